@@ -1,0 +1,113 @@
+"""Pure-Python restatement of the collective operations for TINY inputs.
+
+Written independently of oracle/acc_oracle.c (different language, arbitrary
+Python callables as operators, list-based) so that a slip in either shows up
+as a disagreement.  Definitions follow the same reference comments:
+PrefixSum.hs:137-198 (scans), IndexSpace.hs:144-158 (permute),
+Reduction.hs:37-55,203-215 (fold), Stencil/Extra.hs:198-226 (boundaries).
+"""
+from functools import reduce
+
+
+def scanl(f, z, xs):
+    out = [z]
+    for x in xs:
+        out.append(f(out[-1], x))
+    return out
+
+
+def scanl1(f, xs):
+    out = []
+    for x in xs:
+        out.append(x if not out else f(out[-1], x))
+    return out
+
+
+def scanr(f, z, xs):
+    out = [z]
+    for x in reversed(xs):
+        out.insert(0, f(x, out[0]))
+    return out
+
+
+def scanr1(f, xs):
+    out = []
+    for x in reversed(xs):
+        out.insert(0, x if not out else f(x, out[0]))
+    return out
+
+
+def scanl_p(f, z, xs):
+    r = scanl(f, z, xs)
+    return r[:-1], r[-1]
+
+
+def scanr_p(f, z, xs):
+    r = scanr(f, z, xs)
+    return r[1:], r[0]
+
+
+def fold_left(f, z, xs):
+    """((x0 . x1) . ... . x_{n-1}) . z ; empty -> z"""
+    if not xs:
+        return z
+    return f(reduce(f, xs), z)
+
+
+def fold_right(f, z, xs):
+    """x0 . (x1 . (... (x_{n-1} . z)))"""
+    acc = z
+    for x in reversed(xs):
+        acc = f(x, acc)
+    return acc
+
+
+def fold1_left(f, xs):
+    if not xs:
+        raise ValueError("empty array")
+    return reduce(f, xs)
+
+
+def foldseg(fold, f, z, xs, offsets):
+    return [fold(f, z, xs[offsets[s]:offsets[s + 1]]) for s in range(len(offsets) - 1)]
+
+
+def permute(f, defaults, dst, src, ignore=-1):
+    out = list(defaults)
+    for ix, j in enumerate(dst):
+        if j == ignore:
+            continue
+        out[j] = f(src[ix], out[j])
+    return out
+
+
+def bmap(mode, i, sz):
+    if mode == "clamp":
+        return max(0, min(i, sz - 1))
+    if mode == "mirror":
+        return -i if i < 0 else (sz - (i - sz + 2) if i >= sz else i)
+    if mode == "wrap":
+        return sz + i if i < 0 else (i - sz if i >= sz else i)
+    raise ValueError(mode)
+
+
+def stencil2d(fn, img, offsets, mode, constant=0.0):
+    """fn receives the list of taps in the order of `offsets` [(dy,dx)...]"""
+    h, w = len(img), len(img[0])
+    out = [[None] * w for _ in range(h)]
+    for y in range(h):
+        for x in range(w):
+            taps = []
+            for dy, dx in offsets:
+                yy, xx = y + dy, x + dx
+                if mode == "constant":
+                    taps.append(img[yy][xx] if 0 <= yy < h and 0 <= xx < w else constant)
+                else:
+                    taps.append(img[bmap(mode, yy, h)][bmap(mode, xx, w)])
+            out[y][x] = fn(taps)
+    return out
+
+
+def affine16(x, y):
+    a1, b1, a2, b2 = x >> 16, x & 0xFFFF, y >> 16, y & 0xFFFF
+    return (((a1 * a2) & 0xFFFF) << 16) | ((a1 * b2 + b1) & 0xFFFF)
