@@ -1,0 +1,383 @@
+"""ctypes binding of libacchip (include/acc_hip.h) for tests, the smoke check and
+the bench.  It is a thin, faithful mirror of the C ABI -- the same thing a
+Haskell `foreign import ccall` layer would be -- plus numpy conveniences for
+moving arrays.  It computes nothing itself: every array operation goes through
+the HIP skeletons in the shared library, and loading fails loudly if the
+library has not been built.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libacchip.so")
+CSRC = os.path.join(_HERE, "csrc")
+
+OK, ERR_INVALID, ERR_OOM, ERR_COMPILE, ERR_NOT_FOUND, ERR_HIP, ERR_UNSUPPORTED, ERR_IO = range(8)
+MAX_RANK, MAX_COMP = 8, 8
+
+(SKEL_MAP, SKEL_GENERATE, SKEL_TRANSFORM, SKEL_FOLD, SKEL_FOLD1, SKEL_FOLDSEG, SKEL_FOLD1SEG,
+ SKEL_SCANL, SKEL_SCANL1, SKEL_SCANLP, SKEL_SCANR, SKEL_SCANR1, SKEL_SCANRP, SKEL_PERMUTE,
+ SKEL_STENCIL) = range(15)
+SCAN_KINDS = {"scanl": SKEL_SCANL, "scanl1": SKEL_SCANL1, "scanl'": SKEL_SCANLP,
+              "scanr": SKEL_SCANR, "scanr1": SKEL_SCANR1, "scanr'": SKEL_SCANRP}
+COMBINE_GENERIC, COMBINE_ADD, COMBINE_MIN, COMBINE_MAX, COMBINE_AND, COMBINE_OR, COMBINE_XOR = range(7)
+BOUNDARY = {"clamp": 0, "mirror": 1, "wrap": 2, "constant": 3}
+FLAG_FOLD_RIGHT, FLAG_FAST_MATH = 1, 2
+
+CTYPE = {np.dtype(np.float32): "float", np.dtype(np.float64): "double",
+         np.dtype(np.int8): "Int8", np.dtype(np.int16): "Int16", np.dtype(np.int32): "Int32",
+         np.dtype(np.int64): "Int64", np.dtype(np.uint8): "Word8", np.dtype(np.uint16): "Word16",
+         np.dtype(np.uint32): "Word32", np.dtype(np.uint64): "Word64"}
+
+
+class AccError(RuntimeError):
+    def __init__(self, code, msg):
+        RuntimeError.__init__(self, "libacchip status %d: %s" % (code, msg))
+        self.code = code
+        self.message = msg
+
+
+class acc_array(C.Structure):
+    _fields_ = [("rank", C.c_int32), ("ncomp", C.c_int32),
+                ("shape", C.c_int64 * MAX_RANK), ("ptr", C.c_uint64 * MAX_COMP)]
+
+
+class acc_env_sig(C.Structure):
+    _fields_ = [("rank", C.c_int32), ("ncomp", C.c_int32), ("type", C.c_char_p * MAX_COMP)]
+
+
+class acc_skel_desc(C.Structure):
+    _fields_ = [("kind", C.c_int32), ("flags", C.c_uint32), ("n_env", C.c_int32),
+                ("env", C.POINTER(acc_env_sig)), ("elt_type", C.c_char_p), ("elt_size", C.c_int32),
+                ("out_rank", C.c_int32), ("preamble", C.c_char_p), ("get", C.c_char_p),
+                ("combine", C.c_char_p), ("seed", C.c_char_p), ("permutation", C.c_char_p),
+                ("combine_hint", C.c_int32), ("boundary", C.c_int32), ("boundary_constant", C.c_char_p),
+                ("n_taps", C.c_int32), ("tap_dy", C.POINTER(C.c_int32)), ("tap_dx", C.POINTER(C.c_int32)),
+                ("stencil_fn", C.c_char_p), ("stencil_in_type", C.c_char_p), ("seg_type", C.c_char_p)]
+
+
+class acc_device_props(C.Structure):
+    _fields_ = [("name", C.c_char * 256), ("arch", C.c_char * 64), ("compute_units", C.c_int32),
+                ("wavefront_size", C.c_int32), ("max_threads_per_block", C.c_int32), ("clock_khz", C.c_int32),
+                ("lds_per_block", C.c_int64), ("lds_per_cu", C.c_int64), ("l2_bytes", C.c_int64),
+                ("total_mem", C.c_int64), ("regs_per_block", C.c_int32), ("max_threads_per_cu", C.c_int32)]
+
+
+class acc_cache_stats(C.Structure):
+    _fields_ = [("ram_hits", C.c_uint64), ("disk_hits", C.c_uint64), ("compiles", C.c_uint64),
+                ("disk_errors", C.c_uint64)]
+
+
+class acc_skel_info(C.Structure):
+    _fields_ = [("entry", C.c_char * 64), ("block", C.c_int32), ("blocks_per_cu", C.c_int32),
+                ("num_regs", C.c_int32), ("static_lds", C.c_int32), ("elements_per_block", C.c_int32)]
+
+
+# every symbol include/acc_hip.h declares (tests check that all are exported)
+SYMBOLS = """acc_last_error acc_version acc_init acc_device_count acc_device_get_props acc_context_create
+acc_context_destroy acc_context_device acc_context_sync acc_malloc acc_free acc_mem_info acc_host_alloc
+acc_host_free acc_memcpy_h2d acc_memcpy_d2h acc_memcpy_d2d acc_memcpy_h2d_async acc_memcpy_d2h_async
+acc_memcpy_d2d_async acc_memset32_async acc_stream_create acc_stream_destroy acc_stream_sync
+acc_stream_wait_event acc_event_create acc_event_destroy acc_event_record acc_event_sync acc_event_query
+acc_event_elapsed_ms acc_compile acc_compile_log acc_cache_set_dir acc_cache_dir acc_cache_get_stats
+acc_cache_clear acc_module_load acc_module_unload acc_module_get_function acc_function_attr acc_occupancy
+acc_launch acc_launch_grid acc_skel_create acc_skel_destroy acc_skel_source acc_skel_compile_only
+acc_skel_get_info acc_exec_map acc_exec_fold acc_exec_foldseg acc_exec_scan acc_exec_permute
+acc_exec_stencil acc_exec_stencil_iterate""".split()
+
+
+def build(force=False):
+    """Compile libacchip.so in-tree with the committed Makefile."""
+    if force or not os.path.exists(LIB_PATH):
+        subprocess.check_call(["make", "-C", CSRC, "-j8"] + (["-B"] if force else []), stdout=subprocess.DEVNULL)
+    return LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    """The loaded library.  Raises if it has not been built: there is no fallback."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError("libacchip.so is not built (%s); run `python -c 'import __graft_entry__ as g; g.build()'`"
+                              % LIB_PATH)
+        L = C.CDLL(LIB_PATH)
+        for name in ("acc_last_error", "acc_version", "acc_compile_log", "acc_cache_dir"):
+            getattr(L, name).restype = C.c_char_p
+        L.acc_launch_grid.restype = C.c_int64
+        L.acc_launch_grid.argtypes = [C.c_int64] * 4
+        L.acc_malloc.argtypes = [C.c_void_p, C.c_size_t, C.POINTER(C.c_uint64)]
+        L.acc_free.argtypes = [C.c_void_p, C.c_uint64]
+        L.acc_memcpy_h2d.argtypes = [C.c_void_p, C.c_uint64, C.c_void_p, C.c_size_t]
+        L.acc_memcpy_d2h.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_size_t]
+        L.acc_memcpy_d2d.argtypes = [C.c_void_p, C.c_uint64, C.c_uint64, C.c_size_t]
+        L.acc_memcpy_d2d_async.argtypes = [C.c_void_p, C.c_uint64, C.c_uint64, C.c_size_t, C.c_void_p]
+        L.acc_memset32_async.argtypes = [C.c_void_p, C.c_uint64, C.c_uint32, C.c_size_t, C.c_void_p]
+        L.acc_context_create.argtypes = [C.c_int, C.POINTER(C.c_void_p)]
+        L.acc_context_destroy.argtypes = [C.c_void_p]
+        L.acc_context_sync.argtypes = [C.c_void_p]
+        L.acc_stream_create.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+        L.acc_stream_destroy.argtypes = [C.c_void_p, C.c_void_p]
+        L.acc_stream_sync.argtypes = [C.c_void_p, C.c_void_p]
+        L.acc_event_create.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_void_p)]
+        L.acc_event_destroy.argtypes = [C.c_void_p, C.c_void_p]
+        L.acc_event_record.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+        L.acc_event_sync.argtypes = [C.c_void_p, C.c_void_p]
+        L.acc_event_elapsed_ms.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]
+        L.acc_compile.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.POINTER(C.c_char_p), C.c_int,
+                                  C.POINTER(C.c_void_p), C.POINTER(C.c_size_t)]
+        L.acc_cache_set_dir.argtypes = [C.c_char_p]
+        L.acc_skel_create.argtypes = [C.c_void_p, C.POINTER(acc_skel_desc), C.POINTER(C.c_void_p)]
+        L.acc_skel_destroy.argtypes = [C.c_void_p]
+        L.acc_skel_source.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_char_p)]
+        L.acc_skel_compile_only.argtypes = [C.c_char_p, C.POINTER(acc_skel_desc), C.POINTER(C.c_size_t)]
+        L.acc_skel_get_info.argtypes = [C.c_void_p, C.POINTER(acc_skel_info)]
+        AP = C.POINTER(acc_array)
+        L.acc_exec_map.argtypes = [C.c_void_p, AP, AP, C.c_void_p]
+        L.acc_exec_fold.argtypes = [C.c_void_p, AP, C.c_int32, C.POINTER(C.c_int64), AP, C.c_void_p]
+        L.acc_exec_foldseg.argtypes = [C.c_void_p, AP, C.c_int64, AP, AP, C.c_void_p]
+        L.acc_exec_scan.argtypes = [C.c_void_p, AP, C.c_int64, AP, AP, C.c_void_p]
+        L.acc_exec_permute.argtypes = [C.c_void_p, AP, C.c_int64, AP, AP, C.c_void_p]
+        L.acc_exec_stencil.argtypes = [C.c_void_p, AP, AP, AP, C.c_void_p]
+        L.acc_exec_stencil_iterate.argtypes = [C.c_void_p, AP, AP, AP, C.c_int32, C.c_void_p, C.POINTER(C.c_int32)]
+        _lib = L
+    return _lib
+
+
+def check(rc):
+    if rc != OK:
+        raise AccError(rc, lib().acc_last_error().decode(errors="replace"))
+
+
+def _b(s):
+    return None if s is None else s.encode()
+
+
+def make_desc(kind, elt, env=(), out_rank=0, get=None, combine=None, seed=None, permutation=None,
+              combine_hint=COMBINE_GENERIC, flags=0, preamble=None, boundary="clamp", boundary_constant=None,
+              taps=None, stencil_fn=None, stencil_in=None, seg_type=None, elt_size=0):
+    """env: sequence of (rank, [ctype, ...]) or (rank, ctype).  taps: [(dy, dx), ...] (1-D: [(0, dx)])."""
+    keep = []
+    sigs = (acc_env_sig * max(1, len(env)))()
+    for k, (rank, types) in enumerate(env):
+        if isinstance(types, str):
+            types = [types]
+        sigs[k].rank = rank
+        sigs[k].ncomp = len(types)
+        for c, t in enumerate(types):
+            sigs[k].type[c] = t.encode()
+    d = acc_skel_desc()
+    d.kind, d.flags, d.n_env = kind, flags, len(env)
+    d.env = C.cast(sigs, C.POINTER(acc_env_sig))
+    d.elt_type, d.elt_size, d.out_rank = _b(elt), elt_size, out_rank
+    d.preamble, d.get, d.combine, d.seed = _b(preamble), _b(get), _b(combine), _b(seed)
+    d.permutation, d.combine_hint = _b(permutation), combine_hint
+    d.boundary = BOUNDARY[boundary] if isinstance(boundary, str) else boundary
+    d.boundary_constant = _b(boundary_constant)
+    if taps is not None:
+        dy = (C.c_int32 * len(taps))(*[t[0] for t in taps])
+        dx = (C.c_int32 * len(taps))(*[t[1] for t in taps])
+        keep += [dy, dx]
+        d.n_taps, d.tap_dy, d.tap_dx = len(taps), dy, dx
+    d.stencil_fn, d.stencil_in_type, d.seg_type = _b(stencil_fn), _b(stencil_in), _b(seg_type)
+    d._keep = (sigs, keep)
+    return d
+
+
+def compile_only(desc, target="gfx950"):
+    """hiprtc-compile both variants of a skeleton instance; needs no GPU."""
+    size = C.c_size_t(0)
+    check(lib().acc_skel_compile_only(target.encode(), C.byref(desc), C.byref(size)))
+    return size.value
+
+
+def cache_stats():
+    st = acc_cache_stats()
+    check(lib().acc_cache_get_stats(C.byref(st)))
+    return {"ram_hits": st.ram_hits, "disk_hits": st.disk_hits, "compiles": st.compiles, "disk_errors": st.disk_errors}
+
+
+class DeviceArray(object):
+    """A device-resident array: owner of one acc_malloc'd buffer."""
+
+    def __init__(self, ctx, shape, dtype, ptr=None, owner=True):
+        self.ctx, self.shape, self.dtype = ctx, tuple(int(s) for s in shape), np.dtype(dtype)
+        self.size = int(np.prod(self.shape, dtype=np.int64)) if self.shape else 1
+        self.nbytes = self.size * self.dtype.itemsize
+        self.owner = owner
+        if ptr is None:
+            p = C.c_uint64(0)
+            check(lib().acc_malloc(ctx.handle, self.nbytes, C.byref(p)))
+            ptr = p.value
+        self.ptr = ptr
+
+    def desc(self, shape=None, offset_elems=0):
+        a = acc_array()
+        shape = self.shape if shape is None else tuple(shape)
+        a.rank, a.ncomp = len(shape), 1
+        for i, s in enumerate(shape):
+            a.shape[i] = s
+        a.ptr[0] = self.ptr + offset_elems * self.dtype.itemsize
+        return a
+
+    def get(self):
+        out = np.empty(self.shape, dtype=self.dtype)
+        if self.nbytes:
+            check(lib().acc_memcpy_d2h(self.ctx.handle, out.ctypes.data_as(C.c_void_p), self.ptr, self.nbytes))
+        return out
+
+    def set(self, host):
+        host = np.ascontiguousarray(host, dtype=self.dtype)
+        assert host.size == self.size
+        if self.nbytes:
+            check(lib().acc_memcpy_h2d(self.ctx.handle, self.ptr, host.ctypes.data_as(C.c_void_p), self.nbytes))
+        return self
+
+    def free(self):
+        if self.owner and self.ptr:
+            lib().acc_free(self.ctx.handle, self.ptr)
+            self.ptr = 0
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Context(object):
+    def __init__(self, device=0):
+        h = C.c_void_p()
+        check(lib().acc_init())
+        check(lib().acc_context_create(device, C.byref(h)))
+        self.handle = h
+        self.device = device
+
+    def props(self):
+        p = acc_device_props()
+        check(lib().acc_device_get_props(self.device, C.byref(p)))
+        return p
+
+    def sync(self):
+        check(lib().acc_context_sync(self.handle))
+
+    def empty(self, shape, dtype):
+        if isinstance(shape, int):
+            shape = (shape,)
+        return DeviceArray(self, shape, dtype)
+
+    def array(self, host):
+        host = np.ascontiguousarray(host)
+        return DeviceArray(self, host.shape, host.dtype).set(host)
+
+    def stream(self):
+        s = C.c_void_p()
+        check(lib().acc_stream_create(self.handle, C.byref(s)))
+        return s
+
+    def event(self, timing=True):
+        e = C.c_void_p()
+        check(lib().acc_event_create(self.handle, 1 if timing else 0, C.byref(e)))
+        return e
+
+    def record(self, ev, stream=None):
+        check(lib().acc_event_record(self.handle, ev, stream))
+
+    def elapsed_ms(self, a, b):
+        check(lib().acc_event_sync(self.handle, b))
+        ms = C.c_float(0)
+        check(lib().acc_event_elapsed_ms(self.handle, a, b, C.byref(ms)))
+        return ms.value
+
+    def skeleton(self, *args, **kw):
+        return Skeleton(self, make_desc(*args, **kw))
+
+    def close(self):
+        if self.handle:
+            lib().acc_context_destroy(self.handle)
+            self.handle = None
+
+
+def _env(arrays):
+    if not arrays:
+        return None
+    env = (acc_array * len(arrays))()
+    for k, a in enumerate(arrays):
+        env[k] = a if isinstance(a, acc_array) else a.desc()
+    return env
+
+
+class Skeleton(object):
+    """One compiled skeleton instance (acc_skel)."""
+
+    def __init__(self, ctx, desc):
+        self.ctx, self.desc = ctx, desc
+        h = C.c_void_p()
+        check(lib().acc_skel_create(ctx.handle, C.byref(desc), C.byref(h)))
+        self.handle = h
+
+    def info(self):
+        i = acc_skel_info()
+        check(lib().acc_skel_get_info(self.handle, C.byref(i)))
+        return i
+
+    def source(self, variant=0):
+        s = C.c_char_p()
+        check(lib().acc_skel_source(self.handle, variant, C.byref(s)))
+        return s.value.decode()
+
+    def map(self, env, out, stream=None):
+        check(lib().acc_exec_map(self.handle, _env(env), C.byref(out if isinstance(out, acc_array) else out.desc()), stream))
+
+    def fold(self, env, in_shape, out, stream=None):
+        if isinstance(in_shape, int):
+            in_shape = (in_shape,)
+        sh = (C.c_int64 * len(in_shape))(*in_shape)
+        check(lib().acc_exec_fold(self.handle, _env(env), len(in_shape), sh,
+                                  C.byref(out if isinstance(out, acc_array) else out.desc()), stream))
+
+    def foldseg(self, env, n, offsets, out, stream=None):
+        check(lib().acc_exec_foldseg(self.handle, _env(env), n, C.byref(offsets.desc()), C.byref(out.desc()), stream))
+
+    def scan(self, env, n, out, total=None, stream=None):
+        o = out if isinstance(out, acc_array) else out.desc()
+        t = None if total is None else C.byref(total if isinstance(total, acc_array) else total.desc(shape=()))
+        check(lib().acc_exec_scan(self.handle, _env(env), n, C.byref(o), t, stream))
+
+    def permute(self, env, n_src, defaults, out, stream=None):
+        check(lib().acc_exec_permute(self.handle, _env(env), n_src, C.byref(defaults.desc()), C.byref(out.desc()), stream))
+
+    def stencil(self, env, src, out, stream=None):
+        check(lib().acc_exec_stencil(self.handle, _env(env), C.byref(src.desc()), C.byref(out.desc()), stream))
+
+    def stencil_iterate(self, env, a, b, iters, stream=None):
+        r = C.c_int32(0)
+        check(lib().acc_exec_stencil_iterate(self.handle, _env(env), C.byref(a.desc()), C.byref(b.desc()), iters, stream, C.byref(r)))
+        return b if r.value else a
+
+    def destroy(self):
+        if self.handle:
+            lib().acc_skel_destroy(self.handle)
+            self.handle = None
+
+
+# ---------------------------------------------------------------------------
+# fragments for the benchmark configurations, as the Accelerate code generator
+# would emit them after fusion (CodeGen.hs:714-747 names the array reads)
+
+def linear_stencil_fn(coeffs, divisor=None, ctype="float"):
+    """((c0*t0 + c1*t1) + ...) [/ divisor] with float literals, left to right."""
+    def lit(v):
+        s = repr(float(v))
+        return ("(%sf)" % s) if ctype == "float" else "(%s)" % s
+    e = "%s * t0" % lit(coeffs[0])
+    for k, c in enumerate(coeffs[1:], 1):
+        e = "(%s + %s * t%d)" % (e, lit(c), k)
+    if divisor is not None:
+        e = "(%s / %s)" % (e, lit(divisor))
+    return e

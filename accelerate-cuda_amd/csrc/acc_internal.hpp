@@ -1,0 +1,78 @@
+// Internals shared by the translation units of libacchip.  Not installed.
+#pragma once
+#include <hip/hip_runtime_api.h>
+#include <hip/hiprtc.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../../include/acc_hip.h"
+
+#define ACC_HIP_VERSION "0.1.0"
+
+namespace acc {
+
+// thread-local message of the last failure; returns `code` so that call
+// sites read `return fail(ACC_ERR_INVALID, "...")`
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+int fail_hip(hipError_t e, const char *what);
+void set_compile_log(const std::string &log);
+
+#define ACC_HIP_TRY(expr)                                  \
+  do {                                                     \
+    hipError_t _e = (expr);                                \
+    if (_e != hipSuccess) return ::acc::fail_hip(_e, #expr); \
+  } while (0)
+
+#define ACC_TRY(expr)            \
+  do {                           \
+    int _rc = (expr);            \
+    if (_rc != ACC_OK) return _rc; \
+  } while (0)
+
+// embedded device headers (embed.cpp)
+struct EmbeddedHeader { const char *name; const char *begin; const char *end; };
+const std::vector<EmbeddedHeader> &embedded_headers();
+std::string embedded_text(const char *name);
+
+// A block of device memory lent to one skeleton launch (tile descriptors,
+// block partials, tickets).  Blocks are reused when the borrowing stream is
+// the same (stream order makes that safe) or the event recorded at release
+// has completed.
+enum ScratchProtocol {
+  SCRATCH_FOLD = 0,   // word 0 is a ticket that every launch returns to zero; the rest is don't-care
+  SCRATCH_SCAN = 1    // word 0 is a tile counter used relative to `counter_base`; tile descriptors
+                      // carry `epoch`, so stale ones read as "not yet published"
+};
+
+struct ScratchBlock {
+  void *ptr = nullptr;
+  size_t bytes = 0;
+  int protocol = SCRATCH_FOLD;
+  hipStream_t stream = nullptr;
+  hipEvent_t done = nullptr;
+  bool busy = false;
+  uint32_t epoch = 0;
+  uint32_t counter_base = 0;
+};
+
+}  // namespace acc
+
+struct acc_context_s {
+  int device = 0;
+  hipDeviceProp_t props;
+  std::string arch;          // "gfx950"
+  std::mutex mu;
+  std::vector<acc::ScratchBlock> scratch;
+
+  int make_current() const;
+  // zero-initialised when first allocated; contents persist between uses and
+  // follow the block's protocol
+  int scratch_acquire(size_t bytes, hipStream_t stream, int protocol, int *index);
+  void scratch_release(int index, hipStream_t stream);
+};

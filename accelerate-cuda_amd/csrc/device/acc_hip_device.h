@@ -1,0 +1,184 @@
+/*
+ * acc_hip_device.h -- device-side support for the gfx950 skeleton templates.
+ *
+ * Takes the place of the reference's device headers:
+ *   cubits/accelerate_cuda_type.h:22-30      fixed-width element typedefs
+ *   cubits/accelerate_cuda_function.h:28-193 atomicCAS wrappers, reinterpret, shfl_up/xor
+ * but is written for 64-lane wavefronts: cross-lane traffic uses DPP row
+ * operations and readlane, not 32-wide shuffles, and nothing relies on
+ * warp-synchronous shared memory.
+ *
+ * Every skeleton instance is one translation unit compiled at run time:
+ *     <generated #defines: ACC_ELT, ACC_ENV_PARAMS, ACC_GET, ACC_COMBINE, ...>
+ *     #include "acc_hip_device.h"
+ *     #include "skel_<name>.h"
+ * User fragments are pasted as macros inside the kernel body so that they can
+ * name the kernel's array parameters (arrIn0_0, shIn0_0, ...) directly.
+ */
+#ifndef ACC_HIP_DEVICE_H
+#define ACC_HIP_DEVICE_H
+
+/* element types, named as the Accelerate code generator names them
+ * (CodeGen/Type.hs:106-145: Bool is Word8, Char is Word32, Int is Int64) */
+typedef signed char        Int8;
+typedef short              Int16;
+typedef int                Int32;
+typedef long long          Int64;
+typedef unsigned char      Word8;
+typedef unsigned short     Word16;
+typedef unsigned int       Word32;
+typedef unsigned long long Word64;
+typedef signed char        int8_t;
+typedef short              int16_t;
+typedef int                int32_t;
+typedef long long          int64_t;
+typedef unsigned char      uint8_t;
+typedef unsigned short     uint16_t;
+typedef unsigned int       uint32_t;
+typedef unsigned long long uint64_t;
+
+#define ACC_WAVE 64
+#define ACC_DEV  __device__ __forceinline__
+#define ACC_IGNORE (-1LL)          /* linear image of the index `ignore` */
+
+/* Haskell-flavoured integer helpers the scalar code generator relies on
+ * (CodeGen/Arithmetic.hs:103-134: div/mod round towards minus infinity) */
+template <typename T> ACC_DEV T acc_idiv(T x, T y) { T q = x / y; return ((x % y != 0) && ((x < 0) != (y < 0))) ? q - 1 : q; }
+template <typename T> ACC_DEV T acc_imod(T x, T y) { T r = x % y; return ((r != 0) && ((r < 0) != (y < 0))) ? r + y : r; }
+template <typename T> ACC_DEV T acc_min(T x, T y) { return x < y ? x : y; }
+template <typename T> ACC_DEV T acc_max(T x, T y) { return x > y ? x : y; }
+
+ACC_DEV int acc_lane() { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); }
+
+/* ------------------------------------------------------------------------ */
+/* word-wise movement of arbitrary trivially copyable values across lanes    */
+
+template <typename T> struct acc_words { enum { n = (sizeof(T) + 3) / 4 }; };
+
+/* DPP control words (GFX9 encoding) */
+#define ACC_DPP_ROW_SHL(n)   (0x100 + (n))
+#define ACC_DPP_ROW_SHR(n)   (0x110 + (n))
+#define ACC_DPP_WAVE_SHR1    0x138
+#define ACC_DPP_ROW_BCAST15  0x142
+#define ACC_DPP_ROW_BCAST31  0x143
+
+/* result lane i = src of the lane the control selects; lanes with no source
+ * (or masked out) keep `old` */
+template <int CTRL, int ROW_MASK, typename T>
+ACC_DEV T acc_dpp(const T &old, const T &src)
+{
+  unsigned int o[acc_words<T>::n], s[acc_words<T>::n];
+  o[acc_words<T>::n - 1] = 0; s[acc_words<T>::n - 1] = 0;
+  __builtin_memcpy(o, &old, sizeof(T));
+  __builtin_memcpy(s, &src, sizeof(T));
+#pragma unroll
+  for (int w = 0; w < acc_words<T>::n; ++w)
+    o[w] = (unsigned int)__builtin_amdgcn_update_dpp((int)o[w], (int)s[w], CTRL, ROW_MASK, 0xf, false);
+  T r;
+  __builtin_memcpy(&r, o, sizeof(T));
+  return r;
+}
+
+template <typename T>
+ACC_DEV T acc_readlane(const T &v, int lane)
+{
+  unsigned int s[acc_words<T>::n];
+  s[acc_words<T>::n - 1] = 0;
+  __builtin_memcpy(s, &v, sizeof(T));
+#pragma unroll
+  for (int w = 0; w < acc_words<T>::n; ++w)
+    s[w] = (unsigned int)__builtin_amdgcn_readlane((int)s[w], lane);
+  T r;
+  __builtin_memcpy(&r, s, sizeof(T));
+  return r;
+}
+
+/* ------------------------------------------------------------------------ */
+/* Values that may be absent.  Accelerate's combining functions come with no
+ * identity element (fold1, scanl1, permute), so "nothing here yet" is carried
+ * as a flag and the operator is lifted: absent (+) x = x.                    */
+template <typename T> struct acc_opt { T v; int ok; };
+
+template <typename T> ACC_DEV acc_opt<T> acc_some(const T &v) { acc_opt<T> r; r.v = v; r.ok = 1; return r; }
+template <typename T> ACC_DEV acc_opt<T> acc_none() { acc_opt<T> r; r.v = T(); r.ok = 0; return r; }
+
+template <typename T, typename F>
+struct acc_lifted {
+  F f;
+  ACC_DEV acc_lifted(F f_) : f(f_) {}
+  ACC_DEV acc_opt<T> operator()(const acc_opt<T> &a, const acc_opt<T> &b) const
+  {
+    acc_opt<T> r;
+    r.ok = a.ok | b.ok;
+    r.v  = (a.ok && b.ok) ? f(a.v, b.v) : (a.ok ? a.v : b.v);
+    return r;
+  }
+};
+template <typename T, typename F> ACC_DEV acc_lifted<T, F> acc_lift(F f) { return acc_lifted<T, F>(f); }
+
+/* ------------------------------------------------------------------------ */
+/* wave64 inclusive scan, order preserving: lane i ends with
+ * x_0 (+) x_1 (+) ... (+) x_i, `op(earlier, later)`.  Kogge-Stone inside each
+ * 16-lane DPP row, then the two row-broadcast steps stitch the four rows.    */
+template <typename T, typename F>
+ACC_DEV T acc_wave_scan(T x, F op, int lane)
+{
+  const int r = lane & 15;
+  T t;
+  t = acc_dpp<ACC_DPP_ROW_SHR(1), 0xf>(x, x); if (r >= 1) x = op(t, x);
+  t = acc_dpp<ACC_DPP_ROW_SHR(2), 0xf>(x, x); if (r >= 2) x = op(t, x);
+  t = acc_dpp<ACC_DPP_ROW_SHR(4), 0xf>(x, x); if (r >= 4) x = op(t, x);
+  t = acc_dpp<ACC_DPP_ROW_SHR(8), 0xf>(x, x); if (r >= 8) x = op(t, x);
+  t = acc_dpp<ACC_DPP_ROW_BCAST15, 0xa>(x, x); if (lane & 16) x = op(t, x);
+  t = acc_dpp<ACC_DPP_ROW_BCAST31, 0xc>(x, x); if (lane & 32) x = op(t, x);
+  return x;
+}
+
+/* value of the previous lane (lane 0 keeps its own value: caller masks it) */
+template <typename T> ACC_DEV T acc_wave_shift_up1(const T &x) { return acc_dpp<ACC_DPP_WAVE_SHR1, 0xf>(x, x); }
+
+/* wave64 reduction, order preserving; the result is uniform across the wave */
+template <typename T, typename F>
+ACC_DEV T acc_wave_reduce(T x, F op)
+{
+  T t;
+  t = acc_dpp<ACC_DPP_ROW_SHL(1), 0xf>(x, x); x = op(x, t);
+  t = acc_dpp<ACC_DPP_ROW_SHL(2), 0xf>(x, x); x = op(x, t);
+  t = acc_dpp<ACC_DPP_ROW_SHL(4), 0xf>(x, x); x = op(x, t);
+  t = acc_dpp<ACC_DPP_ROW_SHL(8), 0xf>(x, x); x = op(x, t);
+  /* lane 0 of each row now holds its row; lanes whose partner fell off the
+   * row combined with themselves and are ignored */
+  T r0 = acc_readlane(x, 0), r1 = acc_readlane(x, 16), r2 = acc_readlane(x, 32), r3 = acc_readlane(x, 48);
+  return op(op(r0, r1), op(r2, r3));
+}
+
+/* ------------------------------------------------------------------------ */
+/* atomics on 4- and 8-byte elements of any type, by compare-and-swap on the
+ * bit pattern (replaces cubits/accelerate_cuda_function.h:28-114)            */
+template <int N> struct acc_bits;
+template <> struct acc_bits<4> { typedef unsigned int type; };
+template <> struct acc_bits<8> { typedef unsigned long long type; };
+
+template <typename T, typename F>
+ACC_DEV void acc_atomic_rmw(T *addr, const T &x, F combine_new_old)
+{
+  typedef typename acc_bits<sizeof(T)>::type B;
+  B *p = (B *)addr;
+  B old = *p, assumed;
+  do {
+    assumed = old;
+    T cur, nxt;
+    __builtin_memcpy(&cur, &assumed, sizeof(T));
+    nxt = combine_new_old(x, cur);
+    B nb;
+    __builtin_memcpy(&nb, &nxt, sizeof(T));
+    old = atomicCAS(p, assumed, nb);
+  } while (old != assumed);
+}
+
+/* row-major index helpers (CodeGen/Base.hs:193-218): shapes and indices are
+ * listed innermost dimension LAST, e.g. acc_to_index2(h, w, y, x)            */
+ACC_DEV Int64 acc_to_index2(Int64, Int64 w, Int64 y, Int64 x) { return y * w + x; }
+ACC_DEV Int64 acc_to_index3(Int64, Int64 h, Int64 w, Int64 z, Int64 y, Int64 x) { return (z * h + y) * w + x; }
+
+#endif /* ACC_HIP_DEVICE_H */

@@ -1,0 +1,180 @@
+/*
+ * skel_fold.h -- fold / fold1: reduction of a whole array to one value
+ * (entry foldAll / fold1All) and reduction along the innermost dimension of a
+ * rank > 1 array (entry fold / fold1).
+ *
+ * Takes the place of CodeGen/Reduction.hs:87-215 (mkFoldAll: a first kernel
+ * plus a recursive second one, Execute.hs:291-318) and :221-367 (mkFoldDim),
+ * and of the shared-memory tree reducers at :616-699.
+ *
+ * foldAll is ONE launch: every block strides over tiles of the (fused) input,
+ * each lane reading ACC_UNROLL independent groups of ACC_VEC consecutive
+ * elements per tile; lanes are combined with a wave64 DPP reduction, waves
+ * through a few words of LDS, blocks through one slot each in global memory;
+ * the block that arrives last (atomic ticket) combines the slots, applies the
+ * seed and resets the ticket.  As in the reference the operator must be
+ * associative AND commutative here (the striding reorders elements,
+ * Reduction.hs:160-165), it needs no identity, the seed enters once as the
+ * second operand (Reduction.hs:203-211) and an empty input yields the seed
+ * (:212-214).
+ *
+ * Generated definitions expected: ACC_ENTRY, ACC_ELT, ACC_ENV_PARAMS,
+ * ACC_ENV_ASSUME, ACC_GET(ix), ACC_COMBINE(x,y), ACC_HAS_SEED, ACC_SEED,
+ * ACC_BLOCK, ACC_VEC, ACC_UNROLL, ACC_FOLD_DIM (0: foldAll, 1: innermost dim).
+ */
+
+#define ACC_TILE  (ACC_BLOCK * ACC_VEC * ACC_UNROLL)
+#define ACC_WAVES (ACC_BLOCK / ACC_WAVE)
+
+/* combine the optional per-thread values of a block; result valid in every thread */
+template <typename T, typename F>
+ACC_DEV acc_opt<T> acc_block_reduce(acc_opt<T> x, F f, acc_opt<T> *s_wave)
+{
+  auto lf = acc_lift<T>(f);
+  const int lane = acc_lane();
+  const int wave = (int)(threadIdx.x >> 6);
+  x = acc_wave_reduce(x, lf);
+  if (lane == 0) s_wave[wave] = x;
+  __syncthreads();
+  acc_opt<T> r = s_wave[0];
+#pragma unroll
+  for (int w = 1; w < ACC_WAVES; ++w) r = lf(r, s_wave[w]);
+  __syncthreads();
+  return r;
+}
+
+#if !ACC_FOLD_DIM
+
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+ACC_ENTRY(ACC_ENV_PARAMS
+          ACC_ELT *__restrict__ arrOut_0,
+          const Int64 shIn_0,
+          ACC_ELT *partials, unsigned int *ticket)
+{
+  typedef ACC_ELT T;
+  ACC_ENV_ASSUME
+  __shared__ acc_opt<T> s_wave[ACC_WAVES];
+  __shared__ int s_last;
+
+  auto get = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
+  auto f   = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
+  auto lf  = acc_lift<T>(f);
+
+  const Int64 n = shIn_0;
+  const Int64 full_tiles = n / ACC_TILE;
+
+  /* full tiles: no bounds checks, ACC_UNROLL independent accumulators */
+  T a[ACC_UNROLL];
+  bool have = false;
+  Int64 tile = blockIdx.x;
+  if (tile < full_tiles) {
+    const Int64 base = tile * (Int64)ACC_TILE + (Int64)threadIdx.x * ACC_VEC;
+#pragma unroll
+    for (int u = 0; u < ACC_UNROLL; ++u) {
+      T v = get(base + u * (ACC_BLOCK * ACC_VEC));
+#pragma unroll
+      for (int k = 1; k < ACC_VEC; ++k) v = f(v, get(base + u * (ACC_BLOCK * ACC_VEC) + k));
+      a[u] = v;
+    }
+    have = true;
+    for (tile += gridDim.x; tile < full_tiles; tile += gridDim.x) {
+      const Int64 b2 = tile * (Int64)ACC_TILE + (Int64)threadIdx.x * ACC_VEC;
+      T v[ACC_UNROLL][ACC_VEC];
+#pragma unroll
+      for (int u = 0; u < ACC_UNROLL; ++u)
+#pragma unroll
+        for (int k = 0; k < ACC_VEC; ++k) v[u][k] = get(b2 + u * (ACC_BLOCK * ACC_VEC) + k);
+#pragma unroll
+      for (int u = 0; u < ACC_UNROLL; ++u)
+#pragma unroll
+        for (int k = 0; k < ACC_VEC; ++k) a[u] = f(a[u], v[u][k]);
+    }
+  }
+
+  acc_opt<T> mine = acc_none<T>();
+  if (have) {
+    T v = a[0];
+#pragma unroll
+    for (int u = 1; u < ACC_UNROLL; ++u) v = f(v, a[u]);
+    mine = acc_some(v);
+  }
+
+  /* the ragged last tile, taken by whichever block it falls to */
+  if (full_tiles * (Int64)ACC_TILE < n && (Int64)blockIdx.x == full_tiles % gridDim.x) {
+    const Int64 base = full_tiles * (Int64)ACC_TILE + (Int64)threadIdx.x * ACC_VEC;
+#pragma unroll
+    for (int u = 0; u < ACC_UNROLL; ++u)
+#pragma unroll
+      for (int k = 0; k < ACC_VEC; ++k) {
+        const Int64 ix = base + u * (ACC_BLOCK * ACC_VEC) + k;
+        if (ix < n) mine = lf(mine, acc_some(get(ix)));
+      }
+  }
+
+  acc_opt<T> total = acc_block_reduce(mine, f, s_wave);
+
+  /* hand over to the last block */
+  if (gridDim.x > 1) {
+    if (threadIdx.x == 0) {
+      partials[blockIdx.x] = total.v;            /* host guarantees every block owns >= 1 element */
+      __threadfence();
+      const unsigned int prev = atomicAdd(ticket, 1u);
+      s_last = (prev == gridDim.x - 1);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __threadfence();
+    acc_opt<T> p = acc_none<T>();
+    for (unsigned int i = threadIdx.x; i < gridDim.x; i += ACC_BLOCK) p = lf(p, acc_some(partials[i]));
+    total = acc_block_reduce(p, f, s_wave);
+    if (threadIdx.x == 0) *ticket = 0u;
+  }
+
+  if (threadIdx.x == 0) {
+#if ACC_HAS_SEED
+    const T seed = (ACC_SEED);
+    arrOut_0[0] = total.ok ? f(total.v, seed) : seed;
+#else
+    arrOut_0[0] = total.v;
+#endif
+  }
+}
+
+#else  /* ACC_FOLD_DIM: one wave per innermost row ----------------------------- */
+
+/* rows are the innermost dimension; a wave strides over its row 64*ACC_VEC
+ * elements at a time.  Output has one element per row.                       */
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+ACC_ENTRY(ACC_ENV_PARAMS
+          const Int64 shOut_0, ACC_ELT *__restrict__ arrOut_0,
+          const Int64 shIn_1, const Int64 shIn_0)
+{
+  typedef ACC_ELT T;
+  ACC_ENV_ASSUME
+  (void)shOut_0;
+  auto get = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
+  auto f   = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
+  auto lf  = acc_lift<T>(f);
+
+  const int lane = acc_lane();
+  const Int64 rows = shIn_1, inner = shIn_0;
+  const Int64 wave0 = (Int64)blockIdx.x * ACC_WAVES + (threadIdx.x >> 6);
+  const Int64 nwaves = (Int64)gridDim.x * ACC_WAVES;
+
+  for (Int64 row = wave0; row < rows; row += nwaves) {
+    const Int64 start = row * inner;
+    acc_opt<T> mine = acc_none<T>();
+    for (Int64 i = lane; i < inner; i += ACC_WAVE) mine = lf(mine, acc_some(get(start + i)));
+    acc_opt<T> total = acc_wave_reduce(mine, lf);
+    if (lane == 0) {
+#if ACC_HAS_SEED
+      const T seed = (ACC_SEED);
+      arrOut_0[row] = total.ok ? f(total.v, seed) : seed;      /* Reduction.hs:351-362 */
+#else
+      arrOut_0[row] = total.v;
+#endif
+    }
+  }
+}
+
+#endif

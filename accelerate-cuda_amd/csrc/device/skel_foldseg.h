@@ -1,0 +1,116 @@
+/*
+ * skel_foldseg.h -- foldSeg / fold1Seg: reduce every segment of a vector,
+ * segment s being the index range [offset[s], offset[s+1]).
+ *
+ * Takes the place of CodeGen/Reduction.hs:399-574, which gives each segment a
+ * 32-lane warp (one useful load per lane and a five-step shared-memory tree
+ * for a 32-element row).  With 64-lane waves and short segments most of that
+ * would idle, so the work is split the other way round:
+ *   - a workgroup owns ACC_BLOCK consecutive segments, i.e. ONE contiguous
+ *     range of the input;
+ *   - all its lanes stream that range through LDS in chunks of ACC_CHUNK
+ *     elements, evaluating the (fused) producer with fully coalesced, 128-bit
+ *     reads whatever the segment lengths are;
+ *   - lane i then folds the part of segment i that lies in the chunk, reading
+ *     LDS sequentially, and carries its accumulator to the next chunk.
+ * Every segment is thus combined strictly in index order, the order of a
+ * sequential fold: the operator need only be associative for the result to
+ * be independent of the schedule, and with ACC_FOLD_RIGHT the association is
+ * x0 (+) (x1 (+) (... (+) (x_last (+) z))) instead of
+ * ((x0 (+) x1) (+) ...) (+) z.  The seed is the second operand and an empty
+ * segment yields the seed (Reduction.hs:567-574).
+ *
+ * Generated definitions expected: ACC_ENTRY (via kind), ACC_ELT,
+ * ACC_ENV_PARAMS, ACC_ENV_ASSUME, ACC_GET(ix), ACC_COMBINE(x,y), ACC_HAS_SEED,
+ * ACC_SEED, ACC_SEG_TYPE, ACC_FOLD_RIGHT, ACC_BLOCK, ACC_VEC, ACC_CHUNK.
+ */
+
+static_assert(ACC_CHUNK % (ACC_BLOCK * ACC_VEC) == 0, "chunk must be a whole number of block-wide vector loads");
+
+#if ACC_HAS_SEED
+#define ACC_FOLDSEG_ENTRY foldSeg
+#else
+#define ACC_FOLDSEG_ENTRY fold1Seg
+#endif
+
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
+                  const Int64 shOut_0, ACC_ELT *__restrict__ arrOut_0,
+                  const Int64 shIn_0,
+                  const ACC_SEG_TYPE *__restrict__ arrSeg_0)
+{
+  typedef ACC_ELT T;
+  ACC_ENV_ASSUME
+  __shared__ __attribute__((aligned(16))) T s_val[ACC_CHUNK];
+
+  auto get = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
+  auto f   = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
+
+  const Int64 nseg = shOut_0;
+  const Int64 n = shIn_0;
+  const int tid = threadIdx.x;
+#if ACC_HAS_SEED
+  const T seed = (ACC_SEED);
+#endif
+
+  for (Int64 first = (Int64)blockIdx.x * ACC_BLOCK; first < nseg; first += (Int64)gridDim.x * ACC_BLOCK) {
+    const Int64 seg = first + tid;
+    const bool live = seg < nseg;
+    const Int64 a = live ? (Int64)arrSeg_0[seg] : 0;
+    const Int64 b = live ? (Int64)arrSeg_0[seg + 1] : 0;
+    const Int64 last = acc_min<Int64>(first + ACC_BLOCK, nseg);
+    const Int64 lo = (Int64)arrSeg_0[first], hi = acc_min<Int64>((Int64)arrSeg_0[last], n);
+
+    T acc = T();
+    bool have = false;
+#if ACC_HAS_SEED && ACC_FOLD_RIGHT
+    acc = seed;
+    have = true;
+#endif
+
+    /* chunks start on a vector boundary so that the loads stay aligned */
+    const Int64 lo_al = lo - (lo % ACC_VEC);
+    const Int64 nchunks = hi > lo_al ? (hi - lo_al + ACC_CHUNK - 1) / ACC_CHUNK : 0;
+    for (Int64 q = 0; q < nchunks; ++q) {
+      const Int64 cs = lo_al + (ACC_FOLD_RIGHT ? (nchunks - 1 - q) : q) * (Int64)ACC_CHUNK;
+      const Int64 ce = acc_min<Int64>(cs + ACC_CHUNK, hi);
+      __syncthreads();                               /* the previous chunk has been consumed */
+#pragma unroll
+      for (int u = 0; u < ACC_CHUNK / (ACC_BLOCK * ACC_VEC); ++u) {
+        const int o = (u * ACC_BLOCK + tid) * ACC_VEC;
+        const Int64 ix = cs + o;
+        if (ix + ACC_VEC <= ce && ix >= lo) {
+#pragma unroll
+          for (int k = 0; k < ACC_VEC; ++k) s_val[o + k] = get(ix + k);
+        } else {
+#pragma unroll
+          for (int k = 0; k < ACC_VEC; ++k)
+            if (ix + k >= lo && ix + k < ce) s_val[o + k] = get(ix + k);
+        }
+      }
+      __syncthreads();
+      const Int64 i0 = acc_max(a, cs), i1 = acc_min(b, ce);
+#if ACC_FOLD_RIGHT
+      for (Int64 i = i1 - 1; i >= i0; --i) {
+        const T v = s_val[i - cs];
+        acc = have ? f(v, acc) : v;
+        have = true;
+      }
+#else
+      for (Int64 i = i0; i < i1; ++i) {
+        const T v = s_val[i - cs];
+        acc = have ? f(acc, v) : v;
+        have = true;
+      }
+#endif
+    }
+
+    if (live) {
+#if ACC_HAS_SEED && !ACC_FOLD_RIGHT
+      arrOut_0[seg] = have ? f(acc, seed) : seed;
+#else
+      arrOut_0[seg] = acc;      /* fold1Seg of an empty segment is undefined; T() is written */
+#endif
+    }
+  }
+}

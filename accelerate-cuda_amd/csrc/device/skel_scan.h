@@ -1,0 +1,319 @@
+/*
+ * skel_scan.h -- scanl, scanl1, scanl', scanr, scanr1, scanr' over a vector.
+ *
+ * Takes the place of the reference's three-kernel scan
+ * (CodeGen/PrefixSum.hs:200-365 downsweep, :373-464 upsweep, :470-480 scan of
+ * the interval totals, driven by Execute.hs:364-392).  Here it is ONE kernel:
+ * a single-pass chained scan with decoupled look-back, so the input is read
+ * once and the output written once.
+ *
+ *   - a tile is ACC_BLOCK threads x ACC_ROWS rows x ACC_VEC consecutive items;
+ *     each lane touches ACC_VEC consecutive elements per row, so a wave reads
+ *     64*ACC_VEC contiguous elements per row (128-bit accesses for 4-byte types);
+ *   - inside a wave the row totals are scanned with DPP row shifts / row
+ *     broadcasts (acc_wave_scan), waves are stitched through a few words of LDS;
+ *   - tiles are chained through one descriptor per tile {state, value} in
+ *     global memory.  A tile first publishes its own total (state AGGREGATE),
+ *     then one wave walks back over its predecessors, 64 descriptors per step,
+ *     until it meets an inclusive PREFIX, and finally publishes its own PREFIX.
+ *     Tile numbers are handed out by an atomic counter, so every predecessor
+ *     of a running tile is itself running and the walk cannot deadlock.
+ *   - descriptors are tagged with a launch epoch and the counter is used
+ *     relative to a base, so nothing needs clearing between launches.
+ *
+ * The operator needs no identity and need not commute: `op(earlier, later)`
+ * is applied in logical order only.  For the right-handed scans logical order
+ * is the reverse of memory order and op(a, b) = f(b, a), i.e. the Data.List
+ * convention out[i] = f x[i] out[i+1] (PrefixSum.hs:137-141).
+ *
+ * Output modes (physical index i, logical order as above):
+ *   0  scanl : out[i] = exclusive(i),            out[n] = total     (n+1 results)
+ *   1  scan?1: out[i] = inclusive(i)
+ *   2  scan?': out[i] = exclusive(i),            sum[0] = total
+ *   3  scanr : out[i] = inclusive(i) incl. seed, out[n] = seed      (n+1 results)
+ * which is the pointer arithmetic of Execute.hs:328-362 folded into the kernel.
+ *
+ * Generated definitions expected: ACC_ENTRY, ACC_ELT, ACC_ENV_PARAMS,
+ * ACC_ENV_ASSUME, ACC_GET(ix), ACC_COMBINE(x,y), ACC_HAS_SEED, ACC_SEED,
+ * ACC_SCAN_RIGHT, ACC_SCAN_MODE, ACC_BLOCK, ACC_ROWS, ACC_VEC, ACC_ALIGNED.
+ */
+
+#define ACC_ITEMS (ACC_ROWS * ACC_VEC)
+#define ACC_TILE  (ACC_BLOCK * ACC_ITEMS)
+#define ACC_WAVES (ACC_BLOCK / ACC_WAVE)
+
+#define ACC_ST_AGGREGATE 1u
+#define ACC_ST_PREFIX    2u
+
+/* ---- tile descriptors --------------------------------------------------- */
+/* elements of at most 4 bytes: {flag, value} packed in one 64-bit word that is
+ * read and written with relaxed device-scope atomics -- no fences at all     */
+template <typename T, bool SMALL = (sizeof(T) <= 4)>
+struct acc_scan_desc {
+  unsigned long long *d;
+  ACC_DEV acc_scan_desc(void *p0, void *, void *) : d((unsigned long long *)p0) {}
+  ACC_DEV void put(Int64 tile, unsigned int flag, const T &v) const
+  {
+    unsigned int b = 0;
+    __builtin_memcpy(&b, &v, sizeof(T));
+    __hip_atomic_store(d + tile, ((unsigned long long)flag << 32) | b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  ACC_DEV unsigned int get(Int64 tile, T &v) const
+  {
+    unsigned long long w = __hip_atomic_load(d + tile, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    unsigned int b = (unsigned int)w;
+    __builtin_memcpy(&v, &b, sizeof(T));
+    return (unsigned int)(w >> 32);
+  }
+};
+
+/* wider elements: value slots written plainly, then the flag released; the
+ * reader acquires the flag before touching the slot                          */
+template <typename T>
+struct acc_scan_desc<T, false> {
+  unsigned int *flags; T *agg; T *inc;
+  ACC_DEV acc_scan_desc(void *p0, void *p1, void *p2) : flags((unsigned int *)p0), agg((T *)p1), inc((T *)p2) {}
+  ACC_DEV void put(Int64 tile, unsigned int flag, const T &v) const
+  {
+    T *slot = ((flag & 3u) == ACC_ST_AGGREGATE) ? agg : inc;
+    slot[tile] = v;
+    __hip_atomic_store(flags + tile, flag, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  ACC_DEV unsigned int get(Int64 tile, T &v) const
+  {
+    unsigned int f = __hip_atomic_load(flags + tile, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+    const T *slot = ((f & 3u) == ACC_ST_AGGREGATE) ? agg : inc;
+    v = slot[tile];
+    return f;
+  }
+};
+
+/* ---- full tiles carry plain values, the one ragged tile carries optional
+ *      values so that elements past the end are transparent ---------------- */
+template <typename T, bool PARTIAL> struct acc_sv;
+template <typename T> struct acc_sv<T, false> {
+  typedef T V;
+  static ACC_DEV V some(const T &x) { return x; }
+  static ACC_DEV V none() { return T(); }
+  static ACC_DEV T val(const V &v) { return v; }
+  template <typename F> static ACC_DEV F lift(F f) { return f; }
+};
+template <typename T> struct acc_sv<T, true> {
+  typedef acc_opt<T> V;
+  static ACC_DEV V some(const T &x) { return acc_some(x); }
+  static ACC_DEV V none() { return acc_none<T>(); }
+  static ACC_DEV T val(const V &v) { return v.v; }
+  template <typename F> static ACC_DEV acc_lifted<T, F> lift(F f) { return acc_lift<T>(f); }
+};
+
+/* ---- decoupled look-back, executed by wave 0 of a tile > 0 --------------- */
+template <typename T, typename Op>
+ACC_DEV T acc_scan_lookback(const acc_scan_desc<T> &desc, Int64 tile, const T &block_total, Op op,
+                            unsigned int epoch, int lane)
+{
+  if (lane == 0) desc.put(tile, (epoch << 2) | ACC_ST_AGGREGATE, block_total);
+
+  /* lanes are ordered nearest predecessor first, so a reduction in lane order
+   * must combine (later, earlier) */
+  auto back = acc_lift<T>([&](const T &later, const T &earlier) -> T { return op(earlier, later); });
+  acc_opt<T> run = acc_none<T>();
+
+  for (Int64 look = tile - 1;; look -= ACC_WAVE) {
+    const Int64 idx = look - lane;
+    T v = T();
+    unsigned int st = 0;
+    if (idx >= 0) {
+      unsigned int fl = desc.get(idx, v);
+      while ((fl >> 2) != epoch) {
+        __builtin_amdgcn_s_sleep(1);
+        fl = desc.get(idx, v);
+      }
+      st = fl & 3u;
+    }
+    const unsigned long long prefixes = __ballot(st == ACC_ST_PREFIX);
+    acc_opt<T> c;
+    c.v = v;
+    if (prefixes) {
+      const int first = __ffsll((long long)prefixes) - 1;
+      c.ok = (lane <= first);
+      run = back(run, acc_wave_reduce(c, back));
+      break;
+    }
+    c.ok = 1;                       /* tile 0 always posts a PREFIX, so idx >= 0 here */
+    run = back(run, acc_wave_reduce(c, back));
+  }
+  const T prefix = run.v;
+  if (lane == 0) desc.put(tile, (epoch << 2) | ACC_ST_PREFIX, op(prefix, block_total));
+  return prefix;
+}
+
+/* ---- one tile ------------------------------------------------------------ */
+template <bool PARTIAL, typename T, typename Get, typename Op>
+ACC_DEV void acc_scan_tile(Get get, Op op_raw, const T seed, const Int64 tile, const Int64 base, const Int64 n,
+                           T *__restrict__ out, T *__restrict__ sum, const acc_scan_desc<T> &desc,
+                           const unsigned int epoch, void *s_wave_raw, T *s_prefix)
+{
+  typedef acc_sv<T, PARTIAL> S;
+  typedef typename S::V V;
+  auto op = S::lift(op_raw);
+
+  const int lane = acc_lane();
+  const int wave = (int)(threadIdx.x >> 6);
+  V *s_wave = (V *)s_wave_raw;
+
+  /* load, and scan the ACC_VEC items each lane holds per row */
+  V s[ACC_ROWS][ACC_VEC];
+  Int64 ix0[ACC_ROWS];
+#pragma unroll
+  for (int r = 0; r < ACC_ROWS; ++r) {
+    const int q = ((wave * ACC_ROWS + r) * ACC_WAVE + lane) * ACC_VEC;   /* logical offset in the tile */
+    ix0[r] = base + (ACC_SCAN_RIGHT ? (ACC_TILE - 1 - q) : q);          /* physical index of item k = 0 */
+#pragma unroll
+    for (int k = 0; k < ACC_VEC; ++k) {
+      const Int64 ix = ACC_SCAN_RIGHT ? ix0[r] - k : ix0[r] + k;
+      V v = (!PARTIAL || ix < n) ? S::some(get(ix)) : S::none();
+      s[r][k] = (k == 0) ? v : op(s[r][k - 1], v);
+    }
+  }
+
+  /* scan the per-lane totals of every row across the wave; the rows are
+   * independent chains, which keeps the DPP pipeline busy */
+  V ci[ACC_ROWS];
+#pragma unroll
+  for (int r = 0; r < ACC_ROWS; ++r) ci[r] = acc_wave_scan(s[r][ACC_VEC - 1], op, lane);
+
+  V rowpre[ACC_ROWS];
+  V wave_total = acc_readlane(ci[0], ACC_WAVE - 1);
+  rowpre[0] = wave_total;                                   /* unused */
+#pragma unroll
+  for (int r = 1; r < ACC_ROWS; ++r) {
+    rowpre[r] = wave_total;
+    wave_total = op(wave_total, acc_readlane(ci[r], ACC_WAVE - 1));
+  }
+
+  /* stitch the waves of the block */
+  if (lane == 0) s_wave[wave] = wave_total;
+  __syncthreads();
+  V wavepre = s_wave[0];
+  V block_total = s_wave[0];
+#pragma unroll
+  for (int w = 1; w < ACC_WAVES; ++w) {
+    if (w == wave) wavepre = block_total;
+    block_total = op(block_total, s_wave[w]);
+  }
+
+  /* chain the tiles */
+  T prefix = seed;
+  bool has_prefix = ACC_HAS_SEED;
+  if (tile == 0) {
+    if (threadIdx.x == 0)
+      desc.put(0, (epoch << 2) | ACC_ST_PREFIX,
+               ACC_HAS_SEED ? op_raw(seed, S::val(block_total)) : S::val(block_total));
+  } else {
+    if (wave == 0) {
+      const T p = acc_scan_lookback(desc, tile, S::val(block_total), op_raw, epoch, lane);
+      if (lane == 0) *s_prefix = p;
+    }
+    __syncthreads();
+    prefix = *s_prefix;
+    has_prefix = true;
+  }
+
+  /* apply the prefixes and write */
+#pragma unroll
+  for (int r = 0; r < ACC_ROWS; ++r) {
+    V b = S::some(prefix);
+    bool has_b = has_prefix;
+    if (wave > 0) { b = has_b ? op(b, wavepre) : wavepre; has_b = true; }
+    if (r > 0)    { b = has_b ? op(b, rowpre[r]) : rowpre[r]; has_b = true; }
+
+    const V e = acc_wave_shift_up1(ci[r]);                  /* total of the lanes before this one */
+    V pre;
+    bool has_pre;
+    if (has_b) { pre = (lane == 0) ? b : op(b, e); has_pre = true; }
+    else       { pre = e; has_pre = (lane > 0); }
+
+    V inc[ACC_VEC];
+#pragma unroll
+    for (int k = 0; k < ACC_VEC; ++k) inc[k] = has_pre ? op(pre, s[r][k]) : s[r][k];
+
+    /* the body: one straight run of stores per row so that they merge into
+     * 128-bit accesses */
+    const bool exclusive = (ACC_SCAN_MODE == 0 || ACC_SCAN_MODE == 2);
+#pragma unroll
+    for (int k = 0; k < ACC_VEC; ++k) {
+      const Int64 ix = ACC_SCAN_RIGHT ? ix0[r] - k : ix0[r] + k;
+      if (PARTIAL && ix >= n) continue;
+      out[ix] = exclusive ? S::val(k == 0 ? pre : inc[k - 1]) : S::val(inc[k]);
+    }
+
+    /* the reduction of the whole vector, held by the logically last element */
+    if (ACC_SCAN_MODE == 0 || ACC_SCAN_MODE == 2) {
+      const Int64 last = ACC_SCAN_RIGHT ? 0 : n - 1;
+#pragma unroll
+      for (int k = 0; k < ACC_VEC; ++k) {
+        const Int64 ix = ACC_SCAN_RIGHT ? ix0[r] - k : ix0[r] + k;
+        if (ix == last) {
+          if (ACC_SCAN_MODE == 0) out[n] = S::val(inc[k]);
+          else                    sum[0] = S::val(inc[k]);
+        }
+      }
+    }
+  }
+}
+
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+ACC_ENTRY(ACC_ENV_PARAMS
+          const Int64 shOut_0, ACC_ELT *__restrict__ arrOut_0,
+          ACC_ELT *__restrict__ arrSum_0,
+          const Int64 shIn_0,
+          unsigned int *__restrict__ tile_counter, const unsigned int counter_base,
+          void *desc0, void *desc1, void *desc2,
+          const unsigned int epoch, const Int64 num_tiles)
+{
+  typedef ACC_ELT T;
+  ACC_ENV_ASSUME
+#if ACC_ALIGNED
+  arrOut_0 = (T *)__builtin_assume_aligned(arrOut_0, 16);
+#endif
+  (void)shOut_0;
+
+  __shared__ unsigned int s_tile;
+  __shared__ T s_prefix;
+  __shared__ acc_opt<T> s_wave[ACC_WAVES];
+
+  auto get = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
+  auto f   = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
+  auto op  = [&](const T &earlier, const T &later) -> T { return ACC_SCAN_RIGHT ? f(later, earlier) : f(earlier, later); };
+
+  const Int64 n = shIn_0;
+#if ACC_HAS_SEED
+  const T seed = (ACC_SEED);
+#else
+  const T seed = T();
+#endif
+
+  if (threadIdx.x == 0) s_tile = atomicAdd(tile_counter, 1u) - counter_base;
+  __syncthreads();
+
+  if (n <= 0) {                                   /* PrefixSum.hs:249-251,330-334: scan of nothing is [seed] */
+    if (threadIdx.x == 0 && s_tile == 0) {
+      if (ACC_SCAN_MODE == 0 || ACC_SCAN_MODE == 3) arrOut_0[0] = seed;
+      if (ACC_SCAN_MODE == 2) arrSum_0[0] = seed;
+    }
+    return;
+  }
+
+  const Int64 tile  = (Int64)s_tile;
+  if (tile >= num_tiles) return;
+  const Int64 ptile = ACC_SCAN_RIGHT ? (num_tiles - 1 - tile) : tile;
+  const Int64 base  = ptile * (Int64)ACC_TILE;
+  const acc_scan_desc<T> desc(desc0, desc1, desc2);
+
+  if (ACC_SCAN_MODE == 3 && tile == 0 && threadIdx.x == 0) arrOut_0[n] = seed;
+
+  if (base + ACC_TILE <= n)
+    acc_scan_tile<false, T>(get, op, seed, tile, base, n, arrOut_0, arrSum_0, desc, epoch, (void *)s_wave, &s_prefix);
+  else
+    acc_scan_tile<true, T>(get, op, seed, tile, base, n, arrOut_0, arrSum_0, desc, epoch, (void *)s_wave, &s_prefix);
+}

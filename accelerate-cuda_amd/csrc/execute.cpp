@@ -1,0 +1,387 @@
+// Skeleton drivers: allocate the temporaries a skeleton needs, marshal its
+// arguments, pick the launch shape and enqueue the kernel(s).
+//
+// These are the roles of executeOp / foldCore / foldSegOp / scanCore /
+// permuteOp / stencilOp in CUDA/Execute.hs:264-450, of the argument
+// marshalling at :823-909,930-982 and of the launch arithmetic in
+// CUDA/Analysis/Launch.hs:42-172 -- re-derived for 64-lane wavefronts, 256
+// compute units and single-pass kernels (one launch where the reference needs
+// two or three).
+#include <algorithm>
+#include <cstring>
+#include <deque>
+
+#include "skeleton.hpp"
+
+using acc::fail;
+
+namespace {
+
+// Kernel arguments in launch order.  Every argument of these kernels is at
+// most 8 bytes, so each gets one 8-byte slot whose address is handed to HIP.
+class Args {
+ public:
+  void i64(int64_t v) { push(&v, sizeof(v)); }
+  void u32(uint32_t v) { push(&v, sizeof(v)); }
+  void i32(int32_t v) { push(&v, sizeof(v)); }
+  void ptr(uint64_t v) { push(&v, sizeof(v)); }
+  void **data()
+  {
+    ptrs_.clear();
+    for (uint64_t &s : slots_) ptrs_.push_back(&s);
+    return ptrs_.data();
+  }
+
+ private:
+  void push(const void *p, size_t n)
+  {
+    uint64_t s = 0;
+    std::memcpy(&s, p, n);
+    slots_.push_back(s);
+  }
+  std::deque<uint64_t> slots_;
+  std::vector<void *> ptrs_;
+};
+
+int64_t array_size(const acc_array &a)
+{
+  int64_t n = 1;
+  for (int d = 0; d < a.rank; ++d) n *= a.shape[d];
+  return n;
+}
+
+bool aligned16(uint64_t p) { return (p & 15u) == 0; }
+
+// free array variables first, in Gamma order; per array the extents outermost
+// first, then the component pointers highest component first
+// (CodeGen/Base.hs:344-357, Execute.hs:835-836,946-951)
+int push_env(const acc_skel_s *s, const acc_array *env, Args *args, bool *aligned)
+{
+  const std::vector<acc::EnvSig> &sig = s->spec.env;
+  if (!sig.empty() && !env) return fail(ACC_ERR_INVALID, "%s: env arrays missing", s->entry.c_str());
+  for (size_t k = 0; k < sig.size(); ++k) {
+    const acc_array &a = env[k];
+    if (a.rank != sig[k].rank || a.ncomp != sig[k].ncomp)
+      return fail(ACC_ERR_INVALID, "%s: env array %zu has rank %d / %d components, the kernel was built for %d / %d",
+                  s->entry.c_str(), k, a.rank, a.ncomp, sig[k].rank, sig[k].ncomp);
+    int64_t n = 1;
+    for (int d = 0; d < a.rank; ++d) {
+      if (a.shape[d] < 0) return fail(ACC_ERR_INVALID, "%s: env array %zu has a negative extent", s->entry.c_str(), k);
+      n *= a.shape[d];
+      args->i64(a.shape[d]);
+    }
+    for (int c = a.ncomp - 1; c >= 0; --c) {
+      if (!a.ptr[c] && n > 0) return fail(ACC_ERR_INVALID, "%s: env array %zu component %d is NULL", s->entry.c_str(), k, c);
+      if (!aligned16(a.ptr[c])) *aligned = false;
+      args->ptr(a.ptr[c]);
+    }
+  }
+  return ACC_OK;
+}
+
+int check_out(const acc_skel_s *s, const acc_array *out, int rank, const char *what)
+{
+  if (!out) return fail(ACC_ERR_INVALID, "%s: %s array missing", s->entry.c_str(), what);
+  if (out->rank != rank) return fail(ACC_ERR_INVALID, "%s: %s array has rank %d, expected %d", s->entry.c_str(), what, out->rank, rank);
+  if (out->ncomp != 1) return fail(ACC_ERR_UNSUPPORTED, "%s: tuple-typed %s arrays are not supported", s->entry.c_str(), what);
+  for (int d = 0; d < rank; ++d)
+    if (out->shape[d] < 0) return fail(ACC_ERR_INVALID, "%s: %s array has a negative extent", s->entry.c_str(), what);
+  if (!out->ptr[0] && array_size(*out) > 0) return fail(ACC_ERR_INVALID, "%s: %s array is NULL", s->entry.c_str(), what);
+  return ACC_OK;
+}
+
+void push_out(const acc_array &out, Args *args, bool *aligned)
+{
+  for (int d = 0; d < out.rank; ++d) args->i64(out.shape[d]);
+  if (!aligned16(out.ptr[0])) *aligned = false;
+  args->ptr(out.ptr[0]);
+}
+
+int launch(acc_skel_s *s, int variant, int64_t grid, size_t dyn_lds, hipStream_t stream, Args *args)
+{
+  if (grid < 1 || grid > 0x7fffffffLL) return fail(ACC_ERR_INVALID, "%s: grid of %lld blocks", s->entry.c_str(), (long long)grid);
+  ACC_TRY(s->ensure_variant(variant));
+  ACC_TRY(s->ctx->make_current());
+  ACC_HIP_TRY(hipModuleLaunchKernel(s->variants[variant].fn, static_cast<unsigned>(grid), 1, 1,
+                                    static_cast<unsigned>(s->spec.block), 1, 1, static_cast<unsigned>(dyn_lds), stream,
+                                    args->data(), nullptr));
+  return ACC_OK;
+}
+
+bool kind_is(const acc_skel_s *s, std::initializer_list<int> kinds)
+{
+  return std::find(kinds.begin(), kinds.end(), s->spec.kind) != kinds.end();
+}
+
+size_t round256(size_t n) { return (n + 255) & ~size_t(255); }
+
+// resident-grid cap: compute units x workgroups per unit (Launch.hs:51-55)
+int64_t resident(const acc_skel_s *s, int variant) { return (int64_t)s->ctx->props.multiProcessorCount * s->variants[variant].blocks_per_cu; }
+
+}  // namespace
+
+extern "C" {
+
+int acc_exec_map(acc_skel s, const acc_array *env, const acc_array *out, acc_stream stream)
+{
+  if (!s) return fail(ACC_ERR_INVALID, "acc_exec_map: NULL skeleton");
+  if (!kind_is(s, {ACC_SKEL_MAP, ACC_SKEL_GENERATE, ACC_SKEL_TRANSFORM})) return fail(ACC_ERR_INVALID, "acc_exec_map: skeleton is '%s'", s->entry.c_str());
+  ACC_TRY(check_out(s, out, s->spec.out_rank, "result"));
+  Args args;
+  bool aligned = true;
+  ACC_TRY(push_env(s, env, &args, &aligned));
+  push_out(*out, &args, &aligned);
+  const int64_t n = array_size(*out);
+  if (n == 0) return ACC_OK;
+  const int v = aligned ? 0 : 1;
+  ACC_TRY(s->ensure_variant(v));
+  const int64_t grid = acc_launch_grid(n, s->elements_per_block(), resident(s, v), acc::tune("map.oversub", 8));
+  return launch(s, v, grid, 0, static_cast<hipStream_t>(stream), &args);
+}
+
+int acc_exec_fold(acc_skel s, const acc_array *env, int32_t in_rank, const int64_t *in_shape, const acc_array *out, acc_stream stream)
+{
+  if (!s) return fail(ACC_ERR_INVALID, "acc_exec_fold: NULL skeleton");
+  if (!kind_is(s, {ACC_SKEL_FOLD, ACC_SKEL_FOLD1})) return fail(ACC_ERR_INVALID, "acc_exec_fold: skeleton is '%s'", s->entry.c_str());
+  if (in_rank != s->spec.out_rank + 1 || !in_shape) return fail(ACC_ERR_INVALID, "%s: input rank %d, kernel was built for %d", s->entry.c_str(), in_rank, s->spec.out_rank + 1);
+  ACC_TRY(check_out(s, out, s->spec.out_rank, "result"));
+  for (int d = 0; d < in_rank; ++d)
+    if (in_shape[d] < 0) return fail(ACC_ERR_INVALID, "%s: negative input extent", s->entry.c_str());
+  const int64_t inner = in_shape[in_rank - 1];
+  // fold1 of an empty innermost dimension: Execute.hs:282-285
+  if (inner == 0 && !s->spec.has_seed) return fail(ACC_ERR_INVALID, "%s: empty array", s->entry.c_str());
+  // empty outer extents count as 1: Execute.hs:287-289
+  int64_t rows = 1;
+  for (int d = 0; d + 1 < in_rank; ++d) rows *= std::max<int64_t>(1, in_shape[d]);
+  if (array_size(*out) < rows && !(in_rank == 1)) return fail(ACC_ERR_INVALID, "%s: result holds %lld elements, %lld needed", s->entry.c_str(), (long long)array_size(*out), (long long)rows);
+
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  Args args;
+  bool aligned = true;
+  ACC_TRY(push_env(s, env, &args, &aligned));
+  const int v = aligned ? 0 : 1;
+  ACC_TRY(s->ensure_variant(v));
+
+  if (s->spec.out_rank > 0) {      // one wave per innermost row
+    args.i64(rows);
+    args.ptr(out->ptr[0]);
+    args.i64(rows);
+    args.i64(inner);
+    const int waves = s->spec.block / 64;
+    const int64_t grid = acc_launch_grid(rows, waves, resident(s, v), 4);
+    return launch(s, v, grid, 0, st, &args);
+  }
+
+  const int64_t n = inner;
+  const int64_t tile = s->elements_per_block();
+  const int64_t grid = acc_launch_grid(n, tile, resident(s, v), acc::tune("fold.oversub", 1));
+  int blk = -1;
+  ACC_TRY(s->ctx->scratch_acquire(256 + (size_t)grid * s->spec.elt_size, st, acc::SCRATCH_FOLD, &blk));
+  char *base = static_cast<char *>(s->ctx->scratch[blk].ptr);
+  args.ptr(out->ptr[0]);
+  args.i64(n);
+  args.ptr(reinterpret_cast<uint64_t>(base + 256));
+  args.ptr(reinterpret_cast<uint64_t>(base));
+  const int rc = launch(s, v, grid, 0, st, &args);
+  s->ctx->scratch_release(blk, st);
+  return rc;
+}
+
+int acc_exec_foldseg(acc_skel s, const acc_array *env, int64_t n, const acc_array *offsets, const acc_array *out, acc_stream stream)
+{
+  if (!s) return fail(ACC_ERR_INVALID, "acc_exec_foldseg: NULL skeleton");
+  if (!kind_is(s, {ACC_SKEL_FOLDSEG, ACC_SKEL_FOLD1SEG})) return fail(ACC_ERR_INVALID, "acc_exec_foldseg: skeleton is '%s'", s->entry.c_str());
+  ACC_TRY(check_out(s, offsets, 1, "segment offsets"));
+  ACC_TRY(check_out(s, out, 1, "result"));
+  if (n < 0) return fail(ACC_ERR_INVALID, "%s: negative input extent", s->entry.c_str());
+  // the offsets vector is one longer than the number of segments: Execute.hs:320-324
+  const int64_t nseg = offsets->shape[0] - 1;
+  if (nseg <= 0) return ACC_OK;
+  if (out->shape[0] < nseg) return fail(ACC_ERR_INVALID, "%s: result holds %lld segments, %lld needed", s->entry.c_str(), (long long)out->shape[0], (long long)nseg);
+  Args args;
+  bool aligned = true;
+  ACC_TRY(push_env(s, env, &args, &aligned));
+  args.i64(nseg);
+  args.ptr(out->ptr[0]);
+  args.i64(n);
+  args.ptr(offsets->ptr[0]);
+  const int v = aligned ? 0 : 1;
+  ACC_TRY(s->ensure_variant(v));
+  const int64_t grid = acc_launch_grid(nseg, s->spec.block, resident(s, v), acc::tune("foldseg.oversub", 8));
+  return launch(s, v, grid, 0, static_cast<hipStream_t>(stream), &args);
+}
+
+int acc_exec_scan(acc_skel s, const acc_array *env, int64_t n, const acc_array *out, const acc_array *total, acc_stream stream)
+{
+  if (!s) return fail(ACC_ERR_INVALID, "acc_exec_scan: NULL skeleton");
+  if (!kind_is(s, {ACC_SKEL_SCANL, ACC_SKEL_SCANL1, ACC_SKEL_SCANLP, ACC_SKEL_SCANR, ACC_SKEL_SCANR1, ACC_SKEL_SCANRP}))
+    return fail(ACC_ERR_INVALID, "acc_exec_scan: skeleton is '%s'", s->entry.c_str());
+  if (n < 0) return fail(ACC_ERR_INVALID, "%s: negative input extent", s->entry.c_str());
+  ACC_TRY(check_out(s, out, 1, "result"));
+  const int kind = s->spec.kind;
+  const bool plus_one = (kind == ACC_SKEL_SCANL || kind == ACC_SKEL_SCANR);     // Execute.hs:328-339
+  const bool primed = (kind == ACC_SKEL_SCANLP || kind == ACC_SKEL_SCANRP);     // Execute.hs:352-362
+  if (out->shape[0] < n + (plus_one ? 1 : 0))
+    return fail(ACC_ERR_INVALID, "%s: result holds %lld elements, %lld needed", s->entry.c_str(), (long long)out->shape[0], (long long)(n + (plus_one ? 1 : 0)));
+  uint64_t sum_ptr = 0;
+  if (primed) {
+    ACC_TRY(check_out(s, total, 0, "total"));
+    sum_ptr = total->ptr[0];
+  }
+  if (n == 0 && !plus_one && !primed) return ACC_OK;       // scanl1 / scanr1 of nothing is nothing
+
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  Args args;
+  bool aligned = true;
+  ACC_TRY(push_env(s, env, &args, &aligned));
+  push_out(*out, &args, &aligned);
+  args.ptr(sum_ptr);
+  args.i64(n);
+
+  const int64_t tile = s->elements_per_block();
+  const int64_t tiles = (n + tile - 1) / tile;
+  const int64_t grid = std::max<int64_t>(1, tiles);
+  const size_t esz = s->spec.elt_size;
+  size_t bytes = 256;
+  size_t off_d0 = 256, off_d1 = 0, off_d2 = 0;
+  if (esz <= 4) {
+    bytes += round256((size_t)grid * 8);
+  } else {
+    off_d1 = off_d0 + round256((size_t)grid * 4);
+    off_d2 = off_d1 + round256((size_t)grid * esz);
+    bytes = off_d2 + round256((size_t)grid * esz);
+  }
+  int blk = -1;
+  ACC_TRY(s->ctx->scratch_acquire(bytes, st, acc::SCRATCH_SCAN, &blk));
+  uint32_t epoch, counter_base;
+  char *base;
+  {
+    std::lock_guard<std::mutex> lock(s->ctx->mu);
+    acc::ScratchBlock &b = s->ctx->scratch[blk];
+    base = static_cast<char *>(b.ptr);
+    if (b.epoch + 1 >= (1u << 30)) {          // descriptor tags are 30 bits wide: start over from a clean block
+      hipError_t e = hipMemsetAsync(b.ptr, 0, b.bytes, st);
+      if (e != hipSuccess) { b.busy = false; return acc::fail_hip(e, "hipMemsetAsync(scan state)"); }
+      b.epoch = 0;
+      b.counter_base = 0;
+    }
+    epoch = ++b.epoch;
+    counter_base = b.counter_base;
+    b.counter_base += static_cast<uint32_t>(grid);    // every launched block draws exactly one ticket
+  }
+  args.ptr(reinterpret_cast<uint64_t>(base));
+  args.u32(counter_base);
+  args.ptr(reinterpret_cast<uint64_t>(base + off_d0));
+  args.ptr(reinterpret_cast<uint64_t>(base + off_d1));
+  args.ptr(reinterpret_cast<uint64_t>(base + off_d2));
+  args.u32(epoch);
+  args.i64(tiles);
+  const int rc = launch(s, aligned ? 0 : 1, grid, 0, st, &args);
+  if (rc != ACC_OK) {
+    // nothing ran: take the tickets back so that the block stays consistent
+    std::lock_guard<std::mutex> lock(s->ctx->mu);
+    s->ctx->scratch[blk].counter_base = counter_base;
+  }
+  s->ctx->scratch_release(blk, st);
+  return rc;
+}
+
+int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_array *defaults, const acc_array *out, acc_stream stream)
+{
+  if (!s) return fail(ACC_ERR_INVALID, "acc_exec_permute: NULL skeleton");
+  if (!kind_is(s, {ACC_SKEL_PERMUTE})) return fail(ACC_ERR_INVALID, "acc_exec_permute: skeleton is '%s'", s->entry.c_str());
+  if (n_src < 0) return fail(ACC_ERR_INVALID, "permute: negative source extent");
+  ACC_TRY(check_out(s, out, s->spec.out_rank, "result"));
+  ACC_TRY(check_out(s, defaults, s->spec.out_rank, "defaults"));
+  for (int d = 0; d < out->rank; ++d)
+    if (defaults->shape[d] != out->shape[d]) return fail(ACC_ERR_INVALID, "permute: defaults and result differ in shape");
+  const int64_t ntarget = array_size(*out);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const size_t esz = s->spec.elt_size;
+  ACC_TRY(s->ctx->make_current());
+  // the result starts as a copy of the defaults: Execute.hs:401-406 (no lock array here)
+  if (ntarget > 0 && defaults->ptr[0] != out->ptr[0])
+    ACC_HIP_TRY(hipMemcpyAsync(reinterpret_cast<void *>(out->ptr[0]), reinterpret_cast<void *>(defaults->ptr[0]), (size_t)ntarget * esz, hipMemcpyDeviceToDevice, st));
+  if (n_src == 0 || ntarget == 0) return ACC_OK;
+
+  Args args;
+  bool aligned = true;
+  ACC_TRY(push_env(s, env, &args, &aligned));
+  push_out(*out, &args, &aligned);
+  args.i64(n_src);
+  const int v = aligned ? 0 : 1;
+  ACC_TRY(s->ensure_variant(v));
+
+  // privatise target indices [0, bins) in LDS when the combine has a hardware
+  // atomic and an identity; small targets get one copy per wave to spread
+  // same-address traffic
+  int64_t bins = 0, copies = 1;
+  if (s->spec.combine_hint != ACC_COMBINE_GENERIC) {
+    const int64_t budget = std::min<int64_t>((int64_t)s->ctx->props.sharedMemPerBlock, acc::tune("permute.lds_bytes", 65536)) - s->variants[v].static_lds;
+    const int64_t cap = std::max<int64_t>(0, budget / (int64_t)esz);
+    bins = std::min(ntarget, cap);
+    if (bins == ntarget && bins > 0) copies = std::max<int64_t>(1, std::min<int64_t>(s->spec.block / 64, cap / bins));
+    copies = std::min<int64_t>(copies, acc::tune("permute.max_copies", 16));
+  }
+  const size_t lds = (size_t)(bins * copies) * esz;
+  args.i32(static_cast<int32_t>(bins));
+  args.i32(static_cast<int32_t>(copies));
+  int bpc = 0;
+  hipError_t e = hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&bpc, s->variants[v].fn, s->spec.block, lds);
+  if (e != hipSuccess || bpc < 1) { (void)hipGetLastError(); bpc = 1; }
+  const int64_t grid = acc_launch_grid(n_src, s->elements_per_block(), s->ctx->props.multiProcessorCount, std::min(bpc, acc::tune("permute.max_blocks_per_cu", 4)));
+  return launch(s, v, grid, lds, st, &args);
+}
+
+static int stencil_once(acc_skel s, const acc_array *env, const acc_array *in, const acc_array *out, hipStream_t st)
+{
+  const int rank = s->spec.out_rank;
+  Args args;
+  bool aligned = true;
+  ACC_TRY(push_env(s, env, &args, &aligned));
+  push_out(*out, &args, &aligned);
+  if (!aligned16(in->ptr[0])) aligned = false;
+  args.ptr(in->ptr[0]);
+  const int64_t w = out->shape[rank - 1];
+  const int64_t h = rank == 2 ? out->shape[0] : 1;
+  if (w == 0 || h == 0) return ACC_OK;
+  // rows start on 16-byte boundaries only if the row pitch allows it
+  const size_t in_esz = acc::type_size(s->spec.stencil_in_type) ? acc::type_size(s->spec.stencil_in_type) : s->spec.elt_size;
+  if ((w * (int64_t)s->spec.elt_size) % 16 != 0 || (w * (int64_t)in_esz) % 16 != 0) aligned = false;
+  const int64_t tx = (w + s->spec.tile_w - 1) / s->spec.tile_w;
+  const int64_t ty = (h + s->spec.tile_h - 1) / s->spec.tile_h;
+  return launch(s, aligned ? 0 : 1, tx * ty, 0, st, &args);
+}
+
+static int stencil_check(acc_skel s, const acc_array *in, const acc_array *out)
+{
+  if (!s) return fail(ACC_ERR_INVALID, "acc_exec_stencil: NULL skeleton");
+  if (!kind_is(s, {ACC_SKEL_STENCIL})) return fail(ACC_ERR_INVALID, "acc_exec_stencil: skeleton is '%s'", s->entry.c_str());
+  ACC_TRY(check_out(s, out, s->spec.out_rank, "result"));
+  ACC_TRY(check_out(s, in, s->spec.out_rank, "source"));
+  for (int d = 0; d < out->rank; ++d)
+    if (in->shape[d] != out->shape[d]) return fail(ACC_ERR_INVALID, "stencil: source and result differ in shape");
+  if (in->ptr[0] == out->ptr[0] && array_size(*out) > 0) return fail(ACC_ERR_INVALID, "stencil: source and result must not alias");
+  return ACC_OK;
+}
+
+int acc_exec_stencil(acc_skel s, const acc_array *env, const acc_array *in, const acc_array *out, acc_stream stream)
+{
+  ACC_TRY(stencil_check(s, in, out));
+  return stencil_once(s, env, in, out, static_cast<hipStream_t>(stream));
+}
+
+int acc_exec_stencil_iterate(acc_skel s, const acc_array *env, const acc_array *a, const acc_array *b, int32_t iters, acc_stream stream, int32_t *result_in_b)
+{
+  ACC_TRY(stencil_check(s, a, b));
+  if (iters < 0) return fail(ACC_ERR_INVALID, "stencil: negative iteration count");
+  const acc_array *src = a, *dst = b;
+  for (int32_t i = 0; i < iters; ++i) {
+    ACC_TRY(stencil_once(s, env, src, dst, static_cast<hipStream_t>(stream)));
+    std::swap(src, dst);
+  }
+  if (result_in_b) *result_in_b = (iters & 1);
+  return ACC_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,427 @@
+// Driver layer of libacchip: devices, contexts, memory, transfers, streams,
+// events, modules, occupancy and raw launches over libamdhip64.
+//
+// It stands where accelerate-cuda reaches the `cuda` package:
+//   State.hs:127-132, Context.hs:55-111      initialise / create / destroy
+//   Array/Remote.hs:63-79,191                mallocArray / free / getMemInfo
+//   Array/Prim.hs:189-391                    peek / poke / copy [Async]
+//   Execute/Stream.hs, Execute/Event.hs      stream and event handling
+//   Compile.hs:453-465,505,534               loadData / getFun / requires
+//   Execute.hs:975-978                       launchKernel
+#include <cstring>
+
+#include "acc_internal.hpp"
+
+namespace acc {
+
+static thread_local std::string g_last_error;
+static thread_local std::string g_compile_log;
+
+int fail(int code, const char *fmt, ...)
+{
+  char buf[2048];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  g_last_error = buf;
+  return code;
+}
+
+int fail_hip(hipError_t e, const char *what)
+{
+  // the one error a caller is expected to recover from (Array/Remote.hs:63-67)
+  const int code = (e == hipErrorOutOfMemory) ? ACC_ERR_OOM : ACC_ERR_HIP;
+  (void)hipGetLastError();  // do not let a sticky error leak into the next call
+  return fail(code, "%s: %s (%d)", what, hipGetErrorString(e), static_cast<int>(e));
+}
+
+void set_compile_log(const std::string &log) { g_compile_log = log; }
+
+}  // namespace acc
+
+using acc::fail;
+
+int acc_context_s::make_current() const
+{
+  ACC_HIP_TRY(hipSetDevice(device));
+  return ACC_OK;
+}
+
+int acc_context_s::scratch_acquire(size_t bytes, hipStream_t stream, int protocol, int *index)
+{
+  std::lock_guard<std::mutex> lock(mu);
+  int pick = -1;
+  for (size_t i = 0; i < scratch.size(); ++i) {
+    acc::ScratchBlock &b = scratch[i];
+    if (b.busy || b.bytes < bytes || b.protocol != protocol) continue;
+    bool reusable = (b.stream == stream);
+    if (!reusable && b.done) reusable = (hipEventQuery(b.done) == hipSuccess);
+    if (reusable && (pick < 0 || b.bytes < scratch[pick].bytes)) pick = static_cast<int>(i);
+  }
+  if (pick < 0) {
+    acc::ScratchBlock b;
+    b.bytes = (bytes + 4095) & ~size_t(4095);
+    ACC_HIP_TRY(hipMalloc(&b.ptr, b.bytes));
+    hipError_t e = hipEventCreateWithFlags(&b.done, hipEventDisableTiming);
+    if (e != hipSuccess) { (void)hipFree(b.ptr); return acc::fail_hip(e, "hipEventCreateWithFlags"); }
+    b.protocol = protocol;
+    // cleared once, on the stream that first uses it (not meant to be captured into a graph)
+    e = hipMemsetAsync(b.ptr, 0, b.bytes, stream);
+    if (e != hipSuccess) { (void)hipEventDestroy(b.done); (void)hipFree(b.ptr); return acc::fail_hip(e, "hipMemsetAsync(scratch)"); }
+    scratch.push_back(b);
+    pick = static_cast<int>(scratch.size()) - 1;
+  }
+  acc::ScratchBlock &b = scratch[pick];
+  b.busy = true;
+  b.stream = stream;
+  *index = pick;
+  return ACC_OK;
+}
+
+void acc_context_s::scratch_release(int index, hipStream_t stream)
+{
+  std::lock_guard<std::mutex> lock(mu);
+  acc::ScratchBlock &b = scratch[index];
+  (void)hipEventRecord(b.done, stream);
+  b.stream = stream;
+  b.busy = false;
+}
+
+extern "C" {
+
+const char *acc_last_error(void) { return acc::g_last_error.c_str(); }
+const char *acc_compile_log(void) { return acc::g_compile_log.c_str(); }
+const char *acc_version(void) { return ACC_HIP_VERSION; }
+
+int acc_init(void)
+{
+  ACC_HIP_TRY(hipInit(0));
+  return ACC_OK;
+}
+
+int acc_device_count(int *count)
+{
+  if (!count) return fail(ACC_ERR_INVALID, "acc_device_count: NULL argument");
+  *count = 0;
+  ACC_HIP_TRY(hipGetDeviceCount(count));
+  return ACC_OK;
+}
+
+static void fill_props(const hipDeviceProp_t &p, acc_device_props *out)
+{
+  std::memset(out, 0, sizeof(*out));
+  std::snprintf(out->name, sizeof(out->name), "%s", p.name);
+  std::snprintf(out->arch, sizeof(out->arch), "%.63s", p.gcnArchName);
+  out->compute_units = p.multiProcessorCount;
+  out->wavefront_size = p.warpSize;
+  out->max_threads_per_block = p.maxThreadsPerBlock;
+  out->clock_khz = p.clockRate;
+  out->lds_per_block = static_cast<int64_t>(p.sharedMemPerBlock);
+  out->lds_per_cu = static_cast<int64_t>(p.maxSharedMemoryPerMultiProcessor);
+  out->l2_bytes = p.l2CacheSize;
+  out->total_mem = static_cast<int64_t>(p.totalGlobalMem);
+  out->regs_per_block = p.regsPerBlock;
+  out->max_threads_per_cu = p.maxThreadsPerMultiProcessor;
+}
+
+int acc_device_get_props(int device, acc_device_props *out)
+{
+  if (!out) return fail(ACC_ERR_INVALID, "acc_device_get_props: NULL argument");
+  hipDeviceProp_t p;
+  ACC_HIP_TRY(hipGetDeviceProperties(&p, device));
+  fill_props(p, out);
+  return ACC_OK;
+}
+
+int acc_context_create(int device, acc_context *out)
+{
+  if (!out) return fail(ACC_ERR_INVALID, "acc_context_create: NULL argument");
+  *out = nullptr;
+  int n = 0;
+  ACC_HIP_TRY(hipGetDeviceCount(&n));
+  if (device < 0 || device >= n) return fail(ACC_ERR_NOT_FOUND, "acc_context_create: no device %d (%d present)", device, n);
+  acc_context_s *ctx = new acc_context_s();
+  ctx->device = device;
+  hipError_t e = hipGetDeviceProperties(&ctx->props, device);
+  if (e == hipSuccess) e = hipSetDevice(device);
+  if (e != hipSuccess) { delete ctx; return acc::fail_hip(e, "acc_context_create"); }
+  ctx->arch = ctx->props.gcnArchName;
+  const size_t colon = ctx->arch.find(':');
+  if (colon != std::string::npos) ctx->arch.resize(colon);
+  *out = ctx;
+  return ACC_OK;
+}
+
+int acc_context_destroy(acc_context ctx)
+{
+  if (!ctx) return ACC_OK;
+  (void)hipSetDevice(ctx->device);
+  (void)hipDeviceSynchronize();
+  for (acc::ScratchBlock &b : ctx->scratch) {
+    if (b.done) (void)hipEventDestroy(b.done);
+    if (b.ptr) (void)hipFree(b.ptr);
+  }
+  delete ctx;
+  return ACC_OK;
+}
+
+int acc_context_device(acc_context ctx, int *device)
+{
+  if (!ctx || !device) return fail(ACC_ERR_INVALID, "acc_context_device: NULL argument");
+  *device = ctx->device;
+  return ACC_OK;
+}
+
+int acc_context_sync(acc_context ctx)
+{
+  if (!ctx) return fail(ACC_ERR_INVALID, "acc_context_sync: NULL context");
+  ACC_TRY(ctx->make_current());
+  ACC_HIP_TRY(hipDeviceSynchronize());
+  return ACC_OK;
+}
+
+int acc_malloc(acc_context ctx, size_t bytes, acc_devptr *out)
+{
+  if (!ctx || !out) return fail(ACC_ERR_INVALID, "acc_malloc: NULL argument");
+  *out = 0;
+  ACC_TRY(ctx->make_current());
+  void *p = nullptr;
+  // a zero-sized array still needs a distinct, valid pointer (Array/Prim.hs:150-157)
+  ACC_HIP_TRY(hipMalloc(&p, bytes ? bytes : 1));
+  *out = reinterpret_cast<acc_devptr>(p);
+  return ACC_OK;
+}
+
+int acc_free(acc_context ctx, acc_devptr p)
+{
+  if (!p) return ACC_OK;
+  if (!ctx) return fail(ACC_ERR_INVALID, "acc_free: NULL context");
+  ACC_TRY(ctx->make_current());
+  ACC_HIP_TRY(hipFree(reinterpret_cast<void *>(p)));
+  return ACC_OK;
+}
+
+int acc_mem_info(acc_context ctx, size_t *free_bytes, size_t *total_bytes)
+{
+  if (!ctx || !free_bytes || !total_bytes) return fail(ACC_ERR_INVALID, "acc_mem_info: NULL argument");
+  ACC_TRY(ctx->make_current());
+  ACC_HIP_TRY(hipMemGetInfo(free_bytes, total_bytes));
+  return ACC_OK;
+}
+
+int acc_host_alloc(acc_context ctx, size_t bytes, void **out)
+{
+  if (!ctx || !out) return fail(ACC_ERR_INVALID, "acc_host_alloc: NULL argument");
+  ACC_TRY(ctx->make_current());
+  ACC_HIP_TRY(hipHostMalloc(out, bytes ? bytes : 1, hipHostMallocDefault));
+  return ACC_OK;
+}
+
+int acc_host_free(acc_context ctx, void *p)
+{
+  if (!p) return ACC_OK;
+  if (!ctx) return fail(ACC_ERR_INVALID, "acc_host_free: NULL context");
+  ACC_TRY(ctx->make_current());
+  ACC_HIP_TRY(hipHostFree(p));
+  return ACC_OK;
+}
+
+static int copy(acc_context ctx, void *dst, const void *src, size_t bytes, hipMemcpyKind kind, hipStream_t s, bool async)
+{
+  if (!ctx) return fail(ACC_ERR_INVALID, "memcpy: NULL context");
+  if (bytes == 0) return ACC_OK;
+  if (!dst || !src) return fail(ACC_ERR_INVALID, "memcpy: NULL pointer");
+  ACC_TRY(ctx->make_current());
+  if (async) {
+    ACC_HIP_TRY(hipMemcpyAsync(dst, src, bytes, kind, s));
+  } else {
+    ACC_HIP_TRY(hipMemcpy(dst, src, bytes, kind));
+  }
+  return ACC_OK;
+}
+
+int acc_memcpy_h2d(acc_context c, acc_devptr d, const void *s, size_t n) { return copy(c, reinterpret_cast<void *>(d), s, n, hipMemcpyHostToDevice, nullptr, false); }
+int acc_memcpy_d2h(acc_context c, void *d, acc_devptr s, size_t n) { return copy(c, d, reinterpret_cast<void *>(s), n, hipMemcpyDeviceToHost, nullptr, false); }
+int acc_memcpy_d2d(acc_context c, acc_devptr d, acc_devptr s, size_t n) { return copy(c, reinterpret_cast<void *>(d), reinterpret_cast<void *>(s), n, hipMemcpyDeviceToDevice, nullptr, false); }
+int acc_memcpy_h2d_async(acc_context c, acc_devptr d, const void *s, size_t n, acc_stream st) { return copy(c, reinterpret_cast<void *>(d), s, n, hipMemcpyHostToDevice, static_cast<hipStream_t>(st), true); }
+int acc_memcpy_d2h_async(acc_context c, void *d, acc_devptr s, size_t n, acc_stream st) { return copy(c, d, reinterpret_cast<void *>(s), n, hipMemcpyDeviceToHost, static_cast<hipStream_t>(st), true); }
+int acc_memcpy_d2d_async(acc_context c, acc_devptr d, acc_devptr s, size_t n, acc_stream st) { return copy(c, reinterpret_cast<void *>(d), reinterpret_cast<void *>(s), n, hipMemcpyDeviceToDevice, static_cast<hipStream_t>(st), true); }
+
+int acc_memset32_async(acc_context ctx, acc_devptr dst, uint32_t value, size_t count, acc_stream s)
+{
+  if (!ctx) return fail(ACC_ERR_INVALID, "acc_memset32_async: NULL context");
+  if (count == 0) return ACC_OK;
+  if (!dst) return fail(ACC_ERR_INVALID, "acc_memset32_async: NULL pointer");
+  ACC_TRY(ctx->make_current());
+  ACC_HIP_TRY(hipMemsetD32Async(reinterpret_cast<hipDeviceptr_t>(dst), static_cast<int>(value), count, static_cast<hipStream_t>(s)));
+  return ACC_OK;
+}
+
+int acc_stream_create(acc_context ctx, acc_stream *out)
+{
+  if (!ctx || !out) return fail(ACC_ERR_INVALID, "acc_stream_create: NULL argument");
+  ACC_TRY(ctx->make_current());
+  hipStream_t s;
+  // default priority on purpose; non-blocking w.r.t. the NULL stream as CUDA.Stream.create [] is not
+  ACC_HIP_TRY(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  *out = s;
+  return ACC_OK;
+}
+
+int acc_stream_destroy(acc_context ctx, acc_stream s)
+{
+  if (!s) return ACC_OK;
+  if (!ctx) return fail(ACC_ERR_INVALID, "acc_stream_destroy: NULL context");
+  ACC_TRY(ctx->make_current());
+  ACC_HIP_TRY(hipStreamDestroy(static_cast<hipStream_t>(s)));
+  return ACC_OK;
+}
+
+int acc_stream_sync(acc_context ctx, acc_stream s)
+{
+  if (!ctx) return fail(ACC_ERR_INVALID, "acc_stream_sync: NULL context");
+  ACC_TRY(ctx->make_current());
+  ACC_HIP_TRY(hipStreamSynchronize(static_cast<hipStream_t>(s)));
+  return ACC_OK;
+}
+
+int acc_stream_wait_event(acc_context ctx, acc_stream s, acc_event e)
+{
+  if (!ctx || !e) return fail(ACC_ERR_INVALID, "acc_stream_wait_event: NULL argument");
+  ACC_TRY(ctx->make_current());
+  ACC_HIP_TRY(hipStreamWaitEvent(static_cast<hipStream_t>(s), static_cast<hipEvent_t>(e), 0));
+  return ACC_OK;
+}
+
+int acc_event_create(acc_context ctx, int enable_timing, acc_event *out)
+{
+  if (!ctx || !out) return fail(ACC_ERR_INVALID, "acc_event_create: NULL argument");
+  ACC_TRY(ctx->make_current());
+  hipEvent_t e;
+  ACC_HIP_TRY(hipEventCreateWithFlags(&e, enable_timing ? hipEventDefault : hipEventDisableTiming));
+  *out = e;
+  return ACC_OK;
+}
+
+int acc_event_destroy(acc_context ctx, acc_event e)
+{
+  if (!e) return ACC_OK;
+  if (!ctx) return fail(ACC_ERR_INVALID, "acc_event_destroy: NULL context");
+  ACC_TRY(ctx->make_current());
+  ACC_HIP_TRY(hipEventDestroy(static_cast<hipEvent_t>(e)));
+  return ACC_OK;
+}
+
+int acc_event_record(acc_context ctx, acc_event e, acc_stream s)
+{
+  if (!ctx || !e) return fail(ACC_ERR_INVALID, "acc_event_record: NULL argument");
+  ACC_TRY(ctx->make_current());
+  ACC_HIP_TRY(hipEventRecord(static_cast<hipEvent_t>(e), static_cast<hipStream_t>(s)));
+  return ACC_OK;
+}
+
+int acc_event_sync(acc_context ctx, acc_event e)
+{
+  if (!ctx || !e) return fail(ACC_ERR_INVALID, "acc_event_sync: NULL argument");
+  ACC_TRY(ctx->make_current());
+  ACC_HIP_TRY(hipEventSynchronize(static_cast<hipEvent_t>(e)));
+  return ACC_OK;
+}
+
+int acc_event_query(acc_context ctx, acc_event e, int *done)
+{
+  if (!ctx || !e || !done) return fail(ACC_ERR_INVALID, "acc_event_query: NULL argument");
+  ACC_TRY(ctx->make_current());
+  hipError_t r = hipEventQuery(static_cast<hipEvent_t>(e));
+  if (r == hipSuccess) { *done = 1; return ACC_OK; }
+  if (r == hipErrorNotReady) { *done = 0; (void)hipGetLastError(); return ACC_OK; }
+  return acc::fail_hip(r, "hipEventQuery");
+}
+
+int acc_event_elapsed_ms(acc_context ctx, acc_event start, acc_event stop, float *ms)
+{
+  if (!ctx || !start || !stop || !ms) return fail(ACC_ERR_INVALID, "acc_event_elapsed_ms: NULL argument");
+  ACC_TRY(ctx->make_current());
+  ACC_HIP_TRY(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+  return ACC_OK;
+}
+
+int acc_module_load(acc_context ctx, const void *code, size_t code_size, acc_module *out)
+{
+  if (!ctx || !code || !code_size || !out) return fail(ACC_ERR_INVALID, "acc_module_load: NULL argument");
+  ACC_TRY(ctx->make_current());
+  hipModule_t m;
+  ACC_HIP_TRY(hipModuleLoadData(&m, code));
+  *out = m;
+  return ACC_OK;
+}
+
+int acc_module_unload(acc_context ctx, acc_module m)
+{
+  if (!m) return ACC_OK;
+  if (!ctx) return fail(ACC_ERR_INVALID, "acc_module_unload: NULL context");
+  ACC_TRY(ctx->make_current());
+  ACC_HIP_TRY(hipModuleUnload(static_cast<hipModule_t>(m)));
+  return ACC_OK;
+}
+
+int acc_module_get_function(acc_context ctx, acc_module m, const char *entry, acc_function *out)
+{
+  if (!ctx || !m || !entry || !out) return fail(ACC_ERR_INVALID, "acc_module_get_function: NULL argument");
+  ACC_TRY(ctx->make_current());
+  hipFunction_t f;
+  hipError_t e = hipModuleGetFunction(&f, static_cast<hipModule_t>(m), entry);
+  if (e == hipErrorNotFound) { (void)hipGetLastError(); return fail(ACC_ERR_NOT_FOUND, "no kernel entry '%s' in module", entry); }
+  if (e != hipSuccess) return acc::fail_hip(e, "hipModuleGetFunction");
+  *out = f;
+  return ACC_OK;
+}
+
+int acc_function_attr(acc_context ctx, acc_function f, int which, int *value)
+{
+  if (!ctx || !f || !value) return fail(ACC_ERR_INVALID, "acc_function_attr: NULL argument");
+  hipFunction_attribute a;
+  switch (which) {
+    case ACC_FUNC_NUM_REGS: a = HIP_FUNC_ATTRIBUTE_NUM_REGS; break;
+    case ACC_FUNC_SHARED_SIZE_BYTES: a = HIP_FUNC_ATTRIBUTE_SHARED_SIZE_BYTES; break;
+    case ACC_FUNC_CONST_SIZE_BYTES: a = HIP_FUNC_ATTRIBUTE_CONST_SIZE_BYTES; break;
+    case ACC_FUNC_LOCAL_SIZE_BYTES: a = HIP_FUNC_ATTRIBUTE_LOCAL_SIZE_BYTES; break;
+    case ACC_FUNC_MAX_THREADS: a = HIP_FUNC_ATTRIBUTE_MAX_THREADS_PER_BLOCK; break;
+    default: return fail(ACC_ERR_INVALID, "acc_function_attr: unknown attribute %d", which);
+  }
+  ACC_TRY(ctx->make_current());
+  ACC_HIP_TRY(hipFuncGetAttribute(value, a, static_cast<hipFunction_t>(f)));
+  return ACC_OK;
+}
+
+int acc_occupancy(acc_context ctx, acc_function f, int block, size_t dyn_lds, int *blocks_per_cu)
+{
+  if (!ctx || !f || !blocks_per_cu || block <= 0) return fail(ACC_ERR_INVALID, "acc_occupancy: bad argument");
+  ACC_TRY(ctx->make_current());
+  ACC_HIP_TRY(hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(blocks_per_cu, static_cast<hipFunction_t>(f), block, dyn_lds));
+  return ACC_OK;
+}
+
+int acc_launch(acc_context ctx, acc_function f, uint32_t grid, uint32_t block, uint32_t dyn_lds, acc_stream s, void **args)
+{
+  if (!ctx || !f) return fail(ACC_ERR_INVALID, "acc_launch: NULL argument");
+  if (grid == 0 || block == 0 || block > static_cast<uint32_t>(ctx->props.maxThreadsPerBlock))
+    return fail(ACC_ERR_INVALID, "acc_launch: bad launch shape grid=%u block=%u", grid, block);
+  ACC_TRY(ctx->make_current());
+  ACC_HIP_TRY(hipModuleLaunchKernel(static_cast<hipFunction_t>(f), grid, 1, 1, block, 1, 1, dyn_lds,
+                                    static_cast<hipStream_t>(s), args, nullptr));
+  return ACC_OK;
+}
+
+int64_t acc_launch_grid(int64_t n, int64_t per_block, int64_t cus, int64_t blocks_per_cu)
+{
+  if (per_block < 1) per_block = 1;
+  int64_t need = (n + per_block - 1) / per_block;
+  if (need < 1) need = 1;
+  int64_t cap = cus * blocks_per_cu;
+  if (cap < 1) cap = 1;
+  return need < cap ? need : cap;
+}
+
+}  // extern "C"

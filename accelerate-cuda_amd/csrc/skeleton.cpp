@@ -1,0 +1,454 @@
+// Skeleton instantiation: scalar fragments + a hand-written gfx950 template
+// -> one translation unit -> (cache | hiprtc) -> loaded module -> kernel record.
+//
+// This is the job CUDA/CodeGen.hs:91-136 (dispatch on the array operation),
+// CUDA/CodeGen/Base.hs:69-89,262-383 (naming and ordering of kernel parameters)
+// and CUDA/Compile.hs:444-459,484-566 (build1 / compile / link) do in the
+// reference.  The templates themselves live in device/*.h.
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+#include <sstream>
+
+#include "skeleton.hpp"
+
+namespace acc {
+
+// ---- element types --------------------------------------------------------
+
+int type_size(const std::string &t)
+{
+  static const struct { const char *name; int size; } table[] = {
+      {"float", 4},   {"double", 8},  {"Int8", 1},     {"Int16", 2},    {"Int32", 4},   {"Int64", 8},
+      {"Word8", 1},   {"Word16", 2},  {"Word32", 4},   {"Word64", 8},   {"int8_t", 1},  {"int16_t", 2},
+      {"int32_t", 4}, {"int64_t", 8}, {"uint8_t", 1},  {"uint16_t", 2}, {"uint32_t", 4}, {"uint64_t", 8},
+      {"char", 1},    {"short", 2},   {"int", 4},      {"unsigned", 4}, {"unsigned int", 4},
+      {"long long", 8}, {"unsigned long long", 8}};
+  for (const auto &e : table)
+    if (t == e.name) return e.size;
+  return 0;
+}
+
+static bool is_integer_type(const std::string &t)
+{
+  return type_size(t) != 0 && t != "float" && t != "double";
+}
+
+// one-line form of a fragment so that it can sit in a #define
+static std::string flat(const char *s)
+{
+  std::string r = s ? s : "";
+  for (char &c : r)
+    if (c == '\n' || c == '\r') c = ' ';
+  return r;
+}
+
+// ---- tuning knobs -----------------------------------------------------------
+// ACC_HIP_TUNE="scan.block=512,scan.rows=2,fold.unroll=8" overrides a default,
+// for measurement sweeps; the value becomes part of the source and so of the
+// cache key.
+int tune(const char *name, int dflt)
+{
+  const char *e = std::getenv("ACC_HIP_TUNE");
+  if (!e) return dflt;
+  const std::string all = e, key = std::string(name) + "=";
+  size_t pos = 0;
+  while (pos < all.size()) {
+    size_t end = all.find(',', pos);
+    if (end == std::string::npos) end = all.size();
+    if (all.compare(pos, key.size(), key) == 0) return std::atoi(all.c_str() + pos + key.size());
+    pos = end + 1;
+  }
+  return dflt;
+}
+
+// ---- parameter groups (CodeGen/Base.hs:69-89,348-383) ----------------------
+
+static std::string env_params(const std::vector<EnvSig> &env)
+{
+  std::ostringstream o;
+  for (size_t k = 0; k < env.size(); ++k) {
+    for (int d = env[k].rank - 1; d >= 0; --d) o << "const Int64 shIn" << k << "_" << d << ", ";
+    for (int c = env[k].ncomp - 1; c >= 0; --c)
+      o << "const " << env[k].type[c] << " *__restrict__ arrIn" << k << "_" << c << ", ";
+  }
+  return o.str();
+}
+
+static std::string env_assume(const std::vector<EnvSig> &env, bool aligned)
+{
+  std::ostringstream o;
+  for (size_t k = 0; k < env.size(); ++k) {
+    for (int d = env[k].rank - 1; d >= 0; --d) o << "(void)shIn" << k << "_" << d << "; ";
+    for (int c = env[k].ncomp - 1; c >= 0; --c) {
+      if (aligned)
+        o << "arrIn" << k << "_" << c << " = (const " << env[k].type[c] << " *)__builtin_assume_aligned(arrIn" << k
+          << "_" << c << ", 16); ";
+      else
+        o << "(void)arrIn" << k << "_" << c << "; ";
+    }
+  }
+  return o.str();
+}
+
+static std::string out_params(int rank, const std::string &elt)
+{
+  std::ostringstream o;
+  for (int d = rank - 1; d >= 0; --d) o << "const Int64 shOut_" << d << ", ";
+  o << elt << " *__restrict__ arrOut_0";
+  return o.str();
+}
+
+static std::string out_size(int rank)
+{
+  if (rank == 0) return "1";
+  std::ostringstream o;
+  o << "(";
+  for (int d = rank - 1; d >= 0; --d) o << "shOut_" << d << (d ? " * " : "");
+  o << ")";
+  return o.str();
+}
+
+static const char *kind_name(int kind)
+{
+  static const char *names[] = {"map", "generate", "transform", "fold", "fold1", "foldSeg", "fold1Seg", "scanl",
+                                "scanl1", "scanl'", "scanr", "scanr1", "scanr'", "permute", "stencil"};
+  return (kind >= 0 && kind < ACC_SKEL_KIND_COUNT) ? names[kind] : "?";
+}
+
+// ---- the generator -------------------------------------------------------------
+
+int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::string *source)
+{
+  std::ostringstream o;
+  const int esz = sp.elt_size;
+  int vec = std::max(1, 16 / std::max(1, esz));
+  o << "// accelerate-hip " ACC_HIP_VERSION " skeleton instance: " << kind_name(sp.kind) << "\n";
+  o << "#define ACC_ELT " << sp.elt_type << "\n";
+  o << "#define ACC_ALIGNED " << (aligned ? 1 : 0) << "\n";
+  o << "#define ACC_ENV_PARAMS " << env_params(sp.env) << "\n";
+  o << "#define ACC_ENV_ASSUME " << env_assume(sp.env, aligned) << "\n";
+  if (!sp.get.empty()) o << "#define ACC_GET(ix) " << sp.get << "\n";
+  if (!sp.combine.empty()) o << "#define ACC_COMBINE(x, y) " << sp.combine << "\n";
+  o << "#define ACC_HAS_SEED " << (sp.has_seed ? 1 : 0) << "\n";
+  if (sp.has_seed) o << "#define ACC_SEED " << sp.seed << "\n";
+
+  const char *tmpl = nullptr;
+  switch (sp.kind) {
+    case ACC_SKEL_MAP:
+    case ACC_SKEL_GENERATE:
+    case ACC_SKEL_TRANSFORM:
+      *entry = kind_name(sp.kind);
+      o << "#define ACC_OUT_PARAMS " << out_params(sp.out_rank, sp.elt_type) << "\n";
+      o << "#define ACC_OUT_SIZE " << out_size(sp.out_rank) << "\n";
+      o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_UNROLL " << sp.unroll << "\n";
+      tmpl = "skel_map.h";
+      break;
+    case ACC_SKEL_FOLD:
+    case ACC_SKEL_FOLD1:
+      if (sp.out_rank == 0) *entry = sp.has_seed ? "foldAll" : "fold1All";
+      else *entry = sp.has_seed ? "fold" : "fold1";
+      o << "#define ACC_FOLD_DIM " << (sp.out_rank == 0 ? 0 : 1) << "\n";
+      o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_UNROLL " << sp.unroll << "\n";
+      tmpl = "skel_fold.h";
+      break;
+    case ACC_SKEL_FOLDSEG:
+    case ACC_SKEL_FOLD1SEG:
+      *entry = sp.has_seed ? "foldSeg" : "fold1Seg";
+      o << "#define ACC_SEG_TYPE " << sp.seg_type << "\n";
+      o << "#define ACC_FOLD_RIGHT " << ((sp.flags & ACC_FLAG_FOLD_RIGHT) ? 1 : 0) << "\n";
+      o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_CHUNK " << sp.chunk << "\n";
+      tmpl = "skel_foldseg.h";
+      break;
+    case ACC_SKEL_SCANL: case ACC_SKEL_SCANL1: case ACC_SKEL_SCANLP:
+    case ACC_SKEL_SCANR: case ACC_SKEL_SCANR1: case ACC_SKEL_SCANRP: {
+      const bool right = sp.kind >= ACC_SKEL_SCANR;
+      int mode = 1;
+      if (sp.kind == ACC_SKEL_SCANL) mode = 0;
+      if (sp.kind == ACC_SKEL_SCANLP || sp.kind == ACC_SKEL_SCANRP) mode = 2;
+      if (sp.kind == ACC_SKEL_SCANR) mode = 3;
+      // entry names as the reference builds them: "scan" ++ dir ++ ("1" if seedless), PrefixSum.hs:311
+      *entry = std::string("scan") + (right ? "r" : "l") + (sp.has_seed ? "" : "1");
+      o << "#define ACC_SCAN_RIGHT " << (right ? 1 : 0) << "\n#define ACC_SCAN_MODE " << mode << "\n";
+      o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_ROWS " << sp.rows << "\n";
+      tmpl = "skel_scan.h";
+      break;
+    }
+    case ACC_SKEL_PERMUTE:
+      *entry = "permute";
+      o << "#define ACC_OUT_PARAMS " << out_params(sp.out_rank, sp.elt_type) << "\n";
+      o << "#define ACC_OUT_SIZE " << out_size(sp.out_rank) << "\n";
+      o << "#define ACC_PERMUTATION(ix) " << sp.permutation << "\n";
+      o << "#define ACC_COMBINE_HINT " << sp.combine_hint << "\n";
+      o << "#define ACC_ELT_IS_INTEGER " << (is_integer_type(sp.elt_type) ? 1 : 0) << "\n";
+      o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_UNROLL " << sp.unroll << "\n";
+      tmpl = "skel_permute.h";
+      break;
+    case ACC_SKEL_STENCIL: {
+      *entry = "stencil";
+      int ry = 0, rx = 0;
+      for (size_t k = 0; k < sp.tap_dy.size(); ++k) {
+        ry = std::max(ry, std::abs(sp.tap_dy[k]));
+        rx = std::max(rx, std::abs(sp.tap_dx[k]));
+      }
+      o << "#define ACC_OUT_PARAMS " << out_params(sp.out_rank, sp.elt_type) << "\n";
+      o << "#define ACC_STENCIL_RANK " << sp.out_rank << "\n";
+      o << "#define ACC_IN_ELT " << sp.stencil_in_type << "\n";
+      o << "#define ACC_RADIUS_Y " << ry << "\n#define ACC_RADIUS_X " << rx << "\n";
+      o << "#define ACC_BOUNDARY " << sp.boundary << "\n";
+      o << "#define ACC_BOUNDARY_CONSTANT " << (sp.boundary_constant.empty() ? "0" : sp.boundary_constant) << "\n";
+      // the stencil pattern: one binding per tap, read through whatever accessor the template passes
+      o << "#define ACC_STENCIL_TAPS(READ) ";
+      for (size_t k = 0; k < sp.tap_dy.size(); ++k)
+        o << "const ACC_IN_ELT t" << k << " = READ(" << sp.tap_dy[k] << ", " << sp.tap_dx[k] << "); ";
+      o << "\n";
+      o << "#define ACC_STENCIL_FN " << sp.stencil_fn << "\n";
+      o << "#define ACC_TILE_W " << sp.tile_w << "\n#define ACC_TILE_H " << sp.tile_h << "\n#define ACC_BLOCK " << sp.block << "\n";
+      tmpl = "skel_stencil.h";
+      break;
+    }
+    default:
+      return fail(ACC_ERR_INVALID, "unknown skeleton kind %d", sp.kind);
+  }
+  o << "#define ACC_ENTRY " << *entry << "\n";
+  o << "#include \"acc_hip_device.h\"\n";
+  if (!sp.preamble.empty()) o << sp.preamble << "\n";
+  o << "#include \"" << tmpl << "\"\n";
+  *source = o.str();
+  return ACC_OK;
+}
+
+// ---- description -> spec ---------------------------------------------------------
+
+int make_spec(const acc_skel_desc *d, SkelSpec *sp)
+{
+  if (!d) return fail(ACC_ERR_INVALID, "NULL skeleton description");
+  if (d->kind < 0 || d->kind >= ACC_SKEL_KIND_COUNT) return fail(ACC_ERR_INVALID, "unknown skeleton kind %d", d->kind);
+  if (!d->elt_type || !*d->elt_type) return fail(ACC_ERR_INVALID, "skeleton description: elt_type missing");
+  if (d->n_env < 0 || (d->n_env > 0 && !d->env)) return fail(ACC_ERR_INVALID, "skeleton description: bad env");
+  sp->kind = d->kind;
+  sp->flags = d->flags;
+  sp->elt_type = d->elt_type;
+  sp->elt_size = d->elt_size > 0 ? d->elt_size : type_size(sp->elt_type);
+  if (sp->elt_size <= 0) return fail(ACC_ERR_INVALID, "cannot size element type '%s': set elt_size", d->elt_type);
+  sp->out_rank = d->out_rank;
+  if (sp->out_rank < 0 || sp->out_rank > ACC_MAX_RANK) return fail(ACC_ERR_INVALID, "bad out_rank %d", d->out_rank);
+  for (int k = 0; k < d->n_env; ++k) {
+    const acc_env_sig &e = d->env[k];
+    if (e.rank < 0 || e.rank > ACC_MAX_RANK || e.ncomp < 1 || e.ncomp > ACC_MAX_COMP)
+      return fail(ACC_ERR_INVALID, "env array %d: bad rank/ncomp", k);
+    EnvSig s;
+    s.rank = e.rank;
+    s.ncomp = e.ncomp;
+    for (int c = 0; c < e.ncomp; ++c) {
+      if (!e.type[c] || !*e.type[c]) return fail(ACC_ERR_INVALID, "env array %d: component %d has no type", k, c);
+      s.type.push_back(e.type[c]);
+    }
+    sp->env.push_back(s);
+  }
+  sp->preamble = d->preamble ? d->preamble : "";
+  sp->get = flat(d->get);
+  sp->combine = flat(d->combine);
+  sp->has_seed = d->seed && *d->seed;
+  sp->seed = flat(d->seed);
+  sp->permutation = flat(d->permutation);
+  sp->combine_hint = d->combine_hint;
+  sp->seg_type = (d->seg_type && *d->seg_type) ? d->seg_type : "Int32";
+
+  const bool needs_get = d->kind != ACC_SKEL_STENCIL;
+  if (needs_get && sp->get.empty()) return fail(ACC_ERR_INVALID, "%s: `get` fragment missing", kind_name(d->kind));
+  const bool needs_combine = d->kind >= ACC_SKEL_FOLD && d->kind <= ACC_SKEL_PERMUTE;
+  if (needs_combine && sp->combine.empty()) return fail(ACC_ERR_INVALID, "%s: `combine` fragment missing", kind_name(d->kind));
+
+  switch (d->kind) {
+    case ACC_SKEL_FOLD: case ACC_SKEL_FOLDSEG: case ACC_SKEL_SCANL: case ACC_SKEL_SCANLP:
+    case ACC_SKEL_SCANR: case ACC_SKEL_SCANRP:
+      if (!sp->has_seed) return fail(ACC_ERR_INVALID, "%s: `seed` fragment missing", kind_name(d->kind));
+      break;
+    case ACC_SKEL_FOLD1: case ACC_SKEL_FOLD1SEG: case ACC_SKEL_SCANL1: case ACC_SKEL_SCANR1:
+      if (sp->has_seed) return fail(ACC_ERR_INVALID, "%s takes no seed", kind_name(d->kind));
+      break;
+    default:
+      break;
+  }
+
+  sp->block = 256;
+  sp->unroll = 4;
+  sp->rows = 4;
+  sp->chunk = 4096;
+  switch (d->kind) {
+    case ACC_SKEL_MAP: case ACC_SKEL_GENERATE: case ACC_SKEL_TRANSFORM:
+      sp->block = tune("map.block", 256);
+      sp->unroll = tune("map.unroll", 4);
+      break;
+    case ACC_SKEL_FOLD: case ACC_SKEL_FOLD1:
+      sp->block = tune("fold.block", 256);
+      sp->unroll = tune("fold.unroll", 4);
+      break;
+    case ACC_SKEL_FOLDSEG: case ACC_SKEL_FOLD1SEG:
+      sp->block = tune("foldseg.block", 256);
+      sp->chunk = tune("foldseg.chunk", 4096);
+      break;
+    case ACC_SKEL_PERMUTE:
+      if (sp->permutation.empty()) return fail(ACC_ERR_INVALID, "permute: `permutation` fragment missing");
+      if (sp->out_rank < 1) return fail(ACC_ERR_UNSUPPORTED, "permute into a rank-0 array is not supported");   // IndexSpace.hs:230
+      if (sp->elt_size != 4 && sp->elt_size != 8)
+        return fail(ACC_ERR_UNSUPPORTED, "permute: element size %d has no atomic update", sp->elt_size);
+      if (sp->combine_hint < ACC_COMBINE_GENERIC || sp->combine_hint > ACC_COMBINE_XOR)
+        return fail(ACC_ERR_INVALID, "permute: bad combine_hint %d", sp->combine_hint);
+      if (sp->combine_hint >= ACC_COMBINE_AND && !is_integer_type(sp->elt_type))
+        return fail(ACC_ERR_INVALID, "permute: bitwise combine_hint on non-integer element type '%s'", sp->elt_type.c_str());
+      sp->block = tune("permute.block", 512);
+      sp->unroll = tune("permute.unroll", 4);
+      break;
+    case ACC_SKEL_STENCIL: {
+      if (sp->out_rank != 1 && sp->out_rank != 2) return fail(ACC_ERR_UNSUPPORTED, "stencil: rank %d not supported (1 and 2 are)", sp->out_rank);
+      if (d->n_taps < 1 || d->n_taps > 81 || !d->tap_dx) return fail(ACC_ERR_INVALID, "stencil: bad tap list");
+      if (!d->stencil_fn || !*d->stencil_fn) return fail(ACC_ERR_INVALID, "stencil: `stencil_fn` fragment missing");
+      if (d->boundary < ACC_BOUNDARY_CLAMP || d->boundary > ACC_BOUNDARY_CONSTANT) return fail(ACC_ERR_INVALID, "stencil: bad boundary %d", d->boundary);
+      for (int k = 0; k < d->n_taps; ++k) {
+        const int dy = (sp->out_rank == 2 && d->tap_dy) ? d->tap_dy[k] : 0;
+        if (std::abs(dy) > 4 || std::abs(d->tap_dx[k]) > 4) return fail(ACC_ERR_UNSUPPORTED, "stencil: tap offset beyond 4");
+        sp->tap_dy.push_back(dy);
+        sp->tap_dx.push_back(d->tap_dx[k]);
+      }
+      sp->boundary = d->boundary;
+      sp->boundary_constant = flat(d->boundary_constant);
+      sp->stencil_fn = flat(d->stencil_fn);
+      sp->stencil_in_type = (d->stencil_in_type && *d->stencil_in_type) ? d->stencil_in_type : sp->elt_type;
+      sp->block = tune("stencil.block", 256);
+      sp->tile_w = tune("stencil.tile_w", 256);
+      sp->tile_h = tune("stencil.tile_h", sp->out_rank == 2 ? 16 : 1);
+      if (sp->out_rank == 1) { sp->tile_h = 1; sp->tile_w = sp->block * 4; }
+      break;
+    }
+    default:   // scans
+      sp->block = tune("scan.block", 256);
+      sp->rows = tune("scan.rows", 4);
+      break;
+  }
+  if (sp->block < 64 || sp->block > 1024 || (sp->block & 63)) return fail(ACC_ERR_INVALID, "block size %d is not a multiple of the 64-lane wavefront", sp->block);
+  return ACC_OK;
+}
+
+std::vector<std::string> compile_options(const SkelSpec &sp)
+{
+  std::vector<std::string> o = {"-O3", "-std=c++17"};
+  // scalar operations round one at a time, as the interpreter evaluates them,
+  // unless the caller asks otherwise
+  o.push_back((sp.flags & ACC_FLAG_FAST_MATH) ? "-ffp-contract=fast" : "-ffp-contract=off");
+  // no packed two-lane Float32 instructions: scalar code stays scalar
+  for (const char *f : {"-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"}) o.push_back(f);
+  return o;
+}
+
+}  // namespace acc
+
+using acc::fail;
+
+// ---- acc_skel_s ----------------------------------------------------------------
+
+int acc_skel_s::ensure_variant(int v)
+{
+  acc::Variant &var = variants[v];
+  if (var.ready) return ACC_OK;
+  std::string entry_name;
+  ACC_TRY(acc::generate_source(spec, v == 0, &entry_name, &var.source));
+  entry = entry_name;
+  std::vector<std::string> opts = acc::compile_options(spec);
+  std::vector<const char *> optp;
+  for (const std::string &s : opts) optp.push_back(s.c_str());
+  const void *code = nullptr;
+  size_t size = 0;
+  ACC_TRY(acc_compile(ctx, nullptr, var.source.c_str(), optp.data(), static_cast<int>(optp.size()), &code, &size));
+  ACC_TRY(ctx->make_current());
+  ACC_HIP_TRY(hipModuleLoadData(&var.module, code));
+  hipError_t e = hipModuleGetFunction(&var.fn, var.module, entry.c_str());
+  if (e != hipSuccess) {
+    (void)hipModuleUnload(var.module);
+    var.module = nullptr;
+    return acc::fail_hip(e, ("hipModuleGetFunction(" + entry + ")").c_str());
+  }
+  (void)hipFuncGetAttribute(&var.num_regs, HIP_FUNC_ATTRIBUTE_NUM_REGS, var.fn);
+  (void)hipFuncGetAttribute(&var.static_lds, HIP_FUNC_ATTRIBUTE_SHARED_SIZE_BYTES, var.fn);
+  int bpc = 0;
+  e = hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&bpc, var.fn, spec.block, 0);
+  if (e != hipSuccess || bpc < 1) { (void)hipGetLastError(); bpc = 1; }
+  var.blocks_per_cu = bpc;
+  var.ready = true;
+  return ACC_OK;
+}
+
+extern "C" {
+
+int acc_skel_create(acc_context ctx, const acc_skel_desc *desc, acc_skel *out)
+{
+  if (!ctx || !out) return fail(ACC_ERR_INVALID, "acc_skel_create: NULL argument");
+  *out = nullptr;
+  acc::SkelSpec sp;
+  ACC_TRY(acc::make_spec(desc, &sp));
+  acc_skel_s *s = new acc_skel_s();
+  s->ctx = ctx;
+  s->spec = sp;
+  int rc = s->ensure_variant(0);      // the unaligned variant is built on first need
+  if (rc != ACC_OK) { delete s; return rc; }
+  *out = s;
+  return ACC_OK;
+}
+
+int acc_skel_destroy(acc_skel s)
+{
+  if (!s) return ACC_OK;
+  (void)s->ctx->make_current();
+  for (acc::Variant &v : s->variants)
+    if (v.module) (void)hipModuleUnload(v.module);
+  delete s;
+  return ACC_OK;
+}
+
+int acc_skel_source(acc_skel s, int variant, const char **source)
+{
+  if (!s || !source || variant < 0 || variant > 1) return fail(ACC_ERR_INVALID, "acc_skel_source: bad argument");
+  if (s->variants[variant].source.empty()) {
+    std::string e;
+    ACC_TRY(acc::generate_source(s->spec, variant == 0, &e, &s->variants[variant].source));
+  }
+  *source = s->variants[variant].source.c_str();
+  return ACC_OK;
+}
+
+int acc_skel_compile_only(const char *target, const acc_skel_desc *desc, size_t *code_size)
+{
+  if (!target) return fail(ACC_ERR_INVALID, "acc_skel_compile_only: NULL target");
+  acc::SkelSpec sp;
+  ACC_TRY(acc::make_spec(desc, &sp));
+  std::vector<std::string> opts = acc::compile_options(sp);
+  std::vector<const char *> optp;
+  for (const std::string &o : opts) optp.push_back(o.c_str());
+  size_t total = 0;
+  for (int v = 0; v < 2; ++v) {
+    std::string entry, src;
+    ACC_TRY(acc::generate_source(sp, v == 0, &entry, &src));
+    const void *code = nullptr;
+    size_t size = 0;
+    ACC_TRY(acc_compile(nullptr, target, src.c_str(), optp.data(), static_cast<int>(optp.size()), &code, &size));
+    total += size;
+  }
+  if (code_size) *code_size = total;
+  return ACC_OK;
+}
+
+int acc_skel_get_info(acc_skel s, acc_skel_info *out)
+{
+  if (!s || !out) return fail(ACC_ERR_INVALID, "acc_skel_get_info: NULL argument");
+  std::memset(out, 0, sizeof(*out));
+  std::snprintf(out->entry, sizeof(out->entry), "%s", s->entry.c_str());
+  out->block = s->spec.block;
+  out->blocks_per_cu = s->variants[0].blocks_per_cu;
+  out->num_regs = s->variants[0].num_regs;
+  out->static_lds = s->variants[0].static_lds;
+  out->elements_per_block = s->elements_per_block();
+  return ACC_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,76 @@
+// Skeleton instances: what acc_skel_create builds and acc_exec_* run.
+#pragma once
+#include "acc_internal.hpp"
+
+namespace acc {
+
+struct EnvSig {
+  int rank = 0;
+  int ncomp = 1;
+  std::vector<std::string> type;
+};
+
+// the validated, owned form of an acc_skel_desc plus the tuning of its template
+struct SkelSpec {
+  int kind = 0;
+  uint32_t flags = 0;
+  std::vector<EnvSig> env;
+  std::string elt_type;
+  int elt_size = 0;
+  int out_rank = 0;
+  std::string preamble, get, combine, seed, permutation;
+  bool has_seed = false;
+  int combine_hint = 0;
+  std::string seg_type;
+  // stencil
+  int boundary = 0;
+  std::string boundary_constant, stencil_fn, stencil_in_type;
+  std::vector<int> tap_dy, tap_dx;
+  int tile_w = 256, tile_h = 16;
+  // tuning
+  int block = 256, unroll = 4, rows = 4, chunk = 4096;
+};
+
+// one compiled form of an instance: AccKernel of the reference (AST.hs:51-59)
+struct Variant {
+  bool ready = false;
+  std::string source;
+  hipModule_t module = nullptr;
+  hipFunction_t fn = nullptr;
+  int num_regs = 0;
+  int static_lds = 0;
+  int blocks_per_cu = 1;
+};
+
+int type_size(const std::string &t);
+int tune(const char *name, int dflt);
+int make_spec(const acc_skel_desc *d, SkelSpec *sp);
+int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::string *source);
+std::vector<std::string> compile_options(const SkelSpec &sp);
+
+}  // namespace acc
+
+struct acc_skel_s {
+  acc_context ctx = nullptr;
+  acc::SkelSpec spec;
+  std::string entry;
+  acc::Variant variants[2];   // [0] pointers 16-byte aligned, [1] no assumption
+  std::mutex mu;
+
+  int ensure_variant(int v);
+  int vec() const { int v = 16 / (spec.elt_size > 0 ? spec.elt_size : 1); return v < 1 ? 1 : v; }
+  int elements_per_block() const
+  {
+    switch (spec.kind) {
+      case ACC_SKEL_SCANL: case ACC_SKEL_SCANL1: case ACC_SKEL_SCANLP:
+      case ACC_SKEL_SCANR: case ACC_SKEL_SCANR1: case ACC_SKEL_SCANRP:
+        return spec.block * spec.rows * vec();
+      case ACC_SKEL_STENCIL:
+        return spec.tile_w * spec.tile_h;
+      case ACC_SKEL_FOLDSEG: case ACC_SKEL_FOLD1SEG:
+        return spec.block;   // segments per block
+      default:
+        return spec.block * spec.unroll * vec();
+    }
+  }
+};

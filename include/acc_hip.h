@@ -1,0 +1,358 @@
+/*
+ * acc_hip.h -- C ABI of libacchip, the MI355X (gfx950) runtime under an
+ * Accelerate backend.  It is what a `Data.Array.Accelerate.HIP` module binds
+ * with `foreign import ccall` in place of everything accelerate-cuda reaches
+ * through the `cuda` package (Foreign.CUDA.Driver / Foreign.CUDA.Analysis) and
+ * the external `nvcc`.
+ *
+ * Two layers:
+ *
+ *   A. driver layer   -- devices, memory, transfers, streams, events, modules,
+ *                        run-time compilation with a content-hashed code-object
+ *                        cache, occupancy, raw launches;
+ *   B. skeleton layer -- instantiate one of the hand-written gfx950 skeleton
+ *                        templates with the scalar fragments the code generator
+ *                        produced (acc_skel_create), and run it with the
+ *                        temporaries, launch shapes and multi-kernel protocols
+ *                        it needs (acc_exec_*).  These are the roles of
+ *                        the CUDA/CodeGen modules (templates) and of the skeleton
+ *                        drivers in CUDA/Execute.hs:264-450.
+ *
+ * Conventions
+ *   - plain C: pointers, sizes, fixed-width integers; no C++ or torch types;
+ *   - every function returns an int status (ACC_OK == 0); the message of the
+ *     last failure on the calling thread is acc_last_error(); nothing aborts.
+ *     (The reference throws CUDAException, State.hs:86-88; out-of-memory is its
+ *     one recoverable error, Array/Remote.hs:63-67 -> ACC_ERR_OOM here);
+ *   - device pointers are uint64_t (Haskell does pointer arithmetic itself, as
+ *     with advanceDevPtr / plusDevPtr);
+ *   - acc_stream / acc_event / acc_module / acc_function are the HIP handles
+ *     themselves (hipStream_t, ...); a NULL stream is the default stream;
+ *   - the caller owns every handle it creates; the library owns the kernel
+ *     cache and per-context scratch memory; destroy/free of NULL is a no-op;
+ *   - thread safety: every entry point may be called from any thread; the
+ *     device of the context is made current on entry.  One acc_skel may be
+ *     executed from several threads, calls on the SAME stream are ordered.
+ */
+#ifndef ACC_HIP_H
+#define ACC_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+#if defined(__GNUC__)
+#pragma GCC visibility push(default)
+#endif
+
+/* ---- status codes -------------------------------------------------------- */
+#define ACC_OK               0
+#define ACC_ERR_INVALID      1   /* bad argument, shape mismatch, fold1 of empty array */
+#define ACC_ERR_OOM          2   /* device allocation failed: caller may evict and retry */
+#define ACC_ERR_COMPILE      3   /* run-time compilation failed: see acc_compile_log */
+#define ACC_ERR_NOT_FOUND    4   /* no such kernel entry / device */
+#define ACC_ERR_HIP          5   /* any other HIP runtime error */
+#define ACC_ERR_UNSUPPORTED  6   /* valid Accelerate, not implemented by this backend */
+#define ACC_ERR_IO           7   /* kernel cache file trouble (never fatal to a compile) */
+
+typedef struct acc_context_s *acc_context;
+typedef struct acc_skel_s    *acc_skel;
+typedef void *acc_stream;     /* hipStream_t   */
+typedef void *acc_event;      /* hipEvent_t    */
+typedef void *acc_module;     /* hipModule_t   */
+typedef void *acc_function;   /* hipFunction_t */
+typedef uint64_t acc_devptr;
+
+const char *acc_last_error(void);
+const char *acc_version(void);
+
+/* =========================================================================
+ * A. driver layer
+ * ========================================================================= */
+
+/* CUDA.initialise / count / props: State.hs:127-132, Analysis/Device.hs:31-41 */
+int acc_init(void);
+int acc_device_count(int *count);
+
+typedef struct acc_device_props {
+  char     name[256];
+  char     arch[64];               /* gcnArchName, e.g. "gfx950:sramecc+:xnack-" */
+  int32_t  compute_units;
+  int32_t  wavefront_size;
+  int32_t  max_threads_per_block;
+  int32_t  clock_khz;
+  int64_t  lds_per_block;          /* bytes a single workgroup may use */
+  int64_t  lds_per_cu;
+  int64_t  l2_bytes;
+  int64_t  total_mem;
+  int32_t  regs_per_block;
+  int32_t  max_threads_per_cu;
+} acc_device_props;
+int acc_device_get_props(int device, acc_device_props *out);
+
+/* Context.hs:55-71 (create), :99-111 (destroy).  HIP has one primary context
+ * per device, so there is no push/pop (State.hs:84-92) and no cache config.  */
+int acc_context_create(int device, acc_context *out);
+int acc_context_destroy(acc_context ctx);
+int acc_context_device(acc_context ctx, int *device);
+int acc_context_sync(acc_context ctx);                 /* CUDA.sync */
+
+/* CUDA.mallocArray / free / getMemInfo: Array/Remote.hs:63-79,191 */
+int acc_malloc(acc_context ctx, size_t bytes, acc_devptr *out);
+int acc_free(acc_context ctx, acc_devptr p);
+int acc_mem_info(acc_context ctx, size_t *free_bytes, size_t *total_bytes);
+
+/* pinned host staging buffers for asynchronous transfers */
+int acc_host_alloc(acc_context ctx, size_t bytes, void **out);
+int acc_host_free(acc_context ctx, void *p);
+
+/* pokeArray / peekArray / copyArray [Async], memsetAsync:
+ * Array/Prim.hs:189-391, Execute.hs:405.  stream == NULL: default stream.
+ * The non-async forms return after the copy has completed.                  */
+int acc_memcpy_h2d(acc_context ctx, acc_devptr dst, const void *src, size_t bytes);
+int acc_memcpy_d2h(acc_context ctx, void *dst, acc_devptr src, size_t bytes);
+int acc_memcpy_d2d(acc_context ctx, acc_devptr dst, acc_devptr src, size_t bytes);
+int acc_memcpy_h2d_async(acc_context ctx, acc_devptr dst, const void *src, size_t bytes, acc_stream s);
+int acc_memcpy_d2h_async(acc_context ctx, void *dst, acc_devptr src, size_t bytes, acc_stream s);
+int acc_memcpy_d2d_async(acc_context ctx, acc_devptr dst, acc_devptr src, size_t bytes, acc_stream s);
+int acc_memset32_async(acc_context ctx, acc_devptr dst, uint32_t value, size_t count, acc_stream s);
+
+/* Execute/Stream.hs:102,134 and Execute/Event.hs:70-127, Debug.hs:48-67 */
+int acc_stream_create(acc_context ctx, acc_stream *out);
+int acc_stream_destroy(acc_context ctx, acc_stream s);
+int acc_stream_sync(acc_context ctx, acc_stream s);
+int acc_stream_wait_event(acc_context ctx, acc_stream s, acc_event e);
+int acc_event_create(acc_context ctx, int enable_timing, acc_event *out);
+int acc_event_destroy(acc_context ctx, acc_event e);
+int acc_event_record(acc_context ctx, acc_event e, acc_stream s);
+int acc_event_sync(acc_context ctx, acc_event e);
+int acc_event_query(acc_context ctx, acc_event e, int *done);
+int acc_event_elapsed_ms(acc_context ctx, acc_event start, acc_event stop, float *ms);
+
+/* Run-time compilation with the kernel cache.  Replaces the nvcc subprocess
+ * and the two-level cache: Compile.hs:543-594, Persistent.hs:77-137,218-228,
+ * 305-378.  Key = SHA-256 of (library version, target, compiler version,
+ * options, the device headers, the source text); look-up order is RAM table,
+ * then <cache dir>/<target>/<key>.co (size- and hash-checked, rewritten if
+ * damaged), then hiprtc.  Compilation needs no GPU.
+ *
+ *   target  "gfx950" style ISA name; NULL = the context's device (ctx may be
+ *           NULL only when target is given)
+ *   code    receives a pointer owned by the cache, valid until acc_cache_clear
+ */
+int acc_compile(acc_context ctx, const char *target, const char *source,
+                const char *const *options, int n_options,
+                const void **code, size_t *code_size);
+const char *acc_compile_log(void);                       /* log of the last compile on this thread */
+int acc_cache_set_dir(const char *dir);                  /* NULL/"" = memory only; default
+                                                            $ACC_HIP_CACHE_DIR or ~/.accelerate/accelerate-hip-<ver>/cache */
+const char *acc_cache_dir(void);
+typedef struct acc_cache_stats { uint64_t ram_hits, disk_hits, compiles, disk_errors; } acc_cache_stats;
+int acc_cache_get_stats(acc_cache_stats *out);
+int acc_cache_clear(int also_disk);                      /* -fflush-cache of the reference's debug flags */
+
+/* CUDA.loadData / getFun / unload / requires: Compile.hs:453-465,505,534 */
+int acc_module_load(acc_context ctx, const void *code, size_t code_size, acc_module *out);
+int acc_module_unload(acc_context ctx, acc_module m);
+int acc_module_get_function(acc_context ctx, acc_module m, const char *entry, acc_function *out);
+#define ACC_FUNC_NUM_REGS            0
+#define ACC_FUNC_SHARED_SIZE_BYTES   1
+#define ACC_FUNC_CONST_SIZE_BYTES    2
+#define ACC_FUNC_LOCAL_SIZE_BYTES    3
+#define ACC_FUNC_MAX_THREADS         4
+int acc_function_attr(acc_context ctx, acc_function f, int which, int *value);
+
+/* CUDA.optimalBlockSizeOf / Occupancy: Analysis/Launch.hs:42-102.  Resident
+ * workgroups per compute unit for the given block size and dynamic LDS.      */
+int acc_occupancy(acc_context ctx, acc_function f, int block, size_t dyn_lds, int *blocks_per_cu);
+
+/* CUDA.launchKernel fn (grid,1,1) (cta,1,1) smem stream args: Execute.hs:975-978 */
+int acc_launch(acc_context ctx, acc_function f, uint32_t grid, uint32_t block, uint32_t dyn_lds,
+               acc_stream s, void **args);
+
+/* Pure launch arithmetic of Analysis/Launch.hs, exposed for the host side
+ * and for tests: blocks needed for `n` elements at `per_block` each, at most
+ * `cus * blocks_per_cu`, at least 1 (split, :124-128; maxGrid, :51-55).      */
+int64_t acc_launch_grid(int64_t n, int64_t per_block, int64_t cus, int64_t blocks_per_cu);
+
+/* =========================================================================
+ * B. skeleton layer
+ * ========================================================================= */
+
+#define ACC_MAX_RANK 8
+#define ACC_MAX_COMP 8
+
+/* A device-resident array as the kernels see it: extents outermost first
+ * (row-major, innermost dimension last: CodeGen/Base.hs:193-202) and one
+ * device pointer per tuple component, structure-of-arrays
+ * (Array/Prim.hs:64-110; include/AccFFI.h:10-30 has the same shape/adata
+ * split).  rank 0 is a Scalar (one element).                                */
+typedef struct acc_array {
+  int32_t    rank;
+  int32_t    ncomp;
+  int64_t    shape[ACC_MAX_RANK];
+  acc_devptr ptr[ACC_MAX_COMP];
+} acc_array;
+
+/* signature of one free array variable of the scalar fragments (Gamma,
+ * AST.hs:87-112).  Variable k becomes the kernel parameters
+ *     const Int64 shIn<k>_<rank-1> ... shIn<k>_0,
+ *     const T<ncomp-1>* arrIn<k>_<ncomp-1> ... const T0* arrIn<k>_0
+ * exactly as CodeGen/Base.hs:69-89,348-383 names and orders them, and the
+ * fragments index them as arrIn<k>_<c>[i] (CodeGen.hs:714-747).              */
+typedef struct acc_env_sig {
+  int32_t     rank;
+  int32_t     ncomp;
+  const char *type[ACC_MAX_COMP];   /* C type of each component, component 0 first */
+} acc_env_sig;
+
+/* skeleton kinds: one per entry of CodeGen.hs:91-136 that is built */
+enum {
+  ACC_SKEL_MAP        = 0,   /* entry "map"       Mapping.hs:39-78      */
+  ACC_SKEL_GENERATE   = 1,   /* entry "generate"  IndexSpace.hs:47-83   */
+  ACC_SKEL_TRANSFORM  = 2,   /* entry "transform" IndexSpace.hs:96-141 (backpermute too) */
+  ACC_SKEL_FOLD       = 3,   /* foldAll / fold    Reduction.hs:56-65    */
+  ACC_SKEL_FOLD1      = 4,   /* fold1All / fold1  Reduction.hs:67-75    */
+  ACC_SKEL_FOLDSEG    = 5,   /* foldSeg           Reduction.hs:399-408  */
+  ACC_SKEL_FOLD1SEG   = 6,   /* fold1Seg          Reduction.hs:410-418  */
+  ACC_SKEL_SCANL      = 7,   /* PrefixSum.hs:51-66   */
+  ACC_SKEL_SCANL1     = 8,   /* PrefixSum.hs:77-91   */
+  ACC_SKEL_SCANLP     = 9,   /* scanl'  PrefixSum.hs:102-114 */
+  ACC_SKEL_SCANR      = 10,
+  ACC_SKEL_SCANR1     = 11,
+  ACC_SKEL_SCANRP     = 12,  /* scanr' */
+  ACC_SKEL_PERMUTE    = 13,  /* IndexSpace.hs:160-303 */
+  ACC_SKEL_STENCIL    = 14,  /* Stencil.hs:55-114     */
+  ACC_SKEL_KIND_COUNT = 15
+};
+
+/* how `combine` may be applied atomically by permute */
+enum {
+  ACC_COMBINE_GENERIC = 0,   /* compare-and-swap loop on the element's bits (4/8-byte elements) */
+  ACC_COMBINE_ADD     = 1,   /* combine x y == x + y   -> hardware atomic add   */
+  ACC_COMBINE_MIN     = 2,
+  ACC_COMBINE_MAX     = 3,
+  ACC_COMBINE_AND     = 4,
+  ACC_COMBINE_OR      = 5,
+  ACC_COMBINE_XOR     = 6
+};
+
+/* stencil boundary conditions: Stencil/Extra.hs:112-116 */
+enum { ACC_BOUNDARY_CLAMP = 0, ACC_BOUNDARY_MIRROR = 1, ACC_BOUNDARY_WRAP = 2, ACC_BOUNDARY_CONSTANT = 3 };
+
+/* flags */
+#define ACC_FLAG_FOLD_RIGHT   1u  /* foldSeg: associate x0 (+) (x1 (+) (... (+) z)) instead of ((x0 (+) x1) ...) (+) z */
+#define ACC_FLAG_FAST_MATH    2u  /* allow FMA contraction (default: off, every scalar op rounds as written) */
+
+/* What the code generator hands over for one array operation: the pieces
+ * CUTranslSkel / CUFun1 / CUFun2 / CUExp / CUDelayed carry across the
+ * reference's Compile boundary (CodeGen/Base.hs:98-138), as HIP C++ text.
+ * Fragments are EXPRESSIONS (GNU statement expressions ({ ...; v; }) allow
+ * local bindings) over the names given below and the env parameters.        */
+typedef struct acc_skel_desc {
+  int32_t            kind;          /* ACC_SKEL_*                                           */
+  uint32_t           flags;         /* ACC_FLAG_*                                           */
+  int32_t            n_env;         /* free array variables In0 .. In<n_env-1>              */
+  const acc_env_sig *env;
+  const char        *elt_type;      /* C type of the result element (single component)      */
+  int32_t            elt_size;      /* sizeof(elt_type); 0 = derive from the type's name    */
+  int32_t            out_rank;      /* map family, stencil: rank of the result (>= 0)       */
+  const char        *preamble;      /* file-scope declarations for the fragments, or NULL   */
+  const char        *get;           /* delayed input / element function over `ix` (Int64 linear
+                                       index); map family: value of out[ix].  Not used by stencil. */
+  const char        *combine;       /* over `x`, `y`: fold, foldSeg, scans, permute          */
+  const char        *seed;          /* NULL for the seedless kinds                           */
+  const char        *permutation;   /* permute: linear target index of source `ix`, or
+                                       ACC_IGNORE (-1) to drop the element                   */
+  int32_t            combine_hint;  /* ACC_COMBINE_*: lets permute use hardware atomics      */
+  /* stencil: taps t0 .. t<n-1> at offsets (dy, dx) from the focus (1-D: dy = 0),
+   * `stencil_fn` is an expression over t0.. giving the result element       */
+  int32_t            boundary;      /* ACC_BOUNDARY_*                                       */
+  const char        *boundary_constant;
+  int32_t            n_taps;
+  const int32_t     *tap_dy;
+  const int32_t     *tap_dx;
+  const char        *stencil_fn;
+  const char        *stencil_in_type; /* element type of the source array; NULL = elt_type */
+  const char        *seg_type;      /* foldSeg: C type of the offsets (NULL = "Int32")       */
+} acc_skel_desc;
+
+/* Generate + compile (through the cache) + load one skeleton instance and
+ * work out its launch shape.  The counterpart of build1/compile/link,
+ * Compile.hs:444-459,484-566, which yields the AccKernel record AST.hs:51-59. */
+int acc_skel_create(acc_context ctx, const acc_skel_desc *desc, acc_skel *out);
+int acc_skel_destroy(acc_skel s);
+
+/* The generated translation unit (for -ddump-cc style debugging and tests).
+ * variant 0 = aligned (128-bit accesses assumed legal), 1 = unaligned.      */
+int acc_skel_source(acc_skel s, int variant, const char **source);
+/* compile only (no GPU needed): used by the build check */
+int acc_skel_compile_only(const char *target, const acc_skel_desc *desc, size_t *code_size);
+
+/* kernel record of the instance: AccKernel, AST.hs:51-59 */
+typedef struct acc_skel_info {
+  char    entry[64];
+  int32_t block;              /* threads per workgroup          */
+  int32_t blocks_per_cu;      /* occupancy of the main kernel   */
+  int32_t num_regs;
+  int32_t static_lds;
+  int32_t elements_per_block; /* tile size                      */
+} acc_skel_info;
+int acc_skel_get_info(acc_skel s, acc_skel_info *out);
+
+/* ---- skeleton drivers (Execute.hs:264-450) ----------------------------------
+ * `env` points at n_env arrays in Gamma order.  All work is enqueued on
+ * `stream` and the call returns without waiting.                             */
+
+/* map / generate / transform: executeOp, Execute.hs:264-268.  out has the
+ * desc's out_rank; one element is written per index of out.                 */
+int acc_exec_map(acc_skel s, const acc_array *env, const acc_array *out, acc_stream stream);
+
+/* fold / fold1: foldOp / fold1Op / foldCore / foldRec, Execute.hs:282-318.
+ * in_shape has in_rank >= 1 extents of the delayed input; out has rank
+ * in_rank-1.  fold1 of an empty innermost dimension is ACC_ERR_INVALID
+ * ("empty array", Execute.hs:282-285).                                       */
+int acc_exec_fold(acc_skel s, const acc_array *env, int32_t in_rank, const int64_t *in_shape,
+                  const acc_array *out, acc_stream stream);
+
+/* foldSeg / fold1Seg: foldSegOp, Execute.hs:320-324.  `n` elements in one row;
+ * `offsets` is the manifest vector of nseg+1 segment starts (the front end
+ * has already turned lengths into offsets, CUDA.hs:402); out has nseg
+ * elements.                                                                  */
+int acc_exec_foldseg(acc_skel s, const acc_array *env, int64_t n, const acc_array *offsets,
+                     const acc_array *out, acc_stream stream);
+
+/* scans: scanOp / scan1Op / scan'Op / scanCore, Execute.hs:328-392.
+ *   scanl, scanr    : out holds n+1 elements, `total` is ignored (may be NULL)
+ *   scanl1, scanr1  : out holds n elements
+ *   scanl', scanr'  : out holds n elements, total is a Scalar                */
+int acc_exec_scan(acc_skel s, const acc_array *env, int64_t n, const acc_array *out,
+                  const acc_array *total, acc_stream stream);
+
+/* permute: permuteOp, Execute.hs:396-408.  `n_src` source elements (linear);
+ * out is first filled from `defaults` (same shape), then combined into.
+ * defaults may alias out (then nothing is copied).                           */
+int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_array *defaults,
+                     const acc_array *out, acc_stream stream);
+
+/* stencil: stencilOp, Execute.hs:413-425 (launched once, not twice).  `in` is
+ * the manifest source, out has the same shape (rank 1 or 2).                 */
+int acc_exec_stencil(acc_skel s, const acc_array *env, const acc_array *in, const acc_array *out,
+                     acc_stream stream);
+
+/* `iters` applications of the same stencil, ping-ponging between a and b on
+ * the device with no host round trip (what `awhile` with a counter, or a
+ * repeated run1, computes: Execute.hs:236-244, CUDA.hs:325-333).  The input is
+ * a; *result_in_b tells where the last application wrote.                    */
+int acc_exec_stencil_iterate(acc_skel s, const acc_array *env, const acc_array *a, const acc_array *b,
+                             int32_t iters, acc_stream stream, int32_t *result_in_b);
+
+#if defined(__GNUC__)
+#pragma GCC visibility pop
+#endif
+#ifdef __cplusplus
+}
+#endif
+#endif /* ACC_HIP_H */

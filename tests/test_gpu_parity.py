@@ -1,0 +1,501 @@
+"""Parity of the HIP skeletons against the CPU oracle, through the C ABI.
+
+Bit-exact for integer / index work; Float32 tolerances are written at each
+assertion.  Every case prints its name before touching the GPU so that a
+fault names its case.
+"""
+import json
+import os
+import sys
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+rng = np.random.default_rng(77)
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+F32 = (1, "float")
+I32 = (1, "Int32")
+
+AFFINE_PREAMBLE = """
+__device__ __forceinline__ Word32 affine16(Word32 x, Word32 y) {
+  Word32 a1 = x >> 16, b1 = x & 0xffffu, a2 = y >> 16, b2 = y & 0xffffu;
+  return (((a1 * a2) & 0xffffu) << 16) | ((a1 * b2 + b1) & 0xffffu);
+}
+"""
+
+
+def say(*a):
+    print("[case]", *a)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def A():
+    import acchip
+    return acchip
+
+
+@pytest.fixture(scope="module")
+def ctx(A):
+    c = A.Context(0)
+    p = c.props()
+    say("device", p.name.decode(), p.arch.decode(), "CUs", p.compute_units, "LDS/block", p.lds_per_block,
+        "wave", p.wavefront_size)
+    yield c
+    c.close()
+
+
+SIZES = [0, 1, 5, 63, 64, 65, 4095, 4096, 4097, 100003, (1 << 21) + 17]
+
+
+# --------------------------------------------------------------------------- map family
+
+def test_zipwith_saxpy_generate(A, ctx, orc):
+    mul = ctx.skeleton(A.SKEL_MAP, "float", env=[F32, F32], out_rank=1, get="arrIn0_0[ix] * arrIn1_0[ix]")
+    saxpy = ctx.skeleton(A.SKEL_MAP, "float", env=[F32, F32], out_rank=1, get="2.5f * arrIn0_0[ix] + arrIn1_0[ix]")
+    for n in SIZES:
+        say("zipWith/saxpy n =", n)
+        x = (rng.random(n) * 2 - 1).astype(np.float32)
+        y = (rng.random(n) * 2 - 1).astype(np.float32)
+        dx, dy, do = ctx.array(x), ctx.array(y), ctx.empty(n, np.float32)
+        mul.map([dx, dy], do)
+        assert np.array_equal(do.get(), x * y)
+        saxpy.map([dx, dy], do)
+        exp = (np.float32(2.5) * x).astype(np.float32) + y          # two roundings: contraction is off
+        assert np.array_equal(do.get(), exp)
+    say("generate 2-D iota")
+    gen = ctx.skeleton(A.SKEL_GENERATE, "Int32", out_rank=2, get="(Int32)((ix / shOut_0) * 1000 + ix % shOut_0)")
+    out = ctx.empty((37, 211), np.int32)
+    gen.map([], out)
+    yy, xx = np.mgrid[0:37, 0:211]
+    assert np.array_equal(out.get(), (yy * 1000 + xx).astype(np.int32))
+
+
+def test_backpermute_and_unaligned(A, ctx, orc):
+    gather = ctx.skeleton(A.SKEL_TRANSFORM, "float", env=[F32, I32], out_rank=1, get="arrIn0_0[arrIn1_0[ix]]")
+    for n in (1, 1000, 262147):
+        say("backpermute n =", n)
+        src = rng.random(5000).astype(np.float32)
+        idx = rng.integers(0, 5000, n, dtype=np.int32)
+        out = ctx.empty(n, np.float32)
+        gather.map([ctx.array(src), ctx.array(idx)], out)
+        assert np.array_equal(out.get(), orc.backpermute(src, idx))
+    say("map on pointers that are only 4-byte aligned")
+    copy = ctx.skeleton(A.SKEL_MAP, "float", env=[F32], out_rank=1, get="arrIn0_0[ix] + 1.0f")
+    n = 10001
+    x = rng.random(n + 3).astype(np.float32)
+    dx, do = ctx.array(x), ctx.array(np.zeros(n + 3, np.float32))
+    copy.map([dx.desc(shape=(n,), offset_elems=1)], do.desc(shape=(n,), offset_elems=3))
+    got = do.get()
+    assert np.array_equal(got[3:], x[1:n + 1] + np.float32(1)) and np.all(got[:3] == 0)
+
+
+# --------------------------------------------------------------------------- fold
+
+def test_dot_product(A, ctx, orc):
+    dot = ctx.skeleton(A.SKEL_FOLD, "float", env=[F32, F32], out_rank=0, get="arrIn0_0[ix] * arrIn1_0[ix]",
+                       combine="x + y", seed="0.0f")
+    out = ctx.empty((), np.float32)
+    for n in SIZES + [1 << 22]:
+        say("dot n =", n)
+        x = (rng.random(n) * 2 - 1).astype(np.float32)
+        y = (rng.random(n) * 2 - 1).astype(np.float32)
+        dot.fold([ctx.array(x), ctx.array(y)], n, out)
+        got = float(out.get())
+        truth, cond = orc.dot_f64(x, y), orc.dot_abs_f64(x, y)
+        # tolerance: 1e-4 relative to the interpreter's (sequential Float32) result, with the
+        # denominator floored by the rounding noise of that sequential sum itself
+        ref = float(orc.dot_f32(x, y))
+        floor = n * 2.0 ** -24 * cond
+        assert abs(got - ref) <= 1e-4 * max(abs(ref), floor) + 1e-30, (n, got, ref)
+        # and against the Float64 truth the tree-shaped GPU sum is far inside the classic bound
+        assert abs(got - truth) <= 64 * 2.0 ** -24 * cond + 1e-30
+    say("dot of small integers is exact in any order")
+    n = 1 << 20
+    xi = rng.integers(-8, 8, n).astype(np.float32)
+    yi = rng.integers(-8, 8, n).astype(np.float32)
+    dot.fold([ctx.array(xi), ctx.array(yi)], n, out)
+    assert float(out.get()) == float(orc.dot_f32(xi, yi))
+
+
+def test_fold_integers_and_errors(A, ctx, orc):
+    add = ctx.skeleton(A.SKEL_FOLD, "Int32", env=[I32], out_rank=0, get="arrIn0_0[ix]", combine="x + y", seed="42")
+    mx = ctx.skeleton(A.SKEL_FOLD1, "Int32", env=[I32], out_rank=0, get="arrIn0_0[ix]", combine="acc_max(x, y)")
+    add64 = ctx.skeleton(A.SKEL_FOLD, "Int64", env=[(1, "Int64")], out_rank=0, get="arrIn0_0[ix]", combine="x + y", seed="0")
+    out = ctx.empty((), np.int32)
+    out64 = ctx.empty((), np.int64)
+    for n in SIZES:
+        say("fold (+) / fold1 max n =", n)
+        x = rng.integers(-1000, 1000, n, dtype=np.int32)
+        dx = ctx.array(x)
+        add.fold([dx], n, out)
+        assert int(out.get()) == int(orc.fold(orc.OP_ADD, x, seed=42))
+        if n > 0:
+            mx.fold([dx], n, out)
+            assert int(out.get()) == int(x.max())
+        x64 = rng.integers(-2**40, 2**40, n, dtype=np.int64)
+        add64.fold([ctx.array(x64)], n, out64)
+        assert int(out64.get()) == int(x64.sum())
+    say("fold1 of an empty array is an error")
+    with pytest.raises(A.AccError) as e:
+        mx.fold([ctx.array(np.zeros(0, np.int32))], 0, out)
+    assert e.value.code == A.ERR_INVALID and "empty array" in e.value.message
+    say("repeated launches reuse the ticket")
+    x = rng.integers(-1000, 1000, 1 << 20, dtype=np.int32)
+    dx = ctx.array(x)
+    for _ in range(5):
+        add.fold([dx], x.size, out)
+        assert int(out.get()) == int(x.sum(dtype=np.int64)) + 42
+
+
+def test_fold_innermost_dimension(A, ctx, orc):
+    add = ctx.skeleton(A.SKEL_FOLD, "Int32", env=[(2, "Int32")], out_rank=1, get="arrIn0_0[ix]", combine="x + y", seed="7")
+    mn = ctx.skeleton(A.SKEL_FOLD1, "float", env=[(2, "float")], out_rank=1, get="arrIn0_0[ix]", combine="acc_min(x, y)")
+    for shape in [(1, 1), (3, 0), (17, 5), (300, 64), (33, 1000), (1000, 129)]:
+        say("fold along rows", shape)
+        x = rng.integers(-100, 100, shape, dtype=np.int32)
+        out = ctx.empty(shape[0], np.int32)
+        add.fold([ctx.array(x)], shape, out)
+        assert np.array_equal(out.get(), orc.fold(orc.OP_ADD, x, seed=7))
+        if shape[1] > 0:
+            xf = rng.random(shape).astype(np.float32)
+            outf = ctx.empty(shape[0], np.float32)
+            mn.fold([ctx.array(xf)], shape, outf)
+            assert np.array_equal(outf.get(), xf.min(axis=1))
+
+
+# --------------------------------------------------------------------------- scans
+
+def _run_scan(A, ctx, kind, elt, x, combine, seed, preamble=None, env_type=None):
+    n = x.size
+    sk = ctx.skeleton(A.SCAN_KINDS[kind], elt, env=[(1, env_type or elt)], get="arrIn0_0[ix]", combine=combine,
+                      seed=seed, preamble=preamble)
+    return sk
+
+
+@pytest.mark.parametrize("kind", ["scanl", "scanl1", "scanl'", "scanr", "scanr1", "scanr'"])
+def test_scan_int32_add(A, ctx, orc, kind):
+    seeded = not kind.endswith("1")
+    sk = ctx.skeleton(A.SCAN_KINDS[kind], "Int32", env=[I32], get="arrIn0_0[ix]", combine="x + y",
+                      seed="5" if seeded else None)
+    for n in SIZES + [(1 << 22) + 4099]:
+        say(kind, "(+) Int32 n =", n)
+        x = rng.integers(0, 16, n, dtype=np.int32)
+        plus = 1 if kind in ("scanl", "scanr") else 0
+        out = ctx.array(np.full(n + plus + 2, -777, np.int32))      # two guard words past the end
+        tot = ctx.array(np.array(-1, np.int32))
+        sk.scan([ctx.array(x)], n, out.desc(shape=(n + plus,)), tot if kind.endswith("'") else None)
+        got = out.get()
+        assert np.all(got[n + plus:] == -777), "wrote past the end"
+        exp = orc.scan(kind, orc.OP_ADD, x, seed=5)
+        if kind.endswith("'"):
+            assert np.array_equal(got[:n], exp[0]) and int(tot.get()) == int(exp[1])
+        else:
+            assert np.array_equal(got[:n + plus], exp)
+
+
+def test_scan_repeated_launches_and_sizes_interleaved(A, ctx, orc):
+    """the tile descriptors and the ticket counter are reused between launches"""
+    sk = ctx.skeleton(A.SKEL_SCANL, "Int32", env=[I32], get="arrIn0_0[ix]", combine="x + y", seed="0")
+    for n in [1 << 20, 1000, (1 << 21) + 3, 7, 1 << 20, 1 << 16]:
+        say("scanl relaunch n =", n)
+        x = rng.integers(0, 16, n, dtype=np.int32)
+        out = ctx.empty(n + 1, np.int32)
+        sk.scan([ctx.array(x)], n, out)
+        assert np.array_equal(out.get(), orc.scan("scanl", orc.OP_ADD, x, seed=0))
+
+
+@pytest.mark.parametrize("kind", ["scanl", "scanl1", "scanl'", "scanr", "scanr1", "scanr'"])
+def test_scan_noncommutative(A, ctx, orc, kind):
+    seeded = not kind.endswith("1")
+    sk = ctx.skeleton(A.SCAN_KINDS[kind], "Word32", env=[(1, "Word32")], get="arrIn0_0[ix]",
+                      combine="affine16(x, y)", seed="0x00030005u" if seeded else None, preamble=AFFINE_PREAMBLE)
+    for n in [1, 2, 64, 1000, 4096, 4097, 50001]:
+        say(kind, "affine16 n =", n)
+        x = rng.integers(0, 2**32, n, dtype=np.uint32)
+        plus = 1 if kind in ("scanl", "scanr") else 0
+        out = ctx.empty(n + plus, np.uint32)
+        tot = ctx.empty((), np.uint32)
+        sk.scan([ctx.array(x)], n, out, tot if kind.endswith("'") else None)
+        exp = orc.scan(kind, orc.OP_AFFINE16, x.view(np.int32), seed=0x00030005)
+        if kind.endswith("'"):
+            assert np.array_equal(out.get().view(np.int32), exp[0]) and int(tot.get().view(np.int32)) == int(exp[1])
+        else:
+            assert np.array_equal(out.get().view(np.int32), exp)
+
+
+def test_scan_wide_and_float_elements(A, ctx, orc):
+    for kind in ("scanl", "scanr1", "scanl'"):
+        seeded = not kind.endswith("1")
+        sk = ctx.skeleton(A.SCAN_KINDS[kind], "Int64", env=[(1, "Int64")], get="arrIn0_0[ix]", combine="x + y",
+                          seed="11" if seeded else None)
+        for n in [1, 2047, 2048, 2049, 300001]:
+            say(kind, "Int64 n =", n)
+            x = rng.integers(-2**40, 2**40, n, dtype=np.int64)
+            plus = 1 if kind in ("scanl", "scanr") else 0
+            out = ctx.empty(n + plus, np.int64)
+            tot = ctx.empty((), np.int64)
+            sk.scan([ctx.array(x)], n, out, tot if kind.endswith("'") else None)
+            exp = orc.scan(kind, orc.OP_ADD, x, seed=11)
+            if kind.endswith("'"):
+                assert np.array_equal(out.get(), exp[0]) and int(tot.get()) == int(exp[1])
+            else:
+                assert np.array_equal(out.get(), exp)
+    say("scanl1 (+) Float32: tolerance 1e-5 relative to the running magnitude")
+    sk = ctx.skeleton(A.SKEL_SCANL1, "float", env=[F32], get="arrIn0_0[ix]", combine="x + y")
+    n = 200000
+    x = rng.random(n).astype(np.float32)
+    out = ctx.empty(n, np.float32)
+    sk.scan([ctx.array(x)], n, out)
+    truth = np.cumsum(x.astype(np.float64))
+    assert np.max(np.abs(out.get() - truth) / truth) <= 1e-5
+    say("scanl1 max Float64")
+    sk = ctx.skeleton(A.SKEL_SCANL1, "double", env=[(1, "double")], get="arrIn0_0[ix]", combine="acc_max(x, y)")
+    xd = rng.random(70001)
+    outd = ctx.empty(xd.size, np.float64)
+    sk.scan([ctx.array(xd)], xd.size, outd)
+    assert np.array_equal(outd.get(), np.maximum.accumulate(xd))
+
+
+def test_scan_fused_producer(A, ctx, orc):
+    """the input of a scan is a delayed array: here zipWith (*) fused in"""
+    sk = ctx.skeleton(A.SKEL_SCANL, "Int32", env=[I32, I32], get="arrIn0_0[ix] * arrIn1_0[ix]", combine="x + y", seed="0")
+    n = 123457
+    a = rng.integers(-3, 4, n, dtype=np.int32)
+    b = rng.integers(-3, 4, n, dtype=np.int32)
+    out = ctx.empty(n + 1, np.int32)
+    say("scanl over fused zipWith")
+    sk.scan([ctx.array(a), ctx.array(b)], n, out)
+    assert np.array_equal(out.get(), orc.scan("scanl", orc.OP_ADD, a * b, seed=0))
+
+
+# --------------------------------------------------------------------------- permute
+
+def test_histograms(A, ctx, orc):
+    import workloads as wl
+    hist = ctx.skeleton(A.SKEL_PERMUTE, "Int32", env=[I32], out_rank=1, get="1", combine="x + y",
+                        permutation="arrIn0_0[ix]", combine_hint=A.COMBINE_ADD)
+    for name, keys, bins in [("uniform 256", wl.uniform_i32(1, 1 << 22, 256), 256),
+                             ("uniform 7", wl.uniform_i32(2, 100003, 7), 7),
+                             ("zipf 65536", wl.zipf_i32(3, 1 << 22, 65536), 65536),
+                             ("uniform 1M bins", wl.uniform_i32(4, 1 << 21, 1 << 20), 1 << 20),
+                             ("empty source", np.zeros(0, np.int32), 16)]:
+        say("histogram", name)
+        dfl = rng.integers(0, 5, bins, dtype=np.int32)
+        out = ctx.empty(bins, np.int32)
+        hist.permute([ctx.array(keys)], keys.size, ctx.array(dfl), out)
+        got = out.get()
+        assert np.array_equal(got, orc.permute(orc.OP_ADD, dfl, keys))
+        assert int(got.sum()) - int(dfl.sum()) == keys.size
+    say("histogram with ignored and out-of-range targets, in place over the defaults")
+    keys = wl.uniform_i32(5, 500000, 300)
+    keys[::5] = -1
+    dfl = rng.integers(0, 5, 300, dtype=np.int32)
+    out = ctx.array(dfl)
+    hist.permute([ctx.array(keys)], keys.size, out, out)
+    assert np.array_equal(out.get(), orc.permute(orc.OP_ADD, dfl, keys))
+
+
+def test_permute_other_combines(A, ctx, orc):
+    n, bins = 300000, 1000
+    dst = rng.integers(0, bins, n, dtype=np.int32)
+    dst[::11] = -1
+    src = rng.integers(-10**6, 10**6, n, dtype=np.int32)
+    dd, ds = ctx.array(dst), ctx.array(src)
+    for name, hint, comb, op in [("min", A.COMBINE_MIN, "acc_min(x, y)", orc.OP_MIN),
+                                 ("max", A.COMBINE_MAX, "acc_max(x, y)", orc.OP_MAX),
+                                 ("add generic (CAS loop)", A.COMBINE_GENERIC, "x + y", orc.OP_ADD),
+                                 ("weighted add", A.COMBINE_ADD, "x + y", orc.OP_ADD)]:
+        say("permute", name)
+        sk = ctx.skeleton(A.SKEL_PERMUTE, "Int32", env=[I32, I32], out_rank=1, get="arrIn1_0[ix]", combine=comb,
+                          permutation="arrIn0_0[ix]", combine_hint=hint)
+        dfl = rng.integers(-100, 100, bins, dtype=np.int32)
+        out = ctx.empty(bins, np.int32)
+        sk.permute([dd, ds], n, ctx.array(dfl), out)
+        assert np.array_equal(out.get(), orc.permute(op, dfl, dst, src))
+    say("permute Float32 (+): order of arrival differs, tolerance 1e-4 of the absolute sum")
+    sk = ctx.skeleton(A.SKEL_PERMUTE, "float", env=[I32, F32], out_rank=1, get="arrIn1_0[ix]", combine="x + y",
+                      permutation="arrIn0_0[ix]", combine_hint=A.COMBINE_ADD)
+    srcf = (rng.random(n) * 2 - 1).astype(np.float32)
+    dfl = np.zeros(bins, np.float32)
+    out = ctx.empty(bins, np.float32)
+    sk.permute([dd, ctx.array(srcf)], n, ctx.array(dfl), out)
+    ok = dst >= 0
+    truth = np.bincount(dst[ok], weights=srcf[ok].astype(np.float64), minlength=bins)
+    mag = np.bincount(dst[ok], weights=np.abs(srcf[ok]).astype(np.float64), minlength=bins)
+    assert np.all(np.abs(out.get() - truth) <= 1e-4 * mag + 1e-30)
+    say("permute with a unique target per element (a scatter): FIRST-style combine keeps the new value")
+    perm = rng.permutation(5000).astype(np.int32)
+    vals = rng.integers(0, 10**6, 5000, dtype=np.int32)
+    sk = ctx.skeleton(A.SKEL_PERMUTE, "Int32", env=[I32, I32], out_rank=1, get="arrIn1_0[ix]", combine="x",
+                      permutation="arrIn0_0[ix]")
+    out = ctx.empty(5000, np.int32)
+    sk.permute([ctx.array(perm), ctx.array(vals)], 5000, ctx.array(np.full(5000, -1, np.int32)), out)
+    assert np.array_equal(out.get(), orc.permute(orc.OP_FIRST, np.full(5000, -1, np.int32), perm, vals))
+
+
+# --------------------------------------------------------------------------- stencil
+
+GAUSS_TAPS = [(dy, dx) for dy in (-1, 0, 1) for dx in (-1, 0, 1)]
+LAPLACE_TAPS = [(-1, 0), (0, -1), (0, 0), (0, 1), (1, 0)]
+
+
+@pytest.mark.parametrize("mode", ["clamp", "mirror", "wrap", "constant"])
+def test_stencil_2d(A, ctx, orc, mode):
+    gauss = ctx.skeleton(A.SKEL_STENCIL, "float", out_rank=2, taps=GAUSS_TAPS,
+                         stencil_fn=A.linear_stencil_fn([1, 2, 1, 2, 4, 2, 1, 2, 1], 16), boundary=mode,
+                         boundary_constant="0.25f")
+    lap = ctx.skeleton(A.SKEL_STENCIL, "float", out_rank=2, taps=LAPLACE_TAPS,
+                       stencil_fn=A.linear_stencil_fn([1, 1, -4, 1, 1]), boundary=mode, boundary_constant="0.25f")
+    for shape in [(5, 5), (7, 3), (3, 64), (33, 70), (16, 256), (300, 517), (1024, 1024), (531, 1028)]:
+        say("stencil", mode, shape)
+        img = rng.random(shape).astype(np.float32)
+        d, o = ctx.array(img), ctx.empty(shape, np.float32)
+        gauss.stencil([], d, o)
+        exp = orc.stencil2d(img, orc.GAUSS3X3, divisor=16.0, mode=mode, constant=0.25)
+        assert np.max(np.abs(o.get() - exp)) <= 1e-5          # stated tolerance; in practice identical bits
+        assert np.array_equal(o.get(), exp)
+        lap.stencil([], d, o)
+        exp = orc.stencil2d(img, orc.LAPLACE5, mode=mode, constant=0.25)
+        assert np.max(np.abs(o.get() - exp)) <= 1e-5
+        assert np.array_equal(o.get(), exp)
+
+
+def test_stencil_iterated_and_asymmetric(A, ctx, orc):
+    gauss = ctx.skeleton(A.SKEL_STENCIL, "float", out_rank=2, taps=GAUSS_TAPS,
+                         stencil_fn=A.linear_stencil_fn([1, 2, 1, 2, 4, 2, 1, 2, 1], 16), boundary="clamp")
+    for shape, iters in [((512, 768), 10), ((100, 260), 3), ((64, 256), 0)]:
+        say("gaussian x", iters, shape)
+        img = rng.random(shape).astype(np.float32)
+        a, b = ctx.array(img), ctx.empty(shape, np.float32)
+        res = gauss.stencil_iterate([], a, b, iters)
+        exp = orc.stencil2d(img, orc.GAUSS3X3, divisor=16.0, mode="clamp", iters=iters)
+        assert np.max(np.abs(res.get() - exp)) <= 1e-5
+    say("asymmetric taps, radius 2")
+    taps = [(-2, 1, 3.0), (0, -2, -2.0), (1, 0, 5.0), (2, 2, 1.0)]
+    sk = ctx.skeleton(A.SKEL_STENCIL, "float", out_rank=2, taps=[(t[0], t[1]) for t in taps],
+                      stencil_fn=A.linear_stencil_fn([t[2] for t in taps]), boundary="wrap")
+    img = rng.integers(0, 50, (70, 300)).astype(np.float32)
+    o = ctx.empty(img.shape, np.float32)
+    sk.stencil([], ctx.array(img), o)
+    assert np.array_equal(o.get(), orc.stencil2d(img, taps, mode="wrap"))
+
+
+def test_stencil_1d(A, ctx, orc):
+    for mode in ("clamp", "mirror", "wrap", "constant"):
+        sk = ctx.skeleton(A.SKEL_STENCIL, "float", out_rank=1, taps=[(0, -1), (0, 0), (0, 1)],
+                          stencil_fn=A.linear_stencil_fn([1, -2, 1]), boundary=mode, boundary_constant="0.5f")
+        for n in (1, 2, 5, 1023, 1024, 1025, 100001):
+            if n < 2 and mode in ("mirror",):
+                continue                                        # the index maps assume the array spans the stencil
+            say("stencil 1-D", mode, n)
+            v = rng.random(n).astype(np.float32)
+            o = ctx.empty(n, np.float32)
+            sk.stencil([], ctx.array(v), o)
+            exp = orc.stencil1d(v, [(-1, 1.0), (0, -2.0), (1, 1.0)], mode=mode, constant=0.5)
+            assert np.array_equal(o.get(), exp)
+
+
+# --------------------------------------------------------------------------- foldSeg / SMVM
+
+def _csr(nrows, ncols, mean, empty_every=0):
+    lens = rng.poisson(mean, nrows).astype(np.int32)
+    if empty_every:
+        lens[::empty_every] = 0
+    offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    nnz = int(offs[-1])
+    cols = rng.integers(0, ncols, nnz, dtype=np.int32)
+    vals = (rng.random(nnz) * 2 - 1).astype(np.float32)
+    x = (rng.random(ncols) * 2 - 1).astype(np.float32)
+    return vals, cols, offs, x
+
+
+@pytest.mark.parametrize("right", [False, True])
+def test_smvm(A, ctx, orc, right):
+    smvm = ctx.skeleton(A.SKEL_FOLDSEG, "float", env=[F32, I32, F32], get="arrIn0_0[ix] * arrIn2_0[arrIn1_0[ix]]",
+                        combine="x + y", seed="0.0f", flags=A.FLAG_FOLD_RIGHT if right else 0)
+    d = orc.DIR_RIGHT if right else orc.DIR_LEFT
+    for nrows, ncols, mean, ee in [(1, 10, 3, 0), (255, 100, 8, 0), (256, 100, 32, 7), (257, 100, 32, 0),
+                                   (50000, 4096, 32, 9), (3000, 512, 700, 4), (40, 64, 9000, 3), (100000, 1000, 1, 2)]:
+        say("smvm right" if right else "smvm left", nrows, "rows, mean length", mean)
+        vals, cols, offs, x = _csr(nrows, ncols, mean, ee)
+        y = ctx.array(np.full(nrows, np.nan, np.float32))
+        smvm.foldseg([ctx.array(vals), ctx.array(cols), ctx.array(x)], vals.size, ctx.array(offs), y)
+        exp = orc.smvm_f32(vals, cols, offs, x, d)
+        got = y.get()
+        # the segments are folded in index order, like the sequential interpreter: identical bits.
+        # (stated tolerance for this configuration: 1e-4 relative per row)
+        assert np.array_equal(got, exp)
+        y64, yabs = orc.smvm_f64(vals, cols, offs, x)
+        assert np.all(np.abs(got - y64) <= 1e-4 * np.maximum(np.abs(y64), 1e-3 * yabs) + 1e-30)
+
+
+def test_foldseg_integers(A, ctx, orc):
+    add = ctx.skeleton(A.SKEL_FOLDSEG, "Int32", env=[I32], get="arrIn0_0[ix]", combine="x + y", seed="3")
+    mx = ctx.skeleton(A.SKEL_FOLD1SEG, "Int32", env=[I32], get="arrIn0_0[ix]", combine="acc_max(x, y)")
+    for nseg, mean in [(1, 5), (1000, 3), (70000, 20), (513, 1500)]:
+        say("foldSeg Int32", nseg, "segments, mean", mean)
+        lens = rng.poisson(mean, nseg).astype(np.int32)
+        offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        x = rng.integers(-1000, 1000, int(offs[-1]), dtype=np.int32)
+        out = ctx.empty(nseg, np.int32)
+        add.foldseg([ctx.array(x)], x.size, ctx.array(offs), out)
+        assert np.array_equal(out.get(), orc.foldseg(orc.OP_ADD, x, offs, seed=3))
+        lens1 = np.maximum(lens, 1)
+        offs1 = np.concatenate([[0], np.cumsum(lens1)]).astype(np.int32)
+        x1 = rng.integers(-1000, 1000, int(offs1[-1]), dtype=np.int32)
+        mx.foldseg([ctx.array(x1)], x1.size, ctx.array(offs1), out)
+        assert np.array_equal(out.get(), orc.foldseg(orc.OP_MAX, x1, offs1))
+
+
+# --------------------------------------------------------------------------- committed fixtures
+
+def test_golden_fixtures_on_gpu(A, ctx):
+    """the numpy/scipy-made vectors of tests/golden, through the HIP path"""
+    with open(os.path.join(GOLDEN, "golden.json")) as fh:
+        g = json.load(fh)
+    say("golden scans")
+    x = np.array(g["scan"]["x"], dtype=np.int32)
+    dx = ctx.array(x)
+    for kind, key in (("scanl", "scanl"), ("scanl1", "scanl1"), ("scanr", "scanr")):
+        sk = ctx.skeleton(A.SCAN_KINDS[kind], "Int32", env=[I32], get="arrIn0_0[ix]", combine="x + y",
+                          seed=str(g["scan"]["seed"]) if kind != "scanl1" else None)
+        out = ctx.empty(len(g["scan"][key]), np.int32)
+        sk.scan([dx], x.size, out)
+        assert out.get().tolist() == g["scan"][key]
+    say("golden histogram")
+    keys = np.array(g["hist"]["keys"], dtype=np.int32)
+    hist = ctx.skeleton(A.SKEL_PERMUTE, "Int32", env=[I32], out_rank=1, get="1", combine="x + y",
+                        permutation="arrIn0_0[ix]", combine_hint=A.COMBINE_ADD)
+    out = ctx.empty(g["hist"]["bins"], np.int32)
+    hist.permute([ctx.array(keys)], keys.size, ctx.array(np.zeros(g["hist"]["bins"], np.int32)), out)
+    assert out.get().tolist() == g["hist"]["counts"]
+    say("golden stencils")
+    img = np.array(g["stencil"]["img"], dtype=np.float32)
+    for mode in ("clamp", "mirror", "wrap", "constant"):
+        for name, taps, coef, div in (("gauss_", GAUSS_TAPS, [1, 2, 1, 2, 4, 2, 1, 2, 1], 16),
+                                      ("laplace_", LAPLACE_TAPS, [1, 1, -4, 1, 1], None)):
+            sk = ctx.skeleton(A.SKEL_STENCIL, "float", out_rank=2, taps=taps, stencil_fn=A.linear_stencil_fn(coef, div),
+                              boundary=mode, boundary_constant="%rf" % g["stencil"]["constant"])
+            o = ctx.empty(img.shape, np.float32)
+            sk.stencil([], ctx.array(img), o)
+            assert np.max(np.abs(o.get() - np.array(g["stencil"][name + mode]))) <= 1e-5
+    say("golden smvm and dot")
+    s = g["smvm"]
+    smvm = ctx.skeleton(A.SKEL_FOLDSEG, "float", env=[F32, I32, F32], get="arrIn0_0[ix] * arrIn2_0[arrIn1_0[ix]]",
+                        combine="x + y", seed="0.0f")
+    y = ctx.empty(len(s["y"]), np.float32)
+    smvm.foldseg([ctx.array(np.array(s["vals"], np.float32)), ctx.array(np.array(s["cols"], np.int32)),
+                  ctx.array(np.array(s["x"], np.float32))], len(s["vals"]),
+                 ctx.array(np.array(s["offsets"], np.int32)), y)
+    ref = np.array(s["y"])
+    assert np.max(np.abs(y.get() - ref)) <= 1e-5
+    d = g["dot"]
+    dot = ctx.skeleton(A.SKEL_FOLD, "float", env=[F32, F32], out_rank=0, get="arrIn0_0[ix] * arrIn1_0[ix]",
+                       combine="x + y", seed="0.0f")
+    out = ctx.empty((), np.float32)
+    dot.fold([ctx.array(np.array(d["x"], np.float32)), ctx.array(np.array(d["y"], np.float32))], len(d["x"]), out)
+    assert abs(float(out.get()) - d["dot"]) <= 1e-4 * abs(d["dot"])
