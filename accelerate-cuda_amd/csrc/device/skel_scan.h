@@ -16,8 +16,9 @@
  *     global memory.  A tile first publishes its own total (state AGGREGATE),
  *     then one wave walks back over its predecessors, 64 descriptors per step,
  *     until it meets an inclusive PREFIX, and finally publishes its own PREFIX.
- *     Tile numbers are handed out by an atomic counter, so every predecessor
- *     of a running tile is itself running and the walk cannot deadlock.
+ *     Tile numbers are handed out by an atomic counter to a resident grid of
+ *     persistent workgroups, so every predecessor of a tile being worked on
+ *     is itself held by a running workgroup and the walk cannot deadlock.
  *   - descriptors are tagged with a launch epoch and the counter is used
  *     relative to a base, so nothing needs clearing between launches.
  *
@@ -42,6 +43,14 @@
 #define ACC_TILE  (ACC_BLOCK * ACC_ITEMS)
 #define ACC_WAVES (ACC_BLOCK / ACC_WAVE)
 
+#ifndef ACC_LOOKBACK
+#define ACC_LOOKBACK 4
+#endif
+
+#ifndef ACC_DESC_STRIDE
+#define ACC_DESC_STRIDE 1     /* 8-byte words between the descriptors of consecutive tiles */
+#endif
+
 #define ACC_ST_AGGREGATE 1u
 #define ACC_ST_PREFIX    2u
 
@@ -56,11 +65,11 @@ struct acc_scan_desc {
   {
     unsigned int b = 0;
     __builtin_memcpy(&b, &v, sizeof(T));
-    __hip_atomic_store(d + tile, ((unsigned long long)flag << 32) | b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(d + tile * ACC_DESC_STRIDE, ((unsigned long long)flag << 32) | b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   ACC_DEV unsigned int get(Int64 tile, T &v) const
   {
-    unsigned long long w = __hip_atomic_load(d + tile, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    unsigned long long w = __hip_atomic_load(d + tile * ACC_DESC_STRIDE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     unsigned int b = (unsigned int)w;
     __builtin_memcpy(&v, &b, sizeof(T));
     return (unsigned int)(w >> 32);
@@ -106,41 +115,53 @@ template <typename T> struct acc_sv<T, true> {
   template <typename F> static ACC_DEV acc_lifted<T, F> lift(F f) { return acc_lift<T>(f); }
 };
 
-/* ---- decoupled look-back, executed by wave 0 of a tile > 0 --------------- */
+/* ---- decoupled look-back, executed by wave 0 of a tile > 0 ---------------
+ * Every step inspects ACC_LOOKBACK descriptors per lane, 64 * ACC_LOOKBACK
+ * predecessors in one memory round trip.  The chain of tiles can advance by
+ * at most one such window per round trip, so the window has to be wide
+ * enough for the rate at which tiles retire.                                */
 template <typename T, typename Op>
 ACC_DEV T acc_scan_lookback(const acc_scan_desc<T> &desc, Int64 tile, const T &block_total, Op op,
                             unsigned int epoch, int lane)
 {
-  if (lane == 0) desc.put(tile, (epoch << 2) | ACC_ST_AGGREGATE, block_total);
-
-  /* lanes are ordered nearest predecessor first, so a reduction in lane order
+  /* slots are ordered nearest predecessor first, so a reduction in slot order
    * must combine (later, earlier) */
   auto back = acc_lift<T>([&](const T &later, const T &earlier) -> T { return op(earlier, later); });
   acc_opt<T> run = acc_none<T>();
 
-  for (Int64 look = tile - 1;; look -= ACC_WAVE) {
-    const Int64 idx = look - lane;
-    T v = T();
-    unsigned int st = 0;
-    if (idx >= 0) {
-      unsigned int fl = desc.get(idx, v);
-      while ((fl >> 2) != epoch) {
-        __builtin_amdgcn_s_sleep(1);
-        fl = desc.get(idx, v);
+  for (Int64 look = tile - 1;; look -= ACC_WAVE * ACC_LOOKBACK) {
+    T v[ACC_LOOKBACK];
+    unsigned int fl[ACC_LOOKBACK];
+    Int64 idx[ACC_LOOKBACK];
+#pragma unroll
+    for (int j = 0; j < ACC_LOOKBACK; ++j) {            /* all loads in flight together */
+      idx[j] = look - (lane * ACC_LOOKBACK + j);
+      v[j] = T();
+      fl[j] = 0;
+      if (idx[j] >= 0) fl[j] = desc.get(idx[j], v[j]);
+    }
+    int nearest = ACC_WAVE * ACC_LOOKBACK;              /* slot of the nearest PREFIX, if any */
+#pragma unroll
+    for (int j = 0; j < ACC_LOOKBACK; ++j) {
+      if (idx[j] >= 0) {
+        while ((fl[j] >> 2) != epoch) {
+          __builtin_amdgcn_s_sleep(1);
+          fl[j] = desc.get(idx[j], v[j]);
+        }
       }
-      st = fl & 3u;
+      const unsigned long long m = __ballot(idx[j] >= 0 && (fl[j] & 3u) == ACC_ST_PREFIX);
+      if (m) nearest = acc_min(nearest, (__ffsll((long long)m) - 1) * ACC_LOOKBACK + j);
     }
-    const unsigned long long prefixes = __ballot(st == ACC_ST_PREFIX);
-    acc_opt<T> c;
-    c.v = v;
-    if (prefixes) {
-      const int first = __ffsll((long long)prefixes) - 1;
-      c.ok = (lane <= first);
-      run = back(run, acc_wave_reduce(c, back));
-      break;
+    acc_opt<T> c = acc_none<T>();
+#pragma unroll
+    for (int j = 0; j < ACC_LOOKBACK; ++j) {
+      acc_opt<T> e;
+      e.v = v[j];
+      e.ok = (idx[j] >= 0) && (lane * ACC_LOOKBACK + j <= nearest);
+      c = back(c, e);
     }
-    c.ok = 1;                       /* tile 0 always posts a PREFIX, so idx >= 0 here */
     run = back(run, acc_wave_reduce(c, back));
+    if (nearest < ACC_WAVE * ACC_LOOKBACK) break;       /* tile 0 always posts a PREFIX: the walk ends */
   }
   const T prefix = run.v;
   if (lane == 0) desc.put(tile, (epoch << 2) | ACC_ST_PREFIX, op(prefix, block_total));
@@ -148,10 +169,46 @@ ACC_DEV T acc_scan_lookback(const acc_scan_desc<T> &desc, Int64 tile, const T &b
 }
 
 /* ---- one tile ------------------------------------------------------------ */
-template <bool PARTIAL, typename T, typename Get, typename Op>
-ACC_DEV void acc_scan_tile(Get get, Op op_raw, const T seed, const Int64 tile, const Int64 base, const Int64 n,
-                           T *__restrict__ out, T *__restrict__ sum, const acc_scan_desc<T> &desc,
-                           const unsigned int epoch, void *s_wave_raw, T *s_prefix)
+/* physical index of item 0 of row r of this lane; item k is k further on in
+ * logical order (for right-handed scans: k further back in memory)          */
+ACC_DEV Int64 acc_scan_ix0(const Int64 base, const int wave, const int lane, const int r)
+{
+  const int q = ((wave * ACC_ROWS + r) * ACC_WAVE + lane) * ACC_VEC;     /* logical offset in the tile */
+  return base + (ACC_SCAN_RIGHT ? (ACC_TILE - 1 - q) : q);
+}
+
+/* issue the loads of a tile; nothing here waits for them */
+template <typename T, typename Get>
+ACC_DEV void acc_scan_load(Get get, const Int64 base, const Int64 n, T (&x)[ACC_ROWS][ACC_VEC], const int wave, const int lane)
+{
+  if (base + ACC_TILE <= n) {
+#pragma unroll
+    for (int r = 0; r < ACC_ROWS; ++r) {
+      const Int64 i0 = acc_scan_ix0(base, wave, lane, r);
+#pragma unroll
+      for (int k = 0; k < ACC_VEC; ++k) x[r][k] = get(ACC_SCAN_RIGHT ? i0 - k : i0 + k);
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < ACC_ROWS; ++r) {
+      const Int64 i0 = acc_scan_ix0(base, wave, lane, r);
+#pragma unroll
+      for (int k = 0; k < ACC_VEC; ++k) {
+        const Int64 ix = ACC_SCAN_RIGHT ? i0 - k : i0 + k;
+        x[r][k] = T();
+        if (ix < n) x[r][k] = get(ix);
+      }
+    }
+  }
+}
+
+/* scan one tile whose elements are already in registers.  `prefetch` is
+ * called once the block total is known and before the look-back starts: the
+ * caller uses it to put the next tile's loads in flight behind the wait.     */
+template <bool PARTIAL, typename T, typename Op, typename Prefetch>
+ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op_raw, const T seed, const Int64 tile, const Int64 base,
+                           const Int64 n, T *__restrict__ out, T *__restrict__ sum, const acc_scan_desc<T> &desc,
+                           const unsigned int epoch, void *s_wave_raw, T *s_prefix, Prefetch prefetch)
 {
   typedef acc_sv<T, PARTIAL> S;
   typedef typename S::V V;
@@ -161,17 +218,16 @@ ACC_DEV void acc_scan_tile(Get get, Op op_raw, const T seed, const Int64 tile, c
   const int wave = (int)(threadIdx.x >> 6);
   V *s_wave = (V *)s_wave_raw;
 
-  /* load, and scan the ACC_VEC items each lane holds per row */
+  /* scan the ACC_VEC items each lane holds per row */
   V s[ACC_ROWS][ACC_VEC];
   Int64 ix0[ACC_ROWS];
 #pragma unroll
   for (int r = 0; r < ACC_ROWS; ++r) {
-    const int q = ((wave * ACC_ROWS + r) * ACC_WAVE + lane) * ACC_VEC;   /* logical offset in the tile */
-    ix0[r] = base + (ACC_SCAN_RIGHT ? (ACC_TILE - 1 - q) : q);          /* physical index of item k = 0 */
+    ix0[r] = acc_scan_ix0(base, wave, lane, r);
 #pragma unroll
     for (int k = 0; k < ACC_VEC; ++k) {
       const Int64 ix = ACC_SCAN_RIGHT ? ix0[r] - k : ix0[r] + k;
-      V v = (!PARTIAL || ix < n) ? S::some(get(ix)) : S::none();
+      V v = (!PARTIAL || ix < n) ? S::some(x[r][k]) : S::none();
       s[r][k] = (k == 0) ? v : op(s[r][k - 1], v);
     }
   }
@@ -202,16 +258,23 @@ ACC_DEV void acc_scan_tile(Get get, Op op_raw, const T seed, const Int64 tile, c
     block_total = op(block_total, s_wave[w]);
   }
 
-  /* chain the tiles */
+  /* publish early, then start the next tile's loads, then look back */
   T prefix = seed;
   bool has_prefix = ACC_HAS_SEED;
   if (tile == 0) {
     if (threadIdx.x == 0)
       desc.put(0, (epoch << 2) | ACC_ST_PREFIX,
                ACC_HAS_SEED ? op_raw(seed, S::val(block_total)) : S::val(block_total));
+    prefetch();
   } else {
+    if (threadIdx.x == 0) desc.put(tile, (epoch << 2) | ACC_ST_AGGREGATE, S::val(block_total));
+    prefetch();
     if (wave == 0) {
+#ifdef ACC_SCAN_DEBUG_NO_LOOKBACK
+      const T p = S::val(block_total);
+#else
       const T p = acc_scan_lookback(desc, tile, S::val(block_total), op_raw, epoch, lane);
+#endif
       if (lane == 0) *s_prefix = p;
     }
     __syncthreads();
@@ -262,6 +325,11 @@ ACC_DEV void acc_scan_tile(Get get, Op op_raw, const T seed, const Int64 tile, c
   }
 }
 
+/* The kernel is persistent: a resident grid of workgroups draws tile numbers
+ * from an atomic counter until they run out.  The ticket of the tile after
+ * next is requested while the current tile is being scanned, and the next
+ * tile's elements are loaded while the current tile waits for its prefix, so
+ * neither the ticket nor the look-back leaves the memory system idle.        */
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 ACC_ENTRY(ACC_ENV_PARAMS
           const Int64 shOut_0, ACC_ELT *__restrict__ arrOut_0,
@@ -278,7 +346,7 @@ ACC_ENTRY(ACC_ENV_PARAMS
 #endif
   (void)shOut_0;
 
-  __shared__ unsigned int s_tile;
+  __shared__ unsigned int s_ticket[2];
   __shared__ T s_prefix;
   __shared__ acc_opt<T> s_wave[ACC_WAVES];
 
@@ -292,28 +360,50 @@ ACC_ENTRY(ACC_ENV_PARAMS
 #else
   const T seed = T();
 #endif
+  const int lane = acc_lane();
+  const int wave = (int)(threadIdx.x >> 6);
+  const acc_scan_desc<T> desc(desc0, desc1, desc2);
+  auto tile_base = [&](const Int64 t) -> Int64 { return (ACC_SCAN_RIGHT ? (num_tiles - 1 - t) : t) * (Int64)ACC_TILE; };
 
-  if (threadIdx.x == 0) s_tile = atomicAdd(tile_counter, 1u) - counter_base;
+  if (threadIdx.x == 0) s_ticket[0] = atomicAdd(tile_counter, 1u) - counter_base;
   __syncthreads();
+  Int64 tile = (Int64)s_ticket[0];
 
   if (n <= 0) {                                   /* PrefixSum.hs:249-251,330-334: scan of nothing is [seed] */
-    if (threadIdx.x == 0 && s_tile == 0) {
+    if (threadIdx.x == 0 && tile == 0) {
       if (ACC_SCAN_MODE == 0 || ACC_SCAN_MODE == 3) arrOut_0[0] = seed;
       if (ACC_SCAN_MODE == 2) arrSum_0[0] = seed;
     }
     return;
   }
-
-  const Int64 tile  = (Int64)s_tile;
-  if (tile >= num_tiles) return;
-  const Int64 ptile = ACC_SCAN_RIGHT ? (num_tiles - 1 - tile) : tile;
-  const Int64 base  = ptile * (Int64)ACC_TILE;
-  const acc_scan_desc<T> desc(desc0, desc1, desc2);
-
   if (ACC_SCAN_MODE == 3 && tile == 0 && threadIdx.x == 0) arrOut_0[n] = seed;
 
-  if (base + ACC_TILE <= n)
-    acc_scan_tile<false, T>(get, op, seed, tile, base, n, arrOut_0, arrSum_0, desc, epoch, (void *)s_wave, &s_prefix);
-  else
-    acc_scan_tile<true, T>(get, op, seed, tile, base, n, arrOut_0, arrSum_0, desc, epoch, (void *)s_wave, &s_prefix);
+  T cur[ACC_ROWS][ACC_VEC], nxt[ACC_ROWS][ACC_VEC];
+  if (tile < num_tiles) acc_scan_load(get, tile_base(tile), n, cur, wave, lane);
+
+  int parity = 1;
+  while (tile < num_tiles) {
+    /* ticket for the tile after this one; it is read after the next barrier */
+    if (threadIdx.x == 0) s_ticket[parity] = atomicAdd(tile_counter, 1u) - counter_base;
+
+    Int64 next = num_tiles;
+    auto prefetch = [&]() {
+      next = (Int64)s_ticket[parity];
+      if (next < num_tiles) acc_scan_load(get, tile_base(next), n, nxt, wave, lane);
+    };
+
+    const Int64 base = tile_base(tile);
+    if (base + ACC_TILE <= n)
+      acc_scan_tile<false, T>(cur, op, seed, tile, base, n, arrOut_0, arrSum_0, desc, epoch, (void *)s_wave, &s_prefix, prefetch);
+    else
+      acc_scan_tile<true, T>(cur, op, seed, tile, base, n, arrOut_0, arrSum_0, desc, epoch, (void *)s_wave, &s_prefix, prefetch);
+
+#pragma unroll
+    for (int r = 0; r < ACC_ROWS; ++r)
+#pragma unroll
+      for (int k = 0; k < ACC_VEC; ++k) cur[r][k] = nxt[r][k];
+    tile = next;
+    parity ^= 1;
+    __syncthreads();          /* s_wave and s_prefix are free for the next tile */
+  }
 }

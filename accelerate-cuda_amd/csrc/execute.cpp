@@ -238,18 +238,24 @@ int acc_exec_scan(acc_skel s, const acc_array *env, int64_t n, const acc_array *
   args.ptr(sum_ptr);
   args.i64(n);
 
+  const int v = aligned ? 0 : 1;
+  ACC_TRY(s->ensure_variant(v));
   const int64_t tile = s->elements_per_block();
   const int64_t tiles = (n + tile - 1) / tile;
-  const int64_t grid = std::max<int64_t>(1, tiles);
+  // a resident grid of persistent workgroups; each draws tiles until none are left
+  const int64_t per_cu = std::max(1, std::min(s->variants[v].blocks_per_cu, acc::tune("scan.blocks_per_cu", 2)));
+  const int64_t grid = std::max<int64_t>(1, std::min<int64_t>(tiles, (int64_t)s->ctx->props.multiProcessorCount * per_cu));
+  const int64_t draws = tiles + grid;             // every tile once, plus the draw that tells a workgroup to stop
+  const int64_t ndesc = std::max<int64_t>(1, tiles);
   const size_t esz = s->spec.elt_size;
   size_t bytes = 256;
   size_t off_d0 = 256, off_d1 = 0, off_d2 = 0;
   if (esz <= 4) {
-    bytes += round256((size_t)grid * 8);
+    bytes += round256((size_t)ndesc * 8 * (size_t)acc::tune("scan.desc_stride", 1));
   } else {
-    off_d1 = off_d0 + round256((size_t)grid * 4);
-    off_d2 = off_d1 + round256((size_t)grid * esz);
-    bytes = off_d2 + round256((size_t)grid * esz);
+    off_d1 = off_d0 + round256((size_t)ndesc * 4);
+    off_d2 = off_d1 + round256((size_t)ndesc * esz);
+    bytes = off_d2 + round256((size_t)ndesc * esz);
   }
   int blk = -1;
   ACC_TRY(s->ctx->scratch_acquire(bytes, st, acc::SCRATCH_SCAN, &blk));
@@ -267,7 +273,7 @@ int acc_exec_scan(acc_skel s, const acc_array *env, int64_t n, const acc_array *
     }
     epoch = ++b.epoch;
     counter_base = b.counter_base;
-    b.counter_base += static_cast<uint32_t>(grid);    // every launched block draws exactly one ticket
+    b.counter_base += static_cast<uint32_t>(draws);
   }
   args.ptr(reinterpret_cast<uint64_t>(base));
   args.u32(counter_base);
@@ -276,7 +282,7 @@ int acc_exec_scan(acc_skel s, const acc_array *env, int64_t n, const acc_array *
   args.ptr(reinterpret_cast<uint64_t>(base + off_d2));
   args.u32(epoch);
   args.i64(tiles);
-  const int rc = launch(s, aligned ? 0 : 1, grid, 0, st, &args);
+  const int rc = launch(s, v, grid, 0, st, &args);
   if (rc != ACC_OK) {
     // nothing ran: take the tickets back so that the block stays consistent
     std::lock_guard<std::mutex> lock(s->ctx->mu);

@@ -171,6 +171,9 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       *entry = std::string("scan") + (right ? "r" : "l") + (sp.has_seed ? "" : "1");
       o << "#define ACC_SCAN_RIGHT " << (right ? 1 : 0) << "\n#define ACC_SCAN_MODE " << mode << "\n";
       o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_ROWS " << sp.rows << "\n";
+      o << "#define ACC_LOOKBACK " << tune("scan.lookback", 1) << "\n";
+      o << "#define ACC_DESC_STRIDE " << tune("scan.desc_stride", 1) << "\n";
+      if (tune("scan.debug_nolookback", 0)) o << "#define ACC_SCAN_DEBUG_NO_LOOKBACK 1\n";
       tmpl = "skel_scan.h";
       break;
     }
