@@ -16,9 +16,8 @@
  *     global memory.  A tile first publishes its own total (state AGGREGATE),
  *     then one wave walks back over its predecessors, 64 descriptors per step,
  *     until it meets an inclusive PREFIX, and finally publishes its own PREFIX.
- *     Tile numbers are handed out by an atomic counter to a resident grid of
- *     persistent workgroups, so every predecessor of a tile being worked on
- *     is itself held by a running workgroup and the walk cannot deadlock.
+ *     Every predecessor of a tile that is being worked on is itself held by a
+ *     running workgroup (see the kernel), so the walk cannot deadlock.
  *   - descriptors are tagged with a launch epoch and the counter is used
  *     relative to a base, so nothing needs clearing between launches.
  *
@@ -120,9 +119,29 @@ template <typename T> struct acc_sv<T, true> {
  * predecessors in one memory round trip.  The chain of tiles can advance by
  * at most one such window per round trip, so the window has to be wide
  * enough for the rate at which tiles retire.                                */
+/* first window of the walk: only issues the loads, so that the caller can put
+ * other memory traffic behind them before their results are needed          */
+template <typename T>
+struct acc_scan_window {
+  T v[ACC_LOOKBACK];
+  unsigned int fl[ACC_LOOKBACK];
+};
+
+template <typename T>
+ACC_DEV void acc_scan_window_load(const acc_scan_desc<T> &desc, const Int64 look, const int lane, acc_scan_window<T> &w)
+{
+#pragma unroll
+  for (int j = 0; j < ACC_LOOKBACK; ++j) {
+    const Int64 idx = look - (lane * ACC_LOOKBACK + j);
+    w.v[j] = T();
+    w.fl[j] = 0;
+    if (idx >= 0) w.fl[j] = desc.get(idx, w.v[j]);
+  }
+}
+
 template <typename T, typename Op>
 ACC_DEV T acc_scan_lookback(const acc_scan_desc<T> &desc, Int64 tile, const T &block_total, Op op,
-                            unsigned int epoch, int lane)
+                            unsigned int epoch, int lane, acc_scan_window<T> &w)
 {
   /* slots are ordered nearest predecessor first, so a reduction in slot order
    * must combine (later, earlier) */
@@ -130,34 +149,26 @@ ACC_DEV T acc_scan_lookback(const acc_scan_desc<T> &desc, Int64 tile, const T &b
   acc_opt<T> run = acc_none<T>();
 
   for (Int64 look = tile - 1;; look -= ACC_WAVE * ACC_LOOKBACK) {
-    T v[ACC_LOOKBACK];
-    unsigned int fl[ACC_LOOKBACK];
-    Int64 idx[ACC_LOOKBACK];
-#pragma unroll
-    for (int j = 0; j < ACC_LOOKBACK; ++j) {            /* all loads in flight together */
-      idx[j] = look - (lane * ACC_LOOKBACK + j);
-      v[j] = T();
-      fl[j] = 0;
-      if (idx[j] >= 0) fl[j] = desc.get(idx[j], v[j]);
-    }
+    if (look != tile - 1) acc_scan_window_load(desc, look, lane, w);
     int nearest = ACC_WAVE * ACC_LOOKBACK;              /* slot of the nearest PREFIX, if any */
 #pragma unroll
     for (int j = 0; j < ACC_LOOKBACK; ++j) {
-      if (idx[j] >= 0) {
-        while ((fl[j] >> 2) != epoch) {
+      const Int64 idx = look - (lane * ACC_LOOKBACK + j);
+      if (idx >= 0) {
+        while ((w.fl[j] >> 2) != epoch) {
           __builtin_amdgcn_s_sleep(1);
-          fl[j] = desc.get(idx[j], v[j]);
+          w.fl[j] = desc.get(idx, w.v[j]);
         }
       }
-      const unsigned long long m = __ballot(idx[j] >= 0 && (fl[j] & 3u) == ACC_ST_PREFIX);
+      const unsigned long long m = __ballot(idx >= 0 && (w.fl[j] & 3u) == ACC_ST_PREFIX);
       if (m) nearest = acc_min(nearest, (__ffsll((long long)m) - 1) * ACC_LOOKBACK + j);
     }
     acc_opt<T> c = acc_none<T>();
 #pragma unroll
     for (int j = 0; j < ACC_LOOKBACK; ++j) {
       acc_opt<T> e;
-      e.v = v[j];
-      e.ok = (idx[j] >= 0) && (lane * ACC_LOOKBACK + j <= nearest);
+      e.v = w.v[j];
+      e.ok = (look - (lane * ACC_LOOKBACK + j) >= 0) && (lane * ACC_LOOKBACK + j <= nearest);
       c = back(c, e);
     }
     run = back(run, acc_wave_reduce(c, back));
@@ -268,12 +279,14 @@ ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op_raw, const T s
     prefetch();
   } else {
     if (threadIdx.x == 0) desc.put(tile, (epoch << 2) | ACC_ST_AGGREGATE, S::val(block_total));
+    acc_scan_window<T> win;
+    if (wave == 0) acc_scan_window_load(desc, tile - 1, lane, win);   /* ahead of the prefetch: results return in issue order */
     prefetch();
     if (wave == 0) {
 #ifdef ACC_SCAN_DEBUG_NO_LOOKBACK
       const T p = S::val(block_total);
 #else
-      const T p = acc_scan_lookback(desc, tile, S::val(block_total), op_raw, epoch, lane);
+      const T p = acc_scan_lookback(desc, tile, S::val(block_total), op_raw, epoch, lane, win);
 #endif
       if (lane == 0) *s_prefix = p;
     }
@@ -325,11 +338,117 @@ ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op_raw, const T s
   }
 }
 
-/* The kernel is persistent: a resident grid of workgroups draws tile numbers
- * from an atomic counter until they run out.  The ticket of the tile after
- * next is requested while the current tile is being scanned, and the next
- * tile's elements are loaded while the current tile waits for its prefix, so
- * neither the ticket nor the look-back leaves the memory system idle.        */
+/* The one ragged tile of a scan (elements past the end are transparent).  It
+ * does the same job as acc_scan_tile<true> but keeps almost nothing live:
+ * the per-row scans are simply done twice, once to get the totals and once,
+ * when the prefix is known, to produce the results.  Speed is irrelevant
+ * here (at most one such tile per launch); what matters is that its register
+ * footprint does not dictate the kernel's.                                   */
+template <typename T, typename Op, typename Prefetch>
+ACC_DEV void acc_scan_tile_ragged(const T (&x)[ACC_ROWS][ACC_VEC], Op op_raw, const T seed, const Int64 tile,
+                                  const Int64 base, const Int64 n, T *__restrict__ out, T *__restrict__ sum,
+                                  const acc_scan_desc<T> &desc, const unsigned int epoch, void *s_wave_raw,
+                                  T *s_prefix, Prefetch prefetch)
+{
+  typedef acc_opt<T> V;
+  auto op = acc_lift<T>(op_raw);
+  const int lane = acc_lane();
+  const int wave = (int)(threadIdx.x >> 6);
+  V *s_wave = (V *)s_wave_raw;
+
+  auto item = [&](const int r, const int k) -> V {
+    const Int64 i0 = acc_scan_ix0(base, wave, lane, r);
+    const Int64 ix = ACC_SCAN_RIGHT ? i0 - k : i0 + k;
+    V v;
+    v.v = x[r][k];
+    v.ok = (ix < n);
+    return v;
+  };
+  auto lane_total = [&](const int r) -> V {
+    V t = item(r, 0);
+#pragma unroll
+    for (int k = 1; k < ACC_VEC; ++k) t = op(t, item(r, k));
+    return t;
+  };
+
+  /* pass 1: total of this wave */
+  V wave_total = acc_none<T>();
+#pragma unroll 1
+  for (int r = 0; r < ACC_ROWS; ++r) {
+    const V ci = acc_wave_scan(lane_total(r), op, lane);
+    wave_total = op(wave_total, acc_readlane(ci, ACC_WAVE - 1));
+  }
+  if (lane == 0) s_wave[wave] = wave_total;
+  __syncthreads();
+  V wavepre = acc_none<T>();
+  V block_total = acc_none<T>();
+#pragma unroll 1
+  for (int w = 0; w < ACC_WAVES; ++w) {
+    if (w == wave) wavepre = block_total;
+    block_total = op(block_total, s_wave[w]);
+  }
+
+  T prefix = seed;
+  bool has_prefix = ACC_HAS_SEED;
+  if (tile == 0) {
+    if (threadIdx.x == 0)
+      desc.put(0, (epoch << 2) | ACC_ST_PREFIX, ACC_HAS_SEED ? op_raw(seed, block_total.v) : block_total.v);
+    prefetch();
+  } else {
+    if (threadIdx.x == 0) desc.put(tile, (epoch << 2) | ACC_ST_AGGREGATE, block_total.v);
+    acc_scan_window<T> win;
+    if (wave == 0) acc_scan_window_load(desc, tile - 1, lane, win);
+    prefetch();
+    if (wave == 0) {
+      const T p = acc_scan_lookback(desc, tile, block_total.v, op_raw, epoch, lane, win);
+      if (lane == 0) *s_prefix = p;
+    }
+    __syncthreads();
+    prefix = *s_prefix;
+    has_prefix = true;
+  }
+
+  /* pass 2: redo the row scans, now with everything before them known */
+  V run;                                      /* everything before the current row */
+  run.v = prefix;
+  run.ok = has_prefix;
+  run = op(run, wavepre);
+  const Int64 last = ACC_SCAN_RIGHT ? 0 : n - 1;
+#pragma unroll 1
+  for (int r = 0; r < ACC_ROWS; ++r) {
+    const V ci = acc_wave_scan(lane_total(r), op, lane);
+    V e = acc_wave_shift_up1(ci);
+    if (lane == 0) e = acc_none<T>();
+    V acc = op(run, e);                       /* everything before this lane's first item */
+    const Int64 i0 = acc_scan_ix0(base, wave, lane, r);
+#pragma unroll
+    for (int k = 0; k < ACC_VEC; ++k) {
+      const Int64 ix = ACC_SCAN_RIGHT ? i0 - k : i0 + k;
+      const V before = acc;
+      acc = op(acc, item(r, k));
+      if (ix < n) {
+        const bool exclusive = (ACC_SCAN_MODE == 0 || ACC_SCAN_MODE == 2);
+        out[ix] = exclusive ? before.v : acc.v;
+        if (ix == last) {
+          if (ACC_SCAN_MODE == 0) out[n] = acc.v;
+          if (ACC_SCAN_MODE == 2) sum[0] = acc.v;
+        }
+      }
+    }
+    run = op(run, acc_readlane(ci, ACC_WAVE - 1));
+  }
+}
+
+/* Two ways of handing tiles to workgroups:
+ *
+ * ACC_SCAN_PERSISTENT == 0  one workgroup per tile, tile number = workgroup
+ *   number.  Workgroups are dispatched in increasing order, so every
+ *   predecessor of a running tile has itself been dispatched and the look-back
+ *   always makes progress.
+ * ACC_SCAN_PERSISTENT == 1  a resident grid of workgroups draws tile numbers
+ *   from an atomic counter (two tiles ahead, so the atomic's round trip is
+ *   never waited for) and loads the next tile's elements while the current
+ *   tile waits for its prefix.                                              */
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 ACC_ENTRY(ACC_ENV_PARAMS
           const Int64 shOut_0, ACC_ELT *__restrict__ arrOut_0,
@@ -346,7 +465,6 @@ ACC_ENTRY(ACC_ENV_PARAMS
 #endif
   (void)shOut_0;
 
-  __shared__ unsigned int s_ticket[2];
   __shared__ T s_prefix;
   __shared__ acc_opt<T> s_wave[ACC_WAVES];
 
@@ -365,9 +483,19 @@ ACC_ENTRY(ACC_ENV_PARAMS
   const acc_scan_desc<T> desc(desc0, desc1, desc2);
   auto tile_base = [&](const Int64 t) -> Int64 { return (ACC_SCAN_RIGHT ? (num_tiles - 1 - t) : t) * (Int64)ACC_TILE; };
 
-  if (threadIdx.x == 0) s_ticket[0] = atomicAdd(tile_counter, 1u) - counter_base;
+#if ACC_SCAN_PERSISTENT
+  __shared__ unsigned int s_ticket[4];
+  unsigned int pending = 0;
+  if (threadIdx.x == 0) {
+    s_ticket[0] = atomicAdd(tile_counter, 1u) - counter_base;
+    pending = atomicAdd(tile_counter, 1u);
+  }
   __syncthreads();
   Int64 tile = (Int64)s_ticket[0];
+#else
+  (void)tile_counter; (void)counter_base;
+  Int64 tile = (Int64)blockIdx.x;
+#endif
 
   if (n <= 0) {                                   /* PrefixSum.hs:249-251,330-334: scan of nothing is [seed] */
     if (threadIdx.x == 0 && tile == 0) {
@@ -378,32 +506,43 @@ ACC_ENTRY(ACC_ENV_PARAMS
   }
   if (ACC_SCAN_MODE == 3 && tile == 0 && threadIdx.x == 0) arrOut_0[n] = seed;
 
-  T cur[ACC_ROWS][ACC_VEC], nxt[ACC_ROWS][ACC_VEC];
+  T cur[ACC_ROWS][ACC_VEC];
   if (tile < num_tiles) acc_scan_load(get, tile_base(tile), n, cur, wave, lane);
 
-  int parity = 1;
+#if ACC_SCAN_PERSISTENT
+  T nxt[ACC_ROWS][ACC_VEC];
+  int slot = 1;
   while (tile < num_tiles) {
-    /* ticket for the tile after this one; it is read after the next barrier */
-    if (threadIdx.x == 0) s_ticket[parity] = atomicAdd(tile_counter, 1u) - counter_base;
-
+    /* hand over the ticket drawn one tile ago (read after the next barrier)
+     * and draw another */
+    if (threadIdx.x == 0) {
+      s_ticket[slot] = pending - counter_base;
+      pending = atomicAdd(tile_counter, 1u);
+    }
     Int64 next = num_tiles;
     auto prefetch = [&]() {
-      next = (Int64)s_ticket[parity];
+      next = (Int64)s_ticket[slot];
       if (next < num_tiles) acc_scan_load(get, tile_base(next), n, nxt, wave, lane);
     };
+#else
+  if (tile < num_tiles) {
+    auto prefetch = [&]() {};
+#endif
 
     const Int64 base = tile_base(tile);
     if (base + ACC_TILE <= n)
       acc_scan_tile<false, T>(cur, op, seed, tile, base, n, arrOut_0, arrSum_0, desc, epoch, (void *)s_wave, &s_prefix, prefetch);
     else
-      acc_scan_tile<true, T>(cur, op, seed, tile, base, n, arrOut_0, arrSum_0, desc, epoch, (void *)s_wave, &s_prefix, prefetch);
+      acc_scan_tile_ragged<T>(cur, op, seed, tile, base, n, arrOut_0, arrSum_0, desc, epoch, (void *)s_wave, &s_prefix, prefetch);
 
+#if ACC_SCAN_PERSISTENT
 #pragma unroll
     for (int r = 0; r < ACC_ROWS; ++r)
 #pragma unroll
       for (int k = 0; k < ACC_VEC; ++k) cur[r][k] = nxt[r][k];
     tile = next;
-    parity ^= 1;
+    slot = (slot + 1) & 3;
     __syncthreads();          /* s_wave and s_prefix are free for the next tile */
+#endif
   }
 }

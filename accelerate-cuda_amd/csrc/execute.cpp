@@ -8,6 +8,7 @@
 // compute units and single-pass kernels (one launch where the reference needs
 // two or three).
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <deque>
 
@@ -242,16 +243,20 @@ int acc_exec_scan(acc_skel s, const acc_array *env, int64_t n, const acc_array *
   ACC_TRY(s->ensure_variant(v));
   const int64_t tile = s->elements_per_block();
   const int64_t tiles = (n + tile - 1) / tile;
-  // a resident grid of persistent workgroups; each draws tiles until none are left
-  const int64_t per_cu = std::max(1, std::min(s->variants[v].blocks_per_cu, acc::tune("scan.blocks_per_cu", 2)));
-  const int64_t grid = std::max<int64_t>(1, std::min<int64_t>(tiles, (int64_t)s->ctx->props.multiProcessorCount * per_cu));
-  const int64_t draws = tiles + grid;             // every tile once, plus the draw that tells a workgroup to stop
+  int64_t grid = std::max<int64_t>(1, tiles);     // one workgroup per tile, in dispatch order ...
+  int64_t draws = 0;
+  if (acc::tune("scan.persistent", 0)) {
+    // ... or a resident grid of persistent workgroups, each drawing tiles until none are left
+    const int64_t per_cu = std::max(1, std::min(s->variants[v].blocks_per_cu, acc::tune("scan.blocks_per_cu", 2)));
+    grid = std::max<int64_t>(1, std::min<int64_t>(tiles, (int64_t)s->ctx->props.multiProcessorCount * per_cu));
+    draws = tiles + 2 * grid;                     // every tile once, plus two draws ahead per workgroup
+  }
   const int64_t ndesc = std::max<int64_t>(1, tiles);
   const size_t esz = s->spec.elt_size;
   size_t bytes = 256;
   size_t off_d0 = 256, off_d1 = 0, off_d2 = 0;
   if (esz <= 4) {
-    bytes += round256((size_t)ndesc * 8 * (size_t)acc::tune("scan.desc_stride", 1));
+    bytes += round256((size_t)ndesc * 8 * (size_t)acc::tune("scan.desc_stride", 16));
   } else {
     off_d1 = off_d0 + round256((size_t)ndesc * 4);
     off_d2 = off_d1 + round256((size_t)ndesc * esz);

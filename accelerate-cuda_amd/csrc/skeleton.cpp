@@ -172,8 +172,9 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "#define ACC_SCAN_RIGHT " << (right ? 1 : 0) << "\n#define ACC_SCAN_MODE " << mode << "\n";
       o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_ROWS " << sp.rows << "\n";
       o << "#define ACC_LOOKBACK " << tune("scan.lookback", 1) << "\n";
-      o << "#define ACC_DESC_STRIDE " << tune("scan.desc_stride", 1) << "\n";
+      o << "#define ACC_DESC_STRIDE " << tune("scan.desc_stride", 16) << "\n";
       if (tune("scan.debug_nolookback", 0)) o << "#define ACC_SCAN_DEBUG_NO_LOOKBACK 1\n";
+      o << "#define ACC_SCAN_PERSISTENT " << (tune("scan.persistent", 0) ? 1 : 0) << "\n";
       tmpl = "skel_scan.h";
       break;
     }
@@ -326,8 +327,8 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
       break;
     }
     default:   // scans
-      sp->block = tune("scan.block", 256);
-      sp->rows = tune("scan.rows", 4);
+      sp->block = tune("scan.block", 1024);
+      sp->rows = tune("scan.rows", 8);
       break;
   }
   if (sp->block < 64 || sp->block > 1024 || (sp->block & 63)) return fail(ACC_ERR_INVALID, "block size %d is not a multiple of the 64-lane wavefront", sp->block);
