@@ -57,6 +57,7 @@ struct ScratchBlock {
   hipStream_t stream = nullptr;
   hipEvent_t done = nullptr;
   bool busy = false;
+  bool recorded = false;   // `done` was recorded at the last release
   uint32_t epoch = 0;
   uint32_t counter_base = 0;
 };
@@ -69,6 +70,12 @@ struct acc_context_s {
   std::string arch;          // "gfx950"
   std::mutex mu;
   std::vector<acc::ScratchBlock> scratch;
+  // Completion events are only needed to hand a block from one stream to
+  // another.  While a single stream has used the pool, stream order alone
+  // makes reuse safe and no events are recorded.
+  bool scratch_any_stream = false;
+  bool scratch_multi_stream = false;
+  hipStream_t scratch_first_stream = nullptr;
 
   int make_current() const;
   // zero-initialised when first allocated; contents persist between uses and

@@ -7,16 +7,20 @@
  * plus a recursive second one, Execute.hs:291-318) and :221-367 (mkFoldDim),
  * and of the shared-memory tree reducers at :616-699.
  *
- * foldAll is ONE launch: every block strides over tiles of the (fused) input,
- * each lane reading ACC_UNROLL independent groups of ACC_VEC consecutive
- * elements per tile; lanes are combined with a wave64 DPP reduction, waves
- * through a few words of LDS, blocks through one slot each in global memory;
- * the block that arrives last (atomic ticket) combines the slots, applies the
- * seed and resets the ticket.  As in the reference the operator must be
- * associative AND commutative here (the striding reorders elements,
- * Reduction.hs:160-165), it needs no identity, the seed enters once as the
- * second operand (Reduction.hs:203-211) and an empty input yields the seed
- * (:212-214).
+ * foldAll: every block strides over tiles of the (fused) input, each lane
+ * reading ACC_UNROLL independent groups of ACC_VEC consecutive elements per
+ * tile; lanes are combined with a wave64 DPP reduction, waves through a few
+ * words of LDS, and each block leaves one partial result in global memory.  A
+ * second, single-block launch of <entry>_finish combines the partials and
+ * applies the seed (a lone block does so itself and the second launch is
+ * skipped).  Blocks never meet on an atomic: same-address device-scope
+ * atomics cost tens of nanoseconds each on this part, far more than a
+ * back-to-back launch; and with a fixed grid the association order, hence
+ * the Float32 result, is reproducible from run to run.  As in the reference
+ * the operator must be associative AND commutative here (the striding
+ * reorders elements, Reduction.hs:160-165), it needs no identity, the seed
+ * enters once as the second operand (Reduction.hs:203-211) and an empty input
+ * yields the seed (:212-214).
  *
  * Generated definitions expected: ACC_ENTRY, ACC_ELT, ACC_ENV_PARAMS,
  * ACC_ENV_ASSUME, ACC_GET(ix), ACC_COMBINE(x,y), ACC_HAS_SEED, ACC_SEED,
@@ -49,12 +53,11 @@ extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 ACC_ENTRY(ACC_ENV_PARAMS
           ACC_ELT *__restrict__ arrOut_0,
           const Int64 shIn_0,
-          ACC_ELT *partials, unsigned int *ticket)
+          ACC_ELT *__restrict__ partials)
 {
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
   __shared__ acc_opt<T> s_wave[ACC_WAVES];
-  __shared__ int s_last;
 
   auto get = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
   auto f   = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
@@ -113,31 +116,43 @@ ACC_ENTRY(ACC_ENV_PARAMS
 
   acc_opt<T> total = acc_block_reduce(mine, f, s_wave);
 
-  /* hand over to the last block */
+  if (threadIdx.x != 0) return;
   if (gridDim.x > 1) {
-    if (threadIdx.x == 0) {
-      partials[blockIdx.x] = total.v;            /* host guarantees every block owns >= 1 element */
-      __threadfence();
-      const unsigned int prev = atomicAdd(ticket, 1u);
-      s_last = (prev == gridDim.x - 1);
-    }
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();
-    acc_opt<T> p = acc_none<T>();
-    for (unsigned int i = threadIdx.x; i < gridDim.x; i += ACC_BLOCK) p = lf(p, acc_some(partials[i]));
-    total = acc_block_reduce(p, f, s_wave);
-    if (threadIdx.x == 0) *ticket = 0u;
+    partials[blockIdx.x] = total.v;              /* the host guarantees every block owns >= 1 element */
+    return;
   }
-
-  if (threadIdx.x == 0) {
 #if ACC_HAS_SEED
-    const T seed = (ACC_SEED);
-    arrOut_0[0] = total.ok ? f(total.v, seed) : seed;
+  const T seed = (ACC_SEED);
+  arrOut_0[0] = total.ok ? f(total.v, seed) : seed;
 #else
-    arrOut_0[0] = total.v;
+  arrOut_0[0] = total.v;
 #endif
-  }
+}
+
+#define ACC_CAT2(a, b) a##b
+#define ACC_CAT(a, b) ACC_CAT2(a, b)
+
+/* second launch: one block folds the `count` partial results */
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+ACC_CAT(ACC_ENTRY, _finish)(ACC_ENV_PARAMS
+                            ACC_ELT *__restrict__ arrOut_0,
+                            const ACC_ELT *__restrict__ partials, const Int64 count)
+{
+  typedef ACC_ELT T;
+  ACC_ENV_ASSUME
+  __shared__ acc_opt<T> s_wave[ACC_WAVES];
+  auto f  = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
+  auto lf = acc_lift<T>(f);
+  acc_opt<T> p = acc_none<T>();
+  for (Int64 i = threadIdx.x; i < count; i += ACC_BLOCK) p = lf(p, acc_some(partials[i]));
+  const acc_opt<T> total = acc_block_reduce(p, f, s_wave);
+  if (threadIdx.x != 0) return;
+#if ACC_HAS_SEED
+  const T seed = (ACC_SEED);
+  arrOut_0[0] = total.ok ? f(total.v, seed) : seed;
+#else
+  arrOut_0[0] = total.v;
+#endif
 }
 
 #else  /* ACC_FOLD_DIM: one wave per innermost row ----------------------------- */

@@ -12,12 +12,17 @@
  *     max, and, or, xor) is issued as one atomic; anything else is a
  *     compare-and-swap loop on the element's bits -- no locks either way;
  *   - target indices [0, lds_bins) are privatised in LDS: updates to them are
- *     LDS atomics and reach global memory once per block, at the end, so hot
- *     targets (a 256-bin histogram, the head of a skewed one) do not queue up
- *     on one memory-side atomic unit.  A target that fits entirely gets
- *     `lds_copies` replicas, one per group of waves, to thin out same-address
- *     collisions inside a block.  Privatisation needs an identity for the
- *     combine, so it is only used with a hint.
+ *     LDS atomics and leave the block once, at the end, so hot targets (a
+ *     256-bin histogram, the head of a skewed one) do not queue up on one
+ *     memory-side atomic unit.  A target that fits entirely gets `lds_copies`
+ *     replicas, one per group of waves, to thin out same-address collisions
+ *     inside a block.  Privatisation needs an identity for the combine, so it
+ *     is only used with a hint.
+ *   - the privatised part leaves a block either as one global atomic per
+ *     touched target (few blocks x few bins), or -- when that would again be
+ *     millions of atomics, a thousand to the same address -- as a plain dump of
+ *     the block's bins into a table that a second kernel, permute_merge, folds
+ *     column by column into the result.
  * The new value is the FIRST operand of combine (IndexSpace.hs:207).  Updates
  * arrive in no particular order, as in the reference, so combine must be
  * associative and commutative.  Targets outside the result are dropped.
@@ -61,38 +66,57 @@ ACC_DEV T acc_hint_identity()
 #endif
 }
 
-/* one atomic application of the hinted operator; P is a global or LDS pointer */
-template <typename T, typename F>
+/* one atomic application of the hinted operator at the given scope.  LDS and
+ * a block's private table only need workgroup scope (the atomic is performed
+ * in LDS, or in this compute die's L2); the shared result needs device scope,
+ * which on this part is performed at the memory side and is far slower.      */
+template <int SCOPE, typename T, typename F>
 ACC_DEV void acc_hint_apply(T *p, const T &x, F combine)
 {
 #if ACC_ELT_IS_INTEGER && ACC_COMBINE_HINT != ACC_HINT_GENERIC
-  typedef typename acc_bits<sizeof(T)>::type U;
   (void)combine;
 #if ACC_COMBINE_HINT == ACC_HINT_ADD
-  atomicAdd((U *)p, (U)x);
+  (void)__hip_atomic_fetch_add(p, x, __ATOMIC_RELAXED, SCOPE);
 #elif ACC_COMBINE_HINT == ACC_HINT_AND
-  atomicAnd((U *)p, (U)x);
+  (void)__hip_atomic_fetch_and(p, x, __ATOMIC_RELAXED, SCOPE);
 #elif ACC_COMBINE_HINT == ACC_HINT_OR
-  atomicOr((U *)p, (U)x);
+  (void)__hip_atomic_fetch_or(p, x, __ATOMIC_RELAXED, SCOPE);
 #elif ACC_COMBINE_HINT == ACC_HINT_XOR
-  atomicXor((U *)p, (U)x);
+  (void)__hip_atomic_fetch_xor(p, x, __ATOMIC_RELAXED, SCOPE);
 #elif ACC_COMBINE_HINT == ACC_HINT_MIN
-  if (T(-1) < T(0)) { if (sizeof(T) == 4) atomicMin((int *)p, (int)x); else atomicMin((long long *)p, (long long)x); }
-  else atomicMin((U *)p, (U)x);
+  (void)__hip_atomic_fetch_min(p, x, __ATOMIC_RELAXED, SCOPE);
 #elif ACC_COMBINE_HINT == ACC_HINT_MAX
-  if (T(-1) < T(0)) { if (sizeof(T) == 4) atomicMax((int *)p, (int)x); else atomicMax((long long *)p, (long long)x); }
-  else atomicMax((U *)p, (U)x);
+  (void)__hip_atomic_fetch_max(p, x, __ATOMIC_RELAXED, SCOPE);
 #endif
 #elif !ACC_ELT_IS_INTEGER && ACC_COMBINE_HINT == ACC_HINT_ADD
   (void)combine;
-  atomicAdd(p, x);
+  (void)__hip_atomic_fetch_add(p, x, __ATOMIC_RELAXED, SCOPE);
 #else
-  acc_atomic_rmw(p, x, combine);
+  /* compare-and-swap on the bit pattern (cubits/accelerate_cuda_function.h:28-114) */
+  typedef typename acc_bits<sizeof(T)>::type B;
+  B *q = (B *)p;
+  B old = __hip_atomic_load(q, __ATOMIC_RELAXED, SCOPE);
+  for (;;) {
+    T cur, nxt;
+    __builtin_memcpy(&cur, &old, sizeof(T));
+    nxt = combine(x, cur);
+    B nb;
+    __builtin_memcpy(&nb, &nxt, sizeof(T));
+    if (__hip_atomic_compare_exchange_strong(q, &old, nb, __ATOMIC_RELAXED, __ATOMIC_RELAXED, SCOPE)) break;
+  }
 #endif
 }
 
+#define ACC_SCOPE_BLOCK  __HIP_MEMORY_SCOPE_WORKGROUP
+#define ACC_SCOPE_DEVICE __HIP_MEMORY_SCOPE_AGENT
+
+/* dump == NULL            : privatised bins are flushed into the result with atomics
+ * dump, cols == lds_bins  : privatised bins are dumped to row blockIdx.x of the table
+ * dump, cols == target    : additionally the targets beyond the LDS window are
+ *                           privatised in the rest of this block's table row   */
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
-permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, const int lds_copies)
+permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, const int lds_copies,
+        ACC_ELT *__restrict__ dump, const int dump_cols)
 {
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
@@ -106,56 +130,112 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
   const Int64 n = shIn_0;
   const Int64 ntarget = (ACC_OUT_SIZE);
   const T ident = acc_hint_identity<T>();
+  T *row = dump ? dump + (Int64)blockIdx.x * dump_cols : (T *)0;
+  const bool private_tail = dump && dump_cols > lds_bins;
 
   for (int i = threadIdx.x; i < lds_bins * lds_copies; i += ACC_BLOCK) bins[i] = ident;
+  if (private_tail)
+    for (int i = lds_bins + threadIdx.x; i < dump_cols; i += ACC_BLOCK) row[i] = ident;
   __syncthreads();
   T *mine = bins + ((threadIdx.x >> 6) % lds_copies) * lds_bins;
 
   auto update = [&](const Int64 j, const T &x) {
     if (j < 0 || j >= ntarget) return;            /* `ignore`, or outside the result */
-    if (j < lds_bins) acc_hint_apply(mine + j, x, f);
-    else              acc_hint_apply(arrOut_0 + j, x, f);
+    if (j < lds_bins)      acc_hint_apply<ACC_SCOPE_BLOCK>(mine + j, x, f);
+    else if (private_tail) acc_hint_apply<ACC_SCOPE_BLOCK>(row + j, x, f);
+    else                   acc_hint_apply<ACC_SCOPE_DEVICE>(arrOut_0 + j, x, f);
   };
 
-  const Int64 num_tiles = (n + ACC_TILE - 1) / ACC_TILE;
-  for (Int64 tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {
+  /* full tiles, software-pipelined: the next tile's indices and values are
+   * requested before the current tile's updates are issued, so the atomics'
+   * latency is spent under loads already in flight */
+  const Int64 full_tiles = n / ACC_TILE;
+  Int64 j[ACC_UNROLL][ACC_VEC], jn[ACC_UNROLL][ACC_VEC];
+  T x[ACC_UNROLL][ACC_VEC], xn[ACC_UNROLL][ACC_VEC];
+  auto load = [&](const Int64 tile, Int64 (&jj)[ACC_UNROLL][ACC_VEC], T (&xx)[ACC_UNROLL][ACC_VEC]) {
     const Int64 base = tile * (Int64)ACC_TILE + (Int64)threadIdx.x * ACC_VEC;
-    if ((tile + 1) * (Int64)ACC_TILE <= n) {
-      Int64 j[ACC_UNROLL][ACC_VEC];
-      T x[ACC_UNROLL][ACC_VEC];
 #pragma unroll
-      for (int u = 0; u < ACC_UNROLL; ++u)
+    for (int u = 0; u < ACC_UNROLL; ++u)
 #pragma unroll
-        for (int k = 0; k < ACC_VEC; ++k) {
-          const Int64 ix = base + u * (ACC_BLOCK * ACC_VEC) + k;
-          j[u][k] = perm(ix);
-          x[u][k] = get(ix);
-        }
+      for (int k = 0; k < ACC_VEC; ++k) {
+        const Int64 ix = base + u * (ACC_BLOCK * ACC_VEC) + k;
+        jj[u][k] = perm(ix);
+        xx[u][k] = get(ix);
+      }
+  };
+  Int64 tile = blockIdx.x;
+  if (tile < full_tiles) load(tile, j, x);
+  while (tile < full_tiles) {
+    const Int64 next = tile + gridDim.x;
+    if (next < full_tiles) load(next, jn, xn);
 #pragma unroll
-      for (int u = 0; u < ACC_UNROLL; ++u)
+    for (int u = 0; u < ACC_UNROLL; ++u)
 #pragma unroll
-        for (int k = 0; k < ACC_VEC; ++k) update(j[u][k], x[u][k]);
-    } else {
+      for (int k = 0; k < ACC_VEC; ++k) update(j[u][k], x[u][k]);
 #pragma unroll
-      for (int u = 0; u < ACC_UNROLL; ++u)
+    for (int u = 0; u < ACC_UNROLL; ++u)
 #pragma unroll
-        for (int k = 0; k < ACC_VEC; ++k) {
-          const Int64 ix = base + u * (ACC_BLOCK * ACC_VEC) + k;
-          if (ix < n) update(perm(ix), get(ix));
-        }
-    }
+      for (int k = 0; k < ACC_VEC; ++k) { j[u][k] = jn[u][k]; x[u][k] = xn[u][k]; }
+    tile = next;
   }
 
-  /* flush the privatised part: one global atomic per touched target */
+  /* the ragged last tile, taken by whichever block it falls to */
+  if (full_tiles * (Int64)ACC_TILE < n && (Int64)blockIdx.x == full_tiles % gridDim.x) {
+    const Int64 base = full_tiles * (Int64)ACC_TILE + (Int64)threadIdx.x * ACC_VEC;
+#pragma unroll
+    for (int u = 0; u < ACC_UNROLL; ++u)
+#pragma unroll
+      for (int k = 0; k < ACC_VEC; ++k) {
+        const Int64 ix = base + u * (ACC_BLOCK * ACC_VEC) + k;
+        if (ix < n) update(perm(ix), get(ix));
+      }
+  }
+
+  /* the privatised part leaves the block */
   if (lds_bins > 0) {
     __syncthreads();
     for (int i = threadIdx.x; i < lds_bins; i += ACC_BLOCK) {
       T acc = bins[i];
       for (int c = 1; c < lds_copies; ++c) acc = f(bins[c * lds_bins + i], acc);
-      typename acc_bits<sizeof(T)>::type a, b;
-      __builtin_memcpy(&a, &acc, sizeof(T));
-      __builtin_memcpy(&b, &ident, sizeof(T));
-      if (a != b) acc_hint_apply(arrOut_0 + i, acc, f);
+      if (row) {
+        row[i] = acc;
+      } else {
+        typename acc_bits<sizeof(T)>::type a, b;
+        __builtin_memcpy(&a, &acc, sizeof(T));
+        __builtin_memcpy(&b, &ident, sizeof(T));
+        if (a != b) acc_hint_apply<ACC_SCOPE_DEVICE>(arrOut_0 + i, acc, f);
+      }
     }
+  }
+}
+
+/* folds the table dump[nblocks][cols] into out[0 .. cols).  The rows are split
+ * into `slices` groups handled by different workgroups; with one slice the
+ * result is written plainly, otherwise each group applies its share with one
+ * atomic per target.                                                         */
+extern "C" __global__ void __launch_bounds__(256)
+permute_merge(ACC_ENV_PARAMS ACC_OUT_PARAMS, const ACC_ELT *__restrict__ dump, const int cols, const int nblocks,
+              const int slices)
+{
+  typedef ACC_ELT T;
+  ACC_ENV_ASSUME
+  auto f = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
+  const int column = (int)(blockIdx.x / slices) * 256 + threadIdx.x;
+  const int slice = (int)(blockIdx.x % slices);
+  if (column >= cols) return;
+  const int per = (nblocks + slices - 1) / slices;
+  const int r0 = slice * per, r1 = acc_min(nblocks, r0 + per);
+  if (r0 >= r1) return;
+  T acc = dump[(Int64)r0 * cols + column];
+#pragma unroll 8
+  for (int r = r0 + 1; r < r1; ++r) acc = f(dump[(Int64)r * cols + column], acc);
+  if (slices == 1) {
+    arrOut_0[column] = f(acc, arrOut_0[column]);
+  } else {
+    const T ident = acc_hint_identity<T>();
+    typename acc_bits<sizeof(T)>::type a, b;
+    __builtin_memcpy(&a, &acc, sizeof(T));
+    __builtin_memcpy(&b, &ident, sizeof(T));
+    if (a != b) acc_hint_apply<ACC_SCOPE_DEVICE>(arrOut_0 + column, acc, f);
   }
 }

@@ -136,7 +136,8 @@ int acc_exec_map(acc_skel s, const acc_array *env, const acc_array *out, acc_str
   if (n == 0) return ACC_OK;
   const int v = aligned ? 0 : 1;
   ACC_TRY(s->ensure_variant(v));
-  const int64_t grid = acc_launch_grid(n, s->elements_per_block(), resident(s, v), acc::tune("map.oversub", 8));
+  // streaming with no reuse: one short-lived workgroup per tile keeps the most loads in flight
+  const int64_t grid = acc_launch_grid(n, s->elements_per_block(), resident(s, v), acc::tune("map.oversub", 1 << 20));
   return launch(s, v, grid, 0, static_cast<hipStream_t>(stream), &args);
 }
 
@@ -175,15 +176,35 @@ int acc_exec_fold(acc_skel s, const acc_array *env, int32_t in_rank, const int64
 
   const int64_t n = inner;
   const int64_t tile = s->elements_per_block();
-  const int64_t grid = acc_launch_grid(n, tile, resident(s, v), acc::tune("fold.oversub", 1));
+  const int64_t grid = acc_launch_grid(n, tile, s->ctx->props.multiProcessorCount,
+                                       std::min(s->variants[v].blocks_per_cu, acc::tune("fold.blocks_per_cu", 4)));
+  if (grid == 1) {                 // a lone block finishes the job itself
+    args.ptr(out->ptr[0]);
+    args.i64(n);
+    args.ptr(0);
+    return launch(s, v, 1, 0, st, &args);
+  }
+  // one partial per block, then a single-block launch folds them: foldRec, Execute.hs:304-315,
+  // always exactly one level deep because the first grid never exceeds what is resident
   int blk = -1;
-  ACC_TRY(s->ctx->scratch_acquire(256 + (size_t)grid * s->spec.elt_size, st, acc::SCRATCH_FOLD, &blk));
-  char *base = static_cast<char *>(s->ctx->scratch[blk].ptr);
+  ACC_TRY(s->ctx->scratch_acquire((size_t)grid * s->spec.elt_size, st, acc::SCRATCH_FOLD, &blk));
+  const uint64_t partials = reinterpret_cast<uint64_t>(s->ctx->scratch[blk].ptr);
   args.ptr(out->ptr[0]);
   args.i64(n);
-  args.ptr(reinterpret_cast<uint64_t>(base + 256));
-  args.ptr(reinterpret_cast<uint64_t>(base));
-  const int rc = launch(s, v, grid, 0, st, &args);
+  args.ptr(partials);
+  int rc = launch(s, v, grid, 0, st, &args);
+  if (rc == ACC_OK) {
+    Args fin;
+    bool al = true;
+    rc = push_env(s, env, &fin, &al);
+    fin.ptr(out->ptr[0]);
+    fin.ptr(partials);
+    fin.i64(grid);
+    if (rc == ACC_OK) {
+      hipError_t e = hipModuleLaunchKernel(s->variants[v].fn_finish, 1, 1, 1, static_cast<unsigned>(s->spec.block), 1, 1, 0, st, fin.data(), nullptr);
+      if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(fold finish)");
+    }
+  }
   s->ctx->scratch_release(blk, st);
   return rc;
 }
@@ -326,22 +347,60 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
   // privatise target indices [0, bins) in LDS when the combine has a hardware
   // atomic and an identity; small targets get one copy per wave to spread
   // same-address traffic
+  const int cus = s->ctx->props.multiProcessorCount;
   int64_t bins = 0, copies = 1;
   if (s->spec.combine_hint != ACC_COMBINE_GENERIC) {
-    const int64_t budget = std::min<int64_t>((int64_t)s->ctx->props.sharedMemPerBlock, acc::tune("permute.lds_bytes", 65536)) - s->variants[v].static_lds;
+    const int64_t budget = std::min<int64_t>((int64_t)s->ctx->props.sharedMemPerBlock, acc::tune("permute.lds_bytes", 160 * 1024)) - s->variants[v].static_lds;
     const int64_t cap = std::max<int64_t>(0, budget / (int64_t)esz);
     bins = std::min(ntarget, cap);
     if (bins == ntarget && bins > 0) copies = std::max<int64_t>(1, std::min<int64_t>(s->spec.block / 64, cap / bins));
     copies = std::min<int64_t>(copies, acc::tune("permute.max_copies", 16));
   }
   const size_t lds = (size_t)(bins * copies) * esz;
-  args.i32(static_cast<int32_t>(bins));
-  args.i32(static_cast<int32_t>(copies));
   int bpc = 0;
   hipError_t e = hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&bpc, s->variants[v].fn, s->spec.block, lds);
   if (e != hipSuccess || bpc < 1) { (void)hipGetLastError(); bpc = 1; }
-  const int64_t grid = acc_launch_grid(n_src, s->elements_per_block(), s->ctx->props.multiProcessorCount, std::min(bpc, acc::tune("permute.max_blocks_per_cu", 4)));
-  return launch(s, v, grid, lds, st, &args);
+  const int64_t grid = acc_launch_grid(n_src, s->elements_per_block(), cus, std::min(bpc, acc::tune("permute.max_blocks_per_cu", 1)));
+
+  // how the privatised part leaves the blocks: atomics while they are few,
+  // otherwise a table of per-block bins folded by a second kernel
+  // Targets beyond the LDS window would be hit with device-scope atomics, the
+  // slowest operation on the machine; if a whole table row per block is
+  // affordable, they are privatised there instead (block-scope atomics in L2).
+  const bool private_tail = bins > 0 && bins < ntarget && ntarget < (1 << 30) &&
+                            (int64_t)grid * ntarget * (int64_t)esz <= (int64_t)acc::tune("permute.table_mbytes", 256) << 20;
+  const bool table = private_tail || (bins > 0 && grid * bins > acc::tune("permute.atomic_flush_max", 1 << 16));
+  const int64_t cols = private_tail ? ntarget : bins;
+  int blk = -1;
+  uint64_t dump = 0;
+  if (table) {
+    ACC_TRY(s->ctx->scratch_acquire((size_t)(grid * cols) * esz, st, acc::SCRATCH_FOLD, &blk));
+    dump = reinterpret_cast<uint64_t>(s->ctx->scratch[blk].ptr);
+  }
+  args.i32(static_cast<int32_t>(bins));
+  args.i32(static_cast<int32_t>(copies));
+  args.ptr(dump);
+  args.i32(static_cast<int32_t>(cols));
+  int rc = launch(s, v, grid, lds, st, &args);
+  if (rc == ACC_OK && table) {
+    Args m;
+    bool al = true;
+    rc = push_env(s, env, &m, &al);
+    push_out(*out, &m, &al);
+    // enough workgroups to fill the machine: columns x row slices
+    const int64_t columns = (cols + 255) / 256;
+    const int64_t slices = std::max<int64_t>(1, std::min<int64_t>(grid, (2 * cus + columns - 1) / columns));
+    m.ptr(dump);
+    m.i32(static_cast<int32_t>(cols));
+    m.i32(static_cast<int32_t>(grid));
+    m.i32(static_cast<int32_t>(slices));
+    if (rc == ACC_OK) {
+      e = hipModuleLaunchKernel(s->variants[v].fn_finish, static_cast<unsigned>(columns * slices), 1, 1, 256, 1, 1, 0, st, m.data(), nullptr);
+      if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(permute_merge)");
+    }
+  }
+  if (blk >= 0) s->ctx->scratch_release(blk, st);
+  return rc;
 }
 
 static int stencil_once(acc_skel s, const acc_array *env, const acc_array *in, const acc_array *out, hipStream_t st)

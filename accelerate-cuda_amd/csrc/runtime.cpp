@@ -51,12 +51,21 @@ int acc_context_s::make_current() const
 int acc_context_s::scratch_acquire(size_t bytes, hipStream_t stream, int protocol, int *index)
 {
   std::lock_guard<std::mutex> lock(mu);
+  if (!scratch_any_stream) {
+    scratch_any_stream = true;
+    scratch_first_stream = stream;
+  } else if (!scratch_multi_stream && stream != scratch_first_stream) {
+    // a second stream shows up: settle everything enqueued so far once, and
+    // track completion with events from here on
+    ACC_HIP_TRY(hipDeviceSynchronize());
+    scratch_multi_stream = true;
+  }
   int pick = -1;
   for (size_t i = 0; i < scratch.size(); ++i) {
     acc::ScratchBlock &b = scratch[i];
     if (b.busy || b.bytes < bytes || b.protocol != protocol) continue;
-    bool reusable = (b.stream == stream);
-    if (!reusable && b.done) reusable = (hipEventQuery(b.done) == hipSuccess);
+    bool reusable = (b.stream == stream) || !b.recorded;
+    if (!reusable) reusable = (hipEventQuery(b.done) == hipSuccess);
     if (reusable && (pick < 0 || b.bytes < scratch[pick].bytes)) pick = static_cast<int>(i);
   }
   if (pick < 0) {
@@ -83,7 +92,8 @@ void acc_context_s::scratch_release(int index, hipStream_t stream)
 {
   std::lock_guard<std::mutex> lock(mu);
   acc::ScratchBlock &b = scratch[index];
-  (void)hipEventRecord(b.done, stream);
+  b.recorded = false;
+  if (scratch_multi_stream) b.recorded = (hipEventRecord(b.done, stream) == hipSuccess);
   b.stream = stream;
   b.busy = false;
 }

@@ -283,7 +283,7 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
   switch (d->kind) {
     case ACC_SKEL_MAP: case ACC_SKEL_GENERATE: case ACC_SKEL_TRANSFORM:
       sp->block = tune("map.block", 256);
-      sp->unroll = tune("map.unroll", 4);
+      sp->unroll = tune("map.unroll", 1);
       break;
     case ACC_SKEL_FOLD: case ACC_SKEL_FOLD1:
       sp->block = tune("fold.block", 256);
@@ -302,8 +302,8 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
         return fail(ACC_ERR_INVALID, "permute: bad combine_hint %d", sp->combine_hint);
       if (sp->combine_hint >= ACC_COMBINE_AND && !is_integer_type(sp->elt_type))
         return fail(ACC_ERR_INVALID, "permute: bitwise combine_hint on non-integer element type '%s'", sp->elt_type.c_str());
-      sp->block = tune("permute.block", 512);
-      sp->unroll = tune("permute.unroll", 4);
+      sp->block = tune("permute.block", 1024);
+      sp->unroll = tune("permute.unroll", 2);
       break;
     case ACC_SKEL_STENCIL: {
       if (sp->out_rank != 1 && sp->out_rank != 2) return fail(ACC_ERR_UNSUPPORTED, "stencil: rank %d not supported (1 and 2 are)", sp->out_rank);
@@ -372,6 +372,17 @@ int acc_skel_s::ensure_variant(int v)
     (void)hipModuleUnload(var.module);
     var.module = nullptr;
     return acc::fail_hip(e, ("hipModuleGetFunction(" + entry + ")").c_str());
+  }
+  const bool two_kernels = ((spec.kind == ACC_SKEL_FOLD || spec.kind == ACC_SKEL_FOLD1) && spec.out_rank == 0) ||
+                           spec.kind == ACC_SKEL_PERMUTE;
+  const std::string second = entry + (spec.kind == ACC_SKEL_PERMUTE ? "_merge" : "_finish");
+  if (two_kernels) {
+    e = hipModuleGetFunction(&var.fn_finish, var.module, second.c_str());
+    if (e != hipSuccess) {
+      (void)hipModuleUnload(var.module);
+      var.module = nullptr;
+      return acc::fail_hip(e, ("hipModuleGetFunction(" + second + ")").c_str());
+    }
   }
   (void)hipFuncGetAttribute(&var.num_regs, HIP_FUNC_ATTRIBUTE_NUM_REGS, var.fn);
   (void)hipFuncGetAttribute(&var.static_lds, HIP_FUNC_ATTRIBUTE_SHARED_SIZE_BYTES, var.fn);

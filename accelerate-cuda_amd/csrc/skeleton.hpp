@@ -37,6 +37,7 @@ struct Variant {
   std::string source;
   hipModule_t module = nullptr;
   hipFunction_t fn = nullptr;
+  hipFunction_t fn_finish = nullptr;   // second kernel of a two-launch skeleton (foldAll)
   int num_regs = 0;
   int static_lds = 0;
   int blocks_per_cu = 1;
