@@ -176,6 +176,27 @@ ACC_DEV void acc_atomic_rmw(T *addr, const T &x, F combine_new_old)
   } while (old != assumed);
 }
 
+/* Workgroups are handed to the 8 compute dies (XCDs) round-robin, and each die
+ * has its own L2.  This renumbering gives every die one contiguous run of the
+ * logical work items instead of every eighth one, so that neighbours in the
+ * logical order -- which share halo rows, or continue each other's memory
+ * stream -- also share an L2.  It is a bijection on [0, gridDim.x) whatever
+ * the hardware really does; only the locality depends on the assumption.    */
+#define ACC_XCDS 8
+ACC_DEV Int64 acc_xcd_contiguous_block()
+{
+  const Int64 n = gridDim.x, b = blockIdx.x;
+  const Int64 q = n / ACC_XCDS, r = n % ACC_XCDS;
+  const Int64 xcd = b % ACC_XCDS, i = b / ACC_XCDS;
+  return xcd * q + acc_min<Int64>(xcd, r) + i;
+}
+
+/* A read of an array element that will not be needed again (a manifest input
+ * consumed once, in index order).  It is marked non-temporal so that it does
+ * not evict data that IS reused -- a gathered vector, a small table -- from
+ * the L2.  The code generator uses it for linear reads next to indirect ones. */
+template <typename T> ACC_DEV T acc_stream(const T *p, const Int64 ix) { return __builtin_nontemporal_load(p + ix); }
+
 /* row-major index helpers (CodeGen/Base.hs:193-218): shapes and indices are
  * listed innermost dimension LAST, e.g. acc_to_index2(h, w, y, x)            */
 ACC_DEV Int64 acc_to_index2(Int64, Int64 w, Int64 y, Int64 x) { return y * w + x; }

@@ -33,6 +33,9 @@ static_assert(ACC_CHUNK % (ACC_BLOCK * ACC_VEC) == 0, "chunk must be a whole num
 #define ACC_FOLDSEG_ENTRY fold1Seg
 #endif
 
+#define ACC_LOADS (ACC_CHUNK / (ACC_BLOCK * ACC_VEC))   /* vector loads per lane and chunk */
+#define ACC_EAT 8                                        /* LDS reads kept in flight while folding */
+
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
                   const Int64 shOut_0, ACC_ELT *__restrict__ arrOut_0,
@@ -74,34 +77,56 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
     for (Int64 q = 0; q < nchunks; ++q) {
       const Int64 cs = lo_al + (ACC_FOLD_RIGHT ? (nchunks - 1 - q) : q) * (Int64)ACC_CHUNK;
       const Int64 ce = acc_min<Int64>(cs + ACC_CHUNK, hi);
+
+      /* stage the chunk: every load is issued before any result is used.
+       * Elements of the chunk's first and last vector that belong to a
+       * neighbouring block are loaded too (they exist) and never read back;
+       * only the very end of the array needs a guard. */
+      T v[ACC_LOADS][ACC_VEC];
+      if (cs + ACC_CHUNK <= n) {
+#pragma unroll
+        for (int u = 0; u < ACC_LOADS; ++u)
+#pragma unroll
+          for (int k = 0; k < ACC_VEC; ++k) v[u][k] = get(cs + (u * ACC_BLOCK + tid) * ACC_VEC + k);
+      } else {
+#pragma unroll
+        for (int u = 0; u < ACC_LOADS; ++u)
+#pragma unroll
+          for (int k = 0; k < ACC_VEC; ++k) {
+            const Int64 ix = cs + (u * ACC_BLOCK + tid) * ACC_VEC + k;
+            v[u][k] = T();
+            if (ix < n) v[u][k] = get(ix);
+          }
+      }
       __syncthreads();                               /* the previous chunk has been consumed */
 #pragma unroll
-      for (int u = 0; u < ACC_CHUNK / (ACC_BLOCK * ACC_VEC); ++u) {
-        const int o = (u * ACC_BLOCK + tid) * ACC_VEC;
-        const Int64 ix = cs + o;
-        if (ix + ACC_VEC <= ce && ix >= lo) {
+      for (int u = 0; u < ACC_LOADS; ++u)
 #pragma unroll
-          for (int k = 0; k < ACC_VEC; ++k) s_val[o + k] = get(ix + k);
-        } else {
-#pragma unroll
-          for (int k = 0; k < ACC_VEC; ++k)
-            if (ix + k >= lo && ix + k < ce) s_val[o + k] = get(ix + k);
-        }
-      }
+        for (int k = 0; k < ACC_VEC; ++k) s_val[(u * ACC_BLOCK + tid) * ACC_VEC + k] = v[u][k];
       __syncthreads();
-      const Int64 i0 = acc_max(a, cs), i1 = acc_min(b, ce);
+
+      /* fold this lane's segment, as far as it lies in the chunk, in index order */
+      int p0 = (int)(acc_max(a, cs) - cs), p1 = (int)(acc_min(b, ce) - cs);
 #if ACC_FOLD_RIGHT
-      for (Int64 i = i1 - 1; i >= i0; --i) {
-        const T v = s_val[i - cs];
-        acc = have ? f(v, acc) : v;
-        have = true;
+      if (!have && p0 < p1) { acc = s_val[--p1]; have = true; }
+      for (; p1 - ACC_EAT >= p0; p1 -= ACC_EAT) {
+        T w[ACC_EAT];
+#pragma unroll
+        for (int k = 0; k < ACC_EAT; ++k) w[k] = s_val[p1 - 1 - k];
+#pragma unroll
+        for (int k = 0; k < ACC_EAT; ++k) acc = f(w[k], acc);
       }
+      for (; p1 > p0; --p1) acc = f(s_val[p1 - 1], acc);
 #else
-      for (Int64 i = i0; i < i1; ++i) {
-        const T v = s_val[i - cs];
-        acc = have ? f(acc, v) : v;
-        have = true;
+      if (!have && p0 < p1) { acc = s_val[p0++]; have = true; }
+      for (; p0 + ACC_EAT <= p1; p0 += ACC_EAT) {
+        T w[ACC_EAT];
+#pragma unroll
+        for (int k = 0; k < ACC_EAT; ++k) w[k] = s_val[p0 + k];
+#pragma unroll
+        for (int k = 0; k < ACC_EAT; ++k) acc = f(acc, w[k]);
       }
+      for (; p0 < p1; ++p0) acc = f(acc, s_val[p0]);
 #endif
     }
 

@@ -6,35 +6,46 @@
  * CodeGen/Stencil/Extra.hs:53-128.  The reference reads every tap straight
  * from global memory (relying on the L1 cache, Context.hs:61-68), recovers the
  * multidimensional index with 64-bit divisions and tests a whole warp for
- * "interior" (Stencil.hs:103-110).  Here a workgroup stages a
- * (ACC_TILE_H + 2 ry) x (ACC_TILE_W + 2 rx) patch of the source in LDS once
- * -- 128-bit loads for the body of each row, a handful of scalar loads for the
- * halo columns -- and every tap is an LDS read.  Only tiles that touch the
- * array's edge apply the boundary condition, while they fill the patch; the
- * index maps are exactly those of Stencil/Extra.hs:191-226:
+ * "interior" (Stencil.hs:103-110).  Here the work is cut into strips: one
+ * 64-lane wave owns 256 columns (4 per lane) and walks down ACC_TILE_H rows,
+ * keeping the 2 ry + 1 source rows it currently needs in registers:
+ *   - every source row is fetched once per strip with one 128-bit load per
+ *     lane, ACC_PREFETCH rows ahead of its use, so a wave always has several
+ *     kilobytes in flight and never waits at a barrier;
+ *   - taps to the left and right come from the neighbouring lanes' registers
+ *     through DPP wave shifts; only the first and last lane of a strip load
+ *     their rx halo elements themselves;
+ *   - taps above and below are simply older and newer rows of the register
+ *     window, which rotates by renaming (the row loop is unrolled by the
+ *     window length).
+ * The boundary condition is applied where rows and halo elements are fetched;
+ * the index maps are exactly those of Stencil/Extra.hs:191-226:
  *     clamp    max(0, min(i, sz-1))
  *     mirror   i < 0 ? -i : i >= sz ? sz - (i - sz + 2) : i
  *     wrap     i < 0 ? sz + i : i >= sz ? i - sz : i
  *     constant out-of-range taps read the constant
- * Each lane produces ACC_VEC consecutive results of a row and a workgroup
- * walks down its tile ACC_BLOCK / (ACC_TILE_W / ACC_VEC) rows at a time.
+ * Strips are kept short (ACC_TILE_H rows): the workgroups in flight then sweep
+ * a compact window of the image, which DRAM serves far better than many
+ * distant rows at once; the price is that neighbouring strips re-read each
+ * other's boundary rows.  ACC_XCD_REMAP renumbers the workgroups so that such
+ * neighbours run on the same compute die (acc_xcd_contiguous_block).
+ * Strips that are cut by the right edge, and arrays whose rows are not
+ * 16-byte aligned, take a slower path that maps every element on its own.
  *
  * Generated definitions expected: ACC_ELT, ACC_IN_ELT, ACC_ENV_PARAMS,
  * ACC_ENV_ASSUME, ACC_OUT_PARAMS, ACC_STENCIL_RANK (1|2), ACC_RADIUS_Y,
  * ACC_RADIUS_X, ACC_BOUNDARY, ACC_BOUNDARY_CONSTANT, ACC_STENCIL_TAPS(READ),
- * ACC_STENCIL_FN, ACC_TILE_W, ACC_TILE_H, ACC_BLOCK, ACC_ALIGNED.
+ * ACC_STENCIL_FN, ACC_TILE_H, ACC_PREFETCH, ACC_BLOCK, ACC_ALIGNED.
  */
 
-#define ACC_SVEC 4                                     /* results per lane and row */
-#define ACC_TPR  (ACC_TILE_W / ACC_SVEC)               /* lanes per tile row */
-#define ACC_RPP  (ACC_BLOCK / ACC_TPR)                 /* tile rows per pass */
-#define ACC_LW   (ACC_TILE_W + 2 * ACC_RADIUS_X)
-#define ACC_LH   (ACC_TILE_H + 2 * ACC_RADIUS_Y)
-#define ACC_LPITCH (ACC_LW + ((4 - (ACC_LW & 3)) & 3) + 4)   /* keep rows 16-byte aligned, skew banks */
-#define ACC_LX0  4                                     /* LDS column of tile column 0 (>= rx, multiple of 4) */
+#define ACC_SVEC  4                                   /* results per lane and row */
+#define ACC_STRIP (ACC_WAVE * ACC_SVEC)               /* columns per wave */
+#define ACC_NR    (2 * ACC_RADIUS_Y + 1)              /* rows a result depends on */
+#define ACC_RING  (ACC_NR + ACC_PREFETCH)             /* rows held in registers */
+#define ACC_WW    (ACC_SVEC + 2 * ACC_RADIUS_X)       /* row window of one lane */
+#define ACC_WAVES (ACC_BLOCK / ACC_WAVE)
 
-static_assert(ACC_TILE_W % ACC_SVEC == 0 && ACC_BLOCK % ACC_TPR == 0 && ACC_TILE_H % ACC_RPP == 0, "tile shape does not divide among the lanes");
-static_assert(ACC_RADIUS_X <= ACC_LX0, "stencil too wide for the patch layout");
+static_assert(ACC_RADIUS_X <= ACC_SVEC, "stencil wider than one lane's neighbours can supply");
 
 #define ACC_B_CLAMP 0
 #define ACC_B_MIRROR 1
@@ -50,13 +61,19 @@ ACC_DEV Int64 acc_boundary_index(Int64 i, const Int64 sz)
 #elif ACC_BOUNDARY == ACC_B_WRAP
   i = i < 0 ? sz + i : (i >= sz ? i - sz : i);
 #endif
-  /* positions of a ragged tile that no valid result reads may still lie
-   * outside; keep the address legal */
+  /* the maps assume the array spans the stencil; keep the address legal if not */
   return acc_max<Int64>(0, acc_min<Int64>(i, sz - 1));
 }
 
 struct __attribute__((aligned(16))) acc_in_vec { ACC_IN_ELT v[ACC_SVEC]; };
 struct __attribute__((aligned(16))) acc_out_vec { ACC_ELT v[ACC_SVEC]; };
+
+/* value held by the next lane (the last lane keeps its own: caller masks it) */
+#define ACC_DPP_WAVE_SHL1 0x130
+template <typename T> ACC_DEV T acc_wave_shift_down1(const T &x) { return acc_dpp<ACC_DPP_WAVE_SHL1, 0xf>(x, x); }
+
+/* one source row as a lane sees it: [rx left | ACC_SVEC own | rx right] */
+struct acc_row { ACC_IN_ELT e[ACC_WW]; };
 
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 stencil(ACC_ENV_PARAMS ACC_OUT_PARAMS, const ACC_IN_ELT *__restrict__ arrStencil_0)
@@ -64,81 +81,132 @@ stencil(ACC_ENV_PARAMS ACC_OUT_PARAMS, const ACC_IN_ELT *__restrict__ arrStencil
   typedef ACC_ELT T;
   typedef ACC_IN_ELT S;
   ACC_ENV_ASSUME
-  __shared__ __attribute__((aligned(16))) S patch[ACC_LH][ACC_LPITCH];
-
 #if ACC_STENCIL_RANK == 2
   const Int64 h = shOut_1, w = shOut_0;
 #else
   const Int64 h = 1, w = shOut_0;
 #endif
-  const Int64 tiles_x = (w + ACC_TILE_W - 1) / ACC_TILE_W;
-  const Int64 ty = (Int64)blockIdx.x / tiles_x, tx = (Int64)blockIdx.x % tiles_x;
-  const Int64 y0 = ty * ACC_TILE_H, x0 = tx * ACC_TILE_W;
-
-  const int tid = threadIdx.x;
-  const bool interior = (y0 - ACC_RADIUS_Y >= 0) && (y0 + ACC_TILE_H + ACC_RADIUS_Y <= h) &&
-                        (x0 - ACC_RADIUS_X >= 0) && (x0 + ACC_TILE_W + ACC_RADIUS_X <= w);
-
-  /* ---- stage the patch ---------------------------------------------------- */
-  if (interior) {
-    /* body of every patch row: one vector per lane */
-    for (int i = tid; i < ACC_LH * ACC_TPR; i += ACC_BLOCK) {
-      const int ly = i / ACC_TPR, c = i % ACC_TPR;
-      const S *src = arrStencil_0 + (y0 - ACC_RADIUS_Y + ly) * w + x0 + c * ACC_SVEC;
-#if ACC_ALIGNED
-      *(acc_in_vec *)&patch[ly][ACC_LX0 + c * ACC_SVEC] = *(const acc_in_vec *)src;
+  const int lane = acc_lane();
+  const Int64 strips_x = (w + ACC_STRIP - 1) / ACC_STRIP;
+#if ACC_XCD_REMAP
+  const Int64 strip = acc_xcd_contiguous_block() * ACC_WAVES + (threadIdx.x >> 6);
 #else
-#pragma unroll
-      for (int k = 0; k < ACC_SVEC; ++k) patch[ly][ACC_LX0 + c * ACC_SVEC + k] = src[k];
+  const Int64 strip = (Int64)blockIdx.x * ACC_WAVES + (threadIdx.x >> 6);
 #endif
-    }
-    /* halo columns */
-    if (ACC_RADIUS_X > 0) {
-      for (int i = tid; i < ACC_LH * 2 * ACC_RADIUS_X; i += ACC_BLOCK) {
-        const int ly = i / (2 * ACC_RADIUS_X), e = i % (2 * ACC_RADIUS_X);
-        const int lx = (e < ACC_RADIUS_X) ? (e - ACC_RADIUS_X) : (ACC_TILE_W + e - ACC_RADIUS_X);   /* relative to tile column 0 */
-        patch[ly][ACC_LX0 + lx] = arrStencil_0[(y0 - ACC_RADIUS_Y + ly) * w + x0 + lx];
+  const Int64 y0 = (strip / strips_x) * ACC_TILE_H, x0 = (strip % strips_x) * ACC_STRIP;
+  if (y0 >= h) return;                                   /* whole wave leaves together */
+  const Int64 gx = x0 + lane * ACC_SVEC;
+  const int rows = (int)acc_min<Int64>(ACC_TILE_H, h - y0);
+#if ACC_ALIGNED
+  const bool fast = (x0 + ACC_STRIP <= w);               /* every lane owns a full, aligned vector */
+#else
+  const bool fast = false;
+#endif
+
+  /* fetch source row (y0 - ry + rho) into a window; in the fast path the left
+   * and right parts are only valid in the strip's first and last lane until
+   * acc_row_finish has run */
+  auto fetch = [&](const int rho, acc_row &r) {
+    const Int64 gy = y0 - ACC_RADIUS_Y + rho;
+#if ACC_BOUNDARY == ACC_B_CONSTANT
+    const bool row_inside = gy >= 0 && gy < h;
+    const Int64 my = acc_max<Int64>(0, acc_min<Int64>(gy, h - 1));
+#else
+    const bool row_inside = true;
+    const Int64 my = acc_boundary_index(gy, h);
+#endif
+    const S *src = arrStencil_0 + my * w;
+    if (fast) {
+      const acc_in_vec own = *(const acc_in_vec *)(src + gx);
+#pragma unroll
+      for (int k = 0; k < ACC_SVEC; ++k) r.e[ACC_RADIUS_X + k] = row_inside ? own.v[k] : (S)(ACC_BOUNDARY_CONSTANT);
+#pragma unroll
+      for (int j = 0; j < ACC_RADIUS_X; ++j) {
+        r.e[j] = S();
+        r.e[ACC_RADIUS_X + ACC_SVEC + j] = S();
+        if (lane == 0) {
+          const Int64 xx = x0 - ACC_RADIUS_X + j;
+#if ACC_BOUNDARY == ACC_B_CONSTANT
+          r.e[j] = (row_inside && xx >= 0) ? src[acc_max<Int64>(xx, 0)] : (S)(ACC_BOUNDARY_CONSTANT);
+#else
+          r.e[j] = src[acc_boundary_index(xx, w)];
+#endif
+        }
+        if (lane == ACC_WAVE - 1) {
+          const Int64 xx = x0 + ACC_STRIP + j;
+#if ACC_BOUNDARY == ACC_B_CONSTANT
+          r.e[ACC_RADIUS_X + ACC_SVEC + j] = (row_inside && xx < w) ? src[acc_min<Int64>(xx, w - 1)] : (S)(ACC_BOUNDARY_CONSTANT);
+#else
+          r.e[ACC_RADIUS_X + ACC_SVEC + j] = src[acc_boundary_index(xx, w)];
+#endif
+        }
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < ACC_WW; ++e) {
+        const Int64 xx = gx - ACC_RADIUS_X + e;
+        r.e[e] = S();
+        if (gx < w) {                                    /* lanes past the edge produce nothing */
+#if ACC_BOUNDARY == ACC_B_CONSTANT
+          const bool inside = row_inside && xx >= 0 && xx < w;
+          r.e[e] = inside ? src[xx] : (S)(ACC_BOUNDARY_CONSTANT);
+#else
+          r.e[e] = src[acc_boundary_index(xx, w)];
+#endif
+        }
       }
     }
-  } else {
-    for (int i = tid; i < ACC_LH * ACC_LW; i += ACC_BLOCK) {
-      const int ly = i / ACC_LW, lx = i % ACC_LW - ACC_RADIUS_X;
-      const Int64 gy = y0 - ACC_RADIUS_Y + ly, gx = x0 + lx;
-#if ACC_BOUNDARY == ACC_B_CONSTANT
-      const bool inside = gy >= 0 && gy < h && gx >= 0 && gx < w;
-      const S v = inside ? arrStencil_0[gy * w + gx] : (S)(ACC_BOUNDARY_CONSTANT);
-#else
-      const S v = arrStencil_0[acc_boundary_index(gy, h) * w + acc_boundary_index(gx, w)];
-#endif
-      patch[ly][ACC_LX0 + lx] = v;
-    }
-  }
-  __syncthreads();
+  };
 
-  /* ---- evaluate ------------------------------------------------------------- */
-  const int c = tid % ACC_TPR, r0 = tid / ACC_TPR;
+  /* fast path only: complete the window with the neighbours' elements */
+  auto finish = [&](acc_row &r) {
+    if (!fast) return;
 #pragma unroll
-  for (int p = 0; p < ACC_TILE_H / ACC_RPP; ++p) {
-    const int r = r0 + p * ACC_RPP;
-    const Int64 gy = y0 + r, gx = x0 + c * ACC_SVEC;
-    acc_out_vec res;
-#pragma unroll
-    for (int k = 0; k < ACC_SVEC; ++k) {
-#define ACC_PATCH_READ(dy, dx) patch[r + ACC_RADIUS_Y + (dy)][ACC_LX0 + c * ACC_SVEC + k + (dx)]
-      ACC_STENCIL_TAPS(ACC_PATCH_READ)
-#undef ACC_PATCH_READ
-      res.v[k] = (T)(ACC_STENCIL_FN);
+    for (int j = 0; j < ACC_RADIUS_X; ++j) {
+      const S from_left  = acc_wave_shift_up1(r.e[ACC_SVEC + j]);          /* neighbour's own[SVEC - rx + j] */
+      const S from_right = acc_wave_shift_down1(r.e[ACC_RADIUS_X + j]);    /* neighbour's own[j] */
+      if (lane != 0) r.e[j] = from_left;
+      if (lane != ACC_WAVE - 1) r.e[ACC_RADIUS_X + ACC_SVEC + j] = from_right;
     }
-    if (gy < h) {
-      T *dst = arrOut_0 + gy * w + gx;
-#if ACC_ALIGNED
-      if (gx + ACC_SVEC <= w) *(acc_out_vec *)dst = res;
-      else
-#endif
-      {
+  };
+
+  acc_row ring[ACC_RING];
+  const int total = rows + 2 * ACC_RADIUS_Y;              /* source rows this strip touches */
+
+  /* prologue: the rows the first result needs, minus the newest, plus the prefetch */
 #pragma unroll
-        for (int k = 0; k < ACC_SVEC; ++k)
-          if (gx + k < w) dst[k] = res.v[k];
+  for (int rho = 0; rho < ACC_RING - 1; ++rho)
+    if (rho < total) fetch(rho, ring[rho]);
+#pragma unroll
+  for (int rho = 0; rho < ACC_NR - 1; ++rho) finish(ring[rho]);
+
+  for (int yb = 0; yb < rows; yb += ACC_RING) {
+#pragma unroll
+    for (int s = 0; s < ACC_RING; ++s) {
+      const int y = yb + s;                               /* row of the strip being produced */
+      if (y < rows) {
+        /* newest row needed now is rho = y + 2 ry, in slot (s + NR - 1) % RING; the
+         * slot freed by the previous step takes the row PREFETCH further on */
+        const int rho_new = y + ACC_NR - 1 + ACC_PREFETCH;
+        if (rho_new < total) fetch(rho_new, ring[(s + ACC_RING - 1) % ACC_RING]);
+        finish(ring[(s + ACC_NR - 1) % ACC_RING]);
+
+        acc_out_vec res;
+#pragma unroll
+        for (int k = 0; k < ACC_SVEC; ++k) {
+#define ACC_WINDOW_READ(dy, dx) ring[(s + ACC_RADIUS_Y + (dy)) % ACC_RING].e[ACC_RADIUS_X + k + (dx)]
+          ACC_STENCIL_TAPS(ACC_WINDOW_READ)
+#undef ACC_WINDOW_READ
+          res.v[k] = (T)(ACC_STENCIL_FN);
+        }
+        T *dst = arrOut_0 + (y0 + y) * w + gx;
+        if (fast) {
+          *(acc_out_vec *)dst = res;
+        } else {
+#pragma unroll
+          for (int k = 0; k < ACC_SVEC; ++k)
+            if (gx + k < w) dst[k] = res.v[k];
+        }
       }
     }
   }

@@ -229,7 +229,7 @@ int acc_exec_foldseg(acc_skel s, const acc_array *env, int64_t n, const acc_arra
   args.ptr(offsets->ptr[0]);
   const int v = aligned ? 0 : 1;
   ACC_TRY(s->ensure_variant(v));
-  const int64_t grid = acc_launch_grid(nseg, s->spec.block, resident(s, v), acc::tune("foldseg.oversub", 8));
+  const int64_t grid = acc_launch_grid(nseg, s->spec.block, resident(s, v), acc::tune("foldseg.oversub", 1 << 20));
   return launch(s, v, grid, 0, static_cast<hipStream_t>(stream), &args);
 }
 
@@ -418,9 +418,10 @@ static int stencil_once(acc_skel s, const acc_array *env, const acc_array *in, c
   // rows start on 16-byte boundaries only if the row pitch allows it
   const size_t in_esz = acc::type_size(s->spec.stencil_in_type) ? acc::type_size(s->spec.stencil_in_type) : s->spec.elt_size;
   if ((w * (int64_t)s->spec.elt_size) % 16 != 0 || (w * (int64_t)in_esz) % 16 != 0) aligned = false;
-  const int64_t tx = (w + s->spec.tile_w - 1) / s->spec.tile_w;
-  const int64_t ty = (h + s->spec.tile_h - 1) / s->spec.tile_h;
-  return launch(s, aligned ? 0 : 1, tx * ty, 0, st, &args);
+  // one wave per strip of 256 columns x tile_h rows
+  const int64_t strips = ((w + s->spec.tile_w - 1) / s->spec.tile_w) * ((h + s->spec.tile_h - 1) / s->spec.tile_h);
+  const int64_t waves = s->spec.block / 64;
+  return launch(s, aligned ? 0 : 1, (strips + waves - 1) / waves, 0, st, &args);
 }
 
 static int stencil_check(acc_skel s, const acc_array *in, const acc_array *out)

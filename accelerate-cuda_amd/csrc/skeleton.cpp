@@ -207,7 +207,8 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
         o << "const ACC_IN_ELT t" << k << " = READ(" << sp.tap_dy[k] << ", " << sp.tap_dx[k] << "); ";
       o << "\n";
       o << "#define ACC_STENCIL_FN " << sp.stencil_fn << "\n";
-      o << "#define ACC_TILE_W " << sp.tile_w << "\n#define ACC_TILE_H " << sp.tile_h << "\n#define ACC_BLOCK " << sp.block << "\n";
+      o << "#define ACC_XCD_REMAP " << tune("stencil.xcd_remap", 0) << "\n";
+      o << "#define ACC_TILE_H " << sp.tile_h << "\n#define ACC_PREFETCH " << sp.prefetch << "\n#define ACC_BLOCK " << sp.block << "\n";
       tmpl = "skel_stencil.h";
       break;
     }
@@ -291,7 +292,7 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
       break;
     case ACC_SKEL_FOLDSEG: case ACC_SKEL_FOLD1SEG:
       sp->block = tune("foldseg.block", 256);
-      sp->chunk = tune("foldseg.chunk", 4096);
+      sp->chunk = tune("foldseg.chunk", 2048);
       break;
     case ACC_SKEL_PERMUTE:
       if (sp->permutation.empty()) return fail(ACC_ERR_INVALID, "permute: `permutation` fragment missing");
@@ -321,9 +322,10 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
       sp->stencil_fn = flat(d->stencil_fn);
       sp->stencil_in_type = (d->stencil_in_type && *d->stencil_in_type) ? d->stencil_in_type : sp->elt_type;
       sp->block = tune("stencil.block", 256);
-      sp->tile_w = tune("stencil.tile_w", 256);
-      sp->tile_h = tune("stencil.tile_h", sp->out_rank == 2 ? 16 : 1);
-      if (sp->out_rank == 1) { sp->tile_h = 1; sp->tile_w = sp->block * 4; }
+      sp->tile_w = 256;                                  // one wave's strip: 64 lanes x 4 columns
+      sp->tile_h = sp->out_rank == 2 ? tune("stencil.tile_h", 4) : 1;
+      sp->prefetch = sp->out_rank == 2 ? tune("stencil.prefetch", 3) : 0;
+      if (sp->tile_h < 1 || sp->prefetch < 0 || sp->prefetch > 8) return fail(ACC_ERR_INVALID, "stencil: bad tile shape");
       break;
     }
     default:   // scans

@@ -246,7 +246,8 @@ def main():
         dv, dc, dxv, doff = ctx.array(vals), ctx.array(cols), ctx.array(xv), ctx.array(offs)
         env = envs(dv, dc, dxv)
         y = ctx.empty(rows, np.float32)
-        smvm = ctx.skeleton(A.SKEL_FOLDSEG, "float", env=[F32, I32, F32], get="arrIn0_0[ix] * arrIn2_0[arrIn1_0[ix]]",
+        smvm = ctx.skeleton(A.SKEL_FOLDSEG, "float", env=[F32, I32, F32],
+                            get=os.environ.get("ACC_BENCH_SMVM_GET", "arrIn0_0[ix] * arrIn2_0[arrIn1_0[ix]]"),
                             combine="x + y", seed="0.0f")
         offd, yd = doff.desc(), y.desc()
 
