@@ -84,7 +84,7 @@ acc_memcpy_d2d_async acc_memset32_async acc_stream_create acc_stream_destroy acc
 acc_stream_wait_event acc_event_create acc_event_destroy acc_event_record acc_event_sync acc_event_query
 acc_event_elapsed_ms acc_compile acc_compile_log acc_cache_set_dir acc_cache_dir acc_cache_get_stats
 acc_cache_clear acc_module_load acc_module_unload acc_module_get_function acc_function_attr acc_occupancy
-acc_launch acc_launch_grid acc_skel_create acc_skel_destroy acc_skel_source acc_skel_compile_only
+acc_launch acc_launch_grid acc_skel_create acc_skel_destroy acc_skel_source acc_skel_preview acc_skel_compile_only
 acc_skel_get_info acc_exec_map acc_exec_fold acc_exec_foldseg acc_exec_scan acc_exec_permute
 acc_exec_stencil acc_exec_stencil_iterate""".split()
 
@@ -135,6 +135,7 @@ def lib():
         L.acc_skel_create.argtypes = [C.c_void_p, C.POINTER(acc_skel_desc), C.POINTER(C.c_void_p)]
         L.acc_skel_destroy.argtypes = [C.c_void_p]
         L.acc_skel_source.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_char_p)]
+        L.acc_skel_preview.argtypes = [C.POINTER(acc_skel_desc), C.c_int, C.POINTER(C.c_char_p), C.POINTER(C.c_char_p)]
         L.acc_skel_compile_only.argtypes = [C.c_char_p, C.POINTER(acc_skel_desc), C.POINTER(C.c_size_t)]
         L.acc_skel_get_info.argtypes = [C.c_void_p, C.POINTER(acc_skel_info)]
         AP = C.POINTER(acc_array)
@@ -187,6 +188,13 @@ def make_desc(kind, elt, env=(), out_rank=0, get=None, combine=None, seed=None, 
     d.stencil_fn, d.stencil_in_type, d.seg_type = _b(stencil_fn), _b(stencil_in), _b(seg_type)
     d._keep = (sigs, keep)
     return d
+
+
+def preview(desc, variant=0):
+    """(entry name, generated translation unit) of a description; needs no GPU."""
+    src, entry = C.c_char_p(), C.c_char_p()
+    check(lib().acc_skel_preview(C.byref(desc), variant, C.byref(src), C.byref(entry)))
+    return entry.value.decode(), src.value.decode()
 
 
 def compile_only(desc, target="gfx950"):

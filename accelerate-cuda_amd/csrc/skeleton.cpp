@@ -434,6 +434,18 @@ int acc_skel_source(acc_skel s, int variant, const char **source)
   return ACC_OK;
 }
 
+int acc_skel_preview(const acc_skel_desc *desc, int variant, const char **source, const char **entry)
+{
+  static thread_local std::string text, name;
+  if (!source || variant < 0 || variant > 1) return fail(ACC_ERR_INVALID, "acc_skel_preview: bad argument");
+  acc::SkelSpec sp;
+  ACC_TRY(acc::make_spec(desc, &sp));
+  ACC_TRY(acc::generate_source(sp, variant == 0, &name, &text));
+  *source = text.c_str();
+  if (entry) *entry = name.c_str();
+  return ACC_OK;
+}
+
 int acc_skel_compile_only(const char *target, const acc_skel_desc *desc, size_t *code_size)
 {
   if (!target) return fail(ACC_ERR_INVALID, "acc_skel_compile_only: NULL target");

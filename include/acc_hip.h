@@ -288,6 +288,9 @@ int acc_skel_destroy(acc_skel s);
 /* The generated translation unit (for -ddump-cc style debugging and tests).
  * variant 0 = aligned (128-bit accesses assumed legal), 1 = unaligned.      */
 int acc_skel_source(acc_skel s, int variant, const char **source);
+/* the same text straight from a description, without a context or a GPU; the
+ * string stays valid until the calling thread's next call of this function  */
+int acc_skel_preview(const acc_skel_desc *desc, int variant, const char **source, const char **entry);
 /* compile only (no GPU needed): used by the build check */
 int acc_skel_compile_only(const char *target, const acc_skel_desc *desc, size_t *code_size);
 

@@ -1,0 +1,243 @@
+"""Host-side logic of libacchip that needs no GPU: the C ABI surface, run-time
+compilation for gfx950 (hiprtc works without a device), the kernel cache, the
+skeleton generator's parameter ABI, launch arithmetic and error paths.
+"""
+import ctypes as C
+import os
+import re
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def A():
+    import acchip
+    acchip.build()
+    return acchip
+
+
+def test_library_exports_every_declared_symbol(A):
+    """every function include/acc_hip.h declares is exported by the shared library"""
+    with open(os.path.join(ROOT, "include", "acc_hip.h")) as fh:
+        text = fh.read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    declared = set(re.findall(r"\b(acc_[a-z0-9_]+)\s*\(", text))
+    assert len(declared) >= 50
+    assert declared == set(A.SYMBOLS), declared ^ set(A.SYMBOLS)
+    out = subprocess.check_output(["nm", "-D", "--defined-only", A.LIB_PATH]).decode()
+    exported = set(re.findall(r" T (acc_[a-z0-9_]+)", out))
+    assert declared <= exported, declared - exported
+    L = A.lib()
+    for name in declared:
+        assert getattr(L, name) is not None
+    assert L.acc_version().decode().count(".") == 2
+
+
+def test_no_torch_types_and_no_oracle_in_the_product():
+    """the boundary is plain C and the product never reaches into oracle/"""
+    with open(os.path.join(ROOT, "include", "acc_hip.h")) as fh:
+        hdr = re.sub(r"/\*.*?\*/", "", fh.read(), flags=re.S)
+    assert "torch" not in hdr and "std::" not in hdr and "at::" not in hdr
+    pkg = os.path.join(ROOT, "accelerate-cuda_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".cpp", ".hpp", ".h")):
+                with open(os.path.join(dirpath, f)) as fh:
+                    assert "oracle" not in fh.read().lower(), os.path.join(dirpath, f)
+
+
+def test_every_skeleton_instance_compiles_for_gfx950(A, tmp_path):
+    import __graft_entry__ as g
+    A.lib().acc_cache_set_dir(str(tmp_path).encode())
+    inst = g.standard_instances(A)
+    assert len(inst) >= 18
+    for name, desc in inst.items():
+        assert A.compile_only(desc, "gfx950") > 4000, name
+
+
+def test_kernel_cache_hit_miss_and_corruption(A, tmp_path):
+    L = A.lib()
+    d = str(tmp_path / "cache")
+    L.acc_cache_set_dir(d.encode())
+    assert L.acc_cache_dir().decode() == d
+    src = b'extern "C" __global__ void k(float *p) { p[threadIdx.x] = 1.0f; }\n'
+    opts = (C.c_char_p * 1)(b"-O3")
+    code, size = C.c_void_p(), C.c_size_t()
+
+    def compile_(source=src, options=opts, n=1, target=b"gfx950"):
+        A.check(L.acc_compile(None, target, source, options, n, C.byref(code), C.byref(size)))
+        return C.string_at(code, size.value)
+
+    s0 = A.cache_stats()
+    obj = compile_()
+    assert obj[:4] == b"\x7fELF"
+    s1 = A.cache_stats()
+    assert s1["compiles"] == s0["compiles"] + 1
+    files = [os.path.join(dp, f) for dp, _, fs in os.walk(d) for f in fs]
+    assert len(files) == 1 and files[0].endswith(".co") and os.sep + "gfx950" + os.sep in files[0]
+    # same text: found in memory
+    assert compile_() == obj
+    assert A.cache_stats()["ram_hits"] == s1["ram_hits"] + 1
+    # memory table emptied: found on disk, not compiled again
+    L.acc_cache_clear(0)
+    assert compile_() == obj
+    s2 = A.cache_stats()
+    assert s2["disk_hits"] == s1["disk_hits"] + 1 and s2["compiles"] == s1["compiles"]
+    # anything that decides the object changes the key: text, options, target
+    compile_(source=src + b"// x\n")
+    compile_(options=(C.c_char_p * 1)(b"-O2"))
+    compile_(target=b"gfx942")
+    s3 = A.cache_stats()
+    assert s3["compiles"] == s2["compiles"] + 3
+    assert len([f for dp, _, fs in os.walk(d) for f in fs]) == 4
+    # a damaged entry (truncated, then bit-flipped) is detected, removed and rebuilt
+    for damage in ("truncate", "flip"):
+        L.acc_cache_clear(0)
+        with open(files[0], "rb") as fh:
+            blob = bytearray(fh.read())
+        if damage == "truncate":
+            blob = blob[:len(blob) // 2]
+        else:
+            blob[-10] ^= 0x40
+        with open(files[0], "wb") as fh:
+            fh.write(bytes(blob))
+        before = A.cache_stats()
+        assert compile_() == obj
+        after = A.cache_stats()
+        assert after["compiles"] == before["compiles"] + 1 and after["disk_errors"] == before["disk_errors"] + 1
+        with open(files[0], "rb") as fh:
+            assert fh.read(8) == b"ACCHIPCO"
+    # an unusable directory degrades to memory only, it never fails a compile
+    L.acc_cache_clear(0)
+    L.acc_cache_set_dir(b"/proc/definitely/not/writable")
+    assert compile_() == obj
+    L.acc_cache_set_dir(b"")
+    assert compile_(source=src + b"// y\n")[:4] == b"\x7fELF"
+    # clear(also_disk) removes what this process put there
+    L.acc_cache_set_dir(d.encode())
+    compile_(source=src + b"// z\n")
+    n_before = len([f for dp, _, fs in os.walk(d) for f in fs])
+    L.acc_cache_clear(1)
+    assert len([f for dp, _, fs in os.walk(d) for f in fs]) < n_before
+
+
+def test_compile_error_is_a_status_with_a_log(A):
+    L = A.lib()
+    L.acc_cache_set_dir(b"")
+    code, size = C.c_void_p(), C.c_size_t()
+    rc = L.acc_compile(None, b"gfx950", b"this is not HIP\n", None, 0, C.byref(code), C.byref(size))
+    assert rc == A.ERR_COMPILE
+    assert "error" in L.acc_compile_log().decode()
+    assert "compilation failed" in L.acc_last_error().decode()
+    # a bad scalar fragment surfaces the same way through the skeleton layer
+    bad = A.make_desc(A.SKEL_MAP, "float", env=[(1, "float")], out_rank=1, get="arrIn0_0[ix] +* 2")
+    with pytest.raises(A.AccError) as e:
+        A.compile_only(bad)
+    assert e.value.code == A.ERR_COMPILE and "error" in L.acc_compile_log().decode()
+    assert L.acc_compile(None, None, b"x", None, 0, C.byref(code), C.byref(size)) == A.ERR_INVALID
+    assert L.acc_compile(None, b"gfx950; rm -rf", b"x", None, 0, C.byref(code), C.byref(size)) == A.ERR_INVALID
+
+
+def test_descriptions_are_validated(A):
+    F32 = (1, "float")
+    cases = [
+        (dict(kind=A.SKEL_FOLD, elt="float", env=[F32], get="arrIn0_0[ix]", combine="x + y"), "seed"),            # fold needs a seed
+        (dict(kind=A.SKEL_FOLD1, elt="float", env=[F32], get="arrIn0_0[ix]", combine="x + y", seed="0"), "no seed"),
+        (dict(kind=A.SKEL_SCANL, elt="float", env=[F32], get="arrIn0_0[ix]", seed="0"), "combine"),
+        (dict(kind=A.SKEL_MAP, elt="float", env=[F32], out_rank=1), "get"),
+        (dict(kind=A.SKEL_MAP, elt="quaternion", env=[F32], out_rank=1, get="0"), "elt_size"),
+        (dict(kind=A.SKEL_PERMUTE, elt="Int32", env=[], out_rank=0, get="1", combine="x+y", permutation="0"), "rank-0"),  # IndexSpace.hs:230
+        (dict(kind=A.SKEL_PERMUTE, elt="Int16", env=[], out_rank=1, get="1", combine="x+y", permutation="0", elt_size=2), "atomic"),
+        (dict(kind=A.SKEL_PERMUTE, elt="float", env=[], out_rank=1, get="1", combine="x", permutation="0", combine_hint=A.COMBINE_XOR), "bitwise"),
+        (dict(kind=A.SKEL_STENCIL, elt="float", out_rank=3, taps=[(0, 0)], stencil_fn="t0"), "rank 3"),
+        (dict(kind=A.SKEL_STENCIL, elt="float", out_rank=2, taps=[(0, 9)], stencil_fn="t0"), "offset"),
+        (dict(kind=99, elt="float"), "unknown"),
+    ]
+    for kw, needle in cases:
+        with pytest.raises(A.AccError) as e:
+            A.compile_only(A.make_desc(**kw))
+        assert e.value.code in (A.ERR_INVALID, A.ERR_UNSUPPORTED), kw
+        assert needle in e.value.message, (needle, e.value.message)
+
+
+def test_generated_parameter_abi_follows_the_reference(A):
+    """free array variables first in Gamma order, per array the extents
+    outermost first then the components highest first, then the result group
+    (CodeGen/Base.hs:69-89,344-357,376-383); entry names as CodeGen builds them."""
+    env = [(2, ["float", "Int32"]), (1, "double")]
+    d = A.make_desc(A.SKEL_MAP, "float", env=env, out_rank=2, get="arrIn0_1[ix] + (float)arrIn1_0[0]")
+    entry, src = A.preview(d)
+    assert entry == "map"
+    defs = dict(m.groups() for m in re.finditer(r"^#define (\w+)(?:\([^)]*\))? (.*)$", src, flags=re.M))
+    assert defs["ACC_ENV_PARAMS"].strip() == (
+        "const Int64 shIn0_1, const Int64 shIn0_0, const Int32 *__restrict__ arrIn0_1, "
+        "const float *__restrict__ arrIn0_0, const Int64 shIn1_0, const double *__restrict__ arrIn1_0,")
+    assert defs["ACC_OUT_PARAMS"].strip() == "const Int64 shOut_1, const Int64 shOut_0, float *__restrict__ arrOut_0"
+    assert defs["ACC_OUT_SIZE"].strip() == "(shOut_1 * shOut_0)"
+    assert src.rstrip().endswith('#include "skel_map.h"') and '#include "acc_hip_device.h"' in src
+    assert "__builtin_assume_aligned" in src and "__builtin_assume_aligned" not in A.preview(d, 1)[1]
+    assert A.compile_only(d) > 0
+    # entry names as the reference builds them: PrefixSum.hs:311, Reduction.hs:188,554, IndexSpace.hs:55,109,171, Mapping.hs:49
+    I32 = (1, "Int32")
+    expect = [(A.SKEL_SCANL, "0", "scanl"), (A.SKEL_SCANL1, None, "scanl1"), (A.SKEL_SCANLP, "0", "scanl"),
+              (A.SKEL_SCANR, "0", "scanr"), (A.SKEL_SCANR1, None, "scanr1"), (A.SKEL_SCANRP, "0", "scanr"),
+              (A.SKEL_FOLD, "0", "foldAll"), (A.SKEL_FOLD1, None, "fold1All"),
+              (A.SKEL_FOLDSEG, "0", "foldSeg"), (A.SKEL_FOLD1SEG, None, "fold1Seg")]
+    for kind, seed, name in expect:
+        e, _ = A.preview(A.make_desc(kind, "Int32", env=[I32], get="arrIn0_0[ix]", combine="x + y", seed=seed))
+        assert e == name
+    assert A.preview(A.make_desc(A.SKEL_FOLD, "Int32", env=[(2, "Int32")], out_rank=1, get="arrIn0_0[ix]", combine="x+y", seed="0"))[0] == "fold"
+    assert A.preview(A.make_desc(A.SKEL_GENERATE, "Int32", out_rank=1, get="0"))[0] == "generate"
+    assert A.preview(A.make_desc(A.SKEL_TRANSFORM, "Int32", env=[I32], out_rank=1, get="arrIn0_0[ix]"))[0] == "transform"
+    assert A.preview(A.make_desc(A.SKEL_PERMUTE, "Int32", env=[I32], out_rank=1, get="1", combine="x+y", permutation="arrIn0_0[ix]"))[0] == "permute"
+    # multi-line fragments are flattened so that they fit a #define
+    _, src = A.preview(A.make_desc(A.SKEL_MAP, "float", env=[(1, "float")], out_rank=1, get="({ const float a = arrIn0_0[ix];\n a * a; })"))
+    assert "#define ACC_GET(ix) ({ const float a = arrIn0_0[ix];  a * a; })" in src
+    # tuning knobs reach the text (and so the cache key)
+    os.environ["ACC_HIP_TUNE"] = "scan.block=512,scan.rows=2"
+    try:
+        _, src = A.preview(A.make_desc(A.SKEL_SCANL, "Int32", env=[I32], get="arrIn0_0[ix]", combine="x + y", seed="0"))
+    finally:
+        del os.environ["ACC_HIP_TUNE"]
+    assert "#define ACC_BLOCK 512" in src and "#define ACC_ROWS 2" in src
+
+
+def test_launch_arithmetic(A):
+    """split / maxGrid of Analysis/Launch.hs:51-55,124-128"""
+    g = A.lib().acc_launch_grid
+    assert g(0, 256, 256, 8) == 1                 # at least one block, so that empty folds still write their seed
+    assert g(1, 256, 256, 8) == 1
+    assert g(256, 256, 256, 8) == 1
+    assert g(257, 256, 256, 8) == 2
+    assert g(1 << 26, 4096, 256, 8) == 2048       # capped at what is resident
+    assert g(1 << 26, 4096, 256, 1 << 20) == 16384
+    assert g(100, 0, 1, 1) == 1                   # degenerate arguments do not divide by zero
+
+
+def test_without_a_gpu_the_runtime_reports_an_error_not_a_crash(A):
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    L = A.lib()
+    n = C.c_int(-1)
+    rc = L.acc_device_count(C.byref(n))
+    h = C.c_void_p()
+    rc2 = L.acc_context_create(0, C.byref(h))
+    assert (rc != A.OK or n.value == 0) and rc2 != A.OK and not h.value
+    assert len(L.acc_last_error()) > 0
+    with pytest.raises(A.AccError):
+        A.Context(0)
+
+
+def test_workload_module_is_pure_numpy():
+    import workloads as wl
+    x, y = wl.dot_inputs(1000)
+    assert x.dtype == np.float32 and x.shape == (1000,) and not np.array_equal(x, y)
+    vals, cols, offs, lens, xv = wl.smvm_inputs(nrows=500, mean_len=8, ncols=64)
+    assert offs[0] == 0 and offs[-1] == vals.size == cols.size and np.array_equal(np.diff(offs), lens)
+    assert cols.min() >= 0 and cols.max() < 64 and xv.size == 64
