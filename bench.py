@@ -24,6 +24,7 @@ for p in (ROOT, os.path.join(ROOT, "accelerate-cuda_amd")):
 import numpy as np  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
+SCANL_HBM_TRAFFIC_BYTES = 542100000
 
 
 def log(*a):
@@ -278,7 +279,10 @@ def main():
         "dtype": "int32", "data": "synthetic (seeded SplitMix64, resident in HBM before the timed region)",
         "config": {"workload": workload, "elements": n, "timing": "kernel launches back to back on one stream, inputs device-resident"},
         "roofline": {"bound": "hbm", "achieved": headline["GB_per_s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(headline["GB_per_s"] / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(headline["GB_per_s"] / HBM_PEAK_GBS, 4),
+                     # HBM bytes per scanl launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the
+                     # plain copy of the same size: profiles/scan_2p26_hbm_traffic_pmc.txt
+                     "traffic": SCANL_HBM_TRAFFIC_BYTES if workload.startswith("configs[1]") else None,
                      "kernel": "scanl", "avg_launch_us": headline["avg_launch_us"],
                      "algorithmic_bytes_per_launch": headline["algorithmic_bytes_per_launch"]},
         "cpu_baseline": cpu,
