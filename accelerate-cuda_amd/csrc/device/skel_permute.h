@@ -23,6 +23,11 @@
  *     millions of atomics, a thousand to the same address -- as a plain dump of
  *     the block's bins into a table that a second kernel, permute_merge, folds
  *     column by column into the result.
+ *   - targets beyond the LDS window (the tail of a skewed histogram) are
+ *     updated in one table row per XCD, shared by the workgroups running
+ *     there: a few hundred KB that stay in that XCD's L2, where its atomics
+ *     execute, instead of device-scope atomics that each travel to memory.
+ *     permute_merge folds those rows into the result as well.
  * The new value is the FIRST operand of combine (IndexSpace.hs:207).  Updates
  * arrive in no particular order, as in the reference, so combine must be
  * associative and commutative.  Targets outside the result are dropped.
@@ -110,13 +115,22 @@ ACC_DEV void acc_hint_apply(T *p, const T &x, F combine)
 #define ACC_SCOPE_BLOCK  __HIP_MEMORY_SCOPE_WORKGROUP
 #define ACC_SCOPE_DEVICE __HIP_MEMORY_SCOPE_AGENT
 
-/* dump == NULL            : privatised bins are flushed into the result with atomics
- * dump, cols == lds_bins  : privatised bins are dumped to row blockIdx.x of the table
- * dump, cols == target    : additionally the targets beyond the LDS window are
- *                           privatised in the rest of this block's table row   */
+/* The XCD this workgroup runs on (hardware register XCC_ID, bits 3:0).  Every
+ * XCD has an L2 of its own, and global atomics execute in the L2 of the XCD
+ * that issues them. */
+ACC_DEV int acc_xcd_id() { return (int)(__builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11)) & 15u); }
+#define ACC_XCD_ROWS 16
+
+/* dump == NULL : privatised bins are flushed into the result with atomics
+ * dump         : privatised bins are dumped to row blockIdx.x of the table dump[gridDim.x][lds_bins]
+ * far == NULL  : targets beyond the LDS window are updated in the result with device-scope atomics
+ * far          : ... in row acc_xcd_id() of far[ACC_XCD_ROWS][target size] (filled with the combine's
+ *                identity beforehand), shared by the workgroups of one XCD.  Their atomics meet in
+ *                that XCD's L2, where the row stays resident, and need no wider scope than that
+ *                cache; the rows reach memory when the kernel ends.                                */
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, const int lds_copies,
-        ACC_ELT *__restrict__ dump, const int dump_cols)
+        ACC_ELT *__restrict__ dump, ACC_ELT *__restrict__ far)
 {
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
@@ -130,20 +144,18 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
   const Int64 n = shIn_0;
   const Int64 ntarget = (ACC_OUT_SIZE);
   const T ident = acc_hint_identity<T>();
-  T *row = dump ? dump + (Int64)blockIdx.x * dump_cols : (T *)0;
-  const bool private_tail = dump && dump_cols > lds_bins;
+  T *row = dump ? dump + (Int64)blockIdx.x * lds_bins : (T *)0;
+  T *far_row = far ? far + (Int64)acc_xcd_id() * ntarget : (T *)0;
 
   for (int i = threadIdx.x; i < lds_bins * lds_copies; i += ACC_BLOCK) bins[i] = ident;
-  if (private_tail)
-    for (int i = lds_bins + threadIdx.x; i < dump_cols; i += ACC_BLOCK) row[i] = ident;
   __syncthreads();
   T *mine = bins + ((threadIdx.x >> 6) % lds_copies) * lds_bins;
 
   auto update = [&](const Int64 j, const T &x) {
     if (j < 0 || j >= ntarget) return;            /* `ignore`, or outside the result */
-    if (j < lds_bins)      acc_hint_apply<ACC_SCOPE_BLOCK>(mine + j, x, f);
-    else if (private_tail) acc_hint_apply<ACC_SCOPE_BLOCK>(row + j, x, f);
-    else                   acc_hint_apply<ACC_SCOPE_DEVICE>(arrOut_0 + j, x, f);
+    if (j < lds_bins) acc_hint_apply<ACC_SCOPE_BLOCK>(mine + j, x, f);
+    else if (far_row) acc_hint_apply<ACC_SCOPE_BLOCK>(far_row + j, x, f);
+    else              acc_hint_apply<ACC_SCOPE_DEVICE>(arrOut_0 + j, x, f);
   };
 
   /* full tiles, software-pipelined: the next tile's indices and values are
@@ -209,33 +221,43 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
   }
 }
 
-/* folds the table dump[nblocks][cols] into out[0 .. cols).  The rows are split
- * into `slices` groups handled by different workgroups; with one slice the
- * result is written plainly, otherwise each group applies its share with one
- * atomic per target.                                                         */
+/* fills p[0 .. count) with the combine's identity */
 extern "C" __global__ void __launch_bounds__(256)
-permute_merge(ACC_ENV_PARAMS ACC_OUT_PARAMS, const ACC_ELT *__restrict__ dump, const int cols, const int nblocks,
-              const int slices)
+permute_fill(ACC_ELT *__restrict__ p, const Int64 count)
+{
+  const ACC_ELT ident = acc_hint_identity<ACC_ELT>();
+  for (Int64 i = (Int64)blockIdx.x * 256 + threadIdx.x; i < count; i += (Int64)gridDim.x * 256) p[i] = ident;
+}
+
+/* folds columns [first, first + cols) of the table dump[nrows][stride] into the
+ * same positions of the result.  The rows are split into `slices` groups
+ * handled by different workgroups; with one slice the result is written
+ * plainly, otherwise each group applies its share with one atomic per target. */
+extern "C" __global__ void __launch_bounds__(256)
+permute_merge(ACC_ENV_PARAMS ACC_OUT_PARAMS, const ACC_ELT *__restrict__ dump, const Int64 stride, const Int64 first,
+              const Int64 cols, const int nrows, const int slices)
 {
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
   auto f = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
-  const int column = (int)(blockIdx.x / slices) * 256 + threadIdx.x;
+  const Int64 column = (Int64)(blockIdx.x / slices) * 256 + threadIdx.x;
   const int slice = (int)(blockIdx.x % slices);
   if (column >= cols) return;
-  const int per = (nblocks + slices - 1) / slices;
-  const int r0 = slice * per, r1 = acc_min(nblocks, r0 + per);
+  const int per = (nrows + slices - 1) / slices;
+  const int r0 = slice * per, r1 = acc_min(nrows, r0 + per);
   if (r0 >= r1) return;
-  T acc = dump[(Int64)r0 * cols + column];
+  const T *src = dump + first + column;
+  T acc = src[(Int64)r0 * stride];
 #pragma unroll 8
-  for (int r = r0 + 1; r < r1; ++r) acc = f(dump[(Int64)r * cols + column], acc);
+  for (int r = r0 + 1; r < r1; ++r) acc = f(src[(Int64)r * stride], acc);
+  T *dst = arrOut_0 + first + column;
   if (slices == 1) {
-    arrOut_0[column] = f(acc, arrOut_0[column]);
+    *dst = f(acc, *dst);
   } else {
     const T ident = acc_hint_identity<T>();
     typename acc_bits<sizeof(T)>::type a, b;
     __builtin_memcpy(&a, &acc, sizeof(T));
     __builtin_memcpy(&b, &ident, sizeof(T));
-    if (a != b) acc_hint_apply<ACC_SCOPE_DEVICE>(arrOut_0 + column, acc, f);
+    if (a != b) acc_hint_apply<ACC_SCOPE_DEVICE>(dst, acc, f);
   }
 }

@@ -448,8 +448,15 @@ ACC_DEV void acc_scan_tile_ragged(const T (&x)[ACC_ROWS][ACC_VEC], Op op_raw, co
  * ACC_SCAN_PERSISTENT == 1  a resident grid of workgroups draws tile numbers
  *   from an atomic counter (two tiles ahead, so the atomic's round trip is
  *   never waited for) and loads the next tile's elements while the current
- *   tile waits for its prefix.                                              */
-extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+ *   tile waits for its prefix.
+ * ACC_SCAN_PERSISTENT == 2  the same without the counter: workgroup b takes
+ *   tiles b, b + grid, b + 2 grid, ...  Only valid under a cooperative launch,
+ *   which guarantees that the whole grid is resident at once.               */
+/* second launch bound = waves per SIMD the register allocation must leave room for */
+#ifndef ACC_MIN_WAVES
+#define ACC_MIN_WAVES 1
+#endif
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK, ACC_MIN_WAVES)
 ACC_ENTRY(ACC_ENV_PARAMS
           const Int64 shOut_0, ACC_ELT *__restrict__ arrOut_0,
           ACC_ELT *__restrict__ arrSum_0,
@@ -483,7 +490,7 @@ ACC_ENTRY(ACC_ENV_PARAMS
   const acc_scan_desc<T> desc(desc0, desc1, desc2);
   auto tile_base = [&](const Int64 t) -> Int64 { return (ACC_SCAN_RIGHT ? (num_tiles - 1 - t) : t) * (Int64)ACC_TILE; };
 
-#if ACC_SCAN_PERSISTENT
+#if ACC_SCAN_PERSISTENT == 1
   __shared__ unsigned int s_ticket[4];
   unsigned int pending = 0;
   if (threadIdx.x == 0) {
@@ -509,7 +516,7 @@ ACC_ENTRY(ACC_ENV_PARAMS
   T cur[ACC_ROWS][ACC_VEC];
   if (tile < num_tiles) acc_scan_load(get, tile_base(tile), n, cur, wave, lane);
 
-#if ACC_SCAN_PERSISTENT
+#if ACC_SCAN_PERSISTENT == 1
   T nxt[ACC_ROWS][ACC_VEC];
   int slot = 1;
   while (tile < num_tiles) {
@@ -522,6 +529,13 @@ ACC_ENTRY(ACC_ENV_PARAMS
     Int64 next = num_tiles;
     auto prefetch = [&]() {
       next = (Int64)s_ticket[slot];
+      if (next < num_tiles) acc_scan_load(get, tile_base(next), n, nxt, wave, lane);
+    };
+#elif ACC_SCAN_PERSISTENT == 2
+  T nxt[ACC_ROWS][ACC_VEC];
+  while (tile < num_tiles) {
+    Int64 next = tile + gridDim.x;
+    auto prefetch = [&]() {
       if (next < num_tiles) acc_scan_load(get, tile_base(next), n, nxt, wave, lane);
     };
 #else
@@ -541,7 +555,9 @@ ACC_ENTRY(ACC_ENV_PARAMS
 #pragma unroll
       for (int k = 0; k < ACC_VEC; ++k) cur[r][k] = nxt[r][k];
     tile = next;
+#if ACC_SCAN_PERSISTENT == 1
     slot = (slot + 1) & 3;
+#endif
     __syncthreads();          /* s_wave and s_prefix are free for the next tile */
 #endif
   }

@@ -93,7 +93,15 @@ stencil(ACC_ENV_PARAMS ACC_OUT_PARAMS, const ACC_IN_ELT *__restrict__ arrStencil
 #else
   const Int64 strip = (Int64)blockIdx.x * ACC_WAVES + (threadIdx.x >> 6);
 #endif
+#if ACC_STACK_WAVES
+  /* the waves of a workgroup take vertically adjacent strips: the boundary
+   * rows they share are then requested from the same compute unit, where the
+   * second request merges with the first instead of going out to memory */
+  const Int64 group = strip / ACC_WAVES, within = strip % ACC_WAVES;
+  const Int64 y0 = ((group / strips_x) * ACC_WAVES + within) * ACC_TILE_H, x0 = (group % strips_x) * ACC_STRIP;
+#else
   const Int64 y0 = (strip / strips_x) * ACC_TILE_H, x0 = (strip % strips_x) * ACC_STRIP;
+#endif
   if (y0 >= h) return;                                   /* whole wave leaves together */
   const Int64 gx = x0 + lane * ACC_SVEC;
   const int rows = (int)acc_min<Int64>(ACC_TILE_H, h - y0);

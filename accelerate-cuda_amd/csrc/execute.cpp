@@ -266,11 +266,12 @@ int acc_exec_scan(acc_skel s, const acc_array *env, int64_t n, const acc_array *
   const int64_t tiles = (n + tile - 1) / tile;
   int64_t grid = std::max<int64_t>(1, tiles);     // one workgroup per tile, in dispatch order ...
   int64_t draws = 0;
-  if (acc::tune("scan.persistent", 0)) {
+  const int persistent = acc::tune("scan.persistent", 0);
+  if (persistent) {
     // ... or a resident grid of persistent workgroups, each drawing tiles until none are left
     const int64_t per_cu = std::max(1, std::min(s->variants[v].blocks_per_cu, acc::tune("scan.blocks_per_cu", 2)));
     grid = std::max<int64_t>(1, std::min<int64_t>(tiles, (int64_t)s->ctx->props.multiProcessorCount * per_cu));
-    draws = tiles + 2 * grid;                     // every tile once, plus two draws ahead per workgroup
+    draws = persistent == 1 ? tiles + 2 * grid : 0;   // every tile once, plus two draws ahead per workgroup
   }
   const int64_t ndesc = std::max<int64_t>(1, tiles);
   const size_t esz = s->spec.elt_size;
@@ -308,7 +309,18 @@ int acc_exec_scan(acc_skel s, const acc_array *env, int64_t n, const acc_array *
   args.ptr(reinterpret_cast<uint64_t>(base + off_d2));
   args.u32(epoch);
   args.i64(tiles);
-  const int rc = launch(s, v, grid, 0, st, &args);
+  int rc;
+  if (persistent == 2) {
+    // static tile assignment needs every workgroup resident at once: a cooperative launch promises that
+    rc = s->ctx->make_current();
+    if (rc == ACC_OK) {
+      hipError_t e = hipModuleLaunchCooperativeKernel(s->variants[v].fn, static_cast<unsigned>(grid), 1, 1,
+                                                      static_cast<unsigned>(s->spec.block), 1, 1, 0, st, args.data());
+      if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchCooperativeKernel(scan)");
+    }
+  } else {
+    rc = launch(s, v, grid, 0, st, &args);
+  }
   if (rc != ACC_OK) {
     // nothing ran: take the tickets back so that the block stays consistent
     std::lock_guard<std::mutex> lock(s->ctx->mu);
@@ -362,43 +374,60 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
   if (e != hipSuccess || bpc < 1) { (void)hipGetLastError(); bpc = 1; }
   const int64_t grid = acc_launch_grid(n_src, s->elements_per_block(), cus, std::min(bpc, acc::tune("permute.max_blocks_per_cu", 1)));
 
-  // how the privatised part leaves the blocks: atomics while they are few,
-  // otherwise a table of per-block bins folded by a second kernel
-  // Targets beyond the LDS window would be hit with device-scope atomics, the
-  // slowest operation on the machine; if a whole table row per block is
-  // affordable, they are privatised there instead (block-scope atomics in L2).
-  const bool private_tail = bins > 0 && bins < ntarget && ntarget < (1 << 30) &&
-                            (int64_t)grid * ntarget * (int64_t)esz <= (int64_t)acc::tune("permute.table_mbytes", 256) << 20;
-  const bool table = private_tail || (bins > 0 && grid * bins > acc::tune("permute.atomic_flush_max", 1 << 16));
-  const int64_t cols = private_tail ? ntarget : bins;
+  // How the privatised part leaves the blocks: atomics while they are few, otherwise a table of
+  // per-block bins folded by a second kernel.
+  // Targets beyond the LDS window would be hit with device-scope atomics, the slowest operation on
+  // the machine.  While a row of the whole target stays well inside one XCD's L2, the workgroups of
+  // each XCD share such a row instead, and the rows are folded into the result afterwards.
+  constexpr int64_t XCD_ROWS = 16;                 // what the kernel's XCC_ID field can name
+  const bool far_rows = bins > 0 && bins < ntarget &&
+                        ntarget * (int64_t)esz <= (int64_t)acc::tune("permute.xcd_row_kbytes", 1024) << 10;
+  const bool table = bins > 0 && grid * bins > acc::tune("permute.atomic_flush_max", 1 << 16);
+  const size_t far_bytes = far_rows ? (size_t)(XCD_ROWS * ntarget) * esz : 0;
+  const size_t dump_bytes = table ? (size_t)(grid * bins) * esz : 0;
   int blk = -1;
-  uint64_t dump = 0;
-  if (table) {
-    ACC_TRY(s->ctx->scratch_acquire((size_t)(grid * cols) * esz, st, acc::SCRATCH_FOLD, &blk));
-    dump = reinterpret_cast<uint64_t>(s->ctx->scratch[blk].ptr);
+  uint64_t far = 0, dump = 0;
+  if (far_rows || table) {
+    ACC_TRY(s->ctx->scratch_acquire(far_bytes + dump_bytes, st, acc::SCRATCH_FOLD, &blk));
+    const uint64_t base = reinterpret_cast<uint64_t>(s->ctx->scratch[blk].ptr);
+    if (far_rows) far = base;
+    if (table) dump = base + far_bytes;
+  }
+  int rc = ACC_OK;
+  if (far_rows) {
+    Args f;
+    f.ptr(far);
+    f.i64(XCD_ROWS * ntarget);
+    const int64_t fill_grid = std::min<int64_t>((XCD_ROWS * ntarget + 255) / 256, 8 * (int64_t)cus);
+    e = hipModuleLaunchKernel(s->variants[v].fn_fill, static_cast<unsigned>(fill_grid), 1, 1, 256, 1, 1, 0, st, f.data(), nullptr);
+    if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(permute_fill)");
   }
   args.i32(static_cast<int32_t>(bins));
   args.i32(static_cast<int32_t>(copies));
   args.ptr(dump);
-  args.i32(static_cast<int32_t>(cols));
-  int rc = launch(s, v, grid, lds, st, &args);
-  if (rc == ACC_OK && table) {
+  args.ptr(far);
+  if (rc == ACC_OK) rc = launch(s, v, grid, lds, st, &args);
+  // folds columns [first, first + cols) of a table of `rows` rows into the result
+  auto merge = [&](uint64_t tbl, int64_t stride, int64_t first, int64_t cols, int64_t rows) -> int {
     Args m;
     bool al = true;
-    rc = push_env(s, env, &m, &al);
+    ACC_TRY(push_env(s, env, &m, &al));
     push_out(*out, &m, &al);
     // enough workgroups to fill the machine: columns x row slices
     const int64_t columns = (cols + 255) / 256;
-    const int64_t slices = std::max<int64_t>(1, std::min<int64_t>(grid, (2 * cus + columns - 1) / columns));
-    m.ptr(dump);
-    m.i32(static_cast<int32_t>(cols));
-    m.i32(static_cast<int32_t>(grid));
+    const int64_t slices = std::max<int64_t>(1, std::min<int64_t>(rows, (2 * cus + columns - 1) / columns));
+    m.ptr(tbl);
+    m.i64(stride);
+    m.i64(first);
+    m.i64(cols);
+    m.i32(static_cast<int32_t>(rows));
     m.i32(static_cast<int32_t>(slices));
-    if (rc == ACC_OK) {
-      e = hipModuleLaunchKernel(s->variants[v].fn_finish, static_cast<unsigned>(columns * slices), 1, 1, 256, 1, 1, 0, st, m.data(), nullptr);
-      if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(permute_merge)");
-    }
-  }
+    hipError_t me = hipModuleLaunchKernel(s->variants[v].fn_finish, static_cast<unsigned>(columns * slices), 1, 1, 256, 1, 1, 0, st, m.data(), nullptr);
+    if (me != hipSuccess) return acc::fail_hip(me, "hipModuleLaunchKernel(permute_merge)");
+    return ACC_OK;
+  };
+  if (rc == ACC_OK && table) rc = merge(dump, bins, 0, bins, grid);
+  if (rc == ACC_OK && far_rows) rc = merge(far, ntarget, bins, ntarget - bins, XCD_ROWS);
   if (blk >= 0) s->ctx->scratch_release(blk, st);
   return rc;
 }
@@ -419,9 +448,12 @@ static int stencil_once(acc_skel s, const acc_array *env, const acc_array *in, c
   const size_t in_esz = acc::type_size(s->spec.stencil_in_type) ? acc::type_size(s->spec.stencil_in_type) : s->spec.elt_size;
   if ((w * (int64_t)s->spec.elt_size) % 16 != 0 || (w * (int64_t)in_esz) % 16 != 0) aligned = false;
   // one wave per strip of 256 columns x tile_h rows
-  const int64_t strips = ((w + s->spec.tile_w - 1) / s->spec.tile_w) * ((h + s->spec.tile_h - 1) / s->spec.tile_h);
+  // (for 2-D the waves of a workgroup are stacked vertically, so the row count is rounded up to whole groups)
   const int64_t waves = s->spec.block / 64;
-  return launch(s, aligned ? 0 : 1, (strips + waves - 1) / waves, 0, st, &args);
+  const int64_t strips_x = (w + s->spec.tile_w - 1) / s->spec.tile_w;
+  int64_t bands = (h + s->spec.tile_h - 1) / s->spec.tile_h;
+  if (rank == 2 && acc::tune("stencil.stack", 0)) bands = (bands + waves - 1) / waves * waves;
+  return launch(s, aligned ? 0 : 1, (strips_x * bands + waves - 1) / waves, 0, st, &args);
 }
 
 static int stencil_check(acc_skel s, const acc_array *in, const acc_array *out)

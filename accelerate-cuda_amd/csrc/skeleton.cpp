@@ -174,7 +174,8 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "#define ACC_LOOKBACK " << tune("scan.lookback", 1) << "\n";
       o << "#define ACC_DESC_STRIDE " << tune("scan.desc_stride", 16) << "\n";
       if (tune("scan.debug_nolookback", 0)) o << "#define ACC_SCAN_DEBUG_NO_LOOKBACK 1\n";
-      o << "#define ACC_SCAN_PERSISTENT " << (tune("scan.persistent", 0) ? 1 : 0) << "\n";
+      o << "#define ACC_MIN_WAVES " << tune("scan.min_waves", 1) << "\n";
+      o << "#define ACC_SCAN_PERSISTENT " << tune("scan.persistent", 0) << "\n";
       tmpl = "skel_scan.h";
       break;
     }
@@ -208,6 +209,7 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "\n";
       o << "#define ACC_STENCIL_FN " << sp.stencil_fn << "\n";
       o << "#define ACC_XCD_REMAP " << tune("stencil.xcd_remap", 0) << "\n";
+      o << "#define ACC_STACK_WAVES " << (sp.out_rank == 2 ? tune("stencil.stack", 0) : 0) << "\n";
       o << "#define ACC_TILE_H " << sp.tile_h << "\n#define ACC_PREFETCH " << sp.prefetch << "\n#define ACC_BLOCK " << sp.block << "\n";
       tmpl = "skel_stencil.h";
       break;
@@ -384,6 +386,14 @@ int acc_skel_s::ensure_variant(int v)
       (void)hipModuleUnload(var.module);
       var.module = nullptr;
       return acc::fail_hip(e, ("hipModuleGetFunction(" + second + ")").c_str());
+    }
+  }
+  if (spec.kind == ACC_SKEL_PERMUTE) {
+    e = hipModuleGetFunction(&var.fn_fill, var.module, (entry + "_fill").c_str());
+    if (e != hipSuccess) {
+      (void)hipModuleUnload(var.module);
+      var.module = nullptr;
+      return acc::fail_hip(e, ("hipModuleGetFunction(" + entry + "_fill)").c_str());
     }
   }
   (void)hipFuncGetAttribute(&var.num_regs, HIP_FUNC_ATTRIBUTE_NUM_REGS, var.fn);

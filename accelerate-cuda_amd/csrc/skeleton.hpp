@@ -37,7 +37,8 @@ struct Variant {
   std::string source;
   hipModule_t module = nullptr;
   hipFunction_t fn = nullptr;
-  hipFunction_t fn_finish = nullptr;   // second kernel of a two-launch skeleton (foldAll)
+  hipFunction_t fn_finish = nullptr;   // second kernel of a two-launch skeleton (foldAll, permute's merge)
+  hipFunction_t fn_fill = nullptr;     // permute: fills table rows with the combine's identity
   int num_regs = 0;
   int static_lds = 0;
   int blocks_per_cu = 1;

@@ -201,7 +201,7 @@ def main():
         dk = ctx.array(keys)
         env = envs(dk)
         hist = ctx.skeleton(A.SKEL_PERMUTE, "Int32", env=[I32], out_rank=1, get="1", combine="x + y",
-                            permutation="arrIn0_0[ix]", combine_hint=A.COMBINE_ADD)
+                            permutation=os.environ.get("ACC_BENCH_HIST_PERM", "arrIn0_0[ix]"), combine_hint=A.COMBINE_ADD)
         dfl, out = ctx.array(np.zeros(bins, np.int32)), ctx.empty(bins, np.int32)
         dd, od = dfl.desc(), out.desc()
 
