@@ -197,6 +197,20 @@ ACC_DEV Int64 acc_xcd_contiguous_block()
  * the L2.  The code generator uses it for linear reads next to indirect ones. */
 template <typename T> ACC_DEV T acc_stream(const T *p, const Int64 ix) { return __builtin_nontemporal_load(p + ix); }
 
+/* the bulk stores of a streaming skeleton (a result that this kernel never
+ * reads back): non-temporal if the generator asks for it */
+#ifndef ACC_NT_STORE
+#define ACC_NT_STORE 0
+#endif
+template <typename T> ACC_DEV void acc_store(T *p, const T &v)
+{
+#if ACC_NT_STORE
+  __builtin_nontemporal_store(v, p);
+#else
+  *p = v;
+#endif
+}
+
 /* row-major index helpers (CodeGen/Base.hs:193-218): shapes and indices are
  * listed innermost dimension LAST, e.g. acc_to_index2(h, w, y, x)            */
 ACC_DEV Int64 acc_to_index2(Int64, Int64 w, Int64 y, Int64 x) { return y * w + x; }

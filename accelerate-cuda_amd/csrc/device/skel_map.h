@@ -45,7 +45,7 @@ ACC_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS)
 #pragma unroll
       for (int u = 0; u < ACC_UNROLL; ++u)
 #pragma unroll
-        for (int k = 0; k < ACC_VEC; ++k) arrOut_0[base + u * (ACC_BLOCK * ACC_VEC) + k] = v[u][k];
+        for (int k = 0; k < ACC_VEC; ++k) acc_store(arrOut_0 + (base + u * (ACC_BLOCK * ACC_VEC) + k), v[u][k]);
     } else {
 #pragma unroll
       for (int u = 0; u < ACC_UNROLL; ++u)

@@ -283,11 +283,7 @@ ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op_raw, const T s
     if (wave == 0) acc_scan_window_load(desc, tile - 1, lane, win);   /* ahead of the prefetch: results return in issue order */
     prefetch();
     if (wave == 0) {
-#ifdef ACC_SCAN_DEBUG_NO_LOOKBACK
-      const T p = S::val(block_total);
-#else
       const T p = acc_scan_lookback(desc, tile, S::val(block_total), op_raw, epoch, lane, win);
-#endif
       if (lane == 0) *s_prefix = p;
     }
     __syncthreads();
@@ -320,7 +316,7 @@ ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op_raw, const T s
     for (int k = 0; k < ACC_VEC; ++k) {
       const Int64 ix = ACC_SCAN_RIGHT ? ix0[r] - k : ix0[r] + k;
       if (PARTIAL && ix >= n) continue;
-      out[ix] = exclusive ? S::val(k == 0 ? pre : inc[k - 1]) : S::val(inc[k]);
+      acc_store(out + ix, exclusive ? S::val(k == 0 ? pre : inc[k - 1]) : S::val(inc[k]));
     }
 
     /* the reduction of the whole vector, held by the logically last element */

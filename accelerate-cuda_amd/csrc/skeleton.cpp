@@ -173,7 +173,6 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_ROWS " << sp.rows << "\n";
       o << "#define ACC_LOOKBACK " << tune("scan.lookback", 1) << "\n";
       o << "#define ACC_DESC_STRIDE " << tune("scan.desc_stride", 16) << "\n";
-      if (tune("scan.debug_nolookback", 0)) o << "#define ACC_SCAN_DEBUG_NO_LOOKBACK 1\n";
       o << "#define ACC_MIN_WAVES " << tune("scan.min_waves", 1) << "\n";
       o << "#define ACC_SCAN_PERSISTENT " << tune("scan.persistent", 0) << "\n";
       tmpl = "skel_scan.h";
@@ -218,6 +217,7 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       return fail(ACC_ERR_INVALID, "unknown skeleton kind %d", sp.kind);
   }
   o << "#define ACC_ENTRY " << *entry << "\n";
+  o << "#define ACC_NT_STORE " << tune("nt_store", 1) << "\n";
   o << "#include \"acc_hip_device.h\"\n";
   if (!sp.preamble.empty()) o << sp.preamble << "\n";
   o << "#include \"" << tmpl << "\"\n";

@@ -8,6 +8,11 @@ A step is one pass of a skeleton over its full-size synthetic input (for the
 iterated stencil: the ten applications).  The headline line is the prefix sum
 `scanl (+) 0` over 2^26 Int32; the other configurations are reported under
 "skeletons" in the same JSON line.  One GPU only.
+
+Consecutive steps work on DIFFERENT copies of the input and different result
+buffers (--sets of them, used round robin, together several times the 256 MB
+of the memory-side cache), so that no step finds the previous step's data in a
+cache: the figures are those of data that comes from and goes to HBM.
 """
 import argparse
 import ctypes as C
@@ -24,7 +29,7 @@ for p in (ROOT, os.path.join(ROOT, "accelerate-cuda_amd")):
 import numpy as np  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
-SCANL_HBM_TRAFFIC_BYTES = 542100000
+SCANL_HBM_TRAFFIC_BYTES = 542400000
 
 
 def log(*a):
@@ -41,13 +46,18 @@ class Timer(object):
         self.e0, self.e1 = ctx.event(True), ctx.event(True)
 
     def run(self, step):
-        for _ in range(self.warmup):
-            step()
+        """`step` is one callable, or a list of them (one per buffer set) taken round robin"""
+        steps = step if isinstance(step, (list, tuple)) else [step]
+        k = 0
+        for _ in range(max(self.warmup, len(steps))):
+            steps[k % len(steps)]()
+            k += 1
         self.ctx.sync()
         t0 = time.perf_counter()
         self.ctx.record(self.e0, self.stream)
         for _ in range(self.steps):
-            step()
+            steps[k % len(steps)]()
+            k += 1
         self.ctx.record(self.e1, self.stream)
         self.ctx.sync()
         wall_ms = (time.perf_counter() - t0) * 1e3 / self.steps
@@ -75,6 +85,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--only", type=str, default="")
+    ap.add_argument("--sets", type=int, default=4, help="copies of every configuration's buffers, used round robin")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -95,6 +106,11 @@ def main():
     F32, I32 = (1, "float"), (1, "Int32")
     sk = {}
     headline = None
+    S = max(1, args.sets)
+
+    def rd(k):
+        """fragment text for a linear read of input k at ix"""
+        return ("acc_stream(arrIn%d_0, ix)" if os.environ.get("ACC_BENCH_STREAM", "1") == "1" else "arrIn%d_0[ix]") % k
 
     def envs(*arrs):
         e = (A.acc_array * len(arrs))()
@@ -107,22 +123,22 @@ def main():
     if want("scan"):
         log("prefix sums over 2^26 Int32 ...")
         x = wl.scan_input(n)
-        dx = ctx.array(x)
-        env = envs(dx)
-        out = ctx.empty(n + 1, np.int32)
+        dxs = [ctx.array(x) for _ in range(S)]
+        env_s = [envs(d) for d in dxs]
+        outs = [ctx.empty(n + 1, np.int32) for _ in range(S)]
         for kind in ("scanl", "scanl1", "scanr"):
-            s = ctx.skeleton(A.SCAN_KINDS[kind], "Int32", env=[I32], get="arrIn0_0[ix]", combine="x + y",
-                             seed=None if kind == "scanl1" else "0")
-            od = out.desc(shape=(n + (0 if kind == "scanl1" else 1),))
+            s = ctx.skeleton(A.SCAN_KINDS[kind], "Int32", env=[I32], get=rd(0),
+                             combine="x + y", seed=None if kind == "scanl1" else "0")
+            ods = [o.desc(shape=(n + (0 if kind == "scanl1" else 1),)) for o in outs]
 
-            def step(s=s, od=od):
-                A.check(L.acc_exec_scan(s.handle, env, n, C.byref(od), None, stream))
-            w, e = T.run(step)
+            def step(i, s=s, ods=ods):
+                return lambda: A.check(L.acc_exec_scan(s.handle, env_s[i], n, C.byref(ods[i]), None, stream))
+            w, e = T.run([step(i) for i in range(S)])
             sk[kind] = result(kind + " (+) Int32 2^26", w, e, 1, 2 * n * 4 + 4, n)
             if kind == "scanl":
                 headline = dict(sk[kind], wall_ms=w, event_ms=e)
                 # size-independent check: the last element is the sum, the first the seed
-                got = out.get()
+                got = outs[S - 1].get()
                 if os.environ.get("ACC_BENCH_NOCHECK"):
                     continue
                 assert int(got[0]) == 0 and int(got[-1]) == int(x.sum(dtype=np.int64)), "scanl total mismatch"
@@ -140,7 +156,7 @@ def main():
                              "1 thread of %d host cores; an upper bound on the boxed Haskell interpreter" % (reps, os.cpu_count())}
         else:
             cpu = None
-        del dx, out, x
+        del dxs, outs, env_s, x
     else:
         cpu = None
 
@@ -148,49 +164,52 @@ def main():
     if want("map"):
         log("map: copy and zipWith (*) over 2^26 elements ...")
         x = wl.scan_input(n)
-        dx, out = ctx.array(x), ctx.empty(n, np.int32)
-        env = envs(dx)
-        cp = ctx.skeleton(A.SKEL_MAP, "Int32", env=[I32], out_rank=1, get="arrIn0_0[ix]")
-        od = out.desc()
+        dxs, outs = [ctx.array(x) for _ in range(S)], [ctx.empty(n, np.int32) for _ in range(S)]
+        env_s = [envs(d) for d in dxs]
+        cp = ctx.skeleton(A.SKEL_MAP, "Int32", env=[I32], out_rank=1, get=rd(0))
+        ods = [o.desc() for o in outs]
 
-        def step():
-            A.check(L.acc_exec_map(cp.handle, env, C.byref(od), stream))
-        w, e = T.run(step)
-        assert np.array_equal(out.get(), x)
+        def step(i):
+            return lambda: A.check(L.acc_exec_map(cp.handle, env_s[i], C.byref(ods[i]), stream))
+        w, e = T.run([step(i) for i in range(S)])
+        assert np.array_equal(outs[S - 1].get(), x)
         sk["map_copy"] = result("map id Int32 2^26 (copy)", w, e, 1, 2 * n * 4, n)
+        del dxs, outs, env_s
         fx = x.astype(np.float32)
-        dfx, dfy, fo = ctx.array(fx), ctx.array(fx[::-1].copy()), ctx.empty(n, np.float32)
-        env2 = envs(dfx, dfy)
-        zw = ctx.skeleton(A.SKEL_MAP, "float", env=[F32, F32], out_rank=1, get="arrIn0_0[ix] * arrIn1_0[ix]")
-        fod = fo.desc()
+        fy = fx[::-1].copy()
+        dfx, dfy, fo = [ctx.array(fx) for _ in range(S)], [ctx.array(fy) for _ in range(S)], [ctx.empty(n, np.float32) for _ in range(S)]
+        env2 = [envs(dfx[i], dfy[i]) for i in range(S)]
+        zw = ctx.skeleton(A.SKEL_MAP, "float", env=[F32, F32], out_rank=1, get=rd(0) + " * " + rd(1))
+        fod = [o.desc() for o in fo]
 
-        def step():
-            A.check(L.acc_exec_map(zw.handle, env2, C.byref(fod), stream))
-        w, e = T.run(step)
-        assert np.array_equal(fo.get(), fx * fx[::-1])
+        def step(i):
+            return lambda: A.check(L.acc_exec_map(zw.handle, env2[i], C.byref(fod[i]), stream))
+        w, e = T.run([step(i) for i in range(S)])
+        assert np.array_equal(fo[S - 1].get(), fx * fy)
         sk["zipwith_mul"] = result("zipWith (*) Float32 2^26", w, e, 1, 3 * n * 4, n)
-        del dx, out, dfx, dfy, fo, x, fx
+        del dfx, dfy, fo, env2, x, fx, fy
 
     # ---------------------------------------------------------------- 1: dot product
     if want("dot"):
         log("dot product of two 2^24 Float32 vectors ...")
         nd = 1 << 24
         x, y = wl.dot_inputs(nd)
-        dx, dy = ctx.array(x), ctx.array(y)
-        env = envs(dx, dy)
-        dot = ctx.skeleton(A.SKEL_FOLD, "float", env=[F32, F32], out_rank=0, get="arrIn0_0[ix] * arrIn1_0[ix]",
+        Sd = 4 * S                                  # 128 MB per set: more sets to get past the cache
+        dxs, dys = [ctx.array(x) for _ in range(Sd)], [ctx.array(y) for _ in range(Sd)]
+        env_s = [envs(dxs[i], dys[i]) for i in range(Sd)]
+        dot = ctx.skeleton(A.SKEL_FOLD, "float", env=[F32, F32], out_rank=0, get=rd(0) + " * " + rd(1),
                            combine="x + y", seed="0.0f")
         o = ctx.empty((), np.float32)
         od = o.desc()
         sh = (C.c_int64 * 1)(nd)
 
-        def step():
-            A.check(L.acc_exec_fold(dot.handle, env, 1, sh, C.byref(od), stream))
-        w, e = T.run(step)
+        def step(i):
+            return lambda: A.check(L.acc_exec_fold(dot.handle, env_s[i], 1, sh, C.byref(od), stream))
+        w, e = T.run([step(i) for i in range(Sd)])
         truth = float(np.dot(x.astype(np.float64), y.astype(np.float64)))
         sk["dot"] = result("fold (+) 0 . zipWith (*) 2^24", w, e, 1, 2 * nd * 4 + 4, nd,
                            {"result": float(o.get()), "float64_truth": truth, "GFLOP_per_s": round(2 * nd / (e * 1e-3) / 1e9, 1)})
-        del dx, dy
+        del dxs, dys, env_s
 
     # ---------------------------------------------------------------- 3: histograms
     for name, bins, gen in (("hist256_uniform", 256, wl.hist_uniform_keys), ("hist65536_zipf", 65536, wl.hist_zipf_keys)):
@@ -198,29 +217,29 @@ def main():
             continue
         log("histogram %s over 2^26 Int32 keys ..." % name)
         keys = gen(n, bins)
-        dk = ctx.array(keys)
-        env = envs(dk)
+        dks = [ctx.array(keys) for _ in range(S)]
+        env_s = [envs(d) for d in dks]
         hist = ctx.skeleton(A.SKEL_PERMUTE, "Int32", env=[I32], out_rank=1, get="1", combine="x + y",
-                            permutation=os.environ.get("ACC_BENCH_HIST_PERM", "arrIn0_0[ix]"), combine_hint=A.COMBINE_ADD)
+                            permutation=rd(0), combine_hint=A.COMBINE_ADD)
         dfl, out = ctx.array(np.zeros(bins, np.int32)), ctx.empty(bins, np.int32)
         dd, od = dfl.desc(), out.desc()
 
-        def step():
-            A.check(L.acc_exec_permute(hist.handle, env, n, C.byref(dd), C.byref(od), stream))
-        w, e = T.run(step)
+        def step(i):
+            return lambda: A.check(L.acc_exec_permute(hist.handle, env_s[i], n, C.byref(dd), C.byref(od), stream))
+        w, e = T.run([step(i) for i in range(S)])
         got = out.get()
         assert os.environ.get("ACC_BENCH_NOCHECK") or (int(got.sum()) == n and np.array_equal(got, np.bincount(keys, minlength=bins))), "histogram mismatch"
         sk[name] = result("permute (+) %d bins" % bins, w, e, 1, n * 4 + 2 * bins * 4, n,
                           {"Gkeys_per_s": round(n / (e * 1e-3) / 1e9, 2), "note": "step = defaults copy + permute kernel"})
-        del dk, keys
+        del dks, env_s, keys
 
     # ---------------------------------------------------------------- 4: stencils
     if want("stencil"):
         log("3x3 Gaussian (clamp) x10 and 5-point Laplacian (mirror) on 8192x8192 Float32 ...")
         h = w_ = 8192
         img = wl.stencil_image(h, w_)
-        a, b = ctx.array(img), ctx.empty((h, w_), np.float32)
-        ad, bd = a.desc(), b.desc()
+        a_s, b_s = [ctx.array(img) for _ in range(S)], [ctx.empty((h, w_), np.float32) for _ in range(S)]
+        ad, bd = [a.desc() for a in a_s], [b.desc() for b in b_s]
         taps = [(dy, dx) for dy in (-1, 0, 1) for dx in (-1, 0, 1)]
         gauss = ctx.skeleton(A.SKEL_STENCIL, "float", out_rank=2, taps=taps, boundary="clamp",
                              stencil_fn=A.linear_stencil_fn([1, 2, 1, 2, 4, 2, 1, 2, 1], 16))
@@ -228,33 +247,35 @@ def main():
                            boundary="mirror", stencil_fn=A.linear_stencil_fn([1, 1, -4, 1, 1]))
         rib = C.c_int32(0)
 
-        def step():
-            A.check(L.acc_exec_stencil_iterate(gauss.handle, None, C.byref(ad), C.byref(bd), 10, stream, C.byref(rib)))
-        w, e = T.run(step)
+        def step(i):
+            return lambda: A.check(L.acc_exec_stencil_iterate(gauss.handle, None, C.byref(ad[i]), C.byref(bd[i]), 10, stream, C.byref(rib)))
+        w, e = T.run([step(i) for i in range(S)])
         sk["gaussian3x3_clamp_x10"] = result("stencil 3x3 gaussian x10", w, e, 10, 2 * h * w_ * 4, 10 * h * w_)
 
-        def step2():
-            A.check(L.acc_exec_stencil(lap.handle, None, C.byref(ad), C.byref(bd), stream))
-        w, e = T.run(step2)
+        def step2(i):
+            return lambda: A.check(L.acc_exec_stencil(lap.handle, None, C.byref(ad[i]), C.byref(bd[i]), stream))
+        w, e = T.run([step2(i) for i in range(S)])
         sk["laplace5_mirror"] = result("stencil 5-point laplacian", w, e, 1, 2 * h * w_ * 4, h * w_)
-        del a, b, img
+        del a_s, b_s, img
 
     # ---------------------------------------------------------------- 5: sparse matrix-vector product
     if want("smvm"):
         log("CSR SMVM, 2^20 rows, Poisson(32) row lengths ...")
         vals, cols, offs, lens, xv = wl.smvm_inputs()
         nnz, rows = vals.size, offs.size - 1
-        dv, dc, dxv, doff = ctx.array(vals), ctx.array(cols), ctx.array(xv), ctx.array(offs)
-        env = envs(dv, dc, dxv)
-        y = ctx.empty(rows, np.float32)
+        dv, dc = [ctx.array(vals) for _ in range(S)], [ctx.array(cols) for _ in range(S)]
+        dxv, doff = [ctx.array(xv) for _ in range(S)], [ctx.array(offs) for _ in range(S)]
+        env_s = [envs(dv[i], dc[i], dxv[i]) for i in range(S)]
+        ys = [ctx.empty(rows, np.float32) for _ in range(S)]
         smvm = ctx.skeleton(A.SKEL_FOLDSEG, "float", env=[F32, I32, F32],
-                            get=os.environ.get("ACC_BENCH_SMVM_GET", "arrIn0_0[ix] * arrIn2_0[arrIn1_0[ix]]"),
+                            get=os.environ.get("ACC_BENCH_SMVM_GET", rd(0) + " * arrIn2_0[" + rd(1) + "]"),
                             combine="x + y", seed="0.0f")
-        offd, yd = doff.desc(), y.desc()
+        offd, yd = [d.desc() for d in doff], [y.desc() for y in ys]
 
-        def step():
-            A.check(L.acc_exec_foldseg(smvm.handle, env, nnz, C.byref(offd), C.byref(yd), stream))
-        w, e = T.run(step)
+        def step(i):
+            return lambda: A.check(L.acc_exec_foldseg(smvm.handle, env_s[i], nnz, C.byref(offd[i]), C.byref(yd[i]), stream))
+        w, e = T.run([step(i) for i in range(S)])
+        y = ys[S - 1]
         sk["smvm"] = result("foldSeg (+) . zipWith (*) . gather", w, e, 1, nnz * 8 + rows * 8 + xv.size * 4, nnz,
                             {"nnz": int(nnz), "GFLOP_per_s": round(2 * nnz / (e * 1e-3) / 1e9, 1),
                              "note": "segment offsets precomputed on the device (scanl over the 2^20 lengths is not in the step)"})
@@ -277,7 +298,8 @@ def main():
         "value": headline["GB_per_s"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": headline["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int32", "data": "synthetic (seeded SplitMix64, resident in HBM before the timed region)",
-        "config": {"workload": workload, "elements": n, "timing": "kernel launches back to back on one stream, inputs device-resident"},
+        "config": {"workload": workload, "elements": n, "buffer_sets": S,
+                   "timing": "kernel launches back to back on one stream, inputs device-resident, consecutive launches on different buffer sets"},
         "roofline": {"bound": "hbm", "achieved": headline["GB_per_s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(headline["GB_per_s"] / HBM_PEAK_GBS, 4),
                      # HBM bytes per scanl launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the

@@ -3,6 +3,10 @@
 Checked against the CPU oracle where it runs in a second or two (the C
 restatement handles 2^26 elements comfortably), and through size-independent
 properties otherwise.  Tolerances are the configurations' own.
+
+The fragments spell reads that are consumed once as acc_stream(array, ix), the
+non-temporal load a code generator emits for the linear index of a delayed
+array; indirect reads (the gathered vector of the SMVM) stay plain.
 """
 import sys
 
@@ -43,7 +47,7 @@ def test_config1_dot_product_2_24(A, ctx, wl, orc):
     say("dot 2^24")
     n = 1 << 24
     x, y = wl.dot_inputs(n)
-    dot = ctx.skeleton(A.SKEL_FOLD, "float", env=[F32, F32], out_rank=0, get="arrIn0_0[ix] * arrIn1_0[ix]",
+    dot = ctx.skeleton(A.SKEL_FOLD, "float", env=[F32, F32], out_rank=0, get="acc_stream(arrIn0_0, ix) * acc_stream(arrIn1_0, ix)",
                        combine="x + y", seed="0.0f")
     out = ctx.empty((), np.float32)
     dx, dy = ctx.array(x), ctx.array(y)
@@ -68,7 +72,7 @@ def test_config2_prefix_sums_2_26(A, ctx, wl, orc, kind):
     say(kind, "2^26")
     n = 1 << 26
     x = wl.scan_input(n)
-    sk = ctx.skeleton(A.SCAN_KINDS[kind], "Int32", env=[I32], get="arrIn0_0[ix]", combine="x + y",
+    sk = ctx.skeleton(A.SCAN_KINDS[kind], "Int32", env=[I32], get="acc_stream(arrIn0_0, ix)", combine="x + y",
                       seed=None if kind == "scanl1" else "0")
     m = n if kind == "scanl1" else n + 1
     out = ctx.empty(m, np.int32)
@@ -93,7 +97,7 @@ def test_config3_histograms_2_26(A, ctx, wl, orc, case):
     bins = 256 if case == "uniform256" else 65536
     keys = wl.hist_uniform_keys(n, bins) if case == "uniform256" else wl.hist_zipf_keys(n, bins)
     hist = ctx.skeleton(A.SKEL_PERMUTE, "Int32", env=[I32], out_rank=1, get="1", combine="x + y",
-                        permutation="arrIn0_0[ix]", combine_hint=A.COMBINE_ADD)
+                        permutation="acc_stream(arrIn0_0, ix)", combine_hint=A.COMBINE_ADD)
     zeros = np.zeros(bins, np.int32)
     out = ctx.empty(bins, np.int32)
     dk = ctx.array(keys)
@@ -154,7 +158,7 @@ def test_config5_smvm_2_20_rows(A, ctx, wl, orc):
     doff = ctx.empty(rows + 1, np.int32)
     scan.scan([ctx.array(lens)], rows, doff)
     assert np.array_equal(doff.get(), offs)
-    smvm = ctx.skeleton(A.SKEL_FOLDSEG, "float", env=[F32, I32, F32], get="arrIn0_0[ix] * arrIn2_0[arrIn1_0[ix]]",
+    smvm = ctx.skeleton(A.SKEL_FOLDSEG, "float", env=[F32, I32, F32], get="acc_stream(arrIn0_0, ix) * arrIn2_0[acc_stream(arrIn1_0, ix)]",
                         combine="x + y", seed="0.0f")
     y = ctx.empty(rows, np.float32)
     smvm.foldseg([ctx.array(vals), ctx.array(cols), ctx.array(x)], nnz, doff, y)
