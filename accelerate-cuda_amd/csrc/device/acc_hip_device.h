@@ -197,6 +197,9 @@ ACC_DEV Int64 acc_xcd_contiguous_block()
  * the L2.  The code generator uses it for linear reads next to indirect ones. */
 template <typename T> ACC_DEV T acc_stream(const T *p, const Int64 ix) { return __builtin_nontemporal_load(p + ix); }
 
+/* a compile-time flag passed as a value (to generic lambdas) */
+template <bool B> struct acc_bool { static constexpr bool value = B; };
+
 /* the bulk stores of a streaming skeleton (a result that this kernel never
  * reads back): non-temporal if the generator asks for it */
 #ifndef ACC_NT_STORE

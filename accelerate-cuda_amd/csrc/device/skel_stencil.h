@@ -13,8 +13,9 @@
  *     lane, ACC_PREFETCH rows ahead of its use, so a wave always has several
  *     kilobytes in flight and never waits at a barrier;
  *   - taps to the left and right come from the neighbouring lanes' registers
- *     through DPP wave shifts; only the first and last lane of a strip load
- *     their rx halo elements themselves;
+ *     through DPP wave shifts; the rx elements just outside the strip, for
+ *     all its rows, are fetched by one gather at the start and handed to the
+ *     strip's first and last lane with readlane;
  *   - taps above and below are simply older and newer rows of the register
  *     window, which rotates by renaming (the row loop is unrolled by the
  *     window length).
@@ -44,6 +45,9 @@
 #define ACC_RING  (ACC_NR + ACC_PREFETCH)             /* rows held in registers */
 #define ACC_WW    (ACC_SVEC + 2 * ACC_RADIUS_X)       /* row window of one lane */
 #define ACC_WAVES (ACC_BLOCK / ACC_WAVE)
+#define ACC_TOTAL_MAX  (ACC_TILE_H + 2 * ACC_RADIUS_Y)        /* source rows a strip touches */
+#define ACC_HALO_COUNT (2 * ACC_RADIUS_X * ACC_TOTAL_MAX)     /* elements just outside the strip */
+#define ACC_HALO_LOADS (ACC_HALO_COUNT > 0 ? (ACC_HALO_COUNT + ACC_WAVE - 1) / ACC_WAVE : 1)
 
 static_assert(ACC_RADIUS_X <= ACC_SVEC, "stencil wider than one lane's neighbours can supply");
 
@@ -88,10 +92,14 @@ stencil(ACC_ENV_PARAMS ACC_OUT_PARAMS, const ACC_IN_ELT *__restrict__ arrStencil
 #endif
   const int lane = acc_lane();
   const Int64 strips_x = (w + ACC_STRIP - 1) / ACC_STRIP;
+  /* the wave's number within the workgroup, as a scalar: everything derived
+   * from it (the strip's origin, which path it takes) is then uniform for the
+   * compiler too, and the paths below become scalar branches */
+  const int wave_in_block = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
 #if ACC_XCD_REMAP
-  const Int64 strip = acc_xcd_contiguous_block() * ACC_WAVES + (threadIdx.x >> 6);
+  const Int64 strip = acc_xcd_contiguous_block() * ACC_WAVES + wave_in_block;
 #else
-  const Int64 strip = (Int64)blockIdx.x * ACC_WAVES + (threadIdx.x >> 6);
+  const Int64 strip = (Int64)blockIdx.x * ACC_WAVES + wave_in_block;
 #endif
 #if ACC_STACK_WAVES
   /* the waves of a workgroup take vertically adjacent strips: the boundary
@@ -104,16 +112,58 @@ stencil(ACC_ENV_PARAMS ACC_OUT_PARAMS, const ACC_IN_ELT *__restrict__ arrStencil
 #endif
   if (y0 >= h) return;                                   /* whole wave leaves together */
   const Int64 gx = x0 + lane * ACC_SVEC;
-  const int rows = (int)acc_min<Int64>(ACC_TILE_H, h - y0);
+  const int rows_here = (int)acc_min<Int64>(ACC_TILE_H, h - y0);
 #if ACC_ALIGNED
-  const bool fast = (x0 + ACC_STRIP <= w);               /* every lane owns a full, aligned vector */
+  const bool fast_here = (x0 + ACC_STRIP <= w);          /* every lane owns a full, aligned vector */
 #else
-  const bool fast = false;
+  const bool fast_here = false;
 #endif
 
+  /* the strip, compiled three times: fast and ACC_TILE_H rows tall (all constants),
+   * fast and cut by the bottom edge, and the element-wise path */
+  auto run = [&](auto fast_c, auto full_c) {
+  constexpr bool fast = decltype(fast_c)::value;
+  const int rows = decltype(full_c)::value ? ACC_TILE_H : rows_here;
+
+  const int total = rows + 2 * ACC_RADIUS_Y;              /* source rows this strip touches */
+
+  /* fast path: the 2 rx elements just outside the strip, for every source row
+   * the strip will touch, are requested in one go -- lane q takes element
+   * q = (side * rx + j) * ACC_TOTAL_MAX + rho -- ahead of all row loads; finish()
+   * hands them to the strip's first and last lane.  One instruction for the
+   * strip instead of two per row. */
+  S halo[ACC_HALO_LOADS];
+  if (fast) {
+#pragma unroll
+    for (int g = 0; g < ACC_HALO_LOADS; ++g) {
+      const int q = lane + ACC_WAVE * g;
+      const int side = q / (ACC_RADIUS_X * ACC_TOTAL_MAX), rem = q % (ACC_RADIUS_X * ACC_TOTAL_MAX);
+      const int j = rem / ACC_TOTAL_MAX, rho = rem % ACC_TOTAL_MAX;
+      halo[g] = S();
+      if (q < ACC_HALO_COUNT && rho < total) {
+        const Int64 gy = y0 - ACC_RADIUS_Y + rho;
+        const Int64 xx = side ? x0 + ACC_STRIP + j : x0 - ACC_RADIUS_X + j;
+#if ACC_BOUNDARY == ACC_B_CONSTANT
+        const bool inside = gy >= 0 && gy < h && xx >= 0 && xx < w;
+        const Int64 my = acc_max<Int64>(0, acc_min<Int64>(gy, h - 1)), mx = acc_max<Int64>(0, acc_min<Int64>(xx, w - 1));
+        halo[g] = inside ? arrStencil_0[my * w + mx] : (S)(ACC_BOUNDARY_CONSTANT);
+#else
+        halo[g] = arrStencil_0[acc_boundary_index(gy, h) * w + acc_boundary_index(xx, w)];
+#endif
+      }
+    }
+  }
+  auto halo_of = [&](const int side, const int j, const int rho) -> S {
+    const int q = (side * ACC_RADIUS_X + j) * ACC_TOTAL_MAX + rho;
+    S v = acc_readlane(halo[0], q % ACC_WAVE);
+#pragma unroll
+    for (int g = 1; g < ACC_HALO_LOADS; ++g)
+      if (q / ACC_WAVE == g) v = acc_readlane(halo[g], q % ACC_WAVE);
+    return v;
+  };
+
   /* fetch source row (y0 - ry + rho) into a window; in the fast path the left
-   * and right parts are only valid in the strip's first and last lane until
-   * acc_row_finish has run */
+   * and right parts are only valid once finish() has run */
   auto fetch = [&](const int rho, acc_row &r) {
     const Int64 gy = y0 - ACC_RADIUS_Y + rho;
 #if ACC_BOUNDARY == ACC_B_CONSTANT
@@ -129,25 +179,9 @@ stencil(ACC_ENV_PARAMS ACC_OUT_PARAMS, const ACC_IN_ELT *__restrict__ arrStencil
 #pragma unroll
       for (int k = 0; k < ACC_SVEC; ++k) r.e[ACC_RADIUS_X + k] = row_inside ? own.v[k] : (S)(ACC_BOUNDARY_CONSTANT);
 #pragma unroll
-      for (int j = 0; j < ACC_RADIUS_X; ++j) {
+      for (int j = 0; j < ACC_RADIUS_X; ++j) {           /* filled in by finish() */
         r.e[j] = S();
         r.e[ACC_RADIUS_X + ACC_SVEC + j] = S();
-        if (lane == 0) {
-          const Int64 xx = x0 - ACC_RADIUS_X + j;
-#if ACC_BOUNDARY == ACC_B_CONSTANT
-          r.e[j] = (row_inside && xx >= 0) ? src[acc_max<Int64>(xx, 0)] : (S)(ACC_BOUNDARY_CONSTANT);
-#else
-          r.e[j] = src[acc_boundary_index(xx, w)];
-#endif
-        }
-        if (lane == ACC_WAVE - 1) {
-          const Int64 xx = x0 + ACC_STRIP + j;
-#if ACC_BOUNDARY == ACC_B_CONSTANT
-          r.e[ACC_RADIUS_X + ACC_SVEC + j] = (row_inside && xx < w) ? src[acc_min<Int64>(xx, w - 1)] : (S)(ACC_BOUNDARY_CONSTANT);
-#else
-          r.e[ACC_RADIUS_X + ACC_SVEC + j] = src[acc_boundary_index(xx, w)];
-#endif
-        }
       }
     } else {
 #pragma unroll
@@ -167,26 +201,25 @@ stencil(ACC_ENV_PARAMS ACC_OUT_PARAMS, const ACC_IN_ELT *__restrict__ arrStencil
   };
 
   /* fast path only: complete the window with the neighbours' elements */
-  auto finish = [&](acc_row &r) {
+  auto finish = [&](const int rho, acc_row &r) {
     if (!fast) return;
 #pragma unroll
     for (int j = 0; j < ACC_RADIUS_X; ++j) {
       const S from_left  = acc_wave_shift_up1(r.e[ACC_SVEC + j]);          /* neighbour's own[SVEC - rx + j] */
       const S from_right = acc_wave_shift_down1(r.e[ACC_RADIUS_X + j]);    /* neighbour's own[j] */
-      if (lane != 0) r.e[j] = from_left;
-      if (lane != ACC_WAVE - 1) r.e[ACC_RADIUS_X + ACC_SVEC + j] = from_right;
+      r.e[j] = (lane != 0) ? from_left : halo_of(0, j, rho);
+      r.e[ACC_RADIUS_X + ACC_SVEC + j] = (lane != ACC_WAVE - 1) ? from_right : halo_of(1, j, rho);
     }
   };
 
   acc_row ring[ACC_RING];
-  const int total = rows + 2 * ACC_RADIUS_Y;              /* source rows this strip touches */
 
   /* prologue: the rows the first result needs, minus the newest, plus the prefetch */
 #pragma unroll
   for (int rho = 0; rho < ACC_RING - 1; ++rho)
     if (rho < total) fetch(rho, ring[rho]);
 #pragma unroll
-  for (int rho = 0; rho < ACC_NR - 1; ++rho) finish(ring[rho]);
+  for (int rho = 0; rho < ACC_NR - 1; ++rho) finish(rho, ring[rho]);
 
   for (int yb = 0; yb < rows; yb += ACC_RING) {
 #pragma unroll
@@ -197,7 +230,7 @@ stencil(ACC_ENV_PARAMS ACC_OUT_PARAMS, const ACC_IN_ELT *__restrict__ arrStencil
          * slot freed by the previous step takes the row PREFETCH further on */
         const int rho_new = y + ACC_NR - 1 + ACC_PREFETCH;
         if (rho_new < total) fetch(rho_new, ring[(s + ACC_RING - 1) % ACC_RING]);
-        finish(ring[(s + ACC_NR - 1) % ACC_RING]);
+        finish(y + ACC_NR - 1, ring[(s + ACC_NR - 1) % ACC_RING]);
 
         acc_out_vec res;
 #pragma unroll
@@ -217,5 +250,13 @@ stencil(ACC_ENV_PARAMS ACC_OUT_PARAMS, const ACC_IN_ELT *__restrict__ arrStencil
         }
       }
     }
+  }
+  };   /* run */
+
+  if (fast_here) {
+    if (rows_here == ACC_TILE_H) run(acc_bool<true>(), acc_bool<true>());
+    else                         run(acc_bool<true>(), acc_bool<false>());
+  } else {
+    run(acc_bool<false>(), acc_bool<false>());
   }
 }
