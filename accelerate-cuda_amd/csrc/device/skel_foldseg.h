@@ -12,7 +12,8 @@
  *     elements, evaluating the (fused) producer with fully coalesced, 128-bit
  *     reads whatever the segment lengths are;
  *   - lane i then folds the part of segment i that lies in the chunk, reading
- *     LDS sequentially, and carries its accumulator to the next chunk.
+ *     LDS sequentially, and carries its accumulator to the next chunk; the
+ *     next chunk's loads are already in flight while it does so.
  * Every segment is thus combined strictly in index order, the order of a
  * sequential fold: the operator need only be associative for the result to
  * be independent of the schedule, and with ACC_FOLD_RIGHT the association is
@@ -74,15 +75,13 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
     /* chunks start on a vector boundary so that the loads stay aligned */
     const Int64 lo_al = lo - (lo % ACC_VEC);
     const Int64 nchunks = hi > lo_al ? (hi - lo_al + ACC_CHUNK - 1) / ACC_CHUNK : 0;
-    for (Int64 q = 0; q < nchunks; ++q) {
-      const Int64 cs = lo_al + (ACC_FOLD_RIGHT ? (nchunks - 1 - q) : q) * (Int64)ACC_CHUNK;
-      const Int64 ce = acc_min<Int64>(cs + ACC_CHUNK, hi);
-
-      /* stage the chunk: every load is issued before any result is used.
-       * Elements of the chunk's first and last vector that belong to a
-       * neighbouring block are loaded too (they exist) and never read back;
-       * only the very end of the array needs a guard. */
-      T v[ACC_LOADS][ACC_VEC];
+    /* stage a chunk: every load is issued before any result is used.  Elements
+     * of the chunk's first and last vector that belong to a neighbouring block
+     * are loaded too (they exist) and never read back; only the very end of
+     * the array needs a guard. */
+    T v[ACC_LOADS][ACC_VEC];
+    auto chunk_start = [&](const Int64 q) -> Int64 { return lo_al + (ACC_FOLD_RIGHT ? (nchunks - 1 - q) : q) * (Int64)ACC_CHUNK; };
+    auto stage = [&](const Int64 cs) {
       if (cs + ACC_CHUNK <= n) {
 #pragma unroll
         for (int u = 0; u < ACC_LOADS; ++u)
@@ -98,12 +97,19 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
             if (ix < n) v[u][k] = get(ix);
           }
       }
+    };
+    if (nchunks > 0) stage(chunk_start(0));
+    for (Int64 q = 0; q < nchunks; ++q) {
+      const Int64 cs = chunk_start(q);
+      const Int64 ce = acc_min<Int64>(cs + ACC_CHUNK, hi);
       __syncthreads();                               /* the previous chunk has been consumed */
 #pragma unroll
       for (int u = 0; u < ACC_LOADS; ++u)
 #pragma unroll
         for (int k = 0; k < ACC_VEC; ++k) s_val[(u * ACC_BLOCK + tid) * ACC_VEC + k] = v[u][k];
       __syncthreads();
+      /* the next chunk's loads (and the gathers behind them) travel while this one is folded */
+      if (q + 1 < nchunks) stage(chunk_start(q + 1));
 
       /* fold this lane's segment, as far as it lies in the chunk, in index order */
       int p0 = (int)(acc_max(a, cs) - cs), p1 = (int)(acc_min(b, ce) - cs);

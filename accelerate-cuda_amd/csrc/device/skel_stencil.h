@@ -175,9 +175,16 @@ stencil(ACC_ENV_PARAMS ACC_OUT_PARAMS, const ACC_IN_ELT *__restrict__ arrStencil
 #endif
     const S *src = arrStencil_0 + my * w;
     if (fast) {
+#if ACC_STENCIL_NT & 2
+      typedef S acc_in_native __attribute__((ext_vector_type(ACC_SVEC)));
+      const acc_in_native own = __builtin_nontemporal_load((const acc_in_native *)(src + gx));
+#pragma unroll
+      for (int k = 0; k < ACC_SVEC; ++k) r.e[ACC_RADIUS_X + k] = row_inside ? own[k] : (S)(ACC_BOUNDARY_CONSTANT);
+#else
       const acc_in_vec own = *(const acc_in_vec *)(src + gx);
 #pragma unroll
       for (int k = 0; k < ACC_SVEC; ++k) r.e[ACC_RADIUS_X + k] = row_inside ? own.v[k] : (S)(ACC_BOUNDARY_CONSTANT);
+#endif
 #pragma unroll
       for (int j = 0; j < ACC_RADIUS_X; ++j) {           /* filled in by finish() */
         r.e[j] = S();
@@ -242,7 +249,15 @@ stencil(ACC_ENV_PARAMS ACC_OUT_PARAMS, const ACC_IN_ELT *__restrict__ arrStencil
         }
         T *dst = arrOut_0 + (y0 + y) * w + gx;
         if (fast) {
+#if ACC_STENCIL_NT & 1
+          typedef T acc_out_native __attribute__((ext_vector_type(ACC_SVEC)));
+          acc_out_native nv;
+#pragma unroll
+          for (int k = 0; k < ACC_SVEC; ++k) nv[k] = res.v[k];
+          __builtin_nontemporal_store(nv, (acc_out_native *)dst);
+#else
           *(acc_out_vec *)dst = res;
+#endif
         } else {
 #pragma unroll
           for (int k = 0; k < ACC_SVEC; ++k)
