@@ -219,4 +219,7 @@ template <typename T> ACC_DEV void acc_store(T *p, const T &v)
 ACC_DEV Int64 acc_to_index2(Int64, Int64 w, Int64 y, Int64 x) { return y * w + x; }
 ACC_DEV Int64 acc_to_index3(Int64, Int64 h, Int64 w, Int64 z, Int64 y, Int64 x) { return (z * h + y) * w + x; }
 
+/* the scalar primitives of the expression language */
+#include "acc_prim.h"
+
 #endif /* ACC_HIP_DEVICE_H */

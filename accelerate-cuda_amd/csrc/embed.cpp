@@ -18,6 +18,7 @@
   extern "C" const char acc_embed_##sym##_end[];
 
 ACC_EMBED(device, "device/acc_hip_device.h")
+ACC_EMBED(prim, "device/acc_prim.h")
 ACC_EMBED(map, "device/skel_map.h")
 ACC_EMBED(fold, "device/skel_fold.h")
 ACC_EMBED(foldseg, "device/skel_foldseg.h")
@@ -31,6 +32,7 @@ const std::vector<EmbeddedHeader> &embedded_headers()
 {
   static const std::vector<EmbeddedHeader> headers = {
       {"acc_hip_device.h", acc_embed_device_begin, acc_embed_device_end},
+      {"acc_prim.h", acc_embed_prim_begin, acc_embed_prim_end},
       {"skel_map.h", acc_embed_map_begin, acc_embed_map_end},
       {"skel_fold.h", acc_embed_fold_begin, acc_embed_fold_end},
       {"skel_foldseg.h", acc_embed_foldseg_begin, acc_embed_foldseg_end},

@@ -111,3 +111,45 @@ def stencil2d(fn, img, offsets, mode, constant=0.0):
 def affine16(x, y):
     a1, b1, a2, b2 = x >> 16, x & 0xFFFF, y >> 16, y & 0xFFFF
     return (((a1 * a2) & 0xFFFF) << 16) | ((a1 * b2 + b1) & 0xFFFF)
+
+
+# ---- scalar primitives on fixed-width integers (exact, with Python integers) ---------------
+# The definitions are Haskell's (quot/rem truncate, div/mod floor, rotate modulo the width),
+# which the reference's generated C reproduces (CodeGen/Arithmetic.hs:90-217).
+
+def wrap(v, bits, signed):
+    v &= (1 << bits) - 1
+    if signed and v >> (bits - 1):
+        v -= 1 << bits
+    return v
+
+
+def quot(x, y):
+    q = abs(x) // abs(y)
+    return q if (x < 0) == (y < 0) else -q
+
+
+def rem(x, y):
+    return x - y * quot(x, y)
+
+
+def idiv(x, y):
+    return x // y
+
+
+def imod(x, y):
+    return x % y
+
+
+def signum(x):
+    return (x > 0) - (x < 0)
+
+
+def shift_rl(x, i, bits):
+    return (x & ((1 << bits) - 1)) >> i
+
+
+def rotate_l(x, i, bits):
+    u = x & ((1 << bits) - 1)
+    k = i % bits
+    return ((u << k) | (u >> (bits - k))) & ((1 << bits) - 1) if k else u

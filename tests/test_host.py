@@ -60,6 +60,27 @@ def test_every_skeleton_instance_compiles_for_gfx950(A, tmp_path):
         assert A.compile_only(desc, "gfx950") > 4000, name
 
 
+def test_every_scalar_primitive_compiles_for_every_type(A, tmp_path):
+    """acc_prim.h: one map per element type naming every primitive that type has
+    (CodeGen.hs:406-476); what they compute is checked on the GPU"""
+    A.lib().acc_cache_set_dir(str(tmp_path).encode())
+    X, Y = "arrIn0_0[ix]", "arrIn1_0[ix]"
+    integral = ["acc_quot(X, Y)", "acc_rem(X, Y)", "acc_idiv(X, Y)", "acc_imod(X, Y)", "acc_quot_rem(X, Y).snd",
+                "acc_div_mod(X, Y).fst", "acc_abs(X)", "acc_signum(X)", "acc_pmax(X, Y)", "acc_pmin(X, Y)",
+                "acc_shift_l(X, 1)", "acc_shift_r(X, 1)", "acc_shift_rl(X, 1)", "acc_rotate_l(X, (Int64)Y)",
+                "acc_rotate_r(X, (Int64)Y)", "acc_from_integral<T>(acc_bool_to_int((Word8)(X > Y)))", "(T)acc_ord(acc_chr(X))"]
+    floating = ["acc_recip(X)", "acc_abs(X)", "acc_signum(X)", "acc_pmax(X, Y)", "acc_pmin(X, Y)", "acc_pow(X, Y)",
+                "acc_atan2(X, Y)", "acc_log_base(X, Y)", "(T)acc_is_nan(X)", "(T)acc_truncate<Int32>(X)",
+                "(T)acc_round<Int64>(X)", "(T)acc_floor<Int16>(X)", "(T)acc_ceiling<Word32>(X)"] + \
+               ["acc_%s(X)" % f for f in ("sin", "cos", "tan", "asin", "acos", "atan", "sinh", "cosh", "tanh", "asinh",
+                                          "acosh", "atanh", "exp", "sqrt", "log")]
+    for t in ("Int8", "Int16", "Int32", "Int64", "Word8", "Word16", "Word32", "Word64", "float", "double"):
+        terms = floating if t in ("float", "double") else integral
+        frag = " + ".join("(T)(%s)" % e for e in terms).replace("X", X).replace("Y", Y).replace("T", t)
+        d = A.make_desc(A.SKEL_MAP, t, env=[(1, t), (1, t)], out_rank=1, get=frag)
+        assert A.compile_only(d, "gfx950") > 4000, t
+
+
 def test_kernel_cache_hit_miss_and_corruption(A, tmp_path):
     L = A.lib()
     d = str(tmp_path / "cache")
