@@ -258,6 +258,38 @@ class DeviceArray(object):
             pass
 
 
+class TupleArray(object):
+    """An array of tuples as the array language lays it out: one device array per
+    component (structure of arrays).  `comps` lists the components as the tuple
+    reads, left to right; the kernel ABI numbers them from the right, so the
+    descriptor's ptr[c] is comps[n - 1 - c]."""
+
+    def __init__(self, comps):
+        comps = list(comps)
+        assert comps and all(c.shape == comps[0].shape for c in comps)
+        self.comps, self.shape, self.size = comps, comps[0].shape, comps[0].size
+
+    def desc(self, shape=None, offset_elems=0):
+        a = self.comps[0].desc(shape, offset_elems)
+        n = len(self.comps)
+        a.ncomp = n
+        for c in range(n):
+            comp = self.comps[n - 1 - c]
+            a.ptr[c] = comp.ptr + offset_elems * comp.dtype.itemsize
+        return a
+
+    def ctypes_of(self):
+        """component C types by component index (component 0 = the LAST element), for an env signature"""
+        return [CTYPE_OF[c.dtype.type] for c in reversed(self.comps)]
+
+    def get(self):
+        return tuple(c.get() for c in self.comps)
+
+
+CTYPE_OF = {np.float32: "float", np.float64: "double", np.int8: "Int8", np.int16: "Int16", np.int32: "Int32",
+            np.int64: "Int64", np.uint8: "Word8", np.uint16: "Word16", np.uint32: "Word32", np.uint64: "Word64"}
+
+
 class Context(object):
     def __init__(self, device=0):
         h = C.c_void_p()
@@ -282,6 +314,13 @@ class Context(object):
     def array(self, host):
         host = np.ascontiguousarray(host)
         return DeviceArray(self, host.shape, host.dtype).set(host)
+
+    def tuple_array(self, *hosts):
+        """an array of tuples from its component arrays, listed left to right"""
+        return TupleArray([self.array(h) for h in hosts])
+
+    def empty_tuple(self, shape, dtypes):
+        return TupleArray([self.empty(shape, dt) for dt in dtypes])
 
     def stream(self):
         s = C.c_void_p()

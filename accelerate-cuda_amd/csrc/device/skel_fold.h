@@ -51,7 +51,7 @@ ACC_DEV acc_opt<T> acc_block_reduce(acc_opt<T> x, F f, acc_opt<T> *s_wave)
 
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 ACC_ENTRY(ACC_ENV_PARAMS
-          ACC_ELT *__restrict__ arrOut_0,
+          ACC_OUT_ARRAY(arrOut),
           const Int64 shIn_0,
           ACC_ELT *__restrict__ partials)
 {
@@ -123,9 +123,9 @@ ACC_ENTRY(ACC_ENV_PARAMS
   }
 #if ACC_HAS_SEED
   const T seed = (ACC_SEED);
-  arrOut_0[0] = total.ok ? f(total.v, seed) : seed;
+  ACC_SET(arrOut, 0, total.ok ? f(total.v, seed) : seed);
 #else
-  arrOut_0[0] = total.v;
+  ACC_SET(arrOut, 0, total.v);
 #endif
 }
 
@@ -135,7 +135,7 @@ ACC_ENTRY(ACC_ENV_PARAMS
 /* second launch: one block folds the `count` partial results */
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 ACC_CAT(ACC_ENTRY, _finish)(ACC_ENV_PARAMS
-                            ACC_ELT *__restrict__ arrOut_0,
+                            ACC_OUT_ARRAY(arrOut),
                             const ACC_ELT *__restrict__ partials, const Int64 count)
 {
   typedef ACC_ELT T;
@@ -149,9 +149,9 @@ ACC_CAT(ACC_ENTRY, _finish)(ACC_ENV_PARAMS
   if (threadIdx.x != 0) return;
 #if ACC_HAS_SEED
   const T seed = (ACC_SEED);
-  arrOut_0[0] = total.ok ? f(total.v, seed) : seed;
+  ACC_SET(arrOut, 0, total.ok ? f(total.v, seed) : seed);
 #else
-  arrOut_0[0] = total.v;
+  ACC_SET(arrOut, 0, total.v);
 #endif
 }
 
@@ -161,7 +161,7 @@ ACC_CAT(ACC_ENTRY, _finish)(ACC_ENV_PARAMS
  * elements at a time.  Output has one element per row.                       */
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 ACC_ENTRY(ACC_ENV_PARAMS
-          const Int64 shOut_0, ACC_ELT *__restrict__ arrOut_0,
+          const Int64 shOut_0, ACC_OUT_ARRAY(arrOut),
           const Int64 shIn_1, const Int64 shIn_0)
 {
   typedef ACC_ELT T;
@@ -184,9 +184,9 @@ ACC_ENTRY(ACC_ENV_PARAMS
     if (lane == 0) {
 #if ACC_HAS_SEED
       const T seed = (ACC_SEED);
-      arrOut_0[row] = total.ok ? f(total.v, seed) : seed;      /* Reduction.hs:351-362 */
+      ACC_SET(arrOut, row, total.ok ? f(total.v, seed) : seed);      /* Reduction.hs:351-362 */
 #else
-      arrOut_0[row] = total.v;
+      ACC_SET(arrOut, row, total.v);
 #endif
     }
   }

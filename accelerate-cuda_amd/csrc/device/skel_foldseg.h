@@ -39,7 +39,7 @@ static_assert(ACC_CHUNK % (ACC_BLOCK * ACC_VEC) == 0, "chunk must be a whole num
 
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
-                  const Int64 shOut_0, ACC_ELT *__restrict__ arrOut_0,
+                  const Int64 shOut_0, ACC_OUT_ARRAY(arrOut),
                   const Int64 shIn_0,
                   const ACC_SEG_TYPE *__restrict__ arrSeg_0)
 {
@@ -138,9 +138,9 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
 
     if (live) {
 #if ACC_HAS_SEED && !ACC_FOLD_RIGHT
-      arrOut_0[seg] = have ? f(acc, seed) : seed;
+      ACC_SET(arrOut, seg, have ? f(acc, seed) : seed);
 #else
-      arrOut_0[seg] = acc;      /* fold1Seg of an empty segment is undefined; T() is written */
+      ACC_SET(arrOut, seg, acc);      /* fold1Seg of an empty segment is undefined; T() is written */
 #endif
     }
   }

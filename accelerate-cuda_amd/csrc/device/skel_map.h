@@ -27,7 +27,7 @@ ACC_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS)
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
 #if ACC_ALIGNED
-  arrOut_0 = (T *)__builtin_assume_aligned(arrOut_0, 16);
+  ACC_OUT_ASSUME(arrOut)
 #endif
   auto get = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
 
@@ -45,14 +45,14 @@ ACC_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS)
 #pragma unroll
       for (int u = 0; u < ACC_UNROLL; ++u)
 #pragma unroll
-        for (int k = 0; k < ACC_VEC; ++k) acc_store(arrOut_0 + (base + u * (ACC_BLOCK * ACC_VEC) + k), v[u][k]);
+        for (int k = 0; k < ACC_VEC; ++k) ACC_PUT(arrOut, base + u * (ACC_BLOCK * ACC_VEC) + k, v[u][k]);
     } else {
 #pragma unroll
       for (int u = 0; u < ACC_UNROLL; ++u)
 #pragma unroll
         for (int k = 0; k < ACC_VEC; ++k) {
           const Int64 ix = base + u * (ACC_BLOCK * ACC_VEC) + k;
-          if (ix < n) arrOut_0[ix] = get(ix);
+          if (ix < n) ACC_SET(arrOut, ix, get(ix));
         }
     }
   }

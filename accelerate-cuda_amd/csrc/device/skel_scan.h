@@ -179,6 +179,15 @@ ACC_DEV T acc_scan_lookback(const acc_scan_desc<T> &desc, Int64 tile, const T &b
   return prefix;
 }
 
+/* the result arrays as the tile code sees them */
+template <typename Put, typename Set, typename Total>
+struct acc_scan_out {
+  Put put_;  Set set_;  Total total_;
+  ACC_DEV void put(const Int64 ix, const ACC_ELT &v) const { put_(ix, v); }
+  ACC_DEV void set(const Int64 ix, const ACC_ELT &v) const { set_(ix, v); }
+  ACC_DEV void total(const ACC_ELT &v) const { total_(v); }
+};
+
 /* ---- one tile ------------------------------------------------------------ */
 /* physical index of item 0 of row r of this lane; item k is k further on in
  * logical order (for right-handed scans: k further back in memory)          */
@@ -216,9 +225,9 @@ ACC_DEV void acc_scan_load(Get get, const Int64 base, const Int64 n, T (&x)[ACC_
 /* scan one tile whose elements are already in registers.  `prefetch` is
  * called once the block total is known and before the look-back starts: the
  * caller uses it to put the next tile's loads in flight behind the wait.     */
-template <bool PARTIAL, typename T, typename Op, typename Prefetch>
+template <bool PARTIAL, typename T, typename Op, typename Prefetch, typename Out>
 ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op_raw, const T seed, const Int64 tile, const Int64 base,
-                           const Int64 n, T *__restrict__ out, T *__restrict__ sum, const acc_scan_desc<T> &desc,
+                           const Int64 n, const Out &out, const acc_scan_desc<T> &desc,
                            const unsigned int epoch, void *s_wave_raw, T *s_prefix, Prefetch prefetch)
 {
   typedef acc_sv<T, PARTIAL> S;
@@ -316,7 +325,7 @@ ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op_raw, const T s
     for (int k = 0; k < ACC_VEC; ++k) {
       const Int64 ix = ACC_SCAN_RIGHT ? ix0[r] - k : ix0[r] + k;
       if (PARTIAL && ix >= n) continue;
-      acc_store(out + ix, exclusive ? S::val(k == 0 ? pre : inc[k - 1]) : S::val(inc[k]));
+      out.put(ix, exclusive ? S::val(k == 0 ? pre : inc[k - 1]) : S::val(inc[k]));
     }
 
     /* the reduction of the whole vector, held by the logically last element */
@@ -326,8 +335,8 @@ ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op_raw, const T s
       for (int k = 0; k < ACC_VEC; ++k) {
         const Int64 ix = ACC_SCAN_RIGHT ? ix0[r] - k : ix0[r] + k;
         if (ix == last) {
-          if (ACC_SCAN_MODE == 0) out[n] = S::val(inc[k]);
-          else                    sum[0] = S::val(inc[k]);
+          if (ACC_SCAN_MODE == 0) out.set(n, S::val(inc[k]));
+          else                    out.total(S::val(inc[k]));
         }
       }
     }
@@ -340,9 +349,9 @@ ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op_raw, const T s
  * when the prefix is known, to produce the results.  Speed is irrelevant
  * here (at most one such tile per launch); what matters is that its register
  * footprint does not dictate the kernel's.                                   */
-template <typename T, typename Op, typename Prefetch>
+template <typename T, typename Op, typename Prefetch, typename Out>
 ACC_DEV void acc_scan_tile_ragged(const T (&x)[ACC_ROWS][ACC_VEC], Op op_raw, const T seed, const Int64 tile,
-                                  const Int64 base, const Int64 n, T *__restrict__ out, T *__restrict__ sum,
+                                  const Int64 base, const Int64 n, const Out &out,
                                   const acc_scan_desc<T> &desc, const unsigned int epoch, void *s_wave_raw,
                                   T *s_prefix, Prefetch prefetch)
 {
@@ -424,10 +433,10 @@ ACC_DEV void acc_scan_tile_ragged(const T (&x)[ACC_ROWS][ACC_VEC], Op op_raw, co
       acc = op(acc, item(r, k));
       if (ix < n) {
         const bool exclusive = (ACC_SCAN_MODE == 0 || ACC_SCAN_MODE == 2);
-        out[ix] = exclusive ? before.v : acc.v;
+        out.set(ix, exclusive ? before.v : acc.v);
         if (ix == last) {
-          if (ACC_SCAN_MODE == 0) out[n] = acc.v;
-          if (ACC_SCAN_MODE == 2) sum[0] = acc.v;
+          if (ACC_SCAN_MODE == 0) out.set(n, acc.v);
+          if (ACC_SCAN_MODE == 2) out.total(acc.v);
         }
       }
     }
@@ -454,8 +463,8 @@ ACC_DEV void acc_scan_tile_ragged(const T (&x)[ACC_ROWS][ACC_VEC], Op op_raw, co
 #endif
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK, ACC_MIN_WAVES)
 ACC_ENTRY(ACC_ENV_PARAMS
-          const Int64 shOut_0, ACC_ELT *__restrict__ arrOut_0,
-          ACC_ELT *__restrict__ arrSum_0,
+          const Int64 shOut_0, ACC_OUT_ARRAY(arrOut),
+          ACC_OUT_ARRAY(arrSum),
           const Int64 shIn_0,
           unsigned int *__restrict__ tile_counter, const unsigned int counter_base,
           void *desc0, void *desc1, void *desc2,
@@ -464,7 +473,7 @@ ACC_ENTRY(ACC_ENV_PARAMS
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
 #if ACC_ALIGNED
-  arrOut_0 = (T *)__builtin_assume_aligned(arrOut_0, 16);
+  ACC_OUT_ASSUME(arrOut)
 #endif
   (void)shOut_0;
 
@@ -484,6 +493,11 @@ ACC_ENTRY(ACC_ENV_PARAMS
   const int lane = acc_lane();
   const int wave = (int)(threadIdx.x >> 6);
   const acc_scan_desc<T> desc(desc0, desc1, desc2);
+  /* where results go: one array per component of the element */
+  auto put_fn   = [&](const Int64 ix, const T &v) { ACC_PUT(arrOut, ix, v); };      /* the body, streaming */
+  auto set_fn   = [&](const Int64 ix, const T &v) { ACC_SET(arrOut, ix, v); };
+  auto total_fn = [&](const T &v) { ACC_SET(arrSum, 0, v); };
+  const acc_scan_out<decltype(put_fn), decltype(set_fn), decltype(total_fn)> out = {put_fn, set_fn, total_fn};
   auto tile_base = [&](const Int64 t) -> Int64 { return (ACC_SCAN_RIGHT ? (num_tiles - 1 - t) : t) * (Int64)ACC_TILE; };
 
 #if ACC_SCAN_PERSISTENT == 1
@@ -502,12 +516,12 @@ ACC_ENTRY(ACC_ENV_PARAMS
 
   if (n <= 0) {                                   /* PrefixSum.hs:249-251,330-334: scan of nothing is [seed] */
     if (threadIdx.x == 0 && tile == 0) {
-      if (ACC_SCAN_MODE == 0 || ACC_SCAN_MODE == 3) arrOut_0[0] = seed;
-      if (ACC_SCAN_MODE == 2) arrSum_0[0] = seed;
+      if (ACC_SCAN_MODE == 0 || ACC_SCAN_MODE == 3) ACC_SET(arrOut, 0, seed);
+      if (ACC_SCAN_MODE == 2) ACC_SET(arrSum, 0, seed);
     }
     return;
   }
-  if (ACC_SCAN_MODE == 3 && tile == 0 && threadIdx.x == 0) arrOut_0[n] = seed;
+  if (ACC_SCAN_MODE == 3 && tile == 0 && threadIdx.x == 0) ACC_SET(arrOut, n, seed);
 
   T cur[ACC_ROWS][ACC_VEC];
   if (tile < num_tiles) acc_scan_load(get, tile_base(tile), n, cur, wave, lane);
@@ -541,9 +555,9 @@ ACC_ENTRY(ACC_ENV_PARAMS
 
     const Int64 base = tile_base(tile);
     if (base + ACC_TILE <= n)
-      acc_scan_tile<false, T>(cur, op, seed, tile, base, n, arrOut_0, arrSum_0, desc, epoch, (void *)s_wave, &s_prefix, prefetch);
+      acc_scan_tile<false, T>(cur, op, seed, tile, base, n, out, desc, epoch, (void *)s_wave, &s_prefix, prefetch);
     else
-      acc_scan_tile_ragged<T>(cur, op, seed, tile, base, n, arrOut_0, arrSum_0, desc, epoch, (void *)s_wave, &s_prefix, prefetch);
+      acc_scan_tile_ragged<T>(cur, op, seed, tile, base, n, out, desc, epoch, (void *)s_wave, &s_prefix, prefetch);
 
 #if ACC_SCAN_PERSISTENT
 #pragma unroll

@@ -80,22 +80,37 @@ int push_env(const acc_skel_s *s, const acc_array *env, Args *args, bool *aligne
   return ACC_OK;
 }
 
-int check_out(const acc_skel_s *s, const acc_array *out, int rank, const char *what)
+int check_out(const acc_skel_s *s, const acc_array *out, int rank, const char *what, int ncomp)
 {
   if (!out) return fail(ACC_ERR_INVALID, "%s: %s array missing", s->entry.c_str(), what);
   if (out->rank != rank) return fail(ACC_ERR_INVALID, "%s: %s array has rank %d, expected %d", s->entry.c_str(), what, out->rank, rank);
-  if (out->ncomp != 1) return fail(ACC_ERR_UNSUPPORTED, "%s: tuple-typed %s arrays are not supported", s->entry.c_str(), what);
+  if (out->ncomp != ncomp)
+    return fail(ncomp == 1 ? ACC_ERR_UNSUPPORTED : ACC_ERR_INVALID, "%s: %s array has %d components, the kernel was built for %d",
+                s->entry.c_str(), what, out->ncomp, ncomp);
   for (int d = 0; d < rank; ++d)
     if (out->shape[d] < 0) return fail(ACC_ERR_INVALID, "%s: %s array has a negative extent", s->entry.c_str(), what);
-  if (!out->ptr[0] && array_size(*out) > 0) return fail(ACC_ERR_INVALID, "%s: %s array is NULL", s->entry.c_str(), what);
+  for (int c = 0; c < ncomp; ++c)
+    if (!out->ptr[c] && array_size(*out) > 0) return fail(ACC_ERR_INVALID, "%s: %s array is NULL", s->entry.c_str(), what);
   return ACC_OK;
+}
+
+// an array of the skeleton's element type: one component, or the tuple's
+int check_out(const acc_skel_s *s, const acc_array *out, int rank, const char *what) { return check_out(s, out, rank, what, s->ncomp()); }
+
+// the component pointers of a result array, highest component first; NULL array = that many null pointers
+void push_ptrs(const acc_array *a, int ncomp, Args *args, bool *aligned)
+{
+  for (int c = ncomp - 1; c >= 0; --c) {
+    const uint64_t p = a ? a->ptr[c] : 0;
+    if (a && !aligned16(p)) *aligned = false;
+    args->ptr(p);
+  }
 }
 
 void push_out(const acc_array &out, Args *args, bool *aligned)
 {
   for (int d = 0; d < out.rank; ++d) args->i64(out.shape[d]);
-  if (!aligned16(out.ptr[0])) *aligned = false;
-  args->ptr(out.ptr[0]);
+  push_ptrs(&out, out.ncomp, args, aligned);
 }
 
 int launch(acc_skel_s *s, int variant, int64_t grid, size_t dyn_lds, hipStream_t stream, Args *args)
@@ -166,7 +181,7 @@ int acc_exec_fold(acc_skel s, const acc_array *env, int32_t in_rank, const int64
 
   if (s->spec.out_rank > 0) {      // one wave per innermost row
     args.i64(rows);
-    args.ptr(out->ptr[0]);
+    push_ptrs(out, out->ncomp, &args, &aligned);
     args.i64(rows);
     args.i64(inner);
     const int waves = s->spec.block / 64;
@@ -179,7 +194,7 @@ int acc_exec_fold(acc_skel s, const acc_array *env, int32_t in_rank, const int64
   const int64_t grid = acc_launch_grid(n, tile, s->ctx->props.multiProcessorCount,
                                        std::min(s->variants[v].blocks_per_cu, acc::tune("fold.blocks_per_cu", 4)));
   if (grid == 1) {                 // a lone block finishes the job itself
-    args.ptr(out->ptr[0]);
+    push_ptrs(out, out->ncomp, &args, &aligned);
     args.i64(n);
     args.ptr(0);
     return launch(s, v, 1, 0, st, &args);
@@ -189,7 +204,7 @@ int acc_exec_fold(acc_skel s, const acc_array *env, int32_t in_rank, const int64
   int blk = -1;
   ACC_TRY(s->ctx->scratch_acquire((size_t)grid * s->spec.elt_size, st, acc::SCRATCH_FOLD, &blk));
   const uint64_t partials = reinterpret_cast<uint64_t>(s->ctx->scratch[blk].ptr);
-  args.ptr(out->ptr[0]);
+  push_ptrs(out, out->ncomp, &args, &aligned);
   args.i64(n);
   args.ptr(partials);
   int rc = launch(s, v, grid, 0, st, &args);
@@ -197,7 +212,7 @@ int acc_exec_fold(acc_skel s, const acc_array *env, int32_t in_rank, const int64
     Args fin;
     bool al = true;
     rc = push_env(s, env, &fin, &al);
-    fin.ptr(out->ptr[0]);
+    push_ptrs(out, out->ncomp, &fin, &al);
     fin.ptr(partials);
     fin.i64(grid);
     if (rc == ACC_OK) {
@@ -213,7 +228,7 @@ int acc_exec_foldseg(acc_skel s, const acc_array *env, int64_t n, const acc_arra
 {
   if (!s) return fail(ACC_ERR_INVALID, "acc_exec_foldseg: NULL skeleton");
   if (!kind_is(s, {ACC_SKEL_FOLDSEG, ACC_SKEL_FOLD1SEG})) return fail(ACC_ERR_INVALID, "acc_exec_foldseg: skeleton is '%s'", s->entry.c_str());
-  ACC_TRY(check_out(s, offsets, 1, "segment offsets"));
+  ACC_TRY(check_out(s, offsets, 1, "segment offsets", 1));
   ACC_TRY(check_out(s, out, 1, "result"));
   if (n < 0) return fail(ACC_ERR_INVALID, "%s: negative input extent", s->entry.c_str());
   // the offsets vector is one longer than the number of segments: Execute.hs:320-324
@@ -224,7 +239,7 @@ int acc_exec_foldseg(acc_skel s, const acc_array *env, int64_t n, const acc_arra
   bool aligned = true;
   ACC_TRY(push_env(s, env, &args, &aligned));
   args.i64(nseg);
-  args.ptr(out->ptr[0]);
+  push_ptrs(out, out->ncomp, &args, &aligned);
   args.i64(n);
   args.ptr(offsets->ptr[0]);
   const int v = aligned ? 0 : 1;
@@ -245,11 +260,7 @@ int acc_exec_scan(acc_skel s, const acc_array *env, int64_t n, const acc_array *
   const bool primed = (kind == ACC_SKEL_SCANLP || kind == ACC_SKEL_SCANRP);     // Execute.hs:352-362
   if (out->shape[0] < n + (plus_one ? 1 : 0))
     return fail(ACC_ERR_INVALID, "%s: result holds %lld elements, %lld needed", s->entry.c_str(), (long long)out->shape[0], (long long)(n + (plus_one ? 1 : 0)));
-  uint64_t sum_ptr = 0;
-  if (primed) {
-    ACC_TRY(check_out(s, total, 0, "total"));
-    sum_ptr = total->ptr[0];
-  }
+  if (primed) ACC_TRY(check_out(s, total, 0, "total"));
   if (n == 0 && !plus_one && !primed) return ACC_OK;       // scanl1 / scanr1 of nothing is nothing
 
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -257,7 +268,10 @@ int acc_exec_scan(acc_skel s, const acc_array *env, int64_t n, const acc_array *
   bool aligned = true;
   ACC_TRY(push_env(s, env, &args, &aligned));
   push_out(*out, &args, &aligned);
-  args.ptr(sum_ptr);
+  {
+    bool ignore = true;      // a scalar's alignment decides nothing
+    push_ptrs(primed ? total : nullptr, s->ncomp(), &args, &ignore);
+  }
   args.i64(n);
 
   const int v = aligned ? 0 : 1;
@@ -461,7 +475,7 @@ static int stencil_check(acc_skel s, const acc_array *in, const acc_array *out)
   if (!s) return fail(ACC_ERR_INVALID, "acc_exec_stencil: NULL skeleton");
   if (!kind_is(s, {ACC_SKEL_STENCIL})) return fail(ACC_ERR_INVALID, "acc_exec_stencil: skeleton is '%s'", s->entry.c_str());
   ACC_TRY(check_out(s, out, s->spec.out_rank, "result"));
-  ACC_TRY(check_out(s, in, s->spec.out_rank, "source"));
+  ACC_TRY(check_out(s, in, s->spec.out_rank, "source", 1));
   for (int d = 0; d < out->rank; ++d)
     if (in->shape[d] != out->shape[d]) return fail(ACC_ERR_INVALID, "stencil: source and result differ in shape");
   if (in->ptr[0] == out->ptr[0] && array_size(*out) > 0) return fail(ACC_ERR_INVALID, "stencil: source and result must not alias");

@@ -95,7 +95,8 @@ static std::string out_params(int rank, const std::string &elt)
 {
   std::ostringstream o;
   for (int d = rank - 1; d >= 0; --d) o << "const Int64 shOut_" << d << ", ";
-  o << elt << " *__restrict__ arrOut_0";
+  (void)elt;
+  o << "ACC_OUT_ARRAY(arrOut)";
   return o.str();
 }
 
@@ -121,10 +122,41 @@ static const char *kind_name(int kind)
 int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::string *source)
 {
   std::ostringstream o;
-  const int esz = sp.elt_size;
-  int vec = std::max(1, 16 / std::max(1, esz));
+  int vec = std::max(1, 16 / std::max(1, sp.vec_size));
   o << "// accelerate-hip " ACC_HIP_VERSION " skeleton instance: " << kind_name(sp.kind) << "\n";
   o << "#define ACC_ELT " << sp.elt_type << "\n";
+  // The result array(s): one pointer per component, highest component first (CodeGen/Base.hs:344-357).
+  //   ACC_OUT_ARRAY(name)   the pointer parameters  name_<c>
+  //   ACC_OUT_ASSUME(name)  16-byte alignment of each
+  //   ACC_PUT(name, ix, v)  element ix := v, as a streaming store
+  //   ACC_SET(name, ix, v)  the same as an ordinary store (small results that are read again soon)
+  {
+    const int nc = sp.comp_types.empty() ? 1 : (int)sp.comp_types.size();
+    std::ostringstream arr, assume, put, set;
+    for (int i = 0; i < nc; ++i) {
+      const int c = nc - 1 - i;
+      const std::string t = sp.comp_types.empty() ? std::string("ACC_ELT") : sp.comp_types[i];
+      arr << (i ? ", " : "") << t << " *__restrict__ name##_" << c;
+      assume << "name##_" << c << " = (" << t << " *)__builtin_assume_aligned(name##_" << c << ", 16); ";
+      if (sp.comp_types.empty()) {
+        put << "acc_store(name##_0 + (ix), (v))";
+        set << "name##_0[ix] = (v)";
+      } else {
+        put << "acc_store(name##_" << c << " + (ix), acc_pv.a" << c << "); ";
+        set << "name##_" << c << "[ix] = acc_pv.a" << c << "; ";
+      }
+    }
+    o << "#define ACC_NCOMP " << nc << "\n";
+    o << "#define ACC_OUT_ARRAY(name) " << arr.str() << "\n";
+    o << "#define ACC_OUT_ASSUME(name) " << (aligned ? assume.str() : std::string()) << "\n";
+    if (sp.comp_types.empty()) {
+      o << "#define ACC_PUT(name, ix, v) " << put.str() << "\n";
+      o << "#define ACC_SET(name, ix, v) " << set.str() << "\n";
+    } else {
+      o << "#define ACC_PUT(name, ix, v) do { const ACC_ELT acc_pv = (v); " << put.str() << "} while (0)\n";
+      o << "#define ACC_SET(name, ix, v) do { const ACC_ELT acc_pv = (v); " << set.str() << "} while (0)\n";
+    }
+  }
   o << "#define ACC_ALIGNED " << (aligned ? 1 : 0) << "\n";
   o << "#define ACC_ENV_PARAMS " << env_params(sp.env) << "\n";
   o << "#define ACC_ENV_ASSUME " << env_assume(sp.env, aligned) << "\n";
@@ -220,6 +252,13 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
   o << "#define ACC_ENTRY " << *entry << "\n";
   o << "#define ACC_NT_STORE " << tune("nt_store", 1) << "\n";
   o << "#include \"acc_hip_device.h\"\n";
+  if (!sp.comp_types.empty()) {
+    // a tuple element: fields a<c>, component 0 last, so that brace initialisation reads like the tuple
+    o << "struct acc_elt { ";
+    const int nc = (int)sp.comp_types.size();
+    for (int i = 0; i < nc; ++i) o << sp.comp_types[i] << " a" << (nc - 1 - i) << "; ";
+    o << "};\n";
+  }
   if (!sp.preamble.empty()) o << sp.preamble << "\n";
   o << "#include \"" << tmpl << "\"\n";
   *source = o.str();
@@ -237,8 +276,34 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
   sp->kind = d->kind;
   sp->flags = d->flags;
   sp->elt_type = d->elt_type;
-  sp->elt_size = d->elt_size > 0 ? d->elt_size : type_size(sp->elt_type);
-  if (sp->elt_size <= 0) return fail(ACC_ERR_INVALID, "cannot size element type '%s': set elt_size", d->elt_type);
+  if (sp->elt_type.find(',') != std::string::npos) {
+    // a tuple: "T<n-1>, ..., T0"; laid out as the struct the generator declares
+    size_t pos = 0;
+    int size = 0, align = 1;
+    while (pos <= sp->elt_type.size()) {
+      size_t end = sp->elt_type.find(',', pos);
+      if (end == std::string::npos) end = sp->elt_type.size();
+      std::string t = sp->elt_type.substr(pos, end - pos);
+      t.erase(0, t.find_first_not_of(" \t"));
+      t.erase(t.find_last_not_of(" \t") + 1);
+      const int ts = type_size(t);
+      if (ts <= 0) return fail(ACC_ERR_INVALID, "tuple element type: unknown component type '%s'", t.c_str());
+      sp->comp_types.push_back(t);
+      size = (size + ts - 1) / ts * ts + ts;
+      align = std::max(align, ts);
+      sp->vec_size = std::max(sp->vec_size, ts);
+      pos = end + 1;
+    }
+    if ((int)sp->comp_types.size() > ACC_MAX_COMP) return fail(ACC_ERR_INVALID, "tuple element type: more than %d components", ACC_MAX_COMP);
+    sp->elt_size = (size + align - 1) / align * align;
+    sp->elt_type = "acc_elt";
+    if (d->kind == ACC_SKEL_PERMUTE || d->kind == ACC_SKEL_STENCIL)
+      return fail(ACC_ERR_UNSUPPORTED, "%s: tuple element types are not supported by this skeleton", kind_name(d->kind));
+  } else {
+    sp->elt_size = d->elt_size > 0 ? d->elt_size : type_size(sp->elt_type);
+    if (sp->elt_size <= 0) return fail(ACC_ERR_INVALID, "cannot size element type '%s': set elt_size", d->elt_type);
+    sp->vec_size = sp->elt_size;
+  }
   sp->out_rank = d->out_rank;
   if (sp->out_rank < 0 || sp->out_rank > ACC_MAX_RANK) return fail(ACC_ERR_INVALID, "bad out_rank %d", d->out_rank);
   for (int k = 0; k < d->n_env; ++k) {

@@ -15,8 +15,10 @@ struct SkelSpec {
   int kind = 0;
   uint32_t flags = 0;
   std::vector<EnvSig> env;
-  std::string elt_type;
-  int elt_size = 0;
+  std::string elt_type;                 // C type of the element; "acc_elt" for a tuple
+  int elt_size = 0;                     // sizeof(elt_type)
+  std::vector<std::string> comp_types;  // tuple elements: the component types, left to right (component ncomp-1 first)
+  int vec_size = 0;                     // bytes of the widest component: decides how many elements a lane takes per access
   int out_rank = 0;
   std::string preamble, get, combine, seed, permutation;
   bool has_seed = false;
@@ -60,7 +62,8 @@ struct acc_skel_s {
   std::mutex mu;
 
   int ensure_variant(int v);
-  int vec() const { int v = 16 / (spec.elt_size > 0 ? spec.elt_size : 1); return v < 1 ? 1 : v; }
+  int ncomp() const { return spec.comp_types.empty() ? 1 : (int)spec.comp_types.size(); }
+  int vec() const { int v = 16 / (spec.vec_size > 0 ? spec.vec_size : 1); return v < 1 ? 1 : v; }
   int elements_per_block() const
   {
     switch (spec.kind) {

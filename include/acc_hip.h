@@ -256,7 +256,12 @@ typedef struct acc_skel_desc {
   uint32_t           flags;         /* ACC_FLAG_*                                           */
   int32_t            n_env;         /* free array variables In0 .. In<n_env-1>              */
   const acc_env_sig *env;
-  const char        *elt_type;      /* C type of the result element (single component)      */
+  const char        *elt_type;      /* C type of the result element, or "T<n-1>, ..., T0" for a
+                                     * tuple: the generated code then declares
+                                     *   struct acc_elt { T<n-1> a<n-1>; ...; T0 a0; };
+                                     * fragments produce and take apart acc_elt values, and the
+                                     * result array has one pointer per component (CodeGen/
+                                     * Base.hs:344-357); not for permute and stencil          */
   int32_t            elt_size;      /* sizeof(elt_type); 0 = derive from the type's name    */
   int32_t            out_rank;      /* map family, stencil: rank of the result (>= 0)       */
   const char        *preamble;      /* file-scope declarations for the fragments, or NULL   */

@@ -1,0 +1,164 @@
+"""Tuple element types (structure of arrays, one result pointer per component)
+through map, fold, fold along a dimension, foldSeg and the scans.
+
+What each case is checked against is independent of the kernels: numpy's
+argmax / cumsum / reduceat / minimum / maximum, or a sequential Python loop
+for the non-commutative operator.  Integer components are compared bit for
+bit; the one Float64 sum states its tolerance.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+F32, I32 = (1, "float"), (1, "Int32")
+SIZES = [1, 63, 64, 65, 4097, 100003, (1 << 20) + 17]
+
+
+def say(*a):
+    print("[case]", *a)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def A():
+    import acchip
+    return acchip
+
+
+@pytest.fixture(scope="module")
+def ctx(A):
+    c = A.Context(0)
+    yield c
+    c.close()
+
+
+def test_map_builds_and_takes_apart_pairs(A, ctx):
+    rng = np.random.default_rng(3)
+    zipk = ctx.skeleton(A.SKEL_MAP, "float, Int32", env=[F32, I32], out_rank=1, get="acc_elt{arrIn0_0[ix] * 2.0f, arrIn1_0[ix] + 1}")
+    # a free array of pairs: component 1 is the first element, component 0 the second
+    swap = ctx.skeleton(A.SKEL_MAP, "Int32, float", env=[(1, ["Int32", "float"])], out_rank=1,
+                        get="acc_elt{arrIn0_0[ix], arrIn0_1[ix]}")
+    for n in [0] + SIZES:
+        say("zip / swap, n =", n)
+        x = rng.random(n).astype(np.float32)
+        k = rng.integers(-1000, 1000, n).astype(np.int32)
+        out = ctx.empty_tuple(n, [np.float32, np.int32])
+        zipk.map([ctx.array(x), ctx.array(k)], out)
+        a, b = out.get()
+        assert np.array_equal(a, x * np.float32(2)) and np.array_equal(b, k + 1)
+        out2 = ctx.empty_tuple(n, [np.int32, np.float32])
+        swap.map([out], out2)
+        b2, a2 = out2.get()
+        assert np.array_equal(a2, a) and np.array_equal(b2, b)
+
+
+def test_fold_argmax_of_value_index_pairs(A, ctx):
+    rng = np.random.default_rng(4)
+    argmax = ctx.skeleton(A.SKEL_FOLD, "float, Int32", env=[F32], out_rank=0, get="acc_elt{arrIn0_0[ix], (Int32)ix}",
+                          combine="(x.a1 > y.a1 || (x.a1 == y.a1 && x.a0 < y.a0)) ? x : y", seed="acc_elt{-1.0f, 2147483647}")
+    for n in [0] + SIZES + [1 << 24]:
+        say("argmax, n =", n)
+        x = rng.integers(0, 1000, n).astype(np.float32)          # many ties: the smallest index must win
+        out = ctx.empty_tuple((), [np.float32, np.int32])
+        argmax.fold([ctx.array(x)], n, out)
+        v, i = out.get()
+        if n == 0:
+            assert float(v) == -1.0 and int(i) == 2147483647      # the seed
+        else:
+            assert int(i) == int(np.argmax(x)) and float(v) == float(x.max())
+
+
+def test_fold_along_rows_min_and_max(A, ctx):
+    rng = np.random.default_rng(5)
+    mm = ctx.skeleton(A.SKEL_FOLD, "Int32, Int32", env=[(2, "Int32")], out_rank=1, get="acc_elt{arrIn0_0[ix], arrIn0_0[ix]}",
+                      combine="acc_elt{acc_pmin(x.a1, y.a1), acc_pmax(x.a0, y.a0)}", seed="acc_elt{2147483647, -2147483647 - 1}")
+    for rows, cols in [(1, 1), (7, 100), (300, 65), (64, 4096), (1000, 1001)]:
+        say("row-wise (min, max)", rows, "x", cols)
+        x = rng.integers(-10 ** 9, 10 ** 9, (rows, cols)).astype(np.int32)
+        out = ctx.empty_tuple(rows, [np.int32, np.int32])
+        mm.fold([ctx.array(x)], (rows, cols), out)
+        lo, hi = out.get()
+        assert np.array_equal(lo, x.min(axis=1)) and np.array_equal(hi, x.max(axis=1))
+
+
+def test_foldseg_sum_and_count(A, ctx):
+    rng = np.random.default_rng(6)
+    sc = ctx.skeleton(A.SKEL_FOLDSEG, "double, Int32", env=[F32], get="acc_elt{(double)arrIn0_0[ix], 1}",
+                      combine="acc_elt{x.a1 + y.a1, x.a0 + y.a0}", seed="acc_elt{0.0, 0}")
+    for nseg in [1, 5, 257, 10000]:
+        say("foldSeg (sum, count), segments =", nseg)
+        lens = rng.poisson(20, nseg).astype(np.int32)
+        lens[::7] = 0
+        offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        n = int(offs[-1])
+        x = rng.random(n).astype(np.float32)
+        out = ctx.empty_tuple(nseg, [np.float64, np.int32])
+        sc.foldseg([ctx.array(x)], n, ctx.array(offs), out)
+        s, c = out.get()
+        assert np.array_equal(c, lens)
+        exp = np.array([x[offs[i]:offs[i + 1]].astype(np.float64).sum() for i in range(nseg)])
+        assert np.all(np.abs(s - exp) <= 1e-12 * np.maximum(1.0, np.abs(exp)))      # Float64 sums of <= ~50 Float32 values
+
+
+def segmented_cumsum(flags, vals):
+    out = np.empty_like(vals)
+    run = 0
+    for i in range(vals.size):
+        run = int(vals[i]) if flags[i] else run + int(vals[i])
+        out[i] = np.int32(run)
+    return out
+
+
+@pytest.mark.parametrize("kind", ["scanl1", "scanl", "scanl'", "scanr1"])
+def test_segmented_scan_with_flag_value_pairs(A, ctx, kind):
+    """(f1, v1) (+) (f2, v2) = (f1 | f2, f2 ? v2 : v1 + v2): associative, not commutative"""
+    rng = np.random.default_rng(7)
+    seeded = not kind.endswith("1")
+    right = kind.startswith("scanr")
+    # op(earlier, later) in logical order; the right-handed scans are handed f with its arguments as Data.List has them
+    body = "acc_elt{E.a1 | L.a1, L.a1 ? L.a0 : E.a0 + L.a0}"
+    combine = body.replace("E", "y").replace("L", "x") if right else body.replace("E", "x").replace("L", "y")
+    sk = ctx.skeleton(A.SCAN_KINDS[kind], "Int32, Int32", env=[I32, I32], get="acc_elt{arrIn0_0[ix], arrIn1_0[ix]}",
+                      combine=combine, seed="acc_elt{0, 0}" if seeded else None)
+    for n in SIZES:
+        say(kind, "segmented sum, n =", n)
+        flags = (rng.random(n) < 0.01).astype(np.int32)
+        vals = rng.integers(-100, 100, n).astype(np.int32)
+        m = n + 1 if kind == "scanl" else n
+        out = ctx.empty_tuple(m, [np.int32, np.int32])
+        tot = ctx.empty_tuple((), [np.int32, np.int32]) if kind == "scanl'" else None
+        sk.scan([ctx.array(flags), ctx.array(vals)], n, out, tot)
+        gf, gv = out.get()
+        if right:       # scanr1: the same recurrence walking from the end
+            exp = segmented_cumsum(flags[::-1], vals[::-1])[::-1]
+            assert np.array_equal(gv, exp) and np.array_equal(gf, np.maximum.accumulate(flags[::-1])[::-1])
+            continue
+        inc = segmented_cumsum(flags, vals)                       # inclusive results; the seed (0, 0) is an identity here
+        incf = np.maximum.accumulate(flags)
+        if kind == "scanl1":
+            assert np.array_equal(gv, inc) and np.array_equal(gf, incf)
+        elif kind == "scanl":
+            assert gv[0] == 0 and gf[0] == 0 and np.array_equal(gv[1:], inc) and np.array_equal(gf[1:], incf)
+        else:
+            tf, tv = tot.get()
+            assert gv[0] == 0 and np.array_equal(gv[1:], inc[:-1]) and np.array_equal(gf[1:], incf[:-1])
+            assert int(tv) == int(inc[-1]) and int(tf) == int(incf[-1])
+
+
+def test_tuple_results_need_tuple_arrays_and_are_refused_elsewhere(A, ctx):
+    say("misuse")
+    zipk = ctx.skeleton(A.SKEL_MAP, "float, Int32", env=[F32], out_rank=1, get="acc_elt{arrIn0_0[ix], 0}")
+    x = ctx.array(np.zeros(8, np.float32))
+    with pytest.raises(A.AccError) as e:
+        zipk.map([x], ctx.empty(8, np.float32))                  # one component offered, two needed
+    assert e.value.code == A.ERR_INVALID
+    with pytest.raises(A.AccError) as e:
+        ctx.skeleton(A.SKEL_PERMUTE, "float, Int32", env=[I32], out_rank=1, get="acc_elt{1.0f, 1}", combine="x",
+                     permutation="arrIn0_0[ix]")
+    assert e.value.code == A.ERR_UNSUPPORTED
+    with pytest.raises(A.AccError) as e:
+        ctx.skeleton(A.SKEL_MAP, "float, quux", env=[F32], out_rank=1, get="acc_elt{1.0f, 1}")
+    assert e.value.code == A.ERR_INVALID

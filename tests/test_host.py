@@ -198,7 +198,13 @@ def test_generated_parameter_abi_follows_the_reference(A):
     assert defs["ACC_ENV_PARAMS"].strip() == (
         "const Int64 shIn0_1, const Int64 shIn0_0, const Int32 *__restrict__ arrIn0_1, "
         "const float *__restrict__ arrIn0_0, const Int64 shIn1_0, const double *__restrict__ arrIn1_0,")
-    assert defs["ACC_OUT_PARAMS"].strip() == "const Int64 shOut_1, const Int64 shOut_0, float *__restrict__ arrOut_0"
+    assert defs["ACC_OUT_PARAMS"].strip() == "const Int64 shOut_1, const Int64 shOut_0, ACC_OUT_ARRAY(arrOut)"
+    assert defs["ACC_OUT_ARRAY"].strip() == "ACC_ELT *__restrict__ name##_0" and defs["ACC_ELT"].strip() == "float"
+    # a tuple result: one pointer per component, highest component first, the element a struct with fields a<c>
+    _, tsrc = A.preview(A.make_desc(A.SKEL_MAP, "float, Int32, double", env=env, out_rank=1, get="acc_elt{1.0f, 2, 3.0}"))
+    tdefs = dict(m.groups() for m in re.finditer(r"^#define (\w+)(?:\([^)]*\))? (.*)$", tsrc, flags=re.M))
+    assert tdefs["ACC_OUT_ARRAY"].strip() == "float *__restrict__ name##_2, Int32 *__restrict__ name##_1, double *__restrict__ name##_0"
+    assert "struct acc_elt { float a2; Int32 a1; double a0; };" in tsrc and tdefs["ACC_ELT"].strip() == "acc_elt"
     assert defs["ACC_OUT_SIZE"].strip() == "(shOut_1 * shOut_0)"
     assert src.rstrip().endswith('#include "skel_map.h"') and '#include "acc_hip_device.h"' in src
     assert "__builtin_assume_aligned" in src and "__builtin_assume_aligned" not in A.preview(d, 1)[1]
