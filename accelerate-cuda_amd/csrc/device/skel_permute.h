@@ -221,43 +221,59 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
   }
 }
 
-/* fills p[0 .. count) with the combine's identity */
+/* fills p[0 .. count) with the combine's identity and copies copy_count
+ * elements from copy_src to copy_dst (the defaults into the result): the two
+ * small jobs that precede the main kernel, in one launch */
 extern "C" __global__ void __launch_bounds__(256)
-permute_fill(ACC_ELT *__restrict__ p, const Int64 count)
+permute_fill(ACC_ELT *__restrict__ p, const Int64 count, ACC_ELT *__restrict__ copy_dst,
+             const ACC_ELT *__restrict__ copy_src, const Int64 copy_count)
 {
   const ACC_ELT ident = acc_hint_identity<ACC_ELT>();
-  for (Int64 i = (Int64)blockIdx.x * 256 + threadIdx.x; i < count; i += (Int64)gridDim.x * 256) p[i] = ident;
+  const Int64 first = (Int64)blockIdx.x * 256 + threadIdx.x, step = (Int64)gridDim.x * 256;
+  for (Int64 i = first; i < count; i += step) p[i] = ident;
+  for (Int64 i = first; i < copy_count; i += step) copy_dst[i] = copy_src[i];
 }
 
-/* folds columns [first, first + cols) of the table dump[nrows][stride] into the
- * same positions of the result.  The rows are split into `slices` groups
- * handled by different workgroups; with one slice the result is written
- * plainly, otherwise each group applies its share with one atomic per target. */
+/* one table to fold: columns [first, first + cols) of dump[nrows][stride] go
+ * into the same positions of the result.  The rows are split into `slices`
+ * groups handled by different workgroups; with one slice the result is
+ * written plainly, otherwise each group applies its share with one atomic per
+ * target.                                                                    */
+struct acc_merge_job {
+  const ACC_ELT *dump;
+  Int64 stride, first, cols;
+  int nrows, slices;
+};
+
+/* folds up to two tables in one launch: workgroups [0, blocks_a) take job a,
+ * the rest job b */
 extern "C" __global__ void __launch_bounds__(256)
-permute_merge(ACC_ENV_PARAMS ACC_OUT_PARAMS, const ACC_ELT *__restrict__ dump, const Int64 stride, const Int64 first,
-              const Int64 cols, const int nrows, const int slices)
+permute_merge(ACC_ENV_PARAMS ACC_OUT_PARAMS, const acc_merge_job a, const int blocks_a, const acc_merge_job b)
 {
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
   auto f = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
-  const Int64 column = (Int64)(blockIdx.x / slices) * 256 + threadIdx.x;
-  const int slice = (int)(blockIdx.x % slices);
-  if (column >= cols) return;
-  const int per = (nrows + slices - 1) / slices;
-  const int r0 = slice * per, r1 = acc_min(nrows, r0 + per);
+  const bool second = (int)blockIdx.x >= blocks_a;
+  const acc_merge_job job = second ? b : a;
+  const int block = second ? (int)blockIdx.x - blocks_a : (int)blockIdx.x;
+  const Int64 column = (Int64)(block / job.slices) * 256 + threadIdx.x;
+  const int slice = block % job.slices;
+  if (column >= job.cols) return;
+  const int per = (job.nrows + job.slices - 1) / job.slices;
+  const int r0 = slice * per, r1 = acc_min(job.nrows, r0 + per);
   if (r0 >= r1) return;
-  const T *src = dump + first + column;
-  T acc = src[(Int64)r0 * stride];
+  const T *src = job.dump + job.first + column;
+  T acc = src[(Int64)r0 * job.stride];
 #pragma unroll 8
-  for (int r = r0 + 1; r < r1; ++r) acc = f(src[(Int64)r * stride], acc);
-  T *dst = arrOut_0 + first + column;
-  if (slices == 1) {
+  for (int r = r0 + 1; r < r1; ++r) acc = f(src[(Int64)r * job.stride], acc);
+  T *dst = arrOut_0 + job.first + column;
+  if (job.slices == 1) {
     *dst = f(acc, *dst);
   } else {
     const T ident = acc_hint_identity<T>();
-    typename acc_bits<sizeof(T)>::type a, b;
-    __builtin_memcpy(&a, &acc, sizeof(T));
-    __builtin_memcpy(&b, &ident, sizeof(T));
-    if (a != b) acc_hint_apply<ACC_SCOPE_DEVICE>(dst, acc, f);
+    typename acc_bits<sizeof(T)>::type x, y;
+    __builtin_memcpy(&x, &acc, sizeof(T));
+    __builtin_memcpy(&y, &ident, sizeof(T));
+    if (x != y) acc_hint_apply<ACC_SCOPE_DEVICE>(dst, acc, f);
   }
 }

@@ -26,6 +26,7 @@ class Args {
   void u32(uint32_t v) { push(&v, sizeof(v)); }
   void i32(int32_t v) { push(&v, sizeof(v)); }
   void ptr(uint64_t v) { push(&v, sizeof(v)); }
+  size_t count() const { return slots_.size(); }
   void **data()
   {
     ptrs_.clear();
@@ -358,9 +359,13 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
   const size_t esz = s->spec.elt_size;
   ACC_TRY(s->ctx->make_current());
   // the result starts as a copy of the defaults: Execute.hs:401-406 (no lock array here)
-  if (ntarget > 0 && defaults->ptr[0] != out->ptr[0])
-    ACC_HIP_TRY(hipMemcpyAsync(reinterpret_cast<void *>(out->ptr[0]), reinterpret_cast<void *>(defaults->ptr[0]), (size_t)ntarget * esz, hipMemcpyDeviceToDevice, st));
-  if (n_src == 0 || ntarget == 0) return ACC_OK;
+  const bool copy_defaults = ntarget > 0 && defaults->ptr[0] != out->ptr[0];
+  auto plain_copy = [&]() -> int {
+    if (copy_defaults)
+      ACC_HIP_TRY(hipMemcpyAsync(reinterpret_cast<void *>(out->ptr[0]), reinterpret_cast<void *>(defaults->ptr[0]), (size_t)ntarget * esz, hipMemcpyDeviceToDevice, st));
+    return ACC_OK;
+  };
+  if (n_src == 0 || ntarget == 0) return plain_copy();
 
   Args args;
   bool aligned = true;
@@ -408,40 +413,52 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
     if (table) dump = base + far_bytes;
   }
   int rc = ACC_OK;
-  if (far_rows) {
+  if (far_rows) {                       // one launch: identity into the XCD rows, defaults into the result
     Args f;
     f.ptr(far);
     f.i64(XCD_ROWS * ntarget);
+    f.ptr(out->ptr[0]);
+    f.ptr(defaults->ptr[0]);
+    f.i64(copy_defaults ? ntarget : 0);
     const int64_t fill_grid = std::min<int64_t>((XCD_ROWS * ntarget + 255) / 256, 8 * (int64_t)cus);
     e = hipModuleLaunchKernel(s->variants[v].fn_fill, static_cast<unsigned>(fill_grid), 1, 1, 256, 1, 1, 0, st, f.data(), nullptr);
     if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(permute_fill)");
+  } else {
+    rc = plain_copy();
   }
   args.i32(static_cast<int32_t>(bins));
   args.i32(static_cast<int32_t>(copies));
   args.ptr(dump);
   args.ptr(far);
   if (rc == ACC_OK) rc = launch(s, v, grid, lds, st, &args);
-  // folds columns [first, first + cols) of a table of `rows` rows into the result
-  auto merge = [&](uint64_t tbl, int64_t stride, int64_t first, int64_t cols, int64_t rows) -> int {
+  if (rc == ACC_OK && (table || far_rows)) {
+    // the tables are folded into the result by one launch: the per-block window rows, the per-XCD rows
+    struct MergeJob { uint64_t dump; int64_t stride, first, cols; int32_t nrows, slices; };
+    auto job = [&](uint64_t tbl, int64_t stride, int64_t first, int64_t cols, int64_t rows, int64_t *blocks) {
+      // enough workgroups to fill the machine: columns x row slices
+      const int64_t columns = (cols + 255) / 256;
+      const int64_t slices = std::max<int64_t>(1, std::min<int64_t>(rows, (2 * cus + columns - 1) / columns));
+      *blocks = columns * slices;
+      return MergeJob{tbl, stride, first, cols, static_cast<int32_t>(rows), static_cast<int32_t>(slices)};
+    };
+    int64_t blocks_a = 0, blocks_b = 0;
+    MergeJob ja = {0, 0, 0, 0, 0, 1}, jb = {0, 0, 0, 0, 0, 1};
+    if (table) ja = job(dump, bins, 0, bins, grid, &blocks_a);
+    if (far_rows) jb = job(far, ntarget, bins, ntarget - bins, XCD_ROWS, &blocks_b);
     Args m;
     bool al = true;
-    ACC_TRY(push_env(s, env, &m, &al));
+    rc = push_env(s, env, &m, &al);
     push_out(*out, &m, &al);
-    // enough workgroups to fill the machine: columns x row slices
-    const int64_t columns = (cols + 255) / 256;
-    const int64_t slices = std::max<int64_t>(1, std::min<int64_t>(rows, (2 * cus + columns - 1) / columns));
-    m.ptr(tbl);
-    m.i64(stride);
-    m.i64(first);
-    m.i64(cols);
-    m.i32(static_cast<int32_t>(rows));
-    m.i32(static_cast<int32_t>(slices));
-    hipError_t me = hipModuleLaunchKernel(s->variants[v].fn_finish, static_cast<unsigned>(columns * slices), 1, 1, 256, 1, 1, 0, st, m.data(), nullptr);
-    if (me != hipSuccess) return acc::fail_hip(me, "hipModuleLaunchKernel(permute_merge)");
-    return ACC_OK;
-  };
-  if (rc == ACC_OK && table) rc = merge(dump, bins, 0, bins, grid);
-  if (rc == ACC_OK && far_rows) rc = merge(far, ntarget, bins, ntarget - bins, XCD_ROWS);
+    int32_t blocks_a32 = static_cast<int32_t>(blocks_a);
+    std::vector<void *> margs(m.data(), m.data() + m.count());
+    margs.push_back(&ja);
+    margs.push_back(&blocks_a32);
+    margs.push_back(&jb);
+    if (rc == ACC_OK) {
+      e = hipModuleLaunchKernel(s->variants[v].fn_finish, static_cast<unsigned>(blocks_a + blocks_b), 1, 1, 256, 1, 1, 0, st, margs.data(), nullptr);
+      if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(permute_merge)");
+    }
+  }
   if (blk >= 0) s->ctx->scratch_release(blk, st);
   return rc;
 }
