@@ -45,7 +45,7 @@ std::string embedded_text(const char *name);
 // the same (stream order makes that safe) or the event recorded at release
 // has completed.
 enum ScratchProtocol {
-  SCRATCH_FOLD = 0,   // word 0 is a ticket that every launch returns to zero; the rest is don't-care
+  SCRATCH_FOLD = 0,   // contents are don't-care: every launch writes what it reads (fold partials, permute tables)
   SCRATCH_SCAN = 1    // word 0 is a tile counter used relative to `counter_base`; tile descriptors
                       // carry `epoch`, so stale ones read as "not yet published"
 };

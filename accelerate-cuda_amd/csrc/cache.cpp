@@ -17,6 +17,7 @@
 #include <sys/types.h>
 #include <unistd.h>
 
+#include <atomic>
 #include <cerrno>
 #include <cstdlib>
 #include <cstring>
@@ -103,7 +104,9 @@ bool read_entry(const std::string &path, std::vector<char> *payload)
 bool write_entry(const std::string &dir, const std::string &path, const std::vector<char> &payload)
 {
   if (!mkdirs(dir)) return false;
-  const std::string tmp = path + ".tmp." + std::to_string(static_cast<long>(getpid()));
+  // unique per process and per call: two threads may be writing the same entry
+  static std::atomic<unsigned long> serial{0};
+  const std::string tmp = path + ".tmp." + std::to_string(static_cast<long>(getpid())) + "." + std::to_string(serial.fetch_add(1));
   {
     std::ofstream out(tmp, std::ios::binary | std::ios::trunc);
     if (!out) return false;

@@ -424,6 +424,8 @@ using acc::fail;
 
 int acc_skel_s::ensure_variant(int v)
 {
+  // two threads may meet here on the first launch that needs the unaligned variant
+  std::lock_guard<std::mutex> lock(mu);
   acc::Variant &var = variants[v];
   if (var.ready) return ACC_OK;
   std::string entry_name;

@@ -186,3 +186,37 @@ def test_scratch_pool_with_two_streams(A, ctx, orc):
     for i in range(4):
         assert np.array_equal(outs[i].get(), orc.scan("scanl", orc.OP_ADD, xs[i], seed=0))
         assert int(sums[i].get()) == int(xs[i].sum())
+
+
+def test_one_skeleton_launched_from_several_threads(A, ctx):
+    """the reference runs every computation in a bound thread of its own (State.hs:84-92):
+    threads sharing a context and a skeleton, each on its own stream, misaligned inputs so
+    that the lazily built second variant is first needed by all of them at once"""
+    import threading
+    say("four host threads, one scan skeleton, one stream each")
+    I32 = (1, "Int32")
+    scan = ctx.skeleton(A.SKEL_SCANL1, "Int32", env=[I32], get="arrIn0_0[ix]", combine="x + y")
+    n = (1 << 20) + 5
+    rng = np.random.default_rng(8)
+    results, errors = {}, []
+
+    def work(k):
+        try:
+            st = ctx.stream()
+            x = rng.integers(0, 16, n + 1, dtype=np.int32)
+            dx = ctx.array(x)
+            out = ctx.empty(n, np.int32)
+            for rep in range(5):
+                # a view that starts 4 bytes into the buffer: not 16-byte aligned
+                scan.scan([dx.desc(shape=(n,), offset_elems=1)], n, out, stream=st)
+            A.check(A.lib().acc_stream_sync(ctx.handle, st))
+            results[k] = np.array_equal(out.get(), np.cumsum(x[1:], dtype=np.int32))
+        except Exception as e:                          # noqa: BLE001
+            errors.append(e)
+    threads = [threading.Thread(target=work, args=(k,)) for k in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    assert results == {0: True, 1: True, 2: True, 3: True}

@@ -147,6 +147,45 @@ def test_kernel_cache_hit_miss_and_corruption(A, tmp_path):
     assert len([f for dp, _, fs in os.walk(d) for f in fs]) < n_before
 
 
+def test_concurrent_compilation_from_many_threads(A, tmp_path):
+    """the reference compiles on a pool of worker threads (Compile.hs:620-660): several
+    threads asking for the same and for different kernels at once must all be served,
+    and the disk entries they leave must be whole"""
+    import threading
+    L = A.lib()
+    L.acc_cache_set_dir(str(tmp_path).encode())
+    L.acc_cache_clear(0)
+    before = A.cache_stats()
+    descs = [A.make_desc(A.SKEL_MAP, "float", env=[(1, "float")], out_rank=1, get="arrIn0_0[ix] * %d.0f" % (k % 3))
+             for k in range(12)]                        # 3 distinct kernels, each wanted by 4 threads
+    sizes, errors = [0] * len(descs), []
+
+    def work(k):
+        try:
+            sizes[k] = A.compile_only(descs[k], "gfx950")
+        except Exception as e:                          # noqa: BLE001
+            errors.append(e)
+    threads = [threading.Thread(target=work, args=(k,)) for k in range(len(descs))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors and all(s > 4000 for s in sizes)
+    assert len(set(sizes[k] for k in range(0, 12, 3))) == 1       # the same kernel gives the same object
+    after = A.cache_stats()
+    assert after["disk_errors"] == before["disk_errors"]
+    files = [os.path.join(dp, f) for dp, _, fs in os.walk(str(tmp_path)) for f in fs]
+    assert len(files) == 6 and not any(".tmp." in f for f in files)     # 3 kernels x 2 variants, no leftovers
+    # every entry reads back: drop the RAM table and compile again without a single compiler run
+    L.acc_cache_clear(0)
+    mid = A.cache_stats()
+    for d in descs[:3]:
+        A.compile_only(d, "gfx950")
+    end = A.cache_stats()
+    assert end["compiles"] == mid["compiles"] and end["disk_hits"] == mid["disk_hits"] + 6
+    assert end["disk_errors"] == mid["disk_errors"]
+
+
 def test_compile_error_is_a_status_with_a_log(A):
     L = A.lib()
     L.acc_cache_set_dir(b"")
