@@ -137,12 +137,24 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
   extern __shared__ __attribute__((aligned(16))) unsigned char acc_lds_raw[];
   T *bins = (T *)acc_lds_raw;
 
-  auto get  = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
-  auto perm = [&](const Int64 ix) -> Int64 { return (Int64)(ACC_PERMUTATION(ix)); };
-  auto f    = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
-
+  /* Target indices are handled as unsigned numbers of the width the
+   * permutation produces (32 bits for Int32 keys): `ignore` (-1) and every
+   * other negative index then lie beyond any bound, and each range test
+   * lo <= t < hi is one subtraction and one comparison.  The update loop is
+   * bound by instruction issue as much as by memory -- some twenty vector
+   * instructions per element is all there is room for -- so this matters. */
+  typedef decltype(ACC_PERMUTATION((Int64)0)) acc_perm_result;
+  typedef typename acc_bits<(sizeof(acc_perm_result) <= 4 ? 4 : 8)>::type U;
   const Int64 n = shIn_0;
   const Int64 ntarget = (ACC_OUT_SIZE);
+  /* what a non-negative index of that width can name */
+  const Int64 reach = sizeof(U) == 4 ? acc_min<Int64>(ntarget, (Int64)1 << (acc_is_unsigned<acc_perm_result>::value ? 32 : 31)) : ntarget;
+  const U u_bins = (U)acc_min<Int64>(lds_bins, reach), u_beyond = (U)(reach - acc_min<Int64>(lds_bins, reach));
+
+  auto get  = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
+  auto perm = [&](const Int64 ix) -> U { return (U)(ACC_PERMUTATION(ix)); };
+  auto f    = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
+
   const T ident = acc_hint_identity<T>();
   T *row = dump ? dump + (Int64)blockIdx.x * lds_bins : (T *)0;
   T *far_row = far ? far + (Int64)acc_xcd_id() * ntarget : (T *)0;
@@ -151,20 +163,23 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
   __syncthreads();
   T *mine = bins + ((threadIdx.x >> 6) % lds_copies) * lds_bins;
 
-  auto update = [&](const Int64 j, const T &x) {
-    if (j < 0 || j >= ntarget) return;            /* `ignore`, or outside the result */
-    if (j < lds_bins) acc_hint_apply<ACC_SCOPE_BLOCK>(mine + j, x, f);
-    else if (far_row) acc_hint_apply<ACC_SCOPE_BLOCK>(far_row + j, x, f);
-    else              acc_hint_apply<ACC_SCOPE_DEVICE>(arrOut_0 + j, x, f);
+  /* two independent tests rather than a chain: each becomes a predicated
+   * instruction, not a branch */
+  auto update = [&](const U t, const T &x) {
+    if (t < u_bins) acc_hint_apply<ACC_SCOPE_BLOCK>(mine + t, x, f);
+    if ((U)(t - u_bins) < u_beyond) {
+      if (far_row) acc_hint_apply<ACC_SCOPE_BLOCK>(far_row + t, x, f);
+      else         acc_hint_apply<ACC_SCOPE_DEVICE>(arrOut_0 + t, x, f);
+    }
   };
 
   /* full tiles, software-pipelined: the next tile's indices and values are
    * requested before the current tile's updates are issued, so the atomics'
    * latency is spent under loads already in flight */
   const Int64 full_tiles = n / ACC_TILE;
-  Int64 j[ACC_UNROLL][ACC_VEC], jn[ACC_UNROLL][ACC_VEC];
+  U j[ACC_UNROLL][ACC_VEC], jn[ACC_UNROLL][ACC_VEC];
   T x[ACC_UNROLL][ACC_VEC], xn[ACC_UNROLL][ACC_VEC];
-  auto load = [&](const Int64 tile, Int64 (&jj)[ACC_UNROLL][ACC_VEC], T (&xx)[ACC_UNROLL][ACC_VEC]) {
+  auto load = [&](const Int64 tile, U (&jj)[ACC_UNROLL][ACC_VEC], T (&xx)[ACC_UNROLL][ACC_VEC]) {
     const Int64 base = tile * (Int64)ACC_TILE + (Int64)threadIdx.x * ACC_VEC;
 #pragma unroll
     for (int u = 0; u < ACC_UNROLL; ++u)

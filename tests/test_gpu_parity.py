@@ -499,3 +499,38 @@ def test_golden_fixtures_on_gpu(A, ctx):
     out = ctx.empty((), np.float32)
     dot.fold([ctx.array(np.array(d["x"], np.float32)), ctx.array(np.array(d["y"], np.float32))], len(d["x"]), out)
     assert abs(float(out.get()) - d["dot"]) <= 1e-4 * abs(d["dot"])
+
+
+def test_permute_index_types_and_stray_targets(A, ctx, orc):
+    """targets of every width and signedness a permutation can produce; negative
+    ones, `ignore` and those past the end of the result are dropped, in the LDS
+    window, in the part of the target beyond it, and without any window"""
+    n = 200000
+    for bins in (300, 100000):                                   # inside one LDS window / larger than it
+        base = rng.integers(-50, bins + 50, n)                   # ~ strays on both sides
+        base[::17] = -1
+        dfl = rng.integers(0, 5, bins, dtype=np.int32)
+        keep = (base >= 0) & (base < bins)
+        exp = dfl + np.bincount(base[keep], minlength=bins).astype(np.int32)
+        for tname, dt, frag in (("Int32", np.int32, "arrIn0_0[ix]"), ("Int64", np.int64, "arrIn0_0[ix]"),
+                                ("Int16 widened", np.int32, "(Int16)arrIn0_0[ix]"),
+                                ("Int64 computed", np.int32, "(Int64)arrIn0_0[ix] * 1")):
+            if tname.startswith("Int16") and bins > 30000:
+                continue
+            for hint in (A.COMBINE_ADD, A.COMBINE_GENERIC):
+                say("permute targets as", tname, "bins", bins, "hint", hint)
+                keys = base.astype(dt)
+                sk = ctx.skeleton(A.SKEL_PERMUTE, "Int32", env=[(1, "Int64" if dt == np.int64 else "Int32")], out_rank=1,
+                                  get="1", combine="x + y", permutation=frag, combine_hint=hint)
+                out = ctx.empty(bins, np.int32)
+                sk.permute([ctx.array(keys)], n, ctx.array(dfl), out)
+                assert np.array_equal(out.get(), exp), (tname, bins, hint)
+    say("unsigned 32-bit targets: values of 2^31 and more are simply past the end")
+    keys = rng.integers(0, 400, n).astype(np.uint32)
+    keys[::13] = np.uint32(0x80000005)
+    keys[::29] = np.uint32(0xFFFFFFFF)
+    sk = ctx.skeleton(A.SKEL_PERMUTE, "Int32", env=[(1, "Word32")], out_rank=1, get="1", combine="x + y",
+                      permutation="arrIn0_0[ix]", combine_hint=A.COMBINE_ADD)
+    out = ctx.empty(300, np.int32)
+    sk.permute([ctx.array(keys)], n, ctx.array(np.zeros(300, np.int32)), out)
+    assert np.array_equal(out.get(), np.bincount(keys[keys < 300], minlength=300).astype(np.int32))
