@@ -20,7 +20,7 @@ MAX_RANK, MAX_COMP = 8, 8
 
 (SKEL_MAP, SKEL_GENERATE, SKEL_TRANSFORM, SKEL_FOLD, SKEL_FOLD1, SKEL_FOLDSEG, SKEL_FOLD1SEG,
  SKEL_SCANL, SKEL_SCANL1, SKEL_SCANLP, SKEL_SCANR, SKEL_SCANR1, SKEL_SCANRP, SKEL_PERMUTE,
- SKEL_STENCIL) = range(15)
+ SKEL_STENCIL, SKEL_STENCIL2) = range(16)
 SCAN_KINDS = {"scanl": SKEL_SCANL, "scanl1": SKEL_SCANL1, "scanl'": SKEL_SCANLP,
               "scanr": SKEL_SCANR, "scanr1": SKEL_SCANR1, "scanr'": SKEL_SCANRP}
 COMBINE_GENERIC, COMBINE_ADD, COMBINE_MIN, COMBINE_MAX, COMBINE_AND, COMBINE_OR, COMBINE_XOR = range(7)
@@ -56,7 +56,9 @@ class acc_skel_desc(C.Structure):
                 ("combine", C.c_char_p), ("seed", C.c_char_p), ("permutation", C.c_char_p),
                 ("combine_hint", C.c_int32), ("boundary", C.c_int32), ("boundary_constant", C.c_char_p),
                 ("n_taps", C.c_int32), ("tap_dy", C.POINTER(C.c_int32)), ("tap_dx", C.POINTER(C.c_int32)),
-                ("stencil_fn", C.c_char_p), ("stencil_in_type", C.c_char_p), ("seg_type", C.c_char_p)]
+                ("stencil_fn", C.c_char_p), ("stencil_in_type", C.c_char_p), ("seg_type", C.c_char_p),
+                ("boundary2", C.c_int32), ("boundary2_constant", C.c_char_p), ("n_taps2", C.c_int32),
+                ("tap2_dy", C.POINTER(C.c_int32)), ("tap2_dx", C.POINTER(C.c_int32)), ("stencil_in2_type", C.c_char_p)]
 
 
 class acc_device_props(C.Structure):
@@ -86,7 +88,7 @@ acc_event_elapsed_ms acc_compile acc_compile_log acc_cache_set_dir acc_cache_dir
 acc_cache_clear acc_module_load acc_module_unload acc_module_get_function acc_function_attr acc_occupancy
 acc_launch acc_launch_grid acc_skel_create acc_skel_destroy acc_skel_source acc_skel_preview acc_skel_compile_only
 acc_skel_get_info acc_exec_map acc_exec_fold acc_exec_foldseg acc_exec_scan acc_exec_permute
-acc_exec_stencil acc_exec_stencil_iterate""".split()
+acc_exec_stencil acc_exec_stencil2 acc_exec_stencil_iterate""".split()
 
 
 def build(force=False):
@@ -145,6 +147,7 @@ def lib():
         L.acc_exec_scan.argtypes = [C.c_void_p, AP, C.c_int64, AP, AP, C.c_void_p]
         L.acc_exec_permute.argtypes = [C.c_void_p, AP, C.c_int64, AP, AP, C.c_void_p]
         L.acc_exec_stencil.argtypes = [C.c_void_p, AP, AP, AP, C.c_void_p]
+        L.acc_exec_stencil2.argtypes = [C.c_void_p, AP, AP, AP, AP, C.c_void_p]
         L.acc_exec_stencil_iterate.argtypes = [C.c_void_p, AP, AP, AP, C.c_int32, C.c_void_p, C.POINTER(C.c_int32)]
         _lib = L
     return _lib
@@ -161,7 +164,8 @@ def _b(s):
 
 def make_desc(kind, elt, env=(), out_rank=0, get=None, combine=None, seed=None, permutation=None,
               combine_hint=COMBINE_GENERIC, flags=0, preamble=None, boundary="clamp", boundary_constant=None,
-              taps=None, stencil_fn=None, stencil_in=None, seg_type=None, elt_size=0):
+              taps=None, stencil_fn=None, stencil_in=None, seg_type=None, elt_size=0,
+              taps2=None, boundary2="clamp", boundary2_constant=None, stencil_in2=None):
     """env: sequence of (rank, [ctype, ...]) or (rank, ctype).  taps: [(dy, dx), ...] (1-D: [(0, dx)])."""
     keep = []
     sigs = (acc_env_sig * max(1, len(env)))()
@@ -186,6 +190,13 @@ def make_desc(kind, elt, env=(), out_rank=0, get=None, combine=None, seed=None, 
         keep += [dy, dx]
         d.n_taps, d.tap_dy, d.tap_dx = len(taps), dy, dx
     d.stencil_fn, d.stencil_in_type, d.seg_type = _b(stencil_fn), _b(stencil_in), _b(seg_type)
+    if taps2 is not None:       # stencil2: the second source
+        dy2 = (C.c_int32 * len(taps2))(*[t[0] for t in taps2])
+        dx2 = (C.c_int32 * len(taps2))(*[t[1] for t in taps2])
+        keep += [dy2, dx2]
+        d.n_taps2, d.tap2_dy, d.tap2_dx = len(taps2), dy2, dx2
+    d.boundary2 = BOUNDARY[boundary2] if isinstance(boundary2, str) else boundary2
+    d.boundary2_constant, d.stencil_in2_type = _b(boundary2_constant), _b(stencil_in2)
     d._keep = (sigs, keep)
     return d
 
@@ -401,6 +412,10 @@ class Skeleton(object):
 
     def stencil(self, env, src, out, stream=None):
         check(lib().acc_exec_stencil(self.handle, _env(env), C.byref(src.desc()), C.byref(out.desc()), stream))
+
+    def stencil2(self, env, src1, src2, out, stream=None):
+        check(lib().acc_exec_stencil2(self.handle, _env(env), C.byref(src1.desc()), C.byref(src2.desc()),
+                                      C.byref(out.desc()), stream))
 
     def stencil_iterate(self, env, a, b, iters, stream=None):
         r = C.c_int32(0)

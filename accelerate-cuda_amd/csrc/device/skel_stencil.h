@@ -33,10 +33,19 @@
  * Strips that are cut by the right edge, and arrays whose rows are not
  * 16-byte aligned, take a slower path that maps every element on its own.
  *
+ * With ACC_STENCIL_SOURCES == 2 the same kernel is stencil2
+ * (CodeGen/Stencil.hs:118-237): two source arrays, each with its own taps,
+ * element type, boundary condition and extents; the result covers the
+ * intersection of the two extents and its element is a function of both
+ * neighbourhoods (taps t0.. of the first source, u0.. of the second).
+ *
  * Generated definitions expected: ACC_ELT, ACC_IN_ELT, ACC_ENV_PARAMS,
  * ACC_ENV_ASSUME, ACC_OUT_PARAMS, ACC_STENCIL_RANK (1|2), ACC_RADIUS_Y,
- * ACC_RADIUS_X, ACC_BOUNDARY, ACC_BOUNDARY_CONSTANT, ACC_STENCIL_TAPS(READ),
- * ACC_STENCIL_FN, ACC_TILE_H, ACC_PREFETCH, ACC_BLOCK, ACC_ALIGNED.
+ * ACC_RADIUS_X (the larger of the two sources'), ACC_BOUNDARY,
+ * ACC_BOUNDARY_CONSTANT, ACC_STENCIL_TAPS(READ), ACC_STENCIL_FN, ACC_TILE_H,
+ * ACC_PREFETCH, ACC_BLOCK, ACC_ALIGNED, ACC_STENCIL_SOURCES (1|2) and for the
+ * second source ACC_IN2_ELT, ACC_BOUNDARY2, ACC_BOUNDARY2_CONSTANT,
+ * ACC_STENCIL_TAPS2(READ).
  */
 
 #define ACC_SVEC  4                                   /* results per lane and row */
@@ -56,34 +65,144 @@ static_assert(ACC_RADIUS_X <= ACC_SVEC, "stencil wider than one lane's neighbour
 #define ACC_B_WRAP 2
 #define ACC_B_CONSTANT 3
 
+template <int MODE>
 ACC_DEV Int64 acc_boundary_index(Int64 i, const Int64 sz)
 {
-#if ACC_BOUNDARY == ACC_B_CLAMP
-  i = acc_max<Int64>(0, acc_min<Int64>(i, sz - 1));
-#elif ACC_BOUNDARY == ACC_B_MIRROR
-  i = i < 0 ? -i : (i >= sz ? sz - (i - sz + 2) : i);
-#elif ACC_BOUNDARY == ACC_B_WRAP
-  i = i < 0 ? sz + i : (i >= sz ? i - sz : i);
-#endif
+  if (MODE == ACC_B_CLAMP)  i = acc_max<Int64>(0, acc_min<Int64>(i, sz - 1));
+  if (MODE == ACC_B_MIRROR) i = i < 0 ? -i : (i >= sz ? sz - (i - sz + 2) : i);
+  if (MODE == ACC_B_WRAP)   i = i < 0 ? sz + i : (i >= sz ? i - sz : i);
   /* the maps assume the array spans the stencil; keep the address legal if not */
   return acc_max<Int64>(0, acc_min<Int64>(i, sz - 1));
 }
 
-struct __attribute__((aligned(16))) acc_in_vec { ACC_IN_ELT v[ACC_SVEC]; };
 struct __attribute__((aligned(16))) acc_out_vec { ACC_ELT v[ACC_SVEC]; };
 
 /* value held by the next lane (the last lane keeps its own: caller masks it) */
 #define ACC_DPP_WAVE_SHL1 0x130
 template <typename T> ACC_DEV T acc_wave_shift_down1(const T &x) { return acc_dpp<ACC_DPP_WAVE_SHL1, 0xf>(x, x); }
 
-/* one source row as a lane sees it: [rx left | ACC_SVEC own | rx right] */
-struct acc_row { ACC_IN_ELT e[ACC_WW]; };
+/* One source array as a strip sees it: the register window of ACC_RING rows,
+ * each row [rx left | ACC_SVEC own | rx right] per lane, and what fills it.
+ * S element type, MODE boundary condition, FAST the aligned full-strip path. */
+template <typename S, int MODE, bool FAST>
+struct acc_strip_source {
+  struct row { S e[ACC_WW]; };
+  struct __attribute__((aligned(ACC_SVEC * sizeof(S)))) vec { S v[ACC_SVEC]; };
+
+  const S *base;            /* the array, its extents, the value outside it (constant boundary) */
+  Int64 h, w;
+  S outside;
+  Int64 y0, x0, gx;         /* the strip's origin, this lane's first column */
+  int lane, total;          /* total = source rows the strip touches */
+  row ring[ACC_RING];
+  S halo[ACC_HALO_LOADS];
+
+  /* FAST: the 2 rx elements just outside the strip, for every source row the
+   * strip will touch, are requested in one go -- lane q takes element
+   * q = (side * rx + j) * ACC_TOTAL_MAX + rho -- ahead of all row loads;
+   * finish() hands them to the strip's first and last lane.  One instruction
+   * for the strip instead of two per row. */
+  ACC_DEV void gather_halo()
+  {
+    if (!FAST) return;
+#pragma unroll
+    for (int g = 0; g < ACC_HALO_LOADS; ++g) {
+      const int q = lane + ACC_WAVE * g;
+      const int side = q / (ACC_RADIUS_X * ACC_TOTAL_MAX + (ACC_RADIUS_X == 0)), rem = q % (ACC_RADIUS_X * ACC_TOTAL_MAX + (ACC_RADIUS_X == 0));
+      const int j = rem / ACC_TOTAL_MAX, rho = rem % ACC_TOTAL_MAX;
+      halo[g] = S();
+      if (q < ACC_HALO_COUNT && rho < total) {
+        const Int64 gy = y0 - ACC_RADIUS_Y + rho;
+        const Int64 xx = side ? x0 + ACC_STRIP + j : x0 - ACC_RADIUS_X + j;
+        if (MODE == ACC_B_CONSTANT) {
+          const bool inside = gy >= 0 && gy < h && xx >= 0 && xx < w;
+          const Int64 my = acc_max<Int64>(0, acc_min<Int64>(gy, h - 1)), mx = acc_max<Int64>(0, acc_min<Int64>(xx, w - 1));
+          halo[g] = inside ? base[my * w + mx] : outside;
+        } else {
+          halo[g] = base[acc_boundary_index<MODE>(gy, h) * w + acc_boundary_index<MODE>(xx, w)];
+        }
+      }
+    }
+  }
+  ACC_DEV S halo_of(const int side, const int j, const int rho) const
+  {
+    const int q = (side * ACC_RADIUS_X + j) * ACC_TOTAL_MAX + rho;
+    S v = acc_readlane(halo[0], q % ACC_WAVE);
+#pragma unroll
+    for (int g = 1; g < ACC_HALO_LOADS; ++g)
+      if (q / ACC_WAVE == g) v = acc_readlane(halo[g], q % ACC_WAVE);
+    return v;
+  }
+
+  /* fetch source row (y0 - ry + rho) into ring[slot]; on the FAST path the left
+   * and right parts are only valid once finish() has run */
+  ACC_DEV void fetch(const int rho, const int slot)
+  {
+    row &r = ring[slot];
+    const Int64 gy = y0 - ACC_RADIUS_Y + rho;
+    const bool row_inside = MODE != ACC_B_CONSTANT || (gy >= 0 && gy < h);
+    const Int64 my = MODE == ACC_B_CONSTANT ? acc_max<Int64>(0, acc_min<Int64>(gy, h - 1)) : acc_boundary_index<MODE>(gy, h);
+    const S *src = base + my * w;
+    if (FAST) {
+      const vec own = *(const vec *)(src + gx);
+#pragma unroll
+      for (int k = 0; k < ACC_SVEC; ++k) r.e[ACC_RADIUS_X + k] = row_inside ? own.v[k] : outside;
+#pragma unroll
+      for (int j = 0; j < ACC_RADIUS_X; ++j) {           /* filled in by finish() */
+        r.e[j] = S();
+        r.e[ACC_RADIUS_X + ACC_SVEC + j] = S();
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < ACC_WW; ++e) {
+        const Int64 xx = gx - ACC_RADIUS_X + e;
+        r.e[e] = S();
+        if (gx < w) {                                    /* lanes past the edge produce nothing */
+          if (MODE == ACC_B_CONSTANT) {
+            const bool inside = row_inside && xx >= 0 && xx < w;
+            r.e[e] = inside ? src[acc_max<Int64>(0, acc_min<Int64>(xx, w - 1))] : outside;
+          } else {
+            r.e[e] = src[acc_boundary_index<MODE>(xx, w)];
+          }
+        }
+      }
+    }
+  }
+
+  /* FAST only: complete ring[slot], which holds source row rho, with the neighbours' elements */
+  ACC_DEV void finish(const int rho, const int slot)
+  {
+    if (!FAST) return;
+    row &r = ring[slot];
+#pragma unroll
+    for (int j = 0; j < ACC_RADIUS_X; ++j) {
+      const S from_left  = acc_wave_shift_up1(r.e[ACC_SVEC + j]);          /* neighbour's own[SVEC - rx + j] */
+      const S from_right = acc_wave_shift_down1(r.e[ACC_RADIUS_X + j]);    /* neighbour's own[j] */
+      r.e[j] = (lane != 0) ? from_left : halo_of(0, j, rho);
+      r.e[ACC_RADIUS_X + ACC_SVEC + j] = (lane != ACC_WAVE - 1) ? from_right : halo_of(1, j, rho);
+    }
+  }
+};
+
+#if ACC_STENCIL_SOURCES == 2
+#define ACC_STENCIL_ENTRY stencil2
+/* each source comes with its own extents (Stencil.hs:146-152) */
+#if ACC_STENCIL_RANK == 2
+#define ACC_SOURCE_PARAMS , const Int64 shStencil1_1, const Int64 shStencil1_0, const ACC_IN_ELT *__restrict__ arrStencil1_0 \
+                          , const Int64 shStencil2_1, const Int64 shStencil2_0, const ACC_IN2_ELT *__restrict__ arrStencil2_0
+#else
+#define ACC_SOURCE_PARAMS , const Int64 shStencil1_0, const ACC_IN_ELT *__restrict__ arrStencil1_0 \
+                          , const Int64 shStencil2_0, const ACC_IN2_ELT *__restrict__ arrStencil2_0
+#endif
+#else
+#define ACC_STENCIL_ENTRY stencil
+#define ACC_SOURCE_PARAMS , const ACC_IN_ELT *__restrict__ arrStencil_0
+#endif
 
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
-stencil(ACC_ENV_PARAMS ACC_OUT_PARAMS, const ACC_IN_ELT *__restrict__ arrStencil_0)
+ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS)
 {
   typedef ACC_ELT T;
-  typedef ACC_IN_ELT S;
   ACC_ENV_ASSUME
 #if ACC_STENCIL_RANK == 2
   const Int64 h = shOut_1, w = shOut_0;
@@ -124,109 +243,48 @@ stencil(ACC_ENV_PARAMS ACC_OUT_PARAMS, const ACC_IN_ELT *__restrict__ arrStencil
   auto run = [&](auto fast_c, auto full_c) {
   constexpr bool fast = decltype(fast_c)::value;
   const int rows = decltype(full_c)::value ? ACC_TILE_H : rows_here;
-
   const int total = rows + 2 * ACC_RADIUS_Y;              /* source rows this strip touches */
 
-  /* fast path: the 2 rx elements just outside the strip, for every source row
-   * the strip will touch, are requested in one go -- lane q takes element
-   * q = (side * rx + j) * ACC_TOTAL_MAX + rho -- ahead of all row loads; finish()
-   * hands them to the strip's first and last lane.  One instruction for the
-   * strip instead of two per row. */
-  S halo[ACC_HALO_LOADS];
-  if (fast) {
-#pragma unroll
-    for (int g = 0; g < ACC_HALO_LOADS; ++g) {
-      const int q = lane + ACC_WAVE * g;
-      const int side = q / (ACC_RADIUS_X * ACC_TOTAL_MAX), rem = q % (ACC_RADIUS_X * ACC_TOTAL_MAX);
-      const int j = rem / ACC_TOTAL_MAX, rho = rem % ACC_TOTAL_MAX;
-      halo[g] = S();
-      if (q < ACC_HALO_COUNT && rho < total) {
-        const Int64 gy = y0 - ACC_RADIUS_Y + rho;
-        const Int64 xx = side ? x0 + ACC_STRIP + j : x0 - ACC_RADIUS_X + j;
-#if ACC_BOUNDARY == ACC_B_CONSTANT
-        const bool inside = gy >= 0 && gy < h && xx >= 0 && xx < w;
-        const Int64 my = acc_max<Int64>(0, acc_min<Int64>(gy, h - 1)), mx = acc_max<Int64>(0, acc_min<Int64>(xx, w - 1));
-        halo[g] = inside ? arrStencil_0[my * w + mx] : (S)(ACC_BOUNDARY_CONSTANT);
+  acc_strip_source<ACC_IN_ELT, ACC_BOUNDARY, fast> a;
+#if ACC_STENCIL_SOURCES == 2
+  a.base = arrStencil1_0;
+  a.w = shStencil1_0;
+#if ACC_STENCIL_RANK == 2
+  a.h = shStencil1_1;
 #else
-        halo[g] = arrStencil_0[acc_boundary_index(gy, h) * w + acc_boundary_index(xx, w)];
+  a.h = 1;
 #endif
-      }
-    }
-  }
-  auto halo_of = [&](const int side, const int j, const int rho) -> S {
-    const int q = (side * ACC_RADIUS_X + j) * ACC_TOTAL_MAX + rho;
-    S v = acc_readlane(halo[0], q % ACC_WAVE);
-#pragma unroll
-    for (int g = 1; g < ACC_HALO_LOADS; ++g)
-      if (q / ACC_WAVE == g) v = acc_readlane(halo[g], q % ACC_WAVE);
-    return v;
-  };
+#else
+  a.base = arrStencil_0;
+  a.h = h;
+  a.w = w;
+#endif
+  a.outside = (ACC_IN_ELT)(ACC_BOUNDARY_CONSTANT);
+  a.y0 = y0; a.x0 = x0; a.gx = gx; a.lane = lane; a.total = total;
+#if ACC_STENCIL_SOURCES == 2
+  acc_strip_source<ACC_IN2_ELT, ACC_BOUNDARY2, fast> b;
+  b.base = arrStencil2_0;
+  b.w = shStencil2_0;
+#if ACC_STENCIL_RANK == 2
+  b.h = shStencil2_1;
+#else
+  b.h = 1;
+#endif
+  b.outside = (ACC_IN2_ELT)(ACC_BOUNDARY2_CONSTANT);
+  b.y0 = y0; b.x0 = x0; b.gx = gx; b.lane = lane; b.total = total;
+#define ACC_BOTH(call) do { a.call; b.call; } while (0)
+#else
+#define ACC_BOTH(call) a.call
+#endif
 
-  /* fetch source row (y0 - ry + rho) into a window; in the fast path the left
-   * and right parts are only valid once finish() has run */
-  auto fetch = [&](const int rho, acc_row &r) {
-    const Int64 gy = y0 - ACC_RADIUS_Y + rho;
-#if ACC_BOUNDARY == ACC_B_CONSTANT
-    const bool row_inside = gy >= 0 && gy < h;
-    const Int64 my = acc_max<Int64>(0, acc_min<Int64>(gy, h - 1));
-#else
-    const bool row_inside = true;
-    const Int64 my = acc_boundary_index(gy, h);
-#endif
-    const S *src = arrStencil_0 + my * w;
-    if (fast) {
-#if ACC_STENCIL_NT & 2
-      typedef S acc_in_native __attribute__((ext_vector_type(ACC_SVEC)));
-      const acc_in_native own = __builtin_nontemporal_load((const acc_in_native *)(src + gx));
-#pragma unroll
-      for (int k = 0; k < ACC_SVEC; ++k) r.e[ACC_RADIUS_X + k] = row_inside ? own[k] : (S)(ACC_BOUNDARY_CONSTANT);
-#else
-      const acc_in_vec own = *(const acc_in_vec *)(src + gx);
-#pragma unroll
-      for (int k = 0; k < ACC_SVEC; ++k) r.e[ACC_RADIUS_X + k] = row_inside ? own.v[k] : (S)(ACC_BOUNDARY_CONSTANT);
-#endif
-#pragma unroll
-      for (int j = 0; j < ACC_RADIUS_X; ++j) {           /* filled in by finish() */
-        r.e[j] = S();
-        r.e[ACC_RADIUS_X + ACC_SVEC + j] = S();
-      }
-    } else {
-#pragma unroll
-      for (int e = 0; e < ACC_WW; ++e) {
-        const Int64 xx = gx - ACC_RADIUS_X + e;
-        r.e[e] = S();
-        if (gx < w) {                                    /* lanes past the edge produce nothing */
-#if ACC_BOUNDARY == ACC_B_CONSTANT
-          const bool inside = row_inside && xx >= 0 && xx < w;
-          r.e[e] = inside ? src[xx] : (S)(ACC_BOUNDARY_CONSTANT);
-#else
-          r.e[e] = src[acc_boundary_index(xx, w)];
-#endif
-        }
-      }
-    }
-  };
-
-  /* fast path only: complete the window with the neighbours' elements */
-  auto finish = [&](const int rho, acc_row &r) {
-    if (!fast) return;
-#pragma unroll
-    for (int j = 0; j < ACC_RADIUS_X; ++j) {
-      const S from_left  = acc_wave_shift_up1(r.e[ACC_SVEC + j]);          /* neighbour's own[SVEC - rx + j] */
-      const S from_right = acc_wave_shift_down1(r.e[ACC_RADIUS_X + j]);    /* neighbour's own[j] */
-      r.e[j] = (lane != 0) ? from_left : halo_of(0, j, rho);
-      r.e[ACC_RADIUS_X + ACC_SVEC + j] = (lane != ACC_WAVE - 1) ? from_right : halo_of(1, j, rho);
-    }
-  };
-
-  acc_row ring[ACC_RING];
+  ACC_BOTH(gather_halo());
 
   /* prologue: the rows the first result needs, minus the newest, plus the prefetch */
 #pragma unroll
   for (int rho = 0; rho < ACC_RING - 1; ++rho)
-    if (rho < total) fetch(rho, ring[rho]);
+    if (rho < total) ACC_BOTH(fetch(rho, rho));
 #pragma unroll
-  for (int rho = 0; rho < ACC_NR - 1; ++rho) finish(rho, ring[rho]);
+  for (int rho = 0; rho < ACC_NR - 1; ++rho) ACC_BOTH(finish(rho, rho));
 
   for (int yb = 0; yb < rows; yb += ACC_RING) {
 #pragma unroll
@@ -236,15 +294,20 @@ stencil(ACC_ENV_PARAMS ACC_OUT_PARAMS, const ACC_IN_ELT *__restrict__ arrStencil
         /* newest row needed now is rho = y + 2 ry, in slot (s + NR - 1) % RING; the
          * slot freed by the previous step takes the row PREFETCH further on */
         const int rho_new = y + ACC_NR - 1 + ACC_PREFETCH;
-        if (rho_new < total) fetch(rho_new, ring[(s + ACC_RING - 1) % ACC_RING]);
-        finish(y + ACC_NR - 1, ring[(s + ACC_NR - 1) % ACC_RING]);
+        if (rho_new < total) ACC_BOTH(fetch(rho_new, (s + ACC_RING - 1) % ACC_RING));
+        ACC_BOTH(finish(y + ACC_NR - 1, (s + ACC_NR - 1) % ACC_RING));
 
         acc_out_vec res;
 #pragma unroll
         for (int k = 0; k < ACC_SVEC; ++k) {
-#define ACC_WINDOW_READ(dy, dx) ring[(s + ACC_RADIUS_Y + (dy)) % ACC_RING].e[ACC_RADIUS_X + k + (dx)]
+#define ACC_WINDOW_READ(dy, dx) a.ring[(s + ACC_RADIUS_Y + (dy)) % ACC_RING].e[ACC_RADIUS_X + k + (dx)]
           ACC_STENCIL_TAPS(ACC_WINDOW_READ)
 #undef ACC_WINDOW_READ
+#if ACC_STENCIL_SOURCES == 2
+#define ACC_WINDOW_READ(dy, dx) b.ring[(s + ACC_RADIUS_Y + (dy)) % ACC_RING].e[ACC_RADIUS_X + k + (dx)]
+          ACC_STENCIL_TAPS2(ACC_WINDOW_READ)
+#undef ACC_WINDOW_READ
+#endif
           res.v[k] = (T)(ACC_STENCIL_FN);
         }
         T *dst = arrOut_0 + (y0 + y) * w + gx;
@@ -266,6 +329,7 @@ stencil(ACC_ENV_PARAMS ACC_OUT_PARAMS, const ACC_IN_ELT *__restrict__ arrStencil
       }
     }
   }
+#undef ACC_BOTH
   };   /* run */
 
   if (fast_here) {

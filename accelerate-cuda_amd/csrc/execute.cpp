@@ -463,21 +463,31 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
   return rc;
 }
 
-static int stencil_once(acc_skel s, const acc_array *env, const acc_array *in, const acc_array *out, hipStream_t st)
+// `in2` is the second source of a stencil2, NULL for a stencil
+static int stencil_once(acc_skel s, const acc_array *env, const acc_array *in, const acc_array *in2, const acc_array *out, hipStream_t st)
 {
   const int rank = s->spec.out_rank;
   Args args;
   bool aligned = true;
   ACC_TRY(push_env(s, env, &args, &aligned));
   push_out(*out, &args, &aligned);
-  if (!aligned16(in->ptr[0])) aligned = false;
-  args.ptr(in->ptr[0]);
   const int64_t w = out->shape[rank - 1];
   const int64_t h = rank == 2 ? out->shape[0] : 1;
-  if (w == 0 || h == 0) return ACC_OK;
   // rows start on 16-byte boundaries only if the row pitch allows it
-  const size_t in_esz = acc::type_size(s->spec.stencil_in_type) ? acc::type_size(s->spec.stencil_in_type) : s->spec.elt_size;
-  if ((w * (int64_t)s->spec.elt_size) % 16 != 0 || (w * (int64_t)in_esz) % 16 != 0) aligned = false;
+  auto row_aligned = [&](const acc_array &a, const std::string &type) {
+    const size_t esz = acc::type_size(type) ? acc::type_size(type) : s->spec.elt_size;
+    return aligned16(a.ptr[0]) && (a.shape[rank - 1] * (int64_t)esz) % 16 == 0;
+  };
+  if ((w * (int64_t)s->spec.elt_size) % 16 != 0 || !row_aligned(*in, s->spec.stencil_in_type)) aligned = false;
+  if (in2) {      // each source with its extents (Stencil.hs:146-152)
+    if (!row_aligned(*in2, s->spec.stencil_in2_type)) aligned = false;
+    bool ignore = true;
+    push_out(*in, &args, &ignore);
+    push_out(*in2, &args, &ignore);
+  } else {
+    args.ptr(in->ptr[0]);
+  }
+  if (w == 0 || h == 0) return ACC_OK;
   // one wave per strip of 256 columns x tile_h rows
   // (for 2-D the waves of a workgroup are stacked vertically, so the row count is rounded up to whole groups)
   const int64_t waves = s->spec.block / 64;
@@ -502,7 +512,22 @@ static int stencil_check(acc_skel s, const acc_array *in, const acc_array *out)
 int acc_exec_stencil(acc_skel s, const acc_array *env, const acc_array *in, const acc_array *out, acc_stream stream)
 {
   ACC_TRY(stencil_check(s, in, out));
-  return stencil_once(s, env, in, out, static_cast<hipStream_t>(stream));
+  return stencil_once(s, env, in, nullptr, out, static_cast<hipStream_t>(stream));
+}
+
+int acc_exec_stencil2(acc_skel s, const acc_array *env, const acc_array *in1, const acc_array *in2, const acc_array *out, acc_stream stream)
+{
+  if (!s) return fail(ACC_ERR_INVALID, "acc_exec_stencil2: NULL skeleton");
+  if (!kind_is(s, {ACC_SKEL_STENCIL2})) return fail(ACC_ERR_INVALID, "acc_exec_stencil2: skeleton is '%s'", s->entry.c_str());
+  ACC_TRY(check_out(s, out, s->spec.out_rank, "result"));
+  ACC_TRY(check_out(s, in1, s->spec.out_rank, "first source", 1));
+  ACC_TRY(check_out(s, in2, s->spec.out_rank, "second source", 1));
+  for (int d = 0; d < out->rank; ++d)
+    if (out->shape[d] > std::min(in1->shape[d], in2->shape[d]))
+      return fail(ACC_ERR_INVALID, "stencil2: the result is larger than the intersection of the sources' extents");
+  if (array_size(*out) > 0 && (in1->ptr[0] == out->ptr[0] || in2->ptr[0] == out->ptr[0]))
+    return fail(ACC_ERR_INVALID, "stencil2: a source and the result must not alias");
+  return stencil_once(s, env, in1, in2, out, static_cast<hipStream_t>(stream));
 }
 
 int acc_exec_stencil_iterate(acc_skel s, const acc_array *env, const acc_array *a, const acc_array *b, int32_t iters, acc_stream stream, int32_t *result_in_b)
@@ -511,7 +536,7 @@ int acc_exec_stencil_iterate(acc_skel s, const acc_array *env, const acc_array *
   if (iters < 0) return fail(ACC_ERR_INVALID, "stencil: negative iteration count");
   const acc_array *src = a, *dst = b;
   for (int32_t i = 0; i < iters; ++i) {
-    ACC_TRY(stencil_once(s, env, src, dst, static_cast<hipStream_t>(stream)));
+    ACC_TRY(stencil_once(s, env, src, nullptr, dst, static_cast<hipStream_t>(stream)));
     std::swap(src, dst);
   }
   if (result_in_b) *result_in_b = (iters & 1);

@@ -113,7 +113,7 @@ static std::string out_size(int rank)
 static const char *kind_name(int kind)
 {
   static const char *names[] = {"map", "generate", "transform", "fold", "fold1", "foldSeg", "fold1Seg", "scanl",
-                                "scanl1", "scanl'", "scanr", "scanr1", "scanr'", "permute", "stencil"};
+                                "scanl1", "scanl'", "scanr", "scanr1", "scanr'", "permute", "stencil", "stencil2"};
   return (kind >= 0 && kind < ACC_SKEL_KIND_COUNT) ? names[kind] : "?";
 }
 
@@ -220,15 +220,22 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_UNROLL " << sp.unroll << "\n";
       tmpl = "skel_permute.h";
       break;
-    case ACC_SKEL_STENCIL: {
-      *entry = "stencil";
+    case ACC_SKEL_STENCIL:
+    case ACC_SKEL_STENCIL2: {
+      const bool two = sp.kind == ACC_SKEL_STENCIL2;
+      *entry = two ? "stencil2" : "stencil";
       int ry = 0, rx = 0;
       for (size_t k = 0; k < sp.tap_dy.size(); ++k) {
         ry = std::max(ry, std::abs(sp.tap_dy[k]));
         rx = std::max(rx, std::abs(sp.tap_dx[k]));
       }
+      for (size_t k = 0; k < sp.tap2_dy.size(); ++k) {
+        ry = std::max(ry, std::abs(sp.tap2_dy[k]));
+        rx = std::max(rx, std::abs(sp.tap2_dx[k]));
+      }
       o << "#define ACC_OUT_PARAMS " << out_params(sp.out_rank, sp.elt_type) << "\n";
       o << "#define ACC_STENCIL_RANK " << sp.out_rank << "\n";
+      o << "#define ACC_STENCIL_SOURCES " << (two ? 2 : 1) << "\n";
       o << "#define ACC_IN_ELT " << sp.stencil_in_type << "\n";
       o << "#define ACC_RADIUS_Y " << ry << "\n#define ACC_RADIUS_X " << rx << "\n";
       o << "#define ACC_BOUNDARY " << sp.boundary << "\n";
@@ -238,6 +245,15 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       for (size_t k = 0; k < sp.tap_dy.size(); ++k)
         o << "const ACC_IN_ELT t" << k << " = READ(" << sp.tap_dy[k] << ", " << sp.tap_dx[k] << "); ";
       o << "\n";
+      if (two) {
+        o << "#define ACC_IN2_ELT " << sp.stencil_in2_type << "\n";
+        o << "#define ACC_BOUNDARY2 " << sp.boundary2 << "\n";
+        o << "#define ACC_BOUNDARY2_CONSTANT " << (sp.boundary2_constant.empty() ? "0" : sp.boundary2_constant) << "\n";
+        o << "#define ACC_STENCIL_TAPS2(READ) ";
+        for (size_t k = 0; k < sp.tap2_dy.size(); ++k)
+          o << "const ACC_IN2_ELT u" << k << " = READ(" << sp.tap2_dy[k] << ", " << sp.tap2_dx[k] << "); ";
+        o << "\n";
+      }
       o << "#define ACC_STENCIL_FN " << sp.stencil_fn << "\n";
       o << "#define ACC_XCD_REMAP " << tune("stencil.xcd_remap", 0) << "\n";
       o << "#define ACC_STENCIL_NT " << tune("stencil.nt", 1) << "\n";
@@ -297,7 +313,7 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
     if ((int)sp->comp_types.size() > ACC_MAX_COMP) return fail(ACC_ERR_INVALID, "tuple element type: more than %d components", ACC_MAX_COMP);
     sp->elt_size = (size + align - 1) / align * align;
     sp->elt_type = "acc_elt";
-    if (d->kind == ACC_SKEL_PERMUTE || d->kind == ACC_SKEL_STENCIL)
+    if (d->kind == ACC_SKEL_PERMUTE || d->kind == ACC_SKEL_STENCIL || d->kind == ACC_SKEL_STENCIL2)
       return fail(ACC_ERR_UNSUPPORTED, "%s: tuple element types are not supported by this skeleton", kind_name(d->kind));
   } else {
     sp->elt_size = d->elt_size > 0 ? d->elt_size : type_size(sp->elt_type);
@@ -328,7 +344,7 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
   sp->combine_hint = d->combine_hint;
   sp->seg_type = (d->seg_type && *d->seg_type) ? d->seg_type : "Int32";
 
-  const bool needs_get = d->kind != ACC_SKEL_STENCIL;
+  const bool needs_get = d->kind != ACC_SKEL_STENCIL && d->kind != ACC_SKEL_STENCIL2;
   if (needs_get && sp->get.empty()) return fail(ACC_ERR_INVALID, "%s: `get` fragment missing", kind_name(d->kind));
   const bool needs_combine = d->kind >= ACC_SKEL_FOLD && d->kind <= ACC_SKEL_PERMUTE;
   if (needs_combine && sp->combine.empty()) return fail(ACC_ERR_INVALID, "%s: `combine` fragment missing", kind_name(d->kind));
@@ -374,21 +390,32 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
       sp->block = tune("permute.block", 1024);
       sp->unroll = tune("permute.unroll", 2);
       break;
-    case ACC_SKEL_STENCIL: {
+    case ACC_SKEL_STENCIL:
+    case ACC_SKEL_STENCIL2: {
       if (sp->out_rank != 1 && sp->out_rank != 2) return fail(ACC_ERR_UNSUPPORTED, "stencil: rank %d not supported (1 and 2 are)", sp->out_rank);
-      if (d->n_taps < 1 || d->n_taps > 81 || !d->tap_dx) return fail(ACC_ERR_INVALID, "stencil: bad tap list");
       if (!d->stencil_fn || !*d->stencil_fn) return fail(ACC_ERR_INVALID, "stencil: `stencil_fn` fragment missing");
-      if (d->boundary < ACC_BOUNDARY_CLAMP || d->boundary > ACC_BOUNDARY_CONSTANT) return fail(ACC_ERR_INVALID, "stencil: bad boundary %d", d->boundary);
-      for (int k = 0; k < d->n_taps; ++k) {
-        const int dy = (sp->out_rank == 2 && d->tap_dy) ? d->tap_dy[k] : 0;
-        if (std::abs(dy) > 4 || std::abs(d->tap_dx[k]) > 4) return fail(ACC_ERR_UNSUPPORTED, "stencil: tap offset beyond 4");
-        sp->tap_dy.push_back(dy);
-        sp->tap_dx.push_back(d->tap_dx[k]);
-      }
+      auto taps = [&](int n, const int32_t *dys, const int32_t *dxs, int boundary, std::vector<int> *oy, std::vector<int> *ox) -> int {
+        if (n < 1 || n > 81 || !dxs) return fail(ACC_ERR_INVALID, "stencil: bad tap list");
+        if (boundary < ACC_BOUNDARY_CLAMP || boundary > ACC_BOUNDARY_CONSTANT) return fail(ACC_ERR_INVALID, "stencil: bad boundary %d", boundary);
+        for (int k = 0; k < n; ++k) {
+          const int dy = (sp->out_rank == 2 && dys) ? dys[k] : 0;
+          if (std::abs(dy) > 4 || std::abs(dxs[k]) > 4) return fail(ACC_ERR_UNSUPPORTED, "stencil: tap offset beyond 4");
+          oy->push_back(dy);
+          ox->push_back(dxs[k]);
+        }
+        return ACC_OK;
+      };
+      ACC_TRY(taps(d->n_taps, d->tap_dy, d->tap_dx, d->boundary, &sp->tap_dy, &sp->tap_dx));
       sp->boundary = d->boundary;
       sp->boundary_constant = flat(d->boundary_constant);
       sp->stencil_fn = flat(d->stencil_fn);
       sp->stencil_in_type = (d->stencil_in_type && *d->stencil_in_type) ? d->stencil_in_type : sp->elt_type;
+      if (d->kind == ACC_SKEL_STENCIL2) {
+        ACC_TRY(taps(d->n_taps2, d->tap2_dy, d->tap2_dx, d->boundary2, &sp->tap2_dy, &sp->tap2_dx));
+        sp->boundary2 = d->boundary2;
+        sp->boundary2_constant = flat(d->boundary2_constant);
+        sp->stencil_in2_type = (d->stencil_in2_type && *d->stencil_in2_type) ? d->stencil_in2_type : sp->elt_type;
+      }
       sp->block = tune("stencil.block", 256);
       sp->tile_w = 256;                                  // one wave's strip: 64 lanes x 4 columns
       sp->tile_h = sp->out_rank == 2 ? tune("stencil.tile_h", 4) : 1;

@@ -28,6 +28,10 @@ struct SkelSpec {
   int boundary = 0;
   std::string boundary_constant, stencil_fn, stencil_in_type;
   std::vector<int> tap_dy, tap_dx;
+  // stencil2: the second source
+  int boundary2 = 0;
+  std::string boundary2_constant, stencil_in2_type;
+  std::vector<int> tap2_dy, tap2_dx;
   int tile_w = 256, tile_h = 4, prefetch = 3;
   // tuning
   int block = 256, unroll = 4, rows = 4, chunk = 4096;
@@ -71,6 +75,7 @@ struct acc_skel_s {
       case ACC_SKEL_SCANR: case ACC_SKEL_SCANR1: case ACC_SKEL_SCANRP:
         return spec.block * spec.rows * vec();
       case ACC_SKEL_STENCIL:
+      case ACC_SKEL_STENCIL2:
         return spec.tile_w * spec.tile_h * (spec.block / 64);
       case ACC_SKEL_FOLDSEG: case ACC_SKEL_FOLD1SEG:
         return spec.block;   // segments per block

@@ -225,7 +225,8 @@ enum {
   ACC_SKEL_SCANRP     = 12,  /* scanr' */
   ACC_SKEL_PERMUTE    = 13,  /* IndexSpace.hs:160-303 */
   ACC_SKEL_STENCIL    = 14,  /* Stencil.hs:55-114     */
-  ACC_SKEL_KIND_COUNT = 15
+  ACC_SKEL_STENCIL2   = 15,  /* Stencil.hs:118-237: two sources, result over the intersection of their extents */
+  ACC_SKEL_KIND_COUNT = 16
 };
 
 /* how `combine` may be applied atomically by permute */
@@ -282,6 +283,13 @@ typedef struct acc_skel_desc {
   const char        *stencil_fn;
   const char        *stencil_in_type; /* element type of the source array; NULL = elt_type */
   const char        *seg_type;      /* foldSeg: C type of the offsets (NULL = "Int32")       */
+  /* stencil2 only: the second source, with taps u0 .. u<n-1>; `stencil_fn` is over t0.. and u0.. */
+  int32_t            boundary2;
+  const char        *boundary2_constant;
+  int32_t            n_taps2;
+  const int32_t     *tap2_dy;
+  const int32_t     *tap2_dx;
+  const char        *stencil_in2_type; /* NULL = elt_type */
 } acc_skel_desc;
 
 /* Generate + compile (through the cache) + load one skeleton instance and
@@ -349,6 +357,13 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
  * the manifest source, out has the same shape (rank 1 or 2).                 */
 int acc_exec_stencil(acc_skel s, const acc_array *env, const acc_array *in, const acc_array *out,
                      acc_stream stream);
+
+/* stencil2: stencil2Op, Execute.hs:427-450.  Two manifest sources of the same
+ * rank; out must be no larger than the intersection of their extents (that is
+ * the result's shape, Stencil.hs:118-119).  Each source keeps its own boundary
+ * condition, applied at its own edges.                                        */
+int acc_exec_stencil2(acc_skel s, const acc_array *env, const acc_array *in1, const acc_array *in2,
+                      const acc_array *out, acc_stream stream);
 
 /* `iters` applications of the same stencil, ping-ponging between a and b on
  * the device with no host round trip (what `awhile` with a counter, or a

@@ -153,3 +153,38 @@ def rotate_l(x, i, bits):
     u = x & ((1 << bits) - 1)
     k = i % bits
     return ((u << k) | (u >> (bits - k))) & ((1 << bits) - 1) if k else u
+
+
+# ---- stencil taps as whole arrays (numpy index maps; the boundary rules of Stencil/Extra.hs:191-226) ----
+
+def bmap_np(mode, i, sz):
+    import numpy as np
+    if mode == "clamp":
+        return np.clip(i, 0, sz - 1)
+    if mode == "mirror":
+        return np.where(i < 0, -i, np.where(i >= sz, sz - (i - sz + 2), i))
+    if mode == "wrap":
+        return np.where(i < 0, sz + i, np.where(i >= sz, i - sz, i))
+    raise ValueError(mode)
+
+
+def tap_arrays(img, offsets, mode, constant, out_shape):
+    """for each (dy, dx): the array, of the result's shape, of the source elements at that offset
+    from every result position; the boundary applies at the SOURCE's own edges"""
+    import numpy as np
+    img = np.asarray(img)
+    if img.ndim == 1:
+        img = img[None, :]
+        out_shape = (1, out_shape[-1])
+    h, w = img.shape
+    ys, xs = np.arange(out_shape[0])[:, None], np.arange(out_shape[1])[None, :]
+    taps = []
+    for dy, dx in offsets:
+        yy, xx = ys + dy, xs + dx
+        if mode == "constant":
+            inside = (yy >= 0) & (yy < h) & (xx >= 0) & (xx < w)
+            v = np.where(inside, img[np.clip(yy, 0, h - 1), np.clip(xx, 0, w - 1)], np.asarray(constant, img.dtype))
+        else:
+            v = img[bmap_np(mode, yy, h), bmap_np(mode, xx, w)]
+        taps.append(v)
+    return taps
