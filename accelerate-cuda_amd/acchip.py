@@ -58,7 +58,8 @@ class acc_skel_desc(C.Structure):
                 ("n_taps", C.c_int32), ("tap_dy", C.POINTER(C.c_int32)), ("tap_dx", C.POINTER(C.c_int32)),
                 ("stencil_fn", C.c_char_p), ("stencil_in_type", C.c_char_p), ("seg_type", C.c_char_p),
                 ("boundary2", C.c_int32), ("boundary2_constant", C.c_char_p), ("n_taps2", C.c_int32),
-                ("tap2_dy", C.POINTER(C.c_int32)), ("tap2_dx", C.POINTER(C.c_int32)), ("stencil_in2_type", C.c_char_p)]
+                ("tap2_dy", C.POINTER(C.c_int32)), ("tap2_dx", C.POINTER(C.c_int32)), ("stencil_in2_type", C.c_char_p),
+                ("tap_dz", C.POINTER(C.c_int32)), ("tap2_dz", C.POINTER(C.c_int32))]
 
 
 class acc_device_props(C.Structure):
@@ -166,7 +167,8 @@ def make_desc(kind, elt, env=(), out_rank=0, get=None, combine=None, seed=None, 
               combine_hint=COMBINE_GENERIC, flags=0, preamble=None, boundary="clamp", boundary_constant=None,
               taps=None, stencil_fn=None, stencil_in=None, seg_type=None, elt_size=0,
               taps2=None, boundary2="clamp", boundary2_constant=None, stencil_in2=None):
-    """env: sequence of (rank, [ctype, ...]) or (rank, ctype).  taps: [(dy, dx), ...] (1-D: [(0, dx)])."""
+    """env: sequence of (rank, [ctype, ...]) or (rank, ctype).
+    taps: [(dy, dx), ...] (1-D: [(0, dx)]; 3-D: [(dz, dy, dx), ...])."""
     keep = []
     sigs = (acc_env_sig * max(1, len(env)))()
     for k, (rank, types) in enumerate(env):
@@ -185,16 +187,24 @@ def make_desc(kind, elt, env=(), out_rank=0, get=None, combine=None, seed=None, 
     d.boundary = BOUNDARY[boundary] if isinstance(boundary, str) else boundary
     d.boundary_constant = _b(boundary_constant)
     if taps is not None:
-        dy = (C.c_int32 * len(taps))(*[t[0] for t in taps])
-        dx = (C.c_int32 * len(taps))(*[t[1] for t in taps])
+        dy = (C.c_int32 * len(taps))(*[t[-2] for t in taps])
+        dx = (C.c_int32 * len(taps))(*[t[-1] for t in taps])
         keep += [dy, dx]
         d.n_taps, d.tap_dy, d.tap_dx = len(taps), dy, dx
+        if len(taps[0]) == 3:
+            dz = (C.c_int32 * len(taps))(*[t[0] for t in taps])
+            keep.append(dz)
+            d.tap_dz = dz
     d.stencil_fn, d.stencil_in_type, d.seg_type = _b(stencil_fn), _b(stencil_in), _b(seg_type)
     if taps2 is not None:       # stencil2: the second source
-        dy2 = (C.c_int32 * len(taps2))(*[t[0] for t in taps2])
-        dx2 = (C.c_int32 * len(taps2))(*[t[1] for t in taps2])
+        dy2 = (C.c_int32 * len(taps2))(*[t[-2] for t in taps2])
+        dx2 = (C.c_int32 * len(taps2))(*[t[-1] for t in taps2])
         keep += [dy2, dx2]
         d.n_taps2, d.tap2_dy, d.tap2_dx = len(taps2), dy2, dx2
+        if len(taps2[0]) == 3:
+            dz2 = (C.c_int32 * len(taps2))(*[t[0] for t in taps2])
+            keep.append(dz2)
+            d.tap2_dz = dz2
     d.boundary2 = BOUNDARY[boundary2] if isinstance(boundary2, str) else boundary2
     d.boundary2_constant, d.stencil_in2_type = _b(boundary2_constant), _b(stencil_in2)
     d._keep = (sigs, keep)

@@ -1,6 +1,6 @@
 /*
- * skel_stencil.h -- 1-D and 2-D stencils: every element of the result is a
- * function of the elements of the source at fixed offsets from it.
+ * skel_stencil.h -- 1-D, 2-D and 3-D stencils: every element of the result
+ * is a function of the elements of the source at fixed offsets from it.
  *
  * Takes the place of CodeGen/Stencil.hs:55-114 and the access generator of
  * CodeGen/Stencil/Extra.hs:53-128.  The reference reads every tap straight
@@ -33,6 +33,10 @@
  * Strips that are cut by the right edge, and arrays whose rows are not
  * 16-byte aligned, take a slower path that maps every element on its own.
  *
+ * A 3-D stencil walks its strips plane by plane: a strip lies in one plane z
+ * and keeps a register window per plane offset it reads (2 rz + 1 of them),
+ * all advancing down the rows together.
+ *
  * With ACC_STENCIL_SOURCES == 2 the same kernel is stencil2
  * (CodeGen/Stencil.hs:118-237): two source arrays, each with its own taps,
  * element type, boundary condition and extents; the result covers the
@@ -40,7 +44,7 @@
  * neighbourhoods (taps t0.. of the first source, u0.. of the second).
  *
  * Generated definitions expected: ACC_ELT, ACC_IN_ELT, ACC_ENV_PARAMS,
- * ACC_ENV_ASSUME, ACC_OUT_PARAMS, ACC_STENCIL_RANK (1|2), ACC_RADIUS_Y,
+ * ACC_ENV_ASSUME, ACC_OUT_PARAMS, ACC_STENCIL_RANK (1|2|3), ACC_RADIUS_Z, ACC_RADIUS_Y,
  * ACC_RADIUS_X (the larger of the two sources'), ACC_BOUNDARY,
  * ACC_BOUNDARY_CONSTANT, ACC_STENCIL_TAPS(READ), ACC_STENCIL_FN, ACC_TILE_H,
  * ACC_PREFETCH, ACC_BLOCK, ACC_ALIGNED, ACC_STENCIL_SOURCES (1|2) and for the
@@ -54,8 +58,12 @@
 #define ACC_RING  (ACC_NR + ACC_PREFETCH)             /* rows held in registers */
 #define ACC_WW    (ACC_SVEC + 2 * ACC_RADIUS_X)       /* row window of one lane */
 #define ACC_WAVES (ACC_BLOCK / ACC_WAVE)
-#define ACC_TOTAL_MAX  (ACC_TILE_H + 2 * ACC_RADIUS_Y)        /* source rows a strip touches */
-#define ACC_HALO_COUNT (2 * ACC_RADIUS_X * ACC_TOTAL_MAX)     /* elements just outside the strip */
+#ifndef ACC_RADIUS_Z
+#define ACC_RADIUS_Z 0
+#endif
+#define ACC_NZ    (2 * ACC_RADIUS_Z + 1)              /* planes a result depends on */
+#define ACC_TOTAL_MAX  (ACC_TILE_H + 2 * ACC_RADIUS_Y)        /* source rows a strip touches, per plane */
+#define ACC_HALO_COUNT (2 * ACC_RADIUS_X * ACC_TOTAL_MAX * ACC_NZ)   /* elements just outside the strip */
 #define ACC_HALO_LOADS (ACC_HALO_COUNT > 0 ? (ACC_HALO_COUNT + ACC_WAVE - 1) / ACC_WAVE : 1)
 
 static_assert(ACC_RADIUS_X <= ACC_SVEC, "stencil wider than one lane's neighbours can supply");
@@ -90,11 +98,11 @@ struct acc_strip_source {
   struct __attribute__((aligned(ACC_SVEC * sizeof(S)))) vec { S v[ACC_SVEC]; };
 
   const S *base;            /* the array, its extents, the value outside it (constant boundary) */
-  Int64 h, w;
+  Int64 d, h, w;
   S outside;
-  Int64 y0, x0, gx;         /* the strip's origin, this lane's first column */
-  int lane, total;          /* total = source rows the strip touches */
-  row ring[ACC_RING];
+  Int64 z0, y0, x0, gx;     /* the strip's plane and origin, this lane's first column */
+  int lane, total;          /* total = source rows the strip touches in each plane */
+  row ring[ACC_NZ][ACC_RING];
   S halo[ACC_HALO_LOADS];
 
   /* FAST: the 2 rx elements just outside the strip, for every source row the
@@ -108,25 +116,29 @@ struct acc_strip_source {
 #pragma unroll
     for (int g = 0; g < ACC_HALO_LOADS; ++g) {
       const int q = lane + ACC_WAVE * g;
-      const int side = q / (ACC_RADIUS_X * ACC_TOTAL_MAX + (ACC_RADIUS_X == 0)), rem = q % (ACC_RADIUS_X * ACC_TOTAL_MAX + (ACC_RADIUS_X == 0));
+      const int per_plane = 2 * ACC_RADIUS_X * ACC_TOTAL_MAX + (ACC_RADIUS_X == 0);
+      const int p = q / per_plane, qq = q % per_plane;
+      const int side = qq / (ACC_RADIUS_X * ACC_TOTAL_MAX + (ACC_RADIUS_X == 0)), rem = qq % (ACC_RADIUS_X * ACC_TOTAL_MAX + (ACC_RADIUS_X == 0));
       const int j = rem / ACC_TOTAL_MAX, rho = rem % ACC_TOTAL_MAX;
       halo[g] = S();
       if (q < ACC_HALO_COUNT && rho < total) {
+        const Int64 gz = z0 - ACC_RADIUS_Z + p;
         const Int64 gy = y0 - ACC_RADIUS_Y + rho;
         const Int64 xx = side ? x0 + ACC_STRIP + j : x0 - ACC_RADIUS_X + j;
         if (MODE == ACC_B_CONSTANT) {
-          const bool inside = gy >= 0 && gy < h && xx >= 0 && xx < w;
+          const bool inside = gz >= 0 && gz < d && gy >= 0 && gy < h && xx >= 0 && xx < w;
+          const Int64 mz = acc_max<Int64>(0, acc_min<Int64>(gz, d - 1));
           const Int64 my = acc_max<Int64>(0, acc_min<Int64>(gy, h - 1)), mx = acc_max<Int64>(0, acc_min<Int64>(xx, w - 1));
-          halo[g] = inside ? base[my * w + mx] : outside;
+          halo[g] = inside ? base[(mz * h + my) * w + mx] : outside;
         } else {
-          halo[g] = base[acc_boundary_index<MODE>(gy, h) * w + acc_boundary_index<MODE>(xx, w)];
+          halo[g] = base[(acc_boundary_index<MODE>(gz, d) * h + acc_boundary_index<MODE>(gy, h)) * w + acc_boundary_index<MODE>(xx, w)];
         }
       }
     }
   }
-  ACC_DEV S halo_of(const int side, const int j, const int rho) const
+  ACC_DEV S halo_of(const int p, const int side, const int j, const int rho) const
   {
-    const int q = (side * ACC_RADIUS_X + j) * ACC_TOTAL_MAX + rho;
+    const int q = p * (2 * ACC_RADIUS_X * ACC_TOTAL_MAX) + (side * ACC_RADIUS_X + j) * ACC_TOTAL_MAX + rho;
     S v = acc_readlane(halo[0], q % ACC_WAVE);
 #pragma unroll
     for (int g = 1; g < ACC_HALO_LOADS; ++g)
@@ -134,15 +146,22 @@ struct acc_strip_source {
     return v;
   }
 
-  /* fetch source row (y0 - ry + rho) into ring[slot]; on the FAST path the left
-   * and right parts are only valid once finish() has run */
+  /* fetch source row (y0 - ry + rho) of every plane into ring[.][slot]; on the FAST
+   * path the left and right parts are only valid once finish() has run */
   ACC_DEV void fetch(const int rho, const int slot)
   {
-    row &r = ring[slot];
+#pragma unroll
+    for (int p = 0; p < ACC_NZ; ++p) fetch_plane(p, rho, slot);
+  }
+  ACC_DEV void fetch_plane(const int p, const int rho, const int slot)
+  {
+    row &r = ring[p][slot];
+    const Int64 gz = z0 - ACC_RADIUS_Z + p;
     const Int64 gy = y0 - ACC_RADIUS_Y + rho;
-    const bool row_inside = MODE != ACC_B_CONSTANT || (gy >= 0 && gy < h);
+    const bool row_inside = MODE != ACC_B_CONSTANT || (gy >= 0 && gy < h && gz >= 0 && gz < d);
     const Int64 my = MODE == ACC_B_CONSTANT ? acc_max<Int64>(0, acc_min<Int64>(gy, h - 1)) : acc_boundary_index<MODE>(gy, h);
-    const S *src = base + my * w;
+    const Int64 mz = MODE == ACC_B_CONSTANT ? acc_max<Int64>(0, acc_min<Int64>(gz, d - 1)) : acc_boundary_index<MODE>(gz, d);
+    const S *src = base + (mz * h + my) * w;
     if (FAST) {
       const vec own = *(const vec *)(src + gx);
 #pragma unroll
@@ -169,17 +188,20 @@ struct acc_strip_source {
     }
   }
 
-  /* FAST only: complete ring[slot], which holds source row rho, with the neighbours' elements */
+  /* FAST only: complete ring[.][slot], which holds source row rho, with the neighbours' elements */
   ACC_DEV void finish(const int rho, const int slot)
   {
     if (!FAST) return;
-    row &r = ring[slot];
 #pragma unroll
-    for (int j = 0; j < ACC_RADIUS_X; ++j) {
-      const S from_left  = acc_wave_shift_up1(r.e[ACC_SVEC + j]);          /* neighbour's own[SVEC - rx + j] */
-      const S from_right = acc_wave_shift_down1(r.e[ACC_RADIUS_X + j]);    /* neighbour's own[j] */
-      r.e[j] = (lane != 0) ? from_left : halo_of(0, j, rho);
-      r.e[ACC_RADIUS_X + ACC_SVEC + j] = (lane != ACC_WAVE - 1) ? from_right : halo_of(1, j, rho);
+    for (int p = 0; p < ACC_NZ; ++p) {
+      row &r = ring[p][slot];
+#pragma unroll
+      for (int j = 0; j < ACC_RADIUS_X; ++j) {
+        const S from_left  = acc_wave_shift_up1(r.e[ACC_SVEC + j]);          /* neighbour's own[SVEC - rx + j] */
+        const S from_right = acc_wave_shift_down1(r.e[ACC_RADIUS_X + j]);    /* neighbour's own[j] */
+        r.e[j] = (lane != 0) ? from_left : halo_of(p, 0, j, rho);
+        r.e[ACC_RADIUS_X + ACC_SVEC + j] = (lane != ACC_WAVE - 1) ? from_right : halo_of(p, 1, j, rho);
+      }
     }
   }
 };
@@ -187,7 +209,10 @@ struct acc_strip_source {
 #if ACC_STENCIL_SOURCES == 2
 #define ACC_STENCIL_ENTRY stencil2
 /* each source comes with its own extents (Stencil.hs:146-152) */
-#if ACC_STENCIL_RANK == 2
+#if ACC_STENCIL_RANK == 3
+#define ACC_SOURCE_PARAMS , const Int64 shStencil1_2, const Int64 shStencil1_1, const Int64 shStencil1_0, const ACC_IN_ELT *__restrict__ arrStencil1_0 \
+                          , const Int64 shStencil2_2, const Int64 shStencil2_1, const Int64 shStencil2_0, const ACC_IN2_ELT *__restrict__ arrStencil2_0
+#elif ACC_STENCIL_RANK == 2
 #define ACC_SOURCE_PARAMS , const Int64 shStencil1_1, const Int64 shStencil1_0, const ACC_IN_ELT *__restrict__ arrStencil1_0 \
                           , const Int64 shStencil2_1, const Int64 shStencil2_0, const ACC_IN2_ELT *__restrict__ arrStencil2_0
 #else
@@ -204,10 +229,12 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS)
 {
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
-#if ACC_STENCIL_RANK == 2
-  const Int64 h = shOut_1, w = shOut_0;
+#if ACC_STENCIL_RANK == 3
+  const Int64 d = shOut_2, h = shOut_1, w = shOut_0;
+#elif ACC_STENCIL_RANK == 2
+  const Int64 d = 1, h = shOut_1, w = shOut_0;
 #else
-  const Int64 h = 1, w = shOut_0;
+  const Int64 d = 1, h = 1, w = shOut_0;
 #endif
   const int lane = acc_lane();
   const Int64 strips_x = (w + ACC_STRIP - 1) / ACC_STRIP;
@@ -220,14 +247,22 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS)
 #else
   const Int64 strip = (Int64)blockIdx.x * ACC_WAVES + wave_in_block;
 #endif
+  /* strips are numbered row of strips after row of strips (band), plane after plane */
 #if ACC_STACK_WAVES
   /* the waves of a workgroup take vertically adjacent strips: the boundary
    * rows they share are then requested from the same compute unit, where the
    * second request merges with the first instead of going out to memory */
   const Int64 group = strip / ACC_WAVES, within = strip % ACC_WAVES;
-  const Int64 y0 = ((group / strips_x) * ACC_WAVES + within) * ACC_TILE_H, x0 = (group % strips_x) * ACC_STRIP;
+  const Int64 band = (group / strips_x) * ACC_WAVES + within, x0 = (group % strips_x) * ACC_STRIP;
 #else
-  const Int64 y0 = (strip / strips_x) * ACC_TILE_H, x0 = (strip % strips_x) * ACC_STRIP;
+  const Int64 band = strip / strips_x, x0 = (strip % strips_x) * ACC_STRIP;
+#endif
+#if ACC_STENCIL_RANK == 3
+  const Int64 bands = (h + ACC_TILE_H - 1) / ACC_TILE_H;
+  const Int64 z0 = band / bands, y0 = (band % bands) * ACC_TILE_H;
+  if (z0 >= d) return;
+#else
+  const Int64 z0 = 0, y0 = band * ACC_TILE_H;
 #endif
   if (y0 >= h) return;                                   /* whole wave leaves together */
   const Int64 gx = x0 + lane * ACC_SVEC;
@@ -249,29 +284,36 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS)
 #if ACC_STENCIL_SOURCES == 2
   a.base = arrStencil1_0;
   a.w = shStencil1_0;
-#if ACC_STENCIL_RANK == 2
-  a.h = shStencil1_1;
-#else
   a.h = 1;
+  a.d = 1;
+#if ACC_STENCIL_RANK >= 2
+  a.h = shStencil1_1;
+#endif
+#if ACC_STENCIL_RANK == 3
+  a.d = shStencil1_2;
 #endif
 #else
   a.base = arrStencil_0;
+  a.d = d;
   a.h = h;
   a.w = w;
 #endif
   a.outside = (ACC_IN_ELT)(ACC_BOUNDARY_CONSTANT);
-  a.y0 = y0; a.x0 = x0; a.gx = gx; a.lane = lane; a.total = total;
+  a.z0 = z0; a.y0 = y0; a.x0 = x0; a.gx = gx; a.lane = lane; a.total = total;
 #if ACC_STENCIL_SOURCES == 2
   acc_strip_source<ACC_IN2_ELT, ACC_BOUNDARY2, fast> b;
   b.base = arrStencil2_0;
   b.w = shStencil2_0;
-#if ACC_STENCIL_RANK == 2
-  b.h = shStencil2_1;
-#else
   b.h = 1;
+  b.d = 1;
+#if ACC_STENCIL_RANK >= 2
+  b.h = shStencil2_1;
+#endif
+#if ACC_STENCIL_RANK == 3
+  b.d = shStencil2_2;
 #endif
   b.outside = (ACC_IN2_ELT)(ACC_BOUNDARY2_CONSTANT);
-  b.y0 = y0; b.x0 = x0; b.gx = gx; b.lane = lane; b.total = total;
+  b.z0 = z0; b.y0 = y0; b.x0 = x0; b.gx = gx; b.lane = lane; b.total = total;
 #define ACC_BOTH(call) do { a.call; b.call; } while (0)
 #else
 #define ACC_BOTH(call) a.call
@@ -300,17 +342,17 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS)
         acc_out_vec res;
 #pragma unroll
         for (int k = 0; k < ACC_SVEC; ++k) {
-#define ACC_WINDOW_READ(dy, dx) a.ring[(s + ACC_RADIUS_Y + (dy)) % ACC_RING].e[ACC_RADIUS_X + k + (dx)]
+#define ACC_WINDOW_READ(dz, dy, dx) a.ring[ACC_RADIUS_Z + (dz)][(s + ACC_RADIUS_Y + (dy)) % ACC_RING].e[ACC_RADIUS_X + k + (dx)]
           ACC_STENCIL_TAPS(ACC_WINDOW_READ)
 #undef ACC_WINDOW_READ
 #if ACC_STENCIL_SOURCES == 2
-#define ACC_WINDOW_READ(dy, dx) b.ring[(s + ACC_RADIUS_Y + (dy)) % ACC_RING].e[ACC_RADIUS_X + k + (dx)]
+#define ACC_WINDOW_READ(dz, dy, dx) b.ring[ACC_RADIUS_Z + (dz)][(s + ACC_RADIUS_Y + (dy)) % ACC_RING].e[ACC_RADIUS_X + k + (dx)]
           ACC_STENCIL_TAPS2(ACC_WINDOW_READ)
 #undef ACC_WINDOW_READ
 #endif
           res.v[k] = (T)(ACC_STENCIL_FN);
         }
-        T *dst = arrOut_0 + (y0 + y) * w + gx;
+        T *dst = arrOut_0 + ((z0 * h) + (y0 + y)) * w + gx;
         if (fast) {
 #if ACC_STENCIL_NT & 1
           typedef T acc_out_native __attribute__((ext_vector_type(ACC_SVEC)));

@@ -472,7 +472,8 @@ static int stencil_once(acc_skel s, const acc_array *env, const acc_array *in, c
   ACC_TRY(push_env(s, env, &args, &aligned));
   push_out(*out, &args, &aligned);
   const int64_t w = out->shape[rank - 1];
-  const int64_t h = rank == 2 ? out->shape[0] : 1;
+  const int64_t h = rank >= 2 ? out->shape[rank - 2] : 1;
+  const int64_t planes = rank == 3 ? out->shape[0] : 1;
   // rows start on 16-byte boundaries only if the row pitch allows it
   auto row_aligned = [&](const acc_array &a, const std::string &type) {
     const size_t esz = acc::type_size(type) ? acc::type_size(type) : s->spec.elt_size;
@@ -487,14 +488,14 @@ static int stencil_once(acc_skel s, const acc_array *env, const acc_array *in, c
   } else {
     args.ptr(in->ptr[0]);
   }
-  if (w == 0 || h == 0) return ACC_OK;
+  if (w == 0 || h == 0 || planes == 0) return ACC_OK;
   // one wave per strip of 256 columns x tile_h rows
   // (for 2-D the waves of a workgroup are stacked vertically, so the row count is rounded up to whole groups)
   const int64_t waves = s->spec.block / 64;
   const int64_t strips_x = (w + s->spec.tile_w - 1) / s->spec.tile_w;
   int64_t bands = (h + s->spec.tile_h - 1) / s->spec.tile_h;
   if (rank == 2 && acc::tune("stencil.stack", 0)) bands = (bands + waves - 1) / waves * waves;
-  return launch(s, aligned ? 0 : 1, (strips_x * bands + waves - 1) / waves, 0, st, &args);
+  return launch(s, aligned ? 0 : 1, (strips_x * bands * planes + waves - 1) / waves, 0, st, &args);
 }
 
 static int stencil_check(acc_skel s, const acc_array *in, const acc_array *out)

@@ -224,12 +224,14 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
     case ACC_SKEL_STENCIL2: {
       const bool two = sp.kind == ACC_SKEL_STENCIL2;
       *entry = two ? "stencil2" : "stencil";
-      int ry = 0, rx = 0;
+      int rz = 0, ry = 0, rx = 0;
       for (size_t k = 0; k < sp.tap_dy.size(); ++k) {
+        rz = std::max(rz, std::abs(sp.tap_dz[k]));
         ry = std::max(ry, std::abs(sp.tap_dy[k]));
         rx = std::max(rx, std::abs(sp.tap_dx[k]));
       }
       for (size_t k = 0; k < sp.tap2_dy.size(); ++k) {
+        rz = std::max(rz, std::abs(sp.tap2_dz[k]));
         ry = std::max(ry, std::abs(sp.tap2_dy[k]));
         rx = std::max(rx, std::abs(sp.tap2_dx[k]));
       }
@@ -237,13 +239,13 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "#define ACC_STENCIL_RANK " << sp.out_rank << "\n";
       o << "#define ACC_STENCIL_SOURCES " << (two ? 2 : 1) << "\n";
       o << "#define ACC_IN_ELT " << sp.stencil_in_type << "\n";
-      o << "#define ACC_RADIUS_Y " << ry << "\n#define ACC_RADIUS_X " << rx << "\n";
+      o << "#define ACC_RADIUS_Z " << rz << "\n#define ACC_RADIUS_Y " << ry << "\n#define ACC_RADIUS_X " << rx << "\n";
       o << "#define ACC_BOUNDARY " << sp.boundary << "\n";
       o << "#define ACC_BOUNDARY_CONSTANT " << (sp.boundary_constant.empty() ? "0" : sp.boundary_constant) << "\n";
       // the stencil pattern: one binding per tap, read through whatever accessor the template passes
       o << "#define ACC_STENCIL_TAPS(READ) ";
       for (size_t k = 0; k < sp.tap_dy.size(); ++k)
-        o << "const ACC_IN_ELT t" << k << " = READ(" << sp.tap_dy[k] << ", " << sp.tap_dx[k] << "); ";
+        o << "const ACC_IN_ELT t" << k << " = READ(" << sp.tap_dz[k] << ", " << sp.tap_dy[k] << ", " << sp.tap_dx[k] << "); ";
       o << "\n";
       if (two) {
         o << "#define ACC_IN2_ELT " << sp.stencil_in2_type << "\n";
@@ -251,7 +253,7 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
         o << "#define ACC_BOUNDARY2_CONSTANT " << (sp.boundary2_constant.empty() ? "0" : sp.boundary2_constant) << "\n";
         o << "#define ACC_STENCIL_TAPS2(READ) ";
         for (size_t k = 0; k < sp.tap2_dy.size(); ++k)
-          o << "const ACC_IN2_ELT u" << k << " = READ(" << sp.tap2_dy[k] << ", " << sp.tap2_dx[k] << "); ";
+          o << "const ACC_IN2_ELT u" << k << " = READ(" << sp.tap2_dz[k] << ", " << sp.tap2_dy[k] << ", " << sp.tap2_dx[k] << "); ";
         o << "\n";
       }
       o << "#define ACC_STENCIL_FN " << sp.stencil_fn << "\n";
@@ -392,34 +394,39 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
       break;
     case ACC_SKEL_STENCIL:
     case ACC_SKEL_STENCIL2: {
-      if (sp->out_rank != 1 && sp->out_rank != 2) return fail(ACC_ERR_UNSUPPORTED, "stencil: rank %d not supported (1 and 2 are)", sp->out_rank);
+      if (sp->out_rank < 1 || sp->out_rank > 3) return fail(ACC_ERR_UNSUPPORTED, "stencil: rank %d not supported (1, 2 and 3 are)", sp->out_rank);
       if (!d->stencil_fn || !*d->stencil_fn) return fail(ACC_ERR_INVALID, "stencil: `stencil_fn` fragment missing");
-      auto taps = [&](int n, const int32_t *dys, const int32_t *dxs, int boundary, std::vector<int> *oy, std::vector<int> *ox) -> int {
-        if (n < 1 || n > 81 || !dxs) return fail(ACC_ERR_INVALID, "stencil: bad tap list");
+      auto taps = [&](int n, const int32_t *dzs, const int32_t *dys, const int32_t *dxs, int boundary, std::vector<int> *oz,
+                      std::vector<int> *oy, std::vector<int> *ox) -> int {
+        if (n < 1 || n > 125 || !dxs) return fail(ACC_ERR_INVALID, "stencil: bad tap list");
         if (boundary < ACC_BOUNDARY_CLAMP || boundary > ACC_BOUNDARY_CONSTANT) return fail(ACC_ERR_INVALID, "stencil: bad boundary %d", boundary);
         for (int k = 0; k < n; ++k) {
-          const int dy = (sp->out_rank == 2 && dys) ? dys[k] : 0;
-          if (std::abs(dy) > 4 || std::abs(dxs[k]) > 4) return fail(ACC_ERR_UNSUPPORTED, "stencil: tap offset beyond 4");
+          const int dy = (sp->out_rank >= 2 && dys) ? dys[k] : 0;
+          const int dz = (sp->out_rank == 3 && dzs) ? dzs[k] : 0;
+          if (std::abs(dy) > 4 || std::abs(dxs[k]) > 4 || std::abs(dz) > 2) return fail(ACC_ERR_UNSUPPORTED, "stencil: tap offset beyond 4 (2 across planes)");
+          oz->push_back(dz);
           oy->push_back(dy);
           ox->push_back(dxs[k]);
         }
         return ACC_OK;
       };
-      ACC_TRY(taps(d->n_taps, d->tap_dy, d->tap_dx, d->boundary, &sp->tap_dy, &sp->tap_dx));
+      ACC_TRY(taps(d->n_taps, d->tap_dz, d->tap_dy, d->tap_dx, d->boundary, &sp->tap_dz, &sp->tap_dy, &sp->tap_dx));
       sp->boundary = d->boundary;
       sp->boundary_constant = flat(d->boundary_constant);
       sp->stencil_fn = flat(d->stencil_fn);
       sp->stencil_in_type = (d->stencil_in_type && *d->stencil_in_type) ? d->stencil_in_type : sp->elt_type;
       if (d->kind == ACC_SKEL_STENCIL2) {
-        ACC_TRY(taps(d->n_taps2, d->tap2_dy, d->tap2_dx, d->boundary2, &sp->tap2_dy, &sp->tap2_dx));
+        ACC_TRY(taps(d->n_taps2, d->tap2_dz, d->tap2_dy, d->tap2_dx, d->boundary2, &sp->tap2_dz, &sp->tap2_dy, &sp->tap2_dx));
         sp->boundary2 = d->boundary2;
         sp->boundary2_constant = flat(d->boundary2_constant);
         sp->stencil_in2_type = (d->stencil_in2_type && *d->stencil_in2_type) ? d->stencil_in2_type : sp->elt_type;
       }
       sp->block = tune("stencil.block", 256);
       sp->tile_w = 256;                                  // one wave's strip: 64 lanes x 4 columns
-      sp->tile_h = sp->out_rank == 2 ? tune("stencil.tile_h", 4) : 1;
-      sp->prefetch = sp->out_rank == 2 ? tune("stencil.prefetch", 3) : 0;
+      // rows per strip: short in 2-D (a compact window of the image in flight), taller in 3-D where every row is
+      // read from 2 rz + 1 planes and the boundary rows of a strip cost that much more
+      sp->tile_h = sp->out_rank == 2 ? tune("stencil.tile_h", 4) : (sp->out_rank == 3 ? tune("stencil.tile_h3", 16) : 1);
+      sp->prefetch = sp->out_rank == 2 ? tune("stencil.prefetch", 3) : (sp->out_rank == 3 ? tune("stencil.prefetch3", 1) : 0);
       if (sp->tile_h < 1 || sp->prefetch < 0 || sp->prefetch > 8) return fail(ACC_ERR_INVALID, "stencil: bad tile shape");
       break;
     }

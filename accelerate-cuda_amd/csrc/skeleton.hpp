@@ -27,11 +27,11 @@ struct SkelSpec {
   // stencil
   int boundary = 0;
   std::string boundary_constant, stencil_fn, stencil_in_type;
-  std::vector<int> tap_dy, tap_dx;
+  std::vector<int> tap_dz, tap_dy, tap_dx;
   // stencil2: the second source
   int boundary2 = 0;
   std::string boundary2_constant, stencil_in2_type;
-  std::vector<int> tap2_dy, tap2_dx;
+  std::vector<int> tap2_dz, tap2_dy, tap2_dx;
   int tile_w = 256, tile_h = 4, prefetch = 3;
   // tuning
   int block = 256, unroll = 4, rows = 4, chunk = 4096;

@@ -273,7 +273,7 @@ typedef struct acc_skel_desc {
   const char        *permutation;   /* permute: linear target index of source `ix`, or
                                        ACC_IGNORE (-1) to drop the element                   */
   int32_t            combine_hint;  /* ACC_COMBINE_*: lets permute use hardware atomics      */
-  /* stencil: taps t0 .. t<n-1> at offsets (dy, dx) from the focus (1-D: dy = 0),
+  /* stencil: taps t0 .. t<n-1> at offsets (dy, dx) from the focus (1-D: dy = 0; 3-D: see tap_dz),
    * `stencil_fn` is an expression over t0.. giving the result element       */
   int32_t            boundary;      /* ACC_BOUNDARY_*                                       */
   const char        *boundary_constant;
@@ -290,6 +290,9 @@ typedef struct acc_skel_desc {
   const int32_t     *tap2_dy;
   const int32_t     *tap2_dx;
   const char        *stencil_in2_type; /* NULL = elt_type */
+  /* rank-3 stencils: the taps' offsets across planes (NULL = all in the focus' plane) */
+  const int32_t     *tap_dz;
+  const int32_t     *tap2_dz;
 } acc_skel_desc;
 
 /* Generate + compile (through the cache) + load one skeleton instance and
@@ -354,7 +357,7 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
                      const acc_array *out, acc_stream stream);
 
 /* stencil: stencilOp, Execute.hs:413-425 (launched once, not twice).  `in` is
- * the manifest source, out has the same shape (rank 1 or 2).                 */
+ * the manifest source, out has the same shape (rank 1, 2 or 3).              */
 int acc_exec_stencil(acc_skel s, const acc_array *env, const acc_array *in, const acc_array *out,
                      acc_stream stream);
 

@@ -188,3 +188,24 @@ def tap_arrays(img, offsets, mode, constant, out_shape):
             v = img[bmap_np(mode, yy, h), bmap_np(mode, xx, w)]
         taps.append(v)
     return taps
+
+
+def tap_arrays3(vol, offsets, mode, constant, out_shape):
+    """tap_arrays for a rank-3 source and offsets (dz, dy, dx)"""
+    import numpy as np
+    vol = np.asarray(vol)
+    d, h, w = vol.shape
+    zs = np.arange(out_shape[0])[:, None, None]
+    ys = np.arange(out_shape[1])[None, :, None]
+    xs = np.arange(out_shape[2])[None, None, :]
+    taps = []
+    for dz, dy, dx in offsets:
+        zz, yy, xx = zs + dz, ys + dy, xs + dx
+        if mode == "constant":
+            inside = (zz >= 0) & (zz < d) & (yy >= 0) & (yy < h) & (xx >= 0) & (xx < w)
+            v = np.where(inside, vol[np.clip(zz, 0, d - 1), np.clip(yy, 0, h - 1), np.clip(xx, 0, w - 1)],
+                         np.asarray(constant, vol.dtype))
+        else:
+            v = vol[bmap_np(mode, zz, d), bmap_np(mode, yy, h), bmap_np(mode, xx, w)]
+        taps.append(v)
+    return taps

@@ -1,0 +1,91 @@
+"""Rank-3 stencils (and a rank-3 stencil2) through the C ABI, against numpy
+index maps (tests/pyref.py, tap_arrays3).  Sources hold small integers, so every
+Float32 operation is exact and results are compared bit for bit whatever order
+the sums are taken in; one case with fractional data states its tolerance."""
+import sys
+
+import numpy as np
+import pytest
+
+import pyref
+
+pytestmark = pytest.mark.gpu
+
+F = np.float32
+SEVEN = [(0, 0, 0), (-1, 0, 0), (1, 0, 0), (0, -1, 0), (0, 1, 0), (0, 0, -1), (0, 0, 1)]
+BOX = [(dz, dy, dx) for dz in (-1, 0, 1) for dy in (-1, 0, 1) for dx in (-1, 0, 1)]
+SHAPES = [(1, 1, 1), (3, 3, 3), (5, 7, 9), (3, 33, 70), (4, 64, 256), (6, 37, 517), (2, 16, 1024), (17, 40, 260)]
+
+
+def say(*a):
+    print("[case]", *a)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def A():
+    import acchip
+    return acchip
+
+
+@pytest.fixture(scope="module")
+def ctx(A):
+    c = A.Context(0)
+    yield c
+    c.close()
+
+
+@pytest.mark.parametrize("mode", ["clamp", "mirror", "wrap", "constant"])
+def test_stencil_3d(A, ctx, mode):
+    rng = np.random.default_rng(31)
+    lap = ctx.skeleton(A.SKEL_STENCIL, "float", out_rank=3, taps=SEVEN, boundary=mode, boundary_constant="2.0f",
+                       stencil_fn="t1 + t2 + t3 + t4 + t5 + t6 - 6.0f * t0")
+    box = ctx.skeleton(A.SKEL_STENCIL, "float", out_rank=3, taps=BOX, boundary=mode, boundary_constant="2.0f",
+                       stencil_fn=" + ".join("(float)%d * t%d" % (k % 5 - 2, k) for k in range(27)))
+    for shape in SHAPES:
+        if mode == "mirror" and min(shape) < 2:
+            continue                                   # the index maps assume the array spans the stencil
+        say("stencil 3-D", mode, shape)
+        v = rng.integers(-9, 9, shape).astype(F)
+        dv, out = ctx.array(v), ctx.empty(shape, F)
+        lap.stencil([], dv, out)
+        t = pyref.tap_arrays3(v, SEVEN, mode, 2.0, shape)
+        assert np.array_equal(out.get(), t[1] + t[2] + t[3] + t[4] + t[5] + t[6] - F(6) * t[0])
+        box.stencil([], dv, out)
+        t = pyref.tap_arrays3(v, BOX, mode, 2.0, shape)
+        assert np.array_equal(out.get(), sum(F(k % 5 - 2) * t[k] for k in range(27)))
+    say("stencil 3-D fractional data", mode)
+    v = rng.random((9, 50, 300)).astype(F)
+    out = ctx.empty(v.shape, F)
+    lap.stencil([], ctx.array(v), out)
+    t = pyref.tap_arrays3(v, SEVEN, mode, 2.0, v.shape)
+    exp = ((((t[1] + t[2]) + t[3]) + t[4]) + t[5]) + t[6] - F(6) * t[0]
+    assert np.max(np.abs(out.get() - exp)) <= 1e-5                 # in fact the same operations in the same order:
+    assert np.array_equal(out.get(), exp)
+
+
+def test_stencil2_3d_and_iteration(A, ctx):
+    rng = np.random.default_rng(32)
+    say("stencil2 3-D, sources of different extents")
+    sk = ctx.skeleton(A.SKEL_STENCIL2, "float", out_rank=3, taps=[(-1, 0, 0), (1, 0, 0)], boundary="wrap",
+                      taps2=[(0, 0, -1), (0, 0, 1), (0, -1, 0)], boundary2="constant", boundary2_constant="1.0f",
+                      stencil_fn="(t1 - t0) * (u0 + u1 + u2)")
+    a = rng.integers(-5, 5, (6, 40, 300)).astype(F)
+    b = rng.integers(-5, 5, (5, 44, 260)).astype(F)
+    shape = (5, 40, 260)
+    out = ctx.empty(shape, F)
+    sk.stencil2([], ctx.array(a), ctx.array(b), out)
+    t = pyref.tap_arrays3(a, [(-1, 0, 0), (1, 0, 0)], "wrap", 0, shape)
+    u = pyref.tap_arrays3(b, [(0, 0, -1), (0, 0, 1), (0, -1, 0)], "constant", 1.0, shape)
+    assert np.array_equal(out.get(), (t[1] - t[0]) * (u[0] + u[1] + u[2]))
+    say("3-D stencil iterated on the device")
+    avg = ctx.skeleton(A.SKEL_STENCIL, "float", out_rank=3, taps=SEVEN, boundary="clamp",
+                       stencil_fn="(t0 + t0 + t1 + t2 + t3 + t4 + t5 + t6) * 0.125f")
+    v = (rng.integers(0, 4, (8, 32, 256)) * 8 ** 4).astype(F)      # multiples of 8^4: four halvings by 8 stay exact
+    a_, b_ = ctx.array(v), ctx.empty(v.shape, F)
+    res = avg.stencil_iterate([], a_, b_, 4).get()
+    exp = v
+    for _ in range(4):
+        t = pyref.tap_arrays3(exp, SEVEN, "clamp", 0, v.shape)
+        exp = (t[0] + t[0] + t[1] + t[2] + t[3] + t[4] + t[5] + t[6]) * F(0.125)
+    assert np.array_equal(res, exp)
