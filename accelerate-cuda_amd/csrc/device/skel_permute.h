@@ -40,6 +40,55 @@
 
 #define ACC_TILE (ACC_BLOCK * ACC_VEC * ACC_UNROLL)
 
+#if ACC_PERMUTE_LOCKED
+/* An element no atomic instruction covers -- a tuple, or a scalar of another
+ * size than 4 or 8 bytes -- is updated under a lock per target, which is how
+ * the reference updates everything (IndexSpace.hs:285-303): locks[j] is 0 when
+ * free.  Lanes of one wave may want the same target, and a lane that spins
+ * for a lock held by another lane of its own wave never gets it: the holder
+ * is masked off until the spinning lane leaves the loop.  So nobody spins: the
+ * wave goes round a loop whose condition is a vote of the whole wave, every
+ * lane that still has work tries its lock once per trip, and whoever gets it
+ * updates the element and frees the lock within that trip.  Taking the lock
+ * is an acquire and freeing it a release, both at device scope: the compiler
+ * puts the cache invalidation and write-back around them that make the
+ * element written under the lock the one the next holder reads, on whichever
+ * compute die it runs (acknowledged stores alone are not enough: they are
+ * acknowledged by the die's own L2).  `locks` must be all zero on entry and is
+ * all zero again on exit; the word before it records a lane that gave up.    */
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, int *__restrict__ locks)
+{
+  typedef ACC_ELT T;
+  ACC_ENV_ASSUME
+  auto get  = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
+  auto perm = [&](const Int64 ix) -> Int64 { return (Int64)(ACC_PERMUTATION(ix)); };
+  auto f    = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
+  const Int64 n = shIn_0;
+  const Int64 ntarget = (ACC_OUT_SIZE);
+  for (Int64 ix = (Int64)blockIdx.x * ACC_BLOCK + threadIdx.x; ix < n; ix += (Int64)gridDim.x * ACC_BLOCK) {
+    const Int64 j = perm(ix);
+    if (j < 0 || j >= ntarget) continue;            /* `ignore`, or outside the result */
+    const T x = get(ix);
+    bool done = false;
+    /* Bounded, so that the kernel ends whatever `locks` held on entry.  When every
+     * element wants the same target the last lane waits for all the others, each
+     * of which holds the lock for a few round trips to memory: hence the factor. */
+    Int64 trips = 0;
+    while (__ballot(!done) != 0 && trips < 64 * n + (1 << 20)) {
+      if (!done && __hip_atomic_exchange(locks + j, 1, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) == 0) {
+        const T cur = ACC_READ(arrOut, j);
+        ACC_SET(arrOut, j, f(x, cur));
+        __hip_atomic_store(locks + j, 0, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        done = true;
+      }
+      ++trips;
+    }
+    if (!done) locks[-1] = 1;                       /* never seen in a healthy run: a lock that did not open */
+  }
+}
+#else /* atomics */
+
 #define ACC_HINT_GENERIC 0
 #define ACC_HINT_ADD 1
 #define ACC_HINT_MIN 2
@@ -292,3 +341,4 @@ permute_merge(ACC_ENV_PARAMS ACC_OUT_PARAMS, const acc_merge_job a, const int bl
     if (x != y) acc_hint_apply<ACC_SCOPE_DEVICE>(dst, acc, f);
   }
 }
+#endif /* ACC_PERMUTE_LOCKED */

@@ -358,14 +358,37 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
   hipStream_t st = static_cast<hipStream_t>(stream);
   const size_t esz = s->spec.elt_size;
   ACC_TRY(s->ctx->make_current());
-  // the result starts as a copy of the defaults: Execute.hs:401-406 (no lock array here)
+  // the result starts as a copy of the defaults: Execute.hs:401-406
   const bool copy_defaults = ntarget > 0 && defaults->ptr[0] != out->ptr[0];
   auto plain_copy = [&]() -> int {
-    if (copy_defaults)
-      ACC_HIP_TRY(hipMemcpyAsync(reinterpret_cast<void *>(out->ptr[0]), reinterpret_cast<void *>(defaults->ptr[0]), (size_t)ntarget * esz, hipMemcpyDeviceToDevice, st));
+    if (!copy_defaults) return ACC_OK;
+    const int nc = s->ncomp();
+    for (int c = 0; c < nc; ++c) {
+      const size_t csz = nc == 1 ? esz : (size_t)acc::type_size(s->spec.comp_types[nc - 1 - c]);
+      ACC_HIP_TRY(hipMemcpyAsync(reinterpret_cast<void *>(out->ptr[c]), reinterpret_cast<void *>(defaults->ptr[c]), (size_t)ntarget * csz, hipMemcpyDeviceToDevice, st));
+    }
     return ACC_OK;
   };
   if (n_src == 0 || ntarget == 0) return plain_copy();
+
+  if (s->spec.permute_locked) {
+    // elements no atomic covers: a lock per target (the reference's lock array, Execute.hs:402-405)
+    ACC_TRY(plain_copy());
+    Args largs;
+    bool al = true;
+    ACC_TRY(push_env(s, env, &largs, &al));
+    push_out(*out, &largs, &al);
+    largs.i64(n_src);
+    ACC_TRY(s->ensure_variant(al ? 0 : 1));
+    int lblk = -1;
+    ACC_TRY(s->ctx->scratch_acquire((size_t)ntarget * 4 + 256, st, acc::SCRATCH_LOCKS, &lblk));
+    // the locks start 256 bytes in; the word just before them is the kernel's "a lock never opened" mark
+    largs.ptr(reinterpret_cast<uint64_t>(s->ctx->scratch[lblk].ptr) + 256);
+    const int64_t lgrid = acc_launch_grid(n_src, s->spec.block, s->ctx->props.multiProcessorCount, 8);
+    const int lrc = launch(s, al ? 0 : 1, lgrid, 0, st, &largs);
+    s->ctx->scratch_release(lblk, st);
+    return lrc;
+  }
 
   Args args;
   bool aligned = true;

@@ -132,12 +132,13 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
   //   ACC_SET(name, ix, v)  the same as an ordinary store (small results that are read again soon)
   {
     const int nc = sp.comp_types.empty() ? 1 : (int)sp.comp_types.size();
-    std::ostringstream arr, assume, put, set;
+    std::ostringstream arr, assume, put, set, read;
     for (int i = 0; i < nc; ++i) {
       const int c = nc - 1 - i;
       const std::string t = sp.comp_types.empty() ? std::string("ACC_ELT") : sp.comp_types[i];
       arr << (i ? ", " : "") << t << " *__restrict__ name##_" << c;
       assume << "name##_" << c << " = (" << t << " *)__builtin_assume_aligned(name##_" << c << ", 16); ";
+      read << (i ? ", " : "") << "name##_" << c << "[ix]";
       if (sp.comp_types.empty()) {
         put << "acc_store(name##_0 + (ix), (v))";
         set << "name##_0[ix] = (v)";
@@ -147,6 +148,9 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       }
     }
     o << "#define ACC_NCOMP " << nc << "\n";
+    //   ACC_READ(name, ix)    element ix, assembled from its components
+    if (sp.comp_types.empty()) o << "#define ACC_READ(name, ix) (" << read.str() << ")\n";
+    else o << "#define ACC_READ(name, ix) (ACC_ELT{" << read.str() << "})\n";
     o << "#define ACC_OUT_ARRAY(name) " << arr.str() << "\n";
     o << "#define ACC_OUT_ASSUME(name) " << (aligned ? assume.str() : std::string()) << "\n";
     if (sp.comp_types.empty()) {
@@ -216,6 +220,7 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "#define ACC_OUT_SIZE " << out_size(sp.out_rank) << "\n";
       o << "#define ACC_PERMUTATION(ix) " << sp.permutation << "\n";
       o << "#define ACC_COMBINE_HINT " << sp.combine_hint << "\n";
+      o << "#define ACC_PERMUTE_LOCKED " << (sp.permute_locked ? 1 : 0) << "\n";
       o << "#define ACC_ELT_IS_INTEGER " << (is_integer_type(sp.elt_type) ? 1 : 0) << "\n";
       o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_UNROLL " << sp.unroll << "\n";
       tmpl = "skel_permute.h";
@@ -315,7 +320,7 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
     if ((int)sp->comp_types.size() > ACC_MAX_COMP) return fail(ACC_ERR_INVALID, "tuple element type: more than %d components", ACC_MAX_COMP);
     sp->elt_size = (size + align - 1) / align * align;
     sp->elt_type = "acc_elt";
-    if (d->kind == ACC_SKEL_PERMUTE || d->kind == ACC_SKEL_STENCIL || d->kind == ACC_SKEL_STENCIL2)
+    if (d->kind == ACC_SKEL_STENCIL || d->kind == ACC_SKEL_STENCIL2)
       return fail(ACC_ERR_UNSUPPORTED, "%s: tuple element types are not supported by this skeleton", kind_name(d->kind));
   } else {
     sp->elt_size = d->elt_size > 0 ? d->elt_size : type_size(sp->elt_type);
@@ -383,10 +388,13 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
     case ACC_SKEL_PERMUTE:
       if (sp->permutation.empty()) return fail(ACC_ERR_INVALID, "permute: `permutation` fragment missing");
       if (sp->out_rank < 1) return fail(ACC_ERR_UNSUPPORTED, "permute into a rank-0 array is not supported");   // IndexSpace.hs:230
-      if (sp->elt_size != 4 && sp->elt_size != 8)
-        return fail(ACC_ERR_UNSUPPORTED, "permute: element size %d has no atomic update", sp->elt_size);
       if (sp->combine_hint < ACC_COMBINE_GENERIC || sp->combine_hint > ACC_COMBINE_XOR)
         return fail(ACC_ERR_INVALID, "permute: bad combine_hint %d", sp->combine_hint);
+      // no atomic read-modify-write covers a tuple or an element of another size than 4 or 8 bytes:
+      // those go through a lock per target, as every permute does in the reference (IndexSpace.hs:285-303)
+      sp->permute_locked = !sp->comp_types.empty() || (sp->elt_size != 4 && sp->elt_size != 8);
+      if (sp->permute_locked && sp->combine_hint != ACC_COMBINE_GENERIC)
+        return fail(ACC_ERR_INVALID, "permute: combine_hint needs a 4- or 8-byte single-component element");
       if (sp->combine_hint >= ACC_COMBINE_AND && !is_integer_type(sp->elt_type))
         return fail(ACC_ERR_INVALID, "permute: bitwise combine_hint on non-integer element type '%s'", sp->elt_type.c_str());
       sp->block = tune("permute.block", 1024);
@@ -480,7 +488,7 @@ int acc_skel_s::ensure_variant(int v)
     return acc::fail_hip(e, ("hipModuleGetFunction(" + entry + ")").c_str());
   }
   const bool two_kernels = ((spec.kind == ACC_SKEL_FOLD || spec.kind == ACC_SKEL_FOLD1) && spec.out_rank == 0) ||
-                           spec.kind == ACC_SKEL_PERMUTE;
+                           (spec.kind == ACC_SKEL_PERMUTE && !spec.permute_locked);
   const std::string second = entry + (spec.kind == ACC_SKEL_PERMUTE ? "_merge" : "_finish");
   if (two_kernels) {
     e = hipModuleGetFunction(&var.fn_finish, var.module, second.c_str());
@@ -490,7 +498,7 @@ int acc_skel_s::ensure_variant(int v)
       return acc::fail_hip(e, ("hipModuleGetFunction(" + second + ")").c_str());
     }
   }
-  if (spec.kind == ACC_SKEL_PERMUTE) {
+  if (spec.kind == ACC_SKEL_PERMUTE && !spec.permute_locked) {
     e = hipModuleGetFunction(&var.fn_fill, var.module, (entry + "_fill").c_str());
     if (e != hipSuccess) {
       (void)hipModuleUnload(var.module);

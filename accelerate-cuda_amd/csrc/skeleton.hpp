@@ -23,6 +23,7 @@ struct SkelSpec {
   std::string preamble, get, combine, seed, permutation;
   bool has_seed = false;
   int combine_hint = 0;
+  bool permute_locked = false;          // permute of an element no atomic covers (tuples, 1/2/16-byte types): per-target locks
   std::string seg_type;
   // stencil
   int boundary = 0;

@@ -148,6 +148,44 @@ def test_segmented_scan_with_flag_value_pairs(A, ctx, kind):
             assert int(tv) == int(inc[-1]) and int(tf) == int(incf[-1])
 
 
+def test_permute_of_tuples_and_narrow_elements_under_locks(A, ctx):
+    """elements no atomic instruction covers are combined under a lock per target (IndexSpace.hs:285-303)"""
+    rng = np.random.default_rng(9)
+    n, bins = 300000, 500
+    keys = rng.integers(-3, bins + 3, n).astype(np.int32)            # a few strays on both sides, dropped
+    keys[::19] = -1
+    w = rng.integers(-50, 50, n).astype(np.float32)                  # whole numbers: Float32 sums are exact in any order
+    ok = (keys >= 0) & (keys < bins)
+    say("permute (sum, count) pairs")
+    sk = ctx.skeleton(A.SKEL_PERMUTE, "float, Int32", env=[I32, F32], out_rank=1, get="acc_elt{arrIn1_0[ix], 1}",
+                      combine="acc_elt{x.a1 + y.a1, x.a0 + y.a0}", permutation="arrIn0_0[ix]")
+    d0 = rng.integers(-5, 5, bins).astype(np.float32)
+    d1 = rng.integers(0, 3, bins).astype(np.int32)
+    out = ctx.empty_tuple(bins, [np.float32, np.int32])
+    sk.permute([ctx.array(keys), ctx.array(w)], n, ctx.tuple_array(d0, d1), out)
+    s_, c_ = out.get()
+    assert np.array_equal(c_, d1 + np.bincount(keys[ok], minlength=bins).astype(np.int32))
+    assert np.array_equal(s_, d0 + np.bincount(keys[ok], weights=w[ok].astype(np.float64), minlength=bins).astype(np.float32))
+    say("the same again: the locks were left open")
+    sk.permute([ctx.array(keys), ctx.array(w)], n, ctx.tuple_array(d0, d1), out)
+    assert np.array_equal(out.get()[1], c_)
+    say("permute into Int16 and Word8 targets, every key the same target among them")
+    h16 = ctx.skeleton(A.SKEL_PERMUTE, "Int16", env=[I32], out_rank=1, get="(Int16)1", combine="(Int16)(x + y)", permutation="arrIn0_0[ix]")
+    few = rng.integers(0, 40, 20000).astype(np.int32)
+    few[:3000] = 7
+    o16 = ctx.empty(40, np.int16)
+    h16.permute([ctx.array(few)], few.size, ctx.array(np.zeros(40, np.int16)), o16)
+    assert np.array_equal(o16.get(), np.bincount(few, minlength=40).astype(np.int16))
+    or8 = ctx.skeleton(A.SKEL_PERMUTE, "Word8", env=[I32, (1, "Word8")], out_rank=1, get="arrIn1_0[ix]", combine="(Word8)(x | y)",
+                       permutation="arrIn0_0[ix]")
+    bits = (1 << rng.integers(0, 8, few.size)).astype(np.uint8)
+    o8 = ctx.empty(40, np.uint8)
+    or8.permute([ctx.array(few), ctx.array(bits)], few.size, ctx.array(np.zeros(40, np.uint8)), o8)
+    exp = np.zeros(40, np.uint8)
+    np.bitwise_or.at(exp, few, bits)
+    assert np.array_equal(o8.get(), exp)
+
+
 def test_tuple_results_need_tuple_arrays_and_are_refused_elsewhere(A, ctx):
     say("misuse")
     zipk = ctx.skeleton(A.SKEL_MAP, "float, Int32", env=[F32], out_rank=1, get="acc_elt{arrIn0_0[ix], 0}")
@@ -156,8 +194,7 @@ def test_tuple_results_need_tuple_arrays_and_are_refused_elsewhere(A, ctx):
         zipk.map([x], ctx.empty(8, np.float32))                  # one component offered, two needed
     assert e.value.code == A.ERR_INVALID
     with pytest.raises(A.AccError) as e:
-        ctx.skeleton(A.SKEL_PERMUTE, "float, Int32", env=[I32], out_rank=1, get="acc_elt{1.0f, 1}", combine="x",
-                     permutation="arrIn0_0[ix]")
+        ctx.skeleton(A.SKEL_STENCIL, "float, Int32", out_rank=1, taps=[(0, 0)], stencil_fn="acc_elt{t0, 1}")
     assert e.value.code == A.ERR_UNSUPPORTED
     with pytest.raises(A.AccError) as e:
         ctx.skeleton(A.SKEL_MAP, "float, quux", env=[F32], out_rank=1, get="acc_elt{1.0f, 1}")
