@@ -1,0 +1,607 @@
+"""An embedded array language over libacchip, shaped like the surface a user of
+the reference programs against (Data.Array.Accelerate + Data.Array.Accelerate.CUDA:
+`use`, `map`, `zipWith`, `generate`, `backpermute`, `fold`, `foldSeg`, the scans,
+`permute`, `stencil`, `run`, `run1` -- CUDA.hs:184-200).
+
+    import accelerate_hip as acc
+    def dotp(xs, ys):
+        return acc.fold(lambda a, b: a + b, 0.0, acc.zipWith(lambda a, b: a * b, xs, ys))
+    print(acc.run(dotp(acc.use(x), acc.use(y))))
+
+What it does is what the reference's front end and code generator do for the
+skeleton hot path, in miniature:
+  * scalar functions are Python callables over `Exp` values; applying them builds
+    HIP C++ expression text (the role of CodeGen.hs:338-821), with the primitive
+    table of acc_prim.h behind the operators that are not plain C operators;
+  * `map`, `zipWith`, `generate`, `backpermute` are DELAYED: they are index -> value
+    functions that fuse into whatever consumes them, so `fold (+) 0 (zipWith (*) xs ys)`
+    is one kernel reading two arrays (what the fusion of `convertAccWith` hands the
+    reference's back end as `CUDelayed`, CodeGen/Base.hs:115-138);
+  * consumers (`fold`, `foldSeg`, scans, `permute`, `stencil`, and forcing a delayed
+    array) each become one skeleton instance, created once per distinct generated
+    text and cached; free arrays are numbered in order of first use (the Gamma
+    environment, AST.hs:87-112) and named arrIn<k>_0 in the text.
+Everything runs on the GPU through the C ABI; there is no other execution path.
+"""
+import numbers
+import re
+import weakref
+
+import numpy as np
+
+import acchip as A
+
+__all__ = ["Exp", "constant", "cond", "use", "unit", "map", "zipWith", "generate", "backpermute", "transpose", "reverse", "zip_", "unzip",
+           "fold", "fold1", "foldSeg", "scanl", "scanl1", "scanl_", "scanr", "scanr1", "scanr_", "permute", "ignore",
+           "stencil", "stencil2", "run", "run1", "fst", "snd", "lift", "index_if", "fromIntegral", "truncate", "round_", "floor",
+           "ceiling", "idiv", "mod", "quot", "rem", "min_", "max_", "sqrt", "exp", "log", "sin", "cos", "tan", "abs_",
+           "signum", "Context", "the"]
+
+CTYPE = dict(A.CTYPE_OF)
+NPTYPE = {v: k for k, v in CTYPE.items()}
+FLOATS = ("float", "double")
+RANK = {"Int8": 1, "Word8": 1, "Int16": 2, "Word16": 2, "Int32": 3, "Word32": 3, "Int64": 4, "Word64": 4, "float": 5, "double": 6}
+
+
+# ------------------------------------------------------------------------------ scalar expressions
+
+class Exp(object):
+    """A typed scalar expression: a C type name and text, or, for a tuple, the component expressions
+    (tuples exist only on the host side of the generated text: `fst`/`snd` pick a component, and the
+    braces of the element struct are written where a tuple becomes a skeleton's result)."""
+
+    def __init__(self, ctype, text=None, comps=None):
+        self.ctype, self.comps = ctype, comps
+        if comps is not None:
+            text = "acc_elt{%s}" % ", ".join(c.text for c in comps)
+        self.text = text
+
+    # -- helpers
+    @staticmethod
+    def of(v, like=None):
+        if isinstance(v, Exp):
+            return v
+        if isinstance(v, (tuple, list)):
+            if isinstance(like, tuple):
+                return lift(*[Exp.of(e, t) for e, t in zip(v, like)])
+            return lift(*v)
+        t = like if like is not None else ("double" if isinstance(v, float) else "Int64")
+        return constant(v, t)
+
+    def _bin(self, other, op, result=None):
+        o = Exp.of(other, self.ctype)
+        if o.ctype != self.ctype:
+            raise TypeError("operands of %s differ in type: %s and %s (convert with fromIntegral)" % (op, self.ctype, o.ctype))
+        return Exp(result or self.ctype, "((%s)(%s %s %s))" % (result or self.ctype, self.text, op, o.text))
+
+    def _rbin(self, other, op):
+        return Exp.of(other, self.ctype)._bin(self, op)
+
+    def _call(self, fn, *others):
+        args = [self] + [Exp.of(o, self.ctype) for o in others]
+        for a in args:
+            if a.ctype != self.ctype:
+                raise TypeError("operands of %s differ in type" % fn)
+        return Exp(self.ctype, "%s(%s)" % (fn, ", ".join(a.text for a in args)))
+
+    # -- Num
+    def __add__(self, o): return self._bin(o, "+")
+    def __radd__(self, o): return self._rbin(o, "+")
+    def __sub__(self, o): return self._bin(o, "-")
+    def __rsub__(self, o): return self._rbin(o, "-")
+    def __mul__(self, o): return self._bin(o, "*")
+    def __rmul__(self, o): return self._rbin(o, "*")
+    def __neg__(self): return Exp(self.ctype, "((%s)(-%s))" % (self.ctype, self.text))
+
+    # -- Fractional / Integral: `/` is fdiv on floating types and Haskell's `div` (towards -inf) on integers
+    def __truediv__(self, o):
+        if self.ctype in FLOATS:
+            return self._bin(o, "/")
+        return self._call("acc_idiv", o)
+
+    def __rtruediv__(self, o): return Exp.of(o, self.ctype).__truediv__(self)
+    def __floordiv__(self, o): return self._call("acc_idiv", o)
+    def __mod__(self, o): return self._call("acc_imod", o)
+
+    # -- Bits
+    def __and__(self, o): return self._bin(o, "&")
+    def __or__(self, o): return self._bin(o, "|")
+    def __xor__(self, o): return self._bin(o, "^")
+    def __invert__(self): return Exp(self.ctype, "((%s)(~%s))" % (self.ctype, self.text))
+    def __lshift__(self, o): return Exp(self.ctype, "acc_shift_l(%s, (Int64)%s)" % (self.text, Exp.of(o, "Int64").text))
+    def __rshift__(self, o): return Exp(self.ctype, "acc_shift_r(%s, (Int64)%s)" % (self.text, Exp.of(o, "Int64").text))
+
+    # -- Eq / Ord: Bool is Word8 (CodeGen/Type.hs:139)
+    def __lt__(self, o): return self._bin(o, "<", "Word8")
+    def __le__(self, o): return self._bin(o, "<=", "Word8")
+    def __gt__(self, o): return self._bin(o, ">", "Word8")
+    def __ge__(self, o): return self._bin(o, ">=", "Word8")
+    def eq(self, o): return self._bin(o, "==", "Word8")
+    def ne(self, o): return self._bin(o, "!=", "Word8")
+    def land(self, o): return self._bin(o, "&&", "Word8")
+    def lor(self, o): return self._bin(o, "||", "Word8")
+    def lnot(self): return Exp("Word8", "((Word8)(!%s))" % self.text)
+
+    def __bool__(self):
+        raise TypeError("an Exp has no truth value on the host: use cond(p, t, e)")
+
+
+def _literal(v, ctype):
+    if ctype == "float":
+        f = np.float32(v)
+        if np.isinf(f):
+            return "(-__builtin_inff())" if f < 0 else "__builtin_inff()"
+        return "%sf" % repr(float(f)) if "e" in repr(float(f)) or "." in repr(float(f)) else "%s.0f" % repr(float(f))
+    if ctype == "double":
+        f = float(v)
+        if np.isinf(f):
+            return "(-__builtin_inf())" if f < 0 else "__builtin_inf()"
+        return repr(f)
+    if ctype in ("Int64", "Word64"):
+        i = int(v)
+        if i == -2 ** 63:
+            return "(-9223372036854775807LL - 1)"
+        return "((%s)%d%s)" % (ctype, i, "LL" if ctype == "Int64" else "ULL")
+    i = int(v)
+    if i == -2 ** 31:
+        return "((%s)(-2147483647 - 1))" % ctype
+    return "((%s)%d)" % (ctype, i)
+
+
+def constant(v, ctype):
+    return Exp(ctype, _literal(v, ctype))
+
+
+def lift(*es):
+    """a tuple of expressions as one tuple-typed expression: brace initialiser of the generated struct"""
+    es = [Exp.of(e) for e in es]
+    return Exp(tuple(e.ctype for e in es), comps=es)
+
+
+def _var(ctype, name):
+    """a kernel-side variable of the given type; of a tuple type, its members (a<n-1> is the first component)"""
+    if isinstance(ctype, tuple):
+        n = len(ctype)
+        return Exp(ctype, comps=[Exp(t, "%s.a%d" % (name, n - 1 - k)) for k, t in enumerate(ctype)])
+    return Exp(ctype, name)
+
+
+def _prj(e, k):
+    if not isinstance(e.ctype, tuple):
+        raise TypeError("not a tuple")
+    return e.comps[k]
+
+
+def fst(e): return _prj(e, 0)
+def snd(e): return _prj(e, 1)
+
+
+def cond(p, t, e):
+    t = Exp.of(t, e.ctype if isinstance(e, Exp) else None)
+    e = Exp.of(e, t.ctype)
+    if t.ctype != e.ctype:
+        raise TypeError("branches of cond differ in type")
+    if isinstance(t.ctype, tuple):
+        return lift(*[cond(p, a, b) for a, b in zip(t.comps, e.comps)])
+    return Exp(t.ctype, "(%s ? %s : %s)" % (Exp.of(p).text, t.text, e.text))
+
+
+def fromIntegral(e, to): return Exp(to, "acc_from_integral<%s>(%s)" % (to, e.text))
+def truncate(e, to): return Exp(to, "acc_truncate<%s>(%s)" % (to, e.text))
+def round_(e, to): return Exp(to, "acc_round<%s>(%s)" % (to, e.text))
+def floor(e, to): return Exp(to, "acc_floor<%s>(%s)" % (to, e.text))
+def ceiling(e, to): return Exp(to, "acc_ceiling<%s>(%s)" % (to, e.text))
+def idiv(a, b): return Exp.of(a)._call("acc_idiv", b)
+def mod(a, b): return Exp.of(a)._call("acc_imod", b)
+def quot(a, b): return Exp.of(a)._call("acc_quot", b)
+def rem(a, b): return Exp.of(a)._call("acc_rem", b)
+def min_(a, b): return Exp.of(a)._call("acc_pmin", b)
+def max_(a, b): return Exp.of(a)._call("acc_pmax", b)
+def abs_(a): return a._call("acc_abs")
+def signum(a): return a._call("acc_signum")
+def sqrt(a): return a._call("acc_sqrt")
+def exp(a): return a._call("acc_exp")
+def log(a): return a._call("acc_log")
+def sin(a): return a._call("acc_sin")
+def cos(a): return a._call("acc_cos")
+def tan(a): return a._call("acc_tan")
+
+
+ignore = "ignore"        # the target index that drops an element (IndexSpace.hs:150-151)
+
+
+# ------------------------------------------------------------------------------ arrays
+
+class Acc(object):
+    """An array-valued computation: its shape (outermost first), element type and either a device
+    array (manifest) or an index -> value function (delayed)."""
+
+    def __init__(self, shape, ctype, manifest=None, at=None):
+        self.shape, self.ctype, self.manifest, self.at = tuple(int(s) for s in shape), ctype, manifest, at
+
+    @property
+    def size(self):
+        n = 1
+        for s in self.shape:
+            n *= s
+        return n
+
+    def index(self, ix):
+        """value at linear index `ix` (an Exp of type Int64).  A manifest array is named by a tag that
+        is replaced by its place in the kernel's environment when the kernel is assembled; read at the
+        consuming skeleton's own index `ix` it is a streaming read (each element is wanted once)."""
+        if self.manifest is not None:
+            tag = _tag(self.manifest)
+            if isinstance(self.ctype, tuple):
+                n = len(self.ctype)
+                return Exp(self.ctype, comps=[Exp(t, "%s_%d[%s]" % (tag, n - 1 - i, ix.text)) for i, t in enumerate(self.ctype)])
+            if ix.text == "ix":
+                return Exp(self.ctype, "acc_stream(%s_0, ix)" % tag)
+            return Exp(self.ctype, "%s_0[%s]" % (tag, ix.text))
+        return self.at(ix)
+
+    def stream(self):
+        """value at the consuming skeleton's own linear index"""
+        return self.index(Exp("Int64", "ix"))
+
+    def __getitem__(self, idx):
+        """`arr ! ix` inside a scalar function: idx is a multi-index (a tuple of Exps) or, for a vector, one Exp"""
+        return self.index(_linear(idx, self.shape))
+
+
+_MANIFEST = weakref.WeakValueDictionary()        # tag number -> device array, while some computation still names it
+
+
+def _tag(manifest):
+    _MANIFEST[id(manifest)] = manifest
+    return "@@%d@@" % id(manifest)
+
+
+def _assemble(**fragments):
+    """number the free arrays the fragments name, in order of first appearance (the Gamma environment of
+    AST.hs:87-112), and spell them arrIn<k>: returns (arrays, signature, fragments)"""
+    order = []
+    for text in fragments.values():
+        for m in re.finditer(r"@@(\d+)@@", text or ""):
+            if int(m.group(1)) not in order:
+                order.append(int(m.group(1)))
+    arrays = [_MANIFEST[i] for i in order]
+    out = {}
+    for name, text in fragments.items():
+        if text is not None:
+            for k, i in enumerate(order):
+                text = text.replace("@@%d@@" % i, "arrIn%d" % k)
+        out[name] = text
+    sig = []
+    for m in arrays:
+        if isinstance(m, A.TupleArray):
+            sig.append((len(m.shape), m.ctypes_of()))
+        else:
+            sig.append((len(m.shape), CTYPE[m.dtype.type]))
+    return arrays, sig, out
+
+
+class Context(object):
+    """a device context plus the table of skeleton instances built so far (the kernel table of State.hs:110-119)"""
+    _default = None
+
+    def __init__(self, device=0):
+        self.ctx = A.Context(device)
+        self.skeletons = {}
+
+    @classmethod
+    def default(cls):
+        if cls._default is None:
+            cls._default = Context(0)
+        return cls._default
+
+    def skeleton(self, kind, elt, env, **kw):
+        key = (kind, elt, tuple((r, tuple(t) if isinstance(t, list) else t) for r, t in env),
+               tuple(sorted((k, str(v)) for k, v in kw.items())))
+        sk = self.skeletons.get(key)
+        if sk is None:
+            sk = self.ctx.skeleton(kind, elt, env=env, **kw)
+            self.skeletons[key] = sk
+        return sk
+
+
+def _elt(ctype):
+    return ", ".join(ctype) if isinstance(ctype, tuple) else ctype
+
+
+def _dtype(ctype):
+    return [NPTYPE[c] for c in ctype] if isinstance(ctype, tuple) else NPTYPE[ctype]
+
+
+def _empty(cx, shape, ctype):
+    if isinstance(ctype, tuple):
+        return cx.ctx.empty_tuple(shape, _dtype(ctype))
+    return cx.ctx.empty(shape, _dtype(ctype))
+
+
+def use(host, context=None):
+    """a host array (or a tuple of equally shaped host arrays: an array of tuples) made available on the device"""
+    cx = context or Context.default()
+    if isinstance(host, tuple):
+        hs = [np.ascontiguousarray(h) for h in host]
+        return Acc(hs[0].shape, tuple(CTYPE[h.dtype.type] for h in hs), manifest=cx.ctx.tuple_array(*hs))
+    host = np.ascontiguousarray(host)
+    return Acc(host.shape, CTYPE[host.dtype.type], manifest=cx.ctx.array(host))
+
+
+def unit(value, ctype, context=None):
+    return use(np.array(value, dtype=NPTYPE[ctype]), context)
+
+
+def _unlinear(ix, shape):
+    """multi-index (outermost first) of a linear index, as Exps; extents are literals, so the divisions are by constants"""
+    out, rest = [], ix
+    for d in range(len(shape) - 1, -1, -1):
+        ext = constant(shape[d], "Int64")
+        if d == 0:
+            out.append(rest)
+        else:
+            out.append(Exp("Int64", "(%s %% %s)" % (rest.text, ext.text)))
+            rest = Exp("Int64", "(%s / %s)" % (rest.text, ext.text))
+    return tuple(reversed(out))
+
+
+def _linear(idx, shape):
+    idx = [Exp.of(i, "Int64") for i in (idx if isinstance(idx, (tuple, list)) else (idx,))]
+    idx = [i if i.ctype == "Int64" else fromIntegral(i, "Int64") for i in idx]
+    if len(idx) != len(shape):
+        raise TypeError("index of rank %d into an array of rank %d" % (len(idx), len(shape)))
+    if not shape:
+        return constant(0, "Int64")
+    acc_ = idx[0]
+    for d in range(1, len(shape)):
+        acc_ = acc_ * constant(shape[d], "Int64") + idx[d]
+    return acc_
+
+
+def _probe(f, *ctypes):
+    """result type of a scalar function, found by applying it to dummy operands"""
+    return Exp.of(f(*[_var(c, "_") for c in ctypes])).ctype
+
+
+def map(f, a):
+    t = _probe(f, a.ctype)
+    return Acc(a.shape, t, at=lambda ix: Exp.of(f(a.index(ix))))
+
+
+def _meet(s1, s2):
+    return tuple(min(x, y) for x, y in zip(s1, s2))
+
+
+def zipWith(f, a, b):
+    """extent = intersection of the operands' extents (Accelerate's zipWith)"""
+    if a.shape != b.shape:
+        if len(a.shape) != len(b.shape):
+            raise TypeError("zipWith of arrays of different rank")
+        shape = _meet(a.shape, b.shape)
+        a = a if a.shape == shape else backpermute(shape, lambda *i: i, a)
+        b = b if b.shape == shape else backpermute(shape, lambda *i: i, b)
+    t = _probe(f, a.ctype, b.ctype)
+    return Acc(a.shape, t, at=lambda ix: Exp.of(f(a.index(ix), b.index(ix))))
+
+
+def generate(shape, f):
+    shape = (shape,) if isinstance(shape, numbers.Integral) else tuple(shape)
+    t = _probe(f, *["Int64"] * len(shape))
+    return Acc(shape, t, at=lambda ix: Exp.of(f(*_unlinear(ix, shape))))
+
+
+def backpermute(shape, p, a):
+    """result[i] = a[p(i)]: p takes the result's multi-index and returns a multi-index of `a`"""
+    shape = (shape,) if isinstance(shape, numbers.Integral) else tuple(shape)
+    return Acc(shape, a.ctype, at=lambda ix: a.index(_linear(p(*_unlinear(ix, shape)), a.shape)))
+
+
+def transpose(a):
+    h, w = a.shape
+    return backpermute((w, h), lambda y, x: (x, y), a)
+
+
+def zip_(a, b):
+    """array of pairs over the intersection of the extents"""
+    return zipWith(lambda x, y: lift(x, y), a, b)
+
+
+def unzip(a):
+    return map(fst, a), map(snd, a)
+
+
+def reverse(a):
+    n = a.shape[0]
+    return backpermute((n,), lambda i: (constant(n - 1, "Int64") - i,), a)
+
+
+# ------------------------------------------------------------------------------ execution
+
+def _force(a, cx):
+    """a manifest array holding `a` (one map kernel if it is delayed)"""
+    if a.manifest is not None:
+        return a
+    arrays, sig, fr = _assemble(get=a.stream().text)
+    sk = cx.skeleton(A.SKEL_MAP, _elt(a.ctype), sig, out_rank=len(a.shape), **fr)
+    out = _empty(cx, a.shape, a.ctype)
+    sk.map(arrays, out)
+    return Acc(a.shape, a.ctype, manifest=out)
+
+
+def _combine(f, ctype):
+    r = Exp.of(f(_var(ctype, "x"), _var(ctype, "y")), ctype)
+    if r.ctype != ctype:
+        raise TypeError("the combining function returns %s for elements of type %s" % (r.ctype, ctype))
+    return r
+
+
+def _fold(f, z, a, seedless, context):
+    cx = context or Context.default()
+    out_shape = a.shape[:-1]
+    arrays, sig, fr = _assemble(get=a.stream().text, combine=_combine(f, a.ctype).text,
+                                seed=None if seedless else Exp.of(z, a.ctype).text)
+    sk = cx.skeleton(A.SKEL_FOLD1 if seedless else A.SKEL_FOLD, _elt(a.ctype), sig, out_rank=len(out_shape), **fr)
+    out = _empty(cx, out_shape, a.ctype)
+    sk.fold(arrays, a.shape, out)
+    return Acc(out_shape, a.ctype, manifest=out)
+
+
+def fold(f, z, a, context=None):
+    """reduce the innermost dimension with an associative f; z is combined in once (Reduction.hs:203-211)"""
+    return _fold(f, z, a, False, context)
+
+
+def fold1(f, a, context=None):
+    return _fold(f, None, a, True, context)
+
+
+def foldSeg(f, z, a, seg_lengths, context=None):
+    """reduce each segment of a vector; `seg_lengths` is a vector of segment lengths (Int32), turned into
+    offsets by an exclusive scan on the device as the front end does (CUDA.hs:402)"""
+    cx = context or Context.default()
+    offs = scanl(lambda x, y: x + y, constant(0, seg_lengths.ctype), seg_lengths, context=cx)
+    arrays, sig, fr = _assemble(get=a.stream().text, combine=_combine(f, a.ctype).text, seed=Exp.of(z, a.ctype).text)
+    sk = cx.skeleton(A.SKEL_FOLDSEG, _elt(a.ctype), sig, seg_type=seg_lengths.ctype, **fr)
+    nseg = seg_lengths.shape[0]
+    out = _empty(cx, (nseg,), a.ctype)
+    sk.foldseg(arrays, a.size, offs.manifest, out)
+    return Acc((nseg,), a.ctype, manifest=out)
+
+
+def _scan(kind, f, z, a, context):
+    cx = context or Context.default()
+    if len(a.shape) != 1:
+        raise TypeError("scans are over vectors")
+    arrays, sig, fr = _assemble(get=a.stream().text, combine=_combine(f, a.ctype).text,
+                                seed=Exp.of(z, a.ctype).text if z is not None else None)
+    sk = cx.skeleton(A.SCAN_KINDS[kind], _elt(a.ctype), sig, **fr)
+    n = a.shape[0]
+    m = n + 1 if kind in ("scanl", "scanr") else n
+    out = _empty(cx, (m,), a.ctype)
+    total = _empty(cx, (), a.ctype) if kind.endswith("'") else None
+    sk.scan(arrays, n, out, total)
+    res = Acc((m,), a.ctype, manifest=out)
+    return (res, Acc((), a.ctype, manifest=total)) if total is not None else res
+
+
+def scanl(f, z, a, context=None): return _scan("scanl", f, z, a, context)
+def scanl1(f, a, context=None): return _scan("scanl1", f, None, a, context)
+def scanl_(f, z, a, context=None): return _scan("scanl'", f, z, a, context)      # scanl': (body, total)
+def scanr(f, z, a, context=None): return _scan("scanr", f, z, a, context)
+def scanr1(f, a, context=None): return _scan("scanr1", f, None, a, context)
+def scanr_(f, z, a, context=None): return _scan("scanr'", f, z, a, context)
+
+
+_HINTS = {"+": A.COMBINE_ADD, "min": A.COMBINE_MIN, "max": A.COMBINE_MAX, "&": A.COMBINE_AND, "|": A.COMBINE_OR, "^": A.COMBINE_XOR}
+
+
+def _hint(f, ctype):
+    """recognise a combining function the hardware applies atomically, by its generated text (the check a code
+    generator makes on the expression tree)"""
+    if isinstance(ctype, tuple) or ctype not in ("Int32", "Word32", "Int64", "Word64", "float", "double"):
+        return A.COMBINE_GENERIC
+    text = _combine(f, ctype).text
+    for op, h in _HINTS.items():
+        if len(op) == 1:
+            forms = ("((%s)(x %s y))" % (ctype, op), "((%s)(y %s x))" % (ctype, op))
+        else:
+            forms = ("acc_p%s(x, y)" % op, "acc_p%s(y, x)" % op)
+        if text in forms and (ctype not in FLOATS or op == "+"):
+            return h
+    return A.COMBINE_GENERIC
+
+
+class _Maybe(object):
+    def __init__(self, p, idx):
+        self.p, self.idx = Exp.of(p), idx
+
+
+def index_if(p, idx):
+    """a permutation result that is `idx` where p holds and `ignore` elsewhere"""
+    return _Maybe(p, idx)
+
+
+def permute(f, defaults, p, a, context=None):
+    """forward permutation: out = defaults; out[p(i)] = f(a[i], out[p(i)]) for every source index i;
+    p(i) = ignore (or index_if with a false condition) drops the element"""
+    cx = context or Context.default()
+    dfl = _force(defaults, cx)
+    t = p(*_unlinear(Exp("Int64", "ix"), a.shape))
+    if isinstance(t, str) and t == ignore:
+        perm_text = "ACC_IGNORE"
+    elif isinstance(t, _Maybe):
+        perm_text = "(%s ? %s : ACC_IGNORE)" % (t.p.text, _linear(t.idx, dfl.shape).text)
+    else:
+        perm_text = _linear(t, dfl.shape).text
+    arrays, sig, fr = _assemble(get=a.stream().text, combine=_combine(f, a.ctype).text, permutation=perm_text)
+    sk = cx.skeleton(A.SKEL_PERMUTE, _elt(a.ctype), sig, out_rank=len(dfl.shape), combine_hint=_hint(f, a.ctype), **fr)
+    out = _empty(cx, dfl.shape, a.ctype)
+    sk.permute(arrays, a.size, dfl.manifest, out)
+    return Acc(dfl.shape, a.ctype, manifest=out)
+
+
+def the(a, context=None):
+    """the value of a scalar array, on the host"""
+    return run(a, context)[()]
+
+
+def _taps(pattern, rank):
+    offs = []
+    for t in pattern:
+        t = tuple(t) if isinstance(t, (tuple, list)) else (t,)
+        offs.append((0,) * (max(2, rank) - len(t)) + t)
+    return offs
+
+
+def stencil(pattern, f, boundary, a, context=None, constant_value=None):
+    """result[i] = f(a[i + o] for o in pattern); boundary is "clamp", "mirror", "wrap" or "constant"
+    (Stencil/Extra.hs:112-116); the source is made manifest first, as in the reference (Execute.hs:413-425)"""
+    cx = context or Context.default()
+    src = _force(a, cx)
+    rank = len(src.shape)
+    taps = _taps(pattern, rank)
+    res = Exp.of(f(*[Exp(src.ctype, "t%d" % k) for k in range(len(taps))]))
+    arrays, sig, fr = _assemble(stencil_fn=res.text)
+    sk = cx.skeleton(A.SKEL_STENCIL, res.ctype, sig, out_rank=rank, taps=taps, boundary=boundary,
+                     boundary_constant=None if constant_value is None else _literal(constant_value, src.ctype),
+                     stencil_in=src.ctype, **fr)
+    out = _empty(cx, src.shape, res.ctype)
+    sk.stencil(arrays, src.manifest, out)
+    return Acc(src.shape, res.ctype, manifest=out)
+
+
+def stencil2(pattern1, pattern2, f, boundary1, a, boundary2, b, context=None, constant1=None, constant2=None):
+    """f receives the list of taps of the first source and the list of taps of the second"""
+    cx = context or Context.default()
+    s1, s2 = _force(a, cx), _force(b, cx)
+    rank = len(s1.shape)
+    t1, t2 = _taps(pattern1, rank), _taps(pattern2, rank)
+    res = Exp.of(f([Exp(s1.ctype, "t%d" % k) for k in range(len(t1))], [Exp(s2.ctype, "u%d" % k) for k in range(len(t2))]))
+    arrays, sig, fr = _assemble(stencil_fn=res.text)
+    sk = cx.skeleton(A.SKEL_STENCIL2, res.ctype, sig, out_rank=rank, taps=t1, boundary=boundary1, taps2=t2, boundary2=boundary2,
+                     boundary_constant=None if constant1 is None else _literal(constant1, s1.ctype),
+                     boundary2_constant=None if constant2 is None else _literal(constant2, s2.ctype),
+                     stencil_in=s1.ctype, stencil_in2=s2.ctype, **fr)
+    shape = _meet(s1.shape, s2.shape)
+    out = _empty(cx, shape, res.ctype)
+    sk.stencil2(arrays, s1.manifest, s2.manifest, out)
+    return Acc(shape, res.ctype, manifest=out)
+
+
+def run(a, context=None):
+    """evaluate and bring the result to the host (CUDA.hs:209-216); a tuple of Acc gives a tuple of results"""
+    cx = context or Context.default()
+    if isinstance(a, tuple):
+        return tuple(run(x, cx) for x in a)
+    return _force(a, cx).manifest.get()
+
+
+def run1(f, context=None):
+    """a function from host arrays to host arrays whose kernels are built on the first call and reused afterwards
+    (CUDA.hs:318-333: `run1 f` must be partially applied so that the compiled kernels are shared between calls)"""
+    cx = context or Context.default()
+
+    def go(*hosts):
+        return run(f(*[use(h, cx) for h in hosts]), cx)
+    return go

@@ -1,0 +1,91 @@
+"""The embedded array language without a GPU: what text it generates for the benchmark programs, how it numbers the
+free arrays, and that the generated skeleton instances compile for gfx950.  Device arrays are stood in for by objects
+with a shape and a dtype; nothing is launched."""
+import numpy as np
+import pytest
+
+import acchip as A
+import accelerate_hip as acc
+
+
+class Resident(object):
+    def __init__(self, shape, dt):
+        self.shape, self.dtype = tuple(shape), np.dtype(dt)
+
+
+def use(shape, dt):
+    return acc.Acc(shape, acc.CTYPE[np.dtype(dt).type], manifest=Resident(shape, dt))
+
+
+def add(x, y):
+    return x + y
+
+
+def test_dotp_fuses_into_one_fold_over_two_streamed_arrays():
+    xs, ys = use((100,), np.float32), use((100,), np.float32)
+    d = acc.zipWith(lambda a, b: a * b, xs, ys)
+    arrays, sig, fr = acc._assemble(get=d.stream().text, combine=acc._combine(add, "float").text,
+                                    seed=acc.Exp.of(0.0, "float").text)
+    assert arrays == [xs.manifest, ys.manifest] and sig == [(1, "float"), (1, "float")]
+    assert fr == {"get": "((float)(acc_stream(arrIn0_0, ix) * acc_stream(arrIn1_0, ix)))",
+                  "combine": "((float)(x + y))", "seed": "0.0f"}
+    assert A.compile_only(A.make_desc(A.SKEL_FOLD, "float", env=sig, **fr)) > 0
+    # the same array twice is one environment slot
+    sq = acc.zipWith(lambda a, b: a * b, xs, xs)
+    arrays, sig, fr = acc._assemble(get=sq.stream().text)
+    assert len(arrays) == 1 and fr["get"].count("arrIn0_0") == 2
+
+
+def test_free_arrays_are_numbered_in_order_of_first_use_across_fragments():
+    ks, ws = use((1000,), np.int32), use((1000,), np.int32)
+    target = acc._linear((ks[acc.Exp("Int64", "ix")],), (256,))
+    arrays, sig, fr = acc._assemble(get=ws.stream().text, combine=acc._combine(add, "Int32").text, permutation=target.text)
+    assert arrays == [ws.manifest, ks.manifest]
+    assert fr["permutation"] == "acc_from_integral<Int64>(acc_stream(arrIn1_0, ix))"
+    desc = A.make_desc(A.SKEL_PERMUTE, "Int32", env=sig, out_rank=1, combine_hint=acc._hint(add, "Int32"), **fr)
+    assert A.compile_only(desc) > 0
+
+
+def test_combination_hints_are_read_off_the_generated_text():
+    assert acc._hint(add, "Int32") == A.COMBINE_ADD
+    assert acc._hint(lambda x, y: y + x, "float") == A.COMBINE_ADD
+    assert acc._hint(acc.max_, "Int64") == A.COMBINE_MAX
+    assert acc._hint(acc.min_, "Word32") == A.COMBINE_MIN
+    assert acc._hint(acc.max_, "float") == A.COMBINE_GENERIC           # no floating-point atomic max is assumed
+    assert acc._hint(lambda x, y: x ^ y, "Word64") == A.COMBINE_XOR
+    assert acc._hint(lambda x, y: acc.cond(x > y, x, y), "Int32") == A.COMBINE_GENERIC
+    assert acc._hint(add, "Int16") == A.COMBINE_GENERIC
+
+
+def test_tuples_live_on_the_host_side_of_the_text():
+    ps = acc.Acc((10,), ("Int16", "double"), manifest=Resident((10,), np.int16))
+    sw = acc.map(lambda p: acc.lift(acc.snd(p), acc.fst(p)), ps)
+    assert sw.ctype == ("double", "Int16")
+    text = sw.stream().text
+    assert text.startswith("acc_elt{") and text.index("_0[ix]") < text.index("_1[ix]")      # snd first: component 0
+    c = acc._combine(lambda p, q: acc.cond(acc.fst(p) >= acc.fst(q), p, q), ("float", "Int32"))
+    assert c.text == "acc_elt{(((Word8)(x.a1 >= y.a1)) ? x.a1 : y.a1), (((Word8)(x.a1 >= y.a1)) ? x.a0 : y.a0)}"
+    seed = acc.Exp.of((-np.inf, -1), ("float", "Int32"))
+    assert seed.text == "acc_elt{(-__builtin_inff()), ((Int32)-1)}"
+    desc = A.make_desc(A.SKEL_FOLD, "float, Int32", env=[(1, ["Int32", "float"])],
+                       get="acc_elt{arrIn0_1[ix], arrIn0_0[ix]}", combine=c.text, seed=seed.text)
+    assert A.compile_only(desc) > 0
+
+
+def test_index_arithmetic_of_the_delayed_combinators():
+    m = use((3, 5), np.int32)
+    t = acc.transpose(m)
+    assert t.shape == (5, 3)
+    arrays, sig, fr = acc._assemble(get=t.stream().text)
+    assert sig == [(2, "Int32")]
+    ix = np.arange(15)
+    y, x = ix // 3, ix % 3                       # the result's (row, column)
+    src = eval(fr["get"].replace("arrIn0_0", "src").replace("((Int64)", "(").replace("LL)", ")").replace("/", "//"),
+               {"src": np.arange(15), "ix": ix, "Int64": lambda v: v})
+    assert np.array_equal(src, x * 5 + y)
+    with pytest.raises(TypeError):
+        m[acc.Exp("Int64", "ix")]                # a rank-1 index into a matrix
+    with pytest.raises(TypeError):
+        acc.zipWith(add, m, use((3, 5), np.float32))
+    with pytest.raises(TypeError):
+        acc._combine(lambda x, y: x < y, "Int32")

@@ -1,0 +1,202 @@
+"""The embedded array language (accelerate_hip) against numpy: the benchmark programs written the way a user of
+the reference writes them (accelerate-examples' dotp, scan, histogram via permute, stencil, smvm), plus the
+delayed-array combinators.  Integer results are exact; floating-point sums carry the tolerance stated per test."""
+import numpy as np
+import pytest
+
+import pyref
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def acc():
+    import accelerate_hip
+    return accelerate_hip
+
+
+def add(x, y):
+    return x + y
+
+
+def test_dotp_is_one_kernel(acc):
+    rng = np.random.default_rng(1)
+    x, y = rng.standard_normal(1000003).astype(np.float32), rng.standard_normal(1000003).astype(np.float32)
+    cx = acc.Context.default()
+    before = len(cx.skeletons)
+    r = acc.run(acc.fold(add, 0.0, acc.zipWith(lambda a, b: a * b, acc.use(x), acc.use(y))))
+    assert len(cx.skeletons) == before + 1                      # zipWith fused into the fold
+    assert r.shape == () and abs(float(r) - float(np.dot(x.astype(np.float64), y.astype(np.float64)))) < 1e-3 * np.sqrt(x.size)
+    xi, yi = rng.integers(-1000, 1000, 77777).astype(np.int32), rng.integers(-1000, 1000, 77777).astype(np.int32)
+    r = acc.run(acc.fold(add, 0, acc.zipWith(lambda a, b: a * b, acc.use(xi), acc.use(yi))))
+    assert int(r) == pyref.wrap(int(np.dot(xi.astype(np.int64), yi.astype(np.int64))), 32, True)
+
+
+def test_saxpy_and_run1_reuses_kernels(acc):
+    rng = np.random.default_rng(2)
+    cx = acc.Context.default()
+    saxpy = acc.run1(lambda xs, ys: acc.zipWith(lambda x, y: acc.constant(1.5, "float") * x + y, xs, ys))
+    x, y = rng.standard_normal(4099).astype(np.float32), rng.standard_normal(4099).astype(np.float32)
+    assert np.array_equal(saxpy(x, y), np.float32(1.5) * x + y)
+    n = len(cx.skeletons)
+    x2, y2 = rng.standard_normal(513).astype(np.float32), rng.standard_normal(513).astype(np.float32)
+    assert np.array_equal(saxpy(x2, y2), np.float32(1.5) * x2 + y2)
+    assert len(cx.skeletons) == n
+
+
+def test_six_scans(acc):
+    rng = np.random.default_rng(3)
+    x = rng.integers(-50, 50, 100001).astype(np.int32)
+    xs = acc.use(x)
+    c = np.cumsum(x, dtype=np.int32)
+    rc = np.cumsum(x[::-1], dtype=np.int32)[::-1]
+    assert np.array_equal(acc.run(acc.scanl(add, 0, xs)), np.concatenate([[0], c]).astype(np.int32))
+    assert np.array_equal(acc.run(acc.scanl1(add, xs)), c)
+    body, total = acc.run(acc.scanl_(add, 0, xs))
+    assert np.array_equal(body, np.concatenate([[0], c[:-1]]).astype(np.int32)) and int(total) == int(c[-1])
+    assert np.array_equal(acc.run(acc.scanr(add, 0, xs)), np.concatenate([rc, [0]]).astype(np.int32))
+    assert np.array_equal(acc.run(acc.scanr1(add, xs)), rc)
+    body, total = acc.run(acc.scanr_(add, 0, xs))
+    assert np.array_equal(body, np.concatenate([rc[1:], [0]]).astype(np.int32)) and int(total) == int(rc[0])
+    # a scan of a delayed array with a non-commutative-looking operator: running maximum of squares
+    m = acc.run(acc.scanl1(acc.max_, acc.map(lambda v: v * v, xs)))
+    assert np.array_equal(m, np.maximum.accumulate(x * x))
+
+
+def test_histogram_via_permute_reads_keys_inside_the_permutation(acc):
+    rng = np.random.default_rng(4)
+    bins, n = 256, 300007
+    keys = rng.integers(0, bins, n).astype(np.int32)
+    ks = acc.use(keys)
+    zeros = acc.generate((bins,), lambda i: acc.constant(0, "Int32"))
+    ones = acc.generate((n,), lambda i: acc.constant(1, "Int32"))
+    h = acc.run(acc.permute(add, zeros, lambda i: (ks[i],), ones))
+    assert np.array_equal(h, np.bincount(keys, minlength=bins).astype(np.int32))
+    # weighted, with every odd key dropped
+    w = rng.integers(1, 9, n).astype(np.int32)
+    h = acc.run(acc.permute(add, zeros, lambda i: acc.index_if((ks[i] & 1).eq(0), (ks[i],)), acc.use(w)))
+    even = (keys & 1) == 0
+    assert np.array_equal(h, np.bincount(keys[even], weights=w[even], minlength=bins).astype(np.int32))
+    # nothing lands anywhere
+    h = acc.run(acc.permute(add, acc.use(np.arange(bins, dtype=np.int32)), lambda i: acc.ignore, acc.use(w)))
+    assert np.array_equal(h, np.arange(bins, dtype=np.int32))
+
+
+def test_permute_with_a_generic_combination(acc):
+    rng = np.random.default_rng(5)
+    n, m = 50021, 97
+    t = rng.integers(0, m, n).astype(np.int32)
+    v = rng.integers(-10 ** 6, 10 ** 6, n).astype(np.int64)
+    ts = acc.use(t)
+    first = np.full(m, -2 ** 62, dtype=np.int64)
+    out = acc.run(acc.permute(lambda x, y: acc.cond(x > y, x, y), acc.use(first), lambda i: (ts[i],), acc.use(v)))
+    ref = first.copy()
+    np.maximum.at(ref, t, v)
+    assert np.array_equal(out, ref)
+
+
+def test_stencils(acc):
+    rng = np.random.default_rng(6)
+    img = rng.standard_normal((301, 517)).astype(np.float32)
+    pat = [(dy, dx) for dy in (-1, 0, 1) for dx in (-1, 0, 1)]
+    wts = [1, 2, 1, 2, 4, 2, 1, 2, 1]
+
+    def gauss(*t):
+        s = t[0] * acc.constant(wts[0], "float")
+        for k in range(1, 9):
+            s = s + t[k] * acc.constant(wts[k], "float")
+        return s / acc.constant(16, "float")
+    for mode in ("clamp", "mirror", "wrap"):
+        out = acc.run(acc.stencil(pat, gauss, mode, acc.use(img)))
+        taps = pyref.tap_arrays(img, pat, mode, 0, img.shape)
+        ref = taps[0] * np.float32(wts[0])
+        for k in range(1, 9):
+            ref = ref + taps[k] * np.float32(wts[k])
+        assert np.array_equal(out, ref / np.float32(16)), mode
+    # 1-D second difference of a delayed array (forced to a manifest array first), constant boundary
+    x = rng.integers(-100, 100, 10007).astype(np.int32)
+    out = acc.run(acc.stencil([(-1,), (0,), (1,)], lambda a, b, c: a - 2 * b + c, "constant",
+                              acc.map(lambda v: v + 1, acc.use(x)), constant_value=7))
+    p = np.concatenate([[7], x + 1, [7]]).astype(np.int32)
+    assert np.array_equal(out, p[:-2] - 2 * p[1:-1] + p[2:])
+    # stencil2: difference of a horizontal gradient of one image and a vertical gradient of another
+    img2 = rng.standard_normal((301, 517)).astype(np.float32)
+    out = acc.run(acc.stencil2([(0, -1), (0, 1)], [(-1, 0), (1, 0)], lambda t, u: (t[1] - t[0]) - (u[1] - u[0]),
+                               "clamp", acc.use(img), "wrap", acc.use(img2)))
+    t = pyref.tap_arrays(img, [(0, -1), (0, 1)], "clamp", 0, img.shape)
+    u = pyref.tap_arrays(img2, [(-1, 0), (1, 0)], "wrap", 0, img.shape)
+    assert np.array_equal(out, (t[1] - t[0]) - (u[1] - u[0]))
+
+
+def test_smvm_by_foldseg(acc):
+    rng = np.random.default_rng(7)
+    rows, ncols = 4001, 3000
+    lens = rng.integers(0, 40, rows).astype(np.int32)
+    nnz = int(lens.sum())
+    cols = rng.integers(0, ncols, nnz).astype(np.int32)
+    vals = rng.integers(-9, 10, nnz).astype(np.float32)          # small integers: float sums are exact
+    vec = rng.integers(-9, 10, ncols).astype(np.float32)
+    v = acc.use(vec)
+    products = acc.zipWith(lambda c, a: a * v[c], acc.use(cols), acc.use(vals))
+    y = acc.run(acc.foldSeg(add, 0.0, products, acc.use(lens)))
+    offs = np.concatenate([[0], np.cumsum(lens)])
+    ref = np.array([np.sum(vals[offs[r]:offs[r + 1]] * vec[cols[offs[r]:offs[r + 1]]], dtype=np.float32) for r in range(rows)],
+                   dtype=np.float32)
+    assert np.array_equal(y, ref)
+
+
+def test_index_transformations(acc):
+    rng = np.random.default_rng(8)
+    m = rng.integers(0, 1000, (37, 101)).astype(np.int32)
+    assert np.array_equal(acc.run(acc.transpose(acc.use(m))), m.T)
+    x = rng.integers(0, 1000, 1001).astype(np.int64)
+    assert np.array_equal(acc.run(acc.reverse(acc.use(x))), x[::-1])
+    # zipWith over different extents takes the intersection
+    a, b = rng.integers(0, 9, (5, 9)).astype(np.int32), rng.integers(0, 9, (7, 4)).astype(np.int32)
+    assert np.array_equal(acc.run(acc.zipWith(add, acc.use(a), acc.use(b))), a[:5, :4] + b[:5, :4])
+    # generate over a rank-3 index, fold over the innermost dimension of it
+    g = acc.generate((3, 5, 7), lambda z, y, x_: z * 100 + y * 10 + x_)
+    zz, yy, xx = np.meshgrid(np.arange(3), np.arange(5), np.arange(7), indexing="ij")
+    ref = (zz * 100 + yy * 10 + xx).astype(np.int64)
+    assert np.array_equal(acc.run(g), ref)
+    assert np.array_equal(acc.run(acc.fold(add, 0, g)), ref.sum(axis=2))
+    assert np.array_equal(acc.run(acc.fold1(acc.min_, g)), ref.min(axis=2))
+
+
+def test_integer_division_follows_haskell(acc):
+    a = np.array([7, -7, 7, -7, 0, 5, -5, 2 ** 31 - 1, -2 ** 31], dtype=np.int32)
+    b = np.array([2, 2, -2, -2, 3, 5, 5, -1, 1], dtype=np.int32)
+    xs, ys = acc.use(a), acc.use(b)
+    assert np.array_equal(acc.run(acc.zipWith(lambda x, y: x // y, xs, ys)), a // b)
+    assert np.array_equal(acc.run(acc.zipWith(lambda x, y: x % y, xs, ys)), a % b)
+    assert np.array_equal(acc.run(acc.zipWith(acc.quot, xs, ys)), np.array([pyref.wrap(pyref.quot(int(p), int(q)), 32, True) for p, q in zip(a, b)], dtype=np.int32))
+    assert np.array_equal(acc.run(acc.zipWith(acc.rem, xs, ys)), np.array([pyref.wrap(pyref.rem(int(p), int(q)), 32, True) for p, q in zip(a, b)], dtype=np.int32))
+
+
+def test_tuples_argmax_and_unzip(acc):
+    rng = np.random.default_rng(9)
+    n = 123457
+    x = rng.permutation(n).astype(np.float32)
+    idx = acc.generate((n,), lambda i: acc.fromIntegral(i, "Int32"))
+    pairs = acc.zip_(acc.use(x), idx)
+    best = acc.fold(lambda p, q: acc.cond(acc.fst(p) >= acc.fst(q), p, q), (-np.inf, -1), pairs)
+    val, where = acc.run(best)
+    assert float(val) == float(x.max()) and int(where) == int(np.argmax(x))
+    # a manifest array of pairs read back, swapped
+    ys = rng.integers(0, 100, 1000).astype(np.int16)
+    zs = rng.standard_normal(1000)
+    sw = acc.map(lambda p: acc.lift(acc.snd(p), acc.fst(p)), acc.use((ys, zs)))
+    a, b = acc.run(sw)
+    assert np.array_equal(a, zs) and np.array_equal(b, ys)
+    f, s = acc.unzip(sw)
+    assert np.array_equal(acc.run(s), ys)
+
+
+def test_type_errors_are_reported_before_anything_is_compiled(acc):
+    xs = acc.use(np.zeros(4, dtype=np.int32))
+    with pytest.raises(TypeError):
+        acc.zipWith(add, xs, acc.use(np.zeros(4, dtype=np.float32)))
+    with pytest.raises(TypeError):
+        acc.scanl(add, 0, acc.use(np.zeros((2, 2), dtype=np.int32)))
+    with pytest.raises(TypeError):
+        acc.map(lambda v: 1 if v > 0 else 0, xs)
