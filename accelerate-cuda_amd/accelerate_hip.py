@@ -31,7 +31,7 @@ import numpy as np
 
 import acchip as A
 
-__all__ = ["Exp", "constant", "cond", "use", "unit", "map", "zipWith", "generate", "backpermute", "transpose", "reverse", "zip_", "unzip",
+__all__ = ["Exp", "constant", "cond", "use", "unit", "map", "zipWith", "generate", "backpermute", "transpose", "reverse", "zip_", "unzip", "while_",
            "fold", "fold1", "foldSeg", "scanl", "scanl1", "scanl_", "scanr", "scanr1", "scanr_", "permute", "ignore",
            "stencil", "stencil2", "run", "run1", "fst", "snd", "lift", "index_if", "fromIntegral", "truncate", "round_", "floor",
            "ceiling", "idiv", "mod", "quot", "rem", "min_", "max_", "sqrt", "exp", "log", "sin", "cos", "tan", "abs_",
@@ -45,16 +45,41 @@ RANK = {"Int8": 1, "Word8": 1, "Int16": 2, "Word16": 2, "Int32": 3, "Word32": 3,
 
 # ------------------------------------------------------------------------------ scalar expressions
 
-class Exp(object):
-    """A typed scalar expression: a C type name and text, or, for a tuple, the component expressions
-    (tuples exist only on the host side of the generated text: `fst`/`snd` pick a component, and the
-    braces of the element struct are written where a tuple becomes a skeleton's result)."""
+def _merge(exps):
+    out = []
+    for e in exps:
+        for st in e.binds:
+            if st not in out:
+                out.append(st)
+    return tuple(out)
 
-    def __init__(self, ctype, text=None, comps=None):
+
+class Exp(object):
+    """A typed scalar expression: a C type name, the text of a pure expression (`term`) and the
+    statements that must run before it (`binds`: the loops of `while_`; the local bindings of the
+    reference's code generation monad, CodeGen/Monad.hs).  Of a tuple type it holds the component
+    expressions instead: tuples exist only on the host side of the generated text, `fst`/`snd` pick a
+    component, and the braces of the element struct are written where a tuple becomes a result.
+    `text` is the closed form a skeleton fragment takes: the term alone, or an immediately applied
+    lambda holding the statements."""
+
+    def __init__(self, ctype, term=None, comps=None, binds=()):
         self.ctype, self.comps = ctype, comps
         if comps is not None:
-            text = "acc_elt{%s}" % ", ".join(c.text for c in comps)
-        self.text = text
+            term = "acc_elt{%s}" % ", ".join(c.term for c in comps)
+            binds = _merge(comps)
+        self.term, self.binds = term, tuple(binds)
+
+    @property
+    def text(self):
+        if not self.binds:
+            return self.term
+        return "[&] { %s return %s; }()" % (" ".join(self.binds), self.term)
+
+    @staticmethod
+    def mk(ctype, fmt, *args):
+        """an expression whose text is `fmt` over the operands' terms and which runs their statements first"""
+        return Exp(ctype, fmt % tuple(a.term for a in args), binds=_merge(args))
 
     # -- helpers
     @staticmethod
@@ -72,7 +97,7 @@ class Exp(object):
         o = Exp.of(other, self.ctype)
         if o.ctype != self.ctype:
             raise TypeError("operands of %s differ in type: %s and %s (convert with fromIntegral)" % (op, self.ctype, o.ctype))
-        return Exp(result or self.ctype, "((%s)(%s %s %s))" % (result or self.ctype, self.text, op, o.text))
+        return Exp.mk(result or self.ctype, "((%s)(%%s %s %%s))" % (result or self.ctype, op.replace("%", "%%")), self, o)
 
     def _rbin(self, other, op):
         return Exp.of(other, self.ctype)._bin(self, op)
@@ -82,7 +107,7 @@ class Exp(object):
         for a in args:
             if a.ctype != self.ctype:
                 raise TypeError("operands of %s differ in type" % fn)
-        return Exp(self.ctype, "%s(%s)" % (fn, ", ".join(a.text for a in args)))
+        return Exp.mk(self.ctype, "%s(%s)" % (fn, ", ".join(["%s"] * len(args))), *args)
 
     # -- Num
     def __add__(self, o): return self._bin(o, "+")
@@ -91,7 +116,7 @@ class Exp(object):
     def __rsub__(self, o): return self._rbin(o, "-")
     def __mul__(self, o): return self._bin(o, "*")
     def __rmul__(self, o): return self._rbin(o, "*")
-    def __neg__(self): return Exp(self.ctype, "((%s)(-%s))" % (self.ctype, self.text))
+    def __neg__(self): return Exp.mk(self.ctype, "((%s)(-%%s))" % self.ctype, self)
 
     # -- Fractional / Integral: `/` is fdiv on floating types and Haskell's `div` (towards -inf) on integers
     def __truediv__(self, o):
@@ -107,9 +132,9 @@ class Exp(object):
     def __and__(self, o): return self._bin(o, "&")
     def __or__(self, o): return self._bin(o, "|")
     def __xor__(self, o): return self._bin(o, "^")
-    def __invert__(self): return Exp(self.ctype, "((%s)(~%s))" % (self.ctype, self.text))
-    def __lshift__(self, o): return Exp(self.ctype, "acc_shift_l(%s, (Int64)%s)" % (self.text, Exp.of(o, "Int64").text))
-    def __rshift__(self, o): return Exp(self.ctype, "acc_shift_r(%s, (Int64)%s)" % (self.text, Exp.of(o, "Int64").text))
+    def __invert__(self): return Exp.mk(self.ctype, "((%s)(~%%s))" % self.ctype, self)
+    def __lshift__(self, o): return Exp.mk(self.ctype, "acc_shift_l(%s, (Int64)%s)", self, Exp.of(o, "Int64"))
+    def __rshift__(self, o): return Exp.mk(self.ctype, "acc_shift_r(%s, (Int64)%s)", self, Exp.of(o, "Int64"))
 
     # -- Eq / Ord: Bool is Word8 (CodeGen/Type.hs:139)
     def __lt__(self, o): return self._bin(o, "<", "Word8")
@@ -120,7 +145,7 @@ class Exp(object):
     def ne(self, o): return self._bin(o, "!=", "Word8")
     def land(self, o): return self._bin(o, "&&", "Word8")
     def lor(self, o): return self._bin(o, "||", "Word8")
-    def lnot(self): return Exp("Word8", "((Word8)(!%s))" % self.text)
+    def lnot(self): return Exp.mk("Word8", "((Word8)(!%s))", self)
 
     def __bool__(self):
         raise TypeError("an Exp has no truth value on the host: use cond(p, t, e)")
@@ -183,14 +208,43 @@ def cond(p, t, e):
         raise TypeError("branches of cond differ in type")
     if isinstance(t.ctype, tuple):
         return lift(*[cond(p, a, b) for a, b in zip(t.comps, e.comps)])
-    return Exp(t.ctype, "(%s ? %s : %s)" % (Exp.of(p).text, t.text, e.text))
+    return Exp.mk(t.ctype, "(%s ? %s : %s)", Exp.of(p), t, e)
 
 
-def fromIntegral(e, to): return Exp(to, "acc_from_integral<%s>(%s)" % (to, e.text))
-def truncate(e, to): return Exp(to, "acc_truncate<%s>(%s)" % (to, e.text))
-def round_(e, to): return Exp(to, "acc_round<%s>(%s)" % (to, e.text))
-def floor(e, to): return Exp(to, "acc_floor<%s>(%s)" % (to, e.text))
-def ceiling(e, to): return Exp(to, "acc_ceiling<%s>(%s)" % (to, e.text))
+_FRESH = [0]
+
+
+def while_(p, f, init):
+    """iterate `f` from `init` while `p` holds (the scalar `While` of the expression language,
+    CodeGen.hs:338-821): a loop statement ahead of the expression that uses its result.  Of a tuple,
+    every component is a loop variable."""
+    init = Exp.of(init)
+    _FRESH[0] += 1
+    tup = isinstance(init.ctype, tuple)
+    types = list(init.ctype) if tup else [init.ctype]
+    names = ["w%d_%d" % (_FRESH[0], k) for k in range(len(types))]
+    inits = init.comps if tup else [init]
+    var = lift(*[Exp(t, n) for t, n in zip(types, names)]) if tup else Exp(types[0], names[0])
+    nxt = Exp.of(f(var), init.ctype)
+    if nxt.ctype != init.ctype:
+        raise TypeError("the body of while_ changes the type of its state: %s to %s" % (init.ctype, nxt.ctype))
+    nxts = nxt.comps if tup else [nxt]
+    # statements of the condition and of the body belong inside the loop: their closed forms are used there
+    decl = " ".join("%s %s = %s;" % (t, n, e.term) for t, n, e in zip(types, names, inits))
+    step = " ".join("const %s n%s = %s;" % (t, n, e.text) for t, n, e in zip(types, names, nxts))
+    copy = " ".join("%s = n%s;" % (n, n) for n in names)
+    loop = "%s while (%s) { %s %s }" % (decl, Exp.of(p(var)).text, step, copy)
+    binds = _merge(inits) + (loop,)
+    if tup:
+        return Exp(init.ctype, comps=[Exp(t, n, binds=binds) for t, n in zip(types, names)])
+    return Exp(types[0], names[0], binds=binds)
+
+
+def fromIntegral(e, to): return Exp.mk(to, "acc_from_integral<%s>(%%s)" % to, e)
+def truncate(e, to): return Exp.mk(to, "acc_truncate<%s>(%%s)" % to, e)
+def round_(e, to): return Exp.mk(to, "acc_round<%s>(%%s)" % to, e)
+def floor(e, to): return Exp.mk(to, "acc_floor<%s>(%%s)" % to, e)
+def ceiling(e, to): return Exp.mk(to, "acc_ceiling<%s>(%%s)" % to, e)
 def idiv(a, b): return Exp.of(a)._call("acc_idiv", b)
 def mod(a, b): return Exp.of(a)._call("acc_imod", b)
 def quot(a, b): return Exp.of(a)._call("acc_quot", b)
@@ -234,10 +288,10 @@ class Acc(object):
             tag = _tag(self.manifest)
             if isinstance(self.ctype, tuple):
                 n = len(self.ctype)
-                return Exp(self.ctype, comps=[Exp(t, "%s_%d[%s]" % (tag, n - 1 - i, ix.text)) for i, t in enumerate(self.ctype)])
-            if ix.text == "ix":
+                return Exp(self.ctype, comps=[Exp.mk(t, "%s_%d[%%s]" % (tag, n - 1 - i), ix) for i, t in enumerate(self.ctype)])
+            if ix.term == "ix":
                 return Exp(self.ctype, "acc_stream(%s_0, ix)" % tag)
-            return Exp(self.ctype, "%s_0[%s]" % (tag, ix.text))
+            return Exp.mk(self.ctype, "%s_0[%%s]" % tag, ix)
         return self.at(ix)
 
     def stream(self):
@@ -341,8 +395,8 @@ def _unlinear(ix, shape):
         if d == 0:
             out.append(rest)
         else:
-            out.append(Exp("Int64", "(%s %% %s)" % (rest.text, ext.text)))
-            rest = Exp("Int64", "(%s / %s)" % (rest.text, ext.text))
+            out.append(Exp.mk("Int64", "(%s %% %s)", rest, ext))
+            rest = Exp.mk("Int64", "(%s / %s)", rest, ext)
     return tuple(reversed(out))
 
 
@@ -531,7 +585,7 @@ def permute(f, defaults, p, a, context=None):
     if isinstance(t, str) and t == ignore:
         perm_text = "ACC_IGNORE"
     elif isinstance(t, _Maybe):
-        perm_text = "(%s ? %s : ACC_IGNORE)" % (t.p.text, _linear(t.idx, dfl.shape).text)
+        perm_text = Exp.mk("Int64", "(%s ? %s : ACC_IGNORE)", t.p, _linear(t.idx, dfl.shape)).text
     else:
         perm_text = _linear(t, dfl.shape).text
     arrays, sig, fr = _assemble(get=a.stream().text, combine=_combine(f, a.ctype).text, permutation=perm_text)

@@ -89,3 +89,21 @@ def test_index_arithmetic_of_the_delayed_combinators():
         acc.zipWith(add, m, use((3, 5), np.float32))
     with pytest.raises(TypeError):
         acc._combine(lambda x, y: x < y, "Int32")
+
+
+def test_while_is_a_statement_ahead_of_the_expression_and_compiles():
+    xs = use((64,), np.int64)
+    r = acc.map(lambda v: acc.while_(lambda k: (k + 1) * (k + 1) <= v, lambda k: k + 1, acc.constant(0, "Int64")) + 1, xs)
+    e = r.stream()
+    assert len(e.binds) == 1 and " while (" in e.binds[0] and e.text.startswith("[&] { Int64 w")
+    arrays, sig, fr = acc._assemble(get=e.text)
+    assert A.compile_only(A.make_desc(A.SKEL_MAP, "Int64", env=sig, out_rank=1, **fr)) > 0
+    # the same loop used twice is emitted once
+    twice = acc.map(lambda v: (lambda s: s * s)(acc.while_(lambda k: k < v, lambda k: k + 2, acc.constant(0, "Int64"))), xs).stream()
+    assert len(twice.binds) == 1
+    # a tuple state: every component is a loop variable, components picked afterwards share the loop
+    t = acc.while_(lambda s: s.comps[1] < 10, lambda s: (s.comps[0] * 2, s.comps[1] + 1), acc.lift(acc.constant(1, "Int64"), acc.constant(0, "Int64")))
+    both = t.comps[0] + t.comps[1]
+    assert len(both.binds) == 1
+    with pytest.raises(TypeError):
+        acc.while_(lambda k: k < 3, lambda k: acc.fromIntegral(k, "Int32"), acc.constant(0, "Int64"))

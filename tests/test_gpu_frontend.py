@@ -200,3 +200,52 @@ def test_type_errors_are_reported_before_anything_is_compiled(acc):
         acc.scanl(add, 0, acc.use(np.zeros((2, 2), dtype=np.int32)))
     with pytest.raises(TypeError):
         acc.map(lambda v: 1 if v > 0 else 0, xs)
+
+
+def test_scalar_while_mandelbrot_and_collatz(acc):
+    # Mandelbrot escape counts (accelerate-examples' mandelbrot): state (zr, zi, i) iterated per element
+    h, w, limit = 96, 128, 64
+    f32 = lambda v: acc.constant(v, "float")
+
+    def pixel(y, x):
+        cr = acc.fromIntegral(x, "float") * f32(3.0 / w) - f32(2.25)
+        ci = acc.fromIntegral(y, "float") * f32(2.5 / h) - f32(1.25)
+
+        def inside(s):
+            zr, zi, i = s.comps
+            return (zr * zr + zi * zi <= f32(4.0)).land(i < limit)
+
+        def step(s):
+            zr, zi, i = s.comps
+            return (zr * zr - zi * zi + cr, f32(2.0) * zr * zi + ci, i + 1)
+        return acc.while_(inside, step, acc.lift(f32(0.0), f32(0.0), acc.constant(0, "Int32"))).comps[2]
+    counts = acc.run(acc.generate((h, w), pixel))
+    yy, xx = np.meshgrid(np.arange(h), np.arange(w), indexing="ij")
+    cr = xx.astype(np.float32) * np.float32(3.0 / w) - np.float32(2.25)
+    ci = yy.astype(np.float32) * np.float32(2.5 / h) - np.float32(1.25)
+    zr, zi, it = np.zeros_like(cr), np.zeros_like(cr), np.zeros((h, w), np.int32)
+    for _ in range(limit):
+        live = (zr * zr + zi * zi <= np.float32(4.0)) & (it < limit)
+        nzr = zr * zr - zi * zi + cr
+        nzi = np.float32(2.0) * zr * zi + ci
+        zr, zi, it = np.where(live, nzr, zr), np.where(live, nzi, zi), np.where(live, it + 1, it)
+    assert np.array_equal(counts, it) and 0 < it.min() < it.max() == limit
+    # Collatz steps: a scalar loop state, the loop inside a fold's producer
+    n = np.arange(1, 5001, dtype=np.int64)
+
+    def steps(v):
+        s = acc.while_(lambda t: t.comps[0] > 1,
+                       lambda t: (acc.cond((t.comps[0] & 1).eq(0), t.comps[0] // 2, 3 * t.comps[0] + 1), t.comps[1] + 1),
+                       acc.lift(v, acc.constant(0, "Int64")))
+        return s.comps[1]
+    ref = []
+    for v in n:
+        c = 0
+        while v > 1:
+            v, c = (v // 2 if v % 2 == 0 else 3 * v + 1), c + 1
+        ref.append(c)
+    assert np.array_equal(acc.run(acc.map(steps, acc.use(n))), np.array(ref, dtype=np.int64))
+    assert int(acc.run(acc.fold1(acc.max_, acc.map(steps, acc.use(n))))) == max(ref)
+    # a loop whose state is one scalar: integer square root by counting
+    r = acc.run(acc.map(lambda v: acc.while_(lambda k: (k + 1) * (k + 1) <= v, lambda k: k + 1, acc.constant(0, "Int64")), acc.use(n)))
+    assert np.array_equal(r, np.floor(np.sqrt(n)).astype(np.int64))
