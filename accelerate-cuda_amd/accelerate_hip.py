@@ -335,12 +335,46 @@ def _assemble(**fragments):
     return arrays, sig, out
 
 
+class _Resident(object):
+    """A manifest array under the context's memory table: host storage (the array `use`d, or the place a result is
+    written back to when the device is full) and the table entry keyed by it.  The device address is only known
+    between acquire and release, which bracket every launch (Context.launch)."""
+
+    def __init__(self, cx, host, frozen):
+        self.cx, self.host, self.shape, self.dtype, self.size = cx, host, host.shape, host.dtype, host.size
+        self.key = A.MemTable.key(host)
+        cx.table.malloc(host, frozen)
+        cx.live[self.key] = cx.live.get(self.key, 0) + 1
+
+    def get(self):
+        d = self.cx.table.acquire(self.host)
+        try:
+            return d.get()
+        finally:
+            self.cx.table.release(self.host)
+
+    def __del__(self):
+        try:
+            cx = self.cx
+            cx.live[self.key] -= 1
+            if cx.live[self.key] == 0:
+                del cx.live[self.key]
+                if cx.table.handle:
+                    cx.table.free(self.host)
+        except Exception:
+            pass
+
+
 class Context(object):
-    """a device context plus the table of skeleton instances built so far (the kernel table of State.hs:110-119)"""
+    """a device context, the table of skeleton instances built so far (the kernel table of State.hs:110-119) and the
+    memory table every manifest array lives in (State.hs:120-122): `budget_bytes` bounds the device memory held,
+    0 leaves that to the device"""
     _default = None
 
-    def __init__(self, device=0):
+    def __init__(self, device=0, budget_bytes=0):
         self.ctx = A.Context(device)
+        self.table = A.MemTable(self.ctx, budget_bytes)
+        self.live = {}
         self.skeletons = {}
 
     @classmethod
@@ -358,6 +392,24 @@ class Context(object):
             self.skeletons[key] = sk
         return sk
 
+    def launch(self, manifests, go):
+        """run `go` on the device views of `manifests` (None stays None), keeping them resident meanwhile"""
+        taken = []
+
+        def view(m):
+            if m is None:
+                return None
+            if isinstance(m, A.TupleArray):
+                return A.TupleArray([view(c) for c in m.comps])
+            d = self.table.acquire(m.host)
+            taken.append(m)
+            return d
+        try:
+            return go([view(m) for m in manifests])
+        finally:
+            for m in taken:
+                self.table.release(m.host)
+
 
 def _elt(ctype):
     return ", ".join(ctype) if isinstance(ctype, tuple) else ctype
@@ -368,19 +420,22 @@ def _dtype(ctype):
 
 
 def _empty(cx, shape, ctype):
+    """device memory for a result; its host side is untouched pages until the result is evicted or read"""
     if isinstance(ctype, tuple):
-        return cx.ctx.empty_tuple(shape, _dtype(ctype))
-    return cx.ctx.empty(shape, _dtype(ctype))
+        return A.TupleArray([_Resident(cx, np.empty(shape, dtype=t), False) for t in _dtype(ctype)])
+    return _Resident(cx, np.empty(shape, dtype=_dtype(ctype)), False)
 
 
 def use(host, context=None):
-    """a host array (or a tuple of equally shaped host arrays: an array of tuples) made available on the device"""
+    """a host array (or a tuple of equally shaped host arrays: an array of tuples) made available on the device.
+    It is uploaded when first wanted there and once only, however often it is `use`d (Array/Prim.hs:177-192); it must
+    not be changed afterwards."""
     cx = context or Context.default()
     if isinstance(host, tuple):
         hs = [np.ascontiguousarray(h) for h in host]
-        return Acc(hs[0].shape, tuple(CTYPE[h.dtype.type] for h in hs), manifest=cx.ctx.tuple_array(*hs))
+        return Acc(hs[0].shape, tuple(CTYPE[h.dtype.type] for h in hs), manifest=A.TupleArray([_Resident(cx, h, True) for h in hs]))
     host = np.ascontiguousarray(host)
-    return Acc(host.shape, CTYPE[host.dtype.type], manifest=cx.ctx.array(host))
+    return Acc(host.shape, CTYPE[host.dtype.type], manifest=_Resident(cx, host, True))
 
 
 def unit(value, ctype, context=None):
@@ -479,7 +534,7 @@ def _force(a, cx):
     arrays, sig, fr = _assemble(get=a.stream().text)
     sk = cx.skeleton(A.SKEL_MAP, _elt(a.ctype), sig, out_rank=len(a.shape), **fr)
     out = _empty(cx, a.shape, a.ctype)
-    sk.map(arrays, out)
+    cx.launch(arrays + [out], lambda v: sk.map(v[:-1], v[-1]))
     return Acc(a.shape, a.ctype, manifest=out)
 
 
@@ -497,7 +552,7 @@ def _fold(f, z, a, seedless, context):
                                 seed=None if seedless else Exp.of(z, a.ctype).text)
     sk = cx.skeleton(A.SKEL_FOLD1 if seedless else A.SKEL_FOLD, _elt(a.ctype), sig, out_rank=len(out_shape), **fr)
     out = _empty(cx, out_shape, a.ctype)
-    sk.fold(arrays, a.shape, out)
+    cx.launch(arrays + [out], lambda v: sk.fold(v[:-1], a.shape, v[-1]))
     return Acc(out_shape, a.ctype, manifest=out)
 
 
@@ -519,7 +574,7 @@ def foldSeg(f, z, a, seg_lengths, context=None):
     sk = cx.skeleton(A.SKEL_FOLDSEG, _elt(a.ctype), sig, seg_type=seg_lengths.ctype, **fr)
     nseg = seg_lengths.shape[0]
     out = _empty(cx, (nseg,), a.ctype)
-    sk.foldseg(arrays, a.size, offs.manifest, out)
+    cx.launch(arrays + [offs.manifest, out], lambda v: sk.foldseg(v[:-2], a.size, v[-2], v[-1]))
     return Acc((nseg,), a.ctype, manifest=out)
 
 
@@ -534,7 +589,7 @@ def _scan(kind, f, z, a, context):
     m = n + 1 if kind in ("scanl", "scanr") else n
     out = _empty(cx, (m,), a.ctype)
     total = _empty(cx, (), a.ctype) if kind.endswith("'") else None
-    sk.scan(arrays, n, out, total)
+    cx.launch(arrays + [out, total], lambda v: sk.scan(v[:-2], n, v[-2], v[-1]))
     res = Acc((m,), a.ctype, manifest=out)
     return (res, Acc((), a.ctype, manifest=total)) if total is not None else res
 
@@ -591,7 +646,7 @@ def permute(f, defaults, p, a, context=None):
     arrays, sig, fr = _assemble(get=a.stream().text, combine=_combine(f, a.ctype).text, permutation=perm_text)
     sk = cx.skeleton(A.SKEL_PERMUTE, _elt(a.ctype), sig, out_rank=len(dfl.shape), combine_hint=_hint(f, a.ctype), **fr)
     out = _empty(cx, dfl.shape, a.ctype)
-    sk.permute(arrays, a.size, dfl.manifest, out)
+    cx.launch(arrays + [dfl.manifest, out], lambda v: sk.permute(v[:-2], a.size, v[-2], v[-1]))
     return Acc(dfl.shape, a.ctype, manifest=out)
 
 
@@ -621,7 +676,7 @@ def stencil(pattern, f, boundary, a, context=None, constant_value=None):
                      boundary_constant=None if constant_value is None else _literal(constant_value, src.ctype),
                      stencil_in=src.ctype, **fr)
     out = _empty(cx, src.shape, res.ctype)
-    sk.stencil(arrays, src.manifest, out)
+    cx.launch(arrays + [src.manifest, out], lambda v: sk.stencil(v[:-2], v[-2], v[-1]))
     return Acc(src.shape, res.ctype, manifest=out)
 
 
@@ -639,7 +694,7 @@ def stencil2(pattern1, pattern2, f, boundary1, a, boundary2, b, context=None, co
                      stencil_in=s1.ctype, stencil_in2=s2.ctype, **fr)
     shape = _meet(s1.shape, s2.shape)
     out = _empty(cx, shape, res.ctype)
-    sk.stencil2(arrays, s1.manifest, s2.manifest, out)
+    cx.launch(arrays + [s1.manifest, s2.manifest, out], lambda v: sk.stencil2(v[:-3], v[-3], v[-2], v[-1]))
     return Acc(shape, res.ctype, manifest=out)
 
 

@@ -80,6 +80,12 @@ class acc_skel_info(C.Structure):
 
 
 # every symbol include/acc_hip.h declares (tests check that all are exported)
+class acc_memtable_stats(C.Structure):
+    _fields_ = [(n, C.c_uint64) for n in ("resident_bytes", "nursery_bytes", "arrays", "resident_arrays", "device_allocs",
+                                          "nursery_hits", "uploads", "upload_bytes", "evictions", "writebacks",
+                                          "writeback_bytes")]
+
+
 SYMBOLS = """acc_last_error acc_version acc_init acc_device_count acc_device_get_props acc_context_create
 acc_context_destroy acc_context_device acc_context_sync acc_malloc acc_free acc_mem_info acc_host_alloc
 acc_host_free acc_memcpy_h2d acc_memcpy_d2h acc_memcpy_d2d acc_memcpy_h2d_async acc_memcpy_d2h_async
@@ -89,7 +95,9 @@ acc_event_elapsed_ms acc_compile acc_compile_log acc_cache_set_dir acc_cache_dir
 acc_cache_clear acc_module_load acc_module_unload acc_module_get_function acc_function_attr acc_occupancy
 acc_launch acc_launch_grid acc_skel_create acc_skel_destroy acc_skel_source acc_skel_preview acc_skel_compile_only
 acc_skel_get_info acc_exec_map acc_exec_fold acc_exec_foldseg acc_exec_scan acc_exec_permute
-acc_exec_stencil acc_exec_stencil2 acc_exec_stencil_iterate""".split()
+acc_exec_stencil acc_exec_stencil2 acc_exec_stencil_iterate acc_memtable_create acc_memtable_destroy
+acc_memtable_malloc acc_memtable_acquire acc_memtable_release acc_memtable_free acc_memtable_insert_unmanaged
+acc_memtable_reclaim acc_memtable_get_stats""".split()
 
 
 def build(force=False):
@@ -150,6 +158,15 @@ def lib():
         L.acc_exec_stencil.argtypes = [C.c_void_p, AP, AP, AP, C.c_void_p]
         L.acc_exec_stencil2.argtypes = [C.c_void_p, AP, AP, AP, AP, C.c_void_p]
         L.acc_exec_stencil_iterate.argtypes = [C.c_void_p, AP, AP, AP, C.c_int32, C.c_void_p, C.POINTER(C.c_int32)]
+        L.acc_memtable_create.argtypes = [C.c_void_p, C.c_uint64, C.POINTER(C.c_void_p)]
+        L.acc_memtable_destroy.argtypes = [C.c_void_p]
+        L.acc_memtable_malloc.argtypes = [C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint64, C.c_int, C.POINTER(C.c_int)]
+        L.acc_memtable_acquire.argtypes = [C.c_void_p, C.c_uint64, C.c_void_p, C.POINTER(C.c_uint64)]
+        L.acc_memtable_release.argtypes = [C.c_void_p, C.c_uint64, C.c_void_p]
+        L.acc_memtable_free.argtypes = [C.c_void_p, C.c_uint64]
+        L.acc_memtable_insert_unmanaged.argtypes = [C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint64]
+        L.acc_memtable_reclaim.argtypes = [C.c_void_p]
+        L.acc_memtable_get_stats.argtypes = [C.c_void_p, C.POINTER(acc_memtable_stats)]
         _lib = L
     return _lib
 
@@ -368,6 +385,57 @@ class Context(object):
     def close(self):
         if self.handle:
             lib().acc_context_destroy(self.handle)
+            self.handle = None
+
+
+class MemTable(object):
+    """acc_memtable: host numpy arrays (identified by the address of their storage) and their device copies."""
+
+    def __init__(self, ctx, budget_bytes=0):
+        self.ctx, self.hosts = ctx, {}
+        h = C.c_void_p()
+        check(lib().acc_memtable_create(ctx.handle, budget_bytes, C.byref(h)))
+        self.handle = h
+
+    @staticmethod
+    def key(host):
+        """address and length of the storage (a slice that starts where its parent starts is another array)"""
+        return (host.ctypes.data ^ (host.nbytes * 0x9E3779B97F4A7C15)) & 0xFFFFFFFFFFFFFFFF
+
+    def malloc(self, host, frozen):
+        """enter a C-contiguous host array; returns True if it was not in the table yet"""
+        assert host.flags.c_contiguous
+        new = C.c_int()
+        check(lib().acc_memtable_malloc(self.handle, self.key(host), host.ctypes.data, host.nbytes, int(frozen), C.byref(new)))
+        self.hosts[self.key(host)] = host           # the table reads and writes this storage later
+        return bool(new.value)
+
+    def acquire(self, host, stream=None):
+        p = C.c_uint64()
+        check(lib().acc_memtable_acquire(self.handle, self.key(host), stream, C.byref(p)))
+        return DeviceArray(self.ctx, host.shape, host.dtype, ptr=p.value, owner=False)
+
+    def release(self, host, stream=None):
+        check(lib().acc_memtable_release(self.handle, self.key(host), stream))
+
+    def free(self, host):
+        check(lib().acc_memtable_free(self.handle, self.key(host)))
+        self.hosts.pop(self.key(host), None)
+
+    def insert_unmanaged(self, host, dev):
+        check(lib().acc_memtable_insert_unmanaged(self.handle, self.key(host), dev.ptr, host.nbytes))
+
+    def reclaim(self):
+        check(lib().acc_memtable_reclaim(self.handle))
+
+    def stats(self):
+        st = acc_memtable_stats()
+        check(lib().acc_memtable_get_stats(self.handle, C.byref(st)))
+        return {n: getattr(st, n) for n, _ in acc_memtable_stats._fields_}
+
+    def destroy(self):
+        if self.handle:
+            check(lib().acc_memtable_destroy(self.handle))
             self.handle = None
 
 

@@ -1,0 +1,328 @@
+// Memory table: host array identity -> device block, a nursery of freed blocks
+// keyed by size, and least-recently-used eviction (write-back to the host copy
+// unless that copy is authoritative).  One table belongs to one context, hence
+// one device; every entry point takes the table's lock.
+#include <algorithm>
+#include <unordered_map>
+
+#include "acc_internal.hpp"
+
+using namespace acc;
+
+namespace {
+
+enum Status {
+  CLEAN,      // device == host
+  DIRTY,      // device holds the only current copy
+  EVICTED,    // host holds the only copy; no device block
+  PENDING,    // frozen, not uploaded yet; device block may or may not exist
+  UNMANAGED   // the caller's device memory
+};
+
+struct Entry {
+  void *host = nullptr;
+  uint64_t bytes = 0, rounded = 0;
+  void *dev = nullptr;
+  Status status = CLEAN;
+  bool frozen = false;
+  int pins = 0;
+  uint64_t tick = 0;           // last acquire
+  hipEvent_t last_use = nullptr;
+  bool recorded = false;
+};
+
+uint64_t round_up(uint64_t bytes)
+{
+  uint64_t b = bytes ? bytes : 1;
+  return (b + ACC_MEMTABLE_GRANULE - 1) / ACC_MEMTABLE_GRANULE * ACC_MEMTABLE_GRANULE;
+}
+
+}  // namespace
+
+struct acc_memtable_s {
+  acc_context ctx = nullptr;
+  uint64_t budget = 0;
+  std::mutex mu;
+  std::unordered_map<uint64_t, Entry> table;
+  std::multimap<uint64_t, void *> nursery;     // rounded size -> free block
+  uint64_t clock = 0;
+  acc_memtable_stats st{};
+
+  uint64_t held() const { return st.resident_bytes + st.nursery_bytes; }
+
+  int flush_nursery()
+  {
+    for (auto &kv : nursery) ACC_HIP_TRY(hipFree(kv.second));
+    nursery.clear();
+    st.nursery_bytes = 0;
+    return ACC_OK;
+  }
+
+  // work recorded at the entry's last release has finished?
+  static bool idle(Entry &e)
+  {
+    if (!e.recorded) return true;
+    if (hipEventQuery(e.last_use) == hipSuccess) { e.recorded = false; return true; }
+    (void)hipGetLastError();   // hipErrorNotReady is not a failure
+    return false;
+  }
+
+  // give up the device block of `e`: write back what only the device has, then
+  // hand the block to the nursery (keep == true) or to the device
+  int drop(Entry &e, bool keep)
+  {
+    if (e.recorded) { ACC_HIP_TRY(hipEventSynchronize(e.last_use)); e.recorded = false; }
+    if (e.status == DIRTY) {
+      ACC_HIP_TRY(hipMemcpy(e.host, e.dev, e.bytes, hipMemcpyDeviceToHost));
+      st.writebacks++;
+      st.writeback_bytes += e.bytes;
+    }
+    st.resident_bytes -= e.rounded;
+    st.resident_arrays--;
+    if (keep) {
+      nursery.emplace(e.rounded, e.dev);
+      st.nursery_bytes += e.rounded;
+    } else {
+      ACC_HIP_TRY(hipFree(e.dev));
+    }
+    e.dev = nullptr;
+    return ACC_OK;
+  }
+
+  // least recently used entry that may leave the device; nullptr if none.
+  // Entries whose last use is still running are taken only when nothing idle is left.
+  Entry *victim()
+  {
+    Entry *best = nullptr, *busy = nullptr;
+    for (auto &kv : table) {
+      Entry &e = kv.second;
+      if (!e.dev || e.pins > 0 || e.status == UNMANAGED) continue;
+      Entry *&slot = idle(e) ? best : busy;
+      if (!slot || e.tick < slot->tick) slot = &e;
+    }
+    return best ? best : busy;
+  }
+
+  int evict_one(bool *any)
+  {
+    Entry *v = victim();
+    *any = v != nullptr;
+    if (!v) return ACC_OK;
+    Status after = (v->status == PENDING) ? PENDING : EVICTED;
+    ACC_TRY(drop(*v, false));
+    v->status = after;
+    st.evictions++;
+    return ACC_OK;
+  }
+
+  // a device block of `rounded` bytes: nursery, else the device; makes room first
+  // when a budget says so and afterwards when the device says so
+  int block(uint64_t rounded, void **out)
+  {
+    auto it = nursery.find(rounded);
+    if (it != nursery.end()) {
+      *out = it->second;
+      nursery.erase(it);
+      st.nursery_bytes -= rounded;
+      st.nursery_hits++;
+      return ACC_OK;
+    }
+    if (budget && rounded > budget)
+      return fail(ACC_ERR_OOM, "acc_memtable: an array of %llu bytes exceeds the table's budget of %llu",
+                  (unsigned long long)rounded, (unsigned long long)budget);
+    for (;;) {
+      bool over = budget && held() + rounded > budget;
+      if (!over) {
+        void *p = nullptr;
+        hipError_t e = hipMalloc(&p, rounded);
+        if (e == hipSuccess) { *out = p; st.device_allocs++; return ACC_OK; }
+        (void)hipGetLastError();
+        if (e != hipErrorOutOfMemory) return fail_hip(e, "hipMalloc");
+      }
+      if (!nursery.empty()) { ACC_TRY(flush_nursery()); continue; }
+      bool any = false;
+      ACC_TRY(evict_one(&any));
+      if (!any)
+        return fail(ACC_ERR_OOM, "acc_memtable: %llu bytes do not fit and every resident array is in use "
+                    "(%llu bytes resident%s)", (unsigned long long)rounded, (unsigned long long)st.resident_bytes,
+                    budget ? ", budget reached" : "");
+    }
+  }
+};
+
+extern "C" {
+
+int acc_memtable_create(acc_context ctx, uint64_t budget_bytes, acc_memtable *out)
+{
+  if (!ctx || !out) return fail(ACC_ERR_INVALID, "acc_memtable_create: NULL argument");
+  *out = nullptr;
+  ACC_TRY(ctx->make_current());
+  acc_memtable mt = new acc_memtable_s();
+  mt->ctx = ctx;
+  mt->budget = budget_bytes;
+  *out = mt;
+  return ACC_OK;
+}
+
+int acc_memtable_destroy(acc_memtable mt)
+{
+  if (!mt) return ACC_OK;
+  int rc = ACC_OK;
+  {
+    std::lock_guard<std::mutex> lock(mt->mu);
+    rc = mt->ctx->make_current();
+    if (rc == ACC_OK) {
+      for (auto &kv : mt->table) {
+        Entry &e = kv.second;
+        if (e.recorded) (void)hipEventSynchronize(e.last_use);
+        if (e.last_use) (void)hipEventDestroy(e.last_use);
+        if (e.dev && e.status != UNMANAGED) (void)hipFree(e.dev);
+      }
+      for (auto &kv : mt->nursery) (void)hipFree(kv.second);
+    }
+  }
+  delete mt;
+  return rc;
+}
+
+int acc_memtable_malloc(acc_memtable mt, uint64_t key, void *host, uint64_t bytes, int frozen, int *is_new)
+{
+  if (!mt) return fail(ACC_ERR_INVALID, "acc_memtable_malloc: NULL table");
+  if (!host && bytes) return fail(ACC_ERR_INVALID, "acc_memtable_malloc: an array needs host storage to be evicted to");
+  std::lock_guard<std::mutex> lock(mt->mu);
+  ACC_TRY(mt->ctx->make_current());
+  auto it = mt->table.find(key);
+  if (it != mt->table.end()) {
+    if (it->second.bytes != bytes)
+      return fail(ACC_ERR_INVALID, "acc_memtable_malloc: key %llx is in the table with %llu bytes, not %llu",
+                  (unsigned long long)key, (unsigned long long)it->second.bytes, (unsigned long long)bytes);
+    if (is_new) *is_new = 0;
+    return ACC_OK;
+  }
+  Entry e;
+  e.host = host;
+  e.bytes = bytes;
+  e.rounded = round_up(bytes);
+  e.frozen = frozen != 0;
+  e.tick = ++mt->clock;
+  if (frozen) {
+    e.status = PENDING;       // the block is taken when the array is first wanted on the device
+  } else {
+    ACC_TRY(mt->block(e.rounded, &e.dev));
+    e.status = DIRTY;
+    mt->st.resident_bytes += e.rounded;
+    mt->st.resident_arrays++;
+  }
+  mt->table.emplace(key, e);
+  mt->st.arrays++;
+  if (is_new) *is_new = 1;
+  return ACC_OK;
+}
+
+int acc_memtable_acquire(acc_memtable mt, uint64_t key, acc_stream stream, acc_devptr *out)
+{
+  if (!mt || !out) return fail(ACC_ERR_INVALID, "acc_memtable_acquire: NULL argument");
+  *out = 0;
+  std::lock_guard<std::mutex> lock(mt->mu);
+  ACC_TRY(mt->ctx->make_current());
+  auto it = mt->table.find(key);
+  if (it == mt->table.end())
+    return fail(ACC_ERR_NOT_FOUND, "acc_memtable_acquire: key %llx is not in the table", (unsigned long long)key);
+  Entry &e = it->second;
+  if (e.status == EVICTED || e.status == PENDING) {
+    if (!e.dev) {
+      e.pins++;                               // never its own victim
+      int rc = mt->block(e.rounded, &e.dev);
+      e.pins--;
+      if (rc != ACC_OK) return rc;
+      mt->st.resident_bytes += e.rounded;
+      mt->st.resident_arrays++;
+    }
+    if (e.bytes) {
+      ACC_HIP_TRY(hipMemcpyAsync(e.dev, e.host, e.bytes, hipMemcpyHostToDevice, static_cast<hipStream_t>(stream)));
+      mt->st.uploads++;
+      mt->st.upload_bytes += e.bytes;
+    }
+    // what the device now holds is what the host holds; an array produced on the device is
+    // taken to be changed again by whoever acquires it
+    e.status = e.frozen ? CLEAN : DIRTY;
+  }
+  e.pins++;
+  e.tick = ++mt->clock;
+  *out = reinterpret_cast<acc_devptr>(e.dev);
+  return ACC_OK;
+}
+
+int acc_memtable_release(acc_memtable mt, uint64_t key, acc_stream stream)
+{
+  if (!mt) return fail(ACC_ERR_INVALID, "acc_memtable_release: NULL table");
+  std::lock_guard<std::mutex> lock(mt->mu);
+  ACC_TRY(mt->ctx->make_current());
+  auto it = mt->table.find(key);
+  if (it == mt->table.end())
+    return fail(ACC_ERR_NOT_FOUND, "acc_memtable_release: key %llx is not in the table", (unsigned long long)key);
+  Entry &e = it->second;
+  if (e.pins <= 0) return fail(ACC_ERR_INVALID, "acc_memtable_release: key %llx is not acquired", (unsigned long long)key);
+  if (e.status != UNMANAGED) {
+    if (!e.last_use) ACC_HIP_TRY(hipEventCreateWithFlags(&e.last_use, hipEventDisableTiming));
+    ACC_HIP_TRY(hipEventRecord(e.last_use, static_cast<hipStream_t>(stream)));
+    e.recorded = true;
+  }
+  e.pins--;
+  return ACC_OK;
+}
+
+int acc_memtable_free(acc_memtable mt, uint64_t key)
+{
+  if (!mt) return fail(ACC_ERR_INVALID, "acc_memtable_free: NULL table");
+  std::lock_guard<std::mutex> lock(mt->mu);
+  ACC_TRY(mt->ctx->make_current());
+  auto it = mt->table.find(key);
+  if (it == mt->table.end()) return ACC_OK;       // freeing twice is harmless (Array/Remote.hs:166-168)
+  Entry &e = it->second;
+  if (e.pins > 0) return fail(ACC_ERR_INVALID, "acc_memtable_free: key %llx is still acquired", (unsigned long long)key);
+  if (e.dev && e.status != UNMANAGED) {
+    e.status = CLEAN;                              // nobody will read it: nothing to write back
+    ACC_TRY(mt->drop(e, true));
+    if (mt->budget && mt->held() > mt->budget) ACC_TRY(mt->flush_nursery());
+  }
+  if (e.last_use) (void)hipEventDestroy(e.last_use);
+  mt->table.erase(it);
+  mt->st.arrays--;
+  return ACC_OK;
+}
+
+int acc_memtable_insert_unmanaged(acc_memtable mt, uint64_t key, acc_devptr p, uint64_t bytes)
+{
+  if (!mt || !p) return fail(ACC_ERR_INVALID, "acc_memtable_insert_unmanaged: NULL argument");
+  std::lock_guard<std::mutex> lock(mt->mu);
+  if (mt->table.count(key))
+    return fail(ACC_ERR_INVALID, "acc_memtable_insert_unmanaged: key %llx is already in the table", (unsigned long long)key);
+  Entry e;
+  e.bytes = bytes;
+  e.rounded = 0;                                   // not counted: the table does not hold it
+  e.dev = reinterpret_cast<void *>(p);
+  e.status = UNMANAGED;
+  e.tick = ++mt->clock;
+  mt->table.emplace(key, e);
+  mt->st.arrays++;
+  return ACC_OK;
+}
+
+int acc_memtable_reclaim(acc_memtable mt)
+{
+  if (!mt) return fail(ACC_ERR_INVALID, "acc_memtable_reclaim: NULL table");
+  std::lock_guard<std::mutex> lock(mt->mu);
+  ACC_TRY(mt->ctx->make_current());
+  return mt->flush_nursery();
+}
+
+int acc_memtable_get_stats(acc_memtable mt, acc_memtable_stats *out)
+{
+  if (!mt || !out) return fail(ACC_ERR_INVALID, "acc_memtable_get_stats: NULL argument");
+  std::lock_guard<std::mutex> lock(mt->mu);
+  *out = mt->st;
+  return ACC_OK;
+}
+
+}  // extern "C"

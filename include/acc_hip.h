@@ -375,6 +375,76 @@ int acc_exec_stencil2(acc_skel s, const acc_array *env, const acc_array *in1, co
 int acc_exec_stencil_iterate(acc_skel s, const acc_array *env, const acc_array *a, const acc_array *b,
                              int32_t iters, acc_stream stream, int32_t *result_in_b);
 
+/* =========================================================================
+ * C. memory table
+ * ========================================================================= */
+
+/* The association between host arrays and their device copies, with reuse of
+ * freed blocks and least-recently-used eviction when the device (or a budget)
+ * is full: the roles of Array/Remote.hs:111-196 and of the LRU table it takes
+ * from the `accelerate` base package (Data.Array.Accelerate.Array.Remote.LRU,
+ * accelerate-1.0; not part of the reference tree).
+ *
+ *   key     identity of the host array (the reference uses the StableName of
+ *           its ArrayData; the address of the host storage serves as well)
+ *   host    the host storage of `bytes` bytes: evicted data is written there
+ *           and read from there when the array is wanted again.  It must stay
+ *           valid until acc_memtable_free(key)
+ *   frozen  non-zero: the host copy is authoritative and already holds the
+ *           data (a `use`d array): it is uploaded when first acquired and
+ *           eviction drops the device copy without writing back.  Zero: the
+ *           array is produced on the device; eviction writes it back first
+ *
+ * Device blocks are rounded up to ACC_MEMTABLE_GRANULE bytes (the reference's
+ * remoteAllocationSize, Array/Remote.hs:80) and a freed block waits in a
+ * nursery for the next array of the same rounded size.  When an allocation
+ * does not fit, the nursery is returned to the device first; then arrays that
+ * are neither acquired nor still in use by work recorded at their last release
+ * are evicted, least recently used first.  ACC_ERR_OOM if that is not enough.  */
+typedef struct acc_memtable_s *acc_memtable;
+#define ACC_MEMTABLE_GRANULE 1024
+
+/* budget_bytes: upper bound on device bytes held by the table (arrays +
+ * nursery); 0 = bounded only by what the device gives (new, :103-106)        */
+int acc_memtable_create(acc_context ctx, uint64_t budget_bytes, acc_memtable *out);
+int acc_memtable_destroy(acc_memtable mt);          /* frees every managed block */
+
+/* malloc, Array/Remote.hs:141-155.  *is_new = 0 when the key is already in the
+ * table (nothing is allocated or uploaded again: an array `use`d twice is
+ * uploaded once, Array/Prim.hs:177-192)                                       */
+int acc_memtable_malloc(acc_memtable mt, uint64_t key, void *host, uint64_t bytes, int frozen, int *is_new);
+
+/* withRemote, Array/Remote.hs:113-135, as a bracket the caller closes: acquire
+ * returns the device pointer (allocating and uploading on `stream` first when
+ * the array was evicted or never uploaded) and keeps the array resident until
+ * the matching release; release names the stream the array was used on, and
+ * the array is not evicted before the work queued on that stream at that
+ * moment has completed.  Acquires nest.                                       */
+int acc_memtable_acquire(acc_memtable mt, uint64_t key, acc_stream stream, acc_devptr *out);
+int acc_memtable_release(acc_memtable mt, uint64_t key, acc_stream stream);
+
+/* free, Array/Remote.hs:160-170: the host array is gone.  The block goes to
+ * the nursery once work recorded at the last release has completed.          */
+int acc_memtable_free(acc_memtable mt, uint64_t key);
+
+/* insertUnmanaged, Array/Remote.hs:177-189: device memory the table did not
+ * allocate; it is never evicted, reused or freed by the table                */
+int acc_memtable_insert_unmanaged(acc_memtable mt, uint64_t key, acc_devptr p, uint64_t bytes);
+
+/* reclaim, Array/Remote.hs:195-196: return the nursery to the device         */
+int acc_memtable_reclaim(acc_memtable mt);
+
+typedef struct acc_memtable_stats {
+  uint64_t resident_bytes;     /* device bytes under live keys (rounded sizes) */
+  uint64_t nursery_bytes;
+  uint64_t arrays, resident_arrays;
+  uint64_t device_allocs;      /* hipMalloc calls */
+  uint64_t nursery_hits;       /* allocations served from the nursery */
+  uint64_t uploads, upload_bytes;
+  uint64_t evictions, writebacks, writeback_bytes;
+} acc_memtable_stats;
+int acc_memtable_get_stats(acc_memtable mt, acc_memtable_stats *out);
+
 #if defined(__GNUC__)
 #pragma GCC visibility pop
 #endif

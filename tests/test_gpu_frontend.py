@@ -249,3 +249,30 @@ def test_scalar_while_mandelbrot_and_collatz(acc):
     # a loop whose state is one scalar: integer square root by counting
     r = acc.run(acc.map(lambda v: acc.while_(lambda k: (k + 1) * (k + 1) <= v, lambda k: k + 1, acc.constant(0, "Int64")), acc.use(n)))
     assert np.array_equal(r, np.floor(np.sqrt(n)).astype(np.int64))
+
+
+def test_a_working_set_larger_than_the_memory_budget(acc):
+    """twelve 16 MiB arrays alive under a 64 MiB table: results leave the device for their host side and come back"""
+    cx = acc.Context(0, budget_bytes=64 << 20)
+    n = 4 << 20
+    rng = np.random.default_rng(10)
+    x = rng.integers(-100, 100, n).astype(np.int32)
+    xs = acc.use(x, cx)
+    assert acc.use(x, cx).manifest.key == xs.manifest.key                         # one entry, one upload
+    stages = [xs]
+    for k in range(1, 12):
+        prev = stages[-1]
+        stages.append(acc._force(acc.map(lambda v, k=k: v * 3 + k, prev), cx))   # each stage is a manifest array that stays alive
+    st = cx.table.stats()
+    assert st["arrays"] == 12 and st["resident_bytes"] <= 64 << 20 and st["evictions"] >= 8 and st["writebacks"] >= 7
+    assert st["uploads"] >= 1
+    ref = x.copy()
+    for k in range(1, 12):
+        ref = ref * 3 + k
+        assert np.array_equal(acc.run(stages[k], cx), ref), k                     # evicted stages are re-uploaded to be read
+    total = acc.run(acc.fold(add, 0, acc.zipWith(add, stages[1], stages[11]), context=cx), cx)
+    assert int(total) == pyref.wrap(int((x.astype(np.int64) * 3 + 1).sum() + ref.astype(np.int64).sum()), 32, True)
+    del stages, xs
+    import gc
+    gc.collect()
+    assert cx.table.stats()["arrays"] <= 2                                         # results die with their last reference
