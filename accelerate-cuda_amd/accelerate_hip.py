@@ -343,10 +343,13 @@ class _Resident(object):
     def __init__(self, cx, host, frozen):
         self.cx, self.host, self.shape, self.dtype, self.size = cx, host, host.shape, host.dtype, host.size
         self.key = A.MemTable.key(host)
+        self.stream, self.ready = None, None          # where it was produced, and the event recorded behind that
         cx.table.malloc(host, frozen)
         cx.live[self.key] = cx.live.get(self.key, 0) + 1
 
     def get(self):
+        if self.ready is not None:
+            A.check(A.lib().acc_event_sync(self.cx.ctx.handle, self.ready))
         d = self.cx.table.acquire(self.host)
         try:
             return d.get()
@@ -356,6 +359,8 @@ class _Resident(object):
     def __del__(self):
         try:
             cx = self.cx
+            if self.ready is not None:
+                cx.events.append(self.ready)
             cx.live[self.key] -= 1
             if cx.live[self.key] == 0:
                 del cx.live[self.key]
@@ -368,7 +373,10 @@ class _Resident(object):
 class Context(object):
     """a device context, the table of skeleton instances built so far (the kernel table of State.hs:110-119) and the
     memory table every manifest array lives in (State.hs:120-122): `budget_bytes` bounds the device memory held,
-    0 leaves that to the device"""
+    0 leaves that to the device.  Skeletons are launched asynchronously: a computation continues on the stream that
+    produced its first operand, one whose operands are all `use`d arrays takes the next stream of a small reservoir
+    (Execute/Stream.hs:66-74), and a stream waits for the events of operands produced on other streams
+    (Execute.hs:104-105,183-184), so independent subcomputations overlap and the host never waits before `run`."""
     _default = None
 
     def __init__(self, device=0, budget_bytes=0):
@@ -376,6 +384,7 @@ class Context(object):
         self.table = A.MemTable(self.ctx, budget_bytes)
         self.live = {}
         self.skeletons = {}
+        self.streams, self.turn, self.events = [], 0, []
 
     @classmethod
     def default(cls):
@@ -392,8 +401,32 @@ class Context(object):
             self.skeletons[key] = sk
         return sk
 
-    def launch(self, manifests, go):
-        """run `go` on the device views of `manifests` (None stays None), keeping them resident meanwhile"""
+    N_STREAMS = 4
+
+    def _stream_for(self, inputs):
+        for m in inputs:
+            if m.stream is not None:
+                return m.stream
+        if len(self.streams) < self.N_STREAMS:
+            self.streams.append(self.ctx.stream())
+        self.turn = (self.turn + 1) % len(self.streams)
+        return self.streams[self.turn]
+
+    def launch(self, inputs, outputs, go):
+        """run `go(input views, output views, stream)` with the arrays resident (None stays None), after what
+        produced the inputs; the outputs carry the event recorded behind it"""
+        def parts(ms):
+            for m in ms:
+                if isinstance(m, A.TupleArray):
+                    for c in m.comps:
+                        yield c
+                elif m is not None:
+                    yield m
+        stream = self._stream_for(list(parts(inputs)))
+        L = A.lib()
+        for m in parts(inputs):
+            if m.ready is not None and m.stream is not stream:
+                A.check(L.acc_stream_wait_event(self.ctx.handle, stream, m.ready))
         taken = []
 
         def view(m):
@@ -401,14 +434,19 @@ class Context(object):
                 return None
             if isinstance(m, A.TupleArray):
                 return A.TupleArray([view(c) for c in m.comps])
-            d = self.table.acquire(m.host)
+            d = self.table.acquire(m.host, stream)
             taken.append(m)
             return d
         try:
-            return go([view(m) for m in manifests])
+            go([view(m) for m in inputs], [view(m) for m in outputs], stream)
+            for m in parts(outputs):
+                if m.ready is None:
+                    m.ready = self.events.pop() if self.events else self.ctx.event(timing=False)
+                A.check(L.acc_event_record(self.ctx.handle, m.ready, stream))
+                m.stream = stream
         finally:
             for m in taken:
-                self.table.release(m.host)
+                self.table.release(m.host, stream)
 
 
 def _elt(ctype):
@@ -534,7 +572,7 @@ def _force(a, cx):
     arrays, sig, fr = _assemble(get=a.stream().text)
     sk = cx.skeleton(A.SKEL_MAP, _elt(a.ctype), sig, out_rank=len(a.shape), **fr)
     out = _empty(cx, a.shape, a.ctype)
-    cx.launch(arrays + [out], lambda v: sk.map(v[:-1], v[-1]))
+    cx.launch(arrays, [out], lambda i, o, s: sk.map(i, o[0], stream=s))
     return Acc(a.shape, a.ctype, manifest=out)
 
 
@@ -552,7 +590,7 @@ def _fold(f, z, a, seedless, context):
                                 seed=None if seedless else Exp.of(z, a.ctype).text)
     sk = cx.skeleton(A.SKEL_FOLD1 if seedless else A.SKEL_FOLD, _elt(a.ctype), sig, out_rank=len(out_shape), **fr)
     out = _empty(cx, out_shape, a.ctype)
-    cx.launch(arrays + [out], lambda v: sk.fold(v[:-1], a.shape, v[-1]))
+    cx.launch(arrays, [out], lambda i, o, s: sk.fold(i, a.shape, o[0], stream=s))
     return Acc(out_shape, a.ctype, manifest=out)
 
 
@@ -574,7 +612,7 @@ def foldSeg(f, z, a, seg_lengths, context=None):
     sk = cx.skeleton(A.SKEL_FOLDSEG, _elt(a.ctype), sig, seg_type=seg_lengths.ctype, **fr)
     nseg = seg_lengths.shape[0]
     out = _empty(cx, (nseg,), a.ctype)
-    cx.launch(arrays + [offs.manifest, out], lambda v: sk.foldseg(v[:-2], a.size, v[-2], v[-1]))
+    cx.launch(arrays + [offs.manifest], [out], lambda i, o, s: sk.foldseg(i[:-1], a.size, i[-1], o[0], stream=s))
     return Acc((nseg,), a.ctype, manifest=out)
 
 
@@ -589,7 +627,7 @@ def _scan(kind, f, z, a, context):
     m = n + 1 if kind in ("scanl", "scanr") else n
     out = _empty(cx, (m,), a.ctype)
     total = _empty(cx, (), a.ctype) if kind.endswith("'") else None
-    cx.launch(arrays + [out, total], lambda v: sk.scan(v[:-2], n, v[-2], v[-1]))
+    cx.launch(arrays, [out, total], lambda i, o, s: sk.scan(i, n, o[0], o[1], stream=s))
     res = Acc((m,), a.ctype, manifest=out)
     return (res, Acc((), a.ctype, manifest=total)) if total is not None else res
 
@@ -646,7 +684,7 @@ def permute(f, defaults, p, a, context=None):
     arrays, sig, fr = _assemble(get=a.stream().text, combine=_combine(f, a.ctype).text, permutation=perm_text)
     sk = cx.skeleton(A.SKEL_PERMUTE, _elt(a.ctype), sig, out_rank=len(dfl.shape), combine_hint=_hint(f, a.ctype), **fr)
     out = _empty(cx, dfl.shape, a.ctype)
-    cx.launch(arrays + [dfl.manifest, out], lambda v: sk.permute(v[:-2], a.size, v[-2], v[-1]))
+    cx.launch(arrays + [dfl.manifest], [out], lambda i, o, s: sk.permute(i[:-1], a.size, i[-1], o[0], stream=s))
     return Acc(dfl.shape, a.ctype, manifest=out)
 
 
@@ -676,7 +714,7 @@ def stencil(pattern, f, boundary, a, context=None, constant_value=None):
                      boundary_constant=None if constant_value is None else _literal(constant_value, src.ctype),
                      stencil_in=src.ctype, **fr)
     out = _empty(cx, src.shape, res.ctype)
-    cx.launch(arrays + [src.manifest, out], lambda v: sk.stencil(v[:-2], v[-2], v[-1]))
+    cx.launch(arrays + [src.manifest], [out], lambda i, o, s: sk.stencil(i[:-1], i[-1], o[0], stream=s))
     return Acc(src.shape, res.ctype, manifest=out)
 
 
@@ -694,7 +732,7 @@ def stencil2(pattern1, pattern2, f, boundary1, a, boundary2, b, context=None, co
                      stencil_in=s1.ctype, stencil_in2=s2.ctype, **fr)
     shape = _meet(s1.shape, s2.shape)
     out = _empty(cx, shape, res.ctype)
-    cx.launch(arrays + [s1.manifest, s2.manifest, out], lambda v: sk.stencil2(v[:-3], v[-3], v[-2], v[-1]))
+    cx.launch(arrays + [s1.manifest, s2.manifest], [out], lambda i, o, s: sk.stencil2(i[:-2], i[-2], i[-1], o[0], stream=s))
     return Acc(shape, res.ctype, manifest=out)
 
 

@@ -139,6 +139,7 @@ def lib():
         L.acc_event_destroy.argtypes = [C.c_void_p, C.c_void_p]
         L.acc_event_record.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
         L.acc_event_sync.argtypes = [C.c_void_p, C.c_void_p]
+        L.acc_stream_wait_event.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
         L.acc_event_elapsed_ms.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]
         L.acc_compile.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.POINTER(C.c_char_p), C.c_int,
                                   C.POINTER(C.c_void_p), C.POINTER(C.c_size_t)]

@@ -19,6 +19,12 @@ enum Status {
   UNMANAGED   // the caller's device memory
 };
 
+// the end of the work queued on one stream when an array was last released there
+struct Use {
+  hipStream_t stream = nullptr;
+  hipEvent_t done = nullptr;
+};
+
 struct Entry {
   void *host = nullptr;
   uint64_t bytes = 0, rounded = 0;
@@ -27,8 +33,15 @@ struct Entry {
   bool frozen = false;
   int pins = 0;
   uint64_t tick = 0;           // last acquire
-  hipEvent_t last_use = nullptr;
-  bool recorded = false;
+  std::vector<Use> uses;       // one per stream with work that may still touch the block
+  hipStream_t upload_stream = nullptr;
+  hipEvent_t uploaded = nullptr;   // set while the upload may still be running: other streams wait for it
+};
+
+// a block waiting for reuse, with the work that may still touch it
+struct FreeBlock {
+  void *dev = nullptr;
+  std::vector<Use> uses;
 };
 
 uint64_t round_up(uint64_t bytes)
@@ -44,34 +57,70 @@ struct acc_memtable_s {
   uint64_t budget = 0;
   std::mutex mu;
   std::unordered_map<uint64_t, Entry> table;
-  std::multimap<uint64_t, void *> nursery;     // rounded size -> free block
+  std::multimap<uint64_t, FreeBlock> nursery;  // rounded size -> free block
+  std::vector<hipEvent_t> spare_events;
   uint64_t clock = 0;
   acc_memtable_stats st{};
 
   uint64_t held() const { return st.resident_bytes + st.nursery_bytes; }
 
+  int event(hipEvent_t *out)
+  {
+    if (!spare_events.empty()) { *out = spare_events.back(); spare_events.pop_back(); return ACC_OK; }
+    ACC_HIP_TRY(hipEventCreateWithFlags(out, hipEventDisableTiming));
+    return ACC_OK;
+  }
+
+  // wait for everything in `uses`, which is emptied
+  int settle(std::vector<Use> &uses)
+  {
+    for (Use &u : uses) {
+      ACC_HIP_TRY(hipEventSynchronize(u.done));
+      spare_events.push_back(u.done);
+    }
+    uses.clear();
+    return ACC_OK;
+  }
+
+  // forget the uses that have completed; true if none is left
+  bool idle(std::vector<Use> &uses)
+  {
+    for (size_t i = 0; i < uses.size();) {
+      if (hipEventQuery(uses[i].done) == hipSuccess) {
+        spare_events.push_back(uses[i].done);
+        uses[i] = uses.back();
+        uses.pop_back();
+      } else {
+        (void)hipGetLastError();   // hipErrorNotReady is not a failure
+        ++i;
+      }
+    }
+    return uses.empty();
+  }
+
+  void upload_settled(Entry &e)
+  {
+    if (e.uploaded) { spare_events.push_back(e.uploaded); e.uploaded = nullptr; }
+  }
+
   int flush_nursery()
   {
-    for (auto &kv : nursery) ACC_HIP_TRY(hipFree(kv.second));
+    for (auto &kv : nursery) {
+      ACC_TRY(settle(kv.second.uses));
+      ACC_HIP_TRY(hipFree(kv.second.dev));
+    }
     nursery.clear();
     st.nursery_bytes = 0;
     return ACC_OK;
   }
 
-  // work recorded at the entry's last release has finished?
-  static bool idle(Entry &e)
-  {
-    if (!e.recorded) return true;
-    if (hipEventQuery(e.last_use) == hipSuccess) { e.recorded = false; return true; }
-    (void)hipGetLastError();   // hipErrorNotReady is not a failure
-    return false;
-  }
-
   // give up the device block of `e`: write back what only the device has, then
-  // hand the block to the nursery (keep == true) or to the device
+  // hand the block to the nursery (keep == true; work still reading it goes along
+  // and is waited for when the block is reused) or to the device
   int drop(Entry &e, bool keep)
   {
-    if (e.recorded) { ACC_HIP_TRY(hipEventSynchronize(e.last_use)); e.recorded = false; }
+    if (e.uploaded) { ACC_HIP_TRY(hipEventSynchronize(e.uploaded)); upload_settled(e); }
+    if (e.status == DIRTY || !keep) ACC_TRY(settle(e.uses));
     if (e.status == DIRTY) {
       ACC_HIP_TRY(hipMemcpy(e.host, e.dev, e.bytes, hipMemcpyDeviceToHost));
       st.writebacks++;
@@ -80,7 +129,10 @@ struct acc_memtable_s {
     st.resident_bytes -= e.rounded;
     st.resident_arrays--;
     if (keep) {
-      nursery.emplace(e.rounded, e.dev);
+      FreeBlock fb;
+      fb.dev = e.dev;
+      fb.uses.swap(e.uses);
+      nursery.emplace(e.rounded, std::move(fb));
       st.nursery_bytes += e.rounded;
     } else {
       ACC_HIP_TRY(hipFree(e.dev));
@@ -97,7 +149,7 @@ struct acc_memtable_s {
     for (auto &kv : table) {
       Entry &e = kv.second;
       if (!e.dev || e.pins > 0 || e.status == UNMANAGED) continue;
-      Entry *&slot = idle(e) ? best : busy;
+      Entry *&slot = idle(e.uses) ? best : busy;
       if (!slot || e.tick < slot->tick) slot = &e;
     }
     return best ? best : busy;
@@ -121,7 +173,8 @@ struct acc_memtable_s {
   {
     auto it = nursery.find(rounded);
     if (it != nursery.end()) {
-      *out = it->second;
+      ACC_TRY(settle(it->second.uses));
+      *out = it->second.dev;
       nursery.erase(it);
       st.nursery_bytes -= rounded;
       st.nursery_hits++;
@@ -174,11 +227,12 @@ int acc_memtable_destroy(acc_memtable mt)
     if (rc == ACC_OK) {
       for (auto &kv : mt->table) {
         Entry &e = kv.second;
-        if (e.recorded) (void)hipEventSynchronize(e.last_use);
-        if (e.last_use) (void)hipEventDestroy(e.last_use);
+        (void)mt->settle(e.uses);
+        if (e.uploaded) { (void)hipEventSynchronize(e.uploaded); mt->upload_settled(e); }
         if (e.dev && e.status != UNMANAGED) (void)hipFree(e.dev);
       }
-      for (auto &kv : mt->nursery) (void)hipFree(kv.second);
+      (void)mt->flush_nursery();
+      for (hipEvent_t ev : mt->spare_events) (void)hipEventDestroy(ev);
     }
   }
   delete mt;
@@ -239,13 +293,28 @@ int acc_memtable_acquire(acc_memtable mt, uint64_t key, acc_stream stream, acc_d
       mt->st.resident_arrays++;
     }
     if (e.bytes) {
-      ACC_HIP_TRY(hipMemcpyAsync(e.dev, e.host, e.bytes, hipMemcpyHostToDevice, static_cast<hipStream_t>(stream)));
+      hipStream_t s = static_cast<hipStream_t>(stream);
+      ACC_HIP_TRY(hipMemcpyAsync(e.dev, e.host, e.bytes, hipMemcpyHostToDevice, s));
+      mt->upload_settled(e);
+      ACC_TRY(mt->event(&e.uploaded));
+      ACC_HIP_TRY(hipEventRecord(e.uploaded, s));
+      e.upload_stream = s;
       mt->st.uploads++;
       mt->st.upload_bytes += e.bytes;
     }
     // what the device now holds is what the host holds; an array produced on the device is
     // taken to be changed again by whoever acquires it
     e.status = e.frozen ? CLEAN : DIRTY;
+  }
+  if (e.uploaded) {
+    // an upload queued on another stream: this stream's work starts after it
+    if (hipEventQuery(e.uploaded) == hipSuccess) {
+      mt->upload_settled(e);
+    } else {
+      (void)hipGetLastError();
+      if (e.upload_stream != static_cast<hipStream_t>(stream))
+        ACC_HIP_TRY(hipStreamWaitEvent(static_cast<hipStream_t>(stream), e.uploaded, 0));
+    }
   }
   e.pins++;
   e.tick = ++mt->clock;
@@ -264,9 +333,19 @@ int acc_memtable_release(acc_memtable mt, uint64_t key, acc_stream stream)
   Entry &e = it->second;
   if (e.pins <= 0) return fail(ACC_ERR_INVALID, "acc_memtable_release: key %llx is not acquired", (unsigned long long)key);
   if (e.status != UNMANAGED) {
-    if (!e.last_use) ACC_HIP_TRY(hipEventCreateWithFlags(&e.last_use, hipEventDisableTiming));
-    ACC_HIP_TRY(hipEventRecord(e.last_use, static_cast<hipStream_t>(stream)));
-    e.recorded = true;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    Use *u = nullptr;
+    for (Use &k : e.uses)
+      if (k.stream == s) u = &k;
+    if (!u) {
+      mt->idle(e.uses);                  // keeps the list as short as the streams really in flight
+      Use fresh;
+      fresh.stream = s;
+      ACC_TRY(mt->event(&fresh.done));
+      e.uses.push_back(fresh);
+      u = &e.uses.back();
+    }
+    ACC_HIP_TRY(hipEventRecord(u->done, s));
   }
   e.pins--;
   return ACC_OK;
@@ -286,7 +365,8 @@ int acc_memtable_free(acc_memtable mt, uint64_t key)
     ACC_TRY(mt->drop(e, true));
     if (mt->budget && mt->held() > mt->budget) ACC_TRY(mt->flush_nursery());
   }
-  if (e.last_use) (void)hipEventDestroy(e.last_use);
+  ACC_TRY(mt->settle(e.uses));            // (empty when the block went to the nursery with them)
+  if (e.uploaded) { ACC_HIP_TRY(hipEventSynchronize(e.uploaded)); mt->upload_settled(e); }
   mt->table.erase(it);
   mt->st.arrays--;
   return ACC_OK;

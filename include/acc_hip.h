@@ -418,8 +418,12 @@ int acc_memtable_malloc(acc_memtable mt, uint64_t key, void *host, uint64_t byte
  * returns the device pointer (allocating and uploading on `stream` first when
  * the array was evicted or never uploaded) and keeps the array resident until
  * the matching release; release names the stream the array was used on, and
- * the array is not evicted before the work queued on that stream at that
- * moment has completed.  Acquires nest.                                       */
+ * the block is neither evicted nor handed to another array before the work
+ * queued at that moment on every stream it was released on has completed.
+ * An acquire on another stream while the upload is still in flight makes that
+ * stream wait for the upload.  Ordering between the kernel that produces an
+ * array and its consumers on other streams stays with the caller (events, as
+ * Execute.hs:104-105 does with `after`).  Acquires nest.                      */
 int acc_memtable_acquire(acc_memtable mt, uint64_t key, acc_stream stream, acc_devptr *out);
 int acc_memtable_release(acc_memtable mt, uint64_t key, acc_stream stream);
 

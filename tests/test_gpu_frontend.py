@@ -276,3 +276,30 @@ def test_a_working_set_larger_than_the_memory_budget(acc):
     import gc
     gc.collect()
     assert cx.table.stats()["arrays"] <= 2                                         # results die with their last reference
+
+
+def test_independent_subcomputations_run_on_their_own_streams_and_meet_by_events(acc):
+    cx = acc.Context(0)
+    rng = np.random.default_rng(11)
+    n = 1 << 22
+    x, y = rng.integers(-9, 9, n).astype(np.int64), rng.integers(-9, 9, n).astype(np.int64)
+    xs, ys = acc.use(x, cx), acc.use(y, cx)
+    sx = acc.scanl1(add, xs, context=cx)                       # two independent scans ...
+    sy = acc.scanr1(add, ys, context=cx)
+    assert sx.manifest.stream is not sy.manifest.stream        # ... on two streams
+    both = acc._force(acc.zipWith(lambda a, b: a - b, sx, sy), cx)     # joins them: runs behind sx, waits for sy's event
+    assert both.manifest.stream is sx.manifest.stream
+    chain = both
+    for k in range(5):                                          # a dependent chain stays on one stream
+        chain = acc._force(acc.map(lambda v, k=k: v + k, chain), cx)
+        assert chain.manifest.stream is sx.manifest.stream
+    ref = np.cumsum(x) - np.cumsum(y[::-1])[::-1]
+    assert np.array_equal(acc.run(chain, cx), ref + 10)
+    assert np.array_equal(acc.run(sy, cx), np.cumsum(y[::-1])[::-1])
+    # the same input read from two streams right after its upload was queued on the first
+    z = rng.integers(-9, 9, 1 << 24).astype(np.int32)
+    zs = acc.use(z, cx)
+    f1 = acc.fold(add, 0, zs, context=cx)
+    f2 = acc.fold(acc.max_, -100, acc.map(lambda v: v * 2, zs), context=cx)
+    assert f1.manifest.stream is not f2.manifest.stream and cx.table.stats()["uploads"] == 3
+    assert int(acc.run(f1, cx)) == int(z.sum()) and int(acc.run(f2, cx)) == int(z.max() * 2)

@@ -195,3 +195,50 @@ def test_eviction_waits_for_the_work_recorded_at_release(A, ctx, kernels):
     assert np.array_equal(r, 2 * a)
     mt.destroy()
     A.check(A.lib().acc_stream_destroy(ctx.handle, s))
+
+
+def test_blocks_used_on_two_streams_wait_for_both(A, ctx, kernels):
+    say("two streams, eviction and reuse behind running work")
+    mt = A.MemTable(ctx, budget_bytes=48 * MB)
+    a, = host_arrays(1, 5)
+    r1, r2 = np.zeros(N, np.float32), np.zeros(N, np.float32)
+    s1, s2 = ctx.stream(), ctx.stream()
+    mt.malloc(a, frozen=True)
+    mt.malloc(r1, frozen=False)
+    mt.malloc(r2, frozen=False)
+    da, d1 = mt.acquire(a, s1), mt.acquire(r1, s1)
+    da2, d2 = mt.acquire(a, s2), mt.acquire(r2, s2)              # s2 is made to wait for the upload queued on s1
+    assert da2.ptr == da.ptr and mt.stats()["uploads"] == 1
+    for _ in range(10):
+        kernels["double"].map([da], d1, stream=s1)
+        kernels["add"].map([da2, da2], d2, stream=s2)
+    mt.release(a, s1)
+    mt.release(r1, s1)
+    mt.release(a, s2)
+    mt.release(r2, s2)
+    # everything must leave for a 48 MiB array: each block waits for the streams it was released on
+    filler = np.zeros(3 * N, np.float32)
+    mt.malloc(filler, frozen=False)
+    assert mt.stats()["evictions"] == 3 and mt.stats()["writebacks"] == 2
+    assert np.array_equal(r1, 2 * a) and np.array_equal(r2, a + a)
+    # a block freed while a kernel still writes it is reused only after that kernel
+    mt.free(filler)
+    mt.reclaim()
+    t = np.zeros(N, np.float32)
+    mt.malloc(t, frozen=False)
+    da, dt = mt.acquire(a, s1), mt.acquire(t, s1)
+    for _ in range(10):
+        kernels["double"].map([da], dt, stream=s1)
+    mt.release(a, s1)
+    mt.release(t, s1)
+    mt.free(t)                                                    # returns at once; the block carries s1's event
+    u = (np.arange(N) % 7).astype(np.float32)
+    mt.malloc(u, frozen=True)
+    du = mt.acquire(u, s2)                                        # same size: the same block, uploaded on s2
+    assert du.ptr == dt.ptr and mt.stats()["nursery_hits"] >= 1
+    A.check(A.lib().acc_stream_sync(ctx.handle, s2))
+    assert np.array_equal(du.get(), u)                            # not overwritten by the tail of s1's kernels
+    mt.release(u, s2)
+    mt.destroy()
+    for s in (s1, s2):
+        A.check(A.lib().acc_stream_destroy(ctx.handle, s))
