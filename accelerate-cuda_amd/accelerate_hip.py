@@ -33,7 +33,7 @@ import acchip as A
 
 __all__ = ["Exp", "constant", "cond", "use", "unit", "map", "zipWith", "generate", "backpermute", "transpose", "reverse", "zip_", "unzip", "while_",
            "fold", "fold1", "foldSeg", "scanl", "scanl1", "scanl_", "scanr", "scanr1", "scanr_", "permute", "ignore",
-           "stencil", "stencil2", "run", "run1", "fst", "snd", "lift", "index_if", "fromIntegral", "truncate", "round_", "floor",
+           "stencil", "stencil2", "awhile", "run", "run1", "fst", "snd", "lift", "index_if", "fromIntegral", "truncate", "round_", "floor",
            "ceiling", "idiv", "mod", "quot", "rem", "min_", "max_", "sqrt", "exp", "log", "sin", "cos", "tan", "abs_",
            "signum", "Context", "the"]
 
@@ -470,9 +470,9 @@ def use(host, context=None):
     not be changed afterwards."""
     cx = context or Context.default()
     if isinstance(host, tuple):
-        hs = [np.ascontiguousarray(h) for h in host]
+        hs = [np.asarray(h, order="C") for h in host]
         return Acc(hs[0].shape, tuple(CTYPE[h.dtype.type] for h in hs), manifest=A.TupleArray([_Resident(cx, h, True) for h in hs]))
-    host = np.ascontiguousarray(host)
+    host = np.asarray(host, order="C")                  # (ascontiguousarray would make a scalar array a vector)
     return Acc(host.shape, CTYPE[host.dtype.type], manifest=_Resident(cx, host, True))
 
 
@@ -734,6 +734,26 @@ def stencil2(pattern1, pattern2, f, boundary1, a, boundary2, b, context=None, co
     out = _empty(cx, shape, res.ctype)
     cx.launch(arrays + [s1.manifest, s2.manifest], [out], lambda i, o, s: sk.stencil2(i[:-2], i[-2], i[-1], o[0], stream=s))
     return Acc(shape, res.ctype, manifest=out)
+
+
+def awhile(p, f, a, context=None, limit=None):
+    """iterate the array function `f` from `a` while the scalar array `p(a)` holds a non-zero value
+    (Execute.hs:236-244).  `a` is an Acc or a tuple of them; every iterate is made manifest, and the
+    flag is the one value read back per iteration."""
+    cx = context or Context.default()
+    tup = isinstance(a, tuple)
+    force = lambda v: tuple(_force(x, cx) for x in v) if tup else _force(v, cx)
+    a = force(a)
+    n = 0
+    while limit is None or n < limit:
+        flag = p(*a) if tup else p(a)
+        if flag.shape != ():
+            raise TypeError("the predicate of awhile yields a scalar array")
+        if not the(flag, cx):
+            break
+        a = force(f(*a) if tup else f(a))
+        n += 1
+    return a
 
 
 def run(a, context=None):

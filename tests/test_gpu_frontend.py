@@ -303,3 +303,44 @@ def test_independent_subcomputations_run_on_their_own_streams_and_meet_by_events
     f2 = acc.fold(acc.max_, -100, acc.map(lambda v: v * 2, zs), context=cx)
     assert f1.manifest.stream is not f2.manifest.stream and cx.table.stats()["uploads"] == 3
     assert int(acc.run(f1, cx)) == int(z.sum()) and int(acc.run(f2, cx)) == int(z.max() * 2)
+
+
+def test_awhile_iterates_on_the_device_until_the_flag_clears(acc):
+    cx = acc.Context(0)
+    rng = np.random.default_rng(12)
+    x = rng.integers(1, 50, 100003).astype(np.int64)
+    # double every element until the largest passes a million
+    big = lambda xs: acc.map(lambda m: m < 1000000, acc.fold(acc.max_, 0, xs, context=cx))
+    out = acc.run(acc.awhile(big, lambda xs: acc.map(lambda v: v * 2, xs), acc.use(x, cx), context=cx), cx)
+    ref = x.copy()
+    while ref.max() < 1000000:
+        ref = ref * 2
+    assert np.array_equal(out, ref)
+    # a pair of arrays as the state: Jacobi sweeps of a 1-D heat rod until the update is small, with a sweep counter
+    u0 = np.zeros(4097, np.float64)
+    u0[0], u0[-1] = 1.0, 3.0
+
+    def sweep(u, k):
+        nu = acc.stencil([(-1,), (0,), (1,)], lambda a, b, c: (a + c) / 2.0, "clamp", u, context=cx)
+        n = u.shape[0]
+        fixed = acc.zipWith(lambda new, old: new, nu, u)        # interior from the sweep ...
+        ends = acc.generate((n,), lambda i: acc.cond(i.eq(0).lor(i.eq(n - 1)), acc.constant(1, "Word8"), acc.constant(0, "Word8")))
+        fixed = acc.zipWith(lambda e, p: acc.cond(e, acc.snd(p), acc.fst(p)), ends, acc.zip_(nu, u))   # ... ends kept
+        return fixed, acc.map(lambda c: c + 1, k)
+
+    def moving(u, k):
+        nu, _ = sweep(u, k)
+        delta = acc.fold(acc.max_, 0.0, acc.zipWith(lambda a, b: acc.abs_(a - b), nu, u), context=cx)
+        return acc.zipWith(lambda d, c: (d > 1e-3).land(c < 500), delta, k)
+    u, k = acc.awhile(moving, sweep, (acc.use(u0, cx), acc.unit(0, "Int32", cx)), context=cx)
+    ref, steps = u0.copy(), 0
+    while True:
+        nxt = ref.copy()
+        nxt[1:-1] = (ref[:-2] + ref[2:]) / 2.0
+        if not (np.abs(nxt - ref).max() > 1e-3 and steps < 500):
+            break
+        ref, steps = nxt, steps + 1
+    assert int(acc.run(k, cx)) == steps and steps > 3
+    assert np.array_equal(acc.run(u, cx), ref)
+    with pytest.raises(TypeError):
+        acc.awhile(lambda xs: xs, lambda xs: xs, acc.use(x, cx), context=cx)
