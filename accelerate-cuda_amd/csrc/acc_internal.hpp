@@ -47,8 +47,10 @@ std::string embedded_text(const char *name);
 enum ScratchProtocol {
   SCRATCH_FOLD = 0,   // contents are don't-care: every launch writes what it reads (fold partials, permute tables)
   SCRATCH_LOCKS = 2,  // all zero between uses: every launch leaves it as it found it
-  SCRATCH_SCAN = 1    // word 0 is a tile counter used relative to `counter_base`; tile descriptors
+  SCRATCH_SCAN = 1,   // word 0 is a tile counter used relative to `counter_base`; tile descriptors
                       // carry `epoch`, so stale ones read as "not yet published"
+  SCRATCH_FLAGS = 3   // 64-bit words {epoch, payload}: every launch tags what it writes with its `epoch`,
+                      // anything older reads as "not yet"
 };
 
 struct ScratchBlock {

@@ -49,11 +49,51 @@ ACC_DEV acc_opt<T> acc_block_reduce(acc_opt<T> x, F f, acc_opt<T> *s_wave)
 
 #if !ACC_FOLD_DIM
 
+#if ACC_FOLD_SINGLE
+/* A value handed from one workgroup to another without fences: it is cut into
+ * 4-byte pieces and every piece travels in a 64-bit word of its own together
+ * with the tag of the launch, written and read with relaxed device-scope
+ * atomics (write-through, no cache-wide write-back or invalidate as a
+ * release/acquire pair costs).  The value has arrived when all its words
+ * carry the tag.                                                            */
+template <typename T>
+struct acc_tagged {
+  static constexpr int NW = (int)((sizeof(T) + 3) / 4);
+  unsigned long long *d;
+  ACC_DEV void put(unsigned int slot, unsigned int tag, const T &v) const
+  {
+    unsigned int b[NW] = {};
+    __builtin_memcpy(b, &v, sizeof(T));
+#pragma unroll
+    for (int k = 0; k < NW; ++k)
+      __hip_atomic_store(d + (Int64)slot * NW + k, ((unsigned long long)tag << 32) | b[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  ACC_DEV T wait(unsigned int slot, unsigned int tag) const
+  {
+    unsigned int b[NW];
+#pragma unroll
+    for (int k = 0; k < NW; ++k) {
+      unsigned long long w;
+      while ((unsigned int)((w = __hip_atomic_load(d + (Int64)slot * NW + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >> 32) != tag)
+        __builtin_amdgcn_s_sleep(1);
+      b[k] = (unsigned int)w;
+    }
+    T v;
+    __builtin_memcpy(&v, b, sizeof(T));
+    return v;
+  }
+};
+#endif
+
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 ACC_ENTRY(ACC_ENV_PARAMS
           ACC_OUT_ARRAY(arrOut),
           const Int64 shIn_0,
+#if ACC_FOLD_SINGLE
+          unsigned long long *partials, const unsigned int epoch)
+#else
           ACC_ELT *__restrict__ partials)
+#endif
 {
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
@@ -116,11 +156,29 @@ ACC_ENTRY(ACC_ENV_PARAMS
 
   acc_opt<T> total = acc_block_reduce(mine, f, s_wave);
 
+#if ACC_FOLD_SINGLE
+  /* One launch: every block but the last leaves its partial result, tagged with this launch's epoch
+   * (whatever an earlier launch left carries an older one); the last block collects them.  The grid
+   * never exceeds what is resident at once, so nobody waits for a place on the device meanwhile.   */
+  if (gridDim.x > 1) {
+    const acc_tagged<T> slots = {partials};
+    const unsigned int last = gridDim.x - 1;
+    if (blockIdx.x != last) {
+      if (threadIdx.x == 0) slots.put(blockIdx.x, epoch, total.v);   /* the host guarantees every block owns >= 1 element */
+      return;
+    }
+    acc_opt<T> p = threadIdx.x == 0 ? total : acc_none<T>();
+    for (unsigned int i = threadIdx.x; i < last; i += ACC_BLOCK) p = lf(p, acc_some(slots.wait(i, epoch)));
+    total = acc_block_reduce(p, f, s_wave);
+  }
+  if (threadIdx.x != 0) return;
+#else
   if (threadIdx.x != 0) return;
   if (gridDim.x > 1) {
     partials[blockIdx.x] = total.v;              /* the host guarantees every block owns >= 1 element */
     return;
   }
+#endif
 #if ACC_HAS_SEED
   const T seed = (ACC_SEED);
   ACC_SET(arrOut, 0, total.ok ? f(total.v, seed) : seed);

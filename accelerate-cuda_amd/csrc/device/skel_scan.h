@@ -75,24 +75,40 @@ struct acc_scan_desc {
   }
 };
 
-/* wider elements: value slots written plainly, then the flag released; the
- * reader acquires the flag before touching the slot                          */
+/* wider elements: cut into 4-byte pieces, each in a 64-bit word of its own next to
+ * the same flag, all relaxed device-scope atomics as above.  (A plain value slot
+ * plus a released flag costs a cache-wide write-back per tile and an invalidate
+ * per poll on this part: scans of 8-byte elements ran at a third of the speed.)
+ * A descriptor is complete when all its words carry the same flag; while a tile
+ * replaces its AGGREGATE by its PREFIX a reader may meet both, and reads again. */
 template <typename T>
 struct acc_scan_desc<T, false> {
-  unsigned int *flags; T *agg; T *inc;
-  ACC_DEV acc_scan_desc(void *p0, void *p1, void *p2) : flags((unsigned int *)p0), agg((T *)p1), inc((T *)p2) {}
+  static constexpr int NW = (int)((sizeof(T) + 3) / 4);
+  static constexpr int SLOT = NW > ACC_DESC_STRIDE ? NW : ACC_DESC_STRIDE;     /* 8-byte words per tile */
+  unsigned long long *d;
+  ACC_DEV acc_scan_desc(void *p0, void *, void *) : d((unsigned long long *)p0) {}
   ACC_DEV void put(Int64 tile, unsigned int flag, const T &v) const
   {
-    T *slot = ((flag & 3u) == ACC_ST_AGGREGATE) ? agg : inc;
-    slot[tile] = v;
-    __hip_atomic_store(flags + tile, flag, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    unsigned int b[NW] = {};
+    __builtin_memcpy(b, &v, sizeof(T));
+#pragma unroll
+    for (int k = 0; k < NW; ++k)
+      __hip_atomic_store(d + tile * SLOT + k, ((unsigned long long)flag << 32) | b[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   ACC_DEV unsigned int get(Int64 tile, T &v) const
   {
-    unsigned int f = __hip_atomic_load(flags + tile, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
-    const T *slot = ((f & 3u) == ACC_ST_AGGREGATE) ? agg : inc;
-    v = slot[tile];
-    return f;
+    unsigned int b[NW];
+    unsigned int f = 0;
+    bool same = true;
+#pragma unroll
+    for (int k = 0; k < NW; ++k) {
+      const unsigned long long w = __hip_atomic_load(d + tile * SLOT + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      b[k] = (unsigned int)w;
+      if (k == 0) f = (unsigned int)(w >> 32);
+      else same = same && (unsigned int)(w >> 32) == f;
+    }
+    __builtin_memcpy(&v, b, sizeof(T));
+    return same ? f : 0u;                 /* 0 is no launch's flag: the caller reads again */
   }
 };
 

@@ -192,13 +192,43 @@ int acc_exec_fold(acc_skel s, const acc_array *env, int32_t in_rank, const int64
 
   const int64_t n = inner;
   const int64_t tile = s->elements_per_block();
-  const int64_t grid = acc_launch_grid(n, tile, s->ctx->props.multiProcessorCount,
-                                       std::min(s->variants[v].blocks_per_cu, acc::tune("fold.blocks_per_cu", 4)));
+  int64_t grid = acc_launch_grid(n, tile, s->ctx->props.multiProcessorCount,
+                                 std::min(s->variants[v].blocks_per_cu, acc::tune("fold.blocks_per_cu", 4)));
+  const bool single = acc::tune("fold.single", 1) != 0;       // (the kernel was generated under the same setting)
   if (grid == 1) {                 // a lone block finishes the job itself
     push_ptrs(out, out->ncomp, &args, &aligned);
     args.i64(n);
     args.ptr(0);
+    if (single) args.u32(0);
     return launch(s, v, 1, 0, st, &args);
+  }
+  if (single) {
+    // one launch: every block leaves its partial result in 64-bit words that carry the launch's epoch in their
+    // upper half, and the last block collects them (skel_fold.h).  Every word of the scratch block is only ever
+    // written in that form, so words of earlier launches, whatever their grid or element type, read as "not yet".
+    const size_t words = (s->spec.elt_size + 3) / 4;
+    int blk = -1;
+    ACC_TRY(s->ctx->scratch_acquire((size_t)grid * words * 8, st, acc::SCRATCH_FLAGS, &blk));
+    uint32_t epoch;
+    char *base;
+    {
+      std::lock_guard<std::mutex> lock(s->ctx->mu);
+      acc::ScratchBlock &b = s->ctx->scratch[blk];
+      base = static_cast<char *>(b.ptr);
+      if (b.epoch == 0xFFFFFFFFu) {              // start over from a clean block
+        hipError_t e = hipMemsetAsync(b.ptr, 0, b.bytes, st);
+        if (e != hipSuccess) { b.busy = false; return acc::fail_hip(e, "hipMemsetAsync(fold partials)"); }
+        b.epoch = 0;
+      }
+      epoch = ++b.epoch;
+    }
+    push_ptrs(out, out->ncomp, &args, &aligned);
+    args.i64(n);
+    args.ptr(reinterpret_cast<uint64_t>(base));
+    args.u32(epoch);
+    int rc = launch(s, v, grid, 0, st, &args);
+    s->ctx->scratch_release(blk, st);
+    return rc;
   }
   // one partial per block, then a single-block launch folds them: foldRec, Execute.hs:304-315,
   // always exactly one level deep because the first grid never exceeds what is resident
@@ -290,15 +320,11 @@ int acc_exec_scan(acc_skel s, const acc_array *env, int64_t n, const acc_array *
   }
   const int64_t ndesc = std::max<int64_t>(1, tiles);
   const size_t esz = s->spec.elt_size;
-  size_t bytes = 256;
-  size_t off_d0 = 256, off_d1 = 0, off_d2 = 0;
-  if (esz <= 4) {
-    bytes += round256((size_t)ndesc * 8 * (size_t)acc::tune("scan.desc_stride", 16));
-  } else {
-    off_d1 = off_d0 + round256((size_t)ndesc * 4);
-    off_d2 = off_d1 + round256((size_t)ndesc * esz);
-    bytes = off_d2 + round256((size_t)ndesc * esz);
-  }
+  // one descriptor per tile: 64-bit words {flag, 4 bytes of the value}, `scan.desc_stride` words apart
+  // (more when the element needs more words)
+  const size_t words = std::max<size_t>((esz + 3) / 4, (size_t)acc::tune("scan.desc_stride", 16));
+  const size_t off_d0 = 256, off_d1 = 256, off_d2 = 256;
+  const size_t bytes = 256 + round256((size_t)ndesc * 8 * words);
   int blk = -1;
   ACC_TRY(s->ctx->scratch_acquire(bytes, st, acc::SCRATCH_SCAN, &blk));
   uint32_t epoch, counter_base;

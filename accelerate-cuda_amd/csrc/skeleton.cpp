@@ -185,6 +185,7 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       if (sp.out_rank == 0) *entry = sp.has_seed ? "foldAll" : "fold1All";
       else *entry = sp.has_seed ? "fold" : "fold1";
       o << "#define ACC_FOLD_DIM " << (sp.out_rank == 0 ? 0 : 1) << "\n";
+      o << "#define ACC_FOLD_SINGLE " << tune("fold.single", 1) << "\n";
       o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_UNROLL " << sp.unroll << "\n";
       tmpl = "skel_fold.h";
       break;
