@@ -214,6 +214,43 @@ template <typename T> ACC_DEV void acc_store(T *p, const T &v)
 #endif
 }
 
+/* Loads and stores that meet at device scope: relaxed atomics, which go past the
+ * caches that are not coherent across the compute dies instead of asking for a
+ * cache-wide invalidate or write-back.  Any size: in pieces of 8, 4, 2 or 1 bytes
+ * (an element is only ever accessed this way under a lock, so the pieces need
+ * not be atomic together).                                                   */
+template <int N> struct acc_piece;
+template <> struct acc_piece<8> { typedef unsigned long long type; };
+template <> struct acc_piece<4> { typedef unsigned int type; };
+template <> struct acc_piece<2> { typedef unsigned short type; };
+template <> struct acc_piece<1> { typedef unsigned char type; };
+template <typename T> struct acc_piece_of {
+  static constexpr int N = (sizeof(T) % 8 == 0 && alignof(T) >= 8) ? 8 : (sizeof(T) % 4 == 0 && alignof(T) >= 4) ? 4 :
+                           (sizeof(T) % 2 == 0 && alignof(T) >= 2) ? 2 : 1;
+  typedef typename acc_piece<N>::type type;
+  static constexpr int COUNT = (int)(sizeof(T) / N);
+};
+template <typename T> ACC_DEV T acc_load_device(const T *p)
+{
+  typedef typename acc_piece_of<T>::type P;
+  P b[acc_piece_of<T>::COUNT];
+#pragma unroll
+  for (int k = 0; k < acc_piece_of<T>::COUNT; ++k)
+    b[k] = __hip_atomic_load((const P *)p + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  T v;
+  __builtin_memcpy(&v, b, sizeof(T));
+  return v;
+}
+template <typename T> ACC_DEV void acc_store_device(T *p, const T &v)
+{
+  typedef typename acc_piece_of<T>::type P;
+  P b[acc_piece_of<T>::COUNT];
+  __builtin_memcpy(b, &v, sizeof(T));
+#pragma unroll
+  for (int k = 0; k < acc_piece_of<T>::COUNT; ++k)
+    __hip_atomic_store((P *)p + k, b[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 /* row-major index helpers (CodeGen/Base.hs:193-218): shapes and indices are
  * listed innermost dimension LAST, e.g. acc_to_index2(h, w, y, x)            */
 ACC_DEV Int64 acc_to_index2(Int64, Int64 w, Int64 y, Int64 x) { return y * w + x; }

@@ -49,13 +49,15 @@
  * is masked off until the spinning lane leaves the loop.  So nobody spins: the
  * wave goes round a loop whose condition is a vote of the whole wave, every
  * lane that still has work tries its lock once per trip, and whoever gets it
- * updates the element and frees the lock within that trip.  Taking the lock
- * is an acquire and freeing it a release, both at device scope: the compiler
- * puts the cache invalidation and write-back around them that make the
- * element written under the lock the one the next holder reads, on whichever
- * compute die it runs (acknowledged stores alone are not enough: they are
- * acknowledged by the die's own L2).  `locks` must be all zero on entry and is
- * all zero again on exit; the word before it records a lane that gave up.    */
+ * updates the element and frees the lock within that trip.  The lock and the
+ * element under it are only touched with relaxed device-scope atomics, which
+ * go past the caches that are private to a compute die: the holder waits for
+ * its stores to the element to be acknowledged before it stores the free lock,
+ * and the next holder, on whichever die, loads the element after its exchange
+ * has returned.  (A release/acquire pair would do as well and costs a
+ * cache-wide write-back and invalidate per update: 40 times slower.)  `locks`
+ * must be all zero on entry and is all zero again on exit; the word before it
+ * records a lane that gave up.                                               */
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, int *__restrict__ locks)
 {
@@ -76,10 +78,15 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, int *__restrict__ loc
      * of which holds the lock for a few round trips to memory: hence the factor. */
     Int64 trips = 0;
     while (__ballot(!done) != 0 && trips < 64 * n + (1 << 20)) {
-      if (!done && __hip_atomic_exchange(locks + j, 1, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) == 0) {
-        const T cur = ACC_READ(arrOut, j);
-        ACC_SET(arrOut, j, f(x, cur));
-        __hip_atomic_store(locks + j, 0, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+      const bool got = !done && __hip_atomic_exchange(locks + j, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0;
+      /* failed exchanges queue at the lock's address in front of the store that frees it: a wave that keeps
+       * getting nowhere steps back for a while */
+      if (trips >= 4 && __ballot(got) == 0) __builtin_amdgcn_s_sleep(32);
+      if (got) {
+        const T cur = ACC_READ_DEVICE(arrOut, j);
+        ACC_SET_DEVICE(arrOut, j, f(x, cur));
+        __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory");        /* the stores above are acknowledged ... */
+        __hip_atomic_store(locks + j, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   /* ... before this one leaves */
         done = true;
       }
       ++trips;

@@ -132,25 +132,36 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
   //   ACC_SET(name, ix, v)  the same as an ordinary store (small results that are read again soon)
   {
     const int nc = sp.comp_types.empty() ? 1 : (int)sp.comp_types.size();
-    std::ostringstream arr, assume, put, set, read;
+    std::ostringstream arr, assume, put, set, read, read_dev, set_dev;
     for (int i = 0; i < nc; ++i) {
       const int c = nc - 1 - i;
       const std::string t = sp.comp_types.empty() ? std::string("ACC_ELT") : sp.comp_types[i];
       arr << (i ? ", " : "") << t << " *__restrict__ name##_" << c;
       assume << "name##_" << c << " = (" << t << " *)__builtin_assume_aligned(name##_" << c << ", 16); ";
       read << (i ? ", " : "") << "name##_" << c << "[ix]";
+      read_dev << (i ? ", " : "") << "acc_load_device(name##_" << c << " + (ix))";
       if (sp.comp_types.empty()) {
         put << "acc_store(name##_0 + (ix), (v))";
         set << "name##_0[ix] = (v)";
+        set_dev << "acc_store_device(name##_0 + (ix), (ACC_ELT)(v))";
       } else {
         put << "acc_store(name##_" << c << " + (ix), acc_pv.a" << c << "); ";
         set << "name##_" << c << "[ix] = acc_pv.a" << c << "; ";
+        set_dev << "acc_store_device(name##_" << c << " + (ix), acc_pv.a" << c << "); ";
       }
     }
     o << "#define ACC_NCOMP " << nc << "\n";
     //   ACC_READ(name, ix)    element ix, assembled from its components
-    if (sp.comp_types.empty()) o << "#define ACC_READ(name, ix) (" << read.str() << ")\n";
-    else o << "#define ACC_READ(name, ix) (ACC_ELT{" << read.str() << "})\n";
+    //   ACC_READ_DEVICE / ACC_SET_DEVICE: the same at device scope, past the caches (elements shared under a lock)
+    if (sp.comp_types.empty()) {
+      o << "#define ACC_READ(name, ix) (" << read.str() << ")\n";
+      o << "#define ACC_READ_DEVICE(name, ix) (" << read_dev.str() << ")\n";
+      o << "#define ACC_SET_DEVICE(name, ix, v) " << set_dev.str() << "\n";
+    } else {
+      o << "#define ACC_READ(name, ix) (ACC_ELT{" << read.str() << "})\n";
+      o << "#define ACC_READ_DEVICE(name, ix) (ACC_ELT{" << read_dev.str() << "})\n";
+      o << "#define ACC_SET_DEVICE(name, ix, v) do { const ACC_ELT acc_pv = (v); " << set_dev.str() << "} while (0)\n";
+    }
     o << "#define ACC_OUT_ARRAY(name) " << arr.str() << "\n";
     o << "#define ACC_OUT_ASSUME(name) " << (aligned ? assume.str() : std::string()) << "\n";
     if (sp.comp_types.empty()) {

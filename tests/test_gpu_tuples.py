@@ -186,6 +186,28 @@ def test_permute_of_tuples_and_narrow_elements_under_locks(A, ctx):
     assert np.array_equal(o8.get(), exp)
 
 
+def test_locked_permute_loses_no_update_at_scale(A, ctx):
+    """4 M updates under per-target locks, from every compute die, with hundreds of lanes waiting at each lock and with
+    hardly any: integer sums and counts are exact, so one lost or torn update shows.  (A handful of targets for
+    millions of updates is the case locks are worst at -- every update waits behind all the failed attempts queued at
+    its lock -- and is kept to the small sizes of the test above.)"""
+    rng = np.random.default_rng(23)
+    n = 1 << 22
+    w = rng.integers(-1000, 1000, n).astype(np.int64)
+    sk = ctx.skeleton(A.SKEL_PERMUTE, "Int64, Int32", env=[I32, (1, "Int64")], out_rank=1, get="acc_elt{arrIn1_0[ix], 1}",
+                      combine="acc_elt{x.a1 + y.a1, x.a0 + y.a0}", permutation="arrIn0_0[ix]")
+    for bins in (1000, 100003):
+        say("locked permute, %d updates into %d targets" % (n, bins))
+        keys = rng.integers(0, bins, n).astype(np.int32)
+        out = ctx.empty_tuple(bins, [np.int64, np.int32])
+        sk.permute([ctx.array(keys), ctx.array(w)], n, ctx.tuple_array(np.zeros(bins, np.int64), np.zeros(bins, np.int32)), out)
+        s_, c_ = out.get()
+        assert np.array_equal(c_, np.bincount(keys, minlength=bins).astype(np.int32))
+        ref = np.zeros(bins, np.int64)
+        np.add.at(ref, keys, w)
+        assert np.array_equal(s_, ref)
+
+
 def test_tuple_results_need_tuple_arrays_and_are_refused_elsewhere(A, ctx):
     say("misuse")
     zipk = ctx.skeleton(A.SKEL_MAP, "float, Int32", env=[F32], out_rank=1, get="acc_elt{arrIn0_0[ix], 0}")
