@@ -35,6 +35,9 @@ static_assert(ACC_CHUNK % (ACC_BLOCK * ACC_VEC) == 0, "chunk must be a whole num
 #endif
 
 #define ACC_LOADS (ACC_CHUNK / (ACC_BLOCK * ACC_VEC))   /* vector loads per lane and chunk */
+/* One word of padding per 32 elements of the staged chunk: lanes that fold segments whose starts are a multiple
+ * of 32 elements apart (every segment 32, 64, 128 ... long) would otherwise all read the same LDS bank.       */
+#define ACC_PAD(i) ((i) + ((i) >> 5))
 #define ACC_EAT 8                                        /* LDS reads kept in flight while folding */
 
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
@@ -45,7 +48,7 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
 {
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
-  __shared__ __attribute__((aligned(16))) T s_val[ACC_CHUNK];
+  __shared__ __attribute__((aligned(16))) T s_val[ACC_PAD(ACC_CHUNK)];
 
   auto get = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
   auto f   = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
@@ -106,7 +109,7 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
 #pragma unroll
       for (int u = 0; u < ACC_LOADS; ++u)
 #pragma unroll
-        for (int k = 0; k < ACC_VEC; ++k) s_val[(u * ACC_BLOCK + tid) * ACC_VEC + k] = v[u][k];
+        for (int k = 0; k < ACC_VEC; ++k) s_val[ACC_PAD((u * ACC_BLOCK + tid) * ACC_VEC + k)] = v[u][k];
       __syncthreads();
       /* the next chunk's loads (and the gathers behind them) travel while this one is folded */
       if (q + 1 < nchunks) stage(chunk_start(q + 1));
@@ -114,25 +117,25 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
       /* fold this lane's segment, as far as it lies in the chunk, in index order */
       int p0 = (int)(acc_max(a, cs) - cs), p1 = (int)(acc_min(b, ce) - cs);
 #if ACC_FOLD_RIGHT
-      if (!have && p0 < p1) { acc = s_val[--p1]; have = true; }
+      if (!have && p0 < p1) { --p1; acc = s_val[ACC_PAD(p1)]; have = true; }
       for (; p1 - ACC_EAT >= p0; p1 -= ACC_EAT) {
         T w[ACC_EAT];
 #pragma unroll
-        for (int k = 0; k < ACC_EAT; ++k) w[k] = s_val[p1 - 1 - k];
+        for (int k = 0; k < ACC_EAT; ++k) w[k] = s_val[ACC_PAD(p1 - 1 - k)];
 #pragma unroll
         for (int k = 0; k < ACC_EAT; ++k) acc = f(w[k], acc);
       }
-      for (; p1 > p0; --p1) acc = f(s_val[p1 - 1], acc);
+      for (; p1 > p0; --p1) acc = f(s_val[ACC_PAD(p1 - 1)], acc);
 #else
-      if (!have && p0 < p1) { acc = s_val[p0++]; have = true; }
+      if (!have && p0 < p1) { acc = s_val[ACC_PAD(p0)]; ++p0; have = true; }
       for (; p0 + ACC_EAT <= p1; p0 += ACC_EAT) {
         T w[ACC_EAT];
 #pragma unroll
-        for (int k = 0; k < ACC_EAT; ++k) w[k] = s_val[p0 + k];
+        for (int k = 0; k < ACC_EAT; ++k) w[k] = s_val[ACC_PAD(p0 + k)];
 #pragma unroll
         for (int k = 0; k < ACC_EAT; ++k) acc = f(acc, w[k]);
       }
-      for (; p0 < p1; ++p0) acc = f(acc, s_val[p0]);
+      for (; p0 < p1; ++p0) acc = f(acc, s_val[ACC_PAD(p0)]);
 #endif
     }
 
@@ -141,6 +144,120 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
       ACC_SET(arrOut, seg, have ? f(acc, seed) : seed);
 #else
       ACC_SET(arrOut, seg, acc);      /* fold1Seg of an empty segment is undefined; T() is written */
+#endif
+    }
+  }
+}
+
+/* ---- long segments: a team of lanes per segment ---------------------------
+ * One lane per segment serialises a long segment on that lane, so when the
+ * segments are long on average the host launches this entry instead: a whole
+ * wave (block_team == 0) or a whole workgroup (block_team != 0) takes one
+ * segment at a time.  The team walks the segment in rounds of ACC_TVEC
+ * consecutive elements per lane, each lane folds its own elements in order,
+ * the lanes are combined in lane order (the wave reduction preserves order,
+ * waves meet in LDS in wave order) and the round's value joins the running
+ * one on the proper side: the segment is still combined in index order, only
+ * the association differs from the one-lane-per-segment entry, as the
+ * operator's associativity allows.  ACC_TROUNDS rounds of loads are issued
+ * before the first is used.                                                 */
+#define ACC_TVEC 4
+#define ACC_TROUNDS 4
+#define ACC_FS_WAVES (ACC_BLOCK / ACC_WAVE)
+#define ACC_FS_CAT2(a, b) a##b
+#define ACC_FS_CAT(a, b) ACC_FS_CAT2(a, b)
+
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _team)(ACC_ENV_PARAMS
+                                     const Int64 shOut_0, ACC_OUT_ARRAY(arrOut),
+                                     const Int64 shIn_0,
+                                     const ACC_SEG_TYPE *__restrict__ arrSeg_0,
+                                     const int block_team)
+{
+  typedef ACC_ELT T;
+  ACC_ENV_ASSUME
+  __shared__ acc_opt<T> s_wave[ACC_FS_WAVES];
+
+  auto get = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
+  auto f   = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
+  auto lf  = acc_lift<T>(f);
+
+  const Int64 nseg = shOut_0;
+  const Int64 n = shIn_0;
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int me = block_team ? tid : acc_lane();                    /* place in the team */
+  const Int64 team_lanes = block_team ? ACC_BLOCK : ACC_WAVE;
+  const Int64 team0 = block_team ? (Int64)blockIdx.x : (Int64)blockIdx.x * ACC_FS_WAVES + wave;
+  const Int64 nteams = block_team ? (Int64)gridDim.x : (Int64)gridDim.x * ACC_FS_WAVES;
+  const Int64 round = team_lanes * ACC_TVEC;
+#if ACC_HAS_SEED
+  const T seed = (ACC_SEED);
+#endif
+
+  /* the values of round `r` of [a, b) that fall to this lane, folded in order */
+  auto mine = [&](const Int64 a, const Int64 b, const Int64 r, const T (&v)[ACC_TVEC]) -> acc_opt<T> {
+    const Int64 base = a + r * round + (Int64)me * ACC_TVEC;
+    acc_opt<T> m = acc_none<T>();
+#pragma unroll
+    for (int k = 0; k < ACC_TVEC; ++k)
+      if (base + k < b) m = lf(m, acc_some(v[k]));
+    return m;
+  };
+  auto fetch = [&](const Int64 a, const Int64 b, const Int64 r, T (&v)[ACC_TVEC]) {
+    const Int64 base = a + r * round + (Int64)me * ACC_TVEC;
+#pragma unroll
+    for (int k = 0; k < ACC_TVEC; ++k) {
+      v[k] = T();
+      if (base + k < b) v[k] = get(base + k);
+    }
+  };
+  /* all lanes of the team, in order; uniform over the team (block teams: over the workgroup) */
+  auto team = [&](acc_opt<T> m) -> acc_opt<T> {
+    m = acc_wave_reduce(m, lf);
+    if (!block_team) return m;
+    if (acc_lane() == 0) s_wave[wave] = m;
+    __syncthreads();
+    acc_opt<T> r = s_wave[0];
+#pragma unroll
+    for (int w = 1; w < ACC_FS_WAVES; ++w) r = lf(r, s_wave[w]);
+    __syncthreads();
+    return r;
+  };
+
+  for (Int64 seg = team0; seg < nseg; seg += nteams) {
+    const Int64 a = (Int64)arrSeg_0[seg];
+    const Int64 b = acc_min<Int64>((Int64)arrSeg_0[seg + 1], n);
+    const Int64 nrounds = b > a ? (b - a + round - 1) / round : 0;
+    acc_opt<T> acc = acc_none<T>();
+#if ACC_HAS_SEED && ACC_FOLD_RIGHT
+    acc = acc_some(seed);
+#endif
+    for (Int64 r0 = 0; r0 < nrounds; r0 += ACC_TROUNDS) {
+      T v[ACC_TROUNDS][ACC_TVEC];
+#pragma unroll
+      for (int u = 0; u < ACC_TROUNDS; ++u) {
+        const Int64 r = ACC_FOLD_RIGHT ? nrounds - 1 - (r0 + u) : r0 + u;
+        if (r0 + u < nrounds) fetch(a, b, r, v[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < ACC_TROUNDS; ++u) {
+        const Int64 r = ACC_FOLD_RIGHT ? nrounds - 1 - (r0 + u) : r0 + u;
+        if (r0 + u < nrounds) {                                  /* uniform over the team */
+          const acc_opt<T> t = team(mine(a, b, r, v[u]));
+#if ACC_FOLD_RIGHT
+          acc = lf(t, acc);
+#else
+          acc = lf(acc, t);
+#endif
+        }
+      }
+    }
+    if (me == 0) {
+#if ACC_HAS_SEED && !ACC_FOLD_RIGHT
+      ACC_SET(arrOut, seg, acc.ok ? f(acc.v, seed) : seed);
+#else
+      ACC_SET(arrOut, seg, acc.v);      /* fold1Seg of an empty segment is undefined; T() is written */
 #endif
     }
   }

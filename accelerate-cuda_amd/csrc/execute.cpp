@@ -275,6 +275,22 @@ int acc_exec_foldseg(acc_skel s, const acc_array *env, int64_t n, const acc_arra
   args.ptr(offsets->ptr[0]);
   const int v = aligned ? 0 : 1;
   ACC_TRY(s->ensure_variant(v));
+  // Short segments: a lane per segment over chunks staged in LDS.  Long ones (on average: the lengths themselves are
+  // on the device) would serialise on that lane, so a wave, or from `foldseg.block_team_len` a workgroup, takes one
+  // segment at a time instead.
+  const int64_t avg = n / nseg;
+  if (avg >= acc::tune("foldseg.wave_team_len", 192)) {
+    const int block_team = avg >= acc::tune("foldseg.block_team_len", 16384) ? 1 : 0;
+    args.i32(block_team);
+    const int64_t per_block = block_team ? 1 : s->spec.block / 64;
+    const int64_t tgrid = acc_launch_grid(nseg, per_block, s->ctx->props.multiProcessorCount, 2048 / s->spec.block);
+    ACC_TRY(s->ctx->make_current());
+    hipError_t e = hipModuleLaunchKernel(s->variants[v].fn_finish, static_cast<unsigned>(tgrid), 1, 1,
+                                         static_cast<unsigned>(s->spec.block), 1, 1, 0, static_cast<hipStream_t>(stream),
+                                         args.data(), nullptr);
+    if (e != hipSuccess) return acc::fail_hip(e, "hipModuleLaunchKernel(foldSeg team)");
+    return ACC_OK;
+  }
   const int64_t grid = acc_launch_grid(nseg, s->spec.block, resident(s, v), acc::tune("foldseg.oversub", 1 << 20));
   return launch(s, v, grid, 0, static_cast<hipStream_t>(stream), &args);
 }

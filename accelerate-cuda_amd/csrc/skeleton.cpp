@@ -499,9 +499,10 @@ int acc_skel_s::ensure_variant(int v)
     var.module = nullptr;
     return acc::fail_hip(e, ("hipModuleGetFunction(" + entry + ")").c_str());
   }
+  const bool segmented = spec.kind == ACC_SKEL_FOLDSEG || spec.kind == ACC_SKEL_FOLD1SEG;
   const bool two_kernels = ((spec.kind == ACC_SKEL_FOLD || spec.kind == ACC_SKEL_FOLD1) && spec.out_rank == 0) ||
-                           (spec.kind == ACC_SKEL_PERMUTE && !spec.permute_locked);
-  const std::string second = entry + (spec.kind == ACC_SKEL_PERMUTE ? "_merge" : "_finish");
+                           (spec.kind == ACC_SKEL_PERMUTE && !spec.permute_locked) || segmented;
+  const std::string second = entry + (spec.kind == ACC_SKEL_PERMUTE ? "_merge" : segmented ? "_team" : "_finish");
   if (two_kernels) {
     e = hipModuleGetFunction(&var.fn_finish, var.module, second.c_str());
     if (e != hipSuccess) {

@@ -426,9 +426,11 @@ def test_smvm(A, ctx, orc, right):
         smvm.foldseg([ctx.array(vals), ctx.array(cols), ctx.array(x)], vals.size, ctx.array(offs), y)
         exp = orc.smvm_f32(vals, cols, offs, x, d)
         got = y.get()
-        # the segments are folded in index order, like the sequential interpreter: identical bits.
-        # (stated tolerance for this configuration: 1e-4 relative per row)
-        assert np.array_equal(got, exp)
+        # short segments (one lane each) are folded in index order with the sequential association: identical bits.
+        # Segments long on average go to a wave or a workgroup each: still index order, another association, so the
+        # last bits may differ.  (Stated tolerance for this configuration, checked below for both: 1e-4 relative per row.)
+        if vals.size // nrows < 192:
+            assert np.array_equal(got, exp)
         y64, yabs = orc.smvm_f64(vals, cols, offs, x)
         assert np.all(np.abs(got - y64) <= 1e-4 * np.maximum(np.abs(y64), 1e-3 * yabs) + 1e-30)
 
@@ -443,6 +445,47 @@ def test_foldseg_integers(A, ctx, orc):
         x = rng.integers(-1000, 1000, int(offs[-1]), dtype=np.int32)
         out = ctx.empty(nseg, np.int32)
         add.foldseg([ctx.array(x)], x.size, ctx.array(offs), out)
+        assert np.array_equal(out.get(), orc.foldseg(orc.OP_ADD, x, offs, seed=3))
+        lens1 = np.maximum(lens, 1)
+        offs1 = np.concatenate([[0], np.cumsum(lens1)]).astype(np.int32)
+        x1 = rng.integers(-1000, 1000, int(offs1[-1]), dtype=np.int32)
+        mx.foldseg([ctx.array(x1)], x1.size, ctx.array(offs1), out)
+        assert np.array_equal(out.get(), orc.foldseg(orc.OP_MAX, x1, offs1))
+
+
+def test_foldseg_long_segments_keep_index_order(A, ctx, orc):
+    """segments long on average go to a wave or a workgroup each: same results as the sequential fold, also for an
+    operator that is associative but not commutative, in both association directions, with empty segments between"""
+    first = ctx.skeleton(A.SKEL_FOLDSEG, "Int32", env=[I32], get="arrIn0_0[ix]", combine="x != 0 ? x : y", seed="-7")
+    last = ctx.skeleton(A.SKEL_FOLDSEG, "Int32", env=[I32], get="arrIn0_0[ix]", combine="y != 0 ? y : x", seed="0")
+    last_r = ctx.skeleton(A.SKEL_FOLDSEG, "Int32", env=[I32], get="arrIn0_0[ix]", combine="y != 0 ? y : x", seed="0",
+                          flags=A.FLAG_FOLD_RIGHT)
+    add = ctx.skeleton(A.SKEL_FOLDSEG, "Int32", env=[I32], get="arrIn0_0[ix]", combine="x + y", seed="3")
+    mx = ctx.skeleton(A.SKEL_FOLD1SEG, "Int32", env=[I32], get="arrIn0_0[ix]", combine="acc_max(x, y)")
+    for nseg, mean in [(300, 200), (2000, 1000), (37, 20000), (5, 300000), (1, 1 << 21)]:
+        say("foldSeg, long segments:", nseg, "of mean", mean)
+        lens = rng.poisson(mean, nseg).astype(np.int64)
+        lens[::7] = 0                                        # empty ones in between
+        lens[-1] = mean + 3
+        offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        n = int(offs[-1])
+        x = rng.integers(-3, 4, n, dtype=np.int32)
+        x[rng.random(n) < 0.9] = 0                          # mostly zeros: the first / last non-zero is somewhere inside
+        dx, doffs, out = ctx.array(x), ctx.array(offs), ctx.empty(nseg, np.int32)
+        exp_first = np.full(nseg, -7, np.int32)
+        exp_last = np.zeros(nseg, np.int32)
+        for k in range(nseg):
+            nz = np.flatnonzero(x[offs[k]:offs[k + 1]])
+            if nz.size:
+                exp_first[k] = x[offs[k] + nz[0]]
+                exp_last[k] = x[offs[k] + nz[-1]]
+        first.foldseg([dx], n, doffs, out)
+        assert np.array_equal(out.get(), exp_first)
+        last.foldseg([dx], n, doffs, out)
+        assert np.array_equal(out.get(), exp_last)
+        last_r.foldseg([dx], n, doffs, out)                  # x0 (+) (x1 (+) (... (+) z)): the same value, associated the other way
+        assert np.array_equal(out.get(), exp_last)
+        add.foldseg([dx], n, doffs, out)
         assert np.array_equal(out.get(), orc.foldseg(orc.OP_ADD, x, offs, seed=3))
         lens1 = np.maximum(lens, 1)
         offs1 = np.concatenate([[0], np.cumsum(lens1)]).astype(np.int32)
