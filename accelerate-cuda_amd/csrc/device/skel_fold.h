@@ -1,11 +1,11 @@
 /*
  * skel_fold.h -- fold / fold1: reduction of a whole array to one value
- * (entry foldAll / fold1All) and reduction along the innermost dimension of a
- * rank > 1 array (entry fold / fold1).
+ * (entry foldAll / fold1All).  Reduction along the innermost dimension of a
+ * rank > 1 array is skel_foldseg.h with segments of one length.
  *
  * Takes the place of CodeGen/Reduction.hs:87-215 (mkFoldAll: a first kernel
- * plus a recursive second one, Execute.hs:291-318) and :221-367 (mkFoldDim),
- * and of the shared-memory tree reducers at :616-699.
+ * plus a recursive second one, Execute.hs:291-318) and of the shared-memory
+ * tree reducers at :616-699.
  *
  * foldAll: every block strides over tiles of the (fused) input, each lane
  * reading ACC_UNROLL independent groups of ACC_VEC consecutive elements per
@@ -24,7 +24,7 @@
  *
  * Generated definitions expected: ACC_ENTRY, ACC_ELT, ACC_ENV_PARAMS,
  * ACC_ENV_ASSUME, ACC_GET(ix), ACC_COMBINE(x,y), ACC_HAS_SEED, ACC_SEED,
- * ACC_BLOCK, ACC_VEC, ACC_UNROLL, ACC_FOLD_DIM (0: foldAll, 1: innermost dim).
+ * ACC_BLOCK, ACC_VEC, ACC_UNROLL, ACC_FOLD_SINGLE.
  */
 
 #define ACC_TILE  (ACC_BLOCK * ACC_VEC * ACC_UNROLL)
@@ -46,8 +46,6 @@ ACC_DEV acc_opt<T> acc_block_reduce(acc_opt<T> x, F f, acc_opt<T> *s_wave)
   __syncthreads();
   return r;
 }
-
-#if !ACC_FOLD_DIM
 
 #if ACC_FOLD_SINGLE
 /* A value handed from one workgroup to another without fences: it is cut into
@@ -212,42 +210,3 @@ ACC_CAT(ACC_ENTRY, _finish)(ACC_ENV_PARAMS
   ACC_SET(arrOut, 0, total.v);
 #endif
 }
-
-#else  /* ACC_FOLD_DIM: one wave per innermost row ----------------------------- */
-
-/* rows are the innermost dimension; a wave strides over its row 64*ACC_VEC
- * elements at a time.  Output has one element per row.                       */
-extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
-ACC_ENTRY(ACC_ENV_PARAMS
-          const Int64 shOut_0, ACC_OUT_ARRAY(arrOut),
-          const Int64 shIn_1, const Int64 shIn_0)
-{
-  typedef ACC_ELT T;
-  ACC_ENV_ASSUME
-  (void)shOut_0;
-  auto get = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
-  auto f   = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
-  auto lf  = acc_lift<T>(f);
-
-  const int lane = acc_lane();
-  const Int64 rows = shIn_1, inner = shIn_0;
-  const Int64 wave0 = (Int64)blockIdx.x * ACC_WAVES + (threadIdx.x >> 6);
-  const Int64 nwaves = (Int64)gridDim.x * ACC_WAVES;
-
-  for (Int64 row = wave0; row < rows; row += nwaves) {
-    const Int64 start = row * inner;
-    acc_opt<T> mine = acc_none<T>();
-    for (Int64 i = lane; i < inner; i += ACC_WAVE) mine = lf(mine, acc_some(get(start + i)));
-    acc_opt<T> total = acc_wave_reduce(mine, lf);
-    if (lane == 0) {
-#if ACC_HAS_SEED
-      const T seed = (ACC_SEED);
-      ACC_SET(arrOut, row, total.ok ? f(total.v, seed) : seed);      /* Reduction.hs:351-362 */
-#else
-      ACC_SET(arrOut, row, total.v);
-#endif
-    }
-  }
-}
-
-#endif

@@ -28,10 +28,30 @@
 
 static_assert(ACC_CHUNK % (ACC_BLOCK * ACC_VEC) == 0, "chunk must be a whole number of block-wide vector loads");
 
+/* ACC_SEG_UNIFORM: the segments are the rows of a rank > 1 array, all of the same length -- `fold` / `fold1` along
+ * the innermost dimension (CodeGen/Reduction.hs:221-367, mkFoldDim) is this template with computed offsets.      */
+#ifndef ACC_SEG_UNIFORM
+#define ACC_SEG_UNIFORM 0
+#endif
+#if ACC_SEG_UNIFORM
+#if ACC_HAS_SEED
+#define ACC_FOLDSEG_ENTRY fold
+#else
+#define ACC_FOLDSEG_ENTRY fold1
+#endif
+/* (rows, row length) as the kernel parameters shIn_1, shIn_0 */
+#define ACC_SEG_PARAMS const Int64 shIn_1, const Int64 shIn_0
+#define ACC_SEG_TOTAL (shIn_1 * shIn_0)
+#define ACC_SEG_AT(s) ((Int64)(s) * shIn_0)
+#else
 #if ACC_HAS_SEED
 #define ACC_FOLDSEG_ENTRY foldSeg
 #else
 #define ACC_FOLDSEG_ENTRY fold1Seg
+#endif
+#define ACC_SEG_PARAMS const Int64 shIn_0, const ACC_SEG_TYPE *__restrict__ arrSeg_0
+#define ACC_SEG_TOTAL shIn_0
+#define ACC_SEG_AT(s) ((Int64)arrSeg_0[s])
 #endif
 
 #define ACC_LOADS (ACC_CHUNK / (ACC_BLOCK * ACC_VEC))   /* vector loads per lane and chunk */
@@ -43,8 +63,7 @@ static_assert(ACC_CHUNK % (ACC_BLOCK * ACC_VEC) == 0, "chunk must be a whole num
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
                   const Int64 shOut_0, ACC_OUT_ARRAY(arrOut),
-                  const Int64 shIn_0,
-                  const ACC_SEG_TYPE *__restrict__ arrSeg_0)
+                  ACC_SEG_PARAMS)
 {
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
@@ -54,7 +73,7 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
   auto f   = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
 
   const Int64 nseg = shOut_0;
-  const Int64 n = shIn_0;
+  const Int64 n = ACC_SEG_TOTAL;
   const int tid = threadIdx.x;
 #if ACC_HAS_SEED
   const T seed = (ACC_SEED);
@@ -63,10 +82,10 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
   for (Int64 first = (Int64)blockIdx.x * ACC_BLOCK; first < nseg; first += (Int64)gridDim.x * ACC_BLOCK) {
     const Int64 seg = first + tid;
     const bool live = seg < nseg;
-    const Int64 a = live ? (Int64)arrSeg_0[seg] : 0;
-    const Int64 b = live ? (Int64)arrSeg_0[seg + 1] : 0;
+    const Int64 a = live ? ACC_SEG_AT(seg) : 0;
+    const Int64 b = live ? ACC_SEG_AT(seg + 1) : 0;
     const Int64 last = acc_min<Int64>(first + ACC_BLOCK, nseg);
-    const Int64 lo = (Int64)arrSeg_0[first], hi = acc_min<Int64>((Int64)arrSeg_0[last], n);
+    const Int64 lo = ACC_SEG_AT(first), hi = acc_min<Int64>(ACC_SEG_AT(last), n);
 
     T acc = T();
     bool have = false;
@@ -160,7 +179,13 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
  * one on the proper side: the segment is still combined in index order, only
  * the association differs from the one-lane-per-segment entry, as the
  * operator's associativity allows.  ACC_TROUNDS rounds of loads are issued
- * before the first is used.                                                 */
+ * before the first is used.
+ *
+ * With fewer segments than the device has room for teams, every segment is
+ * cut into `split` consecutive pieces of equal length, each piece goes to
+ * a team that leaves its value (and whether the piece held anything) in
+ * `part` / `part_ok`, and <entry>_join puts the pieces of every segment
+ * together, in order.                                                        */
 #define ACC_TVEC 4
 #define ACC_TROUNDS 4
 #define ACC_FS_WAVES (ACC_BLOCK / ACC_WAVE)
@@ -170,9 +195,9 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _team)(ACC_ENV_PARAMS
                                      const Int64 shOut_0, ACC_OUT_ARRAY(arrOut),
-                                     const Int64 shIn_0,
-                                     const ACC_SEG_TYPE *__restrict__ arrSeg_0,
-                                     const int block_team)
+                                     ACC_SEG_PARAMS,
+                                     const int block_team, const Int64 split,
+                                     ACC_ELT *__restrict__ part, int *__restrict__ part_ok)
 {
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
@@ -183,7 +208,7 @@ ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _team)(ACC_ENV_PARAMS
   auto lf  = acc_lift<T>(f);
 
   const Int64 nseg = shOut_0;
-  const Int64 n = shIn_0;
+  const Int64 n = ACC_SEG_TOTAL;
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
   const int me = block_team ? tid : acc_lane();                    /* place in the team */
@@ -198,6 +223,12 @@ ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _team)(ACC_ENV_PARAMS
   /* the values of round `r` of [a, b) that fall to this lane, folded in order */
   auto mine = [&](const Int64 a, const Int64 b, const Int64 r, const T (&v)[ACC_TVEC]) -> acc_opt<T> {
     const Int64 base = a + r * round + (Int64)me * ACC_TVEC;
+    if (base + ACC_TVEC <= b) {                      /* all there: plain values */
+      T t = v[0];
+#pragma unroll
+      for (int k = 1; k < ACC_TVEC; ++k) t = f(t, v[k]);
+      return acc_some(t);
+    }
     acc_opt<T> m = acc_none<T>();
 #pragma unroll
     for (int k = 0; k < ACC_TVEC; ++k)
@@ -206,6 +237,11 @@ ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _team)(ACC_ENV_PARAMS
   };
   auto fetch = [&](const Int64 a, const Int64 b, const Int64 r, T (&v)[ACC_TVEC]) {
     const Int64 base = a + r * round + (Int64)me * ACC_TVEC;
+    if (base + ACC_TVEC <= b) {
+#pragma unroll
+      for (int k = 0; k < ACC_TVEC; ++k) v[k] = get(base + k);
+      return;
+    }
 #pragma unroll
     for (int k = 0; k < ACC_TVEC; ++k) {
       v[k] = T();
@@ -225,14 +261,16 @@ ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _team)(ACC_ENV_PARAMS
     return r;
   };
 
-  for (Int64 seg = team0; seg < nseg; seg += nteams) {
-    const Int64 a = (Int64)arrSeg_0[seg];
-    const Int64 b = acc_min<Int64>((Int64)arrSeg_0[seg + 1], n);
+  for (Int64 job = team0; job < nseg * split; job += nteams) {
+    const Int64 seg = job / split, part_no = job - seg * split;
+    const Int64 sa = ACC_SEG_AT(seg);
+    const Int64 sb = acc_min<Int64>(ACC_SEG_AT(seg + 1), n);
+    /* `split` pieces of equal length, whole rounds each so that only a segment's last piece is ragged */
+    const Int64 piece = (((sb - sa) + split - 1) / split + round - 1) / round * round;
+    const Int64 a = split > 1 ? acc_min<Int64>(sa + part_no * piece, sb) : sa;
+    const Int64 b = split > 1 ? acc_min<Int64>(a + piece, sb) : sb;
     const Int64 nrounds = b > a ? (b - a + round - 1) / round : 0;
     acc_opt<T> acc = acc_none<T>();
-#if ACC_HAS_SEED && ACC_FOLD_RIGHT
-    acc = acc_some(seed);
-#endif
     for (Int64 r0 = 0; r0 < nrounds; r0 += ACC_TROUNDS) {
       T v[ACC_TROUNDS][ACC_TVEC];
 #pragma unroll
@@ -253,12 +291,49 @@ ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _team)(ACC_ENV_PARAMS
         }
       }
     }
-    if (me == 0) {
-#if ACC_HAS_SEED && !ACC_FOLD_RIGHT
-      ACC_SET(arrOut, seg, acc.ok ? f(acc.v, seed) : seed);
-#else
-      ACC_SET(arrOut, seg, acc.v);      /* fold1Seg of an empty segment is undefined; T() is written */
-#endif
+    if (me != 0) continue;
+    if (split > 1) {
+      part[job] = acc.v;
+      part_ok[job] = acc.ok ? 1 : 0;
+      continue;
     }
+    /* (x0 (+) ... (+) x_last) (+) z in either association direction: the seed is the right operand */
+#if ACC_HAS_SEED
+    ACC_SET(arrOut, seg, acc.ok ? f(acc.v, seed) : seed);
+#else
+    ACC_SET(arrOut, seg, acc.v);        /* fold1Seg of an empty segment is undefined; T() is written */
+#endif
   }
+}
+
+/* the pieces of every segment, in order, and the seed: one wave per segment, every lane a run of
+ * consecutive pieces, the lanes combined in lane order */
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _join)(ACC_ENV_PARAMS
+                                     const Int64 shOut_0, ACC_OUT_ARRAY(arrOut), const Int64 split,
+                                     const ACC_ELT *__restrict__ part, const int *__restrict__ part_ok)
+{
+  typedef ACC_ELT T;
+  ACC_ENV_ASSUME
+  auto f  = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
+  auto lf = acc_lift<T>(f);
+  const int lane = acc_lane();
+  const Int64 seg = (Int64)blockIdx.x * ACC_FS_WAVES + (threadIdx.x >> 6);
+  if (seg >= shOut_0) return;                         /* whole waves leave */
+  const Int64 per = (split + ACC_WAVE - 1) / ACC_WAVE;
+  acc_opt<T> acc = acc_none<T>();
+  for (Int64 k = lane * per; k < acc_min<Int64>((lane + 1) * per, split); ++k) {
+    acc_opt<T> p;
+    p.v = part[seg * split + k];
+    p.ok = part_ok[seg * split + k] != 0;
+    acc = lf(acc, p);
+  }
+  acc = acc_wave_reduce(acc, lf);
+  if (lane != 0) return;
+#if ACC_HAS_SEED
+  const T seed = (ACC_SEED);
+  ACC_SET(arrOut, seg, acc.ok ? f(acc.v, seed) : seed);
+#else
+  ACC_SET(arrOut, seg, acc.v);
+#endif
 }

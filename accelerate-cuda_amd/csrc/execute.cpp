@@ -157,6 +157,74 @@ int acc_exec_map(acc_skel s, const acc_array *env, const acc_array *out, acc_str
   return launch(s, v, grid, 0, static_cast<hipStream_t>(stream), &args);
 }
 
+namespace {
+
+// The segmented fold over `nseg` segments holding `n` elements in all; `args` holds the kernel parameters up to and
+// including the segment description (offsets, or rows and row length).
+//   short segments: a lane per segment over chunks staged in LDS (skel_foldseg.h);
+//   long ones (on average: the lengths themselves are on the device) would serialise on that lane, so a wave, or
+//   from `foldseg.block_team_len` a workgroup, takes one segment at a time;
+//   fewer long segments than the device has room for teams: every segment is cut into `split` pieces, a team
+//   each, and a second launch joins the pieces in order.
+int launch_segmented(acc_skel_s *s, int v, Args *args, const acc_array *env, const acc_array *out, int64_t nseg, int64_t n,
+                     hipStream_t st)
+{
+  const int64_t avg = n / nseg;
+  if (avg < acc::tune("foldseg.wave_team_len", 192)) {
+    const int64_t grid = acc_launch_grid(nseg, s->spec.block, resident(s, v), acc::tune("foldseg.oversub", 1 << 20));
+    return launch(s, v, grid, 0, st, args);
+  }
+  const int block_team = avg >= acc::tune("foldseg.block_team_len", 16384) ? 1 : 0;
+  const int64_t cus = s->ctx->props.multiProcessorCount;
+  const int64_t team_lanes = block_team ? s->spec.block : 64;
+  const int64_t room = cus * (2048 / team_lanes);                    // teams the device holds at once
+  const int64_t min_piece = team_lanes * 64;                          // a piece keeps its team busy for a while
+  int64_t split = 1;
+  if (nseg * 2 <= room) split = std::max<int64_t>(1, std::min<int64_t>({room / nseg, avg / min_piece, acc::tune("foldseg.max_split", 4096)}));
+  int blk = -1;
+  uint64_t part = 0, part_ok = 0;
+  if (split > 1) {
+    const size_t jobs = (size_t)(nseg * split);
+    const size_t ok_off = round256(jobs * s->spec.elt_size);
+    ACC_TRY(s->ctx->scratch_acquire(ok_off + jobs * 4, st, acc::SCRATCH_FOLD, &blk));
+    part = reinterpret_cast<uint64_t>(s->ctx->scratch[blk].ptr);
+    part_ok = part + ok_off;
+  }
+  args->i32(block_team);
+  args->i64(split);
+  args->ptr(part);
+  args->ptr(part_ok);
+  const int64_t per_block = block_team ? 1 : s->spec.block / 64;
+  const int64_t tgrid = acc_launch_grid(nseg * split, per_block, cus, 2048 / s->spec.block);
+  int rc = s->ctx->make_current();
+  if (rc == ACC_OK) {
+    hipError_t e = hipModuleLaunchKernel(s->variants[v].fn_finish, static_cast<unsigned>(tgrid), 1, 1,
+                                         static_cast<unsigned>(s->spec.block), 1, 1, 0, st, args->data(), nullptr);
+    if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(segmented fold, team)");
+  }
+  if (rc == ACC_OK && split > 1) {
+    Args join;
+    bool al = true;
+    rc = push_env(s, env, &join, &al);
+    join.i64(nseg);
+    push_ptrs(out, out->ncomp, &join, &al);
+    join.i64(split);
+    join.ptr(part);
+    join.ptr(part_ok);
+    if (rc == ACC_OK) {
+      const int64_t waves = s->spec.block / 64;
+      const int64_t jgrid = (nseg + waves - 1) / waves;          // a wave per segment
+      hipError_t e = hipModuleLaunchKernel(s->variants[v].fn_fill, static_cast<unsigned>(jgrid), 1, 1,
+                                           static_cast<unsigned>(s->spec.block), 1, 1, 0, st, join.data(), nullptr);
+      if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(segmented fold, join)");
+    }
+  }
+  if (blk >= 0) s->ctx->scratch_release(blk, st);
+  return rc;
+}
+
+}  // namespace
+
 int acc_exec_fold(acc_skel s, const acc_array *env, int32_t in_rank, const int64_t *in_shape, const acc_array *out, acc_stream stream)
 {
   if (!s) return fail(ACC_ERR_INVALID, "acc_exec_fold: NULL skeleton");
@@ -180,14 +248,17 @@ int acc_exec_fold(acc_skel s, const acc_array *env, int32_t in_rank, const int64
   const int v = aligned ? 0 : 1;
   ACC_TRY(s->ensure_variant(v));
 
-  if (s->spec.out_rank > 0) {      // one wave per innermost row
+  if (s->spec.out_rank > 0) {      // along the innermost dimension: a segmented fold over rows of one length
     args.i64(rows);
     push_ptrs(out, out->ncomp, &args, &aligned);
     args.i64(rows);
     args.i64(inner);
-    const int waves = s->spec.block / 64;
-    const int64_t grid = acc_launch_grid(rows, waves, resident(s, v), 4);
-    return launch(s, v, grid, 0, st, &args);
+    if (inner == 0) {
+      // rows without elements: every result is the seed; the one-lane-per-row entry does that
+      const int64_t grid = acc_launch_grid(rows, s->spec.block, resident(s, v), 1 << 20);
+      return launch(s, v, grid, 0, st, &args);
+    }
+    return launch_segmented(s, v, &args, env, out, rows, rows * inner, st);
   }
 
   const int64_t n = inner;
@@ -275,24 +346,7 @@ int acc_exec_foldseg(acc_skel s, const acc_array *env, int64_t n, const acc_arra
   args.ptr(offsets->ptr[0]);
   const int v = aligned ? 0 : 1;
   ACC_TRY(s->ensure_variant(v));
-  // Short segments: a lane per segment over chunks staged in LDS.  Long ones (on average: the lengths themselves are
-  // on the device) would serialise on that lane, so a wave, or from `foldseg.block_team_len` a workgroup, takes one
-  // segment at a time instead.
-  const int64_t avg = n / nseg;
-  if (avg >= acc::tune("foldseg.wave_team_len", 192)) {
-    const int block_team = avg >= acc::tune("foldseg.block_team_len", 16384) ? 1 : 0;
-    args.i32(block_team);
-    const int64_t per_block = block_team ? 1 : s->spec.block / 64;
-    const int64_t tgrid = acc_launch_grid(nseg, per_block, s->ctx->props.multiProcessorCount, 2048 / s->spec.block);
-    ACC_TRY(s->ctx->make_current());
-    hipError_t e = hipModuleLaunchKernel(s->variants[v].fn_finish, static_cast<unsigned>(tgrid), 1, 1,
-                                         static_cast<unsigned>(s->spec.block), 1, 1, 0, static_cast<hipStream_t>(stream),
-                                         args.data(), nullptr);
-    if (e != hipSuccess) return acc::fail_hip(e, "hipModuleLaunchKernel(foldSeg team)");
-    return ACC_OK;
-  }
-  const int64_t grid = acc_launch_grid(nseg, s->spec.block, resident(s, v), acc::tune("foldseg.oversub", 1 << 20));
-  return launch(s, v, grid, 0, static_cast<hipStream_t>(stream), &args);
+  return launch_segmented(s, v, &args, env, out, nseg, n, static_cast<hipStream_t>(stream));
 }
 
 int acc_exec_scan(acc_skel s, const acc_array *env, int64_t n, const acc_array *out, const acc_array *total, acc_stream stream)

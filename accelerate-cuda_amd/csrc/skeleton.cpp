@@ -193,9 +193,16 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       break;
     case ACC_SKEL_FOLD:
     case ACC_SKEL_FOLD1:
-      if (sp.out_rank == 0) *entry = sp.has_seed ? "foldAll" : "fold1All";
-      else *entry = sp.has_seed ? "fold" : "fold1";
-      o << "#define ACC_FOLD_DIM " << (sp.out_rank == 0 ? 0 : 1) << "\n";
+      if (sp.out_rank > 0) {
+        // along the innermost dimension: the segmented fold over rows of one length
+        *entry = sp.has_seed ? "fold" : "fold1";
+        o << "#define ACC_SEG_UNIFORM 1\n";
+        o << "#define ACC_FOLD_RIGHT " << ((sp.flags & ACC_FLAG_FOLD_RIGHT) ? 1 : 0) << "\n";
+        o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_CHUNK " << sp.chunk << "\n";
+        tmpl = "skel_foldseg.h";
+        break;
+      }
+      *entry = sp.has_seed ? "foldAll" : "fold1All";
       o << "#define ACC_FOLD_SINGLE " << tune("fold.single", 1) << "\n";
       o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_UNROLL " << sp.unroll << "\n";
       tmpl = "skel_fold.h";
@@ -392,6 +399,10 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
     case ACC_SKEL_FOLD: case ACC_SKEL_FOLD1:
       sp->block = tune("fold.block", 256);
       sp->unroll = tune("fold.unroll", 4);
+      if (sp->out_rank > 0) {
+        sp->block = tune("foldseg.block", 256);
+        sp->chunk = tune("foldseg.chunk", 2048);
+      }
       break;
     case ACC_SKEL_FOLDSEG: case ACC_SKEL_FOLD1SEG:
       sp->block = tune("foldseg.block", 256);
@@ -499,7 +510,8 @@ int acc_skel_s::ensure_variant(int v)
     var.module = nullptr;
     return acc::fail_hip(e, ("hipModuleGetFunction(" + entry + ")").c_str());
   }
-  const bool segmented = spec.kind == ACC_SKEL_FOLDSEG || spec.kind == ACC_SKEL_FOLD1SEG;
+  const bool segmented = spec.kind == ACC_SKEL_FOLDSEG || spec.kind == ACC_SKEL_FOLD1SEG ||
+                         ((spec.kind == ACC_SKEL_FOLD || spec.kind == ACC_SKEL_FOLD1) && spec.out_rank > 0);
   const bool two_kernels = ((spec.kind == ACC_SKEL_FOLD || spec.kind == ACC_SKEL_FOLD1) && spec.out_rank == 0) ||
                            (spec.kind == ACC_SKEL_PERMUTE && !spec.permute_locked) || segmented;
   const std::string second = entry + (spec.kind == ACC_SKEL_PERMUTE ? "_merge" : segmented ? "_team" : "_finish");
@@ -511,12 +523,13 @@ int acc_skel_s::ensure_variant(int v)
       return acc::fail_hip(e, ("hipModuleGetFunction(" + second + ")").c_str());
     }
   }
-  if (spec.kind == ACC_SKEL_PERMUTE && !spec.permute_locked) {
-    e = hipModuleGetFunction(&var.fn_fill, var.module, (entry + "_fill").c_str());
+  if ((spec.kind == ACC_SKEL_PERMUTE && !spec.permute_locked) || segmented) {
+    const std::string third = entry + (segmented ? "_join" : "_fill");
+    e = hipModuleGetFunction(&var.fn_fill, var.module, third.c_str());
     if (e != hipSuccess) {
       (void)hipModuleUnload(var.module);
       var.module = nullptr;
-      return acc::fail_hip(e, ("hipModuleGetFunction(" + entry + "_fill)").c_str());
+      return acc::fail_hip(e, ("hipModuleGetFunction(" + third + ")").c_str());
     }
   }
   (void)hipFuncGetAttribute(&var.num_regs, HIP_FUNC_ATTRIBUTE_NUM_REGS, var.fn);

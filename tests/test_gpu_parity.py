@@ -462,7 +462,7 @@ def test_foldseg_long_segments_keep_index_order(A, ctx, orc):
                           flags=A.FLAG_FOLD_RIGHT)
     add = ctx.skeleton(A.SKEL_FOLDSEG, "Int32", env=[I32], get="arrIn0_0[ix]", combine="x + y", seed="3")
     mx = ctx.skeleton(A.SKEL_FOLD1SEG, "Int32", env=[I32], get="arrIn0_0[ix]", combine="acc_max(x, y)")
-    for nseg, mean in [(300, 200), (2000, 1000), (37, 20000), (5, 300000), (1, 1 << 21)]:
+    for nseg, mean in [(300, 200), (2000, 1000), (37, 20000), (5, 300000), (1, 1 << 21), (3, 5000), (100, 3000)]:
         say("foldSeg, long segments:", nseg, "of mean", mean)
         lens = rng.poisson(mean, nseg).astype(np.int64)
         lens[::7] = 0                                        # empty ones in between
@@ -492,6 +492,34 @@ def test_foldseg_long_segments_keep_index_order(A, ctx, orc):
         x1 = rng.integers(-1000, 1000, int(offs1[-1]), dtype=np.int32)
         mx.foldseg([ctx.array(x1)], x1.size, ctx.array(offs1), out)
         assert np.array_equal(out.get(), orc.foldseg(orc.OP_MAX, x1, offs1))
+
+
+def test_fold_along_the_innermost_dimension_at_every_shape(A, ctx):
+    """rows of 1 to 2^20 elements, 2^20 rows to one: a lane, a wave, a workgroup or several workgroups per row"""
+    add = ctx.skeleton(A.SKEL_FOLD, "Int32", env=[(2, "Int32")], out_rank=1, get="arrIn0_0[ix]", combine="x + y", seed="5")
+    first = ctx.skeleton(A.SKEL_FOLD1, "Int32", env=[(2, "Int32")], out_rank=1, get="arrIn0_0[ix]", combine="x != 0 ? x : y")
+    add3 = ctx.skeleton(A.SKEL_FOLD, "Int64", env=[(3, "Int32")], out_rank=2, get="(Int64)arrIn0_0[ix]", combine="x + y", seed="0")
+    for rows, inner in [(1 << 18, 1), (70001, 3), (40000, 31), (9999, 64), (3000, 191), (3000, 193), (700, 1000), (129, 16384),
+                        (33, 40001), (7, 300007), (2, 1 << 20), (1, (1 << 21) + 5)]:
+        say("fold of a", rows, "x", inner, "array")
+        x = rng.integers(-5, 6, (rows, inner), dtype=np.int32)
+        x[rng.random((rows, inner)) < 0.8] = 0
+        dx, out = ctx.array(x), ctx.empty(rows, np.int32)
+        add.fold([dx], (rows, inner), out)
+        assert np.array_equal(out.get(), x.sum(axis=1, dtype=np.int32) + 5)
+        first.fold([dx], (rows, inner), out)                    # associative, not commutative: index order must be kept
+        nz = x != 0
+        exp = np.where(nz.any(axis=1), x[np.arange(rows), nz.argmax(axis=1)], 0).astype(np.int32)
+        assert np.array_equal(out.get(), exp)
+    say("fold of a rank-3 array")
+    x = rng.integers(-1000, 1000, (6, 50, 700), dtype=np.int32)
+    out = ctx.empty((6, 50), np.int64)
+    add3.fold([ctx.array(x)], x.shape, out)
+    assert np.array_equal(out.get(), x.sum(axis=2, dtype=np.int64))
+    say("rows without elements yield the seed")
+    out = ctx.empty(17, np.int32)
+    add.fold([ctx.empty((17, 0), np.int32)], (17, 0), out)
+    assert np.array_equal(out.get(), np.full(17, 5, np.int32))
 
 
 # --------------------------------------------------------------------------- committed fixtures
