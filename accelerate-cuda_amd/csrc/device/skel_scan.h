@@ -112,24 +112,6 @@ struct acc_scan_desc<T, false> {
   }
 };
 
-/* ---- full tiles carry plain values, the one ragged tile carries optional
- *      values so that elements past the end are transparent ---------------- */
-template <typename T, bool PARTIAL> struct acc_sv;
-template <typename T> struct acc_sv<T, false> {
-  typedef T V;
-  static ACC_DEV V some(const T &x) { return x; }
-  static ACC_DEV V none() { return T(); }
-  static ACC_DEV T val(const V &v) { return v; }
-  template <typename F> static ACC_DEV F lift(F f) { return f; }
-};
-template <typename T> struct acc_sv<T, true> {
-  typedef acc_opt<T> V;
-  static ACC_DEV V some(const T &x) { return acc_some(x); }
-  static ACC_DEV V none() { return acc_none<T>(); }
-  static ACC_DEV T val(const V &v) { return v.v; }
-  template <typename F> static ACC_DEV acc_lifted<T, F> lift(F f) { return acc_lift<T>(f); }
-};
-
 /* ---- decoupled look-back, executed by wave 0 of a tile > 0 ---------------
  * Every step inspects ACC_LOOKBACK descriptors per lane, 64 * ACC_LOOKBACK
  * predecessors in one memory round trip.  The chain of tiles can advance by
@@ -217,7 +199,7 @@ ACC_DEV Int64 acc_scan_ix0(const Int64 base, const int wave, const int lane, con
 template <typename T, typename Get>
 ACC_DEV void acc_scan_load(Get get, const Int64 base, const Int64 n, T (&x)[ACC_ROWS][ACC_VEC], const int wave, const int lane)
 {
-  if (base + ACC_TILE <= n) {
+  if (base >= 0 && base + ACC_TILE <= n) {
 #pragma unroll
     for (int r = 0; r < ACC_ROWS; ++r) {
       const Int64 i0 = acc_scan_ix0(base, wave, lane, r);
@@ -225,14 +207,23 @@ ACC_DEV void acc_scan_load(Get get, const Int64 base, const Int64 n, T (&x)[ACC_
       for (int k = 0; k < ACC_VEC; ++k) x[r][k] = get(ACC_SCAN_RIGHT ? i0 - k : i0 + k);
     }
   } else {
+    /* a tile that reaches outside the array: vectors that lie inside are read as in a full tile (one 128-bit
+     * access), the one across the edge element by element, those outside not at all -- a tile read and written
+     * element by element takes three times as long as a full one, and it is the last one to finish */
 #pragma unroll
     for (int r = 0; r < ACC_ROWS; ++r) {
       const Int64 i0 = acc_scan_ix0(base, wave, lane, r);
+      const Int64 lo = ACC_SCAN_RIGHT ? i0 - (ACC_VEC - 1) : i0;
+      if (lo >= 0 && lo + ACC_VEC <= n) {
 #pragma unroll
-      for (int k = 0; k < ACC_VEC; ++k) {
-        const Int64 ix = ACC_SCAN_RIGHT ? i0 - k : i0 + k;
-        x[r][k] = T();
-        if (ix < n) x[r][k] = get(ix);
+        for (int k = 0; k < ACC_VEC; ++k) x[r][k] = get(ACC_SCAN_RIGHT ? i0 - k : i0 + k);
+      } else {
+#pragma unroll
+        for (int k = 0; k < ACC_VEC; ++k) {
+          /* outside the array: its nearest element instead; the value never reaches a result */
+          const Int64 ix = ACC_SCAN_RIGHT ? i0 - k : i0 + k;
+          x[r][k] = get(acc_max<Int64>(0, acc_min<Int64>(ix, n - 1)));
+        }
       }
     }
   }
@@ -240,15 +231,28 @@ ACC_DEV void acc_scan_load(Get get, const Int64 base, const Int64 n, T (&x)[ACC_
 
 /* scan one tile whose elements are already in registers.  `prefetch` is
  * called once the block total is known and before the look-back starts: the
- * caller uses it to put the next tile's loads in flight behind the wait.     */
-template <bool PARTIAL, typename T, typename Op, typename Prefetch, typename Out>
-ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op_raw, const T seed, const Int64 tile, const Int64 base,
+ * caller uses it to put the next tile's loads in flight behind the wait.
+ *
+ * GUARD: the tile reaches outside the array.  Tiles are laid so that the
+ * positions outside come LAST in scan order (left-handed scans count tiles
+ * from element 0, right-handed ones from the end of the array rounded up to a
+ * whole vector): whatever stands there only enters results that are never
+ * stored and an aggregate no other tile reads, so the same code runs on it,
+ * with the stores guarded.  The one exception is the rounding of a
+ * right-handed scan: up to ACC_VEC - 1 positions past the end come FIRST, in
+ * the first vector of the first tile, and the lane that holds them starts its
+ * own scan at the first element inside (`lead` below).                       */
+template <bool GUARD, typename T, typename Op, typename Prefetch, typename Out>
+ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op, const T seed, const Int64 tile, const Int64 base,
                            const Int64 n, const Out &out, const acc_scan_desc<T> &desc,
                            const unsigned int epoch, void *s_wave_raw, T *s_prefix, Prefetch prefetch)
 {
-  typedef acc_sv<T, PARTIAL> S;
-  typedef typename S::V V;
-  auto op = S::lift(op_raw);
+  typedef T V;
+  struct S {
+    static ACC_DEV V some(const T &v) { return v; }
+    static ACC_DEV T val(const V &v) { return v; }
+  };
+  auto op_raw = op;
 
   const int lane = acc_lane();
   const int wave = (int)(threadIdx.x >> 6);
@@ -257,14 +261,15 @@ ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op_raw, const T s
   /* scan the ACC_VEC items each lane holds per row */
   V s[ACC_ROWS][ACC_VEC];
   Int64 ix0[ACC_ROWS];
+  int lead[ACC_ROWS];                       /* positions past the end that come first in this lane's vector */
 #pragma unroll
   for (int r = 0; r < ACC_ROWS; ++r) {
     ix0[r] = acc_scan_ix0(base, wave, lane, r);
+    lead[r] = (GUARD && ACC_SCAN_RIGHT) ? (int)acc_max<Int64>(0, acc_min<Int64>(ix0[r] - (n - 1), ACC_VEC - 1)) : 0;
 #pragma unroll
     for (int k = 0; k < ACC_VEC; ++k) {
-      const Int64 ix = ACC_SCAN_RIGHT ? ix0[r] - k : ix0[r] + k;
-      V v = (!PARTIAL || ix < n) ? S::some(x[r][k]) : S::none();
-      s[r][k] = (k == 0) ? v : op(s[r][k - 1], v);
+      const V v = x[r][k];
+      s[r][k] = (k == 0 || (GUARD && ACC_SCAN_RIGHT && k == lead[r])) ? v : op(s[r][k - 1], v);
     }
   }
 
@@ -335,13 +340,25 @@ ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op_raw, const T s
     for (int k = 0; k < ACC_VEC; ++k) inc[k] = has_pre ? op(pre, s[r][k]) : s[r][k];
 
     /* the body: one straight run of stores per row so that they merge into
-     * 128-bit accesses */
+     * 128-bit accesses; in a tile that reaches outside the array only for the
+     * vectors that lie inside it */
     const bool exclusive = (ACC_SCAN_MODE == 0 || ACC_SCAN_MODE == 2);
+    const Int64 lo = ACC_SCAN_RIGHT ? ix0[r] - (ACC_VEC - 1) : ix0[r];
+    if (!GUARD || (lo >= 0 && lo + ACC_VEC <= n)) {
 #pragma unroll
-    for (int k = 0; k < ACC_VEC; ++k) {
-      const Int64 ix = ACC_SCAN_RIGHT ? ix0[r] - k : ix0[r] + k;
-      if (PARTIAL && ix >= n) continue;
-      out.put(ix, exclusive ? S::val(k == 0 ? pre : inc[k - 1]) : S::val(inc[k]));
+      for (int k = 0; k < ACC_VEC; ++k) {
+        const Int64 ix = ACC_SCAN_RIGHT ? ix0[r] - k : ix0[r] + k;
+        out.put(ix, exclusive ? S::val(k == 0 ? pre : inc[k - 1]) : S::val(inc[k]));
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < ACC_VEC; ++k) {
+        const Int64 ix = ACC_SCAN_RIGHT ? ix0[r] - k : ix0[r] + k;
+        if (ix < 0 || ix >= n) continue;
+        const bool first = (k == 0) || (ACC_SCAN_RIGHT && k == lead[r]);
+        const V before = (k == 0) ? pre : (first ? pre : inc[k - 1]);     /* (k == 0 keeps inc[-1] out of the expression) */
+        out.set(ix, exclusive ? S::val(before) : S::val(inc[k]));
+      }
     }
 
     /* the reduction of the whole vector, held by the logically last element */
@@ -356,107 +373,6 @@ ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op_raw, const T s
         }
       }
     }
-  }
-}
-
-/* The one ragged tile of a scan (elements past the end are transparent).  It
- * does the same job as acc_scan_tile<true> but keeps almost nothing live:
- * the per-row scans are simply done twice, once to get the totals and once,
- * when the prefix is known, to produce the results.  Speed is irrelevant
- * here (at most one such tile per launch); what matters is that its register
- * footprint does not dictate the kernel's.                                   */
-template <typename T, typename Op, typename Prefetch, typename Out>
-ACC_DEV void acc_scan_tile_ragged(const T (&x)[ACC_ROWS][ACC_VEC], Op op_raw, const T seed, const Int64 tile,
-                                  const Int64 base, const Int64 n, const Out &out,
-                                  const acc_scan_desc<T> &desc, const unsigned int epoch, void *s_wave_raw,
-                                  T *s_prefix, Prefetch prefetch)
-{
-  typedef acc_opt<T> V;
-  auto op = acc_lift<T>(op_raw);
-  const int lane = acc_lane();
-  const int wave = (int)(threadIdx.x >> 6);
-  V *s_wave = (V *)s_wave_raw;
-
-  auto item = [&](const int r, const int k) -> V {
-    const Int64 i0 = acc_scan_ix0(base, wave, lane, r);
-    const Int64 ix = ACC_SCAN_RIGHT ? i0 - k : i0 + k;
-    V v;
-    v.v = x[r][k];
-    v.ok = (ix < n);
-    return v;
-  };
-  auto lane_total = [&](const int r) -> V {
-    V t = item(r, 0);
-#pragma unroll
-    for (int k = 1; k < ACC_VEC; ++k) t = op(t, item(r, k));
-    return t;
-  };
-
-  /* pass 1: total of this wave */
-  V wave_total = acc_none<T>();
-#pragma unroll 1
-  for (int r = 0; r < ACC_ROWS; ++r) {
-    const V ci = acc_wave_scan(lane_total(r), op, lane);
-    wave_total = op(wave_total, acc_readlane(ci, ACC_WAVE - 1));
-  }
-  if (lane == 0) s_wave[wave] = wave_total;
-  __syncthreads();
-  V wavepre = acc_none<T>();
-  V block_total = acc_none<T>();
-#pragma unroll 1
-  for (int w = 0; w < ACC_WAVES; ++w) {
-    if (w == wave) wavepre = block_total;
-    block_total = op(block_total, s_wave[w]);
-  }
-
-  T prefix = seed;
-  bool has_prefix = ACC_HAS_SEED;
-  if (tile == 0) {
-    if (threadIdx.x == 0)
-      desc.put(0, (epoch << 2) | ACC_ST_PREFIX, ACC_HAS_SEED ? op_raw(seed, block_total.v) : block_total.v);
-    prefetch();
-  } else {
-    if (threadIdx.x == 0) desc.put(tile, (epoch << 2) | ACC_ST_AGGREGATE, block_total.v);
-    acc_scan_window<T> win;
-    if (wave == 0) acc_scan_window_load(desc, tile - 1, lane, win);
-    prefetch();
-    if (wave == 0) {
-      const T p = acc_scan_lookback(desc, tile, block_total.v, op_raw, epoch, lane, win);
-      if (lane == 0) *s_prefix = p;
-    }
-    __syncthreads();
-    prefix = *s_prefix;
-    has_prefix = true;
-  }
-
-  /* pass 2: redo the row scans, now with everything before them known */
-  V run;                                      /* everything before the current row */
-  run.v = prefix;
-  run.ok = has_prefix;
-  run = op(run, wavepre);
-  const Int64 last = ACC_SCAN_RIGHT ? 0 : n - 1;
-#pragma unroll 1
-  for (int r = 0; r < ACC_ROWS; ++r) {
-    const V ci = acc_wave_scan(lane_total(r), op, lane);
-    V e = acc_wave_shift_up1(ci);
-    if (lane == 0) e = acc_none<T>();
-    V acc = op(run, e);                       /* everything before this lane's first item */
-    const Int64 i0 = acc_scan_ix0(base, wave, lane, r);
-#pragma unroll
-    for (int k = 0; k < ACC_VEC; ++k) {
-      const Int64 ix = ACC_SCAN_RIGHT ? i0 - k : i0 + k;
-      const V before = acc;
-      acc = op(acc, item(r, k));
-      if (ix < n) {
-        const bool exclusive = (ACC_SCAN_MODE == 0 || ACC_SCAN_MODE == 2);
-        out.set(ix, exclusive ? before.v : acc.v);
-        if (ix == last) {
-          if (ACC_SCAN_MODE == 0) out.set(n, acc.v);
-          if (ACC_SCAN_MODE == 2) out.total(acc.v);
-        }
-      }
-    }
-    run = op(run, acc_readlane(ci, ACC_WAVE - 1));
   }
 }
 
@@ -514,7 +430,10 @@ ACC_ENTRY(ACC_ENV_PARAMS
   auto set_fn   = [&](const Int64 ix, const T &v) { ACC_SET(arrOut, ix, v); };
   auto total_fn = [&](const T &v) { ACC_SET(arrSum, 0, v); };
   const acc_scan_out<decltype(put_fn), decltype(set_fn), decltype(total_fn)> out = {put_fn, set_fn, total_fn};
-  auto tile_base = [&](const Int64 t) -> Int64 { return (ACC_SCAN_RIGHT ? (num_tiles - 1 - t) : t) * (Int64)ACC_TILE; };
+  /* first physical index of scan tile t (right-handed: tiles count down from the end of the array, rounded up to a
+   * whole vector so that the 128-bit accesses stay aligned; the last tile may start below 0) */
+  const Int64 n_up = (n + ACC_VEC - 1) / ACC_VEC * ACC_VEC;
+  auto tile_base = [&](const Int64 t) -> Int64 { return ACC_SCAN_RIGHT ? n_up - (t + 1) * (Int64)ACC_TILE : t * (Int64)ACC_TILE; };
 
 #if ACC_SCAN_PERSISTENT == 1
   __shared__ unsigned int s_ticket[4];
@@ -570,10 +489,10 @@ ACC_ENTRY(ACC_ENV_PARAMS
 #endif
 
     const Int64 base = tile_base(tile);
-    if (base + ACC_TILE <= n)
+    if (base >= 0 && base + ACC_TILE <= n)
       acc_scan_tile<false, T>(cur, op, seed, tile, base, n, out, desc, epoch, (void *)s_wave, &s_prefix, prefetch);
     else
-      acc_scan_tile_ragged<T>(cur, op, seed, tile, base, n, out, desc, epoch, (void *)s_wave, &s_prefix, prefetch);
+      acc_scan_tile<true, T>(cur, op, seed, tile, base, n, out, desc, epoch, (void *)s_wave, &s_prefix, prefetch);
 
 #if ACC_SCAN_PERSISTENT
 #pragma unroll
