@@ -140,15 +140,25 @@ ACC_ENTRY(ACC_ENV_PARAMS
     mine = acc_some(v);
   }
 
-  /* the ragged last tile, taken by whichever block it falls to */
-  if (full_tiles * (Int64)ACC_TILE < n && (Int64)blockIdx.x == full_tiles % gridDim.x) {
+  /* the ragged last tile, taken by whichever block it falls to ...
+   * but not by the last block of a larger grid, which collects the partial results and should not be late */
+  Int64 ragged_owner = full_tiles % gridDim.x;
+  if (gridDim.x > 1 && ragged_owner == (Int64)gridDim.x - 1) ragged_owner = 0;
+  if (full_tiles * (Int64)ACC_TILE < n && (Int64)blockIdx.x == ragged_owner) {
     const Int64 base = full_tiles * (Int64)ACC_TILE + (Int64)threadIdx.x * ACC_VEC;
+    /* every load is issued before any value is used: positions past the end read the last element instead and are
+     * left out below (a load under `if (ix < n)` waits for its result inside the branch, one round trip each) */
+    T v[ACC_UNROLL][ACC_VEC];
+#pragma unroll
+    for (int u = 0; u < ACC_UNROLL; ++u)
+#pragma unroll
+      for (int k = 0; k < ACC_VEC; ++k) v[u][k] = get(acc_min<Int64>(base + u * (ACC_BLOCK * ACC_VEC) + k, n - 1));
 #pragma unroll
     for (int u = 0; u < ACC_UNROLL; ++u)
 #pragma unroll
       for (int k = 0; k < ACC_VEC; ++k) {
         const Int64 ix = base + u * (ACC_BLOCK * ACC_VEC) + k;
-        if (ix < n) mine = lf(mine, acc_some(get(ix)));
+        if (ix < n) mine = lf(mine, acc_some(v[u][k]));
       }
   }
 
