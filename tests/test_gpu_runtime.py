@@ -220,3 +220,15 @@ def test_one_skeleton_launched_from_several_threads(A, ctx):
         t.join()
     assert not errors, errors
     assert results == {0: True, 1: True, 2: True, 3: True}
+
+
+def test_the_c_client_of_the_abi():
+    """tests/c_abi/client.c: the benchmark programs and the memory table from plain C, checked against loops in C"""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "c_abi", "client")
+    assert os.path.exists(exe), "build it first: make -C tests/c_abi (or __graft_entry__.build())"
+    say("C client")
+    out = subprocess.run([exe], capture_output=True, text=True, timeout=300)
+    print(out.stdout)
+    assert out.returncode == 0 and "all checks passed" in out.stdout, out.stdout + out.stderr

@@ -310,3 +310,13 @@ def test_workload_module_is_pure_numpy():
     vals, cols, offs, lens, xv = wl.smvm_inputs(nrows=500, mean_len=8, ncols=64)
     assert offs[0] == 0 and offs[-1] == vals.size == cols.size and np.array_equal(np.diff(offs), lens)
     assert cols.min() >= 0 and cols.max() < 64 and xv.size == 64
+
+
+def test_c_client_builds_as_c99_and_runs_its_deviceless_part():
+    """include/acc_hip.h is a C header: a C99 program (-pedantic -Werror) includes it, links the library and drives
+    generation and compilation through it"""
+    import subprocess
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "c_abi")
+    subprocess.check_call(["make", "-C", here], stdout=subprocess.DEVNULL)
+    out = subprocess.run([os.path.join(here, "client"), "--no-gpu"], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0 and "all checks passed" in out.stdout, out.stdout + out.stderr
