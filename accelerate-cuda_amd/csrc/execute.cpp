@@ -467,7 +467,15 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
   };
   if (n_src == 0 || ntarget == 0) return plain_copy();
 
-  if (s->spec.permute_locked) {
+  // A combination without an atomic instruction of its own on few targets: compare-and-swap loops on the result
+  // meet on those few addresses (16 M Float32 `max` updates on 1000 targets: 16.6 ms), the tables in LDS of the
+  // locked template do not (74 us).  Such a skeleton carries that template as its variants 2 and 3.
+  const int64_t lds_all = std::min<int64_t>((int64_t)s->ctx->props.sharedMemPerBlock, acc::tune("permute.lds_bytes", 160 * 1024));
+  const bool lds_table_fits = (((int64_t)ntarget * (int64_t)esz + 15) & ~int64_t(15)) + ntarget * 4 <= lds_all &&
+                              n_src >= acc::tune("permute.lock_lds_min_ratio", 4) * ntarget;
+  const bool generic_few = !s->spec.permute_locked && s->spec.combine_hint == ACC_COMBINE_GENERIC && lds_table_fits &&
+                           acc::tune("permute.generic_lds", 1) != 0;
+  if (s->spec.permute_locked || generic_few) {
     // elements no atomic covers: a lock per target (the reference's lock array, Execute.hs:402-405)
     ACC_TRY(plain_copy());
     Args largs;
@@ -475,7 +483,8 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
     ACC_TRY(push_env(s, env, &largs, &al));
     push_out(*out, &largs, &al);
     largs.i64(n_src);
-    ACC_TRY(s->ensure_variant(al ? 0 : 1));
+    const int lv = (al ? 0 : 1) + (s->spec.permute_locked ? 0 : 2);
+    ACC_TRY(s->ensure_variant(lv));
     int lblk = -1;
     ACC_TRY(s->ctx->scratch_acquire((size_t)ntarget * 4 + 256, st, acc::SCRATCH_LOCKS, &lblk));
     // the locks start 256 bytes in; the word just before them is the kernel's "a lock never opened" mark
@@ -485,9 +494,56 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
     // into failed attempts (1000 targets: 12 M updates/s with every compute unit full, 20 times that with 32 lanes
     // per target).
     const int64_t lanes = std::max<int64_t>(64, ntarget * acc::tune("permute.lock_lanes_per_target", 32));
-    const int64_t lgrid = std::min(acc_launch_grid(n_src, s->spec.block, s->ctx->props.multiProcessorCount, 8),
-                                   (lanes + s->spec.block - 1) / s->spec.block);
-    const int lrc = launch(s, al ? 0 : 1, lgrid, 0, st, &largs);
+    int64_t lgrid = std::min(acc_launch_grid(n_src, s->spec.block, s->ctx->props.multiProcessorCount, 8),
+                             (lanes + s->spec.block - 1) / s->spec.block);
+    // With few targets every workgroup combines in a table of its own in LDS (value + state word per target),
+    // leaves it as a row of a table in memory, and a second launch folds the rows into the result: no global lock.
+    const int64_t lds_budget = std::min<int64_t>((int64_t)s->ctx->props.sharedMemPerBlock, acc::tune("permute.lds_bytes", 160 * 1024));
+    auto lds_for = [&](int64_t copies) { return (((int64_t)ntarget * copies * (int64_t)esz + 15) & ~int64_t(15)) + ntarget * copies * 4; };
+    int64_t lds_need = lds_for(1);
+    int32_t lds_bins = 0, lds_copies = 1;
+    int dblk = -1;
+    uint64_t dump_val = 0, dump_ok = 0;
+    if (lds_need <= lds_budget && n_src >= acc::tune("permute.lock_lds_min_ratio", 4) * ntarget) {
+      lds_bins = static_cast<int32_t>(ntarget);
+      // one copy of a small table per wave, within a quarter of the LDS so that several workgroups still fit
+      const int64_t waves = s->spec.block / 64;
+      while (lds_copies * 2 <= waves && lds_for(lds_copies * 2) <= std::min<int64_t>(lds_budget, acc::tune("permute.lock_copies_bytes", 40 * 1024))) lds_copies *= 2;
+      lds_need = lds_for(lds_copies);
+      int bpc = 0;
+      hipError_t oe = hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&bpc, s->variants[lv].fn, s->spec.block, (size_t)lds_need);
+      if (oe != hipSuccess || bpc < 1) { (void)hipGetLastError(); bpc = 1; }
+      // the device full of workgroups, as long as their rows stay within `permute.lock_table_mbytes`
+      const int64_t row_bytes = ntarget * ((int64_t)esz + 4);
+      const int64_t row_cap = std::max<int64_t>(1, ((int64_t)acc::tune("permute.lock_table_mbytes", 64) << 20) / row_bytes);
+      lgrid = std::max<int64_t>(1, std::min<int64_t>(acc_launch_grid(n_src, s->spec.block, s->ctx->props.multiProcessorCount, bpc), row_cap));
+      const size_t ok_off = round256((size_t)(lgrid * ntarget) * esz);
+      const int arc = s->ctx->scratch_acquire(ok_off + (size_t)(lgrid * ntarget) * 4, st, acc::SCRATCH_FOLD, &dblk);
+      if (arc != ACC_OK) { s->ctx->scratch_release(lblk, st); return arc; }
+      dump_val = reinterpret_cast<uint64_t>(s->ctx->scratch[dblk].ptr);
+      dump_ok = dump_val + ok_off;
+    }
+    largs.i32(lds_bins);
+    largs.i32(lds_copies);
+    largs.ptr(dump_val);
+    largs.ptr(dump_ok);
+    int lrc = launch(s, lv, lgrid, lds_bins ? (size_t)lds_need : 0, st, &largs);
+    if (lrc == ACC_OK && lds_bins) {
+      Args j;
+      bool jal = true;
+      lrc = push_env(s, env, &j, &jal);
+      push_out(*out, &j, &jal);
+      j.ptr(dump_val);
+      j.ptr(dump_ok);
+      j.i32(static_cast<int32_t>(lgrid));
+      j.i32(lds_bins);
+      if (lrc == ACC_OK) {
+        hipError_t je = hipModuleLaunchKernel(s->variants[lv].fn_finish, static_cast<unsigned>((ntarget + 3) / 4), 1, 1, 256, 1, 1, 0, st,
+                                              j.data(), nullptr);
+        if (je != hipSuccess) lrc = acc::fail_hip(je, "hipModuleLaunchKernel(permute_join)");
+      }
+    }
+    if (dblk >= 0) s->ctx->scratch_release(dblk, st);
     s->ctx->scratch_release(lblk, st);
     return lrc;
   }

@@ -493,8 +493,11 @@ int acc_skel_s::ensure_variant(int v)
   std::lock_guard<std::mutex> lock(mu);
   acc::Variant &var = variants[v];
   if (var.ready) return ACC_OK;
+  // variants 2 and 3 of a permute: the locked template for an element the atomic template also covers
+  acc::SkelSpec spec = this->spec;
+  if (v >= 2) spec.permute_locked = true;
   std::string entry_name;
-  ACC_TRY(acc::generate_source(spec, v == 0, &entry_name, &var.source));
+  ACC_TRY(acc::generate_source(spec, (v & 1) == 0, &entry_name, &var.source));
   entry = entry_name;
   std::vector<std::string> opts = acc::compile_options(spec);
   std::vector<const char *> optp;
@@ -513,8 +516,8 @@ int acc_skel_s::ensure_variant(int v)
   const bool segmented = spec.kind == ACC_SKEL_FOLDSEG || spec.kind == ACC_SKEL_FOLD1SEG ||
                          ((spec.kind == ACC_SKEL_FOLD || spec.kind == ACC_SKEL_FOLD1) && spec.out_rank > 0);
   const bool two_kernels = ((spec.kind == ACC_SKEL_FOLD || spec.kind == ACC_SKEL_FOLD1) && spec.out_rank == 0) ||
-                           (spec.kind == ACC_SKEL_PERMUTE && !spec.permute_locked) || segmented;
-  const std::string second = entry + (spec.kind == ACC_SKEL_PERMUTE ? "_merge" : segmented ? "_team" : "_finish");
+                           spec.kind == ACC_SKEL_PERMUTE || segmented;
+  const std::string second = entry + (spec.kind == ACC_SKEL_PERMUTE ? (spec.permute_locked ? "_join" : "_merge") : segmented ? "_team" : "_finish");
   if (two_kernels) {
     e = hipModuleGetFunction(&var.fn_finish, var.module, second.c_str());
     if (e != hipSuccess) {

@@ -63,7 +63,8 @@ struct acc_skel_s {
   acc_context ctx = nullptr;
   acc::SkelSpec spec;
   std::string entry;
-  acc::Variant variants[2];   // [0] pointers 16-byte aligned, [1] no assumption
+  acc::Variant variants[4];   // [0] pointers 16-byte aligned, [1] no assumption; [2], [3]: the same for the
+                              // table-in-LDS form of a permute whose combination has no atomic instruction
   std::mutex mu;
 
   int ensure_variant(int v);
