@@ -187,16 +187,15 @@ def test_permute_of_tuples_and_narrow_elements_under_locks(A, ctx):
 
 
 def test_locked_permute_loses_no_update_at_scale(A, ctx):
-    """4 M updates under per-target locks, from every compute die, with hundreds of lanes waiting at each lock and with
-    hardly any: integer sums and counts are exact, so one lost or torn update shows.  (A handful of targets for
-    millions of updates is the case locks are worst at -- every update waits behind all the failed attempts queued at
-    its lock -- and is kept to the small sizes of the test above.)"""
+    """4 M updates: on few targets (tables in LDS under LDS locks, joined by a second launch: 7 targets, where every
+    lane of a workgroup wants the same few locks; 13 000, the largest table that fits) and on many (a lock per target in
+    memory).  Integer sums and counts are exact, so one lost or torn update shows."""
     rng = np.random.default_rng(23)
     n = 1 << 22
     w = rng.integers(-1000, 1000, n).astype(np.int64)
     sk = ctx.skeleton(A.SKEL_PERMUTE, "Int64, Int32", env=[I32, (1, "Int64")], out_rank=1, get="acc_elt{arrIn1_0[ix], 1}",
                       combine="acc_elt{x.a1 + y.a1, x.a0 + y.a0}", permutation="arrIn0_0[ix]")
-    for bins in (1000, 100003):
+    for bins in (7, 1000, 13000, 100003):
         say("locked permute, %d updates into %d targets" % (n, bins))
         keys = rng.integers(0, bins, n).astype(np.int32)
         out = ctx.empty_tuple(bins, [np.int64, np.int32])
@@ -206,6 +205,26 @@ def test_locked_permute_loses_no_update_at_scale(A, ctx):
         ref = np.zeros(bins, np.int64)
         np.add.at(ref, keys, w)
         assert np.array_equal(s_, ref)
+
+
+def test_generic_combination_on_few_targets_goes_through_lds_tables(A, ctx):
+    """a 4-byte element with a combination that is no hardware atomic: compare-and-swap loops on many targets,
+    the locked template's tables in LDS on few -- same results"""
+    rng = np.random.default_rng(29)
+    n = 1 << 21
+    v = rng.integers(-10 ** 6, 10 ** 6, n).astype(np.int32)
+    sk = ctx.skeleton(A.SKEL_PERMUTE, "Int32", env=[I32, I32], out_rank=1, get="arrIn1_0[ix]",
+                      combine="(x > y) ? x : y", permutation="arrIn0_0[ix]")        # max, spelt so that no hint applies
+    for bins in (1, 5, 300, 20000, 200000):
+        say("generic permute (max) into", bins, "targets")
+        keys = rng.integers(-2, bins + 2, n).astype(np.int32)
+        d = rng.integers(-10 ** 6, 10 ** 6, bins).astype(np.int32)
+        out = ctx.empty(bins, np.int32)
+        sk.permute([ctx.array(keys), ctx.array(v)], n, ctx.array(d), out)
+        ok = (keys >= 0) & (keys < bins)
+        ref = d.copy()
+        np.maximum.at(ref, keys[ok], v[ok])
+        assert np.array_equal(out.get(), ref)
 
 
 def test_tuple_results_need_tuple_arrays_and_are_refused_elsewhere(A, ctx):
