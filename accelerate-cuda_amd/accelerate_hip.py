@@ -33,7 +33,8 @@ import acchip as A
 
 __all__ = ["Exp", "constant", "cond", "use", "unit", "map", "zipWith", "generate", "backpermute", "transpose", "reverse", "zip_", "unzip", "while_",
            "fold", "fold1", "foldSeg", "scanl", "scanl1", "scanl_", "scanr", "scanr1", "scanr_", "permute", "ignore",
-           "stencil", "stencil2", "awhile", "run", "run1", "fst", "snd", "lift", "index_if", "fromIntegral", "truncate", "round_", "floor",
+           "stencil", "stencil2", "awhile", "run", "run1", "fill", "enumFromN", "take", "drop", "init", "tail", "gather",
+           "scatter", "foldAll", "sum_", "product", "maximum", "minimum", "and_", "or_", "all_", "any_", "filter_", "fst", "snd", "lift", "index_if", "fromIntegral", "truncate", "round_", "floor",
            "ceiling", "idiv", "mod", "quot", "rem", "min_", "max_", "sqrt", "exp", "log", "sin", "cos", "tan", "abs_",
            "signum", "Context", "the"]
 
@@ -734,6 +735,87 @@ def stencil2(pattern1, pattern2, f, boundary1, a, boundary2, b, context=None, co
     out = _empty(cx, shape, res.ctype)
     cx.launch(arrays + [s1.manifest, s2.manifest], [out], lambda i, o, s: sk.stencil2(i[:-2], i[-2], i[-1], o[0], stream=s))
     return Acc(shape, res.ctype, manifest=out)
+
+
+# ------------------------------------------------------------------------------ library functions
+# What Data.Array.Accelerate.Prelude builds out of the primitive operations, built the same way.
+
+def fill(shape, value, ctype):
+    return generate(shape, lambda *ix: constant(value, ctype))
+
+
+def enumFromN(shape, first, ctype="Int64"):
+    """first, first + 1, ... in row-major order"""
+    shape = (shape,) if isinstance(shape, numbers.Integral) else tuple(shape)
+    def at(ix):
+        i = ix if ctype == "Int64" else fromIntegral(ix, ctype)
+        return i + constant(first, ctype)
+    return Acc(shape, ctype, at=at)
+
+
+def take(n, a):
+    return backpermute((min(int(n), a.shape[0]),), lambda i: (i,), a)
+
+
+def drop(n, a):
+    n = min(int(n), a.shape[0])
+    return backpermute((a.shape[0] - n,), lambda i: (i + n,), a)
+
+
+def init(a):
+    return take(a.shape[0] - 1, a)
+
+
+def tail(a):
+    return drop(1, a)
+
+
+def gather(indices, a):
+    """result[i] = a[indices[i]] (backpermute through an index vector)"""
+    return Acc(indices.shape, a.ctype, at=lambda ix: a[indices.index(ix)])
+
+
+def scatter(indices, defaults, a, context=None):
+    """defaults overwritten at indices[i] by a[i]; which of several writers to one place wins is unspecified"""
+    return permute(lambda new, old: new, defaults, lambda *i: (indices.index(_linear(i, indices.shape)),), a, context)
+
+
+def foldAll(f, z, a, context=None):
+    """reduce every dimension (Prelude's foldAll: a fold over the array seen as a vector)"""
+    return fold(f, z, Acc((a.size,), a.ctype, at=lambda ix: a.index(ix)), context)
+
+
+def _limit(ctype, low):
+    if ctype == "float" or ctype == "double":
+        return -np.inf if low else np.inf
+    info = np.iinfo(NPTYPE[ctype])
+    return info.min if low else info.max
+
+
+def sum_(a, context=None): return foldAll(lambda x, y: x + y, constant(0, a.ctype), a, context)
+def product(a, context=None): return foldAll(lambda x, y: x * y, constant(1, a.ctype), a, context)
+def maximum(a, context=None): return foldAll(max_, constant(_limit(a.ctype, True), a.ctype), a, context)
+def minimum(a, context=None): return foldAll(min_, constant(_limit(a.ctype, False), a.ctype), a, context)
+def and_(a, context=None): return foldAll(lambda x, y: x.land(y), constant(1, "Word8"), a, context)
+def or_(a, context=None): return foldAll(lambda x, y: x.lor(y), constant(0, "Word8"), a, context)
+def all_(p, a, context=None): return and_(map(p, a), context)
+def any_(p, a, context=None): return or_(map(p, a), context)
+
+
+def filter_(p, a, context=None):
+    """the elements of a vector that satisfy p, in order, and how many there are: the scan-then-permute
+    compaction of the Prelude (an exclusive scan of the flags gives every kept element its place)"""
+    cx = context or Context.default()
+    a = _force(a, cx)
+    flags = map(lambda v: cond(p(v), constant(1, "Int32"), constant(0, "Int32")), a)
+    places, count = scanl_(lambda x, y: x + y, 0, flags, context=cx)
+    n = int(the(count, cx))
+    if n == 0:
+        return Acc((0,), a.ctype, at=lambda ix: a.index(ix)), count
+    keep = lambda i: index_if(p(a[i]), (places[i],))
+    # every kept element has a place of its own, so the combination is never applied: defaults are overwritten
+    out = permute(lambda new, old: new, generate((n,), lambda i: a[constant(0, "Int64")]), keep, a, context=cx)
+    return out, count
 
 
 def awhile(p, f, a, context=None, limit=None):

@@ -344,3 +344,36 @@ def test_awhile_iterates_on_the_device_until_the_flag_clears(acc):
     assert np.array_equal(acc.run(u, cx), ref)
     with pytest.raises(TypeError):
         acc.awhile(lambda xs: xs, lambda xs: xs, acc.use(x, cx), context=cx)
+
+
+def test_library_functions_built_from_the_primitives(acc):
+    cx = acc.Context(0)
+    rng = np.random.default_rng(13)
+    x = rng.integers(-1000, 1000, 200003).astype(np.int32)
+    xs = acc.use(x, cx)
+    # filter: scan of the flags, then a permute into the places it gives
+    kept, count = acc.filter_(lambda v: (v % 3).eq(0), xs, context=cx)
+    assert int(acc.run(count, cx)) == int((x % 3 == 0).sum())
+    assert np.array_equal(acc.run(kept, cx), x[x % 3 == 0])
+    none, count = acc.filter_(lambda v: v > 5000, xs, context=cx)
+    assert none.shape == (0,) and int(acc.run(count, cx)) == 0
+    # whole-array reductions of a matrix
+    m = rng.integers(-50, 50, (301, 77)).astype(np.int64)
+    ms = acc.use(m, cx)
+    assert int(acc.run(acc.sum_(ms, cx), cx)) == int(m.sum())
+    assert int(acc.run(acc.maximum(ms, cx), cx)) == int(m.max()) and int(acc.run(acc.minimum(ms, cx), cx)) == int(m.min())
+    assert int(acc.run(acc.all_(lambda v: v < 50, ms, cx), cx)) == 1 and int(acc.run(acc.any_(lambda v: v > 49, ms, cx), cx)) == 0
+    f = rng.integers(1, 3, 40).astype(np.float64)
+    assert float(acc.run(acc.product(acc.use(f, cx), cx), cx)) == float(np.prod(f))
+    # index-space helpers
+    assert np.array_equal(acc.run(acc.take(10, xs), cx), x[:10]) and np.array_equal(acc.run(acc.drop(199990, xs), cx), x[199990:])
+    assert np.array_equal(acc.run(acc.init(xs), cx), x[:-1]) and np.array_equal(acc.run(acc.tail(xs), cx), x[1:])
+    assert np.array_equal(acc.run(acc.enumFromN((3, 4), 5, "Int32"), cx), np.arange(5, 17, dtype=np.int32).reshape(3, 4))
+    assert np.array_equal(acc.run(acc.fill((2, 3), 7, "Int16"), cx), np.full((2, 3), 7, np.int16))
+    idx = rng.permutation(x.size).astype(np.int32)
+    ids = acc.use(idx, cx)
+    assert np.array_equal(acc.run(acc.gather(ids, xs), cx), x[idx])
+    sc = acc.run(acc.scatter(ids, acc.fill((x.size,), 0, "Int32"), xs, context=cx), cx)       # a permutation: no collisions
+    ref = np.zeros_like(x)
+    ref[idx] = x
+    assert np.array_equal(sc, ref)
