@@ -63,10 +63,13 @@
  * in `dump_val` / `dump_ok` (one row per workgroup); permute_join then folds the rows into the result, one wave
  * per target, without any lock.  With few targets that turns millions of contended global lock rounds (1000
  * targets: 0.25 G updates/s at best) into LDS traffic.  Small tables are kept `lds_copies` times, the waves of
- * the workgroup spread over the copies.                                                                   */
+ * the workgroup spread over the copies.  More targets than one table holds are cut into windows of `lds_bins`:
+ * `win_blocks` consecutive workgroups share a window, walk the whole source between them and take the elements
+ * whose target lies in it (as many passes over the source as there are windows, still far cheaper than a round
+ * of global locks per element while the windows are few).                                                 */
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, int *__restrict__ locks, const int lds_bins, const int lds_copies,
-        ACC_ELT *__restrict__ dump_val, int *__restrict__ dump_ok)
+        ACC_ELT *__restrict__ dump_val, int *__restrict__ dump_ok, const int win_blocks)
 {
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
@@ -119,10 +122,12 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, int *__restrict__ loc
   for (int i = threadIdx.x; i < slots; i += ACC_BLOCK) s_state[i] = 0;
   __syncthreads();
   const int mine = (int)((threadIdx.x >> 6) % lds_copies) * lds_bins;     /* this wave's copy */
-  for (Int64 ix0 = (Int64)blockIdx.x * ACC_BLOCK; ix0 < n; ix0 += (Int64)gridDim.x * ACC_BLOCK) {
+  const Int64 first = (Int64)(blockIdx.x / win_blocks) * lds_bins;          /* this workgroup's window of targets */
+  const Int64 past = acc_min<Int64>(first + lds_bins, ntarget);
+  for (Int64 ix0 = (Int64)(blockIdx.x % win_blocks) * ACC_BLOCK; ix0 < n; ix0 += (Int64)win_blocks * ACC_BLOCK) {
     const Int64 ix = ix0 + threadIdx.x;
-    const Int64 j = ix < n ? perm(ix) : -1;
-    const bool active = j >= 0 && j < ntarget;
+    const Int64 j = ix < n ? perm(ix) - first : -1;
+    const bool active = j >= 0 && j < past - first;
     T x = T();
     if (active) x = get(ix);
     bool done = !active;
@@ -155,10 +160,10 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, int *__restrict__ loc
 }
 
 /* out[j] := f(everything the workgroups gathered for j, out[j]): one wave per target, its lanes spread over
- * the rows of the table */
+ * the `rows` rows of the table that belong to the target's window of `bins` targets */
 extern "C" __global__ void __launch_bounds__(256)
 permute_join(ACC_ENV_PARAMS ACC_OUT_PARAMS, const ACC_ELT *__restrict__ dump_val, const int *__restrict__ dump_ok,
-             const int rows, const int bins)
+             const int rows, const int bins, const Int64 ntarget)
 {
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
@@ -166,12 +171,14 @@ permute_join(ACC_ENV_PARAMS ACC_OUT_PARAMS, const ACC_ELT *__restrict__ dump_val
   auto lf = acc_lift<T>(f);
   const int lane = acc_lane();
   const Int64 j = (Int64)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (j >= bins) return;                              /* whole waves leave */
+  if (j >= ntarget) return;                           /* whole waves leave */
+  const Int64 window = j / bins, col = j - window * bins;
   acc_opt<T> acc = acc_none<T>();
   for (int r = lane; r < rows; r += ACC_WAVE) {
+    const Int64 at = (window * rows + r) * bins + col;
     acc_opt<T> p;
-    p.v = dump_val[(Int64)r * bins + j];
-    p.ok = dump_ok[(Int64)r * bins + j] != 0;
+    p.v = dump_val[at];
+    p.ok = dump_ok[at] != 0;
     acc = lf(acc, p);
   }
   acc = acc_wave_reduce(acc, lf);

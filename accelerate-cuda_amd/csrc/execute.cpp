@@ -471,7 +471,10 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
   // meet on those few addresses (16 M Float32 `max` updates on 1000 targets: 16.6 ms), the tables in LDS of the
   // locked template do not (74 us).  Such a skeleton carries that template as its variants 2 and 3.
   const int64_t lds_all = std::min<int64_t>((int64_t)s->ctx->props.sharedMemPerBlock, acc::tune("permute.lds_bytes", 160 * 1024));
-  const bool lds_table_fits = (((int64_t)ntarget * (int64_t)esz + 15) & ~int64_t(15)) + ntarget * 4 <= lds_all &&
+  // targets per table in LDS (value + state word each), and how many such windows the targets need
+  const int64_t lds_cap = std::max<int64_t>(1, (lds_all - 16) / ((int64_t)esz + 4));
+  const int64_t lds_windows = (ntarget + lds_cap - 1) / lds_cap;
+  const bool lds_table_fits = lds_windows <= acc::tune("permute.lock_max_windows", 12) &&
                               n_src >= acc::tune("permute.lock_lds_min_ratio", 4) * ntarget;
   // (Floating-point addition has an LDS atomic, but it runs at a fifth of the integer one's rate -- 16 M updates on
   // 1000 targets: 95 us against 66 us through the tables -- so it goes the same way.)
@@ -501,27 +504,33 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
                              (lanes + s->spec.block - 1) / s->spec.block);
     // With few targets every workgroup combines in a table of its own in LDS (value + state word per target),
     // leaves it as a row of a table in memory, and a second launch folds the rows into the result: no global lock.
-    const int64_t lds_budget = std::min<int64_t>((int64_t)s->ctx->props.sharedMemPerBlock, acc::tune("permute.lds_bytes", 160 * 1024));
-    auto lds_for = [&](int64_t copies) { return (((int64_t)ntarget * copies * (int64_t)esz + 15) & ~int64_t(15)) + ntarget * copies * 4; };
-    int64_t lds_need = lds_for(1);
-    int32_t lds_bins = 0, lds_copies = 1;
+    const int64_t lds_budget = lds_all;
+    int32_t lds_bins = 0, lds_copies = 1, win_blocks = 1;
+    int64_t lds_need = 0;
     int dblk = -1;
     uint64_t dump_val = 0, dump_ok = 0;
-    if (lds_need <= lds_budget && n_src >= acc::tune("permute.lock_lds_min_ratio", 4) * ntarget) {
-      lds_bins = static_cast<int32_t>(ntarget);
-      // one copy of a small table per wave, within a quarter of the LDS so that several workgroups still fit
+    if (lds_table_fits) {
+      // windows of equal size; a single window that is small is kept once per wave, within a quarter of the LDS so
+      // that several workgroups still fit
+      lds_bins = static_cast<int32_t>((ntarget + lds_windows - 1) / lds_windows);
+      auto lds_for = [&](int64_t copies) { return (((int64_t)lds_bins * copies * (int64_t)esz + 15) & ~int64_t(15)) + (int64_t)lds_bins * copies * 4; };
       const int64_t waves = s->spec.block / 64;
-      while (lds_copies * 2 <= waves && lds_for(lds_copies * 2) <= std::min<int64_t>(lds_budget, acc::tune("permute.lock_copies_bytes", 40 * 1024))) lds_copies *= 2;
+      while (lds_windows == 1 && lds_copies * 2 <= waves &&
+             lds_for(lds_copies * 2) <= std::min<int64_t>(lds_budget, acc::tune("permute.lock_copies_bytes", 40 * 1024))) lds_copies *= 2;
       lds_need = lds_for(lds_copies);
       int bpc = 0;
       hipError_t oe = hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&bpc, s->variants[lv].fn, s->spec.block, (size_t)lds_need);
       if (oe != hipSuccess || bpc < 1) { (void)hipGetLastError(); bpc = 1; }
-      // the device full of workgroups, as long as their rows stay within `permute.lock_table_mbytes`
-      const int64_t row_bytes = ntarget * ((int64_t)esz + 4);
-      const int64_t row_cap = std::max<int64_t>(1, ((int64_t)acc::tune("permute.lock_table_mbytes", 64) << 20) / row_bytes);
-      lgrid = std::max<int64_t>(1, std::min<int64_t>(acc_launch_grid(n_src, s->spec.block, s->ctx->props.multiProcessorCount, bpc), row_cap));
-      const size_t ok_off = round256((size_t)(lgrid * ntarget) * esz);
-      const int arc = s->ctx->scratch_acquire(ok_off + (size_t)(lgrid * ntarget) * 4, st, acc::SCRATCH_FOLD, &dblk);
+      // the device full of workgroups, shared out between the windows, as long as their rows stay within
+      // `permute.lock_table_mbytes`
+      const int64_t row_bytes = (int64_t)lds_bins * ((int64_t)esz + 4);
+      const int64_t row_cap = std::max<int64_t>(lds_windows, ((int64_t)acc::tune("permute.lock_table_mbytes", 64) << 20) / row_bytes);
+      const int64_t blocks = std::max<int64_t>(lds_windows, std::min<int64_t>(
+          lds_windows * acc_launch_grid(n_src, s->spec.block, s->ctx->props.multiProcessorCount, bpc), std::min<int64_t>((int64_t)s->ctx->props.multiProcessorCount * bpc, row_cap)));
+      win_blocks = static_cast<int32_t>(std::max<int64_t>(1, blocks / lds_windows));
+      lgrid = lds_windows * win_blocks;
+      const size_t ok_off = round256((size_t)(lgrid * lds_bins) * esz);
+      const int arc = s->ctx->scratch_acquire(ok_off + (size_t)(lgrid * lds_bins) * 4, st, acc::SCRATCH_FOLD, &dblk);
       if (arc != ACC_OK) { s->ctx->scratch_release(lblk, st); return arc; }
       dump_val = reinterpret_cast<uint64_t>(s->ctx->scratch[dblk].ptr);
       dump_ok = dump_val + ok_off;
@@ -530,6 +539,7 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
     largs.i32(lds_copies);
     largs.ptr(dump_val);
     largs.ptr(dump_ok);
+    largs.i32(win_blocks);
     int lrc = launch(s, lv, lgrid, lds_bins ? (size_t)lds_need : 0, st, &largs);
     if (lrc == ACC_OK && lds_bins) {
       Args j;
@@ -538,8 +548,9 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
       push_out(*out, &j, &jal);
       j.ptr(dump_val);
       j.ptr(dump_ok);
-      j.i32(static_cast<int32_t>(lgrid));
+      j.i32(win_blocks);
       j.i32(lds_bins);
+      j.i64(ntarget);
       if (lrc == ACC_OK) {
         hipError_t je = hipModuleLaunchKernel(s->variants[lv].fn_finish, static_cast<unsigned>((ntarget + 3) / 4), 1, 1, 256, 1, 1, 0, st,
                                               j.data(), nullptr);
