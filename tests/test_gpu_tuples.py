@@ -188,14 +188,15 @@ def test_permute_of_tuples_and_narrow_elements_under_locks(A, ctx):
 
 def test_locked_permute_loses_no_update_at_scale(A, ctx):
     """4 M updates: on few targets (tables in LDS under LDS locks, joined by a second launch: 7 targets, where every
-    lane of a workgroup wants the same few locks; 13 000, the largest table that fits) and on many (a lock per target in
-    memory).  Integer sums and counts are exact, so one lost or torn update shows."""
+    lane of a workgroup wants the same few locks; 13 000, about the largest single table; 100 003, ten windows of
+    targets) and on many (3 M: a lock per target in memory).  Integer sums and counts are exact, so one lost or torn
+    update shows."""
     rng = np.random.default_rng(23)
     n = 1 << 22
     w = rng.integers(-1000, 1000, n).astype(np.int64)
     sk = ctx.skeleton(A.SKEL_PERMUTE, "Int64, Int32", env=[I32, (1, "Int64")], out_rank=1, get="acc_elt{arrIn1_0[ix], 1}",
                       combine="acc_elt{x.a1 + y.a1, x.a0 + y.a0}", permutation="arrIn0_0[ix]")
-    for bins in (7, 1000, 13000, 100003):
+    for bins in (7, 1000, 13000, 100003, 3000017):
         say("locked permute, %d updates into %d targets" % (n, bins))
         keys = rng.integers(0, bins, n).astype(np.int32)
         out = ctx.empty_tuple(bins, [np.int64, np.int32])
@@ -215,7 +216,7 @@ def test_generic_combination_on_few_targets_goes_through_lds_tables(A, ctx):
     v = rng.integers(-10 ** 6, 10 ** 6, n).astype(np.int32)
     sk = ctx.skeleton(A.SKEL_PERMUTE, "Int32", env=[I32, I32], out_rank=1, get="arrIn1_0[ix]",
                       combine="(x > y) ? x : y", permutation="arrIn0_0[ix]")        # max, spelt so that no hint applies
-    for bins in (1, 5, 300, 20000, 200000):
+    for bins in (1, 5, 300, 20000, 200000, 1500000):
         say("generic permute (max) into", bins, "targets")
         keys = rng.integers(-2, bins + 2, n).astype(np.int32)
         d = rng.integers(-10 ** 6, 10 ** 6, bins).astype(np.int32)
