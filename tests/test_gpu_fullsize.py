@@ -168,3 +168,38 @@ def test_config5_smvm_2_20_rows(A, ctx, wl, orc):
     # per row 1e-4 relative; rows that cancel to almost nothing are measured against their magnitude
     assert np.all(np.abs(got - y64) <= 1e-4 * np.maximum(np.abs(y64), 1e-3 * yabs) + 1e-30)
     assert np.all(got[lens == 0] == 0.0)
+
+
+def test_more_than_2_31_elements(A, ctx):
+    """indices are 64-bit throughout: map, fold, scan and permute over 2^31 + 1 000 003 bytes"""
+    n = (1 << 31) + 1000003
+    W8 = (1, "Word8")
+    say("beyond 2^31 elements, n =", n)
+    x = np.empty(n, np.uint8)
+    blk = (np.arange(1 << 20, dtype=np.uint32) * 7 % 251).astype(np.uint8)
+    for s in range(0, n, 1 << 20):
+        e = min(n, s + (1 << 20))
+        x[s:e] = blk[:e - s]
+    dx, o = ctx.array(x), ctx.empty(n, np.uint8)
+    say("map")
+    A_map = ctx.skeleton(A.SKEL_MAP, "Word8", env=[W8], out_rank=1, get="(Word8)(arrIn0_0[ix] + 1)")
+    A_map.map([dx], o)
+    got = o.get()
+    assert np.array_equal(got[-5000000:], (x[-5000000:] + 1).astype(np.uint8)) and np.array_equal(got[:1000], (x[:1000] + 1).astype(np.uint8))
+    say("fold")
+    f = ctx.skeleton(A.SKEL_FOLD, "Int64", env=[W8], out_rank=0, get="(Int64)arrIn0_0[ix]", combine="x + y", seed="0")
+    s_ = ctx.empty((), np.int64)
+    f.fold([dx], n, s_)
+    assert int(s_.get().reshape(-1)[0]) == int(x.sum(dtype=np.int64))
+    say("scanl1")
+    sc = ctx.skeleton(A.SKEL_SCANL1, "Word8", env=[W8], get="arrIn0_0[ix]", combine="(Word8)(x ^ y)")
+    sc.scan([dx], n, o)
+    got = o.get()
+    ref = np.bitwise_xor.accumulate(x)
+    assert np.array_equal(got[:100000], ref[:100000]) and np.array_equal(got[-100000:], ref[-100000:])
+    say("permute")
+    p = ctx.skeleton(A.SKEL_PERMUTE, "Int64", env=[W8], out_rank=1, get="(Int64)1", combine="x + y", combine_hint=A.COMBINE_ADD,
+                     permutation="(Int64)arrIn0_0[ix]")
+    h = ctx.empty(256, np.int64)
+    p.permute([dx], n, ctx.array(np.zeros(256, np.int64)), h)
+    assert np.array_equal(h.get(), np.bincount(x, minlength=256).astype(np.int64))
