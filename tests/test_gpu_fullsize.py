@@ -203,3 +203,22 @@ def test_more_than_2_31_elements(A, ctx):
     h = ctx.empty(256, np.int64)
     p.permute([dx], n, ctx.array(np.zeros(256, np.int64)), h)
     assert np.array_equal(h.get(), np.bincount(x, minlength=256).astype(np.int64))
+
+
+def test_stencil_over_more_than_2_31_elements(A, ctx):
+    h, w = 65536, 33000
+    say("5-point stencil over", h * w, "Int8 elements")
+    img = np.empty((h, w), np.int8)
+    row = (np.arange(w, dtype=np.int64) * 5 % 97).astype(np.int8)
+    for y in range(h):
+        img[y] = np.roll(row, y % 131)
+    s = ctx.skeleton(A.SKEL_STENCIL, "Int8", out_rank=2, taps=[(-1, 0), (0, -1), (0, 0), (0, 1), (1, 0)], boundary="clamp",
+                     stencil_fn="(Int8)(t0 + t1 + t2 + t3 + t4)", stencil_in="Int8")
+    b = ctx.empty((h, w), np.int8)
+    s.stencil([], ctx.array(img), b)
+    got = b.get()
+    for y in (0, 1, 777, 32768, 65000, 65534, 65535):          # the rows on both sides of index 2^31 among them
+        up, dn = img[max(y - 1, 0)].astype(np.int32), img[min(y + 1, h - 1)].astype(np.int32)
+        c = img[y].astype(np.int32)
+        left, right = np.concatenate([c[:1], c[:-1]]), np.concatenate([c[1:], c[-1:]])
+        assert np.array_equal(got[y], (up + left + c + right + dn).astype(np.int8)), y
