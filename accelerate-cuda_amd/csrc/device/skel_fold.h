@@ -10,13 +10,16 @@
  * foldAll: every block strides over tiles of the (fused) input, each lane
  * reading ACC_UNROLL independent groups of ACC_VEC consecutive elements per
  * tile; lanes are combined with a wave64 DPP reduction, waves through a few
- * words of LDS, and each block leaves one partial result in global memory.  A
- * second, single-block launch of <entry>_finish combines the partials and
- * applies the seed (a lone block does so itself and the second launch is
- * skipped).  Blocks never meet on an atomic: same-address device-scope
- * atomics cost tens of nanoseconds each on this part, far more than a
- * back-to-back launch; and with a fixed grid the association order, hence
- * the Float32 result, is reproducible from run to run.  As in the reference
+ * words of LDS, and each block leaves one partial result in global memory.
+ * With ACC_FOLD_SINGLE (the default) that is all one launch: the partial
+ * travels as tagged 64-bit words and the last block collects the others'
+ * and applies the seed; without it a second, single-block launch of
+ * <entry>_finish does (a lone block finishes the job itself either way).
+ * Blocks never meet on an atomic or behind a fence: same-address device-scope
+ * atomics cost tens of nanoseconds each on this part and a release/acquire
+ * pair a cache-wide write-back and invalidate; and with a fixed grid the
+ * association order, hence the Float32 result, is reproducible from run to
+ * run.  As in the reference
  * the operator must be associative AND commutative here (the striding
  * reorders elements, Reduction.hs:160-165), it needs no identity, the seed
  * enters once as the second operand (Reduction.hs:203-211) and an empty input

@@ -44,8 +44,8 @@ struct Variant {
   std::string source;
   hipModule_t module = nullptr;
   hipFunction_t fn = nullptr;
-  hipFunction_t fn_finish = nullptr;   // second kernel of a two-launch skeleton (foldAll, permute's merge)
-  hipFunction_t fn_fill = nullptr;     // permute: fills table rows with the combine's identity
+  hipFunction_t fn_finish = nullptr;   // second kernel: foldAll's _finish, permute's _merge / _join, the segmented fold's _team
+  hipFunction_t fn_fill = nullptr;     // third kernel: permute's _fill (identity into the table rows), the segmented fold's _join
   int num_regs = 0;
   int static_lds = 0;
   int blocks_per_cu = 1;
