@@ -711,7 +711,7 @@ def stencil(pattern, f, boundary, a, context=None, constant_value=None):
     taps = _taps(pattern, rank)
     res = Exp.of(f(*[Exp(src.ctype, "t%d" % k) for k in range(len(taps))]))
     arrays, sig, fr = _assemble(stencil_fn=res.text)
-    sk = cx.skeleton(A.SKEL_STENCIL, res.ctype, sig, out_rank=rank, taps=taps, boundary=boundary,
+    sk = cx.skeleton(A.SKEL_STENCIL, _elt(res.ctype), sig, out_rank=rank, taps=taps, boundary=boundary,
                      boundary_constant=None if constant_value is None else _literal(constant_value, src.ctype),
                      stencil_in=src.ctype, **fr)
     out = _empty(cx, src.shape, res.ctype)
@@ -727,7 +727,7 @@ def stencil2(pattern1, pattern2, f, boundary1, a, boundary2, b, context=None, co
     t1, t2 = _taps(pattern1, rank), _taps(pattern2, rank)
     res = Exp.of(f([Exp(s1.ctype, "t%d" % k) for k in range(len(t1))], [Exp(s2.ctype, "u%d" % k) for k in range(len(t2))]))
     arrays, sig, fr = _assemble(stencil_fn=res.text)
-    sk = cx.skeleton(A.SKEL_STENCIL2, res.ctype, sig, out_rank=rank, taps=t1, boundary=boundary1, taps2=t2, boundary2=boundary2,
+    sk = cx.skeleton(A.SKEL_STENCIL2, _elt(res.ctype), sig, out_rank=rank, taps=t1, boundary=boundary1, taps2=t2, boundary2=boundary2,
                      boundary_constant=None if constant1 is None else _literal(constant1, s1.ctype),
                      boundary2_constant=None if constant2 is None else _literal(constant2, s2.ctype),
                      stencil_in=s1.ctype, stencil_in2=s2.ctype, **fr)

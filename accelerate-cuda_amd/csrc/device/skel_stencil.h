@@ -83,7 +83,7 @@ ACC_DEV Int64 acc_boundary_index(Int64 i, const Int64 sz)
   return acc_max<Int64>(0, acc_min<Int64>(i, sz - 1));
 }
 
-struct __attribute__((aligned(16))) acc_out_vec { ACC_ELT v[ACC_SVEC]; };
+struct acc_out_vec { ACC_ELT v[ACC_SVEC]; };
 
 /* value held by the next lane (the last lane keeps its own: caller masks it) */
 #define ACC_DPP_WAVE_SHL1 0x130
@@ -352,22 +352,24 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS)
 #endif
           res.v[k] = (T)(ACC_STENCIL_FN);
         }
-        T *dst = arrOut_0 + ((z0 * h) + (y0 + y)) * w + gx;
-        if (fast) {
-#if ACC_STENCIL_NT & 1
-          typedef T acc_out_native __attribute__((ext_vector_type(ACC_SVEC)));
-          acc_out_native nv;
-#pragma unroll
-          for (int k = 0; k < ACC_SVEC; ++k) nv[k] = res.v[k];
-          __builtin_nontemporal_store(nv, (acc_out_native *)dst);
-#else
-          *(acc_out_vec *)dst = res;
-#endif
-        } else {
-#pragma unroll
-          for (int k = 0; k < ACC_SVEC; ++k)
-            if (gx + k < w) dst[k] = res.v[k];
+        /* one vector store per component of the result (a tuple result is one array per component) */
+        const Int64 at = ((z0 * h) + (y0 + y)) * w + gx;
+#define ACC_STORE_COMPONENT(c, CT)                                                   \
+        {                                                                            \
+          CT *dst = arrOut_##c + at;                                                 \
+          if (fast) {                                                                \
+            typedef CT acc_out_native __attribute__((ext_vector_type(ACC_SVEC)));    \
+            acc_out_native nv;                                                       \
+            _Pragma("unroll") for (int k = 0; k < ACC_SVEC; ++k) nv[k] = ACC_COMPONENT(res.v[k], c); \
+            if (ACC_STENCIL_NT & 1) __builtin_nontemporal_store(nv, (acc_out_native *)dst); \
+            else                    *(acc_out_native *)dst = nv;                     \
+          } else {                                                                   \
+            _Pragma("unroll") for (int k = 0; k < ACC_SVEC; ++k)                     \
+              if (gx + k < w) dst[k] = ACC_COMPONENT(res.v[k], c);                   \
+          }                                                                          \
         }
+        ACC_FOR_COMPONENTS(ACC_STORE_COMPONENT)
+#undef ACC_STORE_COMPONENT
       }
     }
   }

@@ -674,7 +674,13 @@ static int stencil_once(acc_skel s, const acc_array *env, const acc_array *in, c
     const size_t esz = acc::type_size(type) ? acc::type_size(type) : s->spec.elt_size;
     return aligned16(a.ptr[0]) && (a.shape[rank - 1] * (int64_t)esz) % 16 == 0;
   };
-  if ((w * (int64_t)s->spec.elt_size) % 16 != 0 || !row_aligned(*in, s->spec.stencil_in_type)) aligned = false;
+  // (of a tuple result: the rows of every component's array)
+  const int ncomp = s->ncomp();
+  for (int c = 0; c < ncomp; ++c) {
+    const int64_t csz = ncomp == 1 ? (int64_t)s->spec.elt_size : (int64_t)acc::type_size(s->spec.comp_types[ncomp - 1 - c]);
+    if ((w * csz) % 16 != 0) aligned = false;
+  }
+  if (!row_aligned(*in, s->spec.stencil_in_type)) aligned = false;
   if (in2) {      // each source with its extents (Stencil.hs:146-152)
     if (!row_aligned(*in2, s->spec.stencil_in2_type)) aligned = false;
     bool ignore = true;

@@ -151,6 +151,13 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       }
     }
     o << "#define ACC_NCOMP " << nc << "\n";
+    //   ACC_FOR_COMPONENTS(M)  M(c, type) for every component;  ACC_COMPONENT(v, c)  component c of the value v
+    {
+      std::ostringstream each;
+      for (int i = 0; i < nc; ++i) each << "M(" << (nc - 1 - i) << ", " << (sp.comp_types.empty() ? std::string("ACC_ELT") : sp.comp_types[i]) << ") ";
+      o << "#define ACC_FOR_COMPONENTS(M) " << each.str() << "\n";
+      o << "#define ACC_COMPONENT(v, c) " << (sp.comp_types.empty() ? "(v)" : "((v).a##c)") << "\n";
+    }
     //   ACC_READ(name, ix)    element ix, assembled from its components
     //   ACC_READ_DEVICE / ACC_SET_DEVICE: the same at device scope, past the caches (elements shared under a lock)
     if (sp.comp_types.empty()) {
@@ -339,8 +346,11 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
     if ((int)sp->comp_types.size() > ACC_MAX_COMP) return fail(ACC_ERR_INVALID, "tuple element type: more than %d components", ACC_MAX_COMP);
     sp->elt_size = (size + align - 1) / align * align;
     sp->elt_type = "acc_elt";
-    if (d->kind == ACC_SKEL_STENCIL || d->kind == ACC_SKEL_STENCIL2)
-      return fail(ACC_ERR_UNSUPPORTED, "%s: tuple element types are not supported by this skeleton", kind_name(d->kind));
+    // a stencil may produce tuples; its sources are arrays of scalars, whose type must then be given
+    if ((d->kind == ACC_SKEL_STENCIL || d->kind == ACC_SKEL_STENCIL2) && !(d->stencil_in_type && *d->stencil_in_type))
+      return fail(ACC_ERR_INVALID, "%s: a tuple result needs `stencil_in_type` (the sources are arrays of scalars)", kind_name(d->kind));
+    if (d->kind == ACC_SKEL_STENCIL2 && !(d->stencil_in2_type && *d->stencil_in2_type))
+      return fail(ACC_ERR_INVALID, "stencil2: a tuple result needs `stencil_in2_type`");
   } else {
     sp->elt_size = d->elt_size > 0 ? d->elt_size : type_size(sp->elt_type);
     if (sp->elt_size <= 0) return fail(ACC_ERR_INVALID, "cannot size element type '%s': set elt_size", d->elt_type);

@@ -262,7 +262,8 @@ typedef struct acc_skel_desc {
                                      *   struct acc_elt { T<n-1> a<n-1>; ...; T0 a0; };
                                      * fragments produce and take apart acc_elt values, and the
                                      * result array has one pointer per component (CodeGen/
-                                     * Base.hs:344-357); not for stencil                      */
+                                     * Base.hs:344-357).  A stencil may produce tuples; its
+                                     * sources are arrays of scalars (stencil_in_type)        */
   int32_t            elt_size;      /* sizeof(elt_type); 0 = derive from the type's name    */
   int32_t            out_rank;      /* map family, stencil: rank of the result (>= 0)       */
   const char        *preamble;      /* file-scope declarations for the fragments, or NULL   */

@@ -377,3 +377,15 @@ def test_library_functions_built_from_the_primitives(acc):
     ref = np.zeros_like(x)
     ref[idx] = x
     assert np.array_equal(sc, ref)
+
+
+def test_stencil_producing_pairs(acc):
+    cx = acc.Context(0)
+    rng = np.random.default_rng(14)
+    img = rng.integers(-100, 100, (70, 333)).astype(np.float32)
+    g = acc.stencil([(0, -1), (0, 1), (-1, 0), (1, 0)], lambda l, r, u, d: acc.lift(r - l, d - u), "clamp", acc.use(img, cx), context=cx)
+    gx, gy = acc.run(g, cx)
+    t = pyref.tap_arrays(img, [(0, -1), (0, 1), (-1, 0), (1, 0)], "clamp", 0, img.shape)
+    assert np.array_equal(gx, t[1] - t[0]) and np.array_equal(gy, t[3] - t[2])
+    mag = acc.run(acc.map(lambda p: acc.fst(p) * acc.fst(p) + acc.snd(p) * acc.snd(p), g), cx)
+    assert np.array_equal(mag, (t[1] - t[0]) ** 2 + (t[3] - t[2]) ** 2)
