@@ -707,6 +707,17 @@ def stencil(pattern, f, boundary, a, context=None, constant_value=None):
     (Stencil/Extra.hs:112-116); the source is made manifest first, as in the reference (Execute.hs:413-425)"""
     cx = context or Context.default()
     src = _force(a, cx)
+    if isinstance(src.ctype, tuple):
+        # an array of pairs is two arrays: the same pattern over both, as a stencil2 (the sources of the
+        # stencil kernels are arrays of scalars)
+        if len(src.ctype) != 2:
+            raise TypeError("stencil over an array of %d-tuples: take it apart into pairs and scalars first" % len(src.ctype))
+        if constant_value is not None and not isinstance(constant_value, (tuple, list)):
+            raise TypeError("the boundary constant of a stencil over pairs is a pair")
+        c1, c2 = (None, None) if constant_value is None else constant_value
+        comp = [Acc(src.shape, t, manifest=m) for t, m in zip(src.ctype, src.manifest.comps)]
+        return stencil2(pattern, pattern, lambda ts, us: f(*[lift(t, u) for t, u in zip(ts, us)]), boundary, comp[0],
+                        boundary, comp[1], context=cx, constant1=c1, constant2=c2)
     rank = len(src.shape)
     taps = _taps(pattern, rank)
     res = Exp.of(f(*[Exp(src.ctype, "t%d" % k) for k in range(len(taps))]))

@@ -389,3 +389,25 @@ def test_stencil_producing_pairs(acc):
     assert np.array_equal(gx, t[1] - t[0]) and np.array_equal(gy, t[3] - t[2])
     mag = acc.run(acc.map(lambda p: acc.fst(p) * acc.fst(p) + acc.snd(p) * acc.snd(p), g), cx)
     assert np.array_equal(mag, (t[1] - t[0]) ** 2 + (t[3] - t[2]) ** 2)
+
+
+def test_stencil_over_an_array_of_pairs(acc):
+    """complex numbers as (re, im) pairs: a 3-point average along rows, the pairs kept together"""
+    cx = acc.Context(0)
+    rng = np.random.default_rng(15)
+    re, im = rng.integers(-9, 9, (33, 260)).astype(np.float32), rng.integers(-9, 9, (33, 260)).astype(np.float32)
+    z = acc.use((re, im), cx)
+
+    def avg(a, b, c):
+        return acc.lift(acc.fst(a) + acc.fst(b) + acc.fst(c), acc.snd(a) + acc.snd(b) + acc.snd(c))
+    out_re, out_im = acc.run(acc.stencil([(0, -1), (0, 0), (0, 1)], avg, "wrap", z, context=cx), cx)
+    tr = pyref.tap_arrays(re, [(0, -1), (0, 0), (0, 1)], "wrap", 0, re.shape)
+    ti = pyref.tap_arrays(im, [(0, -1), (0, 0), (0, 1)], "wrap", 0, im.shape)
+    assert np.array_equal(out_re, tr[0] + tr[1] + tr[2]) and np.array_equal(out_im, ti[0] + ti[1] + ti[2])
+    # and of a delayed array of pairs, with a constant boundary given as a pair
+    zz = acc.map(lambda p: acc.lift(acc.snd(p), acc.fst(p)), z)
+    o1, o2 = acc.run(acc.stencil([(-1, 0), (1, 0)], lambda u, d: acc.lift(acc.fst(d) - acc.fst(u), acc.snd(d) - acc.snd(u)),
+                                 "constant", zz, context=cx, constant_value=(1.0, -1.0)), cx)
+    ti2 = pyref.tap_arrays(im, [(-1, 0), (1, 0)], "constant", 1.0, im.shape)
+    tr2 = pyref.tap_arrays(re, [(-1, 0), (1, 0)], "constant", -1.0, re.shape)
+    assert np.array_equal(o1, ti2[1] - ti2[0]) and np.array_equal(o2, tr2[1] - tr2[0])
