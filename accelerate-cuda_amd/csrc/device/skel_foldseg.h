@@ -187,7 +187,9 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
  * `part` / `part_ok`, and <entry>_join puts the pieces of every segment
  * together, in order.                                                        */
 #define ACC_TVEC 4
+#ifndef ACC_TROUNDS
 #define ACC_TROUNDS 4
+#endif
 #define ACC_FS_WAVES (ACC_BLOCK / ACC_WAVE)
 #define ACC_FS_CAT2(a, b) a##b
 #define ACC_FS_CAT(a, b) ACC_FS_CAT2(a, b)
