@@ -95,7 +95,9 @@ template <typename T> ACC_DEV T acc_wave_shift_down1(const T &x) { return acc_dp
 template <typename S, int MODE, bool FAST>
 struct acc_strip_source {
   struct row { S e[ACC_WW]; };
-  struct __attribute__((aligned(ACC_SVEC * sizeof(S)))) vec { S v[ACC_SVEC]; };
+  /* one lane's run of a row.  When rows start on 16-byte boundaries (ACC_ALIGNED) the type says so; otherwise
+   * it is only element-aligned, which the memory instructions accept as well */
+  struct __attribute__((aligned(ACC_ALIGNED ? ACC_SVEC * sizeof(S) : alignof(S)))) vec { S v[ACC_SVEC]; };
 
   const S *base;            /* the array, its extents, the value outside it (constant boundary) */
   Int64 d, h, w;
@@ -267,11 +269,7 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS)
   if (y0 >= h) return;                                   /* whole wave leaves together */
   const Int64 gx = x0 + lane * ACC_SVEC;
   const int rows_here = (int)acc_min<Int64>(ACC_TILE_H, h - y0);
-#if ACC_ALIGNED
-  const bool fast_here = (x0 + ACC_STRIP <= w);          /* every lane owns a full, aligned vector */
-#else
-  const bool fast_here = false;
-#endif
+  const bool fast_here = (x0 + ACC_STRIP <= w);          /* every lane owns a full vector */
 
   /* the strip, compiled three times: fast and ACC_TILE_H rows tall (all constants),
    * fast and cut by the bottom edge, and the element-wise path */
@@ -359,10 +357,11 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS)
           CT *dst = arrOut_##c + at;                                                 \
           if (fast) {                                                                \
             typedef CT acc_out_native __attribute__((ext_vector_type(ACC_SVEC)));    \
+            typedef acc_out_native acc_out_stored __attribute__((aligned(ACC_ALIGNED ? ACC_SVEC * sizeof(CT) : alignof(CT)))); \
             acc_out_native nv;                                                       \
             _Pragma("unroll") for (int k = 0; k < ACC_SVEC; ++k) nv[k] = ACC_COMPONENT(res.v[k], c); \
-            if (ACC_STENCIL_NT & 1) __builtin_nontemporal_store(nv, (acc_out_native *)dst); \
-            else                    *(acc_out_native *)dst = nv;                     \
+            if (ACC_STENCIL_NT & 1) __builtin_nontemporal_store(nv, (acc_out_stored *)dst); \
+            else                    *(acc_out_stored *)dst = nv;                     \
           } else {                                                                   \
             _Pragma("unroll") for (int k = 0; k < ACC_SVEC; ++k)                     \
               if (gx + k < w) dst[k] = ACC_COMPONENT(res.v[k], c);                   \
