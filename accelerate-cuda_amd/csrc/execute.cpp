@@ -567,6 +567,64 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
   ACC_TRY(push_env(s, env, &args, &aligned));
   push_out(*out, &args, &aligned);
   args.i64(n_src);
+
+  // A hinted combination on more targets than two LDS tables hold: windows of targets, each with its share of the
+  // workgroups, which walk the whole source (skel_permute.h).  Up to `permute.max_windows` passes are cheaper than
+  // a device-scope atomic per element (27 G/s for the whole device).
+  if (s->spec.combine_hint != ACC_COMBINE_GENERIC) {
+    const int64_t wcap = std::max<int64_t>(1, lds_all / (int64_t)esz);
+    int win_log = 0;                                       // a power of two of windows: targets are dealt out modulo it
+    while (((ntarget + ((int64_t)1 << win_log) - 1) >> win_log) > wcap) ++win_log;
+    const int64_t windows = (int64_t)1 << win_log;
+    if (windows >= acc::tune("permute.windows_from", 2) && windows <= acc::tune("permute.max_windows", 32) && n_src >= 4 * ntarget) {
+      const int wv = (aligned ? 0 : 1) + 4;
+      ACC_TRY(s->ensure_variant(wv));
+      ACC_TRY(plain_copy());
+      const int64_t wbins = (ntarget + windows - 1) >> win_log;
+      const size_t wlds = (size_t)wbins * esz;
+      int bpc = 0;
+      hipError_t oe = hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&bpc, s->variants[wv].fn, s->spec.block, wlds);
+      if (oe != hipSuccess || bpc < 1) { (void)hipGetLastError(); bpc = 1; }
+      const int64_t cus_w = s->ctx->props.multiProcessorCount;
+      const int64_t win_blocks = std::max<int64_t>(1, std::min<int64_t>(cus_w * bpc / windows,
+                                                                         acc_launch_grid(n_src, s->elements_per_block(), cus_w, bpc)));
+      const int64_t wgrid = windows * win_blocks;
+      int wblk = -1;
+      ACC_TRY(s->ctx->scratch_acquire((size_t)(wgrid * wbins) * esz, st, acc::SCRATCH_FOLD, &wblk));
+      const uint64_t wdump = reinterpret_cast<uint64_t>(s->ctx->scratch[wblk].ptr);
+      args.i32(static_cast<int32_t>(wbins));
+      args.i32(1);
+      args.ptr(wdump);
+      args.ptr(0);
+      args.i32(static_cast<int32_t>(win_blocks));
+      args.i32(win_log);
+      int wrc = launch(s, wv, wgrid, wlds, st, &args);
+      if (wrc == ACC_OK) {
+        struct MergeJob { uint64_t dump; int64_t stride, first, cols; int32_t nrows, slices, window_log; };
+        const int64_t columns = (ntarget + 255) / 256;
+        const int64_t slices = std::max<int64_t>(1, std::min<int64_t>(win_blocks, (2 * cus_w + columns - 1) / columns));
+        MergeJob ja = {wdump, wbins, 0, ntarget, static_cast<int32_t>(win_blocks), static_cast<int32_t>(slices), win_log};
+        MergeJob jb = {0, 0, 0, 0, 0, 1, -1};
+        int32_t blocks_a32 = static_cast<int32_t>(columns * slices);
+        Args m;
+        bool mal = true;
+        wrc = push_env(s, env, &m, &mal);
+        push_out(*out, &m, &mal);
+        std::vector<void *> margs(m.data(), m.data() + m.count());
+        margs.push_back(&ja);
+        margs.push_back(&blocks_a32);
+        margs.push_back(&jb);
+        if (wrc == ACC_OK) {
+          hipError_t me = hipModuleLaunchKernel(s->variants[wv].fn_finish, static_cast<unsigned>(blocks_a32), 1, 1, 256, 1, 1, 0, st,
+                                                margs.data(), nullptr);
+          if (me != hipSuccess) wrc = acc::fail_hip(me, "hipModuleLaunchKernel(permute_merge, windows)");
+        }
+      }
+      s->ctx->scratch_release(wblk, st);
+      return wrc;
+    }
+  }
+
   const int v = aligned ? 0 : 1;
   ACC_TRY(s->ensure_variant(v));
 
@@ -628,16 +686,16 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
   if (rc == ACC_OK) rc = launch(s, v, grid, lds, st, &args);
   if (rc == ACC_OK && (table || far_rows)) {
     // the tables are folded into the result by one launch: the per-block window rows, the per-XCD rows
-    struct MergeJob { uint64_t dump; int64_t stride, first, cols; int32_t nrows, slices; };
+    struct MergeJob { uint64_t dump; int64_t stride, first, cols; int32_t nrows, slices, window_log; };
     auto job = [&](uint64_t tbl, int64_t stride, int64_t first, int64_t cols, int64_t rows, int64_t *blocks) {
       // enough workgroups to fill the machine: columns x row slices
       const int64_t columns = (cols + 255) / 256;
       const int64_t slices = std::max<int64_t>(1, std::min<int64_t>(rows, (2 * cus + columns - 1) / columns));
       *blocks = columns * slices;
-      return MergeJob{tbl, stride, first, cols, static_cast<int32_t>(rows), static_cast<int32_t>(slices)};
+      return MergeJob{tbl, stride, first, cols, static_cast<int32_t>(rows), static_cast<int32_t>(slices), -1};
     };
     int64_t blocks_a = 0, blocks_b = 0;
-    MergeJob ja = {0, 0, 0, 0, 0, 1}, jb = {0, 0, 0, 0, 0, 1};
+    MergeJob ja = {0, 0, 0, 0, 0, 1, -1}, jb = {0, 0, 0, 0, 0, 1, -1};
     if (table) ja = job(dump, bins, 0, bins, grid, &blocks_a);
     if (far_rows) jb = job(far, ntarget, bins, ntarget - bins, XCD_ROWS, &blocks_b);
     Args m;

@@ -249,6 +249,7 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "#define ACC_PERMUTATION(ix) " << sp.permutation << "\n";
       o << "#define ACC_COMBINE_HINT " << sp.combine_hint << "\n";
       o << "#define ACC_PERMUTE_LOCKED " << (sp.permute_locked ? 1 : 0) << "\n";
+      o << "#define ACC_PERMUTE_WINDOWS " << (sp.permute_windows ? 1 : 0) << "\n";
       o << "#define ACC_ELT_IS_INTEGER " << (is_integer_type(sp.elt_type) ? 1 : 0) << "\n";
       o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_UNROLL " << sp.unroll << "\n";
       tmpl = "skel_permute.h";
@@ -507,7 +508,8 @@ int acc_skel_s::ensure_variant(int v)
   if (var.ready) return ACC_OK;
   // variants 2 and 3 of a permute: the locked template for an element the atomic template also covers
   acc::SkelSpec spec = this->spec;
-  if (v >= 2) spec.permute_locked = true;
+  if (v >= 2 && v < 4) spec.permute_locked = true;
+  if (v >= 4) spec.permute_windows = true;
   std::string entry_name;
   ACC_TRY(acc::generate_source(spec, (v & 1) == 0, &entry_name, &var.source));
   entry = entry_name;

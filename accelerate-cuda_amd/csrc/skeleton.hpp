@@ -23,6 +23,7 @@ struct SkelSpec {
   std::string preamble, get, combine, seed, permutation;
   bool has_seed = false;
   int combine_hint = 0;
+  bool permute_windows = false;         // hinted permute over several LDS windows of targets (variants 4 and 5)
   bool permute_locked = false;          // permute of an element no atomic covers (tuples, 1/2/16-byte types): per-target locks
   std::string seg_type;
   // stencil
@@ -63,8 +64,9 @@ struct acc_skel_s {
   acc_context ctx = nullptr;
   acc::SkelSpec spec;
   std::string entry;
-  acc::Variant variants[4];   // [0] pointers 16-byte aligned, [1] no assumption; [2], [3]: the same for the
-                              // table-in-LDS form of a permute whose combination has no atomic instruction
+  acc::Variant variants[6];   // [0] pointers 16-byte aligned, [1] no assumption; [2], [3]: the same for the
+                              // table-in-LDS form of a permute whose combination has no atomic instruction;
+                              // [4], [5]: for a hinted permute over several LDS windows of targets
   std::mutex mu;
 
   int ensure_variant(int v);
