@@ -337,6 +337,39 @@ def test_permute_other_combines(A, ctx, orc):
     assert np.array_equal(out.get(), orc.permute(orc.OP_FIRST, np.full(5000, -1, np.int32), perm, vals))
 
 
+def test_permute_hinted_combines_over_windows_of_targets(A, ctx):
+    """more targets than one LDS table holds: 2, 4 and 16 windows, every hinted operator, Int32 and Int64 elements,
+    strays and `ignore` among the targets, a last window that is not full"""
+    n = 1 << 21
+    src = rng.integers(-10**6, 10**6, n, dtype=np.int32)
+    ds = ctx.array(src)
+    for bins in (50001, 150000, 500003):
+        dst = rng.integers(-3, bins + 3, n).astype(np.int32)
+        dst[::13] = -1
+        dd = ctx.array(dst)
+        ok = (dst >= 0) & (dst < bins)
+        for name, hint, comb, ufunc in [("add", A.COMBINE_ADD, "x + y", np.add), ("min", A.COMBINE_MIN, "acc_min(x, y)", np.minimum),
+                                        ("max", A.COMBINE_MAX, "acc_max(x, y)", np.maximum), ("xor", A.COMBINE_XOR, "x ^ y", np.bitwise_xor),
+                                        ("and", A.COMBINE_AND, "x & y", np.bitwise_and), ("or", A.COMBINE_OR, "x | y", np.bitwise_or)]:
+            say("hinted permute", name, "into", bins, "targets")
+            sk = ctx.skeleton(A.SKEL_PERMUTE, "Int32", env=[I32, I32], out_rank=1, get="arrIn1_0[ix]", combine=comb,
+                              permutation="arrIn0_0[ix]", combine_hint=hint)
+            dfl = rng.integers(-100, 100, bins, dtype=np.int32)
+            out = ctx.empty(bins, np.int32)
+            sk.permute([dd, ds], n, ctx.array(dfl), out)
+            ref = dfl.copy()
+            ufunc.at(ref, dst[ok], src[ok])
+            assert np.array_equal(out.get(), ref)
+        say("Int64 sums into", bins, "targets")
+        sk = ctx.skeleton(A.SKEL_PERMUTE, "Int64", env=[I32, I32], out_rank=1, get="(Int64)arrIn1_0[ix] * 1000003", combine="x + y",
+                          permutation="arrIn0_0[ix]", combine_hint=A.COMBINE_ADD)
+        out = ctx.empty(bins, np.int64)
+        sk.permute([dd, ds], n, ctx.array(np.zeros(bins, np.int64)), out)
+        ref = np.zeros(bins, np.int64)
+        np.add.at(ref, dst[ok], src[ok].astype(np.int64) * 1000003)
+        assert np.array_equal(out.get(), ref)
+
+
 # --------------------------------------------------------------------------- stencil
 
 GAUSS_TAPS = [(dy, dx) for dy in (-1, 0, 1) for dx in (-1, 0, 1)]
