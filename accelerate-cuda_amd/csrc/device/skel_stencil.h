@@ -61,7 +61,12 @@
 #ifndef ACC_RADIUS_Z
 #define ACC_RADIUS_Z 0
 #endif
-#define ACC_NZ    (2 * ACC_RADIUS_Z + 1)              /* planes a result depends on */
+#ifndef ACC_TZ
+#define ACC_TZ 1
+#endif
+/* a strip produces ACC_TZ consecutive planes of the result from one register window over
+ * ACC_NZ source planes: a source row fetched once serves the results of up to 2 rz + 1 planes */
+#define ACC_NZ    (2 * ACC_RADIUS_Z + ACC_TZ)         /* planes held */
 #define ACC_TOTAL_MAX  (ACC_TILE_H + 2 * ACC_RADIUS_Y)        /* source rows a strip touches, per plane */
 #define ACC_HALO_COUNT (2 * ACC_RADIUS_X * ACC_TOTAL_MAX * ACC_NZ)   /* elements just outside the strip */
 #define ACC_HALO_LOADS (ACC_HALO_COUNT > 0 ? (ACC_HALO_COUNT + ACC_WAVE - 1) / ACC_WAVE : 1)
@@ -261,7 +266,7 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS)
 #endif
 #if ACC_STENCIL_RANK == 3
   const Int64 bands = (h + ACC_TILE_H - 1) / ACC_TILE_H;
-  const Int64 z0 = band / bands, y0 = (band % bands) * ACC_TILE_H;
+  const Int64 z0 = (band / bands) * ACC_TZ, y0 = (band % bands) * ACC_TILE_H;
   if (z0 >= d) return;
 #else
   const Int64 z0 = 0, y0 = band * ACC_TILE_H;
@@ -337,21 +342,24 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS)
         if (rho_new < total) ACC_BOTH(fetch(rho_new, (s + ACC_RING - 1) % ACC_RING));
         ACC_BOTH(finish(y + ACC_NR - 1, (s + ACC_NR - 1) % ACC_RING));
 
+#pragma unroll
+        for (int pz = 0; pz < ACC_TZ; ++pz) {
+        if (ACC_TZ > 1 && z0 + pz >= d) break;               /* the last band of planes may be short */
         acc_out_vec res;
 #pragma unroll
         for (int k = 0; k < ACC_SVEC; ++k) {
-#define ACC_WINDOW_READ(dz, dy, dx) a.ring[ACC_RADIUS_Z + (dz)][(s + ACC_RADIUS_Y + (dy)) % ACC_RING].e[ACC_RADIUS_X + k + (dx)]
+#define ACC_WINDOW_READ(dz, dy, dx) a.ring[pz + ACC_RADIUS_Z + (dz)][(s + ACC_RADIUS_Y + (dy)) % ACC_RING].e[ACC_RADIUS_X + k + (dx)]
           ACC_STENCIL_TAPS(ACC_WINDOW_READ)
 #undef ACC_WINDOW_READ
 #if ACC_STENCIL_SOURCES == 2
-#define ACC_WINDOW_READ(dz, dy, dx) b.ring[ACC_RADIUS_Z + (dz)][(s + ACC_RADIUS_Y + (dy)) % ACC_RING].e[ACC_RADIUS_X + k + (dx)]
+#define ACC_WINDOW_READ(dz, dy, dx) b.ring[pz + ACC_RADIUS_Z + (dz)][(s + ACC_RADIUS_Y + (dy)) % ACC_RING].e[ACC_RADIUS_X + k + (dx)]
           ACC_STENCIL_TAPS2(ACC_WINDOW_READ)
 #undef ACC_WINDOW_READ
 #endif
           res.v[k] = (T)(ACC_STENCIL_FN);
         }
         /* one vector store per component of the result (a tuple result is one array per component) */
-        const Int64 at = ((z0 * h) + (y0 + y)) * w + gx;
+        const Int64 at = (((z0 + pz) * h) + (y0 + y)) * w + gx;
 #define ACC_STORE_COMPONENT(c, CT)                                                   \
         {                                                                            \
           CT *dst = arrOut_##c + at;                                                 \
@@ -369,6 +377,7 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS)
         }
         ACC_FOR_COMPONENTS(ACC_STORE_COMPONENT)
 #undef ACC_STORE_COMPONENT
+        }   /* pz */
       }
     }
   }

@@ -295,6 +295,7 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "#define ACC_STENCIL_NT " << tune("stencil.nt", 1) << "\n";
       o << "#define ACC_STACK_WAVES " << (sp.out_rank == 2 ? tune("stencil.stack", 0) : 0) << "\n";
       o << "#define ACC_TILE_H " << sp.tile_h << "\n#define ACC_PREFETCH " << sp.prefetch << "\n#define ACC_BLOCK " << sp.block << "\n";
+      o << "#define ACC_TZ " << sp.tile_z << "\n";
       tmpl = "skel_stencil.h";
       break;
     }
@@ -467,11 +468,28 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
       }
       sp->block = tune("stencil.block", 256);
       sp->tile_w = 256;                                  // one wave's strip: 64 lanes x 4 columns
-      // rows per strip: short in 2-D (a compact window of the image in flight), taller in 3-D where every row is
-      // read from 2 rz + 1 planes and the boundary rows of a strip cost that much more
-      sp->tile_h = sp->out_rank == 2 ? tune("stencil.tile_h", 4) : (sp->out_rank == 3 ? tune("stencil.tile_h3", 16) : 1);
       sp->prefetch = sp->out_rank == 2 ? tune("stencil.prefetch", 3) : (sp->out_rank == 3 ? tune("stencil.prefetch3", 1) : 0);
-      if (sp->tile_h < 1 || sp->prefetch < 0 || sp->prefetch > 8) return fail(ACC_ERR_INVALID, "stencil: bad tile shape");
+      // 3-D: a strip that reaches across planes produces up to three planes of the result from one register window
+      // (each source row it fetches then serves several planes instead of one), as many as keep the window of all
+      // sources within 128 registers a lane
+      int planes_per_strip = 1;
+      if (sp->out_rank == 3) {
+        int rz = 0, ry = 0, rx = 0;      // both sources' windows span the larger of the two radii
+        auto reach = [&](const std::vector<int> &dz, const std::vector<int> &dy, const std::vector<int> &dx) {
+          for (size_t k = 0; k < dx.size(); ++k) { rz = std::max(rz, std::abs(dz[k])); ry = std::max(ry, std::abs(dy[k])); rx = std::max(rx, std::abs(dx[k])); }
+        };
+        reach(sp->tap_dz, sp->tap_dy, sp->tap_dx);
+        reach(sp->tap2_dz, sp->tap2_dy, sp->tap2_dx);
+        int words = std::max(1, (type_size(sp->stencil_in_type) + 3) / 4);
+        if (d->kind == ACC_SKEL_STENCIL2) words += std::max(1, (type_size(sp->stencil_in2_type) + 3) / 4);
+        for (int tz = 3; rz > 0 && tz > 1 && planes_per_strip == 1; --tz)
+          if ((2 * rz + tz) * (2 * ry + 1 + sp->prefetch) * (4 + 2 * rx) * words <= 128) planes_per_strip = tz;
+      }
+      sp->tile_z = sp->out_rank == 3 ? tune("stencil.tile_z", planes_per_strip) : 1;
+      // rows per strip: short in 2-D (a compact window of the image in flight), taller in 3-D where every row is
+      // read from 2 rz + tile_z planes and the boundary rows of a strip cost that much more
+      sp->tile_h = sp->out_rank == 2 ? tune("stencil.tile_h", 4) : (sp->out_rank == 3 ? tune("stencil.tile_h3", sp->tile_z > 1 ? 8 : 16) : 1);
+      if (sp->tile_h < 1 || sp->prefetch < 0 || sp->prefetch > 8 || sp->tile_z < 1 || sp->tile_z > 8) return fail(ACC_ERR_INVALID, "stencil: bad tile shape");
       break;
     }
     default:   // scans

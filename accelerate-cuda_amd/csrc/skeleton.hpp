@@ -35,6 +35,7 @@ struct SkelSpec {
   std::string boundary2_constant, stencil_in2_type;
   std::vector<int> tap2_dz, tap2_dy, tap2_dx;
   int tile_w = 256, tile_h = 4, prefetch = 3;
+  int tile_z = 1;                       // rank-3 stencils: result planes per strip
   // tuning
   int block = 256, unroll = 4, rows = 4, chunk = 4096;
 };

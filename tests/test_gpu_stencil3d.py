@@ -89,3 +89,28 @@ def test_stencil2_3d_and_iteration(A, ctx):
         t = pyref.tap_arrays3(exp, SEVEN, "clamp", 0, v.shape)
         exp = (t[0] + t[0] + t[1] + t[2] + t[3] + t[4] + t[5] + t[6]) * F(0.125)
     assert np.array_equal(res, exp)
+
+
+@pytest.mark.parametrize("case", ["wide in x", "two planes either side", "Float64", "within the plane"])
+def test_stencil_3d_window_shapes(A, ctx, case):
+    """Neighbourhoods of other reaches: how many planes of the result a strip produces at once follows the
+    registers its window takes, so each of these runs a different tiling of the depth."""
+    rng = np.random.default_rng(33)
+    taps, ctype, T = SEVEN, "float", F
+    if case == "wide in x":
+        taps = SEVEN + [(0, 0, -2), (0, 0, 2)]
+    elif case == "two planes either side":
+        taps = SEVEN + [(-2, 0, 0), (2, 0, 0)]
+    elif case == "Float64":
+        ctype, T = "double", np.float64
+    else:
+        taps = [(0, dy, dx) for dy in (-1, 0, 1) for dx in (-1, 0, 1)]
+    fn = " + ".join("(%s)%d * t%d" % (ctype, k % 7 - 3, k) for k in range(len(taps)))
+    sk = ctx.skeleton(A.SKEL_STENCIL, ctype, out_rank=3, taps=taps, boundary="mirror", stencil_fn=fn)
+    for shape in [(3, 3, 3), (5, 7, 9), (7, 19, 300), (8, 16, 512), (11, 33, 257)]:
+        say("stencil 3-D", case, shape)
+        v = rng.integers(-9, 9, shape).astype(T)
+        out = ctx.empty(shape, T)
+        sk.stencil([], ctx.array(v), out)
+        t = pyref.tap_arrays3(v, taps, "mirror", 0, shape)
+        assert np.array_equal(out.get(), sum(T(k % 7 - 3) * t[k] for k in range(len(taps))))
