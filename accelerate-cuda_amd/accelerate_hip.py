@@ -1,7 +1,10 @@
 """An embedded array language over libacchip, shaped like the surface a user of
 the reference programs against (Data.Array.Accelerate + Data.Array.Accelerate.CUDA:
 `use`, `map`, `zipWith`, `generate`, `backpermute`, `fold`, `foldSeg`, the scans,
-`permute`, `stencil`, `run`, `run1` -- CUDA.hs:184-200).
+`permute`, `stencil`, and the whole export list of CUDA.hs:184-200: `run`, `run1`,
+`runWith`, `run1With`, `stream`, `streamWith`, `Async`, `wait`, `poll`, `cancel`,
+`runAsync`, `run1Async`, `runAsyncWith`, `run1AsyncWith`, `Context`, `create`,
+`destroy`, `unsafeFree`, `unsafeFreeWith`, `performGC`, `performGCWith`; also `runN`).
 
     import accelerate_hip as acc
     def dotp(xs, ys):
@@ -25,6 +28,7 @@ Everything runs on the GPU through the C ABI; there is no other execution path.
 """
 import numbers
 import re
+import threading
 import weakref
 
 import numpy as np
@@ -36,7 +40,9 @@ __all__ = ["Exp", "constant", "cond", "use", "unit", "map", "zipWith", "generate
            "stencil", "stencil2", "awhile", "run", "run1", "fill", "enumFromN", "take", "drop", "init", "tail", "gather",
            "scatter", "foldAll", "sum_", "product", "maximum", "minimum", "and_", "or_", "all_", "any_", "filter_", "fst", "snd", "lift", "index_if", "fromIntegral", "truncate", "round_", "floor",
            "ceiling", "idiv", "mod", "quot", "rem", "min_", "max_", "sqrt", "exp", "log", "sin", "cos", "tan", "abs_",
-           "signum", "Context", "the"]
+           "signum", "Context", "the", "runWith", "run1With", "runN", "stream", "streamWith", "Async", "wait", "poll",
+           "cancel", "Cancelled", "runAsync", "run1Async", "runAsyncWith", "run1AsyncWith", "create", "destroy",
+           "unsafeFree", "unsafeFreeWith", "performGC", "performGCWith"]
 
 CTYPE = dict(A.CTYPE_OF)
 NPTYPE = {v: k for k, v in CTYPE.items()}
@@ -336,6 +342,28 @@ def _assemble(**fragments):
     return arrays, sig, out
 
 
+def _context(context, *operands):
+    """where a skeleton runs: the context given, else the one its array operands live in (the context of
+    `use ... context`), else the default one (CUDA.hs:205-206 `defaultContext`)"""
+    if context is not None:
+        return context
+    found = None
+    for a in operands:
+        if isinstance(a, Acc) and a.manifest is not None:
+            ms = [a.manifest]
+        elif isinstance(a, (Acc, str)):          # a delayed array, or the text of a fragment: the arrays it names
+            ms = [_MANIFEST[int(i)] for i in re.findall(r"@@(\d+)@@", a if isinstance(a, str) else a.stream().text)]
+        else:
+            continue
+        for m in ms:
+            for c in (m.comps if isinstance(m, A.TupleArray) else [m]):
+                cx = getattr(c, "cx", None)
+                if cx is not None and found is not None and cx is not found:
+                    raise ValueError("the operands of one computation live in different contexts")
+                found = found or cx
+    return found or Context.default()
+
+
 class _Resident(object):
     """A manifest array under the context's memory table: host storage (the array `use`d, or the place a result is
     written back to when the device is full) and the table entry keyed by it.  The device address is only known
@@ -371,6 +399,13 @@ class _Resident(object):
             pass
 
 
+class Cancelled(Exception):
+    """raised inside, and by `wait` on, a computation that `cancel` stopped"""
+
+
+_running = threading.local()     # .asy: the Async whose thread this is
+
+
 class Context(object):
     """a device context, the table of skeleton instances built so far (the kernel table of State.hs:110-119) and the
     memory table every manifest array lives in (State.hs:120-122): `budget_bytes` bounds the device memory held,
@@ -386,6 +421,7 @@ class Context(object):
         self.live = {}
         self.skeletons = {}
         self.streams, self.turn, self.events = [], 0, []
+        self.lock = threading.RLock()      # one host thread at a time evaluates in a context (CUDA.hs:251-252)
 
     @classmethod
     def default(cls):
@@ -423,6 +459,9 @@ class Context(object):
                         yield c
                 elif m is not None:
                     yield m
+        asy = getattr(_running, "asy", None)
+        if asy is not None and asy._cancelled:
+            raise Cancelled()                           # between two skeletons: a launch already made runs to its end
         stream = self._stream_for(list(parts(inputs)))
         L = A.lib()
         for m in parts(inputs):
@@ -585,7 +624,7 @@ def _combine(f, ctype):
 
 
 def _fold(f, z, a, seedless, context):
-    cx = context or Context.default()
+    cx = _context(context, a)
     out_shape = a.shape[:-1]
     arrays, sig, fr = _assemble(get=a.stream().text, combine=_combine(f, a.ctype).text,
                                 seed=None if seedless else Exp.of(z, a.ctype).text)
@@ -607,7 +646,7 @@ def fold1(f, a, context=None):
 def foldSeg(f, z, a, seg_lengths, context=None):
     """reduce each segment of a vector; `seg_lengths` is a vector of segment lengths (Int32), turned into
     offsets by an exclusive scan on the device as the front end does (CUDA.hs:402)"""
-    cx = context or Context.default()
+    cx = _context(context, a, seg_lengths)
     offs = scanl(lambda x, y: x + y, constant(0, seg_lengths.ctype), seg_lengths, context=cx)
     arrays, sig, fr = _assemble(get=a.stream().text, combine=_combine(f, a.ctype).text, seed=Exp.of(z, a.ctype).text)
     sk = cx.skeleton(A.SKEL_FOLDSEG, _elt(a.ctype), sig, seg_type=seg_lengths.ctype, **fr)
@@ -618,7 +657,7 @@ def foldSeg(f, z, a, seg_lengths, context=None):
 
 
 def _scan(kind, f, z, a, context):
-    cx = context or Context.default()
+    cx = _context(context, a)
     if len(a.shape) != 1:
         raise TypeError("scans are over vectors")
     arrays, sig, fr = _assemble(get=a.stream().text, combine=_combine(f, a.ctype).text,
@@ -673,15 +712,15 @@ def index_if(p, idx):
 def permute(f, defaults, p, a, context=None):
     """forward permutation: out = defaults; out[p(i)] = f(a[i], out[p(i)]) for every source index i;
     p(i) = ignore (or index_if with a false condition) drops the element"""
-    cx = context or Context.default()
-    dfl = _force(defaults, cx)
     t = p(*_unlinear(Exp("Int64", "ix"), a.shape))
     if isinstance(t, str) and t == ignore:
         perm_text = "ACC_IGNORE"
     elif isinstance(t, _Maybe):
-        perm_text = Exp.mk("Int64", "(%s ? %s : ACC_IGNORE)", t.p, _linear(t.idx, dfl.shape)).text
+        perm_text = Exp.mk("Int64", "(%s ? %s : ACC_IGNORE)", t.p, _linear(t.idx, defaults.shape)).text
     else:
-        perm_text = _linear(t, dfl.shape).text
+        perm_text = _linear(t, defaults.shape).text
+    cx = _context(context, defaults, a, perm_text)
+    dfl = _force(defaults, cx)
     arrays, sig, fr = _assemble(get=a.stream().text, combine=_combine(f, a.ctype).text, permutation=perm_text)
     sk = cx.skeleton(A.SKEL_PERMUTE, _elt(a.ctype), sig, out_rank=len(dfl.shape), combine_hint=_hint(f, a.ctype), **fr)
     out = _empty(cx, dfl.shape, a.ctype)
@@ -705,7 +744,7 @@ def _taps(pattern, rank):
 def stencil(pattern, f, boundary, a, context=None, constant_value=None):
     """result[i] = f(a[i + o] for o in pattern); boundary is "clamp", "mirror", "wrap" or "constant"
     (Stencil/Extra.hs:112-116); the source is made manifest first, as in the reference (Execute.hs:413-425)"""
-    cx = context or Context.default()
+    cx = _context(context, a)
     src = _force(a, cx)
     if isinstance(src.ctype, tuple):
         # an array of pairs is two arrays: the same pattern over both, as a stencil2 (the sources of the
@@ -732,7 +771,7 @@ def stencil(pattern, f, boundary, a, context=None, constant_value=None):
 
 def stencil2(pattern1, pattern2, f, boundary1, a, boundary2, b, context=None, constant1=None, constant2=None):
     """f receives the list of taps of the first source and the list of taps of the second"""
-    cx = context or Context.default()
+    cx = _context(context, a, b)
     s1, s2 = _force(a, cx), _force(b, cx)
     rank = len(s1.shape)
     t1, t2 = _taps(pattern1, rank), _taps(pattern2, rank)
@@ -816,7 +855,7 @@ def any_(p, a, context=None): return or_(map(p, a), context)
 def filter_(p, a, context=None):
     """the elements of a vector that satisfy p, in order, and how many there are: the scan-then-permute
     compaction of the Prelude (an exclusive scan of the flags gives every kept element its place)"""
-    cx = context or Context.default()
+    cx = _context(context, a)
     a = _force(a, cx)
     flags = map(lambda v: cond(p(v), constant(1, "Int32"), constant(0, "Int32")), a)
     places, count = scanl_(lambda x, y: x + y, 0, flags, context=cx)
@@ -833,7 +872,7 @@ def awhile(p, f, a, context=None, limit=None):
     """iterate the array function `f` from `a` while the scalar array `p(a)` holds a non-zero value
     (Execute.hs:236-244).  `a` is an Acc or a tuple of them; every iterate is made manifest, and the
     flag is the one value read back per iteration."""
-    cx = context or Context.default()
+    cx = _context(context, *(a if isinstance(a, tuple) else (a,)))
     tup = isinstance(a, tuple)
     force = lambda v: tuple(_force(x, cx) for x in v) if tup else _force(v, cx)
     a = force(a)
@@ -851,10 +890,11 @@ def awhile(p, f, a, context=None, limit=None):
 
 def run(a, context=None):
     """evaluate and bring the result to the host (CUDA.hs:209-216); a tuple of Acc gives a tuple of results"""
-    cx = context or Context.default()
-    if isinstance(a, tuple):
-        return tuple(run(x, cx) for x in a)
-    return _force(a, cx).manifest.get()
+    cx = _context(context, *(a if isinstance(a, tuple) else (a,)))
+    with cx.lock:
+        if isinstance(a, tuple):
+            return tuple(run(x, cx) for x in a)
+        return _force(a, cx).manifest.get()
 
 
 def run1(f, context=None):
@@ -865,3 +905,133 @@ def run1(f, context=None):
     def go(*hosts):
         return run(f(*[use(h, cx) for h in hosts]), cx)
     return go
+
+
+def runN(f, context=None):
+    """`run1` for a function of several arrays (`run1` over the uncurried argument tuple)"""
+    return run1(f, context)
+
+
+def runWith(context, a):
+    """`run` in the given context instead of the default one (CUDA.hs:231-234)"""
+    return run(a, context)
+
+
+def run1With(context, f):
+    """`run1` in the given context (CUDA.hs:306-309)"""
+    return run1(f, context)
+
+
+def stream(f, arrays, context=None):
+    """the array function applied to each of a sequence of inputs, kernels built once; like the lazy list of
+    CUDA.hs:338-344 an element is computed when it is asked for"""
+    go = run1(f, context)
+    for a in arrays:
+        yield go(*a) if isinstance(a, tuple) else go(a)
+
+
+def streamWith(context, f, arrays):
+    return stream(f, arrays, context)
+
+
+class Async(object):
+    """A computation running in a host thread of its own (the `Async` of the accelerate package that CUDA.hs:194-196
+    re-exports with `wait`, `poll` and `cancel`; started by `asyncBound`, CUDA.hs:263,323).  Threads of one context
+    take turns; computations in different contexts overlap."""
+
+    def __init__(self, work):
+        self._done, self._cancelled = threading.Event(), False
+        self._value, self._error = None, None
+
+        def body():
+            _running.asy = self
+            try:
+                self._value = work()
+            except BaseException as e:            # delivered to whoever waits
+                self._error = e
+            finally:
+                self._done.set()
+        self._thread = threading.Thread(target=body, daemon=True)
+        self._thread.start()
+
+
+def wait(asy):
+    """block until the computation has finished; its result, or the exception that ended it"""
+    asy._done.wait()
+    if asy._cancelled:
+        raise Cancelled()
+    if asy._error is not None:
+        raise asy._error
+    return asy._value
+
+
+def poll(asy):
+    """None while the computation runs, afterwards what `wait` gives"""
+    return wait(asy) if asy._done.is_set() else None
+
+
+def cancel(asy):
+    """stop the computation at its next skeleton (kernels already launched finish) and drop its result"""
+    asy._cancelled = True
+    asy._done.wait()
+
+
+def runAsync(a, context=None):
+    """`run` without waiting for the result (CUDA.hs:246-263)"""
+    return Async(lambda: run(a, context))
+
+
+def runAsyncWith(context, a):
+    return runAsync(a, context)
+
+
+def run1Async(f, context=None):
+    """`run1` whose applications return at once (CUDA.hs:312-323)"""
+    go = run1(f, context)
+    return lambda *hosts: Async(lambda: go(*hosts))
+
+
+def run1AsyncWith(context, f):
+    return run1Async(f, context)
+
+
+def create(device=0, budget_bytes=0):
+    """a new execution context on the given device (Context.hs:73-84)"""
+    return Context(device, budget_bytes)
+
+
+def destroy(context):
+    """release the context's kernels, streams, events and device memory (Context.hs:100-103); arrays and
+    computations made in it must not be used afterwards"""
+    with context.lock:
+        context.ctx.sync()
+        context.skeletons.clear()
+        context.streams, context.events = [], []
+        context.table.destroy()
+        context.ctx.close()
+    if Context._default is context:
+        Context._default = None
+
+
+def unsafeFree(arrays, context=None):
+    """give back the device copies of host arrays now instead of when their last `use` is dropped (CUDA.hs:421-432).
+    Unsafe as there: a computation that still refers to one of them fails when it looks the array up."""
+    cx = context or Context.default()
+    with cx.lock:
+        for h in (arrays if isinstance(arrays, (tuple, list)) else (arrays,)):
+            cx.table.free(np.asarray(h, order="C"))
+
+
+def unsafeFreeWith(context, arrays):
+    unsafeFree(arrays, context)
+
+
+def performGC(context=None):
+    """return to the device the blocks the memory table keeps for reuse (CUDA.hs:436-441, Array/Remote.hs `cleanup`)"""
+    cx = context or Context.default()
+    with cx.lock:
+        cx.table.reclaim()
+
+
+def performGCWith(context):
+    performGC(context)

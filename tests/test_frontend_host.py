@@ -107,3 +107,34 @@ def test_while_is_a_statement_ahead_of_the_expression_and_compiles():
     assert len(both.binds) == 1
     with pytest.raises(TypeError):
         acc.while_(lambda k: k < 3, lambda k: acc.fromIntegral(k, "Int32"), acc.constant(0, "Int64"))
+
+
+def test_async_wait_poll_cancel_without_a_device():
+    """the thread-backed `Async` on its own: results and exceptions come out of `wait`, `poll` says None while the
+    work runs, a cancelled computation raises `Cancelled`"""
+    import threading
+    gate = threading.Event()
+    a = acc.Async(lambda: (gate.wait(), 42)[1])
+    assert acc.poll(a) is None
+    gate.set()
+    assert acc.wait(a) == 42 and acc.poll(a) == 42
+
+    def boom():
+        raise ValueError("from the worker")
+    with pytest.raises(ValueError, match="from the worker"):
+        acc.wait(acc.Async(boom))
+
+    gate2 = threading.Event()
+    b = acc.Async(lambda: gate2.wait())
+    stopper = threading.Thread(target=acc.cancel, args=(b,))
+    stopper.start()                   # cancel waits for the thread to reach a stopping point: here, the end of its work
+    gate2.set()
+    stopper.join()
+    with pytest.raises(acc.Cancelled):
+        acc.wait(b)
+
+
+def test_the_export_list_of_the_reference_module_is_there():
+    for name in ("run run1 runWith run1With stream streamWith Async wait poll cancel runAsync run1Async runAsyncWith "
+                 "run1AsyncWith Context create destroy unsafeFree unsafeFreeWith performGC performGCWith runN").split():
+        assert callable(getattr(acc, name)), name

@@ -411,3 +411,64 @@ def test_stencil_over_an_array_of_pairs(acc):
     ti2 = pyref.tap_arrays(im, [(-1, 0), (1, 0)], "constant", 1.0, im.shape)
     tr2 = pyref.tap_arrays(re, [(-1, 0), (1, 0)], "constant", -1.0, re.shape)
     assert np.array_equal(o1, ti2[1] - ti2[0]) and np.array_equal(o2, tr2[1] - tr2[0])
+
+
+def test_contexts_streams_of_inputs_and_asynchronous_runs(acc):
+    """the rest of the reference module's export list (CUDA.hs:184-200): *With variants over a context made with
+    `create`, `stream` over a sequence of inputs, `runAsync`/`run1Async` with `wait`/`poll`/`cancel`, `unsafeFree`
+    and `performGC`"""
+    rng = np.random.default_rng(40)
+    cx = acc.create(0)
+    try:
+        x = rng.integers(-9, 9, 50001).astype(np.int32)
+        assert np.array_equal(acc.runWith(cx, acc.scanl1(add, acc.use(x, cx), context=cx)), np.cumsum(x, dtype=np.int32))
+        step = lambda xs: acc.map(lambda v: v * 3 + 1, xs)
+        assert np.array_equal(acc.run1With(cx, step)(x), x * 3 + 1)
+        inputs = [rng.integers(-9, 9, n).astype(np.int32) for n in (1, 1000, 77777)]
+        n_kernels = None
+        for a, r in zip(inputs, acc.streamWith(cx, step, inputs)):
+            assert np.array_equal(r, a * 3 + 1)
+            n_kernels = n_kernels or len(cx.skeletons)
+        assert len(cx.skeletons) == n_kernels                     # built for the first input, reused for the rest
+        # several computations in flight, in this context and the default one
+        ys = [rng.standard_normal(200003).astype(np.float32) for _ in range(4)]
+        dot = lambda a, b: acc.fold(add, 0.0, acc.zipWith(lambda p, q: p * q, a, b))
+        jobs = [acc.runAsyncWith(cx if k % 2 else acc.Context.default(),
+                                 dot(acc.use(y, cx if k % 2 else None), acc.use(ys[0], cx if k % 2 else None)))
+                for k, y in enumerate(ys)]
+        for y, j in zip(ys, jobs):
+            r = acc.wait(j)
+            assert abs(float(r) - float(np.dot(y.astype(np.float64), ys[0].astype(np.float64)))) < 1e-3 * np.sqrt(y.size)
+            assert acc.poll(j) is not None
+        go = acc.run1AsyncWith(cx, step)
+        assert np.array_equal(acc.wait(go(x)), x * 3 + 1)
+        # a cancelled computation stops at its next skeleton and says so
+        import threading
+        gate = threading.Event()
+
+        def slow(xs):
+            gate.wait()
+            return acc.map(lambda v: v + 1, xs)
+        j = acc.Async(lambda: acc.run(slow(acc.use(x, cx)), cx))
+        stopper = threading.Thread(target=acc.cancel, args=(j,))
+        stopper.start()
+        while not j._cancelled:
+            pass
+        gate.set()
+        stopper.join()
+        with pytest.raises(acc.Cancelled):
+            acc.wait(j)
+        # unsafeFree gives the device copy back at once; performGC empties the pool of freed blocks
+        big = rng.integers(0, 9, 1 << 20).astype(np.int32)
+        xs = acc.use(big, cx)
+        assert int(acc.runWith(cx, acc.fold(add, 0, xs, context=cx))) == int(big.sum())
+        resident = cx.table.stats()["resident_arrays"]
+        acc.unsafeFreeWith(cx, big)
+        assert cx.table.stats()["resident_arrays"] == resident - 1
+        with pytest.raises(Exception):
+            acc.runWith(cx, acc.fold(add, 0, xs, context=cx))     # the computation still refers to it: it fails, loudly
+        acc.performGCWith(cx)
+        assert cx.table.stats()["nursery_bytes"] == 0
+    finally:
+        acc.destroy(cx)
+    assert cx.ctx.handle is None
