@@ -1,0 +1,309 @@
+{-# LANGUAGE ForeignFunctionInterface, EmptyDataDecls, DeriveDataTypeable #-}
+-- |
+-- Module      : Data.Array.Accelerate.HIP.FFI
+--
+-- Bindings to libacchip (include/acc_hip.h), one foreign import per entry point of the
+-- library, for a Data.Array.Accelerate.HIP backend that keeps the structure of
+-- Data.Array.Accelerate.CUDA and replaces what that obtains from the `cuda` package,
+-- from nvcc and from its own skeleton templates.
+--
+-- UNCOMPILED: the image this library is built and tested in holds no GHC.  The import
+-- list is checked mechanically against the header (names and argument counts); the
+-- Storable instances use hsc2hs against the same header, so offsets cannot drift.
+--
+-- Calls that can block (compilation, synchronisation, copies, anything that may
+-- allocate) are `safe`; the two string getters and the pure launch arithmetic are `unsafe`.
+-- Every entry point makes the context's device current itself and may be called from any
+-- thread, so the bound-thread / push / pop discipline of State.hs:84-92 is not needed.
+--
+module Data.Array.Accelerate.HIP.FFI where
+
+import Control.Exception
+import Control.Monad
+import Data.Typeable
+import Foreign
+import Foreign.C
+
+#include "acc_hip.h"
+
+data CContext
+data CSkel
+data CMemTable
+type Context  = Ptr CContext
+type Skel     = Ptr CSkel
+type MemTable = Ptr CMemTable
+type Stream   = Ptr ()               -- hipStream_t; nullPtr is the default stream
+type Event    = Ptr ()
+type Module   = Ptr ()
+type Function = Ptr ()
+type DevPtr   = Word64               -- in place of Foreign.CUDA.Ptr.DevicePtr: advanceDevPtr / plusDevPtr are (+)
+type Status   = CInt
+
+-- ---------------------------------------------------------------------------------------------------------
+-- status codes and the exception they become (the reference's CUDAException; State.hs:86-88)
+
+accOK, accErrInvalid, accErrOOM, accErrCompile, accErrNotFound, accErrHIP, accErrUnsupported, accErrIO :: Status
+accOK             = #{const ACC_OK}
+accErrInvalid     = #{const ACC_ERR_INVALID}
+accErrOOM         = #{const ACC_ERR_OOM}
+accErrCompile     = #{const ACC_ERR_COMPILE}
+accErrNotFound    = #{const ACC_ERR_NOT_FOUND}
+accErrHIP         = #{const ACC_ERR_HIP}
+accErrUnsupported = #{const ACC_ERR_UNSUPPORTED}
+accErrIO          = #{const ACC_ERR_IO}
+
+data HIPException = HIPException Status String
+  deriving (Typeable)
+
+instance Show HIPException where
+  show (HIPException s msg) = "libacchip (status " ++ show s ++ "): " ++ msg
+
+instance Exception HIPException
+
+-- | run an entry point; any status but ACC_OK is thrown with the library's message for it
+check :: IO Status -> IO ()
+check io = do
+  s <- io
+  when (s /= accOK) $ do
+    msg <- peekCString =<< c_lastError
+    throwIO (HIPException s msg)
+
+-- | as `check`, for allocation: out of device memory is an ordinary result, so that the caller may evict and
+-- try again (Array/Remote.hs:63-67)
+checkAlloc :: IO Status -> IO Bool
+checkAlloc io = do
+  s <- io
+  if s == accErrOOM then return False else check (return s) >> return True
+
+-- ---------------------------------------------------------------------------------------------------------
+-- structures
+
+-- | a device-resident array as the kernels see it: extents outermost first, one pointer per tuple component
+-- (what Execute.hs:823-873 `Marshalable` flattens into kernel arguments)
+data AccArray = AccArray
+  { arrayShape :: [Int64]            -- rank = length, at most ACC_MAX_RANK
+  , arrayPtrs  :: [DevPtr]           -- component 0 first, at most ACC_MAX_COMP
+  }
+
+instance Storable AccArray where
+  sizeOf    _ = #{size acc_array}
+  alignment _ = #{alignment acc_array}
+  peek p = do
+    rank  <- #{peek acc_array, rank}  p :: IO Int32
+    ncomp <- #{peek acc_array, ncomp} p :: IO Int32
+    sh    <- peekArray (fromIntegral rank)  (#{ptr acc_array, shape} p)
+    ps    <- peekArray (fromIntegral ncomp) (#{ptr acc_array, ptr}   p)
+    return (AccArray sh ps)
+  poke p (AccArray sh ps) = do
+    #{poke acc_array, rank}  p (fromIntegral (length sh) :: Int32)
+    #{poke acc_array, ncomp} p (fromIntegral (length ps) :: Int32)
+    pokeArray (#{ptr acc_array, shape} p) sh
+    pokeArray (#{ptr acc_array, ptr}   p) ps
+
+-- | signature of one free array variable of the scalar fragments (Gamma, AST.hs:87-112)
+data EnvSig = EnvSig
+  { envRank  :: Int32
+  , envTypes :: [CString]            -- C type of each component, component 0 first
+  }
+
+instance Storable EnvSig where
+  sizeOf    _ = #{size acc_env_sig}
+  alignment _ = #{alignment acc_env_sig}
+  peek p = do
+    rank  <- #{peek acc_env_sig, rank}  p
+    ncomp <- #{peek acc_env_sig, ncomp} p :: IO Int32
+    ts    <- peekArray (fromIntegral ncomp) (#{ptr acc_env_sig, type} p)
+    return (EnvSig rank ts)
+  poke p (EnvSig rank ts) = do
+    #{poke acc_env_sig, rank}  p rank
+    #{poke acc_env_sig, ncomp} p (fromIntegral (length ts) :: Int32)
+    pokeArray (#{ptr acc_env_sig, type} p) ts
+
+-- | acc_skel_desc is filled field by field into zeroed memory (every field left out is NULL / 0, which the
+-- library reads as "not given"): see `withSkelDesc`
+data SkelDesc
+data SkelInfo
+data DeviceProps
+data CacheStats
+data MemTableStats
+
+-- | What the code generator hands over for one array operation (CodeGen.hs:91-136 builds a CUTranslSkel; this
+-- is the same information as text fragments)
+data Skeleton = Skeleton
+  { skelKind        :: Int32                 -- ACC_SKEL_*
+  , skelFlags       :: Word32
+  , skelEnv         :: [(Int32, [String])]   -- per free array: rank, component types
+  , skelEltType     :: String
+  , skelOutRank     :: Int32
+  , skelPreamble    :: Maybe String
+  , skelGet         :: Maybe String
+  , skelCombine     :: Maybe String
+  , skelSeed        :: Maybe String
+  , skelPermutation :: Maybe String
+  , skelCombineHint :: Int32
+  , skelSegType     :: Maybe String
+  }
+
+withMaybeCString :: Maybe String -> (CString -> IO a) -> IO a
+withMaybeCString Nothing  k = k nullPtr
+withMaybeCString (Just s) k = withCString s k
+
+withCStrings :: [String] -> ([CString] -> IO a) -> IO a
+withCStrings []     k = k []
+withCStrings (s:ss) k = withCString s $ \c -> withCStrings ss (k . (c:))
+
+-- | marshal a `Skeleton` (map family, folds, scans, permute; a stencil additionally pokes its taps, boundary and
+-- `stencil_fn` the same way) for acc_skel_create / acc_skel_preview
+withSkelDesc :: Skeleton -> (Ptr SkelDesc -> IO a) -> IO a
+withSkelDesc sk k =
+  allocaBytes #{size acc_skel_desc} $ \p ->
+  withEnv (skelEnv sk) $ \envs ->
+  withArrayLen envs $ \n penv ->
+  withCString (skelEltType sk) $ \elt ->
+  withMaybeCString (skelPreamble sk) $ \pre ->
+  withMaybeCString (skelGet sk) $ \get ->
+  withMaybeCString (skelCombine sk) $ \comb ->
+  withMaybeCString (skelSeed sk) $ \seed ->
+  withMaybeCString (skelPermutation sk) $ \perm ->
+  withMaybeCString (skelSegType sk) $ \seg -> do
+    _ <- fillBytes p 0 #{size acc_skel_desc}
+    #{poke acc_skel_desc, kind}         p (skelKind sk)
+    #{poke acc_skel_desc, flags}        p (skelFlags sk)
+    #{poke acc_skel_desc, n_env}        p (fromIntegral n :: Int32)
+    #{poke acc_skel_desc, env}          p penv
+    #{poke acc_skel_desc, elt_type}     p elt
+    #{poke acc_skel_desc, out_rank}     p (skelOutRank sk)
+    #{poke acc_skel_desc, preamble}     p pre
+    #{poke acc_skel_desc, get}          p get
+    #{poke acc_skel_desc, combine}      p comb
+    #{poke acc_skel_desc, seed}         p seed
+    #{poke acc_skel_desc, permutation}  p perm
+    #{poke acc_skel_desc, combine_hint} p (skelCombineHint sk)
+    #{poke acc_skel_desc, seg_type}     p seg
+    k p
+  where
+    withEnv []            kk = kk []
+    withEnv ((r, ts):es)  kk = withCStrings ts $ \cs -> withEnv es (kk . (EnvSig r cs :))
+
+-- | build (or fetch from the kernel cache) the kernels of one array operation: the role of build1 / compile /
+-- link (Compile.hs:444-566).  The handle replaces the AccKernel record (AST.hs:51-59).
+createSkeleton :: Context -> Skeleton -> IO Skel
+createSkeleton ctx sk =
+  withSkelDesc sk $ \pdesc ->
+  alloca $ \pout -> do
+    check (c_skelCreate ctx pdesc pout)
+    peek pout
+
+-- | device memory, or Nothing when the device is full (Array/Remote.hs:63-67 `mallocRemote`)
+mallocDevice :: Context -> Int -> IO (Maybe DevPtr)
+mallocDevice ctx bytes =
+  alloca $ \pout -> do
+    ok <- checkAlloc (c_malloc ctx (fromIntegral bytes) pout)
+    if ok then Just `fmap` peek pout else return Nothing
+
+-- | out[i] = f (in[i]) and the other members of the map family (Execute.hs:264-268 `executeOp`)
+execMap :: Skel -> [AccArray] -> AccArray -> Stream -> IO ()
+execMap sk env out stream =
+  withArray env $ \penv ->
+  with out $ \pout ->
+    check (c_execMap sk penv pout stream)
+
+-- | the six scans (Execute.hs:328-392): `total` is Nothing except for scanl' / scanr'
+execScan :: Skel -> [AccArray] -> Int64 -> AccArray -> Maybe AccArray -> Stream -> IO ()
+execScan sk env n out total stream =
+  withArray env $ \penv ->
+  with out $ \pout ->
+  maybe ($ nullPtr) with total $ \ptot ->
+    check (c_execScan sk penv n pout ptot stream)
+
+-- ---------------------------------------------------------------------------------------------------------
+-- the entry points, in the header's order
+
+-- errors and version
+foreign import ccall unsafe "acc_last_error" c_lastError :: IO CString
+foreign import ccall unsafe "acc_version"    c_version   :: IO CString
+
+-- State.hs:127-132, Analysis/Device.hs:31-41: initialise, count, props
+foreign import ccall safe   "acc_init"             c_init           :: IO Status
+foreign import ccall safe   "acc_device_count"     c_deviceCount    :: Ptr CInt -> IO Status
+foreign import ccall safe   "acc_device_get_props" c_deviceGetProps :: CInt -> Ptr DeviceProps -> IO Status
+
+-- Context.hs:55-111: create / destroy; CUDA.sync
+foreign import ccall safe   "acc_context_create"  c_contextCreate  :: CInt -> Ptr Context -> IO Status
+foreign import ccall safe   "acc_context_destroy" c_contextDestroy :: Context -> IO Status
+foreign import ccall safe   "acc_context_device"  c_contextDevice  :: Context -> Ptr CInt -> IO Status
+foreign import ccall safe   "acc_context_sync"    c_contextSync    :: Context -> IO Status
+
+-- Array/Remote.hs:63-79,191: mallocArray / free / getMemInfo.  ACC_ERR_OOM is the recoverable status
+foreign import ccall safe   "acc_malloc"     c_malloc    :: Context -> CSize -> Ptr DevPtr -> IO Status
+foreign import ccall safe   "acc_free"       c_free      :: Context -> DevPtr -> IO Status
+foreign import ccall safe   "acc_mem_info"   c_memInfo   :: Context -> Ptr CSize -> Ptr CSize -> IO Status
+foreign import ccall safe   "acc_host_alloc" c_hostAlloc :: Context -> CSize -> Ptr (Ptr ()) -> IO Status
+foreign import ccall safe   "acc_host_free"  c_hostFree  :: Context -> Ptr () -> IO Status
+
+-- Array/Prim.hs:189-391, Execute.hs:405: poke / peek / copy [Async], memsetAsync
+foreign import ccall safe   "acc_memcpy_h2d"       c_memcpyH2d      :: Context -> DevPtr -> Ptr () -> CSize -> IO Status
+foreign import ccall safe   "acc_memcpy_d2h"       c_memcpyD2h      :: Context -> Ptr () -> DevPtr -> CSize -> IO Status
+foreign import ccall safe   "acc_memcpy_d2d"       c_memcpyD2d      :: Context -> DevPtr -> DevPtr -> CSize -> IO Status
+foreign import ccall safe   "acc_memcpy_h2d_async" c_memcpyH2dAsync :: Context -> DevPtr -> Ptr () -> CSize -> Stream -> IO Status
+foreign import ccall safe   "acc_memcpy_d2h_async" c_memcpyD2hAsync :: Context -> Ptr () -> DevPtr -> CSize -> Stream -> IO Status
+foreign import ccall safe   "acc_memcpy_d2d_async" c_memcpyD2dAsync :: Context -> DevPtr -> DevPtr -> CSize -> Stream -> IO Status
+foreign import ccall safe   "acc_memset32_async"   c_memset32Async  :: Context -> DevPtr -> Word32 -> CSize -> Stream -> IO Status
+
+-- Execute/Stream.hs:102,134; Execute/Event.hs:70-127; Debug.hs:48-67
+foreign import ccall safe   "acc_stream_create"     c_streamCreate    :: Context -> Ptr Stream -> IO Status
+foreign import ccall safe   "acc_stream_destroy"    c_streamDestroy   :: Context -> Stream -> IO Status
+foreign import ccall safe   "acc_stream_sync"       c_streamSync      :: Context -> Stream -> IO Status
+foreign import ccall safe   "acc_stream_wait_event" c_streamWaitEvent :: Context -> Stream -> Event -> IO Status
+foreign import ccall safe   "acc_event_create"      c_eventCreate     :: Context -> CInt -> Ptr Event -> IO Status
+foreign import ccall safe   "acc_event_destroy"     c_eventDestroy    :: Context -> Event -> IO Status
+foreign import ccall safe   "acc_event_record"      c_eventRecord     :: Context -> Event -> Stream -> IO Status
+foreign import ccall safe   "acc_event_sync"        c_eventSync       :: Context -> Event -> IO Status
+foreign import ccall safe   "acc_event_query"       c_eventQuery      :: Context -> Event -> Ptr CInt -> IO Status
+foreign import ccall safe   "acc_event_elapsed_ms"  c_eventElapsedMs  :: Context -> Event -> Event -> Ptr CFloat -> IO Status
+
+-- Compile.hs:543-594, Persistent.hs: run-time compilation through the kernel cache (blocks while the compiler runs)
+foreign import ccall safe   "acc_compile"         c_compile       :: Context -> CString -> CString -> Ptr CString -> CInt -> Ptr (Ptr ()) -> Ptr CSize -> IO Status
+foreign import ccall unsafe "acc_compile_log"     c_compileLog    :: IO CString
+foreign import ccall safe   "acc_cache_set_dir"   c_cacheSetDir   :: CString -> IO Status
+foreign import ccall unsafe "acc_cache_dir"       c_cacheDir      :: IO CString
+foreign import ccall safe   "acc_cache_get_stats" c_cacheGetStats :: Ptr CacheStats -> IO Status
+foreign import ccall safe   "acc_cache_clear"     c_cacheClear    :: CInt -> IO Status
+
+-- Compile.hs:453-465,505,534; Analysis/Launch.hs:42-102; Execute.hs:975-978: raw modules, occupancy, launch
+foreign import ccall safe   "acc_module_load"         c_moduleLoad        :: Context -> Ptr () -> CSize -> Ptr Module -> IO Status
+foreign import ccall safe   "acc_module_unload"       c_moduleUnload      :: Context -> Module -> IO Status
+foreign import ccall safe   "acc_module_get_function" c_moduleGetFunction :: Context -> Module -> CString -> Ptr Function -> IO Status
+foreign import ccall safe   "acc_function_attr"       c_functionAttr      :: Context -> Function -> CInt -> Ptr CInt -> IO Status
+foreign import ccall safe   "acc_occupancy"           c_occupancy         :: Context -> Function -> CInt -> CSize -> Ptr CInt -> IO Status
+foreign import ccall safe   "acc_launch"              c_launch            :: Context -> Function -> Word32 -> Word32 -> Word32 -> Stream -> Ptr (Ptr ()) -> IO Status
+foreign import ccall unsafe "acc_launch_grid"         c_launchGrid        :: Int64 -> Int64 -> Int64 -> Int64 -> Int64
+
+-- Compile.hs:444-566 + CodeGen/*: one skeleton instance per array operation
+foreign import ccall safe   "acc_skel_create"       c_skelCreate      :: Context -> Ptr SkelDesc -> Ptr Skel -> IO Status
+foreign import ccall safe   "acc_skel_destroy"      c_skelDestroy     :: Skel -> IO Status
+foreign import ccall safe   "acc_skel_source"       c_skelSource      :: Skel -> CInt -> Ptr CString -> IO Status
+foreign import ccall safe   "acc_skel_preview"      c_skelPreview     :: Ptr SkelDesc -> CInt -> Ptr CString -> Ptr CString -> IO Status
+foreign import ccall safe   "acc_skel_compile_only" c_skelCompileOnly :: CString -> Ptr SkelDesc -> Ptr CSize -> IO Status
+foreign import ccall safe   "acc_skel_get_info"     c_skelGetInfo     :: Skel -> Ptr SkelInfo -> IO Status
+
+-- Execute.hs:264-450: the skeleton drivers; everything is enqueued on the stream
+foreign import ccall safe   "acc_exec_map"             c_execMap            :: Skel -> Ptr AccArray -> Ptr AccArray -> Stream -> IO Status
+foreign import ccall safe   "acc_exec_fold"            c_execFold           :: Skel -> Ptr AccArray -> Int32 -> Ptr Int64 -> Ptr AccArray -> Stream -> IO Status
+foreign import ccall safe   "acc_exec_foldseg"         c_execFoldseg        :: Skel -> Ptr AccArray -> Int64 -> Ptr AccArray -> Ptr AccArray -> Stream -> IO Status
+foreign import ccall safe   "acc_exec_scan"            c_execScan           :: Skel -> Ptr AccArray -> Int64 -> Ptr AccArray -> Ptr AccArray -> Stream -> IO Status
+foreign import ccall safe   "acc_exec_permute"         c_execPermute        :: Skel -> Ptr AccArray -> Int64 -> Ptr AccArray -> Ptr AccArray -> Stream -> IO Status
+foreign import ccall safe   "acc_exec_stencil"         c_execStencil        :: Skel -> Ptr AccArray -> Ptr AccArray -> Ptr AccArray -> Stream -> IO Status
+foreign import ccall safe   "acc_exec_stencil2"        c_execStencil2       :: Skel -> Ptr AccArray -> Ptr AccArray -> Ptr AccArray -> Ptr AccArray -> Stream -> IO Status
+foreign import ccall safe   "acc_exec_stencil_iterate" c_execStencilIterate :: Skel -> Ptr AccArray -> Ptr AccArray -> Ptr AccArray -> Int32 -> Stream -> Ptr Int32 -> IO Status
+
+-- Array/Remote.hs, Array/Table.hs, Array/Prim.hs:177-192: the memory table
+foreign import ccall safe   "acc_memtable_create"           c_memtableCreate          :: Context -> Word64 -> Ptr MemTable -> IO Status
+foreign import ccall safe   "acc_memtable_destroy"          c_memtableDestroy         :: MemTable -> IO Status
+foreign import ccall safe   "acc_memtable_malloc"           c_memtableMalloc          :: MemTable -> Word64 -> Ptr () -> Word64 -> CInt -> Ptr CInt -> IO Status
+foreign import ccall safe   "acc_memtable_acquire"          c_memtableAcquire         :: MemTable -> Word64 -> Stream -> Ptr DevPtr -> IO Status
+foreign import ccall safe   "acc_memtable_release"          c_memtableRelease         :: MemTable -> Word64 -> Stream -> IO Status
+foreign import ccall safe   "acc_memtable_free"             c_memtableFree            :: MemTable -> Word64 -> IO Status
+foreign import ccall safe   "acc_memtable_insert_unmanaged" c_memtableInsertUnmanaged :: MemTable -> Word64 -> DevPtr -> Word64 -> IO Status
+foreign import ccall safe   "acc_memtable_reclaim"          c_memtableReclaim         :: MemTable -> IO Status
+foreign import ccall safe   "acc_memtable_get_stats"        c_memtableGetStats        :: MemTable -> Ptr MemTableStats -> IO Status

@@ -320,3 +320,28 @@ def test_c_client_builds_as_c99_and_runs_its_deviceless_part():
     subprocess.check_call(["make", "-C", here], stdout=subprocess.DEVNULL)
     out = subprocess.run([os.path.join(here, "client"), "--no-gpu"], capture_output=True, text=True, timeout=300)
     assert out.returncode == 0 and "all checks passed" in out.stdout, out.stdout + out.stderr
+
+
+def test_haskell_bindings_cover_the_header():
+    """the (uncompiled) Haskell FFI module imports every entry point the header declares, once, with as many
+    arguments as the C declaration has; its structure accesses name fields the header has"""
+    header = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "acc_hip.h")).read(), flags=re.S)
+    hsc = open(os.path.join(ROOT, "accelerate-cuda_amd", "haskell", "Data", "Array", "Accelerate", "HIP", "FFI.hsc")).read()
+    declared = {}
+    for name, params in re.findall(r"^(?:const char \*|int64_t |int )\s*(acc_[a-z0-9_]+)\(([^;]*?)\);", header, flags=re.M | re.S):
+        params = " ".join(params.split())
+        declared[name] = 0 if params == "void" else params.count(",") + 1
+    imported = {}
+    for name, sig in re.findall(r'^foreign import ccall \w+\s+"(acc_\w+)"\s+\w+\s+::\s+(.*)$', hsc, flags=re.M):
+        assert name not in imported, name
+        depth, arrows = 0, 0
+        for k, ch in enumerate(sig):                      # arrows outside parentheses separate the arguments
+            depth += (ch == "(") - (ch == ")")
+            arrows += depth == 0 and sig[k:k + 2] == "->"
+        imported[name] = arrows
+    assert imported == declared
+    for struct, field in re.findall(r"#\{(?:peek|poke|ptr) (\w+), (\w+)\}", hsc):
+        body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (struct, struct), header, flags=re.S).group(1)
+        assert re.search(r"\b%s\b" % field, body), (struct, field)
+    for const in re.findall(r"#\{const (\w+)\}", hsc):
+        assert re.search(r"#define %s\b" % const, header), const
