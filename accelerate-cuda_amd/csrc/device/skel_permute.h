@@ -280,6 +280,30 @@ ACC_DEV int acc_xcd_id() { return (int)(__builtin_amdgcn_s_getreg(20 | (0 << 6) 
  * the elements that belong to it; every workgroup dumps its table (row blockIdx.x of `dump`).  As many passes
  * over the source as windows -- 2^26 uniform keys into 2^18 targets: 8 passes, 0.25 ms, against 2.1 ms of
  * device-scope atomics -- and no worse for skewed keys than for uniform ones.                             */
+/* ACC_PERMUTE_NARROW (integer addition): twice to four times the targets in one LDS table, for counting.  A
+ * target's count is kept in 16 bits, two targets to a word, and grows by additions of at most ACC_NARROW_MAX
+ * (larger addends -- rare in a histogram, where they are all 1 -- go to the result directly).  The lane whose
+ * addition takes a count from below 0x8000 to 0x8000 or above takes 0x8000 out again and adds it to the result;
+ * so a count of 0x8000 or more always has such a correction on its way.  That the count cannot reach 0x10000
+ * (and spill into its neighbour) before the correction lands is not left to timing: a lane that finds a count at
+ * ACC_NARROW_STOP or above waits until it has dropped below that, and since a lane has at most ACC_VEC additions in flight
+ * before it looks, the count ends below ACC_NARROW_STOP + ACC_NARROW_MAX * (1 + ACC_BLOCK * ACC_VEC) < 0x10000.
+ * A wave applies the corrections of a batch before any of its lanes waits, so a lane never waits for its own wave.
+ * What is left in the table at the end leaves as a row of words of `dump`.                                      */
+#ifndef ACC_PERMUTE_NARROW
+#define ACC_PERMUTE_NARROW 0
+#endif
+#if ACC_PERMUTE_NARROW
+#define ACC_NARROW_MAX  3u
+#define ACC_NARROW_HALF 0x8000u
+#ifndef ACC_NARROW_STOP
+#define ACC_NARROW_STOP 0xA000u
+#endif
+static_assert(ACC_NARROW_STOP > ACC_NARROW_HALF, "a lane would wait for a correction nobody owes");
+static_assert(ACC_NARROW_STOP + ACC_NARROW_MAX * (1u + ACC_BLOCK * ACC_VEC) < 0x10000u, "a 16-bit count could spill into its neighbour");
+static_assert(ACC_COMBINE_HINT == ACC_HINT_ADD && ACC_ELT_IS_INTEGER && !ACC_PERMUTE_WINDOWS, "narrow counts are for integer addition");
+#endif
+
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, const int lds_copies,
         ACC_ELT *__restrict__ dump, ACC_ELT *__restrict__ far
@@ -321,14 +345,57 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
   T *far_row = far ? far + (Int64)acc_xcd_id() * ntarget : (T *)0;
   (void)far_row;
 
+#if ACC_PERMUTE_NARROW
+  unsigned *words = (unsigned *)acc_lds_raw;
+  const int nwords = (lds_bins + 1) / 2;
+  for (int i = threadIdx.x; i < nwords; i += ACC_BLOCK) words[i] = 0u;
+  __syncthreads();
+  typedef typename acc_bits<sizeof(T)>::type UT;
+  /* the addition itself: what the count was before it, or ACC_NARROW_HALF (which asks for neither a correction
+   * nor a wait) where no count was touched */
+  /* (Without a branch, so that the additions of a batch are issued one behind the other and waited for together:
+   * a lane with nothing to add adds 0 to a word of its own.) */
+  auto narrow_add = [&](const U t, const T &x) -> unsigned {
+    const UT ux = (UT)x;
+    const bool in = t < u_bins, small = ux <= (UT)ACC_NARROW_MAX;
+    if (in && !small) acc_hint_apply<ACC_SCOPE_DEVICE>(arrOut_0 + t, x, f);
+    const bool take = in && small;
+    const unsigned sh = ((unsigned)t & 1u) * 16u;
+    const unsigned old = __hip_atomic_fetch_add(words + (take ? (unsigned)(t >> 1) : (threadIdx.x & 63u)),
+                                                take ? (unsigned)ux << sh : 0u, __ATOMIC_RELAXED, ACC_SCOPE_BLOCK);
+    return take ? (old >> sh) & 0xFFFFu : ACC_NARROW_HALF;
+  };
+  /* the lane that took the count over the half-way mark moves that half into the result */
+  auto narrow_carry = [&](const U t, const T &x, const unsigned before) {
+    if (before < ACC_NARROW_HALF && before + (unsigned)(UT)x >= ACC_NARROW_HALF) {
+      (void)__hip_atomic_fetch_sub(words + (t >> 1), ACC_NARROW_HALF << (((unsigned)t & 1u) * 16u), __ATOMIC_RELAXED, ACC_SCOPE_BLOCK);
+      acc_hint_apply<ACC_SCOPE_DEVICE>(arrOut_0 + t, (T)ACC_NARROW_HALF, f);
+    }
+  };
+  auto narrow_wait = [&](const U t, const unsigned before) {
+    if (before >= ACC_NARROW_STOP) {
+      const unsigned sh = ((unsigned)t & 1u) * 16u;
+      /* (the correction is a few instructions away in another wave; the bound only makes sure that every wave ends) */
+      for (int polls = 0; polls < (1 << 20) &&
+           ((__hip_atomic_load(words + (t >> 1), __ATOMIC_RELAXED, ACC_SCOPE_BLOCK) >> sh) & 0xFFFFu) >= ACC_NARROW_STOP; ++polls)
+        __builtin_amdgcn_s_sleep(1);
+    }
+  };
+  (void)ident; (void)bins;
+#else
   for (int i = threadIdx.x; i < lds_bins * lds_copies; i += ACC_BLOCK) bins[i] = ident;
   __syncthreads();
   T *mine = bins + ((threadIdx.x >> 6) % lds_copies) * lds_bins;
+#endif
 
   /* two independent tests rather than a chain: each becomes a predicated
    * instruction, not a branch */
   auto update = [&](const U t, const T &x) {
-#if ACC_PERMUTE_WINDOWS
+#if ACC_PERMUTE_NARROW
+    const unsigned before = narrow_add(t, x);
+    narrow_carry(t, x, before);
+    narrow_wait(t, before);
+#elif ACC_PERMUTE_WINDOWS
     if (t < u_reach && (t & u_mask) == u_window) acc_hint_apply<ACC_SCOPE_BLOCK>(mine + (t >> win_log), x, f);
 #else
     if (t < u_bins) acc_hint_apply<ACC_SCOPE_BLOCK>(mine + t, x, f);
@@ -366,10 +433,23 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
   while (tile < full_tiles) {
     const Int64 next = tile + walkers;
     if (next < full_tiles) load(next, jn, xn);
+#if ACC_PERMUTE_NARROW
+#pragma unroll
+    for (int u = 0; u < ACC_UNROLL; ++u) {           /* ACC_VEC additions, then their corrections, then the waits */
+      unsigned before[ACC_VEC];
+#pragma unroll
+      for (int k = 0; k < ACC_VEC; ++k) before[k] = narrow_add(j[u][k], x[u][k]);
+#pragma unroll
+      for (int k = 0; k < ACC_VEC; ++k) narrow_carry(j[u][k], x[u][k], before[k]);
+#pragma unroll
+      for (int k = 0; k < ACC_VEC; ++k) narrow_wait(j[u][k], before[k]);
+    }
+#else
 #pragma unroll
     for (int u = 0; u < ACC_UNROLL; ++u)
 #pragma unroll
       for (int k = 0; k < ACC_VEC; ++k) update(j[u][k], x[u][k]);
+#endif
 #pragma unroll
     for (int u = 0; u < ACC_UNROLL; ++u)
 #pragma unroll
@@ -390,6 +470,14 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
   }
 
   /* the privatised part leaves the block */
+#if ACC_PERMUTE_NARROW
+  __syncthreads();
+  {
+    unsigned *wrow = (unsigned *)dump + (Int64)blockIdx.x * nwords;
+    for (int i = threadIdx.x; i < nwords; i += ACC_BLOCK) wrow[i] = words[i];
+  }
+  (void)row;
+#else
   if (lds_bins > 0) {
     __syncthreads();
     for (int i = threadIdx.x; i < lds_bins; i += ACC_BLOCK) {
@@ -405,6 +493,7 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
       }
     }
   }
+#endif
 }
 
 /* fills p[0 .. count) with the combine's identity and copies copy_count
@@ -433,6 +522,38 @@ struct acc_merge_job {
                              t mod 2^window_log at column t >> window_log; -1: one table, target t at column t */
 };
 
+#if ACC_PERMUTE_NARROW
+/* the rows of packed 16-bit counts, `nwords` words a row, added into the result: a thread per word (two targets),
+ * the rows shared between `slices` workgroups (then each adds its share atomically) */
+extern "C" __global__ void __launch_bounds__(256)
+permute_merge(ACC_ENV_PARAMS ACC_OUT_PARAMS, const unsigned *__restrict__ dump, const Int64 nwords, const int nrows,
+              const int slices, const Int64 ntarget)
+{
+  typedef ACC_ELT T;
+  ACC_ENV_ASSUME
+  auto f = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
+  const Int64 column = (Int64)(blockIdx.x / slices) * 256 + threadIdx.x;
+  const int slice = blockIdx.x % slices;
+  if (column >= nwords) return;
+  const int per = (nrows + slices - 1) / slices;
+  const int r0 = slice * per, r1 = acc_min(nrows, r0 + per);
+  unsigned lo = 0u, hi = 0u;                     /* at most 65536 rows of counts below 0x8000 each */
+#pragma unroll 8
+  for (int r = r0; r < r1; ++r) {
+    const unsigned w = dump[(Int64)r * nwords + column];
+    lo += w & 0xFFFFu;
+    hi += w >> 16;
+  }
+  const Int64 t = 2 * column;
+  if (slices == 1) {
+    arrOut_0[t] = f((T)lo, arrOut_0[t]);
+    if (t + 1 < ntarget) arrOut_0[t + 1] = f((T)hi, arrOut_0[t + 1]);
+  } else {
+    if (lo) acc_hint_apply<ACC_SCOPE_DEVICE>(arrOut_0 + t, (T)lo, f);
+    if (hi && t + 1 < ntarget) acc_hint_apply<ACC_SCOPE_DEVICE>(arrOut_0 + t + 1, (T)hi, f);
+  }
+}
+#else
 /* folds up to two tables in one launch: workgroups [0, blocks_a) take job a,
  * the rest job b */
 extern "C" __global__ void __launch_bounds__(256)
@@ -469,4 +590,5 @@ permute_merge(ACC_ENV_PARAMS ACC_OUT_PARAMS, const acc_merge_job a, const int bl
     if (x != y) acc_hint_apply<ACC_SCOPE_DEVICE>(dst, acc, f);
   }
 }
+#endif /* ACC_PERMUTE_NARROW */
 #endif /* ACC_PERMUTE_LOCKED */

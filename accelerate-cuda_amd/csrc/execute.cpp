@@ -568,6 +568,55 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
   push_out(*out, &args, &aligned);
   args.i64(n_src);
 
+  // Integer addition on more targets than one LDS table of whole elements holds, but no more than one of 16-bit
+  // counts does (65536 Int32 or Int64 targets in 128 KB): one pass over the source instead of one per window.
+  const bool int_add = s->spec.combine_hint == ACC_COMBINE_ADD &&
+                       (s->spec.elt_type == "Int32" || s->spec.elt_type == "Word32" || s->spec.elt_type == "Int64" || s->spec.elt_type == "Word64");
+  // Only where the source is spelt as a small constant -- the counting idiom, `permute (+) zeros bin ones` -- since any
+  // other addend would go to the result one device-scope atomic at a time (`permute.narrow=2` takes every source).
+  const int narrow = acc::tune("permute.narrow", 1);
+  if (int_add && ntarget * (int64_t)esz > lds_all && ((ntarget + 1) / 2) * 4 <= lds_all && n_src >= 4 * ntarget &&
+      (narrow == 2 || (narrow == 1 && s->spec.get_small_constant))) {
+    const int nv = (aligned ? 0 : 1) + 6;
+    ACC_TRY(s->ensure_variant(nv));
+    ACC_TRY(plain_copy());
+    const int64_t nwords = (ntarget + 1) / 2;
+    const size_t nlds = (size_t)nwords * 4;
+    int bpc = 0;
+    hipError_t oe = hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&bpc, s->variants[nv].fn, s->spec.block, nlds);
+    if (oe != hipSuccess || bpc < 1) { (void)hipGetLastError(); bpc = 1; }
+    const int64_t cus_n = s->ctx->props.multiProcessorCount;
+    const int64_t ngrid = acc_launch_grid(n_src, s->elements_per_block(), cus_n, bpc);
+    int nblk = -1;
+    ACC_TRY(s->ctx->scratch_acquire((size_t)(ngrid * nwords) * 4, st, acc::SCRATCH_FOLD, &nblk));
+    const uint64_t ndump = reinterpret_cast<uint64_t>(s->ctx->scratch[nblk].ptr);
+    args.i32(static_cast<int32_t>(ntarget));
+    args.i32(1);
+    args.ptr(ndump);
+    args.ptr(0);
+    int nrc = launch(s, nv, ngrid, nlds, st, &args);
+    if (nrc == ACC_OK) {
+      const int64_t columns = (nwords + 255) / 256;
+      const int64_t slices = std::max<int64_t>(1, std::min<int64_t>(ngrid, (2 * cus_n + columns - 1) / columns));
+      Args m;
+      bool mal = true;
+      nrc = push_env(s, env, &m, &mal);
+      push_out(*out, &m, &mal);
+      m.ptr(ndump);
+      m.i64(nwords);
+      m.i32(static_cast<int32_t>(ngrid));
+      m.i32(static_cast<int32_t>(slices));
+      m.i64(ntarget);
+      if (nrc == ACC_OK) {
+        hipError_t me = hipModuleLaunchKernel(s->variants[nv].fn_finish, static_cast<unsigned>(columns * slices), 1, 1, 256, 1, 1, 0, st,
+                                              m.data(), nullptr);
+        if (me != hipSuccess) nrc = acc::fail_hip(me, "hipModuleLaunchKernel(permute_merge, narrow counts)");
+      }
+    }
+    s->ctx->scratch_release(nblk, st);
+    return nrc;
+  }
+
   // A hinted combination on more targets than two LDS tables hold: windows of targets, each with its share of the
   // workgroups, which walk the whole source (skel_permute.h).  Up to `permute.max_windows` passes are cheaper than
   // a device-scope atomic per element (27 G/s for the whole device).

@@ -6,6 +6,7 @@
 // and CUDA/Compile.hs:444-459,484-566 (build1 / compile / link) do in the
 // reference.  The templates themselves live in device/*.h.
 #include <algorithm>
+#include <cctype>
 #include <cstdlib>
 #include <cstring>
 #include <sstream>
@@ -250,6 +251,8 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "#define ACC_COMBINE_HINT " << sp.combine_hint << "\n";
       o << "#define ACC_PERMUTE_LOCKED " << (sp.permute_locked ? 1 : 0) << "\n";
       o << "#define ACC_PERMUTE_WINDOWS " << (sp.permute_windows ? 1 : 0) << "\n";
+      o << "#define ACC_PERMUTE_NARROW " << (sp.permute_narrow ? 1 : 0) << "\n";
+      if (sp.permute_narrow) o << "#define ACC_NARROW_STOP " << tune("permute.narrow_stop", 0xA000) << "u\n";
       o << "#define ACC_ELT_IS_INTEGER " << (is_integer_type(sp.elt_type) ? 1 : 0) << "\n";
       o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_UNROLL " << sp.unroll << "\n";
       tmpl = "skel_permute.h";
@@ -320,6 +323,31 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
 
 // ---- description -> spec ---------------------------------------------------------
 
+// `text` is an integer literal 0..3, possibly parenthesised and cast: "1", "((Int32)(1))", "(Int64)1u"
+static bool small_literal(std::string t)
+{
+  t.erase(std::remove_if(t.begin(), t.end(), [](unsigned char c) { return std::isspace(c); }), t.end());
+  for (bool again = true; again && !t.empty();) {
+    again = false;
+    if (t.front() == '(' && t.back() == ')') {         // one pair around everything?
+      int depth = 0;
+      size_t k = 0;
+      for (; k < t.size(); ++k) {
+        depth += (t[k] == '(') - (t[k] == ')');
+        if (depth == 0) break;
+      }
+      if (k == t.size() - 1) { t = t.substr(1, t.size() - 2); again = true; continue; }
+    }
+    if (t.front() == '(') {                            // a cast: "(Name)" followed by the rest
+      size_t k = 1;
+      while (k < t.size() && (std::isalnum((unsigned char)t[k]) || t[k] == '_')) ++k;
+      if (k > 1 && k < t.size() - 1 && t[k] == ')') { t = t.substr(k + 1); again = true; }
+    }
+  }
+  while (!t.empty() && (t.back() == 'u' || t.back() == 'U' || t.back() == 'l' || t.back() == 'L')) t.pop_back();
+  return t.size() == 1 && t[0] >= '0' && t[0] <= '3';
+}
+
 int make_spec(const acc_skel_desc *d, SkelSpec *sp)
 {
   if (!d) return fail(ACC_ERR_INVALID, "NULL skeleton description");
@@ -377,6 +405,7 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
   }
   sp->preamble = d->preamble ? d->preamble : "";
   sp->get = flat(d->get);
+  sp->get_small_constant = small_literal(sp->get);
   sp->combine = flat(d->combine);
   sp->has_seed = d->seed && *d->seed;
   sp->seed = flat(d->seed);
@@ -518,6 +547,18 @@ using acc::fail;
 
 // ---- acc_skel_s ----------------------------------------------------------------
 
+namespace acc {
+// what variant v of an instance is generated from (variants beyond 1 exist for permute only)
+SkelSpec spec_of_variant(const SkelSpec &base, int v)
+{
+  SkelSpec spec = base;
+  if (v >= 2 && v < 4) spec.permute_locked = true;
+  if (v >= 4 && v < 6) spec.permute_windows = true;
+  if (v >= 6) spec.permute_narrow = true;
+  return spec;
+}
+}  // namespace acc
+
 int acc_skel_s::ensure_variant(int v)
 {
   // two threads may meet here on the first launch that needs the unaligned variant
@@ -525,9 +566,7 @@ int acc_skel_s::ensure_variant(int v)
   acc::Variant &var = variants[v];
   if (var.ready) return ACC_OK;
   // variants 2 and 3 of a permute: the locked template for an element the atomic template also covers
-  acc::SkelSpec spec = this->spec;
-  if (v >= 2 && v < 4) spec.permute_locked = true;
-  if (v >= 4) spec.permute_windows = true;
+  acc::SkelSpec spec = acc::spec_of_variant(this->spec, v);
   std::string entry_name;
   ACC_TRY(acc::generate_source(spec, (v & 1) == 0, &entry_name, &var.source));
   entry = entry_name;
@@ -618,10 +657,11 @@ int acc_skel_source(acc_skel s, int variant, const char **source)
 int acc_skel_preview(const acc_skel_desc *desc, int variant, const char **source, const char **entry)
 {
   static thread_local std::string text, name;
-  if (!source || variant < 0 || variant > 1) return fail(ACC_ERR_INVALID, "acc_skel_preview: bad argument");
+  if (!source || variant < 0 || variant > 7) return fail(ACC_ERR_INVALID, "acc_skel_preview: bad argument");
   acc::SkelSpec sp;
   ACC_TRY(acc::make_spec(desc, &sp));
-  ACC_TRY(acc::generate_source(sp, variant == 0, &name, &text));
+  if (variant > 1 && sp.kind != ACC_SKEL_PERMUTE) return fail(ACC_ERR_INVALID, "acc_skel_preview: only a permute has variants beyond 1");
+  ACC_TRY(acc::generate_source(acc::spec_of_variant(sp, variant), (variant & 1) == 0, &name, &text));
   *source = text.c_str();
   if (entry) *entry = name.c_str();
   return ACC_OK;

@@ -24,6 +24,8 @@ struct SkelSpec {
   bool has_seed = false;
   int combine_hint = 0;
   bool permute_windows = false;         // hinted permute over several LDS windows of targets (variants 4 and 5)
+  bool get_small_constant = false;      // `get` is a literal 0..3 (under casts and parentheses): a permute that counts
+  bool permute_narrow = false;          // integer addition with 16-bit counts in LDS (variants 6 and 7)
   bool permute_locked = false;          // permute of an element no atomic covers (tuples, 1/2/16-byte types): per-target locks
   std::string seg_type;
   // stencil
@@ -57,6 +59,7 @@ int type_size(const std::string &t);
 int tune(const char *name, int dflt);
 int make_spec(const acc_skel_desc *d, SkelSpec *sp);
 int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::string *source);
+SkelSpec spec_of_variant(const SkelSpec &base, int variant);
 std::vector<std::string> compile_options(const SkelSpec &sp);
 
 }  // namespace acc
@@ -65,9 +68,10 @@ struct acc_skel_s {
   acc_context ctx = nullptr;
   acc::SkelSpec spec;
   std::string entry;
-  acc::Variant variants[6];   // [0] pointers 16-byte aligned, [1] no assumption; [2], [3]: the same for the
+  acc::Variant variants[8];   // [0] pointers 16-byte aligned, [1] no assumption; [2], [3]: the same for the
                               // table-in-LDS form of a permute whose combination has no atomic instruction;
-                              // [4], [5]: for a hinted permute over several LDS windows of targets
+                              // [4], [5]: for a hinted permute over several LDS windows of targets;
+                              // [6], [7]: for integer addition on a table of 16-bit counts in LDS
   std::mutex mu;
 
   int ensure_variant(int v);

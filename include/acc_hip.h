@@ -306,7 +306,10 @@ int acc_skel_destroy(acc_skel s);
  * variant 0 = aligned (128-bit accesses assumed legal), 1 = unaligned.      */
 int acc_skel_source(acc_skel s, int variant, const char **source);
 /* the same text straight from a description, without a context or a GPU; the
- * string stays valid until the calling thread's next call of this function  */
+ * string stays valid until the calling thread's next call of this function.
+ * A permute has further forms the driver chooses between by the number of
+ * targets, at variant + 2 (tables under locks in LDS), + 4 (several LDS
+ * windows of targets), + 6 (16-bit counts in LDS, integer addition)          */
 int acc_skel_preview(const acc_skel_desc *desc, int variant, const char **source, const char **entry);
 /* compile only (no GPU needed): used by the build check */
 int acc_skel_compile_only(const char *target, const acc_skel_desc *desc, size_t *code_size);

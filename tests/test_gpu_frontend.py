@@ -80,6 +80,13 @@ def test_histogram_via_permute_reads_keys_inside_the_permutation(acc):
     # nothing lands anywhere
     h = acc.run(acc.permute(add, acc.use(np.arange(bins, dtype=np.int32)), lambda i: acc.ignore, acc.use(w)))
     assert np.array_equal(h, np.arange(bins, dtype=np.int32))
+    # counting into 65536 targets: the constant source is what lets the driver keep 16-bit counts in LDS
+    keys = np.minimum(rng.zipf(1.3, 1 << 20) - 1, 65535).astype(np.int32)
+    ks = acc.use(keys)
+    h = acc.run(acc.permute(add, acc.fill((65536,), 0, "Int32"), lambda i: (ks[i],), acc.fill((keys.size,), 1, "Int32")))
+    assert np.array_equal(h, np.bincount(keys, minlength=65536).astype(np.int32))
+    h = acc.run(acc.permute(add, acc.fill((65536,), 5, "Int64"), lambda i: (ks[i],), acc.fill((keys.size,), 2, "Int64")))
+    assert np.array_equal(h, 5 + 2 * np.bincount(keys, minlength=65536).astype(np.int64))
 
 
 def test_permute_with_a_generic_combination(acc):

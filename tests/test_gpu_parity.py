@@ -370,6 +370,68 @@ def test_permute_hinted_combines_over_windows_of_targets(A, ctx):
         assert np.array_equal(out.get(), ref)
 
 
+def test_counting_into_a_table_of_16_bit_counts(A, ctx):
+    """a permute that counts (integer `+` over a source spelt as a small constant) into more targets than one LDS
+    table of whole elements holds, but few enough for 16-bit counts: hot targets whose count passes 0x8000 in every
+    workgroup many times over, odd numbers of targets, ignored and stray indices, defaults, Int64 and Word32 results,
+    keys that are not 16-byte aligned"""
+    import workloads as wl
+    n = 1 << 24
+    cases = [("zipf", wl.zipf_i32(7, n, 65536), 65536), ("uniform", wl.uniform_i32(8, n, 65535), 65535),
+             ("one hot target", np.full(n, 4242, np.int32), 50001),
+             ("four hot targets in two words", (rng.integers(0, 4, n) + 70000).astype(np.int32), 81919)]
+    strays = rng.integers(-5, 65536 + 5, 1 << 22).astype(np.int32)
+    strays[::7] = -1
+    cases.append(("strays and ignore", strays, 65536))
+    for ctype, dt, lit in (("Int32", np.int32, "1"), ("Int64", np.int64, "((Int64)(1))"), ("Word32", np.uint32, "3u")):
+        sk = ctx.skeleton(A.SKEL_PERMUTE, ctype, env=[I32], out_rank=1, get=lit, combine="x + y",
+                          permutation="arrIn0_0[ix]", combine_hint=A.COMBINE_ADD)
+        w = 3 if lit == "3u" else 1
+        for name, keys, bins in cases:
+            say("counting", ctype, name, "into", bins)
+            dfl = rng.integers(0, 1000, bins).astype(dt)
+            out = ctx.empty(bins, dt)
+            dk = ctx.array(np.concatenate([np.zeros(1, np.int32), keys]))
+            for view in (dk.desc(shape=(keys.size,), offset_elems=1), ctx.array(keys)):   # 4 bytes off a 16-byte boundary, then on one
+                sk.permute([view], keys.size, ctx.array(dfl), out)
+                ok = (keys >= 0) & (keys < bins)
+                ref = dfl + (np.bincount(keys[ok], minlength=bins) * w).astype(dt)
+                assert np.array_equal(out.get(), ref)
+
+
+def test_16_bit_counts_with_large_addends_and_with_lanes_made_to_wait(A, ctx):
+    """the same table taken for a source that is not a constant (`permute.narrow=2`): addends above 3 and negative
+    ones go to the result directly, the others through the counts; and with the mark at which a lane waits for a
+    pending correction set as low as it goes, so that lanes do wait, on hot targets"""
+    import os
+    n, bins = 1 << 23, 60001
+    dst = rng.integers(0, 40, n).astype(np.int32) * 1500           # 40 hot targets
+    dst[::9] = rng.integers(-2, bins + 2, dst[::9].size)
+    src = rng.integers(-2, 8, n).astype(np.int32)
+    ok = (dst >= 0) & (dst < bins)
+    os.environ["ACC_HIP_TUNE"] = "permute.narrow=2,permute.narrow_stop=32769"
+    try:
+        say("weighted sums through 16-bit counts, waits forced")
+        sk = ctx.skeleton(A.SKEL_PERMUTE, "Int32", env=[I32, I32], out_rank=1, get="arrIn1_0[ix] ", combine="x + y",
+                          permutation="arrIn0_0[ix]", combine_hint=A.COMBINE_ADD)
+        dfl = rng.integers(-100, 100, bins, dtype=np.int32)
+        out = ctx.empty(bins, np.int32)
+        sk.permute([ctx.array(dst), ctx.array(src)], n, ctx.array(dfl), out)
+        ref = dfl.copy()
+        np.add.at(ref, dst[ok], src[ok])
+        assert np.array_equal(out.get(), ref)
+        say("counting with waits forced, one hot target")
+        sk = ctx.skeleton(A.SKEL_PERMUTE, "Int32", env=[I32], out_rank=1, get="(1)", combine="x + y",
+                          permutation="arrIn0_0[ix]", combine_hint=A.COMBINE_ADD)
+        keys = np.full(1 << 24, 31, np.int32)
+        keys[::3] = 30
+        out = ctx.empty(bins, np.int32)
+        sk.permute([ctx.array(keys)], keys.size, ctx.array(dfl), out)
+        assert np.array_equal(out.get(), dfl + np.bincount(keys, minlength=bins).astype(np.int32))
+    finally:
+        del os.environ["ACC_HIP_TUNE"]
+
+
 # --------------------------------------------------------------------------- stencil
 
 GAUSS_TAPS = [(dy, dx) for dy in (-1, 0, 1) for dx in (-1, 0, 1)]
