@@ -281,7 +281,8 @@ ACC_DEV int acc_xcd_id() { return (int)(__builtin_amdgcn_s_getreg(20 | (0 << 6) 
  * over the source as windows -- 2^26 uniform keys into 2^18 targets: 8 passes, 0.25 ms, against 2.1 ms of
  * device-scope atomics -- and no worse for skewed keys than for uniform ones.                             */
 /* ACC_PERMUTE_NARROW (integer addition): twice to four times the targets in one LDS table, for counting.  A
- * target's count is kept in 16 bits, two targets to a word, and grows by additions of at most ACC_NARROW_MAX
+ * target's count is kept in 16 bits, two targets to a word (t and t + half the targets, so that neighbouring hot
+ * targets do not meet on one word), and grows by additions of at most ACC_NARROW_MAX
  * (larger addends -- rare in a histogram, where they are all 1 -- go to the result directly).  The lane whose
  * addition takes a count from below 0x8000 to 0x8000 or above takes 0x8000 out again and adds it to the result;
  * so a count of 0x8000 or more always has such a correction on its way.  That the count cannot reach 0x10000
@@ -351,6 +352,9 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
   for (int i = threadIdx.x; i < nwords; i += ACC_BLOCK) words[i] = 0u;
   __syncthreads();
   typedef typename acc_bits<sizeof(T)>::type UT;
+  const U u_half = (U)nwords;
+  auto narrow_shift = [&](const U t) -> unsigned { return t < u_half ? 0u : 16u; };
+  auto narrow_word  = [&](const U t) -> unsigned { return (unsigned)(t < u_half ? t : t - u_half); };
   /* the addition itself: what the count was before it, or ACC_NARROW_HALF (which asks for neither a correction
    * nor a wait) where no count was touched */
   /* (Without a branch, so that the additions of a batch are issued one behind the other and waited for together:
@@ -360,24 +364,24 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
     const bool in = t < u_bins, small = ux <= (UT)ACC_NARROW_MAX;
     if (in && !small) acc_hint_apply<ACC_SCOPE_DEVICE>(arrOut_0 + t, x, f);
     const bool take = in && small;
-    const unsigned sh = ((unsigned)t & 1u) * 16u;
-    const unsigned old = __hip_atomic_fetch_add(words + (take ? (unsigned)(t >> 1) : (threadIdx.x & 63u)),
+    const unsigned sh = narrow_shift(t);
+    const unsigned old = __hip_atomic_fetch_add(words + (take ? narrow_word(t) : (threadIdx.x & 63u)),
                                                 take ? (unsigned)ux << sh : 0u, __ATOMIC_RELAXED, ACC_SCOPE_BLOCK);
     return take ? (old >> sh) & 0xFFFFu : ACC_NARROW_HALF;
   };
   /* the lane that took the count over the half-way mark moves that half into the result */
   auto narrow_carry = [&](const U t, const T &x, const unsigned before) {
     if (before < ACC_NARROW_HALF && before + (unsigned)(UT)x >= ACC_NARROW_HALF) {
-      (void)__hip_atomic_fetch_sub(words + (t >> 1), ACC_NARROW_HALF << (((unsigned)t & 1u) * 16u), __ATOMIC_RELAXED, ACC_SCOPE_BLOCK);
+      (void)__hip_atomic_fetch_sub(words + narrow_word(t), ACC_NARROW_HALF << narrow_shift(t), __ATOMIC_RELAXED, ACC_SCOPE_BLOCK);
       acc_hint_apply<ACC_SCOPE_DEVICE>(arrOut_0 + t, (T)ACC_NARROW_HALF, f);
     }
   };
   auto narrow_wait = [&](const U t, const unsigned before) {
     if (before >= ACC_NARROW_STOP) {
-      const unsigned sh = ((unsigned)t & 1u) * 16u;
+      const unsigned sh = narrow_shift(t);
       /* (the correction is a few instructions away in another wave; the bound only makes sure that every wave ends) */
       for (int polls = 0; polls < (1 << 20) &&
-           ((__hip_atomic_load(words + (t >> 1), __ATOMIC_RELAXED, ACC_SCOPE_BLOCK) >> sh) & 0xFFFFu) >= ACC_NARROW_STOP; ++polls)
+           ((__hip_atomic_load(words + narrow_word(t), __ATOMIC_RELAXED, ACC_SCOPE_BLOCK) >> sh) & 0xFFFFu) >= ACC_NARROW_STOP; ++polls)
         __builtin_amdgcn_s_sleep(1);
     }
   };
@@ -523,7 +527,8 @@ struct acc_merge_job {
 };
 
 #if ACC_PERMUTE_NARROW
-/* the rows of packed 16-bit counts, `nwords` words a row, added into the result: a thread per word (two targets),
+/* the rows of packed 16-bit counts, `nwords` words a row, added into the result: a thread per word (targets
+ * `column` and `column + nwords`),
  * the rows shared between `slices` workgroups (then each adds its share atomically) */
 extern "C" __global__ void __launch_bounds__(256)
 permute_merge(ACC_ENV_PARAMS ACC_OUT_PARAMS, const unsigned *__restrict__ dump, const Int64 nwords, const int nrows,
@@ -544,13 +549,13 @@ permute_merge(ACC_ENV_PARAMS ACC_OUT_PARAMS, const unsigned *__restrict__ dump, 
     lo += w & 0xFFFFu;
     hi += w >> 16;
   }
-  const Int64 t = 2 * column;
+  const Int64 t = column, t_hi = column + nwords;
   if (slices == 1) {
     arrOut_0[t] = f((T)lo, arrOut_0[t]);
-    if (t + 1 < ntarget) arrOut_0[t + 1] = f((T)hi, arrOut_0[t + 1]);
+    if (t_hi < ntarget) arrOut_0[t_hi] = f((T)hi, arrOut_0[t_hi]);
   } else {
     if (lo) acc_hint_apply<ACC_SCOPE_DEVICE>(arrOut_0 + t, (T)lo, f);
-    if (hi && t + 1 < ntarget) acc_hint_apply<ACC_SCOPE_DEVICE>(arrOut_0 + t + 1, (T)hi, f);
+    if (hi && t_hi < ntarget) acc_hint_apply<ACC_SCOPE_DEVICE>(arrOut_0 + t_hi, (T)hi, f);
   }
 }
 #else

@@ -579,7 +579,17 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
       (narrow == 2 || (narrow == 1 && s->spec.get_small_constant))) {
     const int nv = (aligned ? 0 : 1) + 6;
     ACC_TRY(s->ensure_variant(nv));
-    ACC_TRY(plain_copy());
+    if (copy_defaults) {                 // by a kernel of the instance's own: a third of the time a runtime copy of 256 KB takes
+      Args f;
+      f.ptr(0);
+      f.i64(0);
+      f.ptr(out->ptr[0]);
+      f.ptr(defaults->ptr[0]);
+      f.i64(ntarget);
+      const int64_t fill_grid = std::min<int64_t>((ntarget + 255) / 256, 8 * (int64_t)s->ctx->props.multiProcessorCount);
+      hipError_t fe = hipModuleLaunchKernel(s->variants[nv].fn_fill, static_cast<unsigned>(fill_grid), 1, 1, 256, 1, 1, 0, st, f.data(), nullptr);
+      if (fe != hipSuccess) return acc::fail_hip(fe, "hipModuleLaunchKernel(permute_fill, narrow counts)");
+    }
     const int64_t nwords = (ntarget + 1) / 2;
     const size_t nlds = (size_t)nwords * 4;
     int bpc = 0;
