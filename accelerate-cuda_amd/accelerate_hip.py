@@ -42,7 +42,8 @@ __all__ = ["Exp", "constant", "cond", "use", "unit", "map", "zipWith", "generate
            "ceiling", "idiv", "mod", "quot", "rem", "min_", "max_", "sqrt", "exp", "log", "sin", "cos", "tan", "abs_",
            "signum", "Context", "the", "runWith", "run1With", "runN", "stream", "streamWith", "Async", "wait", "poll",
            "cancel", "Cancelled", "runAsync", "run1Async", "runAsyncWith", "run1AsyncWith", "create", "destroy",
-           "unsafeFree", "unsafeFreeWith", "performGC", "performGCWith"]
+           "unsafeFree", "unsafeFreeWith", "performGC", "performGCWith", "acond", "reshape", "flatten", "replicate", "slice_", "All",
+           "imap", "zipWith3", "iterate"]
 
 CTYPE = dict(A.CTYPE_OF)
 NPTYPE = {v: k for k, v in CTYPE.items()}
@@ -905,6 +906,79 @@ def run1(f, context=None):
     def go(*hosts):
         return run(f(*[use(h, cx) for h in hosts]), cx)
     return go
+
+
+def acond(p, t, e, context=None):
+    """array-level conditional: the scalar array `p` is read back and one of the two computations is returned
+    (Execute.hs:187); `t` and `e` may be Acc values or functions of no argument, so that only the branch taken
+    is built"""
+    taken = t if the(p, context) else e
+    return taken() if callable(taken) else taken
+
+
+def reshape(shape, a):
+    """the same elements in row-major order under another shape of the same size (Execute.hs:198: no kernel, a
+    manifest array keeps its storage; a delayed one is re-indexed)"""
+    shape = (shape,) if isinstance(shape, numbers.Integral) else tuple(int(x) for x in shape)
+    n = 1
+    for x in shape:
+        n *= x
+    if n != a.size:
+        raise ValueError("reshape: %r has %d elements, the array %d" % (shape, n, a.size))
+    if a.manifest is not None:
+        return Acc(shape, a.ctype, manifest=a.manifest)          # device arrays are addressed linearly
+    return Acc(shape, a.ctype, at=a.at)
+
+
+def flatten(a):
+    return reshape((a.size,), a)
+
+
+All = slice(None)
+
+
+def replicate(spec, a):
+    """`replicate (Z :. 3 :. All) xs`: spec has `All` where a dimension of `a` goes and a number where a new
+    dimension of that extent is inserted (fused into the consumer, Execute.hs:216)"""
+    spec = tuple(spec)
+    if sum(1 for x in spec if x is All or x == All) != len(a.shape):
+        raise TypeError("replicate: as many All as the array has dimensions")
+    dims = iter(a.shape)
+    shape = tuple(next(dims) if (x is All or x == All) else int(x) for x in spec)
+    keep = [k for k, x in enumerate(spec) if x is All or x == All]
+    return backpermute(shape, lambda *ix: tuple(ix[k] for k in keep), a)
+
+
+def slice_(a, spec):
+    """`slice arr (Z :. 2 :. All)`: spec has `All` for a dimension that stays and an index (a number or an Exp)
+    for one that is fixed (Execute.hs:217)"""
+    spec = tuple(spec)
+    if len(spec) != len(a.shape):
+        raise TypeError("slice: one entry per dimension of the array")
+    keep = [k for k, x in enumerate(spec) if x is All or (isinstance(x, slice) and x == All)]
+    shape = tuple(a.shape[k] for k in keep)
+
+    def at(*ix):
+        it = iter(ix)
+        return tuple(next(it) if k in keep else spec[k] for k in range(len(spec)))
+    return backpermute(shape, at, a)
+
+
+def imap(f, a):
+    """map with the element's multi-index: f(index tuple, value)"""
+    t = _probe(lambda v: f(tuple(constant(0, "Int64") for _ in a.shape), v), a.ctype)
+    return Acc(a.shape, t, at=lambda ix: Exp.of(f(_unlinear(ix, a.shape), a.index(ix))))
+
+
+def zipWith3(f, a, b, c):
+    return zipWith(lambda xy, z: f(fst(xy), snd(xy), z), zip_(a, b), c)
+
+
+def iterate(n, f, a):
+    """f applied n times (n a host integer)"""
+    for _ in range(int(n)):
+        a = f(a)
+    return a
 
 
 def runN(f, context=None):

@@ -479,3 +479,44 @@ def test_contexts_streams_of_inputs_and_asynchronous_runs(acc):
     finally:
         acc.destroy(cx)
     assert cx.ctx.handle is None
+
+
+def test_reshape_replicate_slice_and_array_level_conditional(acc):
+    rng = np.random.default_rng(41)
+    m = rng.integers(-50, 50, (37, 53)).astype(np.int32)
+    v = rng.integers(-50, 50, 53).astype(np.int32)
+    ms, vs = acc.use(m), acc.use(v)
+    # matrix-vector product the Accelerate way: replicate the vector over the rows, multiply, fold the rows
+    mv = acc.fold(add, 0, acc.zipWith(lambda a, b: a * b, ms, acc.replicate((37, acc.All), vs)))
+    assert np.array_equal(acc.run(mv), m @ v)
+    # a new innermost dimension
+    r = acc.run(acc.replicate((acc.All, 4), vs))
+    assert r.shape == (53, 4) and np.array_equal(r, np.repeat(v[:, None], 4, axis=1))
+    # slices: a row, a column
+    assert np.array_equal(acc.run(acc.map(lambda x: x + 1, acc.slice_(ms, (5, acc.All)))), m[5] + 1)
+    assert np.array_equal(acc.run(acc.map(lambda x: x + 1, acc.slice_(ms, (acc.All, 7)))), m[:, 7] + 1)
+    # reshape of a manifest array (no kernel) and of a delayed one
+    cx = acc.Context.default()
+    n = len(cx.skeletons)
+    flat = acc.flatten(ms)
+    assert flat.manifest is ms.manifest and len(cx.skeletons) == n
+    assert np.array_equal(acc.run(acc.scanl1(add, flat)), np.cumsum(m.reshape(-1), dtype=np.int32))
+    d = acc.reshape((53, 37), acc.map(lambda x: x * 2, ms))
+    assert np.array_equal(acc.run(acc.fold(add, 0, d)), (m * 2).reshape(53, 37).sum(axis=1, dtype=np.int32))
+    with pytest.raises(ValueError):
+        acc.reshape((10, 10), ms)
+    # imap, zipWith3, iterate
+    assert np.array_equal(acc.run(acc.imap(lambda ix, x: x + acc.fromIntegral(ix[0] * 100 + ix[1], "Int32"), ms)),
+                          m + (np.arange(37)[:, None] * 100 + np.arange(53)[None, :]).astype(np.int32))
+    assert np.array_equal(acc.run(acc.zipWith3(lambda a, b, c: a * b + c, vs, vs, vs)), v * v + v)
+    assert np.array_equal(acc.run(acc.iterate(3, lambda a: acc.map(lambda x: x * 2 + 1, a), vs)), ((v * 2 + 1) * 2 + 1) * 2 + 1)
+    # acond: only the branch taken is built
+    built = []
+
+    def branch(tag, k):
+        def go():
+            built.append(tag)
+            return acc.map(lambda x: x + k, vs)
+        return go
+    big = acc.map(lambda s: s > 10 ** 6, acc.fold(add, 0, vs))
+    assert np.array_equal(acc.run(acc.acond(big, branch("then", 1), branch("else", 2))), v + 2) and built == ["else"]
