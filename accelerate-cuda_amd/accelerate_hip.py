@@ -43,7 +43,8 @@ __all__ = ["Exp", "constant", "cond", "use", "unit", "map", "zipWith", "generate
            "signum", "Context", "the", "runWith", "run1With", "runN", "stream", "streamWith", "Async", "wait", "poll",
            "cancel", "Cancelled", "runAsync", "run1Async", "runAsyncWith", "run1AsyncWith", "create", "destroy",
            "unsafeFree", "unsafeFreeWith", "performGC", "performGCWith", "acond", "reshape", "flatten", "replicate", "slice_", "All",
-           "imap", "zipWith3", "iterate"]
+           "imap", "zipWith3", "iterate", "asin", "acos", "atan", "sinh", "cosh", "tanh", "asinh", "acosh", "atanh", "atan2",
+           "pow_", "logBase", "recip", "isNaN", "rotateL", "rotateR", "boolToInt", "ord_", "chr_", "quotRem", "divMod"]
 
 CTYPE = dict(A.CTYPE_OF)
 NPTYPE = {v: k for k, v in CTYPE.items()}
@@ -267,6 +268,35 @@ def log(a): return a._call("acc_log")
 def sin(a): return a._call("acc_sin")
 def cos(a): return a._call("acc_cos")
 def tan(a): return a._call("acc_tan")
+def asin(a): return a._call("acc_asin")
+def acos(a): return a._call("acc_acos")
+def atan(a): return a._call("acc_atan")
+def sinh(a): return a._call("acc_sinh")
+def cosh(a): return a._call("acc_cosh")
+def tanh(a): return a._call("acc_tanh")
+def asinh(a): return a._call("acc_asinh")
+def acosh(a): return a._call("acc_acosh")
+def atanh(a): return a._call("acc_atanh")
+def atan2(y, x): return Exp.of(y)._call("acc_atan2", x)
+def pow_(a, b): return Exp.of(a)._call("acc_pow", b)
+def logBase(base, y): return Exp.of(base)._call("acc_log_base", y)
+def recip(a): return a._call("acc_recip")
+def isNaN(a): return Exp.mk("Word8", "acc_is_nan(%s)", a)
+def rotateL(a, i): return Exp.mk(a.ctype, "acc_rotate_l(%s, (Int64)%s)", a, Exp.of(i, "Int64"))
+def rotateR(a, i): return Exp.mk(a.ctype, "acc_rotate_r(%s, (Int64)%s)", a, Exp.of(i, "Int64"))
+def boolToInt(b): return Exp.mk("Int64", "acc_bool_to_int(%s)", b)
+def ord_(c): return Exp.mk("Int64", "acc_ord(%s)", c)
+def chr_(i): return Exp.mk("Word32", "acc_chr(%s)", i)
+
+
+def quotRem(a, b):
+    """(quotient, remainder) truncated towards zero, as a pair (Arithmetic.hs:90-104)"""
+    return lift(quot(a, b), rem(a, b))
+
+
+def divMod(a, b):
+    """(quotient, remainder) rounded towards minus infinity, as a pair (Arithmetic.hs:106-158)"""
+    return lift(idiv(a, b), mod(a, b))
 
 
 ignore = "ignore"        # the target index that drops an element (IndexSpace.hs:150-151)

@@ -520,3 +520,40 @@ def test_reshape_replicate_slice_and_array_level_conditional(acc):
         return go
     big = acc.map(lambda s: s > 10 ** 6, acc.fold(add, 0, vs))
     assert np.array_equal(acc.run(acc.acond(big, branch("then", 1), branch("else", 2))), v + 2) and built == ["else"]
+
+
+def test_the_rest_of_the_scalar_primitives(acc):
+    """every PrimFun the reference's code generator knows (CodeGen.hs) is reachable from the language: the ones the
+    other tests do not use, against numpy.  Transcendental results within 4 ulp of numpy's Float32 (the device's
+    math library is not bit-identical to the host's); everything else exact."""
+    rng = np.random.default_rng(42)
+    x = (rng.random(5003) * 1.8 - 0.9).astype(np.float32)
+    xs = acc.use(x)
+
+    def close(got, ref, ulps=4):
+        ref = ref.astype(np.float32)
+        return np.all(np.abs(got - ref) <= ulps * np.spacing(np.abs(ref)) + 1e-37)
+    for fn, ref in ((acc.asin, np.arcsin), (acc.acos, np.arccos), (acc.atan, np.arctan), (acc.sinh, np.sinh),
+                    (acc.cosh, np.cosh), (acc.tanh, np.tanh), (acc.asinh, np.arcsinh), (acc.atanh, np.arctanh)):
+        assert close(acc.run(acc.map(fn, xs)), ref(x)), fn.__name__
+    assert close(acc.run(acc.map(lambda v: acc.acosh(v + 2.0), xs)), np.arccosh(x + np.float32(2)))
+    assert close(acc.run(acc.map(lambda v: acc.atan2(v, v * v - 0.5), xs)), np.arctan2(x, x * x - np.float32(0.5)))
+    assert close(acc.run(acc.map(lambda v: acc.pow_(v + 2.0, v), xs)), np.power(x + np.float32(2), x))
+    assert close(acc.run(acc.map(lambda v: acc.logBase(acc.constant(3.0, "float"), v + 2.0), xs)),
+                 np.log(x + np.float32(2)) / np.log(np.float32(3)), ulps=8)
+    assert np.array_equal(acc.run(acc.map(acc.recip, xs)), np.float32(1) / x)
+    nan = x.copy()
+    nan[::7] = np.nan
+    assert np.array_equal(acc.run(acc.map(acc.isNaN, acc.use(nan))), np.isnan(nan).astype(np.uint8))
+    w = rng.integers(0, 2 ** 32, 4001, dtype=np.uint32)
+    ws = acc.use(w)
+    assert np.array_equal(acc.run(acc.map(lambda v: acc.rotateL(v, 7), ws)), (w << np.uint32(7)) | (w >> np.uint32(25)))
+    assert np.array_equal(acc.run(acc.map(lambda v: acc.rotateR(v, 7), ws)), (w >> np.uint32(7)) | (w << np.uint32(25)))
+    assert np.array_equal(acc.run(acc.map(lambda v: acc.boolToInt(v > 2 ** 31), ws)), (w > 2 ** 31).astype(np.int64))
+    assert np.array_equal(acc.run(acc.map(lambda v: acc.ord_(acc.chr_(v)), ws)), w.astype(np.int64))
+    a = rng.integers(-1000, 1000, 4001).astype(np.int32)
+    b = rng.integers(1, 50, 4001).astype(np.int32) * rng.choice([-1, 1], 4001).astype(np.int32)
+    q, r = acc.run(acc.unzip(acc.zipWith(acc.quotRem, acc.use(a), acc.use(b))))
+    assert np.array_equal(q, np.trunc(a / b).astype(np.int32)) and np.array_equal(r, a - b * np.trunc(a / b).astype(np.int32))
+    d, m = acc.run(acc.unzip(acc.zipWith(acc.divMod, acc.use(a), acc.use(b))))
+    assert np.array_equal(d, a // b) and np.array_equal(m, a % b)
