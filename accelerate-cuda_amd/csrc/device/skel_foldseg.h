@@ -168,6 +168,106 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
   }
 }
 
+#if ACC_SEG_UNIFORM
+/* ---- short rows: a lane per row, straight from memory ----------------------
+ * Rows of up to ACC_ROWS_MAX elements (a fold over colour channels, small vectors, 4 x 4 blocks): a lane reads its
+ * row with as few, as wide loads as the row length allows -- the lanes of a wave read one contiguous stretch
+ * between them -- and folds it in index order, in the association of the entry above.  Nothing is staged: the
+ * chunks of the entry above hold whole blocks of segments, which for rows this short leaves most of a chunk unused. */
+#define ACC_ROWS_MAX 16
+template <int W, typename T, typename F>
+ACC_DEV T acc_fold_row(const T (&x)[W], F f, const T &seed)
+{
+  (void)seed;
+#if ACC_FOLD_RIGHT
+  /* x0 (+) (x1 (+) (... (x_last (+) z))) */
+#if ACC_HAS_SEED
+  T acc = f(x[W - 1], seed);
+#else
+  T acc = x[W - 1];
+#endif
+#pragma unroll
+  for (int k = W - 2; k >= 0; --k) acc = f(x[k], acc);
+#else
+  /* ((x0 (+) x1) (+) ... x_last) (+) z */
+  T acc = x[0];
+#pragma unroll
+  for (int k = 1; k < W; ++k) acc = f(acc, x[k]);
+#if ACC_HAS_SEED
+  acc = f(acc, seed);
+#endif
+#endif
+  return acc;
+}
+
+/* A lane takes R consecutive rows -- 4 rows of 1, 2 rows of 2, so that its load is one 128-bit vector and the lanes'
+ * vectors lie side by side; longer rows one at a time, lane after lane -- and U such groups a workgroup-width
+ * apart, so that about 64 bytes per lane are requested before the first is used.  The host computes the same R
+ * and U for the grid.                                                                                            */
+template <int W, typename T, typename G, typename F, typename P>
+ACC_DEV void acc_fold_rows(const Int64 nseg, G get, F f, const T &seed, P put)
+{
+  constexpr int R = W == 1 ? 4 : (W == 2 ? 2 : 1);
+  constexpr int U = (R * W >= 16) ? 1 : 16 / (R * W);
+  const Int64 per_block = (Int64)ACC_BLOCK * R * U;
+  for (Int64 b0 = (Int64)blockIdx.x * per_block; b0 < nseg; b0 += (Int64)gridDim.x * per_block) {
+    if (b0 + per_block <= nseg) {
+      T x[U][R][W];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+          for (int k = 0; k < W; ++k) x[u][r][k] = get((b0 + ((Int64)u * ACC_BLOCK + threadIdx.x) * R + r) * W + k);
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int r = 0; r < R; ++r) put(b0 + ((Int64)u * ACC_BLOCK + threadIdx.x) * R + r, acc_fold_row<W, T>(x[u][r], f, seed));
+    } else {
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const Int64 seg = b0 + ((Int64)u * ACC_BLOCK + threadIdx.x) * R + r;
+          if (seg < nseg) {
+            T x[W];
+#pragma unroll
+            for (int k = 0; k < W; ++k) x[k] = get(seg * W + k);
+            put(seg, acc_fold_row<W, T>(x, f, seed));
+          }
+        }
+    }
+  }
+}
+
+#define ACC_FS_CAT2_(a, b) a##b
+#define ACC_FS_CAT_(a, b) ACC_FS_CAT2_(a, b)
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+ACC_FS_CAT_(ACC_FOLDSEG_ENTRY, _rows)(ACC_ENV_PARAMS
+                                      const Int64 shOut_0, ACC_OUT_ARRAY(arrOut),
+                                      ACC_SEG_PARAMS)
+{
+  typedef ACC_ELT T;
+  ACC_ENV_ASSUME
+  auto get = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
+  auto f   = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
+  auto put = [&](const Int64 seg, const T &v) { ACC_PUT(arrOut, seg, v); };       /* written once, not read again here */
+  (void)shIn_1;
+#if ACC_HAS_SEED
+  const T seed = (ACC_SEED);
+#else
+  const T seed = T();
+#endif
+  switch ((int)shIn_0) {
+#define ACC_ROW_CASE(W) case W: acc_fold_rows<W, T>(shOut_0, get, f, seed, put); break;
+    ACC_ROW_CASE(1) ACC_ROW_CASE(2) ACC_ROW_CASE(3) ACC_ROW_CASE(4) ACC_ROW_CASE(5) ACC_ROW_CASE(6) ACC_ROW_CASE(7) ACC_ROW_CASE(8)
+    ACC_ROW_CASE(9) ACC_ROW_CASE(10) ACC_ROW_CASE(11) ACC_ROW_CASE(12) ACC_ROW_CASE(13) ACC_ROW_CASE(14) ACC_ROW_CASE(15) ACC_ROW_CASE(16)
+#undef ACC_ROW_CASE
+    default: break;                                /* the host does not launch this entry for other lengths */
+  }
+}
+#endif /* ACC_SEG_UNIFORM */
+
 /* ---- long segments: a team of lanes per segment ---------------------------
  * One lane per segment serialises a long segment on that lane, so when the
  * segments are long on average the host launches this entry instead: a whole

@@ -258,6 +258,14 @@ int acc_exec_fold(acc_skel s, const acc_array *env, int32_t in_rank, const int64
       const int64_t grid = acc_launch_grid(rows, s->spec.block, resident(s, v), 1 << 20);
       return launch(s, v, grid, 0, st, &args);
     }
+    if (inner <= std::min(16, acc::tune("fold.rows_max", 7))) {
+      // short rows: a lane reads its row straight from memory (skel_foldseg.h, _rows)
+      const int64_t r = inner == 1 ? 4 : (inner == 2 ? 2 : 1), u = r * inner >= 16 ? 1 : 16 / (r * inner);   // as the kernel's R and U
+      const int64_t grid = acc_launch_grid(rows, s->spec.block * r * u, resident(s, v), acc::tune("foldseg.oversub", 1 << 20));
+      hipError_t e = hipModuleLaunchKernel(s->variants[v].fn_rows, static_cast<unsigned>(grid), 1, 1, static_cast<unsigned>(s->spec.block), 1, 1,
+                                           0, st, args.data(), nullptr);
+      return e == hipSuccess ? ACC_OK : acc::fail_hip(e, "hipModuleLaunchKernel(fold, short rows)");
+    }
     return launch_segmented(s, v, &args, env, out, rows, rows * inner, st);
   }
 

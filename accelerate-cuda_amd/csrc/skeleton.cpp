@@ -606,6 +606,15 @@ int acc_skel_s::ensure_variant(int v)
       return acc::fail_hip(e, ("hipModuleGetFunction(" + third + ")").c_str());
     }
   }
+  if ((spec.kind == ACC_SKEL_FOLD || spec.kind == ACC_SKEL_FOLD1) && spec.out_rank > 0) {
+    const std::string rows = entry + "_rows";
+    e = hipModuleGetFunction(&var.fn_rows, var.module, rows.c_str());
+    if (e != hipSuccess) {
+      (void)hipModuleUnload(var.module);
+      var.module = nullptr;
+      return acc::fail_hip(e, ("hipModuleGetFunction(" + rows + ")").c_str());
+    }
+  }
   (void)hipFuncGetAttribute(&var.num_regs, HIP_FUNC_ATTRIBUTE_NUM_REGS, var.fn);
   (void)hipFuncGetAttribute(&var.static_lds, HIP_FUNC_ATTRIBUTE_SHARED_SIZE_BYTES, var.fn);
   int bpc = 0;

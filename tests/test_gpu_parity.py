@@ -617,6 +617,48 @@ def test_fold_along_the_innermost_dimension_at_every_shape(A, ctx):
     assert np.array_equal(out.get(), np.full(17, 5, np.int32))
 
 
+def test_fold_of_short_rows(A, ctx, orc):
+    """rows of 1 to 16 elements (a lane per row straight from memory up to 7, staged chunks beyond): row counts around
+    the workgroup's share, an operator that is not commutative, Float32 sums bit for bit with the sequential left
+    fold (the association is the same), a fused producer, a source that is not 16-byte aligned"""
+    addf = ctx.skeleton(A.SKEL_FOLD, "float", env=[(2, "float")], out_rank=1, get="arrIn0_0[ix]", combine="x + y", seed="0.5f")
+    sub1 = ctx.skeleton(A.SKEL_FOLD1, "Int32", env=[(2, "Int32")], out_rank=1, get="arrIn0_0[ix]", combine="2 * x - y")
+    prod = ctx.skeleton(A.SKEL_FOLD, "Int64", env=[(2, "Int32"), (2, "Int32")], out_rank=1,
+                        get="(Int64)arrIn0_0[ix] * (Int64)arrIn1_0[ix]", combine="x + y", seed="-3")
+    for inner in range(1, 17):
+        for rows in (1, 255, 4096, 4097, 70001):
+            say("fold of", rows, "rows of", inner)
+            xf = (rng.random((rows, inner)) * 2 - 1).astype(np.float32)
+            out = ctx.empty(rows, np.float32)
+            addf.fold([ctx.array(xf)], (rows, inner), out)
+            ref = xf[:, 0].copy()
+            for k in range(1, inner):
+                ref = ref + xf[:, k]
+            assert np.array_equal(out.get(), ref + np.float32(0.5))               # ((x0 + x1) + ...) + z, as written
+            xi = rng.integers(-9, 10, (rows, inner), dtype=np.int32)
+            outi = ctx.empty(rows, np.int32)
+            sub1.fold([ctx.array(xi)], (rows, inner), outi)
+            ref = xi[:, 0].copy()
+            for k in range(1, inner):
+                ref = 2 * ref - xi[:, k]
+            assert np.array_equal(outi.get(), ref)
+        rows = 30011
+        a, b = rng.integers(-10**4, 10**4, (rows, inner), dtype=np.int32), rng.integers(-10**4, 10**4, (rows, inner), dtype=np.int32)
+        flat = ctx.array(np.concatenate([np.zeros(1, np.int32), a.reshape(-1)]))   # the first source starts 4 bytes off
+        out = ctx.empty(rows, np.int64)
+        prod.fold([flat.desc(shape=(rows, inner), offset_elems=1), ctx.array(b)], (rows, inner), out)
+        assert np.array_equal(out.get(), (a.astype(np.int64) * b).sum(axis=1) - 3)
+    say("rows of pairs")
+    pair = ctx.skeleton(A.SKEL_FOLD, "Int32, float", env=[(2, "Int32"), (2, "float")], out_rank=1,
+                        get="acc_elt{arrIn0_0[ix], arrIn1_0[ix]}", combine="acc_elt{x.a1 + y.a1, acc_max(x.a0, y.a0)}",
+                        seed="acc_elt{0, -1.0e30f}")
+    rows, inner = 50001, 4
+    a, b = rng.integers(-99, 99, (rows, inner), dtype=np.int32), rng.random((rows, inner)).astype(np.float32)
+    out = A.TupleArray([ctx.empty(rows, np.int32), ctx.empty(rows, np.float32)])
+    pair.fold([ctx.array(a), ctx.array(b)], (rows, inner), out)
+    assert np.array_equal(out.comps[0].get(), a.sum(axis=1, dtype=np.int32)) and np.array_equal(out.comps[1].get(), b.max(axis=1))
+
+
 # --------------------------------------------------------------------------- committed fixtures
 
 def test_golden_fixtures_on_gpu(A, ctx):
