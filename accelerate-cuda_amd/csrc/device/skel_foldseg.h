@@ -100,16 +100,16 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
     /* stage a chunk: every load is issued before any result is used.  Elements
      * of the chunk's first and last vector that belong to a neighbouring block
      * are loaded too (they exist) and never read back; only the very end of
-     * the array needs a guard.  A block-wide row of vectors that lies wholly
-     * beyond this block's segments is left out (short segments: 256 of them
-     * fill a fraction of a chunk). */
+     * the array needs a guard.  Vectors that lie wholly beyond this block's
+     * segments are left out: short segments fill a fraction of a chunk, and
+     * behind every element may stand a gather. */
     T v[ACC_LOADS][ACC_VEC];
     auto chunk_start = [&](const Int64 q) -> Int64 { return lo_al + (ACC_FOLD_RIGHT ? (nchunks - 1 - q) : q) * (Int64)ACC_CHUNK; };
     auto stage = [&](const Int64 cs) {
       if (cs + ACC_CHUNK <= n) {
 #pragma unroll
         for (int u = 0; u < ACC_LOADS; ++u)
-          if (u == 0 || cs + (Int64)u * (ACC_BLOCK * ACC_VEC) < hi) {
+          if (cs + (Int64)(u * ACC_BLOCK + tid) * ACC_VEC < hi) {
 #pragma unroll
             for (int k = 0; k < ACC_VEC; ++k) v[u][k] = get(cs + (u * ACC_BLOCK + tid) * ACC_VEC + k);
           }
@@ -131,7 +131,7 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
       __syncthreads();                               /* the previous chunk has been consumed */
 #pragma unroll
       for (int u = 0; u < ACC_LOADS; ++u)
-        if (u == 0 || cs + (Int64)u * (ACC_BLOCK * ACC_VEC) < hi) {
+        if (cs + (Int64)(u * ACC_BLOCK + tid) * ACC_VEC < hi) {
 #pragma unroll
           for (int k = 0; k < ACC_VEC; ++k) s_val[ACC_PAD((u * ACC_BLOCK + tid) * ACC_VEC + k)] = v[u][k];
         }
