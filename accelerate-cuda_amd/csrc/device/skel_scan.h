@@ -208,7 +208,7 @@ ACC_DEV void acc_scan_load(Get get, const Int64 base, const Int64 n, T (&x)[ACC_
     }
   } else {
     /* a tile that reaches outside the array: vectors that lie inside are read as in a full tile (one 128-bit
-     * access), the one across the edge element by element, those outside not at all -- a tile read and written
+     * access), the one across the edge element by element, those outside as one element -- a tile read and written
      * element by element takes three times as long as a full one, and it is the last one to finish */
 #pragma unroll
     for (int r = 0; r < ACC_ROWS; ++r) {
@@ -217,6 +217,12 @@ ACC_DEV void acc_scan_load(Get get, const Int64 base, const Int64 n, T (&x)[ACC_
       if (lo >= 0 && lo + ACC_VEC <= n) {
 #pragma unroll
         for (int k = 0; k < ACC_VEC; ++k) x[r][k] = get(ACC_SCAN_RIGHT ? i0 - k : i0 + k);
+      } else if (lo >= n || lo + ACC_VEC <= 0) {
+        /* a vector wholly outside the array: the array's nearest element in every position (one address for all
+         * of them; the value never reaches a result) */
+        const T edge = get(lo >= n ? n - 1 : (Int64)0);
+#pragma unroll
+        for (int k = 0; k < ACC_VEC; ++k) x[r][k] = edge;
       } else {
 #pragma unroll
         for (int k = 0; k < ACC_VEC; ++k) {
@@ -242,11 +248,16 @@ ACC_DEV void acc_scan_load(Get get, const Int64 base, const Int64 n, T (&x)[ACC_
  * right-handed scan: up to ACC_VEC - 1 positions past the end come FIRST, in
  * the first vector of the first tile, and the lane that holds them starts its
  * own scan at the first element inside (`lead` below).                       */
-template <bool GUARD, typename T, typename Op, typename Prefetch, typename Out>
+/* HOW: 0 the tile lies inside the array, 1 it reaches outside, 2 `outside` says which at run time.  (Two forms
+ * side by side in one kernel cost registers: the compiler moves what they share above the branch between them.
+ * For a right-handed scan of 32 rows that is 275 registers against 184 for the run-time form alone, and 256 is
+ * where a second workgroup stops fitting on the compute unit.  Left-handed scans keep the two compiled forms: 185.) */
+template <int HOW, typename T, typename Op, typename Prefetch, typename Out>
 ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op, const T seed, const Int64 tile, const Int64 base,
                            const Int64 n, const Out &out, const acc_scan_desc<T> &desc,
-                           const unsigned int epoch, void *s_wave_raw, T *s_prefix, Prefetch prefetch)
+                           const unsigned int epoch, void *s_wave_raw, T *s_prefix, Prefetch prefetch, const bool outside)
 {
+  const bool GUARD = HOW == 2 ? outside : (HOW == 1);
   typedef T V;
   struct S {
     static ACC_DEV V some(const T &v) { return v; }
@@ -260,16 +271,26 @@ ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op, const T seed,
 
   /* scan the ACC_VEC items each lane holds per row */
   V s[ACC_ROWS][ACC_VEC];
-  Int64 ix0[ACC_ROWS];
-  int lead[ACC_ROWS];                       /* positions past the end that come first in this lane's vector */
+  /* positions past the end that come first in this lane's vector of row r.  (Neither this nor the row's first index
+   * is kept from here to the stores: a tile of 32 rows would spend 100 registers on them.) */
+  auto lead_of = [&](const Int64 i0) -> int {
+    return (GUARD && ACC_SCAN_RIGHT) ? (int)acc_max<Int64>(0, acc_min<Int64>(i0 - (n - 1), ACC_VEC - 1)) : 0;
+  };
 #pragma unroll
   for (int r = 0; r < ACC_ROWS; ++r) {
-    ix0[r] = acc_scan_ix0(base, wave, lane, r);
-    lead[r] = (GUARD && ACC_SCAN_RIGHT) ? (int)acc_max<Int64>(0, acc_min<Int64>(ix0[r] - (n - 1), ACC_VEC - 1)) : 0;
+    int lead = 0;
+    if (GUARD && ACC_SCAN_RIGHT) {
+      /* worked out when the row's elements have arrived, not before: hoisted above the wait for the loads, the
+       * rows' indices and leads would be alive all at once (the compiler is told that `row_base` depends on the
+       * row's first element) */
+      Int64 row_base = base;
+      asm volatile("" : "+s"(row_base) : "v"(x[r][0]));
+      lead = lead_of(acc_scan_ix0(row_base, wave, lane, r));
+    }
 #pragma unroll
     for (int k = 0; k < ACC_VEC; ++k) {
       const V v = x[r][k];
-      s[r][k] = (k == 0 || (GUARD && ACC_SCAN_RIGHT && k == lead[r])) ? v : op(s[r][k - 1], v);
+      s[r][k] = (k == 0 || (GUARD && ACC_SCAN_RIGHT && k == lead)) ? v : op(s[r][k - 1], v);
     }
   }
 
@@ -321,7 +342,18 @@ ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op, const T seed,
     has_prefix = true;
   }
 
-  /* apply the prefixes and write */
+  /* apply the prefixes and write.  The rows' indices are worked out again from a copy of `base` the compiler cannot
+   * see through: otherwise it keeps the ones of the first loop alive across the whole tile, in the guarded form of
+   * a right-handed scan three registers a row -- and that one tile's form sets the register count of the kernel. */
+  Int64 late_base = base;
+  asm volatile("" : "+s"(late_base));
+  /* where the logically last element of the array sits, if in this tile: offset q in the tile's scan order is
+   * item q % ACC_VEC of lane (q / ACC_VEC) % 64 in row (q / (64 ACC_VEC)) % ACC_ROWS of wave q / (64 ACC_VEC ACC_ROWS) */
+  const Int64 last_q = ACC_SCAN_RIGHT ? base + (ACC_TILE - 1) : (n - 1) - base;
+  const bool holds_last = (ACC_SCAN_MODE == 0 || ACC_SCAN_MODE == 2) && last_q >= 0 && last_q < ACC_TILE;
+  const int last_k = (int)(last_q % ACC_VEC), last_lane = (int)((last_q / ACC_VEC) % ACC_WAVE);
+  const int last_row = (int)((last_q / (ACC_VEC * ACC_WAVE)) % ACC_ROWS), last_wave = (int)(last_q / (ACC_VEC * ACC_WAVE * ACC_ROWS));
+  V whole = V();
 #pragma unroll
   for (int r = 0; r < ACC_ROWS; ++r) {
     V b = S::some(prefix);
@@ -343,37 +375,38 @@ ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op, const T seed,
      * 128-bit accesses; in a tile that reaches outside the array only for the
      * vectors that lie inside it */
     const bool exclusive = (ACC_SCAN_MODE == 0 || ACC_SCAN_MODE == 2);
-    const Int64 lo = ACC_SCAN_RIGHT ? ix0[r] - (ACC_VEC - 1) : ix0[r];
+    const Int64 i0 = acc_scan_ix0(late_base, wave, lane, r);
+    const Int64 lo = ACC_SCAN_RIGHT ? i0 - (ACC_VEC - 1) : i0;
     if (!GUARD || (lo >= 0 && lo + ACC_VEC <= n)) {
 #pragma unroll
       for (int k = 0; k < ACC_VEC; ++k) {
-        const Int64 ix = ACC_SCAN_RIGHT ? ix0[r] - k : ix0[r] + k;
+        const Int64 ix = ACC_SCAN_RIGHT ? i0 - k : i0 + k;
         out.put(ix, exclusive ? S::val(k == 0 ? pre : inc[k - 1]) : S::val(inc[k]));
       }
     } else {
 #pragma unroll
       for (int k = 0; k < ACC_VEC; ++k) {
-        const Int64 ix = ACC_SCAN_RIGHT ? ix0[r] - k : ix0[r] + k;
+        const Int64 ix = ACC_SCAN_RIGHT ? i0 - k : i0 + k;
         if (ix < 0 || ix >= n) continue;
-        const bool first = (k == 0) || (ACC_SCAN_RIGHT && k == lead[r]);
+        const bool first = (k == 0) || (ACC_SCAN_RIGHT && k == lead_of(i0));
         const V before = (k == 0) ? pre : (first ? pre : inc[k - 1]);     /* (k == 0 keeps inc[-1] out of the expression) */
         out.set(ix, exclusive ? S::val(before) : S::val(inc[k]));
       }
     }
 
-    /* the reduction of the whole vector, held by the logically last element: only the tile that holds it
-     * looks for it (32 comparisons per lane are 1.5 % of a tile's time) */
-    const Int64 last = ACC_SCAN_RIGHT ? 0 : n - 1;
-    if ((ACC_SCAN_MODE == 0 || ACC_SCAN_MODE == 2) && last >= base && last < base + ACC_TILE) {
+    /* the reduction of the whole vector is the inclusive value of the logically last element: the row that holds
+     * it keeps the value, and the one lane stores it after the loop (a store per row and position, each under its
+     * own test, made the kernel half as long again, and the exclusive scans 2 % slower than the inclusive ones) */
+    if (holds_last && r == last_row) {
+      V c = inc[0];
 #pragma unroll
-      for (int k = 0; k < ACC_VEC; ++k) {
-        const Int64 ix = ACC_SCAN_RIGHT ? ix0[r] - k : ix0[r] + k;
-        if (ix == last) {
-          if (ACC_SCAN_MODE == 0) out.set(n, S::val(inc[k]));
-          else                    out.total(S::val(inc[k]));
-        }
-      }
+      for (int k = 1; k < ACC_VEC; ++k) c = (k == last_k) ? inc[k] : c;
+      whole = c;
     }
+  }
+  if (holds_last && wave == last_wave && lane == last_lane) {
+    if (ACC_SCAN_MODE == 0) out.set(n, S::val(whole));
+    else                    out.total(S::val(whole));
   }
 }
 
@@ -490,10 +523,8 @@ ACC_ENTRY(ACC_ENV_PARAMS
 #endif
 
     const Int64 base = tile_base(tile);
-    if (base >= 0 && base + ACC_TILE <= n)
-      acc_scan_tile<false, T>(cur, op, seed, tile, base, n, out, desc, epoch, (void *)s_wave, &s_prefix, prefetch);
-    else
-      acc_scan_tile<true, T>(cur, op, seed, tile, base, n, out, desc, epoch, (void *)s_wave, &s_prefix, prefetch);
+    const bool inside = base >= 0 && base + ACC_TILE <= n;
+    acc_scan_tile<2, T>(cur, op, seed, tile, base, n, out, desc, epoch, (void *)s_wave, &s_prefix, prefetch, !inside);
 
 #if ACC_SCAN_PERSISTENT
 #pragma unroll

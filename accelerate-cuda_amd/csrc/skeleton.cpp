@@ -48,6 +48,12 @@ static std::string flat(const char *s)
 // ACC_HIP_TUNE="scan.block=512,scan.rows=2,fold.unroll=8" overrides a default,
 // for measurement sweeps; the value becomes part of the source and so of the
 // cache key.
+// whether ACC_HIP_TUNE names the knob at all
+bool tuned(const char *name)
+{
+  return tune(name, -0x7ffffffe) != -0x7ffffffe;
+}
+
 int tune(const char *name, int dflt)
 {
   const char *e = std::getenv("ACC_HIP_TUNE");
@@ -522,8 +528,13 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
       break;
     }
     default:   // scans
-      sp->block = tune("scan.block", 1024);
-      sp->rows = tune("scan.rows", 8);
+      // A tile of 32 Ki elements either way.  Four waves with 32 rows a lane leave room for two workgroups on a compute
+      // unit, one loading while the other stores, as long as the instance keeps within 256 registers; where it does
+      // not (wide elements, operators that need temporaries) the first build falls back to sixteen waves with 8 rows
+      // (acc_skel_s::ensure_variant).  A shape given by hand is taken as it is.
+      sp->scan_shape_open = !tuned("scan.block") && !tuned("scan.rows");
+      sp->block = tune("scan.block", sp->scan_shape_open ? 256 : 1024);
+      sp->rows = tune("scan.rows", sp->scan_shape_open ? 32 : 8);
       break;
   }
   if (sp->block < 64 || sp->block > 1024 || (sp->block & 63)) return fail(ACC_ERR_INVALID, "block size %d is not a multiple of the 64-lane wavefront", sp->block);
@@ -562,7 +573,7 @@ SkelSpec spec_of_variant(const SkelSpec &base, int v)
 int acc_skel_s::ensure_variant(int v)
 {
   // two threads may meet here on the first launch that needs the unaligned variant
-  std::lock_guard<std::mutex> lock(mu);
+  std::unique_lock<std::mutex> lock(mu);
   acc::Variant &var = variants[v];
   if (var.ready) return ACC_OK;
   // variants 2 and 3 of a permute: the locked template for an element the atomic template also covers
@@ -616,6 +627,18 @@ int acc_skel_s::ensure_variant(int v)
     }
   }
   (void)hipFuncGetAttribute(&var.num_regs, HIP_FUNC_ATTRIBUTE_NUM_REGS, var.fn);
+  if (this->spec.scan_shape_open) {
+    // the first build of a scan decides its tile shape: see make_spec
+    this->spec.scan_shape_open = false;
+    if (var.num_regs > 256) {
+      (void)hipModuleUnload(var.module);
+      var = acc::Variant();
+      this->spec.block = 1024;
+      this->spec.rows = 8;
+      lock.unlock();
+      return ensure_variant(v);
+    }
+  }
   (void)hipFuncGetAttribute(&var.static_lds, HIP_FUNC_ATTRIBUTE_SHARED_SIZE_BYTES, var.fn);
   int bpc = 0;
   e = hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&bpc, var.fn, spec.block, 0);

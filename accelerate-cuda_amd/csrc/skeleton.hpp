@@ -40,6 +40,7 @@ struct SkelSpec {
   int tile_z = 1;                       // rank-3 stencils: result planes per strip
   // tuning
   int block = 256, unroll = 4, rows = 4, chunk = 4096;
+  bool scan_shape_open = false;         // a scan whose tile shape the first build may still change (by its register count)
 };
 
 // one compiled form of an instance: AccKernel of the reference (AST.hs:51-59)
@@ -58,6 +59,7 @@ struct Variant {
 
 int type_size(const std::string &t);
 int tune(const char *name, int dflt);
+bool tuned(const char *name);
 int make_spec(const acc_skel_desc *d, SkelSpec *sp);
 int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::string *source);
 SkelSpec spec_of_variant(const SkelSpec &base, int variant);
