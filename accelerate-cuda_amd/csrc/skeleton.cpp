@@ -528,13 +528,18 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
       break;
     }
     default:   // scans
-      // A tile of 32 Ki elements either way.  Four waves with 32 rows a lane leave room for two workgroups on a compute
-      // unit, one loading while the other stores, as long as the instance keeps within 256 registers; where it does
-      // not (wide elements, operators that need temporaries) the first build falls back to sixteen waves with 8 rows
-      // (acc_skel_s::ensure_variant).  A shape given by hand is taken as it is.
-      sp->scan_shape_open = !tuned("scan.block") && !tuned("scan.rows");
-      sp->block = tune("scan.block", sp->scan_shape_open ? 256 : 1024);
-      sp->rows = tune("scan.rows", sp->scan_shape_open ? 32 : 8);
+      // A tile of 128 KB either way (32 Ki Int32).  Four waves with up to 32 rows a lane leave room for two workgroups
+      // on a compute unit, one loading while the other stores, as long as the instance keeps within 256 registers;
+      // where it does not (operators that need temporaries) the first build falls back to sixteen waves with a
+      // quarter of the rows (acc_skel_s::ensure_variant).  A shape given by hand is taken as it is.
+      {
+        const int per_row = std::max(1, (16 / std::max(1, sp->vec_size)) * std::max(1, sp->elt_size));     // bytes a lane holds per row
+        const int rows4 = std::max(2, std::min(32, 131072 / (256 * per_row)));
+        sp->scan_shape_open = !tuned("scan.block") && !tuned("scan.rows");
+        sp->scan_rows_fallback = std::max(2, std::min(8, 131072 / (1024 * per_row)));
+        sp->block = tune("scan.block", sp->scan_shape_open ? 256 : 1024);
+        sp->rows = tune("scan.rows", sp->scan_shape_open ? rows4 : sp->scan_rows_fallback);
+      }
       break;
   }
   if (sp->block < 64 || sp->block > 1024 || (sp->block & 63)) return fail(ACC_ERR_INVALID, "block size %d is not a multiple of the 64-lane wavefront", sp->block);
@@ -634,7 +639,7 @@ int acc_skel_s::ensure_variant(int v)
       (void)hipModuleUnload(var.module);
       var = acc::Variant();
       this->spec.block = 1024;
-      this->spec.rows = 8;
+      this->spec.rows = this->spec.scan_rows_fallback;
       lock.unlock();
       return ensure_variant(v);
     }

@@ -40,6 +40,7 @@ struct SkelSpec {
   int tile_z = 1;                       // rank-3 stencils: result planes per strip
   // tuning
   int block = 256, unroll = 4, rows = 4, chunk = 4096;
+  int scan_rows_fallback = 8;
   bool scan_shape_open = false;         // a scan whose tile shape the first build may still change (by its register count)
 };
 
