@@ -29,7 +29,7 @@ for p in (ROOT, os.path.join(ROOT, "accelerate-cuda_amd")):
 import numpy as np  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
-SCANL_HBM_TRAFFIC_BYTES = 543200000
+SCANL_HBM_TRAFFIC_BYTES = 542500000
 
 
 def log(*a):
