@@ -47,8 +47,8 @@ std::string embedded_text(const char *name);
 enum ScratchProtocol {
   SCRATCH_FOLD = 0,   // contents are don't-care: every launch writes what it reads (fold partials, permute tables)
   SCRATCH_LOCKS = 2,  // all zero between uses: every launch leaves it as it found it
-  SCRATCH_SCAN = 1,   // word 0 is a tile counter used relative to `counter_base`; tile descriptors
-                      // carry `epoch`, so stale ones read as "not yet published"
+  SCRATCH_SCAN = 1,   // tile descriptors (behind a 256-byte header nothing uses): they carry `epoch`, so stale
+                      // ones read as "not yet published"
   SCRATCH_FLAGS = 3   // 64-bit words {epoch, payload}: every launch tags what it writes with its `epoch`,
                       // anything older reads as "not yet"
 };
@@ -62,7 +62,6 @@ struct ScratchBlock {
   bool busy = false;
   bool recorded = false;   // `done` was recorded at the last release
   uint32_t epoch = 0;
-  uint32_t counter_base = 0;
 };
 
 }  // namespace acc

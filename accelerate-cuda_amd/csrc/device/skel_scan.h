@@ -410,19 +410,10 @@ ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op, const T seed,
   }
 }
 
-/* Two ways of handing tiles to workgroups:
- *
- * ACC_SCAN_PERSISTENT == 0  one workgroup per tile, tile number = workgroup
- *   number.  Workgroups are dispatched in increasing order, so every
- *   predecessor of a running tile has itself been dispatched and the look-back
- *   always makes progress.
- * ACC_SCAN_PERSISTENT == 1  a resident grid of workgroups draws tile numbers
- *   from an atomic counter (two tiles ahead, so the atomic's round trip is
- *   never waited for) and loads the next tile's elements while the current
- *   tile waits for its prefix.
- * ACC_SCAN_PERSISTENT == 2  the same without the counter: workgroup b takes
- *   tiles b, b + grid, b + 2 grid, ...  Only valid under a cooperative launch,
- *   which guarantees that the whole grid is resident at once.               */
+/* One workgroup per tile, tile number = workgroup number.  Workgroups are dispatched in increasing order, so every
+ * predecessor of a running tile has itself been dispatched and the look-back always makes progress.  (Resident
+ * grids of workgroups that draw tiles from a counter, or take them in strides under a cooperative launch, and load
+ * the next tile behind the look-back, were measured at 110-340 us against 96 and are gone.) */
 /* second launch bound = waves per SIMD the register allocation must leave room for */
 #ifndef ACC_MIN_WAVES
 #define ACC_MIN_WAVES 1
@@ -432,7 +423,6 @@ ACC_ENTRY(ACC_ENV_PARAMS
           const Int64 shOut_0, ACC_OUT_ARRAY(arrOut),
           ACC_OUT_ARRAY(arrSum),
           const Int64 shIn_0,
-          unsigned int *__restrict__ tile_counter, const unsigned int counter_base,
           void *desc0, void *desc1, void *desc2,
           const unsigned int epoch, const Int64 num_tiles)
 {
@@ -469,19 +459,7 @@ ACC_ENTRY(ACC_ENV_PARAMS
   const Int64 n_up = (n + ACC_VEC - 1) / ACC_VEC * ACC_VEC;
   auto tile_base = [&](const Int64 t) -> Int64 { return ACC_SCAN_RIGHT ? n_up - (t + 1) * (Int64)ACC_TILE : t * (Int64)ACC_TILE; };
 
-#if ACC_SCAN_PERSISTENT == 1
-  __shared__ unsigned int s_ticket[4];
-  unsigned int pending = 0;
-  if (threadIdx.x == 0) {
-    s_ticket[0] = atomicAdd(tile_counter, 1u) - counter_base;
-    pending = atomicAdd(tile_counter, 1u);
-  }
-  __syncthreads();
-  Int64 tile = (Int64)s_ticket[0];
-#else
-  (void)tile_counter; (void)counter_base;
-  Int64 tile = (Int64)blockIdx.x;
-#endif
+  const Int64 tile = (Int64)blockIdx.x;
 
   if (n <= 0) {                                   /* PrefixSum.hs:249-251,330-334: scan of nothing is [seed] */
     if (threadIdx.x == 0 && tile == 0) {
@@ -495,47 +473,11 @@ ACC_ENTRY(ACC_ENV_PARAMS
   T cur[ACC_ROWS][ACC_VEC];
   if (tile < num_tiles) acc_scan_load(get, tile_base(tile), n, cur, wave, lane);
 
-#if ACC_SCAN_PERSISTENT == 1
-  T nxt[ACC_ROWS][ACC_VEC];
-  int slot = 1;
-  while (tile < num_tiles) {
-    /* hand over the ticket drawn one tile ago (read after the next barrier)
-     * and draw another */
-    if (threadIdx.x == 0) {
-      s_ticket[slot] = pending - counter_base;
-      pending = atomicAdd(tile_counter, 1u);
-    }
-    Int64 next = num_tiles;
-    auto prefetch = [&]() {
-      next = (Int64)s_ticket[slot];
-      if (next < num_tiles) acc_scan_load(get, tile_base(next), n, nxt, wave, lane);
-    };
-#elif ACC_SCAN_PERSISTENT == 2
-  T nxt[ACC_ROWS][ACC_VEC];
-  while (tile < num_tiles) {
-    Int64 next = tile + gridDim.x;
-    auto prefetch = [&]() {
-      if (next < num_tiles) acc_scan_load(get, tile_base(next), n, nxt, wave, lane);
-    };
-#else
   if (tile < num_tiles) {
     auto prefetch = [&]() {};
-#endif
-
     const Int64 base = tile_base(tile);
     const bool inside = base >= 0 && base + ACC_TILE <= n;
     acc_scan_tile<2, T>(cur, op, seed, tile, base, n, out, desc, epoch, (void *)s_wave, &s_prefix, prefetch, !inside);
 
-#if ACC_SCAN_PERSISTENT
-#pragma unroll
-    for (int r = 0; r < ACC_ROWS; ++r)
-#pragma unroll
-      for (int k = 0; k < ACC_VEC; ++k) cur[r][k] = nxt[r][k];
-    tile = next;
-#if ACC_SCAN_PERSISTENT == 1
-    slot = (slot + 1) & 3;
-#endif
-    __syncthreads();          /* s_wave and s_prefix are free for the next tile */
-#endif
   }
 }

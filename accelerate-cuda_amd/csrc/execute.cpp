@@ -387,15 +387,7 @@ int acc_exec_scan(acc_skel s, const acc_array *env, int64_t n, const acc_array *
   ACC_TRY(s->ensure_variant(v));
   const int64_t tile = s->elements_per_block();
   const int64_t tiles = (n + tile - 1) / tile;
-  int64_t grid = std::max<int64_t>(1, tiles);     // one workgroup per tile, in dispatch order ...
-  int64_t draws = 0;
-  const int persistent = acc::tune("scan.persistent", 0);
-  if (persistent) {
-    // ... or a resident grid of persistent workgroups, each drawing tiles until none are left
-    const int64_t per_cu = std::max(1, std::min(s->variants[v].blocks_per_cu, acc::tune("scan.blocks_per_cu", 2)));
-    grid = std::max<int64_t>(1, std::min<int64_t>(tiles, (int64_t)s->ctx->props.multiProcessorCount * per_cu));
-    draws = persistent == 1 ? tiles + 2 * grid : 0;   // every tile once, plus two draws ahead per workgroup
-  }
+  const int64_t grid = std::max<int64_t>(1, tiles);     // one workgroup per tile, in dispatch order
   const int64_t ndesc = std::max<int64_t>(1, tiles);
   const size_t esz = s->spec.elt_size;
   // one descriptor per tile: 64-bit words {flag, 4 bytes of the value}, `scan.desc_stride` words apart
@@ -405,7 +397,7 @@ int acc_exec_scan(acc_skel s, const acc_array *env, int64_t n, const acc_array *
   const size_t bytes = 256 + round256((size_t)ndesc * 8 * words);
   int blk = -1;
   ACC_TRY(s->ctx->scratch_acquire(bytes, st, acc::SCRATCH_SCAN, &blk));
-  uint32_t epoch, counter_base;
+  uint32_t epoch;
   char *base;
   {
     std::lock_guard<std::mutex> lock(s->ctx->mu);
@@ -415,36 +407,15 @@ int acc_exec_scan(acc_skel s, const acc_array *env, int64_t n, const acc_array *
       hipError_t e = hipMemsetAsync(b.ptr, 0, b.bytes, st);
       if (e != hipSuccess) { b.busy = false; return acc::fail_hip(e, "hipMemsetAsync(scan state)"); }
       b.epoch = 0;
-      b.counter_base = 0;
     }
     epoch = ++b.epoch;
-    counter_base = b.counter_base;
-    b.counter_base += static_cast<uint32_t>(draws);
   }
-  args.ptr(reinterpret_cast<uint64_t>(base));
-  args.u32(counter_base);
   args.ptr(reinterpret_cast<uint64_t>(base + off_d0));
   args.ptr(reinterpret_cast<uint64_t>(base + off_d1));
   args.ptr(reinterpret_cast<uint64_t>(base + off_d2));
   args.u32(epoch);
   args.i64(tiles);
-  int rc;
-  if (persistent == 2) {
-    // static tile assignment needs every workgroup resident at once: a cooperative launch promises that
-    rc = s->ctx->make_current();
-    if (rc == ACC_OK) {
-      hipError_t e = hipModuleLaunchCooperativeKernel(s->variants[v].fn, static_cast<unsigned>(grid), 1, 1,
-                                                      static_cast<unsigned>(s->spec.block), 1, 1, 0, st, args.data());
-      if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchCooperativeKernel(scan)");
-    }
-  } else {
-    rc = launch(s, v, grid, 0, st, &args);
-  }
-  if (rc != ACC_OK) {
-    // nothing ran: take the tickets back so that the block stays consistent
-    std::lock_guard<std::mutex> lock(s->ctx->mu);
-    s->ctx->scratch[blk].counter_base = counter_base;
-  }
+  const int rc = launch(s, v, grid, 0, st, &args);
   s->ctx->scratch_release(blk, st);
   return rc;
 }

@@ -245,7 +245,6 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "#define ACC_LOOKBACK " << tune("scan.lookback", 1) << "\n";
       o << "#define ACC_DESC_STRIDE " << tune("scan.desc_stride", 16) << "\n";
       o << "#define ACC_MIN_WAVES " << tune("scan.min_waves", 1) << "\n";
-      o << "#define ACC_SCAN_PERSISTENT " << tune("scan.persistent", 0) << "\n";
       tmpl = "skel_scan.h";
       break;
     }
