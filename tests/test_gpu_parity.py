@@ -742,3 +742,19 @@ def test_permute_index_types_and_stray_targets(A, ctx, orc):
     out = ctx.empty(300, np.int32)
     sk.permute([ctx.array(keys)], n, ctx.array(np.zeros(300, np.int32)), out)
     assert np.array_equal(out.get(), np.bincount(keys[keys < 300], minlength=300).astype(np.int32))
+
+
+def test_scan_tile_shape_follows_the_register_count(A, ctx):
+    """the first build of a scan decides its tile shape: four waves with many rows a lane where that keeps within
+    256 registers, else sixteen waves; tiles hold 128 KB either way, and the results do not depend on the shape"""
+    for ctype, dt, comb in (("Int32", np.int32, "x + y"), ("double", np.float64, "acc_max(x, y)")):
+        sk = ctx.skeleton(A.SKEL_SCANL1, ctype, env=[(1, ctype)], get="arrIn0_0[ix]", combine=comb)
+        info = sk.info()
+        say("scan of", ctype, "block", info.block, "registers", info.num_regs, "elements per tile", info.elements_per_block)
+        assert info.block in (256, 1024) and (info.block == 1024 or info.num_regs <= 256)
+        assert info.elements_per_block * np.dtype(dt).itemsize == 128 * 1024
+        x = rng.integers(-1000, 1000, 3 * info.elements_per_block + 17).astype(dt)
+        out = ctx.empty(x.size, dt)
+        sk.scan([ctx.array(x)], x.size, out)
+        ref = np.cumsum(x, dtype=dt) if ctype == "Int32" else np.maximum.accumulate(x)
+        assert np.array_equal(out.get(), ref)
