@@ -540,10 +540,11 @@ def use(host, context=None):
     It is uploaded when first wanted there and once only, however often it is `use`d (Array/Prim.hs:177-192); it must
     not be changed afterwards."""
     cx = context or Context.default()
+    as_word8 = lambda h: h.view(np.uint8) if h.dtype == np.bool_ else h      # Bool is Word8 on the device (CodeGen/Type.hs)
     if isinstance(host, tuple):
-        hs = [np.asarray(h, order="C") for h in host]
+        hs = [as_word8(np.asarray(h, order="C")) for h in host]
         return Acc(hs[0].shape, tuple(CTYPE[h.dtype.type] for h in hs), manifest=A.TupleArray([_Resident(cx, h, True) for h in hs]))
-    host = np.asarray(host, order="C")                  # (ascontiguousarray would make a scalar array a vector)
+    host = as_word8(np.asarray(host, order="C"))        # (ascontiguousarray would make a scalar array a vector)
     return Acc(host.shape, CTYPE[host.dtype.type], manifest=_Resident(cx, host, True))
 
 
@@ -656,7 +657,8 @@ def _combine(f, ctype):
 
 def _fold(f, z, a, seedless, context):
     cx = _context(context, a)
-    out_shape = a.shape[:-1]
+    # an empty outer extent counts as 1 in the result of a seeded fold (Execute.hs:287-289)
+    out_shape = a.shape[:-1] if seedless else tuple(max(1, d) for d in a.shape[:-1])
     arrays, sig, fr = _assemble(get=a.stream().text, combine=_combine(f, a.ctype).text,
                                 seed=None if seedless else Exp.of(z, a.ctype).text)
     sk = cx.skeleton(A.SKEL_FOLD1 if seedless else A.SKEL_FOLD, _elt(a.ctype), sig, out_rank=len(out_shape), **fr)

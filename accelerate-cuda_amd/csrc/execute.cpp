@@ -233,12 +233,22 @@ int acc_exec_fold(acc_skel s, const acc_array *env, int32_t in_rank, const int64
   ACC_TRY(check_out(s, out, s->spec.out_rank, "result"));
   for (int d = 0; d < in_rank; ++d)
     if (in_shape[d] < 0) return fail(ACC_ERR_INVALID, "%s: negative input extent", s->entry.c_str());
-  const int64_t inner = in_shape[in_rank - 1];
+  int64_t inner = in_shape[in_rank - 1];
   // fold1 of an empty innermost dimension: Execute.hs:282-285
   if (inner == 0 && !s->spec.has_seed) return fail(ACC_ERR_INVALID, "%s: empty array", s->entry.c_str());
-  // empty outer extents count as 1: Execute.hs:287-289
+  // empty outer extents count as 1 in the result of a seeded fold: Execute.hs:287-289.  (The reference then runs its
+  // kernel over rows that do not exist; here such a result is the seed in every position, as for rows without
+  // elements, and a fold1 over no rows has nothing to do.)
   int64_t rows = 1;
-  for (int d = 0; d + 1 < in_rank; ++d) rows *= std::max<int64_t>(1, in_shape[d]);
+  bool no_rows = false;
+  for (int d = 0; d + 1 < in_rank; ++d) {
+    rows *= std::max<int64_t>(1, in_shape[d]);
+    no_rows = no_rows || in_shape[d] == 0;
+  }
+  if (no_rows) {
+    if (!s->spec.has_seed) return ACC_OK;
+    inner = 0;
+  }
   if (array_size(*out) < rows && !(in_rank == 1)) return fail(ACC_ERR_INVALID, "%s: result holds %lld elements, %lld needed", s->entry.c_str(), (long long)array_size(*out), (long long)rows);
 
   hipStream_t st = static_cast<hipStream_t>(stream);

@@ -557,3 +557,30 @@ def test_the_rest_of_the_scalar_primitives(acc):
     assert np.array_equal(q, np.trunc(a / b).astype(np.int32)) and np.array_equal(r, a - b * np.trunc(a / b).astype(np.int32))
     d, m = acc.run(acc.unzip(acc.zipWith(acc.divMod, acc.use(a), acc.use(b))))
     assert np.array_equal(d, a // b) and np.array_equal(m, a % b)
+
+
+def test_empty_arrays_and_booleans(acc):
+    """arrays without elements through every consumer (Reduction.hs:212-214, PrefixSum.hs:249-251, Execute.hs:282-289),
+    and host arrays of booleans, which are Word8 on the device"""
+    e = np.zeros(0, np.int32)
+    assert acc.run(acc.map(lambda v: v + 1, acc.use(e))).shape == (0,)
+    assert int(acc.run(acc.fold(add, 7, acc.use(e)))) == 7
+    assert acc.run(acc.scanl(add, 3, acc.use(e))).tolist() == [3]
+    assert acc.run(acc.scanl1(add, acc.use(e))).shape == (0,)
+    body, total = acc.run(acc.scanl_(add, 3, acc.use(e)))
+    assert body.shape == (0,) and int(total) == 3
+    assert acc.run(acc.permute(add, acc.fill((5,), 1, "Int32"), lambda i: (i,), acc.use(e))).tolist() == [1] * 5
+    with pytest.raises(Exception, match="empty array"):
+        acc.run(acc.fold1(add, acc.use(e)))
+    # rows without elements yield the seed; an empty OUTER extent counts as 1 in a seeded fold's result, and a fold1
+    # over no rows is an empty array
+    assert acc.run(acc.fold(add, 7, acc.use(np.zeros((5, 0), np.int32)))).tolist() == [7] * 5
+    assert acc.run(acc.fold(add, 7, acc.use(np.zeros((0, 5), np.int32)))).tolist() == [7]
+    assert acc.run(acc.fold1(add, acc.use(np.zeros((0, 5), np.int32)))).shape == (0,)
+    assert acc.run(acc.foldSeg(add, 0, acc.use(e), acc.use(e))).shape == (0,)
+    assert acc.run(acc.foldSeg(add, 0, acc.use(np.arange(6, dtype=np.int32)), acc.use(np.array([0, 3, 0, 3, 0], np.int32)))).tolist() == [0, 3, 0, 12, 0]
+    kept, count = acc.run(acc.filter_(lambda v: v > 100, acc.use(np.arange(10, dtype=np.int32))))
+    assert kept.shape == (0,) and int(count) == 0
+    flags = np.array([True, False, True, True])
+    assert acc.run(acc.map(lambda v: v.lnot(), acc.use(flags))).tolist() == [0, 1, 0, 0]
+    assert int(acc.run(acc.sum_(acc.map(lambda v: acc.fromIntegral(v, "Int32"), acc.use(flags))))) == 3
