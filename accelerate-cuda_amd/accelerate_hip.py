@@ -26,6 +26,7 @@ skeleton hot path, in miniature:
     environment, AST.hs:87-112) and named arrIn<k>_0 in the text.
 Everything runs on the GPU through the C ABI; there is no other execution path.
 """
+import collections
 import numbers
 import re
 import threading
@@ -344,8 +345,14 @@ class Acc(object):
 _MANIFEST = weakref.WeakValueDictionary()        # tag number -> device array, while some computation still names it
 
 
+_PENDING = collections.deque(maxlen=16)          # arrays named in text that has not been assembled yet: an array `use`d
+                                                 # inside a scalar function is referred to by nothing else until then
+
+
 def _tag(manifest):
     _MANIFEST[id(manifest)] = manifest
+    if not any(m is manifest for m in _PENDING):
+        _PENDING.append(manifest)
     return "@@%d@@" % id(manifest)
 
 
@@ -358,6 +365,10 @@ def _assemble(**fragments):
             if int(m.group(1)) not in order:
                 order.append(int(m.group(1)))
     arrays = [_MANIFEST[i] for i in order]
+    for m in arrays:                                  # from here on the caller holds them
+        for k in range(len(_PENDING) - 1, -1, -1):
+            if _PENDING[k] is m:
+                del _PENDING[k]
     out = {}
     for name, text in fragments.items():
         if text is not None:

@@ -581,6 +581,9 @@ def test_empty_arrays_and_booleans(acc):
     assert acc.run(acc.foldSeg(add, 0, acc.use(np.arange(6, dtype=np.int32)), acc.use(np.array([0, 3, 0, 3, 0], np.int32)))).tolist() == [0, 3, 0, 12, 0]
     kept, count = acc.run(acc.filter_(lambda v: v > 100, acc.use(np.arange(10, dtype=np.int32))))
     assert kept.shape == (0,) and int(count) == 0
+    # an array `use`d inside the scalar function itself, Int64 indices
+    h = acc.run(acc.permute(add, acc.fill((4,), 0, "Int64"), lambda i: (acc.use(np.array([0, 3, 3, 1], np.int64))[i],), acc.fill((4,), 5, "Int64")))
+    assert h.tolist() == [5, 5, 0, 10]
     flags = np.array([True, False, True, True])
     assert acc.run(acc.map(lambda v: v.lnot(), acc.use(flags))).tolist() == [0, 1, 0, 0]
     assert int(acc.run(acc.sum_(acc.map(lambda v: acc.fromIntegral(v, "Int32"), acc.use(flags))))) == 3
