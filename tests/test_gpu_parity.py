@@ -615,6 +615,13 @@ def test_fold_along_the_innermost_dimension_at_every_shape(A, ctx):
     out = ctx.empty(17, np.int32)
     add.fold([ctx.empty((17, 0), np.int32)], (17, 0), out)
     assert np.array_equal(out.get(), np.full(17, 5, np.int32))
+    say("an empty outer extent: no row exists to be read; a seeded fold gives the seed once (Execute.hs:287-289), fold1 nothing")
+    out = ctx.array(np.full(1, -1, np.int32))
+    add.fold([ctx.empty((0, 5), np.int32)], (0, 5), out)
+    assert out.get().tolist() == [5]
+    out = ctx.array(np.full(3, -1, np.int32))
+    first.fold([ctx.empty((0, 5), np.int32)], (0, 5), out)
+    assert out.get().tolist() == [-1, -1, -1]
 
 
 def test_fold_of_short_rows(A, ctx, orc):
