@@ -345,14 +345,22 @@ class Acc(object):
 _MANIFEST = weakref.WeakValueDictionary()        # tag number -> device array, while some computation still names it
 
 
-_PENDING = collections.deque(maxlen=16)          # arrays named in text that has not been assembled yet: an array `use`d
-                                                 # inside a scalar function is referred to by nothing else until then
+_building = threading.local()     # .pending: arrays named in text that this thread has not assembled yet -- an array
+                                  # `use`d inside a scalar function is referred to by nothing else until then
+
+
+def _pending():
+    q = getattr(_building, "pending", None)
+    if q is None:
+        q = _building.pending = collections.deque(maxlen=16)
+    return q
 
 
 def _tag(manifest):
     _MANIFEST[id(manifest)] = manifest
-    if not any(m is manifest for m in _PENDING):
-        _PENDING.append(manifest)
+    q = _pending()
+    if not any(m is manifest for m in q):
+        q.append(manifest)
     return "@@%d@@" % id(manifest)
 
 
@@ -365,10 +373,11 @@ def _assemble(**fragments):
             if int(m.group(1)) not in order:
                 order.append(int(m.group(1)))
     arrays = [_MANIFEST[i] for i in order]
+    q = _pending()
     for m in arrays:                                  # from here on the caller holds them
-        for k in range(len(_PENDING) - 1, -1, -1):
-            if _PENDING[k] is m:
-                del _PENDING[k]
+        for k in range(len(q) - 1, -1, -1):
+            if q[k] is m:
+                del q[k]
     out = {}
     for name, text in fragments.items():
         if text is not None:
@@ -415,8 +424,9 @@ class _Resident(object):
         self.cx, self.host, self.shape, self.dtype, self.size = cx, host, host.shape, host.dtype, host.size
         self.key = A.MemTable.key(host)
         self.stream, self.ready = None, None          # where it was produced, and the event recorded behind that
-        cx.table.malloc(host, frozen)
-        cx.live[self.key] = cx.live.get(self.key, 0) + 1
+        with cx.lock:
+            cx.table.malloc(host, frozen)
+            cx.live[self.key] = cx.live.get(self.key, 0) + 1
 
     def get(self):
         if self.ready is not None:
@@ -430,13 +440,14 @@ class _Resident(object):
     def __del__(self):
         try:
             cx = self.cx
-            if self.ready is not None:
-                cx.events.append(self.ready)
-            cx.live[self.key] -= 1
-            if cx.live[self.key] == 0:
-                del cx.live[self.key]
-                if cx.table.handle:
-                    cx.table.free(self.host)
+            with cx.lock:
+                if self.ready is not None:
+                    cx.events.append(self.ready)
+                cx.live[self.key] -= 1
+                if cx.live[self.key] == 0:
+                    del cx.live[self.key]
+                    if cx.table.handle:
+                        cx.table.free(self.host)
         except Exception:
             pass
 
@@ -474,10 +485,11 @@ class Context(object):
     def skeleton(self, kind, elt, env, **kw):
         key = (kind, elt, tuple((r, tuple(t) if isinstance(t, list) else t) for r, t in env),
                tuple(sorted((k, str(v)) for k, v in kw.items())))
-        sk = self.skeletons.get(key)
-        if sk is None:
-            sk = self.ctx.skeleton(kind, elt, env=env, **kw)
-            self.skeletons[key] = sk
+        with self.lock:
+            sk = self.skeletons.get(key)
+            if sk is None:
+                sk = self.ctx.skeleton(kind, elt, env=env, **kw)
+                self.skeletons[key] = sk
         return sk
 
     N_STREAMS = 4
@@ -494,6 +506,10 @@ class Context(object):
     def launch(self, inputs, outputs, go):
         """run `go(input views, output views, stream)` with the arrays resident (None stays None), after what
         produced the inputs; the outputs carry the event recorded behind it"""
+        with self.lock:                                  # consumers launch as they are built, from whichever thread
+            return self._launch(inputs, outputs, go)
+
+    def _launch(self, inputs, outputs, go):
         def parts(ms):
             for m in ms:
                 if isinstance(m, A.TupleArray):

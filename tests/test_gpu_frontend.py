@@ -587,3 +587,33 @@ def test_empty_arrays_and_booleans(acc):
     flags = np.array([True, False, True, True])
     assert acc.run(acc.map(lambda v: v.lnot(), acc.use(flags))).tolist() == [0, 1, 0, 0]
     assert int(acc.run(acc.sum_(acc.map(lambda v: acc.fromIntegral(v, "Int32"), acc.use(flags))))) == 3
+
+
+def test_threads_building_computations_in_one_context(acc):
+    """consumers launch as they are built, so threads that share a context meet in its launch path: eight threads,
+    each with its own arrays and a few skeletons in common"""
+    import threading
+    cx = acc.create(0)
+    errors = []
+
+    def work(k):
+        try:
+            rng = np.random.default_rng(100 + k)
+            for rep in range(5):
+                x = rng.integers(-50, 50, 20000 + 37 * k + rep).astype(np.int32)
+                xs = acc.use(x, cx)
+                s = acc.run(acc.scanl1(add, acc.map(lambda v: v * 2, xs)), cx)
+                assert np.array_equal(s, np.cumsum(x * 2, dtype=np.int32))
+                h = acc.run(acc.permute(add, acc.fill((64,), 0, "Int32"), lambda i: (acc.use(np.abs(x) % 64, cx)[i],), acc.fill((x.size,), 1, "Int32")), cx)
+                assert np.array_equal(h, np.bincount(np.abs(x) % 64, minlength=64).astype(np.int32))
+        except Exception as e:                      # reported by the main thread
+            errors.append((k, repr(e)))
+    threads = [threading.Thread(target=work, args=(k,)) for k in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    try:
+        assert not errors, errors
+    finally:
+        acc.destroy(cx)
