@@ -724,8 +724,16 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
     const int64_t fill_grid = std::min<int64_t>((XCD_ROWS * ntarget + 255) / 256, 8 * (int64_t)cus);
     e = hipModuleLaunchKernel(s->variants[v].fn_fill, static_cast<unsigned>(fill_grid), 1, 1, 256, 1, 1, 0, st, f.data(), nullptr);
     if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(permute_fill)");
-  } else {
-    rc = plain_copy();
+  } else if (copy_defaults) {           // the defaults by the same kernel: a runtime copy of 1 KB takes 4 us, this launch 2
+    Args f;
+    f.ptr(0);
+    f.i64(0);
+    f.ptr(out->ptr[0]);
+    f.ptr(defaults->ptr[0]);
+    f.i64(ntarget);
+    const int64_t fill_grid = std::min<int64_t>((ntarget + 255) / 256, 8 * (int64_t)cus);
+    e = hipModuleLaunchKernel(s->variants[v].fn_fill, static_cast<unsigned>(fill_grid), 1, 1, 256, 1, 1, 0, st, f.data(), nullptr);
+    if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(permute_fill, defaults)");
   }
   args.i32(static_cast<int32_t>(bins));
   args.i32(static_cast<int32_t>(copies));
