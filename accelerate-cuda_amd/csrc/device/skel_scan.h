@@ -287,10 +287,18 @@ ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op, const T seed,
       asm volatile("" : "+s"(row_base) : "v"(x[r][0]));
       lead = lead_of(acc_scan_ix0(row_base, wave, lane, r));
     }
+    if (GUARD && ACC_SCAN_RIGHT) {
 #pragma unroll
-    for (int k = 0; k < ACC_VEC; ++k) {
-      const V v = x[r][k];
-      s[r][k] = (k == 0 || (GUARD && ACC_SCAN_RIGHT && k == lead)) ? v : op(s[r][k - 1], v);
+      for (int k = 0; k < ACC_VEC; ++k) {
+        const V v = x[r][k];
+        s[r][k] = (k == 0 || k == lead) ? v : op(s[r][k - 1], v);
+      }
+    } else {                                /* every other tile: no test per element */
+#pragma unroll
+      for (int k = 0; k < ACC_VEC; ++k) {
+        const V v = x[r][k];
+        s[r][k] = (k == 0) ? v : op(s[r][k - 1], v);
+      }
     }
   }
 
