@@ -278,15 +278,7 @@ ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op, const T seed,
   };
 #pragma unroll
   for (int r = 0; r < ACC_ROWS; ++r) {
-    int lead = 0;
-    if (GUARD && ACC_SCAN_RIGHT) {
-      /* worked out when the row's elements have arrived, not before: hoisted above the wait for the loads, the
-       * rows' indices and leads would be alive all at once (the compiler is told that `row_base` depends on the
-       * row's first element) */
-      Int64 row_base = base;
-      asm volatile("" : "+s"(row_base) : "v"(x[r][0]));
-      lead = lead_of(acc_scan_ix0(row_base, wave, lane, r));
-    }
+    const int lead = (GUARD && ACC_SCAN_RIGHT) ? lead_of(acc_scan_ix0(base, wave, lane, r)) : 0;
     if (GUARD && ACC_SCAN_RIGHT) {
 #pragma unroll
       for (int k = 0; k < ACC_VEC; ++k) {

@@ -532,10 +532,12 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
       // where it does not (operators that need temporaries) the first build falls back to sixteen waves with a
       // quarter of the rows (acc_skel_s::ensure_variant).  A shape given by hand is taken as it is.
       {
-        const int per_row = std::max(1, (16 / std::max(1, sp->vec_size)) * std::max(1, sp->elt_size));     // bytes a lane holds per row
-        const int rows4 = std::max(2, std::min(32, 131072 / (256 * per_row)));
+        const int vec = std::max(1, 16 / std::max(1, sp->vec_size));                                       // elements per lane and row
+        const int per_row = std::max(1, vec * std::max(1, sp->elt_size));                                  // bytes of them
+        // (an element takes a register whatever its width: no more than 128 of them a lane, 32 on sixteen waves)
+        const int rows4 = std::max(2, std::min({32, 131072 / (256 * per_row), 128 / vec}));
         sp->scan_shape_open = !tuned("scan.block") && !tuned("scan.rows");
-        sp->scan_rows_fallback = std::max(2, std::min(8, 131072 / (1024 * per_row)));
+        sp->scan_rows_fallback = std::max(2, std::min({8, 131072 / (1024 * per_row), 32 / vec}));
         sp->block = tune("scan.block", sp->scan_shape_open ? 256 : 1024);
         sp->rows = tune("scan.rows", sp->scan_shape_open ? rows4 : sp->scan_rows_fallback);
       }

@@ -751,6 +751,40 @@ def test_permute_index_types_and_stray_targets(A, ctx, orc):
     assert np.array_equal(out.get(), np.bincount(keys[keys < 300], minlength=300).astype(np.int32))
 
 
+def test_right_handed_scans_of_every_element_width(A, ctx):
+    """scanr, scanr1 and scanr' over 1-, 2-, 4- and 8-byte elements and over pairs, at sizes around the tile
+    boundaries and sizes that are no multiple of a vector (the rounding positions of the first vector)"""
+    def rscan(x):                                           # inclusive from the right, in the element type
+        return np.cumsum(x[::-1], dtype=x.dtype)[::-1]
+    for ctype, dt in (("Int8", np.int8), ("Word16", np.uint16), ("Int32", np.int32), ("Int64", np.int64), ("double", np.float64)):
+        lit = "3.0" if ctype == "double" else "3"
+        r0 = ctx.skeleton(A.SKEL_SCANR, ctype, env=[(1, ctype)], get="arrIn0_0[ix]", combine="(%s)(x + y)" % ctype, seed=lit)
+        r1 = ctx.skeleton(A.SKEL_SCANR1, ctype, env=[(1, ctype)], get="arrIn0_0[ix]", combine="(%s)(x + y)" % ctype)
+        rp = ctx.skeleton(A.SKEL_SCANRP, ctype, env=[(1, ctype)], get="arrIn0_0[ix]", combine="(%s)(x + y)" % ctype, seed=lit)
+        tile = r1.info().elements_per_block
+        for n in (1, 3, 17, tile - 1, tile, tile + 1, 3 * tile + 5, 300007):
+            say("right-handed scans of", ctype, "n =", n)
+            x = rng.integers(0, 9, n).astype(dt)
+            inc = rscan(x)
+            out = ctx.empty(n + 1, dt)
+            r0.scan([ctx.array(x)], n, out)
+            assert np.array_equal(out.get(), np.concatenate([inc + dt(3), [dt(3)]]).astype(dt))
+            out = ctx.empty(n, dt)
+            r1.scan([ctx.array(x)], n, out)
+            assert np.array_equal(out.get(), inc)
+            tot = ctx.empty((), dt)
+            rp.scan([ctx.array(x)], n, out, total=tot)
+            assert np.array_equal(out.get(), np.concatenate([inc[1:] + dt(3), [dt(3)]]).astype(dt)) and tot.get()[()] == dt(inc[0] + dt(3))
+    say("right-handed scan of pairs")
+    pr = ctx.skeleton(A.SKEL_SCANR1, "Int32, float", env=[(1, "Int32"), (1, "float")], get="acc_elt{arrIn0_0[ix], arrIn1_0[ix]}",
+                      combine="acc_elt{x.a1 + y.a1, acc_max(x.a0, y.a0)}")
+    n = 100003
+    a, b = rng.integers(-9, 9, n).astype(np.int32), rng.random(n).astype(np.float32)
+    out = A.TupleArray([ctx.empty(n, np.int32), ctx.empty(n, np.float32)])
+    pr.scan([ctx.array(a), ctx.array(b)], n, out)
+    assert np.array_equal(out.comps[0].get(), rscan(a)) and np.array_equal(out.comps[1].get(), np.maximum.accumulate(b[::-1])[::-1])
+
+
 def test_scan_tile_shape_follows_the_register_count(A, ctx):
     """the first build of a scan decides its tile shape: four waves with many rows a lane where that keeps within
     256 registers, else sixteen waves; tiles hold 128 KB either way, and the results do not depend on the shape"""
