@@ -243,6 +243,15 @@ def compile_only(desc, target="gfx950"):
     return size.value
 
 
+def compile_source(source, target="gfx950", options=("-O3", "-std=c++17", "-ffp-contract=off", "-Xclang", "-target-feature",
+                                                      "-Xclang", "-packed-fp32-ops")):
+    """hiprtc-compile one translation unit through the kernel cache; needs no GPU.  Returns the code size."""
+    opts = (C.c_char_p * len(options))(*[o.encode() for o in options])
+    code, size = C.c_void_p(), C.c_size_t(0)
+    check(lib().acc_compile(None, target.encode(), source.encode(), opts, len(options), C.byref(code), C.byref(size)))
+    return size.value
+
+
 def cache_stats():
     st = acc_cache_stats()
     check(lib().acc_cache_get_stats(C.byref(st)))

@@ -60,6 +60,21 @@ def test_every_skeleton_instance_compiles_for_gfx950(A, tmp_path):
         assert A.compile_only(desc, "gfx950") > 4000, name
 
 
+def test_permute_variants_the_driver_chooses_between_all_compile(A, tmp_path):
+    """tables under locks in LDS (+2), several LDS windows of targets (+4), 16-bit counts (+6): generated from the same
+    description, each for aligned and unaligned operands"""
+    A.lib().acc_cache_set_dir(str(tmp_path).encode())
+    hist = A.make_desc(A.SKEL_PERMUTE, "Int32", env=[(1, "Int32")], out_rank=1, get="1", combine="x + y",
+                       permutation="arrIn0_0[ix]", combine_hint=A.COMBINE_ADD)
+    generic = A.make_desc(A.SKEL_PERMUTE, "float", env=[(1, "Int32"), (1, "float")], out_rank=1, get="arrIn1_0[ix]",
+                          combine="acc_max(x, y)", permutation="arrIn0_0[ix]")
+    for desc, variants in ((hist, (0, 1, 4, 5, 6, 7)), (generic, (0, 1, 2, 3))):
+        for v in variants:
+            name, src = A.preview(desc, v)
+            assert name == "permute" and ("ACC_PERMUTE_NARROW 1" in src) == (v >= 6)
+            assert A.compile_source(src) > 4000, v
+
+
 def test_every_scalar_primitive_compiles_for_every_type(A, tmp_path):
     """acc_prim.h: one map per element type naming every primitive that type has
     (CodeGen.hs:406-476); what they compute is checked on the GPU"""
