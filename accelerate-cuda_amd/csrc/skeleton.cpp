@@ -353,6 +353,15 @@ static bool small_literal(std::string t)
   return t.size() == 1 && t[0] >= '0' && t[0] <= '3';
 }
 
+// elements a workgroup of the segmented fold stages at a time: a whole number of its block-wide vector loads (a lane
+// loads 16 bytes, so 16 elements of one byte: one load of 256 lanes is then 4096 of them)
+static int segmented_chunk(const SkelSpec &sp)
+{
+  const int per_load = sp.block * std::max(1, 16 / std::max(1, sp.vec_size));
+  const int want = std::max(tune("foldseg.chunk", 2048), per_load);
+  return (want + per_load - 1) / per_load * per_load;
+}
+
 int make_spec(const acc_skel_desc *d, SkelSpec *sp)
 {
   if (!d) return fail(ACC_ERR_INVALID, "NULL skeleton description");
@@ -449,12 +458,12 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
       sp->unroll = tune("fold.unroll", 4);
       if (sp->out_rank > 0) {
         sp->block = tune("foldseg.block", 256);
-        sp->chunk = tune("foldseg.chunk", 2048);
+        sp->chunk = segmented_chunk(*sp);
       }
       break;
     case ACC_SKEL_FOLDSEG: case ACC_SKEL_FOLD1SEG:
       sp->block = tune("foldseg.block", 256);
-      sp->chunk = tune("foldseg.chunk", 2048);
+      sp->chunk = segmented_chunk(*sp);
       break;
     case ACC_SKEL_PERMUTE:
       if (sp->permutation.empty()) return fail(ACC_ERR_INVALID, "permute: `permutation` fragment missing");

@@ -751,6 +751,28 @@ def test_permute_index_types_and_stray_targets(A, ctx, orc):
     assert np.array_equal(out.get(), np.bincount(keys[keys < 300], minlength=300).astype(np.int32))
 
 
+def test_segmented_and_innermost_folds_of_narrow_elements(A, ctx):
+    """1- and 2-byte elements: a lane loads 16 of them at once, so a workgroup's chunk is larger than for 4-byte ones"""
+    for ctype, dt in (("Word8", np.uint8), ("Int16", np.int16)):
+        seg = ctx.skeleton(A.SKEL_FOLDSEG, ctype, env=[(1, ctype)], get="arrIn0_0[ix]", combine="(%s)(x + y)" % ctype, seed="1")
+        dim = ctx.skeleton(A.SKEL_FOLD, ctype, env=[(2, ctype)], out_rank=1, get="arrIn0_0[ix]", combine="(%s)(x + y)" % ctype, seed="1")
+        for nseg, mean in ((1, 5), (1000, 3), (5000, 40), (300, 3000)):
+            say("foldSeg of", ctype, nseg, "segments of about", mean)
+            lens = rng.poisson(mean, nseg)
+            offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+            x = rng.integers(0, 7, int(offs[-1])).astype(dt)
+            out = ctx.empty(nseg, dt)
+            seg.foldseg([ctx.array(x) if x.size else ctx.empty(0, dt)], x.size, ctx.array(offs), out)
+            ref = np.array([x[a:b].sum(dtype=np.int64) + 1 for a, b in zip(offs[:-1], offs[1:])]).astype(dt)
+            assert np.array_equal(out.get(), ref)
+        for rows, inner in ((7, 3), (1000, 16), (333, 1000), (4, 70001)):
+            say("fold of a", rows, "x", inner, ctype, "array")
+            x = rng.integers(0, 7, (rows, inner)).astype(dt)
+            out = ctx.empty(rows, dt)
+            dim.fold([ctx.array(x)], (rows, inner), out)
+            assert np.array_equal(out.get(), (x.sum(axis=1, dtype=np.int64) + 1).astype(dt))
+
+
 def test_right_handed_scans_of_every_element_width(A, ctx):
     """scanr, scanr1 and scanr' over 1-, 2-, 4- and 8-byte elements and over pairs, at sizes around the tile
     boundaries and sizes that are no multiple of a vector (the rounding positions of the first vector)"""
