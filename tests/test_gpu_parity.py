@@ -11,6 +11,8 @@ import sys
 import numpy as np
 import pytest
 
+import pyref
+
 pytestmark = pytest.mark.gpu
 
 rng = np.random.default_rng(77)
@@ -771,6 +773,35 @@ def test_segmented_and_innermost_folds_of_narrow_elements(A, ctx):
             out = ctx.empty(rows, dt)
             dim.fold([ctx.array(x)], (rows, inner), out)
             assert np.array_equal(out.get(), (x.sum(axis=1, dtype=np.int64) + 1).astype(dt))
+
+
+def test_stencils_of_every_element_width(A, ctx):
+    """2-D stencils in the four boundary modes and a 3-D one over 1-, 2-, 4- and 8-byte elements (integer arithmetic
+    wraps in the element type; Float64 on small integers is exact)"""
+    five = [(-1, 0), (0, -1), (0, 0), (0, 1), (1, 0)]
+    seven = [(0, 0, 0), (-1, 0, 0), (1, 0, 0), (0, -1, 0), (0, 1, 0), (0, 0, -1), (0, 0, 1)]
+    for ctype, dt in (("Int8", np.int8), ("Word16", np.uint16), ("Int64", np.int64), ("double", np.float64)):
+        cast = "(%s)" % ctype
+        wide = (lambda a: a) if ctype == "double" else (lambda a: a.astype(np.int64))
+        for mode in ("clamp", "mirror", "wrap", "constant"):
+            sk = ctx.skeleton(A.SKEL_STENCIL, ctype, out_rank=2, taps=five, boundary=mode, boundary_constant=cast + "2",
+                              stencil_fn=cast + "(t0 + 2 * t1 - t2 + t3 + t4)")
+            for shape in ((5, 7), (33, 300), (7, 1031)):
+                say("stencil of", ctype, mode, shape)
+                v = rng.integers(0, 5, shape).astype(dt)
+                out = ctx.empty(shape, dt)
+                sk.stencil([], ctx.array(v), out)
+                t = [wide(a) for a in pyref.tap_arrays(v, five, mode, 2, shape)]
+                assert np.array_equal(out.get(), (t[0] + 2 * t[1] - t[2] + t[3] + t[4]).astype(dt))
+        sk = ctx.skeleton(A.SKEL_STENCIL, ctype, out_rank=3, taps=seven, boundary="mirror",
+                          stencil_fn=cast + "(t0 + t1 + t2 + t3 + t4 + t5 + 2 * t6)")
+        for shape in ((3, 5, 7), (4, 9, 1031)):
+            say("3-D stencil of", ctype, shape)
+            v = rng.integers(0, 5, shape).astype(dt)
+            out = ctx.empty(shape, dt)
+            sk.stencil([], ctx.array(v), out)
+            t = [wide(a) for a in pyref.tap_arrays3(v, seven, "mirror", 0, shape)]
+            assert np.array_equal(out.get(), (sum(t[:6]) + 2 * t[6]).astype(dt))
 
 
 def test_right_handed_scans_of_every_element_width(A, ctx):
