@@ -197,6 +197,19 @@ ACC_DEV Int64 acc_xcd_contiguous_block()
  * the L2.  The code generator uses it for linear reads next to indirect ones. */
 template <typename T> ACC_DEV T acc_stream(const T *p, const Int64 ix) { return __builtin_nontemporal_load(p + ix); }
 
+/* Keep a value where it was computed.  The compiler otherwise moves the tail of a long dependent chain -- load an
+ * index, gather through it, multiply -- down to its first use, past whatever stands in between, so that its memory
+ * round trips start only there and are waited for one after the other. */
+template <typename T> ACC_DEV void acc_pin(T &v)
+{
+  unsigned int w[acc_words<T>::n];
+  w[acc_words<T>::n - 1] = 0;
+  __builtin_memcpy(w, &v, sizeof(T));
+#pragma unroll
+  for (int k = 0; k < acc_words<T>::n; ++k) asm volatile("" : "+v"(w[k]));
+  __builtin_memcpy(&v, w, sizeof(T));
+}
+
 /* a compile-time flag passed as a value (to generic lambdas) */
 template <bool B> struct acc_bool { static constexpr bool value = B; };
 

@@ -82,8 +82,12 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
   for (Int64 first = (Int64)blockIdx.x * ACC_BLOCK; first < nseg; first += (Int64)gridDim.x * ACC_BLOCK) {
     const Int64 seg = first + tid;
     const bool live = seg < nseg;
-    const Int64 a = live ? ACC_SEG_AT(seg) : 0;
-    const Int64 b = live ? ACC_SEG_AT(seg + 1) : 0;
+    /* both ends of the lane's segment are asked for at once (a lane past the last segment asks for the last one's
+     * and takes nothing) */
+    const Int64 seg_c = acc_min<Int64>(seg, nseg - 1);
+    const Int64 a_c = ACC_SEG_AT(seg_c), b_c = ACC_SEG_AT(seg_c + 1);
+    const Int64 a = live ? a_c : 0;
+    const Int64 b = live ? b_c : 0;
     const Int64 last = acc_min<Int64>(first + ACC_BLOCK, nseg);
     const Int64 lo = ACC_SEG_AT(first), hi = acc_min<Int64>(ACC_SEG_AT(last), n);
 
@@ -97,30 +101,37 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
     /* chunks start on a vector boundary so that the loads stay aligned */
     const Int64 lo_al = lo - (lo % ACC_VEC);
     const Int64 nchunks = hi > lo_al ? (hi - lo_al + ACC_CHUNK - 1) / ACC_CHUNK : 0;
-    /* stage a chunk: every load is issued before any result is used.  Elements
-     * of the chunk's first and last vector that belong to a neighbouring block
-     * are loaded too (they exist) and never read back; only the very end of
-     * the array needs a guard.  Vectors that lie wholly beyond this block's
-     * segments are left out: short segments fill a fraction of a chunk, and
-     * behind every element may stand a gather. */
+    /* stage a chunk: every load is issued before any result is used, with no branch among them, so that all the
+     * loads of a chunk -- and the gathers that may stand behind every element -- are in flight together.  Elements
+     * of the chunk's first and last vector that belong to a neighbouring block are loaded too (they exist) and
+     * never read back.  A vector that lies wholly beyond this block's segments is not wanted (short segments fill
+     * a fraction of a chunk, and every element may cost a gather): its lane reads the block's last vector instead,
+     * which all such lanes of a wave do with one request between them.  Only the block that holds the ragged end
+     * of the array goes element by element. */
     T v[ACC_LOADS][ACC_VEC];
     auto chunk_start = [&](const Int64 q) -> Int64 { return lo_al + (ACC_FOLD_RIGHT ? (nchunks - 1 - q) : q) * (Int64)ACC_CHUNK; };
+    const Int64 last_vec = hi > 0 ? (hi - 1) / ACC_VEC : 0;           /* index of the vector that holds element hi - 1 */
+    const bool whole_vectors = (last_vec + 1) * ACC_VEC <= n;        /* uniform over the block */
     auto stage = [&](const Int64 cs) {
-      if (cs + ACC_CHUNK <= n) {
+      if (whole_vectors) {
+#pragma unroll
+        for (int u = 0; u < ACC_LOADS; ++u) {
+          const Int64 i0 = acc_min<Int64>(cs / ACC_VEC + (u * ACC_BLOCK + tid), last_vec) * ACC_VEC;
+#pragma unroll
+          for (int k = 0; k < ACC_VEC; ++k) v[u][k] = get(i0 + k);
+        }
 #pragma unroll
         for (int u = 0; u < ACC_LOADS; ++u)
-          if (cs + (Int64)(u * ACC_BLOCK + tid) * ACC_VEC < hi) {
 #pragma unroll
-            for (int k = 0; k < ACC_VEC; ++k) v[u][k] = get(cs + (u * ACC_BLOCK + tid) * ACC_VEC + k);
-          }
+          for (int k = 0; k < ACC_VEC; ++k) acc_pin(v[u][k]);
       } else {
 #pragma unroll
         for (int u = 0; u < ACC_LOADS; ++u)
 #pragma unroll
           for (int k = 0; k < ACC_VEC; ++k) {
-            const Int64 ix = cs + (u * ACC_BLOCK + tid) * ACC_VEC + k;
-            v[u][k] = T();
-            if (ix < n) v[u][k] = get(ix);
+            /* past the end of the array: its last element instead, which no segment reads back from there */
+            const Int64 ix = acc_min<Int64>(acc_min<Int64>(cs / ACC_VEC + (u * ACC_BLOCK + tid), last_vec) * ACC_VEC + k, n - 1);
+            v[u][k] = get(ix);
           }
       }
     };
