@@ -94,7 +94,7 @@ acc_stream_wait_event acc_event_create acc_event_destroy acc_event_record acc_ev
 acc_event_elapsed_ms acc_compile acc_compile_log acc_cache_set_dir acc_cache_dir acc_cache_get_stats
 acc_cache_clear acc_module_load acc_module_unload acc_module_get_function acc_function_attr acc_occupancy
 acc_launch acc_launch_grid acc_skel_create acc_skel_destroy acc_skel_source acc_skel_preview acc_skel_compile_only
-acc_skel_get_info acc_exec_map acc_exec_fold acc_exec_foldseg acc_exec_scan acc_exec_permute
+acc_skel_get_info acc_exec_map acc_exec_fold acc_exec_foldseg acc_exec_scan acc_exec_scan_noalloc acc_exec_permute
 acc_exec_stencil acc_exec_stencil2 acc_exec_stencil_iterate acc_memtable_create acc_memtable_destroy
 acc_memtable_malloc acc_memtable_acquire acc_memtable_release acc_memtable_free acc_memtable_insert_unmanaged
 acc_memtable_reclaim acc_memtable_get_stats""".split()
@@ -155,6 +155,7 @@ def lib():
         L.acc_exec_fold.argtypes = [C.c_void_p, AP, C.c_int32, C.POINTER(C.c_int64), AP, C.c_void_p]
         L.acc_exec_foldseg.argtypes = [C.c_void_p, AP, C.c_int64, AP, AP, C.c_void_p]
         L.acc_exec_scan.argtypes = [C.c_void_p, AP, C.c_int64, AP, AP, C.c_void_p]
+        L.acc_exec_scan_noalloc.argtypes = [C.c_void_p, AP, C.c_int64, AP, AP, C.c_void_p]
         L.acc_exec_permute.argtypes = [C.c_void_p, AP, C.c_int64, AP, AP, C.c_void_p]
         L.acc_exec_stencil.argtypes = [C.c_void_p, AP, AP, AP, C.c_void_p]
         L.acc_exec_stencil2.argtypes = [C.c_void_p, AP, AP, AP, AP, C.c_void_p]
@@ -490,10 +491,11 @@ class Skeleton(object):
     def foldseg(self, env, n, offsets, out, stream=None):
         check(lib().acc_exec_foldseg(self.handle, _env(env), n, C.byref(offsets.desc()), C.byref(out.desc()), stream))
 
-    def scan(self, env, n, out, total=None, stream=None):
+    def scan(self, env, n, out, total=None, stream=None, noalloc=False):
         o = out if isinstance(out, acc_array) else out.desc()
         t = None if total is None else C.byref(total if isinstance(total, acc_array) else total.desc(shape=()))
-        check(lib().acc_exec_scan(self.handle, _env(env), n, C.byref(o), t, stream))
+        fn = lib().acc_exec_scan_noalloc if noalloc else lib().acc_exec_scan
+        check(fn(self.handle, _env(env), n, C.byref(o), t, stream))
 
     def permute(self, env, n_src, defaults, out, stream=None):
         check(lib().acc_exec_permute(self.handle, _env(env), n_src, C.byref(defaults.desc()), C.byref(out.desc()), stream))

@@ -15,6 +15,10 @@
 
 #define ACC_HIP_VERSION "0.1.0"
 
+// bytes of the file-scope device array behind acc_exec_scan_noalloc: a 256-byte header and one 128-byte tile
+// descriptor for each of ACC_NOALLOC_MAX_TILES tiles (noalloc.hip)
+#define ACC_NOALLOC_SCRATCH_BYTES (256 + ACC_NOALLOC_MAX_TILES * 128)
+
 namespace acc {
 
 // thread-local message of the last failure; returns `code` so that call
@@ -34,6 +38,10 @@ void set_compile_log(const std::string &log);
     int _rc = (expr);            \
     if (_rc != ACC_OK) return _rc; \
   } while (0)
+
+// the scan's descriptor block for callers that must not allocate (noalloc.hip)
+int noalloc_setup(int device);
+int noalloc_scan_state(int device, size_t bytes, hipStream_t stream, void **base, uint32_t *epoch);
 
 // embedded device headers (embed.cpp)
 struct EmbeddedHeader { const char *name; const char *begin; const char *end; };

@@ -367,11 +367,17 @@ int acc_exec_foldseg(acc_skel s, const acc_array *env, int64_t n, const acc_arra
   return launch_segmented(s, v, &args, env, out, nseg, n, static_cast<hipStream_t>(stream));
 }
 
-int acc_exec_scan(acc_skel s, const acc_array *env, int64_t n, const acc_array *out, const acc_array *total, acc_stream stream)
+namespace {
+
+// scanOp / scan1Op / scan'Op / scanCore, Execute.hs:328-392, as ONE launch.  `noalloc`: the tile descriptors live in
+// the library's file-scope device array instead of a block of the context's pool, and nothing may be allocated,
+// compiled or loaded on the way.
+int scan_core(acc_skel s, const acc_array *env, int64_t n, const acc_array *out, const acc_array *total, acc_stream stream,
+              const bool noalloc, const char *who)
 {
-  if (!s) return fail(ACC_ERR_INVALID, "acc_exec_scan: NULL skeleton");
+  if (!s) return fail(ACC_ERR_INVALID, "%s: NULL skeleton", who);
   if (!kind_is(s, {ACC_SKEL_SCANL, ACC_SKEL_SCANL1, ACC_SKEL_SCANLP, ACC_SKEL_SCANR, ACC_SKEL_SCANR1, ACC_SKEL_SCANRP}))
-    return fail(ACC_ERR_INVALID, "acc_exec_scan: skeleton is '%s'", s->entry.c_str());
+    return fail(ACC_ERR_INVALID, "%s: skeleton is '%s'", who, s->entry.c_str());
   if (n < 0) return fail(ACC_ERR_INVALID, "%s: negative input extent", s->entry.c_str());
   ACC_TRY(check_out(s, out, 1, "result"));
   const int kind = s->spec.kind;
@@ -394,17 +400,43 @@ int acc_exec_scan(acc_skel s, const acc_array *env, int64_t n, const acc_array *
   args.i64(n);
 
   const int v = aligned ? 0 : 1;
-  ACC_TRY(s->ensure_variant(v));
+  if (noalloc) {
+    // building a variant compiles and loads a module: not here
+    if (!s->variant_ready(v))
+      return fail(ACC_ERR_INVALID, "%s: the %s variant of this instance is not loaded yet; run acc_exec_scan once on operands of the same alignment first",
+                  who, aligned ? "aligned" : "unaligned");
+  } else {
+    ACC_TRY(s->ensure_variant(v));
+  }
   const int64_t tile = s->elements_per_block();
   const int64_t tiles = (n + tile - 1) / tile;
   const int64_t grid = std::max<int64_t>(1, tiles);     // one workgroup per tile, in dispatch order
   const int64_t ndesc = std::max<int64_t>(1, tiles);
   const size_t esz = s->spec.elt_size;
-  // one descriptor per tile: 64-bit words {flag, 4 bytes of the value}, `scan.desc_stride` words apart
+  // one descriptor per tile: 64-bit words {flag, 4 bytes of the value}, `desc_stride` words apart
   // (more when the element needs more words)
-  const size_t words = std::max<size_t>((esz + 3) / 4, (size_t)acc::tune("scan.desc_stride", 16));
+  const size_t words = std::max<size_t>((esz + 3) / 4, (size_t)s->spec.scan_desc_stride);
   const size_t off_d0 = 256, off_d1 = 256, off_d2 = 256;
   const size_t bytes = 256 + round256((size_t)ndesc * 8 * words);
+  if (noalloc) {
+    if (tiles > ACC_NOALLOC_MAX_TILES)
+      return fail(ACC_ERR_INVALID, "%s: %lld elements are %lld tiles of %lld, more than the %d the scratch array has descriptors for",
+                  who, (long long)n, (long long)tiles, (long long)tile, ACC_NOALLOC_MAX_TILES);
+    ACC_TRY(s->ctx->make_current());
+    void *nbase = nullptr;
+    uint32_t nepoch = 0;
+    ACC_TRY(acc::noalloc_scan_state(s->ctx->device, bytes, st, &nbase, &nepoch));
+    char *b = static_cast<char *>(nbase);
+    args.ptr(reinterpret_cast<uint64_t>(b + off_d0));
+    args.ptr(reinterpret_cast<uint64_t>(b + off_d1));
+    args.ptr(reinterpret_cast<uint64_t>(b + off_d2));
+    args.u32(nepoch);
+    args.i64(tiles);
+    if (grid < 1 || grid > 0x7fffffffLL) return fail(ACC_ERR_INVALID, "%s: grid of %lld blocks", who, (long long)grid);
+    ACC_HIP_TRY(hipModuleLaunchKernel(s->variants[v].fn, static_cast<unsigned>(grid), 1, 1, static_cast<unsigned>(s->spec.block), 1, 1,
+                                      0, st, args.data(), nullptr));
+    return ACC_OK;
+  }
   int blk = -1;
   ACC_TRY(s->ctx->scratch_acquire(bytes, st, acc::SCRATCH_SCAN, &blk));
   uint32_t epoch;
@@ -428,6 +460,18 @@ int acc_exec_scan(acc_skel s, const acc_array *env, int64_t n, const acc_array *
   const int rc = launch(s, v, grid, 0, st, &args);
   s->ctx->scratch_release(blk, st);
   return rc;
+}
+
+}  // namespace
+
+int acc_exec_scan(acc_skel s, const acc_array *env, int64_t n, const acc_array *out, const acc_array *total, acc_stream stream)
+{
+  return scan_core(s, env, n, out, total, stream, false, "acc_exec_scan");
+}
+
+int acc_exec_scan_noalloc(acc_skel s, const acc_array *env, int64_t n, const acc_array *out, const acc_array *total, acc_stream stream)
+{
+  return scan_core(s, env, n, out, total, stream, true, "acc_exec_scan_noalloc");
 }
 
 int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_array *defaults, const acc_array *out, acc_stream stream)

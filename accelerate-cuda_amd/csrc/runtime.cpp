@@ -156,6 +156,7 @@ int acc_context_create(int device, acc_context *out)
   hipError_t e = hipGetDeviceProperties(&ctx->props, device);
   if (e == hipSuccess) e = hipSetDevice(device);
   if (e != hipSuccess) { delete ctx; return acc::fail_hip(e, "acc_context_create"); }
+  (void)acc::noalloc_setup(device);      // the address of the library's own device array on this device, once
   ctx->arch = ctx->props.gcnArchName;
   const size_t colon = ctx->arch.find(':');
   if (colon != std::string::npos) ctx->arch.resize(colon);

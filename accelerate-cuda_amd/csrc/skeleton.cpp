@@ -243,7 +243,7 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "#define ACC_SCAN_RIGHT " << (right ? 1 : 0) << "\n#define ACC_SCAN_MODE " << mode << "\n";
       o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_ROWS " << sp.rows << "\n";
       o << "#define ACC_LOOKBACK " << tune("scan.lookback", 1) << "\n";
-      o << "#define ACC_DESC_STRIDE " << tune("scan.desc_stride", 16) << "\n";
+      o << "#define ACC_DESC_STRIDE " << sp.scan_desc_stride << "\n";
       o << "#define ACC_MIN_WAVES " << tune("scan.min_waves", 1) << "\n";
       tmpl = "skel_scan.h";
       break;
@@ -545,6 +545,7 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
         const int per_row = std::max(1, vec * std::max(1, sp->elt_size));                                  // bytes of them
         // (an element takes a register whatever its width: no more than 128 of them a lane, 32 on sixteen waves)
         const int rows4 = std::max(2, std::min({32, 131072 / (256 * per_row), 128 / vec}));
+        sp->scan_desc_stride = std::max(1, tune("scan.desc_stride", 16));
         sp->scan_shape_open = !tuned("scan.block") && !tuned("scan.rows");
         sp->scan_rows_fallback = std::max(2, std::min({8, 131072 / (1024 * per_row), 32 / vec}));
         sp->block = tune("scan.block", sp->scan_shape_open ? 256 : 1024);

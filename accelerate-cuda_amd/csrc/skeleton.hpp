@@ -41,6 +41,7 @@ struct SkelSpec {
   // tuning
   int block = 256, unroll = 4, rows = 4, chunk = 4096;
   int scan_rows_fallback = 8;
+  int scan_desc_stride = 16;            // 8-byte words between the tile descriptors of a scan, as generated into the kernel
   bool scan_shape_open = false;         // a scan whose tile shape the first build may still change (by its register count)
 };
 
@@ -79,6 +80,7 @@ struct acc_skel_s {
   std::mutex mu;
 
   int ensure_variant(int v);
+  bool variant_ready(int v) { std::lock_guard<std::mutex> lock(mu); return variants[v].ready; }
   int ncomp() const { return spec.comp_types.empty() ? 1 : (int)spec.comp_types.size(); }
   int vec() const { int v = 16 / (spec.vec_size > 0 ? spec.vec_size : 1); return v < 1 ? 1 : v; }
   int elements_per_block() const

@@ -292,6 +292,7 @@ foreign import ccall safe   "acc_exec_map"             c_execMap            :: S
 foreign import ccall safe   "acc_exec_fold"            c_execFold           :: Skel -> Ptr AccArray -> Int32 -> Ptr Int64 -> Ptr AccArray -> Stream -> IO Status
 foreign import ccall safe   "acc_exec_foldseg"         c_execFoldseg        :: Skel -> Ptr AccArray -> Int64 -> Ptr AccArray -> Ptr AccArray -> Stream -> IO Status
 foreign import ccall safe   "acc_exec_scan"            c_execScan           :: Skel -> Ptr AccArray -> Int64 -> Ptr AccArray -> Ptr AccArray -> Stream -> IO Status
+foreign import ccall safe   "acc_exec_scan_noalloc"    c_execScanNoalloc    :: Skel -> Ptr AccArray -> Int64 -> Ptr AccArray -> Ptr AccArray -> Stream -> IO Status
 foreign import ccall safe   "acc_exec_permute"         c_execPermute        :: Skel -> Ptr AccArray -> Int64 -> Ptr AccArray -> Ptr AccArray -> Stream -> IO Status
 foreign import ccall safe   "acc_exec_stencil"         c_execStencil        :: Skel -> Ptr AccArray -> Ptr AccArray -> Ptr AccArray -> Stream -> IO Status
 foreign import ccall safe   "acc_exec_stencil2"        c_execStencil2       :: Skel -> Ptr AccArray -> Ptr AccArray -> Ptr AccArray -> Ptr AccArray -> Stream -> IO Status

@@ -354,6 +354,22 @@ int acc_exec_foldseg(acc_skel s, const acc_array *env, int64_t n, const acc_arra
 int acc_exec_scan(acc_skel s, const acc_array *env, int64_t n, const acc_array *out,
                   const acc_array *total, acc_stream stream);
 
+/* The same scan for callers that cannot allocate device memory: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid it.  It has no counterpart in the reference (whose scanCore allocates its block
+ * sums on every call, Execute.hs:371-376).  The tile descriptors live in a file-scope array in device memory that
+ * the library holds on every device it has a context on, until the process ends (about 1 MB); the call allocates
+ * nothing, compiles nothing and loads nothing:
+ *   - the input may span at most ACC_NOALLOC_MAX_TILES tiles of acc_skel_info.elements_per_block elements
+ *     (32768 Int32 each: 2^28 elements); more is ACC_ERR_INVALID;
+ *   - the variant for the operands' alignment must have been loaded already (the aligned one is by
+ *     acc_skel_create, the unaligned one by a first acc_exec_scan on such operands), else ACC_ERR_INVALID;
+ *   - every call on a device shares that device's array: calls that overlap in time on one device, from any
+ *     stream, thread or context, race.  Calls ordered on one stream are fine.
+ * Results are those of acc_exec_scan, bit for bit.                                                          */
+#define ACC_NOALLOC_MAX_TILES 8192
+int acc_exec_scan_noalloc(acc_skel s, const acc_array *env, int64_t n, const acc_array *out,
+                          const acc_array *total, acc_stream stream);
+
 /* permute: permuteOp, Execute.hs:396-408.  `n_src` source elements (linear);
  * out is first filled from `defaults` (same shape), then combined into.
  * defaults may alias out (then nothing is copied).                           */
