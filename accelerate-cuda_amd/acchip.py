@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libacchip.so")
 CSRC = os.path.join(_HERE, "csrc")
 
-OK, ERR_INVALID, ERR_OOM, ERR_COMPILE, ERR_NOT_FOUND, ERR_HIP, ERR_UNSUPPORTED, ERR_IO = range(8)
+OK, ERR_INVALID, ERR_OOM, ERR_COMPILE, ERR_NOT_FOUND, ERR_HIP, ERR_UNSUPPORTED, ERR_IO, ERR_STUCK = range(9)
 MAX_RANK, MAX_COMP = 8, 8
 
 (SKEL_MAP, SKEL_GENERATE, SKEL_TRANSFORM, SKEL_FOLD, SKEL_FOLD1, SKEL_FOLDSEG, SKEL_FOLD1SEG,
@@ -87,7 +87,8 @@ class acc_memtable_stats(C.Structure):
 
 
 SYMBOLS = """acc_last_error acc_version acc_init acc_device_count acc_device_get_props acc_context_create
-acc_context_destroy acc_context_device acc_context_sync acc_malloc acc_free acc_mem_info acc_host_alloc
+acc_context_destroy acc_context_device acc_context_sync acc_context_trim acc_context_scratch_bytes
+acc_context_debug_poke_lock acc_malloc acc_free acc_mem_info acc_host_alloc
 acc_host_free acc_memcpy_h2d acc_memcpy_d2h acc_memcpy_d2d acc_memcpy_h2d_async acc_memcpy_d2h_async
 acc_memcpy_d2d_async acc_memset32_async acc_stream_create acc_stream_destroy acc_stream_sync
 acc_stream_wait_event acc_event_create acc_event_destroy acc_event_record acc_event_sync acc_event_query
@@ -132,6 +133,9 @@ def lib():
         L.acc_context_create.argtypes = [C.c_int, C.POINTER(C.c_void_p)]
         L.acc_context_destroy.argtypes = [C.c_void_p]
         L.acc_context_sync.argtypes = [C.c_void_p]
+        L.acc_context_trim.argtypes = [C.c_void_p, C.POINTER(C.c_size_t)]
+        L.acc_context_scratch_bytes.argtypes = [C.c_void_p, C.POINTER(C.c_size_t)]
+        L.acc_context_debug_poke_lock.argtypes = [C.c_void_p, C.c_size_t, C.c_uint32]
         L.acc_stream_create.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
         L.acc_stream_destroy.argtypes = [C.c_void_p, C.c_void_p]
         L.acc_stream_sync.argtypes = [C.c_void_p, C.c_void_p]
@@ -354,6 +358,17 @@ class Context(object):
 
     def sync(self):
         check(lib().acc_context_sync(self.handle))
+
+    def trim(self):
+        """Free the scratch blocks that are not in use; returns the bytes given back."""
+        freed = C.c_size_t()
+        check(lib().acc_context_trim(self.handle, C.byref(freed)))
+        return freed.value
+
+    def scratch_bytes(self):
+        held = C.c_size_t()
+        check(lib().acc_context_scratch_bytes(self.handle, C.byref(held)))
+        return held.value
 
     def empty(self, shape, dtype):
         if isinstance(shape, int):

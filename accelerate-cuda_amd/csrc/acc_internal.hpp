@@ -69,8 +69,28 @@ struct ScratchBlock {
   hipEvent_t done = nullptr;
   bool busy = false;
   bool recorded = false;   // `done` was recorded at the last release
+  bool dirty = false;      // SCRATCH_LOCKS: a launch may have left it non-zero: cleared again before it is lent
   uint32_t epoch = 0;
 };
+
+// What a borrower holds of a block: copies taken under the pool's lock (the pool's vector may move meanwhile).
+// `epoch` is the tag of this use for the SCRATCH_SCAN / SCRATCH_FLAGS protocols (the pool starts a block over from
+// zeroes before its tags run out).
+struct ScratchRef {
+  int index = -1;
+  void *ptr = nullptr;
+  size_t bytes = 0;
+  uint32_t epoch = 0;
+};
+
+// Words of a context's status block (pinned host memory that kernels write, the host reads at synchronisation
+// points): non-zero = a kernel's bounded wait ran out since the block was last read.
+enum StatusWord { STATUS_SCAN_LOOKBACK = 0, STATUS_FOLD_COLLECT = 1, STATUS_PERMUTE_LOCK = 2, STATUS_WORDS = 16 };
+
+// big single-pass scans on different streams of one device are kept from overlapping (runtime.cpp)
+int scan_order_before(int device, hipStream_t stream);    // ACC_OK: the caller launches, then calls scan_order_after
+void scan_order_after(int device);
+void scan_order_forget(int device, hipStream_t stream);
 
 }  // namespace acc
 
@@ -87,9 +107,18 @@ struct acc_context_s {
   bool scratch_multi_stream = false;
   hipStream_t scratch_first_stream = nullptr;
 
+  // kernels report here that a bounded wait ran out (see StatusWord); NULL if the block could not be set up
+  volatile uint32_t *status_host = nullptr;
+  uint64_t status_dev = 0;
+
   int make_current() const;
   // zero-initialised when first allocated; contents persist between uses and
   // follow the block's protocol
-  int scratch_acquire(size_t bytes, hipStream_t stream, int protocol, int *index);
-  void scratch_release(int index, hipStream_t stream);
+  int scratch_acquire(size_t bytes, hipStream_t stream, int protocol, acc::ScratchRef *out);
+  void scratch_release(const acc::ScratchRef &ref, hipStream_t stream);
+  // free every block that is not lent and whose last use has completed; returns the bytes given back
+  size_t scratch_trim();
+  size_t scratch_bytes();
+  // ACC_ERR_STUCK (once) if a kernel has reported a wait that ran out since the last call
+  int check_status(const char *who);
 };

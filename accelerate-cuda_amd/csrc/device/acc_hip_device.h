@@ -191,6 +191,21 @@ ACC_DEV Int64 acc_xcd_contiguous_block()
   return xcd * q + acc_min<Int64>(xcd, r) + i;
 }
 
+/* Waits of one workgroup for another are bounded: after ACC_SPIN_LIMIT polls the waiting lane gives up, says so
+ * in the context's status block -- words in host memory that the host looks at whenever it synchronises -- and
+ * carries on with whatever value it has, so that every kernel ends.  Nothing of that launch's result is to be
+ * trusted then.  A healthy run never writes here.  Word numbers as in the host's StatusWord. */
+#ifndef ACC_SPIN_LIMIT
+#define ACC_SPIN_LIMIT (1 << 22)
+#endif
+#define ACC_STATUS_SCAN_LOOKBACK 0
+#define ACC_STATUS_FOLD_COLLECT  1
+#define ACC_STATUS_PERMUTE_LOCK  2
+ACC_DEV void acc_report(unsigned int *status, const int word)
+{
+  if (status) __hip_atomic_store(status + word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 /* A read of an array element that will not be needed again (a manifest input
  * consumed once, in index order).  It is marked non-temporal so that it does
  * not evict data that IS reused -- a gathered vector, a small table -- from

@@ -69,16 +69,22 @@ struct acc_tagged {
     for (int k = 0; k < NW; ++k)
       __hip_atomic_store(d + (Int64)slot * NW + k, ((unsigned long long)tag << 32) | b[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
-  ACC_DEV T wait(unsigned int slot, unsigned int tag) const
+  /* (bounded: a word that does not turn up within ACC_SPIN_LIMIT polls is taken as it is and reported) */
+  ACC_DEV T wait(unsigned int slot, unsigned int tag, unsigned int *status) const
   {
     unsigned int b[NW];
+    int polls = 0;
 #pragma unroll
     for (int k = 0; k < NW; ++k) {
       unsigned long long w;
-      while ((unsigned int)((w = __hip_atomic_load(d + (Int64)slot * NW + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >> 32) != tag)
+      while ((unsigned int)((w = __hip_atomic_load(d + (Int64)slot * NW + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >> 32) != tag &&
+             polls < ACC_SPIN_LIMIT) {
+        ++polls;
         __builtin_amdgcn_s_sleep(1);
+      }
       b[k] = (unsigned int)w;
     }
+    if (polls >= ACC_SPIN_LIMIT) acc_report(status, ACC_STATUS_FOLD_COLLECT);
     T v;
     __builtin_memcpy(&v, b, sizeof(T));
     return v;
@@ -91,7 +97,7 @@ ACC_ENTRY(ACC_ENV_PARAMS
           ACC_OUT_ARRAY(arrOut),
           const Int64 shIn_0,
 #if ACC_FOLD_SINGLE
-          unsigned long long *partials, const unsigned int epoch)
+          unsigned long long *partials, const unsigned int epoch, unsigned int *acc_status)
 #else
           ACC_ELT *__restrict__ partials)
 #endif
@@ -179,7 +185,7 @@ ACC_ENTRY(ACC_ENV_PARAMS
       return;
     }
     acc_opt<T> p = threadIdx.x == 0 ? total : acc_none<T>();
-    for (unsigned int i = threadIdx.x; i < last; i += ACC_BLOCK) p = lf(p, acc_some(slots.wait(i, epoch)));
+    for (unsigned int i = threadIdx.x; i < last; i += ACC_BLOCK) p = lf(p, acc_some(slots.wait(i, epoch, acc_status)));
     total = acc_block_reduce(p, f, s_wave);
   }
   if (threadIdx.x != 0) return;

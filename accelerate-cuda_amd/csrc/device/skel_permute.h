@@ -56,8 +56,8 @@
  * and the next holder, on whichever die, loads the element after its exchange
  * has returned.  (A release/acquire pair would do as well and costs a
  * cache-wide write-back and invalidate per update: 40 times slower.)  `locks`
- * must be all zero on entry and is all zero again on exit; the word before it
- * records a lane that gave up.                                               */
+ * must be all zero on entry and is all zero again on exit, unless a lane gave
+ * up (then the status block says so, and the host clears the locks).         */
 /* When all targets fit, every workgroup combines its share of the source in a table of its own in LDS, under
  * LDS locks of the same kind (state per target: 0 nothing yet, 1 held, 2 holds a value), and leaves the table
  * in `dump_val` / `dump_ok` (one row per workgroup); permute_join then folds the rows into the result, one wave
@@ -69,7 +69,7 @@
  * of global locks per element while the windows are few).                                                 */
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, int *__restrict__ locks, const int lds_bins, const int lds_copies,
-        ACC_ELT *__restrict__ dump_val, int *__restrict__ dump_ok, const int win_blocks)
+        ACC_ELT *__restrict__ dump_val, int *__restrict__ dump_ok, const int win_blocks, unsigned int *acc_status)
 {
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
@@ -87,7 +87,7 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, int *__restrict__ loc
   auto update_global = [&](const Int64 j, const T &x, const bool active) {
     bool done = !active;
     Int64 trips = 0;
-    while (__ballot(!done) != 0 && trips < 64 * n + (1 << 20)) {
+    while (__ballot(!done) != 0 && trips < 64 * n + ACC_SPIN_LIMIT) {
       const bool got = !done && __hip_atomic_exchange(locks + j, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0;
       /* failed exchanges queue at the lock's address in front of the store that frees it: a wave that keeps
        * getting nowhere steps back for a while */
@@ -101,7 +101,7 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, int *__restrict__ loc
       }
       ++trips;
     }
-    if (!done) locks[-1] = 1;                       /* never seen in a healthy run: a lock that did not open */
+    if (!done) acc_report(acc_status, ACC_STATUS_PERMUTE_LOCK);      /* never in a healthy run: a lock that did not open; the update is lost */
   };
 
   if (lds_bins <= 0) {
@@ -311,6 +311,9 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
 #if ACC_PERMUTE_WINDOWS
         , const int win_blocks, const int win_log
 #endif
+#if ACC_PERMUTE_NARROW
+        , unsigned int *acc_status
+#endif
         )
 {
   typedef ACC_ELT T;
@@ -379,10 +382,15 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
   auto narrow_wait = [&](const U t, const unsigned before) {
     if (before >= ACC_NARROW_STOP) {
       const unsigned sh = narrow_shift(t);
-      /* (the correction is a few instructions away in another wave; the bound only makes sure that every wave ends) */
-      for (int polls = 0; polls < (1 << 20) &&
-           ((__hip_atomic_load(words + narrow_word(t), __ATOMIC_RELAXED, ACC_SCOPE_BLOCK) >> sh) & 0xFFFFu) >= ACC_NARROW_STOP; ++polls)
+      /* (the correction is a few instructions away in another wave; the bound only makes sure that every wave ends,
+       * and a wait that does run out is reported: the count may then have spilt into its neighbour) */
+      int polls = 0;
+      while (((__hip_atomic_load(words + narrow_word(t), __ATOMIC_RELAXED, ACC_SCOPE_BLOCK) >> sh) & 0xFFFFu) >= ACC_NARROW_STOP &&
+             polls < ACC_SPIN_LIMIT) {
+        ++polls;
         __builtin_amdgcn_s_sleep(1);
+      }
+      if (polls >= ACC_SPIN_LIMIT) acc_report(acc_status, ACC_STATUS_PERMUTE_LOCK);
     }
   };
   (void)ident; (void)bins;

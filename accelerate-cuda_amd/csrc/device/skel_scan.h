@@ -139,12 +139,16 @@ ACC_DEV void acc_scan_window_load(const acc_scan_desc<T> &desc, const Int64 look
 
 template <typename T, typename Op>
 ACC_DEV T acc_scan_lookback(const acc_scan_desc<T> &desc, Int64 tile, const T &block_total, Op op,
-                            unsigned int epoch, int lane, acc_scan_window<T> &w)
+                            unsigned int epoch, int lane, acc_scan_window<T> &w, unsigned int *status)
 {
   /* slots are ordered nearest predecessor first, so a reduction in slot order
    * must combine (later, earlier) */
   auto back = acc_lift<T>([&](const T &later, const T &earlier) -> T { return op(earlier, later); });
   acc_opt<T> run = acc_none<T>();
+  /* A descriptor that does not turn up within ACC_SPIN_LIMIT polls of this lane (all its waits together) is given
+   * up: the walk ends there with whatever it has, the status block says so, and this tile still posts a PREFIX, so
+   * that its successors do not wait for it in turn. */
+  int polls = 0;
 
   for (Int64 look = tile - 1;; look -= ACC_WAVE * ACC_LOOKBACK) {
     if (look != tile - 1) acc_scan_window_load(desc, look, lane, w);
@@ -153,7 +157,8 @@ ACC_DEV T acc_scan_lookback(const acc_scan_desc<T> &desc, Int64 tile, const T &b
     for (int j = 0; j < ACC_LOOKBACK; ++j) {
       const Int64 idx = look - (lane * ACC_LOOKBACK + j);
       if (idx >= 0) {
-        while ((w.fl[j] >> 2) != epoch) {
+        while ((w.fl[j] >> 2) != epoch && polls < ACC_SPIN_LIMIT) {
+          ++polls;
           __builtin_amdgcn_s_sleep(1);
           w.fl[j] = desc.get(idx, w.v[j]);
         }
@@ -171,6 +176,10 @@ ACC_DEV T acc_scan_lookback(const acc_scan_desc<T> &desc, Int64 tile, const T &b
     }
     run = back(run, acc_wave_reduce(c, back));
     if (nearest < ACC_WAVE * ACC_LOOKBACK) break;       /* tile 0 always posts a PREFIX: the walk ends */
+    if (__ballot(polls >= ACC_SPIN_LIMIT) != 0) {
+      if (lane == 0) acc_report(status, ACC_STATUS_SCAN_LOOKBACK);
+      break;
+    }
   }
   const T prefix = run.v;
   if (lane == 0) desc.put(tile, (epoch << 2) | ACC_ST_PREFIX, op(prefix, block_total));
@@ -255,7 +264,8 @@ ACC_DEV void acc_scan_load(Get get, const Int64 base, const Int64 n, T (&x)[ACC_
 template <int HOW, typename T, typename Op, typename Prefetch, typename Out>
 ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op, const T seed, const Int64 tile, const Int64 base,
                            const Int64 n, const Out &out, const acc_scan_desc<T> &desc,
-                           const unsigned int epoch, void *s_wave_raw, T *s_prefix, Prefetch prefetch, const bool outside)
+                           const unsigned int epoch, void *s_wave_raw, T *s_prefix, Prefetch prefetch, const bool outside,
+                           unsigned int *status)
 {
   const bool GUARD = HOW == 2 ? outside : (HOW == 1);
   typedef T V;
@@ -334,7 +344,7 @@ ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op, const T seed,
     if (wave == 0) acc_scan_window_load(desc, tile - 1, lane, win);   /* ahead of the prefetch: results return in issue order */
     prefetch();
     if (wave == 0) {
-      const T p = acc_scan_lookback(desc, tile, S::val(block_total), op_raw, epoch, lane, win);
+      const T p = acc_scan_lookback(desc, tile, S::val(block_total), op_raw, epoch, lane, win, status);
       if (lane == 0) *s_prefix = p;
     }
     __syncthreads();
@@ -424,7 +434,7 @@ ACC_ENTRY(ACC_ENV_PARAMS
           ACC_OUT_ARRAY(arrSum),
           const Int64 shIn_0,
           void *desc0, void *desc1, void *desc2,
-          const unsigned int epoch, const Int64 num_tiles)
+          const unsigned int epoch, const Int64 num_tiles, unsigned int *acc_status)
 {
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
@@ -477,7 +487,7 @@ ACC_ENTRY(ACC_ENV_PARAMS
     auto prefetch = [&]() {};
     const Int64 base = tile_base(tile);
     const bool inside = base >= 0 && base + ACC_TILE <= n;
-    acc_scan_tile<2, T>(cur, op, seed, tile, base, n, out, desc, epoch, (void *)s_wave, &s_prefix, prefetch, !inside);
+    acc_scan_tile<2, T>(cur, op, seed, tile, base, n, out, desc, epoch, (void *)s_wave, &s_prefix, prefetch, !inside, acc_status);
 
   }
 }

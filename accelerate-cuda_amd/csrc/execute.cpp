@@ -181,13 +181,13 @@ int launch_segmented(acc_skel_s *s, int v, Args *args, const acc_array *env, con
   const int64_t min_piece = team_lanes * 64;                          // a piece keeps its team busy for a while
   int64_t split = 1;
   if (nseg * 2 <= room) split = std::max<int64_t>(1, std::min<int64_t>({room / nseg, avg / min_piece, acc::tune("foldseg.max_split", 4096)}));
-  int blk = -1;
+  acc::ScratchRef blk;
   uint64_t part = 0, part_ok = 0;
   if (split > 1) {
     const size_t jobs = (size_t)(nseg * split);
     const size_t ok_off = round256(jobs * s->spec.elt_size);
     ACC_TRY(s->ctx->scratch_acquire(ok_off + jobs * 4, st, acc::SCRATCH_FOLD, &blk));
-    part = reinterpret_cast<uint64_t>(s->ctx->scratch[blk].ptr);
+    part = reinterpret_cast<uint64_t>(blk.ptr);
     part_ok = part + ok_off;
   }
   args->i32(block_team);
@@ -219,7 +219,7 @@ int launch_segmented(acc_skel_s *s, int v, Args *args, const acc_array *env, con
       if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(segmented fold, join)");
     }
   }
-  if (blk >= 0) s->ctx->scratch_release(blk, st);
+  s->ctx->scratch_release(blk, st);
   return rc;
 }
 
@@ -288,7 +288,7 @@ int acc_exec_fold(acc_skel s, const acc_array *env, int32_t in_rank, const int64
     push_ptrs(out, out->ncomp, &args, &aligned);
     args.i64(n);
     args.ptr(0);
-    if (single) args.u32(0);
+    if (single) { args.u32(0); args.ptr(s->ctx->status_dev); }
     return launch(s, v, 1, 0, st, &args);
   }
   if (single) {
@@ -296,34 +296,22 @@ int acc_exec_fold(acc_skel s, const acc_array *env, int32_t in_rank, const int64
     // upper half, and the last block collects them (skel_fold.h).  Every word of the scratch block is only ever
     // written in that form, so words of earlier launches, whatever their grid or element type, read as "not yet".
     const size_t words = (s->spec.elt_size + 3) / 4;
-    int blk = -1;
+    acc::ScratchRef blk;
     ACC_TRY(s->ctx->scratch_acquire((size_t)grid * words * 8, st, acc::SCRATCH_FLAGS, &blk));
-    uint32_t epoch;
-    char *base;
-    {
-      std::lock_guard<std::mutex> lock(s->ctx->mu);
-      acc::ScratchBlock &b = s->ctx->scratch[blk];
-      base = static_cast<char *>(b.ptr);
-      if (b.epoch == 0xFFFFFFFFu) {              // start over from a clean block
-        hipError_t e = hipMemsetAsync(b.ptr, 0, b.bytes, st);
-        if (e != hipSuccess) { b.busy = false; return acc::fail_hip(e, "hipMemsetAsync(fold partials)"); }
-        b.epoch = 0;
-      }
-      epoch = ++b.epoch;
-    }
     push_ptrs(out, out->ncomp, &args, &aligned);
     args.i64(n);
-    args.ptr(reinterpret_cast<uint64_t>(base));
-    args.u32(epoch);
+    args.ptr(reinterpret_cast<uint64_t>(blk.ptr));
+    args.u32(blk.epoch);
+    args.ptr(s->ctx->status_dev);
     int rc = launch(s, v, grid, 0, st, &args);
     s->ctx->scratch_release(blk, st);
     return rc;
   }
   // one partial per block, then a single-block launch folds them: foldRec, Execute.hs:304-315,
   // always exactly one level deep because the first grid never exceeds what is resident
-  int blk = -1;
+  acc::ScratchRef blk;
   ACC_TRY(s->ctx->scratch_acquire((size_t)grid * s->spec.elt_size, st, acc::SCRATCH_FOLD, &blk));
-  const uint64_t partials = reinterpret_cast<uint64_t>(s->ctx->scratch[blk].ptr);
+  const uint64_t partials = reinterpret_cast<uint64_t>(blk.ptr);
   push_ptrs(out, out->ncomp, &args, &aligned);
   args.i64(n);
   args.ptr(partials);
@@ -432,32 +420,35 @@ int scan_core(acc_skel s, const acc_array *env, int64_t n, const acc_array *out,
     args.ptr(reinterpret_cast<uint64_t>(b + off_d2));
     args.u32(nepoch);
     args.i64(tiles);
+    args.ptr(s->ctx->status_dev);
     if (grid < 1 || grid > 0x7fffffffLL) return fail(ACC_ERR_INVALID, "%s: grid of %lld blocks", who, (long long)grid);
     ACC_HIP_TRY(hipModuleLaunchKernel(s->variants[v].fn, static_cast<unsigned>(grid), 1, 1, static_cast<unsigned>(s->spec.block), 1, 1,
                                       0, st, args.data(), nullptr));
     return ACC_OK;
   }
-  int blk = -1;
-  ACC_TRY(s->ctx->scratch_acquire(bytes, st, acc::SCRATCH_SCAN, &blk));
-  uint32_t epoch;
-  char *base;
+  // A scan with more tiles than the device holds at once does not share the device with another such scan: tiles of
+  // one could fill a compute die waiting for a tile that another die, full of waiting tiles of the other, has no
+  // room for.  (Not under `noalloc`: calls through that entry that overlap on one device are excluded as it is.)
+  const bool big = grid > resident(s, v);
+  if (big) ACC_TRY(acc::scan_order_before(s->ctx->device, st));
+  acc::ScratchRef blk;
   {
-    std::lock_guard<std::mutex> lock(s->ctx->mu);
-    acc::ScratchBlock &b = s->ctx->scratch[blk];
-    base = static_cast<char *>(b.ptr);
-    if (b.epoch + 1 >= (1u << 30)) {          // descriptor tags are 30 bits wide: start over from a clean block
-      hipError_t e = hipMemsetAsync(b.ptr, 0, b.bytes, st);
-      if (e != hipSuccess) { b.busy = false; return acc::fail_hip(e, "hipMemsetAsync(scan state)"); }
-      b.epoch = 0;
+    const int arc = s->ctx->scratch_acquire(bytes, st, acc::SCRATCH_SCAN, &blk);
+    if (arc != ACC_OK) {
+      if (big) acc::scan_order_after(s->ctx->device);
+      return arc;
     }
-    epoch = ++b.epoch;
   }
+  const uint32_t epoch = blk.epoch;
+  char *base = static_cast<char *>(blk.ptr);
   args.ptr(reinterpret_cast<uint64_t>(base + off_d0));
   args.ptr(reinterpret_cast<uint64_t>(base + off_d1));
   args.ptr(reinterpret_cast<uint64_t>(base + off_d2));
   args.u32(epoch);
   args.i64(tiles);
+  args.ptr(s->ctx->status_dev);
   const int rc = launch(s, v, grid, 0, st, &args);
+  if (big) acc::scan_order_after(s->ctx->device);
   s->ctx->scratch_release(blk, st);
   return rc;
 }
@@ -524,10 +515,10 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
     largs.i64(n_src);
     const int lv = (al ? 0 : 1) + (s->spec.permute_locked ? 0 : 2);
     ACC_TRY(s->ensure_variant(lv));
-    int lblk = -1;
+    acc::ScratchRef lblk;
     ACC_TRY(s->ctx->scratch_acquire((size_t)ntarget * 4 + 256, st, acc::SCRATCH_LOCKS, &lblk));
-    // the locks start 256 bytes in; the word just before them is the kernel's "a lock never opened" mark
-    largs.ptr(reinterpret_cast<uint64_t>(s->ctx->scratch[lblk].ptr) + 256);
+    // the locks start 256 bytes in
+    largs.ptr(reinterpret_cast<uint64_t>(lblk.ptr) + 256);
     // Lanes in flight are kept to a few per target: every failed attempt on a lock is an atomic that queues in front
     // of the holder's own accesses, and with hundreds of lanes waiting per lock the device's whole atomic rate goes
     // into failed attempts (1000 targets: 12 M updates/s with every compute unit full, 20 times that with 32 lanes
@@ -540,7 +531,7 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
     const int64_t lds_budget = lds_all;
     int32_t lds_bins = 0, lds_copies = 1, win_blocks = 1;
     int64_t lds_need = 0;
-    int dblk = -1;
+    acc::ScratchRef dblk;
     uint64_t dump_val = 0, dump_ok = 0;
     if (lds_table_fits) {
       // windows of equal size; a single window that is small is kept once per wave, within a quarter of the LDS so
@@ -565,7 +556,7 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
       const size_t ok_off = round256((size_t)(lgrid * lds_bins) * esz);
       const int arc = s->ctx->scratch_acquire(ok_off + (size_t)(lgrid * lds_bins) * 4, st, acc::SCRATCH_FOLD, &dblk);
       if (arc != ACC_OK) { s->ctx->scratch_release(lblk, st); return arc; }
-      dump_val = reinterpret_cast<uint64_t>(s->ctx->scratch[dblk].ptr);
+      dump_val = reinterpret_cast<uint64_t>(dblk.ptr);
       dump_ok = dump_val + ok_off;
     }
     largs.i32(lds_bins);
@@ -573,6 +564,7 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
     largs.ptr(dump_val);
     largs.ptr(dump_ok);
     largs.i32(win_blocks);
+    largs.ptr(s->ctx->status_dev);
     int lrc = launch(s, lv, lgrid, lds_bins ? (size_t)lds_need : 0, st, &largs);
     if (lrc == ACC_OK && lds_bins) {
       Args j;
@@ -590,7 +582,7 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
         if (je != hipSuccess) lrc = acc::fail_hip(je, "hipModuleLaunchKernel(permute_join)");
       }
     }
-    if (dblk >= 0) s->ctx->scratch_release(dblk, st);
+    s->ctx->scratch_release(dblk, st);
     s->ctx->scratch_release(lblk, st);
     return lrc;
   }
@@ -630,13 +622,14 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
     if (oe != hipSuccess || bpc < 1) { (void)hipGetLastError(); bpc = 1; }
     const int64_t cus_n = s->ctx->props.multiProcessorCount;
     const int64_t ngrid = acc_launch_grid(n_src, s->elements_per_block(), cus_n, bpc);
-    int nblk = -1;
+    acc::ScratchRef nblk;
     ACC_TRY(s->ctx->scratch_acquire((size_t)(ngrid * nwords) * 4, st, acc::SCRATCH_FOLD, &nblk));
-    const uint64_t ndump = reinterpret_cast<uint64_t>(s->ctx->scratch[nblk].ptr);
+    const uint64_t ndump = reinterpret_cast<uint64_t>(nblk.ptr);
     args.i32(static_cast<int32_t>(ntarget));
     args.i32(1);
     args.ptr(ndump);
     args.ptr(0);
+    args.ptr(s->ctx->status_dev);
     int nrc = launch(s, nv, ngrid, nlds, st, &args);
     if (nrc == ACC_OK) {
       const int64_t columns = (nwords + 255) / 256;
@@ -681,9 +674,9 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
       const int64_t win_blocks = std::max<int64_t>(1, std::min<int64_t>(cus_w * bpc / windows,
                                                                          acc_launch_grid(n_src, s->elements_per_block(), cus_w, bpc)));
       const int64_t wgrid = windows * win_blocks;
-      int wblk = -1;
+      acc::ScratchRef wblk;
       ACC_TRY(s->ctx->scratch_acquire((size_t)(wgrid * wbins) * esz, st, acc::SCRATCH_FOLD, &wblk));
-      const uint64_t wdump = reinterpret_cast<uint64_t>(s->ctx->scratch[wblk].ptr);
+      const uint64_t wdump = reinterpret_cast<uint64_t>(wblk.ptr);
       args.i32(static_cast<int32_t>(wbins));
       args.i32(1);
       args.ptr(wdump);
@@ -749,11 +742,11 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
   const bool table = bins > 0 && grid * bins > acc::tune("permute.atomic_flush_max", 1 << 16);
   const size_t far_bytes = far_rows ? (size_t)(XCD_ROWS * ntarget) * esz : 0;
   const size_t dump_bytes = table ? (size_t)(grid * bins) * esz : 0;
-  int blk = -1;
+  acc::ScratchRef blk;
   uint64_t far = 0, dump = 0;
   if (far_rows || table) {
     ACC_TRY(s->ctx->scratch_acquire(far_bytes + dump_bytes, st, acc::SCRATCH_FOLD, &blk));
-    const uint64_t base = reinterpret_cast<uint64_t>(s->ctx->scratch[blk].ptr);
+    const uint64_t base = reinterpret_cast<uint64_t>(blk.ptr);
     if (far_rows) far = base;
     if (table) dump = base + far_bytes;
   }
@@ -812,7 +805,7 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
       if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(permute_merge)");
     }
   }
-  if (blk >= 0) s->ctx->scratch_release(blk, st);
+  s->ctx->scratch_release(blk, st);
   return rc;
 }
 

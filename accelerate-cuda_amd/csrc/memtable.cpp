@@ -193,6 +193,9 @@ struct acc_memtable_s {
         if (e != hipErrorOutOfMemory) return fail_hip(e, "hipMalloc");
       }
       if (!nursery.empty()) { ACC_TRY(flush_nursery()); continue; }
+      // scratch the skeleton drivers are holding on to but not using (only worth anything against the device's
+      // own limit: the budget counts arrays)
+      if (!over && ctx->scratch_trim() > 0) continue;
       bool any = false;
       ACC_TRY(evict_one(&any));
       if (!any)

@@ -48,7 +48,7 @@ int acc_context_s::make_current() const
   return ACC_OK;
 }
 
-int acc_context_s::scratch_acquire(size_t bytes, hipStream_t stream, int protocol, int *index)
+int acc_context_s::scratch_acquire(size_t bytes, hipStream_t stream, int protocol, acc::ScratchRef *out)
 {
   std::lock_guard<std::mutex> lock(mu);
   if (!scratch_any_stream) {
@@ -72,31 +72,172 @@ int acc_context_s::scratch_acquire(size_t bytes, hipStream_t stream, int protoco
     acc::ScratchBlock b;
     b.bytes = (bytes + 4095) & ~size_t(4095);
     ACC_HIP_TRY(hipMalloc(&b.ptr, b.bytes));
-    hipError_t e = hipEventCreateWithFlags(&b.done, hipEventDisableTiming);
-    if (e != hipSuccess) { (void)hipFree(b.ptr); return acc::fail_hip(e, "hipEventCreateWithFlags"); }
+    // into an entry that a trim has emptied, if there is one (it keeps its event)
+    for (size_t i = 0; i < scratch.size() && pick < 0; ++i)
+      if (!scratch[i].ptr && !scratch[i].busy) pick = static_cast<int>(i);
+    if (pick >= 0) {
+      b.done = scratch[pick].done;
+    } else {
+      hipError_t e = hipEventCreateWithFlags(&b.done, hipEventDisableTiming);
+      if (e != hipSuccess) { (void)hipFree(b.ptr); return acc::fail_hip(e, "hipEventCreateWithFlags"); }
+    }
     b.protocol = protocol;
-    // cleared once, on the stream that first uses it (not meant to be captured into a graph)
-    e = hipMemsetAsync(b.ptr, 0, b.bytes, stream);
-    if (e != hipSuccess) { (void)hipEventDestroy(b.done); (void)hipFree(b.ptr); return acc::fail_hip(e, "hipMemsetAsync(scratch)"); }
-    scratch.push_back(b);
-    pick = static_cast<int>(scratch.size()) - 1;
+    b.dirty = true;         // cleared below, on the stream that first uses it (not meant to be captured into a graph)
+    if (pick >= 0) {
+      scratch[pick] = b;
+    } else {
+      scratch.push_back(b);
+      pick = static_cast<int>(scratch.size()) - 1;
+    }
   }
   acc::ScratchBlock &b = scratch[pick];
+  // tags: the scan's are 30 bits wide, the tagged words' 32
+  const bool tags_out = (protocol == acc::SCRATCH_SCAN && b.epoch + 1 >= (1u << 30)) || (protocol == acc::SCRATCH_FLAGS && b.epoch == 0xFFFFFFFFu);
+  if (b.dirty || tags_out) {
+    hipError_t e = hipMemsetAsync(b.ptr, 0, b.bytes, stream);
+    if (e != hipSuccess) return acc::fail_hip(e, "hipMemsetAsync(scratch)");
+    b.dirty = false;
+    b.epoch = 0;
+  }
+  if (protocol == acc::SCRATCH_SCAN || protocol == acc::SCRATCH_FLAGS) ++b.epoch;
   b.busy = true;
   b.stream = stream;
-  *index = pick;
+  out->index = pick;
+  out->ptr = b.ptr;
+  out->bytes = b.bytes;
+  out->epoch = b.epoch;
   return ACC_OK;
 }
 
-void acc_context_s::scratch_release(int index, hipStream_t stream)
+void acc_context_s::scratch_release(const acc::ScratchRef &ref, hipStream_t stream)
 {
+  if (ref.index < 0) return;
   std::lock_guard<std::mutex> lock(mu);
-  acc::ScratchBlock &b = scratch[index];
+  acc::ScratchBlock &b = scratch[ref.index];
   b.recorded = false;
   if (scratch_multi_stream) b.recorded = (hipEventRecord(b.done, stream) == hipSuccess);
   b.stream = stream;
   b.busy = false;
 }
+
+size_t acc_context_s::scratch_bytes()
+{
+  std::lock_guard<std::mutex> lock(mu);
+  size_t total = 0;
+  for (const acc::ScratchBlock &b : scratch) total += b.ptr ? b.bytes : 0;
+  return total;
+}
+
+// Blocks keep their place in the vector (borrowers hold indices): a freed one stays as an empty entry that matches
+// no request and is filled again by the next allocation that finds no block.
+size_t acc_context_s::scratch_trim()
+{
+  std::lock_guard<std::mutex> lock(mu);
+  size_t freed = 0;
+  for (acc::ScratchBlock &b : scratch) {
+    if (b.busy || !b.ptr) continue;
+    if (hipFree(b.ptr) != hipSuccess) { (void)hipGetLastError(); continue; }      // hipFree waits for the device itself
+    freed += b.bytes;
+    b.ptr = nullptr;
+    b.bytes = 0;
+    b.epoch = 0;
+    b.recorded = false;
+  }
+  // empty entries at the end can go
+  while (!scratch.empty() && !scratch.back().ptr && !scratch.back().busy) {
+    if (scratch.back().done) (void)hipEventDestroy(scratch.back().done);
+    scratch.pop_back();
+  }
+  return freed;
+}
+
+int acc_context_s::check_status(const char *who)
+{
+  if (!status_host) return ACC_OK;
+  uint32_t seen[acc::STATUS_WORDS];
+  bool any = false;
+  for (int k = 0; k < acc::STATUS_WORDS; ++k) {
+    seen[k] = status_host[k];
+    any = any || seen[k] != 0;
+  }
+  if (!any) return ACC_OK;
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    for (int k = 0; k < acc::STATUS_WORDS; ++k) status_host[k] = 0;
+    // a lock that never opened is still set: every lock block is cleared before it is lent again
+    for (acc::ScratchBlock &b : scratch)
+      if (b.protocol == acc::SCRATCH_LOCKS) b.dirty = true;
+  }
+  return fail(ACC_ERR_STUCK, "%s: a kernel gave up waiting (%s%s%s): results of the work enqueued since the last successful synchronisation are not valid",
+              who, seen[acc::STATUS_SCAN_LOOKBACK] ? "scan look-back " : "", seen[acc::STATUS_FOLD_COLLECT] ? "fold partial results " : "",
+              seen[acc::STATUS_PERMUTE_LOCK] ? "permute lock" : "");
+}
+
+namespace acc {
+
+// Two single-pass scans whose grids exceed what is resident at once must not share the device: each compute die
+// hands out the workgroups of a launch in order, but the dies do so independently of one another, so tiles of scan A
+// could fill one die waiting for an A tile that another die, full of waiting tiles of scan B, has no room for (and
+// the other way round).  Within a process such scans are therefore chained, per device: a scan on another stream
+// than the last one waits for an event recorded on that stream just then (everything enqueued there so far, the
+// earlier scan included).  Scans that follow one another on one stream -- the common case -- cost nothing.
+// scan_order_before takes the device's lock and scan_order_after gives it back, so that the launch itself lies
+// between them: a second thread must not record its event before the first one's scan is enqueued.
+struct ScanOrder {
+  std::mutex mu;
+  hipEvent_t ev = nullptr;
+  hipStream_t last = nullptr;
+  bool have_last = false;     // `last` is the stream of the most recent big scan (and still exists)
+  bool ev_pending = false;    // that stream is gone; `ev` was recorded on it before it went
+};
+static ScanOrder g_scan_order[64];
+
+int scan_order_before(int device, hipStream_t stream)
+{
+  if (device < 0 || device >= 64) return ACC_OK;
+  ScanOrder &o = g_scan_order[device];
+  o.mu.lock();
+  hipError_t e = hipSuccess;
+  if (o.have_last && o.last != stream) {
+    if (!o.ev) e = hipEventCreateWithFlags(&o.ev, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipEventRecord(o.ev, o.last);
+    if (e == hipSuccess) e = hipStreamWaitEvent(stream, o.ev, 0);
+  } else if (!o.have_last && o.ev_pending) {
+    e = hipStreamWaitEvent(stream, o.ev, 0);
+  }
+  if (e != hipSuccess) {
+    o.mu.unlock();
+    return fail_hip(e, "ordering of scans on different streams");
+  }
+  o.have_last = true;
+  o.last = stream;
+  o.ev_pending = false;
+  return ACC_OK;
+}
+
+void scan_order_after(int device)
+{
+  if (device < 0 || device >= 64) return;
+  g_scan_order[device].mu.unlock();
+}
+
+// a stream is about to be destroyed: what it still holds of a big scan is remembered by an event
+void scan_order_forget(int device, hipStream_t stream)
+{
+  if (device < 0 || device >= 64) return;
+  ScanOrder &o = g_scan_order[device];
+  std::lock_guard<std::mutex> lock(o.mu);
+  if (!o.have_last || o.last != stream) return;
+  o.have_last = false;
+  o.last = nullptr;
+  hipError_t e = hipSuccess;
+  if (!o.ev) e = hipEventCreateWithFlags(&o.ev, hipEventDisableTiming);
+  if (e == hipSuccess) e = hipEventRecord(o.ev, stream);
+  o.ev_pending = (e == hipSuccess);
+  if (e != hipSuccess) { (void)hipGetLastError(); (void)hipStreamSynchronize(stream); }
+}
+
+}  // namespace acc
 
 extern "C" {
 
@@ -157,6 +298,19 @@ int acc_context_create(int device, acc_context *out)
   if (e == hipSuccess) e = hipSetDevice(device);
   if (e != hipSuccess) { delete ctx; return acc::fail_hip(e, "acc_context_create"); }
   (void)acc::noalloc_setup(device);      // the address of the library's own device array on this device, once
+  {
+    // the status block: host memory the device can write (only ever written when a kernel's bounded wait runs out)
+    void *hp = nullptr, *dp = nullptr;
+    if (hipHostMalloc(&hp, acc::STATUS_WORDS * sizeof(uint32_t), hipHostMallocMapped) == hipSuccess &&
+        hipHostGetDevicePointer(&dp, hp, 0) == hipSuccess) {
+      std::memset(hp, 0, acc::STATUS_WORDS * sizeof(uint32_t));
+      ctx->status_host = static_cast<volatile uint32_t *>(hp);
+      ctx->status_dev = reinterpret_cast<uint64_t>(dp);
+    } else {
+      (void)hipGetLastError();
+      if (hp) (void)hipHostFree(hp);
+    }
+  }
   ctx->arch = ctx->props.gcnArchName;
   const size_t colon = ctx->arch.find(':');
   if (colon != std::string::npos) ctx->arch.resize(colon);
@@ -173,6 +327,7 @@ int acc_context_destroy(acc_context ctx)
     if (b.done) (void)hipEventDestroy(b.done);
     if (b.ptr) (void)hipFree(b.ptr);
   }
+  if (ctx->status_host) (void)hipHostFree(const_cast<uint32_t *>(ctx->status_host));
   delete ctx;
   return ACC_OK;
 }
@@ -189,6 +344,42 @@ int acc_context_sync(acc_context ctx)
   if (!ctx) return fail(ACC_ERR_INVALID, "acc_context_sync: NULL context");
   ACC_TRY(ctx->make_current());
   ACC_HIP_TRY(hipDeviceSynchronize());
+  return ctx->check_status("acc_context_sync");
+}
+
+int acc_context_trim(acc_context ctx, size_t *freed_bytes)
+{
+  if (!ctx) return fail(ACC_ERR_INVALID, "acc_context_trim: NULL context");
+  ACC_TRY(ctx->make_current());
+  const size_t freed = ctx->scratch_trim();
+  if (freed_bytes) *freed_bytes = freed;
+  return ACC_OK;
+}
+
+int acc_context_debug_poke_lock(acc_context ctx, size_t word, uint32_t value)
+{
+  if (!ctx) return fail(ACC_ERR_INVALID, "acc_context_debug_poke_lock: NULL context");
+  ACC_TRY(ctx->make_current());
+  ACC_HIP_TRY(hipDeviceSynchronize());
+  void *at = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    const acc::ScratchBlock *found = nullptr;
+    for (const acc::ScratchBlock &b : ctx->scratch)
+      if (b.protocol == acc::SCRATCH_LOCKS && b.ptr && !b.busy) found = &b;
+    if (!found) return fail(ACC_ERR_NOT_FOUND, "acc_context_debug_poke_lock: the context holds no lock block");
+    // (the locks start 256 bytes into their block)
+    if (256 + (word + 1) * 4 > found->bytes) return fail(ACC_ERR_INVALID, "acc_context_debug_poke_lock: word %zu lies outside the block", word);
+    at = static_cast<char *>(found->ptr) + 256 + word * 4;
+  }
+  ACC_HIP_TRY(hipMemcpy(at, &value, 4, hipMemcpyHostToDevice));
+  return ACC_OK;
+}
+
+int acc_context_scratch_bytes(acc_context ctx, size_t *bytes)
+{
+  if (!ctx || !bytes) return fail(ACC_ERR_INVALID, "acc_context_scratch_bytes: NULL argument");
+  *bytes = ctx->scratch_bytes();
   return ACC_OK;
 }
 
@@ -253,7 +444,12 @@ static int copy(acc_context ctx, void *dst, const void *src, size_t bytes, hipMe
 }
 
 int acc_memcpy_h2d(acc_context c, acc_devptr d, const void *s, size_t n) { return copy(c, reinterpret_cast<void *>(d), s, n, hipMemcpyHostToDevice, nullptr, false); }
-int acc_memcpy_d2h(acc_context c, void *d, acc_devptr s, size_t n) { return copy(c, d, reinterpret_cast<void *>(s), n, hipMemcpyDeviceToHost, nullptr, false); }
+int acc_memcpy_d2h(acc_context c, void *d, acc_devptr s, size_t n)
+{
+  // (a blocking copy to the host is where most callers first look at a result: a kernel's report is returned here too)
+  ACC_TRY(copy(c, d, reinterpret_cast<void *>(s), n, hipMemcpyDeviceToHost, nullptr, false));
+  return c->check_status("acc_memcpy_d2h");
+}
 int acc_memcpy_d2d(acc_context c, acc_devptr d, acc_devptr s, size_t n) { return copy(c, reinterpret_cast<void *>(d), reinterpret_cast<void *>(s), n, hipMemcpyDeviceToDevice, nullptr, false); }
 int acc_memcpy_h2d_async(acc_context c, acc_devptr d, const void *s, size_t n, acc_stream st) { return copy(c, reinterpret_cast<void *>(d), s, n, hipMemcpyHostToDevice, static_cast<hipStream_t>(st), true); }
 int acc_memcpy_d2h_async(acc_context c, void *d, acc_devptr s, size_t n, acc_stream st) { return copy(c, d, reinterpret_cast<void *>(s), n, hipMemcpyDeviceToHost, static_cast<hipStream_t>(st), true); }
@@ -285,6 +481,7 @@ int acc_stream_destroy(acc_context ctx, acc_stream s)
   if (!s) return ACC_OK;
   if (!ctx) return fail(ACC_ERR_INVALID, "acc_stream_destroy: NULL context");
   ACC_TRY(ctx->make_current());
+  acc::scan_order_forget(ctx->device, static_cast<hipStream_t>(s));
   ACC_HIP_TRY(hipStreamDestroy(static_cast<hipStream_t>(s)));
   return ACC_OK;
 }
@@ -294,7 +491,7 @@ int acc_stream_sync(acc_context ctx, acc_stream s)
   if (!ctx) return fail(ACC_ERR_INVALID, "acc_stream_sync: NULL context");
   ACC_TRY(ctx->make_current());
   ACC_HIP_TRY(hipStreamSynchronize(static_cast<hipStream_t>(s)));
-  return ACC_OK;
+  return ctx->check_status("acc_stream_sync");
 }
 
 int acc_stream_wait_event(acc_context ctx, acc_stream s, acc_event e)
@@ -337,7 +534,7 @@ int acc_event_sync(acc_context ctx, acc_event e)
   if (!ctx || !e) return fail(ACC_ERR_INVALID, "acc_event_sync: NULL argument");
   ACC_TRY(ctx->make_current());
   ACC_HIP_TRY(hipEventSynchronize(static_cast<hipEvent_t>(e)));
-  return ACC_OK;
+  return ctx->check_status("acc_event_sync");
 }
 
 int acc_event_query(acc_context ctx, acc_event e, int *done)

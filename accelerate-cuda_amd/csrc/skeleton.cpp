@@ -312,6 +312,7 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
   }
   o << "#define ACC_ENTRY " << *entry << "\n";
   o << "#define ACC_NT_STORE " << tune("nt_store", 1) << "\n";
+  if (tuned("spin_limit")) o << "#define ACC_SPIN_LIMIT " << std::max(0, tune("spin_limit", 1 << 22)) << "\n";
   o << "#include \"acc_hip_device.h\"\n";
   if (!sp.comp_types.empty()) {
     // a tuple element: fields a<c>, component 0 last, so that brace initialisation reads like the tuple

@@ -42,7 +42,7 @@ type Status   = CInt
 -- ---------------------------------------------------------------------------------------------------------
 -- status codes and the exception they become (the reference's CUDAException; State.hs:86-88)
 
-accOK, accErrInvalid, accErrOOM, accErrCompile, accErrNotFound, accErrHIP, accErrUnsupported, accErrIO :: Status
+accOK, accErrInvalid, accErrOOM, accErrCompile, accErrNotFound, accErrHIP, accErrUnsupported, accErrIO, accErrStuck :: Status
 accOK             = #{const ACC_OK}
 accErrInvalid     = #{const ACC_ERR_INVALID}
 accErrOOM         = #{const ACC_ERR_OOM}
@@ -51,6 +51,7 @@ accErrNotFound    = #{const ACC_ERR_NOT_FOUND}
 accErrHIP         = #{const ACC_ERR_HIP}
 accErrUnsupported = #{const ACC_ERR_UNSUPPORTED}
 accErrIO          = #{const ACC_ERR_IO}
+accErrStuck       = #{const ACC_ERR_STUCK}
 
 data HIPException = HIPException Status String
   deriving (Typeable)
@@ -233,6 +234,11 @@ foreign import ccall safe   "acc_context_create"  c_contextCreate  :: CInt -> Pt
 foreign import ccall safe   "acc_context_destroy" c_contextDestroy :: Context -> IO Status
 foreign import ccall safe   "acc_context_device"  c_contextDevice  :: Context -> Ptr CInt -> IO Status
 foreign import ccall safe   "acc_context_sync"    c_contextSync    :: Context -> IO Status
+-- scratch memory of the skeleton drivers: give back what is not in use / how much is held
+foreign import ccall safe   "acc_context_trim"          c_contextTrim         :: Context -> Ptr CSize -> IO Status
+foreign import ccall unsafe "acc_context_scratch_bytes" c_contextScratchBytes :: Context -> Ptr CSize -> IO Status
+-- tests of the failure path only
+foreign import ccall safe   "acc_context_debug_poke_lock" c_contextDebugPokeLock :: Context -> CSize -> Word32 -> IO Status
 
 -- Array/Remote.hs:63-79,191: mallocArray / free / getMemInfo.  ACC_ERR_OOM is the recoverable status
 foreign import ccall safe   "acc_malloc"     c_malloc    :: Context -> CSize -> Ptr DevPtr -> IO Status

@@ -56,6 +56,7 @@ extern "C" {
 #define ACC_ERR_HIP          5   /* any other HIP runtime error */
 #define ACC_ERR_UNSUPPORTED  6   /* valid Accelerate, not implemented by this backend */
 #define ACC_ERR_IO           7   /* kernel cache file trouble (never fatal to a compile) */
+#define ACC_ERR_STUCK        8   /* a kernel gave up a wait for another workgroup: see acc_context_sync */
 
 typedef struct acc_context_s *acc_context;
 typedef struct acc_skel_s    *acc_skel;
@@ -98,6 +99,24 @@ int acc_context_create(int device, acc_context *out);
 int acc_context_destroy(acc_context ctx);
 int acc_context_device(acc_context ctx, int *device);
 int acc_context_sync(acc_context ctx);                 /* CUDA.sync */
+/* Waits inside kernels (a scan tile for its predecessors' descriptors, the collecting workgroup of a fold for the
+ * others' partial results, a lane of a permute for a lock) are bounded.  A wait that runs out ends the kernel
+ * normally, with a wrong result, and leaves a mark that the next synchronising call on the context --
+ * acc_context_sync, acc_stream_sync, acc_event_sync, acc_memcpy_d2h -- returns as ACC_ERR_STUCK, once: nothing
+ * enqueued on the context since its last successful synchronisation is then to be trusted.  The reference has no
+ * counterpart: its kernels do not wait for one another (a lock that never opens hangs it, IndexSpace.hs:285-303). */
+
+/* Scratch memory the skeleton drivers keep per context (fold partials, scan descriptors, permute tables and locks,
+ * Execute.hs:304-315,402-405 allocate theirs per use) is reused between calls and grows to the largest request.
+ * acc_context_trim frees every block that is not in use (it waits for the device first) and reports the bytes
+ * given back; acc_context_scratch_bytes says how much is held.  acc_memtable_malloc trims by itself before it
+ * gives up. */
+int acc_context_trim(acc_context ctx, size_t *freed_bytes);
+int acc_context_scratch_bytes(acc_context ctx, size_t *bytes);
+/* For tests of the failure path only: store `value` in the 32-bit word `word` of the per-target lock block that
+ * the context's last locked permute used (ACC_ERR_NOT_FOUND if there is none, ACC_ERR_INVALID past its end).  A
+ * lock left at 1 makes that permute's bounded wait run out. */
+int acc_context_debug_poke_lock(acc_context ctx, size_t word, uint32_t value);
 
 /* CUDA.mallocArray / free / getMemInfo: Array/Remote.hs:63-79,191 */
 int acc_malloc(acc_context ctx, size_t bytes, acc_devptr *out);

@@ -188,6 +188,53 @@ def test_scratch_pool_with_two_streams(A, ctx, orc):
         assert int(sums[i].get()) == int(xs[i].sum())
 
 
+def test_scans_larger_than_the_device_on_two_streams(A, ctx):
+    """scans of many more tiles than the device holds at once, enqueued alternately on two streams and from two
+    threads: the library keeps such scans from sharing the device (tiles of one must not wait for room that waiting
+    tiles of the other hold), so the results are right and nothing is reported"""
+    import threading
+    I32 = (1, "Int32")
+    scan = ctx.skeleton(A.SKEL_SCANL1, "Int32", env=[I32], get="arrIn0_0[ix]", combine="x + y")
+    tile = scan.info().elements_per_block
+    n = 1500 * tile + 11
+    say("scanl1 of", n, "elements =", n // tile + 1, "tiles, twice on each of two streams")
+    rng = np.random.default_rng(9)
+    xs = [rng.integers(0, 16, n, dtype=np.int32) for _ in range(2)]
+    dxs = [ctx.array(x) for x in xs]
+    outs = [ctx.empty(n, np.int32) for _ in range(2)]
+    streams = [ctx.stream(), ctx.stream()]
+    for rep in range(2):
+        for i in range(2):
+            scan.scan([dxs[i]], n, outs[i], stream=streams[i])
+    ctx.sync()
+    for i in range(2):
+        assert np.array_equal(outs[i].get(), np.cumsum(xs[i], dtype=np.int32))
+    say("the same from two host threads")
+    errors = []
+
+    def work(i):
+        try:
+            for rep in range(3):
+                scan.scan([dxs[i]], n, outs[i], stream=streams[i])
+            A.check(A.lib().acc_stream_sync(ctx.handle, streams[i]))
+        except Exception as e:                          # noqa: BLE001
+            errors.append(e)
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for i in range(2):
+        assert np.array_equal(outs[i].get(), np.cumsum(xs[i], dtype=np.int32))
+    for st in streams:                                # a destroyed stream is not waited on by the next big scan
+        A.check(A.lib().acc_stream_destroy(ctx.handle, st))
+    scan.scan([dxs[0]], n, outs[0])
+    ctx.sync()
+    assert np.array_equal(outs[0].get(), np.cumsum(xs[0], dtype=np.int32))
+    scan.destroy()
+
+
 def test_one_skeleton_launched_from_several_threads(A, ctx):
     """the reference runs every computation in a bound thread of its own (State.hs:84-92):
     threads sharing a context and a skeleton, each on its own stream, misaligned inputs so
