@@ -37,7 +37,7 @@ import numpy as np
 import acchip as A
 
 __all__ = ["Exp", "constant", "cond", "use", "unit", "map", "zipWith", "generate", "backpermute", "transpose", "reverse", "zip_", "unzip", "while_",
-           "fold", "fold1", "foldSeg", "scanl", "scanl1", "scanl_", "scanr", "scanr1", "scanr_", "permute", "ignore",
+           "fold", "fold1", "foldSeg", "fold1Seg", "scanl", "scanl1", "scanl_", "scanr", "scanr1", "scanr_", "permute", "ignore",
            "stencil", "stencil2", "awhile", "run", "run1", "fill", "enumFromN", "take", "drop", "init", "tail", "gather",
            "scatter", "foldAll", "sum_", "product", "maximum", "minimum", "and_", "or_", "all_", "any_", "filter_", "fst", "snd", "lift", "index_if", "fromIntegral", "truncate", "round_", "floor",
            "ceiling", "idiv", "mod", "quot", "rem", "min_", "max_", "sqrt", "exp", "log", "sin", "cos", "tan", "abs_",
@@ -703,17 +703,31 @@ def fold1(f, a, context=None):
     return _fold(f, None, a, True, context)
 
 
-def foldSeg(f, z, a, seg_lengths, context=None):
-    """reduce each segment of a vector; `seg_lengths` is a vector of segment lengths (Int32), turned into
-    offsets by an exclusive scan on the device as the front end does (CUDA.hs:402)"""
+def _foldseg(f, z, a, seg_lengths, seedless, context):
     cx = _context(context, a, seg_lengths)
     offs = scanl(lambda x, y: x + y, constant(0, seg_lengths.ctype), seg_lengths, context=cx)
-    arrays, sig, fr = _assemble(get=a.stream().text, combine=_combine(f, a.ctype).text, seed=Exp.of(z, a.ctype).text)
-    sk = cx.skeleton(A.SKEL_FOLDSEG, _elt(a.ctype), sig, seg_type=seg_lengths.ctype, **fr)
+    arrays, sig, fr = _assemble(get=a.stream().text, combine=_combine(f, a.ctype).text,
+                                seed=None if seedless else Exp.of(z, a.ctype).text)
+    rank = len(a.shape)
+    sk = cx.skeleton(A.SKEL_FOLD1SEG if seedless else A.SKEL_FOLDSEG, _elt(a.ctype), sig, out_rank=rank,
+                     seg_type=seg_lengths.ctype, **fr)
     nseg = seg_lengths.shape[0]
-    out = _empty(cx, (nseg,), a.ctype)
-    cx.launch(arrays + [offs.manifest], [out], lambda i, o, s: sk.foldseg(i[:-1], a.size, i[-1], o[0], stream=s))
-    return Acc((nseg,), a.ctype, manifest=out)
+    out_shape = tuple(a.shape[:-1]) + (nseg,)
+    out = _empty(cx, out_shape, a.ctype)
+    cx.launch(arrays + [offs.manifest], [out], lambda i, o, s: sk.foldseg_nd(i[:-1], a.shape, i[-1], o[0], stream=s))
+    return Acc(out_shape, a.ctype, manifest=out)
+
+
+def foldSeg(f, z, a, seg_lengths, context=None):
+    """reduce each segment of the innermost dimension -- of a vector, or of every outer row of an array of higher
+    rank (Reduction.hs:473-474); `seg_lengths` is a vector of segment lengths (Int32), turned into offsets by an
+    exclusive scan on the device as the front end does (CUDA.hs:402)"""
+    return _foldseg(f, z, a, seg_lengths, False, context)
+
+
+def fold1Seg(f, a, seg_lengths, context=None):
+    """foldSeg without a seed: every segment must be non-empty"""
+    return _foldseg(f, None, a, seg_lengths, True, context)
 
 
 def _scan(kind, f, z, a, context):

@@ -95,7 +95,7 @@ acc_stream_wait_event acc_event_create acc_event_destroy acc_event_record acc_ev
 acc_event_elapsed_ms acc_compile acc_compile_log acc_cache_set_dir acc_cache_dir acc_cache_get_stats
 acc_cache_clear acc_module_load acc_module_unload acc_module_get_function acc_function_attr acc_occupancy
 acc_launch acc_launch_grid acc_skel_create acc_skel_destroy acc_skel_source acc_skel_preview acc_skel_compile_only
-acc_skel_get_info acc_exec_map acc_exec_fold acc_exec_foldseg acc_exec_scan acc_exec_scan_noalloc acc_exec_permute
+acc_skel_get_info acc_exec_map acc_exec_fold acc_exec_foldseg acc_exec_foldseg_nd acc_exec_scan acc_exec_scan_noalloc acc_exec_permute
 acc_exec_stencil acc_exec_stencil2 acc_exec_stencil_iterate acc_memtable_create acc_memtable_destroy
 acc_memtable_malloc acc_memtable_acquire acc_memtable_release acc_memtable_free acc_memtable_insert_unmanaged
 acc_memtable_reclaim acc_memtable_get_stats""".split()
@@ -158,6 +158,7 @@ def lib():
         L.acc_exec_map.argtypes = [C.c_void_p, AP, AP, C.c_void_p]
         L.acc_exec_fold.argtypes = [C.c_void_p, AP, C.c_int32, C.POINTER(C.c_int64), AP, C.c_void_p]
         L.acc_exec_foldseg.argtypes = [C.c_void_p, AP, C.c_int64, AP, AP, C.c_void_p]
+        L.acc_exec_foldseg_nd.argtypes = [C.c_void_p, AP, C.c_int32, C.POINTER(C.c_int64), AP, AP, C.c_void_p]
         L.acc_exec_scan.argtypes = [C.c_void_p, AP, C.c_int64, AP, AP, C.c_void_p]
         L.acc_exec_scan_noalloc.argtypes = [C.c_void_p, AP, C.c_int64, AP, AP, C.c_void_p]
         L.acc_exec_permute.argtypes = [C.c_void_p, AP, C.c_int64, AP, AP, C.c_void_p]
@@ -505,6 +506,10 @@ class Skeleton(object):
 
     def foldseg(self, env, n, offsets, out, stream=None):
         check(lib().acc_exec_foldseg(self.handle, _env(env), n, C.byref(offsets.desc()), C.byref(out.desc()), stream))
+
+    def foldseg_nd(self, env, in_shape, offsets, out, stream=None):
+        sh = (C.c_int64 * len(in_shape))(*in_shape)
+        check(lib().acc_exec_foldseg_nd(self.handle, _env(env), len(in_shape), sh, C.byref(offsets.desc()), C.byref(out.desc()), stream))
 
     def scan(self, env, n, out, total=None, stream=None, noalloc=False):
         o = out if isinstance(out, acc_array) else out.desc()

@@ -49,15 +49,36 @@ static_assert(ACC_CHUNK % (ACC_BLOCK * ACC_VEC) == 0, "chunk must be a whole num
 #else
 #define ACC_FOLDSEG_ENTRY fold1Seg
 #endif
+/* ACC_SEG_OUTER: foldSeg / fold1Seg of an array of rank > 1.  The segment descriptor cuts the innermost dimension of
+ * every outer row alike (CodeGen/Reduction.hs:473-474: base = (seg / num_segments) * innerExtent): segment s of the
+ * flattened result is segment s % seg_per_row of row s / seg_per_row, `seg_inner` elements a row.  What a row holds
+ * beyond its last segment belongs to no segment.                                                                  */
+#ifndef ACC_SEG_OUTER
+#define ACC_SEG_OUTER 0
+#endif
+#if ACC_SEG_OUTER
+#define ACC_SEG_PARAMS const Int64 shIn_0, const ACC_SEG_TYPE *__restrict__ arrSeg_0, const Int64 seg_inner, const Int64 seg_per_row
+#define ACC_SEG_TOTAL shIn_0
+#define ACC_SEG_AT(s)  (((Int64)(s) / seg_per_row) * seg_inner + (Int64)arrSeg_0[(Int64)(s) % seg_per_row])
+#define ACC_SEG_END(s) (((Int64)(s) / seg_per_row) * seg_inner + (Int64)arrSeg_0[(Int64)(s) % seg_per_row + 1])
+#else
 #define ACC_SEG_PARAMS const Int64 shIn_0, const ACC_SEG_TYPE *__restrict__ arrSeg_0
 #define ACC_SEG_TOTAL shIn_0
 #define ACC_SEG_AT(s) ((Int64)arrSeg_0[s])
+#endif
+#endif
+/* where segment s ends: where the next one begins, unless rows have tails */
+#ifndef ACC_SEG_END
+#define ACC_SEG_END(s) ACC_SEG_AT((s) + 1)
 #endif
 
 #define ACC_LOADS (ACC_CHUNK / (ACC_BLOCK * ACC_VEC))   /* vector loads per lane and chunk */
 /* One word of padding per 32 elements of the staged chunk: lanes that fold segments whose starts are a multiple
  * of 32 elements apart (every segment 32, 64, 128 ... long) would otherwise all read the same LDS bank.       */
-#define ACC_PAD(i) ((i) + ((i) >> 5))
+#ifndef ACC_PAD_ON
+#define ACC_PAD_ON 1                                     /* 0: for measuring what the padding is worth */
+#endif
+#define ACC_PAD(i) (ACC_PAD_ON ? ((i) + ((i) >> 5)) : (i))
 #define ACC_EAT 8                                        /* LDS reads kept in flight while folding */
 
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
@@ -85,11 +106,11 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
     /* both ends of the lane's segment are asked for at once (a lane past the last segment asks for the last one's
      * and takes nothing) */
     const Int64 seg_c = acc_min<Int64>(seg, nseg - 1);
-    const Int64 a_c = ACC_SEG_AT(seg_c), b_c = ACC_SEG_AT(seg_c + 1);
+    const Int64 a_c = ACC_SEG_AT(seg_c), b_c = ACC_SEG_END(seg_c);
     const Int64 a = live ? a_c : 0;
     const Int64 b = live ? b_c : 0;
     const Int64 last = acc_min<Int64>(first + ACC_BLOCK, nseg);
-    const Int64 lo = ACC_SEG_AT(first), hi = acc_min<Int64>(ACC_SEG_AT(last), n);
+    const Int64 lo = ACC_SEG_AT(first), hi = acc_min<Int64>(ACC_SEG_END(last - 1), n);
 
     T acc = T();
     bool have = false;
@@ -383,7 +404,7 @@ ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _team)(ACC_ENV_PARAMS
   for (Int64 job = team0; job < nseg * split; job += nteams) {
     const Int64 seg = job / split, part_no = job - seg * split;
     const Int64 sa = ACC_SEG_AT(seg);
-    const Int64 sb = acc_min<Int64>(ACC_SEG_AT(seg + 1), n);
+    const Int64 sb = acc_min<Int64>(ACC_SEG_END(seg), n);
     /* `split` pieces of equal length, whole rounds each so that only a segment's last piece is ragged */
     const Int64 piece = (((sb - sa) + split - 1) / split + round - 1) / round * round;
     const Int64 a = split > 1 ? acc_min<Int64>(sa + part_no * piece, sb) : sa;

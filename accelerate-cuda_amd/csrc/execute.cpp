@@ -283,7 +283,7 @@ int acc_exec_fold(acc_skel s, const acc_array *env, int32_t in_rank, const int64
   const int64_t tile = s->elements_per_block();
   int64_t grid = acc_launch_grid(n, tile, s->ctx->props.multiProcessorCount,
                                  std::min(s->variants[v].blocks_per_cu, acc::tune("fold.blocks_per_cu", 4)));
-  const bool single = acc::tune("fold.single", 1) != 0;       // (the kernel was generated under the same setting)
+  const bool single = s->spec.fold_single;       // as generated into the kernel
   if (grid == 1) {                 // a lone block finishes the job itself
     push_ptrs(out, out->ncomp, &args, &aligned);
     args.i64(n);
@@ -332,17 +332,32 @@ int acc_exec_fold(acc_skel s, const acc_array *env, int32_t in_rank, const int64
   return rc;
 }
 
-int acc_exec_foldseg(acc_skel s, const acc_array *env, int64_t n, const acc_array *offsets, const acc_array *out, acc_stream stream)
+int acc_exec_foldseg_nd(acc_skel s, const acc_array *env, int32_t in_rank, const int64_t *in_shape, const acc_array *offsets,
+                        const acc_array *out, acc_stream stream)
 {
   if (!s) return fail(ACC_ERR_INVALID, "acc_exec_foldseg: NULL skeleton");
   if (!kind_is(s, {ACC_SKEL_FOLDSEG, ACC_SKEL_FOLD1SEG})) return fail(ACC_ERR_INVALID, "acc_exec_foldseg: skeleton is '%s'", s->entry.c_str());
+  const int rank = std::max(1, s->spec.out_rank);        // of the input and of the result alike
+  if (in_rank != rank || !in_shape) return fail(ACC_ERR_INVALID, "%s: input rank %d, kernel was built for %d", s->entry.c_str(), in_rank, rank);
   ACC_TRY(check_out(s, offsets, 1, "segment offsets", 1));
-  ACC_TRY(check_out(s, out, 1, "result"));
-  if (n < 0) return fail(ACC_ERR_INVALID, "%s: negative input extent", s->entry.c_str());
-  // the offsets vector is one longer than the number of segments: Execute.hs:320-324
-  const int64_t nseg = offsets->shape[0] - 1;
-  if (nseg <= 0) return ACC_OK;
-  if (out->shape[0] < nseg) return fail(ACC_ERR_INVALID, "%s: result holds %lld segments, %lld needed", s->entry.c_str(), (long long)out->shape[0], (long long)nseg);
+  ACC_TRY(check_out(s, out, rank, "result"));
+  int64_t rows = 1;
+  for (int d = 0; d < rank; ++d) {
+    if (in_shape[d] < 0) return fail(ACC_ERR_INVALID, "%s: negative input extent", s->entry.c_str());
+    if (d + 1 < rank) rows *= in_shape[d];
+  }
+  const int64_t inner = in_shape[rank - 1];
+  // the offsets vector is one longer than the number of segments of a row: Execute.hs:320-324;
+  // the result is  sh :. number of segments  for an input  sh :. inner
+  const int64_t per_row = offsets->shape[0] - 1;
+  if (per_row <= 0 || rows == 0) return ACC_OK;
+  for (int d = 0; d + 1 < rank; ++d)
+    if (out->shape[d] != in_shape[d]) return fail(ACC_ERR_INVALID, "%s: the result's outer extents differ from the input's", s->entry.c_str());
+  if (out->shape[rank - 1] < per_row)
+    return fail(ACC_ERR_INVALID, "%s: result holds %lld segments a row, %lld needed", s->entry.c_str(), (long long)out->shape[rank - 1], (long long)per_row);
+  if (rank > 1 && out->shape[rank - 1] != per_row)
+    return fail(ACC_ERR_INVALID, "%s: the result's rows must be exactly the %lld segments long", s->entry.c_str(), (long long)per_row);
+  const int64_t nseg = rows * per_row, n = rows * inner;
   Args args;
   bool aligned = true;
   ACC_TRY(push_env(s, env, &args, &aligned));
@@ -350,9 +365,20 @@ int acc_exec_foldseg(acc_skel s, const acc_array *env, int64_t n, const acc_arra
   push_ptrs(out, out->ncomp, &args, &aligned);
   args.i64(n);
   args.ptr(offsets->ptr[0]);
+  if (rank > 1) {        // segments restart in every outer row: CodeGen/Reduction.hs:473-474
+    args.i64(inner);
+    args.i64(per_row);
+  }
   const int v = aligned ? 0 : 1;
   ACC_TRY(s->ensure_variant(v));
   return launch_segmented(s, v, &args, env, out, nseg, n, static_cast<hipStream_t>(stream));
+}
+
+int acc_exec_foldseg(acc_skel s, const acc_array *env, int64_t n, const acc_array *offsets, const acc_array *out, acc_stream stream)
+{
+  if (s && std::max(1, s->spec.out_rank) != 1)
+    return fail(ACC_ERR_INVALID, "acc_exec_foldseg: the kernel was built for rank %d: use acc_exec_foldseg_nd", s->spec.out_rank);
+  return acc_exec_foldseg_nd(s, env, 1, &n, offsets, out, stream);
 }
 
 namespace {

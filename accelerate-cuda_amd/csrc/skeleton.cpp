@@ -212,13 +212,15 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
         *entry = sp.has_seed ? "fold" : "fold1";
         o << "#define ACC_SEG_UNIFORM 1\n";
         o << "#define ACC_TROUNDS " << tune("foldseg.team_rounds", 4) << "\n";
+      if (tuned("foldseg.pad")) o << "#define ACC_PAD_ON " << (tune("foldseg.pad", 1) ? 1 : 0) << "\n";
+        if (tuned("foldseg.pad")) o << "#define ACC_PAD_ON " << (tune("foldseg.pad", 1) ? 1 : 0) << "\n";
         o << "#define ACC_FOLD_RIGHT " << ((sp.flags & ACC_FLAG_FOLD_RIGHT) ? 1 : 0) << "\n";
         o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_CHUNK " << sp.chunk << "\n";
         tmpl = "skel_foldseg.h";
         break;
       }
       *entry = sp.has_seed ? "foldAll" : "fold1All";
-      o << "#define ACC_FOLD_SINGLE " << tune("fold.single", 1) << "\n";
+      o << "#define ACC_FOLD_SINGLE " << (sp.fold_single ? 1 : 0) << "\n";
       o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_UNROLL " << sp.unroll << "\n";
       tmpl = "skel_fold.h";
       break;
@@ -226,7 +228,9 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
     case ACC_SKEL_FOLD1SEG:
       *entry = sp.has_seed ? "foldSeg" : "fold1Seg";
       o << "#define ACC_SEG_TYPE " << sp.seg_type << "\n";
+      if (sp.out_rank >= 2) o << "#define ACC_SEG_OUTER 1\n";      // the segments of every outer row: Reduction.hs:473-474
       o << "#define ACC_TROUNDS " << tune("foldseg.team_rounds", 4) << "\n";
+      if (tuned("foldseg.pad")) o << "#define ACC_PAD_ON " << (tune("foldseg.pad", 1) ? 1 : 0) << "\n";
       o << "#define ACC_FOLD_RIGHT " << ((sp.flags & ACC_FLAG_FOLD_RIGHT) ? 1 : 0) << "\n";
       o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_CHUNK " << sp.chunk << "\n";
       tmpl = "skel_foldseg.h";
@@ -457,6 +461,7 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
     case ACC_SKEL_FOLD: case ACC_SKEL_FOLD1:
       sp->block = tune("fold.block", 256);
       sp->unroll = tune("fold.unroll", 4);
+      sp->fold_single = tune("fold.single", 1) != 0;
       if (sp->out_rank > 0) {
         sp->block = tune("foldseg.block", 256);
         sp->chunk = segmented_chunk(*sp);
@@ -597,7 +602,7 @@ int acc_skel_s::ensure_variant(int v)
   acc::SkelSpec spec = acc::spec_of_variant(this->spec, v);
   std::string entry_name;
   ACC_TRY(acc::generate_source(spec, (v & 1) == 0, &entry_name, &var.source));
-  entry = entry_name;
+  if (entry.empty()) entry = entry_name;      // the same for every variant; set once, before the instance is shared
   std::vector<std::string> opts = acc::compile_options(spec);
   std::vector<const char *> optp;
   for (const std::string &s : opts) optp.push_back(s.c_str());
@@ -606,17 +611,17 @@ int acc_skel_s::ensure_variant(int v)
   ACC_TRY(acc_compile(ctx, nullptr, var.source.c_str(), optp.data(), static_cast<int>(optp.size()), &code, &size));
   ACC_TRY(ctx->make_current());
   ACC_HIP_TRY(hipModuleLoadData(&var.module, code));
-  hipError_t e = hipModuleGetFunction(&var.fn, var.module, entry.c_str());
+  hipError_t e = hipModuleGetFunction(&var.fn, var.module, entry_name.c_str());
   if (e != hipSuccess) {
     (void)hipModuleUnload(var.module);
     var.module = nullptr;
-    return acc::fail_hip(e, ("hipModuleGetFunction(" + entry + ")").c_str());
+    return acc::fail_hip(e, ("hipModuleGetFunction(" + entry_name + ")").c_str());
   }
   const bool segmented = spec.kind == ACC_SKEL_FOLDSEG || spec.kind == ACC_SKEL_FOLD1SEG ||
                          ((spec.kind == ACC_SKEL_FOLD || spec.kind == ACC_SKEL_FOLD1) && spec.out_rank > 0);
   const bool two_kernels = ((spec.kind == ACC_SKEL_FOLD || spec.kind == ACC_SKEL_FOLD1) && spec.out_rank == 0) ||
                            spec.kind == ACC_SKEL_PERMUTE || segmented;
-  const std::string second = entry + (spec.kind == ACC_SKEL_PERMUTE ? (spec.permute_locked ? "_join" : "_merge") : segmented ? "_team" : "_finish");
+  const std::string second = entry_name + (spec.kind == ACC_SKEL_PERMUTE ? (spec.permute_locked ? "_join" : "_merge") : segmented ? "_team" : "_finish");
   if (two_kernels) {
     e = hipModuleGetFunction(&var.fn_finish, var.module, second.c_str());
     if (e != hipSuccess) {
@@ -626,7 +631,7 @@ int acc_skel_s::ensure_variant(int v)
     }
   }
   if ((spec.kind == ACC_SKEL_PERMUTE && !spec.permute_locked) || segmented) {
-    const std::string third = entry + (segmented ? "_join" : "_fill");
+    const std::string third = entry_name + (segmented ? "_join" : "_fill");
     e = hipModuleGetFunction(&var.fn_fill, var.module, third.c_str());
     if (e != hipSuccess) {
       (void)hipModuleUnload(var.module);
@@ -635,7 +640,7 @@ int acc_skel_s::ensure_variant(int v)
     }
   }
   if ((spec.kind == ACC_SKEL_FOLD || spec.kind == ACC_SKEL_FOLD1) && spec.out_rank > 0) {
-    const std::string rows = entry + "_rows";
+    const std::string rows = entry_name + "_rows";
     e = hipModuleGetFunction(&var.fn_rows, var.module, rows.c_str());
     if (e != hipSuccess) {
       (void)hipModuleUnload(var.module);

@@ -40,6 +40,7 @@ struct SkelSpec {
   int tile_z = 1;                       // rank-3 stencils: result planes per strip
   // tuning
   int block = 256, unroll = 4, rows = 4, chunk = 4096;
+  bool fold_single = true;              // foldAll in one launch (the last workgroup collects), as generated into the kernel
   int scan_rows_fallback = 8;
   int scan_desc_stride = 16;            // 8-byte words between the tile descriptors of a scan, as generated into the kernel
   bool scan_shape_open = false;         // a scan whose tile shape the first build may still change (by its register count)

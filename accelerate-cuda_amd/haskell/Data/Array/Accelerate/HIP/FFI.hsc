@@ -297,6 +297,7 @@ foreign import ccall safe   "acc_skel_get_info"     c_skelGetInfo     :: Skel ->
 foreign import ccall safe   "acc_exec_map"             c_execMap            :: Skel -> Ptr AccArray -> Ptr AccArray -> Stream -> IO Status
 foreign import ccall safe   "acc_exec_fold"            c_execFold           :: Skel -> Ptr AccArray -> Int32 -> Ptr Int64 -> Ptr AccArray -> Stream -> IO Status
 foreign import ccall safe   "acc_exec_foldseg"         c_execFoldseg        :: Skel -> Ptr AccArray -> Int64 -> Ptr AccArray -> Ptr AccArray -> Stream -> IO Status
+foreign import ccall safe   "acc_exec_foldseg_nd"      c_execFoldsegNd      :: Skel -> Ptr AccArray -> Int32 -> Ptr Int64 -> Ptr AccArray -> Ptr AccArray -> Stream -> IO Status
 foreign import ccall safe   "acc_exec_scan"            c_execScan           :: Skel -> Ptr AccArray -> Int64 -> Ptr AccArray -> Ptr AccArray -> Stream -> IO Status
 foreign import ccall safe   "acc_exec_scan_noalloc"    c_execScanNoalloc    :: Skel -> Ptr AccArray -> Int64 -> Ptr AccArray -> Ptr AccArray -> Stream -> IO Status
 foreign import ccall safe   "acc_exec_permute"         c_execPermute        :: Skel -> Ptr AccArray -> Int64 -> Ptr AccArray -> Ptr AccArray -> Stream -> IO Status

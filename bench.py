@@ -297,6 +297,30 @@ def main():
         mag = abs(Amat) @ np.abs(xv.astype(np.float64))
         assert np.all(np.abs(y.get() - truth) <= 1e-4 * np.maximum(np.abs(truth), 1e-3 * mag) + 1e-30), "smvm mismatch"
 
+    # ---------------------------------------------------------------- not a configuration: fold along rows of 64
+    # (only when named: the rows of a rank-2 array are segments whose starts lie a multiple of 32 elements apart, the
+    # case the padding of the staged chunk in LDS is there for; ACC_HIP_TUNE=foldseg.pad=0 runs it without)
+    if "foldrows64" in only:
+        log("fold (+) along the rows of a 2^20 x 64 Float32 array ...")
+        rows, width = 1 << 20, 64
+        m = wl.dot_inputs(rows * width)[0].reshape(rows, width)
+        dms = [ctx.array(m) for _ in range(S)]
+        env_s = [envs(d) for d in dms]
+        rs = [ctx.empty(rows, np.float32) for _ in range(S)]
+        frow = ctx.skeleton(A.SKEL_FOLD, "float", env=[(2, "float")], out_rank=1, get=rd(0), combine="x + y", seed="0.0f")
+        rds = [r.desc() for r in rs]
+        sh2 = (C.c_int64 * 2)(rows, width)
+
+        def step(i):
+            return lambda: A.check(L.acc_exec_fold(frow.handle, env_s[i], 2, sh2, C.byref(rds[i]), stream))
+        w, e = T.run([step(i) for i in range(S)])
+        want_rows = m[:, 0].copy()
+        for k in range(1, width):
+            want_rows += m[:, k]                      # left to right in Float32, as the kernel folds a row
+        assert np.array_equal(rs[S - 1].get(), want_rows), "row sums mismatch"
+        sk["foldrows64"] = result("fold (+) rows of 64 Float32", w, e, 1, rows * width * 4 + rows * 4, rows * width)
+        del dms, env_s, rs, m
+
     if headline is None:     # --only without scan: report whatever ran first
         k0 = sorted(sk)[0]
         headline = dict(sk[k0], wall_ms=sk[k0]["ms_per_step"], event_ms=sk[k0]["event_ms_per_step"])

@@ -365,6 +365,13 @@ int acc_exec_fold(acc_skel s, const acc_array *env, int32_t in_rank, const int64
  * elements.                                                                  */
 int acc_exec_foldseg(acc_skel s, const acc_array *env, int64_t n, const acc_array *offsets,
                      const acc_array *out, acc_stream stream);
+/* The same for an input of any rank (foldSegOp (sh :. _) (Z :. sz) = executeOp (sh :. sz - 1), Execute.hs:323-324):
+ * the descriptor segments the innermost dimension of EVERY outer row, segment s of a row being
+ * [offsets[s], offsets[s+1]) within it (CodeGen/Reduction.hs:473-474,485-486); what a row holds beyond its last
+ * segment is not read into any result.  in_rank must equal the desc's out_rank (0 and 1 both mean a vector);
+ * out has the input's outer extents and exactly nseg elements a row (a vector may be longer).                  */
+int acc_exec_foldseg_nd(acc_skel s, const acc_array *env, int32_t in_rank, const int64_t *in_shape,
+                        const acc_array *offsets, const acc_array *out, acc_stream stream);
 
 /* scans: scanOp / scan1Op / scan'Op / scanCore, Execute.hs:328-392.
  *   scanl, scanr    : out holds n+1 elements, `total` is ignored (may be NULL)

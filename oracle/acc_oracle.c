@@ -228,6 +228,35 @@ DEF_FOLDSEG(int32_t, i32, 0)
 DEF_FOLDSEG(float,   f32, 1)
 DEF_FOLDSEG(double,  f64, 1)
 
+/* foldSeg / fold1Seg of an array of rank > 1 (`outer` rows of `inner`
+ * elements): the descriptor segments the innermost dimension of every row
+ * alike, segment s of row r being [r*inner + off[s], r*inner + off[s+1])
+ * (CodeGen/Reduction.hs:473-474,485-486: base = (seg / num_segments) *
+ * innerExtent, start = base + off[s], end = base + off[s+1]); the result is
+ * outer x nseg, row-major (Execute.hs:323-324).  What a row holds beyond
+ * off[nseg] belongs to no segment.                                          */
+#define DEF_FOLDSEG_ND(T, SUF, ISF)                                            \
+int orc_foldseg_nd_##SUF(int op, int has_seed, T z, const T *x, int64_t outer, \
+                         int64_t inner, const int32_t *off, int64_t nseg,      \
+                         int dir, T *out)                                      \
+{                                                                              \
+  if (!op_valid(op, ISF) || nseg < 0 || outer < 0 || inner < 0)                \
+    return ORC_ERR_INVALID;                                                    \
+  for (int64_t r = 0; r < outer; ++r)                                          \
+    for (int64_t s = 0; s < nseg; ++s) {                                       \
+      int64_t a = off[s], b = off[s + 1];                                      \
+      if (b < a || a < 0 || b > inner) return ORC_ERR_INVALID;                 \
+      int rc = fold_range_##SUF(op, has_seed, z, x + r * inner + a, b - a,     \
+                                dir, out + r * nseg + s);                      \
+      if (rc) return rc;                                                       \
+    }                                                                          \
+  return ORC_OK;                                                               \
+}
+
+DEF_FOLDSEG_ND(int32_t, i32, 0)
+DEF_FOLDSEG_ND(float,   f32, 1)
+DEF_FOLDSEG_ND(double,  f64, 1)
+
 /* ------------------------------------------------------------------------ */
 /* The two fused Float32 configurations, written out so that no temporary
  * array is needed at full size.                                             */

@@ -102,6 +102,22 @@ def foldseg(op, x, offsets, seed=None, direction=DIR_LEFT):
     return out
 
 
+def foldseg_nd(op, x, offsets, seed=None, direction=DIR_LEFT):
+    """foldSeg / fold1Seg along the innermost dimension of every outer row of `x` (rank >= 1)"""
+    x = _c(x)
+    offsets = _c(offsets, np.int32)
+    suf, ct = _SUF[x.dtype]
+    nseg = offsets.size - 1
+    inner = x.shape[-1]
+    outer = int(np.prod(x.shape[:-1], dtype=np.int64))
+    out = np.empty(x.shape[:-1] + (max(nseg, 0),), dtype=x.dtype)
+    rc = getattr(lib(), "orc_foldseg_nd_" + suf)(
+        C.c_int(op), C.c_int(seed is not None), ct(0 if seed is None else seed), _p(x), C.c_int64(outer), C.c_int64(inner),
+        _p(offsets), C.c_int64(nseg), C.c_int(direction), _p(out))
+    _check(rc, "foldSeg")
+    return out
+
+
 def dot_f32(x, y, direction=DIR_LEFT):
     x = _c(x, np.float32)
     y = _c(y, np.float32)

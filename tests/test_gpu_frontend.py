@@ -152,6 +152,28 @@ def test_smvm_by_foldseg(acc):
     assert np.array_equal(y, ref)
 
 
+def test_foldseg_of_a_matrix_and_fold1seg(acc):
+    """foldSeg over the rows of a matrix (the same segments in every row, Reduction.hs:473-474) fused with its
+    producer, and fold1Seg"""
+    rng = np.random.default_rng(17)
+    m = rng.integers(-50, 50, (301, 64)).astype(np.int32)
+    lens = np.array([5, 0, 20, 1, 30], np.int32)              # 56 of the 64 columns
+    offs = np.concatenate([[0], np.cumsum(lens)])
+    got = acc.run(acc.foldSeg(add, 10, acc.map(lambda v: v * 2, acc.use(m)), acc.use(lens)))
+    ref = np.stack([(2 * m[:, offs[k]:offs[k + 1]]).sum(axis=1) + 10 for k in range(5)], axis=1).astype(np.int32)
+    assert got.shape == (301, 5) and np.array_equal(got, ref)
+    lens1 = np.array([5, 2, 20, 1, 30], np.int32)
+    offs1 = np.concatenate([[0], np.cumsum(lens1)])
+    got = acc.run(acc.fold1Seg(add, acc.use(m), acc.use(lens1)))
+    ref = np.stack([m[:, offs1[k]:offs1[k + 1]].sum(axis=1) for k in range(5)], axis=1).astype(np.int32)
+    assert np.array_equal(got, ref)
+    v = rng.integers(-50, 50, 1000).astype(np.int32)
+    lv = np.array([100, 0, 900], np.int32)
+    assert np.array_equal(acc.run(acc.fold1Seg(add, acc.use(v), acc.use(np.array([100, 900], np.int32)))),
+                          np.array([v[:100].sum(), v[100:].sum()], np.int32))
+    assert np.array_equal(acc.run(acc.foldSeg(add, 0, acc.use(v), acc.use(lv))), np.array([v[:100].sum(), 0, v[100:].sum()], np.int32))
+
+
 def test_index_transformations(acc):
     rng = np.random.default_rng(8)
     m = rng.integers(0, 1000, (37, 101)).astype(np.int32)

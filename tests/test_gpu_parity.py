@@ -591,6 +591,68 @@ def test_foldseg_long_segments_keep_index_order(A, ctx, orc):
         assert np.array_equal(out.get(), orc.foldseg(orc.OP_MAX, x1, offs1))
 
 
+def test_foldseg_of_arrays_of_higher_rank(A, ctx, orc):
+    """the descriptor segments the innermost dimension of every outer row alike (Reduction.hs:473-474): short
+    segments (a lane each), long ones (a wave, a workgroup, several workgroups each), empty ones, a tail of every
+    row that belongs to no segment, an operator that is not commutative, rank 2 and rank 3, a misaligned input"""
+    I2, I3 = (2, "Int32"), (3, "Int32")
+    add = ctx.skeleton(A.SKEL_FOLDSEG, "Int32", env=[I2], out_rank=2, get="arrIn0_0[ix]", combine="x + y", seed="3")
+    first = ctx.skeleton(A.SKEL_FOLDSEG, "Int32", env=[I2], out_rank=2, get="arrIn0_0[ix]", combine="x != 0 ? x : y", seed="-7")
+    last_r = ctx.skeleton(A.SKEL_FOLDSEG, "Int32", env=[I2], out_rank=2, get="arrIn0_0[ix]", combine="y != 0 ? y : x", seed="0",
+                          flags=A.FLAG_FOLD_RIGHT)
+    mx = ctx.skeleton(A.SKEL_FOLD1SEG, "Int32", env=[I2], out_rank=2, get="arrIn0_0[ix]", combine="acc_max(x, y)")
+    add3 = ctx.skeleton(A.SKEL_FOLDSEG, "Int32", env=[I3], out_rank=3, get="arrIn0_0[ix]", combine="x + y", seed="0")
+    for rows, nseg, mean, tail in [(1, 50, 4, 0), (7, 1, 9, 2), (300, 40, 6, 5), (4001, 33, 20, 0), (25, 12, 400, 17),
+                                   (6, 5, 30000, 1), (3, 1, 700000, 3), (2000, 3, 0, 4)]:
+        say("foldSeg of", rows, "rows x", nseg, "segments of mean", mean, "and a tail of", tail)
+        lens = rng.poisson(mean, nseg).astype(np.int64)
+        if nseg > 2:
+            lens[::5] = 0
+        offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        inner = int(offs[-1]) + tail
+        x = rng.integers(-3, 4, (rows, inner), dtype=np.int32)
+        x[rng.random((rows, inner)) < 0.8] = 0
+        dx, doffs, out = ctx.array(x), ctx.array(offs), ctx.array(np.full((rows, nseg), 12345, np.int32))
+        add.foldseg_nd([dx], x.shape, doffs, out)
+        assert np.array_equal(out.get(), orc.foldseg_nd(orc.OP_ADD, x, offs, seed=3))
+        exp_first, exp_last = np.full((rows, nseg), -7, np.int32), np.zeros((rows, nseg), np.int32)
+        for r in range(min(rows, 64)):
+            for k in range(nseg):
+                nz = np.flatnonzero(x[r, offs[k]:offs[k + 1]])
+                if nz.size:
+                    exp_first[r, k] = x[r, offs[k] + nz[0]]
+                    exp_last[r, k] = x[r, offs[k] + nz[-1]]
+        first.foldseg_nd([dx], x.shape, doffs, out)
+        assert np.array_equal(out.get()[:64], exp_first[:64])
+        last_r.foldseg_nd([dx], x.shape, doffs, out)
+        assert np.array_equal(out.get()[:64], exp_last[:64])
+        if mean > 0:
+            lens1 = np.maximum(lens, 1)
+            offs1 = np.concatenate([[0], np.cumsum(lens1)]).astype(np.int32)
+            x1 = rng.integers(-1000, 1000, (rows, int(offs1[-1]) + tail), dtype=np.int32)
+            mx.foldseg_nd([ctx.array(x1)], x1.shape, ctx.array(offs1), out)
+            assert np.array_equal(out.get(), orc.foldseg_nd(orc.OP_MAX, x1, offs1))
+    say("rank 3, and an input that starts 4 bytes off a 16-byte boundary")
+    lens = np.array([2, 0, 7, 1, 30, 0, 3], np.int64)
+    offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    x = rng.integers(-100, 100, (5, 9, 45), dtype=np.int32)
+    out3 = ctx.empty((5, 9, 7), np.int32)
+    add3.foldseg_nd([ctx.array(x)], x.shape, ctx.array(offs), out3)
+    assert np.array_equal(out3.get(), orc.foldseg_nd(orc.OP_ADD, x, offs, seed=0))
+    buf = ctx.array(np.concatenate([[0], x.reshape(-1)]).astype(np.int32))
+    add3.foldseg_nd([buf.desc(shape=x.shape, offset_elems=1)], x.shape, ctx.array(offs), out3)
+    assert np.array_equal(out3.get(), orc.foldseg_nd(orc.OP_ADD, x, offs, seed=0))
+    say("wrong use")
+    with pytest.raises(A.AccError) as e:                     # the rank-1 entry on a rank-2 kernel
+        add.foldseg([ctx.array(x.reshape(-1))], x.size, ctx.array(offs), ctx.empty(7, np.int32))
+    assert e.value.code == A.ERR_INVALID
+    with pytest.raises(A.AccError) as e:                     # a result whose rows are not the segments
+        add.foldseg_nd([ctx.array(x.reshape(45, 45))], (45, 45), ctx.array(offs), ctx.empty((45, 8), np.int32))
+    assert e.value.code == A.ERR_INVALID
+    for s_ in (add, first, last_r, mx, add3):
+        s_.destroy()
+
+
 def test_fold_along_the_innermost_dimension_at_every_shape(A, ctx):
     """rows of 1 to 2^20 elements, 2^20 rows to one: a lane, a wave, a workgroup or several workgroups per row"""
     add = ctx.skeleton(A.SKEL_FOLD, "Int32", env=[(2, "Int32")], out_rank=1, get="arrIn0_0[ix]", combine="x + y", seed="5")

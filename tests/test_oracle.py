@@ -211,6 +211,51 @@ def test_foldseg_vs_numpy_and_empty_segments(orc):
     assert orc.foldseg(orc.OP_MAX, vi, offs, seed=-999).tolist() == ps
 
 
+def test_foldseg_of_higher_rank_restarts_in_every_row(orc):
+    """Reduction.hs:473-474: the descriptor cuts the innermost dimension of every outer row alike; pinned by numpy
+    slicing per row (not by the oracle's own index arithmetic), a row tail that belongs to no segment, empty
+    segments, a non-commutative operator against pure Python, and the rank-1 case against foldseg itself"""
+    rng = np.random.default_rng(21)
+    lens = np.array([3, 0, 5, 1, 0, 4], np.int32)
+    offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)            # 13 of the 16 elements of a row
+    x = rng.integers(-50, 50, (4, 3, 16)).astype(np.int32)
+    got = orc.foldseg_nd(orc.OP_ADD, x, offs, seed=7)
+    assert got.shape == (4, 3, 6)
+    for i in range(4):
+        for j in range(3):
+            for s_ in range(6):
+                assert got[i, j, s_] == x[i, j, offs[s_]:offs[s_ + 1]].sum() + 7
+    # the tail x[..., 13:] reaches no result: changing it changes nothing
+    y = x.copy()
+    y[..., 13:] += 1000
+    assert np.array_equal(orc.foldseg_nd(orc.OP_ADD, y, offs, seed=7), got)
+    # segments of length 1 over the whole row without a seed: the array itself
+    ones = np.arange(17, dtype=np.int32)
+    assert np.array_equal(orc.foldseg_nd(orc.OP_ADD, x, ones), x)
+    # a non-commutative operator: `first` keeps the segment's first element (the seed comes second), `last` the seed
+    xf = rng.random((5, 16)).astype(np.float32)
+    first = orc.foldseg_nd(orc.OP_FIRST, xf, offs, seed=-1.0)
+    last = orc.foldseg_nd(orc.OP_LAST, xf, offs, seed=-1.0)
+    for r in range(5):
+        for s_ in range(6):
+            assert first[r, s_] == (xf[r, offs[s_]] if lens[s_] else np.float32(-1.0))
+            assert last[r, s_] == np.float32(-1.0)
+    # composition of affine maps over Z/2^16 (associative, not commutative) against pure Python, both directions
+    xa = rng.integers(0, 1 << 31, (3, 16)).astype(np.int32)
+    z = int((5 << 16) | 9)
+    for d, pf in ((orc.DIR_LEFT, pyref.fold_left), (orc.DIR_RIGHT, pyref.fold_right)):
+        ps = [pyref.foldseg(pf, pyref.affine16, z, row.tolist(), offs.tolist()) for row in xa]
+        got = orc.foldseg_nd(orc.OP_AFFINE16, xa, offs, seed=z, direction=d)
+        assert (got.astype(np.int64) & 0xFFFFFFFF).tolist() == ps             # the same 32 bits, read as unsigned
+    # rank 1 is foldseg
+    v = x.reshape(-1)[:16]
+    assert np.array_equal(orc.foldseg_nd(orc.OP_MAX, v, offs, seed=-999), orc.foldseg(orc.OP_MAX, v, offs, seed=-999))
+    with pytest.raises(orc.OracleError):                                      # fold1Seg: an empty segment in some row
+        orc.foldseg_nd(orc.OP_ADD, x, offs)
+    with pytest.raises(orc.OracleError):                                      # a descriptor that runs past the row
+        orc.foldseg_nd(orc.OP_ADD, x[..., :12], offs, seed=0)
+
+
 def test_smvm_vs_scipy(orc):
     nrows, ncols = 300, 128
     vals, cols, offs, x = _csr(nrows, ncols, 12)
