@@ -429,6 +429,8 @@ class _Resident(object):
             cx.live[self.key] = cx.live.get(self.key, 0) + 1
 
     def get(self):
+        if self.cx.loop is not None:
+            raise _HostReadInLoop()          # an iteration enqueued ahead cannot wait for the host
         if self.ready is not None:
             A.check(A.lib().acc_event_sync(self.cx.ctx.handle, self.ready))
         d = self.cx.table.acquire(self.host)
@@ -450,6 +452,16 @@ class _Resident(object):
                         cx.table.free(self.host)
         except Exception:
             pass
+
+
+class _HostReadInLoop(Exception):
+    """raised where the body or the predicate of an `awhile` whose iterations are being enqueued ahead asks for a
+    value on the host (`the`, a nested loop): that loop then goes on one iteration at a time"""
+
+
+class _Loop(object):
+    def __init__(self, stream, guard):
+        self.stream, self.guard = stream, guard
 
 
 class Cancelled(Exception):
@@ -475,6 +487,7 @@ class Context(object):
         self.skeletons = {}
         self.streams, self.turn, self.events = [], 0, []
         self.lock = threading.RLock()      # one host thread at a time evaluates in a context (CUDA.hs:251-252)
+        self.loop, self.guard = None, None # the `awhile` being enqueued ahead, if any, and the context's loop guard
 
     @classmethod
     def default(cls):
@@ -486,6 +499,9 @@ class Context(object):
         key = (kind, elt, tuple((r, tuple(t) if isinstance(t, list) else t) for r, t in env),
                tuple(sorted((k, str(v)) for k, v in kw.items())))
         with self.lock:
+            if self.loop is not None:          # kernels that look at the loop's guard: instances of their own
+                kw = dict(kw, flags=kw.get("flags", 0) | A.FLAG_GUARDED)
+                key = key + ("guarded",)
             sk = self.skeletons.get(key)
             if sk is None:
                 sk = self.ctx.skeleton(kind, elt, env=env, **kw)
@@ -495,6 +511,8 @@ class Context(object):
     N_STREAMS = 4
 
     def _stream_for(self, inputs):
+        if self.loop is not None:
+            return self.loop.stream               # everything of a loop enqueued ahead is ordered by one stream
         for m in inputs:
             if m.stream is not None:
                 return m.stream
@@ -942,15 +960,8 @@ def filter_(p, a, context=None):
     return out, count
 
 
-def awhile(p, f, a, context=None, limit=None):
-    """iterate the array function `f` from `a` while the scalar array `p(a)` holds a non-zero value
-    (Execute.hs:236-244).  `a` is an Acc or a tuple of them; every iterate is made manifest, and the
-    flag is the one value read back per iteration."""
-    cx = _context(context, *(a if isinstance(a, tuple) else (a,)))
-    tup = isinstance(a, tuple)
-    force = lambda v: tuple(_force(x, cx) for x in v) if tup else _force(v, cx)
-    a = force(a)
-    n = 0
+def _awhile_stepwise(cx, p, f, a, tup, force, limit, n):
+    """one iteration at a time, the flag read back before every one (as Execute.hs:236-244 does)"""
     while limit is None or n < limit:
         flag = p(*a) if tup else p(a)
         if flag.shape != ():
@@ -960,6 +971,67 @@ def awhile(p, f, a, context=None, limit=None):
         a = force(f(*a) if tup else f(a))
         n += 1
     return a
+
+
+def awhile(p, f, a, context=None, limit=None, ahead=8):
+    """iterate the array function `f` from `a` while the scalar array `p(a)` holds a non-zero value
+    (Execute.hs:236-244).  `a` is an Acc or a tuple of them; every iterate is made manifest.
+
+    The reference reads the flag back before every iteration.  Here `ahead` iterations are enqueued at a time, on one
+    stream, under a guard in device memory: a one-lane kernel behind each predicate folds its flag into the guard,
+    every kernel of the loop looks at the guard and does nothing once it is down, and the host reads the guard --
+    whether the loop still runs and how many iterations were taken -- once per batch.  A predicate or body that
+    needs a value on the host itself (`the`, `filter_`, a loop of its own) makes the loop fall back to one
+    iteration at a time."""
+    cx = _context(context, *(a if isinstance(a, tuple) else (a,)))
+    tup = isinstance(a, tuple)
+    force = lambda v: tuple(_force(x, cx) for x in v) if tup else _force(v, cx)
+    a = force(a)
+    with cx.lock:
+        if cx.loop is not None:
+            raise _HostReadInLoop()              # a loop inside a loop: the outer one goes stepwise, this one ahead
+        if ahead < 2:
+            return _awhile_stepwise(cx, p, f, a, tup, force, limit, 0)
+        stream = cx._stream_for([m for x in (a if tup else (a,)) for m in
+                                 (x.manifest.comps if isinstance(x.manifest, A.TupleArray) else [x.manifest])])
+        if cx.guard is None:
+            cx.guard = A.Guard(cx.ctx)
+        guard = cx.guard
+        guard.attach(stream)
+        guard.reset(stream)
+        cx.loop = _Loop(stream, guard)
+        total, batch, stepwise = 0, [a], False
+        try:
+            while limit is None or total < limit:
+                want = ahead if limit is None else min(ahead, limit - total)
+                batch = [a]
+                try:
+                    for _ in range(want):
+                        cur = batch[-1]
+                        flag = p(*cur) if tup else p(cur)
+                        if flag.shape != ():
+                            raise TypeError("the predicate of awhile yields a scalar array")
+                        if flag.ctype != "Word8":
+                            flag = map(lambda v: v.ne(0), flag)
+                        flag = _force(flag, cx)
+                        cx.launch([flag.manifest], [], lambda i, o, s: guard.latch(i[0], s))
+                        batch.append(force(f(*cur) if tup else f(cur)))
+                except _HostReadInLoop:
+                    stepwise = True
+                alive, count = guard.read(stream)
+                # (a batch cut short by the fall-back may have latched an iteration whose body was never enqueued whole)
+                taken = min(count - total, len(batch) - 1)
+                a = batch[taken]
+                total += taken
+                if stepwise or not alive:
+                    break
+        finally:
+            cx.loop = None
+            guard.detach(stream)
+        del batch
+        if stepwise:
+            return _awhile_stepwise(cx, p, f, a, tup, force, limit, total)
+        return a
 
 
 def run(a, context=None):
@@ -1153,6 +1225,9 @@ def destroy(context):
     with context.lock:
         context.ctx.sync()
         context.skeletons.clear()
+        if context.guard is not None:
+            context.guard.destroy()
+            context.guard = None
         context.streams, context.events = [], []
         context.table.destroy()
         context.ctx.close()

@@ -25,7 +25,7 @@ SCAN_KINDS = {"scanl": SKEL_SCANL, "scanl1": SKEL_SCANL1, "scanl'": SKEL_SCANLP,
               "scanr": SKEL_SCANR, "scanr1": SKEL_SCANR1, "scanr'": SKEL_SCANRP}
 COMBINE_GENERIC, COMBINE_ADD, COMBINE_MIN, COMBINE_MAX, COMBINE_AND, COMBINE_OR, COMBINE_XOR = range(7)
 BOUNDARY = {"clamp": 0, "mirror": 1, "wrap": 2, "constant": 3}
-FLAG_FOLD_RIGHT, FLAG_FAST_MATH = 1, 2
+FLAG_FOLD_RIGHT, FLAG_FAST_MATH, FLAG_GUARDED = 1, 2, 4
 
 CTYPE = {np.dtype(np.float32): "float", np.dtype(np.float64): "double",
          np.dtype(np.int8): "Int8", np.dtype(np.int16): "Int16", np.dtype(np.int32): "Int32",
@@ -96,7 +96,8 @@ acc_event_elapsed_ms acc_compile acc_compile_log acc_cache_set_dir acc_cache_dir
 acc_cache_clear acc_module_load acc_module_unload acc_module_get_function acc_function_attr acc_occupancy
 acc_launch acc_launch_grid acc_skel_create acc_skel_destroy acc_skel_source acc_skel_preview acc_skel_compile_only
 acc_skel_get_info acc_exec_map acc_exec_fold acc_exec_foldseg acc_exec_foldseg_nd acc_exec_scan acc_exec_scan_noalloc acc_exec_permute
-acc_exec_stencil acc_exec_stencil2 acc_exec_stencil_iterate acc_memtable_create acc_memtable_destroy
+acc_exec_stencil acc_exec_stencil2 acc_exec_stencil_iterate acc_guard_create acc_guard_destroy acc_guard_reset
+acc_guard_latch acc_guard_read acc_stream_set_guard acc_memtable_create acc_memtable_destroy
 acc_memtable_malloc acc_memtable_acquire acc_memtable_release acc_memtable_free acc_memtable_insert_unmanaged
 acc_memtable_reclaim acc_memtable_get_stats""".split()
 
@@ -165,6 +166,12 @@ def lib():
         L.acc_exec_stencil.argtypes = [C.c_void_p, AP, AP, AP, C.c_void_p]
         L.acc_exec_stencil2.argtypes = [C.c_void_p, AP, AP, AP, AP, C.c_void_p]
         L.acc_exec_stencil_iterate.argtypes = [C.c_void_p, AP, AP, AP, C.c_int32, C.c_void_p, C.POINTER(C.c_int32)]
+        L.acc_guard_create.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+        L.acc_guard_destroy.argtypes = [C.c_void_p]
+        L.acc_guard_reset.argtypes = [C.c_void_p, C.c_void_p]
+        L.acc_guard_latch.argtypes = [C.c_void_p, AP, C.c_void_p]
+        L.acc_guard_read.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_int32), C.POINTER(C.c_int64)]
+        L.acc_stream_set_guard.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
         L.acc_memtable_create.argtypes = [C.c_void_p, C.c_uint64, C.POINTER(C.c_void_p)]
         L.acc_memtable_destroy.argtypes = [C.c_void_p]
         L.acc_memtable_malloc.argtypes = [C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint64, C.c_int, C.POINTER(C.c_int)]
@@ -412,6 +419,39 @@ class Context(object):
     def close(self):
         if self.handle:
             lib().acc_context_destroy(self.handle)
+            self.handle = None
+
+
+class Guard(object):
+    """acc_guard: the `alive` and `count` words of an array-level loop whose iterations are enqueued ahead"""
+
+    def __init__(self, ctx):
+        self.ctx = ctx
+        h = C.c_void_p()
+        check(lib().acc_guard_create(ctx.handle, C.byref(h)))
+        self.handle = h
+
+    def reset(self, stream=None):
+        check(lib().acc_guard_reset(self.handle, stream))
+
+    def latch(self, pred, stream=None):
+        """`pred`: a rank-0 device array of one byte"""
+        check(lib().acc_guard_latch(self.handle, C.byref(pred.desc()), stream))
+
+    def read(self, stream=None):
+        alive, count = C.c_int32(), C.c_int64()
+        check(lib().acc_guard_read(self.handle, stream, C.byref(alive), C.byref(count)))
+        return bool(alive.value), count.value
+
+    def attach(self, stream):
+        check(lib().acc_stream_set_guard(self.ctx.handle, stream, self.handle))
+
+    def detach(self, stream):
+        check(lib().acc_stream_set_guard(self.ctx.handle, stream, None))
+
+    def destroy(self):
+        if self.handle:
+            lib().acc_guard_destroy(self.handle)
             self.handle = None
 
 

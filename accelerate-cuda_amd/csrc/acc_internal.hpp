@@ -3,6 +3,7 @@
 #include <hip/hip_runtime_api.h>
 #include <hip/hiprtc.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
@@ -88,6 +89,9 @@ struct ScratchRef {
 enum StatusWord { STATUS_SCAN_LOOKBACK = 0, STATUS_FOLD_COLLECT = 1, STATUS_PERMUTE_LOCK = 2, STATUS_WORDS = 16 };
 
 // big single-pass scans on different streams of one device are kept from overlapping (runtime.cpp)
+// device-to-device copy of `bytes` bytes that does nothing when the guard word at `guard` is zero (guard.hip)
+int guarded_copy(uint64_t dst, uint64_t src, size_t bytes, uint64_t guard, hipStream_t stream);
+
 int scan_order_before(int device, hipStream_t stream);    // ACC_OK: the caller launches, then calls scan_order_after
 void scan_order_after(int device);
 void scan_order_forget(int device, hipStream_t stream);
@@ -110,6 +114,17 @@ struct acc_context_s {
   // kernels report here that a bounded wait ran out (see StatusWord); NULL if the block could not be set up
   volatile uint32_t *status_host = nullptr;
   uint64_t status_dev = 0;
+
+  // streams with a loop's guard set (acc_stream_set_guard) and the address of its `alive` word
+  std::map<hipStream_t, uint64_t> guards;
+  std::atomic<int> n_guards{0};
+  uint64_t guard_of(hipStream_t stream)
+  {
+    if (n_guards.load(std::memory_order_acquire) == 0) return 0;
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = guards.find(stream);
+    return it == guards.end() ? 0 : it->second;
+  }
 
   int make_current() const;
   // zero-initialised when first allocated; contents persist between uses and

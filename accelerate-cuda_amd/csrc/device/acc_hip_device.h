@@ -206,6 +206,22 @@ ACC_DEV void acc_report(unsigned int *status, const int word)
   if (status) __hip_atomic_store(status + word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
+/* ACC_GUARDED: the kernels of an instance built for the body or the predicate of an array-level loop take one more
+ * parameter, a word in device memory that says whether the loop is still running, and return at once when it is
+ * zero (a NULL pointer means no loop).  The host can then enqueue several iterations ahead without knowing how
+ * many will be wanted: the ones past the end do nothing.  The test is one scalar load per wave; instances built
+ * without the flag carry neither the parameter nor the test.                                                  */
+#ifndef ACC_GUARDED
+#define ACC_GUARDED 0
+#endif
+#if ACC_GUARDED
+#define ACC_GUARD_PARAM , const unsigned int *__restrict__ acc_guard
+#define ACC_GUARD_CHECK if (acc_guard != (const unsigned int *)0 && *acc_guard == 0u) return;
+#else
+#define ACC_GUARD_PARAM
+#define ACC_GUARD_CHECK
+#endif
+
 /* A read of an array element that will not be needed again (a manifest input
  * consumed once, in index order).  It is marked non-temporal so that it does
  * not evict data that IS reused -- a gathered vector, a small table -- from

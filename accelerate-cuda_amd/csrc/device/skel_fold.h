@@ -97,11 +97,12 @@ ACC_ENTRY(ACC_ENV_PARAMS
           ACC_OUT_ARRAY(arrOut),
           const Int64 shIn_0,
 #if ACC_FOLD_SINGLE
-          unsigned long long *partials, const unsigned int epoch, unsigned int *acc_status)
+          unsigned long long *partials, const unsigned int epoch, unsigned int *acc_status ACC_GUARD_PARAM)
 #else
-          ACC_ELT *__restrict__ partials)
+          ACC_ELT *__restrict__ partials ACC_GUARD_PARAM)
 #endif
 {
+  ACC_GUARD_CHECK
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
   __shared__ acc_opt<T> s_wave[ACC_WAVES];
@@ -211,8 +212,9 @@ ACC_ENTRY(ACC_ENV_PARAMS
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 ACC_CAT(ACC_ENTRY, _finish)(ACC_ENV_PARAMS
                             ACC_OUT_ARRAY(arrOut),
-                            const ACC_ELT *__restrict__ partials, const Int64 count)
+                            const ACC_ELT *__restrict__ partials, const Int64 count ACC_GUARD_PARAM)
 {
+  ACC_GUARD_CHECK
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
   __shared__ acc_opt<T> s_wave[ACC_WAVES];

@@ -84,8 +84,9 @@ static_assert(ACC_CHUNK % (ACC_BLOCK * ACC_VEC) == 0, "chunk must be a whole num
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
                   const Int64 shOut_0, ACC_OUT_ARRAY(arrOut),
-                  ACC_SEG_PARAMS)
+                  ACC_SEG_PARAMS ACC_GUARD_PARAM)
 {
+  ACC_GUARD_CHECK
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
   __shared__ __attribute__((aligned(16))) T s_val[ACC_PAD(ACC_CHUNK)];
@@ -283,8 +284,9 @@ ACC_DEV void acc_fold_rows(const Int64 nseg, G get, F f, const T &seed, P put)
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 ACC_FS_CAT_(ACC_FOLDSEG_ENTRY, _rows)(ACC_ENV_PARAMS
                                       const Int64 shOut_0, ACC_OUT_ARRAY(arrOut),
-                                      ACC_SEG_PARAMS)
+                                      ACC_SEG_PARAMS ACC_GUARD_PARAM)
 {
+  ACC_GUARD_CHECK
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
   auto get = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
@@ -337,8 +339,9 @@ ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _team)(ACC_ENV_PARAMS
                                      const Int64 shOut_0, ACC_OUT_ARRAY(arrOut),
                                      ACC_SEG_PARAMS,
                                      const int block_team, const Int64 split,
-                                     ACC_ELT *__restrict__ part, int *__restrict__ part_ok)
+                                     ACC_ELT *__restrict__ part, int *__restrict__ part_ok ACC_GUARD_PARAM)
 {
+  ACC_GUARD_CHECK
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
   __shared__ acc_opt<T> s_wave[ACC_FS_WAVES];
@@ -451,8 +454,9 @@ ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _team)(ACC_ENV_PARAMS
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _join)(ACC_ENV_PARAMS
                                      const Int64 shOut_0, ACC_OUT_ARRAY(arrOut), const Int64 split,
-                                     const ACC_ELT *__restrict__ part, const int *__restrict__ part_ok)
+                                     const ACC_ELT *__restrict__ part, const int *__restrict__ part_ok ACC_GUARD_PARAM)
 {
+  ACC_GUARD_CHECK
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
   auto f  = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };

@@ -22,8 +22,9 @@
 #define ACC_TILE (ACC_BLOCK * ACC_VEC * ACC_UNROLL)
 
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
-ACC_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS)
+ACC_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_GUARD_PARAM)
 {
+  ACC_GUARD_CHECK
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
 #if ACC_ALIGNED

@@ -69,8 +69,9 @@
  * of global locks per element while the windows are few).                                                 */
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, int *__restrict__ locks, const int lds_bins, const int lds_copies,
-        ACC_ELT *__restrict__ dump_val, int *__restrict__ dump_ok, const int win_blocks, unsigned int *acc_status)
+        ACC_ELT *__restrict__ dump_val, int *__restrict__ dump_ok, const int win_blocks, unsigned int *acc_status ACC_GUARD_PARAM)
 {
+  ACC_GUARD_CHECK
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
   extern __shared__ __attribute__((aligned(16))) unsigned char acc_lds_raw[];
@@ -163,8 +164,9 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, int *__restrict__ loc
  * the `rows` rows of the table that belong to the target's window of `bins` targets */
 extern "C" __global__ void __launch_bounds__(256)
 permute_join(ACC_ENV_PARAMS ACC_OUT_PARAMS, const ACC_ELT *__restrict__ dump_val, const int *__restrict__ dump_ok,
-             const int rows, const int bins, const Int64 ntarget)
+             const int rows, const int bins, const Int64 ntarget ACC_GUARD_PARAM)
 {
+  ACC_GUARD_CHECK
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
   auto f  = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
@@ -314,8 +316,9 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
 #if ACC_PERMUTE_NARROW
         , unsigned int *acc_status
 #endif
-        )
+        ACC_GUARD_PARAM)
 {
+  ACC_GUARD_CHECK
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
   extern __shared__ __attribute__((aligned(16))) unsigned char acc_lds_raw[];
@@ -513,8 +516,9 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
  * small jobs that precede the main kernel, in one launch */
 extern "C" __global__ void __launch_bounds__(256)
 permute_fill(ACC_ELT *__restrict__ p, const Int64 count, ACC_ELT *__restrict__ copy_dst,
-             const ACC_ELT *__restrict__ copy_src, const Int64 copy_count)
+             const ACC_ELT *__restrict__ copy_src, const Int64 copy_count ACC_GUARD_PARAM)
 {
+  ACC_GUARD_CHECK
   const ACC_ELT ident = acc_hint_identity<ACC_ELT>();
   const Int64 first = (Int64)blockIdx.x * 256 + threadIdx.x, step = (Int64)gridDim.x * 256;
   for (Int64 i = first; i < count; i += step) p[i] = ident;
@@ -540,8 +544,9 @@ struct acc_merge_job {
  * the rows shared between `slices` workgroups (then each adds its share atomically) */
 extern "C" __global__ void __launch_bounds__(256)
 permute_merge(ACC_ENV_PARAMS ACC_OUT_PARAMS, const unsigned *__restrict__ dump, const Int64 nwords, const int nrows,
-              const int slices, const Int64 ntarget)
+              const int slices, const Int64 ntarget ACC_GUARD_PARAM)
 {
+  ACC_GUARD_CHECK
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
   auto f = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
@@ -570,8 +575,9 @@ permute_merge(ACC_ENV_PARAMS ACC_OUT_PARAMS, const unsigned *__restrict__ dump, 
 /* folds up to two tables in one launch: workgroups [0, blocks_a) take job a,
  * the rest job b */
 extern "C" __global__ void __launch_bounds__(256)
-permute_merge(ACC_ENV_PARAMS ACC_OUT_PARAMS, const acc_merge_job a, const int blocks_a, const acc_merge_job b)
+permute_merge(ACC_ENV_PARAMS ACC_OUT_PARAMS, const acc_merge_job a, const int blocks_a, const acc_merge_job b ACC_GUARD_PARAM)
 {
+  ACC_GUARD_CHECK
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
   auto f = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };

@@ -434,8 +434,9 @@ ACC_ENTRY(ACC_ENV_PARAMS
           ACC_OUT_ARRAY(arrSum),
           const Int64 shIn_0,
           void *desc0, void *desc1, void *desc2,
-          const unsigned int epoch, const Int64 num_tiles, unsigned int *acc_status)
+          const unsigned int epoch, const Int64 num_tiles, unsigned int *acc_status ACC_GUARD_PARAM)
 {
+  ACC_GUARD_CHECK
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
 #if ACC_ALIGNED

@@ -232,8 +232,9 @@ struct acc_strip_source {
 #endif
 
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
-ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS)
+ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS ACC_GUARD_PARAM)
 {
+  ACC_GUARD_CHECK
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
 #if ACC_STENCIL_RANK == 3

@@ -20,6 +20,16 @@ namespace {
 
 // Kernel arguments in launch order.  Every argument of these kernels is at
 // most 8 bytes, so each gets one 8-byte slot whose address is handed to HIP.
+// What the driver that is running on this thread launches for: the instance's entry name (for the launch trace) and,
+// for an instance built with ACC_FLAG_GUARDED, the address of the guard word that every one of its kernels takes as
+// its last parameter (0: no loop).
+struct Running {
+  const char *entry = "";
+  bool guarded = false;
+  uint64_t guard = 0;
+};
+thread_local Running t_run;
+
 class Args {
  public:
   void i64(int64_t v) { push(&v, sizeof(v)); }
@@ -27,7 +37,17 @@ class Args {
   void i32(int32_t v) { push(&v, sizeof(v)); }
   void ptr(uint64_t v) { push(&v, sizeof(v)); }
   size_t count() const { return slots_.size(); }
+  // the arguments as HIP wants them, the guard's address appended for a guarded instance
   void **data()
+  {
+    if (t_run.guarded && !guard_pushed_) {
+      ptr(t_run.guard);
+      guard_pushed_ = true;
+    }
+    return data_without_guard();
+  }
+  // (for a launch whose last arguments are not 8-byte slots: the caller appends them, then the guard)
+  void **data_without_guard()
   {
     ptrs_.clear();
     for (uint64_t &s : slots_) ptrs_.push_back(&s);
@@ -43,7 +63,34 @@ class Args {
   }
   std::deque<uint64_t> slots_;
   std::vector<void *> ptrs_;
+  bool guard_pushed_ = false;
 };
+
+// Every kernel launch of the drivers.  ACC_HIP_DEBUG=dump-exec prints one line per launch -- entry<<<grid, block,
+// lds>>> and the time on the device -- as the reference's -ddump-exec does (Debug.hs:41-76, hooked at
+// Execute.hs:975-982); timing a launch means waiting for it, so the trace serialises the stream.
+hipError_t launch_kernel(hipFunction_t f, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned by, unsigned bz, unsigned lds,
+                         hipStream_t st, void **args, void **extra)
+{
+  static const bool trace = [] {
+    const char *e = std::getenv("ACC_HIP_DEBUG");
+    return e && std::strstr(e, "dump-exec");
+  }();
+  if (!trace) return hipModuleLaunchKernel(f, gx, gy, gz, bx, by, bz, lds, st, args, extra);
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  const bool timed = hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess && hipEventRecord(e0, st) == hipSuccess;
+  const hipError_t rc = hipModuleLaunchKernel(f, gx, gy, gz, bx, by, bz, lds, st, args, extra);
+  float ms = -1.0f;
+  if (timed && rc == hipSuccess && hipEventRecord(e1, st) == hipSuccess && hipEventSynchronize(e1) == hipSuccess)
+    (void)hipEventElapsedTime(&ms, e0, e1);
+  const char *name = hipKernelNameRef(f);
+  std::fprintf(stderr, "[acc-hip exec] %s: %s<<<%u, %u, %u>>> gpu: %.3f ms%s\n", t_run.entry, name ? name : "?", gx, bx, lds, ms,
+               rc == hipSuccess ? "" : " FAILED");
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  (void)hipGetLastError();
+  return rc;
+}
 
 int64_t array_size(const acc_array &a)
 {
@@ -119,11 +166,36 @@ int launch(acc_skel_s *s, int variant, int64_t grid, size_t dyn_lds, hipStream_t
   if (grid < 1 || grid > 0x7fffffffLL) return fail(ACC_ERR_INVALID, "%s: grid of %lld blocks", s->entry.c_str(), (long long)grid);
   ACC_TRY(s->ensure_variant(variant));
   ACC_TRY(s->ctx->make_current());
-  ACC_HIP_TRY(hipModuleLaunchKernel(s->variants[variant].fn, static_cast<unsigned>(grid), 1, 1,
+  ACC_HIP_TRY(launch_kernel(s->variants[variant].fn, static_cast<unsigned>(grid), 1, 1,
                                     static_cast<unsigned>(s->spec.block), 1, 1, static_cast<unsigned>(dyn_lds), stream,
                                     args->data(), nullptr));
   return ACC_OK;
 }
+
+// For the length of one driver call: what Args::data() and launch_kernel read (see Running).  A stream under a guard
+// only takes instances whose kernels look at it.
+struct RunScope {
+  Running saved;
+  int rc = ACC_OK;
+  RunScope(acc_skel_s *s, hipStream_t st) : saved(t_run)
+  {
+    t_run.entry = s->entry.c_str();
+    t_run.guarded = s->spec.guarded;
+    t_run.guard = 0;
+    const uint64_t g = s->ctx->guard_of(st);
+    if (g && !s->spec.guarded)
+      rc = fail(ACC_ERR_INVALID, "%s: the stream is under a guard (acc_stream_set_guard) and this instance was created without ACC_FLAG_GUARDED",
+                s->entry.c_str());
+    else
+      t_run.guard = g;
+  }
+  ~RunScope() { t_run = saved; }
+  RunScope(const RunScope &) = delete;
+  RunScope &operator=(const RunScope &) = delete;
+};
+#define ACC_RUN_SCOPE(s, st)                          \
+  RunScope run_scope__((s), (st));                    \
+  if (run_scope__.rc != ACC_OK) return run_scope__.rc
 
 bool kind_is(const acc_skel_s *s, std::initializer_list<int> kinds)
 {
@@ -142,6 +214,7 @@ extern "C" {
 int acc_exec_map(acc_skel s, const acc_array *env, const acc_array *out, acc_stream stream)
 {
   if (!s) return fail(ACC_ERR_INVALID, "acc_exec_map: NULL skeleton");
+  ACC_RUN_SCOPE(s, static_cast<hipStream_t>(stream));
   if (!kind_is(s, {ACC_SKEL_MAP, ACC_SKEL_GENERATE, ACC_SKEL_TRANSFORM})) return fail(ACC_ERR_INVALID, "acc_exec_map: skeleton is '%s'", s->entry.c_str());
   ACC_TRY(check_out(s, out, s->spec.out_rank, "result"));
   Args args;
@@ -198,7 +271,7 @@ int launch_segmented(acc_skel_s *s, int v, Args *args, const acc_array *env, con
   const int64_t tgrid = acc_launch_grid(nseg * split, per_block, cus, 2048 / s->spec.block);
   int rc = s->ctx->make_current();
   if (rc == ACC_OK) {
-    hipError_t e = hipModuleLaunchKernel(s->variants[v].fn_finish, static_cast<unsigned>(tgrid), 1, 1,
+    hipError_t e = launch_kernel(s->variants[v].fn_finish, static_cast<unsigned>(tgrid), 1, 1,
                                          static_cast<unsigned>(s->spec.block), 1, 1, 0, st, args->data(), nullptr);
     if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(segmented fold, team)");
   }
@@ -214,7 +287,7 @@ int launch_segmented(acc_skel_s *s, int v, Args *args, const acc_array *env, con
     if (rc == ACC_OK) {
       const int64_t waves = s->spec.block / 64;
       const int64_t jgrid = (nseg + waves - 1) / waves;          // a wave per segment
-      hipError_t e = hipModuleLaunchKernel(s->variants[v].fn_fill, static_cast<unsigned>(jgrid), 1, 1,
+      hipError_t e = launch_kernel(s->variants[v].fn_fill, static_cast<unsigned>(jgrid), 1, 1,
                                            static_cast<unsigned>(s->spec.block), 1, 1, 0, st, join.data(), nullptr);
       if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(segmented fold, join)");
     }
@@ -228,6 +301,7 @@ int launch_segmented(acc_skel_s *s, int v, Args *args, const acc_array *env, con
 int acc_exec_fold(acc_skel s, const acc_array *env, int32_t in_rank, const int64_t *in_shape, const acc_array *out, acc_stream stream)
 {
   if (!s) return fail(ACC_ERR_INVALID, "acc_exec_fold: NULL skeleton");
+  ACC_RUN_SCOPE(s, static_cast<hipStream_t>(stream));
   if (!kind_is(s, {ACC_SKEL_FOLD, ACC_SKEL_FOLD1})) return fail(ACC_ERR_INVALID, "acc_exec_fold: skeleton is '%s'", s->entry.c_str());
   if (in_rank != s->spec.out_rank + 1 || !in_shape) return fail(ACC_ERR_INVALID, "%s: input rank %d, kernel was built for %d", s->entry.c_str(), in_rank, s->spec.out_rank + 1);
   ACC_TRY(check_out(s, out, s->spec.out_rank, "result"));
@@ -272,7 +346,7 @@ int acc_exec_fold(acc_skel s, const acc_array *env, int32_t in_rank, const int64
       // short rows: a lane reads its row straight from memory (skel_foldseg.h, _rows)
       const int64_t r = inner == 1 ? 4 : (inner == 2 ? 2 : 1), u = r * inner >= 16 ? 1 : 16 / (r * inner);   // as the kernel's R and U
       const int64_t grid = acc_launch_grid(rows, s->spec.block * r * u, resident(s, v), acc::tune("foldseg.oversub", 1 << 20));
-      hipError_t e = hipModuleLaunchKernel(s->variants[v].fn_rows, static_cast<unsigned>(grid), 1, 1, static_cast<unsigned>(s->spec.block), 1, 1,
+      hipError_t e = launch_kernel(s->variants[v].fn_rows, static_cast<unsigned>(grid), 1, 1, static_cast<unsigned>(s->spec.block), 1, 1,
                                            0, st, args.data(), nullptr);
       return e == hipSuccess ? ACC_OK : acc::fail_hip(e, "hipModuleLaunchKernel(fold, short rows)");
     }
@@ -324,7 +398,7 @@ int acc_exec_fold(acc_skel s, const acc_array *env, int32_t in_rank, const int64
     fin.ptr(partials);
     fin.i64(grid);
     if (rc == ACC_OK) {
-      hipError_t e = hipModuleLaunchKernel(s->variants[v].fn_finish, 1, 1, 1, static_cast<unsigned>(s->spec.block), 1, 1, 0, st, fin.data(), nullptr);
+      hipError_t e = launch_kernel(s->variants[v].fn_finish, 1, 1, 1, static_cast<unsigned>(s->spec.block), 1, 1, 0, st, fin.data(), nullptr);
       if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(fold finish)");
     }
   }
@@ -336,6 +410,7 @@ int acc_exec_foldseg_nd(acc_skel s, const acc_array *env, int32_t in_rank, const
                         const acc_array *out, acc_stream stream)
 {
   if (!s) return fail(ACC_ERR_INVALID, "acc_exec_foldseg: NULL skeleton");
+  ACC_RUN_SCOPE(s, static_cast<hipStream_t>(stream));
   if (!kind_is(s, {ACC_SKEL_FOLDSEG, ACC_SKEL_FOLD1SEG})) return fail(ACC_ERR_INVALID, "acc_exec_foldseg: skeleton is '%s'", s->entry.c_str());
   const int rank = std::max(1, s->spec.out_rank);        // of the input and of the result alike
   if (in_rank != rank || !in_shape) return fail(ACC_ERR_INVALID, "%s: input rank %d, kernel was built for %d", s->entry.c_str(), in_rank, rank);
@@ -390,6 +465,7 @@ int scan_core(acc_skel s, const acc_array *env, int64_t n, const acc_array *out,
               const bool noalloc, const char *who)
 {
   if (!s) return fail(ACC_ERR_INVALID, "%s: NULL skeleton", who);
+  ACC_RUN_SCOPE(s, static_cast<hipStream_t>(stream));
   if (!kind_is(s, {ACC_SKEL_SCANL, ACC_SKEL_SCANL1, ACC_SKEL_SCANLP, ACC_SKEL_SCANR, ACC_SKEL_SCANR1, ACC_SKEL_SCANRP}))
     return fail(ACC_ERR_INVALID, "%s: skeleton is '%s'", who, s->entry.c_str());
   if (n < 0) return fail(ACC_ERR_INVALID, "%s: negative input extent", s->entry.c_str());
@@ -448,7 +524,7 @@ int scan_core(acc_skel s, const acc_array *env, int64_t n, const acc_array *out,
     args.i64(tiles);
     args.ptr(s->ctx->status_dev);
     if (grid < 1 || grid > 0x7fffffffLL) return fail(ACC_ERR_INVALID, "%s: grid of %lld blocks", who, (long long)grid);
-    ACC_HIP_TRY(hipModuleLaunchKernel(s->variants[v].fn, static_cast<unsigned>(grid), 1, 1, static_cast<unsigned>(s->spec.block), 1, 1,
+    ACC_HIP_TRY(launch_kernel(s->variants[v].fn, static_cast<unsigned>(grid), 1, 1, static_cast<unsigned>(s->spec.block), 1, 1,
                                       0, st, args.data(), nullptr));
     return ACC_OK;
   }
@@ -494,6 +570,7 @@ int acc_exec_scan_noalloc(acc_skel s, const acc_array *env, int64_t n, const acc
 int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_array *defaults, const acc_array *out, acc_stream stream)
 {
   if (!s) return fail(ACC_ERR_INVALID, "acc_exec_permute: NULL skeleton");
+  ACC_RUN_SCOPE(s, static_cast<hipStream_t>(stream));
   if (!kind_is(s, {ACC_SKEL_PERMUTE})) return fail(ACC_ERR_INVALID, "acc_exec_permute: skeleton is '%s'", s->entry.c_str());
   if (n_src < 0) return fail(ACC_ERR_INVALID, "permute: negative source extent");
   ACC_TRY(check_out(s, out, s->spec.out_rank, "result"));
@@ -511,7 +588,10 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
     const int nc = s->ncomp();
     for (int c = 0; c < nc; ++c) {
       const size_t csz = nc == 1 ? esz : (size_t)acc::type_size(s->spec.comp_types[nc - 1 - c]);
-      ACC_HIP_TRY(hipMemcpyAsync(reinterpret_cast<void *>(out->ptr[c]), reinterpret_cast<void *>(defaults->ptr[c]), (size_t)ntarget * csz, hipMemcpyDeviceToDevice, st));
+      if (t_run.guard)      // under a loop's guard the copy, too, must not happen once the loop has ended
+        ACC_TRY(acc::guarded_copy(out->ptr[c], defaults->ptr[c], (size_t)ntarget * csz, t_run.guard, st));
+      else
+        ACC_HIP_TRY(hipMemcpyAsync(reinterpret_cast<void *>(out->ptr[c]), reinterpret_cast<void *>(defaults->ptr[c]), (size_t)ntarget * csz, hipMemcpyDeviceToDevice, st));
     }
     return ACC_OK;
   };
@@ -603,7 +683,7 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
       j.i32(lds_bins);
       j.i64(ntarget);
       if (lrc == ACC_OK) {
-        hipError_t je = hipModuleLaunchKernel(s->variants[lv].fn_finish, static_cast<unsigned>((ntarget + 3) / 4), 1, 1, 256, 1, 1, 0, st,
+        hipError_t je = launch_kernel(s->variants[lv].fn_finish, static_cast<unsigned>((ntarget + 3) / 4), 1, 1, 256, 1, 1, 0, st,
                                               j.data(), nullptr);
         if (je != hipSuccess) lrc = acc::fail_hip(je, "hipModuleLaunchKernel(permute_join)");
       }
@@ -638,7 +718,7 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
       f.ptr(defaults->ptr[0]);
       f.i64(ntarget);
       const int64_t fill_grid = std::min<int64_t>((ntarget + 255) / 256, 8 * (int64_t)s->ctx->props.multiProcessorCount);
-      hipError_t fe = hipModuleLaunchKernel(s->variants[nv].fn_fill, static_cast<unsigned>(fill_grid), 1, 1, 256, 1, 1, 0, st, f.data(), nullptr);
+      hipError_t fe = launch_kernel(s->variants[nv].fn_fill, static_cast<unsigned>(fill_grid), 1, 1, 256, 1, 1, 0, st, f.data(), nullptr);
       if (fe != hipSuccess) return acc::fail_hip(fe, "hipModuleLaunchKernel(permute_fill, narrow counts)");
     }
     const int64_t nwords = (ntarget + 1) / 2;
@@ -670,7 +750,7 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
       m.i32(static_cast<int32_t>(slices));
       m.i64(ntarget);
       if (nrc == ACC_OK) {
-        hipError_t me = hipModuleLaunchKernel(s->variants[nv].fn_finish, static_cast<unsigned>(columns * slices), 1, 1, 256, 1, 1, 0, st,
+        hipError_t me = launch_kernel(s->variants[nv].fn_finish, static_cast<unsigned>(columns * slices), 1, 1, 256, 1, 1, 0, st,
                                               m.data(), nullptr);
         if (me != hipSuccess) nrc = acc::fail_hip(me, "hipModuleLaunchKernel(permute_merge, narrow counts)");
       }
@@ -721,12 +801,15 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
         bool mal = true;
         wrc = push_env(s, env, &m, &mal);
         push_out(*out, &m, &mal);
-        std::vector<void *> margs(m.data(), m.data() + m.count());
+        void **mslots = m.data_without_guard();
+        std::vector<void *> margs(mslots, mslots + m.count());
         margs.push_back(&ja);
         margs.push_back(&blocks_a32);
         margs.push_back(&jb);
+        uint64_t mguard = t_run.guard;
+        if (t_run.guarded) margs.push_back(&mguard);
         if (wrc == ACC_OK) {
-          hipError_t me = hipModuleLaunchKernel(s->variants[wv].fn_finish, static_cast<unsigned>(blocks_a32), 1, 1, 256, 1, 1, 0, st,
+          hipError_t me = launch_kernel(s->variants[wv].fn_finish, static_cast<unsigned>(blocks_a32), 1, 1, 256, 1, 1, 0, st,
                                                 margs.data(), nullptr);
           if (me != hipSuccess) wrc = acc::fail_hip(me, "hipModuleLaunchKernel(permute_merge, windows)");
         }
@@ -785,7 +868,7 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
     f.ptr(defaults->ptr[0]);
     f.i64(copy_defaults ? ntarget : 0);
     const int64_t fill_grid = std::min<int64_t>((XCD_ROWS * ntarget + 255) / 256, 8 * (int64_t)cus);
-    e = hipModuleLaunchKernel(s->variants[v].fn_fill, static_cast<unsigned>(fill_grid), 1, 1, 256, 1, 1, 0, st, f.data(), nullptr);
+    e = launch_kernel(s->variants[v].fn_fill, static_cast<unsigned>(fill_grid), 1, 1, 256, 1, 1, 0, st, f.data(), nullptr);
     if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(permute_fill)");
   } else if (copy_defaults) {           // the defaults by the same kernel: a runtime copy of 1 KB takes 4 us, this launch 2
     Args f;
@@ -795,7 +878,7 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
     f.ptr(defaults->ptr[0]);
     f.i64(ntarget);
     const int64_t fill_grid = std::min<int64_t>((ntarget + 255) / 256, 8 * (int64_t)cus);
-    e = hipModuleLaunchKernel(s->variants[v].fn_fill, static_cast<unsigned>(fill_grid), 1, 1, 256, 1, 1, 0, st, f.data(), nullptr);
+    e = launch_kernel(s->variants[v].fn_fill, static_cast<unsigned>(fill_grid), 1, 1, 256, 1, 1, 0, st, f.data(), nullptr);
     if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(permute_fill, defaults)");
   }
   args.i32(static_cast<int32_t>(bins));
@@ -822,12 +905,15 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
     rc = push_env(s, env, &m, &al);
     push_out(*out, &m, &al);
     int32_t blocks_a32 = static_cast<int32_t>(blocks_a);
-    std::vector<void *> margs(m.data(), m.data() + m.count());
+    void **mslots = m.data_without_guard();
+    std::vector<void *> margs(mslots, mslots + m.count());
     margs.push_back(&ja);
     margs.push_back(&blocks_a32);
     margs.push_back(&jb);
+    uint64_t mguard = t_run.guard;
+    if (t_run.guarded) margs.push_back(&mguard);
     if (rc == ACC_OK) {
-      e = hipModuleLaunchKernel(s->variants[v].fn_finish, static_cast<unsigned>(blocks_a + blocks_b), 1, 1, 256, 1, 1, 0, st, margs.data(), nullptr);
+      e = launch_kernel(s->variants[v].fn_finish, static_cast<unsigned>(blocks_a + blocks_b), 1, 1, 256, 1, 1, 0, st, margs.data(), nullptr);
       if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(permute_merge)");
     }
   }
@@ -838,6 +924,7 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
 // `in2` is the second source of a stencil2, NULL for a stencil
 static int stencil_once(acc_skel s, const acc_array *env, const acc_array *in, const acc_array *in2, const acc_array *out, hipStream_t st)
 {
+  ACC_RUN_SCOPE(s, st);
   const int rank = s->spec.out_rank;
   Args args;
   bool aligned = true;

@@ -316,6 +316,7 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
   }
   o << "#define ACC_ENTRY " << *entry << "\n";
   o << "#define ACC_NT_STORE " << tune("nt_store", 1) << "\n";
+  if (sp.guarded) o << "#define ACC_GUARDED 1\n";
   if (tuned("spin_limit")) o << "#define ACC_SPIN_LIMIT " << std::max(0, tune("spin_limit", 1 << 22)) << "\n";
   o << "#include \"acc_hip_device.h\"\n";
   if (!sp.comp_types.empty()) {
@@ -407,6 +408,7 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
     if (sp->elt_size <= 0) return fail(ACC_ERR_INVALID, "cannot size element type '%s': set elt_size", d->elt_type);
     sp->vec_size = sp->elt_size;
   }
+  sp->guarded = (d->flags & ACC_FLAG_GUARDED) != 0;
   sp->out_rank = d->out_rank;
   if (sp->out_rank < 0 || sp->out_rank > ACC_MAX_RANK) return fail(ACC_ERR_INVALID, "bad out_rank %d", d->out_rank);
   for (int k = 0; k < d->n_env; ++k) {

@@ -40,6 +40,7 @@ struct SkelSpec {
   int tile_z = 1;                       // rank-3 stencils: result planes per strip
   // tuning
   int block = 256, unroll = 4, rows = 4, chunk = 4096;
+  bool guarded = false;                 // ACC_FLAG_GUARDED: every kernel takes the address of a loop's guard word last
   bool fold_single = true;              // foldAll in one launch (the last workgroup collects), as generated into the kernel
   int scan_rows_fallback = 8;
   int scan_desc_stride = 16;            // 8-byte words between the tile descriptors of a scan, as generated into the kernel

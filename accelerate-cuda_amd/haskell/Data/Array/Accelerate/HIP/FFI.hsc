@@ -29,9 +29,11 @@ import Foreign.C
 data CContext
 data CSkel
 data CMemTable
+data CGuard
 type Context  = Ptr CContext
 type Skel     = Ptr CSkel
 type MemTable = Ptr CMemTable
+type Guard    = Ptr CGuard
 type Stream   = Ptr ()               -- hipStream_t; nullPtr is the default stream
 type Event    = Ptr ()
 type Module   = Ptr ()
@@ -304,6 +306,14 @@ foreign import ccall safe   "acc_exec_permute"         c_execPermute        :: S
 foreign import ccall safe   "acc_exec_stencil"         c_execStencil        :: Skel -> Ptr AccArray -> Ptr AccArray -> Ptr AccArray -> Stream -> IO Status
 foreign import ccall safe   "acc_exec_stencil2"        c_execStencil2       :: Skel -> Ptr AccArray -> Ptr AccArray -> Ptr AccArray -> Ptr AccArray -> Stream -> IO Status
 foreign import ccall safe   "acc_exec_stencil_iterate" c_execStencilIterate :: Skel -> Ptr AccArray -> Ptr AccArray -> Ptr AccArray -> Int32 -> Stream -> Ptr Int32 -> IO Status
+
+-- Execute.hs:236-244: awhile with its iterations enqueued ahead; the guard's words say how many were taken
+foreign import ccall safe   "acc_guard_create"     c_guardCreate    :: Context -> Ptr Guard -> IO Status
+foreign import ccall safe   "acc_guard_destroy"    c_guardDestroy   :: Guard -> IO Status
+foreign import ccall safe   "acc_guard_reset"      c_guardReset     :: Guard -> Stream -> IO Status
+foreign import ccall safe   "acc_guard_latch"      c_guardLatch     :: Guard -> Ptr AccArray -> Stream -> IO Status
+foreign import ccall safe   "acc_guard_read"       c_guardRead      :: Guard -> Stream -> Ptr Int32 -> Ptr Int64 -> IO Status
+foreign import ccall safe   "acc_stream_set_guard" c_streamSetGuard :: Context -> Stream -> Guard -> IO Status
 
 -- Array/Remote.hs, Array/Table.hs, Array/Prim.hs:177-192: the memory table
 foreign import ccall safe   "acc_memtable_create"           c_memtableCreate          :: Context -> Word64 -> Ptr MemTable -> IO Status

@@ -265,6 +265,8 @@ enum { ACC_BOUNDARY_CLAMP = 0, ACC_BOUNDARY_MIRROR = 1, ACC_BOUNDARY_WRAP = 2, A
 /* flags */
 #define ACC_FLAG_FOLD_RIGHT   1u  /* foldSeg: associate x0 (+) (x1 (+) (... (+) z)) instead of ((x0 (+) x1) ...) (+) z */
 #define ACC_FLAG_FAST_MATH    2u  /* allow FMA contraction (default: off, every scalar op rounds as written) */
+#define ACC_FLAG_GUARDED      4u  /* the instance may run under an acc_guard (see acc_guard_create): its kernels take the
+                                     guard's address as one more, last, parameter and do nothing once the guard is down */
 
 /* What the code generator hands over for one array operation: the pieces
  * CUTranslSkel / CUFun1 / CUFun2 / CUExp / CUDelayed carry across the
@@ -420,6 +422,30 @@ int acc_exec_stencil2(acc_skel s, const acc_array *env, const acc_array *in1, co
  * a; *result_in_b tells where the last application wrote.                    */
 int acc_exec_stencil_iterate(acc_skel s, const acc_array *env, const acc_array *a, const acc_array *b,
                              int32_t iters, acc_stream stream, int32_t *result_in_b);
+
+/* awhile, Execute.hs:236-244, without a host round trip per iteration.  The reference evaluates the predicate, reads
+ * its Scalar Bool back and decides on the host, every iteration.  Here a guard -- two words in device memory, `alive`
+ * and `count` -- stands between the predicate and the body:
+ *
+ *     acc_guard_create; acc_stream_set_guard(stream, guard); acc_guard_reset         alive = 1, count = 0
+ *     K times:   <the predicate's skeletons>; acc_guard_latch(pred);  <the body's skeletons>
+ *     acc_guard_read -> alive, count;   repeat while alive
+ *
+ * acc_guard_latch takes the predicate's result, a rank-0 array of Bool (one byte), where it lies on the device:
+ * alive becomes alive && pred, and count goes up by one if the loop is still alive, so that count is the number of
+ * times the body has really run.  Every skeleton executed on a stream that has a guard set must have been created with
+ * ACC_FLAG_GUARDED (else ACC_ERR_INVALID): its kernels load `alive` on entry and return at once when it is zero, and so
+ * do the copies the drivers make (a permute's defaults).  The iterations enqueued past the end of the loop therefore
+ * leave their result arrays untouched, and the value of the loop is what the count-th application of the body
+ * produced (the initial value if count is 0).  The host reads the guard once per K iterations instead of once per
+ * iteration.  A guard serves one loop at a time; acc_stream_set_guard(stream, NULL) takes it off the stream.     */
+typedef struct acc_guard_s *acc_guard;
+int acc_guard_create(acc_context ctx, acc_guard *out);
+int acc_guard_destroy(acc_guard g);
+int acc_guard_reset(acc_guard g, acc_stream stream);
+int acc_guard_latch(acc_guard g, const acc_array *pred, acc_stream stream);
+int acc_guard_read(acc_guard g, acc_stream stream, int32_t *alive, int64_t *count);   /* waits for the stream */
+int acc_stream_set_guard(acc_context ctx, acc_stream stream, acc_guard g);
 
 /* =========================================================================
  * C. memory table

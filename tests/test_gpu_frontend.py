@@ -375,6 +375,101 @@ def test_awhile_iterates_on_the_device_until_the_flag_clears(acc):
         acc.awhile(lambda xs: xs, lambda xs: xs, acc.use(x, cx), context=cx)
 
 
+def test_awhile_enqueued_ahead_agrees_with_one_iteration_at_a_time(acc):
+    """the same loops with the flag read back every iteration (ahead=1), every 3 and every 8: identical values and
+    iteration counts; the host reads the guard once per batch; bodies with every kind of skeleton in them; a body that
+    needs the host falls back; limits; loops that never run"""
+    import acchip as A
+    cx = acc.Context(0)
+    rng = np.random.default_rng(31)
+    x = rng.integers(1, 50, 50021).astype(np.int64)
+    reads = []
+    real_read = A.Guard.read
+    A.Guard.read = lambda self, stream=None: (reads.append(1), real_read(self, stream))[1]
+    try:
+        big = lambda xs, k: acc.map(lambda m: m < 3000000, acc.fold(acc.max_, 0, xs, context=cx))
+        step = lambda xs, k: (acc.map(lambda v: v * 2, xs), acc.map(lambda c: c + 1, k))
+        ref, steps = x.copy(), 0
+        while ref.max() < 3000000:
+            ref, steps = ref * 2, steps + 1
+        assert steps > 10
+        for ahead in (1, 3, 8, 64):
+            del reads[:]
+            out, k = acc.awhile(big, step, (acc.use(x, cx), acc.unit(0, "Int32", cx)), context=cx, ahead=ahead)
+            assert np.array_equal(acc.run(out, cx), ref) and int(acc.run(k, cx)) == steps, ahead
+            assert len(reads) == (0 if ahead == 1 else steps // ahead + 1), (ahead, len(reads))
+        # a limit below and above the natural end; a loop that never runs
+        for limit in (0, 1, 5, steps, steps + 7):
+            out, k = acc.awhile(big, step, (acc.use(x, cx), acc.unit(0, "Int32", cx)), context=cx, limit=limit, ahead=4)
+            took = min(limit, steps)
+            assert int(acc.run(k, cx)) == took and np.array_equal(acc.run(out, cx), x * 2 ** took), limit
+        never = lambda xs, k: acc.map(lambda m: m < 0, acc.fold(acc.max_, 0, xs, context=cx))
+        out, k = acc.awhile(never, step, (acc.use(x, cx), acc.unit(0, "Int32", cx)), context=cx)
+        assert int(acc.run(k, cx)) == 0 and np.array_equal(acc.run(out, cx), x)
+
+        # scan, segmented fold, permute (its copy of the defaults included) and a stencil inside the body, an Int32 flag
+        y = rng.integers(0, 7, 4096).astype(np.int32)
+        lens = np.full(64, 64, np.int32)
+
+        def body(v, k):
+            sums = acc.foldSeg(add, 0, v, acc.use(lens, cx), context=cx)                       # 64 block sums
+            hist = acc.permute(add, acc.fill((8,), 0, "Int32"), lambda i: (v[i] & 7,), acc.map(lambda t: t * 0 + 1, v), context=cx)
+            run_ = acc.scanl1(add, v, context=cx)
+            sm = acc.stencil([(-1,), (0,), (1,)], lambda a, b, c: acc.max_(a, acc.max_(b, c)), "clamp", v, context=cx)
+            nv = acc.zipWith(lambda a, b: (a + b) & 1023, sm, run_)
+            nv = acc.zipWith(lambda a, i: a + hist[i & 7] + sums[i & 63], nv, acc.generate((4096,), lambda i: acc.fromIntegral(i, "Int32")))
+            return acc.map(lambda t: t & 4095, nv), acc.map(lambda c: c + 1, k)
+
+        def ref_body(v):
+            sums = v.reshape(64, 64).sum(axis=1).astype(np.int32)
+            hist = np.bincount(v & 7, minlength=8).astype(np.int32)
+            run_ = np.cumsum(v, dtype=np.int32)
+            p = np.concatenate([v[:1], v, v[-1:]])
+            sm = np.maximum(p[:-2], np.maximum(p[1:-1], p[2:]))
+            nv = (sm + run_) & 1023
+            i = np.arange(4096)
+            return ((nv + hist[i & 7] + sums[i & 63]) & 4095).astype(np.int32)
+        cont = lambda v, k: acc.map(lambda m: acc.cond((m % 5).ne(0), acc.constant(1, "Int32"), acc.constant(0, "Int32")),
+                                    acc.fold(add, 0, v, context=cx))
+        ry, rk = y.copy(), 0
+        while int(ry.sum(dtype=np.int32)) % 5 != 0 and rk < 40:
+            ry, rk = ref_body(ry), rk + 1
+        for ahead in (1, 4):
+            out, k = acc.awhile(cont, body, (acc.use(y, cx), acc.unit(0, "Int32", cx)), context=cx, limit=40, ahead=ahead)
+            assert int(acc.run(k, cx)) == rk and np.array_equal(acc.run(out, cx), ry), ahead
+        assert rk >= 1
+
+        # a body that needs a value on the host (filter_ reads the count back): the loop goes on stepwise, same result
+        z = rng.integers(0, 1000, 3001).astype(np.int32)
+
+        def shrink(v):
+            kept, _ = acc.filter_(lambda t: (t % 7).ne(0), v, context=cx)
+            return acc.map(lambda t: t + 1, kept)
+        many = lambda v: acc.map(lambda m: m > 3, acc.fold(acc.max_, 0, acc.map(lambda t: t % 7, v), context=cx))
+        del reads[:]
+        out = acc.run(acc.awhile(many, shrink, acc.use(z, cx), context=cx, limit=6), cx)
+        rz, it = z.copy(), 0
+        while it < 6 and (rz % 7).max() > 3:
+            rz, it = rz[rz % 7 != 0] + 1, it + 1
+        assert np.array_equal(out, rz) and it >= 2
+
+        # a loop inside a loop: the inner one is enqueued ahead, the outer one steps
+        def outer_body(v, k):
+            inner = acc.awhile(lambda w: acc.map(lambda m: m < 100000, acc.fold(acc.max_, 0, w, context=cx)),
+                               lambda w: acc.map(lambda t: t * 3, w), v, context=cx)
+            return acc.map(lambda t: t % 1000 + 1, inner), acc.map(lambda c: c + 1, k)
+        out, k = acc.awhile(lambda v, k: acc.map(lambda c: c < 3, k), outer_body, (acc.use(x, cx), acc.unit(0, "Int32", cx)), context=cx)
+        r = x.copy()
+        for _ in range(3):
+            while r.max() < 100000:
+                r = r * 3
+            r = r % 1000 + 1
+        assert int(acc.run(k, cx)) == 3 and np.array_equal(acc.run(out, cx), r)
+    finally:
+        A.Guard.read = real_read
+        acc.destroy(cx)
+
+
 def test_library_functions_built_from_the_primitives(acc):
     cx = acc.Context(0)
     rng = np.random.default_rng(13)

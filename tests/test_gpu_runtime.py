@@ -235,6 +235,50 @@ def test_scans_larger_than_the_device_on_two_streams(A, ctx):
     scan.destroy()
 
 
+def test_a_loop_enqueued_ahead_under_a_guard(A, ctx):
+    """awhile at the C ABI: twenty iterations of `predicate; latch; body` enqueued without looking at the device, the
+    kernels past the loop's end do nothing, the guard says how many iterations were taken; an instance built
+    without ACC_FLAG_GUARDED is refused on a stream that is under a guard"""
+    I64 = (1, "Int64")
+    n = 100003
+    x = np.random.default_rng(10).integers(1, 50, n).astype(np.int64)
+    G = A.FLAG_GUARDED
+    dbl = ctx.skeleton(A.SKEL_MAP, "Int64", env=[I64], out_rank=1, get="arrIn0_0[ix] * 2", flags=G)
+    mx = ctx.skeleton(A.SKEL_FOLD, "Int64", env=[I64], out_rank=0, get="arrIn0_0[ix]", combine="acc_max(x, y)", seed="0", flags=G)
+    small = ctx.skeleton(A.SKEL_MAP, "Word8", env=[(0, "Int64")], out_rank=0, get="(Word8)(arrIn0_0[0] < 1000000)", flags=G)
+    plain = ctx.skeleton(A.SKEL_MAP, "Int64", env=[I64], out_rank=1, get="arrIn0_0[ix] * 2")
+    st = ctx.stream()
+    guard = A.Guard(ctx)
+    bufs = [ctx.array(x)] + [ctx.array(np.full(n, -1, np.int64)) for _ in range(20)]
+    top, flag = ctx.empty((), np.int64), ctx.empty((), np.uint8)
+    say("twenty iterations enqueued ahead; the doubling stops when the largest element passes a million")
+    guard.attach(st)
+    guard.reset(st)
+    for k in range(20):
+        mx.fold([bufs[k]], n, top, stream=st)
+        small.map([top], flag, stream=st)
+        guard.latch(flag, st)
+        dbl.map([bufs[k]], bufs[k + 1], stream=st)
+    with pytest.raises(A.AccError) as e:
+        plain.map([bufs[0]], bufs[1], stream=st)
+    assert e.value.code == A.ERR_INVALID and "ACC_FLAG_GUARDED" in str(e.value)
+    alive, count = guard.read(st)
+    ref, steps = x.copy(), 0
+    while ref.max() < 1000000:
+        ref, steps = ref * 2, steps + 1
+    assert not alive and count == steps and 10 < steps < 20
+    assert np.array_equal(bufs[count].get(), ref)
+    assert np.all(bufs[count + 1].get() == -1) and np.all(bufs[20].get() == -1)       # the iterations past the end wrote nothing
+    guard.detach(st)
+    plain.map([bufs[0]], bufs[1], stream=st)              # the stream takes any instance again
+    dbl.map([bufs[0]], bufs[2], stream=st)                # and a guarded instance runs unconditionally off a guard
+    ctx.sync()
+    assert np.array_equal(bufs[1].get(), x * 2) and np.array_equal(bufs[2].get(), x * 2)
+    guard.destroy()
+    for s_ in (dbl, mx, small, plain):
+        s_.destroy()
+
+
 def test_one_skeleton_launched_from_several_threads(A, ctx):
     """the reference runs every computation in a bound thread of its own (State.hs:84-92):
     threads sharing a context and a skeleton, each on its own stream, misaligned inputs so
