@@ -97,7 +97,7 @@ acc_cache_clear acc_module_load acc_module_unload acc_module_get_function acc_fu
 acc_launch acc_launch_grid acc_skel_create acc_skel_destroy acc_skel_source acc_skel_preview acc_skel_compile_only
 acc_skel_get_info acc_exec_map acc_exec_fold acc_exec_foldseg acc_exec_foldseg_nd acc_exec_scan acc_exec_scan_noalloc acc_exec_permute
 acc_exec_stencil acc_exec_stencil2 acc_exec_stencil_iterate acc_guard_create acc_guard_destroy acc_guard_reset
-acc_guard_latch acc_guard_read acc_stream_set_guard acc_memtable_create acc_memtable_destroy
+acc_guard_latch acc_guard_read acc_stream_set_guard acc_trace_start acc_trace_stop acc_memtable_create acc_memtable_destroy
 acc_memtable_malloc acc_memtable_acquire acc_memtable_release acc_memtable_free acc_memtable_insert_unmanaged
 acc_memtable_reclaim acc_memtable_get_stats""".split()
 
@@ -172,6 +172,8 @@ def lib():
         L.acc_guard_latch.argtypes = [C.c_void_p, AP, C.c_void_p]
         L.acc_guard_read.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_int32), C.POINTER(C.c_int64)]
         L.acc_stream_set_guard.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+        L.acc_trace_start.argtypes = [C.c_void_p]
+        L.acc_trace_stop.argtypes = [C.c_void_p, C.POINTER(C.c_int32), C.POINTER(C.c_double)]
         L.acc_memtable_create.argtypes = [C.c_void_p, C.c_uint64, C.POINTER(C.c_void_p)]
         L.acc_memtable_destroy.argtypes = [C.c_void_p]
         L.acc_memtable_malloc.argtypes = [C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint64, C.c_int, C.POINTER(C.c_int)]
@@ -366,6 +368,15 @@ class Context(object):
 
     def sync(self):
         check(lib().acc_context_sync(self.handle))
+
+    def trace_start(self):
+        check(lib().acc_trace_start(self.handle))
+
+    def trace_stop(self):
+        """(launches, milliseconds on the device) of what this thread launched since trace_start"""
+        n, ms = C.c_int32(), C.c_double()
+        check(lib().acc_trace_stop(self.handle, C.byref(n), C.byref(ms)))
+        return n.value, ms.value
 
     def trim(self):
         """Free the scratch blocks that are not in use; returns the bytes given back."""

@@ -69,9 +69,28 @@ class Args {
 // Every kernel launch of the drivers.  ACC_HIP_DEBUG=dump-exec prints one line per launch -- entry<<<grid, block,
 // lds>>> and the time on the device -- as the reference's -ddump-exec does (Debug.hs:41-76, hooked at
 // Execute.hs:975-982); timing a launch means waiting for it, so the trace serialises the stream.
+// acc_trace_start .. acc_trace_stop on a thread: an event before and one behind every launch it makes
+struct Trace {
+  bool on = false;
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> spans;
+};
+thread_local Trace t_trace;
+
 hipError_t launch_kernel(hipFunction_t f, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned by, unsigned bz, unsigned lds,
                          hipStream_t st, void **args, void **extra)
 {
+  if (t_trace.on) {
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    const bool timed = hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess && hipEventRecord(e0, st) == hipSuccess;
+    const hipError_t rc = hipModuleLaunchKernel(f, gx, gy, gz, bx, by, bz, lds, st, args, extra);
+    if (timed && rc == hipSuccess && hipEventRecord(e1, st) == hipSuccess) {
+      t_trace.spans.emplace_back(e0, e1);
+    } else {
+      if (e0) (void)hipEventDestroy(e0);
+      if (e1) (void)hipEventDestroy(e1);
+    }
+    return rc;
+  }
   static const bool trace = [] {
     const char *e = std::getenv("ACC_HIP_DEBUG");
     return e && std::strstr(e, "dump-exec");
@@ -210,6 +229,40 @@ int64_t resident(const acc_skel_s *s, int variant) { return (int64_t)s->ctx->pro
 }  // namespace
 
 extern "C" {
+
+int acc_trace_start(acc_context ctx)
+{
+  if (!ctx) return fail(ACC_ERR_INVALID, "acc_trace_start: NULL context");
+  if (t_trace.on) return fail(ACC_ERR_INVALID, "acc_trace_start: this thread is tracing already");
+  t_trace.on = true;
+  return ACC_OK;
+}
+
+int acc_trace_stop(acc_context ctx, int32_t *launches, double *gpu_ms)
+{
+  if (!ctx) return fail(ACC_ERR_INVALID, "acc_trace_stop: NULL context");
+  if (!t_trace.on) return fail(ACC_ERR_INVALID, "acc_trace_stop: this thread is not tracing");
+  t_trace.on = false;
+  int rc = ctx->make_current();
+  double total = 0.0;
+  int32_t count = 0;
+  for (auto &span : t_trace.spans) {
+    float ms = 0.0f;
+    if (rc == ACC_OK) {
+      hipError_t e = hipEventSynchronize(span.second);
+      if (e == hipSuccess) e = hipEventElapsedTime(&ms, span.first, span.second);
+      if (e != hipSuccess) rc = acc::fail_hip(e, "acc_trace_stop");
+    }
+    total += ms;
+    ++count;
+    (void)hipEventDestroy(span.first);
+    (void)hipEventDestroy(span.second);
+  }
+  t_trace.spans.clear();
+  if (launches) *launches = count;
+  if (gpu_ms) *gpu_ms = total;
+  return rc;
+}
 
 int acc_exec_map(acc_skel s, const acc_array *env, const acc_array *out, acc_stream stream)
 {

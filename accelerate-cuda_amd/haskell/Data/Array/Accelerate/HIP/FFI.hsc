@@ -315,6 +315,10 @@ foreign import ccall safe   "acc_guard_latch"      c_guardLatch     :: Guard -> 
 foreign import ccall safe   "acc_guard_read"       c_guardRead      :: Guard -> Stream -> Ptr Int32 -> Ptr Int64 -> IO Status
 foreign import ccall safe   "acc_stream_set_guard" c_streamSetGuard :: Context -> Stream -> Guard -> IO Status
 
+-- Debug.hs:41-76: time on the device of the launches a thread makes
+foreign import ccall safe   "acc_trace_start" c_traceStart :: Context -> IO Status
+foreign import ccall safe   "acc_trace_stop"  c_traceStop  :: Context -> Ptr Int32 -> Ptr CDouble -> IO Status
+
 -- Array/Remote.hs, Array/Table.hs, Array/Prim.hs:177-192: the memory table
 foreign import ccall safe   "acc_memtable_create"           c_memtableCreate          :: Context -> Word64 -> Ptr MemTable -> IO Status
 foreign import ccall safe   "acc_memtable_destroy"          c_memtableDestroy         :: MemTable -> IO Status

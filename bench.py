@@ -29,7 +29,6 @@ for p in (ROOT, os.path.join(ROOT, "accelerate-cuda_amd")):
 import numpy as np  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
-SCANL_HBM_TRAFFIC_BYTES = 542500000
 
 
 def log(*a):
@@ -76,6 +75,51 @@ class Timer(object):
         return wall_ms, event_ms
 
 
+def cpu_leg(fn, what, bytes_per_call, budget_s=3.0):
+    """the oracle's restatement of the reference's algorithm, one thread, timed for about `budget_s` seconds"""
+    reps, t0 = 0, time.perf_counter()
+    while reps == 0 or time.perf_counter() - t0 < budget_s:
+        fn()
+        reps += 1
+    per = (time.perf_counter() - t0) / reps
+    return {"value": round(bytes_per_call / per / 1e9, 3), "unit": "GB/s", "ms_per_step": round(per * 1e3, 3), "cores": 1, "kind": "port",
+            "sample": "%s, %d repetition(s), 1 thread of %d host cores; an upper bound on the boxed Haskell interpreter"
+                      % (what, reps, os.cpu_count())}
+
+
+def end_to_end(ctx, uploads, run, download, reps=3):
+    """what the reference's `run1` does around its kernels (CUDA.hs:382-389, Execute.hs:146-154): the operands go from
+    pageable host memory to the device, the kernels run, the result comes back.  `uploads` pairs device arrays with the
+    host arrays they take; best of `reps`."""
+    best = None
+    for _ in range(reps):
+        ctx.sync()
+        t0 = time.perf_counter()
+        for d, h in uploads:
+            d.set(h)
+        run()
+        out = download.get()
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    moved = sum(h.nbytes for _, h in uploads) + out.nbytes
+    return {"ms": round(best * 1e3, 3), "host_bytes_moved": int(moved),
+            "note": "H2D of the operands from pageable memory + kernels + D2H of the result, device buffers reused; not the headline"}
+
+
+def profiled_traffic(kernel):
+    """HBM bytes per launch of `kernel` as rocprofv3 counted them (FETCH_SIZE and WRITE_SIZE, each scaled by what the
+    same counter reads for a plain copy of known size): read from the committed summary, not measured in this run"""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic_per_launch.txt")
+    try:
+        for line in open(path):
+            f = line.split()
+            if len(f) >= 3 and f[0] == "traffic" and f[1] == kernel:
+                return {"bytes": int(float(f[2])), "source": "profiles/hbm_traffic_per_launch.txt"}
+    except OSError:
+        pass
+    return None
+
+
 def result(name, wall_ms, event_ms, launches_per_step, bytes_per_launch, elements_per_step, extra=None):
     launch_ms = event_ms / launches_per_step
     gbs = bytes_per_launch / (launch_ms * 1e-3) / 1e9
@@ -86,6 +130,10 @@ def result(name, wall_ms, event_ms, launches_per_step, bytes_per_launch, element
          "elements_per_s": round(elements_per_step / (event_ms * 1e-3), 1)}
     if extra:
         r.update(extra)
+    t = profiled_traffic(r.pop("traffic_key", None))
+    if t:
+        r["hbm_traffic_bytes"], r["hbm_traffic_source"] = t["bytes"], t["source"]
+        r["traffic_over_algorithmic"] = round(t["bytes"] / float(bytes_per_launch), 3)
     log("  %-28s %9.3f us/launch  %8.1f GB/s  %5.1f%% of HBM peak" % (name, launch_ms * 1e3, gbs, 100 * gbs / HBM_PEAK_GBS))
     return r
 
@@ -145,8 +193,9 @@ def main():
             def step(i, s=s, ods=ods):
                 return lambda: A.check(L.acc_exec_scan(s.handle, env_s[i], n, C.byref(ods[i]), None, stream))
             w, e = T.run([step(i) for i in range(S)])
-            sk[kind] = result(kind + " (+) Int32 2^26", w, e, 1, 2 * n * 4 + 4, n)
+            sk[kind] = result(kind + " (+) Int32 2^26", w, e, 1, 2 * n * 4 + 4, n, {"traffic_key": kind})
             if kind == "scanl":
+                sk[kind]["end_to_end"] = end_to_end(ctx, [(dxs[0], x)], step(0), outs[0])
                 headline = dict(sk[kind], wall_ms=w, event_ms=e)
                 # size-independent check: the last element is the sum, the first the seed
                 got = outs[S - 1].get()
@@ -184,7 +233,7 @@ def main():
             return lambda: A.check(L.acc_exec_map(cp.handle, env_s[i], C.byref(ods[i]), stream))
         w, e = T.run([step(i) for i in range(S)])
         assert np.array_equal(outs[S - 1].get(), x)
-        sk["map_copy"] = result("map id Int32 2^26 (copy)", w, e, 1, 2 * n * 4, n)
+        sk["map_copy"] = result("map id Int32 2^26 (copy)", w, e, 1, 2 * n * 4, n, {"traffic_key": "map_copy"})
         del dxs, outs, env_s
         fx = x.astype(np.float32)
         fy = fx[::-1].copy()
@@ -198,6 +247,11 @@ def main():
         w, e = T.run([step(i) for i in range(S)])
         assert np.array_equal(fo[S - 1].get(), fx * fy)
         sk["zipwith_mul"] = result("zipWith (*) Float32 2^26", w, e, 1, 3 * n * 4, n)
+        sk["zipwith_mul"]["end_to_end"] = end_to_end(ctx, [(dfx[0], fx), (dfy[0], fy)], step(0), fo[0])
+        if not args.no_cpu:
+            from oracle import oracle as orc
+            orc.build()
+            sk["zipwith_mul"]["cpu_baseline"] = cpu_leg(lambda: orc.zipwith_mul_f32(fx, fy), "oracle/acc_oracle.c orc_zipwith_mul_f32, full 2^26 elements", 3 * n * 4)
         del dfx, dfy, fo, env2, x, fx, fy
 
     # ---------------------------------------------------------------- 1: dot product
@@ -219,7 +273,13 @@ def main():
         w, e = T.run([step(i) for i in range(Sd)])
         truth = float(np.dot(x.astype(np.float64), y.astype(np.float64)))
         sk["dot"] = result("fold (+) 0 . zipWith (*) 2^24", w, e, 1, 2 * nd * 4 + 4, nd,
-                           {"result": float(o.get()), "float64_truth": truth, "GFLOP_per_s": round(2 * nd / (e * 1e-3) / 1e9, 1)})
+                           {"result": float(o.get()), "float64_truth": truth, "GFLOP_per_s": round(2 * nd / (e * 1e-3) / 1e9, 1),
+                            "traffic_key": "foldAll"})
+        sk["dot"]["end_to_end"] = end_to_end(ctx, [(dxs[0], x), (dys[0], y)], step(0), o)
+        if not args.no_cpu:
+            from oracle import oracle as orc
+            orc.build()
+            sk["dot"]["cpu_baseline"] = cpu_leg(lambda: orc.dot_f32(x, y), "oracle/acc_oracle.c orc_dot_f32, full 2^24 elements", 2 * nd * 4 + 4)
         del dxs, dys, env_s
 
     # ---------------------------------------------------------------- 3: histograms
@@ -241,7 +301,15 @@ def main():
         got = out.get()
         assert os.environ.get("ACC_BENCH_NOCHECK") or (int(got.sum()) == n and np.array_equal(got, np.bincount(keys, minlength=bins))), "histogram mismatch"
         sk[name] = result("permute (+) %d bins" % bins, w, e, 1, n * 4 + 2 * bins * 4, n,
-                          {"Gkeys_per_s": round(n / (e * 1e-3) / 1e9, 2), "note": "step = defaults copy + permute kernel"})
+                          {"Gkeys_per_s": round(n / (e * 1e-3) / 1e9, 2), "note": "step = defaults copy + permute kernel(s) + merge",
+                           "traffic_key": name})
+        sk[name]["end_to_end"] = end_to_end(ctx, [(dks[0], keys)], step(0), out)
+        if not args.no_cpu:
+            from oracle import oracle as orc
+            orc.build()
+            zeros = np.zeros(bins, np.int32)
+            sk[name]["cpu_baseline"] = cpu_leg(lambda: orc.permute(orc.OP_ADD, zeros, keys), "oracle/acc_oracle.c orc_permute_i32 (source = 1), full 2^26 keys",
+                                               n * 4 + 2 * bins * 4)
         del dks, env_s, keys
 
     # ---------------------------------------------------------------- 4: stencils
@@ -261,12 +329,26 @@ def main():
         def step(i):
             return lambda: A.check(L.acc_exec_stencil_iterate(gauss.handle, None, C.byref(ad[i]), C.byref(bd[i]), 10, stream, C.byref(rib)))
         w, e = T.run([step(i) for i in range(S)])
-        sk["gaussian3x3_clamp_x10"] = result("stencil 3x3 gaussian x10", w, e, 10, 2 * h * w_ * 4, 10 * h * w_)
+        sk["gaussian3x3_clamp_x10"] = result("stencil 3x3 gaussian x10", w, e, 10, 2 * h * w_ * 4, 10 * h * w_, {"traffic_key": "stencil_gaussian"})
+
+        class _where(object):              # the result of the ten applications lies in a or in b
+            @staticmethod
+            def get():
+                return (b_s[0] if rib.value else a_s[0]).get()
+        sk["gaussian3x3_clamp_x10"]["end_to_end"] = end_to_end(ctx, [(a_s[0], img)], step(0), _where)
+        if not args.no_cpu:
+            from oracle import oracle as orc
+            orc.build()
+            g_taps = [(dy, dx, c) for (dy, dx), c in zip(taps, [1, 2, 1, 2, 4, 2, 1, 2, 1])]
+            sk["gaussian3x3_clamp_x10"]["cpu_baseline"] = cpu_leg(
+                lambda: orc.stencil2d(img, g_taps, 16.0, "clamp", iters=1),
+                "oracle/acc_oracle.c orc_stencil2d_iter_f32, ONE of the ten applications on the full 8192x8192 image (figures per application)",
+                2 * h * w_ * 4, budget_s=2.0)
 
         def step2(i):
             return lambda: A.check(L.acc_exec_stencil(lap.handle, None, C.byref(ad[i]), C.byref(bd[i]), stream))
         w, e = T.run([step2(i) for i in range(S)])
-        sk["laplace5_mirror"] = result("stencil 5-point laplacian", w, e, 1, 2 * h * w_ * 4, h * w_)
+        sk["laplace5_mirror"] = result("stencil 5-point laplacian", w, e, 1, 2 * h * w_ * 4, h * w_, {"traffic_key": "stencil_laplace"})
         del a_s, b_s, img
 
     # ---------------------------------------------------------------- 5: sparse matrix-vector product
@@ -289,13 +371,77 @@ def main():
         y = ys[S - 1]
         sk["smvm"] = result("foldSeg (+) . zipWith (*) . gather", w, e, 1, nnz * 8 + rows * 8 + xv.size * 4, nnz,
                             {"nnz": int(nnz), "GFLOP_per_s": round(2 * nnz / (e * 1e-3) / 1e9, 1),
-                             "note": "segment offsets precomputed on the device (scanl over the 2^20 lengths is not in the step)"})
+                             "note": "segment offsets precomputed on the device (scanl over the 2^20 lengths is not in the step)",
+                             "traffic_key": "foldSeg"})
+        sk["smvm"]["end_to_end"] = end_to_end(ctx, [(dv[0], vals), (dc[0], cols), (dxv[0], xv), (doff[0], offs)], step(0), ys[0])
+        if not args.no_cpu:
+            from oracle import oracle as orc
+            orc.build()
+            sk["smvm"]["cpu_baseline"] = cpu_leg(lambda: orc.smvm_f32(vals, cols, offs, xv), "oracle/acc_oracle.c orc_smvm_f32, full 2^20 rows",
+                                                 nnz * 8 + rows * 8 + xv.size * 4)
         # composition check on the device result: y = A x in float64 within 1e-4 of the row's magnitude
         import scipy.sparse as sp
         Amat = sp.csr_matrix((vals.astype(np.float64), cols, offs), shape=(rows, xv.size))
         truth = Amat @ xv.astype(np.float64)
         mag = abs(Amat) @ np.abs(xv.astype(np.float64))
         assert np.all(np.abs(y.get() - truth) <= 1e-4 * np.maximum(np.abs(truth), 1e-3 * mag) + 1e-30), "smvm mismatch"
+
+    # ---------------------------------------------------------------- the same three computations built by the front end
+    # (dot, scanl and SMVM written as array programs: what `run1` of the front end generates, compiles and launches
+    # for them, timed kernel by kernel (acc_trace_start / acc_trace_stop: an event before and behind every launch),
+    # beside the hand-written fragments above.  Host time per call is Python's and is not in these figures; a launch
+    # onto an idle device carries a few microseconds of dispatch latency that back-to-back launches do not show.)
+    if want("frontend"):
+        log("front end: dotp, scanl and smvm as array programs ...")
+        import accelerate_hip as acc
+        fcx = acc.Context(0)
+        fcx.N_STREAMS = 1                           # one stream: consecutive calls must not share the device, or each looks slower
+        add = lambda a, b: a + b                    # noqa: E731
+        K = max(4, min(args.steps, 20))
+
+        def front(build, sets):
+            acc_r = build(0)                        # builds the skeletons, uploads the operands of set 0
+            for i in range(1, sets):
+                acc_r = build(i)
+            fcx.ctx.sync()
+            fcx.ctx.trace_start()                   # an event before and behind every launch the drivers make
+            for k in range(K):
+                acc_r = build(k % sets)
+            launches, ms = fcx.ctx.trace_stop()
+            return acc_r, round(ms * 1e3 / K, 3), launches // K
+
+        fe = {}
+        nd = 1 << 24
+        x, y = wl.dot_inputs(nd)
+        Sd = 4 * S
+        xs, ys_ = [acc.use(x.copy(), fcx) for _ in range(Sd)], [acc.use(y.copy(), fcx) for _ in range(Sd)]
+        r, us, nk = front(lambda i: acc.fold(add, 0.0, acc.zipWith(lambda a, b: a * b, xs[i], ys_[i]), context=fcx), Sd)
+        fe["dot"] = {"gpu_us_per_call": us, "kernels_per_call": nk, "direct_avg_launch_us": sk.get("dot", {}).get("avg_launch_us"),
+                     "result": float(acc.run(r, fcx))}
+        log("  front end dotp                 %9.3f us/call on the device, %d kernel(s)" % (us, nk))
+        del xs, ys_, r
+        xsc = wl.scan_input(n)
+        xs = [acc.use(xsc.copy(), fcx) for _ in range(S)]
+        r, us, nk = front(lambda i: acc.scanl(add, 0, xs[i], context=fcx), S)
+        got = acc.run(r, fcx)
+        assert int(got[-1]) == int(xsc.sum(dtype=np.int64)), "front end scanl mismatch"
+        fe["scanl"] = {"gpu_us_per_call": us, "kernels_per_call": nk, "direct_avg_launch_us": sk.get("scanl", {}).get("avg_launch_us")}
+        log("  front end scanl                %9.3f us/call on the device, %d kernel(s)" % (us, nk))
+        del xs, r, got, xsc
+        vals, cols, offs, lens, xv = wl.smvm_inputs()
+        vs, cs = [acc.use(vals.copy(), fcx) for _ in range(S)], [acc.use(cols.copy(), fcx) for _ in range(S)]
+        vecs, ls = [acc.use(xv.copy(), fcx) for _ in range(S)], [acc.use(lens.copy(), fcx) for _ in range(S)]
+
+        def smvm_prog(i):
+            v = vecs[i]
+            return acc.foldSeg(add, 0.0, acc.zipWith(lambda c, a: a * v[c], cs[i], vs[i]), ls[i], context=fcx)
+        r, us, nk = front(smvm_prog, S)
+        fe["smvm"] = {"gpu_us_per_call": us, "kernels_per_call": nk, "direct_avg_launch_us": sk.get("smvm", {}).get("avg_launch_us"),
+                      "note": "per call: scanl of the 2^20 segment lengths into offsets, then foldSeg (the direct figure is foldSeg alone)"}
+        log("  front end smvm                 %9.3f us/call on the device, %d kernel(s): offsets scan + foldSeg" % (us, nk))
+        del vs, cs, vecs, ls, r
+        sk["front_end"] = fe
+        acc.destroy(fcx)
 
     # ---------------------------------------------------------------- not a configuration: fold along rows of 64
     # (only when named: the rows of a rank-2 array are segments whose starts lie a multiple of 32 elements apart, the
@@ -322,7 +468,12 @@ def main():
         del dms, env_s, rs, m
 
     if headline is None:     # --only without scan: report whatever ran first
-        k0 = sorted(sk)[0]
+        timed = sorted(k for k in sk if "ms_per_step" in sk[k])
+        if not timed:
+            print(json.dumps({"skeletons": sk}))
+            ctx.close()
+            return
+        k0 = timed[0]
         headline = dict(sk[k0], wall_ms=sk[k0]["ms_per_step"], event_ms=sk[k0]["event_ms_per_step"])
         workload = k0
     else:
@@ -337,9 +488,7 @@ def main():
                    "timing": "kernel launches back to back on one stream, inputs device-resident, consecutive launches on different buffer sets; %d ms of untimed launches once before the first configuration's warm-up steps" % int(Timer.DEVICE_WARMUP_MS)},
         "roofline": {"bound": "hbm", "achieved": headline["GB_per_s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(headline["GB_per_s"] / HBM_PEAK_GBS, 4),
-                     # HBM bytes per scanl launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the
-                     # plain copy of the same size: profiles/scan_2p26_hbm_traffic_pmc.txt
-                     "traffic": SCANL_HBM_TRAFFIC_BYTES if workload.startswith("configs[1]") else None,
+                     "traffic": headline.get("hbm_traffic_bytes"), "traffic_source": headline.get("hbm_traffic_source"),
                      "kernel": "scanl", "avg_launch_us": headline["avg_launch_us"],
                      "algorithmic_bytes_per_launch": headline["algorithmic_bytes_per_launch"]},
         "cpu_baseline": cpu,

@@ -447,6 +447,13 @@ int acc_guard_latch(acc_guard g, const acc_array *pred, acc_stream stream);
 int acc_guard_read(acc_guard g, acc_stream stream, int32_t *alive, int64_t *count);   /* waits for the stream */
 int acc_stream_set_guard(acc_context ctx, acc_stream stream, acc_guard g);
 
+/* Time on the device of the kernels a thread launches through the skeleton drivers between the two calls: an event
+ * before and one behind every launch, summed by acc_trace_stop, which waits for them (Debug.hs:41-76 `timed`, hooked
+ * at Execute.hs:975-982; the reference prints one line per launch under -ddump-exec, which ACC_HIP_DEBUG=dump-exec
+ * in the environment does here).  Per thread; the kernels run as usual.                                           */
+int acc_trace_start(acc_context ctx);
+int acc_trace_stop(acc_context ctx, int32_t *launches, double *gpu_ms);
+
 /* =========================================================================
  * C. memory table
  * ========================================================================= */

@@ -543,13 +543,10 @@ int orc_stencil1d_f32(const float *in, int64_t n, int ntaps, const int32_t *dx,
 int64_t orc_boundary_index(int mode, int64_t i, int64_t sz) { return bmap(mode, i, sz); }
 
 /* ------------------------------------------------------------------------ */
-/* elementwise producers used by the map-family tests                        */
+/* zipWith (*) xs ys (Mapping.hs:59-78: one element function application per
+ * index): every product rounded to Float32.  The CPU side of the map-family
+ * benchmark leg.                                                            */
 void orc_zipwith_mul_f32(const float *x, const float *y, int64_t n, float *out)
 {
   for (int64_t i = 0; i < n; ++i) out[i] = x[i] * y[i];
-}
-
-void orc_saxpy_f32(float a, const float *x, const float *y, int64_t n, float *out)
-{
-  for (int64_t i = 0; i < n; ++i) { float p = a * x[i]; out[i] = p + y[i]; }
 }

@@ -195,6 +195,15 @@ def permute(op, defaults, dst, src=None):
     return out
 
 
+def zipwith_mul_f32(x, y):
+    x = _c(x, np.float32)
+    y = _c(y, np.float32)
+    assert x.shape == y.shape
+    out = np.empty_like(x)
+    lib().orc_zipwith_mul_f32(_p(x), _p(y), C.c_int64(x.size), _p(out))
+    return out
+
+
 def backpermute(arr, idx):
     arr = _c(arr)
     idx = _c(idx, np.int32)

@@ -197,6 +197,16 @@ def _csr(nrows, ncols, mean, integer=False):
     return vals, cols, offs, x
 
 
+def test_zipwith_mul_rounds_every_product_to_float32(orc):
+    rng = np.random.default_rng(33)
+    x = (rng.standard_normal(10007) * 1e3).astype(np.float32)
+    y = (rng.standard_normal(10007) * 1e-3).astype(np.float32)
+    got = orc.zipwith_mul_f32(x, y)
+    assert np.array_equal(got, x * y)                                         # numpy multiplies in Float32 as well
+    assert np.array_equal(got, (x.astype(np.float64) * y.astype(np.float64)).astype(np.float32))   # = the rounded exact product
+    assert orc.zipwith_mul_f32(x[:0], y[:0]).size == 0
+
+
 def test_foldseg_vs_numpy_and_empty_segments(orc):
     vals, _, offs, _ = _csr(200, 50, 8, integer=True)
     vi = vals.astype(np.int32)
