@@ -833,29 +833,28 @@ def _taps(pattern, rank):
     return offs
 
 
+def _boundary_constant(value, ctype):
+    """the value outside the array under a constant boundary, as text: of a tuple source one literal per component"""
+    if value is None:
+        return None
+    if isinstance(ctype, tuple):
+        if not isinstance(value, (tuple, list)) or len(value) != len(ctype):
+            raise TypeError("the boundary constant of a stencil over %d-tuples is a %d-tuple" % (len(ctype), len(ctype)))
+        return ", ".join(_literal(v, t) for v, t in zip(value, ctype))
+    return _literal(value, ctype)
+
+
 def stencil(pattern, f, boundary, a, context=None, constant_value=None):
     """result[i] = f(a[i + o] for o in pattern); boundary is "clamp", "mirror", "wrap" or "constant"
     (Stencil/Extra.hs:112-116); the source is made manifest first, as in the reference (Execute.hs:413-425)"""
     cx = _context(context, a)
     src = _force(a, cx)
-    if isinstance(src.ctype, tuple):
-        # an array of pairs is two arrays: the same pattern over both, as a stencil2 (the sources of the
-        # stencil kernels are arrays of scalars)
-        if len(src.ctype) != 2:
-            raise TypeError("stencil over an array of %d-tuples: take it apart into pairs and scalars first" % len(src.ctype))
-        if constant_value is not None and not isinstance(constant_value, (tuple, list)):
-            raise TypeError("the boundary constant of a stencil over pairs is a pair")
-        c1, c2 = (None, None) if constant_value is None else constant_value
-        comp = [Acc(src.shape, t, manifest=m) for t, m in zip(src.ctype, src.manifest.comps)]
-        return stencil2(pattern, pattern, lambda ts, us: f(*[lift(t, u) for t, u in zip(ts, us)]), boundary, comp[0],
-                        boundary, comp[1], context=cx, constant1=c1, constant2=c2)
     rank = len(src.shape)
     taps = _taps(pattern, rank)
-    res = Exp.of(f(*[Exp(src.ctype, "t%d" % k) for k in range(len(taps))]))
+    res = Exp.of(f(*[_var(src.ctype, "t%d" % k) for k in range(len(taps))]))        # a tap of a tuple source: its members
     arrays, sig, fr = _assemble(stencil_fn=res.text)
     sk = cx.skeleton(A.SKEL_STENCIL, _elt(res.ctype), sig, out_rank=rank, taps=taps, boundary=boundary,
-                     boundary_constant=None if constant_value is None else _literal(constant_value, src.ctype),
-                     stencil_in=src.ctype, **fr)
+                     boundary_constant=_boundary_constant(constant_value, src.ctype), stencil_in=_elt(src.ctype), **fr)
     out = _empty(cx, src.shape, res.ctype)
     cx.launch(arrays + [src.manifest], [out], lambda i, o, s: sk.stencil(i[:-1], i[-1], o[0], stream=s))
     return Acc(src.shape, res.ctype, manifest=out)
@@ -867,12 +866,11 @@ def stencil2(pattern1, pattern2, f, boundary1, a, boundary2, b, context=None, co
     s1, s2 = _force(a, cx), _force(b, cx)
     rank = len(s1.shape)
     t1, t2 = _taps(pattern1, rank), _taps(pattern2, rank)
-    res = Exp.of(f([Exp(s1.ctype, "t%d" % k) for k in range(len(t1))], [Exp(s2.ctype, "u%d" % k) for k in range(len(t2))]))
+    res = Exp.of(f([_var(s1.ctype, "t%d" % k) for k in range(len(t1))], [_var(s2.ctype, "u%d" % k) for k in range(len(t2))]))
     arrays, sig, fr = _assemble(stencil_fn=res.text)
     sk = cx.skeleton(A.SKEL_STENCIL2, _elt(res.ctype), sig, out_rank=rank, taps=t1, boundary=boundary1, taps2=t2, boundary2=boundary2,
-                     boundary_constant=None if constant1 is None else _literal(constant1, s1.ctype),
-                     boundary2_constant=None if constant2 is None else _literal(constant2, s2.ctype),
-                     stencil_in=s1.ctype, stencil_in2=s2.ctype, **fr)
+                     boundary_constant=_boundary_constant(constant1, s1.ctype), boundary2_constant=_boundary_constant(constant2, s2.ctype),
+                     stencil_in=_elt(s1.ctype), stencil_in2=_elt(s2.ctype), **fr)
     shape = _meet(s1.shape, s2.shape)
     out = _empty(cx, shape, res.ctype)
     cx.launch(arrays + [s1.manifest, s2.manifest], [out], lambda i, o, s: sk.stencil2(i[:-2], i[-2], i[-1], o[0], stream=s))

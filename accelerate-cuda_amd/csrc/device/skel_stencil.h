@@ -43,13 +43,17 @@
  * intersection of the two extents and its element is a function of both
  * neighbourhoods (taps t0.. of the first source, u0.. of the second).
  *
- * Generated definitions expected: ACC_ELT, ACC_IN_ELT, ACC_ENV_PARAMS,
- * ACC_ENV_ASSUME, ACC_OUT_PARAMS, ACC_STENCIL_RANK (1|2|3), ACC_RADIUS_Z, ACC_RADIUS_Y,
- * ACC_RADIUS_X (the larger of the two sources'), ACC_BOUNDARY,
- * ACC_BOUNDARY_CONSTANT, ACC_STENCIL_TAPS(READ), ACC_STENCIL_FN, ACC_TILE_H,
- * ACC_PREFETCH, ACC_BLOCK, ACC_ALIGNED, ACC_STENCIL_SOURCES (1|2) and for the
- * second source ACC_IN2_ELT, ACC_BOUNDARY2, ACC_BOUNDARY2_CONSTANT,
- * ACC_STENCIL_TAPS2(READ).
+ * A source of tuples (Stencil/Extra.hs:53-128 reads every component) is one
+ * array per component: each gets its own register window, and a tap is a
+ * struct of the components' values (t0.a1, t0.a0).
+ *
+ * Generated definitions expected: ACC_ELT, ACC_ENV_PARAMS, ACC_ENV_ASSUME,
+ * ACC_OUT_PARAMS, ACC_STENCIL_RANK (1|2|3), ACC_RADIUS_Z, ACC_RADIUS_Y,
+ * ACC_RADIUS_X (the larger of the two sources'), ACC_STENCIL_FN, ACC_TILE_H,
+ * ACC_PREFETCH, ACC_BLOCK, ACC_ALIGNED, ACC_STENCIL_SOURCES (1|2) and per
+ * source n = 1, 2: ACC_BOUNDARY (ACC_BOUNDARY2), ACC_SRC<n>_COMPONENTS(X, arg),
+ * ACC_SRC<n>_PARAMS, ACC_IN<n>_ELT, ACC_STENCIL_TAPS<n>(READ) with
+ * READ(component, dz, dy, dx).
  */
 
 #define ACC_SVEC  4                                   /* results per lane and row */
@@ -213,22 +217,17 @@ struct acc_strip_source {
   }
 };
 
+/* A source is one array per component of its element type; the generator hands over, per source, the list of its
+ * components ACC_SRC<n>_COMPONENTS(X, arg) = X(component, type, value outside, arg) ..., highest component first, and
+ * its kernel parameters ACC_SRC<n>_PARAMS in the same order (for stencil2 each source with its own extents in front,
+ * Stencil.hs:146-152).  Every component gets a register window of its own; they all move together. */
 #if ACC_STENCIL_SOURCES == 2
 #define ACC_STENCIL_ENTRY stencil2
-/* each source comes with its own extents (Stencil.hs:146-152) */
-#if ACC_STENCIL_RANK == 3
-#define ACC_SOURCE_PARAMS , const Int64 shStencil1_2, const Int64 shStencil1_1, const Int64 shStencil1_0, const ACC_IN_ELT *__restrict__ arrStencil1_0 \
-                          , const Int64 shStencil2_2, const Int64 shStencil2_1, const Int64 shStencil2_0, const ACC_IN2_ELT *__restrict__ arrStencil2_0
-#elif ACC_STENCIL_RANK == 2
-#define ACC_SOURCE_PARAMS , const Int64 shStencil1_1, const Int64 shStencil1_0, const ACC_IN_ELT *__restrict__ arrStencil1_0 \
-                          , const Int64 shStencil2_1, const Int64 shStencil2_0, const ACC_IN2_ELT *__restrict__ arrStencil2_0
-#else
-#define ACC_SOURCE_PARAMS , const Int64 shStencil1_0, const ACC_IN_ELT *__restrict__ arrStencil1_0 \
-                          , const Int64 shStencil2_0, const ACC_IN2_ELT *__restrict__ arrStencil2_0
-#endif
+#define ACC_SOURCE_PARAMS ACC_SRC1_PARAMS ACC_SRC2_PARAMS
 #else
 #define ACC_STENCIL_ENTRY stencil
-#define ACC_SOURCE_PARAMS , const ACC_IN_ELT *__restrict__ arrStencil_0
+#define ACC_SOURCE_PARAMS ACC_SRC1_PARAMS
+#define ACC_SRC2_COMPONENTS(X, arg)
 #endif
 
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
@@ -284,44 +283,46 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS ACC_GUARD_PARA
   const int rows = decltype(full_c)::value ? ACC_TILE_H : rows_here;
   const int total = rows + 2 * ACC_RADIUS_Y;              /* source rows this strip touches */
 
-  acc_strip_source<ACC_IN_ELT, ACC_BOUNDARY, fast> a;
+  /* one strip source per component of either source's element: a<c> for the first source, b<c> for the second */
 #if ACC_STENCIL_SOURCES == 2
-  a.base = arrStencil1_0;
-  a.w = shStencil1_0;
-  a.h = 1;
-  a.d = 1;
-#if ACC_STENCIL_RANK >= 2
-  a.h = shStencil1_1;
-#endif
 #if ACC_STENCIL_RANK == 3
-  a.d = shStencil1_2;
-#endif
+#define ACC_SRC1_EXTENTS(o) o.d = shStencil1_2; o.h = shStencil1_1; o.w = shStencil1_0
+#define ACC_SRC2_EXTENTS(o) o.d = shStencil2_2; o.h = shStencil2_1; o.w = shStencil2_0
+#elif ACC_STENCIL_RANK == 2
+#define ACC_SRC1_EXTENTS(o) o.d = 1; o.h = shStencil1_1; o.w = shStencil1_0
+#define ACC_SRC2_EXTENTS(o) o.d = 1; o.h = shStencil2_1; o.w = shStencil2_0
 #else
-  a.base = arrStencil_0;
-  a.d = d;
-  a.h = h;
-  a.w = w;
+#define ACC_SRC1_EXTENTS(o) o.d = 1; o.h = 1; o.w = shStencil1_0
+#define ACC_SRC2_EXTENTS(o) o.d = 1; o.h = 1; o.w = shStencil2_0
 #endif
-  a.outside = (ACC_IN_ELT)(ACC_BOUNDARY_CONSTANT);
-  a.z0 = z0; a.y0 = y0; a.x0 = x0; a.gx = gx; a.lane = lane; a.total = total;
+#define ACC_SRC1_ARRAY(c) arrStencil1_##c
+#define ACC_SRC2_ARRAY(c) arrStencil2_##c
+#else
+#define ACC_SRC1_EXTENTS(o) o.d = d; o.h = h; o.w = w
+#define ACC_SRC1_ARRAY(c) arrStencil_##c
+#endif
+#define ACC_DECLARE_A(c, CT, OUTSIDE, arg)                                         \
+  acc_strip_source<CT, ACC_BOUNDARY, fast> a##c;                                  \
+  a##c.base = ACC_SRC1_ARRAY(c);                                                  \
+  ACC_SRC1_EXTENTS(a##c);                                                         \
+  a##c.outside = (CT)OUTSIDE;                                                     \
+  a##c.z0 = z0; a##c.y0 = y0; a##c.x0 = x0; a##c.gx = gx; a##c.lane = lane; a##c.total = total;
+  ACC_SRC1_COMPONENTS(ACC_DECLARE_A, 0)
+#undef ACC_DECLARE_A
 #if ACC_STENCIL_SOURCES == 2
-  acc_strip_source<ACC_IN2_ELT, ACC_BOUNDARY2, fast> b;
-  b.base = arrStencil2_0;
-  b.w = shStencil2_0;
-  b.h = 1;
-  b.d = 1;
-#if ACC_STENCIL_RANK >= 2
-  b.h = shStencil2_1;
+#define ACC_DECLARE_B(c, CT, OUTSIDE, arg)                                         \
+  acc_strip_source<CT, ACC_BOUNDARY2, fast> b##c;                                 \
+  b##c.base = ACC_SRC2_ARRAY(c);                                                  \
+  ACC_SRC2_EXTENTS(b##c);                                                         \
+  b##c.outside = (CT)OUTSIDE;                                                     \
+  b##c.z0 = z0; b##c.y0 = y0; b##c.x0 = x0; b##c.gx = gx; b##c.lane = lane; b##c.total = total;
+  ACC_SRC2_COMPONENTS(ACC_DECLARE_B, 0)
+#undef ACC_DECLARE_B
 #endif
-#if ACC_STENCIL_RANK == 3
-  b.d = shStencil2_2;
-#endif
-  b.outside = (ACC_IN2_ELT)(ACC_BOUNDARY2_CONSTANT);
-  b.z0 = z0; b.y0 = y0; b.x0 = x0; b.gx = gx; b.lane = lane; b.total = total;
-#define ACC_BOTH(call) do { a.call; b.call; } while (0)
-#else
-#define ACC_BOTH(call) a.call
-#endif
+  /* the same call on every component's window */
+#define ACC_CALL_A(c, CT, OUTSIDE, call) a##c.call;
+#define ACC_CALL_B(c, CT, OUTSIDE, call) b##c.call;
+#define ACC_BOTH(call) do { ACC_SRC1_COMPONENTS(ACC_CALL_A, call) ACC_SRC2_COMPONENTS(ACC_CALL_B, call) } while (0)
 
   ACC_BOTH(gather_halo());
 
@@ -349,11 +350,11 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS ACC_GUARD_PARA
         acc_out_vec res;
 #pragma unroll
         for (int k = 0; k < ACC_SVEC; ++k) {
-#define ACC_WINDOW_READ(dz, dy, dx) a.ring[pz + ACC_RADIUS_Z + (dz)][(s + ACC_RADIUS_Y + (dy)) % ACC_RING].e[ACC_RADIUS_X + k + (dx)]
-          ACC_STENCIL_TAPS(ACC_WINDOW_READ)
+#define ACC_WINDOW_READ(c, dz, dy, dx) a##c.ring[pz + ACC_RADIUS_Z + (dz)][(s + ACC_RADIUS_Y + (dy)) % ACC_RING].e[ACC_RADIUS_X + k + (dx)]
+          ACC_STENCIL_TAPS1(ACC_WINDOW_READ)
 #undef ACC_WINDOW_READ
 #if ACC_STENCIL_SOURCES == 2
-#define ACC_WINDOW_READ(dz, dy, dx) b.ring[pz + ACC_RADIUS_Z + (dz)][(s + ACC_RADIUS_Y + (dy)) % ACC_RING].e[ACC_RADIUS_X + k + (dx)]
+#define ACC_WINDOW_READ(c, dz, dy, dx) b##c.ring[pz + ACC_RADIUS_Z + (dz)][(s + ACC_RADIUS_Y + (dy)) % ACC_RING].e[ACC_RADIUS_X + k + (dx)]
           ACC_STENCIL_TAPS2(ACC_WINDOW_READ)
 #undef ACC_WINDOW_READ
 #endif
@@ -383,6 +384,8 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS ACC_GUARD_PARA
     }
   }
 #undef ACC_BOTH
+#undef ACC_CALL_A
+#undef ACC_CALL_B
   };   /* run */
 
   if (fast_here) {

@@ -986,10 +986,14 @@ static int stencil_once(acc_skel s, const acc_array *env, const acc_array *in, c
   const int64_t w = out->shape[rank - 1];
   const int64_t h = rank >= 2 ? out->shape[rank - 2] : 1;
   const int64_t planes = rank == 3 ? out->shape[0] : 1;
-  // rows start on 16-byte boundaries only if the row pitch allows it
-  auto row_aligned = [&](const acc_array &a, const std::string &type) {
-    const size_t esz = acc::type_size(type) ? acc::type_size(type) : s->spec.elt_size;
-    return aligned16(a.ptr[0]) && (a.shape[rank - 1] * (int64_t)esz) % 16 == 0;
+  // rows start on 16-byte boundaries only if the row pitch allows it: of every component of a source
+  auto row_aligned = [&](const acc_array &a, const std::vector<std::string> &comps) {
+    const int nc = (int)comps.size();
+    for (int c = 0; c < nc; ++c) {
+      const size_t esz = acc::type_size(comps[nc - 1 - c]);          // component c is the (nc - 1 - c)-th in writing order
+      if (!aligned16(a.ptr[c]) || (a.shape[rank - 1] * (int64_t)esz) % 16 != 0) return false;
+    }
+    return true;
   };
   // (of a tuple result: the rows of every component's array)
   const int ncomp = s->ncomp();
@@ -997,14 +1001,15 @@ static int stencil_once(acc_skel s, const acc_array *env, const acc_array *in, c
     const int64_t csz = ncomp == 1 ? (int64_t)s->spec.elt_size : (int64_t)acc::type_size(s->spec.comp_types[ncomp - 1 - c]);
     if ((w * csz) % 16 != 0) aligned = false;
   }
-  if (!row_aligned(*in, s->spec.stencil_in_type)) aligned = false;
+  if (!row_aligned(*in, s->spec.stencil_in_comps)) aligned = false;
   if (in2) {      // each source with its extents (Stencil.hs:146-152)
-    if (!row_aligned(*in2, s->spec.stencil_in2_type)) aligned = false;
+    if (!row_aligned(*in2, s->spec.stencil_in2_comps)) aligned = false;
     bool ignore = true;
     push_out(*in, &args, &ignore);
     push_out(*in2, &args, &ignore);
   } else {
-    args.ptr(in->ptr[0]);
+    bool ignore = true;
+    push_ptrs(in, in->ncomp, &args, &ignore);
   }
   if (w == 0 || h == 0 || planes == 0) return ACC_OK;
   // one wave per strip of 256 columns x tile_h rows
@@ -1022,10 +1027,12 @@ static int stencil_check(acc_skel s, const acc_array *in, const acc_array *out)
   if (!s) return fail(ACC_ERR_INVALID, "acc_exec_stencil: NULL skeleton");
   if (!kind_is(s, {ACC_SKEL_STENCIL})) return fail(ACC_ERR_INVALID, "acc_exec_stencil: skeleton is '%s'", s->entry.c_str());
   ACC_TRY(check_out(s, out, s->spec.out_rank, "result"));
-  ACC_TRY(check_out(s, in, s->spec.out_rank, "source", 1));
+  ACC_TRY(check_out(s, in, s->spec.out_rank, "source", (int)s->spec.stencil_in_comps.size()));
   for (int d = 0; d < out->rank; ++d)
     if (in->shape[d] != out->shape[d]) return fail(ACC_ERR_INVALID, "stencil: source and result differ in shape");
-  if (in->ptr[0] == out->ptr[0] && array_size(*out) > 0) return fail(ACC_ERR_INVALID, "stencil: source and result must not alias");
+  for (int ci = 0; ci < in->ncomp && array_size(*out) > 0; ++ci)
+    for (int co = 0; co < out->ncomp; ++co)
+      if (in->ptr[ci] == out->ptr[co]) return fail(ACC_ERR_INVALID, "stencil: source and result must not alias");
   return ACC_OK;
 }
 
@@ -1040,13 +1047,15 @@ int acc_exec_stencil2(acc_skel s, const acc_array *env, const acc_array *in1, co
   if (!s) return fail(ACC_ERR_INVALID, "acc_exec_stencil2: NULL skeleton");
   if (!kind_is(s, {ACC_SKEL_STENCIL2})) return fail(ACC_ERR_INVALID, "acc_exec_stencil2: skeleton is '%s'", s->entry.c_str());
   ACC_TRY(check_out(s, out, s->spec.out_rank, "result"));
-  ACC_TRY(check_out(s, in1, s->spec.out_rank, "first source", 1));
-  ACC_TRY(check_out(s, in2, s->spec.out_rank, "second source", 1));
+  ACC_TRY(check_out(s, in1, s->spec.out_rank, "first source", (int)s->spec.stencil_in_comps.size()));
+  ACC_TRY(check_out(s, in2, s->spec.out_rank, "second source", (int)s->spec.stencil_in2_comps.size()));
   for (int d = 0; d < out->rank; ++d)
     if (out->shape[d] > std::min(in1->shape[d], in2->shape[d]))
       return fail(ACC_ERR_INVALID, "stencil2: the result is larger than the intersection of the sources' extents");
-  if (array_size(*out) > 0 && (in1->ptr[0] == out->ptr[0] || in2->ptr[0] == out->ptr[0]))
-    return fail(ACC_ERR_INVALID, "stencil2: a source and the result must not alias");
+  for (const acc_array *in : {in1, in2})
+    for (int ci = 0; ci < in->ncomp && array_size(*out) > 0; ++ci)
+      for (int co = 0; co < out->ncomp; ++co)
+        if (in->ptr[ci] == out->ptr[co]) return fail(ACC_ERR_INVALID, "stencil2: a source and the result must not alias");
   return stencil_once(s, env, in1, in2, out, static_cast<hipStream_t>(stream));
 }
 

@@ -69,6 +69,30 @@ int tune(const char *name, int dflt)
   return dflt;
 }
 
+// "a, f(b, c), {d, e}" -> ["a", "f(b, c)", "{d, e}"]: split at the commas that lie inside no bracket
+static std::vector<std::string> split_top_level(const std::string &text)
+{
+  std::vector<std::string> parts;
+  std::string cur;
+  int depth = 0;
+  for (char c : text) {
+    if (c == '(' || c == '{' || c == '[' || c == '<') ++depth;
+    if (c == ')' || c == '}' || c == ']' || c == '>') --depth;
+    if (c == ',' && depth == 0) {
+      parts.push_back(cur);
+      cur.clear();
+    } else {
+      cur.push_back(c);
+    }
+  }
+  parts.push_back(cur);
+  for (std::string &p : parts) {
+    while (!p.empty() && std::isspace((unsigned char)p.front())) p.erase(p.begin());
+    while (!p.empty() && std::isspace((unsigned char)p.back())) p.pop_back();
+  }
+  return parts;
+}
+
 // ---- parameter groups (CodeGen/Base.hs:69-89,348-383) ----------------------
 
 static std::string env_params(const std::vector<EnvSig> &env)
@@ -284,23 +308,47 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "#define ACC_OUT_PARAMS " << out_params(sp.out_rank, sp.elt_type) << "\n";
       o << "#define ACC_STENCIL_RANK " << sp.out_rank << "\n";
       o << "#define ACC_STENCIL_SOURCES " << (two ? 2 : 1) << "\n";
-      o << "#define ACC_IN_ELT " << sp.stencil_in_type << "\n";
       o << "#define ACC_RADIUS_Z " << rz << "\n#define ACC_RADIUS_Y " << ry << "\n#define ACC_RADIUS_X " << rx << "\n";
       o << "#define ACC_BOUNDARY " << sp.boundary << "\n";
-      o << "#define ACC_BOUNDARY_CONSTANT " << (sp.boundary_constant.empty() ? "0" : sp.boundary_constant) << "\n";
-      // the stencil pattern: one binding per tap, read through whatever accessor the template passes
-      o << "#define ACC_STENCIL_TAPS(READ) ";
-      for (size_t k = 0; k < sp.tap_dy.size(); ++k)
-        o << "const ACC_IN_ELT t" << k << " = READ(" << sp.tap_dz[k] << ", " << sp.tap_dy[k] << ", " << sp.tap_dx[k] << "); ";
-      o << "\n";
-      if (two) {
-        o << "#define ACC_IN2_ELT " << sp.stencil_in2_type << "\n";
-        o << "#define ACC_BOUNDARY2 " << sp.boundary2 << "\n";
-        o << "#define ACC_BOUNDARY2_CONSTANT " << (sp.boundary2_constant.empty() ? "0" : sp.boundary2_constant) << "\n";
-        o << "#define ACC_STENCIL_TAPS2(READ) ";
-        for (size_t k = 0; k < sp.tap2_dy.size(); ++k)
-          o << "const ACC_IN2_ELT u" << k << " = READ(" << sp.tap2_dz[k] << ", " << sp.tap2_dy[k] << ", " << sp.tap2_dx[k] << "); ";
+      // A source is one array per component of its element (Stencil/Extra.hs:53-128 reads every component of a tuple
+      // array).  Per source the template gets: the list of its components -- number, type, value outside the array
+      // under a constant boundary -- highest component first; its kernel parameters in that order; and one binding
+      // per tap, read through whatever accessor the template passes, a struct of the components for a tuple.
+      auto source = [&](const char *which, const char *tap_name, const std::string &elt_name, const std::vector<std::string> &comps,
+                        const std::string &constant, const std::vector<int> &dz, const std::vector<int> &dy, const std::vector<int> &dx,
+                        const char *array_name, bool with_extents) -> int {
+        const int nc = (int)comps.size();
+        std::vector<std::string> consts = split_top_level(constant);
+        if (consts.empty() || (consts.size() == 1 && consts[0].empty())) consts.assign(nc, "0");
+        if ((int)consts.size() != nc)
+          return fail(ACC_ERR_INVALID, "stencil: the boundary constant has %d component(s), the source element has %d", (int)consts.size(), nc);
+        o << "#define ACC_SRC" << which << "_COMPONENTS(X, arg)";
+        for (int i = 0; i < nc; ++i) o << " X(" << (nc - 1 - i) << ", " << comps[i] << ", (" << consts[i] << "), arg)";
         o << "\n";
+        o << "#define ACC_SRC" << which << "_PARAMS";
+        if (with_extents)
+          for (int dd = sp.out_rank - 1; dd >= 0; --dd) o << " , const Int64 sh" << array_name << "_" << dd;
+        for (int i = 0; i < nc; ++i) o << " , const " << comps[i] << " *__restrict__ arr" << array_name << "_" << (nc - 1 - i);
+        o << "\n";
+        o << "#define ACC_IN" << which << "_ELT " << (nc == 1 ? comps[0] : elt_name) << "\n";
+        o << "#define ACC_STENCIL_TAPS" << which << "(READ) ";
+        for (size_t k = 0; k < dy.size(); ++k) {
+          o << "const ACC_IN" << which << "_ELT " << tap_name << k << " = ";
+          if (nc > 1) o << "{ ";
+          for (int i = 0; i < nc; ++i)
+            o << (i ? ", " : "") << "READ(" << (nc - 1 - i) << ", " << dz[k] << ", " << dy[k] << ", " << dx[k] << ")";
+          if (nc > 1) o << " }";
+          o << "; ";
+        }
+        o << "\n";
+        return ACC_OK;
+      };
+      ACC_TRY(source("1", "t", "acc_in1_elt", sp.stencil_in_comps, sp.boundary_constant, sp.tap_dz, sp.tap_dy, sp.tap_dx,
+                     two ? "Stencil1" : "Stencil", two));
+      if (two) {
+        o << "#define ACC_BOUNDARY2 " << sp.boundary2 << "\n";
+        ACC_TRY(source("2", "u", "acc_in2_elt", sp.stencil_in2_comps, sp.boundary2_constant, sp.tap2_dz, sp.tap2_dy, sp.tap2_dx,
+                       "Stencil2", true));
       }
       o << "#define ACC_STENCIL_FN " << sp.stencil_fn << "\n";
       o << "#define ACC_XCD_REMAP " << tune("stencil.xcd_remap", 0) << "\n";
@@ -325,6 +373,18 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
     const int nc = (int)sp.comp_types.size();
     for (int i = 0; i < nc; ++i) o << sp.comp_types[i] << " a" << (nc - 1 - i) << "; ";
     o << "};\n";
+  }
+  // a stencil source of tuple type: its taps are values of a struct of their own
+  auto in_struct = [&](const char *name, const std::vector<std::string> &comps) {
+    if (comps.size() < 2) return;
+    o << "struct " << name << " { ";
+    const int nc = (int)comps.size();
+    for (int i = 0; i < nc; ++i) o << comps[i] << " a" << (nc - 1 - i) << "; ";
+    o << "};\n";
+  };
+  if (sp.kind == ACC_SKEL_STENCIL || sp.kind == ACC_SKEL_STENCIL2) {
+    in_struct("acc_in1_elt", sp.stencil_in_comps);
+    in_struct("acc_in2_elt", sp.stencil_in2_comps);
   }
   if (!sp.preamble.empty()) o << sp.preamble << "\n";
   o << "#include \"" << tmpl << "\"\n";
@@ -511,11 +571,21 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
       sp->boundary_constant = flat(d->boundary_constant);
       sp->stencil_fn = flat(d->stencil_fn);
       sp->stencil_in_type = (d->stencil_in_type && *d->stencil_in_type) ? d->stencil_in_type : sp->elt_type;
+      // "T<n-1>, ..., T0": a source of tuples, one array per component (as for elt_type)
+      auto in_comps = [&](const std::string &type, std::vector<std::string> *comps, const char *what) -> int {
+        *comps = split_top_level(type);
+        if (comps->empty() || (int)comps->size() > ACC_MAX_COMP) return fail(ACC_ERR_INVALID, "stencil: %s has too many components", what);
+        for (const std::string &c : *comps)
+          if (c.empty() || type_size(c) <= 0) return fail(ACC_ERR_INVALID, "stencil: cannot size component '%s' of %s", c.c_str(), what);
+        return ACC_OK;
+      };
+      ACC_TRY(in_comps(sp->stencil_in_type, &sp->stencil_in_comps, "stencil_in_type"));
       if (d->kind == ACC_SKEL_STENCIL2) {
         ACC_TRY(taps(d->n_taps2, d->tap2_dz, d->tap2_dy, d->tap2_dx, d->boundary2, &sp->tap2_dz, &sp->tap2_dy, &sp->tap2_dx));
         sp->boundary2 = d->boundary2;
         sp->boundary2_constant = flat(d->boundary2_constant);
         sp->stencil_in2_type = (d->stencil_in2_type && *d->stencil_in2_type) ? d->stencil_in2_type : sp->elt_type;
+        ACC_TRY(in_comps(sp->stencil_in2_type, &sp->stencil_in2_comps, "stencil_in2_type"));
       }
       sp->block = tune("stencil.block", 256);
       sp->tile_w = 256;                                  // one wave's strip: 64 lanes x 4 columns
@@ -531,8 +601,9 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
         };
         reach(sp->tap_dz, sp->tap_dy, sp->tap_dx);
         reach(sp->tap2_dz, sp->tap2_dy, sp->tap2_dx);
-        int words = std::max(1, (type_size(sp->stencil_in_type) + 3) / 4);
-        if (d->kind == ACC_SKEL_STENCIL2) words += std::max(1, (type_size(sp->stencil_in2_type) + 3) / 4);
+        int words = 0;
+        for (const std::string &c : sp->stencil_in_comps) words += std::max(1, (type_size(c) + 3) / 4);
+        for (const std::string &c : sp->stencil_in2_comps) words += std::max(1, (type_size(c) + 3) / 4);
         for (int tz = 3; rz > 0 && tz > 1 && planes_per_strip == 1; --tz)
           if ((2 * rz + tz) * (2 * ry + 1 + sp->prefetch) * (4 + 2 * rx) * words <= 128) planes_per_strip = tz;
       }

@@ -31,6 +31,7 @@ struct SkelSpec {
   // stencil
   int boundary = 0;
   std::string boundary_constant, stencil_fn, stencil_in_type;
+  std::vector<std::string> stencil_in_comps, stencil_in2_comps;   // the sources' element types by component, highest first
   std::vector<int> tap_dz, tap_dy, tap_dx;
   // stencil2: the second source
   int boundary2 = 0;

@@ -283,8 +283,8 @@ typedef struct acc_skel_desc {
                                      *   struct acc_elt { T<n-1> a<n-1>; ...; T0 a0; };
                                      * fragments produce and take apart acc_elt values, and the
                                      * result array has one pointer per component (CodeGen/
-                                     * Base.hs:344-357).  A stencil may produce tuples; its
-                                     * sources are arrays of scalars (stencil_in_type)        */
+                                     * Base.hs:344-357).  A stencil may produce tuples and
+                                     * read them (stencil_in_type)                            */
   int32_t            elt_size;      /* sizeof(elt_type); 0 = derive from the type's name    */
   int32_t            out_rank;      /* map family, stencil: rank of the result (>= 0)       */
   const char        *preamble;      /* file-scope declarations for the fragments, or NULL   */
@@ -298,12 +298,17 @@ typedef struct acc_skel_desc {
   /* stencil: taps t0 .. t<n-1> at offsets (dy, dx) from the focus (1-D: dy = 0; 3-D: see tap_dz),
    * `stencil_fn` is an expression over t0.. giving the result element       */
   int32_t            boundary;      /* ACC_BOUNDARY_*                                       */
-  const char        *boundary_constant;
+  const char        *boundary_constant; /* ACC_BOUNDARY_CONSTANT: the value outside the source; of a
+                                           source of tuples one value per component, "v<n-1>, ..., v0" */
   int32_t            n_taps;
   const int32_t     *tap_dy;
   const int32_t     *tap_dx;
   const char        *stencil_fn;
-  const char        *stencil_in_type; /* element type of the source array; NULL = elt_type */
+  const char        *stencil_in_type; /* element type of the source array; NULL = elt_type.  "T<n-1>, ..., T0" for a
+                                         source of tuples (Stencil/Extra.hs:53-128 reads every component): the
+                                         source acc_array then has one pointer per component, and a tap is a value of
+                                         struct acc_in1_elt { T<n-1> a<n-1>; ...; T0 a0; } (t0.a1, t0.a0; the second
+                                         source of a stencil2: acc_in2_elt, u0.a1, ...) */
   const char        *seg_type;      /* foldSeg: C type of the offsets (NULL = "Int32")       */
   /* stencil2 only: the second source, with taps u0 .. u<n-1>; `stencil_fn` is over t0.. and u0.. */
   int32_t            boundary2;

@@ -291,3 +291,84 @@ def test_tuple_results_need_tuple_arrays(A, ctx):
     with pytest.raises(A.AccError) as e:
         ctx.skeleton(A.SKEL_MAP, "float, quux", env=[F32], out_rank=1, get="acc_elt{1.0f, 1}")
     assert e.value.code == A.ERR_INVALID
+
+
+def test_stencils_over_sources_of_tuple_type(A, ctx):
+    """the source of a stencil may be an array of tuples (Stencil/Extra.hs:53-128 reads every component): one array
+    per component, a register window each, the taps structs of the components.  Components of different widths, a
+    triple, every boundary mode (the constant one with a value per component), aligned and ragged widths, three
+    dimensions, a result that is a tuple again, and a stencil2 with a tuple source and a scalar one"""
+    import pyref
+    rng = np.random.default_rng(47)
+    taps = [(0, -1), (0, 0), (0, 1), (-1, 0), (1, 0)]
+    for (h, w) in [(64, 256), (37, 301), (3, 1030)]:
+        f = rng.integers(-50, 50, (h, w)).astype(np.float32)
+        i = rng.integers(-50, 50, (h, w)).astype(np.int32)
+        for mode in ("clamp", "mirror", "wrap", "constant"):
+            say("5-point stencil over (float, Int32) pairs", h, "x", w, mode)
+            sk = ctx.skeleton(A.SKEL_STENCIL, "float, Int32", out_rank=2, taps=taps, boundary=mode, boundary_constant="1.5f, -3",
+                              stencil_in="float, Int32",
+                              stencil_fn="acc_elt{t0.a1 + t2.a1 - 2.0f * t1.a1 + (float)t3.a0, t3.a0 + t4.a0 - t1.a0 + (Int32)t0.a1}")
+            out = ctx.empty_tuple((h, w), [np.float32, np.int32])
+            sk.stencil([], ctx.tuple_array(f, i), out)
+            of, oi = out.get()
+            tf = pyref.tap_arrays(f, taps, mode, 1.5, (h, w))
+            ti = pyref.tap_arrays(i, taps, mode, -3, (h, w))
+            assert np.array_equal(of, tf[0] + tf[2] - np.float32(2.0) * tf[1] + ti[3].astype(np.float32))
+            assert np.array_equal(oi, ti[3] + ti[4] - ti[1] + tf[0].astype(np.int32))
+            sk.destroy()
+    say("a triple with components of 8, 1 and 2 bytes, scalar result")
+    d = rng.integers(-9, 9, (20, 515)).astype(np.float64)
+    b = rng.integers(0, 2, (20, 515)).astype(np.uint8)
+    s16 = rng.integers(-300, 300, (20, 515)).astype(np.int16)
+    sk = ctx.skeleton(A.SKEL_STENCIL, "double", out_rank=2, taps=[(0, -1), (0, 1)], boundary="mirror", stencil_in="double, Word8, Int16",
+                      stencil_fn="(t0.a1 ? t0.a2 : t1.a2) + (double)(t1.a0 - t0.a0)")
+    out = ctx.empty((20, 515), np.float64)
+    sk.stencil([], ctx.tuple_array(d, b, s16), out)
+    td = pyref.tap_arrays(d, [(0, -1), (0, 1)], "mirror", 0, d.shape)
+    tb = pyref.tap_arrays(b, [(0, -1), (0, 1)], "mirror", 0, d.shape)
+    ts = pyref.tap_arrays(s16, [(0, -1), (0, 1)], "mirror", 0, d.shape)
+    assert np.array_equal(out.get(), np.where(tb[0] != 0, td[0], td[1]) + (ts[1].astype(np.int32) - ts[0].astype(np.int32)).astype(np.float64))
+    sk.destroy()
+    say("1-D and 3-D")
+    x, y = rng.integers(-99, 99, 100003).astype(np.int32), rng.integers(-99, 99, 100003).astype(np.int64)
+    sk = ctx.skeleton(A.SKEL_STENCIL, "Int64", out_rank=1, taps=[(0, -2), (0, 2)], boundary="wrap", stencil_in="Int32, Int64",
+                      stencil_fn="(Int64)t0.a1 * t1.a0 - (Int64)t1.a1 * t0.a0")
+    out = ctx.empty(x.size, np.int64)
+    sk.stencil([], ctx.tuple_array(x, y), out)
+    assert np.array_equal(out.get(), np.roll(x, 2).astype(np.int64) * np.roll(y, -2) - np.roll(x, -2).astype(np.int64) * np.roll(y, 2))
+    sk.destroy()
+    vf, vi = rng.integers(-9, 9, (7, 19, 260)).astype(np.float32), rng.integers(-9, 9, (7, 19, 260)).astype(np.int32)
+    t3 = [(0, 0, 0), (-1, 0, 0), (1, 0, 0), (0, -1, 0), (0, 0, 1)]
+    sk = ctx.skeleton(A.SKEL_STENCIL, "float", out_rank=3, taps=t3, boundary="clamp", stencil_in="float, Int32",
+                      stencil_fn="t1.a1 + t2.a1 + t3.a1 + t4.a1 - 4.0f * t0.a1 + (float)(t1.a0 - t2.a0 + t3.a0 - t4.a0)")
+    out = ctx.empty(vf.shape, np.float32)
+    sk.stencil([], ctx.tuple_array(vf, vi), out)
+    pf, pi = np.pad(vf, 1, mode="edge"), np.pad(vi, 1, mode="edge")
+    c = lambda p, dz, dy, dx: p[1 + dz:p.shape[0] - 1 + dz, 1 + dy:p.shape[1] - 1 + dy, 1 + dx:p.shape[2] - 1 + dx]   # noqa: E731
+    ref = (c(pf, -1, 0, 0) + c(pf, 1, 0, 0) + c(pf, 0, -1, 0) + c(pf, 0, 0, 1) - np.float32(4.0) * vf
+           + (c(pi, -1, 0, 0) - c(pi, 1, 0, 0) + c(pi, 0, -1, 0) - c(pi, 0, 0, 1)).astype(np.float32))
+    assert np.array_equal(out.get(), ref)
+    sk.destroy()
+    say("stencil2: a source of pairs and a scalar one, extents that differ")
+    a1, a0 = rng.integers(-9, 9, (40, 300)).astype(np.float32), rng.integers(-9, 9, (40, 300)).astype(np.float32)
+    m = rng.integers(-9, 9, (33, 310)).astype(np.int32)
+    sk = ctx.skeleton(A.SKEL_STENCIL2, "float", out_rank=2, taps=[(0, -1), (0, 1)], boundary="clamp", taps2=[(-1, 0), (1, 0)], boundary2="constant",
+                      boundary2_constant="5", stencil_in="float, float", stencil_in2="Int32",
+                      stencil_fn="(t1.a1 - t0.a1) * (t1.a0 + t0.a0) + (float)(u1 - u0)")
+    out = ctx.empty((33, 300), np.float32)
+    sk.stencil2([], ctx.tuple_array(a1, a0), ctx.array(m), out)
+    t1 = pyref.tap_arrays(a1, [(0, -1), (0, 1)], "clamp", 0, (33, 300))
+    t0 = pyref.tap_arrays(a0, [(0, -1), (0, 1)], "clamp", 0, (33, 300))
+    u = pyref.tap_arrays(m, [(-1, 0), (1, 0)], "constant", 5, (33, 300))
+    assert np.array_equal(out.get(), (t1[1] - t1[0]) * (t0[1] + t0[0]) + (u[1] - u[0]).astype(np.float32))
+    say("wrong use: a scalar array where the kernel was built for pairs; a constant with too few components")
+    with pytest.raises(A.AccError) as e:
+        sk.stencil2([], ctx.array(a1), ctx.array(m), out)
+    assert e.value.code == A.ERR_INVALID
+    sk.destroy()
+    with pytest.raises(A.AccError) as e:
+        ctx.skeleton(A.SKEL_STENCIL, "float", out_rank=1, taps=[(0, 0)], boundary="constant", boundary_constant="1.0f",
+                     stencil_in="float, Int32", stencil_fn="t0.a1")
+    assert e.value.code == A.ERR_INVALID
+
