@@ -72,6 +72,33 @@ def test_tuples_live_on_the_host_side_of_the_text():
     assert A.compile_only(desc) > 0
 
 
+def test_components_nobody_uses_are_never_loaded():
+    """dead-component elimination (CodeGen.hs:283-314): a fused producer's tuple is a list of component expressions on
+    the host, so what a consumer does not use is not in the text -- neither the arithmetic nor the array read, and an
+    array that only fed a dead component is not even a kernel parameter"""
+    xs, ys = use((100,), np.float32), use((100,), np.int32)
+    pairs = acc.zip_(xs, ys)
+    firsts = acc.map(lambda p: acc.fst(p) * 2.0, pairs)
+    arrays, sig, fr = acc._assemble(get=firsts.stream().text)
+    assert arrays == [xs.manifest] and sig == [(1, "float")] and "arrIn1" not in fr["get"]
+    # a producer that computes two things per element, a consumer that folds one of them
+    both = acc.map(lambda v: acc.lift(acc.sqrt(v), acc.exp(v) + acc.sin(v)), xs)
+    roots = acc.map(acc.fst, both)
+    arrays, sig, fr = acc._assemble(get=roots.stream().text, combine=acc._combine(add, "float").text, seed=acc.Exp.of(0.0, "float").text)
+    assert "acc_sqrt" in fr["get"] and "acc_exp" not in fr["get"] and "acc_sin" not in fr["get"]
+    assert A.compile_only(A.make_desc(A.SKEL_FOLD, "float", env=sig, **fr)) > 0
+    # a manifest array of pairs: only the component that is used is read (the other pointer is passed and left alone)
+    ps = acc.Acc((10,), ("Int16", "double"), manifest=A.TupleArray.__new__(A.TupleArray))
+    ps.manifest.comps = [Resident((10,), np.int16), Resident((10,), np.float64)]
+    seconds = acc.map(acc.snd, ps)
+    text = seconds.stream().text
+    assert "_0" in text and "_1" not in text.replace("acc_stream", "")
+    # through a conditional: each component selects for itself, so a dead component takes its test with it
+    pick = acc.map(lambda p: acc.fst(acc.cond(acc.snd(p) > 0, p, acc.lift(acc.constant(0.0, "float"), acc.snd(p)))), pairs)
+    arrays, sig, fr = acc._assemble(get=pick.stream().text)
+    assert fr["get"].count("arrIn1_0") == 1                                    # the test, once; no select of the dead Int32 component
+
+
 def test_index_arithmetic_of_the_delayed_combinators():
     m = use((3, 5), np.int32)
     t = acc.transpose(m)
