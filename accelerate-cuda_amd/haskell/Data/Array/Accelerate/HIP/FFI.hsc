@@ -55,6 +55,41 @@ accErrUnsupported = #{const ACC_ERR_UNSUPPORTED}
 accErrIO          = #{const ACC_ERR_IO}
 accErrStuck       = #{const ACC_ERR_STUCK}
 
+-- skeleton kinds, combination hints and flags of a skeleton description (acc_skel_desc)
+accSkelMap, accSkelGenerate, accSkelTransform, accSkelFold, accSkelFold1, accSkelFoldSeg, accSkelFold1Seg,
+  accSkelScanl, accSkelScanl1, accSkelScanlP, accSkelScanr, accSkelScanr1, accSkelScanrP, accSkelPermute,
+  accSkelStencil, accSkelStencil2 :: Int32
+accSkelMap       = #{const ACC_SKEL_MAP}
+accSkelGenerate  = #{const ACC_SKEL_GENERATE}
+accSkelTransform = #{const ACC_SKEL_TRANSFORM}
+accSkelFold      = #{const ACC_SKEL_FOLD}
+accSkelFold1     = #{const ACC_SKEL_FOLD1}
+accSkelFoldSeg   = #{const ACC_SKEL_FOLDSEG}
+accSkelFold1Seg  = #{const ACC_SKEL_FOLD1SEG}
+accSkelScanl     = #{const ACC_SKEL_SCANL}
+accSkelScanl1    = #{const ACC_SKEL_SCANL1}
+accSkelScanlP    = #{const ACC_SKEL_SCANLP}
+accSkelScanr     = #{const ACC_SKEL_SCANR}
+accSkelScanr1    = #{const ACC_SKEL_SCANR1}
+accSkelScanrP    = #{const ACC_SKEL_SCANRP}
+accSkelPermute   = #{const ACC_SKEL_PERMUTE}
+accSkelStencil   = #{const ACC_SKEL_STENCIL}
+accSkelStencil2  = #{const ACC_SKEL_STENCIL2}
+
+accCombineGeneric, accCombineAdd, accCombineMin, accCombineMax, accCombineAnd, accCombineOr, accCombineXor :: Int32
+accCombineGeneric = #{const ACC_COMBINE_GENERIC}
+accCombineAdd     = #{const ACC_COMBINE_ADD}
+accCombineMin     = #{const ACC_COMBINE_MIN}
+accCombineMax     = #{const ACC_COMBINE_MAX}
+accCombineAnd     = #{const ACC_COMBINE_AND}
+accCombineOr      = #{const ACC_COMBINE_OR}
+accCombineXor     = #{const ACC_COMBINE_XOR}
+
+accFlagFoldRight, accFlagFastMath, accFlagGuarded :: Word32
+accFlagFoldRight = #{const ACC_FLAG_FOLD_RIGHT}
+accFlagFastMath  = #{const ACC_FLAG_FAST_MATH}
+accFlagGuarded   = #{const ACC_FLAG_GUARDED}
+
 data HIPException = HIPException Status String
   deriving (Typeable)
 

@@ -359,4 +359,32 @@ def test_haskell_bindings_cover_the_header():
         body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (struct, struct), header, flags=re.S).group(1)
         assert re.search(r"\b%s\b" % field, body), (struct, field)
     for const in re.findall(r"#\{const (\w+)\}", hsc):
-        assert re.search(r"#define %s\b" % const, header), const
+        assert re.search(r"#define %s\b|\b%s\s*=" % (const, const), header), const      # a macro, or a member of an enum
+
+
+def test_haskell_modules_use_only_what_the_bindings_and_the_device_headers_have():
+    """the (uncompiled) modules of the Haskell backend -- code generator, compile and execute traversals, front door --
+    call only foreign imports and constants that FFI.hsc defines, and emit only device functions that the headers
+    every generated unit includes define"""
+    hdir = os.path.join(ROOT, "accelerate-cuda_amd", "haskell", "Data", "Array", "Accelerate")
+    hsc = open(os.path.join(hdir, "HIP", "FFI.hsc")).read()
+    bound = set(re.findall(r'^foreign import ccall \w+\s+"acc_\w+"\s+(c_\w+)', hsc, flags=re.M))
+    constants = set(re.findall(r"^(acc[A-Z]\w+)\s+=", hsc, flags=re.M))
+    device = ""
+    for h in ("acc_prim.h", "acc_hip_device.h"):
+        device += open(os.path.join(ROOT, "accelerate-cuda_amd", "csrc", "device", h)).read()
+    defined = set(re.findall(r"\b(acc_[a-z0-9_]+)\s*\(", device)) | set(re.findall(r"#define (ACC_[A-Z_]+)", device))
+    defined |= set(re.findall(r"^ACC_MATH\d\((acc_[a-z0-9_]+),", device, flags=re.M))       # defined through a macro
+    modules = ["HIP.hs", "HIP/CodeGen.hs", "HIP/Compile.hs", "HIP/Execute.hs", "HIP/State.hs"]
+    for m in modules:
+        text = open(os.path.join(hdir, m)).read()
+        assert "UNCOMPILED" in text, m
+        code = re.sub(r"--.*", "", text)
+        for name in set(re.findall(r"\b(c_[a-zA-Z0-9]+)\b", code)):
+            assert name in bound, (m, name)
+        for name in set(re.findall(r"\b(acc(?:Skel|Combine|Flag|Err)[A-Za-z0-9]*)\b", code)):
+            assert name in constants, (m, name)
+        for name in set(re.findall(r'"(acc_[a-z0-9_]+)[<("]', code)):
+            assert name in defined, (m, name)
+        for name in set(re.findall(r"\b(ACC_[A-Z_]+)\b", code)) - {"ACC_FLAG_GUARDED", "ACC_ERR_INVALID", "ACC_ERR_STUCK", "ACC_COMBINE_ADD"}:
+            assert name in defined, (m, name)
