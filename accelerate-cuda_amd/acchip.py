@@ -244,6 +244,14 @@ def make_desc(kind, elt, env=(), out_rank=0, get=None, combine=None, seed=None, 
     return d
 
 
+def make_desc_copy(d):
+    """a description with the same fields (and the same storage behind its pointers), to vary a flag or a hint"""
+    c = acc_skel_desc()
+    C.memmove(C.byref(c), C.byref(d), C.sizeof(acc_skel_desc))
+    c._keep = d._keep
+    return c
+
+
 def preview(desc, variant=0):
     """(entry name, generated translation unit) of a description; needs no GPU."""
     src, entry = C.c_char_p(), C.c_char_p()

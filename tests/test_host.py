@@ -73,6 +73,14 @@ def test_permute_variants_the_driver_chooses_between_all_compile(A, tmp_path):
             name, src = A.preview(desc, v)
             assert name == "permute" and ("ACC_PERMUTE_NARROW 1" in src) == (v >= 6)
             assert A.compile_source(src) > 4000, v
+    # and as a loop's body runs them (ACC_FLAG_GUARDED: one more parameter and a test on entry in every kernel)
+    for desc, variants in ((hist, (4, 6)), (generic, (2,))):
+        g = A.make_desc_copy(desc)
+        g.flags |= A.FLAG_GUARDED
+        for v in variants:
+            name, src = A.preview(g, v)
+            assert "#define ACC_GUARDED 1" in src
+            assert A.compile_source(src) > 4000, v
 
 
 def test_every_scalar_primitive_compiles_for_every_type(A, tmp_path):
