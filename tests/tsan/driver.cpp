@@ -1,0 +1,171 @@
+// Eight host threads on ONE context of libacchip's host code, built under ThreadSanitizer against the stand-in HIP
+// runtime of mock_hip.cpp: what include/acc_hip.h promises ("every entry point may be called from any thread; one
+// acc_skel may be executed from several threads") exercised where data races would sit -- the scratch pool (acquire,
+// release, trim, blocks of several protocols and sizes), the lazily built second variant of a shared instance,
+// instances created and destroyed while others run, the ordering of big scans across streams, guards set on and
+// taken off streams, the status block, the memory table, the launch trace.  Launches do nothing here; the checks are
+// ThreadSanitizer's.  Exit status 0 and no report = pass.
+#include <atomic>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <thread>
+#include <vector>
+
+#include "../../include/acc_hip.h"
+
+extern "C" long mock_hip_launches(void);
+
+#define OK(call)                                                                        \
+  do {                                                                                  \
+    int rc__ = (call);                                                                  \
+    if (rc__ != ACC_OK) {                                                               \
+      std::fprintf(stderr, "%s:%d: %s -> %d: %s\n", __FILE__, __LINE__, #call, rc__, acc_last_error()); \
+      std::exit(2);                                                                     \
+    }                                                                                   \
+  } while (0)
+
+static acc_array vec(uint64_t p, int64_t n)
+{
+  acc_array a;
+  std::memset(&a, 0, sizeof(a));
+  a.rank = 1;
+  a.ncomp = 1;
+  a.shape[0] = n;
+  a.ptr[0] = p;
+  return a;
+}
+
+static acc_skel make(acc_context ctx, int kind, const char *elt, const char *get, const char *combine, const char *seed,
+                     const char *permutation, int hint, uint32_t flags)
+{
+  acc_env_sig env[1];
+  std::memset(env, 0, sizeof(env));
+  env[0].rank = 1;
+  env[0].ncomp = 1;
+  env[0].type[0] = "Int32";
+  acc_skel_desc d;
+  std::memset(&d, 0, sizeof(d));
+  d.kind = kind;
+  d.flags = flags;
+  d.n_env = 1;
+  d.env = env;
+  d.elt_type = elt;
+  d.out_rank = (kind == ACC_SKEL_FOLD) ? 0 : 1;
+  d.get = get;
+  d.combine = combine;
+  d.seed = seed;
+  d.permutation = permutation;
+  d.combine_hint = hint;
+  acc_skel s = nullptr;
+  OK(acc_skel_create(ctx, &d, &s));
+  return s;
+}
+
+int main(int argc, char **argv)
+{
+  const int threads = argc > 1 ? std::atoi(argv[1]) : 8, rounds = argc > 2 ? std::atoi(argv[2]) : 150;
+  OK(acc_init());
+  OK(acc_cache_set_dir(""));
+  acc_context ctx = nullptr;
+  OK(acc_context_create(0, &ctx));
+
+  // shared instances
+  acc_skel scan = make(ctx, ACC_SKEL_SCANL1, "Int32", "arrIn0_0[ix]", "x + y", nullptr, nullptr, 0, 0);
+  acc_skel fold = make(ctx, ACC_SKEL_FOLD, "Int32", "arrIn0_0[ix]", "x + y", "0", nullptr, 0, 0);
+  acc_skel hist = make(ctx, ACC_SKEL_PERMUTE, "Int32", "1", "x + y", nullptr, "arrIn0_0[ix]", ACC_COMBINE_ADD, 0);
+  acc_skel locked = make(ctx, ACC_SKEL_PERMUTE, "Int16", "(Int16)1", "(Int16)(x + y)", nullptr, "arrIn0_0[ix]", 0, 0);
+  acc_skel gmap = make(ctx, ACC_SKEL_MAP, "Int32", "arrIn0_0[ix] + 1", nullptr, nullptr, nullptr, 0, ACC_FLAG_GUARDED);
+  acc_memtable table = nullptr;
+  OK(acc_memtable_create(ctx, 0, &table));
+
+  const int64_t n_max = int64_t(1) << 24;
+  acc_devptr in = 0, out = 0, bins = 0, zeros = 0;
+  OK(acc_malloc(ctx, (size_t)(n_max + 4) * 4, &in));
+  OK(acc_malloc(ctx, (size_t)(n_max + 4) * 4, &out));
+  OK(acc_malloc(ctx, (size_t)(1 << 20) * 4, &bins));
+  OK(acc_malloc(ctx, (size_t)(1 << 20) * 4, &zeros));
+
+  std::atomic<int> failures{0};
+  std::vector<std::thread> pool;
+  for (int t = 0; t < threads; ++t) {
+    pool.emplace_back([&, t] {
+      acc_stream st = nullptr;
+      OK(acc_stream_create(ctx, &st));
+      acc_guard guard = nullptr;
+      OK(acc_guard_create(ctx, &guard));
+      std::vector<char> host(1 << 16);
+      for (int r = 0; r < rounds; ++r) {
+        // sizes from one tile to thousands of them: small and big scans (the big ones are chained across streams),
+        // folds with and without a second workgroup, so that scratch blocks of several sizes and protocols come and go
+        const int64_t n = (r % 5 == 0) ? n_max : (int64_t(1) << (10 + (r * 7 + t * 3) % 12)) + t;
+        // an unaligned operand every few rounds: the second variant of the shared instances is built on first need
+        const uint64_t off = (r % 7 == 3) ? 4 : 0;
+        acc_array a = vec(in + off, n), o = vec(out + off, n), total = vec(out, 1);
+        total.rank = 0;
+        OK(acc_exec_scan(scan, &a, n, &o, nullptr, st));
+        OK(acc_exec_fold(fold, &a, 1, &n, &total, st));
+        const int64_t nb = (r % 3 == 0) ? 256 : ((r % 3 == 1) ? 65536 : 200000);
+        acc_array d = vec(zeros, nb), b = vec(bins, nb);
+        OK(acc_exec_permute(hist, &a, n, &d, &b, st));
+        if (r % 4 == 1) {
+          acc_array d16 = vec(zeros, 3000), b16 = vec(bins, 3000), few = vec(in, 2000);
+          OK(acc_exec_permute(locked, &few, 2000, &d16, &b16, st));
+        }
+        if (r % 6 == 2) {                       // a loop's kernels on this thread's stream, under its guard
+          OK(acc_stream_set_guard(ctx, st, guard));
+          OK(acc_guard_reset(guard, st));
+          acc_array m = vec(out, 1000), mi = vec(in, 1000);
+          OK(acc_exec_map(gmap, &mi, &m, st));
+          int32_t alive = 0;
+          int64_t count = 0;
+          OK(acc_guard_read(guard, st, &alive, &count));
+          OK(acc_stream_set_guard(ctx, st, nullptr));
+        }
+        if (r % 9 == 4) {                       // instances of this thread's own come and go
+          acc_skel mine = make(ctx, ACC_SKEL_SCANL, "Int32", "arrIn0_0[ix] * 2", "x + y", "0", nullptr, 0, 0);
+          acc_array o1 = vec(out, 1001), a1 = vec(in, 1000);
+          OK(acc_exec_scan(mine, &a1, 1000, &o1, nullptr, st));
+          acc_skel_info info;
+          OK(acc_skel_get_info(mine, &info));
+          OK(acc_skel_destroy(mine));
+        }
+        if (r % 11 == 5) {                      // the pool gives back what is not lent, while the others borrow
+          size_t freed = 0, held = 0;
+          OK(acc_context_trim(ctx, &freed));
+          OK(acc_context_scratch_bytes(ctx, &held));
+        }
+        if (r % 5 == 2) {                       // an array of the memory table, keyed by this thread and round
+          const uint64_t key = (uint64_t(t) << 32) | uint64_t(r);
+          int is_new = 0;
+          acc_devptr p = 0;
+          OK(acc_memtable_malloc(table, key, host.data(), host.size(), 1, &is_new));
+          OK(acc_memtable_acquire(table, key, st, &p));
+          OK(acc_memtable_release(table, key, st));
+          OK(acc_memtable_free(table, key));
+        }
+        if (r % 13 == 6) {
+          OK(acc_trace_start(ctx));
+          acc_array o2 = vec(out, 5000), a2 = vec(in, 5000);
+          OK(acc_exec_scan(scan, &a2, 5000, &o2, nullptr, st));
+          int32_t launches = 0;
+          double ms = 0;
+          OK(acc_trace_stop(ctx, &launches, &ms));
+          if (launches != 1) failures.fetch_add(1);
+        }
+        if (r % 8 == 7) OK(acc_stream_sync(ctx, st));
+      }
+      OK(acc_stream_sync(ctx, st));
+      OK(acc_guard_destroy(guard));
+      OK(acc_stream_destroy(ctx, st));
+    });
+  }
+  for (std::thread &th : pool) th.join();
+  OK(acc_context_sync(ctx));
+  OK(acc_memtable_destroy(table));
+  for (acc_skel s : {scan, fold, hist, locked, gmap}) OK(acc_skel_destroy(s));
+  for (acc_devptr p : {in, out, bins, zeros}) OK(acc_free(ctx, p));
+  OK(acc_context_destroy(ctx));
+  std::printf("threads %d rounds %d launches %ld failures %d\n", threads, rounds, mock_hip_launches(), failures.load());
+  return failures.load() ? 1 : 0;
+}
