@@ -360,6 +360,133 @@ static void smvm(acc_context ctx)
   acc_free(ctx, dout);
 }
 
+/* ---- foldSeg over the rows of a matrix: the same segments in every row ------------------------------------- */
+static void segmented_rows(acc_context ctx)
+{
+  enum { ROWS = 300, W = 100, NSEG = 4 };
+  static int32_t m[ROWS * W], got[ROWS * NSEG];
+  static const int32_t offs[NSEG + 1] = {0, 10, 10, 55, 93};          /* an empty segment, and a tail nobody reads */
+  acc_env_sig env[1];
+  acc_skel_desc d;
+  acc_skel sk = NULL;
+  acc_array in, seg, out;
+  acc_devptr dm, doffs, dout;
+  int64_t shape[2] = {ROWS, W};
+  int r, k, i, bad = 0;
+  for (i = 0; i < ROWS * W; ++i) m[i] = (int32_t)(rnd() % 200) - 100;
+  env[0] = sig(2, "Int32");
+  memset(&d, 0, sizeof d);
+  d.kind = ACC_SKEL_FOLDSEG;
+  d.n_env = 1;
+  d.env = env;
+  d.elt_type = "Int32";
+  d.out_rank = 2;                                /* the rank of the input and of the result */
+  d.get = "arrIn0_0[ix]";
+  d.combine = "x + y";
+  d.seed = "7";
+  OK(acc_skel_create(ctx, &d, &sk));
+  dm = upload(ctx, m, sizeof m);
+  doffs = upload(ctx, offs, sizeof offs);
+  OK(acc_malloc(ctx, sizeof got, &dout));
+  memset(&in, 0, sizeof in);
+  in.rank = 2; in.ncomp = 1; in.shape[0] = ROWS; in.shape[1] = W; in.ptr[0] = dm;
+  memset(&out, 0, sizeof out);
+  out.rank = 2; out.ncomp = 1; out.shape[0] = ROWS; out.shape[1] = NSEG; out.ptr[0] = dout;
+  seg = vector_of(doffs, NSEG + 1);
+  OK(acc_exec_foldseg_nd(sk, &in, 2, shape, &seg, &out, NULL));
+  OK(acc_memcpy_d2h(ctx, got, dout, sizeof got));
+  for (r = 0; r < ROWS; ++r)
+    for (k = 0; k < NSEG; ++k) {
+      int32_t sum = 7;
+      for (i = offs[k]; i < offs[k + 1]; ++i) sum += m[r * W + i];
+      if (got[r * NSEG + k] != sum) ++bad;
+    }
+  CHECK(bad == 0, "segmented sums of every row of a matrix");
+  CHECK(acc_exec_foldseg(sk, &in, ROWS * W, &seg, &out, NULL) == ACC_ERR_INVALID, "the vector entry refuses a rank-2 kernel");
+  OK(acc_skel_destroy(sk));
+  acc_free(ctx, dm);
+  acc_free(ctx, doffs);
+  acc_free(ctx, dout);
+}
+
+/* ---- awhile: double a vector until its largest element passes a bound, twelve iterations enqueued ahead -------- */
+static void guarded_loop(acc_context ctx)
+{
+  enum { N = 50000, AHEAD = 12 };
+  static int32_t x[N], got[N];
+  acc_env_sig env[1], senv[1];
+  acc_skel_desc d;
+  acc_skel dbl = NULL, mx = NULL, below = NULL;
+  acc_guard guard = NULL;
+  acc_stream st = NULL;
+  acc_devptr buf[AHEAD + 1], dtop, dflag;
+  acc_array a, b, top, flag;
+  int64_t n = N, count = -1;
+  int32_t alive = -1;
+  int i, k, steps = 0, top_now = 0;
+  for (i = 0; i < N; ++i) { x[i] = (int32_t)(rnd() % 40) + 1; if (x[i] > top_now) top_now = x[i]; }
+  while (top_now < 5000) { top_now *= 2; ++steps; }             /* what the loop should do: `steps` doublings */
+  env[0] = sig(1, "Int32");
+  memset(&d, 0, sizeof d);
+  d.flags = ACC_FLAG_GUARDED;
+  d.n_env = 1;
+  d.env = env;
+  d.elt_type = "Int32";
+  d.kind = ACC_SKEL_MAP;  d.out_rank = 1;  d.get = "arrIn0_0[ix] * 2";
+  OK(acc_skel_create(ctx, &d, &dbl));
+  d.kind = ACC_SKEL_FOLD;  d.out_rank = 0;  d.get = "arrIn0_0[ix]";  d.combine = "acc_max(x, y)";  d.seed = "0";
+  OK(acc_skel_create(ctx, &d, &mx));
+  senv[0] = sig(0, "Int32");
+  memset(&d, 0, sizeof d);
+  d.flags = ACC_FLAG_GUARDED;
+  d.kind = ACC_SKEL_MAP;  d.n_env = 1;  d.env = senv;  d.elt_type = "Word8";  d.out_rank = 0;  d.get = "(Word8)(arrIn0_0[0] < 5000)";
+  OK(acc_skel_create(ctx, &d, &below));
+  OK(acc_stream_create(ctx, &st));
+  OK(acc_guard_create(ctx, &guard));
+  buf[0] = upload(ctx, x, sizeof x);
+  for (k = 1; k <= AHEAD; ++k) OK(acc_malloc(ctx, sizeof x, &buf[k]));
+  OK(acc_malloc(ctx, 256, &dtop));
+  dflag = dtop + 128;
+  memset(&top, 0, sizeof top);   top.ncomp = 1;   top.ptr[0] = dtop;         /* rank 0 */
+  memset(&flag, 0, sizeof flag); flag.ncomp = 1;  flag.ptr[0] = dflag;
+  OK(acc_stream_set_guard(ctx, st, guard));
+  OK(acc_guard_reset(guard, st));
+  for (k = 0; k < AHEAD; ++k) {                  /* predicate; latch; body -- without looking at the device */
+    a = vector_of(buf[k], N);
+    b = vector_of(buf[k + 1], N);
+    OK(acc_exec_fold(mx, &a, 1, &n, &top, st));
+    OK(acc_exec_map(below, &top, &flag, st));
+    OK(acc_guard_latch(guard, &flag, st));
+    OK(acc_exec_map(dbl, &a, &b, st));
+  }
+  OK(acc_guard_read(guard, st, &alive, &count));
+  CHECK(alive == 0 && count == steps && steps > 3 && steps < AHEAD, "the guard counts the iterations that were taken");
+  OK(acc_memcpy_d2h(ctx, got, buf[count], sizeof got));
+  for (i = 0, k = 0; i < N; ++i) k += got[i] != x[i] << steps;
+  CHECK(k == 0, "the loop's value is what the last iteration taken produced");
+  OK(acc_stream_set_guard(ctx, st, NULL));
+  OK(acc_guard_destroy(guard));
+  OK(acc_stream_destroy(ctx, st));
+  OK(acc_skel_destroy(dbl));
+  OK(acc_skel_destroy(mx));
+  OK(acc_skel_destroy(below));
+  for (k = 0; k <= AHEAD; ++k) acc_free(ctx, buf[k]);
+  acc_free(ctx, dtop);
+}
+
+/* ---- the scratch the drivers pool can be had back ------------------------------------------------------------- */
+static void scratch_pool(acc_context ctx)
+{
+  size_t held = 0, freed = 0;
+  OK(acc_context_sync(ctx));
+  OK(acc_context_scratch_bytes(ctx, &held));
+  CHECK(held > 0, "the scans and folds above left scratch in the pool");
+  OK(acc_context_trim(ctx, &freed));
+  CHECK(freed == held, "all of it comes back when nothing is running");
+  OK(acc_context_scratch_bytes(ctx, &held));
+  CHECK(held == 0, "and the pool is empty");
+}
+
 /* ---- memory table: three arrays under a budget that holds two ---------------- */
 static void memory_table(acc_context ctx)
 {
@@ -425,6 +552,9 @@ int main(int argc, char **argv)
   histogram(ctx);
   gaussian(ctx);
   smvm(ctx);
+  segmented_rows(ctx);
+  guarded_loop(ctx);
+  scratch_pool(ctx);
   memory_table(ctx);
   CHECK(acc_context_sync(ctx) == ACC_OK, "device still healthy");
   acc_context_destroy(ctx);
