@@ -56,6 +56,8 @@ std::string embedded_text(const char *name);
 enum ScratchProtocol {
   SCRATCH_FOLD = 0,   // contents are don't-care: every launch writes what it reads (fold partials, permute tables)
   SCRATCH_LOCKS = 2,  // all zero between uses: every launch leaves it as it found it
+  SCRATCH_CARRY = 4,  // the same contract, for the carries of the counting permute (a pool of their own, so that the
+                      // lock blocks stay what acc_context_debug_poke_lock takes them for)
   SCRATCH_SCAN = 1,   // tile descriptors (behind a 256-byte header nothing uses): they carry `epoch`, so stale
                       // ones read as "not yet published"
   SCRATCH_FLAGS = 3   // 64-bit words {epoch, payload}: every launch tags what it writes with its `epoch`,
@@ -70,7 +72,7 @@ struct ScratchBlock {
   hipEvent_t done = nullptr;
   bool busy = false;
   bool recorded = false;   // `done` was recorded at the last release
-  bool dirty = false;      // SCRATCH_LOCKS: a launch may have left it non-zero: cleared again before it is lent
+  bool dirty = false;      // SCRATCH_LOCKS / SCRATCH_CARRY: a launch may have left it non-zero: cleared again before it is lent
   uint32_t epoch = 0;
 };
 

@@ -286,7 +286,8 @@ ACC_DEV int acc_xcd_id() { return (int)(__builtin_amdgcn_s_getreg(20 | (0 << 6) 
  * target's count is kept in 16 bits, two targets to a word (t and t + half the targets, so that neighbouring hot
  * targets do not meet on one word), and grows by additions of at most ACC_NARROW_MAX
  * (larger addends -- rare in a histogram, where they are all 1 -- go to the result directly).  The lane whose
- * addition takes a count from below 0x8000 to 0x8000 or above takes 0x8000 out again and adds it to the result;
+ * addition takes a count from below 0x8000 to 0x8000 or above takes 0x8000 out again and adds it to the target's entry of
+ * a table of carries in memory (`far`, all zero between launches), which permute_merge adds into the result;
  * so a count of 0x8000 or more always has such a correction on its way.  That the count cannot reach 0x10000
  * (and spill into its neighbour) before the correction lands is not left to timing: a lane that finds a count at
  * ACC_NARROW_STOP or above waits until it has dropped below that, and since a lane has at most ACC_VEC additions in flight
@@ -375,11 +376,11 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
                                                 take ? (unsigned)ux << sh : 0u, __ATOMIC_RELAXED, ACC_SCOPE_BLOCK);
     return take ? (old >> sh) & 0xFFFFu : ACC_NARROW_HALF;
   };
-  /* the lane that took the count over the half-way mark moves that half into the result */
+  /* the lane that took the count over the half-way mark moves that half into the target's carry */
   auto narrow_carry = [&](const U t, const T &x, const unsigned before) {
     if (before < ACC_NARROW_HALF && before + (unsigned)(UT)x >= ACC_NARROW_HALF) {
       (void)__hip_atomic_fetch_sub(words + narrow_word(t), ACC_NARROW_HALF << narrow_shift(t), __ATOMIC_RELAXED, ACC_SCOPE_BLOCK);
-      acc_hint_apply<ACC_SCOPE_DEVICE>(arrOut_0 + t, (T)ACC_NARROW_HALF, f);
+      acc_hint_apply<ACC_SCOPE_DEVICE>(far + t, (T)ACC_NARROW_HALF, f);       /* `far` is the table of carries here */
     }
   };
   auto narrow_wait = [&](const U t, const unsigned before) {
@@ -539,36 +540,55 @@ struct acc_merge_job {
 };
 
 #if ACC_PERMUTE_NARROW
-/* the rows of packed 16-bit counts, `nwords` words a row, added into the result: a thread per word (targets
- * `column` and `column + nwords`),
- * the rows shared between `slices` workgroups (then each adds its share atomically) */
+/* result = base + carries + the sum of the workgroups' rows of packed 16-bit counts (`nwords` words a row, targets
+ * `column` and `column + nwords` in a word).  A workgroup takes 64 consecutive words, each of its four waves a
+ * quarter of the rows, eight loads in flight a lane; the waves' sums meet in LDS and the first wave writes the
+ * result -- one thread per pair of targets, so no atomics and nothing that must be in the result beforehand -- and
+ * clears the carries it has taken (the table is all zero between launches).  `base` is the defaults array, or the
+ * result itself where that was filled from the defaults before the main kernel (which then also added to it
+ * directly).                                                                                                */
 extern "C" __global__ void __launch_bounds__(256)
 permute_merge(ACC_ENV_PARAMS ACC_OUT_PARAMS, const unsigned *__restrict__ dump, const Int64 nwords, const int nrows,
-              const int slices, const Int64 ntarget ACC_GUARD_PARAM)
+              const Int64 ntarget, ACC_ELT *carry, const ACC_ELT *base ACC_GUARD_PARAM)
 {
   ACC_GUARD_CHECK
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
+  __shared__ unsigned s_lo[4][64], s_hi[4][64];
   auto f = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
-  const Int64 column = (Int64)(blockIdx.x / slices) * 256 + threadIdx.x;
-  const int slice = blockIdx.x % slices;
-  if (column >= nwords) return;
-  const int per = (nrows + slices - 1) / slices;
-  const int r0 = slice * per, r1 = acc_min(nrows, r0 + per);
-  unsigned lo = 0u, hi = 0u;                     /* at most 65536 rows of counts below 0x8000 each */
-#pragma unroll 8
-  for (int r = r0; r < r1; ++r) {
-    const unsigned w = dump[(Int64)r * nwords + column];
+  const int lane = threadIdx.x & 63, quarter = threadIdx.x >> 6;
+  const Int64 column = (Int64)blockIdx.x * 64 + lane;
+  const Int64 col_c = acc_min<Int64>(column, nwords - 1);       /* lanes past the end read the last word and drop it */
+  unsigned lo = 0u, hi = 0u;                     /* at most 65536 rows of counts below 0x10000 each */
+  int r = quarter;
+  for (; r + 28 < nrows; r += 32) {
+    unsigned w[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) w[k] = __builtin_nontemporal_load(dump + (Int64)(r + 4 * k) * nwords + col_c);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) { lo += w[k] & 0xFFFFu; hi += w[k] >> 16; }
+  }
+  for (; r < nrows; r += 4) {
+    const unsigned w = __builtin_nontemporal_load(dump + (Int64)r * nwords + col_c);
     lo += w & 0xFFFFu;
     hi += w >> 16;
   }
+  s_lo[quarter][lane] = lo;
+  s_hi[quarter][lane] = hi;
+  __syncthreads();
+  if (quarter != 0 || column >= nwords) return;
+  lo = s_lo[0][lane] + s_lo[1][lane] + s_lo[2][lane] + s_lo[3][lane];
+  hi = s_hi[0][lane] + s_hi[1][lane] + s_hi[2][lane] + s_hi[3][lane];
   const Int64 t = column, t_hi = column + nwords;
-  if (slices == 1) {
-    arrOut_0[t] = f((T)lo, arrOut_0[t]);
-    if (t_hi < ntarget) arrOut_0[t_hi] = f((T)hi, arrOut_0[t_hi]);
-  } else {
-    if (lo) acc_hint_apply<ACC_SCOPE_DEVICE>(arrOut_0 + t, (T)lo, f);
-    if (hi && t_hi < ntarget) acc_hint_apply<ACC_SCOPE_DEVICE>(arrOut_0 + t_hi, (T)hi, f);
+  {
+    const T c = carry[t];
+    if (c != T(0)) carry[t] = T(0);
+    arrOut_0[t] = f((T)((T)lo + c), base[t]);
+  }
+  if (t_hi < ntarget) {
+    const T c = carry[t_hi];
+    if (c != T(0)) carry[t_hi] = T(0);
+    arrOut_0[t_hi] = f((T)((T)hi + c), base[t_hi]);
   }
 }
 #else

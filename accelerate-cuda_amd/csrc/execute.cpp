@@ -763,7 +763,13 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
       (narrow == 2 || (narrow == 1 && s->spec.get_small_constant))) {
     const int nv = (aligned ? 0 : 1) + 6;
     ACC_TRY(s->ensure_variant(nv));
-    if (copy_defaults) {                 // by a kernel of the instance's own: a third of the time a runtime copy of 256 KB takes
+    // A source spelt as a small constant never adds to the result directly: its corrections go to a table of carries
+    // (all zero between launches: the merge clears what it reads) and the merge writes  defaults + carries + rows,
+    // so nothing has to be in the result beforehand and the copy of the defaults is not a launch of its own.  Any
+    // other source (`permute.narrow=2`) may hold addends the table does not take; those go to the result, which must
+    // then hold the defaults before the main kernel starts.
+    const bool direct_adds = !s->spec.get_small_constant;
+    if (direct_adds && copy_defaults) {
       Args f;
       f.ptr(0);
       f.i64(0);
@@ -781,18 +787,18 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
     if (oe != hipSuccess || bpc < 1) { (void)hipGetLastError(); bpc = 1; }
     const int64_t cus_n = s->ctx->props.multiProcessorCount;
     const int64_t ngrid = acc_launch_grid(n_src, s->elements_per_block(), cus_n, bpc);
-    acc::ScratchRef nblk;
-    ACC_TRY(s->ctx->scratch_acquire((size_t)(ngrid * nwords) * 4, st, acc::SCRATCH_FOLD, &nblk));
-    const uint64_t ndump = reinterpret_cast<uint64_t>(nblk.ptr);
+    acc::ScratchRef nblk, cblk;
+    ACC_TRY(s->ctx->scratch_acquire((size_t)ntarget * esz, st, acc::SCRATCH_CARRY, &cblk));
+    int nrc = s->ctx->scratch_acquire((size_t)(ngrid * nwords) * 4, st, acc::SCRATCH_FOLD, &nblk);
+    if (nrc != ACC_OK) { s->ctx->scratch_release(cblk, st); return nrc; }
+    const uint64_t ndump = reinterpret_cast<uint64_t>(nblk.ptr), ncarry = reinterpret_cast<uint64_t>(cblk.ptr);
     args.i32(static_cast<int32_t>(ntarget));
     args.i32(1);
     args.ptr(ndump);
-    args.ptr(0);
+    args.ptr(ncarry);
     args.ptr(s->ctx->status_dev);
-    int nrc = launch(s, nv, ngrid, nlds, st, &args);
+    nrc = launch(s, nv, ngrid, nlds, st, &args);
     if (nrc == ACC_OK) {
-      const int64_t columns = (nwords + 255) / 256;
-      const int64_t slices = std::max<int64_t>(1, std::min<int64_t>(ngrid, (2 * cus_n + columns - 1) / columns));
       Args m;
       bool mal = true;
       nrc = push_env(s, env, &m, &mal);
@@ -800,14 +806,17 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
       m.ptr(ndump);
       m.i64(nwords);
       m.i32(static_cast<int32_t>(ngrid));
-      m.i32(static_cast<int32_t>(slices));
       m.i64(ntarget);
+      m.ptr(ncarry);
+      m.ptr(direct_adds ? out->ptr[0] : defaults->ptr[0]);
       if (nrc == ACC_OK) {
-        hipError_t me = launch_kernel(s->variants[nv].fn_finish, static_cast<unsigned>(columns * slices), 1, 1, 256, 1, 1, 0, st,
-                                              m.data(), nullptr);
+        // a workgroup per 64 words of a row, its four waves a quarter of the rows each
+        hipError_t me = launch_kernel(s->variants[nv].fn_finish, static_cast<unsigned>((nwords + 63) / 64), 1, 1, 256, 1, 1, 0, st,
+                                      m.data(), nullptr);
         if (me != hipSuccess) nrc = acc::fail_hip(me, "hipModuleLaunchKernel(permute_merge, narrow counts)");
       }
     }
+    s->ctx->scratch_release(cblk, st);
     s->ctx->scratch_release(nblk, st);
     return nrc;
   }

@@ -166,7 +166,7 @@ int acc_context_s::check_status(const char *who)
     for (int k = 0; k < acc::STATUS_WORDS; ++k) status_host[k] = 0;
     // a lock that never opened is still set: every lock block is cleared before it is lent again
     for (acc::ScratchBlock &b : scratch)
-      if (b.protocol == acc::SCRATCH_LOCKS) b.dirty = true;
+      if (b.protocol == acc::SCRATCH_LOCKS || b.protocol == acc::SCRATCH_CARRY) b.dirty = true;
   }
   return fail(ACC_ERR_STUCK, "%s: a kernel gave up waiting (%s%s%s): results of the work enqueued since the last successful synchronisation are not valid",
               who, seen[acc::STATUS_SCAN_LOOKBACK] ? "scan look-back " : "", seen[acc::STATUS_FOLD_COLLECT] ? "fold partial results " : "",
