@@ -489,8 +489,23 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
 #if ACC_PERMUTE_NARROW
   __syncthreads();
   {
-    unsigned *wrow = (unsigned *)dump + (Int64)blockIdx.x * nwords;
-    for (int i = threadIdx.x; i < nwords; i += ACC_BLOCK) wrow[i] = words[i];
+    /* A count leaves as its low byte: words i and i + nd of the table make one word of the row (bytes: targets
+     * i, i + nwords, i + nd, i + nd + nwords), half of what whole counts would write here and the merge read again.
+     * What a count holds above its low byte goes to the target's carry; few counts do (those of more than 255 of this
+     * workgroup's share of the source), and nothing but speed depends on how few. */
+    const int nd = (nwords + 1) / 2;
+    unsigned *wrow = (unsigned *)dump + (Int64)blockIdx.x * nd;
+    for (int i = threadIdx.x; i < nd; i += ACC_BLOCK) {
+      const unsigned a = words[i];
+      const unsigned b = i + nd < nwords ? words[i + nd] : 0u;
+      if ((a | b) & 0xFF00FF00u) {
+        if (a & 0x0000FF00u) acc_hint_apply<ACC_SCOPE_DEVICE>(far + i, (T)(a & 0xFF00u), f);
+        if (a & 0xFF000000u) acc_hint_apply<ACC_SCOPE_DEVICE>(far + i + nwords, (T)((a >> 16) & 0xFF00u), f);
+        if (b & 0x0000FF00u) acc_hint_apply<ACC_SCOPE_DEVICE>(far + i + nd, (T)(b & 0xFF00u), f);
+        if (b & 0xFF000000u) acc_hint_apply<ACC_SCOPE_DEVICE>(far + i + nd + nwords, (T)((b >> 16) & 0xFF00u), f);
+      }
+      wrow[i] = (a & 0xFFu) | ((a >> 8) & 0xFF00u) | ((b & 0xFFu) << 16) | ((b << 8) & 0xFF000000u);
+    }
   }
   (void)row;
 #else
@@ -540,13 +555,15 @@ struct acc_merge_job {
 };
 
 #if ACC_PERMUTE_NARROW
-/* result = base + carries + the sum of the workgroups' rows of packed 16-bit counts (`nwords` words a row, targets
- * `column` and `column + nwords` in a word).  A workgroup takes 64 consecutive words, each of its four waves a
- * quarter of the rows, eight loads in flight a lane; the waves' sums meet in LDS and the first wave writes the
- * result -- one thread per pair of targets, so no atomics and nothing that must be in the result beforehand -- and
- * clears the carries it has taken (the table is all zero between launches).  `base` is the defaults array, or the
- * result itself where that was filled from the defaults before the main kernel (which then also added to it
- * directly).                                                                                                */
+/* result = base + carries + the sum of the workgroups' rows of packed 8-bit counts.  A row has nd = ceil(nwords / 2)
+ * words; byte q of word `column` is the low byte of the count of target  column + (q & 2 ? nd : 0) + (q & 1 ? nwords : 0)
+ * (the main kernel's table holds targets w and w + nwords in word w, and sends words w and w + nd out as one).  A
+ * workgroup takes 64 consecutive words, each of its four waves a quarter of the rows, eight loads in flight a lane,
+ * whose bytes are added two to a register (8 x 255 fits 16 bits) before they are widened; the waves' sums meet in
+ * LDS and wave q writes the targets of byte q -- one thread per target, so no atomics and nothing that must be in
+ * the result beforehand -- and clears the carries it has taken (the table is all zero between launches).  `base` is
+ * the defaults array, or the result itself where that was filled from the defaults before the main kernel (which
+ * then also added to it directly).                                                                          */
 extern "C" __global__ void __launch_bounds__(256)
 permute_merge(ACC_ENV_PARAMS ACC_OUT_PARAMS, const unsigned *__restrict__ dump, const Int64 nwords, const int nrows,
               const Int64 ntarget, ACC_ELT *carry, const ACC_ELT *base ACC_GUARD_PARAM)
@@ -554,41 +571,40 @@ permute_merge(ACC_ENV_PARAMS ACC_OUT_PARAMS, const unsigned *__restrict__ dump, 
   ACC_GUARD_CHECK
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
-  __shared__ unsigned s_lo[4][64], s_hi[4][64];
+  __shared__ unsigned s_sum[4][4][64];           /* [wave][byte][lane] */
   auto f = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
   const int lane = threadIdx.x & 63, quarter = threadIdx.x >> 6;
+  const Int64 nd = (nwords + 1) / 2;
   const Int64 column = (Int64)blockIdx.x * 64 + lane;
-  const Int64 col_c = acc_min<Int64>(column, nwords - 1);       /* lanes past the end read the last word and drop it */
-  unsigned lo = 0u, hi = 0u;                     /* at most 65536 rows of counts below 0x10000 each */
+  const Int64 col_c = acc_min<Int64>(column, nd - 1);           /* lanes past the end read the last word and drop it */
+  unsigned c0 = 0u, c1 = 0u, c2 = 0u, c3 = 0u;
   int r = quarter;
   for (; r + 28 < nrows; r += 32) {
     unsigned w[8];
 #pragma unroll
-    for (int k = 0; k < 8; ++k) w[k] = __builtin_nontemporal_load(dump + (Int64)(r + 4 * k) * nwords + col_c);
+    for (int k = 0; k < 8; ++k) w[k] = __builtin_nontemporal_load(dump + (Int64)(r + 4 * k) * nd + col_c);
+    unsigned even = 0u, odd = 0u;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) { lo += w[k] & 0xFFFFu; hi += w[k] >> 16; }
+    for (int k = 0; k < 8; ++k) { even += w[k] & 0x00FF00FFu; odd += (w[k] >> 8) & 0x00FF00FFu; }
+    c0 += even & 0xFFFFu; c2 += even >> 16;
+    c1 += odd & 0xFFFFu;  c3 += odd >> 16;
   }
   for (; r < nrows; r += 4) {
-    const unsigned w = __builtin_nontemporal_load(dump + (Int64)r * nwords + col_c);
-    lo += w & 0xFFFFu;
-    hi += w >> 16;
+    const unsigned w = __builtin_nontemporal_load(dump + (Int64)r * nd + col_c);
+    c0 += w & 0xFFu; c1 += (w >> 8) & 0xFFu; c2 += (w >> 16) & 0xFFu; c3 += w >> 24;
   }
-  s_lo[quarter][lane] = lo;
-  s_hi[quarter][lane] = hi;
+  s_sum[quarter][0][lane] = c0;
+  s_sum[quarter][1][lane] = c1;
+  s_sum[quarter][2][lane] = c2;
+  s_sum[quarter][3][lane] = c3;
   __syncthreads();
-  if (quarter != 0 || column >= nwords) return;
-  lo = s_lo[0][lane] + s_lo[1][lane] + s_lo[2][lane] + s_lo[3][lane];
-  hi = s_hi[0][lane] + s_hi[1][lane] + s_hi[2][lane] + s_hi[3][lane];
-  const Int64 t = column, t_hi = column + nwords;
-  {
+  const unsigned total = s_sum[0][quarter][lane] + s_sum[1][quarter][lane] + s_sum[2][quarter][lane] + s_sum[3][quarter][lane];
+  const Int64 word = column + ((quarter & 2) ? nd : 0);          /* the word of the main kernel's table the count sat in */
+  const Int64 t = word + ((quarter & 1) ? nwords : 0);
+  if (column < nd && word < nwords && t < ntarget) {
     const T c = carry[t];
     if (c != T(0)) carry[t] = T(0);
-    arrOut_0[t] = f((T)((T)lo + c), base[t]);
-  }
-  if (t_hi < ntarget) {
-    const T c = carry[t_hi];
-    if (c != T(0)) carry[t_hi] = T(0);
-    arrOut_0[t_hi] = f((T)((T)hi + c), base[t_hi]);
+    arrOut_0[t] = f((T)((T)total + c), base[t]);
   }
 }
 #else

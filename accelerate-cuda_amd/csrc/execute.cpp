@@ -789,7 +789,8 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
     const int64_t ngrid = acc_launch_grid(n_src, s->elements_per_block(), cus_n, bpc);
     acc::ScratchRef nblk, cblk;
     ACC_TRY(s->ctx->scratch_acquire((size_t)ntarget * esz, st, acc::SCRATCH_CARRY, &cblk));
-    int nrc = s->ctx->scratch_acquire((size_t)(ngrid * nwords) * 4, st, acc::SCRATCH_FOLD, &nblk);
+    const int64_t nd = (nwords + 1) / 2;             // words a workgroup's row of 8-bit counts takes
+    int nrc = s->ctx->scratch_acquire((size_t)(ngrid * nd) * 4, st, acc::SCRATCH_FOLD, &nblk);
     if (nrc != ACC_OK) { s->ctx->scratch_release(cblk, st); return nrc; }
     const uint64_t ndump = reinterpret_cast<uint64_t>(nblk.ptr), ncarry = reinterpret_cast<uint64_t>(cblk.ptr);
     args.i32(static_cast<int32_t>(ntarget));
@@ -811,7 +812,7 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
       m.ptr(direct_adds ? out->ptr[0] : defaults->ptr[0]);
       if (nrc == ACC_OK) {
         // a workgroup per 64 words of a row, its four waves a quarter of the rows each
-        hipError_t me = launch_kernel(s->variants[nv].fn_finish, static_cast<unsigned>((nwords + 63) / 64), 1, 1, 256, 1, 1, 0, st,
+        hipError_t me = launch_kernel(s->variants[nv].fn_finish, static_cast<unsigned>((nd + 63) / 64), 1, 1, 256, 1, 1, 0, st,
                                       m.data(), nullptr);
         if (me != hipSuccess) nrc = acc::fail_hip(me, "hipModuleLaunchKernel(permute_merge, narrow counts)");
       }
