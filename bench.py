@@ -40,25 +40,25 @@ class Timer(object):
     """W warm-up steps, then exactly K timed steps: wall clock between two
     device synchronisations, and HIP events recorded on the launch stream."""
 
-    DEVICE_WARMUP_MS = 60.0       # once per process, before the first warm-up step: the device leaves its idle clocks
+    DEVICE_WARMUP_MS = 60.0       # before the first warm-up step of a run that finds the device idle: it leaves its idle clocks
+    IDLE_AFTER_S = 0.25           # (idle = nothing launched for this long: process start, a CPU leg, building inputs)
 
     def __init__(self, A, ctx, stream, steps, warmup):
         self.A, self.ctx, self.stream, self.steps, self.warmup = A, ctx, stream, steps, warmup
         self.e0, self.e1 = ctx.event(True), ctx.event(True)
-        self.device_is_warm = False
+        self.last_busy = None
 
     def run(self, step):
         """`step` is one callable, or a list of them (one per buffer set) taken round robin"""
         steps = step if isinstance(step, (list, tuple)) else [step]
         k = 0
-        if not self.device_is_warm:
+        if self.last_busy is None or time.perf_counter() - self.last_busy > self.IDLE_AFTER_S:
             t_end = time.perf_counter() + self.DEVICE_WARMUP_MS * 1e-3
             while time.perf_counter() < t_end:
                 for _ in range(16):
                     steps[k % len(steps)]()
                     k += 1
                 self.ctx.sync()
-            self.device_is_warm = True
         for _ in range(max(self.warmup, len(steps))):
             steps[k % len(steps)]()
             k += 1
@@ -72,6 +72,7 @@ class Timer(object):
         self.ctx.sync()
         wall_ms = (time.perf_counter() - t0) * 1e3 / self.steps
         event_ms = self.ctx.elapsed_ms(self.e0, self.e1) / self.steps
+        self.last_busy = time.perf_counter()
         return wall_ms, event_ms
 
 
