@@ -310,12 +310,19 @@ ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op, const T seed,
 #pragma unroll
   for (int r = 0; r < ACC_ROWS; ++r) ci[r] = acc_wave_scan(s[r][ACC_VEC - 1], op, lane);
 
-  V rowpre[ACC_ROWS];
+  /* (What the rows before row r of this wave come to is worked out again where it is used, by the same chain of
+   * operations, instead of being kept from here: where the operator has no scalar instruction -- Float64 `+` --
+   * that is two vector registers a row, and the instance then misses the 256 that let two workgroups share a
+   * compute unit.) */
+  /* (Elements of one register keep the values: the compiler holds them in scalar registers, and the headline
+   * scan's code stays what it was measured as.) */
+  constexpr bool KEEP_ROWS = sizeof(T) <= 4;
+  V rowpre[KEEP_ROWS ? ACC_ROWS : 1];
   V wave_total = acc_readlane(ci[0], ACC_WAVE - 1);
   rowpre[0] = wave_total;                                   /* unused */
 #pragma unroll
   for (int r = 1; r < ACC_ROWS; ++r) {
-    rowpre[r] = wave_total;
+    if (KEEP_ROWS) rowpre[r] = wave_total;
     wave_total = op(wave_total, acc_readlane(ci[r], ACC_WAVE - 1));
   }
 
@@ -364,12 +371,16 @@ ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op, const T seed,
   const int last_k = (int)(last_q % ACC_VEC), last_lane = (int)((last_q / ACC_VEC) % ACC_WAVE);
   const int last_row = (int)((last_q / (ACC_VEC * ACC_WAVE)) % ACC_ROWS), last_wave = (int)(last_q / (ACC_VEC * ACC_WAVE * ACC_ROWS));
   V whole = V();
+  V rows_before = V();                                      /* rows 0 .. r - 1 of this wave, for r > 0 */
 #pragma unroll
   for (int r = 0; r < ACC_ROWS; ++r) {
+    if (KEEP_ROWS)   rows_before = rowpre[r];
+    else if (r == 1) rows_before = acc_readlane(ci[0], ACC_WAVE - 1);
+    else if (r > 1)  rows_before = op(rows_before, acc_readlane(ci[r - 1], ACC_WAVE - 1));
     V b = S::some(prefix);
     bool has_b = has_prefix;
     if (wave > 0) { b = has_b ? op(b, wavepre) : wavepre; has_b = true; }
-    if (r > 0)    { b = has_b ? op(b, rowpre[r]) : rowpre[r]; has_b = true; }
+    if (r > 0)    { b = has_b ? op(b, rows_before) : rows_before; has_b = true; }
 
     const V e = acc_wave_shift_up1(ci[r]);                  /* total of the lanes before this one */
     V pre;
