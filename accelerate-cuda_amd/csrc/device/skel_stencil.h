@@ -33,9 +33,16 @@
  * Strips that are cut by the right edge, and arrays whose rows are not
  * 16-byte aligned, take a slower path that maps every element on its own.
  *
- * A 3-D stencil walks its strips plane by plane: a strip lies in one plane z
- * and keeps a register window per plane offset it reads (2 rz + 1 of them),
- * all advancing down the rows together.
+ * A 3-D stencil keeps a register window per plane it reads.  Without taps in
+ * other planes, or with ACC_ZMARCH 0, a strip lies in ACC_TZ planes and all its
+ * windows advance down the rows together.  With ACC_ZMARCH the two axes change
+ * places: a strip is ACC_TZ rows tall and walks through ACC_TILE_H planes, the
+ * windows hold the 2 ry + ACC_TZ rows it reads of each of the 2 rz + 1 planes
+ * in reach (plus the planes requested ahead), and a row fetched once serves
+ * the results of every plane that reads it -- what a walk down the rows reads
+ * 2 rz + ACC_TZ planes for, ACC_TZ at a time.  Everything below is written for
+ * a "marching" axis (the ring) and a "static" axis (the windows side by side);
+ * which of y and z is which is decided in a handful of places marked ACC_ZMARCH.
  *
  * With ACC_STENCIL_SOURCES == 2 the same kernel is stencil2
  * (CodeGen/Stencil.hs:118-237): two source arrays, each with its own taps,
@@ -58,7 +65,17 @@
 
 #define ACC_SVEC  4                                   /* results per lane and row */
 #define ACC_STRIP (ACC_WAVE * ACC_SVEC)               /* columns per wave */
-#define ACC_NR    (2 * ACC_RADIUS_Y + 1)              /* rows a result depends on */
+#ifndef ACC_ZMARCH
+#define ACC_ZMARCH 0
+#endif
+#if ACC_ZMARCH
+#define ACC_RADIUS_M ACC_RADIUS_Z                     /* reach along the axis the strip walks */
+#define ACC_RADIUS_S ACC_RADIUS_Y                     /* reach along the axis its windows lie side by side on */
+#else
+#define ACC_RADIUS_M ACC_RADIUS_Y
+#define ACC_RADIUS_S ACC_RADIUS_Z
+#endif
+#define ACC_NR    (2 * ACC_RADIUS_M + 1)              /* rows (planes) a result depends on */
 #define ACC_RING  (ACC_NR + ACC_PREFETCH)             /* rows held in registers */
 #define ACC_WW    (ACC_SVEC + 2 * ACC_RADIUS_X)       /* row window of one lane */
 #define ACC_WAVES (ACC_BLOCK / ACC_WAVE)
@@ -70,8 +87,8 @@
 #endif
 /* a strip produces ACC_TZ consecutive planes of the result from one register window over
  * ACC_NZ source planes: a source row fetched once serves the results of up to 2 rz + 1 planes */
-#define ACC_NZ    (2 * ACC_RADIUS_Z + ACC_TZ)         /* planes held */
-#define ACC_TOTAL_MAX  (ACC_TILE_H + 2 * ACC_RADIUS_Y)        /* source rows a strip touches, per plane */
+#define ACC_NZ    (2 * ACC_RADIUS_S + ACC_TZ)         /* planes (rows) held side by side */
+#define ACC_TOTAL_MAX  (ACC_TILE_H + 2 * ACC_RADIUS_M)        /* source rows (planes) a strip touches, per window */
 #define ACC_HALO_COUNT (2 * ACC_RADIUS_X * ACC_TOTAL_MAX * ACC_NZ)   /* elements just outside the strip */
 #define ACC_HALO_LOADS (ACC_HALO_COUNT > 0 ? (ACC_HALO_COUNT + ACC_WAVE - 1) / ACC_WAVE : 1)
 
@@ -115,6 +132,25 @@ struct acc_strip_source {
   int lane, total;          /* total = source rows the strip touches in each plane */
   row ring[ACC_NZ][ACC_RING];
   S halo[ACC_HALO_LOADS];
+#if ACC_ZMARCH
+  S halo_ring[ACC_RING];    /* lane (p * 2 + side) * rx + j: the element outside the strip for window p of the slot's plane */
+#endif
+  /* window p, line rho of the strip's walk: which plane and row of the source that is */
+  ACC_DEV Int64 plane_of(const int p, const int rho) const { return ACC_ZMARCH ? z0 - ACC_RADIUS_Z + rho : z0 - ACC_RADIUS_Z + p; }
+  ACC_DEV Int64 row_of(const int p, const int rho) const   { return ACC_ZMARCH ? y0 - ACC_RADIUS_Y + p : y0 - ACC_RADIUS_Y + rho; }
+  /* one element outside the strip: window p, line rho, `side` 0 left 1 right, the j-th of rx */
+  ACC_DEV S outside_element(const int p, const int rho, const int side, const int j) const
+  {
+    const Int64 gz = plane_of(p, rho), gy = row_of(p, rho);
+    const Int64 xx = side ? x0 + ACC_STRIP + j : x0 - ACC_RADIUS_X + j;
+    if (MODE == ACC_B_CONSTANT) {
+      const bool inside = gz >= 0 && gz < d && gy >= 0 && gy < h && xx >= 0 && xx < w;
+      const Int64 mz = acc_max<Int64>(0, acc_min<Int64>(gz, d - 1));
+      const Int64 my = acc_max<Int64>(0, acc_min<Int64>(gy, h - 1)), mx = acc_max<Int64>(0, acc_min<Int64>(xx, w - 1));
+      return inside ? base[(mz * h + my) * w + mx] : outside;
+    }
+    return base[(acc_boundary_index<MODE>(gz, d) * h + acc_boundary_index<MODE>(gy, h)) * w + acc_boundary_index<MODE>(xx, w)];
+  }
 
   /* FAST: the 2 rx elements just outside the strip, for every source row the
    * strip will touch, are requested in one go -- lane q takes element
@@ -123,7 +159,7 @@ struct acc_strip_source {
    * for the strip instead of two per row. */
   ACC_DEV void gather_halo()
   {
-    if (!FAST) return;
+    if (!FAST || ACC_ZMARCH) return;                       /* (a strip that walks through planes asks line by line: fetch) */
 #pragma unroll
     for (int g = 0; g < ACC_HALO_LOADS; ++g) {
       const int q = lane + ACC_WAVE * g;
@@ -132,23 +168,16 @@ struct acc_strip_source {
       const int side = qq / (ACC_RADIUS_X * ACC_TOTAL_MAX + (ACC_RADIUS_X == 0)), rem = qq % (ACC_RADIUS_X * ACC_TOTAL_MAX + (ACC_RADIUS_X == 0));
       const int j = rem / ACC_TOTAL_MAX, rho = rem % ACC_TOTAL_MAX;
       halo[g] = S();
-      if (q < ACC_HALO_COUNT && rho < total) {
-        const Int64 gz = z0 - ACC_RADIUS_Z + p;
-        const Int64 gy = y0 - ACC_RADIUS_Y + rho;
-        const Int64 xx = side ? x0 + ACC_STRIP + j : x0 - ACC_RADIUS_X + j;
-        if (MODE == ACC_B_CONSTANT) {
-          const bool inside = gz >= 0 && gz < d && gy >= 0 && gy < h && xx >= 0 && xx < w;
-          const Int64 mz = acc_max<Int64>(0, acc_min<Int64>(gz, d - 1));
-          const Int64 my = acc_max<Int64>(0, acc_min<Int64>(gy, h - 1)), mx = acc_max<Int64>(0, acc_min<Int64>(xx, w - 1));
-          halo[g] = inside ? base[(mz * h + my) * w + mx] : outside;
-        } else {
-          halo[g] = base[(acc_boundary_index<MODE>(gz, d) * h + acc_boundary_index<MODE>(gy, h)) * w + acc_boundary_index<MODE>(xx, w)];
-        }
-      }
+      if (q < ACC_HALO_COUNT && rho < total) halo[g] = outside_element(p, rho, side, j);
     }
   }
-  ACC_DEV S halo_of(const int p, const int side, const int j, const int rho) const
+  ACC_DEV S halo_of(const int p, const int side, const int j, const int rho, const int slot) const
   {
+#if ACC_ZMARCH
+    (void)rho;
+    return acc_readlane(halo_ring[slot], (p * 2 + side) * ACC_RADIUS_X + j);
+#endif
+    (void)slot;
     const int q = p * (2 * ACC_RADIUS_X * ACC_TOTAL_MAX) + (side * ACC_RADIUS_X + j) * ACC_TOTAL_MAX + rho;
     S v = acc_readlane(halo[0], q % ACC_WAVE);
 #pragma unroll
@@ -161,14 +190,23 @@ struct acc_strip_source {
    * path the left and right parts are only valid once finish() has run */
   ACC_DEV void fetch(const int rho, const int slot)
   {
+#if ACC_ZMARCH
+    /* the 2 rx elements outside the strip of all the windows' rows of this plane: one request, a lane each */
+    static_assert(ACC_NZ * 2 * ACC_RADIUS_X <= ACC_WAVE, "more elements outside the strip than lanes to ask for them");
+    if (FAST && ACC_RADIUS_X > 0) {
+      constexpr int rx = ACC_RADIUS_X > 0 ? ACC_RADIUS_X : 1;
+      halo_ring[slot] = S();
+      if (lane < ACC_NZ * 2 * rx) halo_ring[slot] = outside_element(lane / (2 * rx), rho, (lane / rx) % 2, lane % rx);
+    }
+#endif
 #pragma unroll
     for (int p = 0; p < ACC_NZ; ++p) fetch_plane(p, rho, slot);
   }
   ACC_DEV void fetch_plane(const int p, const int rho, const int slot)
   {
     row &r = ring[p][slot];
-    const Int64 gz = z0 - ACC_RADIUS_Z + p;
-    const Int64 gy = y0 - ACC_RADIUS_Y + rho;
+    const Int64 gz = plane_of(p, rho);
+    const Int64 gy = row_of(p, rho);
     const bool row_inside = MODE != ACC_B_CONSTANT || (gy >= 0 && gy < h && gz >= 0 && gz < d);
     const Int64 my = MODE == ACC_B_CONSTANT ? acc_max<Int64>(0, acc_min<Int64>(gy, h - 1)) : acc_boundary_index<MODE>(gy, h);
     const Int64 mz = MODE == ACC_B_CONSTANT ? acc_max<Int64>(0, acc_min<Int64>(gz, d - 1)) : acc_boundary_index<MODE>(gz, d);
@@ -210,8 +248,12 @@ struct acc_strip_source {
       for (int j = 0; j < ACC_RADIUS_X; ++j) {
         const S from_left  = acc_wave_shift_up1(r.e[ACC_SVEC + j]);          /* neighbour's own[SVEC - rx + j] */
         const S from_right = acc_wave_shift_down1(r.e[ACC_RADIUS_X + j]);    /* neighbour's own[j] */
-        r.e[j] = (lane != 0) ? from_left : halo_of(p, 0, j, rho);
-        r.e[ACC_RADIUS_X + ACC_SVEC + j] = (lane != ACC_WAVE - 1) ? from_right : halo_of(p, 1, j, rho);
+        /* (read by every lane, before the choice: a read of another lane's register made under a condition sees
+         * whatever that lane holds where only the lanes that pass the condition have worked the value out -- for
+         * an element narrower than a register, its widening) */
+        const S outside_left = halo_of(p, 0, j, rho, slot), outside_right = halo_of(p, 1, j, rho, slot);
+        r.e[j] = (lane != 0) ? from_left : outside_left;
+        r.e[ACC_RADIUS_X + ACC_SVEC + j] = (lane != ACC_WAVE - 1) ? from_right : outside_right;
       }
     }
   }
@@ -260,11 +302,19 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS ACC_GUARD_PARA
    * rows they share are then requested from the same compute unit, where the
    * second request merges with the first instead of going out to memory */
   const Int64 group = strip / ACC_WAVES, within = strip % ACC_WAVES;
-  const Int64 band = (group / strips_x) * ACC_WAVES + within, x0 = (group % strips_x) * ACC_STRIP;
+  const Int64 band = (group / strips_x) * ACC_WAVES + within, x0_across = (group % strips_x) * ACC_STRIP;
 #else
-  const Int64 band = strip / strips_x, x0 = (strip % strips_x) * ACC_STRIP;
+  const Int64 band = strip / strips_x, x0_across = (strip % strips_x) * ACC_STRIP;
 #endif
-#if ACC_STENCIL_RANK == 3
+#if ACC_STENCIL_RANK == 3 && ACC_ZMARCH
+  /* strips ACC_TZ rows tall, numbered DOWN a plane first (the waves of a workgroup are vertical neighbours: the rows
+   * they share are asked for by one compute unit at about the same time), then across it, then run of ACC_TILE_H
+   * planes after run */
+  const Int64 bands = (h + ACC_TZ - 1) / ACC_TZ;
+  const Int64 across = strip / bands;
+  const Int64 z0 = (across / strips_x) * ACC_TILE_H, y0 = (strip % bands) * ACC_TZ;
+  if (z0 >= d) return;
+#elif ACC_STENCIL_RANK == 3
   const Int64 bands = (h + ACC_TILE_H - 1) / ACC_TILE_H;
   const Int64 z0 = (band / bands) * ACC_TZ, y0 = (band % bands) * ACC_TILE_H;
   if (z0 >= d) return;
@@ -272,8 +322,15 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS ACC_GUARD_PARA
   const Int64 z0 = 0, y0 = band * ACC_TILE_H;
 #endif
   if (y0 >= h) return;                                   /* whole wave leaves together */
+#if ACC_STENCIL_RANK == 3 && ACC_ZMARCH
+  const Int64 x0 = (across % strips_x) * ACC_STRIP;
+  (void)band; (void)x0_across;
+#else
+  const Int64 x0 = x0_across;
+#endif
   const Int64 gx = x0 + lane * ACC_SVEC;
-  const int rows_here = (int)acc_min<Int64>(ACC_TILE_H, h - y0);
+  /* how far the strip walks: rows, or planes */
+  const int rows_here = (int)acc_min<Int64>(ACC_TILE_H, ACC_ZMARCH ? d - z0 : h - y0);
   const bool fast_here = (x0 + ACC_STRIP <= w);          /* every lane owns a full vector */
 
   /* the strip, compiled three times: fast and ACC_TILE_H rows tall (all constants),
@@ -281,7 +338,7 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS ACC_GUARD_PARA
   auto run = [&](auto fast_c, auto full_c) {
   constexpr bool fast = decltype(fast_c)::value;
   const int rows = decltype(full_c)::value ? ACC_TILE_H : rows_here;
-  const int total = rows + 2 * ACC_RADIUS_Y;              /* source rows this strip touches */
+  const int total = rows + 2 * ACC_RADIUS_M;              /* source rows (planes) this strip touches */
 
   /* one strip source per component of either source's element: a<c> for the first source, b<c> for the second */
 #if ACC_STENCIL_SOURCES == 2
@@ -346,22 +403,28 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS ACC_GUARD_PARA
 
 #pragma unroll
         for (int pz = 0; pz < ACC_TZ; ++pz) {
-        if (ACC_TZ > 1 && z0 + pz >= d) break;               /* the last band of planes may be short */
+        if (ACC_TZ > 1 && (ACC_ZMARCH ? y0 + pz >= h : z0 + pz >= d)) break;   /* the last band of planes (rows) may be short */
         acc_out_vec res;
 #pragma unroll
         for (int k = 0; k < ACC_SVEC; ++k) {
-#define ACC_WINDOW_READ(c, dz, dy, dx) a##c.ring[pz + ACC_RADIUS_Z + (dz)][(s + ACC_RADIUS_Y + (dy)) % ACC_RING].e[ACC_RADIUS_X + k + (dx)]
+#if ACC_ZMARCH
+#define ACC_WINDOW_AT(dz, dy) [pz + ACC_RADIUS_Y + (dy)][(s + ACC_RADIUS_Z + (dz)) % ACC_RING]
+#else
+#define ACC_WINDOW_AT(dz, dy) [pz + ACC_RADIUS_Z + (dz)][(s + ACC_RADIUS_Y + (dy)) % ACC_RING]
+#endif
+#define ACC_WINDOW_READ(c, dz, dy, dx) a##c.ring ACC_WINDOW_AT(dz, dy).e[ACC_RADIUS_X + k + (dx)]
           ACC_STENCIL_TAPS1(ACC_WINDOW_READ)
 #undef ACC_WINDOW_READ
 #if ACC_STENCIL_SOURCES == 2
-#define ACC_WINDOW_READ(c, dz, dy, dx) b##c.ring[pz + ACC_RADIUS_Z + (dz)][(s + ACC_RADIUS_Y + (dy)) % ACC_RING].e[ACC_RADIUS_X + k + (dx)]
+#define ACC_WINDOW_READ(c, dz, dy, dx) b##c.ring ACC_WINDOW_AT(dz, dy).e[ACC_RADIUS_X + k + (dx)]
           ACC_STENCIL_TAPS2(ACC_WINDOW_READ)
 #undef ACC_WINDOW_READ
 #endif
+#undef ACC_WINDOW_AT
           res.v[k] = (T)(ACC_STENCIL_FN);
         }
         /* one vector store per component of the result (a tuple result is one array per component) */
-        const Int64 at = (((z0 + pz) * h) + (y0 + y)) * w + gx;
+        const Int64 at = ACC_ZMARCH ? (((z0 + y) * h) + (y0 + pz)) * w + gx : (((z0 + pz) * h) + (y0 + y)) * w + gx;
 #define ACC_STORE_COMPONENT(c, CT)                                                   \
         {                                                                            \
           CT *dst = arrOut_##c + at;                                                 \

@@ -1028,7 +1028,11 @@ static int stencil_once(acc_skel s, const acc_array *env, const acc_array *in, c
   const int64_t strips_x = (w + s->spec.tile_w - 1) / s->spec.tile_w;
   int64_t bands = (h + s->spec.tile_h - 1) / s->spec.tile_h;
   if (rank == 2 && acc::tune("stencil.stack", 0)) bands = (bands + waves - 1) / waves * waves;
-  const int64_t zbands = (planes + s->spec.tile_z - 1) / s->spec.tile_z;       // tile_z result planes per strip
+  int64_t zbands = (planes + s->spec.tile_z - 1) / s->spec.tile_z;             // tile_z result planes per strip
+  if (s->spec.zmarch) {                  // strips tile_z rows tall that walk through tile_h planes
+    bands = (h + s->spec.tile_z - 1) / s->spec.tile_z;
+    zbands = (planes + s->spec.tile_h - 1) / s->spec.tile_h;
+  }
   return launch(s, aligned ? 0 : 1, (strips_x * bands * zbands + waves - 1) / waves, 0, st, &args);
 }
 

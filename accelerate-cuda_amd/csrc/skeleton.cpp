@@ -356,6 +356,7 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "#define ACC_STACK_WAVES " << (sp.out_rank == 2 ? tune("stencil.stack", 0) : 0) << "\n";
       o << "#define ACC_TILE_H " << sp.tile_h << "\n#define ACC_PREFETCH " << sp.prefetch << "\n#define ACC_BLOCK " << sp.block << "\n";
       o << "#define ACC_TZ " << sp.tile_z << "\n";
+      o << "#define ACC_ZMARCH " << sp.zmarch << "\n";
       tmpl = "skel_stencil.h";
       break;
     }
@@ -594,8 +595,8 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
       // (each source row it fetches then serves several planes instead of one), as many as keep the window of all
       // sources within 128 registers a lane
       int planes_per_strip = 1;
+      int rz = 0, ry = 0, rx = 0;        // both sources' windows span the larger of the two radii
       if (sp->out_rank == 3) {
-        int rz = 0, ry = 0, rx = 0;      // both sources' windows span the larger of the two radii
         auto reach = [&](const std::vector<int> &dz, const std::vector<int> &dy, const std::vector<int> &dx) {
           for (size_t k = 0; k < dx.size(); ++k) { rz = std::max(rz, std::abs(dz[k])); ry = std::max(ry, std::abs(dy[k])); rx = std::max(rx, std::abs(dx[k])); }
         };
@@ -604,13 +605,26 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
         int words = 0;
         for (const std::string &c : sp->stencil_in_comps) words += std::max(1, (type_size(c) + 3) / 4);
         for (const std::string &c : sp->stencil_in2_comps) words += std::max(1, (type_size(c) + 3) / 4);
-        for (int tz = 3; rz > 0 && tz > 1 && planes_per_strip == 1; --tz)
-          if ((2 * rz + tz) * (2 * ry + 1 + sp->prefetch) * (4 + 2 * rx) * words <= 128) planes_per_strip = tz;
+        // Taps in other planes: the strip walks through the planes instead of down the rows, so that a row fetched once
+        // serves all the planes that read it; it is as many rows tall as keep the windows within 144 registers
+        // (2 ry + rows of them side by side, 2 rz + 1 + prefetch planes deep).
+        sp->zmarch = (rz > 0 && 2 * rx * (2 * ry + 1) <= 64) ? (tune("stencil.zmarch", 1) ? 1 : 0) : 0;
+        if (sp->zmarch) {
+          for (int ty = 4; ty > 1 && planes_per_strip == 1; --ty)
+            if ((2 * ry + ty) * (2 * rz + 1 + sp->prefetch) * (4 + 2 * rx) * words <= 144) planes_per_strip = ty;
+          while (2 * rx * (2 * ry + planes_per_strip) > 64) --planes_per_strip;     // one lane each for the elements outside the strip
+        } else {
+          for (int tz = 3; rz > 0 && tz > 1 && planes_per_strip == 1; --tz)
+            if ((2 * rz + tz) * (2 * ry + 1 + sp->prefetch) * (4 + 2 * rx) * words <= 128) planes_per_strip = tz;
+        }
       }
       sp->tile_z = sp->out_rank == 3 ? tune("stencil.tile_z", planes_per_strip) : 1;
       // rows per strip: short in 2-D (a compact window of the image in flight), taller in 3-D where every row is
-      // read from 2 rz + tile_z planes and the boundary rows of a strip cost that much more
-      sp->tile_h = sp->out_rank == 2 ? tune("stencil.tile_h", 4) : (sp->out_rank == 3 ? tune("stencil.tile_h3", sp->tile_z > 1 ? 8 : 16) : 1);
+      // read from 2 rz + tile_z planes and the boundary rows of a strip cost that much more; planes per walk where
+      // the strip goes through planes
+      sp->tile_h = sp->out_rank == 2 ? tune("stencil.tile_h", 4)
+                 : (sp->out_rank == 3 ? (sp->zmarch ? tune("stencil.walk", 64) : tune("stencil.tile_h3", sp->tile_z > 1 ? 8 : 16)) : 1);
+      if (sp->zmarch && 2 * rx * (2 * ry + sp->tile_z) > 64) return fail(ACC_ERR_INVALID, "stencil: strip too tall for its reach");
       if (sp->tile_h < 1 || sp->prefetch < 0 || sp->prefetch > 8 || sp->tile_z < 1 || sp->tile_z > 8) return fail(ACC_ERR_INVALID, "stencil: bad tile shape");
       break;
     }

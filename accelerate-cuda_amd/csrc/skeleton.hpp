@@ -38,7 +38,8 @@ struct SkelSpec {
   std::string boundary2_constant, stencil_in2_type;
   std::vector<int> tap2_dz, tap2_dy, tap2_dx;
   int tile_w = 256, tile_h = 4, prefetch = 3;
-  int tile_z = 1;                       // rank-3 stencils: result planes per strip
+  int tile_z = 1;                       // rank-3 stencils: result planes per strip (rows per strip where the strip walks through planes)
+  int zmarch = 0;                       // rank-3 stencils: strips tile_z rows tall walk through tile_h planes
   // tuning
   int block = 256, unroll = 4, rows = 4, chunk = 4096;
   bool guarded = false;                 // ACC_FLAG_GUARDED: every kernel takes the address of a loop's guard word last

@@ -14,7 +14,9 @@ pytestmark = pytest.mark.gpu
 F = np.float32
 SEVEN = [(0, 0, 0), (-1, 0, 0), (1, 0, 0), (0, -1, 0), (0, 1, 0), (0, 0, -1), (0, 0, 1)]
 BOX = [(dz, dy, dx) for dz in (-1, 0, 1) for dy in (-1, 0, 1) for dx in (-1, 0, 1)]
-SHAPES = [(1, 1, 1), (3, 3, 3), (5, 7, 9), (3, 33, 70), (4, 64, 256), (6, 37, 517), (2, 16, 1024), (17, 40, 260)]
+# (the last two are deeper than one walk through the planes: strips that continue one another, the last one short)
+SHAPES = [(1, 1, 1), (3, 3, 3), (5, 7, 9), (3, 33, 70), (4, 64, 256), (6, 37, 517), (2, 16, 1024), (17, 40, 260),
+          (70, 10, 260), (131, 5, 512)]
 
 
 def say(*a):
@@ -114,3 +116,20 @@ def test_stencil_3d_window_shapes(A, ctx, case):
         sk.stencil([], ctx.array(v), out)
         t = pyref.tap_arrays3(v, taps, "mirror", 0, shape)
         assert np.array_equal(out.get(), sum(T(k % 7 - 3) * t[k] for k in range(len(taps))))
+
+
+def test_stencil_3d_strip_edges_of_narrow_elements(A, ctx):
+    """what a strip reads just outside its 256 columns comes from another lane's register: elements narrower than
+    a register (Int8, Word16) at widths of several strips, first plane included, every boundary mode"""
+    rng = np.random.default_rng(34)
+    for ctype, T in (("Int8", np.int8), ("Word16", np.uint16)):
+        for mode in ("clamp", "mirror", "wrap", "constant"):
+            sk = ctx.skeleton(A.SKEL_STENCIL, ctype, out_rank=3, taps=BOX, boundary=mode, boundary_constant="(%s)3" % ctype,
+                              stencil_fn="(%s)(%s)" % (ctype, " + ".join("t%d" % k for k in range(27))))
+            for shape in ((2, 4, 256), (4, 9, 1031), (66, 6, 512)):
+                say("stencil 3-D", ctype, mode, shape)
+                v = rng.integers(0, 4, shape).astype(T)
+                out = ctx.empty(shape, T)
+                sk.stencil([], ctx.array(v), out)
+                t = pyref.tap_arrays3(v, BOX, mode, 3, shape)
+                assert np.array_equal(out.get(), sum(a.astype(np.int64) for a in t).astype(T))
