@@ -1,0 +1,84 @@
+"""Stencils drawn at random (rank, reach in every dimension, which taps, coefficients, element type, boundary mode)
+on shapes drawn around the strip width and the length of a walk through the planes, against numpy index maps
+(tests/pyref.py).  Sources hold small integers, so every operation is exact in every element type and the results are
+compared bit for bit.  The seed is fixed: the same instances every run."""
+import itertools
+import sys
+
+import numpy as np
+import pytest
+
+import pyref
+
+pytestmark = pytest.mark.gpu
+
+TYPES = [("Int8", np.int8), ("Word16", np.uint16), ("Int32", np.int32), ("Int64", np.int64), ("float", np.float32),
+         ("double", np.float64)]
+
+
+def say(*a):
+    print("[case]", *a)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def A():
+    import acchip
+    return acchip
+
+
+@pytest.fixture(scope="module")
+def ctx(A):
+    c = A.Context(0)
+    yield c
+    c.close()
+
+
+def near(rng, mult, hi):
+    return max(1, int(rng.integers(0, hi // mult + 1)) * mult + int(rng.choice([-3, -1, 0, 0, 1, 2, 5, 17, 100])))
+
+
+@pytest.mark.parametrize("rank", [1, 2, 3])
+def test_random_stencils(A, ctx, rank):
+    rng = np.random.default_rng(1000 + rank)
+    for trial in range(10 if rank < 3 else 14):
+        ctype, T = TYPES[int(rng.integers(0, len(TYPES)))]
+        mode = str(rng.choice(["clamp", "mirror", "wrap", "constant"]))
+        reach = [int(rng.integers(0, 3)) for _ in range(rank)]
+        if rank < 3:
+            reach[-1] = int(rng.integers(0, 5))
+        box = list(itertools.product(*[range(-r, r + 1) for r in reach]))
+        taps = [box[i] for i in rng.choice(len(box), int(rng.integers(1, min(len(box), 9) + 1)), replace=False)]
+        for d in range(rank):                                  # the extremes, so that the reach is what was drawn
+            for sign in (-1, 1):
+                t = [0] * rank
+                t[d] = sign * reach[d]
+                if tuple(t) not in taps:
+                    taps.append(tuple(t))
+        coef = [int(rng.integers(-2, 3)) for _ in taps]
+        whole = np.issubdtype(T, np.integer)
+        fn = " + ".join("(%s)(%d) * t%d" % (ctype, c, k) for k, c in enumerate(coef))
+        sk = ctx.skeleton(A.SKEL_STENCIL, ctype, out_rank=rank, taps=taps if rank > 1 else [(0, t[0]) for t in taps],
+                          boundary=mode, boundary_constant="(%s)2" % ctype, stencil_fn="(%s)(%s)" % (ctype, fn) if whole else fn)
+        for _ in range(2):
+            shape = [near(rng, 256, 1100) if rng.random() < 0.7 else int(rng.integers(1, 80))]
+            if rank >= 2:
+                shape.insert(0, int(rng.integers(1, 70)))
+            if rank == 3:
+                shape.insert(0, near(rng, 64, 140) if rng.random() < 0.5 else int(rng.integers(1, 12)))
+            shape = tuple(max(s, r + 1) for s, r in zip(shape, reach))      # the index maps assume the array spans the stencil
+            say("stencil", ctype, mode, "taps", taps, "shape", shape)
+            v = rng.integers(0, 4, shape).astype(T)
+            out = ctx.empty(shape, T)
+            sk.stencil([], ctx.array(v), out)
+            if rank == 3:
+                t = pyref.tap_arrays3(v, taps, mode, 2, shape)
+            elif rank == 2:
+                t = pyref.tap_arrays(v, taps, mode, 2, shape)
+            else:
+                t = [a[0] for a in pyref.tap_arrays(v.reshape(1, -1), [(0, x[0]) for x in taps], mode, 2, (1, shape[0]))]
+            if whole:
+                ref = sum(np.int64(c) * a.astype(np.int64) for c, a in zip(coef, t)).astype(T)
+            else:
+                ref = sum(T(c) * a for c, a in zip(coef, t)).astype(T)
+            assert np.array_equal(out.get(), ref)
