@@ -486,7 +486,7 @@ def main():
         "ms_per_step": headline["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int32", "data": "synthetic (seeded SplitMix64, resident in HBM before the timed region)",
         "config": {"workload": workload, "elements": n, "buffer_sets": S,
-                   "timing": "kernel launches back to back on one stream, inputs device-resident, consecutive launches on different buffer sets; %d ms of untimed launches once before the first configuration's warm-up steps" % int(Timer.DEVICE_WARMUP_MS)},
+                   "timing": "kernel launches back to back on one stream, inputs device-resident, consecutive launches on different buffer sets; %d ms of untimed launches before the warm-up steps of every configuration that finds the device idle" % int(Timer.DEVICE_WARMUP_MS)},
         "roofline": {"bound": "hbm", "achieved": headline["GB_per_s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(headline["GB_per_s"] / HBM_PEAK_GBS, 4),
                      "traffic": headline.get("hbm_traffic_bytes"), "traffic_source": headline.get("hbm_traffic_source"),
