@@ -162,6 +162,17 @@ def main():
     log("device: arch %s, %d CUs, LDS/workgroup %d, L2 %d" % (props.arch.decode(), props.compute_units, props.lds_per_block, props.l2_bytes))
     stream = ctx.stream()
     T = Timer(A, ctx, stream, args.steps, args.warmup)
+
+    def traced(steps, calls=12):
+        """the same launches one by one onto an idle device, an event before and behind each (acc_trace_start/stop):
+        the way the front-end leg below is timed, for the figure its calls are to be held against"""
+        ctx.sync()
+        ctx.trace_start()
+        for k in range(calls):
+            steps[k % len(steps)]()
+            ctx.sync()
+        launches, ms = ctx.trace_stop()
+        return round(ms * 1e3 / calls, 3)
     L = A.lib()
     F32, I32 = (1, "float"), (1, "Int32")
     sk = {}
@@ -196,6 +207,7 @@ def main():
             w, e = T.run([step(i) for i in range(S)])
             sk[kind] = result(kind + " (+) Int32 2^26", w, e, 1, 2 * n * 4 + 4, n, {"traffic_key": kind})
             if kind == "scanl":
+                sk[kind]["one_by_one_us"] = traced([step(i) for i in range(S)])
                 sk[kind]["end_to_end"] = end_to_end(ctx, [(dxs[0], x)], step(0), outs[0])
                 headline = dict(sk[kind], wall_ms=w, event_ms=e)
                 # size-independent check: the last element is the sum, the first the seed
@@ -272,10 +284,11 @@ def main():
         def step(i):
             return lambda: A.check(L.acc_exec_fold(dot.handle, env_s[i], 1, sh, C.byref(od), stream))
         w, e = T.run([step(i) for i in range(Sd)])
+        dot_one_by_one = traced([step(i) for i in range(Sd)])
         truth = float(np.dot(x.astype(np.float64), y.astype(np.float64)))
         sk["dot"] = result("fold (+) 0 . zipWith (*) 2^24", w, e, 1, 2 * nd * 4 + 4, nd,
                            {"result": float(o.get()), "float64_truth": truth, "GFLOP_per_s": round(2 * nd / (e * 1e-3) / 1e9, 1),
-                            "traffic_key": "foldAll"})
+                            "traffic_key": "foldAll", "one_by_one_us": dot_one_by_one})
         sk["dot"]["end_to_end"] = end_to_end(ctx, [(dxs[0], x), (dys[0], y)], step(0), o)
         if not args.no_cpu:
             from oracle import oracle as orc
@@ -369,11 +382,12 @@ def main():
         def step(i):
             return lambda: A.check(L.acc_exec_foldseg(smvm.handle, env_s[i], nnz, C.byref(offd[i]), C.byref(yd[i]), stream))
         w, e = T.run([step(i) for i in range(S)])
+        smvm_one_by_one = traced([step(i) for i in range(S)])
         y = ys[S - 1]
         sk["smvm"] = result("foldSeg (+) . zipWith (*) . gather", w, e, 1, nnz * 8 + rows * 8 + xv.size * 4, nnz,
                             {"nnz": int(nnz), "GFLOP_per_s": round(2 * nnz / (e * 1e-3) / 1e9, 1),
                              "note": "segment offsets precomputed on the device (scanl over the 2^20 lengths is not in the step)",
-                             "traffic_key": "foldSeg"})
+                             "traffic_key": "foldSeg", "one_by_one_us": smvm_one_by_one})
         sk["smvm"]["end_to_end"] = end_to_end(ctx, [(dv[0], vals), (dc[0], cols), (dxv[0], xv), (doff[0], offs)], step(0), ys[0])
         if not args.no_cpu:
             from oracle import oracle as orc
@@ -418,16 +432,18 @@ def main():
         xs, ys_ = [acc.use(x.copy(), fcx) for _ in range(Sd)], [acc.use(y.copy(), fcx) for _ in range(Sd)]
         r, us, nk = front(lambda i: acc.fold(add, 0.0, acc.zipWith(lambda a, b: a * b, xs[i], ys_[i]), context=fcx), Sd)
         fe["dot"] = {"gpu_us_per_call": us, "kernels_per_call": nk, "direct_avg_launch_us": sk.get("dot", {}).get("avg_launch_us"),
+                     "direct_one_by_one_us": sk.get("dot", {}).get("one_by_one_us"),
                      "result": float(acc.run(r, fcx))}
-        log("  front end dotp                 %9.3f us/call on the device, %d kernel(s)" % (us, nk))
+        log("  front end dotp                 %9.3f us/call on the device, %d kernel(s); the hand-written fragment one by one: %s" % (us, nk, fe["dot"]["direct_one_by_one_us"]))
         del xs, ys_, r
         xsc = wl.scan_input(n)
         xs = [acc.use(xsc.copy(), fcx) for _ in range(S)]
         r, us, nk = front(lambda i: acc.scanl(add, 0, xs[i], context=fcx), S)
         got = acc.run(r, fcx)
         assert int(got[-1]) == int(xsc.sum(dtype=np.int64)), "front end scanl mismatch"
-        fe["scanl"] = {"gpu_us_per_call": us, "kernels_per_call": nk, "direct_avg_launch_us": sk.get("scanl", {}).get("avg_launch_us")}
-        log("  front end scanl                %9.3f us/call on the device, %d kernel(s)" % (us, nk))
+        fe["scanl"] = {"gpu_us_per_call": us, "kernels_per_call": nk, "direct_avg_launch_us": sk.get("scanl", {}).get("avg_launch_us"),
+                       "direct_one_by_one_us": sk.get("scanl", {}).get("one_by_one_us")}
+        log("  front end scanl                %9.3f us/call on the device, %d kernel(s); the hand-written fragment one by one: %s" % (us, nk, fe["scanl"]["direct_one_by_one_us"]))
         del xs, r, got, xsc
         vals, cols, offs, lens, xv = wl.smvm_inputs()
         vs, cs = [acc.use(vals.copy(), fcx) for _ in range(S)], [acc.use(cols.copy(), fcx) for _ in range(S)]
@@ -438,8 +454,9 @@ def main():
             return acc.foldSeg(add, 0.0, acc.zipWith(lambda c, a: a * v[c], cs[i], vs[i]), ls[i], context=fcx)
         r, us, nk = front(smvm_prog, S)
         fe["smvm"] = {"gpu_us_per_call": us, "kernels_per_call": nk, "direct_avg_launch_us": sk.get("smvm", {}).get("avg_launch_us"),
+                      "direct_one_by_one_us": sk.get("smvm", {}).get("one_by_one_us"),
                       "note": "per call: scanl of the 2^20 segment lengths into offsets, then foldSeg (the direct figure is foldSeg alone)"}
-        log("  front end smvm                 %9.3f us/call on the device, %d kernel(s): offsets scan + foldSeg" % (us, nk))
+        log("  front end smvm                 %9.3f us/call on the device, %d kernel(s): offsets scan + foldSeg; the hand-written foldSeg one by one: %s" % (us, nk, fe["smvm"]["direct_one_by_one_us"]))
         del vs, cs, vecs, ls, r
         sk["front_end"] = fe
         acc.destroy(fcx)
