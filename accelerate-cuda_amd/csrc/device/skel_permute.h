@@ -317,6 +317,13 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
 #if ACC_PERMUTE_NARROW
         , unsigned int *acc_status
 #endif
+#if !ACC_PERMUTE_NARROW && !ACC_PERMUTE_WINDOWS
+        /* first_fill != NULL (only where every target has its bin in LDS and the bins leave by atomics): the
+         * result starts as a copy of first_fill, made by workgroup 0 while the others read the source; `ready`
+         * (a word that holds {epoch, 1} once the copy can be seen from every die) is what they look at before
+         * their atomics.  One launch instead of two. */
+        , const ACC_ELT *__restrict__ first_fill, unsigned long long *ready, const unsigned int epoch, unsigned int *acc_status
+#endif
         ACC_GUARD_PARAM)
 {
   ACC_GUARD_CHECK
@@ -324,6 +331,21 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
   ACC_ENV_ASSUME
   extern __shared__ __attribute__((aligned(16))) unsigned char acc_lds_raw[];
   T *bins = (T *)acc_lds_raw;
+#if !ACC_PERMUTE_NARROW && !ACC_PERMUTE_WINDOWS
+  if (first_fill && blockIdx.x == 0) {
+    /* Stores of device scope, which go through this die's L2 to memory, where the others' atomics are performed.
+     * Every wave waits until its own have been acknowledged, the barrier until every wave has, and the word
+     * follows them.  (A fence here, and an acquiring read on the other side, write back and invalidate whole L2s:
+     * 9 us on a launch of 41; the barrier alone does not wait for stores to memory.) */
+    const Int64 count = (ACC_OUT_SIZE);
+    for (Int64 i = threadIdx.x; i < count; i += ACC_BLOCK)
+      __hip_atomic_store(arrOut_0 + i, first_fill[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0)
+      __hip_atomic_store(ready, ((unsigned long long)epoch << 32) | 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+#endif
 
   /* Target indices are handled as unsigned numbers of the width the
    * permutation produces (32 bits for Int32 keys): `ignore` (-1) and every
@@ -510,6 +532,21 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
   (void)row;
 #else
   if (lds_bins > 0) {
+#if !ACC_PERMUTE_WINDOWS
+    if (first_fill && blockIdx.x != 0) {
+      /* workgroup 0 made its copy tens of microseconds ago; the wait is bounded all the same, and one that runs
+       * out is reported (the atomics below would then add to whatever the result held before) */
+      if (threadIdx.x == 0) {
+        int polls = 0;
+        while ((__hip_atomic_load(ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32) != (unsigned long long)epoch &&
+               polls < ACC_SPIN_LIMIT) {
+          ++polls;
+          __builtin_amdgcn_s_sleep(4);
+        }
+        if (polls >= ACC_SPIN_LIMIT) acc_report(acc_status, ACC_STATUS_PERMUTE_LOCK);
+      }
+    }
+#endif
     __syncthreads();
     for (int i = threadIdx.x; i < lds_bins; i += ACC_BLOCK) {
       T acc = bins[i];

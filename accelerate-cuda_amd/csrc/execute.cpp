@@ -922,6 +922,16 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
     if (far_rows) far = base;
     if (table) dump = base + far_bytes;
   }
+  // Where every target has its bin in LDS and the bins leave by atomics, the result's first contents -- the defaults --
+  // are copied by workgroup 0 of the main kernel while the others read the source, and a word in scratch memory
+  // ({epoch, 1}, as the fold's partial results are tagged) tells them when their atomics may follow: one launch.
+  const bool inline_fill = copy_defaults && !far_rows && !table && bins == ntarget && bins > 0 && n_src > 0 &&
+                           acc::tune("permute.inline_fill", 1) != 0;
+  acc::ScratchRef rblk;
+  if (inline_fill) {
+    const int arc = s->ctx->scratch_acquire(256, st, acc::SCRATCH_FLAGS, &rblk);
+    if (arc != ACC_OK) { s->ctx->scratch_release(blk, st); return arc; }
+  }
   int rc = ACC_OK;
   if (far_rows) {                       // one launch: identity into the XCD rows, defaults into the result
     Args f;
@@ -933,7 +943,7 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
     const int64_t fill_grid = std::min<int64_t>((XCD_ROWS * ntarget + 255) / 256, 8 * (int64_t)cus);
     e = launch_kernel(s->variants[v].fn_fill, static_cast<unsigned>(fill_grid), 1, 1, 256, 1, 1, 0, st, f.data(), nullptr);
     if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(permute_fill)");
-  } else if (copy_defaults) {           // the defaults by the same kernel: a runtime copy of 1 KB takes 4 us, this launch 2
+  } else if (copy_defaults && !inline_fill) {   // the defaults by the same kernel: a runtime copy of 1 KB takes 4 us, this launch 2
     Args f;
     f.ptr(0);
     f.i64(0);
@@ -948,7 +958,12 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
   args.i32(static_cast<int32_t>(copies));
   args.ptr(dump);
   args.ptr(far);
+  args.ptr(inline_fill ? defaults->ptr[0] : 0);
+  args.ptr(reinterpret_cast<uint64_t>(rblk.ptr));
+  args.u32(rblk.epoch);
+  args.ptr(s->ctx->status_dev);
   if (rc == ACC_OK) rc = launch(s, v, grid, lds, st, &args);
+  if (inline_fill) s->ctx->scratch_release(rblk, st);
   if (rc == ACC_OK && (table || far_rows)) {
     // the tables are folded into the result by one launch: the per-block window rows, the per-XCD rows
     struct MergeJob { uint64_t dump; int64_t stride, first, cols; int32_t nrows, slices, window_log; };

@@ -315,7 +315,7 @@ def main():
         got = out.get()
         assert os.environ.get("ACC_BENCH_NOCHECK") or (int(got.sum()) == n and np.array_equal(got, np.bincount(keys, minlength=bins))), "histogram mismatch"
         sk[name] = result("permute (+) %d bins" % bins, w, e, 1, n * 4 + 2 * bins * 4, n,
-                          {"Gkeys_per_s": round(n / (e * 1e-3) / 1e9, 2), "note": "step = every launch the call makes: defaults copy + main kernel (256 bins); main kernel + merge (65 536 bins)",
+                          {"Gkeys_per_s": round(n / (e * 1e-3) / 1e9, 2), "note": "step = every launch the call makes: one kernel (256 bins: its first workgroup copies the defaults); main kernel + merge (65 536 bins)",
                            "traffic_key": name})
         sk[name]["end_to_end"] = end_to_end(ctx, [(dks[0], keys)], step(0), out)
         if not args.no_cpu:

@@ -339,6 +339,43 @@ def test_permute_other_combines(A, ctx, orc):
     assert np.array_equal(out.get(), orc.permute(orc.OP_FIRST, np.full(5000, -1, np.int32), perm, vals))
 
 
+def test_permute_whose_first_workgroup_copies_the_defaults(A, ctx):
+    """few enough targets for one LDS table and few enough workgroups for atomics: one launch, workgroup 0 copies
+    the defaults into the result while the others read the source, and they look at a word it leaves before they
+    add their bins.  Defaults that are not the identity, several numbers of targets, Int32 / Int64 / Float32 sums
+    and a maximum, launches that follow one another on one result (the word is tagged anew every time), a result
+    that is its own defaults (no copy), and the same with the copy as a launch of its own."""
+    import os
+    rng_ = np.random.default_rng(77)
+    for ctype, dt in (("Int32", np.int32), ("Int64", np.int64), ("float", np.float32)):
+        for combine, hint, at in (("x + y", A.COMBINE_ADD, np.add.at), ("acc_max(x, y)", A.COMBINE_MAX, np.maximum.at)):
+            for tune in ("", "permute.inline_fill=0"):
+                if tune:
+                    os.environ["ACC_HIP_TUNE"] = tune
+                try:
+                    sk = ctx.skeleton(A.SKEL_PERMUTE, ctype, env=[I32, (1, ctype)], out_rank=1, get="arrIn1_0[ix]", combine=combine,
+                                      permutation="arrIn0_0[ix]", combine_hint=hint)
+                    for bins, n in ((1, 5000), (7, 1), (256, 1 << 22), (4097, 1 << 20), (40960, (1 << 21) + 3)):
+                        say("permute, defaults copied inside the launch", ctype, combine, tune, "bins", bins, "n", n)
+                        keys = rng_.integers(-2, bins + 2, n).astype(np.int32)
+                        src = rng_.integers(0, 9, n).astype(dt)
+                        dfl = rng_.integers(1, 5, bins).astype(dt)
+                        ok = (keys >= 0) & (keys < bins)
+                        ref = dfl.astype(np.int64)
+                        at(ref, keys[ok], src[ok].astype(np.int64))
+                        out = ctx.array(np.full(bins, 99, dt))
+                        dk, ds_, dd = ctx.array(keys), ctx.array(src), ctx.array(dfl)
+                        for _ in range(3):                             # the same result three times over
+                            sk.permute([dk, ds_], n, dd, out)
+                            assert np.array_equal(out.get(), ref.astype(dt))
+                        acc = ctx.array(dfl)                           # the result is its own defaults: it accumulates
+                        sk.permute([dk, ds_], n, acc, acc)
+                        assert np.array_equal(acc.get(), ref.astype(dt))
+                    sk.destroy()
+                finally:
+                    os.environ.pop("ACC_HIP_TUNE", None)
+
+
 def test_permute_hinted_combines_over_windows_of_targets(A, ctx):
     """more targets than one LDS table holds: 2, 4 and 16 windows, every hinted operator, Int32 and Int64 elements,
     strays and `ignore` among the targets, a last window that is not full"""
