@@ -1,0 +1,157 @@
+"""Scans, permutes and segmented and innermost folds on element types, sizes and key distributions drawn at random
+(fixed seed: the same cases every run), against numpy.  Sources hold small integers, so every sum is exact in every
+element type; results are compared bit for bit, and every result array carries two guard words past its end."""
+import sys
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+TYPES = [("Int8", np.int8), ("Word16", np.uint16), ("Int32", np.int32), ("Int64", np.int64), ("float", np.float32),
+         ("double", np.float64)]
+
+
+def say(*a):
+    print("[case]", *a)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def A():
+    import acchip
+    return acchip
+
+
+@pytest.fixture(scope="module")
+def ctx(A):
+    c = A.Context(0)
+    yield c
+    c.close()
+
+
+class View(object):
+    """a result that is the first part of a longer array"""
+    def __init__(self, d):
+        self.d = d
+
+    def desc(self):
+        return self.d
+
+
+def near(rng, mult, hi):
+    return max(1, int(rng.integers(0, hi // mult + 1)) * mult + int(rng.choice([-3, -1, 0, 0, 1, 2, 5, 17, 100])))
+
+
+def test_random_scans(A, ctx):
+    rng = np.random.default_rng(2001)
+    kinds = ["scanl", "scanl1", "scanl'", "scanr", "scanr1", "scanr'"]
+    for trial in range(18):
+        kind = kinds[trial % 6]
+        ctype, T = TYPES[int(rng.integers(0, len(TYPES)))]
+        sk = ctx.skeleton(A.SCAN_KINDS[kind], ctype, env=[(1, ctype)], get="arrIn0_0[ix]", combine="(%s)(x + y)" % ctype,
+                          seed=None if kind.endswith("1") else "(%s)3" % ctype)
+        for _ in range(3):
+            n = near(rng, 32768, 1 << 21) if rng.random() < 0.6 else int(rng.integers(1, 5000))
+            say("scan", kind, ctype, "n", n)
+            x = rng.integers(0, 3, n).astype(T)
+            plus = 1 if kind in ("scanl", "scanr") else 0
+            out = ctx.array(np.full(n + plus + 2, 77, T))
+            tot = ctx.array(np.array(0, T))
+            sk.scan([ctx.array(x)], n, out.desc(shape=(n + plus,)), tot if kind.endswith("'") else None)
+            c = np.cumsum((x if kind.startswith("scanl") else x[::-1]).astype(np.int64))
+            if plus:
+                ref = np.concatenate([[3], 3 + c])
+            elif kind.endswith("1"):
+                ref = c
+            else:
+                ref = np.concatenate([[3], 3 + c[:-1]])
+            if kind.startswith("scanr"):
+                ref = ref[::-1]
+            got = out.get()
+            assert np.array_equal(got[:n + plus], ref.astype(T)) and np.all(got[n + plus:] == 77)
+            if kind.endswith("'"):
+                assert tot.get().reshape(-1)[0] == T(3 + c[-1])
+        sk.destroy()
+
+
+def test_random_permutes(A, ctx):
+    rng = np.random.default_rng(2002)
+    for trial in range(12):
+        ctype, T = [("Int32", np.int32), ("Int64", np.int64), ("float", np.float32), ("Word32", np.uint32)][trial % 4]
+        how = ["count", "weights", "max"][trial % 3]
+        if how == "count":
+            sk = ctx.skeleton(A.SKEL_PERMUTE, ctype, env=[(1, "Int32")], out_rank=1, get="(%s)1" % ctype, combine="x + y",
+                              permutation="arrIn0_0[ix]", combine_hint=A.COMBINE_ADD)
+        elif how == "weights":
+            sk = ctx.skeleton(A.SKEL_PERMUTE, ctype, env=[(1, "Int32"), (1, ctype)], out_rank=1, get="arrIn1_0[ix]", combine="x + y",
+                              permutation="arrIn0_0[ix]", combine_hint=A.COMBINE_ADD)
+        else:
+            sk = ctx.skeleton(A.SKEL_PERMUTE, ctype, env=[(1, "Int32"), (1, ctype)], out_rank=1, get="arrIn1_0[ix]",
+                              combine="acc_max(x, y)", permutation="arrIn0_0[ix]")
+        for _ in range(3):
+            bins = int(rng.choice([1, 7, 256, 1000, 4097, 40960, 40961, 50001, 65536, 81920, 81921, 150000])) + int(rng.integers(0, 3))
+            n = int(rng.choice([0, 1, 1000, 1 << 16, (1 << 20) + 3, 1 << 22]))
+            skew = rng.random() < 0.5
+            say("permute", how, ctype, "targets", bins, "n", n, "zipf keys" if skew else "uniform keys")
+            keys = (np.minimum(rng.zipf(1.2, n) - 1, bins - 1) if skew else rng.integers(0, bins, n)).astype(np.int32)
+            if n:
+                keys[::11] = rng.integers(-3, bins + 3, keys[::11].size)
+            src = rng.integers(0, 5, n).astype(T)
+            dfl = rng.integers(0, 50, bins).astype(T)
+            out = ctx.array(np.full(bins + 2, 99, T))
+            env = [ctx.array(keys)] if how == "count" else [ctx.array(keys), ctx.array(src)]
+            sk.permute(env, n, ctx.array(dfl), View(out.desc(shape=(bins,))))
+            ok = (keys >= 0) & (keys < bins)
+            ref = dfl.astype(np.int64)
+            if how == "count":
+                np.add.at(ref, keys[ok], 1)
+            elif how == "weights":
+                np.add.at(ref, keys[ok], src[ok].astype(np.int64))
+            else:
+                np.maximum.at(ref, keys[ok], src[ok].astype(np.int64))
+            got = out.get()
+            assert np.array_equal(got[:bins], ref.astype(T)) and np.all(got[bins:] == 99)
+        sk.destroy()
+
+
+def test_random_segmented_and_innermost_folds(A, ctx):
+    rng = np.random.default_rng(2003)
+    for trial in range(8):
+        ctype, T = TYPES[int(rng.integers(0, len(TYPES)))]
+        seg = ctx.skeleton(A.SKEL_FOLDSEG, ctype, env=[(1, ctype)], get="arrIn0_0[ix]", combine="(%s)(x + y)" % ctype, seed="(%s)1" % ctype)
+        rows_ = ctx.skeleton(A.SKEL_FOLD, ctype, env=[(2, ctype)], out_rank=1, get="arrIn0_0[ix]", combine="(%s)(x + y)" % ctype,
+                             seed="(%s)1" % ctype)
+        for _ in range(3):
+            nseg = int(rng.choice([1, 2, 255, 256, 257, 5000, 70001]))
+            dist = str(rng.choice(["short", "mixed", "long", "mostly empty"]))
+            if dist == "short":
+                lens = rng.integers(0, 8, nseg)
+            elif dist == "mixed":
+                lens = rng.poisson(rng.choice([1, 4, 32, 100]), nseg)
+            elif dist == "long":
+                lens = rng.integers(0, max(2, (1 << 21) // nseg), nseg)
+            else:
+                lens = np.where(rng.random(nseg) < 0.8, 0, rng.integers(0, 3000, nseg))
+            offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+            n = int(offs[-1])
+            say("foldSeg", ctype, nseg, "segments,", dist, "n", n)
+            x = rng.integers(0, 3, n).astype(T)
+            out = ctx.array(np.full(nseg + 2, 55, T))
+            seg.foldseg([ctx.array(x)], n, ctx.array(offs), View(out.desc(shape=(nseg,))))
+            c = np.concatenate([[0], np.cumsum(x.astype(np.int64))])
+            got = out.get()
+            assert np.array_equal(got[:nseg], (1 + c[offs[1:]] - c[offs[:-1]]).astype(T)) and np.all(got[nseg:] == 55)
+        for _ in range(4):
+            rows = int(rng.choice([1, 3, 255, 4096, 4097, 70001]))
+            inner = int(rng.choice([1, 2, 3, 4, 5, 7, 8, 16, 31, 64, 191, 193, 1000, 16384, 100000]))
+            while rows * inner > (1 << 23):
+                rows = max(1, rows // 2)
+            say("fold along rows", ctype, rows, "x", inner)
+            x = rng.integers(0, 3, (rows, inner)).astype(T)
+            out = ctx.array(np.full(rows + 2, 55, T))
+            rows_.fold([ctx.array(x)], (rows, inner), out.desc(shape=(rows,)))
+            got = out.get()
+            assert np.array_equal(got[:rows], (1 + x.astype(np.int64).sum(axis=1)).astype(T)) and np.all(got[rows:] == 55)
+        seg.destroy()
+        rows_.destroy()
