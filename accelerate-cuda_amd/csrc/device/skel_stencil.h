@@ -387,6 +387,11 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS ACC_GUARD_PARA
 #pragma unroll
   for (int rho = 0; rho < ACC_RING - 1; ++rho)
     if (rho < total) ACC_BOTH(fetch(rho, rho));
+#if ACC_SCHED_BARRIER
+  /* nothing that uses a row moves up between the requests for the rows: left to itself the compiler asks for two
+   * rows, waits for the first to shift its elements between lanes, and only then asks for the others */
+  __builtin_amdgcn_sched_barrier(0);
+#endif
 #pragma unroll
   for (int rho = 0; rho < ACC_NR - 1; ++rho) ACC_BOTH(finish(rho, rho));
 
@@ -399,6 +404,9 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS ACC_GUARD_PARA
          * slot freed by the previous step takes the row PREFETCH further on */
         const int rho_new = y + ACC_NR - 1 + ACC_PREFETCH;
         if (rho_new < total) ACC_BOTH(fetch(rho_new, (s + ACC_RING - 1) % ACC_RING));
+#if ACC_SCHED_BARRIER & 2
+        __builtin_amdgcn_sched_barrier(0);                 /* the requests of this step before anything of the step's results */
+#endif
         ACC_BOTH(finish(y + ACC_NR - 1, (s + ACC_NR - 1) % ACC_RING));
 
 #pragma unroll
