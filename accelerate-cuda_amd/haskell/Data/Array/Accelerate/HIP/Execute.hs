@@ -239,7 +239,7 @@ executeOpenAcc (ExecAcc kernel pacc) aenv stream =
     iterateM k s step = do { s' <- step s; (s :) <$> iterateM (k - 1) s' step }
 
 
--- Supplied by Data.Array.Accelerate.HIP.Array (the memory table brackets, INTEGRATION.md "Memory table") and by the
+-- Supplied by Data.Array.Accelerate.HIP.Array (brackets around the memory table of the header, acc_memtable_*) and by the
 -- host-side expression evaluator the reference already has (Execute.hs:454-560); named here so that the traversal
 -- above reads as a whole.
 aprjInt       :: Int -> Aval aenv -> SomeArrays
