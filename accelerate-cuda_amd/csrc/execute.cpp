@@ -297,8 +297,16 @@ int launch_segmented(acc_skel_s *s, int v, Args *args, const acc_array *env, con
 {
   const int64_t avg = n / nseg;
   if (avg < acc::tune("foldseg.wave_team_len", 192)) {
-    const int64_t grid = acc_launch_grid(nseg, s->spec.block, resident(s, v), acc::tune("foldseg.oversub", 1 << 20));
-    return launch(s, v, grid, 0, st, args);
+    // Segments of 8 elements or more on average stage half as much again at a time (variants 2 and 3 of the
+    // instance, built when first wanted): 2^25 elements in segments of 8 / 32 / 100 on average 36 / 31 / 51 us
+    // -> 32 / 27 / 40; shorter segments lose by it (rows of 4: 46 -> 49 us), and so keep the shorter chunk.
+    int lv = v;
+    if (avg >= acc::tune("foldseg.long_from", 8) && s->spec.chunk_long > s->spec.chunk) {
+      lv = v + 2;
+      ACC_TRY(s->ensure_variant(lv));
+    }
+    const int64_t grid = acc_launch_grid(nseg, s->spec.block, resident(s, lv), acc::tune("foldseg.oversub", 1 << 20));
+    return launch(s, lv, grid, 0, st, args);
   }
   const int block_team = avg >= acc::tune("foldseg.block_team_len", 16384) ? 1 : 0;
   const int64_t cus = s->ctx->props.multiProcessorCount;

@@ -423,10 +423,10 @@ static bool small_literal(std::string t)
 
 // elements a workgroup of the segmented fold stages at a time: a whole number of its block-wide vector loads (a lane
 // loads 16 bytes, so 16 elements of one byte: one load of 256 lanes is then 4096 of them)
-static int segmented_chunk(const SkelSpec &sp)
+static int segmented_chunk(const SkelSpec &sp, bool long_segments = false)
 {
   const int per_load = sp.block * std::max(1, 16 / std::max(1, sp.vec_size));
-  const int want = std::max(tune("foldseg.chunk", 2048), per_load);
+  const int want = std::max(long_segments ? tune("foldseg.chunk_long", 3072) : tune("foldseg.chunk", 2048), per_load);
   return (want + per_load - 1) / per_load * per_load;
 }
 
@@ -529,11 +529,13 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
       if (sp->out_rank > 0) {
         sp->block = tune("foldseg.block", 256);
         sp->chunk = segmented_chunk(*sp);
+        sp->chunk_long = segmented_chunk(*sp, true);
       }
       break;
     case ACC_SKEL_FOLDSEG: case ACC_SKEL_FOLD1SEG:
       sp->block = tune("foldseg.block", 256);
       sp->chunk = segmented_chunk(*sp);
+      sp->chunk_long = segmented_chunk(*sp, true);
       break;
     case ACC_SKEL_PERMUTE:
       if (sp->permutation.empty()) return fail(ACC_ERR_INVALID, "permute: `permutation` fragment missing");
@@ -673,9 +675,13 @@ namespace acc {
 SkelSpec spec_of_variant(const SkelSpec &base, int v)
 {
   SkelSpec spec = base;
-  if (v >= 2 && v < 4) spec.permute_locked = true;
-  if (v >= 4 && v < 6) spec.permute_windows = true;
-  if (v >= 6) spec.permute_narrow = true;
+  if (spec.kind == ACC_SKEL_PERMUTE) {
+    if (v >= 2 && v < 4) spec.permute_locked = true;
+    if (v >= 4 && v < 6) spec.permute_windows = true;
+    if (v >= 6) spec.permute_narrow = true;
+  }
+  // a segmented fold's variants 2 and 3: a longer staged chunk, for segments of 8 elements or more on average
+  if (spec.kind != ACC_SKEL_PERMUTE && v >= 2 && spec.chunk_long > 0) spec.chunk = spec.chunk_long;
   return spec;
 }
 }  // namespace acc
