@@ -595,49 +595,59 @@ struct acc_merge_job {
 /* result = base + carries + the sum of the workgroups' rows of packed 8-bit counts.  A row has nd = ceil(nwords / 2)
  * words; byte q of word `column` is the low byte of the count of target  column + (q & 2 ? nd : 0) + (q & 1 ? nwords : 0)
  * (the main kernel's table holds targets w and w + nwords in word w, and sends words w and w + nd out as one).  A
- * workgroup takes 64 consecutive words, each of its four waves a quarter of the rows, eight loads in flight a lane,
- * whose bytes are added two to a register (8 x 255 fits 16 bits) before they are widened; the waves' sums meet in
+ * workgroup takes 64 consecutive words, each of its ACC_MERGE_WAVES waves its share of the rows, sixteen loads in flight a lane,
+ * whose bytes are added two to a register (16 x 255 fits 16 bits) before they are widened; the waves' sums meet in
  * LDS and wave q writes the targets of byte q -- one thread per target, so no atomics and nothing that must be in
  * the result beforehand -- and clears the carries it has taken (the table is all zero between launches).  `base` is
  * the defaults array, or the result itself where that was filled from the defaults before the main kernel (which
  * then also added to it directly).                                                                          */
-extern "C" __global__ void __launch_bounds__(256)
+#ifndef ACC_MERGE_WAVES
+#define ACC_MERGE_WAVES 4
+#endif
+static_assert(ACC_MERGE_WAVES >= 4 && ACC_MERGE_WAVES <= 16, "a wave for each byte of a row's word");
+extern "C" __global__ void __launch_bounds__(64 * ACC_MERGE_WAVES)
 permute_merge(ACC_ENV_PARAMS ACC_OUT_PARAMS, const unsigned *__restrict__ dump, const Int64 nwords, const int nrows,
               const Int64 ntarget, ACC_ELT *carry, const ACC_ELT *base ACC_GUARD_PARAM)
 {
   ACC_GUARD_CHECK
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
-  __shared__ unsigned s_sum[4][4][64];           /* [wave][byte][lane] */
+  __shared__ unsigned s_sum[ACC_MERGE_WAVES][4][64];   /* [wave][byte][lane] */
   auto f = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
-  const int lane = threadIdx.x & 63, quarter = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  constexpr int waves = ACC_MERGE_WAVES;
   const Int64 nd = (nwords + 1) / 2;
   const Int64 column = (Int64)blockIdx.x * 64 + lane;
   const Int64 col_c = acc_min<Int64>(column, nd - 1);           /* lanes past the end read the last word and drop it */
   unsigned c0 = 0u, c1 = 0u, c2 = 0u, c3 = 0u;
-  int r = quarter;
-  for (; r + 28 < nrows; r += 32) {
-    unsigned w[8];
+  int r = wave;
+#ifndef ACC_MERGE_BATCH
+#define ACC_MERGE_BATCH 16                     /* loads in flight a lane (x 255 fits 16 bits up to 257) */
+#endif
+  for (; r + waves * (ACC_MERGE_BATCH - 1) < nrows; r += waves * ACC_MERGE_BATCH) {
+    unsigned w[ACC_MERGE_BATCH];
 #pragma unroll
-    for (int k = 0; k < 8; ++k) w[k] = __builtin_nontemporal_load(dump + (Int64)(r + 4 * k) * nd + col_c);
+    for (int k = 0; k < ACC_MERGE_BATCH; ++k) w[k] = __builtin_nontemporal_load(dump + (Int64)(r + waves * k) * nd + col_c);
     unsigned even = 0u, odd = 0u;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) { even += w[k] & 0x00FF00FFu; odd += (w[k] >> 8) & 0x00FF00FFu; }
+    for (int k = 0; k < ACC_MERGE_BATCH; ++k) { even += w[k] & 0x00FF00FFu; odd += (w[k] >> 8) & 0x00FF00FFu; }
     c0 += even & 0xFFFFu; c2 += even >> 16;
     c1 += odd & 0xFFFFu;  c3 += odd >> 16;
   }
-  for (; r < nrows; r += 4) {
+  for (; r < nrows; r += waves) {
     const unsigned w = __builtin_nontemporal_load(dump + (Int64)r * nd + col_c);
     c0 += w & 0xFFu; c1 += (w >> 8) & 0xFFu; c2 += (w >> 16) & 0xFFu; c3 += w >> 24;
   }
-  s_sum[quarter][0][lane] = c0;
-  s_sum[quarter][1][lane] = c1;
-  s_sum[quarter][2][lane] = c2;
-  s_sum[quarter][3][lane] = c3;
+  s_sum[wave][0][lane] = c0;
+  s_sum[wave][1][lane] = c1;
+  s_sum[wave][2][lane] = c2;
+  s_sum[wave][3][lane] = c3;
   __syncthreads();
-  const unsigned total = s_sum[0][quarter][lane] + s_sum[1][quarter][lane] + s_sum[2][quarter][lane] + s_sum[3][quarter][lane];
-  const Int64 word = column + ((quarter & 2) ? nd : 0);          /* the word of the main kernel's table the count sat in */
-  const Int64 t = word + ((quarter & 1) ? nwords : 0);
+  if (wave >= 4) return;                                         /* wave q writes the targets of byte q */
+  unsigned total = 0u;
+  for (int w = 0; w < waves; ++w) total += s_sum[w][wave][lane];
+  const Int64 word = column + ((wave & 2) ? nd : 0);             /* the word of the main kernel's table the count sat in */
+  const Int64 t = word + ((wave & 1) ? nwords : 0);
   if (column < nd && word < nwords && t < ntarget) {
     const T c = carry[t];
     if (c != T(0)) carry[t] = T(0);

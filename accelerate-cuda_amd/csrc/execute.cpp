@@ -819,8 +819,9 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
       m.ptr(ncarry);
       m.ptr(direct_adds ? out->ptr[0] : defaults->ptr[0]);
       if (nrc == ACC_OK) {
-        // a workgroup per 64 words of a row, its four waves a quarter of the rows each
-        hipError_t me = launch_kernel(s->variants[nv].fn_finish, static_cast<unsigned>((nd + 63) / 64), 1, 1, 256, 1, 1, 0, st,
+        // a workgroup per 64 words of a row, each of its waves its share of the rows
+        const unsigned merge_threads = 64u * static_cast<unsigned>(s->spec.merge_waves);
+        hipError_t me = launch_kernel(s->variants[nv].fn_finish, static_cast<unsigned>((nd + 63) / 64), 1, 1, merge_threads, 1, 1, 0, st,
                                       m.data(), nullptr);
         if (me != hipSuccess) nrc = acc::fail_hip(me, "hipModuleLaunchKernel(permute_merge, narrow counts)");
       }

@@ -286,6 +286,8 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "#define ACC_PERMUTE_WINDOWS " << (sp.permute_windows ? 1 : 0) << "\n";
       o << "#define ACC_PERMUTE_NARROW " << (sp.permute_narrow ? 1 : 0) << "\n";
       if (sp.permute_narrow) o << "#define ACC_NARROW_STOP " << tune("permute.narrow_stop", 0xA000) << "u\n";
+      if (sp.permute_narrow && tuned("permute.merge_batch")) o << "#define ACC_MERGE_BATCH " << tune("permute.merge_batch", 16) << "\n";
+      if (sp.permute_narrow) o << "#define ACC_MERGE_WAVES " << sp.merge_waves << "\n";
       o << "#define ACC_ELT_IS_INTEGER " << (is_integer_type(sp.elt_type) ? 1 : 0) << "\n";
       o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_UNROLL " << sp.unroll << "\n";
       tmpl = "skel_permute.h";
@@ -550,6 +552,7 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
       if (sp->combine_hint >= ACC_COMBINE_AND && !is_integer_type(sp->elt_type))
         return fail(ACC_ERR_INVALID, "permute: bitwise combine_hint on non-integer element type '%s'", sp->elt_type.c_str());
       sp->block = tune("permute.block", 1024);
+      sp->merge_waves = std::max(4, std::min(16, tune("permute.merge_waves", 4)));
       sp->unroll = tune("permute.unroll", 2);
       break;
     case ACC_SKEL_STENCIL:

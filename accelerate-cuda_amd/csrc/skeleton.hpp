@@ -42,6 +42,7 @@ struct SkelSpec {
   int zmarch = 0;                       // rank-3 stencils: strips tile_z rows tall walk through tile_h planes
   // tuning
   int block = 256, unroll = 4, rows = 4, chunk = 4096;
+  int merge_waves = 4;                  // permute of 16-bit counts: waves of a workgroup of permute_merge
   int chunk_long = 0;                   // segmented folds: the staged chunk of variants 2 and 3 (segments of 8 elements or more on average); 0: none
   bool guarded = false;                 // ACC_FLAG_GUARDED: every kernel takes the address of a loop's guard word last
   bool fold_single = true;              // foldAll in one launch (the last workgroup collects), as generated into the kernel
