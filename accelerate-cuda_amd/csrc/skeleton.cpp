@@ -235,7 +235,7 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
         // along the innermost dimension: the segmented fold over rows of one length
         *entry = sp.has_seed ? "fold" : "fold1";
         o << "#define ACC_SEG_UNIFORM 1\n";
-        o << "#define ACC_TROUNDS " << tune("foldseg.team_rounds", 4) << "\n";
+        o << "#define ACC_TROUNDS " << tune("foldseg.team_rounds", 3) << "\n";
       if (tuned("foldseg.pad")) o << "#define ACC_PAD_ON " << (tune("foldseg.pad", 1) ? 1 : 0) << "\n";
         if (tuned("foldseg.pad")) o << "#define ACC_PAD_ON " << (tune("foldseg.pad", 1) ? 1 : 0) << "\n";
         o << "#define ACC_FOLD_RIGHT " << ((sp.flags & ACC_FLAG_FOLD_RIGHT) ? 1 : 0) << "\n";
@@ -253,7 +253,7 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       *entry = sp.has_seed ? "foldSeg" : "fold1Seg";
       o << "#define ACC_SEG_TYPE " << sp.seg_type << "\n";
       if (sp.out_rank >= 2) o << "#define ACC_SEG_OUTER 1\n";      // the segments of every outer row: Reduction.hs:473-474
-      o << "#define ACC_TROUNDS " << tune("foldseg.team_rounds", 4) << "\n";
+      o << "#define ACC_TROUNDS " << tune("foldseg.team_rounds", 3) << "\n";
       if (tuned("foldseg.pad")) o << "#define ACC_PAD_ON " << (tune("foldseg.pad", 1) ? 1 : 0) << "\n";
       o << "#define ACC_FOLD_RIGHT " << ((sp.flags & ACC_FLAG_FOLD_RIGHT) ? 1 : 0) << "\n";
       o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_CHUNK " << sp.chunk << "\n";
