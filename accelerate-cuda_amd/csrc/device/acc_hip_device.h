@@ -152,6 +152,18 @@ ACC_DEV T acc_wave_reduce(T x, F op)
   return op(op(r0, r1), op(r2, r3));
 }
 
+/* the same over each row of 16 lanes on its own, order preserving; the result is in the row's first lane */
+template <typename T, typename F>
+ACC_DEV T acc_row_reduce(T x, F op)
+{
+  T t;
+  t = acc_dpp<ACC_DPP_ROW_SHL(1), 0xf>(x, x); x = op(x, t);
+  t = acc_dpp<ACC_DPP_ROW_SHL(2), 0xf>(x, x); x = op(x, t);
+  t = acc_dpp<ACC_DPP_ROW_SHL(4), 0xf>(x, x); x = op(x, t);
+  t = acc_dpp<ACC_DPP_ROW_SHL(8), 0xf>(x, x); x = op(x, t);
+  return x;
+}
+
 /* ------------------------------------------------------------------------ */
 /* atomics on 4- and 8-byte elements of any type, by compare-and-swap on the
  * bit pattern (replaces cubits/accelerate_cuda_function.h:28-114)            */

@@ -310,9 +310,11 @@ ACC_FS_CAT_(ACC_FOLDSEG_ENTRY, _rows)(ACC_ENV_PARAMS
 
 /* ---- long segments: a team of lanes per segment ---------------------------
  * One lane per segment serialises a long segment on that lane, so when the
- * segments are long on average the host launches this entry instead: a whole
- * wave (block_team == 0) or a whole workgroup (block_team != 0) takes one
- * segment at a time.  The team walks the segment in rounds of ACC_TVEC
+ * segments are long on average the host launches this entry instead: a row
+ * of 16 lanes (block_team == 2: four segments a wave side by side, for
+ * segments of a few hundred elements, of which a whole wave would ask for
+ * more than they hold), a whole wave (block_team == 0) or a whole workgroup
+ * (block_team == 1) takes one segment at a time.  The team walks the segment in rounds of ACC_TVEC
  * consecutive elements per lane, each lane folds its own elements in order,
  * the lanes are combined in lane order (the wave reduction preserves order,
  * waves meet in LDS in wave order) and the round's value joins the running
@@ -354,10 +356,12 @@ ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _team)(ACC_ENV_PARAMS
   const Int64 n = ACC_SEG_TOTAL;
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
-  const int me = block_team ? tid : acc_lane();                    /* place in the team */
-  const Int64 team_lanes = block_team ? ACC_BLOCK : ACC_WAVE;
-  const Int64 team0 = block_team ? (Int64)blockIdx.x : (Int64)blockIdx.x * ACC_FS_WAVES + wave;
-  const Int64 nteams = block_team ? (Int64)gridDim.x : (Int64)gridDim.x * ACC_FS_WAVES;
+  const bool row_team = block_team == 2, whole_block = block_team == 1;
+  const int me = whole_block ? tid : (row_team ? (acc_lane() & 15) : acc_lane());      /* place in the team */
+  const Int64 team_lanes = whole_block ? ACC_BLOCK : (row_team ? 16 : ACC_WAVE);
+  const Int64 wave0 = (Int64)blockIdx.x * ACC_FS_WAVES + wave;
+  const Int64 team0 = whole_block ? (Int64)blockIdx.x : (row_team ? wave0 * 4 + (acc_lane() >> 4) : wave0);
+  const Int64 nteams = whole_block ? (Int64)gridDim.x : (Int64)gridDim.x * ACC_FS_WAVES * (row_team ? 4 : 1);
   const Int64 round = team_lanes * ACC_TVEC;
 #if ACC_HAS_SEED
   const T seed = (ACC_SEED);
@@ -392,9 +396,11 @@ ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _team)(ACC_ENV_PARAMS
     }
   };
   /* all lanes of the team, in order; uniform over the team (block teams: over the workgroup) */
+  /* (a row team's value is in the row's first lane only, which is the lane that uses it) */
   auto team = [&](acc_opt<T> m) -> acc_opt<T> {
+    if (row_team) return acc_row_reduce(m, lf);
     m = acc_wave_reduce(m, lf);
-    if (!block_team) return m;
+    if (!whole_block) return m;
     if (acc_lane() == 0) s_wave[wave] = m;
     __syncthreads();
     acc_opt<T> r = s_wave[0];

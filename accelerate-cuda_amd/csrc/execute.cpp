@@ -296,7 +296,7 @@ int launch_segmented(acc_skel_s *s, int v, Args *args, const acc_array *env, con
                      hipStream_t st)
 {
   const int64_t avg = n / nseg;
-  if (avg < acc::tune("foldseg.wave_team_len", 192)) {
+  if (avg < acc::tune("foldseg.wave_team_len", 128)) {
     // Segments of 8 elements or more on average stage half as much again at a time (variants 2 and 3 of the
     // instance, built when first wanted): 2^25 elements in segments of 8 / 32 / 100 on average 36 / 31 / 51 us
     // -> 32 / 27 / 40; shorter segments lose by it (rows of 4: 46 -> 49 us), and so keep the shorter chunk.
@@ -308,9 +308,10 @@ int launch_segmented(acc_skel_s *s, int v, Args *args, const acc_array *env, con
     const int64_t grid = acc_launch_grid(nseg, s->spec.block, resident(s, lv), acc::tune("foldseg.oversub", 1 << 20));
     return launch(s, lv, grid, 0, st, args);
   }
-  const int block_team = avg >= acc::tune("foldseg.block_team_len", 16384) ? 1 : 0;
+  // teams: a workgroup (1) from `foldseg.block_team_len`, a row of 16 lanes (2) below `foldseg.row_team_below`, else a wave (0)
+  const int block_team = avg >= acc::tune("foldseg.block_team_len", 16384) ? 1 : (avg < acc::tune("foldseg.row_team_below", 1024) ? 2 : 0);
   const int64_t cus = s->ctx->props.multiProcessorCount;
-  const int64_t team_lanes = block_team ? s->spec.block : 64;
+  const int64_t team_lanes = block_team == 1 ? s->spec.block : (block_team == 2 ? 16 : 64);
   const int64_t room = cus * (2048 / team_lanes);                    // teams the device holds at once
   const int64_t min_piece = team_lanes * 64;                          // a piece keeps its team busy for a while
   int64_t split = 1;
@@ -328,7 +329,7 @@ int launch_segmented(acc_skel_s *s, int v, Args *args, const acc_array *env, con
   args->i64(split);
   args->ptr(part);
   args->ptr(part_ok);
-  const int64_t per_block = block_team ? 1 : s->spec.block / 64;
+  const int64_t per_block = block_team == 1 ? 1 : s->spec.block / team_lanes;
   const int64_t tgrid = acc_launch_grid(nseg * split, per_block, cus, 2048 / s->spec.block);
   int rc = s->ctx->make_current();
   if (rc == ACC_OK) {

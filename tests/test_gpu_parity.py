@@ -563,7 +563,7 @@ def test_smvm(A, ctx, orc, right):
         # short segments (one lane each) are folded in index order with the sequential association: identical bits.
         # Segments long on average go to a wave or a workgroup each: still index order, another association, so the
         # last bits may differ.  (Stated tolerance for this configuration, checked below for both: 1e-4 relative per row.)
-        if vals.size // nrows < 192:
+        if vals.size // nrows < 128:
             assert np.array_equal(got, exp)
         y64, yabs = orc.smvm_f64(vals, cols, offs, x)
         assert np.all(np.abs(got - y64) <= 1e-4 * np.maximum(np.abs(y64), 1e-3 * yabs) + 1e-30)
