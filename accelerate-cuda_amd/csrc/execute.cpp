@@ -669,8 +669,12 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
   const bool lds_table_fits = lds_windows <= acc::tune("permute.lock_max_windows", 12) &&
                               n_src >= acc::tune("permute.lock_lds_min_ratio", 4) * ntarget;
   // (Floating-point addition has an LDS atomic, but it runs at a fifth of the integer one's rate -- 16 M updates on
-  // 1000 targets: 95 us against 66 us through the tables -- so it goes the same way.)
-  const bool fp_add = s->spec.combine_hint == ACC_COMBINE_ADD && (s->spec.elt_type == "float" || s->spec.elt_type == "double");
+  // 1000 targets: 95 us against 63 us through the tables -- so between 48 and 6144 targets it goes the same way.
+  // Below, the tables' locks are what lanes meet on (16 targets 149 us against 93, one target 2.1 ms against 0.12);
+  // above, a table holds half the targets an array of plain values does and the passes over the source multiply
+  // (16 384 targets 123 us against 102, 131 072: 407 against 107).)
+  const bool fp_add = s->spec.combine_hint == ACC_COMBINE_ADD && (s->spec.elt_type == "float" || s->spec.elt_type == "double") &&
+                      ntarget >= acc::tune("permute.fp_tables_from", 48) && ntarget <= acc::tune("permute.fp_tables_to", 6144);
   const bool generic_few = !s->spec.permute_locked && (s->spec.combine_hint == ACC_COMBINE_GENERIC || fp_add) && lds_table_fits &&
                            acc::tune("permute.generic_lds", 1) != 0;
   if (s->spec.permute_locked || generic_few) {
