@@ -766,13 +766,16 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
   args.i64(n_src);
 
   // Integer addition on more targets than one LDS table of whole elements holds, but no more than one of 16-bit
-  // counts does (65536 Int32 or Int64 targets in 128 KB): one pass over the source instead of one per window.
+  // counts does (65536 Int32 or Int64 targets in 128 KB): one pass over the source instead of one per window.  Also
+  // from `permute.narrow_from` targets that whole elements would still hold: a single copy of such a table is what
+  // all sixteen waves add to, and the smaller one does better (2^24 keys into 16 384 / 40 960 targets: 25.2 / 31.4
+  // -> 22.8 / 27.0 us).
   const bool int_add = s->spec.combine_hint == ACC_COMBINE_ADD &&
                        (s->spec.elt_type == "Int32" || s->spec.elt_type == "Word32" || s->spec.elt_type == "Int64" || s->spec.elt_type == "Word64");
   // Only where the source is spelt as a small constant -- the counting idiom, `permute (+) zeros bin ones` -- since any
   // other addend would go to the result one device-scope atomic at a time (`permute.narrow=2` takes every source).
   const int narrow = acc::tune("permute.narrow", 1);
-  if (int_add && ntarget * (int64_t)esz > lds_all && ((ntarget + 1) / 2) * 4 <= lds_all && n_src >= 4 * ntarget &&
+  if (int_add && ntarget > std::min<int64_t>(acc::tune("permute.narrow_from", 8192), lds_all / (int64_t)esz) && ((ntarget + 1) / 2) * 4 <= lds_all && n_src >= 4 * ntarget &&
       (narrow == 2 || (narrow == 1 && s->spec.get_small_constant))) {
     const int nv = (aligned ? 0 : 1) + 6;
     ACC_TRY(s->ensure_variant(nv));
