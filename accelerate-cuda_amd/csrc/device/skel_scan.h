@@ -215,30 +215,48 @@ ACC_DEV void acc_scan_load(Get get, const Int64 base, const Int64 n, T (&x)[ACC_
 #pragma unroll
       for (int k = 0; k < ACC_VEC; ++k) x[r][k] = get(ACC_SCAN_RIGHT ? i0 - k : i0 + k);
     }
+  } else if (n < ACC_VEC) {
+    /* fewer elements than a vector: every position reads the nearest element of the array */
+#pragma unroll
+    for (int r = 0; r < ACC_ROWS; ++r) {
+      const Int64 i0 = acc_scan_ix0(base, wave, lane, r);
+#pragma unroll
+      for (int k = 0; k < ACC_VEC; ++k) {
+        const Int64 ix = ACC_SCAN_RIGHT ? i0 - k : i0 + k;
+        x[r][k] = get(acc_max<Int64>(0, acc_min<Int64>(ix, n - 1)));
+      }
+    }
   } else {
-    /* a tile that reaches outside the array: vectors that lie inside are read as in a full tile (one 128-bit
-     * access), the one across the edge element by element, those outside as one element -- a tile read and written
-     * element by element takes three times as long as a full one, and it is the last one to finish */
+    /* A tile that reaches outside the array, read WITHOUT a branch per row (a branch around a load makes the
+     * compiler wait for that load on the spot, and 32 rows of such waits took 8 us): every row reads one whole
+     * vector -- its own where that lies inside the array, else the last whole vector of the array, whose values
+     * stand in positions that never reach a result -- and the one vector that lies across the end of the array
+     * (there is one if the length is no multiple of the vector) is read once, element by element, by every
+     * lane, and put in the place of the row that holds it. */
+    const Int64 nv = n / ACC_VEC * ACC_VEC;                 /* where the vector across the end begins, if nv < n */
+    T tail[ACC_VEC];
+#pragma unroll
+    for (int k = 0; k < ACC_VEC; ++k) tail[k] = get(acc_min<Int64>(nv + k, n - 1));
+    const Int64 spare = nv - ACC_VEC;                      /* a whole vector inside the array (n >= ACC_VEC) */
 #pragma unroll
     for (int r = 0; r < ACC_ROWS; ++r) {
       const Int64 i0 = acc_scan_ix0(base, wave, lane, r);
       const Int64 lo = ACC_SCAN_RIGHT ? i0 - (ACC_VEC - 1) : i0;
-      if (lo >= 0 && lo + ACC_VEC <= n) {
+      const bool whole = lo >= 0 && lo + ACC_VEC <= n;
+      const Int64 at = whole ? lo : spare;                 /* lowest physical index of the vector read */
+      const Int64 a0 = ACC_SCAN_RIGHT ? at + (ACC_VEC - 1) : at;
 #pragma unroll
-        for (int k = 0; k < ACC_VEC; ++k) x[r][k] = get(ACC_SCAN_RIGHT ? i0 - k : i0 + k);
-      } else if (lo >= n || lo + ACC_VEC <= 0) {
-        /* a vector wholly outside the array: the array's nearest element in every position (one address for all
-         * of them; the value never reaches a result) */
-        const T edge = get(lo >= n ? n - 1 : (Int64)0);
+      for (int k = 0; k < ACC_VEC; ++k) x[r][k] = get(ACC_SCAN_RIGHT ? a0 - k : a0 + k);
+    }
+    /* every load above is in flight before the first result is looked at */
+    __builtin_amdgcn_sched_barrier(0);
+    if (nv < n) {
 #pragma unroll
-        for (int k = 0; k < ACC_VEC; ++k) x[r][k] = edge;
-      } else {
+      for (int r = 0; r < ACC_ROWS; ++r) {
+        const Int64 i0 = acc_scan_ix0(base, wave, lane, r);
+        const bool across = (ACC_SCAN_RIGHT ? i0 - (ACC_VEC - 1) : i0) == nv;
 #pragma unroll
-        for (int k = 0; k < ACC_VEC; ++k) {
-          /* outside the array: its nearest element instead; the value never reaches a result */
-          const Int64 ix = ACC_SCAN_RIGHT ? i0 - k : i0 + k;
-          x[r][k] = get(acc_max<Int64>(0, acc_min<Int64>(ix, n - 1)));
-        }
+        for (int k = 0; k < ACC_VEC; ++k) x[r][k] = across ? tail[ACC_SCAN_RIGHT ? ACC_VEC - 1 - k : k] : x[r][k];
       }
     }
   }

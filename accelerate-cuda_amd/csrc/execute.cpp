@@ -186,7 +186,7 @@ int launch(acc_skel_s *s, int variant, int64_t grid, size_t dyn_lds, hipStream_t
   ACC_TRY(s->ensure_variant(variant));
   ACC_TRY(s->ctx->make_current());
   ACC_HIP_TRY(launch_kernel(s->variants[variant].fn, static_cast<unsigned>(grid), 1, 1,
-                                    static_cast<unsigned>(s->spec.block), 1, 1, static_cast<unsigned>(dyn_lds), stream,
+                                    static_cast<unsigned>(s->variants[variant].block), 1, 1, static_cast<unsigned>(dyn_lds), stream,
                                     args->data(), nullptr));
   return ACC_OK;
 }
@@ -551,16 +551,23 @@ int scan_core(acc_skel s, const acc_array *env, int64_t n, const acc_array *out,
   }
   args.i64(n);
 
-  const int v = aligned ? 0 : 1;
+  // An array of up to 12 MB takes the small-tile variant (4 rows a lane instead of 32): a workgroup runs through the
+  // instructions of all the rows of its tile whether the array fills them or not, and a small array spread over few
+  // large tiles leaves most of the device idle (Int32: 1024 elements 10.6 us -> 4.4, 2^18 8.6 -> 4.1, 2^21 10.0 ->
+  // 8.1, 3 M + 3 14.8 -> 9.3; at 2^22 the two are level, 11.7 and 11.2, and so are 2^21 Float64, 12.0 and 13.2).
+  const bool small = s->spec.scan_small_rows > 0 &&
+                     n * (int64_t)s->spec.elt_size <= (int64_t)acc::tune("scan.small_below_kb", 12288) * 1024;
+  int v = (aligned ? 0 : 1) + (small ? 2 : 0);
   if (noalloc) {
     // building a variant compiles and loads a module: not here
     if (!s->variant_ready(v))
-      return fail(ACC_ERR_INVALID, "%s: the %s variant of this instance is not loaded yet; run acc_exec_scan once on operands of the same alignment first",
-                  who, aligned ? "aligned" : "unaligned");
+      return fail(ACC_ERR_INVALID, "%s: the %s %s-tile variant of this instance is not loaded yet; run acc_exec_scan once on operands of the same alignment and of %s %d KB first",
+                  who, aligned ? "aligned" : "unaligned", small ? "small" : "large", small ? "at most" : "more than", acc::tune("scan.small_below_kb", 12288));
   } else {
     ACC_TRY(s->ensure_variant(v));
   }
-  const int64_t tile = s->elements_per_block();
+  const int block = s->variants[v].block;
+  const int64_t tile = (int64_t)block * s->variants[v].rows * s->vec();
   const int64_t tiles = (n + tile - 1) / tile;
   const int64_t grid = std::max<int64_t>(1, tiles);     // one workgroup per tile, in dispatch order
   const int64_t ndesc = std::max<int64_t>(1, tiles);
@@ -586,7 +593,7 @@ int scan_core(acc_skel s, const acc_array *env, int64_t n, const acc_array *out,
     args.i64(tiles);
     args.ptr(s->ctx->status_dev);
     if (grid < 1 || grid > 0x7fffffffLL) return fail(ACC_ERR_INVALID, "%s: grid of %lld blocks", who, (long long)grid);
-    ACC_HIP_TRY(launch_kernel(s->variants[v].fn, static_cast<unsigned>(grid), 1, 1, static_cast<unsigned>(s->spec.block), 1, 1,
+    ACC_HIP_TRY(launch_kernel(s->variants[v].fn, static_cast<unsigned>(grid), 1, 1, static_cast<unsigned>(block), 1, 1,
                                       0, st, args.data(), nullptr));
     return ACC_OK;
   }

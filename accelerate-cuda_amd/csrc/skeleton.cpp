@@ -649,6 +649,7 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
         sp->scan_rows_fallback = std::max(2, std::min({8, 131072 / (1024 * per_row), 32 / vec}));
         sp->block = tune("scan.block", sp->scan_shape_open ? 256 : 1024);
         sp->rows = tune("scan.rows", sp->scan_shape_open ? rows4 : sp->scan_rows_fallback);
+        sp->scan_small_rows = std::max(0, std::min(tune("scan.small_rows", 4), 32));
       }
       break;
   }
@@ -685,6 +686,12 @@ SkelSpec spec_of_variant(const SkelSpec &base, int v)
   }
   // a segmented fold's variants 2 and 3: a longer staged chunk, for segments of 8 elements or more on average
   if (spec.kind != ACC_SKEL_PERMUTE && v >= 2 && spec.chunk_long > 0) spec.chunk = spec.chunk_long;
+  // a scan's variants 2 and 3: a small tile, for arrays of a few tiles at most (a lone workgroup runs through the
+  // instructions of all its rows one after the other whether the array fills them or not)
+  if (spec.scan_small_rows > 0 && v >= 2) {
+    spec.block = std::min(spec.block, 256);
+    spec.rows = std::min(spec.rows, spec.scan_small_rows);
+  }
   return spec;
 }
 }  // namespace acc
@@ -746,7 +753,9 @@ int acc_skel_s::ensure_variant(int v)
     }
   }
   (void)hipFuncGetAttribute(&var.num_regs, HIP_FUNC_ATTRIBUTE_NUM_REGS, var.fn);
-  if (this->spec.scan_shape_open) {
+  var.block = spec.block;
+  var.rows = spec.rows;
+  if (this->spec.scan_shape_open && v < 2) {
     // the first build of a scan decides its tile shape: see make_spec
     this->spec.scan_shape_open = false;
     if (var.num_regs > 256) {

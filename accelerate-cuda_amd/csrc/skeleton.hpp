@@ -47,6 +47,7 @@ struct SkelSpec {
   bool guarded = false;                 // ACC_FLAG_GUARDED: every kernel takes the address of a loop's guard word last
   bool fold_single = true;              // foldAll in one launch (the last workgroup collects), as generated into the kernel
   int scan_rows_fallback = 8;
+  int scan_small_rows = 0;              // rows a lane of a scan's small-tile variants (2 and 3); 0: none
   int scan_desc_stride = 16;            // 8-byte words between the tile descriptors of a scan, as generated into the kernel
   bool scan_shape_open = false;         // a scan whose tile shape the first build may still change (by its register count)
 };
@@ -63,6 +64,8 @@ struct Variant {
   int num_regs = 0;
   int static_lds = 0;
   int blocks_per_cu = 1;
+  int block = 0;                       // workgroup size and rows a lane of this variant was built with (a scan's small
+  int rows = 0;                        // variant differs from the instance's)
 };
 
 int type_size(const std::string &t);

@@ -394,8 +394,10 @@ int acc_exec_scan(acc_skel s, const acc_array *env, int64_t n, const acc_array *
  * nothing, compiles nothing and loads nothing:
  *   - the input may span at most ACC_NOALLOC_MAX_TILES tiles of acc_skel_info.elements_per_block elements
  *     (32768 Int32 each: 2^28 elements); more is ACC_ERR_INVALID;
- *   - the variant for the operands' alignment must have been loaded already (the aligned one is by
- *     acc_skel_create, the unaligned one by a first acc_exec_scan on such operands), else ACC_ERR_INVALID;
+ *   - the variant that acc_exec_scan takes for such operands must have been loaded already, else ACC_ERR_INVALID.
+ *     There are four: for operands aligned to 16 bytes or not, and for arrays of at most 12 MB (scanned in tiles
+ *     an eighth the size) or more.  acc_skel_create loads the one for large aligned arrays, a first acc_exec_scan
+ *     on operands of the same alignment and on the same side of 12 MB each of the others;
  *   - every call on a device shares that device's array: calls that overlap in time on one device, from any
  *     stream, thread or context, race.  Calls ordered on one stream are fine.
  * Results are those of acc_exec_scan, bit for bit.                                                          */

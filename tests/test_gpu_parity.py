@@ -199,6 +199,42 @@ def test_scan_int32_add(A, ctx, orc, kind):
             assert np.array_equal(got[:n + plus], exp)
 
 
+@pytest.mark.parametrize("small_below_kb", ["0", "2000000"])
+def test_scan_tiles_of_either_size_on_ragged_ends(A, ctx, orc, monkeypatch, small_below_kb):
+    """the driver takes small tiles for arrays up to 12 MB and large ones above: here each kind of tile is forced on
+    sizes either side of that, with ends that fall anywhere in a vector, a row and a tile"""
+    monkeypatch.setenv("ACC_HIP_TUNE", "scan.small_below_kb=" + small_below_kb)
+    sizes = [1, 3, 4, 5, 255, 1027, 4096, 4097, 32767, 32768, 32769, 32771, 65537, 98307, 5 * 32768 + 2, (1 << 21) + 4101]
+    for kind in ("scanl", "scanl1", "scanr", "scanr1", "scanl'", "scanr'"):
+        seeded = not kind.endswith("1")
+        sk = ctx.skeleton(A.SCAN_KINDS[kind], "Int32", env=[I32], get="arrIn0_0[ix]", combine="x + y",
+                          seed="5" if seeded else None)
+        for n in sizes:
+            say(kind, "(+) Int32, scan.small_below_kb =", small_below_kb, "n =", n)
+            x = rng.integers(-9, 16, n, dtype=np.int32)
+            plus = 1 if kind in ("scanl", "scanr") else 0
+            out = ctx.array(np.full(n + plus + 2, -777, np.int32))
+            tot = ctx.array(np.array(-1, np.int32))
+            sk.scan([ctx.array(x)], n, out.desc(shape=(n + plus,)), tot if kind.endswith("'") else None)
+            got = out.get()
+            assert np.all(got[n + plus:] == -777), "wrote past the end"
+            exp = orc.scan(kind, orc.OP_ADD, x, seed=5)
+            if kind.endswith("'"):
+                assert np.array_equal(got[:n], exp[0]) and int(tot.get().reshape(-1)[0]) == int(np.asarray(exp[1]).reshape(-1)[0])
+            else:
+                assert np.array_equal(got[:n + plus], exp)
+    # elements of 1 and 8 bytes (16 and 2 a vector), from the left and from the right
+    for kind, fn in (("scanl1", np.maximum.accumulate), ("scanr1", lambda v: np.maximum.accumulate(v[::-1])[::-1])):
+        for ty, dt in (("Int8", np.int8), ("double", np.float64)):
+            sk = ctx.skeleton(A.SCAN_KINDS[kind], ty, env=[(1, ty)], get="arrIn0_0[ix]", combine="acc_max(x, y)")
+            for n in (1, 15, 17, 2049, 131071, 131073, 300001):
+                say(kind, "max", ty, "scan.small_below_kb =", small_below_kb, "n =", n)
+                x = (rng.standard_normal(n) * 40).astype(dt)
+                out = ctx.empty(n, dt)
+                sk.scan([ctx.array(x)], n, out)
+                assert np.array_equal(out.get(), fn(x)), (kind, ty, n)
+
+
 def test_scan_repeated_launches_and_sizes_interleaved(A, ctx, orc):
     """the tile descriptors and the ticket counter are reused between launches"""
     sk = ctx.skeleton(A.SKEL_SCANL, "Int32", env=[I32], get="arrIn0_0[ix]", combine="x + y", seed="0")
