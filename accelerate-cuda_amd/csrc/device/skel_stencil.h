@@ -30,13 +30,16 @@
  * distant rows at once; the price is that neighbouring strips re-read each
  * other's boundary rows.  ACC_XCD_REMAP renumbers the workgroups so that such
  * neighbours run on the same compute die (acc_xcd_contiguous_block).
- * Strips that are cut by the right edge, and arrays whose rows are not
- * 16-byte aligned, take a slower path that maps every element on its own.
+ * The last strip of a row of strips ends at the right edge (it overlaps its
+ * neighbour rather than reach past the edge); only an array narrower than a
+ * strip takes a slower path that maps every element on its own.  Rows that are
+ * not 16-byte aligned are read with the same 128-bit accesses, element-aligned.
  *
  * A 3-D stencil keeps a register window per plane it reads.  Without taps in
  * other planes, or with ACC_ZMARCH 0, a strip lies in ACC_TZ planes and all its
  * windows advance down the rows together.  With ACC_ZMARCH the two axes change
- * places: a strip is ACC_TZ rows tall and walks through ACC_TILE_H planes, the
+ * places: a strip is ACC_TZ rows tall and walks through ACC_TILE_H planes (or
+ * the fewer the driver asks for on a small volume, `acc_walk`), the
  * windows hold the 2 ry + ACC_TZ rows it reads of each of the 2 rz + 1 planes
  * in reach (plus the planes requested ahead), and a row fetched once serves
  * the results of every plane that reads it -- what a walk down the rows reads
@@ -273,7 +276,7 @@ struct acc_strip_source {
 #endif
 
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
-ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS ACC_GUARD_PARAM)
+ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS, const int acc_walk ACC_GUARD_PARAM)
 {
   ACC_GUARD_CHECK
   typedef ACC_ELT T;
@@ -310,9 +313,10 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS ACC_GUARD_PARA
   /* strips ACC_TZ rows tall, numbered DOWN a plane first (the waves of a workgroup are vertical neighbours: the rows
    * they share are asked for by one compute unit at about the same time), then across it, then run of ACC_TILE_H
    * planes after run */
+  /* (`acc_walk` planes a run: ACC_TILE_H, or fewer where strips that long would be too few to fill the device) */
   const Int64 bands = (h + ACC_TZ - 1) / ACC_TZ;
   const Int64 across = strip / bands;
-  const Int64 z0 = (across / strips_x) * ACC_TILE_H, y0 = (strip % bands) * ACC_TZ;
+  const Int64 z0 = (across / strips_x) * acc_walk, y0 = (strip % bands) * ACC_TZ;
   if (z0 >= d) return;
 #elif ACC_STENCIL_RANK == 3
   const Int64 bands = (h + ACC_TILE_H - 1) / ACC_TILE_H;
@@ -323,14 +327,19 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS ACC_GUARD_PARA
 #endif
   if (y0 >= h) return;                                   /* whole wave leaves together */
 #if ACC_STENCIL_RANK == 3 && ACC_ZMARCH
-  const Int64 x0 = (across % strips_x) * ACC_STRIP;
+  const Int64 x0_grid = (across % strips_x) * ACC_STRIP;
   (void)band; (void)x0_across;
 #else
-  const Int64 x0 = x0_across;
+  const Int64 x0_grid = x0_across;
 #endif
+  /* The last strip of a row of strips is laid to END at the right edge: it overlaps its neighbour, whose columns it
+   * produces a second time (the same values), instead of reaching past the edge, and every lane of it owns a whole
+   * vector like in any other strip.  (An array narrower than a strip has the one strip, on the element-wise path.) */
+  const Int64 x0 = (w >= ACC_STRIP && w - x0_grid >= ACC_SHIFT_MIN) ? acc_min<Int64>(x0_grid, w - ACC_STRIP) : x0_grid;
   const Int64 gx = x0 + lane * ACC_SVEC;
   /* how far the strip walks: rows, or planes */
-  const int rows_here = (int)acc_min<Int64>(ACC_TILE_H, ACC_ZMARCH ? d - z0 : h - y0);
+  const int rows_here = (int)acc_min<Int64>(ACC_ZMARCH ? acc_walk : ACC_TILE_H, ACC_ZMARCH ? d - z0 : h - y0);
+  (void)acc_walk;
   const bool fast_here = (x0 + ACC_STRIP <= w);          /* every lane owns a full vector */
 
   /* the strip, compiled three times: fast and ACC_TILE_H rows tall (all constants),
@@ -403,7 +412,14 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS ACC_GUARD_PARA
         /* newest row needed now is rho = y + 2 ry, in slot (s + NR - 1) % RING; the
          * slot freed by the previous step takes the row PREFETCH further on */
         const int rho_new = y + ACC_NR - 1 + ACC_PREFETCH;
-        if (rho_new < total) ACC_BOTH(fetch(rho_new, (s + ACC_RING - 1) % ACC_RING));
+        if (decltype(full_c)::value) {
+          if (rho_new < total) ACC_BOTH(fetch(rho_new, (s + ACC_RING - 1) % ACC_RING));
+        } else {
+          /* a strip of a length only known at run time asks without a test -- a load under a condition is waited
+           * for on the spot, and with it every row requested ahead: past the strip's end it asks for its last row
+           * again, into a slot nothing reads any more */
+          ACC_BOTH(fetch(acc_min(rho_new, total - 1), (s + ACC_RING - 1) % ACC_RING));
+        }
 #if ACC_SCHED_BARRIER & 2
         __builtin_amdgcn_sched_barrier(0);                 /* the requests of this step before anything of the step's results */
 #endif
