@@ -92,8 +92,9 @@
  * ACC_NZ source planes: a source row fetched once serves the results of up to 2 rz + 1 planes */
 #define ACC_NZ    (2 * ACC_RADIUS_S + ACC_TZ)         /* planes (rows) held side by side */
 #define ACC_TOTAL_MAX  (ACC_TILE_H + 2 * ACC_RADIUS_M)        /* source rows (planes) a strip touches, per window */
-#define ACC_HALO_COUNT (2 * ACC_RADIUS_X * ACC_TOTAL_MAX * ACC_NZ)   /* elements just outside the strip */
-#define ACC_HALO_LOADS (ACC_HALO_COUNT > 0 ? (ACC_HALO_COUNT + ACC_WAVE - 1) / ACC_WAVE : 1)
+/* a strip cut by the right edge of the array gathers up to 2 rx + ACC_SVEC - 1 elements a row and window: where it walks
+ * through planes, a lane each in one request */
+#define ACC_CUT_OK (!ACC_ZMARCH || ACC_NZ * (2 * ACC_RADIUS_X + ACC_SVEC - 1) <= ACC_WAVE)
 
 static_assert(ACC_RADIUS_X <= ACC_SVEC, "stencil wider than one lane's neighbours can supply");
 
@@ -121,8 +122,19 @@ template <typename T> ACC_DEV T acc_wave_shift_down1(const T &x) { return acc_dp
 /* One source array as a strip sees it: the register window of ACC_RING rows,
  * each row [rx left | ACC_SVEC own | rx right] per lane, and what fills it.
  * S element type, MODE boundary condition, FAST the aligned full-strip path. */
-template <typename S, int MODE, bool FAST>
+/* CUT (with FAST): the strip reaches past the right edge of the array.  The lanes whose four columns lie inside work as
+ * in any strip; lane `last` holds the `rem` columns left over (all four if rem is 0), lanes beyond it nothing.  Every
+ * lane still makes one 128-bit request -- from the edge on, for the last whole vector of the row, whose elements the
+ * lane across the edge moves down to where its columns belong -- and what stands right of the array (the rest of that
+ * lane's vector, then the rx elements its results reach for) is gathered like the elements outside a full strip. */
+template <typename S, int MODE, bool FAST, bool CUT = false>
 struct acc_strip_source {
+  static_assert(FAST || !CUT, "a cut strip is a fast strip");
+  static constexpr int RX = ACC_RADIUS_X;
+  static constexpr int RIGHT = CUT ? RX + ACC_SVEC - 1 : RX;       /* gathered elements right of the strip, a row */
+  static constexpr int PER_ROW = RX + RIGHT;                        /* ... either side */
+  static constexpr int HALO_COUNT = PER_ROW * ACC_TOTAL_MAX * ACC_NZ;
+  static constexpr int HALO_LOADS = HALO_COUNT > 0 ? (HALO_COUNT + ACC_WAVE - 1) / ACC_WAVE : 1;
   struct row { S e[ACC_WW]; };
   /* one lane's run of a row.  When rows start on 16-byte boundaries (ACC_ALIGNED) the type says so; otherwise
    * it is only element-aligned, which the memory instructions accept as well */
@@ -133,8 +145,9 @@ struct acc_strip_source {
   S outside;
   Int64 z0, y0, x0, gx;     /* the strip's plane and origin, this lane's first column */
   int lane, total;          /* total = source rows the strip touches in each plane */
+  int last, rem;            /* CUT: the lane across the right edge, and how many of its columns lie inside (0: all) */
   row ring[ACC_NZ][ACC_RING];
-  S halo[ACC_HALO_LOADS];
+  S halo[HALO_LOADS];
 #if ACC_ZMARCH
   S halo_ring[ACC_RING];    /* lane (p * 2 + side) * rx + j: the element outside the strip for window p of the slot's plane */
 #endif
@@ -145,7 +158,7 @@ struct acc_strip_source {
   ACC_DEV S outside_element(const int p, const int rho, const int side, const int j) const
   {
     const Int64 gz = plane_of(p, rho), gy = row_of(p, rho);
-    const Int64 xx = side ? x0 + ACC_STRIP + j : x0 - ACC_RADIUS_X + j;
+    const Int64 xx = side ? (CUT ? w : x0 + ACC_STRIP) + j : x0 - ACC_RADIUS_X + j;
     if (MODE == ACC_B_CONSTANT) {
       const bool inside = gz >= 0 && gz < d && gy >= 0 && gy < h && xx >= 0 && xx < w;
       const Int64 mz = acc_max<Int64>(0, acc_min<Int64>(gz, d - 1));
@@ -162,29 +175,31 @@ struct acc_strip_source {
    * for the strip instead of two per row. */
   ACC_DEV void gather_halo()
   {
-    if (!FAST || ACC_ZMARCH) return;                       /* (a strip that walks through planes asks line by line: fetch) */
+    if (!FAST || ACC_ZMARCH || RX == 0) return;            /* (a strip that walks through planes asks line by line: fetch) */
+    constexpr int per_plane = PER_ROW * ACC_TOTAL_MAX > 0 ? PER_ROW * ACC_TOTAL_MAX : 1;
 #pragma unroll
-    for (int g = 0; g < ACC_HALO_LOADS; ++g) {
+    for (int g = 0; g < HALO_LOADS; ++g) {
       const int q = lane + ACC_WAVE * g;
-      const int per_plane = 2 * ACC_RADIUS_X * ACC_TOTAL_MAX + (ACC_RADIUS_X == 0);
       const int p = q / per_plane, qq = q % per_plane;
-      const int side = qq / (ACC_RADIUS_X * ACC_TOTAL_MAX + (ACC_RADIUS_X == 0)), rem = qq % (ACC_RADIUS_X * ACC_TOTAL_MAX + (ACC_RADIUS_X == 0));
-      const int j = rem / ACC_TOTAL_MAX, rho = rem % ACC_TOTAL_MAX;
+      const int entry = qq / ACC_TOTAL_MAX, rho = qq % ACC_TOTAL_MAX;     /* entries 0 .. rx - 1 left, the others right */
       halo[g] = S();
-      if (q < ACC_HALO_COUNT && rho < total) halo[g] = outside_element(p, rho, side, j);
+      if (q < HALO_COUNT && rho < total) halo[g] = outside_element(p, rho, entry >= RX, entry >= RX ? entry - RX : entry);
     }
   }
+  /* the j-th element left (side 0) or right of the strip, for window p and line rho (held in ring slot `slot`); j may be
+   * a run-time value that is the same in every lane */
   ACC_DEV S halo_of(const int p, const int side, const int j, const int rho, const int slot) const
   {
+    const int entry = side ? RX + j : j;
 #if ACC_ZMARCH
     (void)rho;
-    return acc_readlane(halo_ring[slot], (p * 2 + side) * ACC_RADIUS_X + j);
+    return acc_readlane(halo_ring[slot], p * PER_ROW + entry);
 #endif
     (void)slot;
-    const int q = p * (2 * ACC_RADIUS_X * ACC_TOTAL_MAX) + (side * ACC_RADIUS_X + j) * ACC_TOTAL_MAX + rho;
+    const int q = p * (PER_ROW * ACC_TOTAL_MAX) + entry * ACC_TOTAL_MAX + rho;
     S v = acc_readlane(halo[0], q % ACC_WAVE);
 #pragma unroll
-    for (int g = 1; g < ACC_HALO_LOADS; ++g)
+    for (int g = 1; g < HALO_LOADS; ++g)
       if (q / ACC_WAVE == g) v = acc_readlane(halo[g], q % ACC_WAVE);
     return v;
   }
@@ -195,11 +210,12 @@ struct acc_strip_source {
   {
 #if ACC_ZMARCH
     /* the 2 rx elements outside the strip of all the windows' rows of this plane: one request, a lane each */
-    static_assert(ACC_NZ * 2 * ACC_RADIUS_X <= ACC_WAVE, "more elements outside the strip than lanes to ask for them");
-    if (FAST && ACC_RADIUS_X > 0) {
-      constexpr int rx = ACC_RADIUS_X > 0 ? ACC_RADIUS_X : 1;
+    static_assert(ACC_NZ * PER_ROW <= ACC_WAVE, "more elements outside the strip than lanes to ask for them");
+    if (FAST && RX > 0) {
+      constexpr int per_row = PER_ROW > 0 ? PER_ROW : 1;
+      const int entry = lane % per_row;
       halo_ring[slot] = S();
-      if (lane < ACC_NZ * 2 * rx) halo_ring[slot] = outside_element(lane / (2 * rx), rho, (lane / rx) % 2, lane % rx);
+      if (lane < ACC_NZ * per_row) halo_ring[slot] = outside_element(lane / per_row, rho, entry >= RX, entry >= RX ? entry - RX : entry);
     }
 #endif
 #pragma unroll
@@ -215,7 +231,19 @@ struct acc_strip_source {
     const Int64 mz = MODE == ACC_B_CONSTANT ? acc_max<Int64>(0, acc_min<Int64>(gz, d - 1)) : acc_boundary_index<MODE>(gz, d);
     const S *src = base + (mz * h + my) * w;
     if (FAST) {
-      const vec own = *(const vec *)(src + gx);
+      const Int64 from = CUT ? acc_min<Int64>(gx, w - ACC_SVEC) : gx;
+      vec own = *(const vec *)(src + from);
+      if (CUT) {
+        /* the lane across the edge has asked `down` elements to the left of its own columns: move them down (lanes
+         * beyond it move theirs anywhere: nothing of theirs is used) */
+        const int down = (int)(gx - from);
+        const vec asked = own;
+#pragma unroll
+        for (int k = 0; k + 1 < ACC_SVEC; ++k) {
+#pragma unroll
+          for (int m = 1; k + m < ACC_SVEC; ++m) own.v[k] = (down == m) ? asked.v[k + m] : own.v[k];
+        }
+      }
 #pragma unroll
       for (int k = 0; k < ACC_SVEC; ++k) r.e[ACC_RADIUS_X + k] = row_inside ? own.v[k] : outside;
 #pragma unroll
@@ -247,6 +275,14 @@ struct acc_strip_source {
 #pragma unroll
     for (int p = 0; p < ACC_NZ; ++p) {
       row &r = ring[p][slot];
+      if (CUT && RX > 0) {
+        /* first the columns of the lane across the edge that lie outside the array: its neighbour reads them below */
+#pragma unroll
+        for (int k = 1; k < ACC_SVEC; ++k) {
+          const S outside_own = halo_of(p, 1, acc_max(0, k - rem), rho, slot);
+          r.e[ACC_RADIUS_X + k] = (lane == last && rem != 0 && k >= rem) ? outside_own : r.e[ACC_RADIUS_X + k];
+        }
+      }
 #pragma unroll
       for (int j = 0; j < ACC_RADIUS_X; ++j) {
         const S from_left  = acc_wave_shift_up1(r.e[ACC_SVEC + j]);          /* neighbour's own[SVEC - rx + j] */
@@ -254,9 +290,12 @@ struct acc_strip_source {
         /* (read by every lane, before the choice: a read of another lane's register made under a condition sees
          * whatever that lane holds where only the lanes that pass the condition have worked the value out -- for
          * an element narrower than a register, its widening) */
-        const S outside_left = halo_of(p, 0, j, rho, slot), outside_right = halo_of(p, 1, j, rho, slot);
+        /* (a cut strip: right of the lane across the edge come the columns of its own vector that lie outside the
+         * array, ACC_SVEC - rem of them if any, and then the elements asked for here) */
+        const int beyond = CUT ? (rem ? ACC_SVEC - rem : 0) : 0;
+        const S outside_left = halo_of(p, 0, j, rho, slot), outside_right = halo_of(p, 1, beyond + j, rho, slot);
         r.e[j] = (lane != 0) ? from_left : outside_left;
-        r.e[ACC_RADIUS_X + ACC_SVEC + j] = (lane != ACC_WAVE - 1) ? from_right : outside_right;
+        r.e[ACC_RADIUS_X + ACC_SVEC + j] = (lane != (CUT ? last : ACC_WAVE - 1)) ? from_right : outside_right;
       }
     }
   }
@@ -341,11 +380,22 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS, const int acc
   const int rows_here = (int)acc_min<Int64>(ACC_ZMARCH ? acc_walk : ACC_TILE_H, ACC_ZMARCH ? d - z0 : h - y0);
   (void)acc_walk;
   const bool fast_here = (x0 + ACC_STRIP <= w);          /* every lane owns a full vector */
+  /* a strip cut by the right edge: the last of its lanes with columns inside the array, and how many it has if not all
+   * (a row shorter than one vector is left to the element-wise path) */
+#if ACC_STENCIL_SOURCES == 2
+  const bool same_width = shStencil1_0 == w && shStencil2_0 == w;   /* (a wider source has elements where the result ends) */
+#else
+  const bool same_width = true;
+#endif
+  /* (with few columns inside, mapping each element on its own is cheaper: fewer than ACC_CUT_MIN take that path) */
+  const bool cut_here = ACC_CUT_OK && !fast_here && w >= ACC_SVEC && w - x0 >= ACC_CUT_MIN && same_width;
+  const int cut_last = (int)((w - x0 + ACC_SVEC - 1) / ACC_SVEC) - 1, cut_rem = (int)((w - x0) % ACC_SVEC);
 
-  /* the strip, compiled three times: fast and ACC_TILE_H rows tall (all constants),
-   * fast and cut by the bottom edge, and the element-wise path */
-  auto run = [&](auto fast_c, auto full_c) {
+  /* the strip, compiled four times: fast and ACC_TILE_H rows tall (all constants), fast and cut by the bottom edge,
+   * fast and cut by the right edge, and the element-wise path */
+  auto run = [&](auto fast_c, auto full_c, auto cut_c) {
   constexpr bool fast = decltype(fast_c)::value;
+  constexpr bool cut = decltype(cut_c)::value;
   const int rows = decltype(full_c)::value ? ACC_TILE_H : rows_here;
   const int total = rows + 2 * ACC_RADIUS_M;              /* source rows (planes) this strip touches */
 
@@ -368,7 +418,8 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS, const int acc
 #define ACC_SRC1_ARRAY(c) arrStencil_##c
 #endif
 #define ACC_DECLARE_A(c, CT, OUTSIDE, arg)                                         \
-  acc_strip_source<CT, ACC_BOUNDARY, fast> a##c;                                  \
+  acc_strip_source<CT, ACC_BOUNDARY, fast, cut> a##c;                             \
+  a##c.last = cut_last; a##c.rem = cut_rem;                                       \
   a##c.base = ACC_SRC1_ARRAY(c);                                                  \
   ACC_SRC1_EXTENTS(a##c);                                                         \
   a##c.outside = (CT)OUTSIDE;                                                     \
@@ -377,7 +428,8 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS, const int acc
 #undef ACC_DECLARE_A
 #if ACC_STENCIL_SOURCES == 2
 #define ACC_DECLARE_B(c, CT, OUTSIDE, arg)                                         \
-  acc_strip_source<CT, ACC_BOUNDARY2, fast> b##c;                                 \
+  acc_strip_source<CT, ACC_BOUNDARY2, fast, cut> b##c;                            \
+  b##c.last = cut_last; b##c.rem = cut_rem;                                       \
   b##c.base = ACC_SRC2_ARRAY(c);                                                  \
   ACC_SRC2_EXTENTS(b##c);                                                         \
   b##c.outside = (CT)OUTSIDE;                                                     \
@@ -452,7 +504,7 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS, const int acc
 #define ACC_STORE_COMPONENT(c, CT)                                                   \
         {                                                                            \
           CT *dst = arrOut_##c + at;                                                 \
-          if (fast) {                                                                \
+          if (fast && (!cut || gx + ACC_SVEC <= w)) {                                \
             typedef CT acc_out_native __attribute__((ext_vector_type(ACC_SVEC)));    \
             typedef acc_out_native acc_out_stored __attribute__((aligned(ACC_ALIGNED ? ACC_SVEC * sizeof(CT) : alignof(CT)))); \
             acc_out_native nv;                                                       \
@@ -476,9 +528,11 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS, const int acc
   };   /* run */
 
   if (fast_here) {
-    if (rows_here == ACC_TILE_H) run(acc_bool<true>(), acc_bool<true>());
-    else                         run(acc_bool<true>(), acc_bool<false>());
+    if (rows_here == ACC_TILE_H) run(acc_bool<true>(), acc_bool<true>(), acc_bool<false>());
+    else                         run(acc_bool<true>(), acc_bool<false>(), acc_bool<false>());
+  } else if (cut_here) {
+    run(acc_bool<true>(), acc_bool<false>(), acc_bool<ACC_CUT_OK>());
   } else {
-    run(acc_bool<false>(), acc_bool<false>());
+    run(acc_bool<false>(), acc_bool<false>(), acc_bool<false>());
   }
 }

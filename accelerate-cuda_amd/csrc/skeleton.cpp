@@ -357,6 +357,7 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "#define ACC_STENCIL_NT " << tune("stencil.nt", 1) << "\n";
       o << "#define ACC_SCHED_BARRIER " << tune("stencil.sched_barrier", 3) << "\n";
       o << "#define ACC_SHIFT_MIN " << tune("stencil.shift_min", sp.zmarch ? 1 : 96) << "\n";
+      o << "#define ACC_CUT_MIN " << tune("stencil.cut_min", sp.zmarch ? 4 : 64) << "\n";
       o << "#define ACC_STACK_WAVES " << (sp.out_rank == 2 ? tune("stencil.stack", 0) : 0) << "\n";
       o << "#define ACC_TILE_H " << sp.tile_h << "\n#define ACC_PREFETCH " << sp.prefetch << "\n#define ACC_BLOCK " << sp.block << "\n";
       o << "#define ACC_TZ " << sp.tile_z << "\n";

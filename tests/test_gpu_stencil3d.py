@@ -66,6 +66,25 @@ def test_stencil_3d(A, ctx, mode):
     assert np.array_equal(out.get(), exp)
 
 
+@pytest.mark.parametrize("tune", ["stencil.strips_per_cu=0", "stencil.walk_min=16", "stencil.walk_min=2"])
+def test_stencil_3d_walks_of_every_length(A, ctx, monkeypatch, tune):
+    """the driver shortens a strip's walk through the planes on volumes as small as these (to 4 planes); here the
+    full walk of 64 planes and walks of 16 and of 2 are forced on them: strips that continue one another, the last
+    one short, and the narrow last strip of a row that ends at the right edge"""
+    monkeypatch.setenv("ACC_HIP_TUNE", tune)
+    rng = np.random.default_rng(32)
+    for mode in ("clamp", "wrap", "constant"):
+        lap = ctx.skeleton(A.SKEL_STENCIL, "float", out_rank=3, taps=SEVEN, boundary=mode, boundary_constant="2.0f",
+                           stencil_fn="t1 + t2 + t3 + t4 + t5 + t6 - 6.0f * t0")
+        for shape in [(3, 33, 70), (6, 37, 517), (17, 40, 260), (70, 10, 260), (131, 5, 512), (67, 9, 700)]:
+            say("stencil 3-D", tune, mode, shape)
+            v = rng.integers(-9, 9, shape).astype(F)
+            dv, out = ctx.array(v), ctx.empty(shape, F)
+            lap.stencil([], dv, out)
+            t = pyref.tap_arrays3(v, SEVEN, mode, 2.0, shape)
+            assert np.array_equal(out.get(), t[1] + t[2] + t[3] + t[4] + t[5] + t[6] - F(6) * t[0])
+
+
 def test_stencil2_3d_and_iteration(A, ctx):
     rng = np.random.default_rng(32)
     say("stencil2 3-D, sources of different extents")

@@ -82,3 +82,61 @@ def test_random_stencils(A, ctx, rank):
             else:
                 ref = sum(T(c) * a for c, a in zip(coef, t)).astype(T)
             assert np.array_equal(out.get(), ref)
+
+
+@pytest.mark.parametrize("rank", [2, 3])
+def test_stencils_on_arrays_narrower_than_a_strip(A, ctx, rank):
+    """a strip is 256 columns wide: on narrower arrays (and in the last strip of wider ones, where that is short) the
+    lane across the right edge holds 1 to 4 columns, the lanes beyond it none.  Every width modulo 4, reaches of 1, 2
+    and 4 columns, every boundary mode, elements of 1, 4 and 8 bytes."""
+    rng = np.random.default_rng(2000 + rank)
+    widths = [4, 5, 6, 7, 9, 63, 64, 66, 100, 129, 131, 202, 253, 254, 255, 256 + 65, 256 + 130, 512 + 70]
+    for (ctype, T), mode, rx in itertools.product([("Int8", np.int8), ("float", np.float32), ("double", np.float64)],
+                                                  ["clamp", "mirror", "wrap", "constant"], [1, 2, 4]):
+        if rank == 3 and rx == 4:
+            continue
+        if rank == 2:
+            taps = [(0, 0), (0, -rx), (0, rx), (-1, 1), (1, -1), (1, rx - 1)]
+        else:
+            taps = [(0, 0, 0), (0, 0, -rx), (0, 0, rx), (-1, 0, 1), (1, 1, -1), (0, -1, rx - 1), (1, 0, 0)]
+        coef = [int(rng.integers(-2, 3)) or 1 for _ in taps]
+        whole = np.issubdtype(T, np.integer)
+        fn = " + ".join("(%s)(%d) * t%d" % (ctype, c, k) for k, c in enumerate(coef))
+        sk = ctx.skeleton(A.SKEL_STENCIL, ctype, out_rank=rank, taps=taps, boundary=mode, boundary_constant="(%s)2" % ctype,
+                          stencil_fn="(%s)(%s)" % (ctype, fn) if whole else fn)
+        for w in widths:
+            if w < rx + 1:
+                continue                                           # the index maps assume the array spans the stencil
+            shape = (7, w) if rank == 2 else (6, 5, w)
+            say("narrow stencil", ctype, mode, "reach", rx, "shape", shape)
+            v = rng.integers(0, 4, shape).astype(T)
+            out = ctx.empty(shape, T)
+            sk.stencil([], ctx.array(v), out)
+            t = pyref.tap_arrays3(v, taps, mode, 2, shape) if rank == 3 else pyref.tap_arrays(v, taps, mode, 2, shape)
+            if whole:
+                ref = sum(np.int64(c) * a.astype(np.int64) for c, a in zip(coef, t)).astype(T)
+            else:
+                ref = sum(T(c) * a for c, a in zip(coef, t)).astype(T)
+            assert np.array_equal(out.get(), ref), (ctype, mode, rx, shape)
+
+
+def test_stencil2_on_narrow_sources_of_equal_and_unequal_width(A, ctx):
+    """two sources as wide as the result take the cut strip; a wider source has elements where the result ends"""
+    rng = np.random.default_rng(2100)
+    taps = [(0, -1), (0, 0), (0, 1), (1, 1)]
+    for mode1, mode2 in (("clamp", "wrap"), ("mirror", "constant")):
+        sk = ctx.skeleton(A.SKEL_STENCIL2, "float", out_rank=2, taps=taps, taps2=taps, boundary=mode1, boundary2=mode2,
+                          boundary_constant="2.0f", boundary2_constant="2.0f",
+                          stencil_fn="t0 + 2.0f * t1 + t2 - t3 + u0 - 3.0f * u1 + u2 + u3")
+        for (w1, w2) in ((101, 101), (131, 140), (140, 131), (70, 70), (255, 300), (7, 7)):
+            h1, h2 = 9, 11
+            say("narrow stencil2", mode1, mode2, "widths", w1, w2)
+            a = rng.integers(0, 4, (h1, w1)).astype(np.float32)
+            b = rng.integers(0, 4, (h2, w2)).astype(np.float32)
+            shape = (min(h1, h2), min(w1, w2))
+            out = ctx.empty(shape, np.float32)
+            sk.stencil2([], ctx.array(a), ctx.array(b), out)
+            t = pyref.tap_arrays(a, taps, mode1, 2.0, shape)
+            u = pyref.tap_arrays(b, taps, mode2, 2.0, shape)
+            ref = t[0] + 2 * t[1] + t[2] - t[3] + u[0] - 3 * u[1] + u[2] + u[3]
+            assert np.array_equal(out.get(), ref.astype(np.float32)), (mode1, mode2, w1, w2)
