@@ -962,7 +962,9 @@ def test_right_handed_scans_of_every_element_width(A, ctx):
             assert np.array_equal(out.get(), inc)
             tot = ctx.empty((), dt)
             rp.scan([ctx.array(x)], n, out, total=tot)
-            assert np.array_equal(out.get(), np.concatenate([inc[1:] + dt(3), [dt(3)]]).astype(dt)) and tot.get()[()] == dt(inc[0] + dt(3))
+            with np.errstate(over="ignore"):                       # narrow elements wrap around, here as on the device
+                whole = dt(inc[0] + dt(3))
+            assert np.array_equal(out.get(), np.concatenate([inc[1:] + dt(3), [dt(3)]]).astype(dt)) and tot.get()[()] == whole
     say("right-handed scan of pairs")
     pr = ctx.skeleton(A.SKEL_SCANR1, "Int32, float", env=[(1, "Int32"), (1, "float")], get="acc_elt{arrIn0_0[ix], arrIn1_0[ix]}",
                       combine="acc_elt{x.a1 + y.a1, acc_max(x.a0, y.a0)}")
