@@ -7,7 +7,8 @@
  * from global memory (relying on the L1 cache, Context.hs:61-68), recovers the
  * multidimensional index with 64-bit divisions and tests a whole warp for
  * "interior" (Stencil.hs:103-110).  Here the work is cut into strips: one
- * 64-lane wave owns 256 columns (4 per lane) and walks down ACC_TILE_H rows,
+ * 64-lane wave owns 256 columns (ACC_SVEC = 4 per lane; 2 per lane, 128
+ * columns, of 8-byte elements) and walks down ACC_TILE_H rows,
  * keeping the 2 ry + 1 source rows it currently needs in registers:
  *   - every source row is fetched once per strip with one 128-bit load per
  *     lane, ACC_PREFETCH rows ahead of its use, so a wave always has several
@@ -66,7 +67,9 @@
  * READ(component, dz, dy, dx).
  */
 
+#ifndef ACC_SVEC
 #define ACC_SVEC  4                                   /* results per lane and row */
+#endif
 #define ACC_STRIP (ACC_WAVE * ACC_SVEC)               /* columns per wave */
 #ifndef ACC_ZMARCH
 #define ACC_ZMARCH 0

@@ -356,8 +356,9 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "#define ACC_XCD_REMAP " << tune("stencil.xcd_remap", 0) << "\n";
       o << "#define ACC_STENCIL_NT " << tune("stencil.nt", 1) << "\n";
       o << "#define ACC_SCHED_BARRIER " << tune("stencil.sched_barrier", 3) << "\n";
-      o << "#define ACC_SHIFT_MIN " << tune("stencil.shift_min", sp.zmarch ? 1 : 96) << "\n";
-      o << "#define ACC_CUT_MIN " << tune("stencil.cut_min", sp.zmarch ? 4 : 64) << "\n";
+      o << "#define ACC_SVEC " << sp.svec << "\n";
+      o << "#define ACC_SHIFT_MIN " << tune("stencil.shift_min", sp.zmarch ? 1 : 24 * sp.svec) << "\n";
+      o << "#define ACC_CUT_MIN " << tune("stencil.cut_min", sp.zmarch ? sp.svec : 16 * sp.svec) << "\n";
       o << "#define ACC_STACK_WAVES " << (sp.out_rank == 2 ? tune("stencil.stack", 0) : 0) << "\n";
       o << "#define ACC_TILE_H " << sp.tile_h << "\n#define ACC_PREFETCH " << sp.prefetch << "\n#define ACC_BLOCK " << sp.block << "\n";
       o << "#define ACC_TZ " << sp.tile_z << "\n";
@@ -597,7 +598,23 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
         ACC_TRY(in_comps(sp->stencil_in2_type, &sp->stencil_in2_comps, "stencil_in2_type"));
       }
       sp->block = tune("stencil.block", 256);
-      sp->tile_w = 256;                                  // one wave's strip: 64 lanes x 4 columns
+      // Columns a lane holds of every row: four, or two of an element of 8 bytes -- one 128-bit access either way, and
+      // half the registers for the row windows, so that strips stay as tall as for narrower elements (Float64, 3 x 3
+      // on 8192^2: 202.7 -> 174.6 us; 7 points on 256 x 512 x 512: 249.5 -> 190.3) -- unless the stencil reaches
+      // further to either side than that (the neighbouring lane supplies those columns).  Eight columns of 1- and
+      // 2-byte elements are no gain (an element takes a register whatever its width: Word16 3 x 3 43.1 -> 57.9 us).
+      {
+        int widest = 1, reach_x = 0;
+        for (const std::string &c : sp->stencil_in_comps) widest = std::max(widest, type_size(c));
+        for (const std::string &c : sp->stencil_in2_comps) widest = std::max(widest, type_size(c));
+        for (int t : sp->tap_dx) reach_x = std::max(reach_x, std::abs(t));
+        for (int t : sp->tap2_dx) reach_x = std::max(reach_x, std::abs(t));
+        const int svec = (widest >= 8 && reach_x <= 2) ? 2 : 4;
+        sp->svec = tune("stencil.svec", svec);
+        if (sp->svec != 2 && sp->svec != 4 && sp->svec != 8) return fail(ACC_ERR_INVALID, "stencil: %d columns a lane", sp->svec);
+        if (sp->svec < reach_x) return fail(ACC_ERR_INVALID, "stencil: a reach of %d columns with %d columns a lane", reach_x, sp->svec);
+      }
+      sp->tile_w = 64 * sp->svec;                        // one wave's strip
       sp->prefetch = sp->out_rank == 2 ? tune("stencil.prefetch", 3) : (sp->out_rank == 3 ? tune("stencil.prefetch3", 1) : 0);
       // 3-D: a strip that reaches across planes produces up to three planes of the result from one register window
       // (each source row it fetches then serves several planes instead of one), as many as keep the window of all
@@ -615,15 +632,17 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
         for (const std::string &c : sp->stencil_in2_comps) words += std::max(1, (type_size(c) + 3) / 4);
         // Taps in other planes: the strip walks through the planes instead of down the rows, so that a row fetched once
         // serves all the planes that read it; it is as many rows tall as keep the windows within 144 registers
-        // (2 ry + rows of them side by side, 2 rz + 1 + prefetch planes deep).
+        // (2 ry + rows of them side by side, 2 rz + 1 + prefetch planes deep); within 192 for elements of two words or
+        // more, which would otherwise get strips one row tall that read every row three times (Float64, 7 points,
+        // 256 x 512 x 512: 249.5 us; two rows tall, 207 registers, 231.5).
         sp->zmarch = (rz > 0 && 2 * rx * (2 * ry + 1) <= 64) ? (tune("stencil.zmarch", 1) ? 1 : 0) : 0;
         if (sp->zmarch) {
           for (int ty = 4; ty > 1 && planes_per_strip == 1; --ty)
-            if ((2 * ry + ty) * (2 * rz + 1 + sp->prefetch) * (4 + 2 * rx) * words <= 144) planes_per_strip = ty;
+            if ((2 * ry + ty) * (2 * rz + 1 + sp->prefetch) * (sp->svec + 2 * rx) * words <= (words > 1 ? 192 : 144)) planes_per_strip = ty;
           while (2 * rx * (2 * ry + planes_per_strip) > 64) --planes_per_strip;     // one lane each for the elements outside the strip
         } else {
           for (int tz = 3; rz > 0 && tz > 1 && planes_per_strip == 1; --tz)
-            if ((2 * rz + tz) * (2 * ry + 1 + sp->prefetch) * (4 + 2 * rx) * words <= 128) planes_per_strip = tz;
+            if ((2 * rz + tz) * (2 * ry + 1 + sp->prefetch) * (sp->svec + 2 * rx) * words <= 128) planes_per_strip = tz;
         }
       }
       sp->tile_z = sp->out_rank == 3 ? tune("stencil.tile_z", planes_per_strip) : 1;

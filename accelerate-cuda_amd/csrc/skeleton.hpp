@@ -38,6 +38,7 @@ struct SkelSpec {
   std::string boundary2_constant, stencil_in2_type;
   std::vector<int> tap2_dz, tap2_dy, tap2_dx;
   int tile_w = 256, tile_h = 4, prefetch = 3;
+  int svec = 4;                         // stencils: columns a lane holds of every row (tile_w = 64 of them)
   int tile_z = 1;                       // rank-3 stencils: result planes per strip (rows per strip where the strip walks through planes)
   int zmarch = 0;                       // rank-3 stencils: strips tile_z rows tall walk through tile_h planes
   // tuning
