@@ -1064,7 +1064,14 @@ static int stencil_once(acc_skel s, const acc_array *env, const acc_array *in, c
   // one wave per strip of 256 columns x tile_h rows
   // (for 2-D the waves of a workgroup are stacked vertically, so the row count is rounded up to whole groups)
   const int64_t waves = s->spec.block / 64;
-  const int64_t strips_x = (w + s->spec.tile_w - 1) / s->spec.tile_w;
+  // An array narrower than half a strip (a quarter) takes the variant with half (a quarter) of the columns a lane,
+  // where the stencil's reach allows: the lanes of a strip that lie outside the array do nothing.
+  int narrow = 0;
+  while (narrow < acc::tune("stencil.narrow_max", 2) && (s->spec.svec >> (narrow + 1)) >= std::max(1, s->spec.reach_x) &&
+         w <= (int64_t)64 * (s->spec.svec >> (narrow + 1)))
+    ++narrow;
+  const int64_t tile_w = (int64_t)64 * (s->spec.svec >> narrow);
+  const int64_t strips_x = (w + tile_w - 1) / tile_w;
   int64_t bands = (h + s->spec.tile_h - 1) / s->spec.tile_h;
   if (rank == 2 && acc::tune("stencil.stack", 0)) bands = (bands + waves - 1) / waves * waves;
   int64_t zbands = (planes + s->spec.tile_z - 1) / s->spec.tile_z;             // tile_z result planes per strip
@@ -1080,7 +1087,7 @@ static int stencil_once(acc_skel s, const acc_array *env, const acc_array *in, c
     zbands = (planes + walk - 1) / walk;
   }
   args.i32(static_cast<int32_t>(walk));
-  return launch(s, aligned ? 0 : 1, (strips_x * bands * zbands + waves - 1) / waves, 0, st, &args);
+  return launch(s, (aligned ? 0 : 1) + 2 * narrow, (strips_x * bands * zbands + waves - 1) / waves, 0, st, &args);
 }
 
 static int stencil_check(acc_skel s, const acc_array *in, const acc_array *out)

@@ -611,7 +611,8 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
         for (int t : sp->tap2_dx) reach_x = std::max(reach_x, std::abs(t));
         const int svec = (widest >= 8 && reach_x <= 2) ? 2 : 4;
         sp->svec = tune("stencil.svec", svec);
-        if (sp->svec != 2 && sp->svec != 4 && sp->svec != 8) return fail(ACC_ERR_INVALID, "stencil: %d columns a lane", sp->svec);
+        sp->reach_x = reach_x;
+        if (sp->svec != 1 && sp->svec != 2 && sp->svec != 4 && sp->svec != 8) return fail(ACC_ERR_INVALID, "stencil: %d columns a lane", sp->svec);
         if (sp->svec < reach_x) return fail(ACC_ERR_INVALID, "stencil: a reach of %d columns with %d columns a lane", reach_x, sp->svec);
       }
       sp->tile_w = 64 * sp->svec;                        // one wave's strip
@@ -707,6 +708,12 @@ SkelSpec spec_of_variant(const SkelSpec &base, int v)
   }
   // a segmented fold's variants 2 and 3: a longer staged chunk, for segments of 8 elements or more on average
   if (spec.kind != ACC_SKEL_PERMUTE && v >= 2 && spec.chunk_long > 0) spec.chunk = spec.chunk_long;
+  // a stencil's variants 2 and 3, 4 and 5: half and a quarter of the columns a lane, for arrays narrower than half or a
+  // quarter of a strip, whose lanes would otherwise mostly lie outside the array
+  if ((spec.kind == ACC_SKEL_STENCIL || spec.kind == ACC_SKEL_STENCIL2) && v >= 2) {
+    spec.svec = std::max(1, spec.svec >> (v / 2));
+    spec.tile_w = 64 * spec.svec;
+  }
   // a scan's variants 2 and 3: a small tile, for arrays of a few tiles at most (a lone workgroup runs through the
   // instructions of all its rows one after the other whether the array fills them or not)
   if (spec.scan_small_rows > 0 && v >= 2) {

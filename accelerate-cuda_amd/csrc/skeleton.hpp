@@ -39,6 +39,7 @@ struct SkelSpec {
   std::vector<int> tap2_dz, tap2_dy, tap2_dx;
   int tile_w = 256, tile_h = 4, prefetch = 3;
   int svec = 4;                         // stencils: columns a lane holds of every row (tile_w = 64 of them)
+  int reach_x = 0;                      // stencils: the furthest a tap reaches to either side
   int tile_z = 1;                       // rank-3 stencils: result planes per strip (rows per strip where the strip walks through planes)
   int zmarch = 0;                       // rank-3 stencils: strips tile_z rows tall walk through tile_h planes
   // tuning
@@ -86,7 +87,9 @@ struct acc_skel_s {
   acc::Variant variants[8];   // [0] pointers 16-byte aligned, [1] no assumption; [2], [3]: the same for the
                               // table-in-LDS form of a permute whose combination has no atomic instruction;
                               // [4], [5]: for a hinted permute over several LDS windows of targets;
-                              // [6], [7]: for integer addition on a table of 16-bit counts in LDS
+                              // [6], [7]: for integer addition on a table of 16-bit counts in LDS;
+                              // of a segmented fold [2], [3]: a longer staged chunk; of a scan [2], [3]: small tiles;
+                              // of a stencil [2], [3] and [4], [5]: half and a quarter of the columns a lane
   std::mutex mu;
 
   int ensure_variant(int v);
