@@ -309,8 +309,11 @@ class Acc(object):
     """An array-valued computation: its shape (outermost first), element type and either a device
     array (manifest) or an index -> value function (delayed)."""
 
-    def __init__(self, shape, ctype, manifest=None, at=None):
+    def __init__(self, shape, ctype, manifest=None, at=None, across=False):
         self.shape, self.ctype, self.manifest, self.at = tuple(int(s) for s in shape), ctype, manifest, at
+        # a delayed array that reads a source across its rows (a transpose): the map kernel that makes it manifest
+        # produces it in square tiles (ACC_FLAG_TILED)
+        self.across = bool(across) and manifest is None and len(self.shape) >= 2
 
     @property
     def size(self):
@@ -630,7 +633,7 @@ def _probe(f, *ctypes):
 
 def map(f, a):
     t = _probe(f, a.ctype)
-    return Acc(a.shape, t, at=lambda ix: Exp.of(f(a.index(ix))))
+    return Acc(a.shape, t, at=lambda ix: Exp.of(f(a.index(ix))), across=a.across)
 
 
 def _meet(s1, s2):
@@ -646,7 +649,7 @@ def zipWith(f, a, b):
         a = a if a.shape == shape else backpermute(shape, lambda *i: i, a)
         b = b if b.shape == shape else backpermute(shape, lambda *i: i, b)
     t = _probe(f, a.ctype, b.ctype)
-    return Acc(a.shape, t, at=lambda ix: Exp.of(f(a.index(ix), b.index(ix))))
+    return Acc(a.shape, t, at=lambda ix: Exp.of(f(a.index(ix), b.index(ix))), across=a.across or b.across)
 
 
 def generate(shape, f):
@@ -655,15 +658,16 @@ def generate(shape, f):
     return Acc(shape, t, at=lambda ix: Exp.of(f(*_unlinear(ix, shape))))
 
 
-def backpermute(shape, p, a):
-    """result[i] = a[p(i)]: p takes the result's multi-index and returns a multi-index of `a`"""
+def backpermute(shape, p, a, across=False):
+    """result[i] = a[p(i)]: p takes the result's multi-index and returns a multi-index of `a`.  `across`: p walks
+    down a column of `a` where the result's index moves along a row (see transpose)"""
     shape = (shape,) if isinstance(shape, numbers.Integral) else tuple(shape)
-    return Acc(shape, a.ctype, at=lambda ix: a.index(_linear(p(*_unlinear(ix, shape)), a.shape)))
+    return Acc(shape, a.ctype, at=lambda ix: a.index(_linear(p(*_unlinear(ix, shape)), a.shape)), across=across)
 
 
 def transpose(a):
     h, w = a.shape
-    return backpermute((w, h), lambda y, x: (x, y), a)
+    return backpermute((w, h), lambda y, x: (x, y), a, across=True)
 
 
 def zip_(a, b):
@@ -687,7 +691,7 @@ def _force(a, cx):
     if a.manifest is not None:
         return a
     arrays, sig, fr = _assemble(get=a.stream().text)
-    sk = cx.skeleton(A.SKEL_MAP, _elt(a.ctype), sig, out_rank=len(a.shape), **fr)
+    sk = cx.skeleton(A.SKEL_MAP, _elt(a.ctype), sig, out_rank=len(a.shape), flags=A.FLAG_TILED if a.across else 0, **fr)
     out = _empty(cx, a.shape, a.ctype)
     cx.launch(arrays, [out], lambda i, o, s: sk.map(i, o[0], stream=s))
     return Acc(a.shape, a.ctype, manifest=out)

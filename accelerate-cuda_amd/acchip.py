@@ -25,7 +25,7 @@ SCAN_KINDS = {"scanl": SKEL_SCANL, "scanl1": SKEL_SCANL1, "scanl'": SKEL_SCANLP,
               "scanr": SKEL_SCANR, "scanr1": SKEL_SCANR1, "scanr'": SKEL_SCANRP}
 COMBINE_GENERIC, COMBINE_ADD, COMBINE_MIN, COMBINE_MAX, COMBINE_AND, COMBINE_OR, COMBINE_XOR = range(7)
 BOUNDARY = {"clamp": 0, "mirror": 1, "wrap": 2, "constant": 3}
-FLAG_FOLD_RIGHT, FLAG_FAST_MATH, FLAG_GUARDED = 1, 2, 4
+FLAG_FOLD_RIGHT, FLAG_FAST_MATH, FLAG_GUARDED, FLAG_TILED = 1, 2, 4, 8
 
 CTYPE = {np.dtype(np.float32): "float", np.dtype(np.float64): "double",
          np.dtype(np.int8): "Int8", np.dtype(np.int16): "Int16", np.dtype(np.int32): "Int32",

@@ -278,6 +278,15 @@ int acc_exec_map(acc_skel s, const acc_array *env, const acc_array *out, acc_str
   if (n == 0) return ACC_OK;
   const int v = aligned ? 0 : 1;
   ACC_TRY(s->ensure_variant(v));
+  if (s->spec.map_tiled) {
+    // a wave per tile of 32 x 32 elements of the two innermost dimensions (skel_map.h)
+    const int rank = s->spec.out_rank;
+    const int64_t side = 8 * (int64_t)s->spec.map_tile_block;
+    const int64_t w = out->shape[rank - 1], h = out->shape[rank - 2];
+    const int64_t tiles = ((w + side - 1) / side) * ((h + side - 1) / side) * (n / (w * h));
+    const int64_t waves = s->variants[v].block / 64;
+    return launch(s, v, std::min<int64_t>((tiles + waves - 1) / waves, (int64_t)1 << 22), 0, static_cast<hipStream_t>(stream), &args);
+  }
   // streaming with no reuse: one short-lived workgroup per tile keeps the most loads in flight
   const int64_t grid = acc_launch_grid(n, s->elements_per_block(), resident(s, v), acc::tune("map.oversub", 1 << 20));
   return launch(s, v, grid, 0, static_cast<hipStream_t>(stream), &args);

@@ -227,6 +227,7 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "#define ACC_OUT_PARAMS " << out_params(sp.out_rank, sp.elt_type) << "\n";
       o << "#define ACC_OUT_SIZE " << out_size(sp.out_rank) << "\n";
       o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_UNROLL " << sp.unroll << "\n";
+      o << "#define ACC_MAP_TILED " << (sp.map_tiled ? 1 : 0) << "\n#define ACC_TT " << sp.map_tile_block << "\n";
       tmpl = "skel_map.h";
       break;
     case ACC_SKEL_FOLD:
@@ -476,6 +477,9 @@ int make_spec(const acc_skel_desc *d, SkelSpec *sp)
     sp->vec_size = sp->elt_size;
   }
   sp->guarded = (d->flags & ACC_FLAG_GUARDED) != 0;
+  sp->map_tile_block = std::max(1, std::min(tune("map.tile_block", 4), 8));
+  sp->map_tiled = (d->flags & ACC_FLAG_TILED) != 0 && d->out_rank >= 2 &&
+                  (d->kind == ACC_SKEL_MAP || d->kind == ACC_SKEL_GENERATE || d->kind == ACC_SKEL_TRANSFORM) && tune("map.tiled", 1) != 0;
   sp->out_rank = d->out_rank;
   if (sp->out_rank < 0 || sp->out_rank > ACC_MAX_RANK) return fail(ACC_ERR_INVALID, "bad out_rank %d", d->out_rank);
   for (int k = 0; k < d->n_env; ++k) {

@@ -46,6 +46,8 @@ struct SkelSpec {
   int block = 256, unroll = 4, rows = 4, chunk = 4096;
   int merge_waves = 4;                  // permute of 16-bit counts: waves of a workgroup of permute_merge
   int chunk_long = 0;                   // segmented folds: the staged chunk of variants 2 and 3 (segments of 8 elements or more on average); 0: none
+  bool map_tiled = false;               // ACC_FLAG_TILED on a map of rank 2 or more: tiles of 32 x 32 elements, a wave each
+  int map_tile_block = 4;               // ... a lane's share of a tile: a block of that many elements either way
   bool guarded = false;                 // ACC_FLAG_GUARDED: every kernel takes the address of a loop's guard word last
   bool fold_single = true;              // foldAll in one launch (the last workgroup collects), as generated into the kernel
   int scan_rows_fallback = 8;

@@ -28,7 +28,9 @@ import Data.Array.Accelerate.HIP.FFI
 import Data.Array.Accelerate.HIP.State                          -- HIP monad: the context, the memory table, the stream reservoir
 
 import Control.Monad.Trans                                      ( liftIO )
+import Data.Bits                                              ( (.|.) )
 import Data.Int
+import Data.Word                                              ( Word32 )
 import Data.List                                                ( intercalate )
 
 
@@ -96,7 +98,10 @@ compileOpenAcc guarded (Manifest pacc) =
       kernel accSkelMap g get Nothing Nothing Nothing =<< (ZipWith <$> travF f <*> travD a <*> travD b)
     Backpermute sh p a    -> do
       let (get, g) = gatherThrough p a
-      kernel accSkelTransform g get Nothing Nothing Nothing =<< (Backpermute <$> travE sh <*> travF p <*> travD a)
+          -- an index function that exchanges the two innermost components of the index (`transpose`) reads one
+          -- element of every source row per run of the result: such a kernel produces its result in square tiles
+          across   = if exchangesInnermost p then accFlagTiled else 0
+      kernelWith across accSkelTransform g get Nothing Nothing Nothing =<< (Backpermute <$> travE sh <*> travF p <*> travD a)
     Replicate{}           -> fusedAway "Replicate"
     Slice{}               -> fusedAway "Slice"
 
@@ -157,11 +162,15 @@ compileOpenAcc guarded (Manifest pacc) =
     -- one skeleton instance: fragments -> description -> acc_skel_create (compiled, cached and loaded inside)
     kernel :: Int32 -> Gamma -> Fragment -> Maybe Fragment -> Maybe Fragment -> Maybe Fragment
            -> PreOpenAcc ExecOpenAcc aenv a -> HIP (ExecOpenAcc aenv a)
-    kernel kind gamma get combine seed permutation node = do
+    kernel = kernelWith 0
+
+    kernelWith :: Word32 -> Int32 -> Gamma -> Fragment -> Maybe Fragment -> Maybe Fragment -> Maybe Fragment
+               -> PreOpenAcc ExecOpenAcc aenv a -> HIP (ExecOpenAcc aenv a)
+    kernelWith flags kind gamma get combine seed permutation node = do
       ctx  <- hipContext
       skel <- liftIO $ createSkeleton ctx Skeleton
                 { skelKind        = kind
-                , skelFlags       = if guarded then accFlagGuarded else 0
+                , skelFlags       = flags .|. (if guarded then accFlagGuarded else 0)
                 , skelEnv         = environment gamma
                 , skelEltType     = intercalate ", " (resultTypes node)
                 , skelOutRank     = resultRank node
@@ -213,6 +222,7 @@ environment     :: Gamma -> [(Int32, [String])]
 resultTypes     :: PreOpenAcc ExecOpenAcc aenv a -> [String]
 resultRank      :: PreOpenAcc ExecOpenAcc aenv a -> Int32
 combineHint     :: Fragment -> Int32              -- ACC_COMBINE_ADD .. when the text is literally x + y, acc_pmin(x, y), ...
+exchangesInnermost :: PreOpenFun DelayedOpenAcc () aenv (sh' -> sh) -> Bool   -- \(sh :. y :. x) -> (sh :. x :. y), structurally
 stencilFragment :: PreOpenAcc ExecOpenAcc aenv a -> Fragment
 rebuildExp      :: (forall b. DelayedOpenAcc aenv b -> HIP (ExecOpenAcc aenv b)) -> PreOpenExp DelayedOpenAcc env aenv t -> HIP (PreOpenExp ExecOpenAcc env aenv t)
 fromIndexFun    = undefined
@@ -224,5 +234,6 @@ environment     = undefined
 resultTypes     = undefined
 resultRank      = undefined
 combineHint     = undefined
+exchangesInnermost = undefined
 stencilFragment = undefined
 rebuildExp      = undefined

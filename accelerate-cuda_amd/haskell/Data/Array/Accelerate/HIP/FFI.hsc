@@ -85,10 +85,11 @@ accCombineAnd     = #{const ACC_COMBINE_AND}
 accCombineOr      = #{const ACC_COMBINE_OR}
 accCombineXor     = #{const ACC_COMBINE_XOR}
 
-accFlagFoldRight, accFlagFastMath, accFlagGuarded :: Word32
+accFlagFoldRight, accFlagFastMath, accFlagGuarded, accFlagTiled :: Word32
 accFlagFoldRight = #{const ACC_FLAG_FOLD_RIGHT}
 accFlagFastMath  = #{const ACC_FLAG_FAST_MATH}
 accFlagGuarded   = #{const ACC_FLAG_GUARDED}
+accFlagTiled     = #{const ACC_FLAG_TILED}
 
 data HIPException = HIPException Status String
   deriving (Typeable)

@@ -265,6 +265,10 @@ enum { ACC_BOUNDARY_CLAMP = 0, ACC_BOUNDARY_MIRROR = 1, ACC_BOUNDARY_WRAP = 2, A
 /* flags */
 #define ACC_FLAG_FOLD_RIGHT   1u  /* foldSeg: associate x0 (+) (x1 (+) (... (+) z)) instead of ((x0 (+) x1) ...) (+) z */
 #define ACC_FLAG_FAST_MATH    2u  /* allow FMA contraction (default: off, every scalar op rounds as written) */
+#define ACC_FLAG_TILED        8u  /* map family, out_rank >= 2: produce the result in square tiles of its two innermost
+                                     dimensions instead of runs of the innermost one, for element functions that read
+                                     their sources across rows (a transposing backpermute: IndexSpace.hs:96-141 reads
+                                     one element of every source row per run); the results are the same */
 #define ACC_FLAG_GUARDED      4u  /* the instance may run under an acc_guard (see acc_guard_create): its kernels take the
                                      guard's address as one more, last, parameter and do nothing once the guard is down */
 

@@ -178,6 +178,13 @@ def test_index_transformations(acc):
     rng = np.random.default_rng(8)
     m = rng.integers(0, 1000, (37, 101)).astype(np.int32)
     assert np.array_equal(acc.run(acc.transpose(acc.use(m))), m.T)
+    # a transpose is produced in square tiles, and so is what is fused on top of it
+    big = rng.integers(0, 1000, (300, 517)).astype(np.int32)
+    other = rng.integers(0, 1000, (517, 300)).astype(np.int32)
+    tr = acc.transpose(acc.use(big))
+    assert tr.across and acc.map(lambda v: v + 1, tr).across
+    assert np.array_equal(acc.run(acc.map(lambda v: v * 2 + 1, tr)), big.T * 2 + 1)
+    assert np.array_equal(acc.run(acc.zipWith(lambda a, b: a - b, acc.use(other), tr)), other - big.T)
     x = rng.integers(0, 1000, 1001).astype(np.int64)
     assert np.array_equal(acc.run(acc.reverse(acc.use(x))), x[::-1])
     # zipWith over different extents takes the intersection

@@ -989,3 +989,31 @@ def test_scan_tile_shape_follows_the_register_count(A, ctx):
         sk.scan([ctx.array(x)], x.size, out)
         ref = np.cumsum(x, dtype=dt) if ctype == "Int32" else np.maximum.accumulate(x)
         assert np.array_equal(out.get(), ref)
+
+
+def test_map_in_tiles_gives_what_the_map_in_runs_gives(A, ctx):
+    """ACC_FLAG_TILED changes the order the result is produced in (tiles of 32 x 32, for element functions that read
+    across the rows of their source), never the result: transposes, ragged and narrow shapes, rank 3, a function of
+    the index alone, elements of 1 and 8 bytes"""
+    rng = np.random.default_rng(9)
+    for ctype, dt in (("float", np.float32), ("Int8", np.int8), ("double", np.float64)):
+        tr = ctx.skeleton(A.SKEL_MAP, ctype, env=[(2, ctype)], out_rank=2, flags=A.FLAG_TILED,
+                          get="arrIn0_0[(ix % shOut_0) * shIn0_0 + (ix / shOut_0)]")
+        for (h, w) in ((1, 1), (3, 70), (64, 64), (65, 63), (64, 128), (100, 257), (257, 100), (1, 500), (500, 1), (1030, 515)):
+            say("tiled transpose", ctype, (h, w))
+            src = rng.integers(-100, 100, (w, h)).astype(dt)              # the source is w x h, the result h x w
+            out = ctx.empty((h, w), dt)
+            tr.map([ctx.array(src)], out)
+            assert np.array_equal(out.get(), src.T)
+    say("tiled map of rank 3, a function of the index")
+    g = ctx.skeleton(A.SKEL_GENERATE, "Int32", env=[], out_rank=3, flags=A.FLAG_TILED, get="(Int32)(ix * 7 + 1)")
+    for shape in ((1, 1, 1), (3, 40, 50), (2, 33, 65), (5, 1, 300)):
+        out = ctx.empty(shape, np.int32)
+        g.map([], out)
+        assert np.array_equal(out.get().reshape(-1), (np.arange(int(np.prod(shape)), dtype=np.int64) * 7 + 1).astype(np.int32))
+    say("the flag on a vector is ignored")
+    v = ctx.skeleton(A.SKEL_MAP, "Int32", env=[I32], out_rank=1, flags=A.FLAG_TILED, get="arrIn0_0[ix] + 1")
+    x = rng.integers(0, 9, 1000).astype(np.int32)
+    out = ctx.empty(1000, np.int32)
+    v.map([ctx.array(x)], out)
+    assert np.array_equal(out.get(), x + 1)
