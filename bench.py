@@ -485,6 +485,53 @@ def main():
         sk["foldrows64"] = result("fold (+) rows of 64 Float32", w, e, 1, rows * width * 4 + rows * 4, rows * width)
         del dms, env_s, rs, m
 
+    # ---------------------------------------------------------------- not a configuration: other shapes and sizes
+    # (only when named: small scans, which take small tiles; stencils on volumes of few strips, on arrays narrower than
+    # a strip and over 8-byte elements; a transpose in runs and in tiles)
+    if "shapes" in only:
+        log("other shapes and sizes (us per launch, every launch on the same buffers) ...")
+        shapes = {}
+
+        def one(name, fn, nbytes):
+            w, e = T.run([fn])
+            shapes[name] = {"avg_launch_us": round(e * 1e3, 2), "GB_per_s": round(nbytes / (e * 1e-3) / 1e9, 1)}
+            log("  %-44s %9.2f us/launch  %8.1f GB/s" % (name, e * 1e3, nbytes / (e * 1e-3) / 1e9))
+
+        scan_s = ctx.skeleton(A.SKEL_SCANL, "Int32", env=[I32], get=rd(0), combine="x + y", seed="0")
+        for n in (1 << 10, 49155, 1 << 18, 1 << 21, (3 << 20) + 3, 1 << 22, 1 << 24):
+            x, o = ctx.array(np.ones(n, np.int32)), ctx.empty(n + 1, np.int32)
+            xe, od = envs(x), o.desc()
+            one("scanl (+) Int32 n = %d" % n, lambda: A.check(L.acc_exec_scan(scan_s.handle, xe, n, C.byref(od), None, stream)), 8 * n)
+            del x, o
+        seven = [(0, 0, 0), (-1, 0, 0), (1, 0, 0), (0, -1, 0), (0, 1, 0), (0, 0, -1), (0, 0, 1)]
+        nine = [(dy, dx) for dy in (-1, 0, 1) for dx in (-1, 0, 1)]
+        for ctype, dt in (("float", np.float32), ("double", np.float64)):
+            lap3 = ctx.skeleton(A.SKEL_STENCIL, ctype, out_rank=3, taps=seven, boundary="clamp", stencil_fn="t1 + t2 + t3 + t4 + t5 + t6 - 6 * t0")
+            box2 = ctx.skeleton(A.SKEL_STENCIL, ctype, out_rank=2, taps=nine, boundary="clamp", stencil_fn=" + ".join("t%d" % k for k in range(9)))
+            vols = ((512, 512, 512), (256, 256, 256), (128, 128, 256), (100, 400, 419), (1024, 128, 128), (4096, 64, 64)) if ctype == "float" else ((256, 512, 512),)
+            for shape in vols:
+                a, o = ctx.array(np.ones(shape, dt)), ctx.empty(shape, dt)
+                ad, od = a.desc(), o.desc()
+                one("stencil 7-point %s %d x %d x %d" % ((ctype,) + shape), lambda: A.check(L.acc_exec_stencil(lap3.handle, None, C.byref(ad), C.byref(od), stream)),
+                    2 * int(np.prod(shape)) * np.dtype(dt).itemsize)
+                del a, o
+            imgs = ((1 << 17, 128), (1 << 18, 64), (55924, 300)) if ctype == "float" else ((8192, 8192),)
+            for shape in imgs:
+                a, o = ctx.array(np.ones(shape, dt)), ctx.empty(shape, dt)
+                ad, od = a.desc(), o.desc()
+                one("stencil 3x3 %s %d x %d" % ((ctype,) + shape), lambda: A.check(L.acc_exec_stencil(box2.handle, None, C.byref(ad), C.byref(od), stream)),
+                    2 * int(np.prod(shape)) * np.dtype(dt).itemsize)
+                del a, o
+        side = 8192
+        src, dst = ctx.array(wl.stencil_image(side, side)), ctx.empty((side, side), np.float32)
+        se, dd = envs(src), dst.desc()
+        for name, flags in (("in runs", 0), ("in tiles (ACC_FLAG_TILED)", A.FLAG_TILED)):
+            tr = ctx.skeleton(A.SKEL_MAP, "float", env=[(2, "float")], out_rank=2, flags=flags, get="arrIn0_0[(ix % shOut_0) * shIn0_0 + (ix / shOut_0)]")
+            one("transpose 8192 x 8192 Float32 " + name, lambda: A.check(L.acc_exec_map(tr.handle, se, C.byref(dd), stream)), 8 * side * side)
+        assert np.array_equal(dst.get(), wl.stencil_image(side, side).T), "transpose mismatch"
+        sk["shapes"] = shapes
+        del src, dst
+
     if headline is None:     # --only without scan: report whatever ran first
         timed = sorted(k for k in sk if "ms_per_step" in sk[k])
         if not timed:
