@@ -93,8 +93,9 @@ def test_stencils_on_arrays_narrower_than_a_strip(A, ctx, rank):
     widths = [4, 5, 6, 7, 9, 63, 64, 66, 100, 129, 131, 202, 253, 254, 255, 256 + 65, 256 + 130, 512 + 70]
     for (ctype, T), mode, rx in itertools.product([("Int8", np.int8), ("float", np.float32), ("double", np.float64)],
                                                   ["clamp", "mirror", "wrap", "constant"], [1, 2, 4]):
-        if rank == 3 and rx == 4:
-            continue
+        if rank == 3 and (rx == 4 or (ctype == "double" and (rx != 1 or mode in ("mirror", "wrap"))) or
+                          (ctype == "Int8" and (rx != 2 or mode != "mirror"))):
+            continue                                               # (rank 3 compiles slowly: a selection)
         if rank == 2:
             taps = [(0, 0), (0, -rx), (0, rx), (-1, 1), (1, -1), (1, rx - 1)]
         else:
