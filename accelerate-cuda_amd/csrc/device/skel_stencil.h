@@ -236,7 +236,7 @@ struct acc_strip_source {
     if (FAST) {
       const Int64 from = CUT ? acc_min<Int64>(gx, w - ACC_SVEC) : gx;
       vec own = *(const vec *)(src + from);
-      if (CUT) {
+      if (CUT && rem != 0) {                     /* (the same in every lane: a row that ends with a whole vector skips this) */
         /* the lane across the edge has asked `down` elements to the left of its own columns: move them down (lanes
          * beyond it move theirs anywhere: nothing of theirs is used) */
         const int down = (int)(gx - from);
@@ -278,7 +278,7 @@ struct acc_strip_source {
 #pragma unroll
     for (int p = 0; p < ACC_NZ; ++p) {
       row &r = ring[p][slot];
-      if (CUT && RX > 0) {
+      if (CUT && RX > 0 && rem != 0) {
         /* first the columns of the lane across the edge that lie outside the array: its neighbour reads them below */
 #pragma unroll
         for (int k = 1; k < ACC_SVEC; ++k) {

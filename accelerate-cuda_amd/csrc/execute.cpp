@@ -1079,6 +1079,15 @@ static int stencil_once(acc_skel s, const acc_array *env, const acc_array *in, c
   while (narrow < acc::tune("stencil.narrow_max", 2) && (s->spec.svec >> (narrow + 1)) >= std::max(1, s->spec.reach_x) &&
          w <= (int64_t)64 * (s->spec.svec >> (narrow + 1)))
     ++narrow;
+  // Strips that walk through planes are bound by the instructions of a strip, whatever its share of columns inside the
+  // array: one and a half strips' width is taken as three strips of half the width, not as two of the whole one
+  // (200 x 200 x 300: 35.3 -> 27.4 us), and less than one strip's width as two of half the width, not as one that the
+  // edge of the array cuts (150^3: 17.0 -> 13.3 us).  (In 2-D the columns a last strip produces a second time cost
+  // next to nothing.)
+  if (narrow == 0 && s->spec.zmarch && (s->spec.svec >> 1) >= std::max(1, s->spec.reach_x) && acc::tune("stencil.half_strips", 1) != 0) {
+    const int64_t halves = (w + 32 * s->spec.svec - 1) / (32 * s->spec.svec);
+    if (halves == 3 || (halves == 2 && w < 64 * s->spec.svec)) narrow = 1;
+  }
   const int64_t tile_w = (int64_t)64 * (s->spec.svec >> narrow);
   const int64_t strips_x = (w + tile_w - 1) / tile_w;
   int64_t bands = (h + s->spec.tile_h - 1) / s->spec.tile_h;
