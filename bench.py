@@ -508,7 +508,7 @@ def main():
         for ctype, dt in (("float", np.float32), ("double", np.float64)):
             lap3 = ctx.skeleton(A.SKEL_STENCIL, ctype, out_rank=3, taps=seven, boundary="clamp", stencil_fn="t1 + t2 + t3 + t4 + t5 + t6 - 6 * t0")
             box2 = ctx.skeleton(A.SKEL_STENCIL, ctype, out_rank=2, taps=nine, boundary="clamp", stencil_fn=" + ".join("t%d" % k for k in range(9)))
-            vols = ((512, 512, 512), (256, 256, 256), (128, 128, 256), (100, 400, 419), (1024, 128, 128), (4096, 64, 64)) if ctype == "float" else ((256, 512, 512),)
+            vols = ((512, 512, 512), (384, 384, 384), (300, 300, 300), (256, 256, 256), (150, 150, 150), (128, 128, 256), (100, 400, 419), (1024, 128, 128), (4096, 64, 64)) if ctype == "float" else ((256, 512, 512),)
             for shape in vols:
                 a, o = ctx.array(np.ones(shape, dt)), ctx.empty(shape, dt)
                 ad, od = a.desc(), o.desc()
