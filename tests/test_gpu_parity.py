@@ -233,6 +233,23 @@ def test_scan_tiles_of_either_size_on_ragged_ends(A, ctx, orc, monkeypatch, smal
                 out = ctx.empty(n, dt)
                 sk.scan([ctx.array(x)], n, out)
                 assert np.array_equal(out.get(), fn(x)), (kind, ty, n)
+    # pairs (one array per component), from the left with a seed and from the right without
+    for kind in ("scanl", "scanr1"):
+        pr = ctx.skeleton(A.SCAN_KINDS[kind], "Int32, float", env=[(1, "Int32"), (1, "float")], get="acc_elt{arrIn0_0[ix], arrIn1_0[ix]}",
+                          combine="acc_elt{x.a1 + y.a1, acc_max(x.a0, y.a0)}", seed="acc_elt{3, -1.0f}" if kind == "scanl" else None)
+        for n in (5, 16385, 100003):
+            say(kind, "of pairs, scan.small_below_kb =", small_below_kb, "n =", n)
+            a, b = rng.integers(-9, 9, n).astype(np.int32), rng.random(n).astype(np.float32)
+            plus = 1 if kind == "scanl" else 0
+            out = A.TupleArray([ctx.empty(n + plus, np.int32), ctx.empty(n + plus, np.float32)])
+            pr.scan([ctx.array(a), ctx.array(b)], n, out)
+            if kind == "scanl":
+                want_a = np.concatenate([[3], 3 + np.cumsum(a, dtype=np.int64)]).astype(np.int32)
+                want_b = np.concatenate([[-1.0], np.maximum.accumulate(b)]).astype(np.float32)
+            else:
+                want_a = np.cumsum(a[::-1], dtype=np.int64)[::-1].astype(np.int32)
+                want_b = np.maximum.accumulate(b[::-1])[::-1]
+            assert np.array_equal(out.comps[0].get(), want_a) and np.array_equal(out.comps[1].get(), want_b), (kind, n)
 
 
 def test_scan_repeated_launches_and_sizes_interleaved(A, ctx, orc):
