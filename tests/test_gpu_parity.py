@@ -1028,6 +1028,14 @@ def test_map_in_tiles_gives_what_the_map_in_runs_gives(A, ctx):
         out = ctx.empty(shape, np.int32)
         g.map([], out)
         assert np.array_equal(out.get().reshape(-1), (np.arange(int(np.prod(shape)), dtype=np.int64) * 7 + 1).astype(np.int32))
+    say("tiled map producing pairs (one array per component)")
+    pt = ctx.skeleton(A.SKEL_MAP, "float, Int32", env=[(2, "float"), (2, "Int32")], out_rank=2, flags=A.FLAG_TILED,
+                      get="acc_elt{arrIn0_0[(ix % shOut_0) * shIn0_0 + (ix / shOut_0)] * 2.0f, arrIn1_0[ix] + 1}")
+    for (h, w) in ((5, 7), (64, 96), (70, 131)):
+        fa, ib = rng.integers(-9, 9, (w, h)).astype(np.float32), rng.integers(-9, 9, (h, w)).astype(np.int32)
+        out = ctx.empty_tuple((h, w), [np.float32, np.int32])
+        pt.map([ctx.array(fa), ctx.array(ib)], out)
+        assert np.array_equal(out.comps[0].get(), fa.T * 2) and np.array_equal(out.comps[1].get(), ib + 1)
     say("the flag on a vector is ignored")
     v = ctx.skeleton(A.SKEL_MAP, "Int32", env=[I32], out_rank=1, flags=A.FLAG_TILED, get="arrIn0_0[ix] + 1")
     x = rng.integers(0, 9, 1000).astype(np.int32)
