@@ -80,6 +80,9 @@ static_assert(ACC_CHUNK % (ACC_BLOCK * ACC_VEC) == 0, "chunk must be a whole num
 #endif
 #define ACC_PAD(i) (ACC_PAD_ON ? ((i) + ((i) >> 5)) : (i))
 #define ACC_EAT 8                                        /* LDS reads kept in flight while folding */
+#ifndef ACC_WIDE
+#define ACC_WIDE 256                                     /* elements of one segment in a chunk from which the workgroup folds them together */
+#endif
 
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
@@ -90,9 +93,14 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
   __shared__ __attribute__((aligned(16))) T s_val[ACC_PAD(ACC_CHUNK)];
+  /* for the stretches the whole workgroup folds (below) */
+  __shared__ int s_wide[ACC_BLOCK / ACC_WAVE];
+  __shared__ int s_owner, s_from, s_to;
+  __shared__ acc_opt<T> s_part[ACC_BLOCK / ACC_WAVE];
 
   auto get = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
   auto f   = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
+  auto lf  = acc_lift<T>(f);
 
   const Int64 nseg = shOut_0;
   const Int64 n = ACC_SEG_TOTAL;
@@ -100,6 +108,8 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
 #if ACC_HAS_SEED
   const T seed = (ACC_SEED);
 #endif
+  if (tid == 0) s_owner = ACC_BLOCK;
+  /* (seen by all at the first barrier of the first chunk) */
 
   for (Int64 first = (Int64)blockIdx.x * ACC_BLOCK; first < nseg; first += (Int64)gridDim.x * ACC_BLOCK) {
     const Int64 seg = first + tid;
@@ -168,12 +178,60 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
 #pragma unroll
           for (int k = 0; k < ACC_VEC; ++k) s_val[ACC_PAD((u * ACC_BLOCK + tid) * ACC_VEC + k)] = v[u][k];
         }
+      /* this lane's segment, as far as it lies in the chunk */
+      int p0 = (int)(acc_max(a, cs) - cs), p1 = (int)(acc_min(b, ce) - cs);
+      /* One lane a segment serialises a long segment on its lane while the rest of the workgroup waits: among a
+       * million short segments a single one of 2^23 elements took 130-200 ms.  A stretch of ACC_WIDE elements or more
+       * of one segment in a chunk is therefore folded by the whole workgroup: every lane a run of consecutive
+       * elements, in order, the lanes joined in lane order and the waves in wave order, and the owner of the segment
+       * puts the stretch's value on the proper side of what it holds -- index order still, another association, as
+       * for the segments that teams of lanes fold (below).  Whether a chunk has such a stretch travels with the
+       * barrier that every chunk has anyway. */
+      const bool wide = p1 - p0 >= ACC_WIDE;
+      const bool wide_in_wave = __ballot(wide) != 0;
+      if (acc_lane() == 0) s_wide[tid >> 6] = wide_in_wave ? 1 : 0;
       __syncthreads();
       /* the next chunk's loads (and the gathers behind them) travel while this one is folded */
       if (q + 1 < nchunks) stage(chunk_start(q + 1));
 
+      bool any_wide = false;
+#pragma unroll
+      for (int w = 0; w < ACC_BLOCK / ACC_WAVE; ++w) any_wide = any_wide || s_wide[w] != 0;
+      if (any_wide) {                                              /* the same in every lane */
+        bool pending = wide;
+        for (;;) {
+          if (pending) (void)__hip_atomic_fetch_min(&s_owner, tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);   /* the owners take their turns in lane order */
+          __syncthreads();
+          const int owner = s_owner;
+          if (owner >= ACC_BLOCK) break;                           /* nobody left */
+          if (tid == owner) { s_from = p0; s_to = p1; }
+          __syncthreads();
+          const int from = s_from, to = s_to;
+          const int per = (to - from + ACC_BLOCK - 1) / ACC_BLOCK;
+          const int i0 = acc_min(from + tid * per, to), i1 = acc_min(i0 + per, to);
+          acc_opt<T> m = acc_none<T>();
+          for (int i = i0; i < i1; ++i) m = lf(m, acc_some(s_val[ACC_PAD(i)]));
+          m = acc_wave_reduce(m, lf);
+          if (acc_lane() == 0) s_part[tid >> 6] = m;
+          if (tid == owner) s_owner = ACC_BLOCK;
+          __syncthreads();
+          if (tid == owner) {
+            acc_opt<T> whole = s_part[0];
+#pragma unroll
+            for (int w = 1; w < ACC_BLOCK / ACC_WAVE; ++w) whole = lf(whole, s_part[w]);
+#if ACC_FOLD_RIGHT
+            acc = have ? f(whole.v, acc) : whole.v;
+#else
+            acc = have ? f(acc, whole.v) : whole.v;
+#endif
+            have = true;
+            p0 = p1;                                               /* nothing left of it for the lane alone */
+            pending = false;
+          }
+        }
+      }
+
       /* fold this lane's segment, as far as it lies in the chunk, in index order */
-      int p0 = (int)(acc_max(a, cs) - cs), p1 = (int)(acc_min(b, ce) - cs);
 #if ACC_FOLD_RIGHT
       if (!have && p0 < p1) { --p1; acc = s_val[ACC_PAD(p1)]; have = true; }
       for (; p1 - ACC_EAT >= p0; p1 -= ACC_EAT) {

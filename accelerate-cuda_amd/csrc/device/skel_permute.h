@@ -41,6 +41,10 @@
 #define ACC_TILE (ACC_BLOCK * ACC_VEC * ACC_UNROLL)
 
 #if ACC_PERMUTE_LOCKED
+/* a value and whether a run of equal targets begins at its lane: the inclusive scan of such pairs under
+ * (a, b) -> b begins a run ? b : a (+) b  leaves in every lane the combination of its run up to that lane */
+template <typename T> struct acc_run { T v; int head; };
+#define ACC_DPP_WAVE_SHL1_ 0x130
 /* An element no atomic instruction covers -- a tuple, or a scalar of another
  * size than 4 or 8 bytes -- is updated under a lock per target, which is how
  * the reference updates everything (IndexSpace.hs:285-303): locks[j] is 0 when
@@ -105,13 +109,38 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, int *__restrict__ loc
     if (!done) acc_report(acc_status, ACC_STATUS_PERMUTE_LOCK);      /* never in a healthy run: a lock that did not open; the update is lost */
   };
 
+  /* Sorted or clustered sources send runs of consecutive elements to one target, and the lanes of a wave hold
+   * consecutive elements: a whole run would queue at that target's lock (16 M sorted keys into 4096 targets: 7.6 ms
+   * against 90 us for keys in random order).  Where a wave has such runs, each is combined first -- the scan of
+   * (value, run begins here) pairs above -- and its last lane alone goes on to the lock, with the run's value. */
+  const int lane = acc_lane();
+  auto join_runs = [&](const Int64 j, T &x, bool &active) {
+    const Int64 j_before = acc_dpp<ACC_DPP_WAVE_SHR1, 0xf>(j, j);
+    const int active_before = acc_dpp<ACC_DPP_WAVE_SHR1, 0xf>((int)active, (int)active);
+    const bool continues = lane > 0 && active && active_before != 0 && j_before == j;
+    if (__ballot(continues) == 0) return;                              /* the same in every lane */
+    acc_run<T> r;
+    r.v = x;
+    r.head = continues ? 0 : 1;
+    r = acc_wave_scan(r, [&](const acc_run<T> &a, const acc_run<T> &b) -> acc_run<T> {
+          acc_run<T> c;
+          c.v = b.head ? b.v : f(a.v, b.v);
+          c.head = a.head | b.head;
+          return c;
+        }, lane);
+    const int next_continues = acc_dpp<ACC_DPP_WAVE_SHL1_, 0xf>((int)continues, (int)continues);
+    x = r.v;
+    active = active && (lane == ACC_WAVE - 1 || next_continues == 0);  /* the last lane of its run */
+  };
+
   if (lds_bins <= 0) {
     for (Int64 ix0 = (Int64)blockIdx.x * ACC_BLOCK; ix0 < n; ix0 += (Int64)gridDim.x * ACC_BLOCK) {
       const Int64 ix = ix0 + threadIdx.x;
       const Int64 j = ix < n ? perm(ix) : -1;
-      const bool active = j >= 0 && j < ntarget;        /* else `ignore`, or outside the result */
+      bool active = j >= 0 && j < ntarget;              /* else `ignore`, or outside the result */
       T x = T();
       if (active) x = get(ix);
+      join_runs(j, x, active);
       update_global(j, x, active);
     }
     return;
@@ -128,9 +157,10 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, int *__restrict__ loc
   for (Int64 ix0 = (Int64)(blockIdx.x % win_blocks) * ACC_BLOCK; ix0 < n; ix0 += (Int64)win_blocks * ACC_BLOCK) {
     const Int64 ix = ix0 + threadIdx.x;
     const Int64 j = ix < n ? perm(ix) - first : -1;
-    const bool active = j >= 0 && j < past - first;
+    bool active = j >= 0 && j < past - first;
     T x = T();
     if (active) x = get(ix);
+    join_runs(j, x, active);
     bool done = !active;
     /* whoever holds an LDS lock frees it within the same trip, so every trip makes progress somewhere */
     while (__ballot(!done) != 0) {
@@ -188,6 +218,9 @@ permute_join(ACC_ENV_PARAMS ACC_OUT_PARAMS, const ACC_ELT *__restrict__ dump_val
 }
 #else /* atomics */
 
+#ifndef ACC_RUNS
+#define ACC_RUNS 1
+#endif
 #define ACC_HINT_GENERIC 0
 #define ACC_HINT_ADD 1
 #define ACC_HINT_MIN 2
@@ -492,9 +525,22 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
     }
 #else
 #pragma unroll
-    for (int u = 0; u < ACC_UNROLL; ++u)
+    for (int u = 0; u < ACC_UNROLL; ++u) {
+      /* a lane's ACC_VEC consecutive elements on ONE target (sorted or clustered sources, flat areas of an image):
+       * combined first, one update instead of ACC_VEC on the same address */
+      bool one_target = ACC_RUNS && ACC_VEC > 1;
 #pragma unroll
-      for (int k = 0; k < ACC_VEC; ++k) update(j[u][k], x[u][k]);
+      for (int k = 1; k < ACC_VEC; ++k) one_target = one_target && j[u][k] == j[u][0];
+      if (one_target) {
+        T all = x[u][0];
+#pragma unroll
+        for (int k = 1; k < ACC_VEC; ++k) all = f(all, x[u][k]);
+        update(j[u][0], all);
+      } else {
+#pragma unroll
+        for (int k = 0; k < ACC_VEC; ++k) update(j[u][k], x[u][k]);
+      }
+    }
 #endif
 #pragma unroll
     for (int u = 0; u < ACC_UNROLL; ++u)

@@ -6,6 +6,8 @@ import sys
 import numpy as np
 import pytest
 
+import pyref
+
 pytestmark = pytest.mark.gpu
 
 TYPES = [("Int8", np.int8), ("Word16", np.uint16), ("Int32", np.int32), ("Int64", np.int64), ("float", np.float32),
@@ -155,3 +157,96 @@ def test_random_segmented_and_innermost_folds(A, ctx):
             assert np.array_equal(got[:rows], (1 + x.astype(np.int64).sum(axis=1)).astype(T)) and np.all(got[rows:] == 55)
         seg.destroy()
         rows_.destroy()
+
+
+def test_segments_of_very_unequal_length(A, ctx):
+    """the driver picks the kernel by the average length: among many short segments a few very long ones land on the
+    kernel that gives every segment a lane, which folds their long stretches with the whole workgroup.  Integer sums
+    are exact whatever the association; a non-commutative operator checks the order."""
+    rng = np.random.default_rng(77)
+    I32 = (1, "Int32")
+    fs = ctx.skeleton(A.SKEL_FOLDSEG, "Int32", env=[I32], out_rank=1, get="arrIn0_0[ix]", combine="x + y", seed="5")
+    aff = """
+__device__ __forceinline__ Word32 affine16(Word32 x, Word32 y) {
+  Word32 a1 = x >> 16, b1 = x & 0xffffu, a2 = y >> 16, b2 = y & 0xffffu;
+  return (((a1 * a2) & 0xffffu) << 16) | ((a1 * b2 + b1) & 0xffffu);
+}
+"""
+    f1 = ctx.skeleton(A.SKEL_FOLD1SEG, "Word32", env=[(1, "Word32")], out_rank=1, get="arrIn0_0[ix]", combine="affine16(x, y)", preamble=aff)
+    fr = ctx.skeleton(A.SKEL_FOLDSEG, "Word32", env=[(1, "Word32")], out_rank=1, get="arrIn0_0[ix]", combine="affine16(x, y)", seed="0x00030005u",
+                      preamble=aff, flags=A.FLAG_FOLD_RIGHT)
+    for nseg, mean, longs in ((1000, 3, [(500, 100000)]), (5000, 1, [(0, 3000), (4999, 70001)]), (300, 20, [(7, 255), (8, 256), (9, 257), (200, 5000)]),
+                              (2048, 2, [(k, 300 + k) for k in range(250, 262)]), (100000, 4, [(50000, 1 << 20)])):
+        lens = rng.poisson(mean, nseg).astype(np.int64)
+        for at, ln in longs:
+            lens[at] = ln
+        offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        n = int(offs[-1])
+        say("segments of very unequal length: nseg", nseg, "n", n, "longs", longs[:3])
+        x = rng.integers(-9, 9, n).astype(np.int32)
+        out = ctx.empty(nseg, np.int32)
+        fs.foldseg([ctx.array(x)], n, ctx.array(offs), out)
+        want = np.add.reduceat(np.concatenate([x, [0]]).astype(np.int64), offs[:-1])
+        want[lens == 0] = 0
+        assert np.array_equal(out.get(), (want + 5).astype(np.int32))
+        # composition of affine maps on 16-bit pairs: associative, not commutative -- the order must be the index order
+        u = rng.integers(0, 2**32, n, dtype=np.uint64).astype(np.uint32)
+
+        def chain(seg, right_seed=None):
+            vals = [int(v) for v in seg] + ([right_seed] if right_seed is not None else [])
+            acc = vals[0]
+            for v in vals[1:]:
+                acc = pyref.affine16(acc, v)
+            return acc
+        out1 = ctx.empty(nseg, np.uint32)
+        f1.foldseg([ctx.array(u)], n, ctx.array(offs), out1)
+        got = out1.get()
+        picks = list(range(0, nseg, max(1, nseg // 40))) + [at for at, _ in longs]
+        for s_ in picks:
+            if lens[s_] > 0:
+                assert int(got[s_]) == chain(u[offs[s_]:offs[s_ + 1]]), ("fold1Seg", s_, int(lens[s_]))
+        outr = ctx.empty(nseg, np.uint32)
+        fr.foldseg([ctx.array(u)], n, ctx.array(offs), outr)
+        gotr = outr.get()
+        for s_ in picks:
+            assert int(gotr[s_]) == chain(u[offs[s_]:offs[s_ + 1]], 0x00030005), ("foldSeg right", s_, int(lens[s_]))
+
+
+def test_permute_of_sorted_and_clustered_keys(A, ctx):
+    """runs of consecutive elements with one target: the kernels that update under a lock combine each run in its wave
+    first (any combining function, floating-point addition on few targets, tuples); integer-valued sources, so every
+    sum is exact"""
+    rng = np.random.default_rng(78)
+    I32 = (1, "Int32")
+    generic = ctx.skeleton(A.SKEL_PERMUTE, "Int32", env=[I32, I32], out_rank=1, get="arrIn1_0[ix]", combine="x + y",
+                           permutation="arrIn0_0[ix]", combine_hint=A.COMBINE_GENERIC)
+    fadd = ctx.skeleton(A.SKEL_PERMUTE, "float", env=[I32, (1, "float")], out_rank=1, get="arrIn1_0[ix]", combine="x + y",
+                        permutation="arrIn0_0[ix]", combine_hint=A.COMBINE_ADD)
+    pair = ctx.skeleton(A.SKEL_PERMUTE, "Int32, Int32", env=[I32, I32], out_rank=1, get="acc_elt{arrIn1_0[ix], 1}",
+                        combine="acc_elt{x.a1 + y.a1, x.a0 + y.a0}", permutation="arrIn0_0[ix]")
+    for n, bins, how in ((100000, 7, "sorted"), (300001, 1000, "sorted"), (300001, 1000, "runs"), (200000, 5000, "runs with gaps"),
+                         (65, 3, "sorted"), (1 << 20, 200000, "sorted")):
+        if how == "sorted":
+            keys = np.sort(rng.integers(0, bins, n))
+        else:
+            keys = np.repeat(rng.integers(0, bins, n // 37 + 1), 37)[:n]
+        keys = keys.astype(np.int32)
+        if how == "runs with gaps":
+            keys[rng.random(n) < 0.1] = -1                       # ignored elements inside the runs
+        w = rng.integers(-5, 6, n).astype(np.int32)
+        say("permute of", how, "keys: n", n, "targets", bins)
+        valid = keys >= 0
+        want = np.bincount(keys[valid], weights=w[valid], minlength=bins).astype(np.int64)
+        count = np.bincount(keys[valid], minlength=bins)
+        dk, dw = ctx.array(keys), ctx.array(w)
+        out = ctx.empty(bins, np.int32)
+        generic.permute([dk, dw], n, ctx.array(np.full(bins, 3, np.int32)), out)
+        assert np.array_equal(out.get(), want + 3), ("generic", how, n, bins)
+        outf = ctx.empty(bins, np.float32)
+        fadd.permute([dk, ctx.array(w.astype(np.float32))], n, ctx.array(np.zeros(bins, np.float32)), outf)
+        assert np.array_equal(outf.get(), want.astype(np.float32)), ("float add", how, n, bins)
+        outp = ctx.empty_tuple(bins, [np.int32, np.int32])
+        zero = ctx.empty_tuple(bins, [np.int32, np.int32])
+        zero.comps[0].set(np.zeros(bins, np.int32)); zero.comps[1].set(np.zeros(bins, np.int32))
+        pair.permute([dk, dw], n, zero, outp)
+        assert np.array_equal(outp.comps[0].get(), want) and np.array_equal(outp.comps[1].get(), count), ("pairs", how, n, bins)
