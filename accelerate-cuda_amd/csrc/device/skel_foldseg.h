@@ -187,16 +187,19 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
        * puts the stretch's value on the proper side of what it holds -- index order still, another association, as
        * for the segments that teams of lanes fold (below).  Whether a chunk has such a stretch travels with the
        * barrier that every chunk has anyway. */
-      const bool wide = p1 - p0 >= ACC_WIDE;
-      const bool wide_in_wave = __ballot(wide) != 0;
-      if (acc_lane() == 0) s_wide[tid >> 6] = wide_in_wave ? 1 : 0;
+      constexpr bool wide_stretches = ACC_WIDE <= ACC_CHUNK;      /* (a larger ACC_WIDE switches all of this off) */
+      const bool wide = wide_stretches && p1 - p0 >= ACC_WIDE;
+      if (wide_stretches) {
+        const bool wide_in_wave = __ballot(wide) != 0;
+        if (acc_lane() == 0) s_wide[tid >> 6] = wide_in_wave ? 1 : 0;
+      }
       __syncthreads();
       /* the next chunk's loads (and the gathers behind them) travel while this one is folded */
       if (q + 1 < nchunks) stage(chunk_start(q + 1));
 
       bool any_wide = false;
 #pragma unroll
-      for (int w = 0; w < ACC_BLOCK / ACC_WAVE; ++w) any_wide = any_wide || s_wide[w] != 0;
+      for (int w = 0; w < ACC_BLOCK / ACC_WAVE; ++w) any_wide = any_wide || (wide_stretches && s_wide[w] != 0);
       if (any_wide) {                                              /* the same in every lane */
         bool pending = wide;
         for (;;) {
