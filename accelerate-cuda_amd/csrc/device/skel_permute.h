@@ -421,9 +421,9 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
    * no count was touched */
   /* (Without a branch, so that the additions of a batch are issued one behind the other and waited for together:
    * a lane with nothing to add adds 0 to a word of its own.) */
-  auto narrow_add = [&](const U t, const T &x) -> unsigned {
+  auto narrow_add = [&](const U t, const T &x, const unsigned most) -> unsigned {
     const UT ux = (UT)x;
-    const bool in = t < u_bins, small = ux <= (UT)ACC_NARROW_MAX;
+    const bool in = t < u_bins, small = ux <= (UT)most;
     if (in && !small) acc_hint_apply<ACC_SCOPE_DEVICE>(arrOut_0 + t, x, f);
     const bool take = in && small;
     const unsigned sh = narrow_shift(t);
@@ -463,7 +463,7 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
    * instruction, not a branch */
   auto update = [&](const U t, const T &x) {
 #if ACC_PERMUTE_NARROW
-    const unsigned before = narrow_add(t, x);
+    const unsigned before = narrow_add(t, x, ACC_NARROW_MAX);
     narrow_carry(t, x, before);
     narrow_wait(t, before);
 #elif ACC_PERMUTE_WINDOWS
@@ -508,17 +508,34 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
 #pragma unroll
     for (int u = 0; u < ACC_UNROLL; ++u) {           /* ACC_VEC additions, then their corrections, then the waits */
       unsigned before[ACC_VEC];
+      T added[ACC_VEC];
+      /* a lane's ACC_VEC consecutive elements on ONE target (sorted or clustered sources), each a small addend: one
+       * addition of their sum -- no more than the lane would have had in flight anyway, so the bound above holds */
+      bool one_target = ACC_RUNS && ACC_VEC > 1;
 #pragma unroll
-      for (int k = 0; k < ACC_VEC; ++k) before[k] = narrow_add(j[u][k], x[u][k]);
-      /* ONE test for the batch: a correction or a wait takes a count of ACC_NARROW_HALF - ACC_NARROW_MAX or more, and
+      for (int k = 0; k < ACC_VEC; ++k)
+        one_target = one_target && j[u][k] == j[u][0] && (UT)x[u][k] <= (UT)ACC_NARROW_MAX;
+      if (one_target) {
+        T all = x[u][0];
+#pragma unroll
+        for (int k = 1; k < ACC_VEC; ++k) all = (T)(all + x[u][k]);
+        before[0] = narrow_add(j[u][0], all, ACC_NARROW_MAX * ACC_VEC);
+        added[0] = all;
+#pragma unroll
+        for (int k = 1; k < ACC_VEC; ++k) { before[k] = 0u; added[k] = T(0); }
+      } else {
+#pragma unroll
+        for (int k = 0; k < ACC_VEC; ++k) { before[k] = narrow_add(j[u][k], x[u][k], ACC_NARROW_MAX); added[k] = x[u][k]; }
+      }
+      /* ONE test for the batch: a correction or a wait takes a count within an addend of ACC_NARROW_HALF or more, and
        * nearly no batch has one (a test and a branch per addition, skipped or not, were a third of the loop's
        * instructions; 2^26 Zipf keys into 65 536 targets: 54.2 -> 53.7 us) */
       unsigned top = before[0];
 #pragma unroll
       for (int k = 1; k < ACC_VEC; ++k) top = acc_max(top, before[k]);
-      if (top >= ACC_NARROW_HALF - ACC_NARROW_MAX) {
+      if (top >= ACC_NARROW_HALF - ACC_NARROW_MAX * ACC_VEC) {
 #pragma unroll
-        for (int k = 0; k < ACC_VEC; ++k) narrow_carry(j[u][k], x[u][k], before[k]);
+        for (int k = 0; k < ACC_VEC; ++k) narrow_carry(j[u][k], added[k], before[k]);
 #pragma unroll
         for (int k = 0; k < ACC_VEC; ++k) narrow_wait(j[u][k], before[k]);
       }

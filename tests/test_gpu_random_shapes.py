@@ -250,3 +250,20 @@ def test_permute_of_sorted_and_clustered_keys(A, ctx):
         zero.comps[0].set(np.zeros(bins, np.int32)); zero.comps[1].set(np.zeros(bins, np.int32))
         pair.permute([dk, dw], n, zero, outp)
         assert np.array_equal(outp.comps[0].get(), want) and np.array_equal(outp.comps[1].get(), count), ("pairs", how, n, bins)
+    # counting into more targets than whole counts have room for in LDS (16-bit counts): sorted keys, runs of one key
+    # long enough to take a count past its half-way mark many times over, and runs of 37
+    count = ctx.skeleton(A.SKEL_PERMUTE, "Int32", env=[I32], out_rank=1, get="1", combine="x + y", permutation="arrIn0_0[ix]",
+                         combine_hint=A.COMBINE_ADD)
+    for n, bins, how in ((1 << 22, 65536, "sorted"), (1 << 22, 40000, "one key"), (1 << 21, 50001, "runs")):
+        if how == "sorted":
+            keys = np.sort(rng.integers(0, bins, n))
+        elif how == "one key":
+            keys = np.full(n, 12345)
+            keys[::1000] = rng.integers(0, bins, keys[::1000].size)
+        else:
+            keys = np.repeat(rng.integers(0, bins, n // 37 + 1), 37)[:n]
+        keys = keys.astype(np.int32)
+        say("counting", how, "keys: n", n, "targets", bins)
+        out = ctx.empty(bins, np.int32)
+        count.permute([ctx.array(keys)], n, ctx.array(np.full(bins, 2, np.int32)), out)
+        assert np.array_equal(out.get(), np.bincount(keys, minlength=bins) + 2), ("count", how, n, bins)
