@@ -74,11 +74,15 @@ static_assert(ACC_CHUNK % (ACC_BLOCK * ACC_VEC) == 0, "chunk must be a whole num
 
 #define ACC_LOADS (ACC_CHUNK / (ACC_BLOCK * ACC_VEC))   /* vector loads per lane and chunk */
 /* One word of padding per 32 elements of the staged chunk: lanes that fold segments whose starts are a multiple
- * of 32 elements apart (every segment 32, 64, 128 ... long) would otherwise all read the same LDS bank.       */
+ * of 32 elements apart (every segment 32, 64, 128 ... long) would otherwise all read the same LDS bank.  The padding
+ * moves that worst case to starts 31, 62, 93 ... apart, so rows of ONE length (ACC_SEG_UNIFORM, where the length is
+ * known) are padded only if the length is a multiple of 8: 2^25 Float32 in rows of 31 / 62 / 124 54 -> 25 / 31 / 34 us,
+ * rows of 32 / 64 / 96 stay at 25 / 29 / 31 (68 / 67 / 76 without).                                              */
 #ifndef ACC_PAD_ON
 #define ACC_PAD_ON 1                                     /* 0: for measuring what the padding is worth */
 #endif
-#define ACC_PAD(i) (ACC_PAD_ON ? ((i) + ((i) >> 5)) : (i))
+#define ACC_PAD_SPACE(i) (ACC_PAD_ON ? ((i) + ((i) >> 5)) : (i))
+#define ACC_PAD(i) ((i) + (((i) >> 5) & acc_pad_mask))
 #define ACC_EAT 8                                        /* LDS reads kept in flight while folding */
 #ifndef ACC_WIDE
 #define ACC_WIDE 256                                     /* elements of one segment in a chunk from which the workgroup folds them together */
@@ -92,7 +96,7 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
   ACC_GUARD_CHECK
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
-  __shared__ __attribute__((aligned(16))) T s_val[ACC_PAD(ACC_CHUNK)];
+  __shared__ __attribute__((aligned(16))) T s_val[ACC_PAD_SPACE(ACC_CHUNK)];
   /* for the stretches the whole workgroup folds (below) */
   __shared__ int s_wide[ACC_BLOCK / ACC_WAVE];
   __shared__ int s_owner, s_from, s_to;
@@ -109,6 +113,10 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
   const T seed = (ACC_SEED);
 #endif
   if (tid == 0) s_owner = ACC_BLOCK;
+  /* (the loop over this workgroup's blocks of segments, compiled with and without the padding: an address that adds
+   * the padding under a run-time mask costs the inner loop more than the bank conflicts it avoids) */
+  auto blocks_of_segments = [&](auto padded_c) {
+  constexpr int acc_pad_mask = decltype(padded_c)::value ? ~0 : 0;
   /* (seen by all at the first barrier of the first chunk) */
 
   for (Int64 first = (Int64)blockIdx.x * ACC_BLOCK; first < nseg; first += (Int64)gridDim.x * ACC_BLOCK) {
@@ -266,6 +274,13 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
 #endif
     }
   }
+  };   /* blocks_of_segments */
+#if ACC_SEG_UNIFORM && ACC_PAD_ON
+  if (shIn_0 % 8 == 0) blocks_of_segments(acc_bool<true>());
+  else                 blocks_of_segments(acc_bool<false>());
+#else
+  blocks_of_segments(acc_bool<ACC_PAD_ON != 0>());
+#endif
 }
 
 #if ACC_SEG_UNIFORM
