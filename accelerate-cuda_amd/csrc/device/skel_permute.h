@@ -134,7 +134,13 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, int *__restrict__ loc
   };
 
   if (lds_bins <= 0) {
-    for (Int64 ix0 = (Int64)blockIdx.x * ACC_BLOCK; ix0 < n; ix0 += (Int64)gridDim.x * ACC_BLOCK) {
+    /* every workgroup a stretch of the source of its own, not every gridDim.x-th block of it: under a sorted or
+     * clustered source the workgroups that run at one time then work on targets far apart, instead of all on the
+     * locks of one neighbourhood -- a few cache lines, whose atomics queue (16 M sorted keys into 300 000 targets:
+     * 6.6 ms against 1.4 for keys in random order) */
+    const Int64 rounds = (n + ACC_BLOCK - 1) / ACC_BLOCK;
+    const Int64 mine_first = rounds * (Int64)blockIdx.x / gridDim.x, mine_past = rounds * ((Int64)blockIdx.x + 1) / gridDim.x;
+    for (Int64 ix0 = mine_first * ACC_BLOCK; ix0 < mine_past * ACC_BLOCK; ix0 += ACC_BLOCK) {
       const Int64 ix = ix0 + threadIdx.x;
       const Int64 j = ix < n ? perm(ix) : -1;
       bool active = j >= 0 && j < ntarget;              /* else `ignore`, or outside the result */
