@@ -854,7 +854,11 @@ int acc_skel_preview(const acc_skel_desc *desc, int variant, const char **source
   if (!source || variant < 0 || variant > 7) return fail(ACC_ERR_INVALID, "acc_skel_preview: bad argument");
   acc::SkelSpec sp;
   ACC_TRY(acc::make_spec(desc, &sp));
-  if (variant > 1 && sp.kind != ACC_SKEL_PERMUTE) return fail(ACC_ERR_INVALID, "acc_skel_preview: only a permute has variants beyond 1");
+  // beyond 1: a permute's forms (to 7), a stencil's fewer columns a lane (to 5), a scan's small tiles and a segmented
+  // fold's longer chunk (2 and 3)
+  const bool stencil = sp.kind == ACC_SKEL_STENCIL || sp.kind == ACC_SKEL_STENCIL2;
+  const int most = sp.kind == ACC_SKEL_PERMUTE ? 7 : (stencil ? 5 : ((sp.scan_small_rows > 0 || sp.chunk_long > 0) ? 3 : 1));
+  if (variant > most) return fail(ACC_ERR_INVALID, "acc_skel_preview: this kind of skeleton has variants 0 to %d", most);
   ACC_TRY(acc::generate_source(acc::spec_of_variant(sp, variant), (variant & 1) == 0, &name, &text));
   *source = text.c_str();
   if (entry) *entry = name.c_str();

@@ -83,6 +83,38 @@ def test_permute_variants_the_driver_chooses_between_all_compile(A, tmp_path):
             assert A.compile_source(src) > 4000, v
 
 
+def test_variants_by_shape_of_scans_stencils_and_maps_compile(A, tmp_path):
+    """what the drivers take by the shape of a call: small tiles for scans of small arrays (+2), half and a quarter of
+    the columns a lane for stencils on narrow arrays (+2, +4; two columns a lane of 8-byte elements to begin with), tiles
+    for a map that reads across the rows of its source (ACC_FLAG_TILED, rank 2 or more only)"""
+    A.lib().acc_cache_set_dir(str(tmp_path).encode())
+    scan = A.make_desc(A.SKEL_SCANL, "Int32", env=[(1, "Int32")], get="arrIn0_0[ix]", combine="x + y", seed="0")
+    rows = {}
+    for v in (0, 1, 2, 3):
+        name, src = A.preview(scan, v)
+        assert name == "scanl" and A.compile_source(src) > 4000, v
+        rows[v] = int([l for l in src.splitlines() if l.startswith("#define ACC_ROWS ")][0].split()[-1])
+    assert rows[0] == rows[1] == 32 and rows[2] == rows[3] == 4
+    seven = [(0, 0, 0), (-1, 0, 0), (1, 0, 0), (0, -1, 0), (0, 1, 0), (0, 0, -1), (0, 0, 1)]
+    nine = [(dy, dx) for dy in (-1, 0, 1) for dx in (-1, 0, 1)]
+    for ctype, rank, taps, svecs in (("float", 2, nine, (4, 2, 1)), ("float", 3, seven, (4, 2, 1)), ("double", 3, seven, (2, 1, 1))):
+        st = A.make_desc(A.SKEL_STENCIL, ctype, out_rank=rank, taps=taps, boundary="mirror",
+                         stencil_fn=" + ".join("t%d" % k for k in range(len(taps))))
+        for k, want in enumerate(svecs):
+            for v in (2 * k, 2 * k + 1):
+                name, src = A.preview(st, v)
+                assert "#define ACC_SVEC %d\n" % want in src, (ctype, rank, v)
+                assert A.compile_source(src) > 4000, (ctype, rank, v)
+    wide = A.make_desc(A.SKEL_STENCIL, "float", out_rank=2, taps=[(0, -4), (0, 0), (0, 4)], boundary="clamp", stencil_fn="t0 + t1 + t2")
+    assert "#define ACC_SVEC 4\n" in A.preview(wide, 0)[1]
+    tr = "arrIn0_0[(ix % shOut_0) * shIn0_0 + (ix / shOut_0)]"
+    tiled = A.make_desc(A.SKEL_MAP, "float", env=[(2, "float")], out_rank=2, get=tr, flags=A.FLAG_TILED)
+    name, src = A.preview(tiled, 0)
+    assert name == "map" and "#define ACC_MAP_TILED 1" in src and A.compile_source(src) > 2000
+    vector = A.make_desc(A.SKEL_MAP, "float", env=[(1, "float")], out_rank=1, get="arrIn0_0[ix]", flags=A.FLAG_TILED)
+    assert "#define ACC_MAP_TILED 0" in A.preview(vector, 0)[1]
+
+
 def test_every_scalar_primitive_compiles_for_every_type(A, tmp_path):
     """acc_prim.h: one map per element type naming every primitive that type has
     (CodeGen.hs:406-476); what they compute is checked on the GPU"""
