@@ -95,6 +95,13 @@ def test_variants_by_shape_of_scans_stencils_and_maps_compile(A, tmp_path):
         assert name == "scanl" and A.compile_source(src) > 4000, v
         rows[v] = int([l for l in src.splitlines() if l.startswith("#define ACC_ROWS ")][0].split()[-1])
     assert rows[0] == rows[1] == 32 and rows[2] == rows[3] == 4
+    seg = A.make_desc(A.SKEL_FOLDSEG, "float", env=[(1, "float")], out_rank=1, get="arrIn0_0[ix]", combine="x + y", seed="0.0f")
+    chunks = {}
+    for v in (0, 2, 3):                                            # a longer staged chunk for segments of 8 elements or more
+        name, src = A.preview(seg, v)
+        assert name == "foldSeg" and A.compile_source(src) > 4000, v
+        chunks[v] = int([l for l in src.splitlines() if l.startswith("#define ACC_CHUNK ")][0].split()[-1])
+    assert chunks[2] == chunks[3] > chunks[0]
     seven = [(0, 0, 0), (-1, 0, 0), (1, 0, 0), (0, -1, 0), (0, 1, 0), (0, 0, -1), (0, 0, 1)]
     nine = [(dy, dx) for dy in (-1, 0, 1) for dx in (-1, 0, 1)]
     for ctype, rank, taps, svecs in (("float", 2, nine, (4, 2, 1)), ("float", 3, seven, (4, 2, 1)), ("double", 3, seven, (2, 1, 1))):
