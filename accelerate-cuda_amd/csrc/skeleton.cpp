@@ -237,9 +237,9 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
         *entry = sp.has_seed ? "fold" : "fold1";
         o << "#define ACC_SEG_UNIFORM 1\n";
         o << "#define ACC_TROUNDS " << tune("foldseg.team_rounds", 3) << "\n";
-      if (tuned("foldseg.pad")) o << "#define ACC_PAD_ON " << (tune("foldseg.pad", 1) ? 1 : 0) << "\n";
         if (tuned("foldseg.pad")) o << "#define ACC_PAD_ON " << (tune("foldseg.pad", 1) ? 1 : 0) << "\n";
         if (tuned("foldseg.wide")) o << "#define ACC_WIDE " << std::max(1, tune("foldseg.wide", 256)) << "\n";
+        if (tuned("foldseg.ahead")) o << "#define ACC_AHEAD " << std::max(1, std::min(2, tune("foldseg.ahead", 1))) << "\n";
         o << "#define ACC_FOLD_RIGHT " << ((sp.flags & ACC_FLAG_FOLD_RIGHT) ? 1 : 0) << "\n";
         o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_CHUNK " << sp.chunk << "\n";
         tmpl = "skel_foldseg.h";
@@ -257,6 +257,8 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       if (sp.out_rank >= 2) o << "#define ACC_SEG_OUTER 1\n";      // the segments of every outer row: Reduction.hs:473-474
       o << "#define ACC_TROUNDS " << tune("foldseg.team_rounds", 3) << "\n";
       if (tuned("foldseg.pad")) o << "#define ACC_PAD_ON " << (tune("foldseg.pad", 1) ? 1 : 0) << "\n";
+      if (tuned("foldseg.wide")) o << "#define ACC_WIDE " << std::max(1, tune("foldseg.wide", 256)) << "\n";
+      if (tuned("foldseg.ahead")) o << "#define ACC_AHEAD " << std::max(1, std::min(2, tune("foldseg.ahead", 1))) << "\n";
       o << "#define ACC_FOLD_RIGHT " << ((sp.flags & ACC_FLAG_FOLD_RIGHT) ? 1 : 0) << "\n";
       o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_CHUNK " << sp.chunk << "\n";
       tmpl = "skel_foldseg.h";
