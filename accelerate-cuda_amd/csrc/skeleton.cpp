@@ -239,7 +239,6 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
         o << "#define ACC_TROUNDS " << tune("foldseg.team_rounds", 3) << "\n";
         if (tuned("foldseg.pad")) o << "#define ACC_PAD_ON " << (tune("foldseg.pad", 1) ? 1 : 0) << "\n";
         if (tuned("foldseg.wide")) o << "#define ACC_WIDE " << std::max(1, tune("foldseg.wide", 256)) << "\n";
-        if (tuned("foldseg.ahead")) o << "#define ACC_AHEAD " << std::max(1, std::min(2, tune("foldseg.ahead", 1))) << "\n";
         o << "#define ACC_FOLD_RIGHT " << ((sp.flags & ACC_FLAG_FOLD_RIGHT) ? 1 : 0) << "\n";
         o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_CHUNK " << sp.chunk << "\n";
         tmpl = "skel_foldseg.h";
@@ -258,7 +257,6 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "#define ACC_TROUNDS " << tune("foldseg.team_rounds", 3) << "\n";
       if (tuned("foldseg.pad")) o << "#define ACC_PAD_ON " << (tune("foldseg.pad", 1) ? 1 : 0) << "\n";
       if (tuned("foldseg.wide")) o << "#define ACC_WIDE " << std::max(1, tune("foldseg.wide", 256)) << "\n";
-      if (tuned("foldseg.ahead")) o << "#define ACC_AHEAD " << std::max(1, std::min(2, tune("foldseg.ahead", 1))) << "\n";
       o << "#define ACC_FOLD_RIGHT " << ((sp.flags & ACC_FLAG_FOLD_RIGHT) ? 1 : 0) << "\n";
       o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_CHUNK " << sp.chunk << "\n";
       tmpl = "skel_foldseg.h";
