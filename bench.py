@@ -53,6 +53,11 @@ class Timer(object):
         steps = step if isinstance(step, (list, tuple)) else [step]
         k = 0
         if self.last_busy is None or time.perf_counter() - self.last_busy > self.IDLE_AFTER_S:
+            # (the first call of a step may build a variant of its instance -- seconds of compilation on a machine
+            # with cold caches -- which must not count as time the device was kept busy)
+            steps[0]()
+            k += 1
+            self.ctx.sync()
             t_end = time.perf_counter() + self.DEVICE_WARMUP_MS * 1e-3
             while time.perf_counter() < t_end:
                 for _ in range(16):
@@ -147,7 +152,10 @@ def main():
     ap.add_argument("--only", type=str, default="")
     ap.add_argument("--sets", type=int, default=4, help="copies of every configuration's buffers, used round robin")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--device-warmup-ms", type=float, default=Timer.DEVICE_WARMUP_MS,
+                    help="untimed launches before the warm-up steps of a configuration that finds the device idle")
     args = ap.parse_args()
+    Timer.DEVICE_WARMUP_MS = args.device_warmup_ms
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives, no sharding)" % args.gpus)
 
