@@ -234,12 +234,6 @@ ACC_DEV void acc_report(unsigned int *status, const int word)
 #define ACC_GUARD_CHECK
 #endif
 
-/* A read of an array element that will not be needed again (a manifest input
- * consumed once, in index order).  It is marked non-temporal so that it does
- * not evict data that IS reused -- a gathered vector, a small table -- from
- * the L2.  The code generator uses it for linear reads next to indirect ones. */
-template <typename T> ACC_DEV T acc_stream(const T *p, const Int64 ix) { return __builtin_nontemporal_load(p + ix); }
-
 /* Keep a value where it was computed.  The compiler otherwise moves the tail of a long dependent chain -- load an
  * index, gather through it, multiply -- down to its first use, past whatever stands in between, so that its memory
  * round trips start only there and are waited for one after the other. */
@@ -305,6 +299,39 @@ template <typename T> ACC_DEV void acc_store_device(T *p, const T &v)
 #pragma unroll
   for (int k = 0; k < acc_piece_of<T>::COUNT; ++k)
     __hip_atomic_store((P *)p + k, b[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+/* A read of an array element that will not be needed again (a manifest input
+ * consumed once, in index order).  It is marked non-temporal so that it does
+ * not evict data that IS reused -- a gathered vector, a small table -- from
+ * the L2.  The code generator uses it for linear reads next to indirect ones. */
+#ifndef ACC_STREAM_POLICY
+#define ACC_STREAM_POLICY 1
+#endif
+template <typename T> ACC_DEV T acc_stream(const T *p, const Int64 ix)
+{
+#if ACC_STREAM_POLICY == 0
+  return p[ix];
+#elif ACC_STREAM_POLICY == 2 || ACC_STREAM_POLICY == 3
+  typedef typename acc_piece_of<T>::type P;
+  P b[acc_piece_of<T>::COUNT];
+#pragma unroll
+  for (int k = 0; k < acc_piece_of<T>::COUNT; ++k)
+    b[k] = __hip_atomic_load((const P *)(p + ix) + k, __ATOMIC_RELAXED, ACC_STREAM_POLICY == 2 ? __HIP_MEMORY_SCOPE_AGENT : __HIP_MEMORY_SCOPE_SYSTEM);
+  T v;
+  __builtin_memcpy(&v, b, sizeof(T));
+  return v;
+#elif ACC_STREAM_POLICY >= 100
+  /* (measurement only: buffer loads with the cache-policy bits ACC_STREAM_POLICY - 100: 1 sc0, 2 nt, 16 sc1; byte offsets of 32 bits) */
+  static_assert(sizeof(T) == 4, "measurement path");
+  const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void *)p, 0, 0x7fffffff, 0x00020000);
+  const int w = __builtin_amdgcn_raw_buffer_load_b32(r, (int)ix * 4, 0, ACC_STREAM_POLICY - 100);
+  T v;
+  __builtin_memcpy(&v, &w, 4);
+  return v;
+#else
+  return __builtin_nontemporal_load(p + ix);
+#endif
 }
 
 /* row-major index helpers (CodeGen/Base.hs:193-218): shapes and indices are

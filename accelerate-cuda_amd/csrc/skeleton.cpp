@@ -288,6 +288,7 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "#define ACC_PERMUTE_WINDOWS " << (sp.permute_windows ? 1 : 0) << "\n";
       o << "#define ACC_PERMUTE_NARROW " << (sp.permute_narrow ? 1 : 0) << "\n";
       if (sp.permute_narrow) o << "#define ACC_NARROW_STOP " << tune("permute.narrow_stop", 0xA000) << "u\n";
+      if (sp.permute_narrow && tuned("permute.dump_vec")) o << "#define ACC_NARROW_DUMP_VEC " << (tune("permute.dump_vec", 1) ? 1 : 0) << "\n";
       if (sp.permute_narrow && tuned("permute.merge_batch")) o << "#define ACC_MERGE_BATCH " << tune("permute.merge_batch", 16) << "\n";
       if (sp.permute_narrow) o << "#define ACC_MERGE_WAVES " << sp.merge_waves << "\n";
       if (tuned("permute.runs")) o << "#define ACC_RUNS " << tune("permute.runs", 1) << "\n";
@@ -374,6 +375,7 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
   }
   o << "#define ACC_ENTRY " << *entry << "\n";
   o << "#define ACC_NT_STORE " << tune("nt_store", 1) << "\n";
+  if (tuned("stream.policy")) o << "#define ACC_STREAM_POLICY " << tune("stream.policy", 1) << "\n";
   if (sp.guarded) o << "#define ACC_GUARDED 1\n";
   if (tuned("spin_limit")) o << "#define ACC_SPIN_LIMIT " << std::max(0, tune("spin_limit", 1 << 22)) << "\n";
   o << "#include \"acc_hip_device.h\"\n";

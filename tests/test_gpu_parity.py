@@ -472,6 +472,8 @@ def test_counting_into_a_table_of_16_bit_counts(A, ctx):
     cases = [("zipf", wl.zipf_i32(7, n, 65536), 65536), ("uniform", wl.uniform_i32(8, n, 65535), 65535),
              ("one hot target", np.full(n, 4242, np.int32), 50001),
              ("four hot targets in two words", (rng.integers(0, 4, n) + 70000).astype(np.int32), 81919)]
+    # (a table whose halves are whole 128-bit vectors but no whole number of a wave's 256 words: 65552 targets)
+    cases.append(("hot targets at the ends of the table's quarters", rng.choice(np.array([0, 16387, 16388, 32775, 32776, 49163, 49164, 65551], np.int32), n), 65552))
     strays = rng.integers(-5, 65536 + 5, 1 << 22).astype(np.int32)
     strays[::7] = -1
     cases.append(("strays and ignore", strays, 65536))
