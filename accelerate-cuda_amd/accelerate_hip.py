@@ -38,11 +38,11 @@ import acchip as A
 
 __all__ = ["Exp", "constant", "cond", "use", "unit", "map", "zipWith", "generate", "backpermute", "transpose", "reverse", "zip_", "unzip", "while_",
            "fold", "fold1", "foldSeg", "fold1Seg", "scanl", "scanl1", "scanl_", "scanr", "scanr1", "scanr_", "permute", "ignore",
-           "stencil", "stencil2", "awhile", "run", "run1", "fill", "enumFromN", "take", "drop", "init", "tail", "gather",
+           "stencil", "stencil2", "awhile", "run", "compute", "run1", "fill", "enumFromN", "take", "drop", "init", "tail", "gather",
            "scatter", "foldAll", "sum_", "product", "maximum", "minimum", "and_", "or_", "all_", "any_", "filter_", "fst", "snd", "lift", "index_if", "fromIntegral", "truncate", "round_", "floor",
            "ceiling", "idiv", "mod", "quot", "rem", "min_", "max_", "sqrt", "exp", "log", "sin", "cos", "tan", "abs_",
            "signum", "Context", "the", "runWith", "run1With", "runN", "stream", "streamWith", "Async", "wait", "poll",
-           "cancel", "Cancelled", "runAsync", "run1Async", "runAsyncWith", "run1AsyncWith", "create", "destroy",
+           "cancel", "Cancelled", "streamOut", "streamOutWith", "runAsync", "run1Async", "runAsyncWith", "run1AsyncWith", "create", "destroy",
            "unsafeFree", "unsafeFreeWith", "performGC", "performGCWith", "acond", "reshape", "flatten", "replicate", "slice_", "All",
            "imap", "zipWith3", "iterate", "asin", "acos", "atan", "sinh", "cosh", "tanh", "asinh", "acosh", "atanh", "atan2",
            "pow_", "logBase", "recip", "isNaN", "rotateL", "rotateR", "boolToInt", "ord_", "chr_", "quotRem", "divMod"]
@@ -427,6 +427,7 @@ class _Resident(object):
         self.cx, self.host, self.shape, self.dtype, self.size = cx, host, host.shape, host.dtype, host.size
         self.key = A.MemTable.key(host)
         self.stream, self.ready = None, None          # where it was produced, and the event recorded behind that
+        self.pending = None                           # the launch that will produce it, while that is put off (_Pending)
         with cx.lock:
             cx.table.malloc(host, frozen)
             cx.live[self.key] = cx.live.get(self.key, 0) + 1
@@ -434,6 +435,8 @@ class _Resident(object):
     def get(self):
         if self.cx.loop is not None:
             raise _HostReadInLoop()          # an iteration enqueued ahead cannot wait for the host
+        if self.pending is not None:
+            self.pending.force()
         if self.ready is not None:
             A.check(A.lib().acc_event_sync(self.cx.ctx.handle, self.ready))
         d = self.cx.table.acquire(self.host)
@@ -455,6 +458,42 @@ class _Resident(object):
                         cx.table.free(self.host)
         except Exception:
             pass
+
+
+def _parts(ms):
+    for m in ms:
+        if isinstance(m, A.TupleArray):
+            for c in m.comps:
+                yield c
+        elif m is not None:
+            yield m
+
+
+class _Pending(object):
+    """A skeleton launch that has been put off until its result is wanted.  The instance was created when the
+    consumer was written down -- its compilation runs on the library's worker pool from then on -- and nothing waits
+    for it before `run` (or `the`, or a loop) asks for a value that depends on it: the kernels of a program are
+    compiling side by side while the program is still being built, and execution blocks where a kernel is first used
+    (Compile.hs:451-457,484-538: the reference's compile phase forks every kernel's compilation before its execute
+    phase starts).  The results hold the node; it goes away with them if nobody ever asks."""
+
+    def __init__(self, cx, inputs, outputs, go):
+        self.cx, self.inputs, self.outputs, self.go, self.done = cx, inputs, outputs, go, False
+        for m in _parts(outputs):
+            m.pending = self
+        cx.pending.append(weakref.ref(self))
+
+    def force(self):
+        cx = self.cx
+        with cx.lock:
+            if self.done:
+                return
+            self.done = True
+            inputs, outputs, go = self.inputs, self.outputs, self.go
+            self.inputs = self.outputs = self.go = None
+            for m in _parts(outputs):
+                m.pending = None
+            cx._launch(inputs, outputs, go)
 
 
 class _HostReadInLoop(Exception):
@@ -491,6 +530,8 @@ class Context(object):
         self.streams, self.turn, self.events = [], 0, []
         self.lock = threading.RLock()      # one host thread at a time evaluates in a context (CUDA.hs:251-252)
         self.loop, self.guard = None, None # the `awhile` being enqueued ahead, if any, and the context's loop guard
+        self.pending = []                  # weak references to the launches put off so far (_Pending), oldest first
+        self.lazy = True                   # False: every consumer launches where it is written down
 
     @classmethod
     def default(cls):
@@ -527,17 +568,31 @@ class Context(object):
     def launch(self, inputs, outputs, go):
         """run `go(input views, output views, stream)` with the arrays resident (None stays None), after what
         produced the inputs; the outputs carry the event recorded behind it"""
-        with self.lock:                                  # consumers launch as they are built, from whichever thread
+        with self.lock:
+            # put off until a value is wanted, unless the launch belongs to a loop that is being enqueued ahead (its
+            # kernels go onto the loop's stream now, in order) or produces nothing to wait for
+            if self.lazy and self.loop is None and any(True for _ in _parts(outputs)):
+                _Pending(self, inputs, outputs, go)
+                return
             return self._launch(inputs, outputs, go)
 
+    def flush(self):
+        """launch everything that has been put off, oldest first (before a loop takes a stream under its guard,
+        before arrays are freed by hand, before the context goes away)"""
+        with self.lock:
+            nodes, self.pending = self.pending, []
+            for ref in nodes:
+                node = ref()
+                if node is not None:
+                    node.force()
+
     def _launch(self, inputs, outputs, go):
-        def parts(ms):
-            for m in ms:
-                if isinstance(m, A.TupleArray):
-                    for c in m.comps:
-                        yield c
-                elif m is not None:
-                    yield m
+        parts = _parts
+        for m in list(parts(inputs)):                   # what produces an operand comes first
+            if m.pending is not None:
+                m.pending.force()
+        if len(self.pending) > 256:                     # forget the nodes that are done or gone
+            self.pending = [r for r in self.pending if r() is not None and not r().done]
         asy = getattr(_running, "asy", None)
         if asy is not None and asy._cancelled:
             raise Cancelled()                           # between two skeletons: a launch already made runs to its end
@@ -992,6 +1047,7 @@ def awhile(p, f, a, context=None, limit=None, ahead=8):
     with cx.lock:
         if cx.loop is not None:
             raise _HostReadInLoop()              # a loop inside a loop: the outer one goes stepwise, this one ahead
+        cx.flush()                               # what was put off so far is not the loop's: it runs before, unguarded
         if ahead < 2:
             return _awhile_stepwise(cx, p, f, a, tup, force, limit, 0)
         stream = cx._stream_for([m for x in (a if tup else (a,)) for m in
@@ -1043,6 +1099,20 @@ def run(a, context=None):
         if isinstance(a, tuple):
             return tuple(run(x, cx) for x in a)
         return _force(a, cx).manifest.get()
+
+
+def compute(a, context=None):
+    """evaluate on the device without bringing anything to the host: every kernel the value depends on has been
+    enqueued when this returns (none has been waited for); gives the manifest array, or a tuple of them"""
+    cx = _context(context, *(a if isinstance(a, tuple) else (a,)))
+    with cx.lock:
+        if isinstance(a, tuple):
+            return tuple(compute(x, cx) for x in a)
+        m = _force(a, cx)
+        for part in _parts([m.manifest]):
+            if part.pending is not None:
+                part.pending.force()
+        return m
 
 
 def run1(f, context=None):
@@ -1155,6 +1225,19 @@ def streamWith(context, f, arrays):
     return stream(f, arrays, context)
 
 
+def streamOut(computations, context=None):
+    """the results of a sequence of array computations as a lazy sequence of host arrays: a computation is built,
+    run and collected when its element is asked for, never the whole sequence at once (the `streamOut` of
+    CUDA.hs:349-372, which the reference keeps commented out together with its `Seq` execution; here the sequence is
+    any iterable of Acc values, or of functions of no argument that build one)"""
+    for c in computations:
+        yield run(c() if callable(c) else c, context)
+
+
+def streamOutWith(context, computations):
+    return streamOut(computations, context)
+
+
 class Async(object):
     """A computation running in a host thread of its own (the `Async` of the accelerate package that CUDA.hs:194-196
     re-exports with `wait`, `poll` and `cancel`; started by `asyncBound`, CUDA.hs:263,323).  Threads of one context
@@ -1225,6 +1308,7 @@ def destroy(context):
     """release the context's kernels, streams, events and device memory (Context.hs:100-103); arrays and
     computations made in it must not be used afterwards"""
     with context.lock:
+        context.flush()
         context.ctx.sync()
         context.skeletons.clear()
         if context.guard is not None:
@@ -1242,6 +1326,7 @@ def unsafeFree(arrays, context=None):
     Unsafe as there: a computation that still refers to one of them fails when it looks the array up."""
     cx = context or Context.default()
     with cx.lock:
+        cx.flush()                               # launches put off may still want these arrays
         for h in (arrays if isinstance(arrays, (tuple, list)) else (arrays,)):
             cx.table.free(np.asarray(h, order="C"))
 

@@ -99,7 +99,8 @@ acc_skel_get_info acc_exec_map acc_exec_fold acc_exec_foldseg acc_exec_foldseg_n
 acc_exec_stencil acc_exec_stencil2 acc_exec_stencil_iterate acc_guard_create acc_guard_destroy acc_guard_reset
 acc_guard_latch acc_guard_read acc_stream_set_guard acc_trace_start acc_trace_stop acc_memtable_create acc_memtable_destroy
 acc_memtable_malloc acc_memtable_acquire acc_memtable_release acc_memtable_free acc_memtable_insert_unmanaged
-acc_memtable_reclaim acc_memtable_get_stats""".split()
+acc_memtable_reclaim acc_memtable_get_stats acc_skel_create_async acc_skel_wait acc_skel_poll acc_skel_prefetch acc_compile_threads acc_compile_drain
+acc_tuning_set acc_tuning_text acc_context_set_tuning""".split()
 
 
 def build(force=False):
@@ -120,7 +121,7 @@ def lib():
             raise ImportError("libacchip.so is not built (%s); run `python -c 'import __graft_entry__ as g; g.build()'`"
                               % LIB_PATH)
         L = C.CDLL(LIB_PATH)
-        for name in ("acc_last_error", "acc_version", "acc_compile_log", "acc_cache_dir"):
+        for name in ("acc_last_error", "acc_version", "acc_compile_log", "acc_cache_dir", "acc_tuning_text"):
             getattr(L, name).restype = C.c_char_p
         L.acc_launch_grid.restype = C.c_int64
         L.acc_launch_grid.argtypes = [C.c_int64] * 4
@@ -151,6 +152,12 @@ def lib():
         L.acc_cache_set_dir.argtypes = [C.c_char_p]
         L.acc_skel_create.argtypes = [C.c_void_p, C.POINTER(acc_skel_desc), C.POINTER(C.c_void_p)]
         L.acc_skel_destroy.argtypes = [C.c_void_p]
+        L.acc_skel_create_async.argtypes = [C.c_void_p, C.POINTER(acc_skel_desc), C.POINTER(C.c_void_p)]
+        L.acc_skel_wait.argtypes = [C.c_void_p]
+        L.acc_skel_prefetch.argtypes = [C.c_void_p, C.c_int]
+        L.acc_skel_poll.argtypes = [C.c_void_p, C.POINTER(C.c_int)]
+        L.acc_tuning_set.argtypes = [C.c_char_p]
+        L.acc_context_set_tuning.argtypes = [C.c_void_p, C.c_char_p]
         L.acc_skel_source.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_char_p)]
         L.acc_skel_preview.argtypes = [C.POINTER(acc_skel_desc), C.c_int, C.POINTER(C.c_char_p), C.POINTER(C.c_char_p)]
         L.acc_skel_compile_only.argtypes = [C.c_char_p, C.POINTER(acc_skel_desc), C.POINTER(C.c_size_t)]
@@ -183,6 +190,8 @@ def lib():
         L.acc_memtable_insert_unmanaged.argtypes = [C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint64]
         L.acc_memtable_reclaim.argtypes = [C.c_void_p]
         L.acc_memtable_get_stats.argtypes = [C.c_void_p, C.POINTER(acc_memtable_stats)]
+        import atexit
+        atexit.register(L.acc_compile_drain)     # no worker inside the compiler when exit() tears its static data down
         _lib = L
     return _lib
 
@@ -273,6 +282,28 @@ def compile_source(source, target="gfx950", options=("-O3", "-std=c++17", "-ffp-
     code, size = C.c_void_p(), C.c_size_t(0)
     check(lib().acc_compile(None, target.encode(), source.encode(), opts, len(options), C.byref(code), C.byref(size)))
     return size.value
+
+
+class tuning(object):
+    """with tuning("scan.rows=2", ctx): ... -- the knobs as the process's table (what acc_skel_preview and
+    acc_skel_compile_only read) and, if a context is given, as that context's, for the instances created inside the
+    block; put back afterwards.  Nothing touches the environment."""
+
+    def __init__(self, text, ctx=None):
+        self.text, self.ctx = text, ctx
+
+    def __enter__(self):
+        self.old = lib().acc_tuning_text().decode()
+        check(lib().acc_tuning_set(_b(self.text or "")))
+        if self.ctx is not None:
+            self.ctx.set_tuning(self.text or "")
+        return self
+
+    def __exit__(self, *exc):
+        check(lib().acc_tuning_set(_b(self.old)))
+        if self.ctx is not None:
+            self.ctx.set_tuning(self.old)
+        return False
 
 
 def cache_stats():
@@ -433,7 +464,13 @@ class Context(object):
         return ms.value
 
     def skeleton(self, *args, **kw):
-        return Skeleton(self, make_desc(*args, **kw))
+        """an instance whose compilation runs in the background: whatever first uses it waits for it (wait=True: now)"""
+        wait = kw.pop("wait", False)
+        return Skeleton(self, make_desc(*args, **kw), wait=wait)
+
+    def set_tuning(self, text):
+        """the knobs ("name=value,...") that instances created in this context from now on take; None: the process's"""
+        check(lib().acc_context_set_tuning(self.handle, _b(text)))
 
     def close(self):
         if self.handle:
@@ -537,11 +574,27 @@ def _env(arrays):
 class Skeleton(object):
     """One compiled skeleton instance (acc_skel)."""
 
-    def __init__(self, ctx, desc):
+    def __init__(self, ctx, desc, wait=True):
         self.ctx, self.desc = ctx, desc
         h = C.c_void_p()
-        check(lib().acc_skel_create(ctx.handle, C.byref(desc), C.byref(h)))
+        check((lib().acc_skel_create if wait else lib().acc_skel_create_async)(ctx.handle, C.byref(desc), C.byref(h)))
         self.handle = h
+
+    def wait(self):
+        """block until the instance is compiled and loaded; raises what the compiler had to say"""
+        check(lib().acc_skel_wait(self.handle))
+        return self
+
+    def prefetch(self, variants):
+        """start compiling these variants in the background (the first launch that needs one would otherwise wait)"""
+        for v in variants:
+            check(lib().acc_skel_prefetch(self.handle, v))
+        return self
+
+    def ready(self):
+        r = C.c_int(0)
+        check(lib().acc_skel_poll(self.handle, C.byref(r)))
+        return bool(r.value)
 
     def info(self):
         i = acc_skel_info()

@@ -4,10 +4,12 @@
 #include <hip/hiprtc.h>
 
 #include <atomic>
+#include <condition_variable>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
 #include <map>
+#include <memory>
 #include <mutex>
 #include <string>
 #include <vector>
@@ -27,6 +29,9 @@ namespace acc {
 int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 int fail_hip(hipError_t e, const char *what);
 void set_compile_log(const std::string &log);
+void set_last_error(const std::string &message);
+std::string last_error_text();
+std::string compile_log_text();
 
 #define ACC_HIP_TRY(expr)                                  \
   do {                                                     \
@@ -39,6 +44,91 @@ void set_compile_log(const std::string &log);
     int _rc = (expr);            \
     if (_rc != ACC_OK) return _rc; \
   } while (0)
+
+// ---- tuning knobs -------------------------------------------------------------
+// "scan.block=512,scan.rows=2,fold.unroll=8": overrides of the defaults that the generator and the drivers work
+// with, for measurement sweeps.  The text is parsed ONCE into an immutable table -- the process's when it is first
+// wanted (from ACC_HIP_TUNE in the environment) or set (acc_tuning_set), a context's when it is created or
+// acc_context_set_tuning replaces it, an instance's when it is created -- so that nothing on the path of a driver call
+// reads the environment.  A knob the generator reads becomes part of the source text and so of the cache key.
+struct Tuning {
+  std::vector<std::pair<std::string, int>> kv;      // sorted by name
+  std::string text;
+  int get(const char *name, int dflt) const;
+  bool has(const char *name) const;
+};
+typedef std::shared_ptr<const Tuning> TuningPtr;
+TuningPtr parse_tuning(const char *text);           // NULL or "": no overrides
+TuningPtr default_tuning();                         // the process's table
+void set_default_tuning(TuningPtr t);
+
+// What the drivers look at on every call, resolved when an instance is created: plain integers.
+#define ACC_DRIVER_KNOBS(X)                                                                                          \
+  X(fold_blocks_per_cu, "fold.blocks_per_cu", 4)                                                                       \
+  X(fold_rows_max, "fold.rows_max", 7)                                                                                 \
+  X(foldseg_block_team_len, "foldseg.block_team_len", 16384)                                                           \
+  X(foldseg_long_from, "foldseg.long_from", 8)                                                                         \
+  X(foldseg_max_split, "foldseg.max_split", 4096)                                                                      \
+  X(foldseg_oversub, "foldseg.oversub", 1 << 20)                                                                       \
+  X(foldseg_row_team_below, "foldseg.row_team_below", 1024)                                                            \
+  X(foldseg_wave_team_len, "foldseg.wave_team_len", 128)                                                               \
+  X(map_oversub, "map.oversub", 1 << 20)                                                                               \
+  X(permute_atomic_flush_max, "permute.atomic_flush_max", 1 << 16)                                                     \
+  X(permute_fp_tables_from, "permute.fp_tables_from", 48)                                                              \
+  X(permute_fp_tables_to, "permute.fp_tables_to", 6144)                                                                \
+  X(permute_generic_lds, "permute.generic_lds", 1)                                                                     \
+  X(permute_inline_fill, "permute.inline_fill", 1)                                                                     \
+  X(permute_lds_bytes, "permute.lds_bytes", 160 * 1024)                                                                \
+  X(permute_lock_copies_bytes, "permute.lock_copies_bytes", 40 * 1024)                                                 \
+  X(permute_lock_lanes_per_target, "permute.lock_lanes_per_target", 32)                                                \
+  X(permute_lock_lds_min_ratio, "permute.lock_lds_min_ratio", 4)                                                       \
+  X(permute_lock_max_windows, "permute.lock_max_windows", 12)                                                          \
+  X(permute_lock_table_mbytes, "permute.lock_table_mbytes", 64)                                                        \
+  X(permute_max_blocks_per_cu, "permute.max_blocks_per_cu", 1)                                                         \
+  X(permute_max_copies, "permute.max_copies", 16)                                                                      \
+  X(permute_max_windows, "permute.max_windows", 32)                                                                    \
+  X(permute_narrow, "permute.narrow", 1)                                                                               \
+  X(permute_narrow_from, "permute.narrow_from", 8192)                                                                  \
+  X(permute_windows_from, "permute.windows_from", 2)                                                                   \
+  X(permute_xcd_row_kbytes, "permute.xcd_row_kbytes", 1024)                                                            \
+  X(scan_small_below_kb, "scan.small_below_kb", 12288)                                                                 \
+  X(stencil_half_strips, "stencil.half_strips", 1)                                                                     \
+  X(stencil_narrow_max, "stencil.narrow_max", 2)                                                                       \
+  X(stencil_stack, "stencil.stack", 0)                                                                                 \
+  X(stencil_strips_per_cu, "stencil.strips_per_cu", 3)                                                                 \
+  X(stencil_walk_min, "stencil.walk_min", 4)
+struct Knobs {
+#define ACC_KNOB_FIELD(field, name, dflt) int field = (dflt);
+  ACC_DRIVER_KNOBS(ACC_KNOB_FIELD)
+#undef ACC_KNOB_FIELD
+  void resolve(const Tuning &t)
+  {
+#define ACC_KNOB_GET(field, name, dflt) field = t.get(name, (dflt));
+    ACC_DRIVER_KNOBS(ACC_KNOB_GET)
+#undef ACC_KNOB_GET
+  }
+};
+
+// ---- compilation in the background ----------------------------------------------
+// One run-time compilation handed to the worker pool (Compile.hs:620-660: forked threads bounded by the number of
+// processors, the main thread carries on generating code and blocks at a kernel's first use, :451-457).  The job
+// owns copies of everything the compiler reads, so the instance it was made for may go away meanwhile.
+struct CompileJob {
+  std::string target, source;
+  std::vector<std::string> options;
+  std::mutex mu;
+  std::condition_variable cv;
+  bool done = false;
+  int rc = ACC_OK;
+  std::string error, log;          // acc_last_error / acc_compile_log of the worker, for whoever waits
+  const void *code = nullptr;      // owned by the kernel cache
+  size_t size = 0;
+  void run();                      // compile (through the cache) on the calling thread and mark done
+  int wait();                      // block until done; the outcome, with error and log copied to the calling thread
+};
+bool compile_submit(const std::shared_ptr<CompileJob> &job);     // false: the pool has been drained, nothing was queued
+void compile_drain();
+int compile_pool_threads();
 
 // the scan's descriptor block for callers that must not allocate (noalloc.hip)
 int noalloc_setup(int device);
@@ -112,6 +202,15 @@ struct acc_context_s {
   bool scratch_any_stream = false;
   bool scratch_multi_stream = false;
   hipStream_t scratch_first_stream = nullptr;
+
+  // the tuning table instances created in this context take (set under `mu`)
+  acc::TuningPtr tuning;
+  acc::TuningPtr tuning_now()
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    return tuning;
+  }
+  bool dump_exec = false;      // ACC_HIP_DEBUG=dump-exec was in the environment when the context was created
 
   // kernels report here that a bounded wait ran out (see StatusWord); NULL if the block could not be set up
   volatile uint32_t *status_host = nullptr;

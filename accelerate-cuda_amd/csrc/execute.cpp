@@ -25,6 +25,7 @@ namespace {
 // its last parameter (0: no loop).
 struct Running {
   const char *entry = "";
+  bool dump_exec = false;     // the context was created under ACC_HIP_DEBUG=dump-exec
   bool guarded = false;
   uint64_t guard = 0;
 };
@@ -91,11 +92,7 @@ hipError_t launch_kernel(hipFunction_t f, unsigned gx, unsigned gy, unsigned gz,
     }
     return rc;
   }
-  static const bool trace = [] {
-    const char *e = std::getenv("ACC_HIP_DEBUG");
-    return e && std::strstr(e, "dump-exec");
-  }();
-  if (!trace) return hipModuleLaunchKernel(f, gx, gy, gz, bx, by, bz, lds, st, args, extra);
+  if (!t_run.dump_exec) return hipModuleLaunchKernel(f, gx, gy, gz, bx, by, bz, lds, st, args, extra);
   hipEvent_t e0 = nullptr, e1 = nullptr;
   const bool timed = hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess && hipEventRecord(e0, st) == hipSuccess;
   const hipError_t rc = hipModuleLaunchKernel(f, gx, gy, gz, bx, by, bz, lds, st, args, extra);
@@ -199,6 +196,7 @@ struct RunScope {
   RunScope(acc_skel_s *s, hipStream_t st) : saved(t_run)
   {
     t_run.entry = s->entry.c_str();
+    t_run.dump_exec = s->ctx->dump_exec;
     t_run.guarded = s->spec.guarded;
     t_run.guard = 0;
     const uint64_t g = s->ctx->guard_of(st);
@@ -288,7 +286,7 @@ int acc_exec_map(acc_skel s, const acc_array *env, const acc_array *out, acc_str
     return launch(s, v, std::min<int64_t>((tiles + waves - 1) / waves, (int64_t)1 << 22), 0, static_cast<hipStream_t>(stream), &args);
   }
   // streaming with no reuse: one short-lived workgroup per tile keeps the most loads in flight
-  const int64_t grid = acc_launch_grid(n, s->elements_per_block(), resident(s, v), acc::tune("map.oversub", 1 << 20));
+  const int64_t grid = acc_launch_grid(n, s->elements_per_block(), resident(s, v), s->knobs.map_oversub);
   return launch(s, v, grid, 0, static_cast<hipStream_t>(stream), &args);
 }
 
@@ -305,26 +303,26 @@ int launch_segmented(acc_skel_s *s, int v, Args *args, const acc_array *env, con
                      hipStream_t st)
 {
   const int64_t avg = n / nseg;
-  if (avg < acc::tune("foldseg.wave_team_len", 128)) {
+  if (avg < s->knobs.foldseg_wave_team_len) {
     // Segments of 8 elements or more on average stage half as much again at a time (variants 2 and 3 of the
     // instance, built when first wanted): 2^25 elements in segments of 8 / 32 / 100 on average 36 / 31 / 51 us
     // -> 32 / 27 / 40; shorter segments lose by it (rows of 4: 46 -> 49 us), and so keep the shorter chunk.
     int lv = v;
-    if (avg >= acc::tune("foldseg.long_from", 8) && s->spec.chunk_long > s->spec.chunk) {
+    if (avg >= s->knobs.foldseg_long_from && s->spec.chunk_long > s->spec.chunk) {
       lv = v + 2;
       ACC_TRY(s->ensure_variant(lv));
     }
-    const int64_t grid = acc_launch_grid(nseg, s->spec.block, resident(s, lv), acc::tune("foldseg.oversub", 1 << 20));
+    const int64_t grid = acc_launch_grid(nseg, s->spec.block, resident(s, lv), s->knobs.foldseg_oversub);
     return launch(s, lv, grid, 0, st, args);
   }
   // teams: a workgroup (1) from `foldseg.block_team_len`, a row of 16 lanes (2) below `foldseg.row_team_below`, else a wave (0)
-  const int block_team = avg >= acc::tune("foldseg.block_team_len", 16384) ? 1 : (avg < acc::tune("foldseg.row_team_below", 1024) ? 2 : 0);
+  const int block_team = avg >= s->knobs.foldseg_block_team_len ? 1 : (avg < s->knobs.foldseg_row_team_below ? 2 : 0);
   const int64_t cus = s->ctx->props.multiProcessorCount;
   const int64_t team_lanes = block_team == 1 ? s->spec.block : (block_team == 2 ? 16 : 64);
   const int64_t room = cus * (2048 / team_lanes);                    // teams the device holds at once
   const int64_t min_piece = team_lanes * 64;                          // a piece keeps its team busy for a while
   int64_t split = 1;
-  if (nseg * 2 <= room) split = std::max<int64_t>(1, std::min<int64_t>({room / nseg, avg / min_piece, acc::tune("foldseg.max_split", 4096)}));
+  if (nseg * 2 <= room) split = std::max<int64_t>(1, std::min<int64_t>({room / nseg, avg / min_piece, s->knobs.foldseg_max_split}));
   acc::ScratchRef blk;
   uint64_t part = 0, part_ok = 0;
   if (split > 1) {
@@ -413,10 +411,10 @@ int acc_exec_fold(acc_skel s, const acc_array *env, int32_t in_rank, const int64
       const int64_t grid = acc_launch_grid(rows, s->spec.block, resident(s, v), 1 << 20);
       return launch(s, v, grid, 0, st, &args);
     }
-    if (inner <= std::min(16, acc::tune("fold.rows_max", 7))) {
+    if (inner <= std::min(16, s->knobs.fold_rows_max)) {
       // short rows: a lane reads its row straight from memory (skel_foldseg.h, _rows)
       const int64_t r = inner == 1 ? 4 : (inner == 2 ? 2 : 1), u = r * inner >= 16 ? 1 : 16 / (r * inner);   // as the kernel's R and U
-      const int64_t grid = acc_launch_grid(rows, s->spec.block * r * u, resident(s, v), acc::tune("foldseg.oversub", 1 << 20));
+      const int64_t grid = acc_launch_grid(rows, s->spec.block * r * u, resident(s, v), s->knobs.foldseg_oversub);
       hipError_t e = launch_kernel(s->variants[v].fn_rows, static_cast<unsigned>(grid), 1, 1, static_cast<unsigned>(s->spec.block), 1, 1,
                                            0, st, args.data(), nullptr);
       return e == hipSuccess ? ACC_OK : acc::fail_hip(e, "hipModuleLaunchKernel(fold, short rows)");
@@ -427,7 +425,7 @@ int acc_exec_fold(acc_skel s, const acc_array *env, int32_t in_rank, const int64
   const int64_t n = inner;
   const int64_t tile = s->elements_per_block();
   int64_t grid = acc_launch_grid(n, tile, s->ctx->props.multiProcessorCount,
-                                 std::min(s->variants[v].blocks_per_cu, acc::tune("fold.blocks_per_cu", 4)));
+                                 std::min(s->variants[v].blocks_per_cu, s->knobs.fold_blocks_per_cu));
   const bool single = s->spec.fold_single;       // as generated into the kernel
   if (grid == 1) {                 // a lone block finishes the job itself
     push_ptrs(out, out->ncomp, &args, &aligned);
@@ -565,13 +563,13 @@ int scan_core(acc_skel s, const acc_array *env, int64_t n, const acc_array *out,
   // large tiles leaves most of the device idle (Int32: 1024 elements 10.6 us -> 4.4, 2^18 8.6 -> 4.1, 2^21 10.0 ->
   // 8.1, 3 M + 3 14.8 -> 9.3; at 2^22 the two are level, 11.7 and 11.2, and so are 2^21 Float64, 12.0 and 13.2).
   const bool small = s->spec.scan_small_rows > 0 &&
-                     n * (int64_t)s->spec.elt_size <= (int64_t)acc::tune("scan.small_below_kb", 12288) * 1024;
+                     n * (int64_t)s->spec.elt_size <= (int64_t)s->knobs.scan_small_below_kb * 1024;
   int v = (aligned ? 0 : 1) + (small ? 2 : 0);
   if (noalloc) {
     // building a variant compiles and loads a module: not here
     if (!s->variant_ready(v))
       return fail(ACC_ERR_INVALID, "%s: the %s %s-tile variant of this instance is not loaded yet; run acc_exec_scan once on operands of the same alignment and of %s %d KB first",
-                  who, aligned ? "aligned" : "unaligned", small ? "small" : "large", small ? "at most" : "more than", acc::tune("scan.small_below_kb", 12288));
+                  who, aligned ? "aligned" : "unaligned", small ? "small" : "large", small ? "at most" : "more than", s->knobs.scan_small_below_kb);
   } else {
     ACC_TRY(s->ensure_variant(v));
   }
@@ -678,21 +676,21 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
   // A combination without an atomic instruction of its own on few targets: compare-and-swap loops on the result
   // meet on those few addresses (16 M Float32 `max` updates on 1000 targets: 16.6 ms), the tables in LDS of the
   // locked template do not (74 us).  Such a skeleton carries that template as its variants 2 and 3.
-  const int64_t lds_all = std::min<int64_t>((int64_t)s->ctx->props.sharedMemPerBlock, acc::tune("permute.lds_bytes", 160 * 1024));
+  const int64_t lds_all = std::min<int64_t>((int64_t)s->ctx->props.sharedMemPerBlock, s->knobs.permute_lds_bytes);
   // targets per table in LDS (value + state word each), and how many such windows the targets need
   const int64_t lds_cap = std::max<int64_t>(1, (lds_all - 16) / ((int64_t)esz + 4));
   const int64_t lds_windows = (ntarget + lds_cap - 1) / lds_cap;
-  const bool lds_table_fits = lds_windows <= acc::tune("permute.lock_max_windows", 12) &&
-                              n_src >= acc::tune("permute.lock_lds_min_ratio", 4) * ntarget;
+  const bool lds_table_fits = lds_windows <= s->knobs.permute_lock_max_windows &&
+                              n_src >= s->knobs.permute_lock_lds_min_ratio * ntarget;
   // (Floating-point addition has an LDS atomic, but it runs at a fifth of the integer one's rate -- 16 M updates on
   // 1000 targets: 95 us against 63 us through the tables -- so between 48 and 6144 targets it goes the same way.
   // Below, the tables' locks are what lanes meet on (16 targets 149 us against 93, one target 2.1 ms against 0.12);
   // above, a table holds half the targets an array of plain values does and the passes over the source multiply
   // (16 384 targets 123 us against 102, 131 072: 407 against 107).)
   const bool fp_add = s->spec.combine_hint == ACC_COMBINE_ADD && (s->spec.elt_type == "float" || s->spec.elt_type == "double") &&
-                      ntarget >= acc::tune("permute.fp_tables_from", 48) && ntarget <= acc::tune("permute.fp_tables_to", 6144);
+                      ntarget >= s->knobs.permute_fp_tables_from && ntarget <= s->knobs.permute_fp_tables_to;
   const bool generic_few = !s->spec.permute_locked && (s->spec.combine_hint == ACC_COMBINE_GENERIC || fp_add) && lds_table_fits &&
-                           acc::tune("permute.generic_lds", 1) != 0;
+                           s->knobs.permute_generic_lds != 0;
   if (s->spec.permute_locked || generic_few) {
     // elements no atomic covers: a lock per target (the reference's lock array, Execute.hs:402-405)
     ACC_TRY(plain_copy());
@@ -711,7 +709,7 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
     // of the holder's own accesses, and with hundreds of lanes waiting per lock the device's whole atomic rate goes
     // into failed attempts (1000 targets: 12 M updates/s with every compute unit full, 20 times that with 32 lanes
     // per target).
-    const int64_t lanes = std::max<int64_t>(64, ntarget * acc::tune("permute.lock_lanes_per_target", 32));
+    const int64_t lanes = std::max<int64_t>(64, ntarget * s->knobs.permute_lock_lanes_per_target);
     int64_t lgrid = std::min(acc_launch_grid(n_src, s->spec.block, s->ctx->props.multiProcessorCount, 8),
                              (lanes + s->spec.block - 1) / s->spec.block);
     // With few targets every workgroup combines in a table of its own in LDS (value + state word per target),
@@ -728,7 +726,7 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
       auto lds_for = [&](int64_t copies) { return (((int64_t)lds_bins * copies * (int64_t)esz + 15) & ~int64_t(15)) + (int64_t)lds_bins * copies * 4; };
       const int64_t waves = s->spec.block / 64;
       while (lds_windows == 1 && lds_copies * 2 <= waves &&
-             lds_for(lds_copies * 2) <= std::min<int64_t>(lds_budget, acc::tune("permute.lock_copies_bytes", 40 * 1024))) lds_copies *= 2;
+             lds_for(lds_copies * 2) <= std::min<int64_t>(lds_budget, s->knobs.permute_lock_copies_bytes)) lds_copies *= 2;
       lds_need = lds_for(lds_copies);
       int bpc = 0;
       hipError_t oe = hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&bpc, s->variants[lv].fn, s->spec.block, (size_t)lds_need);
@@ -736,7 +734,7 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
       // the device full of workgroups, shared out between the windows, as long as their rows stay within
       // `permute.lock_table_mbytes`
       const int64_t row_bytes = (int64_t)lds_bins * ((int64_t)esz + 4);
-      const int64_t row_cap = std::max<int64_t>(lds_windows, ((int64_t)acc::tune("permute.lock_table_mbytes", 64) << 20) / row_bytes);
+      const int64_t row_cap = std::max<int64_t>(lds_windows, ((int64_t)s->knobs.permute_lock_table_mbytes << 20) / row_bytes);
       const int64_t blocks = std::max<int64_t>(lds_windows, std::min<int64_t>(
           lds_windows * acc_launch_grid(n_src, s->spec.block, s->ctx->props.multiProcessorCount, bpc), std::min<int64_t>((int64_t)s->ctx->props.multiProcessorCount * bpc, row_cap)));
       win_blocks = static_cast<int32_t>(std::max<int64_t>(1, blocks / lds_windows));
@@ -790,8 +788,8 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
                        (s->spec.elt_type == "Int32" || s->spec.elt_type == "Word32" || s->spec.elt_type == "Int64" || s->spec.elt_type == "Word64");
   // Only where the source is spelt as a small constant -- the counting idiom, `permute (+) zeros bin ones` -- since any
   // other addend would go to the result one device-scope atomic at a time (`permute.narrow=2` takes every source).
-  const int narrow = acc::tune("permute.narrow", 1);
-  if (int_add && ntarget > std::min<int64_t>(acc::tune("permute.narrow_from", 8192), lds_all / (int64_t)esz) && ((ntarget + 1) / 2) * 4 <= lds_all && n_src >= 4 * ntarget &&
+  const int narrow = s->knobs.permute_narrow;
+  if (int_add && ntarget > std::min<int64_t>(s->knobs.permute_narrow_from, lds_all / (int64_t)esz) && ((ntarget + 1) / 2) * 4 <= lds_all && n_src >= 4 * ntarget &&
       (narrow == 2 || (narrow == 1 && s->spec.get_small_constant))) {
     const int nv = (aligned ? 0 : 1) + 6;
     ACC_TRY(s->ensure_variant(nv));
@@ -863,7 +861,7 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
     int win_log = 0;                                       // a power of two of windows: targets are dealt out modulo it
     while (((ntarget + ((int64_t)1 << win_log) - 1) >> win_log) > wcap) ++win_log;
     const int64_t windows = (int64_t)1 << win_log;
-    if (windows >= acc::tune("permute.windows_from", 2) && windows <= acc::tune("permute.max_windows", 32) && n_src >= 4 * ntarget) {
+    if (windows >= s->knobs.permute_windows_from && windows <= s->knobs.permute_max_windows && n_src >= 4 * ntarget) {
       const int wv = (aligned ? 0 : 1) + 4;
       ACC_TRY(s->ensure_variant(wv));
       ACC_TRY(plain_copy());
@@ -924,17 +922,17 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
   const int cus = s->ctx->props.multiProcessorCount;
   int64_t bins = 0, copies = 1;
   if (s->spec.combine_hint != ACC_COMBINE_GENERIC) {
-    const int64_t budget = std::min<int64_t>((int64_t)s->ctx->props.sharedMemPerBlock, acc::tune("permute.lds_bytes", 160 * 1024)) - s->variants[v].static_lds;
+    const int64_t budget = std::min<int64_t>((int64_t)s->ctx->props.sharedMemPerBlock, s->knobs.permute_lds_bytes) - s->variants[v].static_lds;
     const int64_t cap = std::max<int64_t>(0, budget / (int64_t)esz);
     bins = std::min(ntarget, cap);
     if (bins == ntarget && bins > 0) copies = std::max<int64_t>(1, std::min<int64_t>(s->spec.block / 64, cap / bins));
-    copies = std::min<int64_t>(copies, acc::tune("permute.max_copies", 16));
+    copies = std::min<int64_t>(copies, s->knobs.permute_max_copies);
   }
   const size_t lds = (size_t)(bins * copies) * esz;
   int bpc = 0;
   hipError_t e = hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&bpc, s->variants[v].fn, s->spec.block, lds);
   if (e != hipSuccess || bpc < 1) { (void)hipGetLastError(); bpc = 1; }
-  const int64_t grid = acc_launch_grid(n_src, s->elements_per_block(), cus, std::min(bpc, acc::tune("permute.max_blocks_per_cu", 1)));
+  const int64_t grid = acc_launch_grid(n_src, s->elements_per_block(), cus, std::min(bpc, s->knobs.permute_max_blocks_per_cu));
 
   // How the privatised part leaves the blocks: atomics while they are few, otherwise a table of
   // per-block bins folded by a second kernel.
@@ -943,8 +941,8 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
   // each XCD share such a row instead, and the rows are folded into the result afterwards.
   constexpr int64_t XCD_ROWS = 16;                 // what the kernel's XCC_ID field can name
   const bool far_rows = bins > 0 && bins < ntarget &&
-                        ntarget * (int64_t)esz <= (int64_t)acc::tune("permute.xcd_row_kbytes", 1024) << 10;
-  const bool table = bins > 0 && grid * bins > acc::tune("permute.atomic_flush_max", 1 << 16);
+                        ntarget * (int64_t)esz <= (int64_t)s->knobs.permute_xcd_row_kbytes << 10;
+  const bool table = bins > 0 && grid * bins > s->knobs.permute_atomic_flush_max;
   const size_t far_bytes = far_rows ? (size_t)(XCD_ROWS * ntarget) * esz : 0;
   const size_t dump_bytes = table ? (size_t)(grid * bins) * esz : 0;
   acc::ScratchRef blk;
@@ -959,7 +957,7 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
   // are copied by workgroup 0 of the main kernel while the others read the source, and a word in scratch memory
   // ({epoch, 1}, as the fold's partial results are tagged) tells them when their atomics may follow: one launch.
   const bool inline_fill = copy_defaults && !far_rows && !table && bins == ntarget && bins > 0 && n_src > 0 &&
-                           acc::tune("permute.inline_fill", 1) != 0;
+                           s->knobs.permute_inline_fill != 0;
   acc::ScratchRef rblk;
   if (inline_fill) {
     const int arc = s->ctx->scratch_acquire(256, st, acc::SCRATCH_FLAGS, &rblk);
@@ -1076,7 +1074,7 @@ static int stencil_once(acc_skel s, const acc_array *env, const acc_array *in, c
   // An array narrower than half a strip (a quarter) takes the variant with half (a quarter) of the columns a lane,
   // where the stencil's reach allows: the lanes of a strip that lie outside the array do nothing.
   int narrow = 0;
-  while (narrow < acc::tune("stencil.narrow_max", 2) && (s->spec.svec >> (narrow + 1)) >= std::max(1, s->spec.reach_x) &&
+  while (narrow < s->knobs.stencil_narrow_max && (s->spec.svec >> (narrow + 1)) >= std::max(1, s->spec.reach_x) &&
          w <= (int64_t)64 * (s->spec.svec >> (narrow + 1)))
     ++narrow;
   // Strips that walk through planes are bound by the instructions of a strip, whatever its share of columns inside the
@@ -1084,14 +1082,14 @@ static int stencil_once(acc_skel s, const acc_array *env, const acc_array *in, c
   // (200 x 200 x 300: 35.3 -> 27.4 us), and less than one strip's width as two of half the width, not as one that the
   // edge of the array cuts (150^3: 17.0 -> 13.3 us).  (In 2-D the columns a last strip produces a second time cost
   // next to nothing.)
-  if (narrow == 0 && s->spec.zmarch && (s->spec.svec >> 1) >= std::max(1, s->spec.reach_x) && acc::tune("stencil.half_strips", 1) != 0) {
+  if (narrow == 0 && s->spec.zmarch && (s->spec.svec >> 1) >= std::max(1, s->spec.reach_x) && s->knobs.stencil_half_strips != 0) {
     const int64_t halves = (w + 32 * s->spec.svec - 1) / (32 * s->spec.svec);
     if (halves == 3 || (halves == 2 && w < 64 * s->spec.svec)) narrow = 1;
   }
   const int64_t tile_w = (int64_t)64 * (s->spec.svec >> narrow);
   const int64_t strips_x = (w + tile_w - 1) / tile_w;
   int64_t bands = (h + s->spec.tile_h - 1) / s->spec.tile_h;
-  if (rank == 2 && acc::tune("stencil.stack", 0)) bands = (bands + waves - 1) / waves * waves;
+  if (rank == 2 && s->knobs.stencil_stack) bands = (bands + waves - 1) / waves * waves;
   int64_t zbands = (planes + s->spec.tile_z - 1) / s->spec.tile_z;             // tile_z result planes per strip
   int64_t walk = s->spec.tile_h;
   if (s->spec.zmarch) {                  // strips tile_z rows tall that walk through tile_h planes
@@ -1099,8 +1097,8 @@ static int stencil_once(acc_skel s, const acc_array *env, const acc_array *in, c
     // ... or through fewer, halving down to 4, until there are three strips for every compute unit: a volume of
     // 256^3 has 256 strips of 64 planes, a wave for every fourth SIMD (44.1 us; 23.4 with 1024 strips of 16 planes,
     // although each reads 2 rz planes beyond its own; 128 x 128 x 256: 40.5 us -> 6.6 at 4 planes a strip).
-    const int64_t enough = (int64_t)acc::tune("stencil.strips_per_cu", 3) * s->ctx->props.multiProcessorCount;
-    const int64_t shortest = std::max(1, std::min(acc::tune("stencil.walk_min", 4), s->spec.tile_h));
+    const int64_t enough = (int64_t)s->knobs.stencil_strips_per_cu * s->ctx->props.multiProcessorCount;
+    const int64_t shortest = std::max(1, std::min(s->knobs.stencil_walk_min, s->spec.tile_h));
     while (walk / 2 >= shortest && strips_x * bands * ((planes + walk - 1) / walk) < enough) walk /= 2;
     zbands = (planes + walk - 1) / walk;
   }

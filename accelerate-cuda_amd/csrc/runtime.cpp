@@ -8,6 +8,8 @@
 //   Execute/Stream.hs, Execute/Event.hs      stream and event handling
 //   Compile.hs:453-465,505,534               loadData / getFun / requires
 //   Execute.hs:975-978                       launchKernel
+#include <algorithm>
+#include <cstdlib>
 #include <cstring>
 
 #include "acc_internal.hpp"
@@ -37,6 +39,66 @@ int fail_hip(hipError_t e, const char *what)
 }
 
 void set_compile_log(const std::string &log) { g_compile_log = log; }
+void set_last_error(const std::string &message) { g_last_error = message; }
+std::string last_error_text() { return g_last_error; }
+std::string compile_log_text() { return g_compile_log; }
+
+// ---- tuning knobs ------------------------------------------------------------
+
+int Tuning::get(const char *name, int dflt) const
+{
+  auto it = std::lower_bound(kv.begin(), kv.end(), name,
+                             [](const std::pair<std::string, int> &e, const char *n) { return e.first.compare(n) < 0; });
+  return (it != kv.end() && it->first == name) ? it->second : dflt;
+}
+
+bool Tuning::has(const char *name) const
+{
+  auto it = std::lower_bound(kv.begin(), kv.end(), name,
+                             [](const std::pair<std::string, int> &e, const char *n) { return e.first.compare(n) < 0; });
+  return it != kv.end() && it->first == name;
+}
+
+TuningPtr parse_tuning(const char *text)
+{
+  auto t = std::make_shared<Tuning>();
+  t->text = text ? text : "";
+  const std::string &all = t->text;
+  size_t pos = 0;
+  while (pos < all.size()) {
+    size_t end = all.find(',', pos);
+    if (end == std::string::npos) end = all.size();
+    const size_t eq = all.find('=', pos);
+    if (eq != std::string::npos && eq < end && eq > pos) {
+      std::string name = all.substr(pos, eq - pos);
+      while (!name.empty() && name.front() == ' ') name.erase(name.begin());
+      while (!name.empty() && name.back() == ' ') name.pop_back();
+      // the first setting of a name wins, as it did when the text was searched from the left
+      bool seen = false;
+      for (const auto &e : t->kv) seen = seen || e.first == name;
+      if (!seen && !name.empty()) t->kv.emplace_back(name, std::atoi(all.c_str() + eq + 1));
+    }
+    pos = end + 1;
+  }
+  std::sort(t->kv.begin(), t->kv.end());
+  return t;
+}
+
+static std::mutex g_tuning_mu;
+static TuningPtr g_tuning;
+
+TuningPtr default_tuning()
+{
+  std::lock_guard<std::mutex> lock(g_tuning_mu);
+  if (!g_tuning) g_tuning = parse_tuning(std::getenv("ACC_HIP_TUNE"));     // once, when first wanted
+  return g_tuning;
+}
+
+void set_default_tuning(TuningPtr t)
+{
+  std::lock_guard<std::mutex> lock(g_tuning_mu);
+  g_tuning = std::move(t);
+}
 
 }  // namespace acc
 
@@ -311,6 +373,11 @@ int acc_context_create(int device, acc_context *out)
       if (hp) (void)hipHostFree(hp);
     }
   }
+  ctx->tuning = acc::default_tuning();
+  {
+    const char *dbg = std::getenv("ACC_HIP_DEBUG");      // looked at here, never on the path of a launch
+    ctx->dump_exec = dbg && std::strstr(dbg, "dump-exec");
+  }
   ctx->arch = ctx->props.gcnArchName;
   const size_t colon = ctx->arch.find(':');
   if (colon != std::string::npos) ctx->arch.resize(colon);
@@ -329,6 +396,29 @@ int acc_context_destroy(acc_context ctx)
   }
   if (ctx->status_host) (void)hipHostFree(const_cast<uint32_t *>(ctx->status_host));
   delete ctx;
+  return ACC_OK;
+}
+
+int acc_tuning_set(const char *text)
+{
+  // NULL: what ACC_HIP_TUNE holds in the environment now
+  acc::set_default_tuning(acc::parse_tuning(text ? text : std::getenv("ACC_HIP_TUNE")));
+  return ACC_OK;
+}
+
+const char *acc_tuning_text(void)
+{
+  static thread_local std::string text;
+  text = acc::default_tuning()->text;
+  return text.c_str();
+}
+
+int acc_context_set_tuning(acc_context ctx, const char *text)
+{
+  if (!ctx) return fail(ACC_ERR_INVALID, "acc_context_set_tuning: NULL context");
+  acc::TuningPtr t = text ? acc::parse_tuning(text) : acc::default_tuning();
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  ctx->tuning = t;
   return ACC_OK;
 }
 
@@ -482,6 +572,11 @@ int acc_stream_destroy(acc_context ctx, acc_stream s)
   if (!ctx) return fail(ACC_ERR_INVALID, "acc_stream_destroy: NULL context");
   ACC_TRY(ctx->make_current());
   acc::scan_order_forget(ctx->device, static_cast<hipStream_t>(s));
+  {
+    // a guard set on the stream goes with it: a later stream commonly gets the same handle value
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    if (ctx->guards.erase(static_cast<hipStream_t>(s)) != 0) ctx->n_guards.fetch_sub(1, std::memory_order_release);
+  }
   ACC_HIP_TRY(hipStreamDestroy(static_cast<hipStream_t>(s)));
   return ACC_OK;
 }

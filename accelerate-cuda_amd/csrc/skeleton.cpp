@@ -44,31 +44,6 @@ static std::string flat(const char *s)
   return r;
 }
 
-// ---- tuning knobs -----------------------------------------------------------
-// ACC_HIP_TUNE="scan.block=512,scan.rows=2,fold.unroll=8" overrides a default,
-// for measurement sweeps; the value becomes part of the source and so of the
-// cache key.
-// whether ACC_HIP_TUNE names the knob at all
-bool tuned(const char *name)
-{
-  return tune(name, -0x7ffffffe) != -0x7ffffffe;
-}
-
-int tune(const char *name, int dflt)
-{
-  const char *e = std::getenv("ACC_HIP_TUNE");
-  if (!e) return dflt;
-  const std::string all = e, key = std::string(name) + "=";
-  size_t pos = 0;
-  while (pos < all.size()) {
-    size_t end = all.find(',', pos);
-    if (end == std::string::npos) end = all.size();
-    if (all.compare(pos, key.size(), key) == 0) return std::atoi(all.c_str() + pos + key.size());
-    pos = end + 1;
-  }
-  return dflt;
-}
-
 // "a, f(b, c), {d, e}" -> ["a", "f(b, c)", "{d, e}"]: split at the commas that lie inside no bracket
 static std::vector<std::string> split_top_level(const std::string &text)
 {
@@ -152,6 +127,9 @@ static const char *kind_name(int kind)
 
 int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::string *source)
 {
+  const Tuning &knobs = *sp.tuning;
+  auto tune = [&](const char *name, int dflt) { return knobs.get(name, dflt); };
+  auto tuned = [&](const char *name) { return knobs.has(name); };
   std::ostringstream o;
   int vec = std::max(1, 16 / std::max(1, sp.vec_size));
   o << "// accelerate-hip " ACC_HIP_VERSION " skeleton instance: " << kind_name(sp.kind) << "\n";
@@ -435,14 +413,19 @@ static bool small_literal(std::string t)
 // loads 16 bytes, so 16 elements of one byte: one load of 256 lanes is then 4096 of them)
 static int segmented_chunk(const SkelSpec &sp, bool long_segments = false)
 {
+  auto tune = [&](const char *name, int dflt) { return sp.tuning->get(name, dflt); };
   const int per_load = sp.block * std::max(1, 16 / std::max(1, sp.vec_size));
   const int want = std::max(long_segments ? tune("foldseg.chunk_long", 3072) : tune("foldseg.chunk", 2048), per_load);
   return (want + per_load - 1) / per_load * per_load;
 }
 
-int make_spec(const acc_skel_desc *d, SkelSpec *sp)
+int make_spec(const acc_skel_desc *d, const TuningPtr &tuning, SkelSpec *sp)
 {
   if (!d) return fail(ACC_ERR_INVALID, "NULL skeleton description");
+  sp->tuning = tuning ? tuning : default_tuning();
+  const Tuning &knobs = *sp->tuning;
+  auto tune = [&](const char *name, int dflt) { return knobs.get(name, dflt); };
+  auto tuned = [&](const char *name) { return knobs.has(name); };
   if (d->kind < 0 || d->kind >= ACC_SKEL_KIND_COUNT) return fail(ACC_ERR_INVALID, "unknown skeleton kind %d", d->kind);
   if (!d->elt_type || !*d->elt_type) return fail(ACC_ERR_INVALID, "skeleton description: elt_type missing");
   if (d->n_env < 0 || (d->n_env > 0 && !d->env)) return fail(ACC_ERR_INVALID, "skeleton description: bad env");
@@ -732,6 +715,32 @@ SkelSpec spec_of_variant(const SkelSpec &base, int v)
 }
 }  // namespace acc
 
+// the job that compiles variant v (not yet started); fills in the variant's source and entry name
+static int make_job(acc_skel_s *s, int v, std::shared_ptr<acc::CompileJob> *out)
+{
+  acc::Variant &var = s->variants[v];
+  const acc::SkelSpec spec = acc::spec_of_variant(s->spec, v);
+  ACC_TRY(acc::generate_source(spec, (v & 1) == 0, &var.entry, &var.source));
+  if (s->entry.empty()) s->entry = var.entry;      // the same for every variant; set once, before the instance is shared
+  auto job = std::make_shared<acc::CompileJob>();
+  job->target = s->ctx->arch;
+  job->source = var.source;
+  job->options = acc::compile_options(spec);
+  *out = job;
+  return ACC_OK;
+}
+
+int acc_skel_s::start_variant(int v)
+{
+  std::lock_guard<std::mutex> lock(mu);
+  acc::Variant &var = variants[v];
+  if (var.ready || var.job) return ACC_OK;
+  std::shared_ptr<acc::CompileJob> job;
+  ACC_TRY(make_job(this, v, &job));
+  if (acc::compile_submit(job)) var.job = job;      // else: compiled by the thread that first needs it
+  return ACC_OK;
+}
+
 int acc_skel_s::ensure_variant(int v)
 {
   // two threads may meet here on the first launch that needs the unaligned variant
@@ -740,15 +749,17 @@ int acc_skel_s::ensure_variant(int v)
   if (var.ready) return ACC_OK;
   // variants 2 and 3 of a permute: the locked template for an element the atomic template also covers
   acc::SkelSpec spec = acc::spec_of_variant(this->spec, v);
-  std::string entry_name;
-  ACC_TRY(acc::generate_source(spec, (v & 1) == 0, &entry_name, &var.source));
-  if (entry.empty()) entry = entry_name;      // the same for every variant; set once, before the instance is shared
-  std::vector<std::string> opts = acc::compile_options(spec);
-  std::vector<const char *> optp;
-  for (const std::string &s : opts) optp.push_back(s.c_str());
-  const void *code = nullptr;
-  size_t size = 0;
-  ACC_TRY(acc_compile(ctx, nullptr, var.source.c_str(), optp.data(), static_cast<int>(optp.size()), &code, &size));
+  if (!var.job) {                       // nobody has started it: this thread compiles
+    std::shared_ptr<acc::CompileJob> job;
+    ACC_TRY(make_job(this, v, &job));
+    var.job = job;
+    job->run();
+  }
+  // a kernel's first use: here the reference blocks on the compilation it started earlier (Compile.hs:451-457);
+  // a failure is reported to every caller that comes by, with the compiler's log
+  ACC_TRY(var.job->wait());
+  const std::string entry_name = var.entry;
+  const void *code = var.job->code;
   ACC_TRY(ctx->make_current());
   ACC_HIP_TRY(hipModuleLoadData(&var.module, code));
   hipError_t e = hipModuleGetFunction(&var.fn, var.module, entry_name.c_str());
@@ -796,7 +807,7 @@ int acc_skel_s::ensure_variant(int v)
     this->spec.scan_shape_open = false;
     if (var.num_regs > 256) {
       (void)hipModuleUnload(var.module);
-      var = acc::Variant();
+      var = acc::Variant();                   // (its job goes with it: the next build starts from the new shape)
       this->spec.block = 1024;
       this->spec.rows = this->spec.scan_rows_fallback;
       lock.unlock();
@@ -812,20 +823,80 @@ int acc_skel_s::ensure_variant(int v)
   return ACC_OK;
 }
 
+// how many variants an instance of this kind has (the numbering of acc_skel_preview)
+static int variant_count(const acc::SkelSpec &sp)
+{
+  const bool stencil = sp.kind == ACC_SKEL_STENCIL || sp.kind == ACC_SKEL_STENCIL2;
+  return sp.kind == ACC_SKEL_PERMUTE ? 8 : (stencil ? 6 : ((sp.scan_small_rows > 0 || sp.chunk_long > 0) ? 4 : 2));
+}
+
 extern "C" {
 
-int acc_skel_create(acc_context ctx, const acc_skel_desc *desc, acc_skel *out)
+int acc_skel_create_async(acc_context ctx, const acc_skel_desc *desc, acc_skel *out)
 {
   if (!ctx || !out) return fail(ACC_ERR_INVALID, "acc_skel_create: NULL argument");
   *out = nullptr;
   acc::SkelSpec sp;
-  ACC_TRY(acc::make_spec(desc, &sp));
+  ACC_TRY(acc::make_spec(desc, ctx->tuning_now(), &sp));
   acc_skel_s *s = new acc_skel_s();
   s->ctx = ctx;
   s->spec = sp;
-  int rc = s->ensure_variant(0);      // the unaligned variant is built on first need
+  s->knobs.resolve(*sp.tuning);
+  const int rc = s->start_variant(0);     // the other variants are built when a call first needs them
   if (rc != ACC_OK) { delete s; return rc; }
   *out = s;
+  return ACC_OK;
+}
+
+int acc_skel_create(acc_context ctx, const acc_skel_desc *desc, acc_skel *out)
+{
+  acc_skel s = nullptr;
+  ACC_TRY(acc_skel_create_async(ctx, desc, &s));
+  const int rc = s->ensure_variant(0);
+  if (rc != ACC_OK) { acc_skel_destroy(s); return rc; }
+  *out = s;
+  return ACC_OK;
+}
+
+int acc_skel_prefetch(acc_skel s, int variant)
+{
+  if (!s) return fail(ACC_ERR_INVALID, "acc_skel_prefetch: NULL skeleton");
+  if (variant < 0 || variant >= variant_count(s->spec))
+    return fail(ACC_ERR_INVALID, "acc_skel_prefetch: this kind of skeleton has variants 0 to %d", variant_count(s->spec) - 1);
+  // (the locked form of a permute is only generated for elements the atomic template does not take, and the other way round)
+  if (s->spec.kind == ACC_SKEL_PERMUTE && s->spec.permute_locked && variant >= 2)
+    return fail(ACC_ERR_INVALID, "acc_skel_prefetch: a permute under locks has variants 0 and 1");
+  return s->start_variant(variant);
+}
+
+int acc_skel_wait(acc_skel s)
+{
+  if (!s) return fail(ACC_ERR_INVALID, "acc_skel_wait: NULL skeleton");
+  return s->ensure_variant(0);
+}
+
+int acc_skel_poll(acc_skel s, int *ready)
+{
+  if (!s || !ready) return fail(ACC_ERR_INVALID, "acc_skel_poll: NULL argument");
+  std::shared_ptr<acc::CompileJob> job;
+  {
+    std::lock_guard<std::mutex> lock(s->mu);
+    if (s->variants[0].ready) { *ready = 1; return ACC_OK; }
+    job = s->variants[0].job;
+  }
+  *ready = 0;
+  if (job) {
+    std::lock_guard<std::mutex> lock(job->mu);
+    *ready = job->done ? 1 : 0;
+  }
+  return ACC_OK;
+}
+
+int acc_compile_threads(void) { return acc::compile_pool_threads(); }
+
+int acc_compile_drain(void)
+{
+  acc::compile_drain();
   return ACC_OK;
 }
 
@@ -842,6 +913,7 @@ int acc_skel_destroy(acc_skel s)
 int acc_skel_source(acc_skel s, int variant, const char **source)
 {
   if (!s || !source || variant < 0 || variant > 1) return fail(ACC_ERR_INVALID, "acc_skel_source: bad argument");
+  std::lock_guard<std::mutex> lock(s->mu);
   if (s->variants[variant].source.empty()) {
     std::string e;
     ACC_TRY(acc::generate_source(s->spec, variant == 0, &e, &s->variants[variant].source));
@@ -855,11 +927,10 @@ int acc_skel_preview(const acc_skel_desc *desc, int variant, const char **source
   static thread_local std::string text, name;
   if (!source || variant < 0 || variant > 7) return fail(ACC_ERR_INVALID, "acc_skel_preview: bad argument");
   acc::SkelSpec sp;
-  ACC_TRY(acc::make_spec(desc, &sp));
+  ACC_TRY(acc::make_spec(desc, acc::default_tuning(), &sp));
   // beyond 1: a permute's forms (to 7), a stencil's fewer columns a lane (to 5), a scan's small tiles and a segmented
   // fold's longer chunk (2 and 3)
-  const bool stencil = sp.kind == ACC_SKEL_STENCIL || sp.kind == ACC_SKEL_STENCIL2;
-  const int most = sp.kind == ACC_SKEL_PERMUTE ? 7 : (stencil ? 5 : ((sp.scan_small_rows > 0 || sp.chunk_long > 0) ? 3 : 1));
+  const int most = variant_count(sp) - 1;
   if (variant > most) return fail(ACC_ERR_INVALID, "acc_skel_preview: this kind of skeleton has variants 0 to %d", most);
   ACC_TRY(acc::generate_source(acc::spec_of_variant(sp, variant), (variant & 1) == 0, &name, &text));
   *source = text.c_str();
@@ -871,7 +942,7 @@ int acc_skel_compile_only(const char *target, const acc_skel_desc *desc, size_t 
 {
   if (!target) return fail(ACC_ERR_INVALID, "acc_skel_compile_only: NULL target");
   acc::SkelSpec sp;
-  ACC_TRY(acc::make_spec(desc, &sp));
+  ACC_TRY(acc::make_spec(desc, acc::default_tuning(), &sp));
   std::vector<std::string> opts = acc::compile_options(sp);
   std::vector<const char *> optp;
   for (const std::string &o : opts) optp.push_back(o.c_str());
@@ -891,6 +962,7 @@ int acc_skel_compile_only(const char *target, const acc_skel_desc *desc, size_t 
 int acc_skel_get_info(acc_skel s, acc_skel_info *out)
 {
   if (!s || !out) return fail(ACC_ERR_INVALID, "acc_skel_get_info: NULL argument");
+  ACC_TRY(s->ensure_variant(0));          // the record of a kernel that is still being compiled: wait for it
   std::memset(out, 0, sizeof(*out));
   std::snprintf(out->entry, sizeof(out->entry), "%s", s->entry.c_str());
   out->block = s->spec.block;

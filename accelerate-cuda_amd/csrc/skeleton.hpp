@@ -12,6 +12,7 @@ struct EnvSig {
 
 // the validated, owned form of an acc_skel_desc plus the tuning of its template
 struct SkelSpec {
+  TuningPtr tuning;                     // the knobs the generator reads (never NULL once make_spec has run)
   int kind = 0;
   uint32_t flags = 0;
   std::vector<EnvSig> env;
@@ -70,12 +71,12 @@ struct Variant {
   int blocks_per_cu = 1;
   int block = 0;                       // workgroup size and rows a lane of this variant was built with (a scan's small
   int rows = 0;                        // variant differs from the instance's)
+  std::shared_ptr<CompileJob> job;     // its compilation, once started: in the background, or by the thread that needs it
+  std::string entry;                   // the main kernel's name in `job`'s code
 };
 
 int type_size(const std::string &t);
-int tune(const char *name, int dflt);
-bool tuned(const char *name);
-int make_spec(const acc_skel_desc *d, SkelSpec *sp);
+int make_spec(const acc_skel_desc *d, const TuningPtr &tuning, SkelSpec *sp);
 int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::string *source);
 SkelSpec spec_of_variant(const SkelSpec &base, int variant);
 std::vector<std::string> compile_options(const SkelSpec &sp);
@@ -85,6 +86,7 @@ std::vector<std::string> compile_options(const SkelSpec &sp);
 struct acc_skel_s {
   acc_context ctx = nullptr;
   acc::SkelSpec spec;
+  acc::Knobs knobs;           // what the drivers read of the tuning table
   std::string entry;
   acc::Variant variants[8];   // [0] pointers 16-byte aligned, [1] no assumption; [2], [3]: the same for the
                               // table-in-LDS form of a permute whose combination has no atomic instruction;
@@ -94,7 +96,10 @@ struct acc_skel_s {
                               // of a stencil [2], [3] and [4], [5]: half and a quarter of the columns a lane
   std::mutex mu;
 
+  // variant v compiled, loaded and measured; compiles on the calling thread unless a job for it is under way
   int ensure_variant(int v);
+  // start variant v's compilation on the worker pool (nothing if it has been started or is ready)
+  int start_variant(int v);
   bool variant_ready(int v) { std::lock_guard<std::mutex> lock(mu); return variants[v].ready; }
   int ncomp() const { return spec.comp_types.empty() ? 1 : (int)spec.comp_types.size(); }
   int vec() const { int v = 16 / (spec.vec_size > 0 ? spec.vec_size : 1); return v < 1 ? 1 : v; }

@@ -275,6 +275,10 @@ foreign import ccall safe   "acc_context_sync"    c_contextSync    :: Context ->
 -- scratch memory of the skeleton drivers: give back what is not in use / how much is held
 foreign import ccall safe   "acc_context_trim"          c_contextTrim         :: Context -> Ptr CSize -> IO Status
 foreign import ccall unsafe "acc_context_scratch_bytes" c_contextScratchBytes :: Context -> Ptr CSize -> IO Status
+-- tuning knobs: parsed once into a table, per process and per context (Debug.hs:100-140 reads its flags once, too)
+foreign import ccall safe   "acc_tuning_set"         c_tuningSet        :: CString -> IO Status
+foreign import ccall unsafe "acc_tuning_text"        c_tuningText       :: IO CString
+foreign import ccall safe   "acc_context_set_tuning" c_contextSetTuning :: Context -> CString -> IO Status
 -- tests of the failure path only
 foreign import ccall safe   "acc_context_debug_poke_lock" c_contextDebugPokeLock :: Context -> CSize -> Word32 -> IO Status
 
@@ -326,6 +330,13 @@ foreign import ccall unsafe "acc_launch_grid"         c_launchGrid        :: Int
 -- Compile.hs:444-566 + CodeGen/*: one skeleton instance per array operation
 foreign import ccall safe   "acc_skel_create"       c_skelCreate      :: Context -> Ptr SkelDesc -> Ptr Skel -> IO Status
 foreign import ccall safe   "acc_skel_destroy"      c_skelDestroy     :: Skel -> IO Status
+-- compilation on the library's worker pool; the first use of the kernel waits for it (Compile.hs:444-459,620-660)
+foreign import ccall safe   "acc_skel_create_async" c_skelCreateAsync :: Context -> Ptr SkelDesc -> Ptr Skel -> IO Status
+foreign import ccall safe   "acc_skel_wait"         c_skelWait        :: Skel -> IO Status
+foreign import ccall safe   "acc_skel_prefetch"     c_skelPrefetch    :: Skel -> CInt -> IO Status
+foreign import ccall unsafe "acc_skel_poll"         c_skelPoll        :: Skel -> Ptr CInt -> IO Status
+foreign import ccall unsafe "acc_compile_threads"   c_compileThreads  :: IO CInt
+foreign import ccall safe   "acc_compile_drain"     c_compileDrain    :: IO Status
 foreign import ccall safe   "acc_skel_source"       c_skelSource      :: Skel -> CInt -> Ptr CString -> IO Status
 foreign import ccall safe   "acc_skel_preview"      c_skelPreview     :: Ptr SkelDesc -> CInt -> Ptr CString -> Ptr CString -> IO Status
 foreign import ccall safe   "acc_skel_compile_only" c_skelCompileOnly :: CString -> Ptr SkelDesc -> Ptr CSize -> IO Status

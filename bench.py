@@ -423,13 +423,13 @@ def main():
         K = max(4, min(args.steps, 20))
 
         def front(build, sets):
-            acc_r = build(0)                        # builds the skeletons, uploads the operands of set 0
+            acc_r = acc.compute(build(0), fcx)      # builds the skeletons, uploads the operands of set 0
             for i in range(1, sets):
-                acc_r = build(i)
+                acc_r = acc.compute(build(i), fcx)
             fcx.ctx.sync()
             fcx.ctx.trace_start()                   # an event before and behind every launch the drivers make
             for k in range(K):
-                acc_r = build(k % sets)
+                acc_r = acc.compute(build(k % sets), fcx)
             launches, ms = fcx.ctx.trace_stop()
             return acc_r, round(ms * 1e3 / K, 3), launches // K
 

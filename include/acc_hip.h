@@ -118,6 +118,18 @@ int acc_context_scratch_bytes(acc_context ctx, size_t *bytes);
  * lock left at 1 makes that permute's bounded wait run out. */
 int acc_context_debug_poke_lock(acc_context ctx, size_t word, uint32_t value);
 
+/* Tuning knobs, "name=value,name=value": overrides of the defaults the skeleton generator and the drivers work with
+ * (tile shapes, thresholds between kernel forms), for measurement; the counterpart of the reference's
+ * -fflags read once at start-up (Debug.hs:100-140).  The text is parsed once into an immutable table, and no
+ * driver call ever reads the environment.  The process's table comes from ACC_HIP_TUNE in the environment when it
+ * is first wanted; acc_tuning_set replaces it (NULL: read ACC_HIP_TUNE again, now).  A context takes the process's
+ * table when it is created, acc_context_set_tuning gives it another (NULL: the process's); an instance works with
+ * the table its context had when it was created, for as long as it lives.  acc_skel_preview and
+ * acc_skel_compile_only, which have no context, use the process's table.                                     */
+int acc_tuning_set(const char *text);
+const char *acc_tuning_text(void);                  /* the process's table as text; valid until the thread's next call */
+int acc_context_set_tuning(acc_context ctx, const char *text);
+
 /* CUDA.mallocArray / free / getMemInfo: Array/Remote.hs:63-79,191 */
 int acc_malloc(acc_context ctx, size_t bytes, acc_devptr *out);
 int acc_free(acc_context ctx, acc_devptr p);
@@ -331,6 +343,33 @@ typedef struct acc_skel_desc {
  * Compile.hs:444-459,484-566, which yields the AccKernel record AST.hs:51-59. */
 int acc_skel_create(acc_context ctx, const acc_skel_desc *desc, acc_skel *out);
 int acc_skel_destroy(acc_skel s);
+
+/* The same with the compilation left to a pool of worker threads: the description is checked and the source
+ * generated before the call returns (what is wrong with either is reported here), the instance's first variant is
+ * compiled in the background, and whatever first needs the compiled kernel -- acc_exec_*, acc_skel_get_info,
+ * acc_skel_wait -- waits for it and reports a compiler failure then, with acc_compile_log() set as if the caller
+ * had compiled.  This is how the reference builds the kernels of a program: build1 forks one compilation per array
+ * operation, no more at a time than the machine has processors (Compile.hs:484-538,620-660), and the executing thread
+ * blocks where a kernel is first used (the lazy `link`, Compile.hs:444-459) -- so a program of several kernels is
+ * ready after the slowest of them, not after their sum.  acc_skel_create is this call followed by acc_skel_wait.
+ * acc_skel_poll says without waiting whether the compilation has ended (well or badly); acc_compile_threads the
+ * size the pool may grow to: the machine's processors, at most 16 unless ACC_HIP_COMPILE_THREADS in the environment
+ * says otherwise.  An instance may be destroyed while its compilation runs.                                      */
+int acc_skel_create_async(acc_context ctx, const acc_skel_desc *desc, acc_skel *out);
+int acc_skel_wait(acc_skel s);
+/* Start compiling another variant of the instance in the background (numbering as for acc_skel_preview), for a
+ * caller that knows ahead of a launch what its operands will look like -- unaligned, small, narrow; nothing happens
+ * if the variant is ready or under way.  Without it a variant other than 0 is compiled by the first call that needs
+ * it, which waits.                                                                                            */
+int acc_skel_prefetch(acc_skel s, int variant);
+int acc_skel_poll(acc_skel s, int *ready);
+int acc_compile_threads(void);
+/* Before the process exits: abandon the compilations that have not started (whoever waits for one gets
+ * ACC_ERR_COMPILE), wait for the ones that run, end the workers.  exit() tears down the compiler's static data while
+ * a worker may still be inside the compiler; a host that may exit with compilations under way calls this first (from
+ * its own at-exit hook: the reference's forked compiler threads simply die with the Haskell main thread, and its
+ * nvcc is a process of its own).  Instances created afterwards compile on the thread that first needs them.    */
+int acc_compile_drain(void);
 
 /* The generated translation unit (for -ddump-cc style debugging and tests).
  * variant 0 = aligned (128-bit accesses assumed legal), 1 = unaligned.      */

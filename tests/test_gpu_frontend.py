@@ -298,7 +298,7 @@ def test_a_working_set_larger_than_the_memory_budget(acc):
     stages = [xs]
     for k in range(1, 12):
         prev = stages[-1]
-        stages.append(acc._force(acc.map(lambda v, k=k: v * 3 + k, prev), cx))   # each stage is a manifest array that stays alive
+        stages.append(acc.compute(acc.map(lambda v, k=k: v * 3 + k, prev), cx))   # each stage is a manifest array that stays alive
     st = cx.table.stats()
     assert st["arrays"] == 12 and st["resident_bytes"] <= 64 << 20 and st["evictions"] >= 8 and st["writebacks"] >= 7
     assert st["uploads"] >= 1
@@ -320,14 +320,14 @@ def test_independent_subcomputations_run_on_their_own_streams_and_meet_by_events
     n = 1 << 22
     x, y = rng.integers(-9, 9, n).astype(np.int64), rng.integers(-9, 9, n).astype(np.int64)
     xs, ys = acc.use(x, cx), acc.use(y, cx)
-    sx = acc.scanl1(add, xs, context=cx)                       # two independent scans ...
-    sy = acc.scanr1(add, ys, context=cx)
+    sx = acc.compute(acc.scanl1(add, xs, context=cx), cx)      # two independent scans (launched now, not when asked for) ...
+    sy = acc.compute(acc.scanr1(add, ys, context=cx), cx)
     assert sx.manifest.stream is not sy.manifest.stream        # ... on two streams
-    both = acc._force(acc.zipWith(lambda a, b: a - b, sx, sy), cx)     # joins them: runs behind sx, waits for sy's event
+    both = acc.compute(acc.zipWith(lambda a, b: a - b, sx, sy), cx)     # joins them: runs behind sx, waits for sy's event
     assert both.manifest.stream is sx.manifest.stream
     chain = both
     for k in range(5):                                          # a dependent chain stays on one stream
-        chain = acc._force(acc.map(lambda v, k=k: v + k, chain), cx)
+        chain = acc.compute(acc.map(lambda v, k=k: v + k, chain), cx)
         assert chain.manifest.stream is sx.manifest.stream
     ref = np.cumsum(x) - np.cumsum(y[::-1])[::-1]
     assert np.array_equal(acc.run(chain, cx), ref + 10)
@@ -335,8 +335,8 @@ def test_independent_subcomputations_run_on_their_own_streams_and_meet_by_events
     # the same input read from two streams right after its upload was queued on the first
     z = rng.integers(-9, 9, 1 << 24).astype(np.int32)
     zs = acc.use(z, cx)
-    f1 = acc.fold(add, 0, zs, context=cx)
-    f2 = acc.fold(acc.max_, -100, acc.map(lambda v: v * 2, zs), context=cx)
+    f1 = acc.compute(acc.fold(add, 0, zs, context=cx), cx)
+    f2 = acc.compute(acc.fold(acc.max_, -100, acc.map(lambda v: v * 2, zs), context=cx), cx)
     assert f1.manifest.stream is not f2.manifest.stream and cx.table.stats()["uploads"] == 3
     assert int(acc.run(f1, cx)) == int(z.sum()) and int(acc.run(f2, cx)) == int(z.max() * 2)
 

@@ -200,10 +200,10 @@ def test_scan_int32_add(A, ctx, orc, kind):
 
 
 @pytest.mark.parametrize("small_below_kb", ["0", "2000000"])
-def test_scan_tiles_of_either_size_on_ragged_ends(A, ctx, orc, monkeypatch, small_below_kb):
+def test_scan_tiles_of_either_size_on_ragged_ends(A, ctx, orc, tuned, small_below_kb):
     """the driver takes small tiles for arrays up to 12 MB and large ones above: here each kind of tile is forced on
     sizes either side of that, with ends that fall anywhere in a vector, a row and a tile"""
-    monkeypatch.setenv("ACC_HIP_TUNE", "scan.small_below_kb=" + small_below_kb)
+    tuned("scan.small_below_kb=" + small_below_kb)
     sizes = [1, 3, 4, 5, 255, 1027, 4096, 4097, 32767, 32768, 32769, 32771, 65537, 98307, 5 * 32768 + 2, (1 << 21) + 4101]
     for kind in ("scanl", "scanl1", "scanr", "scanr1", "scanl'", "scanr'"):
         seeded = not kind.endswith("1")
@@ -403,8 +403,8 @@ def test_permute_whose_first_workgroup_copies_the_defaults(A, ctx):
     for ctype, dt in (("Int32", np.int32), ("Int64", np.int64), ("float", np.float32)):
         for combine, hint, at in (("x + y", A.COMBINE_ADD, np.add.at), ("acc_max(x, y)", A.COMBINE_MAX, np.maximum.at)):
             for tune in ("", "permute.inline_fill=0"):
-                if tune:
-                    os.environ["ACC_HIP_TUNE"] = tune
+                knobs = A.tuning(tune, ctx)
+                knobs.__enter__()
                 try:
                     sk = ctx.skeleton(A.SKEL_PERMUTE, ctype, env=[I32, (1, ctype)], out_rank=1, get="arrIn1_0[ix]", combine=combine,
                                       permutation="arrIn0_0[ix]", combine_hint=hint)
@@ -426,7 +426,7 @@ def test_permute_whose_first_workgroup_copies_the_defaults(A, ctx):
                         assert np.array_equal(acc.get(), ref.astype(dt))
                     sk.destroy()
                 finally:
-                    os.environ.pop("ACC_HIP_TUNE", None)
+                    knobs.__exit__()
 
 
 def test_permute_hinted_combines_over_windows_of_targets(A, ctx):
@@ -503,7 +503,8 @@ def test_16_bit_counts_with_large_addends_and_with_lanes_made_to_wait(A, ctx):
     dst[::9] = rng.integers(-2, bins + 2, dst[::9].size)
     src = rng.integers(-2, 8, n).astype(np.int32)
     ok = (dst >= 0) & (dst < bins)
-    os.environ["ACC_HIP_TUNE"] = "permute.narrow=2,permute.narrow_stop=32769"
+    knobs = A.tuning("permute.narrow=2,permute.narrow_stop=32769", ctx)
+    knobs.__enter__()
     try:
         say("weighted sums through 16-bit counts, waits forced")
         sk = ctx.skeleton(A.SKEL_PERMUTE, "Int32", env=[I32, I32], out_rank=1, get="arrIn1_0[ix] ", combine="x + y",
@@ -523,7 +524,7 @@ def test_16_bit_counts_with_large_addends_and_with_lanes_made_to_wait(A, ctx):
         sk.permute([ctx.array(keys)], keys.size, ctx.array(dfl), out)
         assert np.array_equal(out.get(), dfl + np.bincount(keys, minlength=bins).astype(np.int32))
     finally:
-        del os.environ["ACC_HIP_TUNE"]
+        knobs.__exit__()
 
 
 # --------------------------------------------------------------------------- stencil

@@ -67,11 +67,11 @@ def test_stencil_3d(A, ctx, mode):
 
 
 @pytest.mark.parametrize("tune", ["stencil.strips_per_cu=0", "stencil.walk_min=16", "stencil.walk_min=2"])
-def test_stencil_3d_walks_of_every_length(A, ctx, monkeypatch, tune):
+def test_stencil_3d_walks_of_every_length(A, ctx, tuned, tune):
     """the driver shortens a strip's walk through the planes on volumes as small as these (to 4 planes); here the
     full walk of 64 planes and walks of 16 and of 2 are forced on them: strips that continue one another, the last
     one short, and the narrow last strip of a row that ends at the right edge"""
-    monkeypatch.setenv("ACC_HIP_TUNE", tune)
+    tuned(tune)
     rng = np.random.default_rng(32)
     for mode in ("clamp", "wrap", "constant"):
         lap = ctx.skeleton(A.SKEL_STENCIL, "float", out_rank=3, taps=SEVEN, boundary=mode, boundary_constant="2.0f",

@@ -28,21 +28,10 @@ def ctx(A):
     c.close()
 
 
-class tuned(object):
-    """ACC_HIP_TUNE for the skeletons created inside the block (the knobs become part of the generated source)"""
-
-    def __init__(self, text):
-        self.text = text
-
-    def __enter__(self):
-        self.old = os.environ.get("ACC_HIP_TUNE")
-        os.environ["ACC_HIP_TUNE"] = self.text
-
-    def __exit__(self, *exc):
-        if self.old is None:
-            del os.environ["ACC_HIP_TUNE"]
-        else:
-            os.environ["ACC_HIP_TUNE"] = self.old
+def tuned(text, ctx):
+    """knobs for the skeletons created inside the block (they become part of the generated source)"""
+    import acchip
+    return acchip.tuning(text, ctx)
 
 
 def test_a_lock_that_never_opens_is_reported_and_cleaned_up(A, ctx):
@@ -52,7 +41,7 @@ def test_a_lock_that_never_opens_is_reported_and_cleaned_up(A, ctx):
     keys = rng.integers(0, bins, n, dtype=np.int32)
     keys[:8] = 5
     want = np.bincount(keys, minlength=bins).astype(np.int16)
-    with tuned("spin_limit=2000"):
+    with tuned("spin_limit=2000", ctx):
         sk = ctx.skeleton(A.SKEL_PERMUTE, "Int16", env=[I32], out_rank=1, get="(Int16)1", combine="(Int16)(x + y)",
                           permutation="arrIn0_0[ix]")
     dk, zero, out = ctx.array(keys), ctx.array(np.zeros(bins, np.int16)), ctx.empty(bins, np.int16)
@@ -89,7 +78,7 @@ def test_scan_and_fold_with_no_patience_still_end(A, ctx, orc):
     n = (1 << 22) + 123
     x = rng.integers(-8, 8, n, dtype=np.int32)
     dx = ctx.array(x)
-    with tuned("spin_limit=0"):
+    with tuned("spin_limit=0", ctx):
         scan0 = ctx.skeleton(A.SKEL_SCANL, "Int32", env=[I32], get="arrIn0_0[ix]", combine="x + y", seed="0")
         fold0 = ctx.skeleton(A.SKEL_FOLD, "Int32", env=[I32], out_rank=0, get="arrIn0_0[ix]", combine="x + y", seed="0")
     scan = ctx.skeleton(A.SKEL_SCANL, "Int32", env=[I32], get="arrIn0_0[ix]", combine="x + y", seed="0")

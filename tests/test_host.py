@@ -330,11 +330,18 @@ def test_generated_parameter_abi_follows_the_reference(A):
     _, src = A.preview(A.make_desc(A.SKEL_MAP, "float", env=[(1, "float")], out_rank=1, get="({ const float a = arrIn0_0[ix];\n a * a; })"))
     assert "#define ACC_GET(ix) ({ const float a = arrIn0_0[ix];  a * a; })" in src
     # tuning knobs reach the text (and so the cache key)
-    os.environ["ACC_HIP_TUNE"] = "scan.block=512,scan.rows=2"
-    try:
+    with A.tuning("scan.block=512,scan.rows=2"):
         _, src = A.preview(A.make_desc(A.SKEL_SCANL, "Int32", env=[I32], get="arrIn0_0[ix]", combine="x + y", seed="0"))
+    # ... and what the environment held when the table was first wanted is what acc_tuning_set(NULL) reads again
+    os.environ["ACC_HIP_TUNE"] = "scan.rows=3"
+    try:
+        A.check(A.lib().acc_tuning_set(None))
+        assert A.lib().acc_tuning_text().decode() == "scan.rows=3"
+        _, src3 = A.preview(A.make_desc(A.SKEL_SCANL, "Int32", env=[I32], get="arrIn0_0[ix]", combine="x + y", seed="0"))
+        assert "#define ACC_ROWS 3" in src3
     finally:
         del os.environ["ACC_HIP_TUNE"]
+        A.check(A.lib().acc_tuning_set(None))
     assert "#define ACC_BLOCK 512" in src and "#define ACC_ROWS 2" in src
 
 

@@ -3,8 +3,10 @@
 // acc_skel may be executed from several threads") exercised where data races would sit -- the scratch pool (acquire,
 // release, trim, blocks of several protocols and sizes), the lazily built second variant of a shared instance,
 // instances created and destroyed while others run, the ordering of big scans across streams, guards set on and
-// taken off streams, the status block, the memory table, the launch trace.  Launches do nothing here; the checks are
-// ThreadSanitizer's.  Exit status 0 and no report = pass.
+// taken off streams, the status block, the memory table, the launch trace; instances whose compilation runs on the
+// library's worker pool, used, waited for, polled and destroyed while it runs; a context's tuning table replaced
+// while instances are created, and a thread that keeps changing the environment meanwhile (no driver call reads
+// it).  Launches do nothing here; the checks are ThreadSanitizer's.  Exit status 0 and no report = pass.
 #include <atomic>
 #include <cstdio>
 #include <cstdlib>
@@ -37,7 +39,7 @@ static acc_array vec(uint64_t p, int64_t n)
 }
 
 static acc_skel make(acc_context ctx, int kind, const char *elt, const char *get, const char *combine, const char *seed,
-                     const char *permutation, int hint, uint32_t flags)
+                     const char *permutation, int hint, uint32_t flags, bool in_background = false)
 {
   acc_env_sig env[1];
   std::memset(env, 0, sizeof(env));
@@ -58,7 +60,8 @@ static acc_skel make(acc_context ctx, int kind, const char *elt, const char *get
   d.permutation = permutation;
   d.combine_hint = hint;
   acc_skel s = nullptr;
-  OK(acc_skel_create(ctx, &d, &s));
+  if (in_background) OK(acc_skel_create_async(ctx, &d, &s));
+  else OK(acc_skel_create(ctx, &d, &s));
   return s;
 }
 
@@ -130,6 +133,22 @@ int main(int argc, char **argv)
           OK(acc_skel_get_info(mine, &info));
           OK(acc_skel_destroy(mine));
         }
+        if (r % 10 == 3) {                      // compiled on the worker pool: used at once, or polled, or dropped while it compiles
+          static const char *bodies[] = {"arrIn0_0[ix] * 3", "arrIn0_0[ix] - 7", "arrIn0_0[ix] ^ 5", "arrIn0_0[ix] + 11"};
+          acc_skel bg = make(ctx, ACC_SKEL_MAP, "Int32", bodies[(r / 10 + t) % 4], nullptr, nullptr, nullptr, 0, 0, true);
+          if ((r / 10) % 3 == 0) {
+            acc_array m = vec(out, 1000), mi = vec(in, 1000);
+            OK(acc_exec_map(bg, &mi, &m, st));            // the first use waits for the compilation
+          } else if ((r / 10) % 3 == 1) {
+            int ready = 0;
+            OK(acc_skel_poll(bg, &ready));
+            OK(acc_skel_wait(bg));
+            OK(acc_skel_poll(bg, &ready));
+            if (!ready) failures.fetch_add(1);
+          }
+          OK(acc_skel_destroy(bg));                       // ... possibly while it still compiles
+        }
+        if (r % 17 == 9 && t == 0) OK(acc_context_set_tuning(ctx, (r & 1) ? "map.oversub=4" : ""));
         if (r % 11 == 5) {                      // the pool gives back what is not lent, while the others borrow
           size_t freed = 0, held = 0;
           OK(acc_context_trim(ctx, &freed));
@@ -161,6 +180,57 @@ int main(int argc, char **argv)
     });
   }
   for (std::thread &th : pool) th.join();
+  {
+    // Driver calls while another thread keeps changing the environment: nothing on their path may read it.  (Only
+    // calls whose variants exist by now: a compilation reads the environment inside the compiler's own library.)
+    std::atomic<bool> stop_env{false};
+    std::thread env_thread([&] {
+      for (int k = 0; !stop_env.load(); ++k) {
+        setenv("ACC_HIP_TUNE", (k & 1) ? "scan.rows=2" : "fold.unroll=2,map.unroll=2", 1);
+        setenv("ACC_HIP_DEBUG", (k & 1) ? "" : "dump-exec", 1);
+        std::this_thread::yield();
+      }
+    });
+    std::vector<std::thread> callers;
+    for (int t = 0; t < threads; ++t) {
+      callers.emplace_back([&, t] {
+        acc_stream st = nullptr;
+        OK(acc_stream_create(ctx, &st));
+        for (int r = 0; r < rounds; ++r) {
+          const int64_t n = (int64_t(1) << (10 + (r * 7 + t * 3) % 12)) + t;
+          const uint64_t off = (r % 7 == 3) ? 4 : 0;
+          acc_array a = vec(in + off, n), o = vec(out + off, n), total = vec(out, 1);
+          total.rank = 0;
+          OK(acc_exec_scan(scan, &a, n, &o, nullptr, st));
+          OK(acc_exec_fold(fold, &a, 1, &n, &total, st));
+          acc_array d = vec(zeros, 256), b = vec(bins, 256);
+          OK(acc_exec_permute(hist, &a, n, &d, &b, st));
+        }
+        OK(acc_stream_sync(ctx, st));
+        OK(acc_stream_destroy(ctx, st));
+      });
+    }
+    for (std::thread &th : callers) th.join();
+    stop_env.store(true);
+    env_thread.join();
+  }
+  {
+    // a stream that goes away takes its guard entry with it: the next stream (often the same handle value) is free of it
+    acc_stream s1 = nullptr, s2 = nullptr;
+    acc_guard g = nullptr;
+    OK(acc_stream_create(ctx, &s1));
+    OK(acc_guard_create(ctx, &g));
+    OK(acc_stream_set_guard(ctx, s1, g));
+    OK(acc_stream_destroy(ctx, s1));
+    OK(acc_stream_create(ctx, &s2));
+    acc_array m = vec(out, 1000), mi = vec(in, 1000);
+    acc_skel plain = make(ctx, ACC_SKEL_MAP, "Int32", "arrIn0_0[ix] + 2", nullptr, nullptr, nullptr, 0, 0);
+    if (s2 == s1) OK(acc_exec_map(plain, &mi, &m, s2));    // was refused: "the stream is under a guard"
+    else std::printf("(the new stream did not take the old one's handle value: guard entry not re-tested)\n");
+    OK(acc_skel_destroy(plain));
+    OK(acc_guard_destroy(g));
+    OK(acc_stream_destroy(ctx, s2));
+  }
   OK(acc_context_sync(ctx));
   OK(acc_memtable_destroy(table));
   for (acc_skel s : {scan, fold, hist, locked, gmap}) OK(acc_skel_destroy(s));
