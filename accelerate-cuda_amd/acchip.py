@@ -335,8 +335,11 @@ class DeviceArray(object):
         a.ptr[0] = self.ptr + offset_elems * self.dtype.itemsize
         return a
 
-    def get(self):
-        out = np.empty(self.shape, dtype=self.dtype)
+    def get(self, out=None):
+        """the array on the host; `out`: a C-contiguous array of the same shape and type to fill instead of a new one"""
+        if out is None:
+            out = np.empty(self.shape, dtype=self.dtype)
+        assert out.flags.c_contiguous and out.dtype == self.dtype and out.size == self.size
         if self.nbytes:
             check(lib().acc_memcpy_d2h(self.ctx.handle, out.ctypes.data_as(C.c_void_p), self.ptr, self.nbytes))
         return out

@@ -126,9 +126,26 @@ struct CompileJob {
   void run();                      // compile (through the cache) on the calling thread and mark done
   int wait();                      // block until done; the outcome, with error and log copied to the calling thread
 };
+// compilation in helper processes (compile_child.cpp): a pool thread attaches, and what it compiles from then on goes
+// to its helper; compile_out_of_process is false where there is none (the caller then compiles in process)
+void compile_child_attach();
+void compile_child_detach();
+bool compile_out_of_process(const std::string &target, const char *source, const std::vector<std::string> &options,
+                            std::vector<char> *code, std::string *log, int *rc);
+// hiprtc on the calling thread (cache.cpp): the code object, the log in the thread's compile log
+int compile_in_process(const std::string &target, const char *source, const std::vector<std::string> &options, std::vector<char> *code);
 bool compile_submit(const std::shared_ptr<CompileJob> &job);     // false: the pool has been drained, nothing was queued
 void compile_drain();
 int compile_pool_threads();
+
+// ---- staged transfers (transfer.cpp) ----------------------------------------------
+class Stager;
+void stager_destroy(acc_context ctx);
+bool wants_staging(acc_context ctx, const void *host, size_t bytes);
+// the upload is handed to the copy engine on the stager's stream `*on`, *done is recorded behind it
+int staged_upload(acc_context ctx, void *dev, const void *host, size_t bytes, hipEvent_t *done, hipStream_t *on);
+int staged_upload_wait(acc_context ctx);
+int staged_download(acc_context ctx, void *host, const void *dev, size_t bytes);     // returns with the data in `host`
 
 // the scan's descriptor block for callers that must not allocate (noalloc.hip)
 int noalloc_setup(int device);
@@ -211,6 +228,11 @@ struct acc_context_s {
     return tuning;
   }
   bool dump_exec = false;      // ACC_HIP_DEBUG=dump-exec was in the environment when the context was created
+
+  // large copies from and to pageable host memory go through pinned buffers of the context's own (transfer.cpp)
+  acc::Stager *stager = nullptr;
+  int copy_helpers = 3;                  // threads that copy beside the caller (knob copy.threads, the caller included)
+  size_t copy_staged_from = 4u << 20;    // bytes from which a pageable copy is staged (knob copy.staged_from_kb; 0 with copy.staged=0: never)
 
   // kernels report here that a bounded wait ran out (see StatusWord); NULL if the block could not be set up
   volatile uint32_t *status_host = nullptr;

@@ -172,6 +172,12 @@ int run_hiprtc(const std::string &target, const char *source, const std::vector<
 }
 
 }  // namespace
+
+int compile_in_process(const std::string &target, const char *source, const std::vector<std::string> &options, std::vector<char> *code)
+{
+  return run_hiprtc(target, source, options, code);
+}
+
 }  // namespace acc
 
 using acc::fail;
@@ -243,10 +249,16 @@ int acc_compile(acc_context ctx, const char *target, const char *source, const c
   h.field(std::to_string(rtc_major) + "." + std::to_string(rtc_minor));
   for (const std::string &o : opts) h.field(o);
   h.field("--");
-  for (const acc::EmbeddedHeader &eh : acc::embedded_headers()) {
-    h.field(eh.name);
-    h.field(std::string(eh.begin, eh.end));
-  }
+  // (the device headers enter the key through their own digest, worked out once: they are 150 KB, a source is 3)
+  static const std::string headers_digest = [] {
+    acc::Sha256 hh;
+    for (const acc::EmbeddedHeader &eh : acc::embedded_headers()) {
+      hh.field(eh.name);
+      hh.field(std::string(eh.begin, eh.end));
+    }
+    return hh.hex();
+  }();
+  h.field(headers_digest);
   h.field(source);
   const std::string key = tgt + "/" + h.hex() + ".co";
 
@@ -279,7 +291,15 @@ int acc_compile(acc_context ctx, const char *target, const char *source, const c
   if (!from_disk) {
     // the lock is not held while compiling: several threads may compile at
     // once, as the reference's worker pool does (Compile.hs:620-660)
-    ACC_TRY(acc::run_hiprtc(tgt, source, opts, payload.get()));
+    // (a thread of the worker pool hands the job to its helper process: hiprtc takes one program at a time per process)
+    int crc = ACC_OK;
+    std::string clog;
+    if (acc::compile_out_of_process(tgt, source, opts, payload.get(), &clog, &crc)) {
+      acc::set_compile_log(clog);
+      if (crc != ACC_OK) return fail(crc, "run-time compilation failed; see acc_compile_log()");
+    } else {
+      ACC_TRY(acc::run_hiprtc(tgt, source, opts, payload.get()));
+    }
     if (!path.empty() && !acc::write_entry(dir + "/" + tgt, path, *payload)) disk_error = true;
   } else {
     acc::set_compile_log("");

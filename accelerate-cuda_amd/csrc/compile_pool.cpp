@@ -117,6 +117,8 @@ class Pool {
 
   void work()
   {
+    compile_child_attach();                 // this thread's compilations run in a helper process of its own
+    struct Detach { ~Detach() { compile_child_detach(); } } detach;
     for (;;) {
       std::shared_ptr<CompileJob> job;
       {

@@ -122,7 +122,9 @@ struct acc_memtable_s {
     if (e.uploaded) { ACC_HIP_TRY(hipEventSynchronize(e.uploaded)); upload_settled(e); }
     if (e.status == DIRTY || !keep) ACC_TRY(settle(e.uses));
     if (e.status == DIRTY) {
-      ACC_HIP_TRY(hipMemcpy(e.host, e.dev, e.bytes, hipMemcpyDeviceToHost));
+      // (every use of the block has been waited for above: nothing the copy must be ordered behind)
+      if (wants_staging(ctx, e.host, e.bytes)) ACC_TRY(staged_download(ctx, e.host, e.dev, e.bytes));
+      else ACC_HIP_TRY(hipMemcpy(e.host, e.dev, e.bytes, hipMemcpyDeviceToHost));
       st.writebacks++;
       st.writeback_bytes += e.bytes;
     }
@@ -297,10 +299,19 @@ int acc_memtable_acquire(acc_memtable mt, uint64_t key, acc_stream stream, acc_d
     }
     if (e.bytes) {
       hipStream_t s = static_cast<hipStream_t>(stream);
-      ACC_HIP_TRY(hipMemcpyAsync(e.dev, e.host, e.bytes, hipMemcpyHostToDevice, s));
       mt->upload_settled(e);
       ACC_TRY(mt->event(&e.uploaded));
-      ACC_HIP_TRY(hipEventRecord(e.uploaded, s));
+      if (wants_staging(mt->ctx, e.host, e.bytes)) {
+        // through the context's pinned buffers, on its copy stream: every stream that wants the array, this one
+        // included, waits for the event recorded there (below)
+        hipStream_t on = nullptr;
+        ACC_TRY(staged_upload(mt->ctx, e.dev, e.host, e.bytes, nullptr, &on));
+        ACC_HIP_TRY(hipEventRecord(e.uploaded, on));
+        s = on;
+      } else {
+        ACC_HIP_TRY(hipMemcpyAsync(e.dev, e.host, e.bytes, hipMemcpyHostToDevice, s));
+        ACC_HIP_TRY(hipEventRecord(e.uploaded, s));
+      }
       e.upload_stream = s;
       mt->st.uploads++;
       mt->st.upload_bytes += e.bytes;

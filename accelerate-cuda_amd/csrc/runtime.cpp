@@ -374,6 +374,8 @@ int acc_context_create(int device, acc_context *out)
     }
   }
   ctx->tuning = acc::default_tuning();
+  ctx->copy_helpers = std::max(1, ctx->tuning->get("copy.threads", 4)) - 1;
+  ctx->copy_staged_from = ctx->tuning->get("copy.staged", 1) ? (size_t)std::max(1, ctx->tuning->get("copy.staged_from_kb", 4096)) << 10 : ~size_t(0);
   {
     const char *dbg = std::getenv("ACC_HIP_DEBUG");      // looked at here, never on the path of a launch
     ctx->dump_exec = dbg && std::strstr(dbg, "dump-exec");
@@ -390,6 +392,7 @@ int acc_context_destroy(acc_context ctx)
   if (!ctx) return ACC_OK;
   (void)hipSetDevice(ctx->device);
   (void)hipDeviceSynchronize();
+  acc::stager_destroy(ctx);
   for (acc::ScratchBlock &b : ctx->scratch) {
     if (b.done) (void)hipEventDestroy(b.done);
     if (b.ptr) (void)hipFree(b.ptr);
@@ -533,11 +536,28 @@ static int copy(acc_context ctx, void *dst, const void *src, size_t bytes, hipMe
   return ACC_OK;
 }
 
-int acc_memcpy_h2d(acc_context c, acc_devptr d, const void *s, size_t n) { return copy(c, reinterpret_cast<void *>(d), s, n, hipMemcpyHostToDevice, nullptr, false); }
+// The blocking copies keep the ordering of a copy on the default stream -- behind the work queued there before, done
+// when the call returns -- also where they are staged through the context's pinned buffers on a stream of its own.
+int acc_memcpy_h2d(acc_context c, acc_devptr d, const void *s, size_t n)
+{
+  if (c && d && s && n && acc::wants_staging(c, s, n)) {
+    ACC_TRY(c->make_current());
+    ACC_HIP_TRY(hipStreamSynchronize(nullptr));
+    ACC_TRY(acc::staged_upload(c, reinterpret_cast<void *>(d), s, n, nullptr, nullptr));
+    return acc::staged_upload_wait(c);
+  }
+  return copy(c, reinterpret_cast<void *>(d), s, n, hipMemcpyHostToDevice, nullptr, false);
+}
 int acc_memcpy_d2h(acc_context c, void *d, acc_devptr s, size_t n)
 {
   // (a blocking copy to the host is where most callers first look at a result: a kernel's report is returned here too)
-  ACC_TRY(copy(c, d, reinterpret_cast<void *>(s), n, hipMemcpyDeviceToHost, nullptr, false));
+  if (c && d && s && n && acc::wants_staging(c, d, n)) {
+    ACC_TRY(c->make_current());
+    ACC_HIP_TRY(hipStreamSynchronize(nullptr));
+    ACC_TRY(acc::staged_download(c, d, reinterpret_cast<void *>(s), n));
+  } else {
+    ACC_TRY(copy(c, d, reinterpret_cast<void *>(s), n, hipMemcpyDeviceToHost, nullptr, false));
+  }
   return c->check_status("acc_memcpy_d2h");
 }
 int acc_memcpy_d2d(acc_context c, acc_devptr d, acc_devptr s, size_t n) { return copy(c, reinterpret_cast<void *>(d), reinterpret_cast<void *>(s), n, hipMemcpyDeviceToDevice, nullptr, false); }

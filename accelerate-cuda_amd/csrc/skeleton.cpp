@@ -944,16 +944,20 @@ int acc_skel_compile_only(const char *target, const acc_skel_desc *desc, size_t 
   acc::SkelSpec sp;
   ACC_TRY(acc::make_spec(desc, acc::default_tuning(), &sp));
   std::vector<std::string> opts = acc::compile_options(sp);
-  std::vector<const char *> optp;
-  for (const std::string &o : opts) optp.push_back(o.c_str());
+  // both variants at once, on the worker pool (a helper process each)
   size_t total = 0;
+  std::shared_ptr<acc::CompileJob> jobs[2];
   for (int v = 0; v < 2; ++v) {
-    std::string entry, src;
-    ACC_TRY(acc::generate_source(sp, v == 0, &entry, &src));
-    const void *code = nullptr;
-    size_t size = 0;
-    ACC_TRY(acc_compile(nullptr, target, src.c_str(), optp.data(), static_cast<int>(optp.size()), &code, &size));
-    total += size;
+    std::string entry;
+    jobs[v] = std::make_shared<acc::CompileJob>();
+    ACC_TRY(acc::generate_source(sp, v == 0, &entry, &jobs[v]->source));
+    jobs[v]->target = target;
+    jobs[v]->options = opts;
+    if (!acc::compile_submit(jobs[v])) jobs[v]->run();
+  }
+  for (int v = 0; v < 2; ++v) {
+    ACC_TRY(jobs[v]->wait());
+    total += jobs[v]->size;
   }
   if (code_size) *code_size = total;
   return ACC_OK;

@@ -95,21 +95,41 @@ def cpu_leg(fn, what, bytes_per_call, budget_s=3.0):
 
 def end_to_end(ctx, uploads, run, download, reps=3):
     """what the reference's `run1` does around its kernels (CUDA.hs:382-389, Execute.hs:146-154): the operands go from
-    pageable host memory to the device, the kernels run, the result comes back.  `uploads` pairs device arrays with the
-    host arrays they take; best of `reps`."""
-    best = None
-    for _ in range(reps):
-        ctx.sync()
-        t0 = time.perf_counter()
-        for d, h in uploads:
-            d.set(h)
-        run()
-        out = download.get()
-        dt = time.perf_counter() - t0
-        best = dt if best is None else min(best, dt)
-    moved = sum(h.nbytes for _, h in uploads) + out.nbytes
-    return {"ms": round(best * 1e3, 3), "host_bytes_moved": int(moved),
-            "note": "H2D of the operands from pageable memory + kernels + D2H of the result, device buffers reused; not the headline"}
+    pageable host memory to the device, the kernels run, the result comes back into pageable host memory.  `uploads`
+    pairs device arrays with the host arrays they take; best of `reps`.  Timed twice: with the library's staged
+    transfers (pinned buffers of its own, chunks copied by a few threads while the copy engine moves the chunks before
+    them), and with the runtime's own copies from and to pageable memory (a second context with `copy.staged=0`)."""
+    import acchip as A
+    L = A.lib()
+    plain = getattr(end_to_end, "plain", None)
+    if plain is None:
+        with A.tuning("copy.staged=0"):
+            plain = end_to_end.plain = A.Context(ctx.device)
+    first = download.get()
+    host_out = np.empty_like(first)
+    host_out[...] = 0                               # its pages exist: the timed copies do not pay for their first touch
+    res = {}
+    for name, handle in (("staged", ctx.handle), ("runtime_pageable", plain.handle)):
+        best = None
+        for _ in range(reps):
+            ctx.sync()
+            t0 = time.perf_counter()
+            for d, h in uploads:
+                A.check(L.acc_memcpy_h2d(handle, d.ptr, h.ctypes.data_as(C.c_void_p), h.nbytes))
+            run()
+            src = download.where() if hasattr(download, "where") else download
+            A.check(L.acc_stream_sync(ctx.handle, end_to_end.stream))
+            A.check(L.acc_memcpy_d2h(handle, host_out.ctypes.data_as(C.c_void_p), src.ptr, src.nbytes))
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        res[name] = best
+    assert np.array_equal(host_out, download.get()), "end to end: the staged and the plain copy disagree"
+    moved = sum(h.nbytes for _, h in uploads) + host_out.nbytes
+    return {"ms": round(res["staged"] * 1e3, 3), "host_bytes_moved": int(moved),
+            "GB_per_s_over_the_link": round(moved / res["staged"] / 1e9, 2),
+            "runtime_pageable_ms": round(res["runtime_pageable"] * 1e3, 3),
+            "runtime_pageable_GB_per_s": round(moved / res["runtime_pageable"] / 1e9, 2),
+            "note": "H2D of the operands from pageable memory + kernels + D2H of the result into pageable memory, device buffers reused; not the headline"}
 
 
 def profiled_traffic(kernel):
@@ -169,6 +189,7 @@ def main():
     props = ctx.props()
     log("device: arch %s, %d CUs, LDS/workgroup %d, L2 %d" % (props.arch.decode(), props.compute_units, props.lds_per_block, props.l2_bytes))
     stream = ctx.stream()
+    end_to_end.stream = stream
     T = Timer(A, ctx, stream, args.steps, args.warmup)
 
     def traced(steps, calls=12):
@@ -355,8 +376,12 @@ def main():
 
         class _where(object):              # the result of the ten applications lies in a or in b
             @staticmethod
+            def where():
+                return b_s[0] if rib.value else a_s[0]
+
+            @staticmethod
             def get():
-                return (b_s[0] if rib.value else a_s[0]).get()
+                return _where.where().get()
         sk["gaussian3x3_clamp_x10"]["end_to_end"] = end_to_end(ctx, [(a_s[0], img)], step(0), _where)
         if not args.no_cpu:
             from oracle import oracle as orc
@@ -396,18 +421,148 @@ def main():
                             {"nnz": int(nnz), "GFLOP_per_s": round(2 * nnz / (e * 1e-3) / 1e9, 1),
                              "note": "segment offsets precomputed on the device (scanl over the 2^20 lengths is not in the step)",
                              "traffic_key": "foldSeg", "one_by_one_us": smvm_one_by_one})
-        sk["smvm"]["end_to_end"] = end_to_end(ctx, [(dv[0], vals), (dc[0], cols), (dxv[0], xv), (doff[0], offs)], step(0), ys[0])
-        if not args.no_cpu:
-            from oracle import oracle as orc
-            orc.build()
-            sk["smvm"]["cpu_baseline"] = cpu_leg(lambda: orc.smvm_f32(vals, cols, offs, xv), "oracle/acc_oracle.c orc_smvm_f32, full 2^20 rows",
-                                                 nnz * 8 + rows * 8 + xv.size * 4)
         # composition check on the device result: y = A x in float64 within 1e-4 of the row's magnitude
         import scipy.sparse as sp
         Amat = sp.csr_matrix((vals.astype(np.float64), cols, offs), shape=(rows, xv.size))
         truth = Amat @ xv.astype(np.float64)
         mag = abs(Amat) @ np.abs(xv.astype(np.float64))
         assert np.all(np.abs(y.get() - truth) <= 1e-4 * np.maximum(np.abs(truth), 1e-3 * mag) + 1e-30), "smvm mismatch"
+        # What bounds it: the same kernel with the product left out (the gather of x alone: one request to the L2 per
+        # non-zero, whatever else the kernel does) and with the gather replaced by a linear read (the kernel's own
+        # structure at the speed of a stream).  The L2s answer a request per channel and clock at best:
+        # 8 XCDs x 16 channels x the L2 clock; the gathers are held against that.
+        legs = {}
+        for leg, get in (("gather_only", "arrIn2_0[" + rd(1) + "]"), ("linear_read_instead_of_gather", rd(0) + " * (float)" + rd(1))):
+            sk_leg = ctx.skeleton(A.SKEL_FOLDSEG, "float", env=[F32, I32, F32], get=get, combine="x + y", seed="0.0f")
+
+            def step_leg(i, sk_leg=sk_leg):
+                return lambda: A.check(L.acc_exec_foldseg(sk_leg.handle, env_s[i], nnz, C.byref(offd[i]), C.byref(yd[i]), stream))
+            wl_, el_ = T.run([step_leg(i) for i in range(S)])
+            legs[leg] = round(el_ * 1e3, 3)
+            log("  %-28s %9.3f us/launch" % ("smvm, " + leg.replace("_", " "), el_ * 1e3))
+        l2_clock_ghz = 2.1                                  # the L2s' clock on this part (the shader clock is 2.4 GHz at its peak)
+        req_peak = 8 * 16 * l2_clock_ghz * 1e9              # requests a second at one a channel and clock
+        req_rate = nnz / (sk["smvm"]["avg_launch_us"] * 1e-6)
+        sk["smvm"].update({
+            "gather_floor_us": legs["gather_only"], "linear_read_us": legs["linear_read_instead_of_gather"],
+            "over_gather_floor": round(sk["smvm"]["avg_launch_us"] / legs["gather_only"], 3),
+            "roofline_l2_requests": {"bound": "l2_requests", "achieved": round(req_rate / 1e9, 1), "peak": round(req_peak / 1e9, 1),
+                                     "unit": "G requests/s", "frac": round(req_rate / req_peak, 3),
+                                     "note": "one 4-byte gather of x per non-zero = one request to an L2 channel; peak = 8 XCDs x 16 channels x %.1f GHz" % l2_clock_ghz}})
+        sk["smvm"]["end_to_end"] = end_to_end(ctx, [(dv[0], vals), (dc[0], cols), (dxv[0], xv), (doff[0], offs)], step(0), ys[0])
+        if not args.no_cpu:
+            from oracle import oracle as orc
+            orc.build()
+            sk["smvm"]["cpu_baseline"] = cpu_leg(lambda: orc.smvm_f32(vals, cols, offs, xv), "oracle/acc_oracle.c orc_smvm_f32, full 2^20 rows",
+                                                 nnz * 8 + rows * 8 + xv.size * 4)
+    # ---------------------------------------------------------------- what a first `run` costs, and what a call costs the host
+    if want("startup"):
+        log("start-up: compilation cold, from the disk cache, from memory; two kernels one after the other and side by side ...")
+        nonce = "// %d.%d" % (os.getpid(), time.time_ns())
+        st = {}
+
+        def build(name, k, wait=True, **kw):
+            t0 = time.perf_counter()
+            skx = ctx.skeleton(*kw.pop("args"), preamble="%s %s %d" % (nonce, name, k), wait=wait, **kw)
+            return skx, (time.perf_counter() - t0) * 1e3
+        kinds = {
+            "scanl": dict(args=(A.SKEL_SCANL, "Int32"), env=[I32], get=rd(0), combine="x + y", seed="0"),
+            "dot": dict(args=(A.SKEL_FOLD, "float"), env=[F32, F32], out_rank=0, get=rd(0) + " * " + rd(1), combine="x + y", seed="0.0f"),
+            "histogram": dict(args=(A.SKEL_PERMUTE, "Int32"), env=[I32], out_rank=1, get="1", combine="x + y", permutation=rd(0), combine_hint=A.COMBINE_ADD),
+            "gaussian3x3": dict(args=(A.SKEL_STENCIL, "float"), out_rank=2, taps=[(dy, dx) for dy in (-1, 0, 1) for dx in (-1, 0, 1)], boundary="clamp",
+                                stencil_fn=A.linear_stencil_fn([1, 2, 1, 2, 4, 2, 1, 2, 1], 16)),
+            "smvm": dict(args=(A.SKEL_FOLDSEG, "float"), env=[F32, I32, F32], get=rd(0) + " * arrIn2_0[" + rd(1) + "]", combine="x + y", seed="0.0f"),
+        }
+        for name, kw in kinds.items():
+            _, cold = build(name, 0, **dict(kw))                  # generated, compiled by hiprtc, loaded
+            A.check(L.acc_cache_clear(0))                         # forget what memory holds, keep the files
+            _, disk = build(name, 0, **dict(kw))
+            _, ram = build(name, 0, **dict(kw))
+            st[name] = {"cold_compile_ms": round(cold, 1), "disk_cache_load_ms": round(disk, 2), "ram_hit_us": round(ram * 1e3, 1)}
+            log("  %-14s cold %8.1f ms   from the disk cache %6.2f ms   from memory %7.1f us" % (name, cold, disk, ram * 1e3))
+        # the SMVM program's two kernels (the scan that makes the offsets, the segmented fold): compiled one after the
+        # other, as acc_skel_create does, and side by side on the worker pool, as the front end's `run` has them
+        t0 = time.perf_counter()
+        build("pair", 1, **dict(kinds["scanl"]))
+        build("pair", 1, **dict(kinds["smvm"]))
+        serial = (time.perf_counter() - t0) * 1e3
+        t0 = time.perf_counter()
+        a_, _ = build("pair", 2, wait=False, **dict(kinds["scanl"]))
+        b_, _ = build("pair", 2, wait=False, **dict(kinds["smvm"]))
+        submitted = (time.perf_counter() - t0) * 1e3
+        a_.wait()
+        b_.wait()
+        together = (time.perf_counter() - t0) * 1e3
+        st["two_kernels"] = {"one_after_the_other_ms": round(serial, 1), "side_by_side_ms": round(together, 1),
+                             "returned_to_the_caller_after_ms": round(submitted, 2), "compile_threads": int(L.acc_compile_threads())}
+        log("  scanl + foldSeg: one after the other %.1f ms, side by side %.1f ms (the caller had both handles after %.2f ms)" % (serial, together, submitted))
+        sk["startup"] = st
+
+    if want("hostcost"):
+        log("host time of a driver call (enqueue only) and small arrays ...")
+        hc = {}
+        small = 1024
+        xs_ = ctx.array(np.arange(small, dtype=np.int32) % 7)
+        o1, o2, tot = ctx.empty(small + 1, np.int32), ctx.empty(256, np.int32), ctx.empty((), np.int32)
+        zero = ctx.array(np.zeros(256, np.int32))
+        e1 = envs(xs_)
+        m_ = ctx.skeleton(A.SKEL_MAP, "Int32", env=[I32], out_rank=1, get="arrIn0_0[ix] + 1", wait=True)
+        f_ = ctx.skeleton(A.SKEL_FOLD, "Int32", env=[I32], out_rank=0, get="arrIn0_0[ix]", combine="x + y", seed="0", wait=True)
+        s_ = ctx.skeleton(A.SKEL_SCANL, "Int32", env=[I32], get="arrIn0_0[ix]", combine="x + y", seed="0", wait=True)
+        p_ = ctx.skeleton(A.SKEL_PERMUTE, "Int32", env=[I32], out_rank=1, get="1", combine="x + y", permutation="arrIn0_0[ix]", combine_hint=A.COMBINE_ADD, wait=True)
+        od1, od1s, od2, zd, td = o1.desc(shape=(small,)), o1.desc(), o2.desc(), zero.desc(), tot.desc()
+        sh1 = (C.c_int64 * 1)(small)
+        calls = {
+            "map": lambda: L.acc_exec_map(m_.handle, e1, C.byref(od1), stream),
+            "fold": lambda: L.acc_exec_fold(f_.handle, e1, 1, sh1, C.byref(td), stream),
+            "scan": lambda: L.acc_exec_scan(s_.handle, e1, small, C.byref(od1s), None, stream),
+            "permute": lambda: L.acc_exec_permute(p_.handle, e1, small, C.byref(zd), C.byref(od2), stream),
+        }
+        empty_call = lambda: L.acc_launch_grid(1, 1, 1, 1)          # what a call through ctypes costs by itself
+        reps = 3000
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            empty_call()
+        ffi_us = (time.perf_counter() - t0) * 1e6 / reps
+        for name, call in calls.items():
+            for _ in range(200):
+                call()
+            ctx.sync()
+            # host time: bursts short enough for the queue to take without the device having to catch up
+            host_us = None
+            for _ in range(12):
+                t0 = time.perf_counter()
+                for _ in range(128):
+                    call()
+                dt = (time.perf_counter() - t0) * 1e6 / 128
+                host_us = dt if host_us is None else min(host_us, dt)
+                ctx.sync()
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                call()
+            ctx.sync()
+            total_us = (time.perf_counter() - t0) * 1e6 / reps
+            hc[name] = {"host_us_per_call": round(host_us, 2), "of_which_the_python_binding_us": round(ffi_us, 2),
+                        "us_per_call_until_the_device_is_done": round(total_us, 2), "elements": small}
+            log("  %-8s %6.2f us of host time a call (%.2f of them the ctypes call itself); %6.2f us a call with the device's work" % (name, host_us, ffi_us, total_us))
+        # small arrays: device time a call, back to back
+        rows = {}
+        for lg in (10, 12, 14, 16, 18):
+            nn = 1 << lg
+            xa, oa = ctx.array(np.arange(nn, dtype=np.int32) % 7), ctx.empty(nn + 1, np.int32)
+            ea, oda, odas = envs(xa), oa.desc(shape=(nn,)), oa.desc()
+            sha = (C.c_int64 * 1)(nn)
+            per = {}
+            for name, call in (("map", lambda: A.check(L.acc_exec_map(m_.handle, ea, C.byref(oda), stream))),
+                               ("fold", lambda: A.check(L.acc_exec_fold(f_.handle, ea, 1, sha, C.byref(td), stream))),
+                               ("scan", lambda: A.check(L.acc_exec_scan(s_.handle, ea, nn, C.byref(odas), None, stream))),
+                               ("permute", lambda: A.check(L.acc_exec_permute(p_.handle, ea, nn, C.byref(zd), C.byref(od2), stream)))):
+                w_, e_ = T.run([call])
+                per[name] = round(e_ * 1e3, 2)
+            rows["2^%d" % lg] = per
+            log("  n = 2^%-2d  us a call on the device, back to back: %s" % (lg, "  ".join("%s %.2f" % kv for kv in per.items())))
+        hc["small_arrays_us_per_call"] = rows
+        sk["host_cost"] = hc
 
     # ---------------------------------------------------------------- the same three computations built by the front end
     # (dot, scanl and SMVM written as array programs: what `run1` of the front end generates, compiles and launches

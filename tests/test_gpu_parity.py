@@ -935,12 +935,20 @@ def test_stencils_of_every_element_width(A, ctx):
     wraps in the element type; Float64 on small integers is exact)"""
     five = [(-1, 0), (0, -1), (0, 0), (0, 1), (1, 0)]
     seven = [(0, 0, 0), (-1, 0, 0), (1, 0, 0), (0, -1, 0), (0, 1, 0), (0, 0, -1), (0, 0, 1)]
-    for ctype, dt in (("Int8", np.int8), ("Word16", np.uint16), ("Int64", np.int64), ("double", np.float64)):
+    types = (("Int8", np.int8), ("Word16", np.uint16), ("Int64", np.int64), ("double", np.float64))
+    sks = {}
+    for ctype, dt in types:                             # all twenty instances first: they compile side by side
+        cast = "(%s)" % ctype
+        for mode in ("clamp", "mirror", "wrap", "constant"):
+            sks[ctype, mode] = ctx.skeleton(A.SKEL_STENCIL, ctype, out_rank=2, taps=five, boundary=mode, boundary_constant=cast + "2",
+                                            stencil_fn=cast + "(t0 + 2 * t1 - t2 + t3 + t4)").prefetch(range(1, 6))
+        sks[ctype, 3] = ctx.skeleton(A.SKEL_STENCIL, ctype, out_rank=3, taps=seven, boundary="mirror",
+                                     stencil_fn=cast + "(t0 + t1 + t2 + t3 + t4 + t5 + 2 * t6)").prefetch(range(1, 6))
+    for ctype, dt in types:
         cast = "(%s)" % ctype
         wide = (lambda a: a) if ctype == "double" else (lambda a: a.astype(np.int64))
         for mode in ("clamp", "mirror", "wrap", "constant"):
-            sk = ctx.skeleton(A.SKEL_STENCIL, ctype, out_rank=2, taps=five, boundary=mode, boundary_constant=cast + "2",
-                              stencil_fn=cast + "(t0 + 2 * t1 - t2 + t3 + t4)")
+            sk = sks[ctype, mode]
             for shape in ((5, 7), (33, 300), (7, 1031)):
                 say("stencil of", ctype, mode, shape)
                 v = rng.integers(0, 5, shape).astype(dt)
@@ -948,8 +956,7 @@ def test_stencils_of_every_element_width(A, ctx):
                 sk.stencil([], ctx.array(v), out)
                 t = [wide(a) for a in pyref.tap_arrays(v, five, mode, 2, shape)]
                 assert np.array_equal(out.get(), (t[0] + 2 * t[1] - t[2] + t[3] + t[4]).astype(dt))
-        sk = ctx.skeleton(A.SKEL_STENCIL, ctype, out_rank=3, taps=seven, boundary="mirror",
-                          stencil_fn=cast + "(t0 + t1 + t2 + t3 + t4 + t5 + 2 * t6)")
+        sk = sks[ctype, 3]
         for shape in ((3, 5, 7), (4, 9, 1031)):
             say("3-D stencil of", ctype, shape)
             v = rng.integers(0, 5, shape).astype(dt)
@@ -964,11 +971,15 @@ def test_right_handed_scans_of_every_element_width(A, ctx):
     boundaries and sizes that are no multiple of a vector (the rounding positions of the first vector)"""
     def rscan(x):                                           # inclusive from the right, in the element type
         return np.cumsum(x[::-1], dtype=x.dtype)[::-1]
-    for ctype, dt in (("Int8", np.int8), ("Word16", np.uint16), ("Int32", np.int32), ("Int64", np.int64), ("double", np.float64)):
+    types = (("Int8", np.int8), ("Word16", np.uint16), ("Int32", np.int32), ("Int64", np.int64), ("double", np.float64))
+    sks = {}
+    for ctype, dt in types:                             # all fifteen instances first, small tiles too: they compile side by side
         lit = "3.0" if ctype == "double" else "3"
-        r0 = ctx.skeleton(A.SKEL_SCANR, ctype, env=[(1, ctype)], get="arrIn0_0[ix]", combine="(%s)(x + y)" % ctype, seed=lit)
-        r1 = ctx.skeleton(A.SKEL_SCANR1, ctype, env=[(1, ctype)], get="arrIn0_0[ix]", combine="(%s)(x + y)" % ctype)
-        rp = ctx.skeleton(A.SKEL_SCANRP, ctype, env=[(1, ctype)], get="arrIn0_0[ix]", combine="(%s)(x + y)" % ctype, seed=lit)
+        sks[ctype] = (ctx.skeleton(A.SKEL_SCANR, ctype, env=[(1, ctype)], get="arrIn0_0[ix]", combine="(%s)(x + y)" % ctype, seed=lit).prefetch([2]),
+                      ctx.skeleton(A.SKEL_SCANR1, ctype, env=[(1, ctype)], get="arrIn0_0[ix]", combine="(%s)(x + y)" % ctype).prefetch([2]),
+                      ctx.skeleton(A.SKEL_SCANRP, ctype, env=[(1, ctype)], get="arrIn0_0[ix]", combine="(%s)(x + y)" % ctype, seed=lit).prefetch([2]))
+    for ctype, dt in types:
+        r0, r1, rp = sks[ctype]
         tile = r1.info().elements_per_block
         for n in (1, 3, 17, tile - 1, tile, tile + 1, 3 * tile + 5, 300007):
             say("right-handed scans of", ctype, "n =", n)

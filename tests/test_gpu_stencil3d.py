@@ -44,6 +44,8 @@ def test_stencil_3d(A, ctx, mode):
                        stencil_fn="t1 + t2 + t3 + t4 + t5 + t6 - 6.0f * t0")
     box = ctx.skeleton(A.SKEL_STENCIL, "float", out_rank=3, taps=BOX, boundary=mode, boundary_constant="2.0f",
                        stencil_fn=" + ".join("(float)%d * t%d" % (k % 5 - 2, k) for k in range(27)))
+    lap.prefetch(range(1, 6))                          # the shapes below take every variant: they compile side by side
+    box.prefetch(range(1, 6))
     for shape in SHAPES:
         if mode == "mirror" and min(shape) < 2:
             continue                                   # the index maps assume the array spans the stencil
@@ -141,10 +143,14 @@ def test_stencil_3d_strip_edges_of_narrow_elements(A, ctx):
     """what a strip reads just outside its 256 columns comes from another lane's register: elements narrower than
     a register (Int8, Word16) at widths of several strips, first plane included, every boundary mode"""
     rng = np.random.default_rng(34)
+    sks = {}
+    for ctype, T in (("Int8", np.int8), ("Word16", np.uint16)):     # the eight instances compile side by side
+        for mode in ("clamp", "mirror", "wrap", "constant"):
+            sks[ctype, mode] = ctx.skeleton(A.SKEL_STENCIL, ctype, out_rank=3, taps=BOX, boundary=mode, boundary_constant="(%s)3" % ctype,
+                                            stencil_fn="(%s)(%s)" % (ctype, " + ".join("t%d" % k for k in range(27)))).prefetch([1])
     for ctype, T in (("Int8", np.int8), ("Word16", np.uint16)):
         for mode in ("clamp", "mirror", "wrap", "constant"):
-            sk = ctx.skeleton(A.SKEL_STENCIL, ctype, out_rank=3, taps=BOX, boundary=mode, boundary_constant="(%s)3" % ctype,
-                              stencil_fn="(%s)(%s)" % (ctype, " + ".join("t%d" % k for k in range(27))))
+            sk = sks[ctype, mode]
             for shape in ((2, 4, 256), (4, 9, 1031), (66, 6, 512)):
                 say("stencil 3-D", ctype, mode, shape)
                 v = rng.integers(0, 4, shape).astype(T)

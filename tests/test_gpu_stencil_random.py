@@ -41,7 +41,8 @@ def near(rng, mult, hi):
 @pytest.mark.parametrize("rank", [1, 2, 3])
 def test_random_stencils(A, ctx, rank):
     rng = np.random.default_rng(1000 + rank)
-    for trial in range(10 if rank < 3 else 14):
+    trials = []
+    for trial in range(10 if rank < 3 else 14):          # every instance first: they compile side by side, variants included
         ctype, T = TYPES[int(rng.integers(0, len(TYPES)))]
         mode = str(rng.choice(["clamp", "mirror", "wrap", "constant"]))
         reach = [int(rng.integers(0, 3)) for _ in range(rank)]
@@ -60,6 +61,9 @@ def test_random_stencils(A, ctx, rank):
         fn = " + ".join("(%s)(%d) * t%d" % (ctype, c, k) for k, c in enumerate(coef))
         sk = ctx.skeleton(A.SKEL_STENCIL, ctype, out_rank=rank, taps=taps if rank > 1 else [(0, t[0]) for t in taps],
                           boundary=mode, boundary_constant="(%s)2" % ctype, stencil_fn="(%s)(%s)" % (ctype, fn) if whole else fn)
+        sk.prefetch(range(1, 6))
+        trials.append((ctype, T, mode, reach, taps, coef, whole, sk))
+    for ctype, T, mode, reach, taps, coef, whole, sk in trials:
         for _ in range(2):
             shape = [near(rng, 256, 1100) if rng.random() < 0.7 else int(rng.integers(1, 80))]
             if rank >= 2:
@@ -91,6 +95,7 @@ def test_stencils_on_arrays_narrower_than_a_strip(A, ctx, rank):
     and 4 columns, every boundary mode, elements of 1, 4 and 8 bytes."""
     rng = np.random.default_rng(2000 + rank)
     widths = [4, 5, 6, 7, 9, 63, 64, 66, 100, 129, 131, 202, 253, 254, 255, 256 + 65, 256 + 130, 512 + 70]
+    cases = []
     for (ctype, T), mode, rx in itertools.product([("Int8", np.int8), ("float", np.float32), ("double", np.float64)],
                                                   ["clamp", "mirror", "wrap", "constant"], [1, 2, 4]):
         if rank == 3 and (rx == 4 or (ctype == "double" and (rx != 1 or mode in ("mirror", "wrap"))) or
@@ -105,6 +110,9 @@ def test_stencils_on_arrays_narrower_than_a_strip(A, ctx, rank):
         fn = " + ".join("(%s)(%d) * t%d" % (ctype, c, k) for k, c in enumerate(coef))
         sk = ctx.skeleton(A.SKEL_STENCIL, ctype, out_rank=rank, taps=taps, boundary=mode, boundary_constant="(%s)2" % ctype,
                           stencil_fn="(%s)(%s)" % (ctype, fn) if whole else fn)
+        sk.prefetch(range(1, 6))                                   # every width below: every variant is wanted
+        cases.append((ctype, T, mode, rx, taps, coef, whole, sk))
+    for ctype, T, mode, rx, taps, coef, whole, sk in cases:        # (the instances have been compiling side by side)
         for w in widths:
             if w < rx + 1:
                 continue                                           # the index maps assume the array spans the stencil

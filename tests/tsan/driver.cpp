@@ -163,6 +163,18 @@ int main(int argc, char **argv)
           OK(acc_memtable_release(table, key, st));
           OK(acc_memtable_free(table, key));
         }
+        if (r % 25 == 8) {                      // copies large enough to be staged through the context's pinned buffers
+          static thread_local std::vector<char> big(9u << 20, 1);
+          OK(acc_memcpy_h2d(ctx, in, big.data(), big.size()));
+          OK(acc_memcpy_d2h(ctx, big.data(), in, big.size()));
+          const uint64_t key = (uint64_t(t) << 32) | uint64_t(r) | (1ull << 60);
+          int is_new = 0;
+          acc_devptr p = 0;
+          OK(acc_memtable_malloc(table, key, big.data(), big.size(), 1, &is_new));
+          OK(acc_memtable_acquire(table, key, st, &p));
+          OK(acc_memtable_release(table, key, st));
+          OK(acc_memtable_free(table, key));
+        }
         if (r % 13 == 6) {
           OK(acc_trace_start(ctx));
           acc_array o2 = vec(out, 5000), a2 = vec(in, 5000);

@@ -57,6 +57,7 @@ hipError_t hipMalloc(void **p, size_t n) { *p = std::malloc(n ? n : 1); return *
 hipError_t hipFree(void *p) { std::free(p); return hipSuccess; }
 hipError_t hipHostMalloc(void **p, size_t n, unsigned) { *p = std::calloc(1, n ? n : 1); return *p ? hipSuccess : hipErrorOutOfMemory; }
 hipError_t hipHostFree(void *p) { std::free(p); return hipSuccess; }
+hipError_t hipPointerGetAttributes(hipPointerAttribute_t *, const void *) { return hipErrorInvalidValue; }    // every host address is pageable here
 hipError_t hipHostGetDevicePointer(void **d, void *h, unsigned) { *d = h; return hipSuccess; }
 hipError_t hipMemGetInfo(size_t *f, size_t *t) { *f = size_t(1) << 35; *t = size_t(1) << 36; return hipSuccess; }
 // (copies and fills are not carried out: two threads of the driver may name the same "device" buffers, as two
