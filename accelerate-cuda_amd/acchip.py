@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libacchip.so")
 CSRC = os.path.join(_HERE, "csrc")
 
 OK, ERR_INVALID, ERR_OOM, ERR_COMPILE, ERR_NOT_FOUND, ERR_HIP, ERR_UNSUPPORTED, ERR_IO, ERR_STUCK = range(9)
-MAX_RANK, MAX_COMP = 8, 8
+MAX_RANK, MAX_COMP = 8, 16
 
 (SKEL_MAP, SKEL_GENERATE, SKEL_TRANSFORM, SKEL_FOLD, SKEL_FOLD1, SKEL_FOLDSEG, SKEL_FOLD1SEG,
  SKEL_SCANL, SKEL_SCANL1, SKEL_SCANLP, SKEL_SCANR, SKEL_SCANR1, SKEL_SCANRP, SKEL_PERMUTE,
@@ -59,7 +59,8 @@ class acc_skel_desc(C.Structure):
                 ("stencil_fn", C.c_char_p), ("stencil_in_type", C.c_char_p), ("seg_type", C.c_char_p),
                 ("boundary2", C.c_int32), ("boundary2_constant", C.c_char_p), ("n_taps2", C.c_int32),
                 ("tap2_dy", C.POINTER(C.c_int32)), ("tap2_dx", C.POINTER(C.c_int32)), ("stencil_in2_type", C.c_char_p),
-                ("tap_dz", C.POINTER(C.c_int32)), ("tap2_dz", C.POINTER(C.c_int32))]
+                ("tap_dz", C.POINTER(C.c_int32)), ("tap2_dz", C.POINTER(C.c_int32)),
+                ("tap_offsets", C.POINTER(C.c_int32)), ("tap2_offsets", C.POINTER(C.c_int32))]
 
 
 class acc_device_props(C.Structure):
@@ -228,7 +229,11 @@ def make_desc(kind, elt, env=(), out_rank=0, get=None, combine=None, seed=None, 
     d.permutation, d.combine_hint = _b(permutation), combine_hint
     d.boundary = BOUNDARY[boundary] if isinstance(boundary, str) else boundary
     d.boundary_constant = _b(boundary_constant)
-    if taps is not None:
+    if taps is not None and len(taps[0]) > 3:          # any rank: rows of offsets, outermost dimension first
+        flat = (C.c_int32 * (len(taps) * len(taps[0])))(*[o for t in taps for o in t])
+        keep.append(flat)
+        d.n_taps, d.tap_offsets = len(taps), flat
+    elif taps is not None:
         dy = (C.c_int32 * len(taps))(*[t[-2] for t in taps])
         dx = (C.c_int32 * len(taps))(*[t[-1] for t in taps])
         keep += [dy, dx]
@@ -238,7 +243,11 @@ def make_desc(kind, elt, env=(), out_rank=0, get=None, combine=None, seed=None, 
             keep.append(dz)
             d.tap_dz = dz
     d.stencil_fn, d.stencil_in_type, d.seg_type = _b(stencil_fn), _b(stencil_in), _b(seg_type)
-    if taps2 is not None:       # stencil2: the second source
+    if taps2 is not None and len(taps2[0]) > 3:
+        flat2 = (C.c_int32 * (len(taps2) * len(taps2[0])))(*[o for t in taps2 for o in t])
+        keep.append(flat2)
+        d.n_taps2, d.tap2_offsets = len(taps2), flat2
+    elif taps2 is not None:       # stencil2: the second source
         dy2 = (C.c_int32 * len(taps2))(*[t[-2] for t in taps2])
         dx2 = (C.c_int32 * len(taps2))(*[t[-1] for t in taps2])
         keep += [dy2, dx2]

@@ -254,6 +254,8 @@ struct acc_context_s {
   // follow the block's protocol
   int scratch_acquire(size_t bytes, hipStream_t stream, int protocol, acc::ScratchRef *out);
   void scratch_release(const acc::ScratchRef &ref, hipStream_t stream);
+  // a borrower could not leave a SCRATCH_LOCKS / SCRATCH_CARRY block as it found it: cleared before it is lent again
+  void scratch_mark_dirty(const acc::ScratchRef &ref);
   // free every block that is not lent and whose last use has completed; returns the bytes given back
   size_t scratch_trim();
   size_t scratch_bytes();

@@ -463,11 +463,16 @@ ACC_ENTRY(ACC_ENV_PARAMS
           ACC_OUT_ARRAY(arrSum),
           const Int64 shIn_0,
           void *desc0, void *desc1, void *desc2,
-          const unsigned int epoch, const Int64 num_tiles, unsigned int *acc_status ACC_GUARD_PARAM)
+          const unsigned int epoch_given, const Int64 num_tiles, unsigned int *acc_status ACC_GUARD_PARAM)
 {
   ACC_GUARD_CHECK
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
+  /* The launch's tag: what the host chose for this launch, or -- 0 given -- what the first word of the 256-byte header
+   * in front of the descriptors holds, put there by a kernel that ran just before on the same stream.  A launch
+   * recorded into a graph keeps its arguments for every replay; its tag must not be among them, or the descriptors
+   * the replay before left behind would read as published. */
+  const unsigned int epoch = epoch_given ? epoch_given : *(const unsigned int *)((const char *)desc0 - 256);
 #if ACC_ALIGNED
   ACC_OUT_ASSUME(arrOut)
 #endif

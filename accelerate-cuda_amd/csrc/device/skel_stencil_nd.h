@@ -1,0 +1,109 @@
+/*
+ * skel_stencil_nd.h -- stencils of any rank and reach, an element of the result a thread.
+ *
+ * Takes the place of CodeGen/Stencil.hs:55-114 as it stands there: the linear index of the element is taken apart
+ * into the index of every dimension (cfromIndex, CodeGen/Base.hs:207-218), every tap adds its offsets, the
+ * boundary condition is applied dimension by dimension (Stencil/Extra.hs:158-226) and the source is read at the
+ * row-major position of the result (ctoIndex, Base.hs:193-202).  skel_stencil.h keeps the rows a strip needs in
+ * registers, which is written for up to three dimensions and for offsets a register window can hold; this template
+ * serves what lies beyond that -- arrays of rank 4 and more, taps further than 2 planes or 4 rows or columns away --
+ * and leaves the reuse of neighbouring elements to the caches, as the reference does.  Same entry names, same
+ * parameters (the strip kernel's `acc_walk` is taken and ignored), same results.
+ *
+ * Generated definitions expected: ACC_ELT, ACC_ENV_PARAMS, ACC_ENV_ASSUME, ACC_OUT_PARAMS, ACC_STENCIL_RANK,
+ * ACC_OUT_EXTENTS (shOut_<rank-1>, ..., shOut_0), ACC_STENCIL_SOURCES (1|2), ACC_STENCIL_FN, ACC_BLOCK and per
+ * source n = 1, 2: ACC_BOUNDARY (ACC_BOUNDARY2), ACC_SRC<n>_COMPONENTS(X, arg), ACC_SRC<n>_PARAMS,
+ * ACC_SRC<n>_EXTENTS (the source's own extents, outermost first), ACC_IN<n>_ELT, ACC_STENCIL_TAPS<n>_ND(READ) with
+ * READ(component, offset of the outermost dimension, ..., offset of the innermost).
+ */
+
+#define ACC_B_CLAMP 0
+#define ACC_B_MIRROR 1
+#define ACC_B_WRAP 2
+#define ACC_B_CONSTANT 3
+
+struct acc_nd_index { Int64 i[ACC_STENCIL_RANK]; };
+struct acc_nd_offset { int o[ACC_STENCIL_RANK]; };
+
+template <int MODE>
+ACC_DEV Int64 acc_nd_boundary(Int64 i, const Int64 sz)
+{
+  if (MODE == ACC_B_CLAMP)  i = acc_max<Int64>(0, acc_min<Int64>(i, sz - 1));
+  if (MODE == ACC_B_MIRROR) i = i < 0 ? -i : (i >= sz ? sz - (i - sz + 2) : i);
+  if (MODE == ACC_B_WRAP)   i = i < 0 ? sz + i : (i >= sz ? i - sz : i);
+  /* the maps assume the array spans the stencil; keep the address legal if not */
+  return acc_max<Int64>(0, acc_min<Int64>(i, sz - 1));
+}
+
+/* the element of `base` (extents `sh`) at `at` + `off`, under the boundary condition; `outside` beyond a constant boundary */
+template <int MODE, typename S>
+ACC_DEV S acc_nd_read(const S *__restrict__ base, const acc_nd_index &sh, const acc_nd_index &at, const acc_nd_offset &off, const S outside)
+{
+  Int64 lin = 0;
+  bool inside = true;
+#pragma unroll
+  for (int d = 0; d < ACC_STENCIL_RANK; ++d) {
+    const Int64 i = at.i[d] + off.o[d];
+    if (MODE == ACC_B_CONSTANT) inside = inside && i >= 0 && i < sh.i[d];
+    lin = lin * sh.i[d] + acc_nd_boundary<MODE>(i, sh.i[d]);
+  }
+  const S v = base[lin];
+  return (MODE == ACC_B_CONSTANT && !inside) ? outside : v;
+}
+
+#if ACC_STENCIL_SOURCES == 2
+#define ACC_STENCIL_ENTRY stencil2
+#define ACC_SOURCE_PARAMS ACC_SRC1_PARAMS ACC_SRC2_PARAMS
+#define ACC_SRC1_ARRAY(c) arrStencil1_##c
+#define ACC_SRC2_ARRAY(c) arrStencil2_##c
+#else
+#define ACC_STENCIL_ENTRY stencil
+#define ACC_SOURCE_PARAMS ACC_SRC1_PARAMS
+#define ACC_SRC1_ARRAY(c) arrStencil_##c
+#define ACC_SRC2_COMPONENTS(X, arg)
+#endif
+
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS, const int acc_walk ACC_GUARD_PARAM)
+{
+  ACC_GUARD_CHECK
+  typedef ACC_ELT T;
+  ACC_ENV_ASSUME
+  (void)acc_walk;
+  const acc_nd_index sh = {{ACC_OUT_EXTENTS}};
+  const acc_nd_index sh1 = {{ACC_SRC1_EXTENTS}};
+#if ACC_STENCIL_SOURCES == 2
+  const acc_nd_index sh2 = {{ACC_SRC2_EXTENTS}};
+#endif
+  Int64 n = 1;
+#pragma unroll
+  for (int d = 0; d < ACC_STENCIL_RANK; ++d) n *= sh.i[d];
+  /* the value outside a constant boundary, component by component */
+#define ACC_DECLARE_OUTSIDE1(c, CT, OUTSIDE, arg) const CT acc_outside1_##c = (CT)OUTSIDE;
+#define ACC_DECLARE_OUTSIDE2(c, CT, OUTSIDE, arg) const CT acc_outside2_##c = (CT)OUTSIDE;
+  ACC_SRC1_COMPONENTS(ACC_DECLARE_OUTSIDE1, 0)
+  ACC_SRC2_COMPONENTS(ACC_DECLARE_OUTSIDE2, 0)
+#undef ACC_DECLARE_OUTSIDE1
+#undef ACC_DECLARE_OUTSIDE2
+
+  for (Int64 ix = (Int64)blockIdx.x * ACC_BLOCK + threadIdx.x; ix < n; ix += (Int64)gridDim.x * ACC_BLOCK) {
+    acc_nd_index at;
+    Int64 rest = ix;
+#pragma unroll
+    for (int d = ACC_STENCIL_RANK - 1; d > 0; --d) {      /* innermost dimension last: Base.hs:207-218 */
+      at.i[d] = rest % sh.i[d];
+      rest /= sh.i[d];
+    }
+    at.i[0] = rest;
+#define ACC_ND_READ1(c, ...) acc_nd_read<ACC_BOUNDARY>(ACC_SRC1_ARRAY(c), sh1, at, acc_nd_offset{{__VA_ARGS__}}, acc_outside1_##c)
+    ACC_STENCIL_TAPS1_ND(ACC_ND_READ1)
+#undef ACC_ND_READ1
+#if ACC_STENCIL_SOURCES == 2
+#define ACC_ND_READ2(c, ...) acc_nd_read<ACC_BOUNDARY2>(ACC_SRC2_ARRAY(c), sh2, at, acc_nd_offset{{__VA_ARGS__}}, acc_outside2_##c)
+    ACC_STENCIL_TAPS2_ND(ACC_ND_READ2)
+#undef ACC_ND_READ2
+#endif
+    const T r = (T)(ACC_STENCIL_FN);
+    ACC_PUT(arrOut, ix, r);
+  }
+}

@@ -25,6 +25,7 @@ ACC_EMBED(foldseg, "device/skel_foldseg.h")
 ACC_EMBED(scan, "device/skel_scan.h")
 ACC_EMBED(permute, "device/skel_permute.h")
 ACC_EMBED(stencil, "device/skel_stencil.h")
+ACC_EMBED(stencil_nd, "device/skel_stencil_nd.h")
 
 namespace acc {
 
@@ -39,6 +40,7 @@ const std::vector<EmbeddedHeader> &embedded_headers()
       {"skel_scan.h", acc_embed_scan_begin, acc_embed_scan_end},
       {"skel_permute.h", acc_embed_permute_begin, acc_embed_permute_end},
       {"skel_stencil.h", acc_embed_stencil_begin, acc_embed_stencil_end},
+      {"skel_stencil_nd.h", acc_embed_stencil_nd_begin, acc_embed_stencil_nd_end},
   };
   return headers;
 }

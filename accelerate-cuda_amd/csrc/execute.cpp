@@ -829,6 +829,7 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
     args.ptr(ncarry);
     args.ptr(s->ctx->status_dev);
     nrc = launch(s, nv, ngrid, nlds, st, &args);
+    const bool main_launched = nrc == ACC_OK;
     if (nrc == ACC_OK) {
       Args m;
       bool mal = true;
@@ -848,6 +849,8 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
         if (me != hipSuccess) nrc = acc::fail_hip(me, "hipModuleLaunchKernel(permute_merge, narrow counts)");
       }
     }
+    // (the merge clears the carries it reads: if the main kernel went out and the merge did not, they stay behind)
+    if (nrc != ACC_OK && main_launched) s->ctx->scratch_mark_dirty(cblk);
     s->ctx->scratch_release(cblk, st);
     s->ctx->scratch_release(nblk, st);
     return nrc;
@@ -1067,7 +1070,15 @@ static int stencil_once(acc_skel s, const acc_array *env, const acc_array *in, c
     bool ignore = true;
     push_ptrs(in, in->ncomp, &args, &ignore);
   }
-  if (w == 0 || h == 0 || planes == 0) return ACC_OK;
+  if (array_size(*out) == 0) return ACC_OK;
+  if (s->spec.stencil_nd) {
+    // an element of the result a thread (skel_stencil_nd.h); the kernel takes the strips' `walk` and ignores it
+    args.i32(0);
+    const int v = aligned ? 0 : 1;
+    ACC_TRY(s->ensure_variant(v));
+    const int64_t grid = acc_launch_grid(array_size(*out), s->spec.block, resident(s, v), s->knobs.map_oversub);
+    return launch(s, v, grid, 0, st, &args);
+  }
   // one wave per strip of 256 columns x tile_h rows
   // (for 2-D the waves of a workgroup are stacked vertically, so the row count is rounded up to whole groups)
   const int64_t waves = s->spec.block / 64;

@@ -16,10 +16,23 @@ static __device__ __align__(256) unsigned char scratch[ACC_NOALLOC_SCRATCH_BYTES
 
 namespace {
 
-// zero `words` 8-byte words from p on (a kernel, not a memset node, so that a caller may capture the launch)
-__global__ void __launch_bounds__(256) acc_noalloc_clear(unsigned long long *p, size_t words)
+// The tag of the next scan: one more than the last one's, kept in the first word of the array's header and read from
+// there by the scan kernel (a launch recorded into a graph carries the same arguments on every replay, so the tag
+// cannot be one of them: this kernel is recorded in front of the scan and counts on the device).  When the 30 bits a
+// descriptor has for its tag run out, the descriptors are cleared and the count starts again -- here too, not on the
+// host, and by stores of a kernel, not by a memset node.
+__global__ void __launch_bounds__(256) acc_noalloc_next_tag(unsigned int *header, unsigned long long *desc, size_t words)
 {
-  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < words; i += (size_t)gridDim.x * 256) p[i] = 0ull;
+  __shared__ unsigned int next;
+  if (threadIdx.x == 0) next = header[0] + 1u;
+  __syncthreads();
+  const unsigned int tag = next;
+  if (tag >= (1u << 30)) {
+    for (size_t i = threadIdx.x; i < words; i += 256) desc[i] = 0ull;
+    if (threadIdx.x == 0) header[0] = 1u;
+  } else if (threadIdx.x == 0) {
+    header[0] = tag;
+  }
 }
 
 constexpr int MAX_DEVICES = 64;
@@ -29,7 +42,6 @@ struct DeviceScratch {
   bool asked = false;
   hipError_t status = hipErrorNotInitialized;
   void *ptr = nullptr;        // the array's address on this device
-  uint32_t epoch = 0;         // tag of the last scan that used it (acc::SCRATCH_SCAN: stale tags read as "not yet")
 };
 DeviceScratch g_dev[MAX_DEVICES];
 
@@ -65,14 +77,13 @@ int noalloc_scan_state(int device, size_t bytes, hipStream_t stream, void **base
   if (bytes > (size_t)ACC_NOALLOC_SCRATCH_BYTES)
     return fail(ACC_ERR_INVALID, "acc_exec_scan_noalloc: %zu bytes of tile descriptors needed, the scratch array holds %d", bytes,
                 (int)ACC_NOALLOC_SCRATCH_BYTES);
-  if (d.epoch + 1 >= (1u << 30)) {            // descriptor tags are 30 bits wide: start over from a clean block
-    hipLaunchKernelGGL(acc_noalloc_clear, dim3(64), dim3(256), 0, stream, static_cast<unsigned long long *>(d.ptr),
-                       (size_t)ACC_NOALLOC_SCRATCH_BYTES / 8);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return fail_hip(e, "acc_noalloc_clear");
-    d.epoch = 0;
-  }
-  *epoch = ++d.epoch;
+  // the launch's tag is counted on the device, by a kernel in front of the scan on the same stream (so that a graph
+  // that records both gets a fresh tag at every replay); the scan is told to look there by a tag of 0
+  hipLaunchKernelGGL(acc_noalloc_next_tag, dim3(1), dim3(256), 0, stream, static_cast<unsigned int *>(d.ptr),
+                     reinterpret_cast<unsigned long long *>(static_cast<char *>(d.ptr) + 256), ((size_t)ACC_NOALLOC_SCRATCH_BYTES - 256) / 8);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail_hip(e, "acc_noalloc_next_tag");
+  *epoch = 0;
   *base = d.ptr;
   return ACC_OK;
 }

@@ -182,6 +182,13 @@ void acc_context_s::scratch_release(const acc::ScratchRef &ref, hipStream_t stre
   b.busy = false;
 }
 
+void acc_context_s::scratch_mark_dirty(const acc::ScratchRef &ref)
+{
+  if (ref.index < 0) return;
+  std::lock_guard<std::mutex> lock(mu);
+  scratch[ref.index].dirty = true;
+}
+
 size_t acc_context_s::scratch_bytes()
 {
   std::lock_guard<std::mutex> lock(mu);

@@ -278,6 +278,62 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
     case ACC_SKEL_STENCIL2: {
       const bool two = sp.kind == ACC_SKEL_STENCIL2;
       *entry = two ? "stencil2" : "stencil";
+      if (sp.stencil_nd) {
+        // an element a thread, any rank and reach (skel_stencil_nd.h)
+        const int rank = sp.out_rank;
+        o << "#define ACC_OUT_PARAMS " << out_params(rank, sp.elt_type) << "\n";
+        o << "#define ACC_STENCIL_RANK " << rank << "\n";
+        o << "#define ACC_STENCIL_SOURCES " << (two ? 2 : 1) << "\n";
+        o << "#define ACC_OUT_EXTENTS";
+        for (int dd = rank - 1; dd >= 0; --dd) o << " shOut_" << dd << (dd ? "," : "");
+        o << "\n";
+        auto source_nd = [&](const char *which, const char *tap_name, const std::string &elt_name, const std::vector<std::string> &comps,
+                             const std::string &constant, const std::vector<int> &off, const char *array_name, bool with_extents) -> int {
+          const int nc = (int)comps.size();
+          std::vector<std::string> consts = split_top_level(constant);
+          if (consts.empty() || (consts.size() == 1 && consts[0].empty())) consts.assign(nc, "0");
+          if ((int)consts.size() != nc)
+            return fail(ACC_ERR_INVALID, "stencil: the boundary constant has %d component(s), the source element has %d", (int)consts.size(), nc);
+          o << "#define ACC_SRC" << which << "_COMPONENTS(X, arg)";
+          for (int i = 0; i < nc; ++i) o << " X(" << (nc - 1 - i) << ", " << comps[i] << ", (" << consts[i] << "), arg)";
+          o << "\n";
+          o << "#define ACC_SRC" << which << "_PARAMS";
+          if (with_extents)
+            for (int dd = rank - 1; dd >= 0; --dd) o << " , const Int64 sh" << array_name << "_" << dd;
+          for (int i = 0; i < nc; ++i) o << " , const " << comps[i] << " *__restrict__ arr" << array_name << "_" << (nc - 1 - i);
+          o << "\n";
+          // a stencil's one source has the result's extents; each source of a stencil2 its own
+          o << "#define ACC_SRC" << which << "_EXTENTS";
+          for (int dd = rank - 1; dd >= 0; --dd) o << " sh" << (with_extents ? array_name : "Out") << "_" << dd << (dd ? "," : "");
+          o << "\n";
+          o << "#define ACC_IN" << which << "_ELT " << (nc == 1 ? comps[0] : elt_name) << "\n";
+          o << "#define ACC_STENCIL_TAPS" << which << "_ND(READ) ";
+          const size_t ntaps = off.size() / (size_t)rank;
+          for (size_t k = 0; k < ntaps; ++k) {
+            o << "const ACC_IN" << which << "_ELT " << tap_name << k << " = ";
+            if (nc > 1) o << "{ ";
+            for (int i = 0; i < nc; ++i) {
+              o << (i ? ", " : "") << "READ(" << (nc - 1 - i);
+              for (int dd = 0; dd < rank; ++dd) o << ", " << off[k * rank + dd];
+              o << ")";
+            }
+            if (nc > 1) o << " }";
+            o << "; ";
+          }
+          o << "\n";
+          return ACC_OK;
+        };
+        ACC_TRY(source_nd("1", "t", "acc_in1_elt", sp.stencil_in_comps, sp.boundary_constant, sp.tap_off, two ? "Stencil1" : "Stencil", two));
+        o << "#define ACC_BOUNDARY " << sp.boundary << "\n";
+        if (two) {
+          o << "#define ACC_BOUNDARY2 " << sp.boundary2 << "\n";
+          ACC_TRY(source_nd("2", "u", "acc_in2_elt", sp.stencil_in2_comps, sp.boundary2_constant, sp.tap2_off, "Stencil2", true));
+        }
+        o << "#define ACC_STENCIL_FN " << sp.stencil_fn << "\n";
+        o << "#define ACC_BLOCK " << sp.block << "\n";
+        tmpl = "skel_stencil_nd.h";
+        break;
+      }
       int rz = 0, ry = 0, rx = 0;
       for (size_t k = 0; k < sp.tap_dy.size(); ++k) {
         rz = std::max(rz, std::abs(sp.tap_dz[k]));
@@ -551,23 +607,41 @@ int make_spec(const acc_skel_desc *d, const TuningPtr &tuning, SkelSpec *sp)
       break;
     case ACC_SKEL_STENCIL:
     case ACC_SKEL_STENCIL2: {
-      if (sp->out_rank < 1 || sp->out_rank > 3) return fail(ACC_ERR_UNSUPPORTED, "stencil: rank %d not supported (1, 2 and 3 are)", sp->out_rank);
+      if (sp->out_rank < 1) return fail(ACC_ERR_INVALID, "stencil: rank %d", sp->out_rank);
       if (!d->stencil_fn || !*d->stencil_fn) return fail(ACC_ERR_INVALID, "stencil: `stencil_fn` fragment missing");
-      auto taps = [&](int n, const int32_t *dzs, const int32_t *dys, const int32_t *dxs, int boundary, std::vector<int> *oz,
-                      std::vector<int> *oy, std::vector<int> *ox) -> int {
-        if (n < 1 || n > 125 || !dxs) return fail(ACC_ERR_INVALID, "stencil: bad tap list");
+      // The taps of one source: as rows of out_rank offsets (`offs`, any rank), or as up to three lists (dz, dy, dx).
+      // Either way they end up in both forms: (oz, oy, ox) for the strips of skel_stencil.h, `all` for the template
+      // that takes any rank and reach, and `beyond` says that only the latter will do.
+      const int rank = sp->out_rank;
+      bool beyond = rank > 3 || tune("stencil.nd", 0) != 0;
+      auto taps = [&](int n, const int32_t *offs, const int32_t *dzs, const int32_t *dys, const int32_t *dxs, int boundary,
+                      std::vector<int> *oz, std::vector<int> *oy, std::vector<int> *ox, std::vector<int> *all) -> int {
+        // (a 9 x 9 x 9 neighbourhood, the widest the array language's stencil patterns describe in three dimensions)
+        if (n < 1 || n > 729 || (!offs && !dxs)) return fail(ACC_ERR_INVALID, "stencil: bad tap list");
+        if (!offs && rank > 3) return fail(ACC_ERR_INVALID, "stencil: a stencil of rank %d gives its taps as `tap_offsets`", rank);
         if (boundary < ACC_BOUNDARY_CLAMP || boundary > ACC_BOUNDARY_CONSTANT) return fail(ACC_ERR_INVALID, "stencil: bad boundary %d", boundary);
         for (int k = 0; k < n; ++k) {
-          const int dy = (sp->out_rank >= 2 && dys) ? dys[k] : 0;
-          const int dz = (sp->out_rank == 3 && dzs) ? dzs[k] : 0;
-          if (std::abs(dy) > 4 || std::abs(dxs[k]) > 4 || std::abs(dz) > 2) return fail(ACC_ERR_UNSUPPORTED, "stencil: tap offset beyond 4 (2 across planes)");
+          int o[ACC_MAX_RANK] = {0};
+          if (offs) {
+            for (int dd = 0; dd < rank; ++dd) o[dd] = offs[k * rank + dd];
+          } else {
+            o[rank - 1] = dxs[k];
+            if (rank >= 2) o[rank - 2] = dys ? dys[k] : 0;
+            if (rank == 3) o[0] = dzs ? dzs[k] : 0;
+          }
+          for (int dd = 0; dd < rank; ++dd) {
+            if (std::abs(o[dd]) > 64) return fail(ACC_ERR_INVALID, "stencil: a tap %d elements away", o[dd]);
+            all->push_back(o[dd]);
+          }
+          const int dx = o[rank - 1], dy = rank >= 2 ? o[rank - 2] : 0, dz = rank == 3 ? o[0] : 0;
+          if (std::abs(dy) > 4 || std::abs(dx) > 4 || std::abs(dz) > 2) beyond = true;      // more than a strip's register windows hold
           oz->push_back(dz);
           oy->push_back(dy);
-          ox->push_back(dxs[k]);
+          ox->push_back(dx);
         }
         return ACC_OK;
       };
-      ACC_TRY(taps(d->n_taps, d->tap_dz, d->tap_dy, d->tap_dx, d->boundary, &sp->tap_dz, &sp->tap_dy, &sp->tap_dx));
+      ACC_TRY(taps(d->n_taps, d->tap_offsets, d->tap_dz, d->tap_dy, d->tap_dx, d->boundary, &sp->tap_dz, &sp->tap_dy, &sp->tap_dx, &sp->tap_off));
       sp->boundary = d->boundary;
       sp->boundary_constant = flat(d->boundary_constant);
       sp->stencil_fn = flat(d->stencil_fn);
@@ -582,13 +656,20 @@ int make_spec(const acc_skel_desc *d, const TuningPtr &tuning, SkelSpec *sp)
       };
       ACC_TRY(in_comps(sp->stencil_in_type, &sp->stencil_in_comps, "stencil_in_type"));
       if (d->kind == ACC_SKEL_STENCIL2) {
-        ACC_TRY(taps(d->n_taps2, d->tap2_dz, d->tap2_dy, d->tap2_dx, d->boundary2, &sp->tap2_dz, &sp->tap2_dy, &sp->tap2_dx));
+        ACC_TRY(taps(d->n_taps2, d->tap2_offsets, d->tap2_dz, d->tap2_dy, d->tap2_dx, d->boundary2, &sp->tap2_dz, &sp->tap2_dy, &sp->tap2_dx, &sp->tap2_off));
         sp->boundary2 = d->boundary2;
         sp->boundary2_constant = flat(d->boundary2_constant);
         sp->stencil_in2_type = (d->stencil_in2_type && *d->stencil_in2_type) ? d->stencil_in2_type : sp->elt_type;
         ACC_TRY(in_comps(sp->stencil_in2_type, &sp->stencil_in2_comps, "stencil_in2_type"));
       }
       sp->block = tune("stencil.block", 256);
+      sp->stencil_nd = beyond;
+      if (sp->stencil_nd) {              // an element a thread: no strips to shape
+        sp->svec = 1;
+        sp->tile_w = sp->block;
+        sp->tile_h = 1;
+        break;
+      }
       // Columns a lane holds of every row: four, or two of an element of 8 bytes -- one 128-bit access either way, and
       // half the registers for the row windows, so that strips stay as tall as for narrower elements (Float64, 3 x 3
       // on 8192^2: 202.7 -> 174.6 us; 7 points on 256 x 512 x 512: 249.5 -> 190.3) -- unless the stencil reaches
@@ -701,7 +782,7 @@ SkelSpec spec_of_variant(const SkelSpec &base, int v)
   if (spec.kind != ACC_SKEL_PERMUTE && v >= 2 && spec.chunk_long > 0) spec.chunk = spec.chunk_long;
   // a stencil's variants 2 and 3, 4 and 5: half and a quarter of the columns a lane, for arrays narrower than half or a
   // quarter of a strip, whose lanes would otherwise mostly lie outside the array
-  if ((spec.kind == ACC_SKEL_STENCIL || spec.kind == ACC_SKEL_STENCIL2) && v >= 2) {
+  if ((spec.kind == ACC_SKEL_STENCIL || spec.kind == ACC_SKEL_STENCIL2) && v >= 2 && !spec.stencil_nd) {
     spec.svec = std::max(1, spec.svec >> (v / 2));
     spec.tile_w = 64 * spec.svec;
   }
@@ -827,7 +908,7 @@ int acc_skel_s::ensure_variant(int v)
 static int variant_count(const acc::SkelSpec &sp)
 {
   const bool stencil = sp.kind == ACC_SKEL_STENCIL || sp.kind == ACC_SKEL_STENCIL2;
-  return sp.kind == ACC_SKEL_PERMUTE ? 8 : (stencil ? 6 : ((sp.scan_small_rows > 0 || sp.chunk_long > 0) ? 4 : 2));
+  return sp.kind == ACC_SKEL_PERMUTE ? 8 : (stencil ? (sp.stencil_nd ? 2 : 6) : ((sp.scan_small_rows > 0 || sp.chunk_long > 0) ? 4 : 2));
 }
 
 extern "C" {

@@ -38,6 +38,8 @@ struct SkelSpec {
   int boundary2 = 0;
   std::string boundary2_constant, stencil_in2_type;
   std::vector<int> tap2_dz, tap2_dy, tap2_dx;
+  bool stencil_nd = false;              // an element a thread (skel_stencil_nd.h): rank > 3, or taps further away than the strips' windows hold
+  std::vector<int> tap_off, tap2_off;   // ... its taps: n_taps rows of out_rank offsets, outermost dimension first
   int tile_w = 256, tile_h = 4, prefetch = 3;
   int svec = 4;                         // stencils: columns a lane holds of every row (tile_w = 64 of them)
   int reach_x = 0;                      // stencils: the furthest a tap reaches to either side

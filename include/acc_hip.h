@@ -213,7 +213,7 @@ int64_t acc_launch_grid(int64_t n, int64_t per_block, int64_t cus, int64_t block
  * ========================================================================= */
 
 #define ACC_MAX_RANK 8
-#define ACC_MAX_COMP 8
+#define ACC_MAX_COMP 16     /* components of a (flattened) tuple element: Accelerate's tuples have up to 15 */
 
 /* A device-resident array as the kernels see it: extents outermost first
  * (row-major, innermost dimension last: CodeGen/Base.hs:193-202) and one
@@ -336,6 +336,12 @@ typedef struct acc_skel_desc {
   /* rank-3 stencils: the taps' offsets across planes (NULL = all in the focus' plane) */
   const int32_t     *tap_dz;
   const int32_t     *tap2_dz;
+  /* stencils of any rank (Stencil.hs:55-114 serves every rank through cfromIndex, Base.hs:207-218): the taps'
+   * offsets as n_taps rows of out_rank numbers, outermost dimension first.  Where given, tap_dz / tap_dy / tap_dx
+   * are not read; required for out_rank > 3.  (Offsets of up to 2 planes and 4 rows and columns in up to three
+   * dimensions run on strips of rows held in registers; anything else an element a thread, as the reference does.) */
+  const int32_t     *tap_offsets;
+  const int32_t     *tap2_offsets;
 } acc_skel_desc;
 
 /* Generate + compile (through the cache) + load one skeleton instance and
@@ -444,7 +450,13 @@ int acc_exec_scan(acc_skel s, const acc_array *env, int64_t n, const acc_array *
  *     an eighth the size) or more.  acc_skel_create loads the one for large aligned arrays, a first acc_exec_scan
  *     on operands of the same alignment and on the same side of 12 MB each of the others;
  *   - every call on a device shares that device's array: calls that overlap in time on one device, from any
- *     stream, thread or context, race.  Calls ordered on one stream are fine.
+ *     stream, thread or context, race.  Calls ordered on one stream are fine.  A call of more tiles than the device
+ *     holds at once must not overlap ANY other scan of that size on the device either, acc_exec_scan's included:
+ *     acc_exec_scan chains such scans across streams with events, which this entry point, possibly under capture,
+ *     does not;
+ *   - a call makes two launches: a small kernel that counts the launch's tag in the array's header, and the scan,
+ *     which reads it there.  A graph that records the call therefore gets a fresh tag at every replay; were the tag
+ *     an argument of the recorded launch, a replay would take the descriptors its predecessor left for its own.
  * Results are those of acc_exec_scan, bit for bit.                                                          */
 #define ACC_NOALLOC_MAX_TILES 8192
 int acc_exec_scan_noalloc(acc_skel s, const acc_array *env, int64_t n, const acc_array *out,
@@ -457,7 +469,7 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
                      const acc_array *out, acc_stream stream);
 
 /* stencil: stencilOp, Execute.hs:413-425 (launched once, not twice).  `in` is
- * the manifest source, out has the same shape (rank 1, 2 or 3).              */
+ * the manifest source, out has the same shape (any rank up to ACC_MAX_RANK).  */
 int acc_exec_stencil(acc_skel s, const acc_array *env, const acc_array *in, const acc_array *out,
                      acc_stream stream);
 

@@ -108,6 +108,29 @@ def stencil2d(fn, img, offsets, mode, constant=0.0):
     return out
 
 
+def tap_arrays_nd(v, taps, mode, constant):
+    """for every tap (a tuple of one offset per dimension, outermost first) the array of what that tap reads at
+    every element of the numpy array `v`, under the boundary condition (Stencil/Extra.hs:198-226), dimension by
+    dimension: index arrays made with `bmap`, one numpy take per dimension"""
+    import numpy as np
+    out = []
+    for off in taps:
+        a = v
+        inside = np.ones(v.shape, bool)
+        for d, o in enumerate(off):
+            sz = v.shape[d]
+            want = [i + o for i in range(sz)]
+            idx = [max(0, min(i, sz - 1)) if mode == "constant" else max(0, min(bmap(mode, i, sz), sz - 1)) for i in want]
+            a = np.take(a, idx, axis=d)
+            if mode == "constant":
+                ok = np.array([0 <= i < sz for i in want])
+                shape = [1] * v.ndim
+                shape[d] = sz
+                inside &= ok.reshape(shape)
+        out.append(np.where(inside, a, np.asarray(constant, dtype=v.dtype)) if mode == "constant" else a)
+    return out
+
+
 def affine16(x, y):
     a1, b1, a2, b2 = x >> 16, x & 0xFFFF, y >> 16, y & 0xFFFF
     return (((a1 * a2) & 0xFFFF) << 16) | ((a1 * b2 + b1) & 0xFFFF)

@@ -372,3 +372,27 @@ def test_stencils_over_sources_of_tuple_type(A, ctx):
                      stencil_in="float, Int32", stencil_fn="t0.a1")
     assert e.value.code == A.ERR_INVALID
 
+
+
+def test_tuples_of_twelve_components(A, ctx):
+    """the kernel ABI names tuple components without a bound (CodeGen/Base.hs:69-79) and the array language's tuples have
+    up to 15: a map that produces twelve components, a fold that reads an array of twelve"""
+    n = 70001
+    x = np.random.default_rng(12).integers(-1000, 1000, n).astype(np.int32)
+    elt = ", ".join(["Int32"] * 12)
+    make = ctx.skeleton(A.SKEL_MAP, elt, env=[I32], out_rank=1,
+                        get="acc_elt{" + ", ".join("arrIn0_0[ix] * %d + %d" % (k + 1, k) for k in range(11, -1, -1)) + "}")
+    out = ctx.empty_tuple(n, [np.int32] * 12)
+    make.map([ctx.array(x)], out)
+    got = out.get()                                           # components as the tuple reads: a11 first
+    for i, g in enumerate(got):
+        k = 11 - i
+        assert np.array_equal(g, x * (k + 1) + k), k
+    total = ctx.skeleton(A.SKEL_FOLD, "Int64", env=[(1, ["Int32"] * 12)], out_rank=0,
+                         get=" + ".join("(Int64)arrIn0_%d[ix]" % k for k in range(12)), combine="x + y", seed="0")
+    res = ctx.empty((), np.int64)
+    total.fold([out], n, res)
+    assert int(res.get()) == int(sum(int(g.astype(np.int64).sum()) for g in got))
+    with pytest.raises(A.AccError) as e:                      # seventeen are too many
+        ctx.skeleton(A.SKEL_MAP, ", ".join(["Int32"] * 17), env=[I32], out_rank=1, get="acc_elt{" + ", ".join(["0"] * 17) + "}")
+    assert e.value.code == A.ERR_INVALID

@@ -277,10 +277,10 @@ def test_descriptions_are_validated(A):
         (dict(kind=A.SKEL_PERMUTE, elt="Int16", env=[], out_rank=1, get="1", combine="x+y", permutation="0", combine_hint=A.COMBINE_ADD),
          "4- or 8-byte"),                                                                                        # no hardware atomic on 2 bytes
         (dict(kind=A.SKEL_PERMUTE, elt="float", env=[], out_rank=1, get="1", combine="x", permutation="0", combine_hint=A.COMBINE_XOR), "bitwise"),
-        (dict(kind=A.SKEL_STENCIL, elt="float", out_rank=4, taps=[(0, 0)], stencil_fn="t0"), "rank 4"),
-        (dict(kind=A.SKEL_STENCIL, elt="float", out_rank=3, taps=[(3, 0, 0)], stencil_fn="t0"), "across planes"),
+        (dict(kind=A.SKEL_STENCIL, elt="float", out_rank=4, taps=[(0, 0)], stencil_fn="t0"), "tap_offsets"),     # rank 4: taps as rows of offsets
+        (dict(kind=A.SKEL_STENCIL, elt="float", out_rank=3, taps=[(300, 0, 0)], stencil_fn="t0"), "elements away"),
         (dict(kind=A.SKEL_STENCIL2, elt="float", out_rank=2, taps=[(0, 0)], stencil_fn="t0"), "tap list"),       # second source missing
-        (dict(kind=A.SKEL_STENCIL, elt="float", out_rank=2, taps=[(0, 9)], stencil_fn="t0"), "offset"),
+        (dict(kind=A.SKEL_STENCIL, elt="float", out_rank=2, taps=[(0, 99)], stencil_fn="t0"), "elements away"),
         (dict(kind=99, elt="float"), "unknown"),
     ]
     for kw, needle in cases:
@@ -379,6 +379,28 @@ def test_workload_module_is_pure_numpy():
     vals, cols, offs, lens, xv = wl.smvm_inputs(nrows=500, mean_len=8, ncols=64)
     assert offs[0] == 0 and offs[-1] == vals.size == cols.size and np.array_equal(np.diff(offs), lens)
     assert cols.min() >= 0 and cols.max() < 64 and xv.size == 64
+
+
+def test_stencils_of_any_rank_and_reach_generate_and_compile(A):
+    """rank 4 (taps as rows of offsets), and a tap five rows away in two dimensions: both take the template that maps an
+    element a thread; a stencil within the strips' reach does not, unless the knob asks for it"""
+    import itertools
+    taps4 = list(itertools.product((-1, 0, 1), repeat=4))
+    d4 = A.make_desc(A.SKEL_STENCIL, "float", out_rank=4, taps=taps4, boundary="mirror", stencil_fn=" + ".join("t%d" % k for k in range(81)))
+    name, src = A.preview(d4, 0)
+    assert name == "stencil" and '#include "skel_stencil_nd.h"' in src and "shOut_3" in src and "READ(0, -1, 0, 1, -1)" in src
+    assert A.compile_only(d4) > 0
+    far = A.make_desc(A.SKEL_STENCIL, "double", out_rank=2, taps=[(0, 0), (-5, 0), (0, 6)], boundary="constant", boundary_constant="1.0",
+                      stencil_fn="t0 + t1 + t2")
+    assert "skel_stencil_nd.h" in A.preview(far, 0)[1] and A.compile_only(far) > 0
+    near = A.make_desc(A.SKEL_STENCIL, "double", out_rank=2, taps=[(0, 0), (-4, 0), (0, 4)], boundary="clamp", stencil_fn="t0 + t1 + t2")
+    assert '#include "skel_stencil.h"' in A.preview(near, 0)[1]
+    with A.tuning("stencil.nd=1"):
+        assert "skel_stencil_nd.h" in A.preview(near, 0)[1]
+    with pytest.raises(A.AccError) as e:                       # a rank-4 stencil cannot say its taps in three lists
+        bad = A.make_desc(A.SKEL_STENCIL, "float", out_rank=4, taps=[(0, 0, 0)], stencil_fn="t0")
+        A.preview(bad, 0)
+    assert e.value.code == A.ERR_INVALID
 
 
 def test_c_client_builds_as_c99_and_runs_its_deviceless_part():

@@ -98,3 +98,61 @@ def test_noalloc_scan_refuses_what_it_cannot_do_without_allocating(A, ctx):
     out2 = ctx.empty(n + 4, np.int32)
     sk.scan([shifted_in], n, out2, noalloc=True)
     assert np.array_equal(out2.get()[:n], ref) and np.array_equal(ref, np.cumsum(x[1:n + 1], dtype=np.int32))
+
+
+def test_noalloc_scan_recorded_into_a_graph_and_replayed_on_changing_inputs(A, ctx, orc):
+    """The entry point is for callers under HIP graph capture.  A recorded launch keeps its arguments, so the launch's
+    tag is not among them: it is counted on the device by a kernel recorded in front of the scan.  Here one call is
+    recorded and the graph replayed several times, the input changed between the replays (the second input is chosen
+    so that tiles published by the first replay would give a wrong result if they were taken for this one's), eager
+    scans and synchronisations of the program's own in between; every replay is checked against the eager result."""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+    for name in ("hipStreamBeginCapture", "hipStreamEndCapture", "hipGraphInstantiate", "hipGraphLaunch", "hipGraphExecDestroy",
+                 "hipGraphDestroy", "hipStreamSynchronize"):
+        getattr(hip, name).restype = C.c_int
+    hip.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+    hip.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+    hip.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+    hip.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+    hip.hipGraphExecDestroy.argtypes = [C.c_void_p]
+    hip.hipGraphDestroy.argtypes = [C.c_void_p]
+    hip.hipStreamSynchronize.argtypes = [C.c_void_p]
+    rng = np.random.default_rng(6)
+    sk = ctx.skeleton(A.SKEL_SCANL, "Int32", env=[I32], get="arrIn0_0[ix]", combine="x + y", seed="0", wait=True)
+    tile = sk.info().elements_per_block
+    n = 700 * tile + 77                           # more tiles than are resident at once: the look-back really waits
+    stream = ctx.stream()
+    dx, got, ref = ctx.empty(n, np.int32), ctx.empty(n + 1, np.int32), ctx.empty(n + 1, np.int32)
+    x0 = rng.integers(-50, 50, size=n, dtype=np.int32)
+    dx.set(x0)
+    sk.scan([dx], n, ref, stream=stream)          # the variant is loaded; and the eager result of the first input
+    sk.scan([dx], n, got, stream=stream, noalloc=True)
+    ctx.sync()
+    assert np.array_equal(got.get(), ref.get())
+    sk.scan([dx], 3 * tile + 1, ref, stream=stream)            # (loads the small-tile variant the calls between the replays take)
+    graph, graph_exec = C.c_void_p(), C.c_void_p()
+    assert hip.hipStreamBeginCapture(stream, 2) == 0          # hipStreamCaptureModeRelaxed
+    try:
+        sk.scan([dx], n, got, stream=stream, noalloc=True)
+    finally:
+        rc = hip.hipStreamEndCapture(stream, C.byref(graph))
+    assert rc == 0 and graph.value
+    assert hip.hipGraphInstantiate(C.byref(graph_exec), graph, None, None, 0) == 0
+    try:
+        for replay in range(5):
+            x = rng.integers(-50, 50, size=n, dtype=np.int32) if replay != 1 else (x0 // 2).astype(np.int32)
+            say("graph replay", replay)
+            dx.set(x)
+            got.set(np.full(n + 1, -1, np.int32))
+            assert hip.hipGraphLaunch(graph_exec, stream) == 0
+            assert hip.hipStreamSynchronize(stream) == 0
+            want = orc.scan("scanl", orc.OP_ADD, x, seed=0)
+            assert np.array_equal(got.get(), want), replay
+            # the program's own eager work between the replays: an allocating scan and a smaller no-alloc one
+            sk.scan([dx], n, ref, stream=stream)
+            sk.scan([dx], 3 * tile + 1, ref, stream=stream, noalloc=True)
+            ctx.sync()
+    finally:
+        hip.hipGraphExecDestroy(graph_exec)
+        hip.hipGraphDestroy(graph)
