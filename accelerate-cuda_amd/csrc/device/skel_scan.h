@@ -457,6 +457,9 @@ ACC_DEV void acc_scan_tile(const T (&x)[ACC_ROWS][ACC_VEC], Op op, const T seed,
 #ifndef ACC_MIN_WAVES
 #define ACC_MIN_WAVES 1
 #endif
+#ifndef ACC_SCAN_TICKET
+#define ACC_SCAN_TICKET 0
+#endif
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK, ACC_MIN_WAVES)
 ACC_ENTRY(ACC_ENV_PARAMS
           const Int64 shOut_0, ACC_OUT_ARRAY(arrOut),
@@ -504,7 +507,18 @@ ACC_ENTRY(ACC_ENV_PARAMS
   const Int64 n_up = (n + ACC_VEC - 1) / ACC_VEC * ACC_VEC;
   auto tile_base = [&](const Int64 t) -> Int64 { return ACC_SCAN_RIGHT ? n_up - (t + 1) * (Int64)ACC_TILE : t * (Int64)ACC_TILE; };
 
+#if ACC_SCAN_TICKET
+  /* (measurement: tiles numbered by a counter in the header, zeroed by the host before the launch, instead of by
+   * workgroup index -- no reliance on the order in which workgroups are dispatched, at the price of one device-scope
+   * addition on one address per tile) */
+  __shared__ unsigned int s_ticket;
+  if (threadIdx.x == 0)
+    s_ticket = __hip_atomic_fetch_add((unsigned int *)((char *)desc0 - 256 + 64), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  const Int64 tile = (Int64)s_ticket;
+#else
   const Int64 tile = (Int64)blockIdx.x;
+#endif
 
   if (n <= 0) {                                   /* PrefixSum.hs:249-251,330-334: scan of nothing is [seed] */
     if (threadIdx.x == 0 && tile == 0) {

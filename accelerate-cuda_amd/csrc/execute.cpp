@@ -619,6 +619,7 @@ int scan_core(acc_skel s, const acc_array *env, int64_t n, const acc_array *out,
   }
   const uint32_t epoch = blk.epoch;
   char *base = static_cast<char *>(blk.ptr);
+  if (s->spec.scan_ticket) (void)hipMemsetAsync(base + 64, 0, 4, st);      // (measurement knob scan.ticket: the counter tiles are drawn from)
   args.ptr(reinterpret_cast<uint64_t>(base + off_d0));
   args.ptr(reinterpret_cast<uint64_t>(base + off_d1));
   args.ptr(reinterpret_cast<uint64_t>(base + off_d2));

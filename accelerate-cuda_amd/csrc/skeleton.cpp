@@ -253,6 +253,7 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "#define ACC_LOOKBACK " << tune("scan.lookback", 1) << "\n";
       o << "#define ACC_DESC_STRIDE " << sp.scan_desc_stride << "\n";
       o << "#define ACC_MIN_WAVES " << tune("scan.min_waves", 1) << "\n";
+      if (sp.scan_ticket) o << "#define ACC_SCAN_TICKET 1\n";
       tmpl = "skel_scan.h";
       break;
     }
@@ -744,6 +745,7 @@ int make_spec(const acc_skel_desc *d, const TuningPtr &tuning, SkelSpec *sp)
         sp->block = tune("scan.block", sp->scan_shape_open ? 256 : 1024);
         sp->rows = tune("scan.rows", sp->scan_shape_open ? rows4 : sp->scan_rows_fallback);
         sp->scan_small_rows = std::max(0, std::min(tune("scan.small_rows", 4), 32));
+        sp->scan_ticket = tune("scan.ticket", 0) != 0;
       }
       break;
   }

@@ -56,6 +56,7 @@ struct SkelSpec {
   int scan_rows_fallback = 8;
   int scan_small_rows = 0;              // rows a lane of a scan's small-tile variants (2 and 3); 0: none
   int scan_desc_stride = 16;            // 8-byte words between the tile descriptors of a scan, as generated into the kernel
+  bool scan_ticket = false;             // measurement: tiles drawn from a counter instead of numbered by workgroup (knob scan.ticket)
   bool scan_shape_open = false;         // a scan whose tile shape the first build may still change (by its register count)
 };
 

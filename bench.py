@@ -101,6 +101,8 @@ def end_to_end(ctx, uploads, run, download, reps=3):
     them), and with the runtime's own copies from and to pageable memory (a second context with `copy.staged=0`)."""
     import acchip as A
     L = A.lib()
+    if getattr(end_to_end, "skip", False):
+        return None
     plain = getattr(end_to_end, "plain", None)
     if plain is None:
         with A.tuning("copy.staged=0"):
@@ -132,15 +134,43 @@ def end_to_end(ctx, uploads, run, download, reps=3):
             "note": "H2D of the operands from pageable memory + kernels + D2H of the result into pageable memory, device buffers reused; not the headline"}
 
 
+def kernel_sources_hash():
+    """SHA-256 over what decides the code of every kernel: the device templates and the generator.  The profile
+    summaries under profiles/ carry the hash of the tree they were measured on; a summary whose hash is not the
+    tree's describes other kernels than the ones this run launches."""
+    import glob
+    import hashlib
+    csrc = os.path.join(ROOT, "accelerate-cuda_amd", "csrc")
+    h = hashlib.sha256()
+    for path in sorted(glob.glob(os.path.join(csrc, "device", "*.h"))) + [os.path.join(csrc, "skeleton.cpp")]:
+        h.update(os.path.basename(path).encode() + b"\0")
+        h.update(open(path, "rb").read())
+    return h.hexdigest()
+
+
+def profile_hash(path):
+    """the `kernel-sources-sha256:` line of a profile summary, or None"""
+    try:
+        for line in open(path):
+            if line.startswith("kernel-sources-sha256:"):
+                return line.split()[1]
+    except OSError:
+        pass
+    return None
+
+
 def profiled_traffic(kernel):
     """HBM bytes per launch of `kernel` as rocprofv3 counted them (FETCH_SIZE and WRITE_SIZE, each scaled by what the
-    same counter reads for a plain copy of known size): read from the committed summary, not measured in this run"""
+    same counter reads for a plain copy of known size): read from the committed summary, not measured in this run;
+    `stale` says whether the summary was measured on other kernel sources than this tree's"""
     path = os.path.join(ROOT, "profiles", "hbm_traffic_per_launch.txt")
     try:
         for line in open(path):
             f = line.split()
             if len(f) >= 3 and f[0] == "traffic" and f[1] == kernel:
-                return {"bytes": int(float(f[2])), "source": "profiles/hbm_traffic_per_launch.txt"}
+                measured_on = profile_hash(path)
+                return {"bytes": int(float(f[2])), "source": "profiles/hbm_traffic_per_launch.txt",
+                        "kernel_sources_sha256": measured_on, "stale": measured_on != kernel_sources_hash()}
     except OSError:
         pass
     return None
@@ -159,6 +189,7 @@ def result(name, wall_ms, event_ms, launches_per_step, bytes_per_launch, element
     t = profiled_traffic(r.pop("traffic_key", None))
     if t:
         r["hbm_traffic_bytes"], r["hbm_traffic_source"] = t["bytes"], t["source"]
+        r["hbm_traffic_stale"] = t["stale"]
         r["traffic_over_algorithmic"] = round(t["bytes"] / float(bytes_per_launch), 3)
     log("  %-28s %9.3f us/launch  %8.1f GB/s  %5.1f%% of HBM peak" % (name, launch_ms * 1e3, gbs, 100 * gbs / HBM_PEAK_GBS))
     return r
@@ -172,10 +203,20 @@ def main():
     ap.add_argument("--only", type=str, default="")
     ap.add_argument("--sets", type=int, default=4, help="copies of every configuration's buffers, used round robin")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--plain", action="store_true",
+                    help="only the warm-up and the timed steps of every configuration: no one-by-one, end-to-end or CPU legs "
+                         "(a counter run then sees a known number of dispatches per kernel)")
+    ap.add_argument("--kernel-sources-hash", action="store_true", help="print the hash the profile summaries are tied to, and leave")
     ap.add_argument("--device-warmup-ms", type=float, default=Timer.DEVICE_WARMUP_MS,
                     help="untimed launches before the warm-up steps of a configuration that finds the device idle")
     args = ap.parse_args()
+    if args.kernel_sources_hash:
+        print(kernel_sources_hash())
+        return
     Timer.DEVICE_WARMUP_MS = args.device_warmup_ms
+    if args.plain:
+        args.no_cpu = True
+        Timer.IDLE_AFTER_S = -1.0             # every configuration starts with its first call on its own: the same number of dispatches each
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives, no sharding)" % args.gpus)
 
@@ -190,11 +231,14 @@ def main():
     log("device: arch %s, %d CUs, LDS/workgroup %d, L2 %d" % (props.arch.decode(), props.compute_units, props.lds_per_block, props.l2_bytes))
     stream = ctx.stream()
     end_to_end.stream = stream
+    end_to_end.skip = args.plain
     T = Timer(A, ctx, stream, args.steps, args.warmup)
 
     def traced(steps, calls=12):
         """the same launches one by one onto an idle device, an event before and behind each (acc_trace_start/stop):
         the way the front-end leg below is timed, for the figure its calls are to be held against"""
+        if args.plain:
+            return None
         ctx.sync()
         ctx.trace_start()
         for k in range(calls):
@@ -717,6 +761,8 @@ def main():
         "roofline": {"bound": "hbm", "achieved": headline["GB_per_s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(headline["GB_per_s"] / HBM_PEAK_GBS, 4),
                      "traffic": headline.get("hbm_traffic_bytes"), "traffic_source": headline.get("hbm_traffic_source"),
+                     "traffic_kernel_sources_sha256": profile_hash(os.path.join(ROOT, "profiles", "hbm_traffic_per_launch.txt")),
+                     "kernel_sources_sha256": kernel_sources_hash(), "stale": headline.get("hbm_traffic_stale"),
                      "kernel": "scanl", "avg_launch_us": headline["avg_launch_us"],
                      "algorithmic_bytes_per_launch": headline["algorithmic_bytes_per_launch"]},
         "cpu_baseline": cpu,
