@@ -464,3 +464,22 @@ def test_haskell_modules_use_only_what_the_bindings_and_the_device_headers_have(
             assert name in defined, (m, name)
         for name in set(re.findall(r"\b(ACC_[A-Z_]+)\b", code)) - {"ACC_FLAG_GUARDED", "ACC_ERR_INVALID", "ACC_ERR_STUCK", "ACC_COMBINE_ADD"}:
             assert name in defined, (m, name)
+
+
+def test_profile_summaries_were_measured_on_this_tree_s_kernel_sources():
+    """every summary under profiles/ names the commit it was measured on and carries the SHA-256 of the kernel sources
+    (csrc/device/*.h and skeleton.cpp) of that tree: a change to a kernel's source without collecting the counters
+    again fails here, and bench.py marks the traffic figures it reads from them as stale"""
+    import glob
+    import re
+    import bench
+    now = bench.kernel_sources_hash()
+    files = sorted(glob.glob(os.path.join(ROOT, "profiles", "*.txt")))
+    assert len(files) >= 7
+    for path in files:
+        text = open(path).read()
+        assert re.search(r"^git-head: [0-9a-f]{40}$", text, re.M), path
+        assert bench.profile_hash(path) == now, "%s was measured on other kernel sources than this tree's" % os.path.basename(path)
+        assert "rocprofv3" in text and "bench.py" in text, path      # the command that made it
+    t = bench.profiled_traffic("scanl")
+    assert t and t["stale"] is False and t["bytes"] > 2 * (1 << 26) * 4
