@@ -1,3 +1,4 @@
+{-# LANGUAGE BangPatterns #-}
 -- |
 -- Module      : Data.Array.Accelerate.HIP
 --
@@ -18,6 +19,7 @@ module Data.Array.Accelerate.HIP (
 
   -- * Synchronous execution
   run, run1, runN, stream, runWith, run1With, streamWith,
+  streamOut, streamOutWith,
 
   -- * Asynchronous execution
   Async, wait, poll, cancel,
@@ -32,7 +34,7 @@ module Data.Array.Accelerate.HIP (
 import Data.Array.Accelerate.Trafo                              ( convertAccWith, convertAfunWith, Phase(..), phases )
 import Data.Array.Accelerate.Smart                              ( Acc )
 import Data.Array.Accelerate.Array.Sugar                       ( Arrays )
-import Data.Array.Accelerate.Async
+import Data.Array.Accelerate.Async                             ( Async, async, wait, poll, cancel )
 
 import Data.Array.Accelerate.HIP.Compile
 import Data.Array.Accelerate.HIP.Execute
@@ -84,21 +86,34 @@ stream :: (Arrays a, Arrays b) => (Acc a -> Acc b) -> [a] -> [b]
 stream = streamWith defaultEnv
 
 streamWith :: (Arrays a, Arrays b) => Context -> (Acc a -> Acc b) -> [a] -> [b]
-streamWith env f = map (run1With env f)
+streamWith env f = map go
+  where
+    !go = run1With env f
 
--- | CUDA.hs:232-316: the computation in a thread of its own; `wait`, `poll` and `cancel` from
--- Data.Array.Accelerate.Async
-runAsync :: Arrays a => Acc a -> Async a
+-- | the results of a sequence of computations as a lazy list: an element is compiled, run and collected when it is
+-- asked for, never the whole sequence at once.  The reference keeps its `streamOut` (CUDA.hs:349-372) commented out
+-- together with the `Seq` language it ran (accelerate-1.0 has none); this is the part of it that does not need
+-- one: the sequence is a list of array computations.
+streamOut :: Arrays a => [Acc a] -> [a]
+streamOut = streamOutWith defaultEnv
+
+streamOutWith :: Arrays a => Context -> [Acc a] -> [a]
+streamOutWith env = map (runWith env)
+
+-- | CUDA.hs:256-333: the computation in a thread of its own; `wait`, `poll` and `cancel` from
+-- Data.Array.Accelerate.Async.  The reference forks a BOUND thread, because a CUDA context belongs to an operating
+-- system thread; every entry point of libacchip makes its context's device current itself, so any thread will do.
+runAsync :: Arrays a => Acc a -> IO (Async a)
 runAsync = runAsyncWith defaultEnv
 
-runAsyncWith :: Arrays a => Context -> Acc a -> Async a
-runAsyncWith env a = unsafePerformIO (async (evaluate env a))
+runAsyncWith :: Arrays a => Context -> Acc a -> IO (Async a)
+runAsyncWith env a = async (evaluate env a)
 
-run1Async :: (Arrays a, Arrays b) => (Acc a -> Acc b) -> a -> Async b
+run1Async :: (Arrays a, Arrays b) => (Acc a -> Acc b) -> a -> IO (Async b)
 run1Async = run1AsyncWith defaultEnv
 
-run1AsyncWith :: (Arrays a, Arrays b) => Context -> (Acc a -> Acc b) -> a -> Async b
-run1AsyncWith env f = \a -> unsafePerformIO (async (return $! go a))
+run1AsyncWith :: (Arrays a, Arrays b) => Context -> (Acc a -> Acc b) -> a -> IO (Async b)
+run1AsyncWith env f = \a -> async (return $! go a)
   where
     !go = run1With env f
 

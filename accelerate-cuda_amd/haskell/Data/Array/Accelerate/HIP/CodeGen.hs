@@ -1,4 +1,4 @@
-{-# LANGUAGE GADTs, RankNTypes, ScopedTypeVariables, PatternGuards #-}
+{-# LANGUAGE GADTs, RankNTypes, ScopedTypeVariables, PatternGuards, ExistentialQuantification #-}
 -- |
 -- Module      : Data.Array.Accelerate.HIP.CodeGen
 --
@@ -20,10 +20,12 @@
 --
 module Data.Array.Accelerate.HIP.CodeGen (
 
-  Gamma, emptyGamma, gammaArrays,
+  Gamma, ArrayVar(..), emptyGamma, gammaArrays, gammaSignature,
   Fragment, fragmentText,
-  codegenFun1, codegenFun2, codegenExp, codegenDelayed, codegenPermutation, codegenStencilFun,
-  eltTypeNames, cTypeOf,
+  codegenFun1, codegenFun2, codegenExp, codegenDelayed, codegenMap, codegenZipWith, codegenIndexFun, codegenIndexedBy,
+  codegenPermutation,
+  codegenStencilFun, codegenBoundary,
+  eltTypeNames, cTypeOf, outExtents,
 
 ) where
 
@@ -31,12 +33,12 @@ import Data.Array.Accelerate.AST
 import Data.Array.Accelerate.Trafo                              ( DelayedOpenAcc(..), DelayedOpenExp, DelayedOpenFun )
 import Data.Array.Accelerate.Type
 import Data.Array.Accelerate.Array.Sugar                       ( Elt, Shape, eltType, Array )
-import Data.Array.Accelerate.Array.Representation              ( SliceIndex(..) )
 import qualified Data.Array.Accelerate.Array.Sugar             as Sugar
-import qualified Data.Array.Accelerate.Analysis.Shape          as Sugar
 
 import Control.Monad.State.Strict
-import Data.List                                                ( intercalate )
+import Data.Int                                                 ( Int32 )
+import Data.List                                                ( intercalate, sortBy )
+import Data.Ord                                                 ( comparing )
 import qualified Data.IntMap.Strict                             as IM
 
 
@@ -47,32 +49,44 @@ import qualified Data.IntMap.Strict                             as IM
 -- shIn<k>_<d> in the text and becomes entry k of the `env` arrays handed to acc_exec_*
 -- (AST.hs:87-112 `Gamma`, Execute.hs:835-836).
 
-data Gamma = Gamma
+-- | an array variable together with what is known of its type where it was met: the execution phase looks its
+-- value up in the array environment and needs the extent and the components (the `Idx_` of AST.hs:96-98)
+data ArrayVar aenv = forall sh e. (Shape sh, Elt e) => ArrayVar (Idx aenv (Array sh e))
+
+data Gamma aenv = Gamma
   { gammaNext :: !Int
-  , gammaSlot :: !(IM.IntMap Int)               -- de Bruijn index of the array variable -> slot
+  , gammaSlot :: !(IM.IntMap (Int, ArrayVar aenv))   -- de Bruijn index of the array variable -> its slot, and the variable
   }
 
-emptyGamma :: Gamma
+emptyGamma :: Gamma aenv
 emptyGamma = Gamma 0 IM.empty
 
--- | de Bruijn indices of the arrays to pass, in slot order
-gammaArrays :: Gamma -> [Int]
-gammaArrays g = map snd . IM.toAscList . IM.fromList $ [ (s, v) | (v, s) <- IM.toList (gammaSlot g) ]
+-- | the arrays to pass, in slot order
+gammaArrays :: Gamma aenv -> [ArrayVar aenv]
+gammaArrays g = map snd (sortBy (comparing fst) (IM.elems (gammaSlot g)))
 
-type Gen = State (Gamma, Int)                    -- the environment so far, and a supply of names for local bindings
+-- | what acc_skel_desc.env says of them: rank, and the C type of every component, component 0 first
+gammaSignature :: Gamma aenv -> [(Int32, [String])]
+gammaSignature g = [ sig v | v <- gammaArrays g ]
+  where
+    sig :: ArrayVar aenv -> (Int32, [String])
+    sig (ArrayVar (_ :: Idx aenv (Array sh e))) =
+      (fromIntegral (Sugar.rank (undefined :: sh)), reverse (eltTypeNames (undefined :: e)))
 
-slotOf :: Idx aenv a -> Gen Int
+type Gen aenv = State (Gamma aenv, Int)          -- the environment so far, and a supply of names for local bindings
+
+slotOf :: (Shape sh, Elt e) => Idx aenv (Array sh e) -> Gen aenv Int
 slotOf ix = do
   (g, n) <- get
   let v = idxToInt ix
   case IM.lookup v (gammaSlot g) of
-    Just s  -> return s
-    Nothing -> do
+    Just (s, _) -> return s
+    Nothing     -> do
       let s = gammaNext g
-      put (g { gammaNext = s + 1, gammaSlot = IM.insert v s (gammaSlot g) }, n)
+      put (g { gammaNext = s + 1, gammaSlot = IM.insert v (s, ArrayVar ix) (gammaSlot g) }, n)
       return s
 
-fresh :: Gen String
+fresh :: Gen aenv String
 fresh = do
   (g, n) <- get
   put (g, n + 1)
@@ -161,43 +175,75 @@ prj (SuccIdx ix) (Push val _) = prj ix val
 -- -----------
 
 -- | a closed scalar expression (a seed, a shape): Execute.hs evaluates shapes on the host instead
-codegenExp :: Gamma -> DelayedOpenExp () aenv t -> (Fragment, Gamma)
+codegenExp :: Gamma aenv -> DelayedOpenExp () aenv t -> (Fragment, Gamma aenv)
 codegenExp g e = close g (expr e Empty)
 
 -- | \x -> body, its argument spelt `x` (components x.a<n-1> .. x.a0 when it is a tuple)
-codegenFun1 :: forall aenv a b. Elt a => Gamma -> DelayedOpenFun () aenv (a -> b) -> (Fragment, Gamma)
+codegenFun1 :: forall aenv a b. Elt a => Gamma aenv -> DelayedOpenFun () aenv (a -> b) -> (Fragment, Gamma aenv)
 codegenFun1 g (Lam (Body b)) = close g (expr b (Empty `Push` argument "x" (eltTypeNames (undefined :: a))))
 codegenFun1 _ _              = error "codegenFun1: expected a unary function"
 
 -- | \x y -> body: the `combine` fragment of folds, scans and permute.  The new value is x (IndexSpace.hs:207).
-codegenFun2 :: forall aenv a b c. (Elt a, Elt b) => Gamma -> DelayedOpenFun () aenv (a -> b -> c) -> (Fragment, Gamma)
+codegenFun2 :: forall aenv a b c. (Elt a, Elt b) => Gamma aenv -> DelayedOpenFun () aenv (a -> b -> c) -> (Fragment, Gamma aenv)
 codegenFun2 g (Lam (Lam (Body b))) =
   close g (expr b (Empty `Push` argument "x" (eltTypeNames (undefined :: a)) `Push` argument "y" (eltTypeNames (undefined :: b))))
 codegenFun2 _ _ = error "codegenFun2: expected a binary function"
 
--- | a stencil's function over its taps t0, t1, ... (u0, ... for the second source of a stencil2), in the order
--- the stencil pattern lists them; a tap of a tuple source is a struct of its components (include/acc_hip.h)
-codegenStencilFun :: Gamma -> [(String, [String])] -> (Val () -> Gen ([String], [String])) -> (Fragment, Gamma)
-codegenStencilFun g _taps body = close g (body Empty)
+-- | a function of an index of the result, over the linear index `ix` the map family's kernels count in: the
+-- argument is `ix` taken apart by the result's extents shOut_<d> (generate, backpermute: IndexSpace.hs:47-141)
+codegenIndexFun :: forall aenv sh e. Shape sh => Gamma aenv -> DelayedOpenFun () aenv (sh -> e) -> (Fragment, Gamma aenv)
+codegenIndexFun g (Lam (Body b)) = close g (expr b (Empty `Push` fromIndex (outExtents (Sugar.rank (undefined :: sh))) "ix"))
+codegenIndexFun _ _              = error "codegenIndexFun: expected a unary function"
+
+-- | a source array read through an index function of the result: backpermute's `get`
+codegenIndexedBy :: forall aenv sh sh' e. (Shape sh, Shape sh', Elt e)
+                 => Gamma aenv -> DelayedOpenFun () aenv (sh' -> sh) -> DelayedOpenAcc aenv (Array sh e) -> (Fragment, Gamma aenv)
+codegenIndexedBy g (Lam (Body p)) a = close g $ do
+  (b1, ix) <- expr p (Empty `Push` fromIndex (outExtents (Sugar.rank (undefined :: sh'))) "ix")
+  (b2, vs) <- expr (Index a (Var ZeroIdx)) (Empty `Push` ix)
+  return (b1 ++ b2, vs)
+codegenIndexedBy _ _ _ = error "codegenIndexedBy: expected a unary function"
+
+-- | the extents of the result as the kernels name them, outermost first
+outExtents :: Int -> [String]
+outExtents r = [ "shOut_" ++ show d | d <- reverse [0 .. r - 1] ]
+
+-- | a stencil's function over its taps: t0, t1, ... in the order the stencil pattern lists them, flattened left to
+-- right (u0, ... for the second source of a stencil2).  `sources` gives, per source, the name of its taps, how
+-- many there are and how many components an element has: a tap of a source of tuples is a struct of its
+-- components, t<k>.a<m-1> .. t<k>.a0 (include/acc_hip.h, stencil_in_type)
+codegenStencilFun :: Gamma aenv -> [(String, Int, Int)] -> DelayedOpenFun () aenv f -> (Fragment, Gamma aenv)
+codegenStencilFun g sources f = close g (go f sources Empty)
+  where
+    go :: DelayedOpenFun env aenv t -> [(String, Int, Int)] -> Val env -> Gen aenv ([String], [String])
+    go (Body b) []                     env = expr b env
+    go (Lam l)  ((name, n, m) : rest)  env = go l rest (env `Push` concat [ tap name k m | k <- [0 .. n - 1] ])
+    go _        _                      _   = error "codegenStencilFun: one argument per source"
+    tap name k 1 = [ name ++ show k ]
+    tap name k m = [ name ++ show k ++ ".a" ++ show c | c <- reverse [0 .. m - 1] ]
+
+-- | the value a constant boundary condition gives outside the source, as acc_skel_desc wants it: one literal per
+-- component, "v<n-1>, ..., v0" (Stencil/Extra.hs:112-116)
+codegenBoundary :: forall e. Elt e => e -> Boundary (Sugar.EltRepr e) -> Maybe String
+codegenBoundary _ (Constant c) = Just (intercalate ", " (constants (eltType (undefined :: e)) c))
+codegenBoundary _ _            = Nothing
 
 argument :: String -> [String] -> [String]
 argument name [_] = [name]
 argument name ts  = [ name ++ ".a" ++ show k | k <- reverse [0 .. length ts - 1] ]
 
-close :: Gamma -> Gen ([String], [String]) -> (Fragment, Gamma)
+close :: Gamma aenv -> Gen aenv ([String], [String]) -> (Fragment, Gamma aenv)
 close g m = let ((binds, comps), (g', _)) = runState m (g, 0) in (Fragment binds comps, g')
 
 -- the statements an expression needs run before it, and its components
-expr :: forall env aenv t. DelayedOpenExp env aenv t -> Val env -> Gen ([String], [String])
+expr :: forall env aenv t. DelayedOpenExp env aenv t -> Val env -> Gen aenv ([String], [String])
 expr e env = case e of
   Var ix                -> pure' (prj ix env)
   Const c               -> pure' (constants (eltType (undefined :: t)) c)
   PrimConst c           -> pure' [primConst c]
   Let bnd body          -> do
     (bs, vs) <- expr bnd env
-    -- every component is bound once, so that a value used twice is computed once (CodeGen/Monad.hs `bind`)
-    names    <- mapM (const fresh) vs
-    let decls = [ "const auto " ++ n ++ " = " ++ v ++ ";" | (n, v) <- zip names vs ]
+    (decls, names) <- bindLocals vs
     (bs', vs') <- expr body (env `Push` names)
     return (bs ++ decls ++ bs', vs')
   Tuple tup             -> tuple tup
@@ -253,7 +299,7 @@ expr e env = case e of
     pure' vs = return ([], vs)
     unsupported what = error ("Data.Array.Accelerate.HIP.CodeGen: " ++ what ++ " in a scalar expression is not generated")
 
-    tuple :: Tuple (DelayedOpenExp env aenv) s -> Gen ([String], [String])
+    tuple :: Tuple (DelayedOpenExp env aenv) s -> Gen aenv ([String], [String])
     tuple NilTup          = pure' []
     tuple (SnocTup tup x) = do
       (b1, v1) <- tuple tup
@@ -272,55 +318,100 @@ expr e env = case e of
           loop   = "for (;;) { " ++ unwords bp ++ " if (!(" ++ vp ++ ")) break; " ++ unwords (bf ++ steps ++ copies) ++ " }"
       return (bx ++ inits ++ [loop], names)
 
-    funOver :: DelayedOpenFun env aenv (a -> b) -> [String] -> Gen ([String], [String])
+    funOver :: DelayedOpenFun env aenv (a -> b) -> [String] -> Gen aenv ([String], [String])
     funOver (Lam (Body b)) names = expr b (env `Push` names)
     funOver _              _     = error "while: expected a unary function"
 
-    -- the extents of an array variable are kernel parameters (CodeGen/Base.hs:69-89)
-    shapeOf :: forall sh e. Shape sh => DelayedOpenAcc aenv (Array sh e) -> Gen ([String], [String])
-    shapeOf (Manifest (Avar ix)) = do
-      k <- slotOf ix
-      let r = Sugar.rank (undefined :: sh)
-      pure' [ "shIn" ++ show k ++ "_" ++ show d | d <- reverse [0 .. r - 1] ]
-    shapeOf Delayed{ extentD = sh } = expr (weakenE sh) env
-    shapeOf _                       = error "shape of an array that is neither a variable nor delayed"
 
-    -- reading an array inside a scalar function: a gather, left to the caches (no non-temporal hint)
-    indexArray :: forall sh e. Elt e => DelayedOpenAcc aenv (Array sh e) -> [String] -> String -> Gen ([String], [String])
-    indexArray (Manifest (Avar ix)) bs i = do
-      k <- slotOf ix
-      let n = length (eltTypeNames (undefined :: e))
-      return (bs, [ "arrIn" ++ show k ++ "_" ++ show c ++ "[" ++ i ++ "]" | c <- reverse [0 .. n - 1] ])
-    indexArray Delayed{ linearIndexD = Lam (Body b) } bs i = do
-      (bs', vs) <- expr (weakenE b) (env `Push` [i])
-      return (bs ++ bs', vs)
-    indexArray _ _ _ = error "index into an array that is neither a variable nor delayed"
+-- Arrays inside fragments
+-- ------------------------
 
-    -- the fragments of a delayed array are closed over the scalar environment: lift them into this one
-    weakenE :: DelayedOpenExp env' aenv s -> DelayedOpenExp env aenv s
-    weakenE = error "weakenE: Data.Array.Accelerate.Trafo.Substitution.weaken over the scalar environment"
+-- the extents of an array variable are kernel parameters (CodeGen/Base.hs:69-89); those of a delayed array are an
+-- expression, closed over the scalar environment: it is generated in the empty one
+shapeOf :: forall aenv sh e. (Shape sh, Elt e) => DelayedOpenAcc aenv (Array sh e) -> Gen aenv ([String], [String])
+shapeOf (Manifest (Avar ix)) = do
+  k <- slotOf ix
+  let r = Sugar.rank (undefined :: sh)
+  return ([], [ "shIn" ++ show k ++ "_" ++ show d | d <- reverse [0 .. r - 1] ])
+shapeOf Delayed{ extentD = sh } = expr sh Empty
+shapeOf _                       = error "shape of an array that is neither a variable nor delayed"
 
+-- reading an array inside a scalar function: a gather, left to the caches (no non-temporal hint)
+indexArray :: forall aenv sh e. (Shape sh, Elt e) => DelayedOpenAcc aenv (Array sh e) -> [String] -> String -> Gen aenv ([String], [String])
+indexArray (Manifest (Avar ix)) bs i = do
+  k <- slotOf ix
+  let n = length (eltTypeNames (undefined :: e))
+  return (bs, [ "arrIn" ++ show k ++ "_" ++ show c ++ "[" ++ i ++ "]" | c <- reverse [0 .. n - 1] ])
+indexArray Delayed{ linearIndexD = Lam (Body b) } bs i = do
+  (bs', vs) <- expr b (Empty `Push` [i])
+  return (bs ++ bs', vs)
+indexArray _ _ _ = error "index into an array that is neither a variable nor delayed"
 
--- | a delayed (or manifest) array as the `get` fragment of a consumer: its element at linear index `ix`.
--- A manifest array consumed in index order is read with a non-temporal load, so that it does not evict what IS
--- reused (gathered vectors, small tables) from the L2.
-codegenDelayed :: forall aenv sh e. (Shape sh, Elt e) => Gamma -> DelayedOpenAcc aenv (Array sh e) -> (Fragment, Gamma)
-codegenDelayed g (Manifest (Avar ix)) = close g $ do
+-- the operand of a skeleton at linear index `ix`.  A manifest array consumed in index order is read with a
+-- non-temporal load, so that it does not evict what IS reused (gathered vectors, small tables) from the L2.
+operandAt :: forall aenv sh e. (Shape sh, Elt e) => DelayedOpenAcc aenv (Array sh e) -> Gen aenv ([String], [String])
+operandAt (Manifest (Avar ix)) = do
   k <- slotOf ix
   let n = length (eltTypeNames (undefined :: e))
   return ([], [ "acc_stream(arrIn" ++ show k ++ "_" ++ show c ++ ", ix)" | c <- reverse [0 .. n - 1] ])
-codegenDelayed g Delayed{ linearIndexD = Lam (Body b) } = close g (expr b (Empty `Push` ["ix"]))
-codegenDelayed _ _ = error "codegenDelayed: the operand of a skeleton is an array variable or a delayed array"
+operandAt Delayed{ linearIndexD = Lam (Body b) } = expr b (Empty `Push` ["ix"])
+operandAt _ = error "the operand of a skeleton is an array variable or a delayed array"
+
+-- the operand of a skeleton whose extents may differ from the result's (zipWith, whose result covers the
+-- intersection): `ix` taken apart by the result's extents and put together again over the operand's own
+operandThrough :: forall aenv sh e. (Shape sh, Elt e) => DelayedOpenAcc aenv (Array sh e) -> Gen aenv ([String], [String])
+operandThrough a
+  | Sugar.rank (undefined :: sh) <= 1 = operandAt a             -- the linear index of the result IS the operand's
+  | otherwise                         = do
+      (bs, sh) <- shapeOf a
+      indexArray a bs (toIndex sh (fromIndex (outExtents (Sugar.rank (undefined :: sh))) "ix"))
+
+-- every component bound to a local once, so that a value used twice is computed once (CodeGen/Monad.hs `bind`)
+bindLocals :: [String] -> Gen aenv ([String], [String])
+bindLocals vs = do
+  names <- mapM (const fresh) vs
+  return ([ "const auto " ++ n ++ " = " ++ v ++ ";" | (n, v) <- zip names vs ], names)
+
+
+-- | a delayed (or manifest) array as the `get` fragment of a consumer: its element at linear index `ix`
+codegenDelayed :: forall aenv sh e. (Shape sh, Elt e) => Gamma aenv -> DelayedOpenAcc aenv (Array sh e) -> (Fragment, Gamma aenv)
+codegenDelayed g a = close g (operandAt a)
+
+-- | map f a as one `get`: the operand's element at `ix` bound to the function's argument (Mapping.hs:39-78)
+codegenMap :: forall aenv sh a b. (Shape sh, Elt a)
+           => Gamma aenv -> DelayedOpenFun () aenv (a -> b) -> DelayedOpenAcc aenv (Array sh a) -> (Fragment, Gamma aenv)
+codegenMap g (Lam (Body f)) a = close g $ do
+  (b1, xs) <- operandAt a
+  (b2, ns) <- bindLocals xs
+  (b3, r)  <- expr f (Empty `Push` ns)
+  return (b1 ++ b2 ++ b3, r)
+codegenMap _ _ _ = error "codegenMap: expected a unary function"
+
+-- | zipWith f a b as one `get` over the result's index space, the intersection of the operands' extents
+codegenZipWith :: forall aenv sh a b c. (Shape sh, Elt a, Elt b)
+               => Gamma aenv -> DelayedOpenFun () aenv (a -> b -> c)
+               -> DelayedOpenAcc aenv (Array sh a) -> DelayedOpenAcc aenv (Array sh b) -> (Fragment, Gamma aenv)
+codegenZipWith g (Lam (Lam (Body f))) a b = close g $ do
+  (b1, xs) <- operandThrough a
+  (b2, ys) <- operandThrough b
+  (b3, nx) <- bindLocals xs
+  (b4, ny) <- bindLocals ys
+  (b5, r)  <- expr f (Empty `Push` nx `Push` ny)
+  return (b1 ++ b2 ++ b3 ++ b4 ++ b5, r)
+codegenZipWith _ _ _ _ = error "codegenZipWith: expected a binary function"
 
 -- | permute's index function as the linear target index of source element `ix`, ACC_IGNORE for `ignore`
--- (IndexSpace.hs:160-303; `ignore` is the index whose every component is -1)
-codegenPermutation :: forall aenv sh sh'. (Shape sh, Shape sh')
-                   => Gamma -> [String] -> [String] -> DelayedOpenFun () aenv (sh -> sh') -> (Fragment, Gamma)
-codegenPermutation g shIn shOut (Lam (Body b)) = close g $ do
+-- (IndexSpace.hs:160-303; `ignore` is the index whose every component is -1).  `ix` is taken apart by the
+-- extents of the source, the target index put together over those of the result, shOut_<d>
+codegenPermutation :: forall aenv sh sh' e. (Shape sh, Shape sh', Elt e)
+                   => Gamma aenv -> DelayedOpenAcc aenv (Array sh e) -> DelayedOpenFun () aenv (sh -> sh') -> (Fragment, Gamma aenv)
+codegenPermutation g a (Lam (Body b)) = close g $ do
+  (b0, shIn)   <- shapeOf a
   (bs, target) <- expr b (Empty `Push` fromIndex shIn "ix")
-  let ignored = intercalate " && " [ "(" ++ t ++ ") == -1" | t <- target ]
-  return (bs, [ if null target then "0" else "((" ++ ignored ++ ") ? ACC_IGNORE : " ++ toIndex shOut target ++ ")" ])
-codegenPermutation _ _ _ _ = error "codegenPermutation: expected a unary function"
+  let shOut   = outExtents (Sugar.rank (undefined :: sh'))
+      ignored = intercalate " && " [ "(" ++ t ++ ") == -1" | t <- target ]
+  return (b0 ++ bs, [ if null target then "0" else "((" ++ ignored ++ ") ? ACC_IGNORE : " ++ toIndex shOut target ++ ")" ])
+codegenPermutation _ _ _ = error "codegenPermutation: expected a unary function"
 
 
 -- Index arithmetic (row-major, outermost extent first)

@@ -1,4 +1,4 @@
-{-# LANGUAGE GADTs, ScopedTypeVariables, BangPatterns #-}
+{-# LANGUAGE GADTs, ScopedTypeVariables, BangPatterns, RankNTypes #-}
 -- |
 -- Module      : Data.Array.Accelerate.HIP.Execute
 --
@@ -18,13 +18,16 @@ module Data.Array.Accelerate.HIP.Execute (
 ) where
 
 import Data.Array.Accelerate.AST
-import Data.Array.Accelerate.Array.Sugar                       ( Array(..), Arrays, Shape, Elt, Scalar, Vector, Segments, Z(..), (:.)(..) )
+import Data.Array.Accelerate.Array.Sugar                       ( Array(..), Arrays, Shape, Elt, Scalar, Vector, Segments, Z(..), (:.)(..), Any(..) )
+import Data.Array.Accelerate.Array.Representation              ( SliceIndex(..) )
+import Data.Array.Accelerate.Interpreter                       ( evalPrim, evalPrimConst, evalPrj )
 import qualified Data.Array.Accelerate.Array.Sugar             as Sugar
 
+import Data.Array.Accelerate.HIP.CodeGen                       ( ArrayVar(..) )
 import Data.Array.Accelerate.HIP.Compile
 import Data.Array.Accelerate.HIP.FFI
 import Data.Array.Accelerate.HIP.State
-import Data.Array.Accelerate.HIP.Array                          -- allocateArray / useArray / peekScalar over acc_memtable_*
+import Data.Array.Accelerate.HIP.Array                          -- arrays and their device copies, over acc_memtable_*
 
 import Control.Monad
 import Control.Monad.Trans                                      ( liftIO )
@@ -53,7 +56,7 @@ executeAcc acc = withStream $ \stream -> do
 -- | CUDA.hs:318-333 `run1`: the kernels were built once, by compileAfun
 executeAfun1 :: (Arrays a, Arrays b) => ExecAfun (a -> b) -> a -> HIP b
 executeAfun1 (Alam (Abody f)) a = withStream $ \stream -> do
-  useArrays a stream
+  useArrays a
   r   <- executeOpenAcc f (Aempty `Apush` a) stream
   ctx <- hipContext
   liftIO $ check (c_streamSync ctx stream)
@@ -74,8 +77,8 @@ executeOpenAcc (ExecAcc kernel pacc) aenv stream =
     Aprj ix tup           -> evalPrj ix . Sugar.fromAtuple <$> travA tup
     Acond p t e           -> do { c <- travE p; if c then travA t else travA e }
     Awhile p f a          -> awhile p f =<< travA a
-    Use arrs              -> do { let a = Sugar.toArr arrs; useArrays a stream; return a }
-    Unit e                -> unitArray stream =<< travE e
+    Use arrs              -> do { let a = Sugar.toArr arrs; useArrays a; return a }
+    Unit e                -> unitArray =<< travE e
     Reshape sh a          -> reshapeArray <$> travE sh <*> travA a       -- same device storage, new extents
 
     -- one driver call each (Execute.hs:264-450)
@@ -116,7 +119,7 @@ executeOpenAcc (ExecAcc kernel pacc) aenv stream =
 
     -- scalar expressions that run on the host (extents, conditions): Execute.hs:454-560, unchanged in structure
     travE :: PreExp ExecOpenAcc aenv t -> HIP t
-    travE e = evalHostExp e aenv stream
+    travE e = evalHostExp e Empty aenv stream
 
     -- the extent of an operand: of a manifest one its array's, of a fused one its extent expression
     extent :: Shape sh => ExecOpenAcc aenv (Array sh e) -> HIP sh
@@ -125,7 +128,7 @@ executeOpenAcc (ExecAcc kernel pacc) aenv stream =
 
     -- the node's free arrays as the kernel wants them, in the order the fragments numbered them
     environment :: ([AccArray] -> HIP r) -> HIP r
-    environment = withArrays stream [ deviceArrayOf (aprjInt v aenv) | v <- gamma ]
+    environment = withArrays stream [ SomeArray (aprj ix aenv) | ArrayVar ix <- gamma ]
 
     run :: IO Status -> HIP ()
     run = liftIO . check
@@ -239,26 +242,84 @@ executeOpenAcc (ExecAcc kernel pacc) aenv stream =
     iterateM k s step = do { s' <- step s; (s :) <$> iterateM (k - 1) s' step }
 
 
--- Supplied by Data.Array.Accelerate.HIP.Array (brackets around the memory table of the header, acc_memtable_*) and by the
--- host-side expression evaluator the reference already has (Execute.hs:454-560); named here so that the traversal
--- above reads as a whole.
-aprjInt       :: Int -> Aval aenv -> SomeArrays
-evalPrj       :: TupleIdx t a -> t -> a
-evalHostExp   :: PreExp ExecOpenAcc aenv t -> Aval aenv -> Stream -> HIP t
-useArrays     :: Arrays a => a -> Stream -> HIP ()
-unitArray     :: Elt e => Stream -> e -> HIP (Scalar e)
-reshapeArray  :: (Shape sh, Shape sh') => sh -> Array sh' e -> Array sh e
-deviceArrayOf :: SomeArrays -> SomeDeviceArray
-withArrays    :: Stream -> [SomeDeviceArray] -> ([AccArray] -> HIP r) -> HIP r
-withDevice    :: Stream -> Array sh e -> (AccArray -> HIP r) -> HIP r
-aprjInt       = undefined
-evalPrj       = undefined
-evalHostExp   = undefined
-useArrays     = undefined
-unitArray     = undefined
-reshapeArray  = undefined
-deviceArrayOf = undefined
-withArrays    = undefined
-withDevice    = undefined
-data SomeArrays
-data SomeDeviceArray
+-- Scalar expressions on the host
+-- -------------------------------
+
+-- the values of the bound scalar variables
+data Val env where
+  Empty :: Val ()
+  Push  :: Val env -> t -> Val (env, t)
+
+prj :: Idx env t -> Val env -> t
+prj ZeroIdx      (Push _   v) = v
+prj (SuccIdx ix) (Push val _) = prj ix val
+
+-- | extents, conditions, the seeds of units: scalar code that did not go into a kernel is interpreted, with the
+-- primitives of the reference interpreter; an array it names is computed first and the one element it wants read
+-- back from the device (Execute.hs:706-768 `executeOpenExp`)
+evalHostExp :: forall env aenv t. PreOpenExp ExecOpenAcc env aenv t -> Val env -> Aval aenv -> Stream -> HIP t
+evalHostExp root env aenv stream = go root
+  where
+    go :: forall s. PreOpenExp ExecOpenAcc env aenv s -> HIP s
+    go e = case e of
+      Var ix              -> return (prj ix env)
+      Let a b             -> do { x <- go a; evalHostExp b (env `Push` x) aenv stream }
+      Const c             -> return (Sugar.toElt c)
+      PrimConst c         -> return (evalPrimConst c)
+      PrimApp f x         -> evalPrim f <$> go x
+      Tuple t             -> Sugar.toTuple <$> goT t
+      Prj ix x            -> evalPrj ix . Sugar.fromTuple <$> go x
+      Cond p t f          -> do { c <- go p; if c then go t else go f }
+      While p f x         -> while p f =<< go x
+      IndexAny            -> return Any
+      IndexNil            -> return Z
+      IndexCons sh i      -> (:.) <$> go sh <*> go i
+      IndexHead sh        -> (\(_ :. i) -> i) <$> go sh
+      IndexTail sh        -> (\(t :. _) -> t) <$> go sh
+      IndexSlice ix s sh  -> restrictTo ix <$> go s <*> go sh
+      IndexFull ix s sl   -> extendTo ix <$> go s <*> go sl
+      ToIndex sh ix       -> Sugar.toIndex <$> go sh <*> go ix
+      FromIndex sh i      -> Sugar.fromIndex <$> go sh <*> go i
+      Intersect a b       -> Sugar.intersect <$> go a <*> go b
+      Union a b           -> Sugar.union <$> go a <*> go b
+      ShapeSize sh        -> Sugar.size <$> go sh
+      Shape a             -> extentOf a
+      Index a ix          -> do { arr <- goA a; i <- go ix; indexArray stream arr (Sugar.toIndex (Sugar.shape arr) i) }
+      LinearIndex a i     -> do { arr <- goA a; indexArray stream arr =<< go i }
+      Foreign{}           -> error "Data.Array.Accelerate.HIP: foreign scalar functions are not supported by this backend"
+
+    goT :: forall s. Tuple (PreOpenExp ExecOpenAcc env aenv) s -> HIP s
+    goT NilTup        = return ()
+    goT (SnocTup t x) = (,) <$> goT t <*> go x
+
+    goA :: forall a. ExecOpenAcc aenv a -> HIP a
+    goA acc = executeOpenAcc acc aenv stream
+
+    -- the extent of a fused array is an expression of its own; nothing is computed for it
+    extentOf :: forall sh e. Shape sh => ExecOpenAcc aenv (Array sh e) -> HIP sh
+    extentOf (ExecFused sh) = evalHostExp sh Empty aenv stream
+    extentOf acc            = Sugar.shape <$> goA acc
+
+    apply1 :: forall a b. PreOpenFun ExecOpenAcc env aenv (a -> b) -> a -> HIP b
+    apply1 (Lam (Body b)) x = evalHostExp b (env `Push` x) aenv stream
+    apply1 _              _ = error "expected a unary function"
+
+    while :: forall a. PreOpenFun ExecOpenAcc env aenv (a -> Bool) -> PreOpenFun ExecOpenAcc env aenv (a -> a) -> a -> HIP a
+    while p f x = do { ok <- apply1 p x; if ok then while p f =<< apply1 f x else return x }
+
+    -- a slice index cuts dimensions out of a shape, or puts them back (Execute.hs:744-764)
+    restrictTo :: (Elt slix, Elt sh, Elt sl) => SliceIndex (Sugar.EltRepr slix) (Sugar.EltRepr sl) co (Sugar.EltRepr sh) -> slix -> sh -> sl
+    restrictTo ix slix sh = Sugar.toElt (cut ix (Sugar.fromElt slix) (Sugar.fromElt sh))
+      where
+        cut :: SliceIndex a b c d -> a -> d -> b
+        cut SliceNil        ()       ()       = ()
+        cut (SliceAll r)    (sx, ()) (sl, sz) = (cut r sx sl, sz)
+        cut (SliceFixed r)  (sx, _)  (sl, _)  = cut r sx sl
+
+    extendTo :: (Elt slix, Elt sh, Elt sl) => SliceIndex (Sugar.EltRepr slix) (Sugar.EltRepr sl) co (Sugar.EltRepr sh) -> slix -> sl -> sh
+    extendTo ix slix sl = Sugar.toElt (grow ix (Sugar.fromElt slix) (Sugar.fromElt sl))
+      where
+        grow :: SliceIndex a b c d -> a -> b -> d
+        grow SliceNil        ()       ()       = ()
+        grow (SliceAll r)    (sx, ()) (sh, sz) = (grow r sx sh, sz)
+        grow (SliceFixed r)  (sx, sz) sh       = (grow r sx sh, sz)

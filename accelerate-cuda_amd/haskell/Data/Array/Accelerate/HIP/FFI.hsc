@@ -85,6 +85,12 @@ accCombineAnd     = #{const ACC_COMBINE_AND}
 accCombineOr      = #{const ACC_COMBINE_OR}
 accCombineXor     = #{const ACC_COMBINE_XOR}
 
+accBoundaryClamp, accBoundaryMirror, accBoundaryWrap, accBoundaryConstant :: Int32
+accBoundaryClamp    = #{const ACC_BOUNDARY_CLAMP}
+accBoundaryMirror   = #{const ACC_BOUNDARY_MIRROR}
+accBoundaryWrap     = #{const ACC_BOUNDARY_WRAP}
+accBoundaryConstant = #{const ACC_BOUNDARY_CONSTANT}
+
 accFlagFoldRight, accFlagFastMath, accFlagGuarded, accFlagTiled :: Word32
 accFlagFoldRight = #{const ACC_FLAG_FOLD_RIGHT}
 accFlagFastMath  = #{const ACC_FLAG_FAST_MATH}
@@ -181,7 +187,25 @@ data Skeleton = Skeleton
   , skelPermutation :: Maybe String
   , skelCombineHint :: Int32
   , skelSegType     :: Maybe String
+  , skelStencilFn   :: Maybe String          -- stencils: the function over the taps t0.. (and u0..)
+  , skelSources     :: [StencilSource]       -- one for a stencil, two for a stencil2
   }
+
+-- | one source of a stencil: its element type ("T<n-1>, ..., T0" for tuples), its boundary condition, and its taps as
+-- rows of out_rank offsets, outermost dimension first (acc_skel_desc.tap_offsets)
+data StencilSource = StencilSource
+  { sourceType     :: String
+  , sourceBoundary :: Int32                  -- ACC_BOUNDARY_*
+  , sourceConstant :: Maybe String
+  , sourceTaps     :: [[Int32]]
+  }
+
+-- | a description with nothing given: the fields a kind does not use stay as they are here
+emptySkeleton :: Skeleton
+emptySkeleton = Skeleton
+  { skelKind = accSkelMap, skelFlags = 0, skelEnv = [], skelEltType = "Int32", skelOutRank = 0, skelPreamble = Nothing
+  , skelGet = Nothing, skelCombine = Nothing, skelSeed = Nothing, skelPermutation = Nothing
+  , skelCombineHint = accCombineGeneric, skelSegType = Nothing, skelStencilFn = Nothing, skelSources = [] }
 
 withMaybeCString :: Maybe String -> (CString -> IO a) -> IO a
 withMaybeCString Nothing  k = k nullPtr
@@ -191,8 +215,7 @@ withCStrings :: [String] -> ([CString] -> IO a) -> IO a
 withCStrings []     k = k []
 withCStrings (s:ss) k = withCString s $ \c -> withCStrings ss (k . (c:))
 
--- | marshal a `Skeleton` (map family, folds, scans, permute; a stencil additionally pokes its taps, boundary and
--- `stencil_fn` the same way) for acc_skel_create / acc_skel_preview
+-- | marshal a `Skeleton` for acc_skel_create[_async] / acc_skel_preview
 withSkelDesc :: Skeleton -> (Ptr SkelDesc -> IO a) -> IO a
 withSkelDesc sk k =
   allocaBytes #{size acc_skel_desc} $ \p ->
@@ -204,7 +227,10 @@ withSkelDesc sk k =
   withMaybeCString (skelCombine sk) $ \comb ->
   withMaybeCString (skelSeed sk) $ \seed ->
   withMaybeCString (skelPermutation sk) $ \perm ->
-  withMaybeCString (skelSegType sk) $ \seg -> do
+  withMaybeCString (skelSegType sk) $ \seg ->
+  withMaybeCString (skelStencilFn sk) $ \sfn ->
+  withSource (source 0) $ \(ty1, bc1, n1, taps1) ->
+  withSource (source 1) $ \(ty2, bc2, n2, taps2) -> do
     _ <- fillBytes p 0 #{size acc_skel_desc}
     #{poke acc_skel_desc, kind}         p (skelKind sk)
     #{poke acc_skel_desc, flags}        p (skelFlags sk)
@@ -219,8 +245,28 @@ withSkelDesc sk k =
     #{poke acc_skel_desc, permutation}  p perm
     #{poke acc_skel_desc, combine_hint} p (skelCombineHint sk)
     #{poke acc_skel_desc, seg_type}     p seg
+    #{poke acc_skel_desc, stencil_fn}          p sfn
+    #{poke acc_skel_desc, stencil_in_type}     p ty1
+    #{poke acc_skel_desc, boundary}            p (maybe accBoundaryClamp sourceBoundary (source 0))
+    #{poke acc_skel_desc, boundary_constant}   p bc1
+    #{poke acc_skel_desc, n_taps}              p (n1 :: Int32)
+    #{poke acc_skel_desc, tap_offsets}         p taps1
+    #{poke acc_skel_desc, stencil_in2_type}    p ty2
+    #{poke acc_skel_desc, boundary2}           p (maybe accBoundaryClamp sourceBoundary (source 1))
+    #{poke acc_skel_desc, boundary2_constant}  p bc2
+    #{poke acc_skel_desc, n_taps2}             p (n2 :: Int32)
+    #{poke acc_skel_desc, tap2_offsets}        p taps2
     k p
   where
+    source i = case drop i (skelSources sk) of { (x : _) -> Just x; [] -> Nothing }
+    -- element type, constant, number of taps, and the taps' offsets row after row
+    withSource :: Maybe StencilSource -> ((CString, CString, Int32, Ptr Int32) -> IO b) -> IO b
+    withSource Nothing   kk = kk (nullPtr, nullPtr, 0, nullPtr)
+    withSource (Just sc) kk =
+      withCString (sourceType sc) $ \ty ->
+      withMaybeCString (sourceConstant sc) $ \bc ->
+      withArray (concat (sourceTaps sc)) $ \taps ->
+        kk (ty, bc, fromIntegral (length (sourceTaps sc)), taps)
     withEnv []            kk = kk []
     withEnv ((r, ts):es)  kk = withCStrings ts $ \cs -> withEnv es (kk . (EnvSig r cs :))
 
@@ -231,6 +277,17 @@ createSkeleton ctx sk =
   withSkelDesc sk $ \pdesc ->
   alloca $ \pout -> do
     check (c_skelCreate ctx pdesc pout)
+    peek pout
+
+-- | the same with the compilation left to the library's pool of workers: the description is checked and the source
+-- generated before this returns, and whatever first needs the kernel (acc_exec_*, acc_skel_wait) waits for it --
+-- build1 forks its compilation and the executing thread blocks where the kernel is first used (Compile.hs:444-459,
+-- 484-538), so a program's kernels compile side by side
+createSkeletonAsync :: Context -> Skeleton -> IO Skel
+createSkeletonAsync ctx sk =
+  withSkelDesc sk $ \pdesc ->
+  alloca $ \pout -> do
+    check (c_skelCreateAsync ctx pdesc pout)
     peek pout
 
 -- | device memory, or Nothing when the device is full (Array/Remote.hs:63-67 `mallocRemote`)
@@ -254,6 +311,17 @@ execScan sk env n out total stream =
   with out $ \pout ->
   maybe ($ nullPtr) with total $ \ptot ->
     check (c_execScan sk penv n pout ptot stream)
+
+-- | have the library's compilations wound up when the process exits (acc_compile_drain: exit() tears down the
+-- compiler's static data, and a worker must not be inside the compiler then).  The C function itself is
+-- registered with the C library's atexit: a Haskell callback could not run there, the run-time system being gone
+-- by then.  Registered after the library (and with it the compiler) was loaded, it runs before their own
+-- destructors.  (Its int result is ignored by the caller, which is harmless under the C ABIs in question.)
+foreign import ccall unsafe "stdlib.h atexit" registerAtExit  :: FunPtr (IO Status) -> IO CInt
+foreign import ccall        "&acc_compile_drain" compileDrainPtr :: FunPtr (IO Status)
+
+drainCompilationsAtExit :: IO ()
+drainCompilationsAtExit = void (registerAtExit compileDrainPtr)
 
 -- ---------------------------------------------------------------------------------------------------------
 -- the entry points, in the header's order

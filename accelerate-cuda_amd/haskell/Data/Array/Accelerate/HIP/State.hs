@@ -56,6 +56,7 @@ withStream body = do
 createEnv :: Int -> IO Env
 createEnv device = do
   check c_init
+  drainCompilationsAtExit                           -- once per context is harmless: the second drain finds nothing to do
   ctx <- alloca $ \p -> check (c_contextCreate (fromIntegral device) p) >> peek p
   mt  <- alloca $ \p -> check (c_memtableCreate ctx 0 p) >> peek p
   Env ctx mt <$> newMVar []

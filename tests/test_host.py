@@ -451,7 +451,7 @@ def test_haskell_modules_use_only_what_the_bindings_and_the_device_headers_have(
         device += open(os.path.join(ROOT, "accelerate-cuda_amd", "csrc", "device", h)).read()
     defined = set(re.findall(r"\b(acc_[a-z0-9_]+)\s*\(", device)) | set(re.findall(r"#define (ACC_[A-Z_]+)", device))
     defined |= set(re.findall(r"^ACC_MATH\d\((acc_[a-z0-9_]+),", device, flags=re.M))       # defined through a macro
-    modules = ["HIP.hs", "HIP/CodeGen.hs", "HIP/Compile.hs", "HIP/Execute.hs", "HIP/State.hs"]
+    modules = ["HIP.hs", "HIP/CodeGen.hs", "HIP/Compile.hs", "HIP/Execute.hs", "HIP/State.hs", "HIP/Array.hs"]
     for m in modules:
         text = open(os.path.join(hdir, m)).read()
         assert "UNCOMPILED" in text, m
@@ -464,6 +464,60 @@ def test_haskell_modules_use_only_what_the_bindings_and_the_device_headers_have(
             assert name in defined, (m, name)
         for name in set(re.findall(r"\b(ACC_[A-Z_]+)\b", code)) - {"ACC_FLAG_GUARDED", "ACC_ERR_INVALID", "ACC_ERR_STUCK", "ACC_COMBINE_ADD"}:
             assert name in defined, (m, name)
+
+
+def test_haskell_modules_are_whole():
+    """every Data.Array.Accelerate.HIP.* module that one of them imports is in the tree; no binding is left
+    `undefined` (or an `error` that names what is missing); every name a module exports, and every name another
+    module imports from it by name, has a definition in it; the front door exports what Data.Array.Accelerate.CUDA
+    does (CUDA.hs:184-200) and the two names the task adds, runN and streamOut"""
+    root = os.path.join(ROOT, "accelerate-cuda_amd", "haskell")
+    paths = {}
+    for d, _, files in os.walk(root):
+        for f in files:
+            if f.endswith((".hs", ".hsc")):
+                rel = os.path.relpath(os.path.join(d, f), root)
+                paths[rel.rsplit(".", 1)[0].replace(os.sep, ".")] = os.path.join(d, f)
+    assert "Data.Array.Accelerate.HIP.Array" in paths
+
+    def strip(text):
+        text = re.sub(r"\{-.*?-\}", "", text, flags=re.S)
+        return re.sub(r"--.*", "", text)
+
+    def defined(code):
+        names = set(re.findall(r"^([a-z_][A-Za-z0-9_']*)\s*(?:::|[^=\n]*=)", code, flags=re.M))            # bindings, signatures
+        names |= set(re.findall(r"^(?:data|type|newtype|class)\s+([A-Z][A-Za-z0-9_']*)", code, flags=re.M))
+        names |= set(re.findall(r'^foreign import ccall.*?"\s+(\w+)\s+::', code, flags=re.M))
+        for body in re.findall(r"^data\s.*?(?=^\S)", code, flags=re.M | re.S):                        # constructors, fields
+            names |= set(re.findall(r"[=|]\s*(?:forall [^.]*\.\s*)?(?:\([^)]*\)\s*=>\s*)?([A-Z][A-Za-z0-9_']*)", body))
+            names |= set(re.findall(r"^\s+([A-Z][A-Za-z0-9_']*)\s*::", body, flags=re.M))              # GADT constructors
+            names |= set(re.findall(r"[{,]\s*([a-z][A-Za-z0-9_']*)\s*::", body))
+        return names
+
+    codes = {m: strip(open(p).read()) for m, p in paths.items()}
+    defs = {m: defined(c) for m, c in codes.items()}
+    for m, code in codes.items():
+        assert not re.search(r"=\s*undefined\b", code), m
+        assert not re.search(r"^\w+\s*=\s*error\b", code, flags=re.M), m
+        for line in re.findall(r"^import\s+(?:qualified\s+)?(Data\.Array\.Accelerate\.HIP[.\w]*)(.*)$", code, flags=re.M):
+            mod, rest = line
+            assert mod in paths, (m, "imports", mod)
+            listed = re.search(r"\(\s*(.*)\)", rest)
+            if listed and "hiding" not in rest:
+                for name in re.findall(r"\b([A-Za-z_][A-Za-z0-9_']*)\b(?:\(\.\.\))?", listed.group(1)):
+                    assert name in defs[mod], (m, "imports", name, "from", mod)
+        head = re.search(r"^module\s+[\w.]+\s*\((.*?)\)\s*where", code, flags=re.M | re.S)
+        if head:
+            for name in re.findall(r"\b([A-Za-z_][A-Za-z0-9_']*)\b", re.sub(r"\(\.\.\)", "", head.group(1))):
+                if name in ("module",):
+                    continue
+                imported = re.search(r"^import\s+.*\b%s\b" % re.escape(name), code, flags=re.M)           # re-exported
+                assert name in defs[m] or imported, (m, "exports", name)
+    front = re.search(r"^module\s+[\w.]+\s*\((.*?)\)\s*where", codes["Data.Array.Accelerate.HIP"], flags=re.M | re.S).group(1)
+    exported = set(re.findall(r"\b([A-Za-z_][A-Za-z0-9_']*)\b", front))
+    reference = """Arrays run run1 runWith run1With stream streamWith Async wait poll cancel runAsync run1Async runAsyncWith
+                   run1AsyncWith Context create destroy unsafeFree unsafeFreeWith performGC performGCWith""".split()
+    assert set(reference) | {"runN", "streamOut", "streamOutWith"} <= exported
 
 
 def test_profile_summaries_were_measured_on_this_tree_s_kernel_sources():
