@@ -358,7 +358,7 @@ def main():
             return lambda: A.check(L.acc_exec_fold(dot.handle, env_s[i], 1, sh, C.byref(od), stream))
         w, e = T.run([step(i) for i in range(Sd)])
         dot_one_by_one = traced([step(i) for i in range(Sd)])
-        truth = float(np.dot(x.astype(np.float64), y.astype(np.float64)))
+        truth = float((x.astype(np.float64) * y.astype(np.float64)).sum())     # (not np.dot: its BLAS threads keep spinning for milliseconds and would take the cores from the copies of the end-to-end leg)
         sk["dot"] = result("fold (+) 0 . zipWith (*) 2^24", w, e, 1, 2 * nd * 4 + 4, nd,
                            {"result": float(o.get()), "float64_truth": truth, "GFLOP_per_s": round(2 * nd / (e * 1e-3) / 1e9, 1),
                             "traffic_key": "foldAll", "one_by_one_us": dot_one_by_one})
