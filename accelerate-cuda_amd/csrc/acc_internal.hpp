@@ -9,6 +9,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <map>
+#include <set>
 #include <memory>
 #include <mutex>
 #include <string>
@@ -237,6 +238,13 @@ struct acc_context_s {
   // kernels report here that a bounded wait ran out (see StatusWord); NULL if the block could not be set up
   volatile uint32_t *status_host = nullptr;
   uint64_t status_dev = 0;
+
+  // Streams and events that were given back while nothing was pending on them wait here for the next request
+  // (the reservoir of Execute/Stream.hs:118-140 and the event table of Execute/Event.hs:63-85), under `mu`.
+  std::vector<hipStream_t> spare_streams;
+  std::vector<hipEvent_t> spare_events[2];          // [0] without timing, [1] with
+  std::set<hipEvent_t> timed_events;                // the events of acc_event_create that record times (an event does not say)
+  static constexpr size_t SPARE_MAX = 64;
 
   // streams with a loop's guard set (acc_stream_set_guard) and the address of its `alive` word
   std::map<hipStream_t, uint64_t> guards;

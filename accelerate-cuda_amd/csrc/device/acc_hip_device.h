@@ -321,14 +321,6 @@ template <typename T> ACC_DEV T acc_stream(const T *p, const Int64 ix)
   T v;
   __builtin_memcpy(&v, b, sizeof(T));
   return v;
-#elif ACC_STREAM_POLICY >= 100
-  /* (measurement only: buffer loads with the cache-policy bits ACC_STREAM_POLICY - 100: 1 sc0, 2 nt, 16 sc1; byte offsets of 32 bits) */
-  static_assert(sizeof(T) == 4, "measurement path");
-  const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void *)p, 0, 0x7fffffff, 0x00020000);
-  const int w = __builtin_amdgcn_raw_buffer_load_b32(r, (int)ix * 4, 0, ACC_STREAM_POLICY - 100);
-  T v;
-  __builtin_memcpy(&v, &w, 4);
-  return v;
 #else
   return __builtin_nontemporal_load(p + ix);
 #endif

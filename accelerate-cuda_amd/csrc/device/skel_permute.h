@@ -342,6 +342,10 @@ ACC_DEV int acc_xcd_id() { return (int)(__builtin_amdgcn_s_getreg(20 | (0 << 6) 
 #ifndef ACC_NARROW_DUMP_VEC
 #define ACC_NARROW_DUMP_VEC 1
 #endif
+#ifndef ACC_NARROW_DUMP_NT
+#define ACC_NARROW_DUMP_NT 0     /* the rows leave in plain stores: behind non-temporal ones the additions to the carries that follow them
+                                    took 1.3 us of a launch instead of 0.4 (2^26 Zipf keys: 53.4 -> 52.5 us a step; uniform keys the same) */
+#endif
 #ifndef ACC_NARROW_STOP
 #define ACC_NARROW_STOP 0xA000u
 #endif
@@ -618,7 +622,11 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
           high = (a.x | a.y | a.z | a.w | b.x | b.y | b.z | b.w) & 0xFF00FF00u;
           acc_u4 o;
           o.x = pack(a.x, b.x); o.y = pack(a.y, b.y); o.z = pack(a.z, b.z); o.w = pack(a.w, b.w);
+#if ACC_NARROW_DUMP_NT
           __builtin_nontemporal_store(o, (acc_u4 *)(wrow + i));
+#else
+          *(acc_u4 *)(wrow + i) = o;
+#endif
         }
         if (__ballot(high != 0u) != 0) {
           for (int q = 0; q < 4; ++q) {

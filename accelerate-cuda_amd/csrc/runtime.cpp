@@ -400,6 +400,9 @@ int acc_context_destroy(acc_context ctx)
   (void)hipSetDevice(ctx->device);
   (void)hipDeviceSynchronize();
   acc::stager_destroy(ctx);
+  for (hipStream_t st : ctx->spare_streams) (void)hipStreamDestroy(st);
+  for (auto &pool : ctx->spare_events)
+    for (hipEvent_t ev : pool) (void)hipEventDestroy(ev);
   for (acc::ScratchBlock &b : ctx->scratch) {
     if (b.done) (void)hipEventDestroy(b.done);
     if (b.ptr) (void)hipFree(b.ptr);
@@ -586,6 +589,15 @@ int acc_stream_create(acc_context ctx, acc_stream *out)
 {
   if (!ctx || !out) return fail(ACC_ERR_INVALID, "acc_stream_create: NULL argument");
   ACC_TRY(ctx->make_current());
+  {
+    // one that was given back idle, if there is one (Execute/Stream.hs:66-74 looks into its reservoir first)
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    if (!ctx->spare_streams.empty()) {
+      *out = ctx->spare_streams.back();
+      ctx->spare_streams.pop_back();
+      return ACC_OK;
+    }
+  }
   hipStream_t s;
   // default priority on purpose; non-blocking w.r.t. the NULL stream as CUDA.Stream.create [] is not
   ACC_HIP_TRY(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
@@ -603,6 +615,18 @@ int acc_stream_destroy(acc_context ctx, acc_stream s)
     // a guard set on the stream goes with it: a later stream commonly gets the same handle value
     std::lock_guard<std::mutex> lock(ctx->mu);
     if (ctx->guards.erase(static_cast<hipStream_t>(s)) != 0) ctx->n_guards.fetch_sub(1, std::memory_order_release);
+  }
+  // A stream with nothing pending is kept for the next acc_stream_create (Execute/Stream.hs:118-140 returns a
+  // stream to the reservoir once its work is done); one that still has work is destroyed, which lets that work
+  // finish and frees the stream behind it.
+  if (hipStreamQuery(static_cast<hipStream_t>(s)) == hipSuccess) {
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    if (ctx->spare_streams.size() < acc_context_s::SPARE_MAX) {
+      ctx->spare_streams.push_back(static_cast<hipStream_t>(s));
+      return ACC_OK;
+    }
+  } else {
+    (void)hipGetLastError();                      // hipErrorNotReady is no error of this call
   }
   ACC_HIP_TRY(hipStreamDestroy(static_cast<hipStream_t>(s)));
   return ACC_OK;
@@ -628,8 +652,21 @@ int acc_event_create(acc_context ctx, int enable_timing, acc_event *out)
 {
   if (!ctx || !out) return fail(ACC_ERR_INVALID, "acc_event_create: NULL argument");
   ACC_TRY(ctx->make_current());
+  {
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    auto &pool = ctx->spare_events[enable_timing ? 1 : 0];
+    if (!pool.empty()) {
+      *out = pool.back();
+      pool.pop_back();
+      return ACC_OK;
+    }
+  }
   hipEvent_t e;
   ACC_HIP_TRY(hipEventCreateWithFlags(&e, enable_timing ? hipEventDefault : hipEventDisableTiming));
+  {
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    if (enable_timing) ctx->timed_events.insert(e);
+  }
   *out = e;
   return ACC_OK;
 }
@@ -639,6 +676,20 @@ int acc_event_destroy(acc_context ctx, acc_event e)
   if (!e) return ACC_OK;
   if (!ctx) return fail(ACC_ERR_INVALID, "acc_event_destroy: NULL context");
   ACC_TRY(ctx->make_current());
+  // An event that is not waiting for anything (never recorded, or what it was recorded behind has completed) is
+  // kept for the next acc_event_create of its kind (Execute/Event.hs:63-85 keeps a table of such events).
+  const hipError_t q = hipEventQuery(static_cast<hipEvent_t>(e));
+  if (q != hipSuccess) (void)hipGetLastError();
+  {
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    const bool timed = ctx->timed_events.count(static_cast<hipEvent_t>(e)) != 0;
+    auto &pool = ctx->spare_events[timed ? 1 : 0];
+    if (q == hipSuccess && pool.size() < acc_context_s::SPARE_MAX) {
+      pool.push_back(static_cast<hipEvent_t>(e));
+      return ACC_OK;
+    }
+    if (timed) ctx->timed_events.erase(static_cast<hipEvent_t>(e));
+  }
   ACC_HIP_TRY(hipEventDestroy(static_cast<hipEvent_t>(e)));
   return ACC_OK;
 }

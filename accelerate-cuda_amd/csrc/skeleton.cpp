@@ -268,6 +268,7 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "#define ACC_PERMUTE_NARROW " << (sp.permute_narrow ? 1 : 0) << "\n";
       if (sp.permute_narrow) o << "#define ACC_NARROW_STOP " << tune("permute.narrow_stop", 0xA000) << "u\n";
       if (sp.permute_narrow && tuned("permute.dump_vec")) o << "#define ACC_NARROW_DUMP_VEC " << (tune("permute.dump_vec", 1) ? 1 : 0) << "\n";
+      if (sp.permute_narrow && tuned("permute.dump_nt")) o << "#define ACC_NARROW_DUMP_NT " << (tune("permute.dump_nt", 0) ? 1 : 0) << "\n";
       if (sp.permute_narrow && tuned("permute.merge_batch")) o << "#define ACC_MERGE_BATCH " << tune("permute.merge_batch", 16) << "\n";
       if (sp.permute_narrow) o << "#define ACC_MERGE_WAVES " << sp.merge_waves << "\n";
       if (tuned("permute.runs")) o << "#define ACC_RUNS " << tune("permute.runs", 1) << "\n";

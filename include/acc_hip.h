@@ -150,7 +150,10 @@ int acc_memcpy_d2h_async(acc_context ctx, void *dst, acc_devptr src, size_t byte
 int acc_memcpy_d2d_async(acc_context ctx, acc_devptr dst, acc_devptr src, size_t bytes, acc_stream s);
 int acc_memset32_async(acc_context ctx, acc_devptr dst, uint32_t value, size_t count, acc_stream s);
 
-/* Execute/Stream.hs:102,134 and Execute/Event.hs:70-127, Debug.hs:48-67 */
+/* Execute/Stream.hs:102,134 and Execute/Event.hs:70-127, Debug.hs:48-67.  A stream that is destroyed with nothing
+ * pending on it, and an event that is destroyed while it waits for nothing, are kept by the context (up to 64 of
+ * each) and handed out by the next create of their kind: the reservoir of Execute/Stream.hs:118-140 and the event
+ * table of Execute/Event.hs:63-85.                                                                            */
 int acc_stream_create(acc_context ctx, acc_stream *out);
 int acc_stream_destroy(acc_context ctx, acc_stream s);
 int acc_stream_sync(acc_context ctx, acc_stream s);

@@ -94,6 +94,23 @@ def test_streams_events_and_pinned_transfers(A, ctx):
         A.check(L.acc_stream_destroy(ctx.handle, st))
     A.check(L.acc_host_free(ctx.handle, hp))
     A.check(L.acc_host_free(ctx.handle, hq))
+    say("streams and events that are given back idle are handed out again")
+    given = {st.value for st in (s, s2)}
+    again = [ctx.stream(), ctx.stream()]
+    assert {st.value for st in again} == given
+    timed = {e0.value, e1.value}
+    e2, e3 = ctx.event(False), ctx.event(True)
+    assert e3.value in timed and e2.value not in timed              # pooled by kind: an untimed event is a new one
+    # a stream that is given back with work pending is not kept: the work still completes
+    busy = again[0]
+    big = ctx.empty(1 << 26, np.int32)
+    A.check(L.acc_memset32_async(ctx.handle, C.c_uint64(big.ptr), 7, C.c_size_t(1 << 26), busy))
+    A.check(L.acc_stream_destroy(ctx.handle, busy))
+    ctx.sync()
+    assert int(big.get()[-1]) == 7
+    A.check(L.acc_stream_destroy(ctx.handle, again[1]))
+    for ev in (e2, e3):
+        A.check(L.acc_event_destroy(ctx.handle, ev))
 
 
 def test_compile_load_launch_a_raw_kernel(A, ctx):

@@ -237,8 +237,18 @@ int main(int argc, char **argv)
     OK(acc_stream_create(ctx, &s2));
     acc_array m = vec(out, 1000), mi = vec(in, 1000);
     acc_skel plain = make(ctx, ACC_SKEL_MAP, "Int32", "arrIn0_0[ix] + 2", nullptr, nullptr, nullptr, 0, 0);
-    if (s2 == s1) OK(acc_exec_map(plain, &mi, &m, s2));    // was refused: "the stream is under a guard"
-    else std::printf("(the new stream did not take the old one's handle value: guard entry not re-tested)\n");
+    // (an idle stream that is given back is the next one handed out: the context keeps it)
+    if (s2 != s1) { std::printf("a stream given back idle was not handed out again\n"); ++failures; }
+    OK(acc_exec_map(plain, &mi, &m, s2));                  // was refused: "the stream is under a guard"
+    acc_event e1 = nullptr, e2 = nullptr, e3 = nullptr;
+    OK(acc_event_create(ctx, 1, &e1));
+    OK(acc_event_record(ctx, e1, s2));
+    OK(acc_event_destroy(ctx, e1));
+    OK(acc_event_create(ctx, 0, &e3));                     // another kind: not the timed one that waits in the pool
+    OK(acc_event_create(ctx, 1, &e2));
+    if (e2 != e1 || e3 == e1) { std::printf("events are not pooled by kind\n"); ++failures; }
+    OK(acc_event_destroy(ctx, e2));
+    OK(acc_event_destroy(ctx, e3));
     OK(acc_skel_destroy(plain));
     OK(acc_guard_destroy(g));
     OK(acc_stream_destroy(ctx, s2));
