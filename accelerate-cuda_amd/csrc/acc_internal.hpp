@@ -233,7 +233,7 @@ struct acc_context_s {
   // large copies from and to pageable host memory go through pinned buffers of the context's own (transfer.cpp)
   acc::Stager *stager = nullptr;
   int copy_helpers = 3;                  // threads that copy beside the caller (knob copy.threads, the caller included)
-  size_t copy_staged_from = 4u << 20;    // bytes from which a pageable copy is staged (knob copy.staged_from_kb; 0 with copy.staged=0: never)
+  size_t copy_staged_from = 4u << 20;    // bytes from which a pageable copy is staged (knob copy.staged_from_kb; the largest size_t with copy.staged=0: never)
 
   // kernels report here that a bounded wait ran out (see StatusWord); NULL if the block could not be set up
   volatile uint32_t *status_host = nullptr;

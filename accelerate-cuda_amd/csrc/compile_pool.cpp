@@ -3,10 +3,10 @@
 // The reference compiles on forked threads, no more at a time than the machine has processors, while its main
 // thread goes on generating code, and blocks only where a kernel is first used (Compile.hs:444-459 `link`, :484-538
 // `build1`, :620-660 `enqueueProcess` / `workers`): that is why a program's kernels take as long to get ready as the
-// slowest of them, not as all of them together.  Here the compiler is hiprtc, in process, and the pool is a set of
-// threads started when the first job arrives.  A job holds copies of all the compiler reads; whoever needs its code
-// waits for it (acc_skel_s::ensure_variant), and gets the worker's error text and compile log as if it had compiled
-// itself.
+// slowest of them, not as all of them together.  Here the compiler is hiprtc and the pool is a set of threads started
+// as jobs arrive, each with a helper process of its own to compile in (compile_child.cpp: hiprtc takes one program at
+// a time per process).  A job holds copies of all the compiler reads; whoever needs its code waits for it
+// (acc_skel_s::ensure_variant), and gets the worker's error text and compile log as if it had compiled itself.
 #include <algorithm>
 #include <cstdlib>
 #include <deque>
@@ -51,7 +51,7 @@ namespace {
 // The pool lives until the process ends.  A worker that is still inside the compiler when exit() starts tearing down
 // static data -- the compiler's own among it, some of it created in the middle of a compilation and therefore torn
 // down BEFORE this pool -- crashes the process on its way out; so a host calls acc_compile_drain before it exits
-// (the Python binding registers it with `atexit`, a Haskell host calls it next to hs_exit).  The destructor does the
+// (the Python binding registers it with `atexit`, the Haskell one registers the C function with the C library's).  The destructor does the
 // same for what is left, which is too late only for a compilation in flight at that moment.
 class Pool {
  public:
