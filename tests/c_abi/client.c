@@ -526,6 +526,65 @@ static void memory_table(acc_context ctx)
   OK(acc_memtable_destroy(mt));
 }
 
+/* ---- kernels compiled in the background, knobs per context, a stencil of rank 4 ------------------------------- */
+static void background_compilation(acc_context ctx)
+{
+  enum { D = 6, N = D * D * D * D };
+  static float v[N], got[N];
+  static int32_t offsets[81 * 4];
+  char fn[81 * 8];
+  acc_skel_desc d;
+  acc_skel_info info;
+  acc_skel box = NULL, twice = NULL;
+  acc_env_sig env[1];
+  acc_array src, out;
+  acc_devptr dsrc, dout;
+  int ready = -1, i, k = 0, a, b, c, e, bad = 0;
+  size_t at = 0;
+  for (i = 0; i < N; ++i) v[i] = (float)(rnd() % 7);
+  for (a = -1; a <= 1; ++a) for (b = -1; b <= 1; ++b) for (c = -1; c <= 1; ++c) for (e = -1; e <= 1; ++e) {
+    offsets[4 * k] = a; offsets[4 * k + 1] = b; offsets[4 * k + 2] = c; offsets[4 * k + 3] = e;
+    at += (size_t)sprintf(fn + at, k ? " + t%d" : "t%d", k);
+    ++k;
+  }
+  CHECK(acc_compile_threads() >= 1, "the pool has room for a worker");
+  OK(acc_context_set_tuning(ctx, "map.block=128"));            /* instances created from now on take the knob ... */
+  memset(&d, 0, sizeof d);
+  env[0] = sig(1, "float");
+  d.kind = ACC_SKEL_MAP;  d.n_env = 1;  d.env = env;  d.elt_type = "float";  d.out_rank = 1;  d.get = "arrIn0_0[ix] * 2.0f";
+  OK(acc_skel_create_async(ctx, &d, &twice));                   /* both handles at once: the kernels compile side by side */
+  OK(acc_context_set_tuning(ctx, NULL));                        /* ... and the process's table is back for the next one */
+  memset(&d, 0, sizeof d);
+  d.kind = ACC_SKEL_STENCIL;  d.elt_type = "float";  d.out_rank = 4;  d.boundary = ACC_BOUNDARY_WRAP;
+  d.n_taps = 81;  d.tap_offsets = offsets;  d.stencil_fn = fn;
+  OK(acc_skel_create_async(ctx, &d, &box));
+  OK(acc_skel_poll(box, &ready));
+  CHECK(ready == 0 || ready == 1, "poll says whether the compilation has ended");
+  OK(acc_skel_prefetch(twice, 1));                              /* the unaligned variant, ahead of any launch that wants it */
+  OK(acc_skel_wait(twice));
+  OK(acc_skel_get_info(twice, &info));
+  CHECK(info.block == 128, "the instance took the knob its context had when it was created");
+  dsrc = upload(ctx, v, sizeof v);
+  OK(acc_malloc(ctx, sizeof v, &dout));
+  memset(&src, 0, sizeof src);  src.rank = 4;  src.ncomp = 1;  src.ptr[0] = dsrc;
+  for (i = 0; i < 4; ++i) src.shape[i] = D;
+  out = src;  out.ptr[0] = dout;
+  OK(acc_exec_stencil(box, NULL, &src, &out, NULL));            /* the first use waits for the kernel */
+  OK(acc_memcpy_d2h(ctx, got, dout, sizeof got));
+  for (a = 0; a < D; ++a) for (b = 0; b < D; ++b) for (c = 0; c < D; ++c) for (e = 0; e < D; ++e) {
+    float sum = 0.0f;                                           /* small integers: exact in any order */
+    for (k = 0; k < 81; ++k)
+      sum += v[((((a + offsets[4 * k] + D) % D) * D + (b + offsets[4 * k + 1] + D) % D) * D + (c + offsets[4 * k + 2] + D) % D) * D +
+               (e + offsets[4 * k + 3] + D) % D];
+    bad += got[((a * D + b) * D + c) * D + e] != sum;
+  }
+  CHECK(bad == 0, "a 3 x 3 x 3 x 3 stencil that wraps round");
+  OK(acc_skel_destroy(box));
+  OK(acc_skel_destroy(twice));
+  acc_free(ctx, dsrc);
+  acc_free(ctx, dout);
+}
+
 int main(int argc, char **argv)
 {
   acc_context ctx = NULL;
@@ -556,8 +615,10 @@ int main(int argc, char **argv)
   guarded_loop(ctx);
   scratch_pool(ctx);
   memory_table(ctx);
+  background_compilation(ctx);
   CHECK(acc_context_sync(ctx) == ACC_OK, "device still healthy");
   acc_context_destroy(ctx);
+  CHECK(acc_compile_drain() == ACC_OK, "nothing is compiling when the process ends");
   printf(failures ? "%d check(s) FAILED\n" : "all checks passed\n", failures);
   return failures ? 1 : 0;
 }
