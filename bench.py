@@ -666,7 +666,6 @@ def main():
                 best = dt
             assert int(res1[-1]) == int(xsc.sum(dtype=np.int64))
             del res1, fresh
-            acc.performGC(fcx)
         fe["scanl"]["run1_ms"] = round(best * 1e3, 3)
         fe["scanl"]["run1_GB_per_s_over_the_link"] = round((2 * n * 4 + 4) / best / 1e9, 2)
         log("  front end run1 scanl           %9.3f ms a call, host array to host array (%.1f GB/s over the link)" % (best * 1e3, (2 * n * 4 + 4) / best / 1e9))
