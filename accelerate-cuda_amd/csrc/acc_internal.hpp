@@ -71,6 +71,9 @@ void set_default_tuning(TuningPtr t);
   X(foldseg_long_from, "foldseg.long_from", 8)                                                                         \
   X(foldseg_max_split, "foldseg.max_split", 4096)                                                                      \
   X(foldseg_oversub, "foldseg.oversub", 1 << 20)                                                                       \
+  X(foldseg_giants, "foldseg.giants", 0)                                                                               \
+  X(foldseg_giant_chunks, "foldseg.giant_chunks", 4)                                                                   \
+  X(foldseg_sweep_per_cu, "foldseg.sweep_per_cu", 4)                                                                   \
   X(foldseg_row_team_below, "foldseg.row_team_below", 1024)                                                            \
   X(foldseg_wave_team_len, "foldseg.wave_team_len", 128)                                                               \
   X(map_oversub, "map.oversub", 1 << 20)                                                                               \

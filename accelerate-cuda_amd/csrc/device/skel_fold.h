@@ -50,48 +50,6 @@ ACC_DEV acc_opt<T> acc_block_reduce(acc_opt<T> x, F f, acc_opt<T> *s_wave)
   return r;
 }
 
-#if ACC_FOLD_SINGLE
-/* A value handed from one workgroup to another without fences: it is cut into
- * 4-byte pieces and every piece travels in a 64-bit word of its own together
- * with the tag of the launch, written and read with relaxed device-scope
- * atomics (write-through, no cache-wide write-back or invalidate as a
- * release/acquire pair costs).  The value has arrived when all its words
- * carry the tag.                                                            */
-template <typename T>
-struct acc_tagged {
-  static constexpr int NW = (int)((sizeof(T) + 3) / 4);
-  unsigned long long *d;
-  ACC_DEV void put(unsigned int slot, unsigned int tag, const T &v) const
-  {
-    unsigned int b[NW] = {};
-    __builtin_memcpy(b, &v, sizeof(T));
-#pragma unroll
-    for (int k = 0; k < NW; ++k)
-      __hip_atomic_store(d + (Int64)slot * NW + k, ((unsigned long long)tag << 32) | b[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-  /* (bounded: a word that does not turn up within ACC_SPIN_LIMIT polls is taken as it is and reported) */
-  ACC_DEV T wait(unsigned int slot, unsigned int tag, unsigned int *status) const
-  {
-    unsigned int b[NW];
-    int polls = 0;
-#pragma unroll
-    for (int k = 0; k < NW; ++k) {
-      unsigned long long w;
-      while ((unsigned int)((w = __hip_atomic_load(d + (Int64)slot * NW + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >> 32) != tag &&
-             polls < ACC_SPIN_LIMIT) {
-        ++polls;
-        __builtin_amdgcn_s_sleep(1);
-      }
-      b[k] = (unsigned int)w;
-    }
-    if (polls >= ACC_SPIN_LIMIT) acc_report(status, ACC_STATUS_FOLD_COLLECT);
-    T v;
-    __builtin_memcpy(&v, b, sizeof(T));
-    return v;
-  }
-};
-#endif
-
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 ACC_ENTRY(ACC_ENV_PARAMS
           ACC_OUT_ARRAY(arrOut),

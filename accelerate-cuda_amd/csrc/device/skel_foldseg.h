@@ -72,6 +72,51 @@ static_assert(ACC_CHUNK % (ACC_BLOCK * ACC_VEC) == 0, "chunk must be a whole num
 #define ACC_SEG_END(s) ACC_SEG_AT((s) + 1)
 #endif
 
+/* ACC_GIANTS: among many short segments a few may hold most of the source (the rows of a power-law graph).  The
+ * workgroup that owns such a segment would stream it alone, chunk after chunk, long after the others have ended: one
+ * segment of 2^23 elements among a million short ones took 6-12 ms.  So where a workgroup has folded a stretch of a
+ * segment together (ACC_WIDE, below) and ACC_GIANT_FROM elements or more of that segment lie beyond the chunk, the
+ * rest is handed over: the owner enters it in a table of jobs in scratch memory, with the value of what it has
+ * folded of the segment so far, and goes on with the chunk in which the segment ends.  A second launch, <entry>_sweep
+ * at the end of this file, takes the jobs in pieces of ACC_GIANT_PIECE elements, by ticket, until none is left; a
+ * piece is folded in index order, all lanes together, and its value left as tagged words.  A job's tickets come
+ * from ACC_GIANT_LINES counters, a cache line of their own each, every one for a run of consecutive pieces
+ * (additions to one word, and to the words of one cache line, are performed one after the other).  Whoever draws
+ * the ticket behind the last piece of the last line puts the owner's value and the pieces together, in order, and
+ * writes the segment's result.  The only wait is that workgroup's, for pieces whose tickets were drawn before its
+ * own -- by workgroups that are running, or done; it is bounded like every wait.  With no room in the table the
+ * segment stays with its owner as if there were no table.  The table and the values carry the launch's tag
+ * (nothing is cleared between launches).  Index order, another association than the sequential fold's: as for
+ * every long segment.
+ *   Off unless the instance is built with `foldseg.giants=1`.  The code in this kernel lies behind the test for a
+ * stretch that the workgroup folds together, and yet, with it compiled in and no such segment in the source, 2^25
+ * elements in segments of 2 / 8 / 32 took 101 / 36 / 29 us instead of 89 / 33 / 27 and the sparse matrix-vector
+ * product 193 instead of 190; the second launch costs a source without such segments 2-3 us more.  (A test of
+ * every block of segments ahead of its first chunk, by way of a barrier that carries the lanes' verdicts, made the
+ * segments of two elements 117 us: the block's first loads then wait for the lanes' offsets.)                   */
+#ifndef ACC_GIANTS
+#define ACC_GIANTS 0
+#endif
+#if ACC_SEG_UNIFORM || ACC_SEG_OUTER
+#undef ACC_GIANTS
+#define ACC_GIANTS 0                                     /* (segments of one length; rows with segments of their own) */
+#endif
+#if ACC_GIANTS
+#define ACC_GIANT_PARAMS , unsigned long long *__restrict__ acc_jobs, const unsigned int acc_epoch, unsigned int *acc_status
+#ifndef ACC_GIANT_CHUNKS
+#define ACC_GIANT_CHUNKS 4
+#endif
+#define ACC_GIANT_PIECE ((Int64)ACC_GIANT_CHUNKS * ACC_CHUNK)
+#define ACC_GIANT_FROM  (2 * ACC_GIANT_PIECE)
+#define ACC_GIANT_JOBS  32                               /* the host sizes the scratch block by these three */
+#define ACC_GIANT_HEAD  8                                /* 64-bit words in front of the jobs */
+#define ACC_GIANT_LINES 16                               /* ticket counters a job, each for a run of its pieces */
+#define ACC_GIANT_SPREAD 32                              /* words between two counters: additions to one cache line queue like additions to one word */
+#define ACC_GIANT_JOB   (8 + ACC_GIANT_LINES * ACC_GIANT_SPREAD)           /* 64-bit words a job: tag, segment, first, end, lines that have run out, 3 unused, the counters */
+#else
+#define ACC_GIANT_PARAMS
+#endif
+
 #define ACC_LOADS (ACC_CHUNK / (ACC_BLOCK * ACC_VEC))   /* vector loads per lane and chunk */
 /* One word of padding per 32 elements of the staged chunk: lanes that fold segments whose starts are a multiple
  * of 32 elements apart (every segment 32, 64, 128 ... long) would otherwise all read the same LDS bank.  The padding
@@ -88,15 +133,57 @@ static_assert(ACC_CHUNK % (ACC_BLOCK * ACC_VEC) == 0, "chunk must be a whole num
 #define ACC_WIDE 256                                     /* elements of one segment in a chunk from which the workgroup folds them together */
 #endif
 
+#if ACC_GIANTS
+/* enter elements [a, b) of segment `seg` in the table of jobs; the job's number, or -1 if the table is full */
+ACC_DEV int acc_giant_enter(unsigned long long *jobs, const unsigned int epoch, const Int64 seg, const Int64 a, const Int64 b)
+{
+  unsigned long long h = __hip_atomic_load(jobs, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  unsigned int at;
+  for (;;) {                                     /* the head word: {tag of the launch, jobs entered so far} */
+    at = (unsigned int)(h >> 32) == epoch ? (unsigned int)h : 0u;
+    if (at >= ACC_GIANT_JOBS) return -1;
+    const unsigned long long want = ((unsigned long long)epoch << 32) | (at + 1u);
+    if (__hip_atomic_compare_exchange_strong(jobs, &h, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) break;
+  }
+  unsigned long long *j = jobs + ACC_GIANT_HEAD + (Int64)at * ACC_GIANT_JOB;
+  __hip_atomic_store(j + 1, (unsigned long long)seg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(j + 2, (unsigned long long)a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(j + 3, (unsigned long long)b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(j + 4, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  for (int k = 0; k < ACC_GIANT_LINES; ++k) __hip_atomic_store(j + 8 + k * ACC_GIANT_SPREAD, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      /* the job is whole before its tag says that it is there */
+  __hip_atomic_store(j, (unsigned long long)epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      /* and the tag is there before the owner itself comes to look */
+  return (int)at;
+}
+
+/* where the value that a job's owner has folded itself goes: behind the two values for every piece of the source */
+ACC_DEV unsigned int acc_giant_edge_slot(const Int64 n, const int job) { return (unsigned int)(2 * (n / ACC_GIANT_PIECE + 2) + job); }
+
+/* one more of the launch's jobs has no ticket left: the word behind the head word, {tag of the launch, such jobs} */
+ACC_DEV void acc_giant_ran_out(unsigned long long *jobs, const unsigned int epoch)
+{
+  unsigned long long h = __hip_atomic_load(jobs + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  for (;;) {
+    const unsigned int at = (unsigned int)(h >> 32) == epoch ? (unsigned int)h : 0u;
+    const unsigned long long want = ((unsigned long long)epoch << 32) | (at + 1u);
+    if (__hip_atomic_compare_exchange_strong(jobs + 1, &h, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) break;
+  }
+}
+#endif
+
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
                   const Int64 shOut_0, ACC_OUT_ARRAY(arrOut),
-                  ACC_SEG_PARAMS ACC_GUARD_PARAM)
+                  ACC_SEG_PARAMS ACC_GIANT_PARAMS ACC_GUARD_PARAM)
 {
   ACC_GUARD_CHECK
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
   __shared__ __attribute__((aligned(16))) T s_val[ACC_PAD_SPACE(ACC_CHUNK)];
+#if ACC_GIANTS
+  __shared__ int s_skip;
+#endif
   /* for the stretches the whole workgroup folds (below) */
   __shared__ int s_wide[ACC_BLOCK / ACC_WAVE];
   __shared__ int s_owner, s_from, s_to;
@@ -113,6 +200,9 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
   const T seed = (ACC_SEED);
 #endif
   if (tid == 0) s_owner = ACC_BLOCK;
+#if ACC_GIANTS
+  if (tid == 0) s_skip = -1;
+#endif
   /* (the loop over this workgroup's blocks of segments, compiled with and without the padding: an address that adds
    * the padding under a run-time mask costs the inner loop more than the bank conflicts it avoids) */
   auto blocks_of_segments = [&](auto padded_c) {
@@ -126,10 +216,11 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
      * and takes nothing) */
     const Int64 seg_c = acc_min<Int64>(seg, nseg - 1);
     const Int64 a_c = ACC_SEG_AT(seg_c), b_c = ACC_SEG_END(seg_c);
-    const Int64 a = live ? a_c : 0;
-    const Int64 b = live ? b_c : 0;
+    Int64 a = live ? a_c : 0;
+    Int64 b = live ? b_c : 0;
     const Int64 last = acc_min<Int64>(first + ACC_BLOCK, nseg);
     const Int64 lo = ACC_SEG_AT(first), hi = acc_min<Int64>(ACC_SEG_END(last - 1), n);
+    bool handed = false;                             /* this lane's segment has been handed over (below) */
 
     T acc = T();
     bool have = false;
@@ -269,13 +360,43 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
 #endif
             have = true;
             pending = false;
+#if ACC_GIANTS
+            /* What is left of the segment beyond this chunk, if that is ACC_GIANT_FROM elements or more, is handed
+             * over: entered in the table of jobs, together with the value of what has been folded so far, and this
+             * workgroup goes on with the chunk in which the segment ends. */
+            const Int64 rest = ACC_FOLD_RIGHT ? cs - a : b - ce;
+            if (acc_jobs && rest >= ACC_GIANT_FROM) {
+              const int job = ACC_FOLD_RIGHT ? acc_giant_enter(acc_jobs, acc_epoch, seg, a, cs) : acc_giant_enter(acc_jobs, acc_epoch, seg, ce, b);
+              if (job >= 0) {                                      /* (no room in the table: the segment stays here) */
+                const acc_tagged<T> values_of = {acc_jobs + ACC_GIANT_HEAD + ACC_GIANT_JOBS * ACC_GIANT_JOB};
+                values_of.put(acc_giant_edge_slot(n, job), acc_epoch, acc);
+                s_skip = ACC_FOLD_RIGHT ? (int)(nchunks - 1 - (a - lo_al) / ACC_CHUNK) : (int)((b - lo_al) / ACC_CHUNK);
+                handed = true;
+#if ACC_FOLD_RIGHT
+                a = b;                                             /* nothing of it is this lane's any more */
+#else
+                b = a;
+#endif
+              }
+            }
+#endif
           }
         }
+#if ACC_GIANTS
+        /* (the turns end with a barrier: what an owner has written is seen by all) */
+        const int skip_to = s_skip;
+        if (skip_to >= 0) {                                        /* the same in every lane */
+          __syncthreads();
+          if (tid == 0) s_skip = -1;
+          if (skip_to < nchunks) stage(chunk_start(skip_to));      /* (in place of the chunk asked for above) */
+          q = skip_to - 1;
+        }
+#endif
       }
 
     }
 
-    if (live) {
+    if (live && !handed) {
 #if ACC_HAS_SEED && !ACC_FOLD_RIGHT
       ACC_SET(arrOut, seg, have ? f(acc, seed) : seed);
 #else
@@ -290,6 +411,7 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
 #else
   blocks_of_segments(acc_bool<ACC_PAD_ON != 0>());
 #endif
+
 }
 
 #if ACC_SEG_UNIFORM
@@ -572,3 +694,176 @@ ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _join)(ACC_ENV_PARAMS
   ACC_SET(arrOut, seg, acc.v);
 #endif
 }
+
+#if ACC_GIANTS
+/* ---- the segments that were handed over -------------------------------------
+ * <entry>_sweep, launched behind <entry> with as many workgroups as the device holds at once: they take the jobs'
+ * pieces by ticket until none is left, and the workgroup that draws the ticket behind a job's last piece puts the
+ * owner's value and the pieces together and writes the segment's result.  (As a part of <entry> -- every workgroup
+ * looking at the table when its own segments were done -- this took 20 registers of it, and a segment met by the
+ * workgroup that is started last found nobody left to take pieces.)  With an empty table the launch is a read of
+ * 16 bytes a workgroup.  Same parameters as <entry>. */
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _sweep)(ACC_ENV_PARAMS
+                                      const Int64 shOut_0, ACC_OUT_ARRAY(arrOut),
+                                      ACC_SEG_PARAMS ACC_GIANT_PARAMS ACC_GUARD_PARAM)
+{
+  ACC_GUARD_CHECK
+  typedef ACC_ELT T;
+  ACC_ENV_ASSUME
+  (void)shOut_0;
+  (void)arrSeg_0;
+  __shared__ __attribute__((aligned(16))) T s_val[ACC_PAD_SPACE(ACC_CHUNK)];
+  __shared__ unsigned long long s_job[8 + ACC_GIANT_LINES];
+  __shared__ acc_opt<T> s_part[ACC_BLOCK / ACC_WAVE];
+  auto get = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
+  auto f   = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
+  auto lf  = acc_lift<T>(f);
+  const Int64 n = ACC_SEG_TOTAL;
+  const int tid = threadIdx.x;
+#if ACC_HAS_SEED
+  const T seed = (ACC_SEED);
+#endif
+  /* an ordered fold of s_val[from .. to) by all lanes: every lane a run of consecutive elements, the lanes joined in
+   * lane order and the waves in wave order */
+  auto together = [&](const int from, const int to) -> acc_opt<T> {
+    constexpr int acc_pad_mask = ACC_PAD_ON ? ~0 : 0;
+    const int per = (to - from + ACC_BLOCK - 1) / ACC_BLOCK;
+    const int i0 = acc_min(from + tid * per, to), i1 = acc_min(i0 + per, to);
+    acc_opt<T> m = acc_none<T>();
+    for (int i = i0; i < i1; ++i) m = lf(m, acc_some(s_val[ACC_PAD(i)]));
+    m = acc_wave_reduce(m, lf);
+    if (acc_lane() == 0) s_part[tid >> 6] = m;
+    __syncthreads();
+    acc_opt<T> whole = s_part[0];
+#pragma unroll
+    for (int w = 1; w < ACC_BLOCK / ACC_WAVE; ++w) whole = lf(whole, s_part[w]);
+    return whole;
+  };
+  /* elements [from, to) of the source folded by the whole workgroup, chunk by chunk in index order (to > from) */
+  auto fold_range = [&](const Int64 from, const Int64 to) -> acc_opt<T> {
+    constexpr int acc_pad_mask = ACC_PAD_ON ? ~0 : 0;
+    acc_opt<T> value = acc_none<T>();
+    for (Int64 cs = from - from % ACC_VEC; cs < to; cs += ACC_CHUNK) {
+      __syncthreads();                                              /* the chunk before has been read */
+      {
+        T w[ACC_LOADS][ACC_VEC];
+        const bool whole = cs + ACC_CHUNK <= n;                     /* (the same in every lane) */
+#pragma unroll
+        for (int u = 0; u < ACC_LOADS; ++u)
+#pragma unroll
+          for (int k = 0; k < ACC_VEC; ++k) {
+            const Int64 ix = cs + (u * ACC_BLOCK + tid) * ACC_VEC + k;
+            w[u][k] = get(whole ? ix : acc_min<Int64>(ix, n - 1));  /* (what lies beyond `to` is never read back) */
+          }
+#pragma unroll
+        for (int u = 0; u < ACC_LOADS; ++u)
+#pragma unroll
+          for (int k = 0; k < ACC_VEC; ++k) s_val[ACC_PAD((u * ACC_BLOCK + tid) * ACC_VEC + k)] = w[u][k];
+      }
+      __syncthreads();
+      value = lf(value, together((int)(acc_max(from, cs) - cs), (int)(acc_min(to, cs + ACC_CHUNK) - cs)));
+    }
+    return value;
+  };
+  {
+    const acc_tagged<T> pieces_of = {acc_jobs + ACC_GIANT_HEAD + ACC_GIANT_JOBS * ACC_GIANT_JOB};
+    if (tid < 2) s_job[tid] = __hip_atomic_load(acc_jobs + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    const unsigned long long head = s_job[0], out = s_job[1];
+    const int entered = (unsigned int)(head >> 32) == acc_epoch ? (int)acc_min<unsigned int>((unsigned int)head, ACC_GIANT_JOBS) : 0;
+    const int ran_out = (unsigned int)(out >> 32) == acc_epoch ? (int)(unsigned int)out : 0;
+    /* as many jobs without a ticket left as there are jobs: nothing to take (most workgroups of a large launch come
+     * here after the last piece has gone, and are spared the look at every job) */
+    const int jobs_in = ran_out >= entered ? 0 : entered;
+    for (int j = 0; j < jobs_in; ++j) {
+      unsigned long long *job = acc_jobs + ACC_GIANT_HEAD + (Int64)j * ACC_GIANT_JOB;
+      __syncthreads();
+      if (tid < 8 + ACC_GIANT_LINES) s_job[tid] = __hip_atomic_load(job + (tid < 8 ? tid : 8 + (tid - 8) * ACC_GIANT_SPREAD), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __syncthreads();
+      if ((unsigned int)s_job[0] != acc_epoch) continue;            /* (entered and not filled in: not after the launch that enters them has ended) */
+      const Int64 g_seg = (Int64)s_job[1], g_a = (Int64)s_job[2], g_b = (Int64)s_job[3];
+      const Int64 p_first = g_a / ACC_GIANT_PIECE, p_count = (g_b - 1) / ACC_GIANT_PIECE - p_first + 1;
+      /* Tickets are drawn from ACC_GIANT_LINES counters, each for a run of `p_line` consecutive pieces, and a
+       * workgroup starts at the counter its number names: additions to ONE word are performed one after the other,
+       * 0.1 us each, so that the thousand workgroups that end together and ask for a ticket at the same moment were
+       * handed theirs over 100 us.  And a look before a ticket is drawn: a counter that has run out (as the words
+       * just read say) is not asked again -- thousands of workgroups that each drew a ticket only to find the job
+       * done kept a launch busy for 200 us. */
+      const Int64 p_line = (p_count + ACC_GIANT_LINES - 1) / ACC_GIANT_LINES;
+      const Int64 lines_in_use = (p_count + p_line - 1) / p_line;
+      /* Where a piece's value goes: two values for every piece of the source.  A handed-over segment is at least two
+       * pieces long, so a piece of the source is shared by two of them at most -- one that ends in it and one that
+       * begins in it -- and the one that begins there (its piece 0) takes the odd place. */
+      auto slot_of = [&](const Int64 piece) -> unsigned int { return (unsigned int)(2 * (p_first + piece) + (piece == 0 ? 1 : 0)); };
+      /* A workgroup goes to the line its number names; when that has run out it looks at the counters again and goes
+       * to the next line that has not, until none is left.  (A line has one ticket more than pieces: whoever draws it
+       * knows that the line has run out, and a counter beyond it says so to everybody who looks.) */
+      auto line_first = [&](const int l) -> Int64 { return acc_min<Int64>((Int64)l * p_line, p_count); };
+      auto line_count = [&](const int l) -> Int64 { return acc_min<Int64>(line_first(l) + p_line, p_count) - line_first(l); };
+      for (int turn = 0; turn <= ACC_GIANT_LINES; ++turn) {
+      if (turn > 0) {                                               /* the counters as they stand now */
+        __syncthreads();
+        if (tid < ACC_GIANT_LINES) s_job[8 + tid] = __hip_atomic_load(job + 8 + tid * ACC_GIANT_SPREAD, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+      }
+      int line = -1;
+      for (int k = 0; k < ACC_GIANT_LINES && line < 0; ++k) {
+        const int l = (int)((blockIdx.x + (unsigned int)k) % ACC_GIANT_LINES);
+        if (line_count(l) > 0 && (Int64)s_job[8 + l] <= line_count(l)) line = l;
+      }
+      if (line < 0) break;                                          /* every line has run out */
+      const Int64 l_first = line_first(line), l_count = line_count(line);
+      for (;;) {
+        __syncthreads();
+        if (tid == 0) {
+          unsigned long long t = __hip_atomic_fetch_add(job + 8 + line * ACC_GIANT_SPREAD, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          /* the ticket behind a line's last piece: one line more has run out; the last such line ends the job */
+          if ((Int64)t == l_count &&
+              (Int64)__hip_atomic_fetch_add(job + 4, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1 == lines_in_use) {
+            acc_giant_ran_out(acc_jobs, acc_epoch);
+            t = ~0ull;
+          }
+          s_job[0] = t;
+        }
+        __syncthreads();
+        const Int64 ticket = s_job[0] == ~0ull ? -1 : (Int64)s_job[0];
+        if (ticket >= l_count) break;
+        if (ticket < 0) {
+          /* Every piece of every line has been drawn (whoever folds a piece asks for another ticket afterwards, so the
+           * ticket behind a line's last piece is always drawn, and by one workgroup): the pieces are put together
+           * here, in order.  Each is waited for by its tag -- the workgroups that drew them are running, or done. */
+          const Int64 per = (p_count + ACC_BLOCK - 1) / ACC_BLOCK;
+          const Int64 i0 = acc_min<Int64>((Int64)tid * per, p_count), i1 = acc_min<Int64>(i0 + per, p_count);
+          acc_opt<T> m = acc_none<T>();
+          for (Int64 i = i0; i < i1; ++i) m = lf(m, acc_some(pieces_of.wait(slot_of(i), acc_epoch, acc_status)));
+          m = acc_wave_reduce(m, lf);
+          if (acc_lane() == 0) s_part[tid >> 6] = m;
+          __syncthreads();
+          if (tid == 0) {
+            acc_opt<T> whole = s_part[0];
+#pragma unroll
+            for (int w = 1; w < ACC_BLOCK / ACC_WAVE; ++w) whole = lf(whole, s_part[w]);
+            /* and joined with what the owner folded itself before it handed the rest over */
+            const T edge = pieces_of.wait(acc_giant_edge_slot(n, j), acc_epoch, acc_status);
+#if ACC_FOLD_RIGHT
+            ACC_SET(arrOut, g_seg, f(whole.v, edge));               /* (a seed is in the owner's value already) */
+#elif ACC_HAS_SEED
+            ACC_SET(arrOut, g_seg, f(f(edge, whole.v), seed));
+#else
+            ACC_SET(arrOut, g_seg, f(edge, whole.v));
+#endif
+          }
+          break;
+        }
+        /* piece p_first + l_first + ticket of the source, as far as it belongs to the segment, chunk by chunk in index order */
+        const Int64 piece = l_first + ticket;
+        const Int64 from = acc_max(g_a, (p_first + piece) * ACC_GIANT_PIECE), to = acc_min(g_b, (p_first + piece + 1) * ACC_GIANT_PIECE);
+        const acc_opt<T> value = fold_range(from, to);
+        if (tid == 0) pieces_of.put(slot_of(piece), acc_epoch, value.v);
+      }
+      }   /* lines */
+    }
+  }
+}
+#endif

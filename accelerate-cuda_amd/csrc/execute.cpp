@@ -299,8 +299,11 @@ namespace {
 //   from `foldseg.block_team_len` a workgroup, takes one segment at a time;
 //   fewer long segments than the device has room for teams: every segment is cut into `split` pieces, a team
 //   each, and a second launch joins the pieces in order.
+//   `giants` (foldSeg of a vector): the kernel of the short segments hands segments of 8 chunks or more over to a
+//   table of jobs that every workgroup helps with when its own segments are done (skel_foldseg.h, ACC_GIANTS); the
+//   table and the pieces' values live in a block of tagged words sized by the source.
 int launch_segmented(acc_skel_s *s, int v, Args *args, const acc_array *env, const acc_array *out, int64_t nseg, int64_t n,
-                     hipStream_t st)
+                     hipStream_t st, bool giants = false)
 {
   const int64_t avg = n / nseg;
   if (avg < s->knobs.foldseg_wave_team_len) {
@@ -313,7 +316,28 @@ int launch_segmented(acc_skel_s *s, int v, Args *args, const acc_array *env, con
       ACC_TRY(s->ensure_variant(lv));
     }
     const int64_t grid = acc_launch_grid(nseg, s->spec.block, resident(s, lv), s->knobs.foldseg_oversub);
-    return launch(s, lv, grid, 0, st, args);
+    // an instance built with `foldseg.giants=1` takes a table of jobs (skel_foldseg.h, ACC_GIANTS): head, 32 jobs of
+    // 8 words and 16 ticket counters 32 words apart, then values of tagged words -- two for every piece of 4 chunks
+    // the source has, and one a job
+    if (!giants || s->knobs.foldseg_giants == 0) return launch(s, lv, grid, 0, st, args);
+    const int64_t piece = (int64_t)std::max(1, s->knobs.foldseg_giant_chunks) * (int64_t)(lv >= 2 ? s->spec.chunk_long : s->spec.chunk);
+    const size_t words_a_value = ((size_t)s->spec.elt_size + 3) / 4;
+    const size_t bytes = (8 + 32 * (8 + 16 * 32) + (2 * (size_t)(n / piece + 2) + 32) * words_a_value) * 8;
+    acc::ScratchRef jobs;
+    ACC_TRY(s->ctx->scratch_acquire(bytes, st, acc::SCRATCH_FLAGS, &jobs));
+    args->ptr(reinterpret_cast<uint64_t>(jobs.ptr));
+    args->u32(jobs.epoch);
+    args->ptr(s->ctx->status_dev);
+    int rc = launch(s, lv, grid, 0, st, args);
+    if (rc == ACC_OK) {
+      // the second launch, which takes what the first has entered in the table: as many workgroups as the device holds
+      const int64_t sweepers = (int64_t)s->ctx->props.multiProcessorCount * std::max(1, std::min(s->knobs.foldseg_sweep_per_cu, 2048 / s->spec.block));
+      hipError_t e = launch_kernel(s->variants[lv].fn_sweep, static_cast<unsigned>(sweepers), 1, 1, static_cast<unsigned>(s->spec.block), 1, 1, 0, st,
+                                   args->data(), nullptr);
+      if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(segmented fold, sweep)");
+    }
+    s->ctx->scratch_release(jobs, st);
+    return rc;
   }
   // teams: a workgroup (1) from `foldseg.block_team_len`, a row of 16 lanes (2) below `foldseg.row_team_below`, else a wave (0)
   const int block_team = avg >= s->knobs.foldseg_block_team_len ? 1 : (avg < s->knobs.foldseg_row_team_below ? 2 : 0);
@@ -515,7 +539,7 @@ int acc_exec_foldseg_nd(acc_skel s, const acc_array *env, int32_t in_rank, const
   }
   const int v = aligned ? 0 : 1;
   ACC_TRY(s->ensure_variant(v));
-  return launch_segmented(s, v, &args, env, out, nseg, n, static_cast<hipStream_t>(stream));
+  return launch_segmented(s, v, &args, env, out, nseg, n, static_cast<hipStream_t>(stream), rank == 1);
 }
 
 int acc_exec_foldseg(acc_skel s, const acc_array *env, int64_t n, const acc_array *offsets, const acc_array *out, acc_stream stream)

@@ -411,6 +411,8 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
   }
   o << "#define ACC_ENTRY " << *entry << "\n";
   o << "#define ACC_NT_STORE " << tune("nt_store", 1) << "\n";
+  if (tune("foldseg.giants", 0) != 0) o << "#define ACC_GIANTS 1\n";
+  if (tuned("foldseg.giant_chunks")) o << "#define ACC_GIANT_CHUNKS " << std::max(1, tune("foldseg.giant_chunks", 4)) << "\n";
   if (tuned("stream.policy")) o << "#define ACC_STREAM_POLICY " << tune("stream.policy", 1) << "\n";
   if (sp.guarded) o << "#define ACC_GUARDED 1\n";
   if (tuned("spin_limit")) o << "#define ACC_SPIN_LIMIT " << std::max(0, tune("spin_limit", 1 << 22)) << "\n";
@@ -872,6 +874,15 @@ int acc_skel_s::ensure_variant(int v)
       (void)hipModuleUnload(var.module);
       var.module = nullptr;
       return acc::fail_hip(e, ("hipModuleGetFunction(" + third + ")").c_str());
+    }
+  }
+  if ((spec.kind == ACC_SKEL_FOLDSEG || spec.kind == ACC_SKEL_FOLD1SEG) && spec.out_rank <= 1 && knobs.foldseg_giants != 0) {
+    const std::string sweep = entry_name + "_sweep";
+    e = hipModuleGetFunction(&var.fn_sweep, var.module, sweep.c_str());
+    if (e != hipSuccess) {
+      (void)hipModuleUnload(var.module);
+      var.module = nullptr;
+      return acc::fail_hip(e, ("hipModuleGetFunction(" + sweep + ")").c_str());
     }
   }
   if ((spec.kind == ACC_SKEL_FOLD || spec.kind == ACC_SKEL_FOLD1) && spec.out_rank > 0) {

@@ -69,6 +69,7 @@ struct Variant {
   hipFunction_t fn_finish = nullptr;   // second kernel: foldAll's _finish, permute's _merge / _join, the segmented fold's _team
   hipFunction_t fn_fill = nullptr;     // third kernel: permute's _fill (identity into the table rows), the segmented fold's _join
   hipFunction_t fn_rows = nullptr;     // fold along the innermost dimension: _rows, a lane per short row
+  hipFunction_t fn_sweep = nullptr;    // a segmented fold built with `foldseg.giants=1`: _sweep, the segments that were handed over
   int num_regs = 0;
   int static_lds = 0;
   int blocks_per_cu = 1;

@@ -754,8 +754,32 @@ def main():
             tr = ctx.skeleton(A.SKEL_MAP, "float", env=[(2, "float")], out_rank=2, flags=flags, get="arrIn0_0[(ix % shOut_0) * shIn0_0 + (ix / shOut_0)]")
             one("transpose 8192 x 8192 Float32 " + name, lambda: A.check(L.acc_exec_map(tr.handle, se, C.byref(dd), stream)), 8 * side * side)
         assert np.array_equal(dst.get(), wl.stencil_image(side, side).T), "transpose mismatch"
-        sk["shapes"] = shapes
         del src, dst
+        # segmented sums whose lengths are very unequal: a million segments of 8 elements on average, one of which holds
+        # half of the source (the rows of a power-law graph); the same elements all in segments of 8; and the former
+        # through an instance built with `foldseg.giants=1`, which hands the long segment over to all workgroups
+        nseg, big = 1 << 20, 1 << 23
+        for name, giant, knobs in (("every segment short", 0, ""), ("one segment of 2^23 elements among them", big, ""),
+                                   ("one segment of 2^23 elements among them, foldseg.giants=1", big, "foldseg.giants=1")):
+            with A.tuning(knobs, ctx):
+                seg_s = ctx.skeleton(A.SKEL_FOLDSEG, "float", env=[F32], get=rd(0), combine="x + y", seed="0.0f")
+            rng_l = np.random.default_rng(5)
+            lens = rng_l.poisson(8, nseg).astype(np.int64)
+            if giant:
+                lens[nseg // 3] = giant
+            else:
+                lens = np.concatenate([lens, rng_l.poisson(8, big // 8).astype(np.int64)])
+            offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+            nel = int(offs[-1])
+            xv_ = ctx.array(np.ones(nel, np.float32))
+            do_, out_ = ctx.array(offs), ctx.empty(lens.size, np.float32)
+            xe, dd_, od_ = envs(xv_), do_.desc(), out_.desc()
+            one("foldSeg (+) Float32, %d segments, %s" % (lens.size, name),
+                lambda: A.check(L.acc_exec_foldseg(seg_s.handle, xe, nel, C.byref(dd_), C.byref(od_), stream)), 4 * nel + 8 * lens.size)
+            assert np.array_equal(out_.get(), lens.astype(np.float32)), "segmented sums mismatch"
+            del xv_, do_, out_
+            seg_s.destroy()
+        sk["shapes"] = shapes
 
     if headline is None:     # --only without scan: report whatever ran first
         timed = sorted(k for k in sk if "ms_per_step" in sk[k])

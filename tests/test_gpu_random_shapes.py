@@ -212,6 +212,81 @@ __device__ __forceinline__ Word32 affine16(Word32 x, Word32 y) {
             assert int(gotr[s_]) == chain(u[offs[s_]:offs[s_ + 1]], 0x00030005), ("foldSeg right", s_, int(lens[s_]))
 
 
+def test_segments_that_are_handed_over(A, ctx, tuned):
+    """instances built with `foldseg.giants=1`: among short segments, segments that go on for eight staged chunks or
+    more beyond the chunk in which the workgroup first folds a stretch of them together.  Their owner enters the rest
+    in a table of jobs and the workgroups take pieces of it when their own segments are done.  Several in one block of
+    256 segments, next to one another, first and last of the array, more of them than the table has room for (the rest
+    stay with their owners), the whole array one segment; sums of integers (exact), a non-commutative operator in both
+    associations (the order of the pieces and of the owner's own part), pairs (a value of several tagged words), and
+    the same inputs through instances built without the table."""
+    rng = np.random.default_rng(88)
+    aff = """
+__device__ __forceinline__ Word32 affine16(Word32 x, Word32 y) {
+  Word32 a1 = x >> 16, b1 = x & 0xffffu, a2 = y >> 16, b2 = y & 0xffffu;
+  return (((a1 * a2) & 0xffffu) << 16) | ((a1 * b2 + b1) & 0xffffu);
+}
+"""
+    G = 30000                                        # above eight chunks of either staged length (2048, 3072)
+    cases = [
+        ("one in the middle", 3000, 3, {1500: 5 * G}),
+        ("first and last", 2000, 5, {0: 2 * G + 1, 1999: 3 * G + 7}),
+        ("three in one block, two of them neighbours", 1000, 2, {300: G, 301: 2 * G + 3, 420: G + 5}),
+        ("behind empty segments", 700, 0, {5: 4 * G}),
+        ("more than the table holds", 40 * 256, 1, {256 * k + 7: G + k for k in range(40)}),
+        ("the whole array", 1, 0, {0: 6 * G + 11}),
+        ("long ones that stay beside one that goes", 600, 4, {100: G - 5000, 101: 3 * G, 102: 12000, 103: 300}),
+    ]
+
+    def run_all(label):
+        fs = ctx.skeleton(A.SKEL_FOLDSEG, "Int32", env=[(1, "Int32")], out_rank=1, get="arrIn0_0[ix]", combine="x + y", seed="5")
+        f1 = ctx.skeleton(A.SKEL_FOLD1SEG, "Word32", env=[(1, "Word32")], out_rank=1, get="arrIn0_0[ix]", combine="affine16(x, y)", preamble=aff)
+        fr = ctx.skeleton(A.SKEL_FOLDSEG, "Word32", env=[(1, "Word32")], out_rank=1, get="arrIn0_0[ix]", combine="affine16(x, y)",
+                          seed="0x00030005u", preamble=aff, flags=A.FLAG_FOLD_RIGHT)
+        fp = ctx.skeleton(A.SKEL_FOLDSEG, "Int64, Int32", env=[(1, "Int32")], out_rank=1, get="acc_elt{(Int64)arrIn0_0[ix], 1}",
+                          combine="acc_elt{x.a1 + y.a1, x.a0 + y.a0}", seed="acc_elt{0, 0}")
+        for name, nseg, mean, longs in cases:
+            lens = rng.poisson(mean, nseg).astype(np.int64) if mean else np.zeros(nseg, np.int64)
+            for at, ln in longs.items():
+                lens[at] = ln
+            offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+            n = int(offs[-1])
+            say("segments handed over:", label, name, "nseg", nseg, "n", n)
+            x = rng.integers(-9, 9, n).astype(np.int32)
+            c = np.concatenate([[0], np.cumsum(x.astype(np.int64))])
+            sums = c[offs[1:]] - c[offs[:-1]]
+            out = ctx.empty(nseg, np.int32)
+            fs.foldseg([ctx.array(x)], n, ctx.array(offs), out)
+            assert np.array_equal(out.get(), (sums + 5).astype(np.int32)), name
+            pair = ctx.empty_tuple(nseg, [np.int64, np.int32])
+            fp.foldseg([ctx.array(x)], n, ctx.array(offs), pair)
+            got_sum, got_count = pair.get()
+            assert np.array_equal(got_sum, sums) and np.array_equal(got_count, lens.astype(np.int32)), name
+            u = rng.integers(0, 2**32, n, dtype=np.uint64).astype(np.uint32)
+
+            def chain(seg, right_seed=None):
+                vals = [int(v) for v in seg] + ([right_seed] if right_seed is not None else [])
+                acc = vals[0]
+                for v in vals[1:]:
+                    acc = pyref.affine16(acc, v)
+                return acc
+            picks = sorted(set(list(range(0, nseg, max(1, nseg // 25))) + list(longs) + [k + 1 for k in longs if k + 1 < nseg]))
+            g1, gr = ctx.empty(nseg, np.uint32), ctx.empty(nseg, np.uint32)
+            du, do = ctx.array(u), ctx.array(offs)
+            f1.foldseg([du], n, do, g1)
+            fr.foldseg([du], n, do, gr)
+            got1, gotr = g1.get(), gr.get()
+            for s_ in picks:
+                if lens[s_] > 0:
+                    assert int(got1[s_]) == chain(u[offs[s_]:offs[s_ + 1]]), (name, "fold1Seg", s_, int(lens[s_]))
+                assert int(gotr[s_]) == chain(u[offs[s_]:offs[s_ + 1]], 0x00030005), (name, "foldSeg right", s_, int(lens[s_]))
+        for sk_ in (fs, f1, fr, fp):
+            sk_.destroy()
+    run_all("(built without the table)")
+    tuned("foldseg.giants=1")
+    run_all("")
+
+
 def test_permute_of_sorted_and_clustered_keys(A, ctx):
     """runs of consecutive elements with one target: the kernels that update under a lock combine each run in its wave
     first (any combining function, floating-point addition on few targets, tuples); integer-valued sources, so every
