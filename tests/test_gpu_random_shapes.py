@@ -245,6 +245,8 @@ __device__ __forceinline__ Word32 affine16(Word32 x, Word32 y) {
                           seed="0x00030005u", preamble=aff, flags=A.FLAG_FOLD_RIGHT)
         fp = ctx.skeleton(A.SKEL_FOLDSEG, "Int64, Int32", env=[(1, "Int32")], out_rank=1, get="acc_elt{(Int64)arrIn0_0[ix], 1}",
                           combine="acc_elt{x.a1 + y.a1, x.a0 + y.a0}", seed="acc_elt{0, 0}")
+        f1r = ctx.skeleton(A.SKEL_FOLD1SEG, "Word32", env=[(1, "Word32")], out_rank=1, get="arrIn0_0[ix]", combine="affine16(x, y)",
+                           preamble=aff, flags=A.FLAG_FOLD_RIGHT)
         for name, nseg, mean, longs in cases:
             lens = rng.poisson(mean, nseg).astype(np.int64) if mean else np.zeros(nseg, np.int64)
             for at, ln in longs.items():
@@ -271,16 +273,18 @@ __device__ __forceinline__ Word32 affine16(Word32 x, Word32 y) {
                     acc = pyref.affine16(acc, v)
                 return acc
             picks = sorted(set(list(range(0, nseg, max(1, nseg // 25))) + list(longs) + [k + 1 for k in longs if k + 1 < nseg]))
-            g1, gr = ctx.empty(nseg, np.uint32), ctx.empty(nseg, np.uint32)
+            g1, gr, g1r = ctx.empty(nseg, np.uint32), ctx.empty(nseg, np.uint32), ctx.empty(nseg, np.uint32)
             du, do = ctx.array(u), ctx.array(offs)
             f1.foldseg([du], n, do, g1)
             fr.foldseg([du], n, do, gr)
-            got1, gotr = g1.get(), gr.get()
+            f1r.foldseg([du], n, do, g1r)
+            got1, gotr, got1r = g1.get(), gr.get(), g1r.get()
             for s_ in picks:
                 if lens[s_] > 0:
                     assert int(got1[s_]) == chain(u[offs[s_]:offs[s_ + 1]]), (name, "fold1Seg", s_, int(lens[s_]))
+                    assert int(got1r[s_]) == chain(u[offs[s_]:offs[s_ + 1]]), (name, "fold1Seg right", s_, int(lens[s_]))
                 assert int(gotr[s_]) == chain(u[offs[s_]:offs[s_ + 1]], 0x00030005), (name, "foldSeg right", s_, int(lens[s_]))
-        for sk_ in (fs, f1, fr, fp):
+        for sk_ in (fs, f1, fr, fp, f1r):
             sk_.destroy()
     run_all("(built without the table)")
     tuned("foldseg.giants=1")
