@@ -27,6 +27,7 @@ skeleton hot path, in miniature:
 Everything runs on the GPU through the C ABI; there is no other execution path.
 """
 import collections
+import ctypes as C
 import numbers
 import re
 import threading
@@ -418,6 +419,63 @@ def _context(context, *operands):
     return found or Context.default()
 
 
+class _ResultPool(object):
+    """Host memory for the results that `run` hands out, page-locked and used again.  A result of 256 MB in a new
+    array costs 4 ms before a byte has arrived (the kernel clears every page when it is first touched) and comes
+    through the library's staging buffers; into page-locked memory the device writes directly, at the link's rate,
+    and a buffer whose array the program has dropped has its pages already.  Page-locking is dear (tens of ms for
+    such a buffer), so a size is served from here from the second time it is asked for -- the program that calls a
+    `run1` function over and over -- and the pool never holds more than `limit` bytes, handed out or not; everything
+    else gets an ordinary array.  A buffer comes back when the last array (or view) on it is collected."""
+    GRAIN = 1 << 20
+
+    def __init__(self, ctx, limit):
+        self.ctx, self.limit, self.held, self.closed = ctx, limit, 0, False
+        self.spare, self.asked = {}, {}
+        self.lock = threading.Lock()       # (collection may happen on any thread, at any time)
+
+    def array(self, shape, dtype):
+        dtype = np.dtype(dtype)
+        size = int(np.prod(shape, dtype=np.int64))
+        nbytes = size * dtype.itemsize
+        if nbytes < self.GRAIN or self.closed:
+            return None
+        room = -(-nbytes // self.GRAIN) * self.GRAIN
+        with self.lock:
+            spare = self.spare.get(room)
+            if spare:
+                addr = spare.pop()
+            else:
+                self.asked[room] = self.asked.get(room, 0) + 1
+                if self.asked[room] < 2 or self.held + room > self.limit:
+                    return None
+                p = C.c_void_p()
+                if A.lib().acc_host_alloc(self.ctx.handle, room, C.byref(p)) != 0 or not p.value:
+                    return None
+                addr = p.value
+                self.held += room
+        buf = (C.c_ubyte * nbytes).from_address(addr)
+        weakref.finalize(buf, self._back, room, addr).atexit = False
+        return np.frombuffer(buf, dtype=dtype, count=size).reshape(shape)
+
+    def _back(self, room, addr):
+        with self.lock:
+            if not self.closed:
+                self.spare.setdefault(room, []).append(addr)
+                return
+        A.lib().acc_host_free(None, C.c_void_p(addr))      # its context has gone: the memory is the process's
+
+    def trim(self, close=False):
+        """give the buffers that nobody holds back to the system (and, closing, take no more back)"""
+        with self.lock:
+            addrs = [(room, a) for room, lst in self.spare.items() for a in lst]
+            self.spare = {}
+            self.held -= sum(room for room, _ in addrs)
+            self.closed = self.closed or close
+        for _, a in addrs:
+            A.lib().acc_host_free(self.ctx.handle, C.c_void_p(a))
+
+
 class _Resident(object):
     """A manifest array under the context's memory table: host storage (the array `use`d, or the place a result is
     written back to when the device is full) and the table entry keyed by it.  The device address is only known
@@ -441,7 +499,7 @@ class _Resident(object):
             A.check(A.lib().acc_event_sync(self.cx.ctx.handle, self.ready))
         d = self.cx.table.acquire(self.host)
         try:
-            return d.get()
+            return d.get(self.cx.results.array(self.shape, self.dtype))
         finally:
             self.cx.table.release(self.host)
 
@@ -522,9 +580,10 @@ class Context(object):
     (Execute.hs:104-105,183-184), so independent subcomputations overlap and the host never waits before `run`."""
     _default = None
 
-    def __init__(self, device=0, budget_bytes=0):
+    def __init__(self, device=0, budget_bytes=0, result_pool_bytes=1 << 30):
         self.ctx = A.Context(device)
         self.table = A.MemTable(self.ctx, budget_bytes)
+        self.results = _ResultPool(self.ctx, result_pool_bytes)   # page-locked host memory for results, used again
         self.live = {}
         self.skeletons = {}
         self.streams, self.turn, self.events = [], 0, []
@@ -1299,9 +1358,10 @@ def run1AsyncWith(context, f):
     return run1Async(f, context)
 
 
-def create(device=0, budget_bytes=0):
-    """a new execution context on the given device (Context.hs:73-84)"""
-    return Context(device, budget_bytes)
+def create(device=0, budget_bytes=0, result_pool_bytes=1 << 30):
+    """a new execution context on the given device (Context.hs:73-84); `result_pool_bytes`: how much page-locked host
+    memory the context may keep for the results it hands out (0: none, every result in an ordinary array)"""
+    return Context(device, budget_bytes, result_pool_bytes)
 
 
 def destroy(context):
@@ -1316,6 +1376,7 @@ def destroy(context):
             context.guard = None
         context.streams, context.events = [], []
         context.table.destroy()
+        context.results.trim(close=True)
         context.ctx.close()
     if Context._default is context:
         Context._default = None
@@ -1340,6 +1401,7 @@ def performGC(context=None):
     cx = context or Context.default()
     with cx.lock:
         cx.table.reclaim()
+    cx.results.trim()
 
 
 def performGCWith(context):

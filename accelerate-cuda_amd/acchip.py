@@ -128,6 +128,8 @@ def lib():
         L.acc_launch_grid.argtypes = [C.c_int64] * 4
         L.acc_malloc.argtypes = [C.c_void_p, C.c_size_t, C.POINTER(C.c_uint64)]
         L.acc_free.argtypes = [C.c_void_p, C.c_uint64]
+        L.acc_host_alloc.argtypes = [C.c_void_p, C.c_size_t, C.POINTER(C.c_void_p)]
+        L.acc_host_free.argtypes = [C.c_void_p, C.c_void_p]
         L.acc_memcpy_h2d.argtypes = [C.c_void_p, C.c_uint64, C.c_void_p, C.c_size_t]
         L.acc_memcpy_d2h.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_size_t]
         L.acc_memcpy_d2d.argtypes = [C.c_void_p, C.c_uint64, C.c_uint64, C.c_size_t]

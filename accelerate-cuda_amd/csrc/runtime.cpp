@@ -526,8 +526,9 @@ int acc_host_alloc(acc_context ctx, size_t bytes, void **out)
 int acc_host_free(acc_context ctx, void *p)
 {
   if (!p) return ACC_OK;
-  if (!ctx) return fail(ACC_ERR_INVALID, "acc_host_free: NULL context");
-  ACC_TRY(ctx->make_current());
+  // (page-locked memory belongs to the process, not to a device: a buffer may outlive the context it was asked
+  // from, and is then given back with no context)
+  if (ctx) ACC_TRY(ctx->make_current());
   ACC_HIP_TRY(hipHostFree(p));
   return ACC_OK;
 }

@@ -135,7 +135,8 @@ int acc_malloc(acc_context ctx, size_t bytes, acc_devptr *out);
 int acc_free(acc_context ctx, acc_devptr p);
 int acc_mem_info(acc_context ctx, size_t *free_bytes, size_t *total_bytes);
 
-/* pinned host staging buffers for asynchronous transfers */
+/* pinned host staging buffers for asynchronous transfers (the memory is the process's: it may be given back after
+ * its context has been destroyed, with a NULL context) */
 int acc_host_alloc(acc_context ctx, size_t bytes, void **out);
 int acc_host_free(acc_context ctx, void *p);
 

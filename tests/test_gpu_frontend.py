@@ -741,3 +741,37 @@ def test_threads_building_computations_in_one_context(acc):
         assert not errors, errors
     finally:
         acc.destroy(cx)
+
+
+def test_results_of_a_repeated_call_come_in_page_locked_memory_that_is_used_again(acc):
+    """`run` hands large results out in host memory that the device writes directly and that is used again when the
+    program has dropped the array: not the first time a size is asked for, never beyond the pool's limit, and a buffer
+    stays away from the pool for as long as any view of its array lives -- or its context does not."""
+    rng = np.random.default_rng(12)
+    cx = acc.create(0, result_pool_bytes=5 << 20)
+    n = (1 << 19) + 3                                     # 2 MB and a little: a buffer of 3 MB
+    inc = acc.run1(lambda a: acc.map(lambda v: v + acc.constant(1, "Int32"), a), cx)
+    x = rng.integers(0, 1000, n).astype(np.int32)
+    r1 = inc(x.copy())
+    assert np.array_equal(r1, x + 1) and cx.results.held == 0        # an ordinary array the first time
+    r2 = inc(x.copy())
+    assert np.array_equal(r2, x + 1) and cx.results.held == 3 << 20
+    where = r2.ctypes.data
+    tail = r2[-5:]                                        # a view keeps the buffer out of the pool
+    del r2
+    r3 = inc(x.copy())
+    assert r3.ctypes.data != where and cx.results.held == 3 << 20    # the limit: an ordinary array again
+    assert np.array_equal(tail, x[-5:] + 1)
+    del tail
+    r4 = inc(x.copy())
+    assert r4.ctypes.data == where and np.array_equal(r4, x + 1) and r4.flags.writeable
+    r4 += 1                                               # the array is the program's to change
+    assert np.array_equal(r4, x + 2)
+    small = acc.run(acc.map(lambda v: v + acc.constant(1, "Int32"), acc.use(x[:100].copy(), cx)), cx)
+    small = acc.run(acc.map(lambda v: v + acc.constant(1, "Int32"), acc.use(x[:100].copy(), cx)), cx)
+    assert np.array_equal(small, x[:100] + 1) and cx.results.held == 3 << 20      # small results: ordinary arrays
+    acc.performGC(cx)
+    assert cx.results.held == 3 << 20                     # r4 still holds its buffer
+    acc.destroy(cx)
+    assert np.array_equal(r4, x + 2)                      # and keeps it when the context has gone
+    del r4                                                # (given back to the system, not to the pool)
