@@ -112,7 +112,7 @@ static_assert(ACC_CHUNK % (ACC_BLOCK * ACC_VEC) == 0, "chunk must be a whole num
 #define ACC_GIANT_HEAD  8                                /* 64-bit words in front of the jobs */
 #define ACC_GIANT_LINES 16                               /* ticket counters a job, each for a run of its pieces */
 #define ACC_GIANT_SPREAD 32                              /* words between two counters: additions to one cache line queue like additions to one word */
-#define ACC_GIANT_JOB   (8 + ACC_GIANT_LINES * ACC_GIANT_SPREAD)           /* 64-bit words a job: tag, segment, first, end, lines that have run out, 3 unused, the counters */
+#define ACC_GIANT_JOB   (8 + ACC_GIANT_LINES * ACC_GIANT_SPREAD)           /* 64-bit words a job: tag; the low halves of segment, first, end; lines that have run out; the high halves; the counters */
 #else
 #define ACC_GIANT_PARAMS
 #endif
@@ -146,14 +146,19 @@ ACC_DEV int acc_giant_enter(unsigned long long *jobs, const unsigned int epoch, 
     if (__hip_atomic_compare_exchange_strong(jobs, &h, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) break;
   }
   unsigned long long *j = jobs + ACC_GIANT_HEAD + (Int64)at * ACC_GIANT_JOB;
-  __hip_atomic_store(j + 1, (unsigned long long)seg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __hip_atomic_store(j + 2, (unsigned long long)a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __hip_atomic_store(j + 3, (unsigned long long)b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  /* (words whose upper half may be anything but zero carry the launch's tag there, like every word of this memory
+   * that others read by its tag: an offset beyond 2^32 left as it is would read as a tag of some later launch) */
+  const unsigned long long tag = (unsigned long long)epoch << 32;
+  const unsigned long long what[3] = {(unsigned long long)seg, (unsigned long long)a, (unsigned long long)b};
+#pragma unroll
+  for (int k = 0; k < 3; ++k) {
+    __hip_atomic_store(j + 1 + k, tag | (unsigned int)what[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(j + 5 + k, tag | (unsigned int)(what[k] >> 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
   __hip_atomic_store(j + 4, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   for (int k = 0; k < ACC_GIANT_LINES; ++k) __hip_atomic_store(j + 8 + k * ACC_GIANT_SPREAD, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      /* the job is whole before its tag says that it is there */
-  __hip_atomic_store(j, (unsigned long long)epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      /* and the tag is there before the owner itself comes to look */
+  /* (nobody looks at a job before this launch has ended: no order among these stores is needed) */
+  __hip_atomic_store(j, tag | 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   return (int)at;
 }
 
@@ -781,8 +786,9 @@ ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _sweep)(ACC_ENV_PARAMS
       __syncthreads();
       if (tid < 8 + ACC_GIANT_LINES) s_job[tid] = __hip_atomic_load(job + (tid < 8 ? tid : 8 + (tid - 8) * ACC_GIANT_SPREAD), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __syncthreads();
-      if ((unsigned int)s_job[0] != acc_epoch) continue;            /* (entered and not filled in: not after the launch that enters them has ended) */
-      const Int64 g_seg = (Int64)s_job[1], g_a = (Int64)s_job[2], g_b = (Int64)s_job[3];
+      if ((unsigned int)(s_job[0] >> 32) != acc_epoch) continue;            /* (not a job of this launch: cannot be, below the head word's count) */
+      auto whole_of = [&](const int k) -> Int64 { return (Int64)(((unsigned long long)(unsigned int)s_job[5 + k] << 32) | (unsigned int)s_job[1 + k]); };
+      const Int64 g_seg = whole_of(0), g_a = whole_of(1), g_b = whole_of(2);
       const Int64 p_first = g_a / ACC_GIANT_PIECE, p_count = (g_b - 1) / ACC_GIANT_PIECE - p_first + 1;
       /* Tickets are drawn from ACC_GIANT_LINES counters, each for a run of `p_line` consecutive pieces, and a
        * workgroup starts at the counter its number names: additions to ONE word are performed one after the other,
