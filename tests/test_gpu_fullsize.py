@@ -171,7 +171,7 @@ def test_config5_smvm_2_20_rows(A, ctx, wl, orc):
 
 
 def test_more_than_2_31_elements(A, ctx):
-    """indices are 64-bit throughout: map, fold, scan and permute over 2^31 + 1 000 003 bytes"""
+    """indices are 64-bit throughout: map, fold, scan, permute and segmented fold over 2^31 + 1 000 003 bytes"""
     n = (1 << 31) + 1000003
     W8 = (1, "Word8")
     say("beyond 2^31 elements, n =", n)
@@ -203,6 +203,24 @@ def test_more_than_2_31_elements(A, ctx):
     h = ctx.empty(256, np.int64)
     p.permute([dx], n, ctx.array(np.zeros(256, np.int64)), h)
     assert np.array_equal(h.get(), np.bincount(x, minlength=256).astype(np.int64))
+    say("foldSeg, 64-bit offsets")
+    rng = np.random.default_rng(31)
+    lens = rng.integers(0, 129, 1 << 25).astype(np.int64)           # 64 elements a segment on average
+    lens[12345] = 300000                                            # and one that the workgroup folds together
+    offs = np.concatenate([[0], np.cumsum(lens)])
+    offs = offs[offs <= n]
+    nseg = offs.size - 1
+    assert offs[-1] > (1 << 31)
+    want = np.add.reduceat(x[:offs[-1]], offs[:-1].clip(max=offs[-1] - 1), dtype=np.int64)
+    want[offs[1:] == offs[:-1]] = 0                                 # (reduceat gives an empty segment its neighbour's first element)
+    doffs = ctx.array(offs)
+    for knobs in ("", "foldseg.giants=1"):
+        with A.tuning(knobs, ctx):
+            fsg = ctx.skeleton(A.SKEL_FOLDSEG, "Int32", env=[W8], out_rank=1, get="(Int32)arrIn0_0[ix]", combine="x + y", seed="3", seg_type="Int64")
+        sums = ctx.empty(nseg, np.int32)
+        fsg.foldseg([dx], int(offs[-1]), doffs, sums)
+        assert np.array_equal(sums.get(), (want + 3).astype(np.int32)), knobs
+        fsg.destroy()
 
 
 def test_stencil_over_more_than_2_31_elements(A, ctx):
