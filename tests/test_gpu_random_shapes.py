@@ -289,6 +289,30 @@ __device__ __forceinline__ Word32 affine16(Word32 x, Word32 y) {
     run_all("(built without the table)")
     tuned("foldseg.giants=1")
     run_all("")
+    # the same under a loop's guard: both launches look at it, so an iteration past the loop's end writes nothing
+    say("segments handed over: under a guard")
+    fg = ctx.skeleton(A.SKEL_FOLDSEG, "Int32", env=[(1, "Int32")], out_rank=1, get="arrIn0_0[ix]", combine="x + y", seed="5", flags=A.FLAG_GUARDED)
+    lens = rng.poisson(3, 3000).astype(np.int64)
+    lens[1500] = 5 * G
+    offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    n = int(offs[-1])
+    x = rng.integers(-9, 9, n).astype(np.int32)
+    c = np.concatenate([[0], np.cumsum(x.astype(np.int64))])
+    want = (c[offs[1:]] - c[offs[:-1]] + 5).astype(np.int32)
+    st, guard = ctx.stream(), A.Guard(ctx)
+    dx, do = ctx.array(x), ctx.array(offs)
+    first, second = ctx.array(np.full(3000, -1, np.int32)), ctx.array(np.full(3000, -1, np.int32))
+    guard.attach(st)
+    guard.reset(st)
+    fg.foldseg([dx], n, do, first, stream=st)
+    guard.latch(ctx.empty((), np.uint8).set(np.zeros(1, np.uint8)), st)      # the predicate says no: the loop has ended
+    fg.foldseg([dx], n, do, second, stream=st)
+    alive, count = guard.read(st)
+    assert not alive and count == 0
+    assert np.array_equal(first.get(), want) and np.all(second.get() == -1)
+    guard.detach(st)
+    guard.destroy()
+    fg.destroy()
 
 
 def test_permute_of_sorted_and_clustered_keys(A, ctx):
