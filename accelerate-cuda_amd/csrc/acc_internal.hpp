@@ -71,7 +71,7 @@ void set_default_tuning(TuningPtr t);
   X(foldseg_long_from, "foldseg.long_from", 8)                                                                         \
   X(foldseg_max_split, "foldseg.max_split", 4096)                                                                      \
   X(foldseg_oversub, "foldseg.oversub", 1 << 20)                                                                       \
-  X(foldseg_giants, "foldseg.giants", 0)                                                                               \
+  X(foldseg_giants, "foldseg.giants", 2)                                                                               \
   X(foldseg_giant_chunks, "foldseg.giant_chunks", 4)                                                                   \
   X(foldseg_sweep_per_cu, "foldseg.sweep_per_cu", 4)                                                                   \
   X(foldseg_row_team_below, "foldseg.row_team_below", 1024)                                                            \
@@ -200,6 +200,10 @@ struct ScratchRef {
 // Words of a context's status block (pinned host memory that kernels write, the host reads at synchronisation
 // points): non-zero = a kernel's bounded wait ran out since the block was last read.
 enum StatusWord { STATUS_SCAN_LOOKBACK = 0, STATUS_FOLD_COLLECT = 1, STATUS_PERMUTE_LOCK = 2, STATUS_WORDS = 16 };
+// Behind them, in the same block: words that say something else than "a wait ran out" -- a kernel of a segmented fold
+// met a very long segment (execute.cpp, launch_segmented).  An instance takes the next word in turn; two instances
+// that share one may each take the other's hint for its own, which costs them a variant they did not need.
+enum { HINT_WORDS = 1024 };
 
 // big single-pass scans on different streams of one device are kept from overlapping (runtime.cpp)
 // device-to-device copy of `bytes` bytes that does nothing when the guard word at `guard` is zero (guard.hip)
@@ -240,6 +244,7 @@ struct acc_context_s {
 
   // kernels report here that a bounded wait ran out (see StatusWord); NULL if the block could not be set up
   volatile uint32_t *status_host = nullptr;
+  std::atomic<unsigned> next_hint{0};
   uint64_t status_dev = 0;
 
   // Streams and events that were given back while nothing was pending on them wait here for the next request

@@ -88,12 +88,14 @@ static_assert(ACC_CHUNK % (ACC_BLOCK * ACC_VEC) == 0, "chunk must be a whole num
  * segment stays with its owner as if there were no table.  The table and the values carry the launch's tag
  * (nothing is cleared between launches).  Index order, another association than the sequential fold's: as for
  * every long segment.
- *   Off unless the instance is built with `foldseg.giants=1`.  The code in this kernel lies behind the test for a
- * stretch that the workgroup folds together, and yet, with it compiled in and no such segment in the source, 2^25
- * elements in segments of 2 / 8 / 32 took 101 / 36 / 29 us instead of 89 / 33 / 27 and the sparse matrix-vector
- * product 193 instead of 190; the second launch costs a source without such segments 2-3 us more.  (A test of
- * every block of segments ahead of its first chunk, by way of a barrier that carries the lanes' verdicts, made the
- * segments of two elements 117 us: the block's first loads then wait for the lanes' offsets.)                   */
+ *   Variants 4 to 7 of an instance are built like this, and the host takes them once a look at the segment lengths
+ * (<entry>_probe, at the end of this file) has found such a segment.  Not every instance, not from the start: the code
+ * in this kernel lies behind the test for a stretch that the workgroup folds together, and yet, with it compiled in
+ * and no such segment in the source, 2^25 elements in segments of 2 / 8 / 32 took 101 / 36 / 29 us instead of
+ * 89 / 33 / 27 and the sparse matrix-vector product 193 instead of 190; the second launch costs a source without
+ * such segments 2-3 us more.  (A test of every block of segments ahead of its first chunk, by way of a barrier that
+ * carries the lanes' verdicts, made the segments of two elements 117 us: the block's first loads then wait for the
+ * lanes' offsets.)                                                                                               */
 #ifndef ACC_GIANTS
 #define ACC_GIANTS 0
 #endif
@@ -101,13 +103,13 @@ static_assert(ACC_CHUNK % (ACC_BLOCK * ACC_VEC) == 0, "chunk must be a whole num
 #undef ACC_GIANTS
 #define ACC_GIANTS 0                                     /* (segments of one length; rows with segments of their own) */
 #endif
-#if ACC_GIANTS
-#define ACC_GIANT_PARAMS , unsigned long long *__restrict__ acc_jobs, const unsigned int acc_epoch, unsigned int *acc_status
 #ifndef ACC_GIANT_CHUNKS
 #define ACC_GIANT_CHUNKS 4
 #endif
 #define ACC_GIANT_PIECE ((Int64)ACC_GIANT_CHUNKS * ACC_CHUNK)
 #define ACC_GIANT_FROM  (2 * ACC_GIANT_PIECE)
+#if ACC_GIANTS
+#define ACC_GIANT_PARAMS , unsigned long long *__restrict__ acc_jobs, const unsigned int acc_epoch, unsigned int *acc_status
 #define ACC_GIANT_JOBS  32                               /* the host sizes the scratch block by these three */
 #define ACC_GIANT_HEAD  8                                /* 64-bit words in front of the jobs */
 #define ACC_GIANT_LINES 16                               /* ticket counters a job, each for a run of its pieces */
@@ -416,7 +418,6 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
 #else
   blocks_of_segments(acc_bool<ACC_PAD_ON != 0>());
 #endif
-
 }
 
 #if ACC_SEG_UNIFORM
@@ -699,6 +700,24 @@ ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _join)(ACC_ENV_PARAMS
   ACC_SET(arrOut, seg, acc.v);
 #endif
 }
+
+#if !ACC_GIANTS && !ACC_SEG_UNIFORM && !ACC_SEG_OUTER
+/* ---- is there a segment that a build with the table of jobs would hand over? ----
+ * <entry>_probe, which the host launches behind <entry> on an instance's calls number 1, 2, 4, 8 ...: a look at the
+ * segment lengths, and a word of host memory set if one of them is as long as that; the host then has variants 4 to
+ * 7 built and takes them once they are there.  (The question asked inside <entry> -- a comparison a segment and a
+ * store that never happens, wherever they stand -- costs the sparse matrix-vector product 1.1 us of 190.)  The
+ * parameters of <entry>, and the word's address behind them. */
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _probe)(ACC_ENV_PARAMS
+                                      const Int64 shOut_0, ACC_OUT_ARRAY(arrOut),
+                                      ACC_SEG_PARAMS ACC_GUARD_PARAM, unsigned int *acc_hint)
+{
+  (void)shIn_0;
+  for (Int64 s = (Int64)blockIdx.x * ACC_BLOCK + threadIdx.x; s < shOut_0; s += (Int64)gridDim.x * ACC_BLOCK)
+    if ((Int64)arrSeg_0[s + 1] - (Int64)arrSeg_0[s] >= ACC_GIANT_FROM + 2 * ACC_CHUNK) *acc_hint = 1u;
+}
+#endif
 
 #if ACC_GIANTS
 /* ---- the segments that were handed over -------------------------------------

@@ -316,11 +316,43 @@ int launch_segmented(acc_skel_s *s, int v, Args *args, const acc_array *env, con
       ACC_TRY(s->ensure_variant(lv));
     }
     const int64_t grid = acc_launch_grid(nseg, s->spec.block, resident(s, lv), s->knobs.foldseg_oversub);
-    // an instance built with `foldseg.giants=1` takes a table of jobs (skel_foldseg.h, ACC_GIANTS): head, 32 jobs of
-    // 8 words and 16 ticket counters 32 words apart, then values of tagged words -- two for every piece of 4 chunks
-    // the source has, and one a job
-    if (!giants || s->knobs.foldseg_giants == 0) return launch(s, lv, grid, 0, st, args);
-    const int64_t piece = (int64_t)std::max(1, s->knobs.foldseg_giant_chunks) * (int64_t)(lv >= 2 ? s->spec.chunk_long : s->spec.chunk);
+    if (!giants) return launch(s, lv, grid, 0, st, args);      // (rows of an array: the kernels have no such parameters)
+    // Very long segments among short ones (skel_foldseg.h, ACC_GIANTS).  Variants 4 to 7 hand what is left of such a
+    // segment over to a second launch, at a cost to sources that have none; so an instance takes them once a look at
+    // its segment lengths has found such a segment -- a small kernel behind calls number 1, 2, 4, 8 ... of the
+    // instance, which says so in a word of host memory -- and once they are compiled, which happens in the
+    // background meanwhile.  `foldseg.giants`: 2 this, 1 always, 0 never.
+    bool hand_over = s->knobs.foldseg_giants == 1;
+    bool look = false;
+    if (s->knobs.foldseg_giants == 2 && s->hint_slot >= 0) {
+      if (!s->met_giants.load(std::memory_order_relaxed) && s->ctx->status_host[acc::STATUS_WORDS + s->hint_slot] != 0)
+        s->met_giants.store(true, std::memory_order_relaxed);
+      if (s->met_giants.load(std::memory_order_relaxed)) {
+        ACC_TRY(s->start_variant(lv + 4));
+        hand_over = s->variant_compiled(lv + 4);
+      } else {
+        const unsigned call = s->seg_calls.fetch_add(1, std::memory_order_relaxed) + 1;
+        look = (call & (call - 1)) == 0;
+      }
+    }
+    if (!hand_over) {
+      int rc = launch(s, lv, grid, 0, st, args);
+      if (rc == ACC_OK && look) {
+        (void)args->data();                                   // (a guard's address, if there is one, comes before the word's)
+        args->ptr(s->ctx->status_dev + (uint64_t)(acc::STATUS_WORDS + s->hint_slot) * sizeof(uint32_t));
+        const int64_t lookers = std::min<int64_t>((nseg + s->spec.block - 1) / s->spec.block, (int64_t)s->ctx->props.multiProcessorCount * 8);
+        hipError_t e = launch_kernel(s->variants[lv].fn_sweep, static_cast<unsigned>(lookers), 1, 1, static_cast<unsigned>(s->spec.block), 1, 1, 0, st,
+                                     args->data_without_guard(), nullptr);
+        if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(segmented fold, probe)");
+      }
+      return rc;
+    }
+    lv += 4;
+    ACC_TRY(s->ensure_variant(lv));
+    const int64_t grid4 = acc_launch_grid(nseg, s->spec.block, resident(s, lv), s->knobs.foldseg_oversub);
+    // the table of jobs: head, 32 jobs of 8 words and 16 ticket counters 32 words apart, then values of tagged words --
+    // two for every piece of 4 chunks the source has, and one a job
+    const int64_t piece = (int64_t)std::max(1, s->knobs.foldseg_giant_chunks) * (int64_t)((lv & 2) ? s->spec.chunk_long : s->spec.chunk);
     const size_t words_a_value = ((size_t)s->spec.elt_size + 3) / 4;
     const size_t bytes = (8 + 32 * (8 + 16 * 32) + (2 * (size_t)(n / piece + 2) + 32) * words_a_value) * 8;
     acc::ScratchRef jobs;
@@ -328,7 +360,7 @@ int launch_segmented(acc_skel_s *s, int v, Args *args, const acc_array *env, con
     args->ptr(reinterpret_cast<uint64_t>(jobs.ptr));
     args->u32(jobs.epoch);
     args->ptr(s->ctx->status_dev);
-    int rc = launch(s, lv, grid, 0, st, args);
+    int rc = launch(s, lv, grid4, 0, st, args);
     if (rc == ACC_OK) {
       // the second launch, which takes what the first has entered in the table: as many workgroups as the device holds
       const int64_t sweepers = (int64_t)s->ctx->props.multiProcessorCount * std::max(1, std::min(s->knobs.foldseg_sweep_per_cu, 2048 / s->spec.block));

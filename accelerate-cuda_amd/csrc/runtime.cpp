@@ -370,9 +370,9 @@ int acc_context_create(int device, acc_context *out)
   {
     // the status block: host memory the device can write (only ever written when a kernel's bounded wait runs out)
     void *hp = nullptr, *dp = nullptr;
-    if (hipHostMalloc(&hp, acc::STATUS_WORDS * sizeof(uint32_t), hipHostMallocMapped) == hipSuccess &&
+    if (hipHostMalloc(&hp, (acc::STATUS_WORDS + acc::HINT_WORDS) * sizeof(uint32_t), hipHostMallocMapped) == hipSuccess &&
         hipHostGetDevicePointer(&dp, hp, 0) == hipSuccess) {
-      std::memset(hp, 0, acc::STATUS_WORDS * sizeof(uint32_t));
+      std::memset(hp, 0, (acc::STATUS_WORDS + acc::HINT_WORDS) * sizeof(uint32_t));
       ctx->status_host = static_cast<volatile uint32_t *>(hp);
       ctx->status_dev = reinterpret_cast<uint64_t>(dp);
     } else {

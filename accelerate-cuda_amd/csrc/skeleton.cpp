@@ -411,7 +411,7 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
   }
   o << "#define ACC_ENTRY " << *entry << "\n";
   o << "#define ACC_NT_STORE " << tune("nt_store", 1) << "\n";
-  if (tune("foldseg.giants", 0) != 0) o << "#define ACC_GIANTS 1\n";
+  if (sp.foldseg_giants) o << "#define ACC_GIANTS 1\n";
   if (tuned("foldseg.giant_chunks")) o << "#define ACC_GIANT_CHUNKS " << std::max(1, tune("foldseg.giant_chunks", 4)) << "\n";
   if (tuned("stream.policy")) o << "#define ACC_STREAM_POLICY " << tune("stream.policy", 1) << "\n";
   if (sp.guarded) o << "#define ACC_GUARDED 1\n";
@@ -783,8 +783,10 @@ SkelSpec spec_of_variant(const SkelSpec &base, int v)
     if (v >= 4 && v < 6) spec.permute_windows = true;
     if (v >= 6) spec.permute_narrow = true;
   }
-  // a segmented fold's variants 2 and 3: a longer staged chunk, for segments of 8 elements or more on average
-  if (spec.kind != ACC_SKEL_PERMUTE && v >= 2 && spec.chunk_long > 0) spec.chunk = spec.chunk_long;
+  // a segmented fold's variants 2 and 3 (6 and 7): a longer staged chunk, for segments of 8 elements or more on
+  // average; 4 to 7: what is left of a very long segment is handed over to a second launch
+  if (spec.kind != ACC_SKEL_PERMUTE && (v & 2) && spec.chunk_long > 0) spec.chunk = spec.chunk_long;
+  if ((spec.kind == ACC_SKEL_FOLDSEG || spec.kind == ACC_SKEL_FOLD1SEG) && spec.out_rank <= 1 && v >= 4) spec.foldseg_giants = true;
   // a stencil's variants 2 and 3, 4 and 5: half and a quarter of the columns a lane, for arrays narrower than half or a
   // quarter of a strip, whose lanes would otherwise mostly lie outside the array
   if ((spec.kind == ACC_SKEL_STENCIL || spec.kind == ACC_SKEL_STENCIL2) && v >= 2 && !spec.stencil_nd) {
@@ -825,6 +827,19 @@ int acc_skel_s::start_variant(int v)
   ACC_TRY(make_job(this, v, &job));
   if (acc::compile_submit(job)) var.job = job;      // else: compiled by the thread that first needs it
   return ACC_OK;
+}
+
+bool acc_skel_s::variant_compiled(int v)
+{
+  std::shared_ptr<acc::CompileJob> job;
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    if (variants[v].ready) return true;
+    job = variants[v].job;
+  }
+  if (!job) return false;
+  std::lock_guard<std::mutex> lock(job->mu);
+  return job->done;
 }
 
 int acc_skel_s::ensure_variant(int v)
@@ -876,8 +891,9 @@ int acc_skel_s::ensure_variant(int v)
       return acc::fail_hip(e, ("hipModuleGetFunction(" + third + ")").c_str());
     }
   }
-  if ((spec.kind == ACC_SKEL_FOLDSEG || spec.kind == ACC_SKEL_FOLD1SEG) && spec.out_rank <= 1 && knobs.foldseg_giants != 0) {
-    const std::string sweep = entry_name + "_sweep";
+  if ((spec.kind == ACC_SKEL_FOLDSEG || spec.kind == ACC_SKEL_FOLD1SEG) && spec.out_rank <= 1) {
+    // variants 4 to 7: the launch that takes what was handed over; 0 to 3: the look at the segment lengths
+    const std::string sweep = entry_name + (spec.foldseg_giants ? "_sweep" : "_probe");
     e = hipModuleGetFunction(&var.fn_sweep, var.module, sweep.c_str());
     if (e != hipSuccess) {
       (void)hipModuleUnload(var.module);
@@ -922,6 +938,7 @@ int acc_skel_s::ensure_variant(int v)
 static int variant_count(const acc::SkelSpec &sp)
 {
   const bool stencil = sp.kind == ACC_SKEL_STENCIL || sp.kind == ACC_SKEL_STENCIL2;
+  if ((sp.kind == ACC_SKEL_FOLDSEG || sp.kind == ACC_SKEL_FOLD1SEG) && sp.out_rank <= 1) return 8;
   return sp.kind == ACC_SKEL_PERMUTE ? 8 : (stencil ? (sp.stencil_nd ? 2 : 6) : ((sp.scan_small_rows > 0 || sp.chunk_long > 0) ? 4 : 2));
 }
 
@@ -937,6 +954,10 @@ int acc_skel_create_async(acc_context ctx, const acc_skel_desc *desc, acc_skel *
   s->ctx = ctx;
   s->spec = sp;
   s->knobs.resolve(*sp.tuning);
+  if ((sp.kind == ACC_SKEL_FOLDSEG || sp.kind == ACC_SKEL_FOLD1SEG) && sp.out_rank <= 1 && ctx->status_host) {
+    s->hint_slot = static_cast<int>(ctx->next_hint.fetch_add(1) % acc::HINT_WORDS);
+    ctx->status_host[acc::STATUS_WORDS + s->hint_slot] = 0;
+  }
   const int rc = s->start_variant(0);     // the other variants are built when a call first needs them
   if (rc != ACC_OK) { delete s; return rc; }
   *out = s;

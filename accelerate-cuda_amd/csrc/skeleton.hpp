@@ -52,6 +52,7 @@ struct SkelSpec {
   bool map_tiled = false;               // ACC_FLAG_TILED on a map of rank 2 or more: tiles of 32 x 32 elements, a wave each
   int map_tile_block = 4;               // ... a lane's share of a tile: a block of that many elements either way
   bool guarded = false;                 // ACC_FLAG_GUARDED: every kernel takes the address of a loop's guard word last
+  bool foldseg_giants = false;          // a segmented fold's variants 4-7: very long segments are handed over to a second launch (skel_foldseg.h)
   bool fold_single = true;              // foldAll in one launch (the last workgroup collects), as generated into the kernel
   int scan_rows_fallback = 8;
   int scan_small_rows = 0;              // rows a lane of a scan's small-tile variants (2 and 3); 0: none
@@ -69,7 +70,8 @@ struct Variant {
   hipFunction_t fn_finish = nullptr;   // second kernel: foldAll's _finish, permute's _merge / _join, the segmented fold's _team
   hipFunction_t fn_fill = nullptr;     // third kernel: permute's _fill (identity into the table rows), the segmented fold's _join
   hipFunction_t fn_rows = nullptr;     // fold along the innermost dimension: _rows, a lane per short row
-  hipFunction_t fn_sweep = nullptr;    // a segmented fold built with `foldseg.giants=1`: _sweep, the segments that were handed over
+  hipFunction_t fn_sweep = nullptr;    // a segmented fold's variants 4-7: _sweep, the segments that were handed over;
+                                       // its variants 0-3: _probe, a look at the segment lengths
   int num_regs = 0;
   int static_lds = 0;
   int blocks_per_cu = 1;
@@ -96,8 +98,12 @@ struct acc_skel_s {
                               // table-in-LDS form of a permute whose combination has no atomic instruction;
                               // [4], [5]: for a hinted permute over several LDS windows of targets;
                               // [6], [7]: for integer addition on a table of 16-bit counts in LDS;
-                              // of a segmented fold [2], [3]: a longer staged chunk; of a scan [2], [3]: small tiles;
+                              // of a segmented fold [2], [3]: a longer staged chunk, [4]-[7]: the same four with the table of
+                              // jobs for very long segments; of a scan [2], [3]: small tiles;
                               // of a stencil [2], [3] and [4], [5]: half and a quarter of the columns a lane
+  int hint_slot = -1;         // a segmented fold: its word among the context's hints (its segments were looked at: a very long one)
+  std::atomic<bool> met_giants{false};   // ... and that the word has been seen set
+  std::atomic<unsigned> seg_calls{0};    // ... and how often it has been launched (the look happens on calls 1, 2, 4, 8 ...)
   std::mutex mu;
 
   // variant v compiled, loaded and measured; compiles on the calling thread unless a job for it is under way
@@ -105,6 +111,8 @@ struct acc_skel_s {
   // start variant v's compilation on the worker pool (nothing if it has been started or is ready)
   int start_variant(int v);
   bool variant_ready(int v) { std::lock_guard<std::mutex> lock(mu); return variants[v].ready; }
+  // ... or its compilation has ended, so that ensure_variant would not wait for the compiler
+  bool variant_compiled(int v);
   int ncomp() const { return spec.comp_types.empty() ? 1 : (int)spec.comp_types.size(); }
   int vec() const { int v = 16 / (spec.vec_size > 0 ? spec.vec_size : 1); return v < 1 ? 1 : v; }
   int elements_per_block() const

@@ -756,10 +756,11 @@ def main():
         assert np.array_equal(dst.get(), wl.stencil_image(side, side).T), "transpose mismatch"
         del src, dst
         # segmented sums whose lengths are very unequal: a million segments of 8 elements on average, one of which holds
-        # half of the source (the rows of a power-law graph); the same elements all in segments of 8; and the former
-        # through an instance built with `foldseg.giants=1`, which hands the long segment over to all workgroups
+        # half of the source (the rows of a power-law graph), folded by its workgroup alone (`foldseg.giants=0`) and handed
+        # over to a second launch (`=1`; as the knobs stand an instance goes from the one to the other by itself, once
+        # it has looked at its segment lengths and the other variant is compiled); the same elements all in segments of 8
         nseg, big = 1 << 20, 1 << 23
-        for name, giant, knobs in (("every segment short", 0, ""), ("one segment of 2^23 elements among them", big, ""),
+        for name, giant, knobs in (("every segment short", 0, ""), ("one segment of 2^23 elements among them, foldseg.giants=0", big, "foldseg.giants=0"),
                                    ("one segment of 2^23 elements among them, foldseg.giants=1", big, "foldseg.giants=1")):
             with A.tuning(knobs, ctx):
                 seg_s = ctx.skeleton(A.SKEL_FOLDSEG, "float", env=[F32], get=rd(0), combine="x + y", seed="0.0f")

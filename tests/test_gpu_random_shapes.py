@@ -213,13 +213,13 @@ __device__ __forceinline__ Word32 affine16(Word32 x, Word32 y) {
 
 
 def test_segments_that_are_handed_over(A, ctx, tuned):
-    """instances built with `foldseg.giants=1`: among short segments, segments that go on for eight staged chunks or
+    """the variants of an instance with the table of jobs (`foldseg.giants=1`: always taken): among short segments, segments that go on for eight staged chunks or
     more beyond the chunk in which the workgroup first folds a stretch of them together.  Their owner enters the rest
     in a table of jobs and the workgroups take pieces of it when their own segments are done.  Several in one block of
     256 segments, next to one another, first and last of the array, more of them than the table has room for (the rest
     stay with their owners), the whole array one segment; sums of integers (exact), a non-commutative operator in both
     associations (the order of the pieces and of the owner's own part), pairs (a value of several tagged words), and
-    the same inputs through instances built without the table."""
+    the same inputs through the variants without the table (`foldseg.giants=0`)."""
     rng = np.random.default_rng(88)
     aff = """
 __device__ __forceinline__ Word32 affine16(Word32 x, Word32 y) {
@@ -286,7 +286,8 @@ __device__ __forceinline__ Word32 affine16(Word32 x, Word32 y) {
                 assert int(gotr[s_]) == chain(u[offs[s_]:offs[s_ + 1]], 0x00030005), (name, "foldSeg right", s_, int(lens[s_]))
         for sk_ in (fs, f1, fr, fp, f1r):
             sk_.destroy()
-    run_all("(built without the table)")
+    tuned("foldseg.giants=0")
+    run_all("(without the table)")
     tuned("foldseg.giants=1")
     run_all("")
     # the same under a loop's guard: both launches look at it, so an iteration past the loop's end writes nothing
@@ -313,6 +314,52 @@ __device__ __forceinline__ Word32 affine16(Word32 x, Word32 y) {
     guard.detach(st)
     guard.destroy()
     fg.destroy()
+
+
+def test_an_instance_that_has_met_a_very_long_segment_takes_the_table(A, ctx):
+    """as the knobs stand, an instance looks at its segment lengths behind calls number 1, 2, 4, 8 ... and, when it
+    has found a segment that the variants with the table of jobs would hand over, has them compiled in the background
+    and takes them when they are there: the same results before, while and after, and the launch trace names the
+    second kernel from then on; an instance that sees no such segment never does"""
+    import time
+    rng = np.random.default_rng(89)
+
+    def inputs(longest):
+        lens = rng.poisson(6, 5000).astype(np.int64)
+        lens[1234] = longest
+        offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        x = rng.integers(-9, 9, int(offs[-1])).astype(np.int32)
+        c = np.concatenate([[0], np.cumsum(x.astype(np.int64))])
+        return ctx.array(x), ctx.array(offs), int(offs[-1]), (c[offs[1:]] - c[offs[:-1]] + 7).astype(np.int32)
+
+    def kernels_of_a_call(sk, dx, do, n):
+        out = ctx.empty(5000, np.int32)
+        ctx.trace_start()
+        sk.foldseg([dx], n, do, out)
+        ctx.sync()
+        return ctx.trace_stop()[0], out.get()
+
+    for longest, switches in ((200000, True), (3000, False)):
+        sk = ctx.skeleton(A.SKEL_FOLDSEG, "Int32", env=[(1, "Int32")], out_rank=1, get="arrIn0_0[ix]", combine="x + y", seed="7")
+        dx, do, n, want = inputs(longest)
+        say("segments of up to", longest, "elements: does the instance take the table?")
+        launches, got = kernels_of_a_call(sk, dx, do, n)
+        assert np.array_equal(got, want) and launches == 2          # the fold, and the look at the segment lengths
+        deadline, taken = time.time() + 60, False
+        for call in range(2, 4000):
+            launches, got = kernels_of_a_call(sk, dx, do, n)
+            assert np.array_equal(got, want), call
+            if switches:                                            # (the first look has found the segment: no more of them)
+                taken = taken or launches == 2                      # the fold and the launch that takes what it handed over
+                assert launches == (2 if taken else 1), (call, launches)
+            else:
+                assert launches == (2 if (call & (call - 1)) == 0 else 1), (call, launches)
+            if (taken and call > 100) or (not switches and call > 300) or time.time() > deadline:
+                break
+            if switches and not taken:
+                time.sleep(0.005)                                   # (the compiler is at work meanwhile)
+        assert taken == switches
+        sk.destroy()
 
 
 def test_permute_of_sorted_and_clustered_keys(A, ctx):
