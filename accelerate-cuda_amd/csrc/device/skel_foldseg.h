@@ -167,16 +167,6 @@ ACC_DEV int acc_giant_enter(unsigned long long *jobs, const unsigned int epoch, 
 /* where the value that a job's owner has folded itself goes: behind the two values for every piece of the source */
 ACC_DEV unsigned int acc_giant_edge_slot(const Int64 n, const int job) { return (unsigned int)(2 * (n / ACC_GIANT_PIECE + 2) + job); }
 
-/* one more of the launch's jobs has no ticket left: the word behind the head word, {tag of the launch, such jobs} */
-ACC_DEV void acc_giant_ran_out(unsigned long long *jobs, const unsigned int epoch)
-{
-  unsigned long long h = __hip_atomic_load(jobs + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  for (;;) {
-    const unsigned int at = (unsigned int)(h >> 32) == epoch ? (unsigned int)h : 0u;
-    const unsigned long long want = ((unsigned long long)epoch << 32) | (at + 1u);
-    if (__hip_atomic_compare_exchange_strong(jobs + 1, &h, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) break;
-  }
-}
 #endif
 
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
@@ -738,7 +728,8 @@ ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _sweep)(ACC_ENV_PARAMS
   (void)shOut_0;
   (void)arrSeg_0;
   __shared__ __attribute__((aligned(16))) T s_val[ACC_PAD_SPACE(ACC_CHUNK)];
-  __shared__ unsigned long long s_job[8 + ACC_GIANT_LINES];
+  __shared__ unsigned long long s_jobs[ACC_GIANT_JOBS][8 + ACC_GIANT_LINES], s_tick;
+  __shared__ int s_pick;
   __shared__ acc_opt<T> s_part[ACC_BLOCK / ACC_WAVE];
   auto get = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
   auto f   = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
@@ -764,7 +755,8 @@ ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _sweep)(ACC_ENV_PARAMS
     for (int w = 1; w < ACC_BLOCK / ACC_WAVE; ++w) whole = lf(whole, s_part[w]);
     return whole;
   };
-  /* elements [from, to) of the source folded by the whole workgroup, chunk by chunk in index order (to > from) */
+  /* elements [from, to) of the source folded by the whole workgroup, chunk by chunk in index order (to > from).
+   * (The loads of two or four chunks in flight together make no piece faster: 36-39 us either way.) */
   auto fold_range = [&](const Int64 from, const Int64 to) -> acc_opt<T> {
     constexpr int acc_pad_mask = ACC_PAD_ON ? ~0 : 0;
     acc_opt<T> value = acc_none<T>();
@@ -792,67 +784,75 @@ ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _sweep)(ACC_ENV_PARAMS
   };
   {
     const acc_tagged<T> pieces_of = {acc_jobs + ACC_GIANT_HEAD + ACC_GIANT_JOBS * ACC_GIANT_JOB};
-    if (tid < 2) s_job[tid] = __hip_atomic_load(acc_jobs + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0) s_tick = __hip_atomic_load(acc_jobs, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
-    const unsigned long long head = s_job[0], out = s_job[1];
-    const int entered = (unsigned int)(head >> 32) == acc_epoch ? (int)acc_min<unsigned int>((unsigned int)head, ACC_GIANT_JOBS) : 0;
-    const int ran_out = (unsigned int)(out >> 32) == acc_epoch ? (int)(unsigned int)out : 0;
-    /* as many jobs without a ticket left as there are jobs: nothing to take (most workgroups of a large launch come
-     * here after the last piece has gone, and are spared the look at every job) */
-    const int jobs_in = ran_out >= entered ? 0 : entered;
-    for (int j = 0; j < jobs_in; ++j) {
+    const unsigned long long head = s_tick;          /* {tag of the launch, jobs entered} */
+    const int jobs_in = (unsigned int)(head >> 32) == acc_epoch ? (int)acc_min<unsigned int>((unsigned int)head, ACC_GIANT_JOBS) : 0;
+    /* Tickets are drawn from ACC_GIANT_LINES counters a job, each for a run of `p_line` consecutive pieces: additions
+     * to ONE word are performed one after the other, 0.1 us each, so that a thousand workgroups that ask for a ticket
+     * at the same moment were handed theirs over 100 us.  A line has one ticket more than pieces: whoever draws it
+     * knows that the line has run out, and a counter beyond it says so to everybody who looks.  And a look comes
+     * before every ticket: a counter that has run out is not asked again -- thousands of workgroups that each drew a
+     * ticket only to find the job done kept a launch busy for 200 us. */
+    struct acc_job_shape { Int64 seg, a, b, p_first, p_count, p_line; };
+    auto shape_of = [&](const unsigned long long *sj) -> acc_job_shape {
+      auto whole_of = [&](const int k) -> Int64 { return (Int64)(((unsigned long long)(unsigned int)sj[5 + k] << 32) | (unsigned int)sj[1 + k]); };
+      acc_job_shape g;
+      g.seg = whole_of(0); g.a = whole_of(1); g.b = whole_of(2);
+      g.p_first = g.a / ACC_GIANT_PIECE;
+      g.p_count = (g.b - 1) / ACC_GIANT_PIECE - g.p_first + 1;
+      g.p_line = (g.p_count + ACC_GIANT_LINES - 1) / ACC_GIANT_LINES;
+      return g;
+    };
+    auto line_first = [&](const acc_job_shape &g, const int l) -> Int64 { return acc_min<Int64>((Int64)l * g.p_line, g.p_count); };
+    auto line_count = [&](const acc_job_shape &g, const int l) -> Int64 { return acc_min<Int64>(line_first(g, l) + g.p_line, g.p_count) - line_first(g, l); };
+    /* A round: a look at every job's words, all in one round trip; of the lines that have a ticket left the one
+     * nearest to the job and the line that this workgroup's number names (so that the workgroups begin spread over
+     * all of them); tickets of that line until it has run out.  Then the next round, until a look finds no line.
+     * (Job after job, each looked at when its turn came, thirty segments of 2^18 elements took 240 us: most of a
+     * workgroup's time went into finding out, one round trip a job, that the others had done it already.) */
+    const int j0 = jobs_in > 0 ? (int)((blockIdx.x / ACC_GIANT_LINES) % (unsigned int)jobs_in) : 0, l0 = (int)(blockIdx.x % ACC_GIANT_LINES);
+    for (int round = 0; round < 2 * ACC_GIANT_JOBS * ACC_GIANT_LINES && jobs_in > 0; ++round) {
+      __syncthreads();                                              /* (the round before has read these words) */
+      if (tid == 0) s_pick = 0x7fffffff;
+      for (int i = tid; i < jobs_in * (8 + ACC_GIANT_LINES); i += ACC_BLOCK) {
+        const int jn = i / (8 + ACC_GIANT_LINES), wn = i % (8 + ACC_GIANT_LINES);
+        s_jobs[jn][wn] = __hip_atomic_load(acc_jobs + ACC_GIANT_HEAD + (Int64)jn * ACC_GIANT_JOB + (wn < 8 ? wn : 8 + (wn - 8) * ACC_GIANT_SPREAD),
+                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      __syncthreads();
+      for (int c = tid; c < jobs_in * ACC_GIANT_LINES; c += ACC_BLOCK) {
+        const int jn = c / ACC_GIANT_LINES, l = c % ACC_GIANT_LINES;
+        const acc_job_shape g = shape_of(s_jobs[jn]);
+        if ((unsigned int)(s_jobs[jn][0] >> 32) == acc_epoch && line_count(g, l) > 0 && (Int64)s_jobs[jn][8 + l] <= line_count(g, l))
+          (void)__hip_atomic_fetch_min(&s_pick, ((jn - j0 + jobs_in) % jobs_in) * ACC_GIANT_LINES + (l - l0 + ACC_GIANT_LINES) % ACC_GIANT_LINES,
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
+      __syncthreads();
+      const int pick = s_pick;
+      if (pick == 0x7fffffff) break;                                /* no line of any job has a ticket left */
+      const int j = (j0 + pick / ACC_GIANT_LINES) % jobs_in, line = (l0 + pick % ACC_GIANT_LINES) % ACC_GIANT_LINES;
       unsigned long long *job = acc_jobs + ACC_GIANT_HEAD + (Int64)j * ACC_GIANT_JOB;
-      __syncthreads();
-      if (tid < 8 + ACC_GIANT_LINES) s_job[tid] = __hip_atomic_load(job + (tid < 8 ? tid : 8 + (tid - 8) * ACC_GIANT_SPREAD), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __syncthreads();
-      if ((unsigned int)(s_job[0] >> 32) != acc_epoch) continue;            /* (not a job of this launch: cannot be, below the head word's count) */
-      auto whole_of = [&](const int k) -> Int64 { return (Int64)(((unsigned long long)(unsigned int)s_job[5 + k] << 32) | (unsigned int)s_job[1 + k]); };
-      const Int64 g_seg = whole_of(0), g_a = whole_of(1), g_b = whole_of(2);
-      const Int64 p_first = g_a / ACC_GIANT_PIECE, p_count = (g_b - 1) / ACC_GIANT_PIECE - p_first + 1;
-      /* Tickets are drawn from ACC_GIANT_LINES counters, each for a run of `p_line` consecutive pieces, and a
-       * workgroup starts at the counter its number names: additions to ONE word are performed one after the other,
-       * 0.1 us each, so that the thousand workgroups that end together and ask for a ticket at the same moment were
-       * handed theirs over 100 us.  And a look before a ticket is drawn: a counter that has run out (as the words
-       * just read say) is not asked again -- thousands of workgroups that each drew a ticket only to find the job
-       * done kept a launch busy for 200 us. */
-      const Int64 p_line = (p_count + ACC_GIANT_LINES - 1) / ACC_GIANT_LINES;
-      const Int64 lines_in_use = (p_count + p_line - 1) / p_line;
+      const acc_job_shape g = shape_of(s_jobs[j]);
+      const Int64 g_seg = g.seg, g_a = g.a, g_b = g.b, p_first = g.p_first, p_count = g.p_count;
+      const Int64 lines_in_use = (p_count + g.p_line - 1) / g.p_line;
       /* Where a piece's value goes: two values for every piece of the source.  A handed-over segment is at least two
        * pieces long, so a piece of the source is shared by two of them at most -- one that ends in it and one that
        * begins in it -- and the one that begins there (its piece 0) takes the odd place. */
       auto slot_of = [&](const Int64 piece) -> unsigned int { return (unsigned int)(2 * (p_first + piece) + (piece == 0 ? 1 : 0)); };
-      /* A workgroup goes to the line its number names; when that has run out it looks at the counters again and goes
-       * to the next line that has not, until none is left.  (A line has one ticket more than pieces: whoever draws it
-       * knows that the line has run out, and a counter beyond it says so to everybody who looks.) */
-      auto line_first = [&](const int l) -> Int64 { return acc_min<Int64>((Int64)l * p_line, p_count); };
-      auto line_count = [&](const int l) -> Int64 { return acc_min<Int64>(line_first(l) + p_line, p_count) - line_first(l); };
-      for (int turn = 0; turn <= ACC_GIANT_LINES; ++turn) {
-      if (turn > 0) {                                               /* the counters as they stand now */
-        __syncthreads();
-        if (tid < ACC_GIANT_LINES) s_job[8 + tid] = __hip_atomic_load(job + 8 + tid * ACC_GIANT_SPREAD, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __syncthreads();
-      }
-      int line = -1;
-      for (int k = 0; k < ACC_GIANT_LINES && line < 0; ++k) {
-        const int l = (int)((blockIdx.x + (unsigned int)k) % ACC_GIANT_LINES);
-        if (line_count(l) > 0 && (Int64)s_job[8 + l] <= line_count(l)) line = l;
-      }
-      if (line < 0) break;                                          /* every line has run out */
-      const Int64 l_first = line_first(line), l_count = line_count(line);
+      const Int64 l_first = line_first(g, line), l_count = line_count(g, line);
       for (;;) {
         __syncthreads();
         if (tid == 0) {
           unsigned long long t = __hip_atomic_fetch_add(job + 8 + line * ACC_GIANT_SPREAD, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           /* the ticket behind a line's last piece: one line more has run out; the last such line ends the job */
           if ((Int64)t == l_count &&
-              (Int64)__hip_atomic_fetch_add(job + 4, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1 == lines_in_use) {
-            acc_giant_ran_out(acc_jobs, acc_epoch);
+              (Int64)__hip_atomic_fetch_add(job + 4, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1 == lines_in_use)
             t = ~0ull;
-          }
-          s_job[0] = t;
+          s_tick = t;
         }
         __syncthreads();
-        const Int64 ticket = s_job[0] == ~0ull ? -1 : (Int64)s_job[0];
+        const Int64 ticket = s_tick == ~0ull ? -1 : (Int64)s_tick;
         if (ticket >= l_count) break;
         if (ticket < 0) {
           /* Every piece of every line has been drawn (whoever folds a piece asks for another ticket afterwards, so the
@@ -887,8 +887,7 @@ ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _sweep)(ACC_ENV_PARAMS
         const acc_opt<T> value = fold_range(from, to);
         if (tid == 0) pieces_of.put(slot_of(piece), acc_epoch, value.v);
       }
-      }   /* lines */
-    }
+    }   /* rounds */
   }
 }
 #endif

@@ -362,6 +362,38 @@ def test_an_instance_that_has_met_a_very_long_segment_takes_the_table(A, ctx):
         sk.destroy()
 
 
+def test_sparse_matrix_with_a_few_very_long_rows(A, ctx, tuned):
+    """the sparse matrix-vector product of a graph with a few hubs: rows of 40 000 to 200 000 non-zeros among rows of
+    eight, with and without the table of jobs; Float32 sums in index order with another association than the
+    sequential one, so against Float64 within 1e-5 of the sum of the magnitudes"""
+    import scipy.sparse as sp
+    rng = np.random.default_rng(90)
+    rows, ncols = 6000, 50000
+    lens = rng.poisson(8, rows).astype(np.int64)
+    for at, ln in ((17, 200000), (18, 40000), (3000, 90001), (5999, 65536)):
+        lens[at] = ln
+    offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    nnz = int(offs[-1])
+    vals = rng.standard_normal(nnz).astype(np.float32)
+    cols = rng.integers(0, ncols, nnz).astype(np.int32)
+    x = rng.standard_normal(ncols).astype(np.float32)
+    m = sp.csr_matrix((vals.astype(np.float64), cols.copy(), offs.copy()), shape=(rows, ncols))     # (scipy may put its arrays in order)
+    want = m @ x.astype(np.float64)
+    size = abs(m) @ np.abs(x.astype(np.float64))
+    dv, dc, dx, do = ctx.array(vals), ctx.array(cols), ctx.array(x), ctx.array(offs)
+    for knobs in ("foldseg.giants=0", "foldseg.giants=1"):
+        say("sparse matrix-vector product with four very long rows,", knobs)
+        tuned(knobs)
+        smvm = ctx.skeleton(A.SKEL_FOLDSEG, "float", env=[(1, "float"), (1, "Int32"), (1, "float")],
+                            get="acc_stream(arrIn0_0, ix) * arrIn2_0[acc_stream(arrIn1_0, ix)]", combine="x + y", seed="0.0f")
+        y = ctx.empty(rows, np.float32)
+        smvm.foldseg([dv, dc, dx], nnz, do, y)
+        got = y.get()
+        assert np.all(np.abs(got - want) <= 1e-5 * size + 1e-30), knobs
+        assert np.all(got[lens == 0] == 0.0)
+        smvm.destroy()
+
+
 def test_permute_of_sorted_and_clustered_keys(A, ctx):
     """runs of consecutive elements with one target: the kernels that update under a lock combine each run in its wave
     first (any combining function, floating-point addition on few targets, tuples); integer-valued sources, so every
