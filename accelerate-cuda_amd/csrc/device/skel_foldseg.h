@@ -88,6 +88,8 @@ static_assert(ACC_CHUNK % (ACC_BLOCK * ACC_VEC) == 0, "chunk must be a whole num
  * segment stays with its owner as if there were no table.  The table and the values carry the launch's tag
  * (nothing is cleared between launches).  Index order, another association than the sequential fold's: as for
  * every long segment.
+ *   The teams of lanes that take segments which are long on average (<entry>_team, below) enter a segment that is
+ * far longer than the rest in the same table, whole and with no value of their own.
  *   Variants 4 to 7 of an instance are built like this, and the host takes them once a look at the segment lengths
  * (<entry>_probe, at the end of this file) has found such a segment.  Not every instance, not from the start: the code
  * in this kernel lies behind the test for a stretch that the workgroup folds together, and yet, with it compiled in
@@ -108,6 +110,7 @@ static_assert(ACC_CHUNK % (ACC_BLOCK * ACC_VEC) == 0, "chunk must be a whole num
 #endif
 #define ACC_GIANT_PIECE ((Int64)ACC_GIANT_CHUNKS * ACC_CHUNK)
 #define ACC_GIANT_FROM  (2 * ACC_GIANT_PIECE)
+#define ACC_GIANT_TIMES 32                               /* ... and, for a team of lanes, so many times the average segment */
 #if ACC_GIANTS
 #define ACC_GIANT_PARAMS , unsigned long long *__restrict__ acc_jobs, const unsigned int acc_epoch, unsigned int *acc_status
 #define ACC_GIANT_JOBS  32                               /* the host sizes the scratch block by these three */
@@ -136,8 +139,9 @@ static_assert(ACC_CHUNK % (ACC_BLOCK * ACC_VEC) == 0, "chunk must be a whole num
 #endif
 
 #if ACC_GIANTS
-/* enter elements [a, b) of segment `seg` in the table of jobs; the job's number, or -1 if the table is full */
-ACC_DEV int acc_giant_enter(unsigned long long *jobs, const unsigned int epoch, const Int64 seg, const Int64 a, const Int64 b)
+/* enter elements [a, b) of segment `seg` in the table of jobs; the job's number, or -1 if the table is full.
+ * `with_value`: the owner has folded a part of the segment itself and leaves its value for whoever joins the pieces */
+ACC_DEV int acc_giant_enter(unsigned long long *jobs, const unsigned int epoch, const Int64 seg, const Int64 a, const Int64 b, const bool with_value)
 {
   unsigned long long h = __hip_atomic_load(jobs, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   unsigned int at;
@@ -160,7 +164,7 @@ ACC_DEV int acc_giant_enter(unsigned long long *jobs, const unsigned int epoch, 
   __hip_atomic_store(j + 4, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   for (int k = 0; k < ACC_GIANT_LINES; ++k) __hip_atomic_store(j + 8 + k * ACC_GIANT_SPREAD, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   /* (nobody looks at a job before this launch has ended: no order among these stores is needed) */
-  __hip_atomic_store(j, tag | 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(j, tag | (with_value ? 1u : 2u), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   return (int)at;
 }
 
@@ -363,7 +367,7 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
              * workgroup goes on with the chunk in which the segment ends. */
             const Int64 rest = ACC_FOLD_RIGHT ? cs - a : b - ce;
             if (acc_jobs && rest >= ACC_GIANT_FROM) {
-              const int job = ACC_FOLD_RIGHT ? acc_giant_enter(acc_jobs, acc_epoch, seg, a, cs) : acc_giant_enter(acc_jobs, acc_epoch, seg, ce, b);
+              const int job = ACC_FOLD_RIGHT ? acc_giant_enter(acc_jobs, acc_epoch, seg, a, cs, true) : acc_giant_enter(acc_jobs, acc_epoch, seg, ce, b, true);
               if (job >= 0) {                                      /* (no room in the table: the segment stays here) */
                 const acc_tagged<T> values_of = {acc_jobs + ACC_GIANT_HEAD + ACC_GIANT_JOBS * ACC_GIANT_JOB};
                 values_of.put(acc_giant_edge_slot(n, job), acc_epoch, acc);
@@ -544,12 +548,15 @@ ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _team)(ACC_ENV_PARAMS
                                      const Int64 shOut_0, ACC_OUT_ARRAY(arrOut),
                                      ACC_SEG_PARAMS,
                                      const int block_team, const Int64 split,
-                                     ACC_ELT *__restrict__ part, int *__restrict__ part_ok ACC_GUARD_PARAM)
+                                     ACC_ELT *__restrict__ part, int *__restrict__ part_ok ACC_GIANT_PARAMS ACC_GUARD_PARAM)
 {
   ACC_GUARD_CHECK
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
   __shared__ acc_opt<T> s_wave[ACC_FS_WAVES];
+#if ACC_GIANTS
+  __shared__ int s_entered;
+#endif
 
   auto get = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
   auto f   = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
@@ -613,6 +620,9 @@ ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _team)(ACC_ENV_PARAMS
     return r;
   };
 
+#if ACC_GIANTS
+  const Int64 giant_from = acc_max<Int64>(ACC_GIANT_FROM, ACC_GIANT_TIMES * (n / acc_max<Int64>(nseg, 1)));
+#endif
   for (Int64 job = team0; job < nseg * split; job += nteams) {
     const Int64 seg = job / split, part_no = job - seg * split;
     const Int64 sa = ACC_SEG_AT(seg);
@@ -621,6 +631,24 @@ ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _team)(ACC_ENV_PARAMS
     const Int64 piece = (((sb - sa) + split - 1) / split + round - 1) / round * round;
     const Int64 a = split > 1 ? acc_min<Int64>(sa + part_no * piece, sb) : sa;
     const Int64 b = split > 1 ? acc_min<Int64>(a + piece, sb) : sb;
+#if ACC_GIANTS
+    /* A segment far longer than the rest -- a team would walk it alone long after the others have ended: one of 2^23
+     * elements among segments of 256 to 4096 took 14-44 ms -- is entered in the table of jobs whole and left to the
+     * launch that takes the jobs (ACC_GIANTS, above).  (Not where every segment is cut into pieces anyway.)  The
+     * team's first lane enters it and tells the others. */
+    if (acc_jobs && split == 1) {
+      int entered = (me == 0 && sb - sa >= giant_from) ? (acc_giant_enter(acc_jobs, acc_epoch, seg, sa, sb, false) >= 0 ? 1 : 0) : 0;
+      if (whole_block) {
+        if (tid == 0) s_entered = entered;
+        __syncthreads();
+        entered = s_entered;
+        __syncthreads();
+      } else {
+        entered = __shfl(entered, row_team ? (acc_lane() & ~15) : 0);
+      }
+      if (entered) continue;
+    }
+#endif
     const Int64 nrounds = b > a ? (b - a + round - 1) / round : 0;
     acc_opt<T> acc = acc_none<T>();
     for (Int64 r0 = 0; r0 < nrounds; r0 += ACC_TROUNDS) {
@@ -703,9 +731,10 @@ ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _probe)(ACC_ENV_PARAMS
                                       const Int64 shOut_0, ACC_OUT_ARRAY(arrOut),
                                       ACC_SEG_PARAMS ACC_GUARD_PARAM, unsigned int *acc_hint)
 {
-  (void)shIn_0;
+  /* (what the kernels with the table take for such a segment: the staged one, and the teams of lanes) */
+  const Int64 from = acc_max<Int64>(ACC_GIANT_FROM + 2 * ACC_CHUNK, ACC_GIANT_TIMES * (shIn_0 / acc_max<Int64>(shOut_0, 1)));
   for (Int64 s = (Int64)blockIdx.x * ACC_BLOCK + threadIdx.x; s < shOut_0; s += (Int64)gridDim.x * ACC_BLOCK)
-    if ((Int64)arrSeg_0[s + 1] - (Int64)arrSeg_0[s] >= ACC_GIANT_FROM + 2 * ACC_CHUNK) *acc_hint = 1u;
+    if ((Int64)arrSeg_0[s + 1] - (Int64)arrSeg_0[s] >= from) *acc_hint = 1u;
 }
 #endif
 
@@ -869,15 +898,23 @@ ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _sweep)(ACC_ENV_PARAMS
             acc_opt<T> whole = s_part[0];
 #pragma unroll
             for (int w = 1; w < ACC_BLOCK / ACC_WAVE; ++w) whole = lf(whole, s_part[w]);
-            /* and joined with what the owner folded itself before it handed the rest over */
-            const T edge = pieces_of.wait(acc_giant_edge_slot(n, j), acc_epoch, acc_status);
+            /* and joined with what the owner folded itself before it handed the rest over, if it did */
+            if ((unsigned int)s_jobs[j][0] == 1u) {
+              const T edge = pieces_of.wait(acc_giant_edge_slot(n, j), acc_epoch, acc_status);
 #if ACC_FOLD_RIGHT
-            ACC_SET(arrOut, g_seg, f(whole.v, edge));               /* (a seed is in the owner's value already) */
+              ACC_SET(arrOut, g_seg, f(whole.v, edge));             /* (a seed is in the owner's value already) */
 #elif ACC_HAS_SEED
-            ACC_SET(arrOut, g_seg, f(f(edge, whole.v), seed));
+              ACC_SET(arrOut, g_seg, f(f(edge, whole.v), seed));
 #else
-            ACC_SET(arrOut, g_seg, f(edge, whole.v));
+              ACC_SET(arrOut, g_seg, f(edge, whole.v));
 #endif
+            } else {
+#if ACC_HAS_SEED
+              ACC_SET(arrOut, g_seg, f(whole.v, seed));             /* the seed is the last operand in either association */
+#else
+              ACC_SET(arrOut, g_seg, whole.v);
+#endif
+            }
           }
           break;
         }

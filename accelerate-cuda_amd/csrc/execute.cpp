@@ -302,6 +302,67 @@ namespace {
 //   `giants` (foldSeg of a vector): the kernel of the short segments hands segments of 8 chunks or more over to a
 //   table of jobs that every workgroup helps with when its own segments are done (skel_foldseg.h, ACC_GIANTS); the
 //   table and the pieces' values live in a block of tagged words sized by the source.
+// Very long segments among the others (skel_foldseg.h, ACC_GIANTS).  Variants 4 to 7 of a segmented fold hand such a
+// segment over to a second launch, at a cost to sources that have none; so an instance takes them once a look at its
+// segment lengths has found such a segment -- a small kernel behind calls number 1, 2, 4, 8 ... of the instance, which
+// says so in a word of host memory -- and once they are compiled, which happens in the background meanwhile.
+// `foldseg.giants`: 2 this, 1 always, 0 never.
+struct GiantsPlan {
+  bool hand_over = false;      // this call takes variant `lv + 4`
+  bool look = false;           // this call is followed by the look at the segment lengths
+};
+
+int plan_giants(acc_skel_s *s, int lv, GiantsPlan *plan)
+{
+  plan->hand_over = s->knobs.foldseg_giants == 1;
+  if (s->knobs.foldseg_giants != 2 || s->hint_slot < 0) return ACC_OK;
+  if (!s->met_giants.load(std::memory_order_relaxed) && s->ctx->status_host[acc::STATUS_WORDS + s->hint_slot] != 0)
+    s->met_giants.store(true, std::memory_order_relaxed);
+  if (s->met_giants.load(std::memory_order_relaxed)) {
+    ACC_TRY(s->start_variant(lv + 4));
+    plan->hand_over = s->variant_compiled(lv + 4);
+  } else {
+    const unsigned call = s->seg_calls.fetch_add(1, std::memory_order_relaxed) + 1;
+    plan->look = (call & (call - 1)) == 0;
+  }
+  return ACC_OK;
+}
+
+// the look: the parameters of the fold's own kernel (`common`, a guard's address behind them) and the word's address
+int launch_probe(acc_skel_s *s, int lv, Args *common, int64_t nseg, hipStream_t st)
+{
+  (void)common->data();
+  common->ptr(s->ctx->status_dev + (uint64_t)(acc::STATUS_WORDS + s->hint_slot) * sizeof(uint32_t));
+  const int64_t lookers = std::min<int64_t>((nseg + s->spec.block - 1) / s->spec.block, (int64_t)s->ctx->props.multiProcessorCount * 8);
+  hipError_t e = launch_kernel(s->variants[lv].fn_sweep, static_cast<unsigned>(lookers), 1, 1, static_cast<unsigned>(s->spec.block), 1, 1, 0, st,
+                               common->data_without_guard(), nullptr);
+  return e == hipSuccess ? ACC_OK : acc::fail_hip(e, "hipModuleLaunchKernel(segmented fold, probe)");
+}
+
+// the table of jobs: head, 32 jobs of 8 words and 16 ticket counters 32 words apart, then values of tagged words -- two
+// for every piece of 4 chunks the source has, and one a job
+int acquire_jobs(acc_skel_s *s, int lv, int64_t n, hipStream_t st, acc::ScratchRef *jobs)
+{
+  const int64_t piece = (int64_t)std::max(1, s->knobs.foldseg_giant_chunks) * (int64_t)((lv & 2) ? s->spec.chunk_long : s->spec.chunk);
+  const size_t words_a_value = ((size_t)s->spec.elt_size + 3) / 4;
+  const size_t bytes = (8 + 32 * (8 + 16 * 32) + (2 * (size_t)(n / piece + 2) + 32) * words_a_value) * 8;
+  return s->ctx->scratch_acquire(bytes, st, acc::SCRATCH_FLAGS, jobs);
+}
+
+// the second launch, which takes what the first has entered in the table: `common` with the table behind it
+int launch_sweep(acc_skel_s *s, int lv, Args *common, const acc::ScratchRef &jobs, hipStream_t st)
+{
+  common->ptr(reinterpret_cast<uint64_t>(jobs.ptr));
+  common->u32(jobs.epoch);
+  common->ptr(s->ctx->status_dev);
+  const int64_t sweepers = (int64_t)s->ctx->props.multiProcessorCount * std::max(1, std::min(s->knobs.foldseg_sweep_per_cu, 2048 / s->spec.block));
+  hipError_t e = launch_kernel(s->variants[lv].fn_sweep, static_cast<unsigned>(sweepers), 1, 1, static_cast<unsigned>(s->spec.block), 1, 1, 0, st,
+                               common->data(), nullptr);
+  return e == hipSuccess ? ACC_OK : acc::fail_hip(e, "hipModuleLaunchKernel(segmented fold, sweep)");
+}
+
+// `args`: the parameters every kernel of the template begins with (free arrays, result, segments).  `giants`: the
+// segments are a vector's (the kernels of rows and of arrays of rank > 1 know no table).
 int launch_segmented(acc_skel_s *s, int v, Args *args, const acc_array *env, const acc_array *out, int64_t nseg, int64_t n,
                      hipStream_t st, bool giants = false)
 {
@@ -315,59 +376,25 @@ int launch_segmented(acc_skel_s *s, int v, Args *args, const acc_array *env, con
       lv = v + 2;
       ACC_TRY(s->ensure_variant(lv));
     }
-    const int64_t grid = acc_launch_grid(nseg, s->spec.block, resident(s, lv), s->knobs.foldseg_oversub);
-    if (!giants) return launch(s, lv, grid, 0, st, args);      // (rows of an array: the kernels have no such parameters)
-    // Very long segments among short ones (skel_foldseg.h, ACC_GIANTS).  Variants 4 to 7 hand what is left of such a
-    // segment over to a second launch, at a cost to sources that have none; so an instance takes them once a look at
-    // its segment lengths has found such a segment -- a small kernel behind calls number 1, 2, 4, 8 ... of the
-    // instance, which says so in a word of host memory -- and once they are compiled, which happens in the
-    // background meanwhile.  `foldseg.giants`: 2 this, 1 always, 0 never.
-    bool hand_over = s->knobs.foldseg_giants == 1;
-    bool look = false;
-    if (s->knobs.foldseg_giants == 2 && s->hint_slot >= 0) {
-      if (!s->met_giants.load(std::memory_order_relaxed) && s->ctx->status_host[acc::STATUS_WORDS + s->hint_slot] != 0)
-        s->met_giants.store(true, std::memory_order_relaxed);
-      if (s->met_giants.load(std::memory_order_relaxed)) {
-        ACC_TRY(s->start_variant(lv + 4));
-        hand_over = s->variant_compiled(lv + 4);
-      } else {
-        const unsigned call = s->seg_calls.fetch_add(1, std::memory_order_relaxed) + 1;
-        look = (call & (call - 1)) == 0;
-      }
-    }
-    if (!hand_over) {
+    GiantsPlan plan;
+    if (giants) ACC_TRY(plan_giants(s, lv, &plan));
+    if (!plan.hand_over) {
+      const int64_t grid = acc_launch_grid(nseg, s->spec.block, resident(s, lv), s->knobs.foldseg_oversub);
       int rc = launch(s, lv, grid, 0, st, args);
-      if (rc == ACC_OK && look) {
-        (void)args->data();                                   // (a guard's address, if there is one, comes before the word's)
-        args->ptr(s->ctx->status_dev + (uint64_t)(acc::STATUS_WORDS + s->hint_slot) * sizeof(uint32_t));
-        const int64_t lookers = std::min<int64_t>((nseg + s->spec.block - 1) / s->spec.block, (int64_t)s->ctx->props.multiProcessorCount * 8);
-        hipError_t e = launch_kernel(s->variants[lv].fn_sweep, static_cast<unsigned>(lookers), 1, 1, static_cast<unsigned>(s->spec.block), 1, 1, 0, st,
-                                     args->data_without_guard(), nullptr);
-        if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(segmented fold, probe)");
-      }
+      if (rc == ACC_OK && plan.look) rc = launch_probe(s, lv, args, nseg, st);
       return rc;
     }
     lv += 4;
     ACC_TRY(s->ensure_variant(lv));
-    const int64_t grid4 = acc_launch_grid(nseg, s->spec.block, resident(s, lv), s->knobs.foldseg_oversub);
-    // the table of jobs: head, 32 jobs of 8 words and 16 ticket counters 32 words apart, then values of tagged words --
-    // two for every piece of 4 chunks the source has, and one a job
-    const int64_t piece = (int64_t)std::max(1, s->knobs.foldseg_giant_chunks) * (int64_t)((lv & 2) ? s->spec.chunk_long : s->spec.chunk);
-    const size_t words_a_value = ((size_t)s->spec.elt_size + 3) / 4;
-    const size_t bytes = (8 + 32 * (8 + 16 * 32) + (2 * (size_t)(n / piece + 2) + 32) * words_a_value) * 8;
+    const int64_t grid = acc_launch_grid(nseg, s->spec.block, resident(s, lv), s->knobs.foldseg_oversub);
     acc::ScratchRef jobs;
-    ACC_TRY(s->ctx->scratch_acquire(bytes, st, acc::SCRATCH_FLAGS, &jobs));
-    args->ptr(reinterpret_cast<uint64_t>(jobs.ptr));
-    args->u32(jobs.epoch);
-    args->ptr(s->ctx->status_dev);
-    int rc = launch(s, lv, grid4, 0, st, args);
-    if (rc == ACC_OK) {
-      // the second launch, which takes what the first has entered in the table: as many workgroups as the device holds
-      const int64_t sweepers = (int64_t)s->ctx->props.multiProcessorCount * std::max(1, std::min(s->knobs.foldseg_sweep_per_cu, 2048 / s->spec.block));
-      hipError_t e = launch_kernel(s->variants[lv].fn_sweep, static_cast<unsigned>(sweepers), 1, 1, static_cast<unsigned>(s->spec.block), 1, 1, 0, st,
-                                   args->data(), nullptr);
-      if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(segmented fold, sweep)");
-    }
+    ACC_TRY(acquire_jobs(s, lv, n, st, &jobs));
+    Args first = *args;
+    first.ptr(reinterpret_cast<uint64_t>(jobs.ptr));
+    first.u32(jobs.epoch);
+    first.ptr(s->ctx->status_dev);
+    int rc = launch(s, lv, grid, 0, st, &first);
+    if (rc == ACC_OK) rc = launch_sweep(s, lv, args, jobs, st);
     s->ctx->scratch_release(jobs, st);
     return rc;
   }
@@ -379,25 +406,40 @@ int launch_segmented(acc_skel_s *s, int v, Args *args, const acc_array *env, con
   const int64_t min_piece = team_lanes * 64;                          // a piece keeps its team busy for a while
   int64_t split = 1;
   if (nseg * 2 <= room) split = std::max<int64_t>(1, std::min<int64_t>({room / nseg, avg / min_piece, s->knobs.foldseg_max_split}));
-  acc::ScratchRef blk;
+  // (segments that are all cut into pieces are not looked at, and none is handed over)
+  GiantsPlan plan;
+  if (giants && split == 1) ACC_TRY(plan_giants(s, v, &plan));
+  const int tv = plan.hand_over ? v + 4 : v;
+  if (plan.hand_over) ACC_TRY(s->ensure_variant(tv));
+  acc::ScratchRef blk, jobs;
   uint64_t part = 0, part_ok = 0;
   if (split > 1) {
-    const size_t jobs = (size_t)(nseg * split);
-    const size_t ok_off = round256(jobs * s->spec.elt_size);
-    ACC_TRY(s->ctx->scratch_acquire(ok_off + jobs * 4, st, acc::SCRATCH_FOLD, &blk));
+    const size_t pieces = (size_t)(nseg * split);
+    const size_t ok_off = round256(pieces * s->spec.elt_size);
+    ACC_TRY(s->ctx->scratch_acquire(ok_off + pieces * 4, st, acc::SCRATCH_FOLD, &blk));
     part = reinterpret_cast<uint64_t>(blk.ptr);
     part_ok = part + ok_off;
   }
-  args->i32(block_team);
-  args->i64(split);
-  args->ptr(part);
-  args->ptr(part_ok);
+  if (plan.hand_over) {
+    const int rj = acquire_jobs(s, tv, n, st, &jobs);
+    if (rj != ACC_OK) { s->ctx->scratch_release(blk, st); return rj; }
+  }
+  Args team = *args;
+  team.i32(block_team);
+  team.i64(split);
+  team.ptr(part);
+  team.ptr(part_ok);
+  if (plan.hand_over) {
+    team.ptr(reinterpret_cast<uint64_t>(jobs.ptr));
+    team.u32(jobs.epoch);
+    team.ptr(s->ctx->status_dev);
+  }
   const int64_t per_block = block_team == 1 ? 1 : s->spec.block / team_lanes;
   const int64_t tgrid = acc_launch_grid(nseg * split, per_block, cus, 2048 / s->spec.block);
   int rc = s->ctx->make_current();
   if (rc == ACC_OK) {
-    hipError_t e = launch_kernel(s->variants[v].fn_finish, static_cast<unsigned>(tgrid), 1, 1,
-                                         static_cast<unsigned>(s->spec.block), 1, 1, 0, st, args->data(), nullptr);
+    hipError_t e = launch_kernel(s->variants[tv].fn_finish, static_cast<unsigned>(tgrid), 1, 1,
+                                         static_cast<unsigned>(s->spec.block), 1, 1, 0, st, team.data(), nullptr);
     if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(segmented fold, team)");
   }
   if (rc == ACC_OK && split > 1) {
@@ -417,7 +459,10 @@ int launch_segmented(acc_skel_s *s, int v, Args *args, const acc_array *env, con
       if (e != hipSuccess) rc = acc::fail_hip(e, "hipModuleLaunchKernel(segmented fold, join)");
     }
   }
+  if (rc == ACC_OK && plan.hand_over) rc = launch_sweep(s, tv, args, jobs, st);
+  if (rc == ACC_OK && plan.look) rc = launch_probe(s, v, args, nseg, st);
   s->ctx->scratch_release(blk, st);
+  if (plan.hand_over) s->ctx->scratch_release(jobs, st);
   return rc;
 }
 

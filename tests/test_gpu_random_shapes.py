@@ -324,30 +324,31 @@ def test_an_instance_that_has_met_a_very_long_segment_takes_the_table(A, ctx):
     import time
     rng = np.random.default_rng(89)
 
-    def inputs(longest):
-        lens = rng.poisson(6, 5000).astype(np.int64)
+    def inputs(longest, mean, nseg):
+        lens = rng.poisson(mean, nseg).astype(np.int64)
         lens[1234] = longest
         offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
         x = rng.integers(-9, 9, int(offs[-1])).astype(np.int32)
         c = np.concatenate([[0], np.cumsum(x.astype(np.int64))])
         return ctx.array(x), ctx.array(offs), int(offs[-1]), (c[offs[1:]] - c[offs[:-1]] + 7).astype(np.int32)
 
-    def kernels_of_a_call(sk, dx, do, n):
-        out = ctx.empty(5000, np.int32)
+    def kernels_of_a_call(sk, dx, do, n, nseg):
+        out = ctx.empty(nseg, np.int32)
         ctx.trace_start()
         sk.foldseg([dx], n, do, out)
         ctx.sync()
         return ctx.trace_stop()[0], out.get()
 
-    for longest, switches in ((200000, True), (3000, False)):
+    # (the last two: segments that rows of 16 lanes take, where "very long" is 32 times the average)
+    for longest, switches, mean, nseg in ((200000, True, 6, 5000), (3000, False, 6, 5000), (300000, True, 300, 20000), (9000, False, 300, 20000)):
         sk = ctx.skeleton(A.SKEL_FOLDSEG, "Int32", env=[(1, "Int32")], out_rank=1, get="arrIn0_0[ix]", combine="x + y", seed="7")
-        dx, do, n, want = inputs(longest)
-        say("segments of up to", longest, "elements: does the instance take the table?")
-        launches, got = kernels_of_a_call(sk, dx, do, n)
+        dx, do, n, want = inputs(longest, mean, nseg)
+        say("segments of", mean, "elements on average and one of", longest, ": does the instance take the table?")
+        launches, got = kernels_of_a_call(sk, dx, do, n, nseg)
         assert np.array_equal(got, want) and launches == 2          # the fold, and the look at the segment lengths
         deadline, taken = time.time() + 60, False
         for call in range(2, 4000):
-            launches, got = kernels_of_a_call(sk, dx, do, n)
+            launches, got = kernels_of_a_call(sk, dx, do, n, nseg)
             assert np.array_equal(got, want), call
             if switches:                                            # (the first look has found the segment: no more of them)
                 taken = taken or launches == 2                      # the fold and the launch that takes what it handed over
@@ -392,6 +393,61 @@ def test_sparse_matrix_with_a_few_very_long_rows(A, ctx, tuned):
         assert np.all(np.abs(got - want) <= 1e-5 * size + 1e-30), knobs
         assert np.all(got[lens == 0] == 0.0)
         smvm.destroy()
+
+
+def test_a_very_long_segment_among_segments_that_teams_of_lanes_fold(A, ctx, tuned):
+    """segments of a few hundred to a few ten thousand elements on average go to rows of 16 lanes, waves or workgroups,
+    a segment each; one that is far longer than the rest is entered in the table of jobs whole (`foldseg.giants=1`: the
+    variants with the table, always) and folded in pieces by the launch behind.  Sums of integers, a non-commutative
+    operator with and without a seed in both associations, and the same through the variants without the table."""
+    rng = np.random.default_rng(91)
+    aff = """
+__device__ __forceinline__ Word32 affine16(Word32 x, Word32 y) {
+  Word32 a1 = x >> 16, b1 = x & 0xffffu, a2 = y >> 16, b2 = y & 0xffffu;
+  return (((a1 * a2) & 0xffffu) << 16) | ((a1 * b2 + b1) & 0xffffu);
+}
+"""
+    cases = [("rows of 16 lanes", 300, 20000, {7000: 300000, 19999: 40000}), ("waves", 2000, 5000, {0: 250000, 2500: 2000 * 32 + 5}),
+             ("workgroups", 20000, 1100, {550: 20000 * 32 + 1})]
+
+    def chain(seg, right_seed=None):
+        vals = [int(v) for v in seg] + ([right_seed] if right_seed is not None else [])
+        acc = vals[0]
+        for v in vals[1:]:
+            acc = pyref.affine16(acc, v)
+        return acc
+
+    for knobs in ("foldseg.giants=1", "foldseg.giants=0"):
+        tuned(knobs)
+        fs = ctx.skeleton(A.SKEL_FOLDSEG, "Int32", env=[(1, "Int32")], out_rank=1, get="arrIn0_0[ix]", combine="x + y", seed="5")
+        f1 = ctx.skeleton(A.SKEL_FOLD1SEG, "Word32", env=[(1, "Word32")], out_rank=1, get="arrIn0_0[ix]", combine="affine16(x, y)", preamble=aff)
+        fr = ctx.skeleton(A.SKEL_FOLDSEG, "Word32", env=[(1, "Word32")], out_rank=1, get="arrIn0_0[ix]", combine="affine16(x, y)",
+                          seed="0x00030005u", preamble=aff, flags=A.FLAG_FOLD_RIGHT)
+        for name, mean, nseg, longs in cases:
+            lens = rng.poisson(mean, nseg).astype(np.int64)
+            lens[::97] = 0
+            for at, ln in longs.items():
+                lens[at] = ln
+            offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+            n = int(offs[-1])
+            say("a very long segment among teams of lanes:", knobs, name, "nseg", nseg, "n", n)
+            x = rng.integers(-9, 9, n).astype(np.int32)
+            c = np.concatenate([[0], np.cumsum(x.astype(np.int64))])
+            out = ctx.empty(nseg, np.int32)
+            fs.foldseg([ctx.array(x)], n, ctx.array(offs), out)
+            assert np.array_equal(out.get(), (c[offs[1:]] - c[offs[:-1]] + 5).astype(np.int32)), name
+            u = rng.integers(0, 2**32, n, dtype=np.uint64).astype(np.uint32)
+            g1, gr = ctx.empty(nseg, np.uint32), ctx.empty(nseg, np.uint32)
+            du, do = ctx.array(u), ctx.array(offs)
+            f1.foldseg([du], n, do, g1)
+            fr.foldseg([du], n, do, gr)
+            got1, gotr = g1.get(), gr.get()
+            for s_ in sorted(set(list(range(1, nseg, max(1, nseg // 12))) + list(longs) + [k + 1 for k in longs if k + 1 < nseg])):
+                if lens[s_] > 0:
+                    assert int(got1[s_]) == chain(u[offs[s_]:offs[s_ + 1]]), (name, "fold1Seg", s_, int(lens[s_]))
+                assert int(gotr[s_]) == chain(u[offs[s_]:offs[s_ + 1]], 0x00030005), (name, "foldSeg right", s_, int(lens[s_]))
+        for sk_ in (fs, f1, fr):
+            sk_.destroy()
 
 
 def test_permute_of_sorted_and_clustered_keys(A, ctx):
