@@ -316,7 +316,9 @@ int plan_giants(acc_skel_s *s, int lv, GiantsPlan *plan)
 {
   plan->hand_over = s->knobs.foldseg_giants == 1;
   if (s->knobs.foldseg_giants != 2 || s->hint_slot < 0) return ACC_OK;
-  if (!s->met_giants.load(std::memory_order_relaxed) && s->ctx->status_host[acc::STATUS_WORDS + s->hint_slot] != 0)
+  // (the word is the device's to write, at any time: read as such)
+  if (!s->met_giants.load(std::memory_order_relaxed) &&
+      __atomic_load_n(const_cast<uint32_t *>(s->ctx->status_host) + acc::STATUS_WORDS + s->hint_slot, __ATOMIC_RELAXED) != 0)
     s->met_giants.store(true, std::memory_order_relaxed);
   if (s->met_giants.load(std::memory_order_relaxed)) {
     ACC_TRY(s->start_variant(lv + 4));

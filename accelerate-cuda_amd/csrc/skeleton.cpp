@@ -956,7 +956,7 @@ int acc_skel_create_async(acc_context ctx, const acc_skel_desc *desc, acc_skel *
   s->knobs.resolve(*sp.tuning);
   if ((sp.kind == ACC_SKEL_FOLDSEG || sp.kind == ACC_SKEL_FOLD1SEG) && sp.out_rank <= 1 && ctx->status_host) {
     s->hint_slot = static_cast<int>(ctx->next_hint.fetch_add(1) % acc::HINT_WORDS);
-    ctx->status_host[acc::STATUS_WORDS + s->hint_slot] = 0;
+    __atomic_store_n(const_cast<uint32_t *>(ctx->status_host) + acc::STATUS_WORDS + s->hint_slot, 0u, __ATOMIC_RELAXED);
   }
   const int rc = s->start_variant(0);     // the other variants are built when a call first needs them
   if (rc != ACC_OK) { delete s; return rc; }

@@ -3,7 +3,8 @@
 // acc_skel may be executed from several threads") exercised where data races would sit -- the scratch pool (acquire,
 // release, trim, blocks of several protocols and sizes), the lazily built second variant of a shared instance,
 // instances created and destroyed while others run, the ordering of big scans across streams, guards set on and
-// taken off streams, the status block, the memory table, the launch trace; instances whose compilation runs on the
+// taken off streams, the status block, the memory table, the launch trace; a segmented fold that goes over to its
+// variants with a table of jobs while it is being launched; instances whose compilation runs on the
 // library's worker pool, used, waited for, polled and destroyed while it runs; a context's tuning table replaced
 // while instances are created, and a thread that keeps changing the environment meanwhile (no driver call reads
 // it).  Launches do nothing here; the checks are ThreadSanitizer's.  Exit status 0 and no report = pass.
@@ -17,6 +18,8 @@
 #include "../../include/acc_hip.h"
 
 extern "C" long mock_hip_launches(void);
+extern "C" void mock_hip_probe_finds(int argument);
+extern "C" long mock_hip_sweeps(void);
 
 #define OK(call)                                                                        \
   do {                                                                                  \
@@ -79,6 +82,7 @@ int main(int argc, char **argv)
   acc_skel hist = make(ctx, ACC_SKEL_PERMUTE, "Int32", "1", "x + y", nullptr, "arrIn0_0[ix]", ACC_COMBINE_ADD, 0);
   acc_skel locked = make(ctx, ACC_SKEL_PERMUTE, "Int16", "(Int16)1", "(Int16)(x + y)", nullptr, "arrIn0_0[ix]", 0, 0);
   acc_skel gmap = make(ctx, ACC_SKEL_MAP, "Int32", "arrIn0_0[ix] + 1", nullptr, nullptr, nullptr, 0, ACC_FLAG_GUARDED);
+  acc_skel segs = make(ctx, ACC_SKEL_FOLDSEG, "Int32", "arrIn0_0[ix]", "x + y", "0", nullptr, 0, 0);
   acc_memtable table = nullptr;
   OK(acc_memtable_create(ctx, 0, &table));
 
@@ -111,6 +115,15 @@ int main(int argc, char **argv)
         const int64_t nb = (r % 3 == 0) ? 256 : ((r % 3 == 1) ? 65536 : 200000);
         acc_array d = vec(zeros, nb), b = vec(bins, nb);
         OK(acc_exec_permute(hist, &a, n, &d, &b, st));
+        {
+          // a segmented fold, segments short or long on average; from a third of the way on its look at the segment
+          // lengths "finds" a very long one (mock_hip.cpp), and the instance goes over to its variants with a table of
+          // jobs -- compiled in the background, taken when they are there -- while all threads keep launching it
+          if (t == 0 && r == rounds / 3) mock_hip_probe_finds(6);      // env (extent, pointer), result (extent, pointer), source extent, offsets: the word comes 7th
+          const int64_t nseg = (r % 2 == 0) ? n / 8 + 1 : n / 700 + 1;
+          acc_array offs = vec(in, nseg + 1), sums = vec(out, nseg);
+          OK(acc_exec_foldseg(segs, &a, n, &offs, &sums, st));
+        }
         if (r % 4 == 1) {
           acc_array d16 = vec(zeros, 3000), b16 = vec(bins, 3000), few = vec(in, 2000);
           OK(acc_exec_permute(locked, &few, 2000, &d16, &b16, st));
@@ -255,7 +268,11 @@ int main(int argc, char **argv)
   }
   OK(acc_context_sync(ctx));
   OK(acc_memtable_destroy(table));
-  for (acc_skel s : {scan, fold, hist, locked, gmap}) OK(acc_skel_destroy(s));
+  if (mock_hip_sweeps() == 0) {
+    std::fprintf(stderr, "the segmented fold never went over to its variants with the table of jobs\n");
+    return 3;
+  }
+  for (acc_skel s : {scan, fold, hist, locked, gmap, segs}) OK(acc_skel_destroy(s));
   for (acc_devptr p : {in, out, bins, zeros}) OK(acc_free(ctx, p));
   OK(acc_context_destroy(ctx));
   std::printf("threads %d rounds %d launches %ld failures %d\n", threads, rounds, mock_hip_launches(), failures.load());

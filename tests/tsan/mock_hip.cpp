@@ -101,12 +101,27 @@ hipError_t hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(int *n, hipFunctio
   *n = std::max(1, std::min({8, 2048 / std::max(64, block), by_lds}));
   return hipSuccess;
 }
-hipError_t hipModuleLaunchKernel(hipFunction_t, unsigned, unsigned, unsigned, unsigned, unsigned, unsigned, unsigned, hipStream_t,
-                                 void **, void **)
+// The one kernel that does something here: a segmented fold's look at its segment lengths (<entry>_probe) finds a very
+// long segment once the driver says so -- it sets the word whose address is its argument number `g_probe_arg`, as the
+// kernel would -- so that the instance's change to its other variants happens among the threads that launch it.
+static std::atomic<int> g_probe_arg{-1};
+static std::atomic<long> g_sweeps{0};
+hipError_t hipModuleLaunchKernel(hipFunction_t f, unsigned, unsigned, unsigned, unsigned, unsigned, unsigned, unsigned, hipStream_t,
+                                 void **params, void **)
 {
   g_launches.fetch_add(1);
+  const char *name = reinterpret_cast<const Function *>(f)->name;
+  const size_t len = std::strlen(name);
+  const int at = g_probe_arg.load();
+  if (len > 6 && std::strcmp(name + len - 6, "_sweep") == 0) g_sweeps.fetch_add(1);
+  if (at >= 0 && params && len > 6 && std::strcmp(name + len - 6, "_probe") == 0) {
+    unsigned int *word = *reinterpret_cast<unsigned int **>(params[at]);
+    __atomic_store_n(word, 1u, __ATOMIC_RELAXED);
+  }
   return hipSuccess;
 }
+void mock_hip_probe_finds(int argument) { g_probe_arg.store(argument); }
+long mock_hip_sweeps(void) { return g_sweeps.load(); }
 
 }  // extern "C"
 
