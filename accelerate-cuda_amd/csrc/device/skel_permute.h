@@ -40,6 +40,10 @@
 
 #define ACC_TILE (ACC_BLOCK * ACC_VEC * ACC_UNROLL)
 
+#ifndef ACC_GATHER
+#define ACC_GATHER 1                                     /* 0: for measuring what the combining of a hot target's lanes is worth */
+#endif
+#define ACC_GATHER_MIN 4                                 /* lanes that share the target, from which they combine first */
 #if ACC_PERMUTE_LOCKED
 /* a value and whether a run of equal targets begins at its lane: the inclusive scan of such pairs under
  * (a, b) -> b begins a run ? b : a (+) b  leaves in every lane the combination of its run up to that lane */
@@ -95,8 +99,15 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, int *__restrict__ loc
     while (__ballot(!done) != 0 && trips < 64 * n + ACC_SPIN_LIMIT) {
       const bool got = !done && __hip_atomic_exchange(locks + j, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0;
       /* failed exchanges queue at the lock's address in front of the store that frees it: a wave that keeps
-       * getting nowhere steps back for a while */
-      if (trips >= 4 && __ballot(got) == 0) __builtin_amdgcn_s_sleep(32);
+       * getting nowhere steps back, for longer every time (up to a third of a millisecond: with the leaders of
+       * eight thousand waves after one lock -- half of 2^22 pairs on one target of three million -- and an
+       * exchange served every 0.1 us, each must stay away that long for the queue to stay short; stepping back for
+       * a microsecond at most, such a launch took 6.8 s) */
+      if (trips >= 4 && __ballot(got) == 0) {
+        const int naps = (int)acc_min<Int64>(trips - 3, 96);
+        for (int k = 0; k < naps; ++k) __builtin_amdgcn_s_sleep(127);
+        trips += naps;                                               /* (they count: the bound below is one of time) */
+      }
       if (got) {
         const T cur = ACC_READ_DEVICE(arrOut, j);
         ACC_SET_DEVICE(arrOut, j, f(x, cur));
@@ -116,9 +127,31 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, int *__restrict__ loc
   const int lane = acc_lane();
   auto join_runs = [&](const Int64 j, T &x, bool &active) {
     const Int64 j_before = acc_dpp<ACC_DPP_WAVE_SHR1, 0xf>(j, j);
-    const int active_before = acc_dpp<ACC_DPP_WAVE_SHR1, 0xf>((int)active, (int)active);
-    const bool continues = lane > 0 && active && active_before != 0 && j_before == j;
-    if (__ballot(continues) == 0) return;                              /* the same in every lane */
+    auto continues_now = [&]() -> bool {
+      const int active_before = acc_dpp<ACC_DPP_WAVE_SHR1, 0xf>((int)active, (int)active);
+      return lane > 0 && active && active_before != 0 && j_before == j;
+    };
+    bool continues = continues_now();
+    const unsigned long long runs = __ballot(continues);
+    if (runs == 0) return;                                             /* the same in every lane */
+#if ACC_GATHER
+    /* A hot target among others, in no order (half of 2^22 sources on one target of 100 000: 4.3-6.9 ms against
+     * 0.13-0.15 for uniform targets): its lanes stand all over the wave, a few of them side by side -- which is how
+     * it is found.  The lanes that share the target of the first run combine, wherever they stand, and the first of
+     * them goes on with the value. */
+    {
+      const Int64 hot = acc_readlane(j, (int)__builtin_ctzll(runs));
+      const bool same = active && j == hot;
+      const unsigned long long sharing = __ballot(same);
+      if (__builtin_popcountll(sharing) >= ACC_GATHER_MIN) {
+        const acc_opt<T> all = acc_wave_reduce(same ? acc_some(x) : acc_none<T>(), acc_lift<T>(f));
+        if (lane == (int)__builtin_ctzll(sharing)) x = all.v;
+        else if (same) active = false;
+        continues = continues_now();
+        if (__ballot(continues) == 0) return;
+      }
+    }
+#endif
     acc_run<T> r;
     r.v = x;
     r.head = continues ? 0 : 1;
@@ -301,6 +334,29 @@ ACC_DEV void acc_hint_apply(T *p, const T &x, F combine)
 
 #define ACC_SCOPE_BLOCK  __HIP_MEMORY_SCOPE_WORKGROUP
 #define ACC_SCOPE_DEVICE __HIP_MEMORY_SCOPE_AGENT
+
+/* A combination applied by compare-and-swap gives way under a hot target: every lane that finds the word changed
+ * tries again, and half of 2^22 sources on ONE target of 100 000 (in no order) took 4.3 ms against 0.13 for uniform
+ * targets.  So the lanes of a wave that share a target combine first and one of them applies the result, wherever in
+ * the wave they stand (neighbouring elements of one lane are taken care of by ACC_RUNS).  To find out, a lane looks
+ * at its neighbour's target only: with a hot target some two neighbours share it, and where no two neighbours share
+ * a target -- nearly always, for targets that are spread -- all this is five instructions an element.           */
+#define ACC_PERMUTE_CAS (ACC_COMBINE_HINT == ACC_HINT_GENERIC || (!ACC_ELT_IS_INTEGER && ACC_COMBINE_HINT != ACC_HINT_ADD))
+template <typename U, typename T, typename F>
+ACC_DEV void acc_wave_gather(U &t, T &x, F f)
+{
+  const int lane = acc_lane();
+  const U before = acc_wave_shift_up1(t);
+  const unsigned long long pairs = __ballot(lane > 0 && t == before);
+  if (pairs == 0) return;                                /* (the same in every lane) */
+  const U hot = acc_readlane(t, (int)__builtin_ctzll(pairs));
+  const bool same = t == hot;
+  const unsigned long long sharing = __ballot(same);
+  if (__builtin_popcountll(sharing) < ACC_GATHER_MIN) return;
+  const acc_opt<T> all = acc_wave_reduce(same ? acc_some(x) : acc_none<T>(), acc_lift<T>(f));
+  if (lane == (int)__builtin_ctzll(sharing)) x = all.v;
+  else if (same) t = (U)~(U)0;                           /* (beyond every bound: dropped, like `ignore`) */
+}
 
 /* The XCD this workgroup runs on (hardware register XCC_ID, bits 3:0).  Every
  * XCD has an L2 of its own, and global atomics execute in the L2 of the XCD
@@ -561,6 +617,16 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
       bool one_target = ACC_RUNS && ACC_VEC > 1;
 #pragma unroll
       for (int k = 1; k < ACC_VEC; ++k) one_target = one_target && j[u][k] == j[u][0];
+#if ACC_GATHER && ACC_PERMUTE_CAS
+      if (one_target) {
+#pragma unroll
+        for (int k = 1; k < ACC_VEC; ++k) { x[u][0] = f(x[u][0], x[u][k]); j[u][k] = (U)~(U)0; }
+      }
+#pragma unroll
+      for (int k = 0; k < ACC_VEC; ++k) acc_wave_gather(j[u][k], x[u][k], f);
+#pragma unroll
+      for (int k = 0; k < ACC_VEC; ++k) update(j[u][k], x[u][k]);
+#else
       if (one_target) {
         T all = x[u][0];
 #pragma unroll
@@ -570,6 +636,7 @@ permute(ACC_ENV_PARAMS ACC_OUT_PARAMS, const Int64 shIn_0, const int lds_bins, c
 #pragma unroll
         for (int k = 0; k < ACC_VEC; ++k) update(j[u][k], x[u][k]);
       }
+#endif
     }
 #endif
 #pragma unroll

@@ -272,6 +272,7 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       if (sp.permute_narrow && tuned("permute.merge_batch")) o << "#define ACC_MERGE_BATCH " << tune("permute.merge_batch", 16) << "\n";
       if (sp.permute_narrow) o << "#define ACC_MERGE_WAVES " << sp.merge_waves << "\n";
       if (tuned("permute.runs")) o << "#define ACC_RUNS " << tune("permute.runs", 1) << "\n";
+      if (tuned("permute.gather")) o << "#define ACC_GATHER " << (tune("permute.gather", 1) ? 1 : 0) << "\n";
       o << "#define ACC_ELT_IS_INTEGER " << (is_integer_type(sp.elt_type) ? 1 : 0) << "\n";
       o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_UNROLL " << sp.unroll << "\n";
       tmpl = "skel_permute.h";

@@ -450,6 +450,52 @@ __device__ __forceinline__ Word32 affine16(Word32 x, Word32 y) {
             sk_.destroy()
 
 
+def test_permute_with_a_hot_target_among_many(A, ctx, tuned):
+    """a third to a half of the sources on one or two targets, the rest spread, in no order: the lanes of a wave that
+    share the hot target combine first wherever they stand (tables under locks in LDS, locks in memory for tuples on
+    more targets than the tables hold, compare-and-swap on the result for scalars there); with ignored elements among
+    them; integer sums (exact), a maximum, pairs; and the same with `permute.gather=0`"""
+    rng = np.random.default_rng(92)
+    I32 = (1, "Int32")
+    for knobs in ("", "permute.gather=0"):
+        tuned(knobs)
+        generic = ctx.skeleton(A.SKEL_PERMUTE, "Int32", env=[I32, I32], out_rank=1, get="arrIn1_0[ix]", combine="x + y",
+                               permutation="arrIn0_0[ix]", combine_hint=A.COMBINE_GENERIC)
+        biggest = ctx.skeleton(A.SKEL_PERMUTE, "float", env=[I32, I32], out_rank=1, get="(float)arrIn1_0[ix]", combine="acc_max(x, y)",
+                               permutation="arrIn0_0[ix]", combine_hint=A.COMBINE_GENERIC)
+        pair = ctx.skeleton(A.SKEL_PERMUTE, "Int32, Int32", env=[I32, I32], out_rank=1, get="acc_elt{arrIn1_0[ix], 1}",
+                            combine="acc_elt{x.a1 + y.a1, x.a0 + y.a0}", permutation="arrIn0_0[ix]")
+        # (targets: few enough for one table in LDS; for several; more than the tables are taken for, whatever the element)
+        for n, bins, hot in ((200003, 900, (17,)), (500000, 100000, (7, 99999)), (1 << 18, 3000000, (123456,)), (70, 5, (2,))):
+            if knobs and bins > 1000000:
+                continue          # (a hundred thousand rounds on one lock in memory, one after the other: what the combining is there to avoid)
+            keys = rng.integers(0, bins, n)
+            for h in hot:
+                keys[rng.random(n) < 0.45 / len(hot)] = h
+            keys[rng.random(n) < 0.05] = -1
+            keys = keys.astype(np.int32)
+            w = rng.integers(-5, 6, n).astype(np.int32)
+            say("permute with hot targets", hot, ": n", n, "targets", bins, knobs)
+            valid = keys >= 0
+            want = np.bincount(keys[valid], weights=w[valid], minlength=bins).astype(np.int64)
+            count = np.bincount(keys[valid], minlength=bins)
+            dk, dw = ctx.array(keys), ctx.array(w)
+            out = ctx.empty(bins, np.int32)
+            generic.permute([dk, dw], n, ctx.array(np.full(bins, 3, np.int32)), out)
+            assert np.array_equal(out.get(), want + 3), ("generic", n, bins)
+            top = np.full(bins, -100.0, np.float32)
+            np.maximum.at(top, keys[valid], w[valid].astype(np.float32))
+            outf = ctx.empty(bins, np.float32)
+            biggest.permute([dk, dw], n, ctx.array(np.full(bins, -100.0, np.float32)), outf)
+            assert np.array_equal(outf.get(), top), ("max", n, bins)
+            outp, zero = ctx.empty_tuple(bins, [np.int32, np.int32]), ctx.empty_tuple(bins, [np.int32, np.int32])
+            zero.comps[0].set(np.zeros(bins, np.int32)); zero.comps[1].set(np.zeros(bins, np.int32))
+            pair.permute([dk, dw], n, zero, outp)
+            assert np.array_equal(outp.comps[0].get(), want) and np.array_equal(outp.comps[1].get(), count), ("pairs", n, bins)
+        for sk_ in (generic, biggest, pair):
+            sk_.destroy()
+
+
 def test_permute_of_sorted_and_clustered_keys(A, ctx):
     """runs of consecutive elements with one target: the kernels that update under a lock combine each run in its wave
     first (any combining function, floating-point addition on few targets, tuples); integer-valued sources, so every
