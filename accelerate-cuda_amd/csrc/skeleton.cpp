@@ -790,7 +790,14 @@ SkelSpec spec_of_variant(const SkelSpec &base, int v)
   if ((spec.kind == ACC_SKEL_FOLDSEG || spec.kind == ACC_SKEL_FOLD1SEG) && spec.out_rank <= 1 && v >= 4) spec.foldseg_giants = true;
   // a stencil's variants 2 and 3, 4 and 5: half and a quarter of the columns a lane, for arrays narrower than half or a
   // quarter of a strip, whose lanes would otherwise mostly lie outside the array
-  if ((spec.kind == ACC_SKEL_STENCIL || spec.kind == ACC_SKEL_STENCIL2) && v >= 2 && !spec.stencil_nd) {
+  // ... and 6 and 7: an element a thread (the form of stencils that strips cannot take), for arrays of a few columns,
+  // where nearly every lane of a strip would lie outside the array
+  if ((spec.kind == ACC_SKEL_STENCIL || spec.kind == ACC_SKEL_STENCIL2) && v >= 6 && !spec.stencil_nd) {
+    spec.stencil_nd = true;
+    spec.svec = 1;
+    spec.tile_w = spec.block;
+    spec.tile_h = 1;
+  } else if ((spec.kind == ACC_SKEL_STENCIL || spec.kind == ACC_SKEL_STENCIL2) && v >= 2 && !spec.stencil_nd) {
     spec.svec = std::max(1, spec.svec >> (v / 2));
     spec.tile_w = 64 * spec.svec;
   }
@@ -940,7 +947,7 @@ static int variant_count(const acc::SkelSpec &sp)
 {
   const bool stencil = sp.kind == ACC_SKEL_STENCIL || sp.kind == ACC_SKEL_STENCIL2;
   if ((sp.kind == ACC_SKEL_FOLDSEG || sp.kind == ACC_SKEL_FOLD1SEG) && sp.out_rank <= 1) return 8;
-  return sp.kind == ACC_SKEL_PERMUTE ? 8 : (stencil ? (sp.stencil_nd ? 2 : 6) : ((sp.scan_small_rows > 0 || sp.chunk_long > 0) ? 4 : 2));
+  return sp.kind == ACC_SKEL_PERMUTE ? 8 : (stencil ? (sp.stencil_nd ? 2 : 8) : ((sp.scan_small_rows > 0 || sp.chunk_long > 0) ? 4 : 2));
 }
 
 extern "C" {

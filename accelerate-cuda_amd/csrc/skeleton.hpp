@@ -100,7 +100,8 @@ struct acc_skel_s {
                               // [6], [7]: for integer addition on a table of 16-bit counts in LDS;
                               // of a segmented fold [2], [3]: a longer staged chunk, [4]-[7]: the same four with the table of
                               // jobs for very long segments; of a scan [2], [3]: small tiles;
-                              // of a stencil [2], [3] and [4], [5]: half and a quarter of the columns a lane
+                              // of a stencil [2], [3] and [4], [5]: half and a quarter of the columns a lane, [6], [7]: an
+                              // element a thread
   int hint_slot = -1;         // a segmented fold: its word among the context's hints (its segments were looked at: a very long one)
   std::atomic<bool> met_giants{false};   // ... and that the word has been seen set
   std::atomic<unsigned> seg_calls{0};    // ... and how often it has been launched (the look happens on calls 1, 2, 4, 8 ...)
