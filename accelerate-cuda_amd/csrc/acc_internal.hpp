@@ -97,6 +97,8 @@ void set_default_tuning(TuningPtr t);
   X(permute_xcd_row_kbytes, "permute.xcd_row_kbytes", 1024)                                                            \
   X(scan_small_below_kb, "scan.small_below_kb", 12288)                                                                 \
   X(stencil_half_strips, "stencil.half_strips", 1)                                                                     \
+  X(map_tiled_min_w, "map.tiled_min_w", 33)                                                                          \
+  X(map_tiled_min_h, "map.tiled_min_h", 10)                                                                          \
   X(stencil_thin_2d, "stencil.thin_2d", 20)                                                                          \
   X(stencil_thin_3d, "stencil.thin_3d", 6)                                                                           \
   X(stencil_narrow_max, "stencil.narrow_max", 2)                                                                       \

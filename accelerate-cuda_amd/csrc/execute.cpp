@@ -274,9 +274,16 @@ int acc_exec_map(acc_skel s, const acc_array *env, const acc_array *out, acc_str
   push_out(*out, &args, &aligned);
   const int64_t n = array_size(*out);
   if (n == 0) return ACC_OK;
-  const int v = aligned ? 0 : 1;
+  int v = aligned ? 0 : 1;
+  // A result of a few columns or rows leaves most of every tile outside it (a transpose of 2^23 x 2 either way:
+  // 170 us in tiles, 23-34 in runs): such a call takes variants 2 and 3, the same map in runs.  (A result of 2^20 rows
+  // of 8 / 16 / 24 / 32 columns: 45 / 56 / 100 / 44 us in tiles, 10 / 20 / 40 / 41 in runs, and 29 against 52 for 33
+  // columns.  Of 6 / 8 / 12 / 16 rows of 2^20 columns: 41 / 41 / 43 / 43 in tiles, 17 / 31 / 82 / 151 in runs.)
+  const bool in_tiles = s->spec.map_tiled && out->shape[s->spec.out_rank - 1] >= s->knobs.map_tiled_min_w &&
+                        out->shape[s->spec.out_rank - 2] >= s->knobs.map_tiled_min_h;
+  if (s->spec.map_tiled && !in_tiles) v += 2;
   ACC_TRY(s->ensure_variant(v));
-  if (s->spec.map_tiled) {
+  if (in_tiles) {
     // a wave per tile of 32 x 32 elements of the two innermost dimensions (skel_map.h)
     const int rank = s->spec.out_rank;
     const int64_t side = 8 * (int64_t)s->spec.map_tile_block;
@@ -299,9 +306,6 @@ namespace {
 //   from `foldseg.block_team_len` a workgroup, takes one segment at a time;
 //   fewer long segments than the device has room for teams: every segment is cut into `split` pieces, a team
 //   each, and a second launch joins the pieces in order.
-//   `giants` (foldSeg of a vector): the kernel of the short segments hands segments of 8 chunks or more over to a
-//   table of jobs that every workgroup helps with when its own segments are done (skel_foldseg.h, ACC_GIANTS); the
-//   table and the pieces' values live in a block of tagged words sized by the source.
 // Very long segments among the others (skel_foldseg.h, ACC_GIANTS).  Variants 4 to 7 of a segmented fold hand such a
 // segment over to a second launch, at a cost to sources that have none; so an instance takes them once a look at its
 // segment lengths has found such a segment -- a small kernel behind calls number 1, 2, 4, 8 ... of the instance, which

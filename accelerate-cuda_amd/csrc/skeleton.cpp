@@ -784,6 +784,8 @@ SkelSpec spec_of_variant(const SkelSpec &base, int v)
     if (v >= 4 && v < 6) spec.permute_windows = true;
     if (v >= 6) spec.permute_narrow = true;
   }
+  // a map in tiles: its variants 2 and 3 are the same map in runs, for results too thin for tiles
+  if (spec.map_tiled && v >= 2) spec.map_tiled = false;
   // a segmented fold's variants 2 and 3 (6 and 7): a longer staged chunk, for segments of 8 elements or more on
   // average; 4 to 7: what is left of a very long segment is handed over to a second launch
   if (spec.kind != ACC_SKEL_PERMUTE && (v & 2) && spec.chunk_long > 0) spec.chunk = spec.chunk_long;
@@ -947,6 +949,7 @@ static int variant_count(const acc::SkelSpec &sp)
 {
   const bool stencil = sp.kind == ACC_SKEL_STENCIL || sp.kind == ACC_SKEL_STENCIL2;
   if ((sp.kind == ACC_SKEL_FOLDSEG || sp.kind == ACC_SKEL_FOLD1SEG) && sp.out_rank <= 1) return 8;
+  if (sp.map_tiled) return 4;
   return sp.kind == ACC_SKEL_PERMUTE ? 8 : (stencil ? (sp.stencil_nd ? 2 : 8) : ((sp.scan_small_rows > 0 || sp.chunk_long > 0) ? 4 : 2));
 }
 

@@ -393,7 +393,7 @@ int acc_skel_source(acc_skel s, int variant, const char **source);
  * segmented fold of a vector the forms that hand segments far longer than
  * the rest over to a second launch at + 4; a stencil half and a quarter of
  * the columns a lane at + 2 and + 4, and an element a thread (for arrays of
- * a few columns) at + 6                                                      */
+ * a few columns) at + 6; a map in tiles the map in runs at + 2                */
 int acc_skel_preview(const acc_skel_desc *desc, int variant, const char **source, const char **entry);
 /* compile only (no GPU needed): used by the build check */
 int acc_skel_compile_only(const char *target, const acc_skel_desc *desc, size_t *code_size);

@@ -1024,13 +1024,15 @@ def test_scan_tile_shape_follows_the_register_count(A, ctx):
 
 def test_map_in_tiles_gives_what_the_map_in_runs_gives(A, ctx):
     """ACC_FLAG_TILED changes the order the result is produced in (tiles of 32 x 32, for element functions that read
-    across the rows of their source), never the result: transposes, ragged and narrow shapes, rank 3, a function of
-    the index alone, elements of 1 and 8 bytes"""
+    across the rows of their source), never the result: transposes, ragged and narrow shapes, shapes too thin for
+    tiles (which take the instance's variants in runs), rank 3, a function of the index alone, elements of 1 and 8 bytes"""
     rng = np.random.default_rng(9)
     for ctype, dt in (("float", np.float32), ("Int8", np.int8), ("double", np.float64)):
         tr = ctx.skeleton(A.SKEL_MAP, ctype, env=[(2, ctype)], out_rank=2, flags=A.FLAG_TILED,
                           get="arrIn0_0[(ix % shOut_0) * shIn0_0 + (ix / shOut_0)]")
-        for (h, w) in ((1, 1), (3, 70), (64, 64), (65, 63), (64, 128), (100, 257), (257, 100), (1, 500), (500, 1), (1030, 515)):
+        # (results of fewer than 10 rows or 33 columns are produced in runs after all: both sides of either bound)
+        for (h, w) in ((1, 1), (3, 70), (64, 64), (65, 63), (64, 128), (100, 257), (257, 100), (1, 500), (500, 1), (1030, 515),
+                       (40000, 5), (9, 70000), (10, 70000), (30011, 32), (30011, 33)):
             say("tiled transpose", ctype, (h, w))
             src = rng.integers(-100, 100, (w, h)).astype(dt)              # the source is w x h, the result h x w
             out = ctx.empty((h, w), dt)
