@@ -99,8 +99,8 @@ void set_default_tuning(TuningPtr t);
   X(stencil_half_strips, "stencil.half_strips", 1)                                                                     \
   X(map_tiled_min_w, "map.tiled_min_w", 33)                                                                          \
   X(map_tiled_min_h, "map.tiled_min_h", 10)                                                                          \
-  X(stencil_thin_2d, "stencil.thin_2d", 27)                                                                          \
-  X(stencil_thin_3d, "stencil.thin_3d", 8)                                                                           \
+  X(stencil_thin_2d, "stencil.thin_2d", 36)                                                                          \
+  X(stencil_thin_3d, "stencil.thin_3d", 16)                                                                          \
   X(stencil_narrow_max, "stencil.narrow_max", 2)                                                                       \
   X(stencil_stack, "stencil.stack", 0)                                                                                 \
   X(stencil_strips_per_cu, "stencil.strips_per_cu", 3)                                                                 \

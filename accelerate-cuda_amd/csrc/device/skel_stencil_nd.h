@@ -22,30 +22,33 @@
 #define ACC_B_WRAP 2
 #define ACC_B_CONSTANT 3
 
-struct acc_nd_index { Int64 i[ACC_STENCIL_RANK]; };
+/* Indices are 32 bits wide where the arrays allow it (fewer than 2^31 elements each): the index of an element is
+ * taken apart and the position of every tap put together with divisions, multiplications and comparisons, which cost
+ * twice to five times as much on 64-bit numbers -- 3 x 3 on 2^24 x 3 elements: 200 us with 64-bit indices. */
+template <typename I> struct acc_nd_index { I i[ACC_STENCIL_RANK]; };
 struct acc_nd_offset { int o[ACC_STENCIL_RANK]; };
 
-template <int MODE>
-ACC_DEV Int64 acc_nd_boundary(Int64 i, const Int64 sz)
+template <int MODE, typename I>
+ACC_DEV I acc_nd_boundary(I i, const I sz)
 {
-  if (MODE == ACC_B_CLAMP)  i = acc_max<Int64>(0, acc_min<Int64>(i, sz - 1));
+  if (MODE == ACC_B_CLAMP)  i = acc_max<I>(0, acc_min<I>(i, sz - 1));
   if (MODE == ACC_B_MIRROR) i = i < 0 ? -i : (i >= sz ? sz - (i - sz + 2) : i);
   if (MODE == ACC_B_WRAP)   i = i < 0 ? sz + i : (i >= sz ? i - sz : i);
   /* the maps assume the array spans the stencil; keep the address legal if not */
-  return acc_max<Int64>(0, acc_min<Int64>(i, sz - 1));
+  return acc_max<I>(0, acc_min<I>(i, sz - 1));
 }
 
 /* the element of `base` (extents `sh`) at `at` + `off`, under the boundary condition; `outside` beyond a constant boundary */
-template <int MODE, typename S>
-ACC_DEV S acc_nd_read(const S *__restrict__ base, const acc_nd_index &sh, const acc_nd_index &at, const acc_nd_offset &off, const S outside)
+template <int MODE, typename S, typename I>
+ACC_DEV S acc_nd_read(const S *__restrict__ base, const acc_nd_index<I> &sh, const acc_nd_index<I> &at, const acc_nd_offset &off, const S outside)
 {
-  Int64 lin = 0;
+  I lin = 0;
   bool inside = true;
 #pragma unroll
   for (int d = 0; d < ACC_STENCIL_RANK; ++d) {
-    const Int64 i = at.i[d] + off.o[d];
+    const I i = at.i[d] + (I)off.o[d];
     if (MODE == ACC_B_CONSTANT) inside = inside && i >= 0 && i < sh.i[d];
-    lin = lin * sh.i[d] + acc_nd_boundary<MODE>(i, sh.i[d]);
+    lin = lin * sh.i[d] + acc_nd_boundary<MODE, I>(i, sh.i[d]);
   }
   const S v = base[lin];
   return (MODE == ACC_B_CONSTANT && !inside) ? outside : v;
@@ -70,14 +73,20 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS, const int acc
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
   (void)acc_walk;
-  const acc_nd_index sh = {{ACC_OUT_EXTENTS}};
-  const acc_nd_index sh1 = {{ACC_SRC1_EXTENTS}};
+  const Int64 acc_extents[ACC_STENCIL_RANK] = {ACC_OUT_EXTENTS};
+  const Int64 acc_extents1[ACC_STENCIL_RANK] = {ACC_SRC1_EXTENTS};
 #if ACC_STENCIL_SOURCES == 2
-  const acc_nd_index sh2 = {{ACC_SRC2_EXTENTS}};
+  const Int64 acc_extents2[ACC_STENCIL_RANK] = {ACC_SRC2_EXTENTS};
 #endif
-  Int64 n = 1;
+  Int64 n = 1, n1 = 1, n2 = 1;
 #pragma unroll
-  for (int d = 0; d < ACC_STENCIL_RANK; ++d) n *= sh.i[d];
+  for (int d = 0; d < ACC_STENCIL_RANK; ++d) {
+    n *= acc_extents[d];
+    n1 *= acc_extents1[d];
+#if ACC_STENCIL_SOURCES == 2
+    n2 *= acc_extents2[d];
+#endif
+  }
   /* the value outside a constant boundary, component by component */
 #define ACC_DECLARE_OUTSIDE1(c, CT, OUTSIDE, arg) const CT acc_outside1_##c = (CT)OUTSIDE;
 #define ACC_DECLARE_OUTSIDE2(c, CT, OUTSIDE, arg) const CT acc_outside2_##c = (CT)OUTSIDE;
@@ -86,24 +95,38 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS, const int acc
 #undef ACC_DECLARE_OUTSIDE1
 #undef ACC_DECLARE_OUTSIDE2
 
-  for (Int64 ix = (Int64)blockIdx.x * ACC_BLOCK + threadIdx.x; ix < n; ix += (Int64)gridDim.x * ACC_BLOCK) {
-    acc_nd_index at;
-    Int64 rest = ix;
+  auto elements = [&](auto width) {
+    typedef decltype(width) I;
+    acc_nd_index<I> sh, sh1;
 #pragma unroll
-    for (int d = ACC_STENCIL_RANK - 1; d > 0; --d) {      /* innermost dimension last: Base.hs:207-218 */
-      at.i[d] = rest % sh.i[d];
-      rest /= sh.i[d];
-    }
-    at.i[0] = rest;
+    for (int d = 0; d < ACC_STENCIL_RANK; ++d) { sh.i[d] = (I)acc_extents[d]; sh1.i[d] = (I)acc_extents1[d]; }
+#if ACC_STENCIL_SOURCES == 2
+    acc_nd_index<I> sh2;
+#pragma unroll
+    for (int d = 0; d < ACC_STENCIL_RANK; ++d) sh2.i[d] = (I)acc_extents2[d];
+#endif
+    for (Int64 ix = (Int64)blockIdx.x * ACC_BLOCK + threadIdx.x; ix < n; ix += (Int64)gridDim.x * ACC_BLOCK) {
+      acc_nd_index<I> at;
+      I rest = (I)ix;
+#pragma unroll
+      for (int d = ACC_STENCIL_RANK - 1; d > 0; --d) {      /* innermost dimension last: Base.hs:207-218 */
+        at.i[d] = rest % sh.i[d];
+        rest /= sh.i[d];
+      }
+      at.i[0] = rest;
 #define ACC_ND_READ1(c, ...) acc_nd_read<ACC_BOUNDARY>(ACC_SRC1_ARRAY(c), sh1, at, acc_nd_offset{{__VA_ARGS__}}, acc_outside1_##c)
-    ACC_STENCIL_TAPS1_ND(ACC_ND_READ1)
+      ACC_STENCIL_TAPS1_ND(ACC_ND_READ1)
 #undef ACC_ND_READ1
 #if ACC_STENCIL_SOURCES == 2
 #define ACC_ND_READ2(c, ...) acc_nd_read<ACC_BOUNDARY2>(ACC_SRC2_ARRAY(c), sh2, at, acc_nd_offset{{__VA_ARGS__}}, acc_outside2_##c)
-    ACC_STENCIL_TAPS2_ND(ACC_ND_READ2)
+      ACC_STENCIL_TAPS2_ND(ACC_ND_READ2)
 #undef ACC_ND_READ2
 #endif
-    const T r = (T)(ACC_STENCIL_FN);
-    ACC_PUT(arrOut, ix, r);
-  }
+      const T r = (T)(ACC_STENCIL_FN);
+      ACC_PUT(arrOut, ix, r);
+    }
+  };
+  /* (the extents with a tap's offset added must fit as well: a stencil reaches 64 elements at most) */
+  if (n < 0x7fff0000LL && n1 < 0x7fff0000LL && n2 < 0x7fff0000LL) elements((int)0);
+  else elements((Int64)0);
 }

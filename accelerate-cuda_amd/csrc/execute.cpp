@@ -1181,9 +1181,9 @@ static int stencil_once(acc_skel s, const acc_array *env, const acc_array *in, c
   if (array_size(*out) == 0) return ACC_OK;
   // An array of a few columns leaves nearly every lane of a strip outside it (3 x 3 on 2^24 x 3: 1.9 ms, 7 points on
   // 2^22 x 2 x 2 and 2^24 x 1 x 1: 0.76 and 2.8 ms): variants 6 and 7 of the instance, an element a thread as for the
-  // stencils that strips cannot take, run at 2.0 (2-D) and 1.3 TB/s (3-D) whatever the shape, which is more than the
-  // strips reach up to 27 columns in 2-D (2^20 rows of 21 / 24 / 28: 117 us in strips, 89 / 100 / 117 so; 40: 60 against
-  // 84) and 8 in 3-D (2^19 x 4 x 8: 125 against 104; 2^17 x 8 x 16: 74 against 104).
+  // stencils that strips cannot take, run at 2.8 (2-D) and 2.1 TB/s (3-D) whatever the shape, which is more than the
+  // strips reach up to 36 columns in 2-D (2^20 rows of 28 / 33: 117 / 119 us in strips, 84 / 98 so; 2^19 of 40: 60
+  // either way) and 16 in 3-D (2^17 x 8 x 16: 74 against 65; 2^14 x 32 x 32: 51 against 65).
   const bool thin = !s->spec.stencil_nd && ((rank == 2 && w <= s->knobs.stencil_thin_2d) || (rank == 3 && w <= s->knobs.stencil_thin_3d));
   if (s->spec.stencil_nd || thin) {
     // an element of the result a thread (skel_stencil_nd.h); the kernel takes the strips' `walk` and ignores it

@@ -92,11 +92,11 @@ def test_random_stencils(A, ctx, rank):
 def test_stencils_on_arrays_narrower_than_a_strip(A, ctx, rank):
     """a strip is 256 columns wide: on narrower arrays (and in the last strip of wider ones, where that is short) the
     lane across the right edge holds 1 to 4 columns, the lanes beyond it none.  Every width modulo 4, reaches of 1, 2
-    and 4 columns, every boundary mode, elements of 1, 4 and 8 bytes.  Arrays of up to 27 columns (8 in three
+    and 4 columns, every boundary mode, elements of 1, 4 and 8 bytes.  Arrays of up to 36 columns (16 in three
     dimensions) take the variants that give a thread an element instead: both sides of that bound, and tall arrays of
     two and three columns."""
     rng = np.random.default_rng(2000 + rank)
-    widths = [2, 3, 4, 5, 6, 7, 8, 9, 27, 28, 63, 64, 66, 100, 129, 131, 202, 253, 254, 255, 256 + 65, 256 + 130, 512 + 70]
+    widths = [2, 3, 4, 5, 6, 7, 9, 16, 17, 36, 37, 63, 64, 66, 100, 129, 131, 202, 253, 254, 255, 256 + 65, 256 + 130, 512 + 70]
     cases = []
     for (ctype, T), mode, rx in itertools.product([("Int8", np.int8), ("float", np.float32), ("double", np.float64)],
                                                   ["clamp", "mirror", "wrap", "constant"], [1, 2, 4]):
