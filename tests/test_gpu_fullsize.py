@@ -240,3 +240,17 @@ def test_stencil_over_more_than_2_31_elements(A, ctx):
         c = img[y].astype(np.int32)
         left, right = np.concatenate([c[:1], c[:-1]]), np.concatenate([c[1:], c[-1:]])
         assert np.array_equal(got[y], (up + left + c + right + dn).astype(np.int8)), y
+    del img, got, b
+    # the same on an array of three columns, which goes an element a thread (with 64-bit indices: too many for 32)
+    h, w = (1 << 31) // 3 + 3000, 3
+    say("5-point stencil over", h * w, "Int8 elements in three columns")
+    img = (np.arange(h * w, dtype=np.int64) * 7 % 101).astype(np.int8).reshape(h, w)
+    b = ctx.empty((h, w), np.int8)
+    s.stencil([], ctx.array(img), b)
+    got = b.get()
+    for y0 in (0, 1 << 20, (1 << 31) // 3 - 500, h - 1000):    # (the rows on both sides of index 2^31 among them)
+        rows = np.arange(y0, y0 + 1000)
+        c = img[rows].astype(np.int32)
+        up, dn = img[np.maximum(rows - 1, 0)].astype(np.int32), img[np.minimum(rows + 1, h - 1)].astype(np.int32)
+        left, right = np.concatenate([c[:, :1], c[:, :-1]], axis=1), np.concatenate([c[:, 1:], c[:, -1:]], axis=1)
+        assert np.array_equal(got[rows], (up + left + c + right + dn).astype(np.int8)), y0
