@@ -733,14 +733,14 @@ def main():
         for ctype, dt in (("float", np.float32), ("double", np.float64)):
             lap3 = ctx.skeleton(A.SKEL_STENCIL, ctype, out_rank=3, taps=seven, boundary="clamp", stencil_fn="t1 + t2 + t3 + t4 + t5 + t6 - 6 * t0")
             box2 = ctx.skeleton(A.SKEL_STENCIL, ctype, out_rank=2, taps=nine, boundary="clamp", stencil_fn=" + ".join("t%d" % k for k in range(9)))
-            vols = ((512, 512, 512), (384, 384, 384), (300, 300, 300), (256, 256, 256), (150, 150, 150), (128, 128, 256), (100, 400, 419), (1024, 128, 128), (4096, 64, 64)) if ctype == "float" else ((256, 512, 512),)
+            vols = ((512, 512, 512), (384, 384, 384), (300, 300, 300), (256, 256, 256), (150, 150, 150), (128, 128, 256), (100, 400, 419), (1024, 128, 128), (4096, 64, 64), (1 << 22, 2, 2)) if ctype == "float" else ((256, 512, 512),)
             for shape in vols:
                 a, o = ctx.array(np.ones(shape, dt)), ctx.empty(shape, dt)
                 ad, od = a.desc(), o.desc()
                 one("stencil 7-point %s %d x %d x %d" % ((ctype,) + shape), lambda: A.check(L.acc_exec_stencil(lap3.handle, None, C.byref(ad), C.byref(od), stream)),
                     2 * int(np.prod(shape)) * np.dtype(dt).itemsize)
                 del a, o
-            imgs = ((1 << 17, 128), (1 << 18, 64), (55924, 300)) if ctype == "float" else ((8192, 8192),)
+            imgs = ((1 << 17, 128), (1 << 18, 64), (55924, 300), (1 << 24, 3)) if ctype == "float" else ((8192, 8192),)
             for shape in imgs:
                 a, o = ctx.array(np.ones(shape, dt)), ctx.empty(shape, dt)
                 ad, od = a.desc(), o.desc()
@@ -755,6 +755,14 @@ def main():
             one("transpose 8192 x 8192 Float32 " + name, lambda: A.check(L.acc_exec_map(tr.handle, se, C.byref(dd), stream)), 8 * side * side)
         assert np.array_equal(dst.get(), wl.stencil_image(side, side).T), "transpose mismatch"
         del src, dst
+        # (a result of two rows or two columns: most of every tile would lie outside it, so the tiled instance goes in runs)
+        for shape in ((1 << 23, 2), (2, 1 << 23)):
+            thin = np.arange(shape[0] * shape[1], dtype=np.float32).reshape(shape)
+            src, dst = ctx.array(thin), ctx.empty((shape[1], shape[0]), np.float32)
+            se, dd = envs(src), dst.desc()
+            one("transpose %d x %d Float32 (ACC_FLAG_TILED)" % shape, lambda: A.check(L.acc_exec_map(tr.handle, se, C.byref(dd), stream)), 8 * thin.size)
+            assert np.array_equal(dst.get(), thin.T), "transpose mismatch"
+            del src, dst
         # segmented sums whose lengths are very unequal: a million segments of 8 elements on average, one of which holds
         # half of the source (the rows of a power-law graph), folded by its workgroup alone (`foldseg.giants=0`) and handed
         # over to a second launch (`=1`; as the knobs stand an instance goes from the one to the other by itself, once
