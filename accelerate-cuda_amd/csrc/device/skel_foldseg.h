@@ -96,7 +96,7 @@ static_assert(ACC_CHUNK % (ACC_BLOCK * ACC_VEC) == 0, "chunk must be a whole num
  * and no such segment in the source, 2^25 elements in segments of 2 / 8 / 32 took 101 / 36 / 29 us instead of
  * 89 / 33 / 27 and the sparse matrix-vector product 193 instead of 190; the second launch costs a source without
  * such segments 2-3 us more.  (A test of every block of segments ahead of its first chunk, by way of a barrier that
- * carries the lanes' verdicts, made the segments of two elements 117 us: the block's first loads then wait for the
+ * carries the lanes' answers, made the segments of two elements 117 us: the block's first loads then wait for the
  * lanes' offsets.)                                                                                               */
 #ifndef ACC_GIANTS
 #define ACC_GIANTS 0
