@@ -14,9 +14,13 @@
  * ACC_OUT_EXTENTS (shOut_<rank-1>, ..., shOut_0), ACC_STENCIL_SOURCES (1|2), ACC_STENCIL_FN, ACC_BLOCK and per
  * source n = 1, 2: ACC_BOUNDARY (ACC_BOUNDARY2), ACC_SRC<n>_COMPONENTS(X, arg), ACC_SRC<n>_PARAMS,
  * ACC_SRC<n>_EXTENTS (the source's own extents, outermost first), ACC_IN<n>_ELT, ACC_STENCIL_TAPS<n>_ND(READ) with
- * READ(component, offset of the outermost dimension, ..., offset of the innermost).
+ * READ(component, offset of the outermost dimension, ..., offset of the innermost), ACC_SRC<n>_REACH_LO / _HI (how far
+ * the taps reach towards the beginning and the end of every dimension, outermost first).
  */
 
+#ifndef ACC_ND_INNER
+#define ACC_ND_INNER 1                                   /* 0: every element takes the way of the elements at the boundary */
+#endif
 #define ACC_B_CLAMP 0
 #define ACC_B_MIRROR 1
 #define ACC_B_WRAP 2
@@ -97,14 +101,35 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS, const int acc
 
   auto elements = [&](auto width) {
     typedef decltype(width) I;
-    acc_nd_index<I> sh, sh1;
+    acc_nd_index<I> sh, sh1, step1;
 #pragma unroll
     for (int d = 0; d < ACC_STENCIL_RANK; ++d) { sh.i[d] = (I)acc_extents[d]; sh1.i[d] = (I)acc_extents1[d]; }
+    /* (elements between neighbours along every dimension: the row-major position of an index is their inner product) */
+    step1.i[ACC_STENCIL_RANK - 1] = 1;
+#pragma unroll
+    for (int d = ACC_STENCIL_RANK - 2; d >= 0; --d) step1.i[d] = step1.i[d + 1] * sh1.i[d + 1];
+    constexpr int lo1[ACC_STENCIL_RANK] = ACC_SRC1_REACH_LO, hi1[ACC_STENCIL_RANK] = ACC_SRC1_REACH_HI;
 #if ACC_STENCIL_SOURCES == 2
-    acc_nd_index<I> sh2;
+    acc_nd_index<I> sh2, step2;
 #pragma unroll
     for (int d = 0; d < ACC_STENCIL_RANK; ++d) sh2.i[d] = (I)acc_extents2[d];
+    step2.i[ACC_STENCIL_RANK - 1] = 1;
+#pragma unroll
+    for (int d = ACC_STENCIL_RANK - 2; d >= 0; --d) step2.i[d] = step2.i[d + 1] * sh2.i[d + 1];
+    constexpr int lo2[ACC_STENCIL_RANK] = ACC_SRC2_REACH_LO, hi2[ACC_STENCIL_RANK] = ACC_SRC2_REACH_HI;
 #endif
+    auto inner_product = [&](const acc_nd_index<I> &a, const acc_nd_index<I> &b) -> I {
+      I v = 0;
+#pragma unroll
+      for (int d = 0; d < ACC_STENCIL_RANK; ++d) v += a.i[d] * b.i[d];
+      return v;
+    };
+    auto of_offset = [&](const acc_nd_offset &o, const acc_nd_index<I> &b) -> I {
+      I v = 0;
+#pragma unroll
+      for (int d = 0; d < ACC_STENCIL_RANK; ++d) v += (I)o.o[d] * b.i[d];
+      return v;
+    };
     for (Int64 ix = (Int64)blockIdx.x * ACC_BLOCK + threadIdx.x; ix < n; ix += (Int64)gridDim.x * ACC_BLOCK) {
       acc_nd_index<I> at;
       I rest = (I)ix;
@@ -114,15 +139,42 @@ ACC_STENCIL_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_SOURCE_PARAMS, const int acc
         rest /= sh.i[d];
       }
       at.i[0] = rest;
+      /* An element whose taps all lie inside the source(s) -- nearly every element of an array that is not thin --
+       * needs no boundary condition: a tap is then the element's own position plus a distance that is the same for
+       * all elements (nine planes of 256^3 floats: 93 -> 50 us; 3 x 3 on 4096^2: 59 -> 40 us). */
+      bool inside = ACC_ND_INNER != 0;
+#pragma unroll
+      for (int d = 0; d < ACC_STENCIL_RANK; ++d) {
+        inside = inside && at.i[d] >= (I)lo1[d] && at.i[d] < sh1.i[d] - (I)hi1[d];
+#if ACC_STENCIL_SOURCES == 2
+        inside = inside && at.i[d] >= (I)lo2[d] && at.i[d] < sh2.i[d] - (I)hi2[d];
+#endif
+      }
+      /* (wave by wave: a wave with an element at the boundary among its 64 would go both ways, one after the other) */
+      T r;
+      if (__ballot(!inside) == 0) {
+        const I here1 = inner_product(at, step1);
+#define ACC_ND_READ1(c, ...) ACC_SRC1_ARRAY(c)[here1 + of_offset(acc_nd_offset{{__VA_ARGS__}}, step1)]
+        ACC_STENCIL_TAPS1_ND(ACC_ND_READ1)
+#undef ACC_ND_READ1
+#if ACC_STENCIL_SOURCES == 2
+        const I here2 = inner_product(at, step2);
+#define ACC_ND_READ2(c, ...) ACC_SRC2_ARRAY(c)[here2 + of_offset(acc_nd_offset{{__VA_ARGS__}}, step2)]
+        ACC_STENCIL_TAPS2_ND(ACC_ND_READ2)
+#undef ACC_ND_READ2
+#endif
+        r = (T)(ACC_STENCIL_FN);
+      } else {
 #define ACC_ND_READ1(c, ...) acc_nd_read<ACC_BOUNDARY>(ACC_SRC1_ARRAY(c), sh1, at, acc_nd_offset{{__VA_ARGS__}}, acc_outside1_##c)
-      ACC_STENCIL_TAPS1_ND(ACC_ND_READ1)
+        ACC_STENCIL_TAPS1_ND(ACC_ND_READ1)
 #undef ACC_ND_READ1
 #if ACC_STENCIL_SOURCES == 2
 #define ACC_ND_READ2(c, ...) acc_nd_read<ACC_BOUNDARY2>(ACC_SRC2_ARRAY(c), sh2, at, acc_nd_offset{{__VA_ARGS__}}, acc_outside2_##c)
-      ACC_STENCIL_TAPS2_ND(ACC_ND_READ2)
+        ACC_STENCIL_TAPS2_ND(ACC_ND_READ2)
 #undef ACC_ND_READ2
 #endif
-      const T r = (T)(ACC_STENCIL_FN);
+        r = (T)(ACC_STENCIL_FN);
+      }
       ACC_PUT(arrOut, ix, r);
     }
   };

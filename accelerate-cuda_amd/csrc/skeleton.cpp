@@ -286,6 +286,7 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
         const int rank = sp.out_rank;
         o << "#define ACC_OUT_PARAMS " << out_params(rank, sp.elt_type) << "\n";
         o << "#define ACC_STENCIL_RANK " << rank << "\n";
+        if (tuned("stencil.nd_inner")) o << "#define ACC_ND_INNER " << (tune("stencil.nd_inner", 1) ? 1 : 0) << "\n";
         o << "#define ACC_STENCIL_SOURCES " << (two ? 2 : 1) << "\n";
         o << "#define ACC_OUT_EXTENTS";
         for (int dd = rank - 1; dd >= 0; --dd) o << " shOut_" << dd << (dd ? "," : "");
@@ -310,8 +311,18 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
           for (int dd = rank - 1; dd >= 0; --dd) o << " sh" << (with_extents ? array_name : "Out") << "_" << dd << (dd ? "," : "");
           o << "\n";
           o << "#define ACC_IN" << which << "_ELT " << (nc == 1 ? comps[0] : elt_name) << "\n";
-          o << "#define ACC_STENCIL_TAPS" << which << "_ND(READ) ";
           const size_t ntaps = off.size() / (size_t)rank;
+          // how far the taps reach towards the beginning and the end of every dimension (outermost first)
+          for (const char *side : {"LO", "HI"}) {
+            o << "#define ACC_SRC" << which << "_REACH_" << side << " {";
+            for (int dd = 0; dd < rank; ++dd) {
+              int most = 0;
+              for (size_t k = 0; k < ntaps; ++k) most = std::max(most, side[0] == 'L' ? -off[k * rank + dd] : off[k * rank + dd]);
+              o << (dd ? ", " : "") << most;
+            }
+            o << "}\n";
+          }
+          o << "#define ACC_STENCIL_TAPS" << which << "_ND(READ) ";
           for (size_t k = 0; k < ntaps; ++k) {
             o << "const ACC_IN" << which << "_ELT " << tap_name << k << " = ";
             if (nc > 1) o << "{ ";
