@@ -781,7 +781,7 @@ def backpermute(shape, p, a, across=False):
 
 def transpose(a):
     h, w = a.shape
-    return backpermute((w, h), lambda y, x: (x, y), a, across=True)
+    return backpermute((w, h), lambda y, x: (x, y), a, across=not a.across)
 
 
 def zip_(a, b):
@@ -824,7 +824,9 @@ def _fold(f, z, a, seedless, context):
     out_shape = a.shape[:-1] if seedless else tuple(max(1, d) for d in a.shape[:-1])
     arrays, sig, fr = _assemble(get=a.stream().text, combine=_combine(f, a.ctype).text,
                                 seed=None if seedless else Exp.of(z, a.ctype).text)
-    sk = cx.skeleton(A.SKEL_FOLD1 if seedless else A.SKEL_FOLD, _elt(a.ctype), sig, out_rank=len(out_shape), **fr)
+    # rows that lie across memory (the fold of a transposed matrix, of a product of replicated operands): a lane a row
+    sk = cx.skeleton(A.SKEL_FOLD1 if seedless else A.SKEL_FOLD, _elt(a.ctype), sig, out_rank=len(out_shape),
+                     flags=A.FLAG_TILED if a.across and len(out_shape) >= 1 else 0, **fr)
     out = _empty(cx, out_shape, a.ctype)
     cx.launch(arrays, [out], lambda i, o, s: sk.fold(i, a.shape, o[0], stream=s))
     return Acc(out_shape, a.ctype, manifest=out)
@@ -1222,7 +1224,8 @@ def replicate(spec, a):
     dims = iter(a.shape)
     shape = tuple(next(dims) if (x is All or x == All) else int(x) for x in spec)
     keep = [k for k, x in enumerate(spec) if x is All or x == All]
-    return backpermute(shape, lambda *ix: tuple(ix[k] for k in keep), a)
+    # (the innermost dimension of the result is the innermost one of `a`: what `a` reads across, the result does)
+    return backpermute(shape, lambda *ix: tuple(ix[k] for k in keep), a, across=a.across and keep[-1] == len(spec) - 1)
 
 
 def slice_(a, spec):

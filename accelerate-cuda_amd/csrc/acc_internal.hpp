@@ -67,6 +67,8 @@ void set_default_tuning(TuningPtr t);
 #define ACC_DRIVER_KNOBS(X)                                                                                          \
   X(fold_blocks_per_cu, "fold.blocks_per_cu", 4)                                                                       \
   X(fold_rows_max, "fold.rows_max", 7)                                                                                 \
+  X(fold_across, "fold.across", 2)                                                                                     \
+  X(fold_across_min_piece, "fold.across_min_piece", 64)                                                                \
   X(foldseg_block_team_len, "foldseg.block_team_len", 16384)                                                           \
   X(foldseg_long_from, "foldseg.long_from", 8)                                                                         \
   X(foldseg_max_split, "foldseg.max_split", 4096)                                                                      \

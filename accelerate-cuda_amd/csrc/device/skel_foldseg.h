@@ -513,6 +513,80 @@ ACC_FS_CAT_(ACC_FOLDSEG_ENTRY, _rows)(ACC_ENV_PARAMS
     default: break;                                /* the host does not launch this entry for other lengths */
   }
 }
+
+/* ---- rows that lie across memory: a lane per row, whatever the length ------
+ * <entry>_across, for an element function that, where the ROW index moves by one, reads neighbouring addresses --
+ * the fold of a transposed matrix (sums down its columns), of a matrix product written as a fold over
+ * `zipWith (*)` of two replicated operands, one of them transposed (ACC_FLAG_TILED says so: the host cannot see it).
+ * A team of lanes along such a row asks for 64 cache lines with every load; a lane per row, neighbouring rows in
+ * neighbouring lanes, asks for one.  Lane t takes piece t / rows of row t % rows: with fewer rows than the device
+ * has lanes the rows are cut into `split` pieces of consecutive elements, whose values <entry>_join puts together in
+ * order; with split == 1 the lane writes the row's result itself.  Every piece is folded in index order, eight
+ * elements requested before the first is used.                                                                   */
+#define ACC_ACROSS_UNROLL 8
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+ACC_FS_CAT_(ACC_FOLDSEG_ENTRY, _across)(ACC_ENV_PARAMS
+                                        const Int64 shOut_0, ACC_OUT_ARRAY(arrOut),
+                                        ACC_SEG_PARAMS,
+                                        const Int64 split, ACC_ELT *__restrict__ part, int *__restrict__ part_ok ACC_GUARD_PARAM)
+{
+  ACC_GUARD_CHECK
+  typedef ACC_ELT T;
+  ACC_ENV_ASSUME
+  auto get = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
+  auto f   = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
+  (void)shIn_1;
+  const Int64 rows = shOut_0, len = shIn_0;
+  const Int64 piece = (len + split - 1) / split;
+  for (Int64 t = (Int64)blockIdx.x * ACC_BLOCK + threadIdx.x; t < rows * split; t += (Int64)gridDim.x * ACC_BLOCK) {
+    const Int64 p = t / rows, row = t - p * rows;
+    const Int64 k0 = acc_min<Int64>(p * piece, len), k1 = acc_min<Int64>(k0 + piece, len);
+    if (k0 >= k1) {                                        /* (a last piece without elements; the host launches no empty rows) */
+      if (split > 1) part_ok[row * split + p] = 0;
+      continue;
+    }
+    const Int64 base = row * len;
+    T x[ACC_ACROSS_UNROLL];
+#if ACC_HAS_SEED
+    const T seed = (ACC_SEED);
+#endif
+#if ACC_FOLD_RIGHT
+    /* x0 (+) (x1 (+) (... (x_last (+) z))), as the other entries associate a row */
+    T acc = get(base + k1 - 1);
+#if ACC_HAS_SEED
+    if (split == 1) acc = f(acc, seed);
+#endif
+    Int64 k = k1 - 1;
+    for (; k - ACC_ACROSS_UNROLL >= k0; k -= ACC_ACROSS_UNROLL) {
+#pragma unroll
+      for (int u = 0; u < ACC_ACROSS_UNROLL; ++u) x[u] = get(base + k - 1 - u);
+#pragma unroll
+      for (int u = 0; u < ACC_ACROSS_UNROLL; ++u) acc = f(x[u], acc);
+    }
+    for (; k > k0; --k) acc = f(get(base + k - 1), acc);
+#else
+    T acc = get(base + k0);
+    Int64 k = k0 + 1;
+    for (; k + ACC_ACROSS_UNROLL <= k1; k += ACC_ACROSS_UNROLL) {
+#pragma unroll
+      for (int u = 0; u < ACC_ACROSS_UNROLL; ++u) x[u] = get(base + k + u);
+#pragma unroll
+      for (int u = 0; u < ACC_ACROSS_UNROLL; ++u) acc = f(acc, x[u]);
+    }
+    for (; k < k1; ++k) acc = f(acc, get(base + k));
+#endif
+    if (split > 1) {
+      part[row * split + p] = acc;
+      part_ok[row * split + p] = 1;
+    } else {
+#if ACC_HAS_SEED && !ACC_FOLD_RIGHT
+      ACC_PUT(arrOut, row, f(acc, seed));                  /* ((x0 (+) x1) (+) ... x_last) (+) z */
+#else
+      ACC_PUT(arrOut, row, acc);
+#endif
+    }
+  }
+}
 #endif /* ACC_SEG_UNIFORM */
 
 /* ---- long segments: a team of lanes per segment ---------------------------

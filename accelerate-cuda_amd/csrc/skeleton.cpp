@@ -539,6 +539,7 @@ int make_spec(const acc_skel_desc *d, const TuningPtr &tuning, SkelSpec *sp)
   sp->map_tile_block = std::max(1, std::min(tune("map.tile_block", 4), 8));
   sp->map_tiled = (d->flags & ACC_FLAG_TILED) != 0 && d->out_rank >= 2 &&
                   (d->kind == ACC_SKEL_MAP || d->kind == ACC_SKEL_GENERATE || d->kind == ACC_SKEL_TRANSFORM) && tune("map.tiled", 1) != 0;
+  sp->fold_across = (d->flags & ACC_FLAG_TILED) != 0 && d->out_rank >= 1 && (d->kind == ACC_SKEL_FOLD || d->kind == ACC_SKEL_FOLD1);
   sp->out_rank = d->out_rank;
   if (sp->out_rank < 0 || sp->out_rank > ACC_MAX_RANK) return fail(ACC_ERR_INVALID, "bad out_rank %d", d->out_rank);
   for (int k = 0; k < d->n_env; ++k) {
@@ -929,6 +930,13 @@ int acc_skel_s::ensure_variant(int v)
       (void)hipModuleUnload(var.module);
       var.module = nullptr;
       return acc::fail_hip(e, ("hipModuleGetFunction(" + rows + ")").c_str());
+    }
+    const std::string across = entry_name + "_across";
+    e = hipModuleGetFunction(&var.fn_across, var.module, across.c_str());
+    if (e != hipSuccess) {
+      (void)hipModuleUnload(var.module);
+      var.module = nullptr;
+      return acc::fail_hip(e, ("hipModuleGetFunction(" + across + ")").c_str());
     }
   }
   (void)hipFuncGetAttribute(&var.num_regs, HIP_FUNC_ATTRIBUTE_NUM_REGS, var.fn);

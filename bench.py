@@ -788,6 +788,21 @@ def main():
             assert np.array_equal(out_.get(), lens.astype(np.float32)), "segmented sums mismatch"
             del xv_, do_, out_
             seg_s.destroy()
+        # sums down the columns of a matrix, written as the fold of its transpose: the rows that the fold sees lie
+        # across memory -- teams of lanes along them (no flag) against a lane a row (ACC_FLAG_TILED)
+        for shape in ((4096, 4096), (1 << 16, 256)):
+            mat = np.ones(shape, np.float32)
+            src, dst = ctx.array(mat), ctx.empty(shape[1], np.float32)
+            se, dd = envs(src), dst.desc()
+            ext = (C.c_int64 * 2)(shape[1], shape[0])
+            for name, flags in (("teams of lanes", 0), ("a lane a row (ACC_FLAG_TILED)", A.FLAG_TILED)):
+                cs = ctx.skeleton(A.SKEL_FOLD, "float", env=[(2, "float")], out_rank=1, flags=flags, combine="x + y", seed="0.0f",
+                                  get="arrIn0_0[(ix % shIn0_1) * shIn0_0 + ix / shIn0_1]")
+                one("fold (+) of the transpose of %d x %d Float32, %s" % (shape + (name,)),
+                    lambda: A.check(L.acc_exec_fold(cs.handle, se, 2, ext, C.byref(dd), stream)), 4 * mat.size)
+                assert np.array_equal(dst.get(), mat.sum(axis=0)), "column sums mismatch"
+                cs.destroy()
+            del src, dst
         sk["shapes"] = shapes
 
     if headline is None:     # --only without scan: report whatever ran first

@@ -284,7 +284,13 @@ enum { ACC_BOUNDARY_CLAMP = 0, ACC_BOUNDARY_MIRROR = 1, ACC_BOUNDARY_WRAP = 2, A
 #define ACC_FLAG_TILED        8u  /* map family, out_rank >= 2: produce the result in square tiles of its two innermost
                                      dimensions instead of runs of the innermost one, for element functions that read
                                      their sources across rows (a transposing backpermute: IndexSpace.hs:96-141 reads
-                                     one element of every source row per run); the results are the same */
+                                     one element of every source row per run); the results are the same.
+                                     fold / fold1 along the innermost dimension (out_rank >= 1): the same statement
+                                     about the element function -- where the ROW of the folded array moves by one, it
+                                     reads neighbouring addresses (the fold of a transposed matrix, a matrix product
+                                     written as a fold over replicated operands) -- and a lane then takes a row,
+                                     neighbouring rows in neighbouring lanes, instead of a team of lanes along a row;
+                                     the operands meet in index order as always */
 #define ACC_FLAG_GUARDED      4u  /* the instance may run under an acc_guard (see acc_guard_create): its kernels take the
                                      guard's address as one more, last, parameter and do nothing once the guard is down */
 

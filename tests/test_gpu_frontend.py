@@ -813,3 +813,39 @@ def test_pagerank_on_a_graph_with_hubs(acc):
         assert np.all(np.abs(rank - ref) <= 1e-4 * ref.max()), k
         if k == 11:
             time.sleep(1.0)                 # (the variants with the table are compiled by now: the second half takes them)
+
+
+def test_column_sums_and_a_matrix_product_written_as_folds(acc):
+    """`fold (+) 0 (transpose m)` and the matrix product of the reference's examples, `fold (+) 0 (zipWith (*)
+    (replicate (Z :. All :. n :. All) a) (replicate (Z :. m :. All :. All) (transpose b)))`: the fold's rows lie
+    across memory, which the front end knows and says (ACC_FLAG_TILED), so a lane takes a row.  One kernel each,
+    integer results exact; a transpose of a transpose reads along the rows again."""
+    rng = np.random.default_rng(31)
+    cx = acc.Context.default()
+    m = rng.integers(-50, 50, (3001, 257)).astype(np.int32)
+    t = acc.transpose(acc.use(m))
+    assert t.across and not acc.transpose(t).across
+    before = len(cx.skeletons)
+    got = acc.run(acc.fold(add, 0, t))
+    assert len(cx.skeletons) == before + 1
+    assert np.array_equal(got, m.sum(axis=0, dtype=np.int32))
+    assert np.array_equal(acc.run(acc.fold(add, 0, acc.transpose(t))), m.sum(axis=1, dtype=np.int32))
+    mm, kk, nn = 70, 333, 129
+    a = rng.integers(-9, 9, (mm, kk)).astype(np.int32)
+    b = rng.integers(-9, 9, (kk, nn)).astype(np.int32)
+
+    def mmult(x, y):
+        xr = acc.replicate((acc.All, nn, acc.All), x)
+        yr = acc.replicate((mm, acc.All, acc.All), acc.transpose(y))
+        assert yr.across and not xr.across
+        return acc.fold(add, 0, acc.zipWith(lambda p, q: p * q, xr, yr))
+    before = len(cx.skeletons)
+    got = acc.run1(mmult)(a, b)
+    assert len(cx.skeletons) == before + 1
+    assert np.array_equal(got, a @ b)
+    fa, fb = a.astype(np.float32) / 8, b.astype(np.float32) / 4            # exact in Float32 whatever the order
+    def mmultf(x, y):
+        xr = acc.replicate((acc.All, nn, acc.All), x)
+        yr = acc.replicate((mm, acc.All, acc.All), acc.transpose(y))
+        return acc.fold(add, 0.0, acc.zipWith(lambda p, q: p * q, xr, yr))
+    assert np.array_equal(acc.run1(mmultf)(fa, fb), fa @ fb)

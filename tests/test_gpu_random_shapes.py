@@ -551,3 +551,75 @@ def test_permute_of_sorted_and_clustered_keys(A, ctx):
         out = ctx.empty(bins, np.int32)
         count.permute([ctx.array(keys)], n, ctx.array(np.full(bins, 2, np.int32)), out)
         assert np.array_equal(out.get(), np.bincount(keys, minlength=bins) + 2), ("count", how, n, bins)
+
+
+def test_fold_of_rows_that_lie_across_memory(A, ctx):
+    """`ACC_FLAG_TILED` on a fold along the innermost dimension: the element function reads a matrix down its columns
+    (the fold of a transposed matrix), and a lane takes a row.  Many short rows, rows just beyond what the
+    one-lane-per-short-row entry takes, a few long rows (cut into pieces that a second launch joins) and one row;
+    sums of integers, a non-commutative operator in both associations, fold1, pairs and Float64 -- and the same
+    through `fold.across=1` on a plain row-major source, which takes the same kernels."""
+    rng = np.random.default_rng(4711)
+    aff = """
+__device__ __forceinline__ Word32 affine16(Word32 x, Word32 y) {
+  Word32 a1 = x >> 16, b1 = x & 0xffffu, a2 = y >> 16, b2 = y & 0xffffu;
+  return (((a1 * a2) & 0xffffu) << 16) | ((a1 * b2 + b1) & 0xffffu);
+}
+"""
+    def chain(vals):
+        acc = int(vals[0])
+        for v in vals[1:]:
+            acc = pyref.affine16(acc, int(v))
+        return acc
+
+    # (h, w): the matrix in memory; the fold sees its transpose, w rows of h elements (the extents are read from the
+    # source's descriptor, so that one instance serves every shape)
+    across = "arrIn0_0[(ix % shIn0_1) * shIn0_0 + ix / shIn0_1]"
+    fs = ctx.skeleton(A.SKEL_FOLD, "Int32", env=[(2, "Int32")], out_rank=1, get=across, combine="x + y", seed="5", flags=A.FLAG_TILED)
+    fp = ctx.skeleton(A.SKEL_FOLD, "Int64, Int32", env=[(2, "Int32")], out_rank=1, get="acc_elt{(Int64)%s, 1}" % across,
+                      combine="acc_elt{x.a1 + y.a1, x.a0 + y.a0}", seed="acc_elt{0, 0}", flags=A.FLAG_TILED)
+    fd = ctx.skeleton(A.SKEL_FOLD1, "double", env=[(2, "double")], out_rank=1, get=across, combine="x + y", flags=A.FLAG_TILED)
+    affine = [(flags, seed, ctx.skeleton(A.SKEL_FOLD if seed else A.SKEL_FOLD1, "Word32", env=[(2, "Word32")], out_rank=1, get=across,
+                                         combine="affine16(x, y)", seed=seed, preamble=aff, flags=flags))
+              for flags, seed in ((A.FLAG_TILED, "0x00030005u"), (A.FLAG_TILED | A.FLAG_FOLD_RIGHT, "0x00030005u"), (A.FLAG_TILED, None),
+                                  (A.FLAG_TILED | A.FLAG_FOLD_RIGHT, None))]
+    for h, w in ((17, 70000), (40, 3000), (1000, 999), (5000, 33), (70000, 5), (300000, 1), (1, 4000), (129, 257)):
+        say("fold across", h, w)
+        m = rng.integers(-9, 9, (h, w)).astype(np.int32)
+        dm = ctx.array(m)
+        out = ctx.array(np.full(w + 2, 77, np.int32))
+        fs.fold([dm], (w, h), out.desc(shape=(w,)))
+        got = out.get()
+        assert np.array_equal(got[:w], m.sum(axis=0, dtype=np.int32) + 5), (h, w)
+        assert np.array_equal(got[w:], [77, 77]), (h, w)
+        # pairs: (sum as Int64, count)
+        pair = ctx.empty_tuple(w, [np.int64, np.int32])
+        fp.fold([dm], (w, h), pair)
+        s_, c_ = pair.get()
+        assert np.array_equal(s_, m.sum(axis=0, dtype=np.int64)) and np.array_equal(c_, np.full(w, h, np.int32)), (h, w)
+        # Float64, small integers: exact
+        md = ctx.array(m.astype(np.float64))
+        od = ctx.empty(w, np.float64)
+        fd.fold([md], (w, h), od)
+        assert np.array_equal(od.get(), m.sum(axis=0).astype(np.float64)), (h, w)
+        # a non-commutative operator, both associations, with and without a seed
+        u = rng.integers(0, 2**32, (h, w), dtype=np.uint64).astype(np.uint32)
+        du = ctx.array(u)
+        picks = sorted(set([0, w - 1, w // 2] + [int(c) for c in rng.integers(0, w, 6)]))
+        plain = {c: chain(u[:, c]) for c in picks}
+        for flags, seed, fa in affine:
+            oa = ctx.empty(w, np.uint32)
+            fa.fold([du], (w, h), oa)
+            ga = oa.get()
+            for c in picks:
+                want = pyref.affine16(plain[c], 0x00030005) if seed else plain[c]
+                assert int(ga[c]) == want, ("affine", h, w, c, flags, seed)
+    # a plain row-major source through the same kernels
+    with A.tuning("fold.across=1", ctx):
+        fs = ctx.skeleton(A.SKEL_FOLD, "Int32", env=[(2, "Int32")], out_rank=1, get="arrIn0_0[ix]", combine="x + y", seed="0")
+    for rows, inner in ((3000, 40), (7, 100000), (100000, 17)):
+        say("fold across, forced", rows, inner)
+        m = rng.integers(-9, 9, (rows, inner)).astype(np.int32)
+        out = ctx.empty(rows, np.int32)
+        fs.fold([ctx.array(m)], (rows, inner), out)
+        assert np.array_equal(out.get(), m.sum(axis=1, dtype=np.int32)), (rows, inner)
