@@ -716,6 +716,15 @@ def unit(value, ctype, context=None):
 
 def _unlinear(ix, shape):
     """multi-index (outermost first) of a linear index, as Exps; extents are literals, so the divisions are by constants"""
+    if ix.term == "ix" and getattr(_building, "rows_of", None) == tuple(shape) and len(shape) >= 2:
+        # inside a fold along the innermost dimension that gives every row to a lane: the row and the place within
+        # it are names of the kernel, and what depends on the row alone leaves the lane's loop
+        return _unlinear(Exp("Int64", "acc_row"), shape[:-1]) + (Exp("Int64", "acc_col"),)
+    made_of = getattr(ix, "made_of", None)
+    if made_of is not None and made_of[1] == tuple(shape):
+        # the linear index of this very multi-index (an index function applied to the result of another, as where a
+        # transposed array is replicated): taking it apart again gives the multi-index back, without a division
+        return made_of[0]
     out, rest = [], ix
     for d in range(len(shape) - 1, -1, -1):
         ext = constant(shape[d], "Int64")
@@ -737,6 +746,9 @@ def _linear(idx, shape):
     acc_ = idx[0]
     for d in range(1, len(shape)):
         acc_ = acc_ * constant(shape[d], "Int64") + idx[d]
+    if acc_ is idx[0]:
+        acc_ = Exp(acc_.ctype, acc_.term, binds=acc_.binds)     # (an object of its own to hang the note on)
+    acc_.made_of = (tuple(idx), tuple(shape))
     return acc_
 
 
@@ -822,8 +834,12 @@ def _fold(f, z, a, seedless, context):
     cx = _context(context, a)
     # an empty outer extent counts as 1 in the result of a seeded fold (Execute.hs:287-289)
     out_shape = a.shape[:-1] if seedless else tuple(max(1, d) for d in a.shape[:-1])
-    arrays, sig, fr = _assemble(get=a.stream().text, combine=_combine(f, a.ctype).text,
-                                seed=None if seedless else Exp.of(z, a.ctype).text)
+    _building.rows_of = tuple(a.shape) if a.across else None
+    try:
+        get = a.stream().text
+    finally:
+        _building.rows_of = None
+    arrays, sig, fr = _assemble(get=get, combine=_combine(f, a.ctype).text, seed=None if seedless else Exp.of(z, a.ctype).text)
     # rows that lie across memory (the fold of a transposed matrix, of a product of replicated operands): a lane a row
     sk = cx.skeleton(A.SKEL_FOLD1 if seedless else A.SKEL_FOLD, _elt(a.ctype), sig, out_rank=len(out_shape),
                      flags=A.FLAG_TILED if a.across and len(out_shape) >= 1 else 0, **fr)

@@ -43,7 +43,13 @@ static_assert(ACC_CHUNK % (ACC_BLOCK * ACC_VEC) == 0, "chunk must be a whole num
 #define ACC_SEG_PARAMS const Int64 shIn_1, const Int64 shIn_0
 #define ACC_SEG_TOTAL (shIn_1 * shIn_0)
 #define ACC_SEG_AT(s) ((Int64)(s) * shIn_0)
+/* The element function of such a fold may name acc_row and acc_col, the row of the folded array and the place within
+ * it (ix == acc_row * row length + acc_col).  The entries that give a row to a lane know both as they stand; the
+ * others divide, where the names are used at all. */
+#define ACC_GET_AT_IX [&](const Int64 ix) -> T { const Int64 acc_row = ix / shIn_0, acc_col = ix - acc_row * shIn_0; (void)acc_row; (void)acc_col; return (ACC_GET(ix)); }
+#define ACC_GET_AT_ROW_COL [&](const Int64 acc_row, const Int64 acc_col) -> T { const Int64 ix = acc_row * shIn_0 + acc_col; (void)ix; return (ACC_GET(ix)); }
 #else
+#define ACC_GET_AT_IX [&](const Int64 ix) -> T { return (ACC_GET(ix)); }
 #if ACC_HAS_SEED
 #define ACC_FOLDSEG_ENTRY foldSeg
 #else
@@ -190,7 +196,7 @@ ACC_FOLDSEG_ENTRY(ACC_ENV_PARAMS
   __shared__ int s_owner, s_from, s_to;
   __shared__ acc_opt<T> s_part[ACC_BLOCK / ACC_WAVE];
 
-  auto get = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
+  auto get = ACC_GET_AT_IX;
   auto f   = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
   auto lf  = acc_lift<T>(f);
 
@@ -464,7 +470,7 @@ ACC_DEV void acc_fold_rows(const Int64 nseg, G get, F f, const T &seed, P put)
 #pragma unroll
         for (int r = 0; r < R; ++r)
 #pragma unroll
-          for (int k = 0; k < W; ++k) x[u][r][k] = get((b0 + ((Int64)u * ACC_BLOCK + threadIdx.x) * R + r) * W + k);
+          for (int k = 0; k < W; ++k) x[u][r][k] = get(b0 + ((Int64)u * ACC_BLOCK + threadIdx.x) * R + r, k);
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -478,7 +484,7 @@ ACC_DEV void acc_fold_rows(const Int64 nseg, G get, F f, const T &seed, P put)
           if (seg < nseg) {
             T x[W];
 #pragma unroll
-            for (int k = 0; k < W; ++k) x[k] = get(seg * W + k);
+            for (int k = 0; k < W; ++k) x[k] = get(seg, k);
             put(seg, acc_fold_row<W, T>(x, f, seed));
           }
         }
@@ -496,7 +502,7 @@ ACC_FS_CAT_(ACC_FOLDSEG_ENTRY, _rows)(ACC_ENV_PARAMS
   ACC_GUARD_CHECK
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
-  auto get = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
+  auto get = ACC_GET_AT_ROW_COL;
   auto f   = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
   auto put = [&](const Int64 seg, const T &v) { ACC_PUT(arrOut, seg, v); };       /* written once, not read again here */
   (void)shIn_1;
@@ -533,7 +539,7 @@ ACC_FS_CAT_(ACC_FOLDSEG_ENTRY, _across)(ACC_ENV_PARAMS
   ACC_GUARD_CHECK
   typedef ACC_ELT T;
   ACC_ENV_ASSUME
-  auto get = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
+  auto get = ACC_GET_AT_ROW_COL;
   auto f   = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
   (void)shIn_1;
   const Int64 rows = shOut_0, len = shIn_0;
@@ -545,35 +551,34 @@ ACC_FS_CAT_(ACC_FOLDSEG_ENTRY, _across)(ACC_ENV_PARAMS
       if (split > 1) part_ok[row * split + p] = 0;
       continue;
     }
-    const Int64 base = row * len;
     T x[ACC_ACROSS_UNROLL];
 #if ACC_HAS_SEED
     const T seed = (ACC_SEED);
 #endif
 #if ACC_FOLD_RIGHT
     /* x0 (+) (x1 (+) (... (x_last (+) z))), as the other entries associate a row */
-    T acc = get(base + k1 - 1);
+    T acc = get(row, k1 - 1);
 #if ACC_HAS_SEED
     if (split == 1) acc = f(acc, seed);
 #endif
     Int64 k = k1 - 1;
     for (; k - ACC_ACROSS_UNROLL >= k0; k -= ACC_ACROSS_UNROLL) {
 #pragma unroll
-      for (int u = 0; u < ACC_ACROSS_UNROLL; ++u) x[u] = get(base + k - 1 - u);
+      for (int u = 0; u < ACC_ACROSS_UNROLL; ++u) x[u] = get(row, k - 1 - u);
 #pragma unroll
       for (int u = 0; u < ACC_ACROSS_UNROLL; ++u) acc = f(x[u], acc);
     }
-    for (; k > k0; --k) acc = f(get(base + k - 1), acc);
+    for (; k > k0; --k) acc = f(get(row, k - 1), acc);
 #else
-    T acc = get(base + k0);
+    T acc = get(row, k0);
     Int64 k = k0 + 1;
     for (; k + ACC_ACROSS_UNROLL <= k1; k += ACC_ACROSS_UNROLL) {
 #pragma unroll
-      for (int u = 0; u < ACC_ACROSS_UNROLL; ++u) x[u] = get(base + k + u);
+      for (int u = 0; u < ACC_ACROSS_UNROLL; ++u) x[u] = get(row, k + u);
 #pragma unroll
       for (int u = 0; u < ACC_ACROSS_UNROLL; ++u) acc = f(acc, x[u]);
     }
-    for (; k < k1; ++k) acc = f(acc, get(base + k));
+    for (; k < k1; ++k) acc = f(acc, get(row, k));
 #endif
     if (split > 1) {
       part[row * split + p] = acc;
@@ -632,7 +637,7 @@ ACC_FS_CAT(ACC_FOLDSEG_ENTRY, _team)(ACC_ENV_PARAMS
   __shared__ int s_entered;
 #endif
 
-  auto get = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
+  auto get = ACC_GET_AT_IX;
   auto f   = [&](const T &x, const T &y) -> T { return (ACC_COMBINE(x, y)); };
   auto lf  = acc_lift<T>(f);
 

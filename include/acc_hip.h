@@ -290,7 +290,11 @@ enum { ACC_BOUNDARY_CLAMP = 0, ACC_BOUNDARY_MIRROR = 1, ACC_BOUNDARY_WRAP = 2, A
                                      reads neighbouring addresses (the fold of a transposed matrix, a matrix product
                                      written as a fold over replicated operands) -- and a lane then takes a row,
                                      neighbouring rows in neighbouring lanes, instead of a team of lanes along a row;
-                                     the operands meet in index order as always */
+                                     the operands meet in index order as always.  (The element function of any fold
+                                     with out_rank >= 1 may name `acc_row` and `acc_col`, the row of the folded array
+                                     and the place within it: ix == acc_row * row length + acc_col.  Kernels that give
+                                     a row to a lane know both without a division, and what depends on acc_row alone
+                                     leaves the lane's loop.) */
 #define ACC_FLAG_GUARDED      4u  /* the instance may run under an acc_guard (see acc_guard_create): its kernels take the
                                      guard's address as one more, last, parameter and do nothing once the guard is down */
 

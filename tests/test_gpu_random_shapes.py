@@ -557,8 +557,9 @@ def test_fold_of_rows_that_lie_across_memory(A, ctx):
     """`ACC_FLAG_TILED` on a fold along the innermost dimension: the element function reads a matrix down its columns
     (the fold of a transposed matrix), and a lane takes a row.  Many short rows, rows just beyond what the
     one-lane-per-short-row entry takes, a few long rows (cut into pieces that a second launch joins) and one row;
-    sums of integers, a non-commutative operator in both associations, fold1, pairs and Float64 -- and the same
-    through `fold.across=1` on a plain row-major source, which takes the same kernels."""
+    sums of integers, a non-commutative operator in both associations, fold1, pairs and Float64; the element function
+    written over the kernel's names `acc_row` and `acc_col`; and `fold.across=1` on a plain row-major source, which
+    takes the same kernels."""
     rng = np.random.default_rng(4711)
     aff = """
 __device__ __forceinline__ Word32 affine16(Word32 x, Word32 y) {
@@ -583,15 +584,21 @@ __device__ __forceinline__ Word32 affine16(Word32 x, Word32 y) {
                                          combine="affine16(x, y)", seed=seed, preamble=aff, flags=flags))
               for flags, seed in ((A.FLAG_TILED, "0x00030005u"), (A.FLAG_TILED | A.FLAG_FOLD_RIGHT, "0x00030005u"), (A.FLAG_TILED, None),
                                   (A.FLAG_TILED | A.FLAG_FOLD_RIGHT, None))]
-    for h, w in ((17, 70000), (40, 3000), (1000, 999), (5000, 33), (70000, 5), (300000, 1), (1, 4000), (129, 257)):
+    # the same element function written with the kernel's names for the row and the place within it, in an instance
+    # that gives rows to lanes (which knows both) and in one that does not (which divides)
+    by_name = "arrIn0_0[acc_col * shIn0_0 + acc_row]"
+    named = [ctx.skeleton(A.SKEL_FOLD, "Int32", env=[(2, "Int32")], out_rank=1, get=by_name, combine="x + y", seed="5", flags=flags)
+             for flags in (A.FLAG_TILED, 0)]
+    for h, w in ((17, 70000), (40, 3000), (1000, 999), (5000, 33), (70000, 5), (300000, 1), (1, 4000), (129, 257), (5, 1000), (16, 300)):
         say("fold across", h, w)
         m = rng.integers(-9, 9, (h, w)).astype(np.int32)
         dm = ctx.array(m)
-        out = ctx.array(np.full(w + 2, 77, np.int32))
-        fs.fold([dm], (w, h), out.desc(shape=(w,)))
-        got = out.get()
-        assert np.array_equal(got[:w], m.sum(axis=0, dtype=np.int32) + 5), (h, w)
-        assert np.array_equal(got[w:], [77, 77]), (h, w)
+        for sk_ in [fs] + named:
+            out = ctx.array(np.full(w + 2, 77, np.int32))
+            sk_.fold([dm], (w, h), out.desc(shape=(w,)))
+            got = out.get()
+            assert np.array_equal(got[:w], m.sum(axis=0, dtype=np.int32) + 5), (h, w)
+            assert np.array_equal(got[w:], [77, 77]), (h, w)
         # pairs: (sum as Int64, count)
         pair = ctx.empty_tuple(w, [np.int64, np.int32])
         fp.fold([dm], (w, h), pair)
