@@ -795,9 +795,11 @@ def main():
             src, dst = ctx.array(mat), ctx.empty(shape[1], np.float32)
             se, dd = envs(src), dst.desc()
             ext = (C.c_int64 * 2)(shape[1], shape[0])
-            for name, flags in (("teams of lanes", 0), ("a lane a row (ACC_FLAG_TILED)", A.FLAG_TILED)):
-                cs = ctx.skeleton(A.SKEL_FOLD, "float", env=[(2, "float")], out_rank=1, flags=flags, combine="x + y", seed="0.0f",
-                                  get="arrIn0_0[(ix % shIn0_1) * shIn0_0 + ix / shIn0_1]")
+            # (the index as a code generator writes it: the extents as literals; over the kernel's names for the row
+            # and the place within it where a lane takes a row)
+            for name, flags, text in (("teams of lanes", 0, "arrIn0_0[(ix %% %dLL) * %dLL + ix / %dLL]" % (shape[0], shape[1], shape[0])),
+                                      ("a lane a row (ACC_FLAG_TILED)", A.FLAG_TILED, "arrIn0_0[acc_col * %dLL + acc_row]" % shape[1])):
+                cs = ctx.skeleton(A.SKEL_FOLD, "float", env=[(2, "float")], out_rank=1, flags=flags, combine="x + y", seed="0.0f", get=text)
                 one("fold (+) of the transpose of %d x %d Float32, %s" % (shape + (name,)),
                     lambda: A.check(L.acc_exec_fold(cs.handle, se, 2, ext, C.byref(dd), stream)), 4 * mat.size)
                 assert np.array_equal(dst.get(), mat.sum(axis=0)), "column sums mismatch"
