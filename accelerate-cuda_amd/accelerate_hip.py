@@ -784,16 +784,52 @@ def generate(shape, f):
     return Acc(shape, t, at=lambda ix: Exp.of(f(*_unlinear(ix, shape))))
 
 
-def backpermute(shape, p, a, across=False):
+def _steps_of(p, shape, src_shape):
+    """how far `p` moves through the source (in elements of its row-major order) where the result's index moves by
+    one along the innermost and along the second innermost dimension: found by applying `p` to plain numbers, which
+    an index function made of arithmetic alone accepts.  None where it does not, or where the result is too small
+    to take a step."""
+    if len(shape) < 2 or shape[-1] < 2 or shape[-2] < 2:
+        return None
+
+    def place(idx):
+        r = p(*idx)
+        r = tuple(r) if isinstance(r, (tuple, list)) else (r,)
+        if len(r) != len(src_shape) or not all(isinstance(v, numbers.Integral) for v in r):
+            raise TypeError
+        at = 0
+        for v, ext in zip(r, src_shape):
+            at = at * ext + int(v)
+        return at
+    try:
+        zero = [0] * len(shape)
+        here = place(zero)
+        return place(zero[:-1] + [1]) - here, place(zero[:-2] + [1, 0]) - here
+    except Exception:
+        return None
+
+
+def backpermute(shape, p, a, across=None):
     """result[i] = a[p(i)]: p takes the result's multi-index and returns a multi-index of `a`.  `across`: p walks
-    down a column of `a` where the result's index moves along a row (see transpose)"""
+    down a column of `a` where the result's index moves along a row (see transpose); where it is not given, an index
+    function made of arithmetic alone is asked by applying it to numbers."""
     shape = (shape,) if isinstance(shape, numbers.Integral) else tuple(shape)
+    if across is None:
+        steps = _steps_of(p, shape, a.shape)
+        if steps is None:
+            across = False
+        elif abs(steps[0]) == 1:
+            across = a.across              # along the rows of `a`: what `a` reads across, the result does
+        elif abs(steps[1]) == 1 and steps[0] != 0:
+            across = not a.across          # down the columns of `a`
+        else:
+            across = False
     return Acc(shape, a.ctype, at=lambda ix: a.index(_linear(p(*_unlinear(ix, shape)), a.shape)), across=across)
 
 
 def transpose(a):
     h, w = a.shape
-    return backpermute((w, h), lambda y, x: (x, y), a, across=not a.across)
+    return backpermute((w, h), lambda y, x: (x, y), a)
 
 
 def zip_(a, b):
@@ -1240,8 +1276,7 @@ def replicate(spec, a):
     dims = iter(a.shape)
     shape = tuple(next(dims) if (x is All or x == All) else int(x) for x in spec)
     keep = [k for k, x in enumerate(spec) if x is All or x == All]
-    # (the innermost dimension of the result is the innermost one of `a`: what `a` reads across, the result does)
-    return backpermute(shape, lambda *ix: tuple(ix[k] for k in keep), a, across=a.across and keep[-1] == len(spec) - 1)
+    return backpermute(shape, lambda *ix: tuple(ix[k] for k in keep), a)
 
 
 def slice_(a, spec):

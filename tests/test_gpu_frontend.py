@@ -830,6 +830,13 @@ def test_column_sums_and_a_matrix_product_written_as_folds(acc):
     assert len(cx.skeletons) == before + 1
     assert np.array_equal(got, m.sum(axis=0, dtype=np.int32))
     assert np.array_equal(acc.run(acc.fold(add, 0, acc.transpose(t))), m.sum(axis=1, dtype=np.int32))
+    # an index function of the user's own that exchanges the two innermost dimensions of a rank-3 array: found out by
+    # applying it to numbers
+    c = rng.integers(-50, 50, (5, 60, 70)).astype(np.int32)
+    swapped = acc.backpermute((5, 70, 60), lambda i, k, j: (i, j, k), acc.use(c))
+    assert swapped.across and not acc.backpermute((60, 5, 70), lambda j, i, k: (i, j, k), acc.use(c)).across
+    assert np.array_equal(acc.run(swapped), c.transpose(0, 2, 1))
+    assert np.array_equal(acc.run(acc.fold(add, 0, swapped)), c.sum(axis=1, dtype=np.int32))
     mm, kk, nn = 70, 333, 129
     a = rng.integers(-9, 9, (mm, kk)).astype(np.int32)
     b = rng.integers(-9, 9, (kk, nn)).astype(np.int32)
