@@ -853,6 +853,35 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
                       ntarget >= s->knobs.permute_fp_tables_from && ntarget <= s->knobs.permute_fp_tables_to;
   const bool generic_few = !s->spec.permute_locked && (s->spec.combine_hint == ACC_COMBINE_GENERIC || fp_add) && lds_table_fits &&
                            s->knobs.permute_generic_lds != 0;
+  if (s->spec.permute_locked && s->spec.permute_replace && n_src <= (int64_t)0xffffffffLL) {
+    // `permute const` of an element that no single store covers: nothing is read or locked.  A scalar of one or two
+    // bytes is stored; of a tuple the source whose index stays in the target's word of a table wins, whole
+    // (skel_permute.h, permute_claim / permute_place).
+    ACC_TRY(plain_copy());
+    Args pargs;
+    bool al = true;
+    ACC_TRY(push_env(s, env, &pargs, &al));
+    push_out(*out, &pargs, &al);
+    pargs.i64(n_src);
+    const int pv = al ? 0 : 1;
+    ACC_TRY(s->ensure_variant(pv));
+    acc::ScratchRef wblk;
+    const bool tuple = s->ncomp() > 1;
+    if (tuple) ACC_TRY(s->ctx->scratch_acquire((size_t)ntarget * 4, st, acc::SCRATCH_FOLD, &wblk));
+    pargs.ptr(reinterpret_cast<uint64_t>(wblk.ptr));
+    const int64_t pgrid = acc_launch_grid(n_src, 256 * 4, s->ctx->props.multiProcessorCount, 32);
+    int prc = ACC_OK;
+    if (tuple) {
+      hipError_t ce = launch_kernel(s->variants[pv].fn_claim, static_cast<unsigned>(pgrid), 1, 1, 256, 1, 1, 0, st, pargs.data(), nullptr);
+      if (ce != hipSuccess) prc = acc::fail_hip(ce, "hipModuleLaunchKernel(permute_claim)");
+    }
+    if (prc == ACC_OK) {
+      hipError_t pe = launch_kernel(s->variants[pv].fn_place, static_cast<unsigned>(pgrid), 1, 1, 256, 1, 1, 0, st, pargs.data(), nullptr);
+      if (pe != hipSuccess) prc = acc::fail_hip(pe, "hipModuleLaunchKernel(permute_place)");
+    }
+    s->ctx->scratch_release(wblk, st);
+    return prc;
+  }
   if (s->spec.permute_locked || generic_few) {
     // elements no atomic covers: a lock per target (the reference's lock array, Execute.hs:402-405)
     ACC_TRY(plain_copy());

@@ -262,7 +262,7 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "#define ACC_OUT_PARAMS " << out_params(sp.out_rank, sp.elt_type) << "\n";
       o << "#define ACC_OUT_SIZE " << out_size(sp.out_rank) << "\n";
       o << "#define ACC_PERMUTATION(ix) " << sp.permutation << "\n";
-      o << "#define ACC_COMBINE_HINT " << sp.combine_hint << "\n";
+      o << "#define ACC_COMBINE_HINT " << (sp.permute_replace && !sp.permute_locked ? 7 : sp.combine_hint) << "\n";
       o << "#define ACC_PERMUTE_LOCKED " << (sp.permute_locked ? 1 : 0) << "\n";
       o << "#define ACC_PERMUTE_WINDOWS " << (sp.permute_windows ? 1 : 0) << "\n";
       o << "#define ACC_PERMUTE_NARROW " << (sp.permute_narrow ? 1 : 0) << "\n";
@@ -614,6 +614,16 @@ int make_spec(const acc_skel_desc *d, const TuningPtr &tuning, SkelSpec *sp)
       // no atomic read-modify-write covers a tuple or an element of another size than 4 or 8 bytes:
       // those go through a lock per target, as every permute does in the reference (IndexSpace.hs:285-303)
       sp->permute_locked = !sp->comp_types.empty() || (sp->elt_size != 4 && sp->elt_size != 8);
+      {
+        // `permute const`: the combination is the new value, whatever its spelling's blanks and brackets
+        std::string c = d->combine ? d->combine : "";
+        c.erase(std::remove_if(c.begin(), c.end(), [](unsigned char ch) { return std::isspace(ch) || ch == '(' || ch == ')'; }), c.end());
+        // (a tuple's spelling: its components, first to last)
+        std::string whole = "acc_elt{";
+        for (size_t k = sp->comp_types.size(); k-- > 0;) whole += "x.a" + std::to_string(k) + (k ? "," : "}");
+        sp->permute_replace = sp->combine_hint == ACC_COMBINE_GENERIC && (c == "x" || (!sp->comp_types.empty() && c == whole)) &&
+                              tune("permute.replace", 1) != 0;
+      }
       if (sp->permute_locked && sp->combine_hint != ACC_COMBINE_GENERIC)
         return fail(ACC_ERR_INVALID, "permute: combine_hint needs a 4- or 8-byte single-component element");
       if (sp->combine_hint >= ACC_COMBINE_AND && !is_integer_type(sp->elt_type))
@@ -911,6 +921,17 @@ int acc_skel_s::ensure_variant(int v)
       (void)hipModuleUnload(var.module);
       var.module = nullptr;
       return acc::fail_hip(e, ("hipModuleGetFunction(" + third + ")").c_str());
+    }
+  }
+  if (spec.kind == ACC_SKEL_PERMUTE && spec.permute_locked) {
+    // `permute const` without locks: see skel_permute.h
+    for (const char *name : {"permute_claim", "permute_place"}) {
+      e = hipModuleGetFunction(name[8] == 'c' ? &var.fn_claim : &var.fn_place, var.module, name);
+      if (e != hipSuccess) {
+        (void)hipModuleUnload(var.module);
+        var.module = nullptr;
+        return acc::fail_hip(e, (std::string("hipModuleGetFunction(") + name + ")").c_str());
+      }
     }
   }
   if ((spec.kind == ACC_SKEL_FOLDSEG || spec.kind == ACC_SKEL_FOLD1SEG) && spec.out_rank <= 1) {

@@ -50,6 +50,7 @@ struct SkelSpec {
   int merge_waves = 4;                  // permute of 16-bit counts: waves of a workgroup of permute_merge
   int chunk_long = 0;                   // segmented folds: the staged chunk of variants 2 and 3 (segments of 8 elements or more on average); 0: none
   bool fold_across = false;             // ACC_FLAG_TILED on a fold along the innermost dimension: neighbouring rows are neighbours in memory
+  bool permute_replace = false;         // permute whose combination is spelt `x` (the new value): plain stores
   bool map_tiled = false;               // ACC_FLAG_TILED on a map of rank 2 or more: tiles of 32 x 32 elements, a wave each
   int map_tile_block = 4;               // ... a lane's share of a tile: a block of that many elements either way
   bool guarded = false;                 // ACC_FLAG_GUARDED: every kernel takes the address of a loop's guard word last
@@ -71,6 +72,8 @@ struct Variant {
   hipFunction_t fn_finish = nullptr;   // second kernel: foldAll's _finish, permute's _merge / _join, the segmented fold's _team
   hipFunction_t fn_fill = nullptr;     // third kernel: permute's _fill (identity into the table rows), the segmented fold's _join
   hipFunction_t fn_rows = nullptr;     // fold along the innermost dimension: _rows, a lane per short row
+  hipFunction_t fn_claim = nullptr;    // a permute under locks: permute_claim and permute_place, for a combination that is the new value
+  hipFunction_t fn_place = nullptr;
   hipFunction_t fn_across = nullptr;   // fold along the innermost dimension: _across, a lane per row of any length
   hipFunction_t fn_sweep = nullptr;    // a segmented fold's variants 4-7: _sweep, the segments that were handed over;
                                        // its variants 0-3: _probe, a look at the segment lengths

@@ -805,6 +805,32 @@ def main():
                 assert np.array_equal(dst.get(), mat.sum(axis=0)), "column sums mismatch"
                 cs.destroy()
             del src, dst
+        # `permute const`, every target written once: the scatter of a stream compaction (half of the sources kept, in
+        # order) and of a stable sorting pass by a 4-bit digit; stores (as the knobs stand) against a read and a
+        # compare-and-swap an element (`permute.replace=0`)
+        nper = 1 << 24
+        rng_p = np.random.default_rng(9)
+        vals_p = rng_p.integers(0, 1 << 30, nper).astype(np.int32)
+        keep_p = rng_p.random(nper) < 0.5
+        places_p = np.where(keep_p, np.cumsum(keep_p) - keep_p, -1).astype(np.int32)
+        order_p = np.argsort(vals_p & 15, kind="stable")
+        dest_p = np.empty(nper, np.int32)
+        dest_p[order_p] = np.arange(nper, dtype=np.int32)
+        dv_p = ctx.array(vals_p)
+        for name, tgt, nt in (("a compaction, half of the sources kept", places_p, int(keep_p.sum())), ("a sorting pass by a 4-bit digit", dest_p, nper)):
+            dk_p, dfl_p, out_p = ctx.array(tgt), ctx.array(np.zeros(nt, np.int32)), ctx.empty(nt, np.int32)
+            pe, pd, po = envs(dk_p, dv_p), dfl_p.desc(), out_p.desc()
+            want_p = np.zeros(nt, np.int32)
+            want_p[tgt[tgt >= 0]] = vals_p[tgt >= 0]
+            for knobs in ("", "permute.replace=0"):
+                with A.tuning(knobs, ctx):
+                    pc = ctx.skeleton(A.SKEL_PERMUTE, "Int32", env=[I32, I32], out_rank=1, get="arrIn1_0[ix]", combine="x", permutation="(Int64)arrIn0_0[ix]")
+                one("permute const Int32, 2^24 sources, %s%s" % (name, ", " + knobs if knobs else ""),
+                    lambda: A.check(L.acc_exec_permute(pc.handle, pe, nper, C.byref(pd), C.byref(po), stream)), 8 * nper + 8 * nt)
+                assert np.array_equal(out_p.get(), want_p), "permute const mismatch"
+                pc.destroy()
+            del dk_p, dfl_p, out_p
+        del dv_p
         sk["shapes"] = shapes
 
     if headline is None:     # --only without scan: report whatever ran first

@@ -320,7 +320,12 @@ typedef struct acc_skel_desc {
   const char        *preamble;      /* file-scope declarations for the fragments, or NULL   */
   const char        *get;           /* delayed input / element function over `ix` (Int64 linear
                                        index); map family: value of out[ix].  Not used by stencil. */
-  const char        *combine;       /* over `x`, `y`: fold, foldSeg, scans, permute          */
+  const char        *combine;       /* over `x`, `y`: fold, foldSeg, scans, permute.  A permute
+                                       whose combination is spelt as its first operand alone -- `x`, or
+                                       `acc_elt{x.a<n-1>, ..., x.a0}` for a tuple: `permute const`, the
+                                       scatter of a compaction or of a sorting pass -- stores the new
+                                       values and reads and locks nothing; of several sources on one
+                                       target one wins whole */
   const char        *seed;          /* NULL for the seedless kinds                           */
   const char        *permutation;   /* permute: linear target index of source `ix`, or
                                        ACC_IGNORE (-1) to drop the element                   */

@@ -630,3 +630,88 @@ __device__ __forceinline__ Word32 affine16(Word32 x, Word32 y) {
         out = ctx.empty(rows, np.int32)
         fs.fold([ctx.array(m)], (rows, inner), out)
         assert np.array_equal(out.get(), m.sum(axis=1, dtype=np.int32)), (rows, inner)
+
+
+def test_permute_whose_combination_is_the_new_value(A, ctx):
+    """`permute const`: the scatter of a stream compaction (targets in order, half of the sources ignored), of a
+    stable sorting pass by a 4-bit digit and of a random permutation -- every target written once, so the result is
+    exact -- for elements of 4 and 8 bytes, spelt `x` and `(x)`; with several sources on a target the result holds
+    one of them whole; and the same through the compare-and-swap loop (`permute.replace=0`).  An instance whose
+    combination is spelt so stores and reads nothing."""
+    rng = np.random.default_rng(515)
+    n = 300007
+    keep = rng.random(n) < 0.5
+    places = np.where(keep, np.cumsum(keep) - keep, -1).astype(np.int32)
+    digit = rng.integers(0, 16, n)
+    order = np.argsort(digit, kind="stable")
+    dest = np.empty(n, np.int32)
+    dest[order] = np.arange(n, dtype=np.int32)
+    for knobs in ("", "permute.replace=0"):
+        for ctype, dt in (("Int32", np.int32), ("float", np.float32), ("Int64", np.int64), ("double", np.float64)):
+            for spelt in ("x", "( x )"):
+                if knobs and spelt != "x":
+                    continue
+                say("permute const", knobs or "-", ctype, repr(spelt))
+                with A.tuning(knobs, ctx):
+                    sk = ctx.skeleton(A.SKEL_PERMUTE, ctype, env=[(1, "Int32"), (1, ctype)], out_rank=1, get="arrIn1_0[ix]",
+                                      combine=spelt, permutation="(Int64)arrIn0_0[ix]")
+                vals = rng.integers(-10**6, 10**6, n).astype(dt)
+                dv = ctx.array(vals)
+                for tgt, nt in ((places, int(keep.sum())), (dest, n), (rng.permutation(n).astype(np.int32), n)):
+                    dfl = rng.integers(0, 100, nt + 2).astype(dt)
+                    out = ctx.array(np.full(nt + 2, 77, dt))
+                    dd = ctx.array(dfl)
+                    sk.permute([ctx.array(tgt), dv], n, View(dd.desc(shape=(nt,))), View(out.desc(shape=(nt,))))
+                    want = dfl[:nt].copy()
+                    m = tgt >= 0
+                    want[tgt[m]] = vals[m]
+                    got = out.get()
+                    assert np.array_equal(got[:nt], want) and np.all(got[nt:] == 77), (knobs, ctype, nt)
+                # eight sources a target: one of them, whole
+                many = (np.arange(n) // 8).astype(np.int32)
+                nt = int(many[-1]) + 1
+                wide = (vals.astype(np.int64) * 0x100000001).astype(dt) if dt == np.int64 else vals
+                out = ctx.empty(nt, dt)
+                sk.permute([ctx.array(many), ctx.array(wide)], n, ctx.array(np.zeros(nt, dt)), out)
+                got = out.get()
+                cand = np.full((nt, 8), wide[0], dt)
+                cand.reshape(-1)[:n] = wide
+                cand[-1, n - 8 * (nt - 1):] = wide[n - 1]
+                assert np.all((cand == got[:, None]).any(axis=1)), (knobs, ctype)
+    # pairs (components are arrays of their own: of several sources on a target one must win whole) and small scalars
+    for knobs in ("", "permute.replace=0"):
+        say("permute const, pairs and small scalars", knobs or "-")
+        with A.tuning(knobs, ctx):
+            sp = ctx.skeleton(A.SKEL_PERMUTE, "Int32, Int32", env=[(1, "Int32"), (1, "Int32")], out_rank=1,
+                              get="acc_elt{arrIn1_0[ix], (Int32)ix}", combine="acc_elt{x.a1, x.a0}", permutation="(Int64)arrIn0_0[ix]")
+            sb = ctx.skeleton(A.SKEL_PERMUTE, "Int8", env=[(1, "Int32"), (1, "Int32")], out_rank=1, get="(Int8)arrIn1_0[ix]",
+                              combine="x", permutation="(Int64)arrIn0_0[ix]")
+            sh = ctx.skeleton(A.SKEL_PERMUTE, "Word16", env=[(1, "Int32"), (1, "Int32")], out_rank=1, get="(Word16)arrIn1_0[ix]",
+                              combine="x", permutation="(Int64)arrIn0_0[ix]")
+        vals = rng.integers(-10**6, 10**6, n).astype(np.int32)
+        dv = ctx.array(vals)
+        for tgt, nt in ((places, int(keep.sum())), (dest, n)):
+            m = tgt >= 0
+            dk = ctx.array(tgt)
+            out = ctx.empty_tuple(nt, [np.int32, np.int32])
+            sp.permute([dk, dv], n, ctx.tuple_array(np.full(nt, 5, np.int32), np.full(nt, 6, np.int32)), out)
+            a1, a0 = out.get()
+            w1 = np.full(nt, 5, np.int32); w1[tgt[m]] = vals[m]
+            w0 = np.full(nt, 6, np.int32); w0[tgt[m]] = np.arange(n, dtype=np.int32)[m]
+            assert np.array_equal(a1, w1) and np.array_equal(a0, w0), (knobs, nt)
+            for sk_, dt in ((sb, np.int8), (sh, np.uint16)):
+                out = ctx.array(np.full(nt + 2, 77, dt))
+                dd = ctx.array(np.full(nt, 9, dt))
+                sk_.permute([dk, dv], n, dd, View(out.desc(shape=(nt,))))
+                w = np.full(nt, 9, dt); w[tgt[m]] = vals[m].astype(dt)
+                got = out.get()
+                assert np.array_equal(got[:nt], w) and np.all(got[nt:] == 77), (knobs, dt, nt)
+        many = (np.arange(n) // 8).astype(np.int32)
+        many[::1000] = -1                                # (some are ignored)
+        nt = n // 8 + 1
+        out = ctx.empty_tuple(nt, [np.int32, np.int32])
+        sp.permute([ctx.array(many), dv], n, ctx.tuple_array(np.zeros(nt, np.int32), np.full(nt, -1, np.int32)), out)
+        a1, a0 = out.get()
+        hit = a0 >= 0
+        assert hit.sum() >= nt - 1
+        assert np.array_equal(many[a0[hit]], np.arange(nt, dtype=np.int32)[hit]) and np.array_equal(vals[a0[hit]], a1[hit]), knobs
