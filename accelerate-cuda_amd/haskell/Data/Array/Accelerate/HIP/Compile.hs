@@ -204,7 +204,10 @@ compileOpenAcc guarded (Manifest pacc) =
       let (get, g0)  = codegenDelayed emptyGamma a
           (comb, g1) = codegenFun2 g0 f
           (seed, g2) = maybe (Nothing, g1) (\e -> let (s, g') = codegenExp g1 e in (Just s, g')) z
-      kernel kind g2 get (Just comb) seed Nothing =<< (rebuild <$> travF f <*> traverse travE z <*> travD a)
+          -- an operand that reads its source across the rows (`fold f z (transpose m)`): the rows the fold sees lie
+          -- across memory, and the kernel gives a row to a lane instead of a team of lanes (ACC_FLAG_TILED)
+          across     = if readsAcross a then accFlagTiled else 0
+      kernelWith across kind g2 get (Just comb) seed Nothing =<< (rebuild <$> travF f <*> traverse travE z <*> travD a)
 
     segmented kind f z a s = do
       let (get, g0)  = codegenDelayed emptyGamma a
@@ -342,6 +345,22 @@ exchangesInnermost (Lam (Body (IndexCons (IndexCons rest a) b)))
     outer IndexNil                              = True
     outer _                                     = False
 exchangesInnermost _ = False
+
+-- | a delayed array whose element at (sh :. y :. x) is a manifest array's element at (sh :. x :. y), whatever is done
+-- to the element afterwards: what fusion makes of `map f (transpose m)`
+readsAcross :: DelayedOpenAcc aenv (Array sh e) -> Bool
+readsAcross Delayed{ indexD = f } = across f
+  where
+    across :: DelayedOpenFun () aenv (sh -> e) -> Bool
+    across (Lam (Body b)) = reads b
+    across _              = False
+    reads :: DelayedOpenExp env aenv t -> Bool
+    reads (Index Manifest{} (IndexCons (IndexCons _ a) b))
+      | IndexHead (Var ZeroIdx)             <- a
+      , IndexHead (IndexTail (Var ZeroIdx)) <- b = True
+    reads (PrimApp _ x)                         = reads x
+    reads _                                     = False
+readsAcross _ = False
 
 -- | scalar code that stays on the host: the arrays it names are compiled, the expression is rebuilt around them
 -- (Compile.hs:237-300 `travE`)
