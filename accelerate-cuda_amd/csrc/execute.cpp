@@ -866,7 +866,7 @@ int acc_exec_permute(acc_skel s, const acc_array *env, int64_t n_src, const acc_
     const int pv = al ? 0 : 1;
     ACC_TRY(s->ensure_variant(pv));
     acc::ScratchRef wblk;
-    const bool tuple = s->ncomp() > 1;
+    const bool tuple = s->ncomp() > 1 || esz > 8;      // (what no single store of at most 8 bytes writes)
     if (tuple) ACC_TRY(s->ctx->scratch_acquire((size_t)ntarget * 4, st, acc::SCRATCH_FOLD, &wblk));
     pargs.ptr(reinterpret_cast<uint64_t>(wblk.ptr));
     const int64_t pgrid = acc_launch_grid(n_src, 256 * 4, s->ctx->props.multiProcessorCount, 32);
