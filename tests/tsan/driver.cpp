@@ -81,6 +81,11 @@ int main(int argc, char **argv)
   acc_skel fold = make(ctx, ACC_SKEL_FOLD, "Int32", "arrIn0_0[ix]", "x + y", "0", nullptr, 0, 0);
   acc_skel hist = make(ctx, ACC_SKEL_PERMUTE, "Int32", "1", "x + y", nullptr, "arrIn0_0[ix]", ACC_COMBINE_ADD, 0);
   acc_skel locked = make(ctx, ACC_SKEL_PERMUTE, "Int16", "(Int16)1", "(Int16)(x + y)", nullptr, "arrIn0_0[ix]", 0, 0);
+  // `permute const` (stores: a kernel of its own for the small element, the atomics template for the 4-byte one) and a
+  // fold along the innermost dimension that gives a row to a lane (pieces in scratch memory where the rows are few)
+  acc_skel scatter16 = make(ctx, ACC_SKEL_PERMUTE, "Int16", "(Int16)ix", "x", nullptr, "arrIn0_0[ix]", 0, 0);
+  acc_skel scatter32 = make(ctx, ACC_SKEL_PERMUTE, "Int32", "(Int32)ix", "( x )", nullptr, "arrIn0_0[ix]", 0, 0);
+  acc_skel across = make(ctx, ACC_SKEL_FOLD1, "Int32", "arrIn0_0[ix]", "x + y", nullptr, nullptr, 0, ACC_FLAG_TILED);
   acc_skel gmap = make(ctx, ACC_SKEL_MAP, "Int32", "arrIn0_0[ix] + 1", nullptr, nullptr, nullptr, 0, ACC_FLAG_GUARDED);
   acc_skel segs = make(ctx, ACC_SKEL_FOLDSEG, "Int32", "arrIn0_0[ix]", "x + y", "0", nullptr, 0, 0);
   acc_memtable table = nullptr;
@@ -127,6 +132,16 @@ int main(int argc, char **argv)
         if (r % 4 == 1) {
           acc_array d16 = vec(zeros, 3000), b16 = vec(bins, 3000), few = vec(in, 2000);
           OK(acc_exec_permute(locked, &few, 2000, &d16, &b16, st));
+        }
+        if (r % 5 == 2) {
+          acc_array d16 = vec(zeros, 3000), b16 = vec(bins, 3000), few = vec(in, 2000);
+          OK(acc_exec_permute(scatter16, &few, 2000, &d16, &b16, st));
+          acc_array d32 = vec(zeros, 5000), b32 = vec(out, 5000);
+          OK(acc_exec_permute(scatter32, &few, 2000, &d32, &b32, st));
+          const int64_t few_rows[2] = {7, 3000}, many_rows[2] = {3000, 40};
+          acc_array r7 = vec(out, 7), r3000 = vec(out, 3000);
+          OK(acc_exec_fold(across, &a, 2, few_rows, &r7, st));
+          OK(acc_exec_fold(across, &a, 2, many_rows, &r3000, st));
         }
         if (r % 6 == 2) {                       // a loop's kernels on this thread's stream, under its guard
           OK(acc_stream_set_guard(ctx, st, guard));
@@ -272,7 +287,7 @@ int main(int argc, char **argv)
     std::fprintf(stderr, "the segmented fold never went over to its variants with the table of jobs\n");
     return 3;
   }
-  for (acc_skel s : {scan, fold, hist, locked, gmap, segs}) OK(acc_skel_destroy(s));
+  for (acc_skel s : {scan, fold, hist, locked, scatter16, scatter32, across, gmap, segs}) OK(acc_skel_destroy(s));
   for (acc_devptr p : {in, out, bins, zeros}) OK(acc_free(ctx, p));
   OK(acc_context_destroy(ctx));
   std::printf("threads %d rounds %d launches %ld failures %d\n", threads, rounds, mock_hip_launches(), failures.load());
