@@ -725,6 +725,19 @@ def _unlinear(ix, shape):
         # the linear index of this very multi-index (an index function applied to the result of another, as where a
         # transposed array is replicated): taking it apart again gives the multi-index back, without a division
         return made_of[0]
+    count = 1
+    for ext in shape:
+        count *= ext
+    if 0 < count < 2 ** 31 and len(shape) > 1:
+        # an index into fewer than 2^31 elements is taken apart in 32 bits: a division by a literal is then a
+        # multiplication and a shift, where the 64-bit one is twenty instructions (generate over 500^3: 240 -> 100 us)
+        out, rest = [], Exp.mk("Word32", "((Word32)%s)", ix)
+        for d in range(len(shape) - 1, 0, -1):
+            ext = Exp("Word32", "%du" % shape[d])
+            out.append(Exp.mk("Int64", "((Int64)(%s %% %s))", rest, ext))
+            rest = Exp.mk("Word32", "(%s / %s)", rest, ext)
+        out.append(Exp.mk("Int64", "((Int64)%s)", rest))
+        return tuple(reversed(out))
     out, rest = [], ix
     for d in range(len(shape) - 1, -1, -1):
         ext = constant(shape[d], "Int64")

@@ -77,3 +77,18 @@ def test_a_fold_whose_rows_lie_across_memory_is_written_over_the_row_and_the_pla
     assert text.count("acc_col") == 2 and "%" in text
     plain = z.stream().text
     assert "acc_row" not in plain and "ix" in plain
+
+
+def test_an_index_into_fewer_than_2_to_the_31_elements_is_taken_apart_in_32_bits():
+    ix = acc.Exp("Int64", "ix")
+    small = acc._unlinear(ix, (500, 500, 500))
+    assert all(p.ctype == "Int64" for p in small)
+    assert "(Word32)ix" in small[2].term and "500u" in small[2].term and "LL" not in small[2].term
+    # 2^31 elements and more: 64-bit arithmetic throughout
+    big = acc._unlinear(ix, (70000, 70000))
+    assert all("Word32" not in p.term for p in big) and "70000LL" in big[1].term
+    # an array without elements has no index to take apart (and no division by zero is written)
+    none = acc._unlinear(ix, (0, 5))
+    assert all("Word32" not in p.term for p in none)
+    # a vector's index is the linear one
+    assert acc._unlinear(ix, (9,))[0].term == "ix"
