@@ -371,6 +371,41 @@ template <typename T> ACC_DEV T acc_stream(const T *p, const Int64 ix)
 ACC_DEV Int64 acc_to_index2(Int64, Int64 w, Int64 y, Int64 x) { return y * w + x; }
 ACC_DEV Int64 acc_to_index3(Int64, Int64 h, Int64 w, Int64 z, Int64 y, Int64 x) { return (z * h + y) * w + x; }
 
+/* The multi-index of a linear index (cfromIndex, CodeGen/Base.hs:207-218): acc_from_index<R>({ext_0, ..., ext_<R-1>},
+ * ix).i[d], outermost dimension first.  An index into fewer than 2^31 elements is taken apart in 32 bits -- a 64-bit
+ * division by an extent that is not a literal is a hundred instructions, the 32-bit one a quarter of that; the test
+ * is the same in every lane.  (A generator that knows the extents writes them as literals instead, and the divisions
+ * become multiplications.) */
+template <int R> struct acc_multi_index { Int64 i[R]; };
+template <int R>
+ACC_DEV acc_multi_index<R> acc_from_index(const Int64 (&sh)[R], const Int64 ix)
+{
+  acc_multi_index<R> m;
+  Int64 count = 1;
+#pragma unroll
+  for (int d = 0; d < R; ++d) count *= sh[d];
+  if (count > 0 && count < (Int64)0x7fffffff) {
+    unsigned int rest = (unsigned int)ix;
+#pragma unroll
+    for (int d = R - 1; d > 0; --d) {
+      const unsigned int ext = (unsigned int)sh[d];
+      m.i[d] = (Int64)(rest % ext);
+      rest /= ext;
+    }
+    m.i[0] = (Int64)rest;
+  } else {
+    Int64 rest = ix;
+#pragma unroll
+    for (int d = R - 1; d > 0; --d) {
+      const Int64 ext = sh[d] > 0 ? sh[d] : 1;
+      m.i[d] = rest % ext;
+      rest /= ext;
+    }
+    m.i[0] = rest;
+  }
+  return m;
+}
+
 /* the scalar primitives of the expression language */
 #include "acc_prim.h"
 

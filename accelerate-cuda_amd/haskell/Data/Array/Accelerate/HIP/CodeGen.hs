@@ -420,16 +420,15 @@ codegenPermutation _ _ _ = error "codegenPermutation: expected a unary function"
 toIndex :: [String] -> [String] -> String
 toIndex sh ix = foldl (\acc (s, i) -> "(" ++ acc ++ " * " ++ s ++ " + " ++ i ++ ")") "((Int64)0)" (zip sh ix)
 
+-- the device header's acc_from_index takes an index into fewer than 2^31 elements apart in 32 bits (the extents are
+-- kernel parameters here, not literals: a 64-bit division by one of them is a hundred instructions); the compiler
+-- makes one decomposition of the components' identical calls
 fromIndex :: [String] -> String -> [String]
-fromIndex sh i = [ component d | d <- [0 .. n - 1] ]
+fromIndex []  _ = []
+fromIndex [_] i = [i]
+fromIndex sh  i = [ "acc_from_index<" ++ show n ++ ">({" ++ intercalate ", " [ "(Int64)(" ++ s ++ ")" | s <- sh ] ++ "}, " ++ i ++ ").i[" ++ show d ++ "]" | d <- [0 .. n - 1] ]
   where
     n = length sh
-    component d
-      | d == 0    = quotient d
-      | otherwise = "(" ++ quotient d ++ " % " ++ (sh !! d) ++ ")"
-    quotient d = case drop (d + 1) sh of
-                   []   -> i
-                   rest -> "(" ++ i ++ " / " ++ product' rest ++ ")"
 
 product' :: [String] -> String
 product' [] = "((Int64)1)"

@@ -254,3 +254,30 @@ def test_stencil_over_more_than_2_31_elements(A, ctx):
         up, dn = img[np.maximum(rows - 1, 0)].astype(np.int32), img[np.minimum(rows + 1, h - 1)].astype(np.int32)
         left, right = np.concatenate([c[:, :1], c[:, :-1]], axis=1), np.concatenate([c[:, 1:], c[:, -1:]], axis=1)
         assert np.array_equal(got[rows], (up + left + c + right + dn).astype(np.int8)), y0
+
+
+def test_the_device_header_s_multi_index_of_a_linear_index(A, ctx):
+    """`acc_from_index<R>({extents}, ix)` in an element function: ranks 2 to 4 with extents that are no powers of two,
+    a result without elements, and an array of more than 2^31 elements (64-bit arithmetic; rows on both sides of
+    index 2^31 are looked at)."""
+    for shape in ((7, 11), (37, 1, 53), (3, 5, 7, 11), (1000, 999), (0, 5)):
+        r = len(shape)
+        ext = ", ".join("shOut_%d" % d for d in range(r - 1, -1, -1))
+        parts = " + ".join("%d * acc_from_index<%d>({%s}, ix).i[%d]" % (10 ** (2 * (r - 1 - d)), r, ext, d) for d in range(r))
+        say("acc_from_index", shape)
+        sk = ctx.skeleton(A.SKEL_GENERATE, "Int64", out_rank=r, get="(Int64)(%s)" % parts)
+        out = ctx.empty(shape, np.int64)
+        sk.map([], out)
+        idx = np.indices(shape, dtype=np.int64) if all(shape) else np.zeros((r,) + shape, np.int64)
+        want = sum(idx[d] * 10 ** (2 * (r - 1 - d)) for d in range(r))
+        assert np.array_equal(out.get(), want), shape
+    h, w = 46400, 46400                                   # 2 152 960 000 elements
+    say("acc_from_index beyond 2^31 elements", h, w)
+    sk = ctx.skeleton(A.SKEL_GENERATE, "Word8", out_rank=2,
+                      get="(Word8)(acc_from_index<2>({shOut_1, shOut_0}, ix).i[0] * 7 + acc_from_index<2>({shOut_1, shOut_0}, ix).i[1])")
+    out = ctx.empty((h, w), np.uint8)
+    sk.map([], out)
+    got = out.get()
+    xs = np.arange(w, dtype=np.int64)
+    for y in (0, 1, 46280, 46281, 46282, h - 1):            # (index 2^31 lies in row 46 281)
+        assert np.array_equal(got[y], ((y * 7 + xs) & 255).astype(np.uint8)), y
