@@ -313,8 +313,10 @@ class Acc(object):
     def __init__(self, shape, ctype, manifest=None, at=None, across=False):
         self.shape, self.ctype, self.manifest, self.at = tuple(int(s) for s in shape), ctype, manifest, at
         # a delayed array that reads a source across its rows (a transpose): the map kernel that makes it manifest
-        # produces it in square tiles (ACC_FLAG_TILED)
-        self.across = bool(across) and manifest is None and len(self.shape) >= 2
+        # produces it in square tiles (ACC_FLAG_TILED).  The number of the result's dimension, counted from the
+        # innermost, along which the source is read: 1 for a transpose, 2 and more for a volume that was turned
+        # (ACC_FLAG_TILE_DIM); 0 for an array read along its rows.
+        self.across = int(across) if (across and manifest is None and len(self.shape) >= 2) else 0
 
     @property
     def size(self):
@@ -799,9 +801,9 @@ def generate(shape, f):
 
 def _steps_of(p, shape, src_shape):
     """how far `p` moves through the source (in elements of its row-major order) where the result's index moves by
-    one along the innermost and along the second innermost dimension: found by applying `p` to plain numbers, which
-    an index function made of arithmetic alone accepts.  None where it does not, or where the result is too small
-    to take a step."""
+    one along each of its dimensions, the innermost first: found by applying `p` to plain numbers, which an index
+    function made of arithmetic alone accepts.  None where it does not, or where the result is too small to take a
+    step along its two innermost dimensions."""
     if len(shape) < 2 or shape[-1] < 2 or shape[-2] < 2:
         return None
 
@@ -817,7 +819,10 @@ def _steps_of(p, shape, src_shape):
     try:
         zero = [0] * len(shape)
         here = place(zero)
-        return place(zero[:-1] + [1]) - here, place(zero[:-2] + [1, 0]) - here
+        steps = []
+        for d in range(len(shape) - 1, -1, -1):               # innermost dimension first
+            steps.append(place(zero[:d] + [1] + zero[d + 1:]) - here if shape[d] >= 2 else 0)
+        return steps
     except Exception:
         return None
 
@@ -829,14 +834,19 @@ def backpermute(shape, p, a, across=None):
     shape = (shape,) if isinstance(shape, numbers.Integral) else tuple(shape)
     if across is None:
         steps = _steps_of(p, shape, a.shape)
+        across = 0
         if steps is None:
-            across = False
+            pass
         elif abs(steps[0]) == 1:
-            across = a.across              # along the rows of `a`: what `a` reads across, the result does
-        elif abs(steps[1]) == 1 and steps[0] != 0:
-            across = not a.across          # down the columns of `a`
-        else:
-            across = False
+            across = a.across if a.across <= 1 else 0    # along the rows of `a`: what `a` reads across, the result does
+        elif steps[0] != 0 and a.across == 0:
+            # the dimension of the result along which `a` is read side by side: the second innermost (a transpose),
+            # or one further out (a volume turned so that its innermost dimension becomes an outer one)
+            for d in range(1, len(steps)):
+                if abs(steps[d]) == 1:
+                    across = d
+                    break
+        # (an exchange of the two innermost dimensions of an array that is itself read across: along the rows again)
     return Acc(shape, a.ctype, at=lambda ix: a.index(_linear(p(*_unlinear(ix, shape)), a.shape)), across=across)
 
 
@@ -866,7 +876,8 @@ def _force(a, cx):
     if a.manifest is not None:
         return a
     arrays, sig, fr = _assemble(get=a.stream().text)
-    sk = cx.skeleton(A.SKEL_MAP, _elt(a.ctype), sig, out_rank=len(a.shape), flags=A.FLAG_TILED if a.across else 0, **fr)
+    sk = cx.skeleton(A.SKEL_MAP, _elt(a.ctype), sig, out_rank=len(a.shape),
+                     flags=(A.FLAG_TILED | A.FLAG_TILE_DIM(a.across)) if a.across else 0, **fr)
     out = _empty(cx, a.shape, a.ctype)
     cx.launch(arrays, [out], lambda i, o, s: sk.map(i, o[0], stream=s))
     return Acc(a.shape, a.ctype, manifest=out)
@@ -883,7 +894,7 @@ def _fold(f, z, a, seedless, context):
     cx = _context(context, a)
     # an empty outer extent counts as 1 in the result of a seeded fold (Execute.hs:287-289)
     out_shape = a.shape[:-1] if seedless else tuple(max(1, d) for d in a.shape[:-1])
-    _building.rows_of = tuple(a.shape) if a.across else None
+    _building.rows_of = tuple(a.shape) if a.across == 1 else None
     try:
         get = a.stream().text
     finally:
@@ -891,7 +902,7 @@ def _fold(f, z, a, seedless, context):
     arrays, sig, fr = _assemble(get=get, combine=_combine(f, a.ctype).text, seed=None if seedless else Exp.of(z, a.ctype).text)
     # rows that lie across memory (the fold of a transposed matrix, of a product of replicated operands): a lane a row
     sk = cx.skeleton(A.SKEL_FOLD1 if seedless else A.SKEL_FOLD, _elt(a.ctype), sig, out_rank=len(out_shape),
-                     flags=A.FLAG_TILED if a.across and len(out_shape) >= 1 else 0, **fr)
+                     flags=A.FLAG_TILED if a.across == 1 and len(out_shape) >= 1 else 0, **fr)
     out = _empty(cx, out_shape, a.ctype)
     cx.launch(arrays, [out], lambda i, o, s: sk.fold(i, a.shape, o[0], stream=s))
     return Acc(out_shape, a.ctype, manifest=out)

@@ -27,6 +27,11 @@ COMBINE_GENERIC, COMBINE_ADD, COMBINE_MIN, COMBINE_MAX, COMBINE_AND, COMBINE_OR,
 BOUNDARY = {"clamp": 0, "mirror": 1, "wrap": 2, "constant": 3}
 FLAG_FOLD_RIGHT, FLAG_FAST_MATH, FLAG_GUARDED, FLAG_TILED = 1, 2, 4, 8
 
+
+def FLAG_TILE_DIM(d):
+    """with FLAG_TILED on a map of rank >= 3: the tiles' second dimension is the d-th above the innermost one"""
+    return int(d) << 8
+
 CTYPE = {np.dtype(np.float32): "float", np.dtype(np.float64): "double",
          np.dtype(np.int8): "Int8", np.dtype(np.int16): "Int16", np.dtype(np.int32): "Int32",
          np.dtype(np.int64): "Int64", np.dtype(np.uint8): "Word8", np.dtype(np.uint16): "Word16",

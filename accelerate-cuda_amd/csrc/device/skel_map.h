@@ -51,11 +51,15 @@ ACC_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_GUARD_PARAM)
   ACC_ENV_ASSUME
   auto get = [&](const Int64 ix) -> T { return (ACC_GET(ix)); };
 
-  const Int64 w = shOut_0, h = shOut_1;
+  /* The tiles' second dimension is the second innermost one of the result, or one further out (ACC_TILE_H its
+   * extent, ACC_TILE_STRIDE the elements between neighbours along it: a volume turned so that its innermost
+   * dimension becomes its outermost reads its source along that one).  What lies between that dimension and the
+   * innermost (`mids` rows for every place along it) and outside it (`outers`) is walked tile by tile. */
+  const Int64 w = shOut_0, h = ACC_TILE_H, stride = ACC_TILE_STRIDE;
   const Int64 n = (ACC_OUT_SIZE);
-  const Int64 planes = (w > 0 && h > 0) ? n / (w * h) : 0;
+  const Int64 mids = w > 0 ? stride / w : 0, outers = (h > 0 && stride > 0) ? n / (h * stride) : 0;
   const Int64 tiles_x = (w + ACC_TSIDE - 1) / ACC_TSIDE, tiles_y = (h + ACC_TSIDE - 1) / ACC_TSIDE;
-  const Int64 tiles = tiles_x * tiles_y * planes;
+  const Int64 tiles = tiles_x * tiles_y * mids * outers;
   const int lane = acc_lane();
   const int lx = lane & 7, ly = lane >> 3;
   const Int64 wave = (Int64)blockIdx.x * (ACC_BLOCK / ACC_WAVE) + (Int64)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -63,25 +67,26 @@ ACC_ENTRY(ACC_ENV_PARAMS ACC_OUT_PARAMS ACC_GUARD_PARAM)
 
   for (Int64 tile = wave; tile < tiles; tile += step) {
     const Int64 tx = tile % tiles_x, ty = (tile / tiles_x) % tiles_y, plane = tile / (tiles_x * tiles_y);
+    const Int64 mid = plane % mids, outer = plane / mids;
     const Int64 x = tx * ACC_TSIDE + lx * ACC_TT, y = ty * ACC_TSIDE + ly * ACC_TT;
-    const Int64 base = (plane * h + y) * w + x;
+    const Int64 base = ((outer * h + y) * mids + mid) * w + x;
     if ((tx + 1) * ACC_TSIDE <= w && (ty + 1) * ACC_TSIDE <= h) {
       T v[ACC_TT][ACC_TT];
       /* down the columns first: what a transposed source holds side by side */
 #pragma unroll
       for (int k = 0; k < ACC_TT; ++k)
 #pragma unroll
-        for (int i = 0; i < ACC_TT; ++i) v[i][k] = get(base + i * w + k);
+        for (int i = 0; i < ACC_TT; ++i) v[i][k] = get(base + i * stride + k);
 #pragma unroll
       for (int i = 0; i < ACC_TT; ++i)
 #pragma unroll
-        for (int k = 0; k < ACC_TT; ++k) ACC_SET(arrOut, base + i * w + k, v[i][k]);
+        for (int k = 0; k < ACC_TT; ++k) ACC_SET(arrOut, base + i * stride + k, v[i][k]);
     } else {
 #pragma unroll
       for (int i = 0; i < ACC_TT; ++i)
 #pragma unroll
         for (int k = 0; k < ACC_TT; ++k)
-          if (x + k < w && y + i < h) ACC_SET(arrOut, base + i * w + k, get(base + i * w + k));
+          if (x + k < w && y + i < h) ACC_SET(arrOut, base + i * stride + k, get(base + i * stride + k));
     }
   }
 }

@@ -280,14 +280,15 @@ int acc_exec_map(acc_skel s, const acc_array *env, const acc_array *out, acc_str
   // of 8 / 16 / 24 / 32 columns: 45 / 56 / 100 / 44 us in tiles, 10 / 20 / 40 / 41 in runs, and 29 against 52 for 33
   // columns.  Of 6 / 8 / 12 / 16 rows of 2^20 columns: 41 / 41 / 43 / 43 in tiles, 17 / 31 / 82 / 151 in runs.)
   const bool in_tiles = s->spec.map_tiled && out->shape[s->spec.out_rank - 1] >= s->knobs.map_tiled_min_w &&
-                        out->shape[s->spec.out_rank - 2] >= s->knobs.map_tiled_min_h;
+                        out->shape[s->spec.out_rank - 1 - s->spec.map_tile_dim] >= s->knobs.map_tiled_min_h;
   if (s->spec.map_tiled && !in_tiles) v += 2;
   ACC_TRY(s->ensure_variant(v));
   if (in_tiles) {
-    // a wave per tile of 32 x 32 elements of the two innermost dimensions (skel_map.h)
+    // a wave per tile of 32 x 32 elements of the innermost dimension and the second innermost one, or the one that
+    // ACC_FLAG_TILE_DIM names (skel_map.h)
     const int rank = s->spec.out_rank;
     const int64_t side = 8 * (int64_t)s->spec.map_tile_block;
-    const int64_t w = out->shape[rank - 1], h = out->shape[rank - 2];
+    const int64_t w = out->shape[rank - 1], h = out->shape[rank - 1 - s->spec.map_tile_dim];
     const int64_t tiles = ((w + side - 1) / side) * ((h + side - 1) / side) * (n / (w * h));
     const int64_t waves = s->variants[v].block / 64;
     return launch(s, v, std::min<int64_t>((tiles + waves - 1) / waves, (int64_t)1 << 22), 0, static_cast<hipStream_t>(stream), &args);

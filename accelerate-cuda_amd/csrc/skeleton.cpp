@@ -206,6 +206,12 @@ int generate_source(const SkelSpec &sp, bool aligned, std::string *entry, std::s
       o << "#define ACC_OUT_SIZE " << out_size(sp.out_rank) << "\n";
       o << "#define ACC_BLOCK " << sp.block << "\n#define ACC_VEC " << vec << "\n#define ACC_UNROLL " << sp.unroll << "\n";
       o << "#define ACC_MAP_TILED " << (sp.map_tiled ? 1 : 0) << "\n#define ACC_TT " << sp.map_tile_block << "\n";
+      if (sp.map_tiled) {
+        // the tiles' second dimension: its extent, and the elements between neighbours along it
+        o << "#define ACC_TILE_H shOut_" << sp.map_tile_dim << "\n#define ACC_TILE_STRIDE (";
+        for (int dd = 0; dd < sp.map_tile_dim; ++dd) o << (dd ? " * " : "") << "shOut_" << dd;
+        o << ")\n";
+      }
       tmpl = "skel_map.h";
       break;
     case ACC_SKEL_FOLD:
@@ -539,6 +545,10 @@ int make_spec(const acc_skel_desc *d, const TuningPtr &tuning, SkelSpec *sp)
   sp->map_tile_block = std::max(1, std::min(tune("map.tile_block", 4), 8));
   sp->map_tiled = (d->flags & ACC_FLAG_TILED) != 0 && d->out_rank >= 2 &&
                   (d->kind == ACC_SKEL_MAP || d->kind == ACC_SKEL_GENERATE || d->kind == ACC_SKEL_TRANSFORM) && tune("map.tiled", 1) != 0;
+  sp->map_tile_dim = (int)((d->flags >> 8) & 15u);
+  if (sp->map_tile_dim == 0) sp->map_tile_dim = 1;
+  if (sp->map_tiled && sp->map_tile_dim >= d->out_rank)
+    return fail(ACC_ERR_INVALID, "%s: ACC_FLAG_TILE_DIM(%d) on a result of rank %d", kind_name(d->kind), sp->map_tile_dim, d->out_rank);
   sp->fold_across = (d->flags & ACC_FLAG_TILED) != 0 && d->out_rank >= 1 && (d->kind == ACC_SKEL_FOLD || d->kind == ACC_SKEL_FOLD1);
   sp->out_rank = d->out_rank;
   if (sp->out_rank < 0 || sp->out_rank > ACC_MAX_RANK) return fail(ACC_ERR_INVALID, "bad out_rank %d", d->out_rank);

@@ -51,6 +51,7 @@ struct SkelSpec {
   int chunk_long = 0;                   // segmented folds: the staged chunk of variants 2 and 3 (segments of 8 elements or more on average); 0: none
   bool fold_across = false;             // ACC_FLAG_TILED on a fold along the innermost dimension: neighbouring rows are neighbours in memory
   bool permute_replace = false;         // permute whose combination is spelt `x` (the new value): plain stores
+  int map_tile_dim = 1;                 // ACC_FLAG_TILE_DIM: which dimension of the result, counted from the innermost, the tiles pair with it
   bool map_tiled = false;               // ACC_FLAG_TILED on a map of rank 2 or more: tiles of 32 x 32 elements, a wave each
   int map_tile_block = 4;               // ... a lane's share of a tile: a block of that many elements either way
   bool guarded = false;                 // ACC_FLAG_GUARDED: every kernel takes the address of a loop's guard word last

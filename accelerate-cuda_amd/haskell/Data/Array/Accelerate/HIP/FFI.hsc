@@ -97,6 +97,11 @@ accFlagFastMath  = #{const ACC_FLAG_FAST_MATH}
 accFlagGuarded   = #{const ACC_FLAG_GUARDED}
 accFlagTiled     = #{const ACC_FLAG_TILED}
 
+-- | ACC_FLAG_TILE_DIM(d): with 'accFlagTiled', which dimension of the result (counted from the innermost) the tiles
+-- pair with the innermost one
+accFlagTileDim :: Int -> Word32
+accFlagTileDim d = fromIntegral d `shiftL` 8
+
 data HIPException = HIPException Status String
   deriving (Typeable)
 

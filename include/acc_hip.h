@@ -295,6 +295,11 @@ enum { ACC_BOUNDARY_CLAMP = 0, ACC_BOUNDARY_MIRROR = 1, ACC_BOUNDARY_WRAP = 2, A
                                      and the place within it: ix == acc_row * row length + acc_col.  Kernels that give
                                      a row to a lane know both without a division, and what depends on acc_row alone
                                      leaves the lane's loop.) */
+#define ACC_FLAG_TILE_DIM(d)  ((uint32_t)(d) << 8)  /* with ACC_FLAG_TILED on a map of rank >= 3: the tiles' second dimension
+                                     is the d-th above the innermost one (1, and what 0 means: the second innermost; 2: the
+                                     third innermost, ...), for an element function that reads its sources along THAT
+                                     dimension of the result -- a volume turned so that what was its innermost dimension
+                                     becomes its outermost; 1 <= d < out_rank */
 #define ACC_FLAG_GUARDED      4u  /* the instance may run under an acc_guard (see acc_guard_create): its kernels take the
                                      guard's address as one more, last, parameter and do nothing once the guard is down */
 

@@ -58,6 +58,9 @@ def test_index_functions_are_asked_by_applying_them_to_numbers():
     # too small to take a step, a vector: not across
     assert not acc.transpose(source("T", (1, 9))).across
     assert not acc.backpermute((9,), lambda i: (8 - i,), source("V", (9,))).across
+    # a volume turned: which dimension of the result, counted from the innermost, the source is read along
+    assert acc.backpermute((7, 5, 6), lambda k, i, j: (i, j, k), c).across == 2
+    assert acc.backpermute((5, 7, 6), lambda i, k, j: (i, j, k), c).across == 1
     # map and zipWith pass it on
     t = acc.transpose(m)
     assert acc.map(lambda v: v + v, t).across and acc.zipWith(lambda p, q: p * q, t, source("N", (32, 64))).across

@@ -837,6 +837,15 @@ def test_column_sums_and_a_matrix_product_written_as_folds(acc):
     assert swapped.across and not acc.backpermute((60, 5, 70), lambda j, i, k: (i, j, k), acc.use(c)).across
     assert np.array_equal(acc.run(swapped), c.transpose(0, 2, 1))
     assert np.array_equal(acc.run(acc.fold(add, 0, swapped)), c.sum(axis=1, dtype=np.int32))
+    # a volume turned so that its innermost dimension becomes the outermost: the source is read along the result's
+    # outermost dimension, and the tiles pair that one with the innermost (ACC_FLAG_TILE_DIM)
+    turned = acc.backpermute((70, 5, 60), lambda k, i, j: (i, j, k), acc.use(c))
+    assert turned.across == 2
+    assert np.array_equal(acc.run(turned), c.transpose(2, 0, 1))
+    c4 = rng.integers(-50, 50, (3, 40, 5, 70)).astype(np.int32)
+    turned4 = acc.backpermute((3, 70, 5, 40), lambda a_, l, k, j: (a_, j, k, l), acc.use(c4))
+    assert turned4.across == 2
+    assert np.array_equal(acc.run(acc.map(lambda v: v + v, turned4)), 2 * c4.transpose(0, 3, 2, 1))
     mm, kk, nn = 70, 333, 129
     a = rng.integers(-9, 9, (mm, kk)).astype(np.int32)
     b = rng.integers(-9, 9, (kk, nn)).astype(np.int32)

@@ -1044,6 +1044,24 @@ def test_map_in_tiles_gives_what_the_map_in_runs_gives(A, ctx):
         out = ctx.empty(shape, np.int32)
         g.map([], out)
         assert np.array_equal(out.get().reshape(-1), (np.arange(int(np.prod(shape)), dtype=np.int64) * 7 + 1).astype(np.int32))
+    say("tiles of the innermost dimension and one further out than the second innermost (ACC_FLAG_TILE_DIM)")
+    for rank, dim, shapes in ((3, 2, ((1, 1, 1), (40, 3, 50), (33, 2, 65), (300, 1, 5), (70, 40, 33))), (4, 2, ((2, 40, 3, 50),)),
+                              (4, 3, ((40, 2, 3, 50), (33, 1, 1, 65)))):
+        g = ctx.skeleton(A.SKEL_GENERATE, "Int32", env=[], out_rank=rank, flags=A.FLAG_TILED | A.FLAG_TILE_DIM(dim), get="(Int32)(ix * 7 + 1)")
+        for shape in shapes:
+            out = ctx.array(np.full(int(np.prod(shape)) + 2, 77, np.int32))
+            g.map([], out.desc(shape=shape))
+            got = out.get()
+            assert np.array_equal(got[:-2], (np.arange(int(np.prod(shape)), dtype=np.int64) * 7 + 1).astype(np.int32)), (rank, dim, shape)
+            assert np.array_equal(got[-2:], [77, 77])
+    vol = rng.integers(-100, 100, (30, 45, 70)).astype(np.int32)               # turned: result[k, i, j] = vol[i, j, k]
+    tv = ctx.skeleton(A.SKEL_MAP, "Int32", env=[(3, "Int32")], out_rank=3, flags=A.FLAG_TILED | A.FLAG_TILE_DIM(2),
+                      get="arrIn0_0[((ix / shOut_0) % shOut_1) * (shIn0_1 * shIn0_0) + (ix % shOut_0) * shIn0_0 + ix / (shOut_0 * shOut_1)]")
+    out = ctx.empty((70, 30, 45), np.int32)
+    tv.map([ctx.array(vol)], out)
+    assert np.array_equal(out.get(), vol.transpose(2, 0, 1))
+    with pytest.raises(A.AccError):
+        ctx.skeleton(A.SKEL_GENERATE, "Int32", env=[], out_rank=2, flags=A.FLAG_TILED | A.FLAG_TILE_DIM(2), get="(Int32)ix", wait=True)
     say("tiled map producing pairs (one array per component)")
     pt = ctx.skeleton(A.SKEL_MAP, "float, Int32", env=[(2, "float"), (2, "Int32")], out_rank=2, flags=A.FLAG_TILED,
                       get="acc_elt{arrIn0_0[(ix % shOut_0) * shIn0_0 + (ix / shOut_0)] * 2.0f, arrIn1_0[ix] + 1}")
