@@ -892,6 +892,22 @@ def _combine(f, ctype):
 
 def _fold(f, z, a, seedless, context):
     cx = _context(context, a)
+    if a.across >= 2 and len(a.shape) > a.across:
+        # The source is read side by side along a dimension of `a` further out than the second innermost (the sum
+        # over the middle dimension of a volume, written as a fold of the volume turned): the fold of `a` with that
+        # dimension and the second innermost exchanged gives a row to a lane with neighbouring rows side by side in
+        # memory, and its result with the two exchanged back (delayed: whoever consumes it reads it across) is the
+        # fold of `a`.
+        r = len(a.shape)
+        i1, id_ = r - 2, r - 1 - a.across
+
+        def exchanged(ix):
+            ix = list(ix)
+            ix[i1], ix[id_] = ix[id_], ix[i1]
+            return tuple(ix)
+        turned = backpermute(exchanged(a.shape), lambda *ix: exchanged(ix), a, across=1)
+        folded = _fold(f, z, turned, seedless, cx)
+        return backpermute(exchanged(folded.shape), lambda *ix: exchanged(ix), folded)
     # an empty outer extent counts as 1 in the result of a seeded fold (Execute.hs:287-289)
     out_shape = a.shape[:-1] if seedless else tuple(max(1, d) for d in a.shape[:-1])
     _building.rows_of = tuple(a.shape) if a.across == 1 else None

@@ -842,10 +842,16 @@ def test_column_sums_and_a_matrix_product_written_as_folds(acc):
     turned = acc.backpermute((70, 5, 60), lambda k, i, j: (i, j, k), acc.use(c))
     assert turned.across == 2
     assert np.array_equal(acc.run(turned), c.transpose(2, 0, 1))
+    # its fold -- the sum over the volume's middle dimension -- goes through the fold of the volume with the two
+    # dimensions exchanged, a lane a row, and comes back exchanged
+    before = len(cx.skeletons)
+    assert np.array_equal(acc.run(acc.fold(add, 0, turned)), c.sum(axis=1, dtype=np.int32).T)
+    assert np.array_equal(acc.run(acc.fold1(lambda p, q: acc.cond(p > q, p, q), turned)), c.max(axis=1).T)
     c4 = rng.integers(-50, 50, (3, 40, 5, 70)).astype(np.int32)
     turned4 = acc.backpermute((3, 70, 5, 40), lambda a_, l, k, j: (a_, j, k, l), acc.use(c4))
     assert turned4.across == 2
     assert np.array_equal(acc.run(acc.map(lambda v: v + v, turned4)), 2 * c4.transpose(0, 3, 2, 1))
+    assert np.array_equal(acc.run(acc.fold(add, 0, turned4)), c4.transpose(0, 3, 2, 1).sum(axis=3, dtype=np.int32))
     mm, kk, nn = 70, 333, 129
     a = rng.integers(-9, 9, (mm, kk)).astype(np.int32)
     b = rng.integers(-9, 9, (kk, nn)).astype(np.int32)
