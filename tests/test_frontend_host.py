@@ -111,7 +111,7 @@ def test_index_arithmetic_of_the_delayed_combinators():
     y, x = ix // 3, ix % 3                       # the result's (row, column)
     # (the text as Python reads it: casts and literal suffixes off -- the index of so small an array is taken apart in
     # 32 bits -- and the division a floor division)
-    text = fr["get"].replace("arrIn0_0", "src").replace("((Int64)", "(").replace("((Word32)", "(").replace("LL)", ")")
+    text = re.sub(r"\((Int64|Word32)\)", "", fr["get"].replace("arrIn0_0", "src")).replace("LL)", ")")
     text = re.sub(r"(\d)u\b", r"\1", text).replace("/", "//")
     src = eval(text, {"src": np.arange(15), "ix": ix})
     assert np.array_equal(src, x * 5 + y)
